@@ -1,0 +1,26 @@
+"""MI355X-native fused equivariant message-passing convolution.
+
+Public names follow the reference package for this path: `Convolution`,
+`convolution`, `convolution_bwd`, `GraphCSR`, `Coef4D`, `O3Space`, `config`.
+Importing the package does not load the kernel library; the first operator call does,
+and fails if `e3j_amd/lib/libe3j_amd.so` has not been built.
+"""
+
+from .coef import Coef, Coef4D, resolve_val_dtype
+from .convolution import Convolution
+from .graph import DUMMY_INDEX, GraphCSR
+from .ops import (ConvolutionBatchingWarning, ConvolutionParams, CUDAConvolutionParams,
+                  convolution, convolution_batched, convolution_bwd)
+from .options import Config, GraphOrdering, Layout, TensorProductNormalization, config
+from .scalar_mixing import ScalarMixing
+from .spaces import O3Irrep, O3Space
+from .tensor_product import TensorProduct
+
+Space = O3Space
+
+__all__ = [
+    "Coef", "Coef4D", "Config", "Convolution", "ConvolutionBatchingWarning", "ConvolutionParams",
+    "CUDAConvolutionParams", "DUMMY_INDEX", "GraphCSR", "GraphOrdering", "Layout", "O3Irrep",
+    "O3Space", "ScalarMixing", "Space", "TensorProduct", "TensorProductNormalization", "config",
+    "convolution", "convolution_batched", "convolution_bwd", "resolve_val_dtype",
+]

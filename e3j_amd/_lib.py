@@ -1,0 +1,95 @@
+"""ctypes binding of `libe3j_amd.so` (declarations of `include/e3j_amd.h`).
+
+There is no fallback: if the library has not been built, loading raises and
+every operator of this package fails.  Takes the place of the reference's
+`e3j_ops` pybind11 module and its registration (`lib/e3j_ops/ffi/e3j_ops.cpp:79-100`,
+`src/e3j/ops/__init__.py:22-23`).
+"""
+
+from __future__ import annotations
+
+import ctypes
+import os
+
+_HERE = os.path.dirname(os.path.abspath(__file__))
+LIB_PATH = os.path.join(_HERE, "lib", "libe3j_amd.so")
+
+OK, INVALID_ARGUMENT, UNIMPLEMENTED, INTERNAL = 0, 1, 2, 3
+LAYOUT_LEADING, LAYOUT_TRAILING = 0, 1
+F32, F64 = 0, 1
+
+
+class ConvParams(ctypes.Structure):
+    """`e3j_amd_conv_params`."""
+
+    _fields_ = [
+        ("num_nodes", ctypes.c_int32),
+        ("num_edges", ctypes.c_int64),
+        ("num_coef", ctypes.c_int32),
+        ("num_x", ctypes.c_int32),
+        ("num_y", ctypes.c_int32),
+        ("num_out", ctypes.c_int32),
+        ("num_scalars", ctypes.c_int32),
+        ("channels", ctypes.c_int32),
+        ("layout", ctypes.c_int32),
+        ("val_dtype", ctypes.c_int32),
+        ("coef_idx_bytes", ctypes.c_int32),
+        ("signature", ctypes.c_int32),
+        ("coef_scale", ctypes.c_float),
+        ("debug", ctypes.c_int32),
+    ]
+
+
+class E3jAmdError(RuntimeError):
+    """Failure reported by the kernel library; `.code` is the status code."""
+
+    def __init__(self, code: int, message: str):
+        super().__init__(message)
+        self.code = code
+
+
+_P = ctypes.c_void_p
+_PARAMS = ctypes.POINTER(ConvParams)
+
+#: name -> (restype, argtypes): every symbol `include/e3j_amd.h` declares.
+SYMBOLS = {
+    "e3j_amd_last_error": (ctypes.c_char_p, []),
+    "e3j_amd_version": (ctypes.c_char_p, []),
+    "e3j_amd_convolution_fwd": (ctypes.c_int, [_PARAMS] + [_P] * 9),
+    "e3j_amd_convolution_bwd_sender": (ctypes.c_int, [_PARAMS] + [_P] * 12),
+    "e3j_amd_convolution_bwd_receiver": (ctypes.c_int, [_PARAMS] + [_P] * 12),
+    "e3j_amd_find_signature": (ctypes.c_int, [_P] + [ctypes.c_int32] * 9 + [ctypes.POINTER(ctypes.c_float)]),
+    "e3j_amd_num_signatures": (ctypes.c_int, []),
+    "e3j_amd_signature_name": (ctypes.c_char_p, [ctypes.c_int]),
+    "e3j_amd_csr_workspace_bytes": (ctypes.c_size_t, [ctypes.c_int32, ctypes.c_int64]),
+    "e3j_amd_csr_row_ptr": (ctypes.c_int, [_P, ctypes.c_int64, ctypes.c_int32, _P, _P, _P]),
+    "e3j_amd_sort_edges": (ctypes.c_int, [_P, _P, ctypes.c_int64, ctypes.c_int32, _P, _P, _P, _P, _P]),
+    "e3j_amd_xla_convolution": (_P, [_P]),
+    "e3j_amd_xla_convolution_bwd": (_P, [_P]),
+    "e3j_amd_xla_convolution_bwd_receiver": (_P, [_P]),
+}
+
+_lib = None
+
+
+def load() -> ctypes.CDLL:
+    """Load the library once; raise if it is missing or lacks a declared symbol."""
+    global _lib
+    if _lib is not None:
+        return _lib
+    if not os.path.exists(LIB_PATH):
+        raise ImportError(
+            f"{LIB_PATH} is missing: build it with `python -m e3j_amd.build` "
+            "(hipcc, gfx950). e3j_amd has no fallback implementation.")
+    lib = ctypes.CDLL(LIB_PATH)
+    for name, (restype, argtypes) in SYMBOLS.items():
+        fn = getattr(lib, name)  # AttributeError if the export is missing
+        fn.restype = restype
+        fn.argtypes = argtypes
+    _lib = lib
+    return lib
+
+
+def check(code: int) -> None:
+    if code != OK:
+        raise E3jAmdError(code, load().e3j_amd_last_error().decode())

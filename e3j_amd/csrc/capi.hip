@@ -1,0 +1,197 @@
+// C-ABI entry points: argument validation, kernel selection, error reporting.
+
+#include <cmath>
+#include <cstring>
+
+#include "common.h"
+
+namespace e3j_amd {
+
+static thread_local std::string g_last_error;
+
+int set_error(int code, const std::string &msg) {
+    const char *cls = code == E3J_AMD_INVALID_ARGUMENT ? "InvalidArgument"
+                    : code == E3J_AMD_UNIMPLEMENTED    ? "Unimplemented"
+                                                       : "Internal";
+    g_last_error = std::string("E3J_AMD_ERROR[") + cls + "]: " + msg;
+    return code;
+}
+
+int check_hip(hipError_t err, const char *what) {
+    if (err == hipSuccess) return E3J_AMD_OK;
+    return set_error(E3J_AMD_INTERNAL, std::string(what) + ": " + hipGetErrorString(err));
+}
+
+namespace {
+
+int validate(const e3j_amd_conv_params *p, const char *op) {
+    const std::string name(op);
+    if (p == nullptr) return set_error(E3J_AMD_INVALID_ARGUMENT, name + ": null params");
+    if (p->num_nodes < 0 || p->num_edges < 0 || p->num_coef < 0)
+        return set_error(E3J_AMD_INVALID_ARGUMENT, name + ": negative size");
+    if (p->num_x < 1 || p->num_y < 1 || p->num_out < 1 || p->num_scalars < 1 || p->channels < 1)
+        return set_error(E3J_AMD_INVALID_ARGUMENT,
+                         name + ": num_x, num_y, num_out, num_scalars and channels must be >= 1");
+    if (p->layout != E3J_AMD_LAYOUT_LEADING && p->layout != E3J_AMD_LAYOUT_TRAILING)
+        return set_error(E3J_AMD_INVALID_ARGUMENT, name + ": unknown layout " + std::to_string(p->layout));
+    if (p->val_dtype != E3J_AMD_F32 && p->val_dtype != E3J_AMD_F64)
+        return set_error(E3J_AMD_INVALID_ARGUMENT, name + ": unsupported (IDX, VAL) dtype pair");
+    if (p->coef_idx_bytes != 1 && p->coef_idx_bytes != 4)
+        return set_error(E3J_AMD_INVALID_ARGUMENT, name + ": unsupported (IDX, VAL) dtype pair");
+    if (p->num_edges > 0x7fffffffLL)
+        return set_error(E3J_AMD_INVALID_ARGUMENT, name + ": edge positions are int32");
+    if (p->signature >= num_signatures())
+        return set_error(E3J_AMD_INVALID_ARGUMENT,
+                         name + ": unknown signature id " + std::to_string(p->signature));
+    if (p->signature >= 0) {
+        const Signature &sg = signature(p->signature);
+        if (p->val_dtype != E3J_AMD_F32 || sg.num_x != p->num_x || sg.num_y != p->num_y ||
+            sg.num_out != p->num_out || sg.num_scalars != p->num_scalars ||
+            sg.channels != p->channels || sg.layout != p->layout)
+            return set_error(E3J_AMD_INVALID_ARGUMENT,
+                             name + ": operand shapes do not match signature " + sg.name);
+    }
+    return E3J_AMD_OK;
+}
+
+bool missing(const void *ptr, int64_t count) { return count > 0 && ptr == nullptr; }
+
+int finish(const e3j_amd_conv_params *p, hipStream_t stream, int rc, const char *op) {
+    if (rc != E3J_AMD_OK || p->debug <= 0) return rc;
+    return check_hip(hipStreamSynchronize(stream), op);
+}
+
+}  // namespace
+
+int run_backward(const e3j_amd_conv_params *p, bool group_is_receiver, const void *coef,
+                 const void *x, const void *y, const void *s, const void *dm,
+                 const int32_t *other, const int32_t *row_ptr, const int32_t *edge_perm,
+                 void *dx, void *dy, void *ds, hipStream_t stream, bool coef_cols_ji) {
+    const char *op = group_is_receiver ? "convolution_bwd_receiver" : "convolution_bwd";
+    int rc = validate(p, op);
+    if (rc) return rc;
+    if (p->num_nodes == 0 && p->num_edges == 0) return E3J_AMD_OK;
+    if (missing(x, p->num_nodes) || missing(dm, p->num_nodes) || missing(dx, p->num_nodes) ||
+        row_ptr == nullptr || missing(other, p->num_edges) || missing(y, p->num_edges) ||
+        missing(s, p->num_edges) || missing(dy, p->num_edges) || missing(ds, p->num_edges) ||
+        (p->signature < 0 && missing(coef, p->num_coef)))
+        return set_error(E3J_AMD_INVALID_ARGUMENT, std::string(op) + ": null operand");
+    if (p->num_nodes == 0) return E3J_AMD_OK;
+    if (p->signature >= 0 && group_is_receiver && signature(p->signature).bwd != nullptr) {
+        rc = signature(p->signature).bwd(*p, static_cast<const float *>(x),
+                                         static_cast<const float *>(y), static_cast<const float *>(s),
+                                         static_cast<const float *>(dm), other, row_ptr, edge_perm,
+                                         static_cast<float *>(dx), static_cast<float *>(dy),
+                                         static_cast<float *>(ds), stream);
+    } else {
+        if (coef == nullptr && p->num_coef > 0)
+            return set_error(E3J_AMD_INVALID_ARGUMENT,
+                             std::string(op) + ": this grouping runs the table-driven kernel and needs `coef`");
+        rc = launch_generic_bwd(*p, group_is_receiver, coef, x, y, s, dm, other, row_ptr, edge_perm,
+                                dx, dy, ds, stream, coef_cols_ji);
+    }
+    return finish(p, stream, rc, op);
+}
+
+}  // namespace e3j_amd
+
+using namespace e3j_amd;
+
+extern "C" {
+
+const char *e3j_amd_last_error(void) { return g_last_error.c_str(); }
+
+const char *e3j_amd_version(void) { return "e3j_amd 0.1 (gfx950)"; }
+
+int e3j_amd_convolution_fwd(const e3j_amd_conv_params *p, const void *coef, const void *x,
+                            const void *y, const void *s, const int32_t *sender,
+                            const int32_t *receiver_ptr, const int32_t *edge_perm, void *out,
+                            void *stream_) {
+    int rc = validate(p, "convolution");
+    if (rc) return rc;
+    hipStream_t stream = static_cast<hipStream_t>(stream_);
+    if (p->num_nodes == 0) return E3J_AMD_OK;
+    if (missing(out, p->num_nodes) || missing(x, p->num_nodes) || receiver_ptr == nullptr ||
+        missing(sender, p->num_edges) || missing(y, p->num_edges) || missing(s, p->num_edges) ||
+        (p->signature < 0 && missing(coef, p->num_coef)))
+        return set_error(E3J_AMD_INVALID_ARGUMENT, "convolution: null operand");
+    if (p->signature >= 0) {
+        rc = signature(p->signature).fwd(*p, static_cast<const float *>(x), static_cast<const float *>(y),
+                                         static_cast<const float *>(s), sender, receiver_ptr,
+                                         edge_perm, static_cast<float *>(out), stream);
+    } else {
+        rc = launch_generic_fwd(*p, coef, x, y, s, sender, receiver_ptr, edge_perm, out, stream);
+    }
+    return finish(p, stream, rc, "convolution");
+}
+
+int e3j_amd_convolution_bwd_sender(const e3j_amd_conv_params *p, const void *coef, const void *x,
+                                   const void *y, const void *s, const void *dm,
+                                   const int32_t *receiver_t, const int32_t *sender_ptr,
+                                   const int32_t *edge_perm, void *dx, void *dy, void *ds,
+                                   void *stream) {
+    return run_backward(p, false, coef, x, y, s, dm, receiver_t, sender_ptr, edge_perm, dx, dy, ds,
+                        static_cast<hipStream_t>(stream), false);
+}
+
+int e3j_amd_convolution_bwd_receiver(const e3j_amd_conv_params *p, const void *coef, const void *x,
+                                     const void *y, const void *s, const void *dm,
+                                     const int32_t *sender, const int32_t *receiver_ptr,
+                                     const int32_t *edge_perm, void *dx, void *dy, void *ds,
+                                     void *stream) {
+    return run_backward(p, true, coef, x, y, s, dm, sender, receiver_ptr, edge_perm, dx, dy, ds,
+                        static_cast<hipStream_t>(stream), false);
+}
+
+int e3j_amd_num_signatures(void) { return num_signatures(); }
+
+const char *e3j_amd_signature_name(int id) {
+    if (id < 0 || id >= num_signatures()) return "";
+    return signature(id).name;
+}
+
+int e3j_amd_find_signature(const void *coef_host, int32_t coef_idx_bytes, int32_t val_dtype,
+                           int32_t num_coef, int32_t num_x, int32_t num_y, int32_t num_out,
+                           int32_t num_scalars, int32_t channels, int32_t layout,
+                           float *coef_scale) {
+    if (coef_scale) *coef_scale = 1.0f;
+    if (coef_host == nullptr || val_dtype != E3J_AMD_F32 || num_coef <= 0) return -1;
+    if (coef_idx_bytes != 1 && coef_idx_bytes != 4) return -1;
+    const size_t item = coef_idx_bytes == 1 ? sizeof(Coef4D<uint8_t, float>) : sizeof(Coef4D<int32_t, float>);
+    const unsigned char *bytes = static_cast<const unsigned char *>(coef_host);
+    for (int id = 0; id < num_signatures(); id++) {
+        const Signature &sg = signature(id);
+        if (sg.num_coef != num_coef || sg.num_x != num_x || sg.num_y != num_y ||
+            sg.num_out != num_out || sg.num_scalars != num_scalars || sg.channels != channels ||
+            sg.layout != layout)
+            continue;
+        // One uniform positive factor is allowed between the tables; it is taken from
+        // the entry of largest magnitude and every entry must agree to float32 rounding.
+        int big = 0;
+        for (int n = 1; n < num_coef; n++)
+            if (std::fabs(sg.val[n]) > std::fabs(sg.val[big])) big = n;
+        float vbig;
+        std::memcpy(&vbig, bytes + big * item, sizeof(float));
+        const double scale = (double)vbig / (double)sg.val[big];
+        bool same = scale > 0.0 && std::isfinite(scale);
+        for (int n = 0; n < num_coef && same; n++) {
+            float v;
+            int32_t idx[4];
+            std::memcpy(&v, bytes + n * item, sizeof(float));
+            for (int t = 0; t < 4; t++) {
+                if (coef_idx_bytes == 1) idx[t] = bytes[n * item + 4 + t];
+                else std::memcpy(&idx[t], bytes + n * item + 4 + 4 * t, 4);
+            }
+            const double want = scale * (double)sg.val[n];
+            same = std::fabs((double)v - want) <= 4e-7 * std::fabs(want);
+            for (int t = 0; t < 4 && same; t++) same = idx[t] == (int32_t)sg.idx[4 * n + t];
+        }
+        if (same) {
+            if (coef_scale) *coef_scale = (float)scale;
+            return id;
+        }
+    }
+    return -1;
+}
+
+}  // extern "C"

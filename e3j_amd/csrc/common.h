@@ -1,0 +1,89 @@
+// Shared declarations of the gfx950 convolution library (internal).
+#ifndef E3J_AMD_CSRC_COMMON_H_
+#define E3J_AMD_CSRC_COMMON_H_
+
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+
+#include <string>
+
+#include "../../include/e3j_amd.h"
+
+namespace e3j_amd {
+
+constexpr int kWave = 64;  // gfx950 wavefront width
+
+// Packed coefficient entry: the struct behind the opaque `coef` operand
+// (field order and padding of lib/e3j_ops/cuda/convolution.cuh:31-44).
+template <typename Idx, typename Val> struct CoefAlign;
+template <> struct CoefAlign<uint8_t, float>  { static constexpr int value = 8; };
+template <> struct CoefAlign<int32_t, float>  { static constexpr int value = 32; };
+template <> struct CoefAlign<uint8_t, double> { static constexpr int value = 16; };
+template <> struct CoefAlign<int32_t, double> { static constexpr int value = 32; };
+
+template <typename Idx, typename Val>
+struct alignas(CoefAlign<Idx, Val>::value) Coef4D {
+    Val val;
+    Idx i, j, k, l;
+};
+static_assert(sizeof(Coef4D<uint8_t, float>) == 8, "packed size");
+static_assert(sizeof(Coef4D<int32_t, float>) == 32, "packed size");
+static_assert(sizeof(Coef4D<uint8_t, double>) == 16, "packed size");
+static_assert(sizeof(Coef4D<int32_t, double>) == 32, "packed size");
+
+// Element strides of a (rows, dim, channels) operand in either layout.
+struct RowLayout {
+    int64_t row;   // elements between consecutive rows
+    int32_t dim;   // stride of the irreps coordinate
+    int32_t chan;  // stride of the channel
+};
+
+inline RowLayout make_layout(int layout, int dim, int channels) {
+    RowLayout r;
+    r.row = (int64_t)dim * channels;
+    if (layout == E3J_AMD_LAYOUT_TRAILING) { r.dim = channels; r.chan = 1; }
+    else                                   { r.dim = 1;        r.chan = dim; }
+    return r;
+}
+
+// Error reporting ------------------------------------------------------
+int set_error(int code, const std::string &msg);
+int check_hip(hipError_t err, const char *what);
+
+// Entry point shared by the C ABI and the XLA-FFI handlers.
+int run_backward(const e3j_amd_conv_params *p, bool group_is_receiver, const void *coef,
+                 const void *x, const void *y, const void *s, const void *dm,
+                 const int32_t *other, const int32_t *row_ptr, const int32_t *edge_perm,
+                 void *dx, void *dy, void *ds, hipStream_t stream, bool coef_cols_ji);
+
+// Table-driven kernels (conv_generic.hip) ---------------------------------
+int launch_generic_fwd(const e3j_amd_conv_params &p, const void *coef, const void *x, const void *y,
+                       const void *s, const int32_t *other, const int32_t *row_ptr,
+                       const int32_t *edge_perm, void *out, hipStream_t stream);
+int launch_generic_bwd(const e3j_amd_conv_params &p, bool group_is_receiver, const void *coef,
+                       const void *x, const void *y, const void *s, const void *dm,
+                       const int32_t *other, const int32_t *row_ptr, const int32_t *edge_perm,
+                       void *dx, void *dy, void *ds, hipStream_t stream,
+                       bool coef_cols_ji = false);
+int launch_fill_zero(void *ptr, size_t bytes, hipStream_t stream);
+
+// Compile-time-unrolled kernels (generated, sig_*.hip) ----------------------
+struct Signature {
+    const char *name;
+    int32_t num_x, num_y, num_out, num_scalars, num_coef;
+    int32_t channels;  // channel count the kernels were built for
+    int32_t layout;
+    const float *val;      // (num_coef) forward table, as float32
+    const uint8_t *idx;    // (num_coef, 4) i, j, k, l
+    int (*fwd)(const e3j_amd_conv_params &p, const float *x, const float *y, const float *s,
+               const int32_t *sender, const int32_t *receiver_ptr, const int32_t *edge_perm,
+               float *out, hipStream_t stream);
+    int (*bwd)(const e3j_amd_conv_params &p, const float *x, const float *y, const float *s,
+               const float *dm, const int32_t *sender, const int32_t *receiver_ptr,
+               const int32_t *edge_perm, float *dx, float *dy, float *ds, hipStream_t stream);
+};
+int num_signatures();
+const Signature &signature(int id);
+
+}  // namespace e3j_amd
+#endif

@@ -1,0 +1,340 @@
+// Table-driven convolution kernels for gfx950: any coefficient table, any
+// channel count, both layouts, float32/float64.  They are the fallback behind
+// the compile-time-unrolled kernels and the carrier of every edge-case rule.
+//
+// Mapping: one 64-lane wavefront owns one CSR row (a node); a lane owns one
+// channel of a 64-channel chunk.  Each lane keeps its operands and
+// accumulators in a private column of LDS (dynamic indexing by the table's
+// coordinates), so no barrier or cross-lane traffic is needed except the
+// channel reduction of dy.  Coefficients, y and the adjacency are
+// wave-uniform and travel through scalar loads.
+//
+// Semantics restated from lib/e3j_ops/cuda/convolution/fwd.cuh:289-403 and
+// bwd.cuh:116-321: zero rows for nodes without live edges, padding edges
+// skipped by a bounds check on the gathered endpoint, dy/ds of padding edges
+// written as zeros, dx rows zero-filled before accumulation.
+
+#include "common.h"
+
+namespace e3j_amd {
+namespace {
+
+template <typename Val>
+__device__ inline Val wave_sum(Val v) {
+#pragma unroll
+    for (int off = kWave / 2; off > 0; off >>= 1) v += __shfl_xor(v, off, kWave);
+    return v;
+}
+
+template <typename Idx, typename Val>
+__global__ void generic_fwd_kernel(const Coef4D<Idx, Val> *__restrict__ coef, int num_coef,
+                                   const Val *__restrict__ x, RowLayout lx,
+                                   const Val *__restrict__ y, int num_y,
+                                   const Val *__restrict__ s, RowLayout ls,
+                                   const int32_t *__restrict__ other,
+                                   const int32_t *__restrict__ row_ptr,
+                                   const int32_t *__restrict__ perm,
+                                   Val *__restrict__ out, RowLayout lo,
+                                   int num_nodes, int channels, int X, int S, int Z, int nchunks) {
+    extern __shared__ __align__(16) unsigned char smem_raw[];
+    const int lane = threadIdx.x;
+    const int wave = threadIdx.y;
+    const int64_t item = (int64_t)blockIdx.x * blockDim.y + wave;
+    if (item >= (int64_t)num_nodes * nchunks) return;  // uniform per wave; no barriers below
+    const int r = (int)(item / nchunks);
+    const int c = (int)(item % nchunks) * kWave + lane;
+    const bool active = c < channels;
+
+    Val *acc = reinterpret_cast<Val *>(smem_raw) + (size_t)wave * (Z + X + S) * kWave + lane;
+    Val *xs = acc + (size_t)Z * kWave;
+    Val *ss = xs + (size_t)X * kWave;
+    for (int i = 0; i < Z; i++) acc[i * kWave] = Val(0);
+
+    const int e0 = row_ptr[r], e1 = row_ptr[r + 1];
+    for (int e = e0; e < e1; e++) {
+        const int snd = other[e];
+        if ((unsigned)snd >= (unsigned)num_nodes) continue;  // padding edge
+        const int64_t ee = perm ? (int64_t)perm[e] : (int64_t)e;
+        const Val *xrow = x + (int64_t)snd * lx.row + (int64_t)c * lx.chan;
+        const Val *srow = s + ee * ls.row + (int64_t)c * ls.chan;
+        for (int j = 0; j < X; j++) xs[j * kWave] = active ? xrow[(int64_t)j * lx.dim] : Val(0);
+        for (int l = 0; l < S; l++) ss[l * kWave] = active ? srow[(int64_t)l * ls.dim] : Val(0);
+        const Val *ye = y + ee * num_y;
+
+        int cur_i = -1, cur_l = 0;
+        Val msg = Val(0);
+        for (int n = 0; n < num_coef; n++) {
+            const Coef4D<Idx, Val> cf = coef[n];
+            const int ci = (int)cf.i, cl = (int)cf.l;
+            if (ci != cur_i || cl != cur_l) {
+                if (cur_i >= 0) acc[cur_i * kWave] += ss[cur_l * kWave] * msg;
+                cur_i = ci; cur_l = cl; msg = Val(0);
+            }
+            msg += (xs[(int)cf.j * kWave] * ye[(int)cf.k]) * cf.val;
+        }
+        if (cur_i >= 0) acc[cur_i * kWave] += ss[cur_l * kWave] * msg;
+    }
+    if (active) {
+        Val *orow = out + (int64_t)r * lo.row + (int64_t)c * lo.chan;
+        for (int i = 0; i < Z; i++) orow[(int64_t)i * lo.dim] = acc[i * kWave];
+    }
+}
+
+// kGroupIsReceiver: rows are receivers (dm row fixed, x gathered, dx scattered with
+// atomics into a zero-filled buffer).  Otherwise rows are senders (x row fixed, dm
+// gathered, dx accumulated in place by the owning wave).
+template <typename Idx, typename Val, bool kGroupIsReceiver>
+__global__ void generic_bwd_kernel(const Coef4D<Idx, Val> *__restrict__ coef, int num_coef,
+                                   const Val *__restrict__ x, RowLayout lx,
+                                   const Val *__restrict__ y, int num_y,
+                                   const Val *__restrict__ s, RowLayout ls,
+                                   const Val *__restrict__ dm, RowLayout lo,
+                                   const int32_t *__restrict__ other,
+                                   const int32_t *__restrict__ row_ptr,
+                                   const int32_t *__restrict__ perm,
+                                   Val *__restrict__ dx, Val *__restrict__ dy, Val *__restrict__ ds,
+                                   int num_nodes, int channels, int X, int S, int Z, int nchunks,
+                                   int cols_ji) {
+    extern __shared__ __align__(16) unsigned char smem_raw[];
+    const int lane = threadIdx.x;
+    const int wave = threadIdx.y;
+    const int64_t item = (int64_t)blockIdx.x * blockDim.y + wave;
+    if (item >= (int64_t)num_nodes) return;
+    const int g = (int)item;
+
+    const int per_wave = Z + 2 * X + 2 * S + num_y;
+    Val *zc = reinterpret_cast<Val *>(smem_raw) + (size_t)wave * per_wave * kWave + lane;
+    Val *xc = zc + (size_t)Z * kWave;
+    Val *sc = xc + (size_t)X * kWave;
+    Val *dsc = sc + (size_t)S * kWave;
+    Val *dxc = dsc + (size_t)S * kWave;
+    Val *dyc = dxc + (size_t)X * kWave;
+
+    if (!kGroupIsReceiver) {
+        for (int q = 0; q < nchunks; q++) {
+            const int c = q * kWave + lane;
+            if (c < channels) {
+                Val *row = dx + (int64_t)g * lx.row + (int64_t)c * lx.chan;
+                for (int j = 0; j < X; j++) row[(int64_t)j * lx.dim] = Val(0);
+            }
+        }
+    }
+
+    const int e0 = row_ptr[g], e1 = row_ptr[g + 1];
+    for (int e = e0; e < e1; e++) {
+        const int o = other[e];
+        if ((unsigned)o >= (unsigned)num_nodes) continue;  // padding edge: zero-filled separately
+        const int64_t ee = perm ? (int64_t)perm[e] : (int64_t)e;
+        const int xnode = kGroupIsReceiver ? o : g;
+        const int znode = kGroupIsReceiver ? g : o;
+        const Val *ye = y + ee * num_y;
+        for (int k = 0; k < num_y; k++) dyc[k * kWave] = Val(0);
+
+        for (int q = 0; q < nchunks; q++) {
+            const int c = q * kWave + lane;
+            const bool active = c < channels;
+            const Val *xrow = x + (int64_t)xnode * lx.row + (int64_t)c * lx.chan;
+            const Val *zrow = dm + (int64_t)znode * lo.row + (int64_t)c * lo.chan;
+            const Val *srow = s + ee * ls.row + (int64_t)c * ls.chan;
+            for (int i = 0; i < Z; i++) zc[i * kWave] = active ? zrow[(int64_t)i * lo.dim] : Val(0);
+            for (int j = 0; j < X; j++) {
+                xc[j * kWave] = active ? xrow[(int64_t)j * lx.dim] : Val(0);
+                dxc[j * kWave] = Val(0);
+            }
+            for (int l = 0; l < S; l++) {
+                sc[l * kWave] = active ? srow[(int64_t)l * ls.dim] : Val(0);
+                dsc[l * kWave] = Val(0);
+            }
+            for (int n = 0; n < num_coef; n++) {
+                const Coef4D<Idx, Val> cf = coef[n];
+                // cols_ji: the table's first two columns hold (x, output) coordinates, as in the
+                // dx-transposed copy the reference passes (src/e3j/ops/convolution.py:367).
+                const int ci = cols_ji ? (int)cf.j : (int)cf.i, cj = cols_ji ? (int)cf.i : (int)cf.j;
+                const int ck = (int)cf.k, cl = (int)cf.l;
+                const Val dz = zc[ci * kWave];
+                const Val xv = xc[cj * kWave];
+                const Val gz = dz * sc[cl * kWave];
+                const Val t = cf.val * ye[ck];
+                dxc[cj * kWave] += t * gz;
+                dsc[cl * kWave] += (t * dz) * xv;
+                dyc[ck * kWave] += (cf.val * gz) * xv;
+            }
+            if (active) {
+                Val *dsrow = ds + ee * ls.row + (int64_t)c * ls.chan;
+                for (int l = 0; l < S; l++) dsrow[(int64_t)l * ls.dim] = dsc[l * kWave];
+                Val *dxrow = dx + (int64_t)xnode * lx.row + (int64_t)c * lx.chan;
+                for (int j = 0; j < X; j++) {
+                    if (kGroupIsReceiver) unsafeAtomicAdd(dxrow + (int64_t)j * lx.dim, dxc[j * kWave]);
+                    else dxrow[(int64_t)j * lx.dim] += dxc[j * kWave];
+                }
+            }
+        }
+        for (int k = 0; k < num_y; k++) {
+            const Val total = wave_sum(dyc[k * kWave]);
+            if (lane == 0) dy[ee * num_y + k] = total;
+        }
+    }
+}
+
+// dy/ds rows of padding edges: positions past the last row, or whose gathered
+// endpoint is out of range (lib/e3j_ops/cuda/convolution/bwd.cuh:308-319).
+template <typename Val>
+__global__ void zero_padding_edges_kernel(const int32_t *__restrict__ other,
+                                          const int32_t *__restrict__ row_ptr,
+                                          const int32_t *__restrict__ perm, int num_nodes,
+                                          int64_t num_edges, Val *__restrict__ dy, int num_y,
+                                          Val *__restrict__ ds, int64_t ds_row) {
+    const int lane = threadIdx.x;
+    const int64_t live_end = row_ptr[num_nodes];
+    for (int64_t e = (int64_t)blockIdx.x * blockDim.y + threadIdx.y; e < num_edges;
+         e += (int64_t)gridDim.x * blockDim.y) {
+        const int o = other[e];
+        if (e < live_end && (unsigned)o < (unsigned)num_nodes) continue;
+        const int64_t ee = perm ? (int64_t)perm[e] : e;
+        for (int k = lane; k < num_y; k += kWave) dy[ee * num_y + k] = Val(0);
+        for (int64_t t = lane; t < ds_row; t += kWave) ds[ee * ds_row + t] = Val(0);
+    }
+}
+
+__global__ void fill_zero_kernel(uint32_t *__restrict__ p, size_t n_words) {
+    const size_t stride = (size_t)gridDim.x * blockDim.x;
+    for (size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x; i < n_words; i += stride) p[i] = 0u;
+}
+
+constexpr size_t kMaxLds = 160 * 1024;  // LDS per CU / per workgroup on gfx950
+
+// waves per block such that the block's LDS stays within `budget`
+int pick_waves(size_t per_wave_bytes, size_t budget) {
+    int w = (int)(budget / per_wave_bytes);
+    return w < 1 ? 1 : (w > 4 ? 4 : w);
+}
+
+template <typename Idx, typename Val>
+int run_fwd(const e3j_amd_conv_params &p, const void *coef, const void *x, const void *y,
+            const void *s, const int32_t *other, const int32_t *row_ptr, const int32_t *perm,
+            void *out, hipStream_t stream) {
+    const int nchunks = (p.channels + kWave - 1) / kWave;
+    const size_t per_wave = (size_t)(p.num_out + p.num_x + p.num_scalars) * kWave * sizeof(Val);
+    if (per_wave > kMaxLds)
+        return set_error(E3J_AMD_UNIMPLEMENTED, "convolution: num_out + num_x + num_scalars = " +
+                         std::to_string(p.num_out + p.num_x + p.num_scalars) +
+                         " exceeds the LDS capacity of the table-driven kernel");
+    const int waves = pick_waves(per_wave, 64 * 1024);
+    const size_t lds = per_wave * waves;
+    auto kernel = generic_fwd_kernel<Idx, Val>;
+    if (lds > 64 * 1024) {
+        int rc = check_hip(hipFuncSetAttribute(reinterpret_cast<const void *>(kernel),
+                                               hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds),
+                           "hipFuncSetAttribute(fwd)");
+        if (rc) return rc;
+    }
+    const int64_t items = (int64_t)p.num_nodes * nchunks;
+    const int64_t blocks = (items + waves - 1) / waves;
+    if (blocks > 0x7fffffffLL) return set_error(E3J_AMD_INVALID_ARGUMENT, "convolution: grid too large");
+    hipLaunchKernelGGL(kernel, dim3((unsigned)blocks), dim3(kWave, waves), lds, stream,
+                       static_cast<const Coef4D<Idx, Val> *>(coef), p.num_coef,
+                       static_cast<const Val *>(x), make_layout(p.layout, p.num_x, p.channels),
+                       static_cast<const Val *>(y), p.num_y,
+                       static_cast<const Val *>(s), make_layout(p.layout, p.num_scalars, p.channels),
+                       other, row_ptr, perm,
+                       static_cast<Val *>(out), make_layout(p.layout, p.num_out, p.channels),
+                       p.num_nodes, p.channels, p.num_x, p.num_scalars, p.num_out, nchunks);
+    return check_hip(hipGetLastError(), "convolution forward launch");
+}
+
+template <typename Idx, typename Val>
+int run_bwd(const e3j_amd_conv_params &p, bool group_is_receiver, const void *coef, const void *x,
+            const void *y, const void *s, const void *dm, const int32_t *other,
+            const int32_t *row_ptr, const int32_t *perm, void *dx, void *dy, void *ds,
+            hipStream_t stream, bool cols_ji) {
+    const int nchunks = (p.channels + kWave - 1) / kWave;
+    const size_t per_wave =
+        (size_t)(p.num_out + 2 * p.num_x + 2 * p.num_scalars + p.num_y) * kWave * sizeof(Val);
+    if (per_wave > kMaxLds)
+        return set_error(E3J_AMD_UNIMPLEMENTED,
+                         "convolution_bwd: irreps dimensions exceed the LDS capacity of the "
+                         "table-driven kernel");
+    const int waves = pick_waves(per_wave, 64 * 1024);
+    const size_t lds = per_wave * waves;
+    const int64_t blocks = ((int64_t)p.num_nodes + waves - 1) / waves;
+    const RowLayout lx = make_layout(p.layout, p.num_x, p.channels);
+    const RowLayout ls = make_layout(p.layout, p.num_scalars, p.channels);
+    const RowLayout lo = make_layout(p.layout, p.num_out, p.channels);
+    int rc = 0;
+    if (group_is_receiver) {
+        rc = launch_fill_zero(dx, (size_t)p.num_nodes * p.num_x * p.channels * sizeof(Val), stream);
+        if (rc) return rc;
+    }
+    if (p.num_edges > 0) {
+        const int64_t zblocks = std::min<int64_t>((p.num_edges + 3) / 4, 4096);
+        hipLaunchKernelGGL(zero_padding_edges_kernel<Val>, dim3((unsigned)zblocks), dim3(kWave, 4), 0,
+                           stream, other, row_ptr, perm, p.num_nodes, p.num_edges,
+                           static_cast<Val *>(dy), p.num_y, static_cast<Val *>(ds),
+                           (int64_t)p.num_scalars * p.channels);
+        rc = check_hip(hipGetLastError(), "convolution backward padding launch");
+        if (rc) return rc;
+    }
+#define E3J_LAUNCH_BWD(FLAG)                                                                      \
+    do {                                                                                          \
+        auto kernel = generic_bwd_kernel<Idx, Val, FLAG>;                                         \
+        if (lds > 64 * 1024) {                                                                    \
+            rc = check_hip(hipFuncSetAttribute(reinterpret_cast<const void *>(kernel),            \
+                                               hipFuncAttributeMaxDynamicSharedMemorySize,        \
+                                               (int)lds),                                         \
+                           "hipFuncSetAttribute(bwd)");                                           \
+            if (rc) return rc;                                                                    \
+        }                                                                                         \
+        hipLaunchKernelGGL(kernel, dim3((unsigned)blocks), dim3(kWave, waves), lds, stream,       \
+                           static_cast<const Coef4D<Idx, Val> *>(coef), p.num_coef,               \
+                           static_cast<const Val *>(x), lx, static_cast<const Val *>(y), p.num_y, \
+                           static_cast<const Val *>(s), ls, static_cast<const Val *>(dm), lo,     \
+                           other, row_ptr, perm, static_cast<Val *>(dx), static_cast<Val *>(dy),  \
+                           static_cast<Val *>(ds), p.num_nodes, p.channels, p.num_x,              \
+                           p.num_scalars, p.num_out, nchunks, cols_ji ? 1 : 0);                   \
+    } while (0)
+    if (group_is_receiver) E3J_LAUNCH_BWD(true);
+    else E3J_LAUNCH_BWD(false);
+#undef E3J_LAUNCH_BWD
+    return check_hip(hipGetLastError(), "convolution backward launch");
+}
+
+}  // namespace
+
+int launch_fill_zero(void *ptr, size_t bytes, hipStream_t stream) {
+    if (bytes == 0) return E3J_AMD_OK;
+    if (bytes % 4 != 0 || (reinterpret_cast<uintptr_t>(ptr) % 4) != 0)
+        return set_error(E3J_AMD_INVALID_ARGUMENT, "fill: buffer must be 4-byte aligned");
+    const size_t words = bytes / 4;
+    const size_t blocks = std::min<size_t>((words + 255) / 256, 8192);
+    hipLaunchKernelGGL(fill_zero_kernel, dim3((unsigned)blocks), dim3(256), 0, stream,
+                       static_cast<uint32_t *>(ptr), words);
+    return check_hip(hipGetLastError(), "fill launch");
+}
+
+#define E3J_DISPATCH(CALL)                                                                  \
+    if (p.val_dtype == E3J_AMD_F32 && p.coef_idx_bytes == 1) return CALL(uint8_t, float);   \
+    if (p.val_dtype == E3J_AMD_F32 && p.coef_idx_bytes == 4) return CALL(int32_t, float);   \
+    if (p.val_dtype == E3J_AMD_F64 && p.coef_idx_bytes == 1) return CALL(uint8_t, double);  \
+    if (p.val_dtype == E3J_AMD_F64 && p.coef_idx_bytes == 4) return CALL(int32_t, double);  \
+    return set_error(E3J_AMD_INVALID_ARGUMENT, "unsupported (IDX, VAL) dtype pair")
+
+int launch_generic_fwd(const e3j_amd_conv_params &p, const void *coef, const void *x, const void *y,
+                       const void *s, const int32_t *other, const int32_t *row_ptr,
+                       const int32_t *edge_perm, void *out, hipStream_t stream) {
+#define E3J_FWD(I, V) run_fwd<I, V>(p, coef, x, y, s, other, row_ptr, edge_perm, out, stream)
+    E3J_DISPATCH(E3J_FWD);
+#undef E3J_FWD
+}
+
+int launch_generic_bwd(const e3j_amd_conv_params &p, bool group_is_receiver, const void *coef,
+                       const void *x, const void *y, const void *s, const void *dm,
+                       const int32_t *other, const int32_t *row_ptr, const int32_t *edge_perm,
+                       void *dx, void *dy, void *ds, hipStream_t stream, bool coef_cols_ji) {
+#define E3J_BWD(I, V)                                                                            \
+    run_bwd<I, V>(p, group_is_receiver, coef, x, y, s, dm, other, row_ptr, edge_perm, dx, dy, ds, \
+                  stream, coef_cols_ji)
+    E3J_DISPATCH(E3J_BWD);
+#undef E3J_BWD
+}
+
+}  // namespace e3j_amd

@@ -1,0 +1,128 @@
+// Graph preparation on the device: CSR row pointers and the stable edge sort
+// behind the unsorted (GraphOrdering NONE) path and the transposed adjacency.
+//
+// Restates GraphCSR (src/e3j/data/graph.py:49-73): row_ptr = [0] +
+// cumsum(bincount(key, length = N)) with out-of-range keys dropped, and
+// sort = stable argsort by key.  The sort is rocPRIM's radix sort (via hipCUB)
+// on unsigned keys, so sentinel and negative keys land after every live row.
+
+#include <hipcub/hipcub.hpp>
+
+#include "common.h"
+
+namespace e3j_amd {
+namespace {
+
+__global__ void count_keys_kernel(const int32_t *__restrict__ key, int64_t num_edges, int num_nodes,
+                                  int32_t *__restrict__ counts) {
+    const int64_t stride = (int64_t)gridDim.x * blockDim.x;
+    for (int64_t e = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; e < num_edges; e += stride) {
+        const int k = key[e];
+        if ((unsigned)k < (unsigned)num_nodes) atomicAdd(&counts[k + 1], 1);
+    }
+}
+
+__global__ void iota_kernel(int32_t *__restrict__ out, int64_t n) {
+    const int64_t stride = (int64_t)gridDim.x * blockDim.x;
+    for (int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; i < n; i += stride)
+        out[i] = (int32_t)i;
+}
+
+__global__ void gather_kernel(const int32_t *__restrict__ src, const int32_t *__restrict__ perm,
+                              int32_t *__restrict__ dst, int64_t n) {
+    const int64_t stride = (int64_t)gridDim.x * blockDim.x;
+    for (int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; i < n; i += stride)
+        dst[i] = src[perm[i]];
+}
+
+size_t align_up(size_t v, size_t a = 256) { return (v + a - 1) / a * a; }
+
+unsigned grid_for(int64_t n) { return (unsigned)std::max<int64_t>(1, std::min<int64_t>((n + 255) / 256, 4096)); }
+
+size_t scan_temp_bytes(int32_t num_nodes) {
+    size_t bytes = 0;
+    hipcub::DeviceScan::InclusiveSum(nullptr, bytes, (int32_t *)nullptr, (int32_t *)nullptr,
+                                     num_nodes + 1);
+    return bytes;
+}
+
+size_t sort_temp_bytes(int64_t num_edges) {
+    size_t bytes = 0;
+    hipcub::DeviceRadixSort::SortPairs(nullptr, bytes, (const uint32_t *)nullptr, (uint32_t *)nullptr,
+                                       (const int32_t *)nullptr, (int32_t *)nullptr, (int)num_edges);
+    return bytes;
+}
+
+int row_ptr_impl(const int32_t *key, int64_t num_edges, int32_t num_nodes, int32_t *row_ptr,
+                 void *temp, size_t temp_bytes, hipStream_t stream) {
+    int rc = launch_fill_zero(row_ptr, sizeof(int32_t) * ((size_t)num_nodes + 1), stream);
+    if (rc) return rc;
+    if (num_edges > 0) {
+        hipLaunchKernelGGL(count_keys_kernel, dim3(grid_for(num_edges)), dim3(256), 0, stream, key,
+                           num_edges, num_nodes, row_ptr);
+        rc = check_hip(hipGetLastError(), "csr count launch");
+        if (rc) return rc;
+    }
+    return check_hip(hipcub::DeviceScan::InclusiveSum(temp, temp_bytes, row_ptr, row_ptr,
+                                                      num_nodes + 1, stream),
+                     "csr scan");
+}
+
+}  // namespace
+}  // namespace e3j_amd
+
+using namespace e3j_amd;
+
+extern "C" {
+
+size_t e3j_amd_csr_workspace_bytes(int32_t num_nodes, int64_t num_edges) {
+    if (num_nodes < 0 || num_edges < 0) return 0;
+    // [scan temp | sort temp | keys_out (E) | iota (E)]
+    return align_up(scan_temp_bytes(num_nodes)) + align_up(sort_temp_bytes(num_edges)) +
+           2 * align_up(sizeof(int32_t) * (size_t)num_edges) + 256;
+}
+
+int e3j_amd_csr_row_ptr(const int32_t *key, int64_t num_edges, int32_t num_nodes, int32_t *row_ptr,
+                        void *workspace, void *stream_) {
+    if (num_nodes < 0 || num_edges < 0 || num_edges > 0x7fffffffLL)
+        return set_error(E3J_AMD_INVALID_ARGUMENT, "csr_row_ptr: bad sizes");
+    if (row_ptr == nullptr || workspace == nullptr || (num_edges > 0 && key == nullptr))
+        return set_error(E3J_AMD_INVALID_ARGUMENT, "csr_row_ptr: null operand");
+    return row_ptr_impl(key, num_edges, num_nodes, row_ptr, workspace, scan_temp_bytes(num_nodes),
+                        static_cast<hipStream_t>(stream_));
+}
+
+int e3j_amd_sort_edges(const int32_t *key, const int32_t *other, int64_t num_edges,
+                       int32_t num_nodes, int32_t *perm, int32_t *other_sorted, int32_t *row_ptr,
+                       void *workspace, void *stream_) {
+    if (num_nodes < 0 || num_edges < 0 || num_edges > 0x7fffffffLL)
+        return set_error(E3J_AMD_INVALID_ARGUMENT, "sort_edges: bad sizes");
+    if (row_ptr == nullptr || workspace == nullptr ||
+        (num_edges > 0 && (key == nullptr || other == nullptr || perm == nullptr || other_sorted == nullptr)))
+        return set_error(E3J_AMD_INVALID_ARGUMENT, "sort_edges: null operand");
+    hipStream_t stream = static_cast<hipStream_t>(stream_);
+    unsigned char *ws = static_cast<unsigned char *>(workspace);
+    const size_t scan_bytes = scan_temp_bytes(num_nodes);
+    const size_t sort_bytes = sort_temp_bytes(num_edges);
+    void *scan_temp = ws;
+    void *sort_temp = ws + align_up(scan_bytes);
+    uint32_t *keys_out = reinterpret_cast<uint32_t *>(ws + align_up(scan_bytes) + align_up(sort_bytes));
+    int32_t *iota = reinterpret_cast<int32_t *>(reinterpret_cast<unsigned char *>(keys_out) +
+                                                align_up(sizeof(int32_t) * (size_t)num_edges));
+    int rc = row_ptr_impl(key, num_edges, num_nodes, row_ptr, scan_temp, scan_bytes, stream);
+    if (rc || num_edges == 0) return rc;
+    hipLaunchKernelGGL(iota_kernel, dim3(grid_for(num_edges)), dim3(256), 0, stream, iota, num_edges);
+    rc = check_hip(hipGetLastError(), "sort iota launch");
+    if (rc) return rc;
+    size_t temp_bytes = sort_bytes;
+    rc = check_hip(hipcub::DeviceRadixSort::SortPairs(sort_temp, temp_bytes,
+                                                      reinterpret_cast<const uint32_t *>(key), keys_out,
+                                                      iota, perm, (int)num_edges, 0, 32, stream),
+                   "edge sort");
+    if (rc) return rc;
+    hipLaunchKernelGGL(gather_kernel, dim3(grid_for(num_edges)), dim3(256), 0, stream, other, perm,
+                       other_sorted, num_edges);
+    return check_hip(hipGetLastError(), "sort gather launch");
+}
+
+}  // extern "C"

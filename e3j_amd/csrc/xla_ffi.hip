@@ -1,0 +1,222 @@
+// XLA-FFI handlers: decode an XLA_FFI_CallFrame and call the launchers.
+//
+// Operand order of the reference's targets (lib/e3j_ops/ffi/e3j_ops.h:457-472,575-594):
+//   "convolution":      coef, x, y, s, sender, receiver_ptr [, coef_ranges]   -> out
+//   "convolution_bwd":  coef, x, y, s, dm, sender_t, receiver_ptr_t, edge_perm [, coef_ranges]
+//                                                                   -> dx, dy, ds
+// `coef_ranges` is accepted and ignored.  `coef` of "convolution_bwd" may be the
+// forward table (rank 2) or the reference's stack of three transposed tables
+// (3, nnz, numel) / (3*nnz, numel) flagged by the attribute coef_stacked = 1;
+// the first of the three, sorted for dx with columns (j, i, k, l), is then used.
+// A third target, "convolution_bwd_receiver", takes the forward's receiver CSR:
+//   coef, x, y, s, dm, sender, receiver_ptr, edge_perm -> dx, dy, ds.
+// Attributes: num_nodes, debug (reference); layout, signature, coef_scale,
+// coef_stacked (optional).  Handlers are re-entrant, allocate nothing and
+// enqueue on the stream XLA hands over; they answer the metadata query.
+
+#include <cstring>
+
+#include "common.h"
+#include "xla_ffi_abi.h"
+
+namespace e3j_amd {
+namespace {
+
+void *make_error(const XlaCallFrame *frame, int code, const std::string &msg) {
+    XlaErrorCreateArgs args;
+    args.struct_size = sizeof(XlaErrorCreateArgs);
+    args.extension_start = nullptr;
+    args.message = msg.c_str();
+    args.errc = code == E3J_AMD_INVALID_ARGUMENT ? kXlaErrInvalidArgument
+              : code == E3J_AMD_UNIMPLEMENTED    ? kXlaErrUnimplemented
+                                                 : kXlaErrInternal;
+    return frame->api->error_create(&args);
+}
+
+void *status_to_error(const XlaCallFrame *frame, int rc) {
+    return rc == E3J_AMD_OK ? nullptr : make_error(frame, rc, e3j_amd_last_error());
+}
+
+// Returns true when the frame is a metadata query (and answers it).
+bool answer_metadata(XlaCallFrame *frame) {
+    XlaExtensionBase *ext = frame->extension_start;
+    if (ext == nullptr || ext->type != kXlaExtMetadata) return false;
+    XlaMetadata *md = reinterpret_cast<XlaMetadataExtension *>(ext)->metadata;
+    md->api_version.major_version = kXlaFfiApiMajor;
+    md->api_version.minor_version = kXlaFfiApiMinor;
+    md->traits = 0;
+    if (md->struct_size >= offsetof(XlaMetadata, state_type_id) + sizeof(int64_t))
+        md->state_type_id = 0;  // stateless handler
+    return true;
+}
+
+const XlaBuffer *arg(const XlaCallFrame *f, int64_t i) {
+    if (i >= f->args.size || f->args.types[i] != kXlaArgBuffer) return nullptr;
+    return static_cast<const XlaBuffer *>(f->args.args[i]);
+}
+const XlaBuffer *ret(const XlaCallFrame *f, int64_t i) {
+    if (i >= f->rets.size || f->rets.types[i] != kXlaRetBuffer) return nullptr;
+    return static_cast<const XlaBuffer *>(f->rets.rets[i]);
+}
+int64_t count(const XlaBuffer *b) {
+    int64_t n = 1;
+    for (int64_t d = 0; d < b->rank; d++) n *= b->dims[d];
+    return n;
+}
+
+// Scalar attribute by name; `found` reports presence.
+template <typename T>
+T attr(const XlaCallFrame *f, const char *name, int32_t dtype, T fallback, bool *found = nullptr) {
+    if (found) *found = false;
+    const size_t len = std::strlen(name);
+    for (int64_t i = 0; i < f->attrs.size; i++) {
+        const XlaByteSpan *nm = f->attrs.names[i];
+        if (nm->len != len || std::memcmp(nm->ptr, name, len) != 0) continue;
+        if (f->attrs.types[i] != kXlaAttrScalar) return fallback;
+        const XlaScalar *sc = static_cast<const XlaScalar *>(f->attrs.attrs[i]);
+        if (sc->dtype != dtype) return fallback;
+        if (found) *found = true;
+        T v;
+        std::memcpy(&v, sc->value, sizeof(T));
+        return v;
+    }
+    return fallback;
+}
+
+struct Decoded {
+    e3j_amd_conv_params p;
+    hipStream_t stream;
+};
+
+// Fills sizes from the buffers, following the reference's handler
+// (lib/e3j_ops/ffi/e3j_ops.h:393-414,496-519).  Returns an XLA error or nullptr.
+void *decode_common(XlaCallFrame *f, const char *op, const XlaBuffer *coef, const XlaBuffer *x,
+                    const XlaBuffer *y, const XlaBuffer *s, const XlaBuffer *node_rows, Decoded *d) {
+    const std::string name(op);
+    if (!coef || !x || !y || !s || !node_rows)
+        return make_error(f, E3J_AMD_INVALID_ARGUMENT, name + ": missing or non-buffer operand");
+    if (x->rank < 2 || x->rank > 3 || y->rank < 2 || s->rank < 2 || node_rows->rank < 2)
+        return make_error(f, E3J_AMD_INVALID_ARGUMENT, name + ": operand rank");
+    e3j_amd_conv_params &p = d->p;
+    std::memset(&p, 0, sizeof(p));
+    bool has_nodes = false;
+    p.num_nodes = attr<int32_t>(f, "num_nodes", kXlaS32, 0, &has_nodes);
+    if (!has_nodes) return make_error(f, E3J_AMD_INVALID_ARGUMENT, name + ": attribute num_nodes (i32) is required");
+    p.debug = attr<int32_t>(f, "debug", kXlaS32, 0);
+    p.layout = attr<int32_t>(f, "layout", kXlaS32, E3J_AMD_LAYOUT_TRAILING);
+    p.signature = attr<int32_t>(f, "signature", kXlaS32, -1);
+    p.coef_scale = attr<float>(f, "coef_scale", kXlaF32, 1.0f);
+    p.num_edges = y->dims[0];
+    p.num_y = (int32_t)y->dims[1];
+    if (y->rank == 3 && y->dims[2] != 1)
+        return make_error(f, E3J_AMD_UNIMPLEMENTED, name + ": RHS y should have only one channel.");
+    const bool leading = p.layout == E3J_AMD_LAYOUT_LEADING;
+    if (x->rank == 2) {
+        p.channels = 1;
+        p.num_x = (int32_t)x->dims[1];
+        p.num_scalars = (int32_t)s->dims[1];
+        p.num_out = (int32_t)node_rows->dims[1];
+    } else {
+        p.channels = (int32_t)(leading ? x->dims[1] : x->dims[2]);
+        p.num_x = (int32_t)(leading ? x->dims[2] : x->dims[1]);
+        p.num_scalars = (int32_t)(s->rank == 3 ? (leading ? s->dims[2] : s->dims[1]) : s->dims[1]);
+        p.num_out = (int32_t)(node_rows->rank == 3 ? (leading ? node_rows->dims[2] : node_rows->dims[1])
+                                                    : node_rows->dims[1]);
+    }
+    if (x->dims[0] != p.num_nodes || node_rows->dims[0] != p.num_nodes)
+        return make_error(f, E3J_AMD_INVALID_ARGUMENT, name + ": node operands must have num_nodes rows");
+    if (s->dims[0] != p.num_edges)
+        return make_error(f, E3J_AMD_INVALID_ARGUMENT, name + ": y and s must have one row per edge");
+    if (coef->dtype == kXlaU8) p.coef_idx_bytes = 1;
+    else if (coef->dtype == kXlaS32) p.coef_idx_bytes = 4;
+    else return make_error(f, E3J_AMD_INVALID_ARGUMENT, "unsupported (IDX, VAL) dtype pair");
+    if (x->dtype == kXlaF32) p.val_dtype = E3J_AMD_F32;
+    else if (x->dtype == kXlaF64) p.val_dtype = E3J_AMD_F64;
+    else return make_error(f, E3J_AMD_INVALID_ARGUMENT, "unsupported (IDX, VAL) dtype pair");
+    if (y->dtype != x->dtype || s->dtype != x->dtype || node_rows->dtype != x->dtype)
+        return make_error(f, E3J_AMD_INVALID_ARGUMENT, name + ": value operands must share one dtype");
+
+    XlaStreamGetArgs sg;
+    sg.struct_size = sizeof(XlaStreamGetArgs);
+    sg.extension_start = nullptr;
+    sg.ctx = f->ctx;
+    sg.stream = nullptr;
+    if (void *err = f->api->stream_get(&sg)) return err;
+    d->stream = static_cast<hipStream_t>(sg.stream);
+    return nullptr;
+}
+
+bool is_s32_vector(const XlaBuffer *b) { return b && b->dtype == kXlaS32 && b->rank == 1; }
+
+void *backward_handler(XlaCallFrame *f, bool group_is_receiver) {
+    const char *op = group_is_receiver ? "convolution_bwd_receiver" : "convolution_bwd";
+    if (answer_metadata(f)) return nullptr;
+    if (f->stage != kXlaStageExecute) return nullptr;
+    if (f->args.size < 8 || f->rets.size != 3)
+        return make_error(f, E3J_AMD_INVALID_ARGUMENT,
+                          std::string(op) + ": expected 8 or 9 operands and 3 results");
+    const XlaBuffer *coef = arg(f, 0), *x = arg(f, 1), *y = arg(f, 2), *s = arg(f, 3), *dm = arg(f, 4);
+    const XlaBuffer *other = arg(f, 5), *row_ptr = arg(f, 6), *perm = arg(f, 7);
+    const XlaBuffer *dx = ret(f, 0), *dy = ret(f, 1), *ds = ret(f, 2);
+    Decoded d;
+    if (void *err = decode_common(f, op, coef, x, y, s, dm, &d)) return err;
+    if (!is_s32_vector(other) || !is_s32_vector(row_ptr) || !is_s32_vector(perm) || !dx || !dy || !ds)
+        return make_error(f, E3J_AMD_INVALID_ARGUMENT, std::string(op) + ": adjacency operands must be S32 vectors");
+    if (count(other) != d.p.num_edges || count(row_ptr) != (int64_t)d.p.num_nodes + 1 ||
+        (count(perm) != 0 && count(perm) != d.p.num_edges))
+        return make_error(f, E3J_AMD_INVALID_ARGUMENT, std::string(op) + ": adjacency operand sizes");
+    if (count(dx) != count(x) || count(dy) != count(y) || count(ds) != count(s))
+        return make_error(f, E3J_AMD_INVALID_ARGUMENT, std::string(op) + ": result shapes");
+    const int32_t stacked = attr<int32_t>(f, "coef_stacked", kXlaS32, coef->rank == 3 ? 1 : 0);
+    const int64_t numel = coef->dims[coef->rank - 1];
+    d.p.num_coef = (int32_t)(count(coef) / numel / (stacked ? 3 : 1));
+    const int32_t *perm_ptr = count(perm) ? static_cast<const int32_t *>(perm->data) : nullptr;
+    const int rc = run_backward(&d.p, group_is_receiver, coef->data, x->data, y->data, s->data, dm->data,
+                                static_cast<const int32_t *>(other->data),
+                                static_cast<const int32_t *>(row_ptr->data), perm_ptr, dx->data,
+                                dy->data, ds->data, d.stream, stacked != 0);
+    return status_to_error(f, rc);
+}
+
+}  // namespace
+}  // namespace e3j_amd
+
+using namespace e3j_amd;
+
+extern "C" {
+
+void *e3j_amd_xla_convolution(void *call_frame) {
+    XlaCallFrame *f = static_cast<XlaCallFrame *>(call_frame);
+    if (answer_metadata(f)) return nullptr;
+    if (f->stage != kXlaStageExecute) return nullptr;
+    if (f->args.size < 6 || f->rets.size != 1)
+        return make_error(f, E3J_AMD_INVALID_ARGUMENT, "convolution: expected 6 to 8 operands and 1 result");
+    const XlaBuffer *coef = arg(f, 0), *x = arg(f, 1), *y = arg(f, 2), *s = arg(f, 3);
+    const XlaBuffer *sender = arg(f, 4), *row_ptr = arg(f, 5), *out = ret(f, 0);
+    // operand 6 is the reference's coef_ranges (ignored); operand 7, if present, an edge permutation
+    const XlaBuffer *perm = f->args.size >= 8 ? arg(f, 7) : nullptr;
+    Decoded d;
+    if (void *err = decode_common(f, "convolution", coef, x, y, s, out, &d)) return err;
+    if (!is_s32_vector(sender) || !is_s32_vector(row_ptr) || (f->args.size >= 8 && !is_s32_vector(perm)))
+        return make_error(f, E3J_AMD_INVALID_ARGUMENT, "convolution: adjacency operands must be S32 vectors");
+    if (count(sender) != d.p.num_edges || count(row_ptr) != (int64_t)d.p.num_nodes + 1 ||
+        (perm && count(perm) != 0 && count(perm) != d.p.num_edges))
+        return make_error(f, E3J_AMD_INVALID_ARGUMENT, "convolution: adjacency operand sizes");
+    d.p.num_coef = (int32_t)coef->dims[0];
+    const int32_t *perm_ptr = (perm && count(perm)) ? static_cast<const int32_t *>(perm->data) : nullptr;
+    const int rc = e3j_amd_convolution_fwd(&d.p, coef->data, x->data, y->data, s->data,
+                                           static_cast<const int32_t *>(sender->data),
+                                           static_cast<const int32_t *>(row_ptr->data), perm_ptr,
+                                           out->data, d.stream);
+    return status_to_error(f, rc);
+}
+
+void *e3j_amd_xla_convolution_bwd(void *call_frame) {
+    return backward_handler(static_cast<XlaCallFrame *>(call_frame), false);
+}
+
+void *e3j_amd_xla_convolution_bwd_receiver(void *call_frame) {
+    return backward_handler(static_cast<XlaCallFrame *>(call_frame), true);
+}
+
+}  // extern "C"

@@ -1,0 +1,145 @@
+"""CSR adjacency of a directed graph, built on the device.
+
+Mirrors `GraphCSR` of the reference (`src/e3j/data/graph.py:21-91`): edges are
+grouped by receiver so a kernel can reduce a receiver's messages without
+atomics; `DUMMY_INDEX` (INT32_MAX) marks padding endpoints, which drop out of
+the adjacency.  The derived buffers (`receiver_ptr`, the permutations of `sort`
+and `transpose`) are int32 and are computed by the HIP kernels of
+`csrc/graph.hip`; the index arithmetic of `mask_edges` and of the folding
+helpers is plain tensor arithmetic.
+"""
+
+from __future__ import annotations
+
+import ctypes
+
+import numpy as np
+import torch
+
+from . import _lib
+
+DUMMY_INDEX = int(np.iinfo(np.int32).max)
+INDEX_DTYPE = torch.int32
+
+
+def is_dummy_index(index: torch.Tensor) -> torch.Tensor:
+    return index == DUMMY_INDEX
+
+
+def is_dummy_edge(sender: torch.Tensor, receiver: torch.Tensor) -> torch.Tensor:
+    return is_dummy_index(sender) | is_dummy_index(receiver)
+
+
+def _require_device(*tensors: torch.Tensor) -> torch.device:
+    device = tensors[0].device
+    for t in tensors:
+        if t.device.type != "cuda":
+            raise RuntimeError("e3j_amd graph kernels need tensors in GPU memory; got a "
+                               f"{t.device.type} tensor (there is no CPU implementation)")
+        if t.device != device:
+            raise RuntimeError("adjacency tensors must live on one device")
+    return device
+
+
+def _stream_ptr(device: torch.device) -> int:
+    return int(torch.cuda.current_stream(device).cuda_stream)
+
+
+def _as_index(t: torch.Tensor) -> torch.Tensor:
+    return t.to(INDEX_DTYPE).contiguous()
+
+
+def _workspace(num_nodes: int, num_edges: int, device) -> torch.Tensor:
+    nbytes = _lib.load().e3j_amd_csr_workspace_bytes(num_nodes, num_edges)
+    return torch.empty(max(int(nbytes), 256), dtype=torch.uint8, device=device)
+
+
+def csr_row_ptr(key: torch.Tensor, num_nodes: int) -> torch.Tensor:
+    """`[0] + cumsum(bincount(key, length=num_nodes))` as int32; out-of-range keys dropped."""
+    device = _require_device(key)
+    key = _as_index(key)
+    row_ptr = torch.empty(num_nodes + 1, dtype=INDEX_DTYPE, device=device)
+    ws = _workspace(num_nodes, key.numel(), device)
+    with torch.cuda.device(device):
+        _lib.check(_lib.load().e3j_amd_csr_row_ptr(
+            key.data_ptr(), key.numel(), num_nodes, row_ptr.data_ptr(), ws.data_ptr(),
+            _stream_ptr(device)))
+    return row_ptr
+
+
+def sort_edges(key: torch.Tensor, other: torch.Tensor, num_nodes: int):
+    """Stable sort of edge positions by `key`: `(perm, other[perm], row_ptr)`, all int32."""
+    device = _require_device(key, other)
+    key, other = _as_index(key), _as_index(other)
+    num_edges = key.numel()
+    perm = torch.empty(num_edges, dtype=INDEX_DTYPE, device=device)
+    other_sorted = torch.empty(num_edges, dtype=INDEX_DTYPE, device=device)
+    row_ptr = torch.empty(num_nodes + 1, dtype=INDEX_DTYPE, device=device)
+    ws = _workspace(num_nodes, num_edges, device)
+    with torch.cuda.device(device):
+        _lib.check(_lib.load().e3j_amd_sort_edges(
+            key.data_ptr(), other.data_ptr(), num_edges, num_nodes, perm.data_ptr(),
+            other_sorted.data_ptr(), row_ptr.data_ptr(), ws.data_ptr(), _stream_ptr(device)))
+    return perm, other_sorted, row_ptr
+
+
+class GraphCSR:
+    """Edges grouped by receiver (`src/e3j/data/graph.py:38-73`)."""
+
+    def __init__(self, num_nodes: int, sender: torch.Tensor, receiver: torch.Tensor,
+                 receiver_ptr: torch.Tensor | None = None):
+        self.num_nodes = int(num_nodes)
+        self.sender = sender
+        self.receiver = receiver
+        self._receiver_ptr = receiver_ptr
+
+    @property
+    def receiver_ptr(self) -> torch.Tensor:
+        if self._receiver_ptr is None:
+            self._receiver_ptr = csr_row_ptr(self.receiver, self.num_nodes)
+        return self._receiver_ptr
+
+    @property
+    def num_neighbors(self) -> torch.Tensor:
+        return self.receiver_ptr[1:] - self.receiver_ptr[:-1]
+
+    @classmethod
+    def sort(cls, num_nodes: int, sender: torch.Tensor, receiver: torch.Tensor):
+        """`(sigma, graph', sigma_inv)` sorting edges by receiver (stable)."""
+        perm, sender_sorted, ptr = sort_edges(receiver, sender, num_nodes)
+        graph = cls(num_nodes, sender_sorted, _as_index(receiver)[perm.long()], receiver_ptr=ptr)
+        inverse = torch.empty_like(perm)
+        inverse[perm.long()] = torch.arange(perm.numel(), dtype=INDEX_DTYPE, device=perm.device)
+        return perm, graph, inverse
+
+    def transpose(self):
+        """`(sigma, graph_t, sigma_inv)` sorting edges by sender instead."""
+        return GraphCSR.sort(self.num_nodes, self.receiver, self.sender)
+
+    @staticmethod
+    def mask_edges(sender: torch.Tensor, receiver: torch.Tensor, node_mask: torch.Tensor):
+        """Mark edges touching a padding node (at or past `count_nonzero(node_mask)`) as dummies."""
+        num_real = torch.count_nonzero(node_mask)
+        keep = (sender < num_real) & (receiver < num_real)
+        dummy = torch.full_like(sender, DUMMY_INDEX)
+        return torch.where(keep, sender, dummy), torch.where(keep, receiver, dummy)
+
+
+def wrap_global_index(index: torch.Tensor, num_nodes: int) -> torch.Tensor:
+    """Reduce modulo `num_nodes`, keeping the sentinel (`src/e3j/ops/convolution.py:39-51`)."""
+    local = torch.where(is_dummy_index(index), index, index % num_nodes)
+    return local.to(INDEX_DTYPE)
+
+
+def fold_endpoints(group: torch.Tensor, guard: torch.Tensor, axis_size: int, num_nodes: int):
+    """Fold `axis_size` graphs into one disjoint graph (`src/e3j/ops/convolution.py:54-78`).
+
+    `group`, `guard`: `(axis_size, E)`.  Padding grouping endpoints move to their
+    graph's last node so the folded key stays non-decreasing; guard endpoints keep
+    the sentinel so kernels skip the edge.
+    """
+    offsets = (torch.arange(axis_size, dtype=group.dtype, device=group.device) * num_nodes)[:, None]
+    last = offsets + (num_nodes - 1)
+    group = torch.where(is_dummy_index(group), last.expand_as(group), group + offsets)
+    guard = torch.where(is_dummy_index(guard), guard, guard + offsets)
+    return group.reshape(-1), guard.reshape(-1)

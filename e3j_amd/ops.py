@@ -1,0 +1,393 @@
+"""The fused convolution operators: `convolution` and `convolution_bwd`.
+
+Same signatures, argument meaning and errors as the reference's primitives
+(`src/e3j/ops/convolution.py:106-116,334-345`), with tensors in GPU memory
+and the HIP library of this package behind them instead of the CUDA `e3j_ops`
+binding.  `convolution` is differentiable in `(x, y, s)` to any reverse-mode
+order: its backward is `convolution_bwd`, whose own backward is expressed with
+three `convolution` and three `convolution_bwd` calls
+(`src/e3j/ops/convolution.py:535-562`).
+
+Extensions over the reference's operator: a `layout` keyword (the reference's
+fused kernel is trailing-channels only), any channel count (no power-of-two
+rule), and `GraphOrdering.NONE` (edges are sorted on the device first).
+"""
+
+from __future__ import annotations
+
+import ctypes
+import dataclasses
+import warnings
+
+import numpy as np
+import torch
+
+from . import _lib
+from .coef import Coef4D
+from .graph import (DUMMY_INDEX, INDEX_DTYPE, csr_row_ptr, fold_endpoints, sort_edges,
+                    wrap_global_index)
+from .options import GraphOrdering, Layout, config
+
+
+@dataclasses.dataclass
+class ConvolutionParams:
+    """Static sizes of the operator (`src/e3j/ops/convolution.py:81-84`)."""
+
+    num_out: int
+    num_scalars: int
+
+
+#: name used by code written against the reference
+CUDAConvolutionParams = ConvolutionParams
+
+
+class ConvolutionBatchingWarning(UserWarning):
+    """Emitted when the convolution is batched over graph adjacencies."""
+
+
+_VAL_DTYPES = {torch.float32: (_lib.F32, np.float32), torch.float64: (_lib.F64, np.float64)}
+
+
+class _Table:
+    """A packed coefficient table with its device copies and kernel selection."""
+
+    _cache: dict = {}
+
+    def __init__(self, packed: np.ndarray, val_np_dtype):
+        self.packed = np.ascontiguousarray(packed)
+        self.idx_bytes = self.packed.dtype.itemsize
+        self.val_np_dtype = np.dtype(val_np_dtype)
+        self.num_coef = int(self.packed.shape[0])
+        self._device = {}
+        self._signature = {}
+
+    @classmethod
+    def get(cls, coef, val_np_dtype) -> "_Table":
+        if isinstance(coef, torch.Tensor):
+            raise TypeError("`coef` must be concrete: it is read on the host.")
+        packed = np.asarray(coef)
+        if packed.dtype not in (np.dtype(np.uint8), np.dtype(np.int32)):
+            raise TypeError(f"unsupported coefficient index dtype {packed.dtype}")
+        key = (packed.dtype.str, packed.shape, packed.tobytes(), np.dtype(val_np_dtype).str)
+        table = cls._cache.get(key)
+        if table is None:
+            if len(cls._cache) > 256:
+                cls._cache.clear()
+            table = cls._cache[key] = cls(packed, val_np_dtype)
+        return table
+
+    def unpack(self) -> Coef4D:
+        return Coef4D.unpack(self.packed, self.val_np_dtype)
+
+    def device(self, device: torch.device) -> torch.Tensor:
+        t = self._device.get(device)
+        if t is None:
+            t = torch.from_numpy(self.packed.view(np.uint8).reshape(-1).copy()).to(device)
+            self._device[device] = t
+        return t
+
+    def signature(self, dims, channels: int, layout: Layout):
+        """`(id, scale)` of a built-in unrolled kernel, `(-1, 1.0)` if none matches."""
+        key = (dims, channels, layout)
+        hit = self._signature.get(key)
+        if hit is None:
+            scale = ctypes.c_float(1.0)
+            val_code = _lib.F32 if self.val_np_dtype == np.float32 else _lib.F64
+            sig = _lib.load().e3j_amd_find_signature(
+                self.packed.ctypes.data, self.idx_bytes, val_code, self.num_coef, dims[0], dims[1],
+                dims[2], dims[3], channels, layout.value, ctypes.byref(scale))
+            hit = self._signature[key] = (int(sig), float(scale.value))
+        return hit
+
+
+@dataclasses.dataclass
+class _Meta:
+    """Everything static about one call."""
+
+    table: _Table
+    signed_table: _Table | None  # forward table under SENDER ordering
+    params: ConvolutionParams
+    ordering: GraphOrdering
+    layout: Layout
+    y_parity: np.ndarray | None
+    num_nodes: int
+    squeeze_channels: bool       # x was (N, X): channel axis added internally
+    y_shape: tuple
+
+
+def _stream(device) -> int:
+    return int(torch.cuda.current_stream(device).cuda_stream)
+
+
+def _fill_params(meta: _Meta, x: torch.Tensor, y: torch.Tensor, s: torch.Tensor, forward: bool,
+                 use_signature: bool = True):
+    layout = meta.layout
+    if layout == Layout.TRAILING_CHANNELS:
+        num_x, channels = x.shape[1], x.shape[2]
+        num_s = s.shape[1]
+    else:
+        channels, num_x = x.shape[1], x.shape[2]
+        num_s = s.shape[2]
+    val_code = _VAL_DTYPES[x.dtype][0]
+    table = meta.signed_table if (forward and meta.signed_table is not None) else meta.table
+    dims = (int(num_x), int(y.shape[1]), int(meta.params.num_out), int(num_s))
+    sig, scale = table.signature(dims, int(channels), layout) if use_signature else (-1, 1.0)
+    cfg = config()
+    p = _lib.ConvParams(
+        num_nodes=int(x.shape[0]), num_edges=int(y.shape[0]), num_coef=table.num_coef,
+        num_x=dims[0], num_y=dims[1], num_out=dims[2], num_scalars=dims[3], channels=int(channels),
+        layout=layout.value, val_dtype=val_code, coef_idx_bytes=table.idx_bytes,
+        signature=sig, coef_scale=scale, debug=int(cfg.debug_level))
+    return p, table
+
+
+def _check_operands(x, y, s, sender, receiver):
+    for name, t in (("x", x), ("y", y), ("s", s), ("sender", sender), ("receiver", receiver)):
+        if not isinstance(t, torch.Tensor):
+            raise TypeError(f"`{name}` must be a torch.Tensor")
+        if t.device.type != "cuda":
+            raise RuntimeError(f"`{name}` must live in GPU memory; e3j_amd has no CPU implementation")
+    if x.dtype not in _VAL_DTYPES:
+        raise TypeError(f"Fused ops support value dtypes ('float32', 'float64'), got {x.dtype}. "
+                        "Cast the operands.")
+    if y.dtype != x.dtype or s.dtype != x.dtype:
+        raise TypeError("x, y and s must share one dtype")
+
+
+def _forward_graph(meta: _Meta, sender: torch.Tensor, receiver: torch.Tensor):
+    """CSR used by the forward kernel: `(other, row_ptr, perm)`."""
+    n = meta.num_nodes
+    sender_l, receiver_l = wrap_global_index(sender, n), wrap_global_index(receiver, n)
+    if meta.ordering == GraphOrdering.RECEIVER:
+        return sender_l.contiguous(), csr_row_ptr(receiver_l, n), None
+    if meta.ordering == GraphOrdering.SENDER:
+        # aggregate over reversed edges; y parities are folded into the coefficients
+        return receiver_l.contiguous(), csr_row_ptr(sender_l, n), None
+    perm, sender_sorted, row_ptr = sort_edges(receiver_l, sender_l, n)
+    return sender_sorted, row_ptr, perm
+
+
+def _raw_forward(meta: _Meta, x, y, s, sender, receiver) -> torch.Tensor:
+    x, y, s = x.contiguous(), y.contiguous(), s.contiguous()
+    p, table = _fill_params(meta, x, y, s, forward=True)
+    other, row_ptr, perm = _forward_graph(meta, sender, receiver)
+    if meta.layout == Layout.TRAILING_CHANNELS:
+        out = torch.empty((x.shape[0], meta.params.num_out, x.shape[2]), dtype=x.dtype, device=x.device)
+    else:
+        out = torch.empty((x.shape[0], x.shape[1], meta.params.num_out), dtype=x.dtype, device=x.device)
+    with torch.cuda.device(x.device):
+        _lib.check(_lib.load().e3j_amd_convolution_fwd(
+            ctypes.byref(p), table.device(x.device).data_ptr(), x.data_ptr(), y.data_ptr(), s.data_ptr(),
+            other.data_ptr(), row_ptr.data_ptr(), perm.data_ptr() if perm is not None else None,
+            out.data_ptr(), _stream(x.device)))
+    return out
+
+
+def _raw_backward(meta: _Meta, x, y, s, dm, sender, receiver):
+    x, y, s, dm = x.contiguous(), y.contiguous(), s.contiguous(), dm.contiguous()
+    n = meta.num_nodes
+    sender_l, receiver_l = wrap_global_index(sender, n), wrap_global_index(receiver, n)
+    dx, dy, ds = torch.empty_like(x), torch.empty_like(y), torch.empty_like(s)
+    lib = _lib.load()
+    deterministic = config().deterministic
+    if meta.ordering == GraphOrdering.SENDER:
+        # already grouped by sender: rows own their dx, no permutation
+        group_receiver, other, row_ptr, perm = False, receiver_l.contiguous(), csr_row_ptr(sender_l, n), None
+    elif deterministic:
+        perm, other, row_ptr = sort_edges(sender_l, receiver_l, n)
+        group_receiver = False
+    elif meta.ordering == GraphOrdering.RECEIVER:
+        group_receiver, other, row_ptr, perm = True, sender_l.contiguous(), csr_row_ptr(receiver_l, n), None
+    else:
+        perm, other, row_ptr = sort_edges(receiver_l, sender_l, n)
+        group_receiver = True
+    p, table = _fill_params(meta, x, y, s, forward=False, use_signature=group_receiver)
+    fn = lib.e3j_amd_convolution_bwd_receiver if group_receiver else lib.e3j_amd_convolution_bwd_sender
+    with torch.cuda.device(x.device):
+        _lib.check(fn(ctypes.byref(p), table.device(x.device).data_ptr(), x.data_ptr(), y.data_ptr(),
+                      s.data_ptr(), dm.data_ptr(), other.data_ptr(), row_ptr.data_ptr(),
+                      perm.data_ptr() if perm is not None else None,
+                      dx.data_ptr(), dy.data_ptr(), ds.data_ptr(), _stream(x.device)))
+    return dx, dy, ds
+
+
+def _sum(*terms):
+    terms = [t for t in terms if t is not None]
+    if not terms:
+        return None
+    total = terms[0]
+    for t in terms[1:]:
+        total = total + t
+    return total
+
+
+class _Convolution(torch.autograd.Function):
+    @staticmethod
+    def forward(ctx, x, y, s, sender, receiver, meta):
+        ctx.meta = meta
+        ctx.save_for_backward(x, y, s, sender, receiver)
+        return _raw_forward(meta, x, y, s, sender, receiver)
+
+    @staticmethod
+    def backward(ctx, dm):
+        x, y, s, sender, receiver = ctx.saved_tensors
+        dx, dy, ds = _ConvolutionBwd.apply(x, y, s, dm, sender, receiver, ctx.meta)
+        return dx, dy, ds, None, None, None
+
+
+class _ConvolutionBwd(torch.autograd.Function):
+    @staticmethod
+    def forward(ctx, x, y, s, dm, sender, receiver, meta):
+        ctx.meta = meta
+        ctx.save_for_backward(x, y, s, dm, sender, receiver)
+        return _raw_backward(meta, x, y, s, dm, sender, receiver)
+
+    @staticmethod
+    def backward(ctx, ddx, ddy, dds):
+        # (Dx, Dy, Ds, Ddm) from (Ddx, Ddy, Dds): the trilinear form's second variation
+        # (`src/e3j/ops/convolution.py:535-562`).
+        x, y, s, dm, sender, receiver = ctx.saved_tensors
+        meta = ctx.meta
+
+        def conv(a, b, c):
+            return _Convolution.apply(a, b, c, sender, receiver, meta)
+
+        def conv_bwd(a, b, c):
+            return _ConvolutionBwd.apply(a, b, c, dm, sender, receiver, meta)
+
+        d_dm, d_x, d_y, d_s = [], [], [], []
+        if ddx is not None:
+            d_dm.append(conv(ddx, y, s))
+            _, gy, gs = conv_bwd(ddx, y, s)
+            d_y.append(gy)
+            d_s.append(gs)
+        if ddy is not None:
+            d_dm.append(conv(x, ddy, s))
+            gx, _, gs = conv_bwd(x, ddy, s)
+            d_x.append(gx)
+            d_s.append(gs)
+        if dds is not None:
+            d_dm.append(conv(x, y, dds))
+            gx, gy, _ = conv_bwd(x, y, dds)
+            d_x.append(gx)
+            d_y.append(gy)
+        return _sum(*d_x), _sum(*d_y), _sum(*d_s), _sum(*d_dm), None, None, None
+
+
+def _make_meta(coef, x, y, s, params, graph_ordering, y_parity, layout) -> _Meta:
+    ordering = GraphOrdering.parse(graph_ordering)
+    layout = Layout.parse(layout)
+    val_np = _VAL_DTYPES[x.dtype][1]
+    table = _Table.get(coef, val_np)
+    signed = None
+    if ordering == GraphOrdering.SENDER:
+        if y_parity is None:
+            raise ValueError("SENDER graph ordering requires `y_parity`.")
+        c = table.unpack()
+        signs = np.asarray(y_parity, dtype=c.val.dtype)[c.idx[:, 2].astype(np.int64)]
+        signed = _Table.get(Coef4D(c.val * signs, c.idx, c.val_dtype, c.idx_dtype).pack(), val_np)
+    return _Meta(table=table, signed_table=signed, params=params, ordering=ordering, layout=layout,
+                 y_parity=None if y_parity is None else np.asarray(y_parity),
+                 num_nodes=int(x.shape[0]), squeeze_channels=False, y_shape=tuple(y.shape))
+
+
+def _canonical(x, y, s, layout: Layout):
+    """Add the channel axis of a 2-D `x`/`s`, drop a unit channel axis of `y`."""
+    squeeze = x.ndim == 2
+    if y.ndim == x.ndim and y.shape[-1] != 1 and not squeeze:
+        raise NotImplementedError("RHS y should have only one channel.")
+    if squeeze:
+        axis = -1 if layout == Layout.TRAILING_CHANNELS else 1
+        x = x.unsqueeze(axis)
+        if s.ndim == 2:
+            s = s.unsqueeze(axis)
+        if y.ndim == 3:
+            y = y.reshape(y.shape[0], -1)
+    elif y.ndim == 3:
+        y = y[..., 0]
+    if x.ndim != 3 or s.ndim != 3 or y.ndim != 2:
+        raise ValueError(f"unexpected operand ranks: x {tuple(x.shape)}, y {tuple(y.shape)}, "
+                         f"s {tuple(s.shape)}")
+    return x, y, s, squeeze
+
+
+def convolution(coef, x, y, s, sender, receiver, params: ConvolutionParams,
+                graph_ordering=GraphOrdering.RECEIVER, y_parity=None, *,
+                layout=Layout.TRAILING_CHANNELS) -> torch.Tensor:
+    """`out[r] = sum_{e: recv(e)=r} (x[send(e)] (x) y[e]) . s[e]` with the fused HIP kernels.
+
+    Args:
+        coef: packed `Coef4D` table (host numpy array, opaque index dtype).
+        x: node features `(num_nodes, num_x, channels)` [leading layout: `(num_nodes, channels, num_x)`].
+        y: edge embeddings `(num_edges, num_y)`, single channel.
+        s: radial scalars `(num_edges, num_scalars, channels)` [leading: `(num_edges, channels, num_scalars)`].
+        sender, receiver: `(num_edges,)` integer endpoints; `DUMMY_INDEX` marks padding.
+            Sorted by receiver (RECEIVER) or sender (SENDER), or in any order (NONE).
+        params: `ConvolutionParams(num_out, num_scalars)`.
+        y_parity: per-`y`-component parity, required under SENDER ordering.
+    """
+    _check_operands(x, y, s, sender, receiver)
+    layout = Layout.parse(layout)
+    y_in_shape = tuple(y.shape)
+    x3, y2, s3, squeeze = _canonical(x, y, s, layout)
+    meta = _make_meta(coef, x3, y2, s3, params, graph_ordering, y_parity, layout)
+    out = _Convolution.apply(x3, y2, s3, sender, receiver, meta)
+    del y_in_shape
+    if squeeze:
+        out = out.squeeze(-1 if layout == Layout.TRAILING_CHANNELS else 1)
+    return out
+
+
+def convolution_bwd(coef, x, y, s, sender, receiver, dm, params: ConvolutionParams,
+                    graph_ordering=GraphOrdering.RECEIVER, y_parity=None, *,
+                    layout=Layout.TRAILING_CHANNELS):
+    """Cotangents `(dx, dy, ds)` of `convolution` for the output cotangent `dm`."""
+    _check_operands(x, y, s, sender, receiver)
+    layout = Layout.parse(layout)
+    y_in_shape = tuple(y.shape)
+    x3, y2, s3, squeeze = _canonical(x, y, s, layout)
+    dm3 = dm.unsqueeze(-1 if layout == Layout.TRAILING_CHANNELS else 1) if squeeze else dm
+    meta = _make_meta(coef, x3, y2, s3, params, graph_ordering, y_parity, layout)
+    dx, dy, ds = _ConvolutionBwd.apply(x3, y2, s3, dm3, sender, receiver, meta)
+    if squeeze:
+        axis = -1 if layout == Layout.TRAILING_CHANNELS else 1
+        dx = dx.squeeze(axis)
+        if s.ndim == 2:
+            ds = ds.squeeze(axis)
+    return dx, dy.reshape(y_in_shape), ds
+
+
+def convolution_batched(coef, x, y, s, sender, receiver, params: ConvolutionParams,
+                        graph_ordering=GraphOrdering.RECEIVER, y_parity=None, *,
+                        layout=Layout.TRAILING_CHANNELS) -> torch.Tensor:
+    """Batch of graphs on a leading axis, folded into one disjoint graph.
+
+    The counterpart of the reference's batching rule (`src/e3j/ops/convolution.py:271-308`):
+    `x (B, N, ...)`, `y (B, E, Y)`, `s (B, E, ...)`; `sender`/`receiver` either `(E,)`
+    (one graph shared by the batch) or `(B, E)` (one graph per batch entry, which
+    emits `ConvolutionBatchingWarning`).
+    """
+    ordering = GraphOrdering.parse(graph_ordering)
+    batch, num_nodes, num_edges = x.shape[0], x.shape[1], y.shape[1]
+    if sender.ndim != receiver.ndim:
+        raise ValueError("Graph adjacency inconsistently batched.")
+    if sender.ndim == 2:
+        warnings.warn("Convolution is being batched over graph adjacency. Batch graphs into a "
+                      "single, disconnected graph upstream or silence this warning by filtering "
+                      "`ConvolutionBatchingWarning`.", ConvolutionBatchingWarning, stacklevel=2)
+    else:
+        sender = sender.unsqueeze(0).expand(batch, -1)
+        receiver = receiver.unsqueeze(0).expand(batch, -1)
+    sender, receiver = sender.to(torch.int64), receiver.to(torch.int64)
+    if ordering == GraphOrdering.SENDER:
+        sender_f, receiver_f = fold_endpoints(sender, receiver, batch, num_nodes)
+    else:
+        receiver_f, sender_f = fold_endpoints(receiver, sender, batch, num_nodes)
+    out = convolution(coef, x.reshape((batch * num_nodes,) + tuple(x.shape[2:])),
+                      y.reshape((batch * num_edges,) + tuple(y.shape[2:])),
+                      s.reshape((batch * num_edges,) + tuple(s.shape[2:])),
+                      sender_f, receiver_f, params, ordering, y_parity, layout=layout)
+    return out.reshape((batch, num_nodes) + tuple(out.shape[1:]))
+
+
+convolution.Params = ConvolutionParams

@@ -1,0 +1,127 @@
+"""Option enums and the small configuration object of the fused convolution path.
+
+Mirrors the option names of the reference (`src/e3j/utils/options.py:76-180`,
+`src/e3j/utils/config.py:42-216`) for the one path this package implements.
+There is deliberately no unfused/CPU evaluation strategy here: the only
+evaluation strategy is the HIP kernel library, and it fails loudly when the
+library is missing.
+"""
+
+from __future__ import annotations
+
+import contextlib
+import dataclasses
+import os
+from enum import Enum
+
+
+class _ParsedEnum(Enum):
+    """Enum with a forgiving `parse` accepting members, names and values."""
+
+    @classmethod
+    def parse(cls, value):
+        if isinstance(value, cls):
+            return value
+        if isinstance(value, str):
+            key = value.strip().upper()
+            if key in cls.__members__:
+                return cls.__members__[key]
+        for member in cls:
+            if member.value == value:
+                return member
+        raise ValueError(f"{value!r} is not a valid {cls.__name__}; "
+                         f"expected one of {list(cls.__members__)}")
+
+
+class Layout(_ParsedEnum):
+    """Memory layout of equivariant arrays (`src/e3j/utils/options.py:122-151`).
+
+    LEADING_CHANNELS: `(rows, channels, dim)`; TRAILING_CHANNELS: `(rows, dim, channels)`.
+    The integer values are the ones the reference hands to its FFI.
+    """
+
+    LEADING_CHANNELS = 0
+    TRAILING_CHANNELS = 1
+
+
+class GraphOrdering(_ParsedEnum):
+    """Edge ordering contract (`src/e3j/utils/options.py:95-112`).
+
+    RECEIVER / SENDER: edges sorted by that endpoint. NONE: no ordering is
+    promised; the kernel library then sorts on the device before reducing.
+    """
+
+    RECEIVER = "RECEIVER"
+    SENDER = "SENDER"
+    NONE = "NONE"
+
+
+class TensorProductNormalization(_ParsedEnum):
+    """Scaling of the stacked Clebsch-Gordan blocks (`src/e3j/utils/options.py:171-180`)."""
+
+    NONE = "NONE"
+    SQRT_DIM_OUT = "SQRT_DIM_OUT"
+
+
+class Convolution(_ParsedEnum):
+    """Evaluation strategy of `e3j_amd.Convolution` (`src/e3j/utils/options.py:76-92`).
+
+    FUSED_HIP is the only strategy: hand-written gfx950 kernels behind the C ABI.
+    """
+
+    FUSED_HIP = "FUSED_HIP"
+
+
+@dataclasses.dataclass(frozen=True)
+class Config:
+    """Frozen settings snapshot (`src/e3j/utils/config.py:42-105`)."""
+
+    layout: Layout = Layout.TRAILING_CHANNELS
+    convolution: Convolution = Convolution.FUSED_HIP
+    #: 0 = asynchronous launches; >0 = synchronise the stream after each launch
+    #: so that device-side failures surface at the faulting call.
+    debug_level: int = 0
+    #: atomic-free backward for `dx` (bit-reproducible, slower).
+    deterministic: bool = False
+
+
+class _ConfigHolder:
+    """Mutable process-wide holder with `use(**kw)` scoping (`src/e3j/utils/config.py:107-216`)."""
+
+    def __init__(self):
+        self._current = Config(
+            debug_level=int(os.environ.get("E3J_AMD_DEBUG", "0")),
+            deterministic=os.environ.get("E3J_AMD_DETERMINISTIC", "0") not in ("0", ""),
+        )
+
+    def __call__(self, **updates) -> Config:
+        if updates:
+            self._current = self._coerce(updates)
+        return self._current
+
+    def _coerce(self, updates) -> Config:
+        fields = {f.name for f in dataclasses.fields(Config)}
+        unknown = set(updates) - fields
+        if unknown:
+            raise TypeError(f"unknown config field(s): {sorted(unknown)}")
+        if "layout" in updates:
+            updates["layout"] = Layout.parse(updates["layout"])
+        if "convolution" in updates:
+            updates["convolution"] = Convolution.parse(updates["convolution"])
+        return dataclasses.replace(self._current, **updates)
+
+    @contextlib.contextmanager
+    def use(self, **updates):
+        previous = self._current
+        self._current = self._coerce(updates)
+        try:
+            yield self._current
+        finally:
+            self._current = previous
+
+    def snapshot(self, config: Config | None = None) -> Config:
+        """Modules freeze the settings they were built under."""
+        return self._current if config is None else config
+
+
+config = _ConfigHolder()

@@ -1,0 +1,133 @@
+"""Host-side construction of the stacked Clebsch-Gordan coefficient table.
+
+Only the parts of the reference's `TensorProduct` that the fused convolution
+consumes are here: selection rules, block stacking and the canonical sort of
+output blocks (`src/e3j/core/tensor_product.py:169-274`,
+`src/e3j/core/permutation.py:55-74`).  Evaluating a stand-alone tensor
+product is a different operator and is not part of this package.
+"""
+
+from __future__ import annotations
+
+import itertools
+
+import numpy as np
+
+from .clebsch_gordan import clebsch_gordan
+from .options import Layout, TensorProductNormalization, config as _config
+from .sparse import SparseCOO, sparse_coo
+from .spaces import O3Space
+
+
+def block_sort_permutation(space: O3Space):
+    """Coordinate permutation sorting the blocks of `space` by (degree, parity).
+
+    Returns `(sigma, sigma_inv, target)`: `sorted[i] = unsorted[sigma[i]]`, and
+    `target` is the sorted space with equal irreps merged
+    (`src/e3j/core/permutation.py:55-74`).
+    """
+    space = O3Space(space)
+    sorted_space, order = space.sort(return_inverse=True)
+    slices = space.slices()
+    sigma = np.concatenate(
+        [np.arange(slices[b].start, slices[b].stop) for b in order]
+    ) if len(order) else np.zeros((0,), dtype=np.int64)
+    return sigma, np.argsort(sigma), sorted_space.regroup()
+
+
+class TensorProduct:
+    r"""Coefficients of the bilinear map `z_i = \sum_{jk} c_{ijk} x_j y_k`."""
+
+    def __init__(self, source, target=None, coef: SparseCOO | None = None, sort: bool = True,
+                 config=None, layout=Layout.LEADING_CHANNELS,
+                 normalization=TensorProductNormalization.NONE):
+        if len(source) != 2:
+            raise TypeError("TensorProduct expects a binary tuple as source argument.")
+        self.source = tuple(O3Space(s) for s in source)
+        self.config = _config.snapshot(config)
+        self.layout = Layout.parse(layout)
+        self.normalization = TensorProductNormalization.parse(normalization)
+        infer = coef is None
+        if target is None:
+            self.target = self.infer_target(self.source)
+        elif infer:
+            self.target = self.infer_target(self.source, O3Space(target))
+        else:
+            self.target = O3Space(target)
+        self._coef = coef
+        if sort and infer:
+            other = self.sort()
+            self.target, self._coef = other.target, other.coef
+
+    # --- coefficient access ----------------------------------------------
+    @property
+    def coef(self) -> SparseCOO:
+        if self._coef is None:
+            self._coef = self.clebsch_gordan(self.target, *self.source, self.normalization)
+        return self._coef
+
+    @coef.setter
+    def coef(self, value: SparseCOO):
+        self._coef = value
+
+    @property
+    def values(self) -> np.ndarray:
+        return self.coef.data
+
+    @property
+    def indices(self) -> np.ndarray:
+        return self.coef.indices
+
+    @property
+    def shape(self):
+        return self.coef.shape
+
+    # --- construction ----------------------------------------------------
+    @staticmethod
+    def infer_target(source, target=None, sort: bool = False) -> O3Space:
+        return O3Space.otimes(source[0], source[1], target, sort)
+
+    def sort(self) -> "TensorProduct":
+        """Permute output coordinates so blocks are ordered by (degree, parity)."""
+        _, sigma_inv, target = block_sort_permutation(self.target)
+        idx = self.indices.astype(np.int64)
+        idx = np.concatenate((sigma_inv[idx[:, 0]][:, None], idx[:, 1:]), axis=-1)
+        return TensorProduct(self.source, target, coef=sparse_coo(self.values, idx, self.shape),
+                             sort=False, config=self.config, layout=self.layout,
+                             normalization=self.normalization)
+
+    @staticmethod
+    def clebsch_gordan(target, source_1, source_2,
+                       normalization=TensorProductNormalization.NONE) -> SparseCOO:
+        """Stack one Clebsch-Gordan block per path, in x-major / y / l_out order.
+
+        `target` only filters which `(l, p)` are kept; the output coordinates are
+        laid out path after path (`src/e3j/core/tensor_product.py:202-274`).
+        """
+        target, in1, in2 = O3Space(target), O3Space(source_1), O3Space(source_2)
+        normalization = TensorProductNormalization.parse(normalization)
+        keep = {(ir.l, ir.p) for _, ir in target}
+        values, indices, begin_out = [], [], 0
+        for ((m1, ir1), s1), ((m2, ir2), s2) in itertools.product(
+                zip(in1, in1.slices()), zip(in2, in2.slices())):
+            k1, k2 = np.mgrid[:m1, :m2].reshape(2, -1)
+            for _, ir0 in ir1 * ir2:
+                if (ir0.l, ir0.p) not in keep:
+                    continue
+                dense = clebsch_gordan(ir0.l, ir1.l, ir2.l)
+                nz = np.nonzero(dense)
+                data = dense[nz]
+                if normalization == TensorProductNormalization.SQRT_DIM_OUT:
+                    data = data * np.sqrt(2 * ir0.l + 1)
+                block_idx = np.stack(nz, axis=-1)
+                values.append(np.tile(data, m1 * m2))
+                offset = np.array([begin_out, s1.start, s2.start])
+                dims = np.array([ir0.dim, ir1.dim, ir2.dim])
+                mul_grid = np.stack((k1 * m2 + k2, k1, k2), axis=-1)
+                offsets = offset + mul_grid * dims
+                indices.append((block_idx[None, :] + offsets[:, None]).reshape(-1, 3))
+                begin_out += m1 * m2 * ir0.dim
+        shape = (target.dim, in1.dim, in2.dim)
+        if not values:
+            return sparse_coo(np.zeros((0,)), np.zeros((0, 3), dtype=np.int64), shape)
+        return sparse_coo(np.concatenate(values), np.concatenate(indices, axis=0), shape)

@@ -1,0 +1,143 @@
+/* C ABI of the MI355X (gfx950) fused message-passing convolution library.
+ *
+ * Every entry point takes plain device pointers, sizes and a HIP stream and
+ * returns a status code; nothing here names a tensor framework.  The operand
+ * lists are those of the reference's two XLA-FFI targets for this path,
+ * "convolution" and "convolution_bwd" (lib/e3j_ops/ffi/e3j_ops.h:379-472 and
+ * :478-594), minus `coef_ranges` (a CUDA launch-balancing artefact) and plus
+ * the memory layout, an optional edge permutation on the forward and the id of
+ * a compile-time-unrolled kernel.
+ *
+ * Conventions
+ *  - Values are float32 (or float64 on the table-driven kernels); indices int32.
+ *  - TRAILING layout: x (N, X, K), s (E, S, K), out/dm (N, Z, K).
+ *    LEADING  layout: x (N, K, X), s (E, K, S), out/dm (N, K, Z).  y is (E, Y).
+ *  - A CSR adjacency groups edge positions by one endpoint: `row_ptr` (N+1)
+ *    and, per position, the other endpoint `other` (E).  A position whose
+ *    `other` lies outside [0, N), or that lies at or past row_ptr[N], is a
+ *    padding edge: it contributes nothing and gets dy = ds = 0
+ *    (lib/e3j_ops/cuda/convolution/fwd.cuh:368, bwd.cuh:225-226,308-319).
+ *  - `edge_perm` (E) maps a CSR position to the row of y / s / dy / ds it
+ *    refers to; NULL means identity (lib/e3j_ops/ffi/e3j_ops.h:543-548).
+ *  - `coef` is the packed table {val; i; j; k; l} of lib/e3j_ops/cuda/convolution.cuh:31-44,
+ *    resident in device memory; `coef_idx_bytes` is 1 (uint8) or 4 (int32).
+ *  - Launches are asynchronous on `stream`; with debug > 0 the stream is
+ *    synchronised before returning so device faults surface at the call
+ *    (lib/e3j_ops/cuda/convolution/launch_fwd.cuh:255-263).
+ *  - Rows of nodes without live edges are written as exact zeros.
+ */
+#ifndef E3J_AMD_H_
+#define E3J_AMD_H_
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+/* Status codes; names follow the reference's error classes (lib/e3j_ops/ffi/error.h:22-105). */
+enum {
+    E3J_AMD_OK = 0,
+    E3J_AMD_INVALID_ARGUMENT = 1,
+    E3J_AMD_UNIMPLEMENTED = 2,
+    E3J_AMD_INTERNAL = 3
+};
+
+enum { E3J_AMD_LAYOUT_LEADING = 0, E3J_AMD_LAYOUT_TRAILING = 1 }; /* src/e3j/utils/options.py:144-145 */
+enum { E3J_AMD_F32 = 0, E3J_AMD_F64 = 1 };
+
+/* Problem sizes, the counterpart of convolution::Params (lib/e3j_ops/cuda/convolution.cuh:46-60). */
+typedef struct e3j_amd_conv_params {
+    int32_t num_nodes;
+    int64_t num_edges;
+    int32_t num_coef;
+    int32_t num_x;
+    int32_t num_y;
+    int32_t num_out;
+    int32_t num_scalars;
+    int32_t channels;
+    int32_t layout;         /* E3J_AMD_LAYOUT_* */
+    int32_t val_dtype;      /* E3J_AMD_F32 / E3J_AMD_F64 */
+    int32_t coef_idx_bytes; /* 1 or 4 */
+    int32_t signature;      /* id from e3j_amd_find_signature, or -1: table-driven kernel */
+    float   coef_scale;     /* unrolled kernels: table = coef_scale * built-in table (1 by default) */
+    int32_t debug;
+} e3j_amd_conv_params;
+
+/* Message of the last failure on the calling thread ("" if none). */
+const char *e3j_amd_last_error(void);
+
+/* Library version string. */
+const char *e3j_amd_version(void);
+
+/* Forward: replaces the "convolution" target (lib/e3j_ops/ffi/e3j_ops.h:379-472;
+ * kernel lib/e3j_ops/cuda/convolution/fwd.cuh:289-403).
+ * CSR grouped by receiver: other = sender per position, row_ptr = receiver_ptr. */
+int e3j_amd_convolution_fwd(const e3j_amd_conv_params *p, const void *coef,
+                            const void *x, const void *y, const void *s,
+                            const int32_t *sender, const int32_t *receiver_ptr,
+                            const int32_t *edge_perm, void *out, void *stream);
+
+/* Backward, operands of the reference: replaces the "convolution_bwd" target
+ * (lib/e3j_ops/ffi/e3j_ops.h:478-594; kernel lib/e3j_ops/cuda/convolution/bwd.cuh:116-321).
+ * CSR grouped by SENDER (the transposed adjacency): receiver_t = receiver per
+ * position, sender_ptr = row pointer by sender, edge_perm = position -> original
+ * edge (NULL under SENDER ordering).  `coef` is the FORWARD table (i, j, k, l);
+ * the reference's three transposed copies are not needed.  dx is accumulated
+ * row-locally without atomics: results are bit-reproducible run to run. */
+int e3j_amd_convolution_bwd_sender(const e3j_amd_conv_params *p, const void *coef,
+                                   const void *x, const void *y, const void *s, const void *dm,
+                                   const int32_t *receiver_t, const int32_t *sender_ptr,
+                                   const int32_t *edge_perm,
+                                   void *dx, void *dy, void *ds, void *stream);
+
+/* Backward on the forward's own receiver-grouped CSR (no transpose, no sort):
+ * same results as e3j_amd_convolution_bwd_sender up to the summation order of dx,
+ * which is accumulated with float atomics.  This is the grouping the reference
+ * recommends for its Mosaic-GPU backend (src/e3j/core/convolution.py:77-82). */
+int e3j_amd_convolution_bwd_receiver(const e3j_amd_conv_params *p, const void *coef,
+                                     const void *x, const void *y, const void *s, const void *dm,
+                                     const int32_t *sender, const int32_t *receiver_ptr,
+                                     const int32_t *edge_perm,
+                                     void *dx, void *dy, void *ds, void *stream);
+
+/* Match a HOST copy of a packed forward table against the tables of the
+ * compile-time-unrolled kernels built into the library, up to one uniform
+ * positive factor (the 1/avg_num_neighbors the reference folds into the values,
+ * src/e3j/core/convolution.py:135-140), which is returned in *coef_scale.
+ * Returns the signature id (>= 0) or -1.  Takes the place of the reference's
+ * trace-time launch planning (src/e3j/ops/convolution.py:178-208). */
+int e3j_amd_find_signature(const void *coef_host, int32_t coef_idx_bytes, int32_t val_dtype,
+                           int32_t num_coef, int32_t num_x, int32_t num_y, int32_t num_out,
+                           int32_t num_scalars, int32_t channels, int32_t layout,
+                           float *coef_scale);
+
+/* Number of built-in signatures and a printable description of one. */
+int e3j_amd_num_signatures(void);
+const char *e3j_amd_signature_name(int signature);
+
+/* Graph preparation on the device, replacing the per-call XLA ops of
+ * GraphCSR (src/e3j/data/graph.py:49-73).
+ * e3j_amd_csr_row_ptr: row_ptr = [0] + cumsum(bincount(key, length = num_nodes)),
+ *   keys outside [0, num_nodes) dropped.  workspace: >= e3j_amd_csr_workspace_bytes(). */
+size_t e3j_amd_csr_workspace_bytes(int32_t num_nodes, int64_t num_edges);
+int e3j_amd_csr_row_ptr(const int32_t *key, int64_t num_edges, int32_t num_nodes,
+                        int32_t *row_ptr, void *workspace, void *stream);
+/* e3j_amd_sort_edges: stable counting sort of edge positions by key (out-of-range
+ *   keys last): perm (E), other_sorted = other[perm] (E), row_ptr (N+1). */
+int e3j_amd_sort_edges(const int32_t *key, const int32_t *other, int64_t num_edges,
+                       int32_t num_nodes, int32_t *perm, int32_t *other_sorted,
+                       int32_t *row_ptr, void *workspace, void *stream);
+
+/* XLA-FFI handlers (C ABI of xla/ffi/api/c_api.h): `XLA_FFI_Error* handler(XLA_FFI_CallFrame*)`.
+ * Operand order of "convolution"/"convolution_bwd" as in lib/e3j_ops/ffi/e3j_ops.h:457-472,575-594;
+ * attrs: num_nodes, debug (reference) + layout, signature (optional). */
+void *e3j_amd_xla_convolution(void *call_frame);
+void *e3j_amd_xla_convolution_bwd(void *call_frame);
+void *e3j_amd_xla_convolution_bwd_receiver(void *call_frame);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* E3J_AMD_H_ */

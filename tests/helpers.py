@@ -1,0 +1,109 @@
+"""Shared builders and the parity criterion of the test-suite."""
+
+from __future__ import annotations
+
+import ctypes
+
+import numpy as np
+
+from oracle import conv_oracle as O
+
+EPS32 = float(np.finfo(np.float32).eps)
+
+
+# ---------------------------------------------------------------------------
+# problem builders
+# ---------------------------------------------------------------------------
+def random_table(rng, nnz, num_x, num_y, num_out, num_scalars):
+    """Random sparse table covering every out/x/y coordinate, sorted by output index.
+
+    Construction of the reference's op tests (tests/test_ops/test_convolution_op.py:102-131).
+    Returns idx (nnz, 3), val (nnz,), mix_idx (num_out,).
+    """
+    def make(dim):
+        extra = rng.integers(0, max(dim - 1, 1), size=max(nnz - dim, 0))
+        return np.concatenate([np.arange(dim), extra])[:max(nnz, dim)]
+    n = max(nnz, num_x, num_y, num_out)
+    cols = []
+    for dim in (num_out, num_x, num_y):
+        c = make(dim)
+        if c.shape[0] < n:
+            c = np.concatenate([c, rng.integers(0, dim, size=n - c.shape[0])])
+        cols.append(c[:n])
+    order = np.argsort(cols[0], kind="stable")
+    idx = np.stack(cols, axis=-1)[order]
+    val = rng.normal(size=n).astype(np.float32)
+    mix = np.sort(np.concatenate([np.arange(num_scalars),
+                                  rng.integers(0, num_scalars, size=num_out - num_scalars)]))
+    return idx, val, mix
+
+
+def random_graph(rng, num_nodes, num_edges, sort_by="receiver"):
+    sender = rng.integers(0, num_nodes, size=num_edges).astype(np.int32)
+    receiver = rng.integers(0, num_nodes, size=num_edges).astype(np.int32)
+    if sort_by == "receiver":
+        order = np.argsort(receiver, kind="stable")
+    elif sort_by == "sender":
+        order = np.argsort(sender, kind="stable")
+    else:
+        order = np.arange(num_edges)
+    return sender[order], receiver[order]
+
+
+def random_operands(rng, num_nodes, num_edges, num_x, num_y, num_scalars, channels, num_out,
+                    dtype=np.float32):
+    x = rng.normal(size=(num_nodes, num_x, channels)).astype(dtype)
+    y = rng.normal(size=(num_edges, num_y)).astype(dtype)
+    s = rng.normal(size=(num_edges, num_scalars, channels)).astype(dtype)
+    dm = rng.normal(size=(num_nodes, num_out, channels)).astype(dtype)
+    return x, y, s, dm
+
+
+def pack_table(idx, val, mix_idx, val_dtype=np.float32, idx_dtype=None):
+    from e3j_amd.coef import Coef4D
+    from e3j_amd.sparse import narrow_index_dtype
+    idx = np.asarray(idx)
+    idx4 = np.concatenate([idx, np.asarray(mix_idx)[idx[:, 0]][:, None]], axis=1)
+    if idx_dtype is None:
+        idx_dtype = narrow_index_dtype((int(idx4.max()) + 1,) if idx4.size else (1,))
+    return Coef4D(np.asarray(val), idx4, val_dtype=val_dtype, idx_dtype=idx_dtype).pack()
+
+
+# ---------------------------------------------------------------------------
+# parity criterion
+# ---------------------------------------------------------------------------
+def forward_reference(idx, val, mix, x, y, s, snd, rcv, num_out, leading=False):
+    """float64 value and the sum of absolute terms of every output element."""
+    ref = O.convolution_unfused(idx, val, mix, x, y, s, snd, rcv, num_out, leading=leading,
+                                dtype=np.float64)
+    mag = O.convolution_unfused(idx, np.abs(val), mix, np.abs(x), np.abs(y), np.abs(s), snd, rcv,
+                                num_out, leading=leading, dtype=np.float64)
+    return ref, mag
+
+
+def backward_reference(idx, val, mix, x, y, s, snd, rcv, dm, leading=False):
+    ref = O.convolution_vjp(idx, val, mix, x, y, s, snd, rcv, dm, leading=leading, dtype=np.float64)
+    mag = O.convolution_vjp(idx, np.abs(val), mix, np.abs(x), np.abs(y), np.abs(s), snd, rcv,
+                            np.abs(dm), leading=leading, dtype=np.float64)
+    return ref, mag
+
+
+def assert_parity(result, ref64, mag64, what="", rtol=1e-5, atol=1e-6, ulps=16.0):
+    """|result - ref| <= atol + rtol*|ref| elementwise (1e-5 relative / 1e-6 absolute);
+    an element outside that must lie within `ulps` float32 roundings of the sum of the
+    absolute values of its terms - the float32 summation-order allowance."""
+    result = np.asarray(result, dtype=np.float64)
+    assert result.shape == ref64.shape, f"{what}: shape {result.shape} != {ref64.shape}"
+    assert np.isfinite(result).all(), f"{what}: non-finite values"
+    err = np.abs(result - ref64)
+    ok = (err <= atol + rtol * np.abs(ref64)) | (err <= ulps * EPS32 * mag64)
+    if not ok.all():
+        bad = np.argwhere(~ok)[0]
+        t = tuple(bad)
+        raise AssertionError(
+            f"{what}: {int((~ok).sum())} of {ok.size} elements out of tolerance; first at {t}: "
+            f"got {result[t]!r}, want {ref64[t]!r}, err {err[t]:.3e}, term magnitude {mag64[t]:.3e}")
+
+
+def float32_noise_bound(ref64, mag64, rtol=1e-5, atol=1e-6, ulps=16.0):
+    return np.maximum(atol + rtol * np.abs(ref64), ulps * EPS32 * mag64)
