@@ -12,7 +12,8 @@ import ctypes
 import os
 
 _HERE = os.path.dirname(os.path.abspath(__file__))
-LIB_PATH = os.path.join(_HERE, "lib", "libe3j_amd.so")
+#: E3J_AMD_LIBRARY overrides the in-tree build (e.g. to compare two builds of the kernels).
+LIB_PATH = os.environ.get("E3J_AMD_LIBRARY") or os.path.join(_HERE, "lib", "libe3j_amd.so")
 
 OK, INVALID_ARGUMENT, UNIMPLEMENTED, INTERNAL = 0, 1, 2, 3
 LAYOUT_LEADING, LAYOUT_TRAILING = 0, 1

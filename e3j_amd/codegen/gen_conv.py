@@ -1,0 +1,347 @@
+"""Generator of the compile-time-unrolled convolution kernels.
+
+For one irreps signature (x irreps, y irreps, output filter, channel count) it
+turns the stacked Clebsch-Gordan table into straight-line HIP: every non-zero
+coefficient becomes a fused multiply-add with a literal constant, and nothing
+of the table is read at run time.  This is the gfx950 counterpart of the
+trace-time unrolling of the reference's Pallas kernels
+(`src/e3j/pallas_ops/convolution/mosaic_gpu/fwd.py:162-177`,
+`src/e3j/pallas_ops/utils/coef.py:102-126`); the reference's CUDA kernel walks
+the table at run time instead (`lib/e3j_ops/cuda/convolution/fwd.cuh:88-153`).
+
+Per edge and lane (a lane owns CPL channels; `y` is the same for all lanes):
+
+    p_m      = |c_m| * y[k_m]                      one product per distinct (|c|, k)
+    w_ij     = sum of +-p_m                         the edge's (output, x) weights
+    forward  : msg_i = sum_j w_ij x_j ;  acc_i += s_l(i) msg_i
+    backward : g_i = dm_i s_l(i) ;  dx_j += w_ij g_i ;  ds_l += dm_i sum_j w_ij x_j
+               dy_k += c_ijk * sum_channels(g_i x_j)
+
+`python -m e3j_amd.codegen.gen_conv` rewrites `e3j_amd/csrc/generated/`.
+"""
+
+from __future__ import annotations
+
+import os
+import struct
+from collections import OrderedDict
+
+import numpy as np
+
+from ..options import Layout
+from ..scalar_mixing import ScalarMixing
+from ..tensor_product import TensorProduct
+
+#: Signatures compiled into the library: (name, x irreps, y irreps, output filter, channels).
+#: They are the irreps/channel combinations of the benchmark configurations
+#: (SQRT_DIM_OUT normalisation, the default of `Convolution`).
+BUILTIN_SIGNATURES = [
+    ("l1_l2_to_l2_k32", "0e+1o", "0e+1o+2e", "0e+1o+2e", 32),
+    ("l2_l3_to_l2_k64", "0e+1o+2e", "0e+1o+2e+3o", "0e+1o+2e", 64),
+    ("l2_l3_to_l3_k64", "0e+1o+2e", "0e+1o+2e+3o", "0e+1o+2e+3o", 64),
+    ("l3_l3_to_l3_k64", "0e+1o+2e+3o", "0e+1o+2e+3o", "0e+1o+2e+3o", 64),
+    ("l3_l3_to_l3_k128", "0e+1o+2e+3o", "0e+1o+2e+3o", "0e+1o+2e+3o", 128),
+]
+
+#: launch shapes per channel count: (channels per lane, waves per block) variants for fwd
+#: and bwd.  Variant 0 is the default; the others are selected with the environment
+#: variables E3J_AMD_FWD_VARIANT / E3J_AMD_BWD_VARIANT (read once) for tuning runs.
+LAUNCH = {
+    32: dict(fwd=[(1, 4)], bwd=[(1, 4)]),
+    64: dict(fwd=[(1, 4), (1, 2)], bwd=[(1, 4), (1, 2)]),
+    128: dict(fwd=[(1, 4), (2, 4), (1, 2)], bwd=[(1, 4), (2, 4), (1, 2)]),
+}
+
+
+def _f32_bits(v: float) -> int:
+    return struct.unpack("<I", struct.pack("<f", float(v)))[0]
+
+
+def _lit(v: float) -> str:
+    """Exact float32 literal."""
+    f = np.float32(v)
+    text = repr(float(f))
+    if "e" not in text and "." not in text and "inf" not in text and "nan" not in text:
+        text += ".0"
+    return text + "f"
+
+
+class Table:
+    """A forward table `(val; i, j, k, l)` organised for emission.
+
+    Output coordinates are grouped by their scalar index `l`: one group is one
+    Clebsch-Gordan path (one output irrep copy), whose rows share an x block, a y
+    block and one normalisation, so the products `|c| * y[k]` of a group are few
+    and die with the group.
+    """
+
+    def __init__(self, val, idx4, num_x, num_y, num_out, num_scalars):
+        self.val = np.asarray(val, dtype=np.float32)
+        self.idx = np.asarray(idx4, dtype=np.int64)
+        self.X, self.Y, self.Z, self.S = int(num_x), int(num_y), int(num_out), int(num_scalars)
+        # paths[l] = OrderedDict i -> OrderedDict j -> [(c, k)]
+        self.paths = OrderedDict()
+        row_scalar = {}
+        for v, (i, j, k, l) in zip(self.val, self.idx):
+            if v == 0:
+                continue
+            if row_scalar.setdefault(int(i), int(l)) != int(l):
+                raise ValueError("an output coordinate must map to one scalar")
+            rows = self.paths.setdefault(int(l), OrderedDict())
+            rows.setdefault(int(i), OrderedDict()).setdefault(int(j), []).append((float(v), int(k)))
+
+    @staticmethod
+    def path_products(rows):
+        """Distinct `(|c|, k)` of one path -> local product id, and their definitions."""
+        ids = OrderedDict()
+        for cols in rows.values():
+            for terms in cols.values():
+                for c, k in terms:
+                    ids.setdefault((_f32_bits(abs(c)), k), len(ids))
+        defs = []
+        for (bits, k), m in ids.items():
+            c = struct.unpack("<f", struct.pack("<I", bits))[0]
+            defs.append(f"            const float p{m} = {_lit(c)} * y[{k}];")
+        return ids, defs
+
+    @staticmethod
+    def weight_expr(terms, ids):
+        """C expression of w_ij and whether it is a bare (possibly negated) product."""
+        parts = [(c < 0, ids[(_f32_bits(abs(c)), k)]) for c, k in terms]
+        if len(parts) == 1:
+            neg, m = parts[0]
+            return ("-" if neg else "") + f"p{m}", True
+        expr = ""
+        for n, (neg, m) in enumerate(parts):
+            if n == 0:
+                expr = ("-" if neg else "") + f"p{m}"
+            else:
+                expr += (" - " if neg else " + ") + f"p{m}"
+        return expr, False
+
+    def op_counts(self):
+        """(products, weight adds, (i, j) pairs, coefficients, rows) - VALU work per edge and lane."""
+        prods = sum(len(self.path_products(rows)[0]) for rows in self.paths.values())
+        pairs = sum(len(cols) for rows in self.paths.values() for cols in rows.values())
+        nnz = sum(len(t) for rows in self.paths.values() for cols in rows.values() for t in cols.values())
+        nrows = sum(len(rows) for rows in self.paths.values())
+        return prods, nnz - pairs, pairs, nnz, nrows
+
+
+FENCE = "        __builtin_amdgcn_sched_barrier(0);"
+
+
+def emit_edge_fwd(t: Table) -> list[str]:
+    lines = ["    template <int C>",
+             "    __device__ static __forceinline__ void edge_fwd(const Vec<C> *x, const float *y,",
+             "                                                     const Vec<C> *s, Vec<C> *acc) {"]
+    for l, rows in t.paths.items():
+        ids, defs = Table.path_products(rows)
+        lines.append(f"        {{  // path {l}: rows {min(rows)}..{max(rows)}")
+        lines += defs
+        for i, cols in rows.items():
+            lines.append("            {")
+            first = True
+            for j, terms in cols.items():
+                expr, bare = Table.weight_expr(terms, ids)
+                if not bare:
+                    lines.append(f"                const float w{j} = {expr};")
+                    expr = f"w{j}"
+                if first:
+                    lines.append(f"                Vec<C> m = vmul(x[{j}], {expr});")
+                    first = False
+                else:
+                    lines.append(f"                m = vfma(x[{j}], {expr}, m);")
+            lines.append(f"                acc[{i}] = vfmav(s[{l}], m, acc[{i}]);")
+            lines.append("            }")
+        lines.append("        }")
+        lines.append(FENCE)
+    lines.append("    }")
+    return lines
+
+
+def emit_edge_bwd(t: Table) -> list[str]:
+    lines = ["    // dx, dy: written here (every coordinate); ds rows are stored path by path.",
+             "    template <int C, int K>",
+             "    __device__ static __forceinline__ void edge_bwd(const Vec<C> *x, const float *y,",
+             "                                                     const Vec<C> *s, const Vec<C> *dm,",
+             "                                                     Vec<C> *dx, float *dy, float *ds_row,",
+             "                                                     bool active) {"]
+    dx_init, dy_init, ds_done = set(), set(), set()
+    for l, rows in t.paths.items():
+        ids, defs = Table.path_products(rows)
+        lines.append(f"        {{  // path {l}: rows {min(rows)}..{max(rows)}")
+        lines += defs
+        lines.append("            Vec<C> dsl;")
+        first_ds = True
+        for i, cols in rows.items():
+            lines.append("            {")
+            lines.append(f"                const Vec<C> g = vmulv(dm[{i}], s[{l}]);")
+            first_tp = True
+            for j, terms in cols.items():
+                expr, bare = Table.weight_expr(terms, ids)
+                if not bare:
+                    lines.append(f"                const float w{j} = {expr};")
+                    expr = f"w{j}"
+                if j in dx_init:
+                    lines.append(f"                dx[{j}] = vfma(g, {expr}, dx[{j}]);")
+                else:
+                    lines.append(f"                dx[{j}] = vmul(g, {expr});")
+                    dx_init.add(j)
+                if first_tp:
+                    lines.append(f"                Vec<C> tp = vmul(x[{j}], {expr});")
+                    first_tp = False
+                else:
+                    lines.append(f"                tp = vfma(x[{j}], {expr}, tp);")
+                lines.append(f"                {{ const float h = hsum(vmulv(g, x[{j}]));")
+                for c, k in terms:
+                    if k in dy_init:
+                        lines.append(f"                  dy[{k}] = fmaf(h, {_lit(c)}, dy[{k}]);")
+                    else:
+                        lines.append(f"                  dy[{k}] = h * {_lit(c)};")
+                        dy_init.add(k)
+                lines.append("                }")
+            if first_ds:
+                lines.append(f"                dsl = vmulv(dm[{i}], tp);")
+                first_ds = False
+            else:
+                lines.append(f"                dsl = vfmav(dm[{i}], tp, dsl);")
+            lines.append("            }")
+        lines.append(f"            if (active) store_vec<C>(ds_row + {l} * K, dsl);")
+        ds_done.add(l)
+        lines.append("        }")
+        lines.append(FENCE)
+    # coordinates no coefficient touches get exact zeros
+    for j in range(t.X):
+        if j not in dx_init:
+            lines.append(f"        dx[{j}] = vzero<C>();")
+    for l in range(t.S):
+        if l not in ds_done:
+            lines.append(f"        if (active) store_vec<C>(ds_row + {l} * K, vzero<C>());")
+    for k in range(t.Y):
+        if k not in dy_init:
+            lines.append(f"        dy[{k}] = 0.f;")
+    lines.append("    }")
+    return lines
+
+
+def build_table(x_irreps, y_irreps, out_filter):
+    tp = TensorProduct((x_irreps, y_irreps), out_filter, normalization="SQRT_DIM_OUT")
+    mix = ScalarMixing(tp.target)
+    idx = tp.indices.astype(np.int64)
+    idx4 = np.concatenate([idx, mix.mix_indices[idx[:, 0]][:, None]], axis=1)
+    return Table(tp.values, idx4, tp.source[0].dim, tp.source[1].dim, tp.target.dim, mix.num_irreps), tp
+
+
+def emit_signature(sig_id: int, name: str, x_irreps: str, y_irreps: str, out_filter: str,
+                   channels: int) -> str:
+    t, tp = build_table(x_irreps, y_irreps, out_filter)
+    launch = LAUNCH[channels]
+    struct_name = f"Sig_{name}"
+    vals = ", ".join(_lit(v) for v in t.val)
+    idxs = ", ".join(str(int(a)) for row in t.idx for a in row)
+    desc = (f"{name}: x {tp.source[0]} | y {tp.source[1]} -> {tp.target}, "
+            f"K={channels}, trailing, nnz={len(t.val)}")
+    out = [
+        "// GENERATED by e3j_amd/codegen/gen_conv.py -- do not edit.",
+        f"// {desc}",
+        '#include "../unrolled.h"',
+        "",
+        "namespace e3j_amd {",
+        "namespace {",
+        "",
+        f"struct {struct_name} {{",
+        f"    static constexpr int X = {t.X}, Y = {t.Y}, S = {t.S}, Z = {t.Z};",
+        "",
+    ]
+    out += emit_edge_fwd(t)
+    out.append("")
+    out += emit_edge_bwd(t)
+    out += ["};", "", "}  // namespace", "",
+            "// both passes: the device pass needs the kernels instantiated"]
+    for cpl, wpb in launch["fwd"]:
+        out += [f"template __global__ void unrolled_fwd_kernel<{struct_name}, {channels}, {cpl}, {wpb}>(",
+                "    const float *, const float *, const float *, const int32_t *, const int32_t *,",
+                "    const int32_t *, float *, int, float);"]
+    for cpl, wpb in launch["bwd"]:
+        out += [f"template __global__ void unrolled_bwd_kernel<{struct_name}, {channels}, {cpl}, {wpb}>(",
+                "    const float *, const float *, const float *, const float *, const int32_t *,",
+                "    const int32_t *, const int32_t *, float *, float *, float *, int, float);"]
+    out += ["", "// host pass only: the registry entry holds host function pointers",
+            "#if !defined(__HIP_DEVICE_COMPILE__)",
+            f"static const float kVal[] = {{{vals}}};",
+            f"static const uint8_t kIdx[] = {{{idxs}}};",
+            "",
+            "static int run_fwd(const e3j_amd_conv_params &p, const float *x, const float *y, const float *s,",
+            "                   const int32_t *sender, const int32_t *row_ptr, const int32_t *perm,",
+            "                   float *out, hipStream_t stream) {",
+            "    switch (tuning().fwd_variant) {"]
+    for n, (cpl, wpb) in reversed(list(enumerate(launch["fwd"]))):
+        label = f"case {n}:" if n else "default:"
+        out.append(f"        {label} return launch_unrolled_fwd<{struct_name}, {channels}, {cpl}, {wpb}>("
+                   "p, x, y, s, sender, row_ptr, perm, out, stream);")
+    out += ["    }", "}", "",
+            "static int run_bwd(const e3j_amd_conv_params &p, const float *x, const float *y, const float *s,",
+            "                   const float *dm, const int32_t *sender, const int32_t *row_ptr,",
+            "                   const int32_t *perm, float *dx, float *dy, float *ds, hipStream_t stream) {",
+            "    switch (tuning().bwd_variant) {"]
+    for n, (cpl, wpb) in reversed(list(enumerate(launch["bwd"]))):
+        label = f"case {n}:" if n else "default:"
+        out.append(f"        {label} return launch_unrolled_bwd<{struct_name}, {channels}, {cpl}, {wpb}>("
+                   "p, x, y, s, dm, sender, row_ptr, perm, dx, dy, ds, stream);")
+    out += ["    }", "}", "",
+            f"extern const Signature kSignature_{sig_id} = {{",
+            f'    "{desc}",',
+            f"    {t.X}, {t.Y}, {t.Z}, {t.S}, {len(t.val)}, {channels}, E3J_AMD_LAYOUT_TRAILING, kVal, kIdx,",
+            "    &run_fwd, &run_bwd,",
+            "};",
+            "#endif",
+            "",
+            "}  // namespace e3j_amd",
+            ""]
+    return "\n".join(out)
+
+
+def emit_registry(count: int) -> str:
+    out = ["// GENERATED by e3j_amd/codegen/gen_conv.py -- do not edit.",
+           '#include "../common.h"', "", "namespace e3j_amd {", ""]
+    for n in range(count):
+        out.append(f"extern const Signature kSignature_{n};")
+    out += ["", f"int num_signatures() {{ return {count}; }}", "",
+            "const Signature &signature(int id) {",
+            "    static const Signature *const table[] = {" +
+            ", ".join(f"&kSignature_{n}" for n in range(count)) + (", " if count else "") + "nullptr};",
+            "    return *table[id];", "}", "", "}  // namespace e3j_amd", ""]
+    return "\n".join(out)
+
+
+def _write_if_changed(path: str, text: str) -> None:
+    if os.path.exists(path):
+        with open(path) as fh:
+            if fh.read() == text:
+                return
+    with open(path, "w") as fh:
+        fh.write(text)
+
+
+def write_all(out_dir: str, signatures=None) -> list[str]:
+    signatures = BUILTIN_SIGNATURES if signatures is None else signatures
+    os.makedirs(out_dir, exist_ok=True)
+    wanted = {"registry.hip"}
+    paths = []
+    for n, (name, xi, yi, oi, k) in enumerate(signatures):
+        fname = f"sig_{name}.hip"
+        wanted.add(fname)
+        _write_if_changed(os.path.join(out_dir, fname), emit_signature(n, name, xi, yi, oi, k))
+        paths.append(os.path.join(out_dir, fname))
+    _write_if_changed(os.path.join(out_dir, "registry.hip"), emit_registry(len(signatures)))
+    for stale in os.listdir(out_dir):
+        if stale.endswith(".hip") and stale not in wanted:
+            os.remove(os.path.join(out_dir, stale))
+    return paths
+
+
+if __name__ == "__main__":
+    here = os.path.dirname(os.path.abspath(__file__))
+    for p in write_all(os.path.join(os.path.dirname(here), "csrc", "generated")):
+        print(p)

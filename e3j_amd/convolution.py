@@ -83,7 +83,8 @@ class Convolution:
         return packed
 
     def _fused_eval(self, node_features, edge_features, edge_scalars, senders, receivers):
-        dtype = torch.result_type(torch.result_type(node_features, edge_features), edge_scalars)
+        dtype = torch.promote_types(torch.promote_types(node_features.dtype, edge_features.dtype),
+                                    edge_scalars.dtype)
         val_dtype = resolve_val_dtype(_NP_OF_TORCH.get(dtype, "int64"))
         if val_dtype == "float16":
             raise TypeError("Fused ops support value dtypes ('float32', 'float64'), got 'float16'. "

@@ -1,6 +1,7 @@
 // C-ABI entry points: argument validation, kernel selection, error reporting.
 
 #include <cmath>
+#include <cstdlib>
 #include <cstring>
 
 #include "common.h"
@@ -20,6 +21,16 @@ int set_error(int code, const std::string &msg) {
 int check_hip(hipError_t err, const char *what) {
     if (err == hipSuccess) return E3J_AMD_OK;
     return set_error(E3J_AMD_INTERNAL, std::string(what) + ": " + hipGetErrorString(err));
+}
+
+const Tuning &tuning() {
+    static const Tuning t = [] {
+        Tuning v{0, 0};
+        if (const char *e = std::getenv("E3J_AMD_FWD_VARIANT")) v.fwd_variant = std::atoi(e);
+        if (const char *e = std::getenv("E3J_AMD_BWD_VARIANT")) v.bwd_variant = std::atoi(e);
+        return v;
+    }();
+    return t;
 }
 
 namespace {

@@ -66,6 +66,17 @@ int launch_generic_bwd(const e3j_amd_conv_params &p, bool group_is_receiver, con
                        void *dx, void *dy, void *ds, hipStream_t stream,
                        bool coef_cols_ji = false);
 int launch_fill_zero(void *ptr, size_t bytes, hipStream_t stream);
+// Zero the dy/ds rows of padding edges (float32 operands).
+int launch_zero_padding(const e3j_amd_conv_params &p, const int32_t *other, const int32_t *row_ptr,
+                        const int32_t *perm, float *dy, float *ds, hipStream_t stream);
+
+// Launch-shape variants of the unrolled kernels, from E3J_AMD_FWD_VARIANT /
+// E3J_AMD_BWD_VARIANT (read once; 0 = default).  For tuning runs.
+struct Tuning {
+    int fwd_variant;
+    int bwd_variant;
+};
+const Tuning &tuning();
 
 // Compile-time-unrolled kernels (generated, sig_*.hip) ----------------------
 struct Signature {

@@ -242,6 +242,17 @@ int run_fwd(const e3j_amd_conv_params &p, const void *coef, const void *x, const
     return check_hip(hipGetLastError(), "convolution forward launch");
 }
 
+template <typename Val>
+int zero_padding(const e3j_amd_conv_params &p, const int32_t *other, const int32_t *row_ptr,
+                 const int32_t *perm, Val *dy, Val *ds, hipStream_t stream) {
+    if (p.num_edges == 0) return E3J_AMD_OK;
+    const int64_t zblocks = std::min<int64_t>((p.num_edges + 3) / 4, 4096);
+    hipLaunchKernelGGL(zero_padding_edges_kernel<Val>, dim3((unsigned)zblocks), dim3(kWave, 4), 0,
+                       stream, other, row_ptr, perm, p.num_nodes, p.num_edges, dy, p.num_y, ds,
+                       (int64_t)p.num_scalars * p.channels);
+    return check_hip(hipGetLastError(), "convolution backward padding launch");
+}
+
 template <typename Idx, typename Val>
 int run_bwd(const e3j_amd_conv_params &p, bool group_is_receiver, const void *coef, const void *x,
             const void *y, const void *s, const void *dm, const int32_t *other,
@@ -265,15 +276,8 @@ int run_bwd(const e3j_amd_conv_params &p, bool group_is_receiver, const void *co
         rc = launch_fill_zero(dx, (size_t)p.num_nodes * p.num_x * p.channels * sizeof(Val), stream);
         if (rc) return rc;
     }
-    if (p.num_edges > 0) {
-        const int64_t zblocks = std::min<int64_t>((p.num_edges + 3) / 4, 4096);
-        hipLaunchKernelGGL(zero_padding_edges_kernel<Val>, dim3((unsigned)zblocks), dim3(kWave, 4), 0,
-                           stream, other, row_ptr, perm, p.num_nodes, p.num_edges,
-                           static_cast<Val *>(dy), p.num_y, static_cast<Val *>(ds),
-                           (int64_t)p.num_scalars * p.channels);
-        rc = check_hip(hipGetLastError(), "convolution backward padding launch");
-        if (rc) return rc;
-    }
+    rc = zero_padding<Val>(p, other, row_ptr, perm, static_cast<Val *>(dy), static_cast<Val *>(ds), stream);
+    if (rc) return rc;
 #define E3J_LAUNCH_BWD(FLAG)                                                                      \
     do {                                                                                          \
         auto kernel = generic_bwd_kernel<Idx, Val, FLAG>;                                         \
@@ -309,6 +313,11 @@ int launch_fill_zero(void *ptr, size_t bytes, hipStream_t stream) {
     hipLaunchKernelGGL(fill_zero_kernel, dim3((unsigned)blocks), dim3(256), 0, stream,
                        static_cast<uint32_t *>(ptr), words);
     return check_hip(hipGetLastError(), "fill launch");
+}
+
+int launch_zero_padding(const e3j_amd_conv_params &p, const int32_t *other, const int32_t *row_ptr,
+                        const int32_t *perm, float *dy, float *ds, hipStream_t stream) {
+    return zero_padding<float>(p, other, row_ptr, perm, dy, ds, stream);
 }
 
 #define E3J_DISPATCH(CALL)                                                                  \

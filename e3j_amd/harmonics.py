@@ -1,0 +1,94 @@
+"""Real spherical harmonics of edge vectors, in the convention of the reference.
+
+`Harmonics(l_max)(r)` returns `(..., (l_max+1)^2)` values ordered by degree and,
+within a degree, `m = -l..l`; the harmonic frame maps the physical axes
+`(X, Y, Z)` of the usual definition to the input components `(z, x, y)`, so the
+degree-1 block is proportional to `(x, y, z)` of the input
+(`src/e3j/utils/spherical_harmonics.py:33-38,66-75`).  Normalisations follow
+`src/e3j/core/harmonics.py:25-42`: "integral" (unit L2 norm on the sphere),
+"component" (`|Y^l|^2 = 2l+1`, the default) and "norm" (`|Y^l| = 1`).
+
+The reference builds explicit polynomials with ladder operators; here the same
+functions come from the recurrences of the associated Legendre polynomials and
+of `(X + iY)^m`, written with tensor operations so they run on the GPU and are
+differentiable with respect to the positions.  The values are pinned by the
+closed forms of degrees 0-2, the addition theorem and the Clebsch-Gordan
+coupling of this package, not by the reference's third-party comparison
+(`tests/test_harmonics.py:178-182`), which needs e3nn.
+"""
+
+from __future__ import annotations
+
+import math
+
+import torch
+
+from .spaces import O3Space, harmonics_space
+
+
+def _normalization_factor(l: int, normalization: str) -> float:
+    if normalization == "integral":
+        return 1.0
+    if normalization == "component":
+        return math.sqrt(4.0 * math.pi)
+    if normalization == "norm":
+        return math.sqrt(4.0 * math.pi / (2 * l + 1))
+    raise NotImplementedError(
+        f"We don't support {normalization} normalization for now. "
+        'We only support "integral", "component" and "norm"')
+
+
+class Harmonics:
+    def __init__(self, target: int | str, normalize: bool = False, normalization: str = "component"):
+        self.target = O3Space(target) if isinstance(target, str) else harmonics_space(int(target))
+        self.degrees = [ir.l for mul, ir in self.target for _ in range(mul)]
+        self.normalize = normalize
+        self.normalization = normalization
+        for l in set(self.degrees):
+            _normalization_factor(l, normalization)
+
+    def __call__(self, r: torch.Tensor) -> torch.Tensor:
+        if self.normalize:
+            norm = torch.linalg.vector_norm(r, dim=-1, keepdim=True)
+            r = r / torch.where(norm > 0, norm, torch.ones_like(norm))
+        x_in, y_in, z_in = r[..., 0], r[..., 1], r[..., 2]
+        X, Y, Z = z_in, x_in, y_in           # harmonic frame
+        l_max = max(self.degrees)
+        r2 = X * X + Y * Y + Z * Z           # 1 on the sphere; keeps the polynomials homogeneous
+        # c_m + i s_m = (X + iY)^m
+        c, s = [torch.ones_like(X)], [torch.zeros_like(X)]
+        for m in range(1, l_max + 1):
+            c.append(c[-1] * X - s[-1] * Y)
+            s.append(s[m - 1] * X + c[m - 1] * Y)
+        # q[l][m]: associated Legendre polynomial without the Condon-Shortley phase, divided by
+        # (1 - Z^2)^(m/2) and made homogeneous of degree l - m with r2.
+        q = [[None] * (l + 1) for l in range(l_max + 1)]
+        for m in range(l_max + 1):
+            q[m][m] = torch.full_like(X, float(_double_factorial(2 * m - 1)))
+            if m + 1 <= l_max:
+                q[m + 1][m] = (2 * m + 1) * Z * q[m][m]
+            for l in range(m + 2, l_max + 1):
+                q[l][m] = ((2 * l - 1) * Z * q[l - 1][m] - (l + m - 1) * r2 * q[l - 2][m]) / (l - m)
+        blocks = []
+        for l in self.degrees:
+            scale = _normalization_factor(l, self.normalization)
+            comps = [None] * (2 * l + 1)
+            for m in range(0, l + 1):
+                n_lm = math.sqrt((2 * l + 1) / (4.0 * math.pi)
+                                 * math.factorial(l - m) / math.factorial(l + m))
+                if m == 0:
+                    comps[l] = (scale * n_lm) * q[l][0]
+                else:
+                    f = scale * math.sqrt(2.0) * n_lm
+                    comps[l + m] = f * q[l][m] * c[m]
+                    comps[l - m] = f * q[l][m] * s[m]
+            blocks.append(torch.stack(comps, dim=-1))
+        return torch.cat(blocks, dim=-1)
+
+
+def _double_factorial(n: int) -> int:
+    out = 1
+    while n > 1:
+        out *= n
+        n -= 2
+    return out

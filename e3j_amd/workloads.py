@@ -1,0 +1,212 @@
+"""Synthetic inputs of the benchmark configurations (seeded).
+
+Atoms at uniformly random positions in a cubic box, a radius graph with a 5
+Angstrom cutoff (periodic boxes use the minimum image), spherical harmonics of
+the unit edge vectors as `y`, normal node features and per-edge per-path radial
+weights of variance `1/fan_in`.  Positions and graphs always come from
+`numpy.random.default_rng(seed)`.  The large value arrays come from the same
+generator when the workload is built on the host, and from a seeded
+`torch.Generator` of the device when it is built in GPU memory (the 1M-edge
+configuration holds 11 GB of radial weights; drawing them on the host and
+copying them would take minutes).
+"""
+
+from __future__ import annotations
+
+import dataclasses
+import math
+
+import numpy as np
+import torch
+
+from .convolution import Convolution
+from .harmonics import Harmonics
+
+
+@dataclasses.dataclass
+class Workload:
+    name: str
+    module: Convolution
+    x: torch.Tensor         # (N, X, K)
+    y: torch.Tensor         # (E, Y)
+    s: torch.Tensor         # (E, S, K)
+    dm: torch.Tensor        # (N, Z, K)
+    sender: torch.Tensor    # (E,) int32
+    receiver: torch.Tensor  # (E,) int32
+    positions: np.ndarray
+    box: float
+
+    def to(self, device) -> "Workload":
+        return dataclasses.replace(self, **{f: getattr(self, f).to(device) for f in
+                                            ("x", "y", "s", "dm", "sender", "receiver")})
+
+    def numpy(self) -> dict:
+        """Host copies of the operands, for the CPU checker."""
+        return {f: getattr(self, f).cpu().numpy() for f in ("x", "y", "s", "dm", "sender", "receiver")}
+
+    def table(self):
+        """`(idx (nnz, 3), val, mix_idx)` of the module's coefficient table."""
+        c = self.module.coef
+        idx = np.asarray(c.idx, dtype=np.int64)
+        mix = np.zeros(self.module.target.dim, dtype=np.int64)
+        mix[idx[:, 0]] = idx[:, 3]
+        return idx[:, :3], np.asarray(c.val, dtype=np.float32), self.module._mix.mix_indices
+
+    def head(self, num_receivers: int) -> "Workload":
+        """Sub-problem of the first `num_receivers` receivers' edges (receiver-sorted workloads).
+
+        Senders keep their global indices, so `x` is kept whole.
+        """
+        e = int((self.receiver < num_receivers).sum().item())
+        return dataclasses.replace(self, s=self.s[:e], y=self.y[:e], sender=self.sender[:e],
+                                   receiver=self.receiver[:e])
+
+    @property
+    def num_nodes(self) -> int:
+        return int(self.x.shape[0])
+
+    @property
+    def num_edges(self) -> int:
+        return int(self.y.shape[0])
+
+    @property
+    def channels(self) -> int:
+        return int(self.x.shape[2])
+
+    def algorithmic_bytes(self, sorted_edges: bool = True) -> dict:
+        """Compulsory traffic: each operand element read once, each result written once."""
+        n, e, k = self.num_nodes, self.num_edges, self.channels
+        X, Y, S, Z = (int(t.shape[1]) for t in (self.x, self.y, self.s, self.dm))
+        fwd = 4 * (n * X * k + e * Y + e * S * k + n * Z * k) + 4 * (e + n + 1)
+        bwd = 4 * (2 * n * X * k + 2 * e * Y + 2 * e * S * k + n * Z * k) + 4 * (2 * e + n + 1)
+        if not sorted_edges:
+            fwd += 4 * e
+            bwd += 4 * e
+        return {"fwd": fwd, "bwd": bwd, "fwd_bwd": fwd + bwd}
+
+
+def periodic_box_length(num_atoms: int, neighbours: float, cutoff: float) -> float:
+    """Edge of the cube whose density gives `neighbours` atoms within `cutoff`."""
+    density = neighbours / (4.0 / 3.0 * math.pi * cutoff ** 3)
+    return (num_atoms / density) ** (1.0 / 3.0)
+
+
+def radius_graph(positions: np.ndarray, cutoff: float, box: float | None):
+    """Directed edges `(sender, receiver)` with `|r_s - r_r| < cutoff`, and the vectors r_s - r_r.
+
+    `box`: edge of the periodic cube (minimum image) or None for an open box.
+    Edges come out sorted by receiver, then sender.
+    """
+    from scipy.spatial import cKDTree
+    pos = np.asarray(positions, dtype=np.float64)
+    if box is not None:
+        pos = np.mod(pos, box)
+        tree = cKDTree(pos, boxsize=box)
+    else:
+        tree = cKDTree(pos)
+    pairs = tree.query_pairs(cutoff, output_type="ndarray")
+    a = np.concatenate([pairs[:, 0], pairs[:, 1]])
+    b = np.concatenate([pairs[:, 1], pairs[:, 0]])
+    order = np.lexsort((a, b))
+    sender, receiver = a[order], b[order]
+    vec = pos[sender] - pos[receiver]
+    if box is not None:
+        vec -= box * np.round(vec / box)
+    return sender.astype(np.int32), receiver.astype(np.int32), vec
+
+
+def path_fan_in(module: Convolution) -> np.ndarray:
+    """Number of (x irrep, y irrep) paths feeding each output irrep, per path."""
+    degrees = []
+    for mul, ir in module.target:
+        degrees += [(ir.l, ir.p)] * mul
+    counts = {d: degrees.count(d) for d in set(degrees)}
+    return np.array([counts[d] for d in degrees], dtype=np.float64)
+
+
+def _harmonics(vec: np.ndarray, l_max: int, device) -> torch.Tensor:
+    unit = torch.from_numpy(vec / np.linalg.norm(vec, axis=-1, keepdims=True)).to(device)
+    return Harmonics(l_max, normalization="component")(unit).to(torch.float32)
+
+
+def _normal(shape, seed: int, device) -> torch.Tensor:
+    device = torch.device(device)
+    if device.type == "cpu":
+        return torch.from_numpy(np.random.default_rng(seed).standard_normal(shape, dtype=np.float32))
+    gen = torch.Generator(device=device)
+    gen.manual_seed(seed)
+    return torch.randn(shape, dtype=torch.float32, device=device, generator=gen)
+
+
+def make_workload(name: str, num_atoms: int, x_irreps: str, l_max: int, out_irreps: str,
+                  channels: int, seeds: tuple, *, neighbours: float | None = 30.0,
+                  box: float | None = None, periodic: bool = True, cutoff: float = 5.0,
+                  device="cpu") -> Workload:
+    seed_pos, seed_x, seed_s, seed_dm = seeds
+    if box is None:
+        box = periodic_box_length(num_atoms, neighbours, cutoff)
+    pos = np.random.default_rng(seed_pos).uniform(0.0, box, size=(num_atoms, 3))
+    sender, receiver, vec = radius_graph(pos, cutoff, box if periodic else None)
+    y_irreps = "+".join(f"{l}{'e' if l % 2 == 0 else 'o'}" for l in range(l_max + 1))
+    module = Convolution((x_irreps, y_irreps), out_irreps, graph_ordering="RECEIVER")
+    X, Z, S = module.source[0].dim, module.target.dim, module.params.num_scalars
+    E = sender.shape[0]
+    x = _normal((num_atoms, X, channels), seed_x, device)
+    y = _harmonics(vec, l_max, device)
+    std = torch.from_numpy((1.0 / np.sqrt(path_fan_in(module))).astype(np.float32)).to(device)
+    s = _normal((E, S, channels), seed_s, device)
+    s *= std[None, :, None]
+    dm = _normal((num_atoms, Z, channels), seed_dm, device)
+    return Workload(name, module, x, y, s, dm, torch.from_numpy(sender).to(device),
+                    torch.from_numpy(receiver).to(device), pos, box)
+
+
+def config1(scale: float = 1.0, device="cpu") -> Workload:
+    """1 000 atoms in an open 20 A box, 32 channels, 0e+1o x lmax 2 -> 0e+1o+2e."""
+    n = max(8, int(1000 * scale))
+    return make_workload("cfg1", n, "0e+1o", 2, "0e+1o+2e", 32, (1, 2, 3, 4),
+                         box=20.0 * scale ** (1.0 / 3.0), periodic=False, device=device)
+
+
+def config2(scale: float = 1.0, out_irreps: str = "0e+1o+2e", device="cpu") -> Workload:
+    """5 000 atoms, ~30 neighbours (~150k edges), 64 channels, 0e+1o+2e x lmax 3."""
+    n = max(8, int(5000 * scale))
+    return make_workload("cfg2", n, "0e+1o+2e", 3, out_irreps, 64, (11, 12, 13, 14), device=device)
+
+
+def config3(scale: float = 1.0, channels: int = 128, device="cpu") -> Workload:
+    """32 000 atoms, ~30 neighbours (~1M edges), 128 channels, 0e..3o x lmax 3 -> 0e..3o."""
+    n = max(8, int(32000 * scale))
+    return make_workload("cfg3", n, "0e+1o+2e+3o", 3, "0e+1o+2e+3o", channels, (21, 22, 23, 24),
+                         device=device)
+
+
+def config4(scale: float = 1.0, device="cpu") -> Workload:
+    """Shapes of config 2 with a skewed degree distribution and edges in random order.
+
+    10 % of the atoms (hubs) receive about 120 edges drawn from a pool of 40 % of the
+    atoms, the rest about 20; edge vectors are random unit vectors.
+    """
+    n = max(40, int(5000 * scale))
+    rng = np.random.default_rng(31)
+    hubs = rng.permutation(n)[: n // 10]
+    pool = rng.permutation(n)[: max(4, (4 * n) // 10)]
+    is_hub = np.zeros(n, dtype=bool)
+    is_hub[hubs] = True
+    degree = np.where(is_hub, rng.poisson(120, n), rng.poisson(20, n))
+    receiver = np.repeat(np.arange(n), degree)
+    sender = np.where(is_hub[receiver], pool[rng.integers(0, pool.shape[0], receiver.shape[0])],
+                      rng.integers(0, n, receiver.shape[0]))
+    shuffle = np.random.default_rng(32).permutation(receiver.shape[0])
+    sender, receiver = sender[shuffle].astype(np.int32), receiver[shuffle].astype(np.int32)
+    vec = np.random.default_rng(33).standard_normal((receiver.shape[0], 3))
+    module = Convolution(("0e+1o+2e", "0e+1o+2e+3o"), "0e+1o+2e", graph_ordering="NONE")
+    X, Z, S = module.source[0].dim, module.target.dim, module.params.num_scalars
+    E = sender.shape[0]
+    x = _normal((n, X, 64), 34, device)
+    y = _harmonics(vec, 3, device)
+    std = torch.from_numpy((1.0 / np.sqrt(path_fan_in(module))).astype(np.float32)).to(device)
+    s = _normal((E, S, 64), 35, device) * std[None, :, None]
+    dm = _normal((n, Z, 64), 36, device)
+    return Workload("cfg4", module, x, y, s, dm, torch.from_numpy(sender).to(device),
+                    torch.from_numpy(receiver).to(device), np.zeros((n, 3)), 0.0)
