@@ -43,13 +43,15 @@ BUILTIN_SIGNATURES = [
     ("l3_l3_to_l3_k128", "0e+1o+2e+3o", "0e+1o+2e+3o", "0e+1o+2e+3o", 128),
 ]
 
-#: launch shapes per channel count: (channels per lane, waves per block) variants for fwd
-#: and bwd.  Variant 0 is the default; the others are selected with the environment
-#: variables E3J_AMD_FWD_VARIANT / E3J_AMD_BWD_VARIANT (read once) for tuning runs.
+#: launch shapes per channel count: (channels per lane, waves per block, parts) variants for
+#: fwd and bwd.  `parts` splits the paths of the signature over that many waves.  Variant 0
+#: is the default; the others are selected with the environment variables
+#: E3J_AMD_FWD_VARIANT / E3J_AMD_BWD_VARIANT (read once) for tuning runs.
 LAUNCH = {
-    32: dict(fwd=[(1, 4)], bwd=[(1, 4)]),
-    64: dict(fwd=[(1, 4), (1, 2)], bwd=[(1, 4), (1, 2)]),
-    128: dict(fwd=[(1, 4), (2, 4), (1, 2)], bwd=[(1, 4), (2, 4), (1, 2)]),
+    32: dict(fwd=[(1, 4, 1)], bwd=[(1, 4, 1)]),
+    64: dict(fwd=[(1, 4, 1), (1, 4, 2)], bwd=[(1, 4, 2), (1, 4, 1), (1, 4, 3), (1, 4, 4)]),
+    128: dict(fwd=[(1, 4, 1), (1, 4, 2), (2, 4, 2), (2, 4, 4)],
+              bwd=[(1, 4, 2), (1, 4, 1), (1, 4, 3), (1, 4, 4), (2, 4, 4)]),
 }
 
 
@@ -128,14 +130,71 @@ class Table:
         return prods, nnz - pairs, pairs, nnz, nrows
 
 
-FENCE = "        __builtin_amdgcn_sched_barrier(0);"
+class Part:
+    """A subset of the paths of a table with its local row numbering."""
+
+    def __init__(self, t: Table, paths: list[int], extra_zero_rows=(), extra_zero_paths=()):
+        self.t = t
+        self.paths = OrderedDict((l, t.paths[l]) for l in paths)
+        self.zero_paths = list(extra_zero_paths)      # paths without coefficients: ds = 0
+        z_rows = sorted({i for rows in self.paths.values() for i in rows} | set(extra_zero_rows))
+        x_rows = sorted({j for rows in self.paths.values() for cols in rows.values() for j in cols})
+        self.kZ, self.kX, self.kS = z_rows, x_rows, list(self.paths)
+        self.zi = {i: n for n, i in enumerate(self.kZ)}
+        self.xj = {j: n for n, j in enumerate(self.kX)}
+        self.sl = {l: n for n, l in enumerate(self.kS)}
+
+    def cost(self) -> int:
+        return sum(len(terms) for rows in self.paths.values() for cols in rows.values()
+                   for terms in cols.values())
 
 
-def emit_edge_fwd(t: Table) -> list[str]:
+def split_parts(t: Table, count: int) -> list[Part]:
+    """Split the paths into at most `count` parts that read disjoint sets of x rows.
+
+    Paths are first grouped by the x rows they read (one group per x irrep block), so a
+    part's x gathers and dx scatters are never repeated by another part; the groups are
+    then packed into parts of similar work, largest first.
+    """
+    def path_cost(l):
+        return sum(len(terms) for cols in t.paths[l].values() for terms in cols.values())
+
+    groups = []  # [set of x rows, [paths]]
+    for l, rows in t.paths.items():
+        xs = {j for cols in rows.values() for j in cols}
+        merged = [xs, [l]]
+        rest = []
+        for g in groups:
+            if g[0] & merged[0]:
+                merged = [g[0] | merged[0], g[1] + merged[1]]
+            else:
+                rest.append(g)
+        groups = rest + [merged]
+    groups.sort(key=lambda g: -sum(path_cost(l) for l in g[1]))
+    count = max(1, min(count, len(groups)))
+    bins = [[] for _ in range(count)]
+    load = [0] * count
+    for _, paths in groups:
+        b = load.index(min(load))
+        bins[b] += paths
+        load[b] += sum(path_cost(l) for l in paths)
+    covered_rows = {i for rows in t.paths.values() for i in rows}
+    gap_rows = [i for i in range(t.Z) if i not in covered_rows]
+    gap_paths = [l for l in range(t.S) if l not in t.paths]
+    return [Part(t, sorted(b), gap_rows if n == 0 else (), gap_paths if n == 0 else ())
+            for n, b in enumerate(bins)]
+
+
+def _arr(name: str, values) -> str:
+    body = ", ".join(str(v) for v in values) if values else "0"
+    return f"    static constexpr int {name}[{max(len(values), 1)}] = {{{body}}};"
+
+
+def emit_edge_fwd(p: Part) -> list[str]:
     lines = ["    template <int C>",
              "    __device__ static __forceinline__ void edge_fwd(const Vec<C> *x, const float *y,",
              "                                                     const Vec<C> *s, Vec<C> *acc) {"]
-    for l, rows in t.paths.items():
+    for l, rows in p.paths.items():
         ids, defs = Table.path_products(rows)
         lines.append(f"        {{  // path {l}: rows {min(rows)}..{max(rows)}")
         lines += defs
@@ -148,52 +207,54 @@ def emit_edge_fwd(t: Table) -> list[str]:
                     lines.append(f"                const float w{j} = {expr};")
                     expr = f"w{j}"
                 if first:
-                    lines.append(f"                Vec<C> m = vmul(x[{j}], {expr});")
+                    lines.append(f"                Vec<C> m = vmul(x[{p.xj[j]}], {expr});")
                     first = False
                 else:
-                    lines.append(f"                m = vfma(x[{j}], {expr}, m);")
-            lines.append(f"                acc[{i}] = vfmav(s[{l}], m, acc[{i}]);")
+                    lines.append(f"                m = vfma(x[{p.xj[j]}], {expr}, m);")
+            lines.append(f"                acc[{p.zi[i]}] = vfmav(s[{p.sl[l]}], m, acc[{p.zi[i]}]);")
             lines.append("            }")
         lines.append("        }")
-        lines.append(FENCE)
     lines.append("    }")
     return lines
 
 
-def emit_edge_bwd(t: Table) -> list[str]:
-    lines = ["    // dx, dy: written here (every coordinate); ds rows are stored path by path.",
+def emit_edge_bwd(p: Part) -> list[str]:
+    t = p.t
+    lines = ["    // dx (this part's x rows) and dy (all Y) are written here; ds rows are stored path by path.",
              "    template <int C, int K>",
              "    __device__ static __forceinline__ void edge_bwd(const Vec<C> *x, const float *y,",
              "                                                     const Vec<C> *s, const Vec<C> *dm,",
              "                                                     Vec<C> *dx, float *dy, float *ds_row,",
              "                                                     bool active) {"]
-    dx_init, dy_init, ds_done = set(), set(), set()
-    for l, rows in t.paths.items():
+    dx_init, dy_init = set(), set()
+    for l, rows in p.paths.items():
         ids, defs = Table.path_products(rows)
         lines.append(f"        {{  // path {l}: rows {min(rows)}..{max(rows)}")
         lines += defs
         lines.append("            Vec<C> dsl;")
         first_ds = True
         for i, cols in rows.items():
+            zi = p.zi[i]
             lines.append("            {")
-            lines.append(f"                const Vec<C> g = vmulv(dm[{i}], s[{l}]);")
+            lines.append(f"                const Vec<C> g = vmulv(dm[{zi}], s[{p.sl[l]}]);")
             first_tp = True
             for j, terms in cols.items():
+                xj = p.xj[j]
                 expr, bare = Table.weight_expr(terms, ids)
                 if not bare:
                     lines.append(f"                const float w{j} = {expr};")
                     expr = f"w{j}"
                 if j in dx_init:
-                    lines.append(f"                dx[{j}] = vfma(g, {expr}, dx[{j}]);")
+                    lines.append(f"                dx[{xj}] = vfma(g, {expr}, dx[{xj}]);")
                 else:
-                    lines.append(f"                dx[{j}] = vmul(g, {expr});")
+                    lines.append(f"                dx[{xj}] = vmul(g, {expr});")
                     dx_init.add(j)
                 if first_tp:
-                    lines.append(f"                Vec<C> tp = vmul(x[{j}], {expr});")
+                    lines.append(f"                Vec<C> tp = vmul(x[{xj}], {expr});")
                     first_tp = False
                 else:
-                    lines.append(f"                tp = vfma(x[{j}], {expr}, tp);")
-                lines.append(f"                {{ const float h = hsum(vmulv(g, x[{j}]));")
+                    lines.append(f"                tp = vfma(x[{xj}], {expr}, tp);")
+                lines.append(f"                {{ const float h = hsum(vmulv(g, x[{xj}]));")
                 for c, k in terms:
                     if k in dy_init:
                         lines.append(f"                  dy[{k}] = fmaf(h, {_lit(c)}, dy[{k}]);")
@@ -202,27 +263,33 @@ def emit_edge_bwd(t: Table) -> list[str]:
                         dy_init.add(k)
                 lines.append("                }")
             if first_ds:
-                lines.append(f"                dsl = vmulv(dm[{i}], tp);")
+                lines.append(f"                dsl = vmulv(dm[{zi}], tp);")
                 first_ds = False
             else:
-                lines.append(f"                dsl = vfmav(dm[{i}], tp, dsl);")
+                lines.append(f"                dsl = vfmav(dm[{zi}], tp, dsl);")
             lines.append("            }")
         lines.append(f"            if (active) store_vec<C>(ds_row + {l} * K, dsl);")
-        ds_done.add(l)
         lines.append("        }")
-        lines.append(FENCE)
-    # coordinates no coefficient touches get exact zeros
-    for j in range(t.X):
-        if j not in dx_init:
-            lines.append(f"        dx[{j}] = vzero<C>();")
-    for l in range(t.S):
-        if l not in ds_done:
-            lines.append(f"        if (active) store_vec<C>(ds_row + {l} * K, vzero<C>());")
+    for l in p.zero_paths:  # paths no coefficient touches get exact zeros
+        lines.append(f"        if (active) store_vec<C>(ds_row + {l} * K, vzero<C>());")
     for k in range(t.Y):
         if k not in dy_init:
             lines.append(f"        dy[{k}] = 0.f;")
     lines.append("    }")
     return lines
+
+
+def emit_part(struct_name: str, p: Part) -> list[str]:
+    t = p.t
+    out = [f"struct {struct_name} {{",
+           f"    static constexpr int X = {t.X}, Y = {t.Y}, S = {t.S}, Z = {t.Z};",
+           f"    static constexpr int NX = {len(p.kX)}, NS = {len(p.kS)}, NZ = {len(p.kZ)};",
+           _arr("kX", p.kX), _arr("kS", p.kS), _arr("kZ", p.kZ), ""]
+    out += emit_edge_fwd(p)
+    out.append("")
+    out += emit_edge_bwd(p)
+    out += ["};", ""]
+    return out
 
 
 def build_table(x_irreps, y_irreps, out_filter):
@@ -237,7 +304,6 @@ def emit_signature(sig_id: int, name: str, x_irreps: str, y_irreps: str, out_fil
                    channels: int) -> str:
     t, tp = build_table(x_irreps, y_irreps, out_filter)
     launch = LAUNCH[channels]
-    struct_name = f"Sig_{name}"
     vals = ", ".join(_lit(v) for v in t.val)
     idxs = ", ".join(str(int(a)) for row in t.idx for a in row)
     desc = (f"{name}: x {tp.source[0]} | y {tp.source[1]} -> {tp.target}, "
@@ -250,21 +316,23 @@ def emit_signature(sig_id: int, name: str, x_irreps: str, y_irreps: str, out_fil
         "namespace e3j_amd {",
         "namespace {",
         "",
-        f"struct {struct_name} {{",
-        f"    static constexpr int X = {t.X}, Y = {t.Y}, S = {t.S}, Z = {t.Z};",
-        "",
     ]
-    out += emit_edge_fwd(t)
-    out.append("")
-    out += emit_edge_bwd(t)
-    out += ["};", "", "}  // namespace", "",
-            "// both passes: the device pass needs the kernels instantiated"]
-    for cpl, wpb in launch["fwd"]:
-        out += [f"template __global__ void unrolled_fwd_kernel<{struct_name}, {channels}, {cpl}, {wpb}>(",
+    splits = sorted({v[2] for v in launch["fwd"] + launch["bwd"]})
+    part_names = {}
+    for zs in splits:
+        names = []
+        for n, part in enumerate(split_parts(t, zs)):
+            sname = f"Sig_{name}_z{zs}p{n}"
+            out += emit_part(sname, part)
+            names.append(sname)
+        part_names[zs] = ", ".join(names)
+    out += ["}  // namespace", "", "// both passes: the device pass needs the kernels instantiated"]
+    for cpl, wpb, zs in launch["fwd"]:
+        out += [f"template __global__ void unrolled_fwd_kernel<{channels}, {cpl}, {wpb}, {part_names[zs]}>(",
                 "    const float *, const float *, const float *, const int32_t *, const int32_t *,",
                 "    const int32_t *, float *, int, float);"]
-    for cpl, wpb in launch["bwd"]:
-        out += [f"template __global__ void unrolled_bwd_kernel<{struct_name}, {channels}, {cpl}, {wpb}>(",
+    for cpl, wpb, zs in launch["bwd"]:
+        out += [f"template __global__ void unrolled_bwd_kernel<{channels}, {cpl}, {wpb}, {part_names[zs]}>(",
                 "    const float *, const float *, const float *, const float *, const int32_t *,",
                 "    const int32_t *, const int32_t *, float *, float *, float *, int, float);"]
     out += ["", "// host pass only: the registry entry holds host function pointers",
@@ -276,19 +344,19 @@ def emit_signature(sig_id: int, name: str, x_irreps: str, y_irreps: str, out_fil
             "                   const int32_t *sender, const int32_t *row_ptr, const int32_t *perm,",
             "                   float *out, hipStream_t stream) {",
             "    switch (tuning().fwd_variant) {"]
-    for n, (cpl, wpb) in reversed(list(enumerate(launch["fwd"]))):
+    for n, (cpl, wpb, zs) in reversed(list(enumerate(launch["fwd"]))):
         label = f"case {n}:" if n else "default:"
-        out.append(f"        {label} return launch_unrolled_fwd<{struct_name}, {channels}, {cpl}, {wpb}>("
+        out.append(f"        {label} return launch_unrolled_fwd<{channels}, {cpl}, {wpb}, {part_names[zs]}>("
                    "p, x, y, s, sender, row_ptr, perm, out, stream);")
     out += ["    }", "}", "",
             "static int run_bwd(const e3j_amd_conv_params &p, const float *x, const float *y, const float *s,",
             "                   const float *dm, const int32_t *sender, const int32_t *row_ptr,",
             "                   const int32_t *perm, float *dx, float *dy, float *ds, hipStream_t stream) {",
             "    switch (tuning().bwd_variant) {"]
-    for n, (cpl, wpb) in reversed(list(enumerate(launch["bwd"]))):
+    for n, (cpl, wpb, zs) in reversed(list(enumerate(launch["bwd"]))):
         label = f"case {n}:" if n else "default:"
-        out.append(f"        {label} return launch_unrolled_bwd<{struct_name}, {channels}, {cpl}, {wpb}>("
-                   "p, x, y, s, dm, sender, row_ptr, perm, dx, dy, ds, stream);")
+        out.append(f"        {label} return launch_unrolled_bwd<{channels}, {cpl}, {wpb}, {t.Y}, {t.X}, "
+                   f"{part_names[zs]}>(p, x, y, s, dm, sender, row_ptr, perm, dx, dy, ds, stream);")
     out += ["    }", "}", "",
             f"extern const Signature kSignature_{sig_id} = {{",
             f'    "{desc}",',

@@ -105,74 +105,104 @@ __device__ __forceinline__ void store_vec<4>(float *p, const Vec<4> &a) {
 
 __device__ __forceinline__ int uniform(int v) { return __builtin_amdgcn_readfirstlane(v); }
 
-constexpr int next_pow2_c(int n) { return n <= 1 ? 1 : 2 * next_pow2_c((n + 1) / 2); }
+// Pin a wave-uniform value (scalar register) into a vector register.  A VALU operation
+// reads at most one scalar or literal operand, so `literal * y` with y in a scalar
+// register would make the compiler park every coefficient literal in a vector register
+// for the whole kernel; with y in a vector register the literals stay inline.
+__device__ __forceinline__ float to_vgpr(float v) {
+    asm volatile("" : "+v"(v));
+    return v;
+}
 
-// Sum NV per-lane values over the 64 lanes of a wave.  Halving exchange: at each
-// step a lane keeps one half of its values and receives the partner's partial sums
-// of that half, so NV values cost about 2*NV exchanges instead of 6*NV.  On return
-// the total of value k sits in v[0] of every lane whose `slot(lane)` equals k.
+// Sum NV (<= 16) per-lane values over the 64 lanes of a wave with about 3*NV + 4
+// VALU operations instead of 6*NV exchanges.  Halving exchange: at each of the four
+// in-row steps a lane keeps one half of its values and adds the partner's partial sums
+// of that half.  The partner comes from a DPP row permutation that flips the lane bit of
+// the step and keeps the lower ones (xor 1, xor 2, rotate by 4, rotate by 8 within a row
+// of 16), the half is picked with a bit-field insert under a per-lane
+// mask (never a register-array select, which the compiler would lower to a chain of
+// compares), and two cross-row exchanges finish the sum.  On return every lane holds
+// in v[0] the total of value `slot(lane)`.
 template <int NV>
 struct WaveReduce {
-    static constexpr int P = next_pow2_c(NV) > 64 ? 64 : next_pow2_c(NV);
-    static_assert(NV <= 64, "at most 64 values");
+    static_assert(NV >= 1 && NV <= 16, "at most 16 values");
+    static constexpr int P = 16;  // values are padded to 16 by the caller
     __device__ static __forceinline__ int slot(int lane) {
-        int k = 0;
-        int off = 32;
-#pragma unroll
-        for (int n = P; n > 1; n >>= 1, off >>= 1) k = 2 * k + ((lane & off) ? 1 : 0);
-        return k;
+        return ((lane & 1) << 3) | ((lane & 2) << 1) | ((lane & 4) >> 1) | ((lane & 8) >> 3);
     }
-    // number of low lane bits over which results are replicated
-    static constexpr int replicated() { return 64 / P; }
-    __device__ static __forceinline__ float run(float (&v)[P], int lane) {
-        int off = 32;
+    template <int CTRL>
+    __device__ static __forceinline__ float dpp(float v) {
+        return __int_as_float(__builtin_amdgcn_mov_dpp(__float_as_int(v), CTRL, 0xf, 0xf, true));
+    }
+    // (a where mask is all ones, b where it is zero)
+    __device__ static __forceinline__ float pick(float a, float b, unsigned mask) {
+        return __uint_as_float((__float_as_uint(a) & mask) | (__float_as_uint(b) & ~mask));
+    }
+    template <int CTRL, int N>
+    __device__ static __forceinline__ void level(float (&v)[P], unsigned upper) {
 #pragma unroll
-        for (int n = P; n > 1; n >>= 1, off >>= 1) {
-            const bool upper = (lane & off) != 0;
-#pragma unroll
-            for (int t = 0; t < n / 2; t++) {
-                const float send = upper ? v[t] : v[t + n / 2];
-                const float keep = upper ? v[t + n / 2] : v[t];
-                v[t] = keep + __shfl_xor(send, off, kWave);
-            }
+        for (int t = 0; t < N / 2; t++) {
+            const float keep = pick(v[t + N / 2], v[t], upper);
+            const float send = pick(v[t], v[t + N / 2], upper);
+            v[t] = keep + dpp<CTRL>(send);
         }
-#pragma unroll
-        for (; off > 0; off >>= 1) v[0] += __shfl_xor(v[0], off, kWave);
+    }
+    __device__ static __forceinline__ float run(float (&v)[P], int lane) {
+        level<0xB1, 16>(v, (lane & 1) ? ~0u : 0u);   // quad_perm [1,0,3,2]
+        level<0x4E, 8>(v, (lane & 2) ? ~0u : 0u);    // quad_perm [2,3,0,1]
+        level<0x124, 4>(v, (lane & 4) ? ~0u : 0u);   // row_ror:4 (the source lane differs in bit 2)
+        level<0x128, 2>(v, (lane & 8) ? ~0u : 0u);   // row_ror:8 (= xor 8)
+        v[0] += __shfl_xor(v[0], 16, kWave);
+        v[0] += __shfl_xor(v[0], 32, kWave);
         return v[0];
     }
 };
 
 // ---------------------------------------------------------------------------
+// A generated `Part` covers a subset of the Clebsch-Gordan paths of a signature
+// (all of them when the signature is not split).  It names the rows it touches:
+//   kX[NX]  x coordinates it reads (and whose dx it produces)
+//   kS[NS]  paths: rows of s it reads / of ds it writes
+//   kZ[NZ]  output coordinates it accumulates (rows of out / dm)
+// and supplies edge_fwd / edge_bwd on arrays indexed by those local positions.
+// Splitting a signature over several waves divides the register-resident
+// accumulators (out rows forward, dm rows backward) between them.
+// ---------------------------------------------------------------------------
+
+template <int K, int CPL>
+struct Slice {
+    static constexpr int WIDTH = kWave * CPL;                 // channels per wave
+    static constexpr int COUNT = (K + WIDTH - 1) / WIDTH;     // waves per row
+    static constexpr bool FULL = (K % WIDTH) == 0;            // no idle lanes
+    static_assert(K % CPL == 0, "channels must be a multiple of the per-lane vector width");
+};
+
+// ---------------------------------------------------------------------------
 // forward
 // ---------------------------------------------------------------------------
-template <typename Sig, int K, int CPL, int WPB>
-__global__ __launch_bounds__(kWave *WPB) void unrolled_fwd_kernel(
+template <typename Part, int K, int CPL>
+__device__ __forceinline__ void unrolled_fwd_part(
     const float *__restrict__ x, const float *__restrict__ y, const float *__restrict__ s,
     const int32_t *__restrict__ sender, const int32_t *__restrict__ row_ptr,
-    const int32_t *__restrict__ perm, float *__restrict__ out, int num_nodes, float scale) {
-    constexpr int X = Sig::X, Y = Sig::Y, S = Sig::S, Z = Sig::Z;
-    constexpr int SLICE = kWave * CPL;
-    constexpr int CW = (K + SLICE - 1) / SLICE;
-    static_assert(K % CPL == 0, "channels must be a multiple of the per-lane vector width");
+    const int32_t *__restrict__ perm, float *__restrict__ out, int num_nodes, float scale,
+    int r, int slice, int lane) {
+    constexpr int NX = Part::NX, NS = Part::NS, NZ = Part::NZ, Y = Part::Y;
+    constexpr int X = Part::X, S = Part::S, Z = Part::Z;
     using V = Vec<CPL>;
+    using SL = Slice<K, CPL>;
 
-    const int lane = threadIdx.x;
-    const int item = uniform(blockIdx.x * WPB + threadIdx.y);
-    if (item >= num_nodes * CW) return;
-    const int r = item / CW;
-    const int c_raw = (item % CW) * SLICE + lane * CPL;
-    // every lane owns channels when K fills whole slices: no predication in that case
-    const bool active = (K % SLICE == 0) || c_raw < K;
+    const int c_raw = slice * SL::WIDTH + lane * CPL;
+    const bool active = SL::FULL || c_raw < K;
     const int c0 = active ? c_raw : 0;  // idle lanes read channel 0 and never store
 
-    V acc[Z];
+    V acc[NZ];
 #pragma unroll
-    for (int i = 0; i < Z; i++) acc[i] = vzero<CPL>();
+    for (int i = 0; i < NZ; i++) acc[i] = vzero<CPL>();
 
     int e = row_ptr[r];
     const int e1 = row_ptr[r + 1];
 
-    V xn[X], sn[S];
+    V xn[NX], sn[NS];
     float yn[Y];
     bool valid_n = false;
     auto fetch = [&](int pos) {
@@ -184,64 +214,94 @@ __global__ __launch_bounds__(kWave *WPB) void unrolled_fwd_kernel(
         const float *sr = s + ee * (int64_t)(S * K) + c0;
         const float *yr = y + ee * Y;
 #pragma unroll
-        for (int j = 0; j < X; j++) xn[j] = load_vec<CPL>(xr + j * K);
+        for (int j = 0; j < NX; j++) xn[j] = load_vec<CPL>(xr + Part::kX[j] * K);
 #pragma unroll
-        for (int l = 0; l < S; l++) sn[l] = load_vec<CPL>(sr + l * K);
+        for (int l = 0; l < NS; l++) sn[l] = load_vec<CPL>(sr + Part::kS[l] * K);
 #pragma unroll
         for (int k = 0; k < Y; k++) yn[k] = yr[k];
     };
     if (e < e1) fetch(e);
     while (e < e1) {
-        V xc[X], sc[S];
+        V xc[NX], sc[NS];
         float yc[Y];
 #pragma unroll
-        for (int j = 0; j < X; j++) xc[j] = xn[j];
+        for (int j = 0; j < NX; j++) xc[j] = xn[j];
 #pragma unroll
-        for (int l = 0; l < S; l++) sc[l] = sn[l];
+        for (int l = 0; l < NS; l++) sc[l] = sn[l];
 #pragma unroll
-        for (int k = 0; k < Y; k++) yc[k] = yn[k];
+        for (int k = 0; k < Y; k++) yc[k] = to_vgpr(yn[k]);
         const bool valid = valid_n;
         e++;
         if (e < e1) fetch(e);
-        if (valid) Sig::template edge_fwd<CPL>(xc, yc, sc, acc);
+        if (valid) Part::template edge_fwd<CPL>(xc, yc, sc, acc);
     }
     if (active) {
         float *orow = out + (int64_t)r * (Z * K) + c0;
 #pragma unroll
-        for (int i = 0; i < Z; i++) store_vec<CPL>(orow + i * K, vmul(acc[i], scale));
+        for (int i = 0; i < NZ; i++) store_vec<CPL>(orow + Part::kZ[i] * K, vmul(acc[i], scale));
     }
 }
 
+template <int K, int CPL, int I>
+__device__ __forceinline__ void dispatch_fwd(int, const float *, const float *, const float *,
+                                             const int32_t *, const int32_t *, const int32_t *,
+                                             float *, int, float, int, int, int) {}
+template <int K, int CPL, int I, typename Part, typename... Rest>
+__device__ __forceinline__ void dispatch_fwd(int part, const float *x, const float *y, const float *s,
+                                             const int32_t *sender, const int32_t *row_ptr,
+                                             const int32_t *perm, float *out, int num_nodes,
+                                             float scale, int r, int slice, int lane) {
+    if (part == I)
+        unrolled_fwd_part<Part, K, CPL>(x, y, s, sender, row_ptr, perm, out, num_nodes, scale, r,
+                                        slice, lane);
+    else
+        dispatch_fwd<K, CPL, I + 1, Rest...>(part, x, y, s, sender, row_ptr, perm, out, num_nodes,
+                                             scale, r, slice, lane);
+}
+
+// One wave per (receiver, channel slice, part); consecutive waves share a receiver.
+template <int K, int CPL, int WPB, typename... Parts>
+__global__ __launch_bounds__(kWave *WPB) void unrolled_fwd_kernel(
+    const float *__restrict__ x, const float *__restrict__ y, const float *__restrict__ s,
+    const int32_t *__restrict__ sender, const int32_t *__restrict__ row_ptr,
+    const int32_t *__restrict__ perm, float *__restrict__ out, int num_nodes, float scale) {
+    constexpr int NP = sizeof...(Parts);
+    constexpr int CW = Slice<K, CPL>::COUNT;
+    const int64_t item = (int64_t)blockIdx.x * WPB + threadIdx.y;
+    if (item >= (int64_t)num_nodes * (CW * NP)) return;
+    const int part = uniform((int)(item % NP));
+    const int slice = uniform((int)((item / NP) % CW));
+    const int r = uniform((int)(item / (NP * CW)));
+    dispatch_fwd<K, CPL, 0, Parts...>(part, x, y, s, sender, row_ptr, perm, out, num_nodes, scale, r,
+                                      slice, threadIdx.x);
+}
+
 // ---------------------------------------------------------------------------
-// backward, receiver-grouped: dm row resident, x gathered, dx scattered by atomics
+// backward, receiver-grouped: dm rows resident, x gathered, dx scattered by atomics
 // ---------------------------------------------------------------------------
-template <typename Sig, int K, int CPL, int WPB>
-__global__ __launch_bounds__(kWave *WPB) void unrolled_bwd_kernel(
+template <typename Part, int K, int CPL, bool kAtomicDy>
+__device__ __forceinline__ void unrolled_bwd_part(
     const float *__restrict__ x, const float *__restrict__ y, const float *__restrict__ s,
     const float *__restrict__ dm, const int32_t *__restrict__ sender,
     const int32_t *__restrict__ row_ptr, const int32_t *__restrict__ perm,
     float *__restrict__ dx, float *__restrict__ dy, float *__restrict__ ds, int num_nodes,
-    float scale) {
-    constexpr int X = Sig::X, Y = Sig::Y, S = Sig::S, Z = Sig::Z;
-    constexpr int SLICE = kWave * CPL;
-    constexpr int CW = (K + SLICE - 1) / SLICE;
+    float scale, int r, int slice, int lane) {
+    constexpr int NX = Part::NX, NS = Part::NS, NZ = Part::NZ, Y = Part::Y;
+    constexpr int X = Part::X, S = Part::S, Z = Part::Z;
     using V = Vec<CPL>;
+    using SL = Slice<K, CPL>;
     using Red = WaveReduce<Y>;
 
-    const int lane = threadIdx.x;
-    const int item = uniform(blockIdx.x * WPB + threadIdx.y);
-    if (item >= num_nodes * CW) return;
-    const int r = item / CW;
-    const int c_raw = (item % CW) * SLICE + lane * CPL;
-    const bool active = (K % SLICE == 0) || c_raw < K;
+    const int c_raw = slice * SL::WIDTH + lane * CPL;
+    const bool active = SL::FULL || c_raw < K;
     const int c0 = active ? c_raw : 0;
 
-    V dmr[Z];
+    V dmr[NZ];
     {
         const float *zr = dm + (int64_t)r * (Z * K) + c0;
 #pragma unroll
-        for (int i = 0; i < Z; i++) {
-            dmr[i] = vmul(load_vec<CPL>(zr + i * K), scale);
+        for (int i = 0; i < NZ; i++) {
+            dmr[i] = vmul(load_vec<CPL>(zr + Part::kZ[i] * K), scale);
             if (!active) dmr[i] = vzero<CPL>();  // idle lanes must add nothing to dy
         }
     }
@@ -249,7 +309,7 @@ __global__ __launch_bounds__(kWave *WPB) void unrolled_bwd_kernel(
     int e = row_ptr[r];
     const int e1 = row_ptr[r + 1];
 
-    V xn[X], sn[S];
+    V xn[NX], sn[NS];
     float yn[Y];
     bool valid_n = false;
     int snd_n = 0;
@@ -263,22 +323,22 @@ __global__ __launch_bounds__(kWave *WPB) void unrolled_bwd_kernel(
         const float *sr = s + ee_n * (int64_t)(S * K) + c0;
         const float *yr = y + ee_n * Y;
 #pragma unroll
-        for (int j = 0; j < X; j++) xn[j] = load_vec<CPL>(xr + j * K);
+        for (int j = 0; j < NX; j++) xn[j] = load_vec<CPL>(xr + Part::kX[j] * K);
 #pragma unroll
-        for (int l = 0; l < S; l++) sn[l] = load_vec<CPL>(sr + l * K);
+        for (int l = 0; l < NS; l++) sn[l] = load_vec<CPL>(sr + Part::kS[l] * K);
 #pragma unroll
         for (int k = 0; k < Y; k++) yn[k] = yr[k];
     };
     if (e < e1) fetch(e);
     while (e < e1) {
-        V xc[X], sc[S];
+        V xc[NX], sc[NS];
         float yc[Y];
 #pragma unroll
-        for (int j = 0; j < X; j++) xc[j] = xn[j];
+        for (int j = 0; j < NX; j++) xc[j] = xn[j];
 #pragma unroll
-        for (int l = 0; l < S; l++) sc[l] = sn[l];
+        for (int l = 0; l < NS; l++) sc[l] = sn[l];
 #pragma unroll
-        for (int k = 0; k < Y; k++) yc[k] = yn[k];
+        for (int k = 0; k < Y; k++) yc[k] = to_vgpr(yn[k]);
         const bool valid = valid_n;
         const int snd = snd_n;
         const int64_t ee = ee_n;
@@ -286,61 +346,98 @@ __global__ __launch_bounds__(kWave *WPB) void unrolled_bwd_kernel(
         if (e < e1) fetch(e);
         if (!valid) continue;  // padding edge: its dy/ds rows are zero-filled separately
 
-        V dxe[X];
+        V dxe[NX];
         float dye[Red::P];
-        Sig::template edge_bwd<CPL, K>(xc, yc, sc, dmr, dxe, dye, ds + ee * (int64_t)(S * K) + c0,
-                                       active);
+        Part::template edge_bwd<CPL, K>(xc, yc, sc, dmr, dxe, dye, ds + ee * (int64_t)(S * K) + c0,
+                                        active);
 #pragma unroll
         for (int k = Y; k < Red::P; k++) dye[k] = 0.f;
 
         if (active) {
             float *dxr = dx + (int64_t)snd * (X * K) + c0;
 #pragma unroll
-            for (int j = 0; j < X; j++) {
+            for (int j = 0; j < NX; j++) {
 #pragma unroll
-                for (int t = 0; t < CPL; t++) unsafeAtomicAdd(dxr + j * K + t, dxe[j].v[t]);
+                for (int t = 0; t < CPL; t++) unsafeAtomicAdd(dxr + Part::kX[j] * K + t, dxe[j].v[t]);
             }
         }
         const float total = Red::run(dye, lane);
         const int k = Red::slot(lane);
-        if ((lane & (Red::replicated() - 1)) == 0 && k < Y) {
-            if (CW == 1) dy[ee * Y + k] = total;
-            else unsafeAtomicAdd(dy + ee * Y + k, total);  // dy zero-filled by the launcher
+        if (lane < 16 && k < Y) {
+            if (kAtomicDy) unsafeAtomicAdd(dy + ee * Y + k, total);  // dy zero-filled by the launcher
+            else dy[ee * Y + k] = total;
         }
     }
 }
 
-template <typename Sig, int K, int CPL, int WPB>
+template <int K, int CPL, bool A, int I>
+__device__ __forceinline__ void dispatch_bwd(int, const float *, const float *, const float *,
+                                             const float *, const int32_t *, const int32_t *,
+                                             const int32_t *, float *, float *, float *, int, float,
+                                             int, int, int) {}
+template <int K, int CPL, bool A, int I, typename Part, typename... Rest>
+__device__ __forceinline__ void dispatch_bwd(int part, const float *x, const float *y, const float *s,
+                                             const float *dm, const int32_t *sender,
+                                             const int32_t *row_ptr, const int32_t *perm, float *dx,
+                                             float *dy, float *ds, int num_nodes, float scale, int r,
+                                             int slice, int lane) {
+    if (part == I)
+        unrolled_bwd_part<Part, K, CPL, A>(x, y, s, dm, sender, row_ptr, perm, dx, dy, ds, num_nodes,
+                                           scale, r, slice, lane);
+    else
+        dispatch_bwd<K, CPL, A, I + 1, Rest...>(part, x, y, s, dm, sender, row_ptr, perm, dx, dy, ds,
+                                                num_nodes, scale, r, slice, lane);
+}
+
+template <int K, int CPL, int WPB, typename... Parts>
+__global__ __launch_bounds__(kWave *WPB)
+void unrolled_bwd_kernel(
+    const float *__restrict__ x, const float *__restrict__ y, const float *__restrict__ s,
+    const float *__restrict__ dm, const int32_t *__restrict__ sender,
+    const int32_t *__restrict__ row_ptr, const int32_t *__restrict__ perm,
+    float *__restrict__ dx, float *__restrict__ dy, float *__restrict__ ds, int num_nodes,
+    float scale) {
+    constexpr int NP = sizeof...(Parts);
+    constexpr int CW = Slice<K, CPL>::COUNT;
+    constexpr bool kAtomicDy = NP * CW > 1;  // several waves add into one dy row
+    const int64_t item = (int64_t)blockIdx.x * WPB + threadIdx.y;
+    if (item >= (int64_t)num_nodes * (CW * NP)) return;
+    const int part = uniform((int)(item % NP));
+    const int slice = uniform((int)((item / NP) % CW));
+    const int r = uniform((int)(item / (NP * CW)));
+    dispatch_bwd<K, CPL, kAtomicDy, 0, Parts...>(part, x, y, s, dm, sender, row_ptr, perm, dx, dy, ds,
+                                                 num_nodes, scale, r, slice, threadIdx.x);
+}
+
+template <int K, int CPL, int WPB, typename... Parts>
 int launch_unrolled_fwd(const e3j_amd_conv_params &p, const float *x, const float *y, const float *s,
                         const int32_t *sender, const int32_t *row_ptr, const int32_t *perm,
                         float *out, hipStream_t stream) {
-    constexpr int CW = (K + kWave * CPL - 1) / (kWave * CPL);
-    const int64_t items = (int64_t)p.num_nodes * CW;
-    const int64_t blocks = (items + WPB - 1) / WPB;
+    constexpr int64_t PER_NODE = (int64_t)Slice<K, CPL>::COUNT * sizeof...(Parts);
+    const int64_t blocks = ((int64_t)p.num_nodes * PER_NODE + WPB - 1) / WPB;
     if (blocks > 0x7fffffffLL) return set_error(E3J_AMD_INVALID_ARGUMENT, "convolution: grid too large");
-    hipLaunchKernelGGL((unrolled_fwd_kernel<Sig, K, CPL, WPB>), dim3((unsigned)blocks),
+    hipLaunchKernelGGL((unrolled_fwd_kernel<K, CPL, WPB, Parts...>), dim3((unsigned)blocks),
                        dim3(kWave, WPB), 0, stream, x, y, s, sender, row_ptr, perm, out,
                        p.num_nodes, p.coef_scale);
     return check_hip(hipGetLastError(), "convolution forward launch");
 }
 
-template <typename Sig, int K, int CPL, int WPB>
+template <int K, int CPL, int WPB, int Y, int X, typename... Parts>
 int launch_unrolled_bwd(const e3j_amd_conv_params &p, const float *x, const float *y, const float *s,
                         const float *dm, const int32_t *sender, const int32_t *row_ptr,
                         const int32_t *perm, float *dx, float *dy, float *ds, hipStream_t stream) {
-    constexpr int CW = (K + kWave * CPL - 1) / (kWave * CPL);
-    int rc = launch_fill_zero(dx, sizeof(float) * (size_t)p.num_nodes * Sig::X * K, stream);
+    constexpr int64_t PER_NODE = (int64_t)Slice<K, CPL>::COUNT * sizeof...(Parts);
+    int rc = launch_fill_zero(dx, sizeof(float) * (size_t)p.num_nodes * X * K, stream);
     if (rc) return rc;
-    if (CW > 1) {
-        rc = launch_fill_zero(dy, sizeof(float) * (size_t)p.num_edges * Sig::Y, stream);
+    if (PER_NODE > 1) {
+        rc = launch_fill_zero(dy, sizeof(float) * (size_t)p.num_edges * Y, stream);
         if (rc) return rc;
     }
     rc = launch_zero_padding(p, sender, row_ptr, perm, dy, ds, stream);
     if (rc) return rc;
-    const int64_t items = (int64_t)p.num_nodes * CW;
-    const int64_t blocks = (items + WPB - 1) / WPB;
+    const int64_t blocks = ((int64_t)p.num_nodes * PER_NODE + WPB - 1) / WPB;
     if (blocks > 0x7fffffffLL) return set_error(E3J_AMD_INVALID_ARGUMENT, "convolution_bwd: grid too large");
-    hipLaunchKernelGGL((unrolled_bwd_kernel<Sig, K, CPL, WPB>), dim3((unsigned)blocks),
+    hipLaunchKernelGGL((unrolled_bwd_kernel<K, CPL, WPB, Parts...>), dim3((unsigned)blocks),
                        dim3(kWave, WPB), 0, stream, x, y, s, dm, sender, row_ptr, perm, dx, dy, ds,
                        p.num_nodes, p.coef_scale);
     return check_hip(hipGetLastError(), "convolution backward launch");
