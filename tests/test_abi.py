@@ -1,0 +1,182 @@
+"""The C-ABI library: exports, argument validation and XLA-FFI frame decoding (no kernel launch)."""
+
+import ctypes as C
+import os
+import re
+
+import numpy as np
+import pytest
+
+from e3j_amd import Convolution, _lib
+from tests.xla_frame import ERR_INVALID_ARGUMENT, ERR_UNIMPLEMENTED, F32, F64, S32, U8, FakeXla
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+
+
+def _params(**kw):
+    base = dict(num_nodes=4, num_edges=6, num_coef=3, num_x=2, num_y=3, num_out=2, num_scalars=1,
+                channels=8, layout=1, val_dtype=0, coef_idx_bytes=1, signature=-1, coef_scale=1.0, debug=0)
+    base.update(kw)
+    return _lib.ConvParams(**base)
+
+
+def test_every_declared_symbol_is_exported():
+    header = open(os.path.join(ROOT, "include", "e3j_amd.h")).read()
+    declared = set(re.findall(r"\b(e3j_amd_[a-z0-9_]+)\s*\(", header))
+    assert declared == set(_lib.SYMBOLS), "binding table and header disagree"
+    lib = _lib.load()
+    for name in declared:
+        assert getattr(lib, name) is not None
+    assert lib.e3j_amd_version().startswith(b"e3j_amd")
+
+
+def test_params_struct_matches_header():
+    header = open(os.path.join(ROOT, "include", "e3j_amd.h")).read()
+    body = re.search(r"typedef struct e3j_amd_conv_params \{(.*?)\} e3j_amd_conv_params;", header, re.S).group(1)
+    fields = re.findall(r"^\s*(int32_t|int64_t|float)\s+(\w+);", body, re.M)
+    assert [name for _, name in fields] == [name for name, _ in _lib.ConvParams._fields_]
+    ctype = {"int32_t": C.c_int32, "int64_t": C.c_int64, "float": C.c_float}
+    assert [ctype[t] for t, _ in fields] == [t for _, t in _lib.ConvParams._fields_]
+
+
+@pytest.mark.parametrize("kw, code, needle", [
+    (dict(layout=7), _lib.INVALID_ARGUMENT, "unknown layout"),
+    (dict(channels=0), _lib.INVALID_ARGUMENT, "must be >= 1"),
+    (dict(val_dtype=5), _lib.INVALID_ARGUMENT, "unsupported (IDX, VAL) dtype pair"),
+    (dict(coef_idx_bytes=2), _lib.INVALID_ARGUMENT, "unsupported (IDX, VAL) dtype pair"),
+    (dict(num_edges=-1), _lib.INVALID_ARGUMENT, "negative size"),
+    (dict(signature=10_000), _lib.INVALID_ARGUMENT, "unknown signature"),
+    (dict(), _lib.INVALID_ARGUMENT, "null operand"),
+])
+def test_forward_argument_errors(kw, code, needle):
+    lib = _lib.load()
+    p = _params(**kw)
+    rc = lib.e3j_amd_convolution_fwd(C.byref(p), None, None, None, None, None, None, None, None, None)
+    assert rc == code
+    message = lib.e3j_amd_last_error().decode()
+    assert needle in message and message.startswith("E3J_AMD_ERROR[")
+    with pytest.raises(_lib.E3jAmdError, match=re.escape(needle)):
+        _lib.check(rc)
+
+
+def test_null_params_and_backward_errors():
+    lib = _lib.load()
+    assert lib.e3j_amd_convolution_fwd(None, *([None] * 9)) == _lib.INVALID_ARGUMENT
+    p = _params()
+    for fn in (lib.e3j_amd_convolution_bwd_sender, lib.e3j_amd_convolution_bwd_receiver):
+        assert fn(C.byref(p), *([None] * 12)) == _lib.INVALID_ARGUMENT
+        assert "null operand" in lib.e3j_amd_last_error().decode()
+    # mismatching shapes for a built-in signature
+    p = _params(signature=0)
+    assert lib.e3j_amd_convolution_fwd(C.byref(p), *([None] * 9)) == _lib.INVALID_ARGUMENT
+    assert "do not match signature" in lib.e3j_amd_last_error().decode()
+
+
+def test_empty_problem_is_a_no_op():
+    lib = _lib.load()
+    p = _params(num_nodes=0, num_edges=0)
+    assert lib.e3j_amd_convolution_fwd(C.byref(p), *([None] * 9)) == _lib.OK
+    assert lib.e3j_amd_convolution_bwd_receiver(C.byref(p), *([None] * 12)) == _lib.OK
+
+
+def test_graph_entry_point_errors():
+    lib = _lib.load()
+    assert lib.e3j_amd_csr_row_ptr(None, -1, 4, None, None, None) == _lib.INVALID_ARGUMENT
+    assert lib.e3j_amd_sort_edges(None, None, 4, 4, None, None, None, None, None) == _lib.INVALID_ARGUMENT
+    assert lib.e3j_amd_csr_workspace_bytes(1000, 100000) > 0
+
+
+def test_find_signature_matches_benchmark_tables():
+    lib = _lib.load()
+    assert lib.e3j_amd_num_signatures() >= 5
+    module = Convolution(("0e+1o+2e+3o", "0e+1o+2e+3o"), "0e+1o+2e+3o", graph_ordering="RECEIVER")
+    packed = module._packed_coef("float32")
+    scale = C.c_float(0)
+
+    def find(buf, channels, idx_bytes=1, layout=1):
+        return lib.e3j_amd_find_signature(buf.ctypes.data, idx_bytes, _lib.F32, buf.shape[0], 16, 16, 99, 23,
+                                          channels, layout, C.byref(scale))
+    sig = find(packed, 128)
+    assert sig >= 0 and scale.value == 1.0
+    assert b"K=128" in lib.e3j_amd_signature_name(sig)
+    assert find(packed, 64) >= 0 and find(packed, 64) != sig
+    assert find(packed, 256) == -1                       # no kernel built for 256 channels
+    assert find(packed, 128, layout=0) == -1             # leading layout: table-driven kernel
+    # int32 indices describe the same table
+    from e3j_amd.coef import Coef4D
+    c = module.coef
+    wide = Coef4D(c.val, c.idx, "float32", "int32").pack()
+    assert find(wide, 128, idx_bytes=4) == sig
+    # a uniform positive factor is recognised and returned
+    scaled = Convolution(("0e+1o+2e+3o", "0e+1o+2e+3o"), "0e+1o+2e+3o", graph_ordering="RECEIVER",
+                         avg_num_neighbors=12.5)._packed_coef("float32")
+    assert find(scaled, 128) == sig and abs(scale.value - 0.08) < 1e-7
+    # one changed value or index breaks the match
+    broken = packed.copy()
+    broken[5, 4] ^= 1
+    assert find(broken, 128) == -1
+    v = packed.copy().view(np.uint8)
+    c2 = Coef4D(c.val.copy(), c.idx, "float32", "uint8")
+    c2.val[7] *= 1.001
+    assert find(c2.pack(), 128) == -1
+
+
+# --- XLA-FFI handlers -----------------------------------------------------------------
+def test_xla_metadata_query():
+    lib = _lib.load()
+    for handler in (lib.e3j_amd_xla_convolution, lib.e3j_amd_xla_convolution_bwd,
+                    lib.e3j_amd_xla_convolution_bwd_receiver):
+        xla = FakeXla()
+        frame, md = xla.metadata_frame()
+        assert handler(C.addressof(frame)) is None
+        assert (md.api_version.major_version, md.api_version.minor_version) == (0, 2)
+        assert md.traits == 0 and md.state_type_id == 0
+        assert not xla.errors
+
+
+def _conv_frame(xla, *, x_dtype=F32, coef_dtype=U8, y_dims=(6, 3), n_attr=4, drop=None, channels=8):
+    bufs = dict(coef=xla.buffer(coef_dtype, 0x1000, (3, 8)), x=xla.buffer(x_dtype, 0x2000, (4, 2, channels)),
+                y=xla.buffer(F32, 0x3000, y_dims), s=xla.buffer(F32, 0x4000, (6, 1, channels)),
+                sender=xla.buffer(S32, 0x5000, (6,)), ptr=xla.buffer(S32, 0x6000, (5,)),
+                ranges=xla.buffer(S32, 0x7000, (1,)))
+    out = xla.buffer(F32, 0x8000, (4, 2, channels))
+    attrs = {"num_nodes": (S32, C.c_int32(n_attr)), "debug": (S32, C.c_int32(0))}
+    if drop:
+        attrs.pop(drop)
+    return xla.frame(list(bufs.values()), [out], attrs)
+
+
+@pytest.mark.parametrize("kw, code, needle", [
+    (dict(x_dtype=10), ERR_INVALID_ARGUMENT, "unsupported (IDX, VAL) dtype pair"),
+    (dict(coef_dtype=F32), ERR_INVALID_ARGUMENT, "unsupported (IDX, VAL) dtype pair"),
+    (dict(y_dims=(6, 3, 2)), ERR_UNIMPLEMENTED, "RHS y should have only one channel"),
+    (dict(n_attr=5), ERR_INVALID_ARGUMENT, "num_nodes rows"),
+    (dict(drop="num_nodes"), ERR_INVALID_ARGUMENT, "num_nodes (i32) is required"),
+])
+def test_xla_forward_decoding_errors(kw, code, needle):
+    lib = _lib.load()
+    xla = FakeXla()
+    frame = _conv_frame(xla, **kw)
+    err = lib.e3j_amd_xla_convolution(C.addressof(frame))
+    assert err is not None and len(xla.errors) == 1
+    assert xla.errors[0][0] == code and needle in xla.errors[0][1]
+
+
+def test_xla_wrong_operand_count_and_stage():
+    lib = _lib.load()
+    xla = FakeXla()
+    frame = xla.frame([xla.buffer(U8, 0x1000, (3, 8))], [], {"num_nodes": (S32, C.c_int32(4))})
+    assert lib.e3j_amd_xla_convolution(C.addressof(frame)) is not None
+    assert "expected 6 to 8 operands" in xla.errors[-1][1]
+    assert lib.e3j_amd_xla_convolution_bwd(C.addressof(frame)) is not None
+    assert "expected 8 or 9 operands" in xla.errors[-1][1]
+    # stages other than EXECUTE are accepted and ignored
+    frame = xla.frame([], [], {}, stage=1)
+    assert lib.e3j_amd_xla_convolution(C.addressof(frame)) is None
+
+
+def test_missing_library_fails_loudly(monkeypatch, tmp_path):
+    monkeypatch.setattr(_lib, "_lib", None)
+    monkeypatch.setattr(_lib, "LIB_PATH", str(tmp_path / "absent.so"))
+    with pytest.raises(ImportError, match="no fallback"):
+        _lib.load()

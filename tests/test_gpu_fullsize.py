@@ -1,0 +1,78 @@
+"""Full-size benchmark workloads: comparison with the C checker where it finishes in
+seconds, and size-independent properties at the 1M-edge configuration."""
+
+import numpy as np
+import pytest
+import torch
+
+import e3j_amd
+from e3j_amd import workloads as W
+from oracle import c_oracle
+from tests import helpers as H
+
+pytestmark = pytest.mark.gpu
+
+
+def _run(w, ordering=None):
+    m = w.module
+    coef = m._packed_coef("float32")
+    ordering = ordering or m.graph_ordering
+    out = e3j_amd.convolution(coef, w.x, w.y, w.s, w.sender, w.receiver, m.params, ordering)
+    grads = e3j_amd.convolution_bwd(coef, w.x, w.y, w.s, w.sender, w.receiver, w.dm, m.params, ordering)
+    return out, grads
+
+
+def _against_c_oracle(w, out, grads, tag):
+    """float32 C checker + float32 noise bound from the term magnitudes (|.| inputs through the same code)."""
+    idx, val, mix = w.table()
+    a = w.numpy()
+    Z = w.module.params.num_out
+    args = (a["x"], a["y"], a["s"], a["sender"], a["receiver"])
+    mag_args = tuple(np.abs(t) for t in args[:3]) + args[3:]
+    ref = c_oracle.convolution(idx, val, mix, *args, Z)
+    mag = c_oracle.convolution(idx, np.abs(val), mix, *mag_args, Z)
+    H.assert_parity(out.cpu().numpy(), ref.astype(np.float64), 2.0 * mag.astype(np.float64), f"{tag} out", ulps=32.0)
+    refs = c_oracle.convolution_vjp(idx, val, mix, *args, a["dm"])
+    mags = c_oracle.convolution_vjp(idx, np.abs(val), mix, *mag_args, np.abs(a["dm"]))
+    for g, r, m, name in zip(grads, refs, mags, ("dx", "dy", "ds")):
+        H.assert_parity(g.cpu().numpy(), r.astype(np.float64), 2.0 * m.astype(np.float64), f"{tag} {name}", ulps=32.0)
+
+
+def test_config1_and_config2_full_size_match_checker():
+    for w in (W.config1(device="cuda"), W.config2(device="cuda")):
+        out, grads = _run(w)
+        _against_c_oracle(w, out, grads, w.name)
+
+
+def test_config4_unsorted_skewed_matches_checker():
+    """Random edge order and hubs with ~120 incoming edges, through the device sort."""
+    w = W.config4(device="cuda")
+    assert w.module.graph_ordering.value == "NONE"
+    assert not bool((w.receiver[1:] >= w.receiver[:-1]).all())
+    out, grads = _run(w)
+    _against_c_oracle(w, out, grads, "cfg4")
+
+
+def test_config3_full_size_properties():
+    """32 000 atoms, ~0.96 M edges, 128 channels: properties that need no CPU reference."""
+    w = W.config3(device="cuda")
+    assert 0.9e6 < w.num_edges < 1.05e6
+    out, (dx, dy, ds) = _run(w)
+    # Euler's identity of a trilinear form: <x,dx> = <y,dy> = <s,ds> = <out,dm>
+    total = float((out.double() * w.dm.double()).sum())
+    for a, g, name in ((w.x, dx, "x"), (w.y, dy, "y"), (w.s, ds, "s")):
+        assert abs(float((a.double() * g.double()).sum()) - total) <= 2e-5 * abs(total), name
+    # linearity in x and in s
+    out2, _ = _run(W.Workload(**{**w.__dict__, "x": 2.0 * w.x}))
+    torch.testing.assert_close(out2, 2.0 * out, rtol=1e-6, atol=1e-5)
+    # the forward is bit-reproducible
+    again, _ = _run(w)
+    assert torch.equal(out, again)
+    # a head of the workload agrees with the C checker
+    head = w.head(64)
+    idx, val, mix = w.table()
+    a = head.numpy()
+    ref = c_oracle.convolution(idx, val, mix, a["x"], a["y"], a["s"], a["sender"], a["receiver"],
+                               w.module.params.num_out)
+    got = out[:64].cpu().numpy()
+    assert np.abs(got - ref[:64]).max() <= 2e-5 * np.abs(ref[:64]).max()

@@ -104,3 +104,137 @@ def test_random_table_fwd_bwd(channels, grouping):
     x, y, s, dm = H.random_operands(rng, N, E, X, Y, S, channels, Z)
     res = run_abi(idx, val, mix, x, y, s, dm, snd, rcv, Z, grouping=grouping)
     check_all(idx, val, mix, x, y, s, dm, snd, rcv, Z, res, tag=f"K={channels} {grouping}")
+
+
+# ---------------------------------------------------------------------------
+# layouts, dtypes, index widths
+# ---------------------------------------------------------------------------
+@pytest.mark.parametrize("dtype", [np.float32, np.float64])
+@pytest.mark.parametrize("leading", [False, True])
+@pytest.mark.parametrize("idx_dtype", [np.uint8, np.int32])
+def test_layout_dtype_grid(dtype, leading, idx_dtype):
+    rng = np.random.default_rng(7)
+    N, E, X, Y, Z, S, K, nnz = 9, 40, 5, 7, 6, 4, 24, 60
+    idx, val, mix = H.random_table(rng, nnz, X, Y, Z, S)
+    snd, rcv = H.random_graph(rng, N, E)
+    x, y, s, dm = H.random_operands(rng, N, E, X, Y, S, K, Z, dtype=dtype)
+    args = [a.swapaxes(1, 2).copy() if leading else a for a in (x, s, dm)]
+    out, dx, dy, ds = run_abi(idx, val, mix, args[0], y, args[1], args[2], snd, rcv, Z, leading=leading,
+                              dtype=dtype, idx_dtype=idx_dtype)
+    ref, mag = H.forward_reference(idx, val, mix, args[0], y, args[1], snd, rcv, Z, leading=leading)
+    (rx, ry, rs), (mx, my, ms) = H.backward_reference(idx, val, mix, args[0], y, args[1], snd, rcv,
+                                                      args[2], leading=leading)
+    tol = dict(rtol=1e-5, atol=1e-6) if dtype == np.float32 else dict(rtol=1e-12, atol=1e-12, ulps=0.0)
+    for got, r, m, name in ((out, ref, mag, "out"), (dx, rx, mx, "dx"), (dy, ry, my, "dy"), (ds, rs, ms, "ds")):
+        H.assert_parity(got, r, m, f"{name} leading={leading} {np.dtype(dtype).name}", **tol)
+
+
+# scalar irreps at 4096 / vector edges at 8192 channels (tests/test_ops/test_convolution_op.py:257-301)
+@pytest.mark.parametrize("X, Y, Z, S, nnz, K", [(1, 1, 1, 1, 1, 4096), (1, 4, 4, 1, 4, 8192)])
+def test_wide_channels(X, Y, Z, S, nnz, K):
+    rng = np.random.default_rng(K)
+    idx, val, mix = H.random_table(rng, nnz, X, Y, Z, S)
+    snd, rcv = H.random_graph(rng, 8, 24)
+    x, y, s, dm = H.random_operands(rng, 8, 24, X, Y, S, K, Z)
+    res = run_abi(idx, val, mix, x, y, s, dm, snd, rcv, Z)
+    check_all(idx, val, mix, x, y, s, dm, snd, rcv, Z, res, tag=f"K={K}")
+
+
+# ---------------------------------------------------------------------------
+# padding, empty rows, gaps (each rule has a reference test, see include/e3j_amd.h)
+# ---------------------------------------------------------------------------
+def _padded_problem(rng, K=16):
+    N, X, Y, Z, S, nnz = 6, 4, 5, 6, 3, 40
+    idx, val, mix = H.random_table(rng, nnz, X, Y, Z, S)
+    # node 2 has no incoming edge; 3 trailing padding edges; 1 sender-only padding edge inside node 4's row
+    snd = np.array([1, 3, 0, 5, 4, 0, O.DUMMY_INDEX, 2, 1, O.DUMMY_INDEX, O.DUMMY_INDEX, O.DUMMY_INDEX], dtype=np.int32)
+    rcv = np.array([0, 0, 1, 1, 3, 4, 4, 4, 5, O.DUMMY_INDEX, O.DUMMY_INDEX, O.DUMMY_INDEX], dtype=np.int32)
+    x, y, s, dm = H.random_operands(rng, N, len(snd), X, Y, S, K, Z)
+    dead = (snd == O.DUMMY_INDEX) | (rcv == O.DUMMY_INDEX)
+    y[dead] = np.nan          # features of padding edges may hold anything
+    s[dead] = np.inf
+    return idx, val, mix, x, y, s, dm, snd, rcv, Z, dead
+
+
+@pytest.mark.parametrize("grouping", ["receiver", "sender"])
+def test_padding_edges_and_empty_rows(grouping):
+    """Zero rows for nodes without live edges, NaN/Inf on padding edges never read, dy/ds of
+    padding edges written as exact zeros over poisoned memory
+    (tests/test_ops/test_convolution_jax_transforms.py:229-306)."""
+    idx, val, mix, x, y, s, dm, snd, rcv, Z, dead = _padded_problem(np.random.default_rng(3))
+    out, dx, dy, ds = run_abi(idx, val, mix, x, y, s, dm, snd, rcv, Z, grouping=grouping)
+    assert not out[2].any() and np.isfinite(out).all()
+    assert not dy[dead].any() and not ds[dead].any()
+    live = ~dead
+    ref, mag = H.forward_reference(idx, val, mix, x, y[live], s[live], snd[live], rcv[live], Z)
+    H.assert_parity(out, ref, mag, "out")
+    (rx, ry, rs), (mx, my, ms) = H.backward_reference(idx, val, mix, x, y[live], s[live], snd[live],
+                                                      rcv[live], dm)
+    H.assert_parity(dx, rx, mx, "dx")
+    H.assert_parity(dy[live], ry, my, "dy")
+    H.assert_parity(ds[live], rs, ms, "ds")
+
+
+def test_no_edges():
+    """E = 0: all-zero out and dx (tests/test_pallas_mosaic_gpu_convolution.py:1566-1589)."""
+    rng = np.random.default_rng(4)
+    idx, val, mix = H.random_table(rng, 20, 3, 3, 4, 2)
+    x, y, s, dm = H.random_operands(rng, 5, 0, 3, 3, 2, 8, 4)
+    empty = np.zeros((0,), dtype=np.int32)
+    out, dx, dy, ds = run_abi(idx, val, mix, x, y, s, dm, empty, empty, 4)
+    assert not out.any() and not dx.any() and dy.shape == (0, 3) and ds.shape == (0, 2, 8)
+
+
+@pytest.mark.parametrize("grouping", ["receiver", "sender"])
+def test_gap_rows_are_zero(grouping):
+    """Coordinates no coefficient touches yield zeros, not garbage (tests/test_ops/test_zero_gap_rows.py:15-26)."""
+    rng = np.random.default_rng(5)
+    X, Y, Z, S, K = 6, 5, 7, 4, 8
+    idx = np.array([[0, 0, 0], [0, 2, 1], [3, 2, 4], [6, 5, 1]])   # out rows 1,2,4,5; x rows 1,3,4; y 2,3; scalar 2 untouched
+    val = rng.normal(size=4).astype(np.float32)
+    mix = np.array([0, 0, 1, 1, 2, 2, 3])
+    snd, rcv = H.random_graph(rng, 5, 14)
+    x, y, s, dm = H.random_operands(rng, 5, 14, X, Y, S, K, Z)
+    out, dx, dy, ds = run_abi(idx, val, mix, x, y, s, dm, snd, rcv, Z, grouping=grouping)
+    assert not out[:, [1, 2, 4, 5]].any() and not dx[:, [1, 3, 4]].any()
+    assert not dy[:, [2, 3]].any() and not ds[:, 2].any()
+    check_all(idx, val, mix, x, y, s, dm, snd, rcv, Z, (out, dx, dy, ds), tag="gaps")
+
+
+def test_unsorted_edges_through_permutation():
+    """Edges in any order: CSR positions refer to y/s rows through edge_perm."""
+    rng = np.random.default_rng(6)
+    N, E, X, Y, Z, S, K, nnz = 10, 60, 4, 6, 5, 3, 32, 50
+    idx, val, mix = H.random_table(rng, nnz, X, Y, Z, S)
+    snd, rcv = H.random_graph(rng, N, E, sort_by=None)
+    x, y, s, dm = H.random_operands(rng, N, E, X, Y, S, K, Z)
+    perm = np.argsort(rcv, kind="stable").astype(np.int32)
+    res = run_abi(idx, val, mix, x, y, s, dm, snd, rcv, Z, perm=perm)
+    check_all(idx, val, mix, x, y, s, dm, snd, rcv, Z, res, tag="perm")
+
+
+def test_repeated_senders_accumulate():
+    """Several edges from one sender (tests/test_pallas_mosaic_gpu_convolution.py:325-350)."""
+    rng = np.random.default_rng(8)
+    idx, val, mix = H.random_table(rng, 30, 3, 4, 4, 2)
+    snd = np.zeros(12, dtype=np.int32)
+    rcv = np.sort(rng.integers(0, 4, 12)).astype(np.int32)
+    x, y, s, dm = H.random_operands(rng, 4, 12, 3, 4, 2, 16, 4)
+    res = run_abi(idx, val, mix, x, y, s, dm, snd, rcv, 4)
+    check_all(idx, val, mix, x, y, s, dm, snd, rcv, 4, res, tag="repeated")
+    assert not res[1][1:].any()
+
+
+def test_sorted_path_is_bit_reproducible():
+    """Forward and the sender-grouped backward give identical bits run to run
+    (tests/test_ops/test_convolution_op.py:322-342)."""
+    rng = np.random.default_rng(9)
+    N, E, X, Y, Z, S, K, nnz = 128, 4096, 16, 16, 4, 4, 32, 64
+    idx, val, mix = H.random_table(rng, nnz, X, Y, Z, S)
+    snd, rcv = H.random_graph(rng, N, E)
+    x, y, s, dm = H.random_operands(rng, N, E, X, Y, S, K, Z)
+    base = run_abi(idx, val, mix, x, y, s, dm, snd, rcv, Z, grouping="sender")
+    for _ in range(5):
+        again = run_abi(idx, val, mix, x, y, s, dm, snd, rcv, Z, grouping="sender")
+        for a, b in zip(base, again):
+            assert np.array_equal(a, b)

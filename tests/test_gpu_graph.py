@@ -1,0 +1,58 @@
+"""Device graph preparation (CSR row pointers, stable edge sort) against numpy."""
+
+import numpy as np
+import pytest
+import torch
+
+from e3j_amd.graph import DUMMY_INDEX, GraphCSR, csr_row_ptr, fold_endpoints, sort_edges, wrap_global_index
+from oracle import conv_oracle as O
+
+pytestmark = pytest.mark.gpu
+
+
+def dev(a):
+    return torch.from_numpy(np.ascontiguousarray(a)).cuda()
+
+
+@pytest.mark.parametrize("num_nodes, num_edges", [(4, 9), (1000, 30000), (32000, 200000), (5, 0)])
+def test_row_ptr_and_sort(num_nodes, num_edges):
+    rng = np.random.default_rng(num_edges)
+    key = rng.integers(0, num_nodes, num_edges).astype(np.int32)
+    other = rng.integers(0, num_nodes, num_edges).astype(np.int32)
+    if num_edges:
+        key[rng.integers(0, num_edges, max(1, num_edges // 50))] = DUMMY_INDEX
+        key[rng.integers(0, num_edges, 2)] = -3          # negative keys are padding too
+    ptr = csr_row_ptr(dev(key), num_nodes)
+    assert ptr.dtype == torch.int32
+    np.testing.assert_array_equal(ptr.cpu().numpy(), O.receiver_ptr(key, num_nodes))
+    perm, other_sorted, ptr2 = sort_edges(dev(key), dev(other), num_nodes)
+    np.testing.assert_array_equal(ptr2.cpu().numpy(), O.receiver_ptr(key, num_nodes))
+    want = np.argsort(key.view(np.uint32), kind="stable")
+    np.testing.assert_array_equal(perm.cpu().numpy(), want)
+    np.testing.assert_array_equal(other_sorted.cpu().numpy(), other[want])
+
+
+def test_graph_csr_with_dummy_edges():
+    """tests/test_graph.py:86-141."""
+    sender = np.array([1, 2, 0, 1, 3, 2] + [DUMMY_INDEX] * 3, dtype=np.int32)
+    receiver = np.array([0, 1, 1, 2, 2, 3] + [DUMMY_INDEX] * 3, dtype=np.int32)
+    s_l, r_l = wrap_global_index(dev(sender), 4), wrap_global_index(dev(receiver), 4)
+    graph = GraphCSR(4, s_l, r_l)
+    assert graph.receiver_ptr.tolist() == [0, 1, 3, 5, 6]
+    assert graph.num_neighbors.tolist() == [1, 2, 2, 1]
+    perm, graph_t, inverse = graph.transpose()
+    assert graph_t.receiver_ptr.tolist() == [0, 1, 3, 5, 6]
+    assert perm[inverse.long()].tolist() == list(range(9))
+    assert graph_t.sender.tolist()[:6] == receiver[perm.cpu().numpy()][:6].tolist()
+    # folding two graphs keeps the grouping key non-decreasing and counts every edge
+    r_f, s_f = fold_endpoints(dev(np.stack([receiver, receiver])).long(), dev(np.stack([sender, sender])).long(), 2, 4)
+    assert bool((r_f[1:] >= r_f[:-1]).all())
+    assert int(csr_row_ptr(r_f, 8)[-1]) == 18
+    assert int((s_f == DUMMY_INDEX).sum()) == 6
+    masked_s, masked_r = GraphCSR.mask_edges(dev(sender[:6]), dev(receiver[:6]), dev(np.arange(4) < 3))
+    assert ((masked_s == DUMMY_INDEX) | (masked_r == DUMMY_INDEX)).tolist() == [False, False, False, False, True, True]
+
+
+def test_cpu_tensors_are_rejected():
+    with pytest.raises(RuntimeError, match="no CPU implementation"):
+        csr_row_ptr(torch.zeros(4, dtype=torch.int32), 4)

@@ -1,0 +1,256 @@
+"""The torch-facing operators and the Convolution module on the GPU, against the CPU oracle."""
+
+import warnings
+
+import numpy as np
+import pytest
+import torch
+
+import e3j_amd
+from e3j_amd import Convolution, ConvolutionParams, GraphOrdering, convolution, convolution_bwd
+from e3j_amd.harmonics import Harmonics
+from oracle import conv_oracle as O
+from tests import helpers as H
+
+pytestmark = pytest.mark.gpu
+
+
+def dev(a, **kw):
+    return torch.from_numpy(np.ascontiguousarray(a)).cuda().requires_grad_(kw.get("grad", False))
+
+
+def _problem(seed, N=12, E=70, X=5, Y=6, Z=7, S=4, K=16, nnz=60, sort_by="receiver", dtype=np.float32):
+    rng = np.random.default_rng(seed)
+    idx, val, mix = H.random_table(rng, nnz, X, Y, Z, S)
+    snd, rcv = H.random_graph(rng, N, E, sort_by=sort_by)
+    x, y, s, dm = H.random_operands(rng, N, E, X, Y, S, K, Z, dtype=dtype)
+    coef = H.pack_table(idx, val, mix, val_dtype=dtype)
+    return dict(idx=idx, val=val, mix=mix, snd=snd, rcv=rcv, x=x, y=y, s=s, dm=dm, coef=coef,
+                params=ConvolutionParams(num_out=Z, num_scalars=S))
+
+
+def _check(p, out, grads, tol=None):
+    tol = tol or {}
+    ref, mag = H.forward_reference(p["idx"], p["val"], p["mix"], p["x"], p["y"], p["s"], p["snd"], p["rcv"],
+                                   p["params"].num_out)
+    H.assert_parity(out.detach().cpu().numpy(), ref, mag, "out", **tol)
+    refs, mags = H.backward_reference(p["idx"], p["val"], p["mix"], p["x"], p["y"], p["s"], p["snd"],
+                                      p["rcv"], p["dm"])
+    for g, r, m, name in zip(grads, refs, mags, ("dx", "dy", "ds")):
+        H.assert_parity(g.detach().cpu().numpy(), r, m, name, **tol)
+
+
+@pytest.mark.parametrize("ordering", ["RECEIVER", "NONE"])
+@pytest.mark.parametrize("deterministic", [False, True])
+def test_autograd_matches_oracle(ordering, deterministic):
+    p = _problem(1, sort_by="receiver" if ordering == "RECEIVER" else None)
+    x, y, s = (dev(p[k], grad=True) for k in ("x", "y", "s"))
+    with e3j_amd.config.use(deterministic=deterministic, debug_level=1):
+        out = convolution(p["coef"], x, y, s, dev(p["snd"]), dev(p["rcv"]), p["params"], ordering)
+        grads = torch.autograd.grad(out, (x, y, s), dev(p["dm"]))
+    _check(p, out, grads)
+
+
+def test_convolution_bwd_direct_and_deterministic_bits():
+    p = _problem(2, N=64, E=2000, K=32)
+    args = [dev(p[k]) for k in ("x", "y", "s")]
+    snd, rcv, dm = dev(p["snd"]), dev(p["rcv"]), dev(p["dm"])
+    with e3j_amd.config.use(deterministic=True):
+        base = convolution_bwd(p["coef"], *args, snd, rcv, dm, p["params"])
+        for _ in range(5):
+            again = convolution_bwd(p["coef"], *args, snd, rcv, dm, p["params"])
+            for a, b in zip(base, again):
+                assert torch.equal(a, b)
+    fast = convolution_bwd(p["coef"], *args, snd, rcv, dm, p["params"])
+    out = convolution(p["coef"], *args, snd, rcv, p["params"])
+    _check(p, out, fast)
+    _check(p, out, base)
+
+
+def test_two_dimensional_x_means_one_channel():
+    p = _problem(3, K=1)
+    x, y, s = dev(p["x"][:, :, 0], grad=True), dev(p["y"], grad=True), dev(p["s"], grad=True)
+    out = convolution(p["coef"], x, y, s, dev(p["snd"]), dev(p["rcv"]), p["params"])
+    assert out.shape == (p["x"].shape[0], p["params"].num_out)
+    grads = torch.autograd.grad(out, (x, y, s), dev(p["dm"][:, :, 0]))
+    assert grads[0].shape == x.shape
+    _check(p, out.unsqueeze(-1), (grads[0].unsqueeze(-1), grads[1], grads[2]))
+
+
+def test_leading_layout_and_float64():
+    p = _problem(4, dtype=np.float64)
+    xl, sl, dml = (np.ascontiguousarray(p[k].swapaxes(1, 2)) for k in ("x", "s", "dm"))
+    x, y, s = dev(xl, grad=True), dev(p["y"], grad=True), dev(sl, grad=True)
+    out = convolution(p["coef"], x, y, s, dev(p["snd"]), dev(p["rcv"]), p["params"], layout="LEADING_CHANNELS")
+    grads = torch.autograd.grad(out, (x, y, s), dev(dml))
+    tol = dict(rtol=1e-12, atol=1e-12, ulps=0.0)
+    _check(p, out.transpose(1, 2), (grads[0].transpose(1, 2), grads[1], grads[2].transpose(1, 2)), tol)
+
+
+def _dense_reference(p, x, y, s):
+    """Independent torch restatement (dense einsum), differentiable to any order."""
+    Z, X, Y = p["params"].num_out, p["x"].shape[1], p["y"].shape[1]
+    dense = torch.zeros((Z, X, Y), dtype=x.dtype, device=x.device)
+    dense.index_put_(tuple(torch.as_tensor(p["idx"].T, device=x.device)),
+                     torch.as_tensor(p["val"], dtype=x.dtype, device=x.device), accumulate=True)
+    snd = torch.as_tensor(p["snd"], dtype=torch.long, device=x.device)
+    rcv = torch.as_tensor(p["rcv"], dtype=torch.long, device=x.device)
+    msg = torch.einsum("ijk,ejc,ek->eic", dense, x[snd], y) * s[:, torch.as_tensor(p["mix"], device=x.device), :]
+    return torch.zeros((x.shape[0], Z, x.shape[2]), dtype=x.dtype, device=x.device).index_add(0, rcv, msg)
+
+
+def test_double_backward_matches_autograd_of_dense_form():
+    """Hessian-vector products through convolution_bwd's own backward
+    (src/e3j/ops/convolution.py:535-562; tests/test_ops/test_convolution_jax_transforms.py:644-767)."""
+    p = _problem(5, N=6, E=20, K=4, dtype=np.float64)
+    snd, rcv = dev(p["snd"]), dev(p["rcv"])
+
+    def scalar(fn, x, y, s):
+        out = fn(x, y, s)
+        g = torch.autograd.grad(out, (x, y, s), dev(p["dm"]), create_graph=True)
+        return sum((gi ** 2).sum() for gi in g) + (out ** 3).sum()
+
+    ours = [dev(p[k], grad=True) for k in ("x", "y", "s")]
+    theirs = [dev(p[k], grad=True) for k in ("x", "y", "s")]
+    a = scalar(lambda x, y, s: convolution(p["coef"], x, y, s, snd, rcv, p["params"]), *ours)
+    b = scalar(lambda x, y, s: _dense_reference(p, x, y, s), *theirs)
+    torch.testing.assert_close(a, b, rtol=1e-10, atol=1e-10)
+    ga = torch.autograd.grad(a, ours)
+    gb = torch.autograd.grad(b, theirs)
+    for u, v in zip(ga, gb):
+        torch.testing.assert_close(u, v, rtol=1e-9, atol=1e-9)
+
+
+def test_sender_ordering_on_symmetric_graph():
+    """SENDER ordering = RECEIVER ordering on a symmetric graph with y_ba = p y_ab, s_ba = s_ab
+    (tests/test_convolution.py:351-456)."""
+    rng = np.random.default_rng(6)
+    N, K = 10, 16
+    pos = rng.normal(size=(N, 3))
+    pairs = [(a, b) for a in range(N) for b in range(N) if a != b and np.linalg.norm(pos[a] - pos[b]) < 1.6]
+    snd = np.array([a for a, b in pairs], dtype=np.int32)
+    rcv = np.array([b for a, b in pairs], dtype=np.int32)
+    module_r = Convolution(("0e+1o", "0e+1o+2e"), "0e+1o+2e", graph_ordering="RECEIVER")
+    module_s = Convolution(("0e+1o", "0e+1o+2e"), "0e+1o+2e", graph_ordering="SENDER")
+    vec = torch.from_numpy(pos[snd] - pos[rcv])
+    y = Harmonics(2, normalize=True)(vec).float().numpy()
+    dist = np.linalg.norm(pos[snd] - pos[rcv], axis=-1)
+    S = module_r.params.num_scalars
+    w = rng.normal(size=(S, K)).astype(np.float32)
+    s = (np.cos(dist)[:, None, None] * w[None]).astype(np.float32)        # symmetric in (a, b)
+    x = rng.normal(size=(N, 4, K)).astype(np.float32)
+    dm = rng.normal(size=(N, module_r.target.dim, K)).astype(np.float32)
+
+    def run(module, order):
+        xs, ys, ss = dev(x, grad=True), dev(y[order], grad=True), dev(s[order], grad=True)
+        out = module(xs, ys, ss, dev(snd[order]), dev(rcv[order]))
+        gx, gy, gs = torch.autograd.grad(out, (xs, ys, ss), dev(dm))
+        inverse = np.argsort(order)
+        return out, gx, gy[inverse], gs[inverse]
+
+    by_receiver = run(module_r, np.argsort(rcv, kind="stable"))
+    by_sender = run(module_s, np.argsort(snd, kind="stable"))
+    for a, b in zip(by_receiver, by_sender):
+        torch.testing.assert_close(a, b, rtol=2e-5, atol=2e-5)
+
+
+def test_batched_graphs_fold_with_padding():
+    """A batch of padded graphs folded into one graph equals a loop over the graphs
+    (tests/test_ops/test_convolution_jax_transforms.py:197-226)."""
+    B, p = 3, _problem(7, N=8, E=30)
+    rng = np.random.default_rng(8)
+    xs = rng.normal(size=(B,) + p["x"].shape).astype(np.float32)
+    ys = rng.normal(size=(B,) + p["y"].shape).astype(np.float32)
+    ss = rng.normal(size=(B,) + p["s"].shape).astype(np.float32)
+    snd = np.stack([p["snd"]] * B)
+    rcv = np.stack([p["rcv"]] * B)
+    for b in range(B):                          # tail padding of different lengths per graph
+        snd[b, 30 - 2 * (b + 1):] = O.DUMMY_INDEX
+        rcv[b, 30 - 2 * (b + 1):] = O.DUMMY_INDEX
+    with warnings.catch_warnings(record=True) as caught:
+        warnings.simplefilter("always")
+        out = e3j_amd.convolution_batched(p["coef"], dev(xs), dev(ys), dev(ss), dev(snd), dev(rcv), p["params"])
+    assert any(issubclass(w.category, e3j_amd.ConvolutionBatchingWarning) for w in caught)
+    for b in range(B):
+        ref, mag = H.forward_reference(p["idx"], p["val"], p["mix"], xs[b], ys[b], ss[b], snd[b], rcv[b],
+                                       p["params"].num_out)
+        H.assert_parity(out[b].cpu().numpy(), ref, mag, f"graph {b}")
+    shared = e3j_amd.convolution_batched(p["coef"], dev(xs), dev(ys), dev(ss), dev(p["snd"]), dev(p["rcv"]),
+                                         p["params"])
+    ref, mag = H.forward_reference(p["idx"], p["val"], p["mix"], xs[1], ys[1], ss[1], p["snd"], p["rcv"],
+                                   p["params"].num_out)
+    H.assert_parity(shared[1].cpu().numpy(), ref, mag, "shared graph")
+
+
+# --- module level -----------------------------------------------------------------------
+def _wigner_d(space, rot):
+    from tests.test_host_logic import _wigner_d as one
+    blocks = [one(ir.l, rot) * (ir.p ** 0) for mul, ir in space for _ in range(mul)]
+    dim = sum(b.shape[0] for b in blocks)
+    out, at = np.zeros((dim, dim)), 0
+    for b in blocks:
+        out[at:at + b.shape[0], at:at + b.shape[0]] = b
+        at += b.shape[0]
+    return out
+
+
+def test_module_is_equivariant_and_shapes():
+    """Rotating node features and edge harmonics rotates the messages (tests/test_convolution.py:112-167)."""
+    from scipy.spatial.transform import Rotation
+    rng = np.random.default_rng(9)
+    N, E, K = 7, 40, 8
+    module = Convolution(("0e+1o+2e", "0e+1o+2e"), "0e+1o+2e", graph_ordering="RECEIVER", avg_num_neighbors=5.0)
+    snd, rcv = H.random_graph(rng, N, E)
+    vec = rng.normal(size=(E, 3))
+    rot = Rotation.from_rotvec([0.4, 0.2, -0.9]).as_matrix()
+    sh = Harmonics(2, normalize=True)
+    x = rng.normal(size=(N, module.source[0].dim, K))
+    s = rng.normal(size=(E, module.params.num_scalars, K))
+    d_x, d_out = _wigner_d(module.source[0], rot), _wigner_d(module.target, rot)
+
+    def run(x_, vec_):
+        y_ = sh(torch.from_numpy(vec_)).cuda()
+        return module(dev(x_), y_, dev(s), dev(snd), dev(rcv)).cpu().numpy()
+
+    out = run(x, vec)
+    assert out.shape == (N, module.target.dim, K)
+    out_rot = run(np.einsum("ij,njc->nic", d_x, x), vec @ rot.T)
+    # coefficient values are stored as float32 (like the reference's tables): equivariance holds to that rounding
+    np.testing.assert_allclose(out_rot, np.einsum("ij,njc->nic", d_out, out), rtol=0, atol=5e-6)
+
+
+def test_module_node_mask_and_dtype_promotion():
+    w_name = "0e+1o"
+    module = Convolution((w_name, "0e+1o"), None, graph_ordering="RECEIVER")
+    rng = np.random.default_rng(10)
+    N, E, K = 6, 24, 4
+    # padding nodes (4, 5) lie at the tail and padding edges only connect padding nodes, as the
+    # reference requires (src/e3j/core/convolution.py:367-372): they form the tail of the sorted list
+    rcv = np.sort(np.concatenate([rng.integers(0, 4, E - 6), rng.integers(4, 6, 6)])).astype(np.int32)
+    snd = np.where(rcv < 4, rng.integers(0, 4, E), rng.integers(4, 6, E)).astype(np.int32)
+    x = rng.normal(size=(N, 4, K)).astype(np.float32)
+    y = rng.normal(size=(E, 4)).astype(np.float32)
+    s = rng.normal(size=(E, module.params.num_scalars, K)).astype(np.float32)
+    mask = np.arange(N) < 4
+    out = module(dev(x), dev(y), dev(s), dev(snd), dev(rcv), node_mask=dev(mask))
+    keep = (snd < 4) & (rcv < 4)
+    ref = module(dev(x), dev(y[keep]), dev(s[keep]), dev(snd[keep]), dev(rcv[keep]))
+    torch.testing.assert_close(out, ref, rtol=1e-6, atol=1e-6)
+    assert not out[4:].any()
+    assert module(dev(x.astype(np.float64)), dev(y), dev(s), dev(snd), dev(rcv)).dtype == torch.float64
+
+
+# --- errors of the reference's operator ------------------------------------------------
+def test_operator_errors():
+    p = _problem(11)
+    x, y, s, snd, rcv = (dev(p[k]) for k in ("x", "y", "s", "snd", "rcv"))
+    with pytest.raises(RuntimeError, match="no CPU implementation"):
+        convolution(p["coef"], x.cpu(), y, s, snd, rcv, p["params"])
+    with pytest.raises(NotImplementedError, match="only one channel"):
+        convolution(p["coef"], x, torch.stack([y, y], -1), s, snd, rcv, p["params"])
+    with pytest.raises(TypeError, match="concrete"):
+        convolution(torch.from_numpy(p["coef"]), x, y, s, snd, rcv, p["params"])
+    with pytest.raises(ValueError, match="y_parity"):
+        convolution(p["coef"], x, y, s, snd, rcv, p["params"], GraphOrdering.SENDER)
+    with pytest.raises(TypeError, match="Cast the operands"):
+        convolution(p["coef"], x.half(), y.half(), s.half(), snd, rcv, p["params"])

@@ -1,0 +1,96 @@
+"""The XLA-FFI handlers driven with hand-built call frames over GPU buffers."""
+
+import ctypes as C
+
+import numpy as np
+import pytest
+import torch
+
+from e3j_amd import _lib
+from e3j_amd.coef import Coef4D
+from oracle import conv_oracle as O
+from tests import helpers as H
+from tests.xla_frame import F32, S32, U8, FakeXla
+
+pytestmark = pytest.mark.gpu
+
+
+def dev(a):
+    return torch.from_numpy(np.ascontiguousarray(a)).cuda()
+
+
+def _buf(xla, t, dtype):
+    xla._keep.append(t)  # the frame only holds the address: keep the tensor alive
+    return xla.buffer(dtype, t.data_ptr(), tuple(t.shape))
+
+
+def _problem():
+    rng = np.random.default_rng(12)
+    N, E, X, Y, Z, S, K, nnz = 9, 50, 4, 5, 6, 3, 32, 40
+    idx, val, mix = H.random_table(rng, nnz, X, Y, Z, S)
+    snd, rcv = H.random_graph(rng, N, E)
+    x, y, s, dm = H.random_operands(rng, N, E, X, Y, S, K, Z)
+    return idx, val, mix, x, y, s, dm, snd, rcv, Z
+
+
+def test_forward_and_both_backward_targets():
+    idx, val, mix, x, y, s, dm, snd, rcv, Z = _problem()
+    lib = _lib.load()
+    xla = FakeXla(stream=torch.cuda.current_stream().cuda_stream)
+    n = x.shape[0]
+    packed = H.pack_table(idx, val, mix)
+    coef = dev(packed)
+    xd, yd, sd, dmd = dev(x), dev(y), dev(s), dev(dm)
+    ptr = dev(O.receiver_ptr(rcv, n))
+    ranges = dev(np.array([len(val)], dtype=np.int32))
+    attrs = lambda: {"num_nodes": (S32, C.c_int32(n)), "debug": (S32, C.c_int32(1))}  # noqa: E731
+
+    # "convolution": reference operand order, coef_ranges present and ignored
+    out = torch.full((n, Z, x.shape[2]), float("nan"), device="cuda")
+    frame = xla.frame([_buf(xla, coef, U8), _buf(xla, xd, F32), _buf(xla, yd, F32), _buf(xla, sd, F32),
+                       _buf(xla, dev(snd), S32), _buf(xla, ptr, S32), _buf(xla, ranges, S32)],
+                      [_buf(xla, out, F32)], attrs())
+    keep = [frame]
+    assert lib.e3j_amd_xla_convolution(C.addressof(frame)) is None, xla.errors
+    torch.cuda.synchronize()
+    ref, mag = H.forward_reference(idx, val, mix, x, y, s, snd, rcv, Z)
+    H.assert_parity(out.cpu().numpy(), ref, mag, "xla out")
+
+    refs, mags = H.backward_reference(idx, val, mix, x, y, s, snd, rcv, dm)
+
+    def check(dx, dy, ds, tag):
+        torch.cuda.synchronize()
+        for g, r, m, name in zip((dx, dy, ds), refs, mags, ("dx", "dy", "ds")):
+            H.assert_parity(g.cpu().numpy(), r, m, f"{tag} {name}")
+
+    # "convolution_bwd": transposed CSR, permutation, and the reference's stack of three
+    # transposed tables (src/e3j/ops/convolution.py:366-369,401-403)
+    c = Coef4D.unpack(packed, np.float32)
+    stacked = np.stack([c.transpose(a).pack() for a in ((1, 0, 2, 3), (2, 0, 1, 3), (3, 0, 2, 1))])
+    perm, recv_t, sptr = O.transpose_graph(snd, rcv, n)
+    dx, dy, ds = (torch.full_like(t, float("nan")) for t in (xd, yd, sd))
+    operands = [_buf(xla, dev(stacked), U8), _buf(xla, xd, F32), _buf(xla, yd, F32), _buf(xla, sd, F32),
+                _buf(xla, dmd, F32), _buf(xla, dev(recv_t.astype(np.int32)), S32), _buf(xla, dev(sptr), S32),
+                _buf(xla, dev(perm), S32), _buf(xla, ranges, S32)]
+    keep.append(operands)
+    frame = xla.frame(operands, [_buf(xla, dx, F32), _buf(xla, dy, F32), _buf(xla, ds, F32)], attrs())
+    assert lib.e3j_amd_xla_convolution_bwd(C.addressof(frame)) is None, xla.errors
+    check(dx, dy, ds, "stacked tables")
+
+    # same target with the forward table
+    dx, dy, ds = (torch.full_like(t, float("nan")) for t in (xd, yd, sd))
+    operands[0] = _buf(xla, coef, U8)
+    frame = xla.frame(operands, [_buf(xla, dx, F32), _buf(xla, dy, F32), _buf(xla, ds, F32)], attrs())
+    assert lib.e3j_amd_xla_convolution_bwd(C.addressof(frame)) is None, xla.errors
+    check(dx, dy, ds, "forward table")
+
+    # "convolution_bwd_receiver": forward CSR, empty permutation
+    dx, dy, ds = (torch.full_like(t, float("nan")) for t in (xd, yd, sd))
+    empty = torch.zeros(0, dtype=torch.int32, device="cuda")
+    frame = xla.frame([_buf(xla, coef, U8), _buf(xla, xd, F32), _buf(xla, yd, F32), _buf(xla, sd, F32),
+                       _buf(xla, dmd, F32), _buf(xla, dev(snd), S32), _buf(xla, ptr, S32),
+                       xla.buffer(S32, 0, (0,))],
+                      [_buf(xla, dx, F32), _buf(xla, dy, F32), _buf(xla, ds, F32)], attrs())
+    assert lib.e3j_amd_xla_convolution_bwd_receiver(C.addressof(frame)) is None, xla.errors
+    check(dx, dy, ds, "receiver grouping")
+    del empty, keep
