@@ -33,6 +33,13 @@ if ROOT not in sys.path:
 
 HBM_PEAK_GBS = 8000.0
 
+#: HBM bytes per launch of the backward kernel on the full cfg3 workload, from two
+#: `rocprofv3 --pmc` runs of this script (FETCH_SIZE and WRITE_SIZE, KiB per dispatch), each
+#: scaled by what the same counter reads for a 1 GiB device copy (`--calibrate-copy`):
+#: 2.0 * 10.24e6 KiB fetched + 1.0 * 18.96e6 KiB written.  Only quoted for that workload.
+MEASURED_TRAFFIC_BYTES = {("cfg3", 1.0): {"backward": 2.0 * 10.236e6 * 1024 + 18.959e6 * 1024,
+                                          "forward": 2.0 * 9.399e6 * 1024 + 1.584e6 * 1024}}
+
 
 def parse_args():
     ap = argparse.ArgumentParser()
@@ -45,6 +52,9 @@ def parse_args():
     ap.add_argument("--cpu-seconds", type=float, default=15.0)
     ap.add_argument("--kernel-only", action="store_true",
                     help="time the C-ABI launches only (no operator-level step)")
+    ap.add_argument("--calibrate-copy", action="store_true",
+                    help="also run a 1 GiB device copy, the known-size kernel that hardware "
+                         "traffic counters are scaled by")
     return ap.parse_args()
 
 
@@ -141,11 +151,14 @@ def cpu_baseline(w, seconds: float) -> dict:
         c_oracle.convolution_vjp(idx, val, mix, x, a["y"], a["s"], a["sender"], a["receiver"], dm)
         return h.num_edges, time.perf_counter() - t0
 
-    probe_nodes = min(w.num_nodes, 64)
-    edges, t = run(probe_nodes)
-    rate = edges / max(t, 1e-9)
-    want_nodes = int(min(w.num_nodes, max(probe_nodes, probe_nodes * seconds * rate / max(edges, 1))))
+    # grow the sample until it takes about `seconds` (the first calls pay thread start-up)
+    want_nodes = min(w.num_nodes, 256)
     edges, t = run(want_nodes)
+    for _ in range(4):
+        if t >= 0.6 * seconds or want_nodes >= w.num_nodes:
+            break
+        want_nodes = int(min(w.num_nodes, max(2 * want_nodes, want_nodes * seconds / max(t, 1e-3))))
+        edges, t = run(want_nodes)
     return {"value": edges / t, "unit": "edges/s", "cores": cores, "kind": "port",
             "sample": f"forward + VJP on the edges of the first {want_nodes} receivers "
                       f"({edges} edges) of the same workload, {t:.1f} s"}
@@ -178,6 +191,14 @@ def main():
         grads = e3j_amd.convolution_bwd(coef, w.x, w.y, w.s, w.sender, w.receiver, w.dm,
                                         module.params, module.graph_ordering)
         return out, grads
+
+    if args.calibrate_copy:
+        src = torch.empty(1 << 28, dtype=torch.float32, device=device).normal_()
+        dst = torch.empty_like(src)
+        for _ in range(3):
+            dst.copy_(src)
+        torch.cuda.synchronize()
+        del src, dst
 
     abi = AbiCalls(w)
     if args.kernel_only:
@@ -228,9 +249,10 @@ def main():
         "roofline": {
             "bound": "hbm", "kernel": "convolution backward (unrolled_bwd_kernel + dx zero fill)",
             "achieved": bwd_gbs, "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": bwd_gbs / HBM_PEAK_GBS,
-            "traffic": None,
+            "traffic": MEASURED_TRAFFIC_BYTES.get((args.config, args.scale), {}).get("backward"),
             "algorithmic_bytes": bytes_["bwd"], "ms": bwd_ms,
             "forward": {"achieved": fwd_gbs, "frac": fwd_gbs / HBM_PEAK_GBS,
+                        "traffic": MEASURED_TRAFFIC_BYTES.get((args.config, args.scale), {}).get("forward"),
                         "algorithmic_bytes": bytes_["fwd"], "ms": fwd_ms},
             "forward_plus_backward": {"achieved": both_gbs, "frac": both_gbs / HBM_PEAK_GBS,
                                       "algorithmic_bytes": bytes_["fwd_bwd"], "ms": fwd_ms + bwd_ms},
