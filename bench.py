@@ -3,8 +3,9 @@
     python bench.py [--gpus 1] [--steps K] [--warmup W] [--config cfg3|cfg2|cfg4]
 
 A step is one pass of the hot path over one batch of synthetic input: the
-operator `convolution` (CSR build + forward kernel) followed by
-`convolution_bwd` (cotangents of node features, harmonics and radial weights)
+operator `convolution` (graph preparation + forward kernel) followed by its VJP
+through autograd (`convolution_bwd`: cotangents of node features, harmonics and
+radial weights)
 on the MACE-scale layer: 32 000 atoms, ~30 neighbours (~0.96 M edges), 128
 channels, irreps 0e+1o+2e+3o, harmonics up to l = 3, all paths up to l_out = 3,
 receiver-sorted edges, trailing-channels layout.  Inputs are resident in HBM
@@ -52,19 +53,22 @@ def parse_args():
     ap.add_argument("--cpu-seconds", type=float, default=15.0)
     ap.add_argument("--kernel-only", action="store_true",
                     help="time the C-ABI launches only (no operator-level step)")
+    ap.add_argument("--spatial-sort", action="store_true",
+                    help="cfg3 only: number the atoms along a space-filling curve instead of at random "
+                         "(a secondary figure; the headline keeps the random numbering)")
     ap.add_argument("--calibrate-copy", action="store_true",
                     help="also run a 1 GiB device copy, the known-size kernel that hardware "
                          "traffic counters are scaled by")
     return ap.parse_args()
 
 
-def build_workload(name: str, scale: float, device):
+def build_workload(name: str, scale: float, device, spatial_sort: bool = False):
     from e3j_amd import workloads as W
     if name == "cfg2":
         return W.config2(scale, device=device)
     if name == "cfg4":
         return W.config4(scale, device=device)
-    return W.config3(scale, device=device)
+    return W.config3(scale, device=device, spatial_sort=spatial_sort)
 
 
 class AbiCalls:
@@ -74,7 +78,8 @@ class AbiCalls:
         import numpy as np
         import torch
         from e3j_amd import _lib
-        from e3j_amd.graph import csr_row_ptr, sort_edges
+        from e3j_amd.graph import csr_row_ptr, locality_order, sort_edges
+        from e3j_amd.options import config
         from e3j_amd.ops import _Table
         self.torch, self.lib, self._lib = torch, _lib.load(), _lib
         self.w = w
@@ -95,6 +100,9 @@ class AbiCalls:
         else:
             self.perm, self.other = None, w.sender.contiguous()
             self.ptr = csr_row_ptr(w.receiver, w.num_nodes)
+        rounds = config().locality_rounds
+        self.order = locality_order(w.sender, w.receiver, w.num_nodes, rounds) if rounds > 0 else None
+        self.params.row_order = self.order.data_ptr() if self.order is not None else None
         self.out = torch.empty_like(w.dm)
         self.dx, self.dy, self.ds = torch.empty_like(w.x), torch.empty_like(w.y), torch.empty_like(w.s)
 
@@ -180,16 +188,18 @@ def main():
     device = torch.device("cuda:0")
     torch.cuda.set_device(device)
 
-    w = build_workload(args.config, args.scale, device)
+    w = build_workload(args.config, args.scale, device, args.spatial_sort)
     module = w.module
     coef = module._packed_coef("float32")
     bytes_ = w.algorithmic_bytes(sorted_edges=module.graph_ordering.value != "NONE")
 
+    xg, yg, sg = (t.detach().requires_grad_(True) for t in (w.x, w.y, w.s))
+
     def step():
-        out = e3j_amd.convolution(coef, w.x, w.y, w.s, w.sender, w.receiver, module.params,
+        # forward, then the VJP of (x, y, s) for the cotangent dm, as autograd runs them
+        out = e3j_amd.convolution(coef, xg, yg, sg, w.sender, w.receiver, module.params,
                                   module.graph_ordering)
-        grads = e3j_amd.convolution_bwd(coef, w.x, w.y, w.s, w.sender, w.receiver, w.dm,
-                                        module.params, module.graph_ordering)
+        grads = torch.autograd.grad(out, (xg, yg, sg), w.dm)
         return out, grads
 
     if args.calibrate_copy:
@@ -242,6 +252,7 @@ def main():
                         f"{module.graph_ordering.value.lower()}-ordered edges, trailing-channels layout, "
                         "forward + VJP (dx, dy, ds)",
             "scale": args.scale,
+            "atom_numbering": "space-filling curve" if args.spatial_sort else "random",
             "signature": abi.signature,
             "signature_name": (_lib.load().e3j_amd_signature_name(abi.signature).decode()
                                if abi.signature >= 0 else "table-driven kernel"),
@@ -249,10 +260,10 @@ def main():
         "roofline": {
             "bound": "hbm", "kernel": "convolution backward (unrolled_bwd_kernel + dx zero fill)",
             "achieved": bwd_gbs, "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": bwd_gbs / HBM_PEAK_GBS,
-            "traffic": MEASURED_TRAFFIC_BYTES.get((args.config, args.scale), {}).get("backward"),
+            "traffic": MEASURED_TRAFFIC_BYTES.get((args.config, args.scale if not args.spatial_sort else -1), {}).get("backward"),
             "algorithmic_bytes": bytes_["bwd"], "ms": bwd_ms,
             "forward": {"achieved": fwd_gbs, "frac": fwd_gbs / HBM_PEAK_GBS,
-                        "traffic": MEASURED_TRAFFIC_BYTES.get((args.config, args.scale), {}).get("forward"),
+                        "traffic": MEASURED_TRAFFIC_BYTES.get((args.config, args.scale if not args.spatial_sort else -1), {}).get("forward"),
                         "algorithmic_bytes": bytes_["fwd"], "ms": fwd_ms},
             "forward_plus_backward": {"achieved": both_gbs, "frac": both_gbs / HBM_PEAK_GBS,
                                       "algorithmic_bytes": bytes_["fwd_bwd"], "ms": fwd_ms + bwd_ms},

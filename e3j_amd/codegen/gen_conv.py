@@ -330,11 +330,11 @@ def emit_signature(sig_id: int, name: str, x_irreps: str, y_irreps: str, out_fil
     for cpl, wpb, zs in launch["fwd"]:
         out += [f"template __global__ void unrolled_fwd_kernel<{channels}, {cpl}, {wpb}, {part_names[zs]}>(",
                 "    const float *, const float *, const float *, const int32_t *, const int32_t *,",
-                "    const int32_t *, float *, int, float);"]
+                "    const int32_t *, const int32_t *, float *, int, float);"]
     for cpl, wpb, zs in launch["bwd"]:
         out += [f"template __global__ void unrolled_bwd_kernel<{channels}, {cpl}, {wpb}, {part_names[zs]}>(",
                 "    const float *, const float *, const float *, const float *, const int32_t *,",
-                "    const int32_t *, const int32_t *, float *, float *, float *, int, float);"]
+                "    const int32_t *, const int32_t *, const int32_t *, float *, float *, float *, int, float);"]
     out += ["", "// host pass only: the registry entry holds host function pointers",
             "#if !defined(__HIP_DEVICE_COMPILE__)",
             f"static const float kVal[] = {{{vals}}};",

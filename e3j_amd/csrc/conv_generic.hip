@@ -34,6 +34,7 @@ __global__ void generic_fwd_kernel(const Coef4D<Idx, Val> *__restrict__ coef, in
                                    const int32_t *__restrict__ other,
                                    const int32_t *__restrict__ row_ptr,
                                    const int32_t *__restrict__ perm,
+                                   const int32_t *__restrict__ row_order,
                                    Val *__restrict__ out, RowLayout lo,
                                    int num_nodes, int channels, int X, int S, int Z, int nchunks) {
     extern __shared__ __align__(16) unsigned char smem_raw[];
@@ -41,7 +42,8 @@ __global__ void generic_fwd_kernel(const Coef4D<Idx, Val> *__restrict__ coef, in
     const int wave = threadIdx.y;
     const int64_t item = (int64_t)blockIdx.x * blockDim.y + wave;
     if (item >= (int64_t)num_nodes * nchunks) return;  // uniform per wave; no barriers below
-    const int r = (int)(item / nchunks);
+    const int q = (int)(item / nchunks);
+    const int r = row_order ? row_order[q] : q;
     const int c = (int)(item % nchunks) * kWave + lane;
     const bool active = c < channels;
 
@@ -92,6 +94,7 @@ __global__ void generic_bwd_kernel(const Coef4D<Idx, Val> *__restrict__ coef, in
                                    const int32_t *__restrict__ other,
                                    const int32_t *__restrict__ row_ptr,
                                    const int32_t *__restrict__ perm,
+                                   const int32_t *__restrict__ row_order,
                                    Val *__restrict__ dx, Val *__restrict__ dy, Val *__restrict__ ds,
                                    int num_nodes, int channels, int X, int S, int Z, int nchunks,
                                    int cols_ji) {
@@ -100,7 +103,7 @@ __global__ void generic_bwd_kernel(const Coef4D<Idx, Val> *__restrict__ coef, in
     const int wave = threadIdx.y;
     const int64_t item = (int64_t)blockIdx.x * blockDim.y + wave;
     if (item >= (int64_t)num_nodes) return;
-    const int g = (int)item;
+    const int g = row_order ? row_order[item] : (int)item;
 
     const int per_wave = Z + 2 * X + 2 * S + num_y;
     Val *zc = reinterpret_cast<Val *>(smem_raw) + (size_t)wave * per_wave * kWave + lane;
@@ -236,7 +239,7 @@ int run_fwd(const e3j_amd_conv_params &p, const void *coef, const void *x, const
                        static_cast<const Val *>(x), make_layout(p.layout, p.num_x, p.channels),
                        static_cast<const Val *>(y), p.num_y,
                        static_cast<const Val *>(s), make_layout(p.layout, p.num_scalars, p.channels),
-                       other, row_ptr, perm,
+                       other, row_ptr, perm, p.row_order,
                        static_cast<Val *>(out), make_layout(p.layout, p.num_out, p.channels),
                        p.num_nodes, p.channels, p.num_x, p.num_scalars, p.num_out, nchunks);
     return check_hip(hipGetLastError(), "convolution forward launch");
@@ -292,7 +295,8 @@ int run_bwd(const e3j_amd_conv_params &p, bool group_is_receiver, const void *co
                            static_cast<const Coef4D<Idx, Val> *>(coef), p.num_coef,               \
                            static_cast<const Val *>(x), lx, static_cast<const Val *>(y), p.num_y, \
                            static_cast<const Val *>(s), ls, static_cast<const Val *>(dm), lo,     \
-                           other, row_ptr, perm, static_cast<Val *>(dx), static_cast<Val *>(dy),  \
+                           other, row_ptr, perm, p.row_order, static_cast<Val *>(dx),             \
+                           static_cast<Val *>(dy),                                               \
                            static_cast<Val *>(ds), p.num_nodes, p.channels, p.num_x,              \
                            p.num_scalars, p.num_out, nchunks, cols_ji ? 1 : 0);                   \
     } while (0)

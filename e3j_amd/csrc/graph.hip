@@ -35,6 +35,25 @@ __global__ void gather_kernel(const int32_t *__restrict__ src, const int32_t *__
         dst[i] = src[perm[i]];
 }
 
+// One sweep of minimum-label propagation: next[n] = min(cur[n], cur[m] for every neighbour m).
+__global__ void min_label_kernel(const int32_t *__restrict__ sender,
+                                 const int32_t *__restrict__ receiver, int64_t num_edges,
+                                 int num_nodes, const int32_t *__restrict__ cur,
+                                 int32_t *__restrict__ next) {
+    const int64_t stride = (int64_t)gridDim.x * blockDim.x;
+    for (int64_t e = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; e < num_edges; e += stride) {
+        const int a = sender[e], b = receiver[e];
+        if ((unsigned)a >= (unsigned)num_nodes || (unsigned)b >= (unsigned)num_nodes) continue;
+        atomicMin(&next[b], cur[a]);
+        atomicMin(&next[a], cur[b]);
+    }
+}
+
+__global__ void copy_i32_kernel(const int32_t *__restrict__ src, int32_t *__restrict__ dst, int64_t n) {
+    const int64_t stride = (int64_t)gridDim.x * blockDim.x;
+    for (int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; i < n; i += stride) dst[i] = src[i];
+}
+
 size_t align_up(size_t v, size_t a = 256) { return (v + a - 1) / a * a; }
 
 unsigned grid_for(int64_t n) { return (unsigned)std::max<int64_t>(1, std::min<int64_t>((n + 255) / 256, 4096)); }
@@ -90,6 +109,64 @@ int e3j_amd_csr_row_ptr(const int32_t *key, int64_t num_edges, int32_t num_nodes
         return set_error(E3J_AMD_INVALID_ARGUMENT, "csr_row_ptr: null operand");
     return row_ptr_impl(key, num_edges, num_nodes, row_ptr, workspace, scan_temp_bytes(num_nodes),
                         static_cast<hipStream_t>(stream_));
+}
+
+size_t e3j_amd_order_workspace_bytes(int32_t num_nodes) {
+    if (num_nodes < 0) return 0;
+    // [sort temp | label a | label b | keys in | keys out | order tmp]
+    return align_up(sort_temp_bytes(num_nodes)) + 5 * align_up(sizeof(int32_t) * (size_t)num_nodes) + 256;
+}
+
+int e3j_amd_locality_order(const int32_t *sender, const int32_t *receiver, int64_t num_edges,
+                           int32_t num_nodes, int32_t rounds, int32_t *order, void *workspace,
+                           void *stream_) {
+    if (num_nodes < 0 || num_edges < 0 || rounds < 0 || rounds > 64)
+        return set_error(E3J_AMD_INVALID_ARGUMENT, "locality_order: bad sizes");
+    if (num_nodes == 0) return E3J_AMD_OK;
+    if (order == nullptr || workspace == nullptr || (num_edges > 0 && (!sender || !receiver)))
+        return set_error(E3J_AMD_INVALID_ARGUMENT, "locality_order: null operand");
+    hipStream_t stream = static_cast<hipStream_t>(stream_);
+    unsigned char *ws = static_cast<unsigned char *>(workspace);
+    const size_t sort_bytes = sort_temp_bytes(num_nodes);
+    const size_t vec = align_up(sizeof(int32_t) * (size_t)num_nodes);
+    void *sort_temp = ws;
+    int32_t *lab_a = reinterpret_cast<int32_t *>(ws + align_up(sort_bytes));
+    int32_t *lab_b = reinterpret_cast<int32_t *>(ws + align_up(sort_bytes) + vec);
+    uint32_t *keys_in = reinterpret_cast<uint32_t *>(ws + align_up(sort_bytes) + 2 * vec);
+    uint32_t *keys_out = reinterpret_cast<uint32_t *>(ws + align_up(sort_bytes) + 3 * vec);
+    int32_t *order_tmp = reinterpret_cast<int32_t *>(ws + align_up(sort_bytes) + 4 * vec);
+    const unsigned ngrid = grid_for(num_nodes), egrid = grid_for(num_edges);
+
+    hipLaunchKernelGGL(iota_kernel, dim3(ngrid), dim3(256), 0, stream, lab_a, (int64_t)num_nodes);
+    hipLaunchKernelGGL(iota_kernel, dim3(ngrid), dim3(256), 0, stream, order, (int64_t)num_nodes);
+    int rc = check_hip(hipGetLastError(), "locality_order init");
+    if (rc) return rc;
+    // Levels: after 1, 2, 4, 8, ... sweeps the labels name ever larger clusters.  The order is
+    // refined from the finest level to the coarsest with stable sorts, so the coarsest clusters
+    // are contiguous and, inside them, the finer ones.
+    int done = 0;
+    for (int level = 1; level <= rounds; level *= 2) {
+        for (; done < level; done++) {
+            hipLaunchKernelGGL(copy_i32_kernel, dim3(ngrid), dim3(256), 0, stream, lab_a, lab_b,
+                               (int64_t)num_nodes);
+            if (num_edges > 0)
+                hipLaunchKernelGGL(min_label_kernel, dim3(egrid), dim3(256), 0, stream, sender,
+                                   receiver, num_edges, num_nodes, lab_a, lab_b);
+            int32_t *t = lab_a; lab_a = lab_b; lab_b = t;
+        }
+        hipLaunchKernelGGL(gather_kernel, dim3(ngrid), dim3(256), 0, stream, lab_a, order,
+                           reinterpret_cast<int32_t *>(keys_in), (int64_t)num_nodes);
+        rc = check_hip(hipGetLastError(), "locality_order sweep");
+        if (rc) return rc;
+        size_t temp_bytes = sort_bytes;
+        rc = check_hip(hipcub::DeviceRadixSort::SortPairs(sort_temp, temp_bytes, keys_in, keys_out, order,
+                                                          order_tmp, (int)num_nodes, 0, 32, stream),
+                       "locality_order sort");
+        if (rc) return rc;
+        hipLaunchKernelGGL(copy_i32_kernel, dim3(ngrid), dim3(256), 0, stream, order_tmp, order,
+                           (int64_t)num_nodes);
+    }
+    return check_hip(hipGetLastError(), "locality_order");
 }
 
 int e3j_amd_sort_edges(const int32_t *key, const int32_t *other, int64_t num_edges,

@@ -169,6 +169,17 @@ struct WaveReduce {
 // accumulators (out rows forward, dm rows backward) between them.
 // ---------------------------------------------------------------------------
 
+// Consecutive workgroups of a launch are dealt round-robin to the 8 XCDs, each with its own
+// L2.  Logical block numbers are therefore handed out so that every XCD walks one contiguous
+// eighth of the work list: rows that are neighbours in the list (and, with a locality-aware
+// row order, in space) share an L2.  The grid is padded to a multiple of 8 blocks.
+constexpr int kXcds = 8;
+__device__ __forceinline__ int64_t logical_block() {
+    const unsigned per_xcd = gridDim.x / kXcds;
+    return (int64_t)(blockIdx.x % kXcds) * per_xcd + blockIdx.x / kXcds;
+}
+inline int64_t padded_grid(int64_t blocks) { return (blocks + kXcds - 1) / kXcds * kXcds; }
+
 template <int K, int CPL>
 struct Slice {
     static constexpr int WIDTH = kWave * CPL;                 // channels per wave
@@ -264,14 +275,16 @@ template <int K, int CPL, int WPB, typename... Parts>
 __global__ __launch_bounds__(kWave *WPB) void unrolled_fwd_kernel(
     const float *__restrict__ x, const float *__restrict__ y, const float *__restrict__ s,
     const int32_t *__restrict__ sender, const int32_t *__restrict__ row_ptr,
-    const int32_t *__restrict__ perm, float *__restrict__ out, int num_nodes, float scale) {
+    const int32_t *__restrict__ perm, const int32_t *__restrict__ row_order,
+    float *__restrict__ out, int num_nodes, float scale) {
     constexpr int NP = sizeof...(Parts);
     constexpr int CW = Slice<K, CPL>::COUNT;
-    const int64_t item = (int64_t)blockIdx.x * WPB + threadIdx.y;
+    const int64_t item = logical_block() * WPB + threadIdx.y;
     if (item >= (int64_t)num_nodes * (CW * NP)) return;
     const int part = uniform((int)(item % NP));
     const int slice = uniform((int)((item / NP) % CW));
-    const int r = uniform((int)(item / (NP * CW)));
+    const int q = uniform((int)(item / (NP * CW)));
+    const int r = row_order ? row_order[q] : q;
     dispatch_fwd<K, CPL, 0, Parts...>(part, x, y, s, sender, row_ptr, perm, out, num_nodes, scale, r,
                                       slice, threadIdx.x);
 }
@@ -395,16 +408,17 @@ void unrolled_bwd_kernel(
     const float *__restrict__ x, const float *__restrict__ y, const float *__restrict__ s,
     const float *__restrict__ dm, const int32_t *__restrict__ sender,
     const int32_t *__restrict__ row_ptr, const int32_t *__restrict__ perm,
-    float *__restrict__ dx, float *__restrict__ dy, float *__restrict__ ds, int num_nodes,
-    float scale) {
+    const int32_t *__restrict__ row_order, float *__restrict__ dx, float *__restrict__ dy,
+    float *__restrict__ ds, int num_nodes, float scale) {
     constexpr int NP = sizeof...(Parts);
     constexpr int CW = Slice<K, CPL>::COUNT;
     constexpr bool kAtomicDy = NP * CW > 1;  // several waves add into one dy row
-    const int64_t item = (int64_t)blockIdx.x * WPB + threadIdx.y;
+    const int64_t item = logical_block() * WPB + threadIdx.y;
     if (item >= (int64_t)num_nodes * (CW * NP)) return;
     const int part = uniform((int)(item % NP));
     const int slice = uniform((int)((item / NP) % CW));
-    const int r = uniform((int)(item / (NP * CW)));
+    const int q = uniform((int)(item / (NP * CW)));
+    const int r = row_order ? row_order[q] : q;
     dispatch_bwd<K, CPL, kAtomicDy, 0, Parts...>(part, x, y, s, dm, sender, row_ptr, perm, dx, dy, ds,
                                                  num_nodes, scale, r, slice, threadIdx.x);
 }
@@ -414,10 +428,10 @@ int launch_unrolled_fwd(const e3j_amd_conv_params &p, const float *x, const floa
                         const int32_t *sender, const int32_t *row_ptr, const int32_t *perm,
                         float *out, hipStream_t stream) {
     constexpr int64_t PER_NODE = (int64_t)Slice<K, CPL>::COUNT * sizeof...(Parts);
-    const int64_t blocks = ((int64_t)p.num_nodes * PER_NODE + WPB - 1) / WPB;
+    const int64_t blocks = padded_grid(((int64_t)p.num_nodes * PER_NODE + WPB - 1) / WPB);
     if (blocks > 0x7fffffffLL) return set_error(E3J_AMD_INVALID_ARGUMENT, "convolution: grid too large");
     hipLaunchKernelGGL((unrolled_fwd_kernel<K, CPL, WPB, Parts...>), dim3((unsigned)blocks),
-                       dim3(kWave, WPB), 0, stream, x, y, s, sender, row_ptr, perm, out,
+                       dim3(kWave, WPB), 0, stream, x, y, s, sender, row_ptr, perm, p.row_order, out,
                        p.num_nodes, p.coef_scale);
     return check_hip(hipGetLastError(), "convolution forward launch");
 }
@@ -435,11 +449,11 @@ int launch_unrolled_bwd(const e3j_amd_conv_params &p, const float *x, const floa
     }
     rc = launch_zero_padding(p, sender, row_ptr, perm, dy, ds, stream);
     if (rc) return rc;
-    const int64_t blocks = ((int64_t)p.num_nodes * PER_NODE + WPB - 1) / WPB;
+    const int64_t blocks = padded_grid(((int64_t)p.num_nodes * PER_NODE + WPB - 1) / WPB);
     if (blocks > 0x7fffffffLL) return set_error(E3J_AMD_INVALID_ARGUMENT, "convolution_bwd: grid too large");
     hipLaunchKernelGGL((unrolled_bwd_kernel<K, CPL, WPB, Parts...>), dim3((unsigned)blocks),
-                       dim3(kWave, WPB), 0, stream, x, y, s, dm, sender, row_ptr, perm, dx, dy, ds,
-                       p.num_nodes, p.coef_scale);
+                       dim3(kWave, WPB), 0, stream, x, y, s, dm, sender, row_ptr, perm, p.row_order,
+                       dx, dy, ds, p.num_nodes, p.coef_scale);
     return check_hip(hipGetLastError(), "convolution backward launch");
 }
 

@@ -83,6 +83,26 @@ def sort_edges(key: torch.Tensor, other: torch.Tensor, num_nodes: int):
     return perm, other_sorted, row_ptr
 
 
+def locality_order(sender: torch.Tensor, receiver: torch.Tensor, num_nodes: int,
+                   rounds: int = 4) -> torch.Tensor:
+    """Processing order of the nodes in which graph neighbours are close together (int32 permutation).
+
+    Kernels that walk rows in this order gather sender rows that the rows running beside them
+    gather too, so those rows are served from cache.  Results do not depend on the order.
+    """
+    device = _require_device(sender, receiver)
+    sender, receiver = _as_index(sender), _as_index(receiver)
+    order = torch.empty(num_nodes, dtype=INDEX_DTYPE, device=device)
+    lib = _lib.load()
+    ws = torch.empty(max(int(lib.e3j_amd_order_workspace_bytes(num_nodes)), 256), dtype=torch.uint8,
+                     device=device)
+    with torch.cuda.device(device):
+        _lib.check(lib.e3j_amd_locality_order(sender.data_ptr(), receiver.data_ptr(), sender.numel(),
+                                              num_nodes, int(rounds), order.data_ptr(), ws.data_ptr(),
+                                              _stream_ptr(device)))
+    return order
+
+
 class GraphCSR:
     """Edges grouped by receiver (`src/e3j/data/graph.py:38-73`)."""
 

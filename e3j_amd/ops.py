@@ -24,8 +24,8 @@ import torch
 
 from . import _lib
 from .coef import Coef4D
-from .graph import (DUMMY_INDEX, INDEX_DTYPE, csr_row_ptr, fold_endpoints, sort_edges,
-                    wrap_global_index)
+from .graph import (DUMMY_INDEX, INDEX_DTYPE, csr_row_ptr, fold_endpoints, locality_order,
+                    sort_edges, wrap_global_index)
 from .options import GraphOrdering, Layout, config
 
 
@@ -120,7 +120,7 @@ def _stream(device) -> int:
 
 
 def _fill_params(meta: _Meta, x: torch.Tensor, y: torch.Tensor, s: torch.Tensor, forward: bool,
-                 use_signature: bool = True):
+                 use_signature: bool = True, row_order: torch.Tensor | None = None):
     layout = meta.layout
     if layout == Layout.TRAILING_CHANNELS:
         num_x, channels = x.shape[1], x.shape[2]
@@ -137,7 +137,8 @@ def _fill_params(meta: _Meta, x: torch.Tensor, y: torch.Tensor, s: torch.Tensor,
         num_nodes=int(x.shape[0]), num_edges=int(y.shape[0]), num_coef=table.num_coef,
         num_x=dims[0], num_y=dims[1], num_out=dims[2], num_scalars=dims[3], channels=int(channels),
         layout=layout.value, val_dtype=val_code, coef_idx_bytes=table.idx_bytes,
-        signature=sig, coef_scale=scale, debug=int(cfg.debug_level))
+        signature=sig, coef_scale=scale, debug=int(cfg.debug_level),
+        row_order=row_order.data_ptr() if row_order is not None else None)
     return p, table
 
 
@@ -154,23 +155,32 @@ def _check_operands(x, y, s, sender, receiver):
         raise TypeError("x, y and s must share one dtype")
 
 
+def _row_order(sender_l: torch.Tensor, receiver_l: torch.Tensor, n: int):
+    """Locality-aware processing order of the rows, or None when switched off."""
+    rounds = config().locality_rounds
+    if rounds <= 0 or n < 2 or sender_l.numel() == 0:
+        return None
+    return locality_order(sender_l, receiver_l, n, rounds)
+
+
 def _forward_graph(meta: _Meta, sender: torch.Tensor, receiver: torch.Tensor):
-    """CSR used by the forward kernel: `(other, row_ptr, perm)`."""
+    """CSR used by the forward kernel: `(other, row_ptr, perm, row_order)`."""
     n = meta.num_nodes
     sender_l, receiver_l = wrap_global_index(sender, n), wrap_global_index(receiver, n)
+    order = _row_order(sender_l, receiver_l, n)
     if meta.ordering == GraphOrdering.RECEIVER:
-        return sender_l.contiguous(), csr_row_ptr(receiver_l, n), None
+        return sender_l.contiguous(), csr_row_ptr(receiver_l, n), None, order
     if meta.ordering == GraphOrdering.SENDER:
         # aggregate over reversed edges; y parities are folded into the coefficients
-        return receiver_l.contiguous(), csr_row_ptr(sender_l, n), None
+        return receiver_l.contiguous(), csr_row_ptr(sender_l, n), None, order
     perm, sender_sorted, row_ptr = sort_edges(receiver_l, sender_l, n)
-    return sender_sorted, row_ptr, perm
+    return sender_sorted, row_ptr, perm, order
 
 
-def _raw_forward(meta: _Meta, x, y, s, sender, receiver) -> torch.Tensor:
+def _raw_forward(meta: _Meta, x, y, s, sender, receiver, graph=None) -> torch.Tensor:
     x, y, s = x.contiguous(), y.contiguous(), s.contiguous()
-    p, table = _fill_params(meta, x, y, s, forward=True)
-    other, row_ptr, perm = _forward_graph(meta, sender, receiver)
+    other, row_ptr, perm, order = graph if graph is not None else _forward_graph(meta, sender, receiver)
+    p, table = _fill_params(meta, x, y, s, forward=True, row_order=order)
     if meta.layout == Layout.TRAILING_CHANNELS:
         out = torch.empty((x.shape[0], meta.params.num_out, x.shape[2]), dtype=x.dtype, device=x.device)
     else:
@@ -183,25 +193,32 @@ def _raw_forward(meta: _Meta, x, y, s, sender, receiver) -> torch.Tensor:
     return out
 
 
-def _raw_backward(meta: _Meta, x, y, s, dm, sender, receiver):
+def _raw_backward(meta: _Meta, x, y, s, dm, sender, receiver, graph=None):
+    """`graph`: the forward's `(other, row_ptr, perm, row_order)` when it can be reused."""
     x, y, s, dm = x.contiguous(), y.contiguous(), s.contiguous(), dm.contiguous()
     n = meta.num_nodes
-    sender_l, receiver_l = wrap_global_index(sender, n), wrap_global_index(receiver, n)
     dx, dy, ds = torch.empty_like(x), torch.empty_like(y), torch.empty_like(s)
     lib = _lib.load()
     deterministic = config().deterministic
-    if meta.ordering == GraphOrdering.SENDER:
-        # already grouped by sender: rows own their dx, no permutation
-        group_receiver, other, row_ptr, perm = False, receiver_l.contiguous(), csr_row_ptr(sender_l, n), None
-    elif deterministic:
-        perm, other, row_ptr = sort_edges(sender_l, receiver_l, n)
-        group_receiver = False
-    elif meta.ordering == GraphOrdering.RECEIVER:
-        group_receiver, other, row_ptr, perm = True, sender_l.contiguous(), csr_row_ptr(receiver_l, n), None
-    else:
-        perm, other, row_ptr = sort_edges(receiver_l, sender_l, n)
+    reuse = graph is not None and not deterministic and meta.ordering != GraphOrdering.SENDER
+    if reuse:
+        other, row_ptr, perm, order = graph
         group_receiver = True
-    p, table = _fill_params(meta, x, y, s, forward=False, use_signature=group_receiver)
+    else:
+        sender_l, receiver_l = wrap_global_index(sender, n), wrap_global_index(receiver, n)
+        order = graph[3] if graph is not None else _row_order(sender_l, receiver_l, n)
+        if meta.ordering == GraphOrdering.SENDER:
+            # already grouped by sender: rows own their dx, no permutation
+            group_receiver, other, row_ptr, perm = False, receiver_l.contiguous(), csr_row_ptr(sender_l, n), None
+        elif deterministic:
+            perm, other, row_ptr = sort_edges(sender_l, receiver_l, n)
+            group_receiver = False
+        elif meta.ordering == GraphOrdering.RECEIVER:
+            group_receiver, other, row_ptr, perm = True, sender_l.contiguous(), csr_row_ptr(receiver_l, n), None
+        else:
+            perm, other, row_ptr = sort_edges(receiver_l, sender_l, n)
+            group_receiver = True
+    p, table = _fill_params(meta, x, y, s, forward=False, use_signature=group_receiver, row_order=order)
     fn = lib.e3j_amd_convolution_bwd_receiver if group_receiver else lib.e3j_amd_convolution_bwd_sender
     with torch.cuda.device(x.device):
         _lib.check(fn(ctypes.byref(p), table.device(x.device).data_ptr(), x.data_ptr(), y.data_ptr(),
@@ -223,24 +240,27 @@ def _sum(*terms):
 
 class _Convolution(torch.autograd.Function):
     @staticmethod
-    def forward(ctx, x, y, s, sender, receiver, meta):
+    def forward(ctx, x, y, s, sender, receiver, meta, graph=None):
         ctx.meta = meta
         ctx.save_for_backward(x, y, s, sender, receiver)
-        return _raw_forward(meta, x, y, s, sender, receiver)
+        # the adjacency prepared here also serves the backward of this call
+        ctx.graph = graph if graph is not None else _forward_graph(meta, sender, receiver)
+        return _raw_forward(meta, x, y, s, sender, receiver, ctx.graph)
 
     @staticmethod
     def backward(ctx, dm):
         x, y, s, sender, receiver = ctx.saved_tensors
-        dx, dy, ds = _ConvolutionBwd.apply(x, y, s, dm, sender, receiver, ctx.meta)
-        return dx, dy, ds, None, None, None
+        dx, dy, ds = _ConvolutionBwd.apply(x, y, s, dm, sender, receiver, ctx.meta, ctx.graph)
+        return dx, dy, ds, None, None, None, None
 
 
 class _ConvolutionBwd(torch.autograd.Function):
     @staticmethod
-    def forward(ctx, x, y, s, dm, sender, receiver, meta):
+    def forward(ctx, x, y, s, dm, sender, receiver, meta, graph=None):
         ctx.meta = meta
+        ctx.graph = graph
         ctx.save_for_backward(x, y, s, dm, sender, receiver)
-        return _raw_backward(meta, x, y, s, dm, sender, receiver)
+        return _raw_backward(meta, x, y, s, dm, sender, receiver, graph)
 
     @staticmethod
     def backward(ctx, ddx, ddy, dds):
@@ -249,11 +269,13 @@ class _ConvolutionBwd(torch.autograd.Function):
         x, y, s, dm, sender, receiver = ctx.saved_tensors
         meta = ctx.meta
 
+        graph = ctx.graph
+
         def conv(a, b, c):
-            return _Convolution.apply(a, b, c, sender, receiver, meta)
+            return _Convolution.apply(a, b, c, sender, receiver, meta, graph)
 
         def conv_bwd(a, b, c):
-            return _ConvolutionBwd.apply(a, b, c, dm, sender, receiver, meta)
+            return _ConvolutionBwd.apply(a, b, c, dm, sender, receiver, meta, graph)
 
         d_dm, d_x, d_y, d_s = [], [], [], []
         if ddx is not None:
@@ -271,7 +293,7 @@ class _ConvolutionBwd(torch.autograd.Function):
             gx, gy, _ = conv_bwd(x, y, dds)
             d_x.append(gx)
             d_y.append(gy)
-        return _sum(*d_x), _sum(*d_y), _sum(*d_s), _sum(*d_dm), None, None, None
+        return _sum(*d_x), _sum(*d_y), _sum(*d_s), _sum(*d_dm), None, None, None, None
 
 
 def _make_meta(coef, x, y, s, params, graph_ordering, y_parity, layout) -> _Meta:

@@ -83,6 +83,9 @@ class Config:
     debug_level: int = 0
     #: atomic-free backward for `dx` (bit-reproducible, slower).
     deterministic: bool = False
+    #: sweeps of label propagation behind the locality-aware row order of the kernels
+    #: (0 = rows are processed in index order).
+    locality_rounds: int = 2
 
 
 class _ConfigHolder:
@@ -92,6 +95,7 @@ class _ConfigHolder:
         self._current = Config(
             debug_level=int(os.environ.get("E3J_AMD_DEBUG", "0")),
             deterministic=os.environ.get("E3J_AMD_DETERMINISTIC", "0") not in ("0", ""),
+            locality_rounds=int(os.environ.get("E3J_AMD_LOCALITY_ROUNDS", "2")),
         )
 
     def __call__(self, **updates) -> Config:

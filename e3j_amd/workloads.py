@@ -138,14 +138,26 @@ def _normal(shape, seed: int, device) -> torch.Tensor:
     return torch.randn(shape, dtype=torch.float32, device=device, generator=gen)
 
 
+def morton_order(positions: np.ndarray, box: float, bits: int = 10) -> np.ndarray:
+    """Permutation sorting points along a Z-order curve (atoms numbered coherently in space)."""
+    cells = np.clip((positions / box * (1 << bits)).astype(np.int64), 0, (1 << bits) - 1)
+    code = np.zeros(len(positions), dtype=np.int64)
+    for b in range(bits):
+        for axis in range(3):
+            code |= ((cells[:, axis] >> b) & 1) << (3 * b + axis)
+    return np.argsort(code, kind="stable")
+
+
 def make_workload(name: str, num_atoms: int, x_irreps: str, l_max: int, out_irreps: str,
                   channels: int, seeds: tuple, *, neighbours: float | None = 30.0,
                   box: float | None = None, periodic: bool = True, cutoff: float = 5.0,
-                  device="cpu") -> Workload:
+                  device="cpu", spatial_sort: bool = False) -> Workload:
     seed_pos, seed_x, seed_s, seed_dm = seeds
     if box is None:
         box = periodic_box_length(num_atoms, neighbours, cutoff)
     pos = np.random.default_rng(seed_pos).uniform(0.0, box, size=(num_atoms, 3))
+    if spatial_sort:  # same atoms, numbered along a space-filling curve instead of at random
+        pos = pos[morton_order(pos, box)]
     sender, receiver, vec = radius_graph(pos, cutoff, box if periodic else None)
     y_irreps = "+".join(f"{l}{'e' if l % 2 == 0 else 'o'}" for l in range(l_max + 1))
     module = Convolution((x_irreps, y_irreps), out_irreps, graph_ordering="RECEIVER")
@@ -174,11 +186,11 @@ def config2(scale: float = 1.0, out_irreps: str = "0e+1o+2e", device="cpu") -> W
     return make_workload("cfg2", n, "0e+1o+2e", 3, out_irreps, 64, (11, 12, 13, 14), device=device)
 
 
-def config3(scale: float = 1.0, channels: int = 128, device="cpu") -> Workload:
+def config3(scale: float = 1.0, channels: int = 128, device="cpu", spatial_sort: bool = False) -> Workload:
     """32 000 atoms, ~30 neighbours (~1M edges), 128 channels, 0e..3o x lmax 3 -> 0e..3o."""
     n = max(8, int(32000 * scale))
     return make_workload("cfg3", n, "0e+1o+2e+3o", 3, "0e+1o+2e+3o", channels, (21, 22, 23, 24),
-                         device=device)
+                         device=device, spatial_sort=spatial_sort)
 
 
 def config4(scale: float = 1.0, device="cpu") -> Workload:

@@ -63,6 +63,10 @@ typedef struct e3j_amd_conv_params {
     int32_t signature;      /* id from e3j_amd_find_signature, or -1: table-driven kernel */
     float   coef_scale;     /* unrolled kernels: table = coef_scale * built-in table (1 by default) */
     int32_t debug;
+    /* Optional processing order of the CSR rows (device, num_nodes entries, a permutation of
+     * 0..num_nodes-1), e.g. from e3j_amd_locality_order; NULL = natural order.  It only
+     * changes which rows run together (cache reuse of gathered rows), never the results. */
+    const int32_t *row_order;
 } e3j_amd_conv_params;
 
 /* Message of the last failure on the calling thread ("" if none). */
@@ -129,6 +133,17 @@ int e3j_amd_csr_row_ptr(const int32_t *key, int64_t num_edges, int32_t num_nodes
 int e3j_amd_sort_edges(const int32_t *key, const int32_t *other, int64_t num_edges,
                        int32_t num_nodes, int32_t *perm, int32_t *other_sorted,
                        int32_t *row_ptr, void *workspace, void *stream);
+
+/* e3j_amd_locality_order: a processing order of the nodes in which nodes that are close in
+ *   the graph are close in the order, from `rounds` sweeps of minimum-label propagation over
+ *   the edges (clusters of nodes within `rounds` hops of a local minimum id), ordered
+ *   hierarchically.  order (N): a permutation.  workspace: >= e3j_amd_order_workspace_bytes().
+ *   No counterpart in the reference, whose kernels walk the rows in index order
+ *   (lib/e3j_ops/cuda/convolution/fwd.cuh:346). */
+size_t e3j_amd_order_workspace_bytes(int32_t num_nodes);
+int e3j_amd_locality_order(const int32_t *sender, const int32_t *receiver, int64_t num_edges,
+                           int32_t num_nodes, int32_t rounds, int32_t *order, void *workspace,
+                           void *stream);
 
 /* XLA-FFI handlers (C ABI of xla/ffi/api/c_api.h): `XLA_FFI_Error* handler(XLA_FFI_CallFrame*)`.
  * Operand order of "convolution"/"convolution_bwd" as in lib/e3j_ops/ffi/e3j_ops.h:457-472,575-594;

@@ -4,7 +4,8 @@ import numpy as np
 import pytest
 import torch
 
-from e3j_amd.graph import DUMMY_INDEX, GraphCSR, csr_row_ptr, fold_endpoints, sort_edges, wrap_global_index
+from e3j_amd.graph import (DUMMY_INDEX, GraphCSR, csr_row_ptr, fold_endpoints, locality_order, sort_edges,
+                           wrap_global_index)
 from oracle import conv_oracle as O
 
 pytestmark = pytest.mark.gpu
@@ -56,3 +57,28 @@ def test_graph_csr_with_dummy_edges():
 def test_cpu_tensors_are_rejected():
     with pytest.raises(RuntimeError, match="no CPU implementation"):
         csr_row_ptr(torch.zeros(4, dtype=torch.int32), 4)
+
+
+@pytest.mark.parametrize("rounds", [0, 1, 3])
+def test_locality_order_is_a_permutation_that_groups_neighbours(rounds):
+    from e3j_amd import workloads as W
+    w = W.config2(0.2)
+    n = w.num_nodes
+    order = locality_order(w.sender.cuda(), w.receiver.cuda(), n, rounds).cpu().numpy()
+    assert sorted(order.tolist()) == list(range(n))
+    if rounds == 0:
+        assert order.tolist() == list(range(n))
+        return
+    # neighbours in the graph end up closer in the order than in a random numbering
+    position = np.empty(n, dtype=np.int64)
+    position[order] = np.arange(n)
+    snd, rcv = w.sender.numpy(), w.receiver.numpy()
+    window = 64
+    close = (np.abs(position[snd] - position[rcv]) <= window).mean()
+    close_before = (np.abs(snd.astype(np.int64) - rcv) <= window).mean()
+    assert close > 3.0 * close_before, (close, close_before)
+    # padding endpoints are ignored
+    snd2 = snd.copy()
+    snd2[::7] = DUMMY_INDEX
+    order2 = locality_order(dev(snd2), w.receiver.cuda(), n, rounds).cpu().numpy()
+    assert sorted(order2.tolist()) == list(range(n))

@@ -51,6 +51,18 @@ def test_autograd_matches_oracle(ordering, deterministic):
     _check(p, out, grads)
 
 
+def test_row_order_does_not_change_results():
+    """The locality-aware row order only changes which rows run together: forward bits are identical."""
+    p = _problem(12, N=200, E=3000, K=32)
+    args = [dev(p[k]) for k in ("x", "y", "s")]
+    snd, rcv = dev(p["snd"]), dev(p["rcv"])
+    outs = []
+    for rounds in (0, 1, 4):
+        with e3j_amd.config.use(locality_rounds=rounds):
+            outs.append(convolution(p["coef"], *args, snd, rcv, p["params"]))
+    assert torch.equal(outs[0], outs[1]) and torch.equal(outs[0], outs[2])
+
+
 def test_convolution_bwd_direct_and_deterministic_bits():
     p = _problem(2, N=64, E=2000, K=32)
     args = [dev(p[k]) for k in ("x", "y", "s")]
