@@ -101,7 +101,7 @@ class AbiCalls:
             self.perm, self.other = None, w.sender.contiguous()
             self.ptr = csr_row_ptr(w.receiver, w.num_nodes)
         rounds = config().locality_rounds
-        self.order = locality_order(w.sender, w.receiver, w.num_nodes, rounds) if rounds > 0 else None
+        self.order = locality_order(self.other, self.ptr, w.num_nodes, rounds) if rounds > 0 else None
         self.params.row_order = self.order.data_ptr() if self.order is not None else None
         self.out = torch.empty_like(w.dm)
         self.dx, self.dy, self.ds = torch.empty_like(w.x), torch.empty_like(w.y), torch.empty_like(w.s)

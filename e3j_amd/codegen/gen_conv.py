@@ -14,8 +14,9 @@ Per edge and lane (a lane owns CPL channels; `y` is the same for all lanes):
     p_m      = |c_m| * y[k_m]                      one product per distinct (|c|, k)
     w_ij     = sum of +-p_m                         the edge's (output, x) weights
     forward  : msg_i = sum_j w_ij x_j ;  acc_i += s_l(i) msg_i
-    backward : g_i = dm_i s_l(i) ;  dx_j += w_ij g_i ;  ds_l += dm_i sum_j w_ij x_j
-               dy_k += c_ijk * sum_channels(g_i x_j)
+    backward : g_i = dm_i s_l(i) ;  dx_j += w_ij g_i
+               a_k = sum_ij c_ijk (dm_i x_j) per path ;  ds_l = sum_k y_k a_k ;
+               dy_k += sum_channels(s_l a_k)
 
 `python -m e3j_amd.codegen.gen_conv` rewrites `e3j_amd/csrc/generated/`.
 """
@@ -219,6 +220,15 @@ def emit_edge_fwd(p: Part) -> list[str]:
 
 
 def emit_edge_bwd(p: Part) -> list[str]:
+    """Backward of one edge for the paths of a part.
+
+    Per path l (rows i, x columns j, y components k):
+        a_k   = sum_{ij} c_ijk (dm_i x_j)          channel-wise, independent of s and y
+        ds_l  = sum_k y_k a_k
+        dy_k += sum_channels s_l a_k
+        dx_j += w_ij (dm_i s_l),  w_ij = sum_k c_ijk y_k
+    One product dm_i x_j per (i, j) pair serves both ds and dy.
+    """
     t = p.t
     lines = ["    // dx (this part's x rows) and dy (all Y) are written here; ds rows are stored path by path.",
              "    template <int C, int K>",
@@ -229,15 +239,16 @@ def emit_edge_bwd(p: Part) -> list[str]:
     dx_init, dy_init = set(), set()
     for l, rows in p.paths.items():
         ids, defs = Table.path_products(rows)
-        lines.append(f"        {{  // path {l}: rows {min(rows)}..{max(rows)}")
+        ks = sorted({k for cols in rows.values() for terms in cols.values() for _, k in terms})
+        lines.append(f"        {{  // path {l}: rows {min(rows)}..{max(rows)}, y components {ks[0]}..{ks[-1]}")
         lines += defs
-        lines.append("            Vec<C> dsl;")
-        first_ds = True
+        a_init = set()
+        for k in ks:
+            lines.append(f"            Vec<C> a{k};")
         for i, cols in rows.items():
             zi = p.zi[i]
             lines.append("            {")
             lines.append(f"                const Vec<C> g = vmulv(dm[{zi}], s[{p.sl[l]}]);")
-            first_tp = True
             for j, terms in cols.items():
                 xj = p.xj[j]
                 expr, bare = Table.weight_expr(terms, ids)
@@ -249,25 +260,27 @@ def emit_edge_bwd(p: Part) -> list[str]:
                 else:
                     lines.append(f"                dx[{xj}] = vmul(g, {expr});")
                     dx_init.add(j)
-                if first_tp:
-                    lines.append(f"                Vec<C> tp = vmul(x[{xj}], {expr});")
-                    first_tp = False
-                else:
-                    lines.append(f"                tp = vfma(x[{xj}], {expr}, tp);")
-                lines.append(f"                {{ const float h = hsum(vmulv(g, x[{xj}]));")
+                lines.append(f"                {{ const Vec<C> pr = vmulv(dm[{zi}], x[{xj}]);")
                 for c, k in terms:
-                    if k in dy_init:
-                        lines.append(f"                  dy[{k}] = fmaf(h, {_lit(c)}, dy[{k}]);")
+                    if k in a_init:
+                        lines.append(f"                  a{k} = vfma(pr, {_lit(c)}, a{k});")
                     else:
-                        lines.append(f"                  dy[{k}] = h * {_lit(c)};")
-                        dy_init.add(k)
+                        lines.append(f"                  a{k} = vmul(pr, {_lit(c)});")
+                        a_init.add(k)
                 lines.append("                }")
-            if first_ds:
-                lines.append(f"                dsl = vmulv(dm[{zi}], tp);")
-                first_ds = False
-            else:
-                lines.append(f"                dsl = vfmav(dm[{zi}], tp, dsl);")
             lines.append("            }")
+        first = True
+        for k in ks:
+            if first:
+                lines.append(f"            Vec<C> dsl = vmul(a{k}, y[{k}]);")
+                first = False
+            else:
+                lines.append(f"            dsl = vfma(a{k}, y[{k}], dsl);")
+            if k in dy_init:
+                lines.append(f"            dy[{k}] += hsum(vmulv(s[{p.sl[l]}], a{k}));")
+            else:
+                lines.append(f"            dy[{k}] = hsum(vmulv(s[{p.sl[l]}], a{k}));")
+                dy_init.add(k)
         lines.append(f"            if (active) store_vec<C>(ds_row + {l} * K, dsl);")
         lines.append("        }")
     for l in p.zero_paths:  # paths no coefficient touches get exact zeros

@@ -181,6 +181,9 @@ __global__ void generic_bwd_kernel(const Coef4D<Idx, Val> *__restrict__ coef, in
 
 // dy/ds rows of padding edges: positions past the last row, or whose gathered
 // endpoint is out of range (lib/e3j_ops/cuda/convolution/bwd.cuh:308-319).
+// A wave inspects 64 positions at a time (one per lane) and then zeroes the rows of the
+// padding positions among them together; live graphs have few, so this is one pass over
+// the index array.
 template <typename Val>
 __global__ void zero_padding_edges_kernel(const int32_t *__restrict__ other,
                                           const int32_t *__restrict__ row_ptr,
@@ -189,13 +192,21 @@ __global__ void zero_padding_edges_kernel(const int32_t *__restrict__ other,
                                           Val *__restrict__ ds, int64_t ds_row) {
     const int lane = threadIdx.x;
     const int64_t live_end = row_ptr[num_nodes];
-    for (int64_t e = (int64_t)blockIdx.x * blockDim.y + threadIdx.y; e < num_edges;
-         e += (int64_t)gridDim.x * blockDim.y) {
-        const int o = other[e];
-        if (e < live_end && (unsigned)o < (unsigned)num_nodes) continue;
-        const int64_t ee = perm ? (int64_t)perm[e] : e;
-        for (int k = lane; k < num_y; k += kWave) dy[ee * num_y + k] = Val(0);
-        for (int64_t t = lane; t < ds_row; t += kWave) ds[ee * ds_row + t] = Val(0);
+    const int64_t stride = (int64_t)gridDim.x * blockDim.y * kWave;
+    for (int64_t base = ((int64_t)blockIdx.x * blockDim.y + threadIdx.y) * kWave; base < num_edges;
+         base += stride) {
+        const int64_t e = base + lane;
+        bool padding = false;
+        if (e < num_edges) padding = e >= live_end || (unsigned)other[e] >= (unsigned)num_nodes;
+        uint64_t mask = __ballot(padding);
+        while (mask) {
+            const int src = __ffsll((unsigned long long)mask) - 1;
+            mask &= mask - 1;
+            const int64_t pos = base + src;
+            const int64_t ee = perm ? (int64_t)perm[pos] : pos;
+            for (int k = lane; k < num_y; k += kWave) dy[ee * num_y + k] = Val(0);
+            for (int64_t t = lane; t < ds_row; t += kWave) ds[ee * ds_row + t] = Val(0);
+        }
     }
 }
 
@@ -249,7 +260,7 @@ template <typename Val>
 int zero_padding(const e3j_amd_conv_params &p, const int32_t *other, const int32_t *row_ptr,
                  const int32_t *perm, Val *dy, Val *ds, hipStream_t stream) {
     if (p.num_edges == 0) return E3J_AMD_OK;
-    const int64_t zblocks = std::min<int64_t>((p.num_edges + 3) / 4, 4096);
+    const int64_t zblocks = std::min<int64_t>((p.num_edges + 4 * kWave - 1) / (4 * kWave), 2048);
     hipLaunchKernelGGL(zero_padding_edges_kernel<Val>, dim3((unsigned)zblocks), dim3(kWave, 4), 0,
                        stream, other, row_ptr, perm, p.num_nodes, p.num_edges, dy, p.num_y, ds,
                        (int64_t)p.num_scalars * p.channels);

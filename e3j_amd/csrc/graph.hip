@@ -13,12 +13,24 @@
 namespace e3j_amd {
 namespace {
 
+// Histogram of the in-range keys into counts[key + 1].  A thread walks a short run of
+// consecutive positions and issues one atomic per run of equal keys: sorted keys (the
+// common case) then cost one atomic per thread instead of one per edge on a hot address.
+constexpr int kCountChunk = 16;
 __global__ void count_keys_kernel(const int32_t *__restrict__ key, int64_t num_edges, int num_nodes,
                                   int32_t *__restrict__ counts) {
-    const int64_t stride = (int64_t)gridDim.x * blockDim.x;
-    for (int64_t e = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; e < num_edges; e += stride) {
-        const int k = key[e];
-        if ((unsigned)k < (unsigned)num_nodes) atomicAdd(&counts[k + 1], 1);
+    const int64_t stride = (int64_t)gridDim.x * blockDim.x * kCountChunk;
+    for (int64_t base = ((int64_t)blockIdx.x * blockDim.x + threadIdx.x) * kCountChunk;
+         base < num_edges; base += stride) {
+        const int64_t end = base + kCountChunk < num_edges ? base + kCountChunk : num_edges;
+        int run_key = key[base], run = 1;
+        for (int64_t e = base + 1; e < end; e++) {
+            const int k = key[e];
+            if (k == run_key) { run++; continue; }
+            if ((unsigned)run_key < (unsigned)num_nodes) atomicAdd(&counts[run_key + 1], run);
+            run_key = k; run = 1;
+        }
+        if ((unsigned)run_key < (unsigned)num_nodes) atomicAdd(&counts[run_key + 1], run);
     }
 }
 
@@ -35,18 +47,19 @@ __global__ void gather_kernel(const int32_t *__restrict__ src, const int32_t *__
         dst[i] = src[perm[i]];
 }
 
-// One sweep of minimum-label propagation: next[n] = min(cur[n], cur[m] for every neighbour m).
-__global__ void min_label_kernel(const int32_t *__restrict__ sender,
-                                 const int32_t *__restrict__ receiver, int64_t num_edges,
-                                 int num_nodes, const int32_t *__restrict__ cur,
-                                 int32_t *__restrict__ next) {
-    const int64_t stride = (int64_t)gridDim.x * blockDim.x;
-    for (int64_t e = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; e < num_edges; e += stride) {
-        const int a = sender[e], b = receiver[e];
-        if ((unsigned)a >= (unsigned)num_nodes || (unsigned)b >= (unsigned)num_nodes) continue;
-        atomicMin(&next[b], cur[a]);
-        atomicMin(&next[a], cur[b]);
+// One sweep of minimum-label propagation over a CSR adjacency:
+// next[n] = min(cur[n], cur[m] for every m in row n).  One thread per row, no atomics.
+__global__ void min_label_kernel(const int32_t *__restrict__ other,
+                                 const int32_t *__restrict__ row_ptr, int num_nodes,
+                                 const int32_t *__restrict__ cur, int32_t *__restrict__ next) {
+    const int n = blockIdx.x * blockDim.x + threadIdx.x;
+    if (n >= num_nodes) return;
+    int best = cur[n];
+    for (int e = row_ptr[n]; e < row_ptr[n + 1]; e++) {
+        const int m = other[e];
+        if ((unsigned)m < (unsigned)num_nodes) best = min(best, cur[m]);
     }
+    next[n] = best;
 }
 
 __global__ void copy_i32_kernel(const int32_t *__restrict__ src, int32_t *__restrict__ dst, int64_t n) {
@@ -77,14 +90,29 @@ int row_ptr_impl(const int32_t *key, int64_t num_edges, int32_t num_nodes, int32
     int rc = launch_fill_zero(row_ptr, sizeof(int32_t) * ((size_t)num_nodes + 1), stream);
     if (rc) return rc;
     if (num_edges > 0) {
-        hipLaunchKernelGGL(count_keys_kernel, dim3(grid_for(num_edges)), dim3(256), 0, stream, key,
-                           num_edges, num_nodes, row_ptr);
+        hipLaunchKernelGGL(count_keys_kernel, dim3(grid_for((num_edges + kCountChunk - 1) / kCountChunk)),
+                           dim3(256), 0, stream, key, num_edges, num_nodes, row_ptr);
         rc = check_hip(hipGetLastError(), "csr count launch");
         if (rc) return rc;
     }
     return check_hip(hipcub::DeviceScan::InclusiveSum(temp, temp_bytes, row_ptr, row_ptr,
                                                       num_nodes + 1, stream),
                      "csr scan");
+}
+
+// Global node ids of a sharded graph reduced to shard-local ids; the sentinel stays.
+__global__ void wrap_index_kernel(const int32_t *__restrict__ index, int64_t n, int32_t num_nodes,
+                                  int32_t *__restrict__ out) {
+    const int64_t stride = (int64_t)gridDim.x * blockDim.x;
+    for (int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; i < n; i += stride) {
+        const int32_t v = index[i];
+        int32_t r = v;
+        if (v != INT32_MAX) {
+            r = v % num_nodes;          // Python semantics: the result takes the divisor's sign
+            if (r < 0) r += num_nodes;
+        }
+        out[i] = r;
+    }
 }
 
 }  // namespace
@@ -111,19 +139,30 @@ int e3j_amd_csr_row_ptr(const int32_t *key, int64_t num_edges, int32_t num_nodes
                         static_cast<hipStream_t>(stream_));
 }
 
+int e3j_amd_wrap_index(const int32_t *index, int64_t n, int32_t num_nodes, int32_t *out,
+                       void *stream_) {
+    if (n < 0 || num_nodes <= 0)
+        return set_error(E3J_AMD_INVALID_ARGUMENT, "wrap_index: bad sizes");
+    if (n == 0) return E3J_AMD_OK;
+    if (index == nullptr || out == nullptr)
+        return set_error(E3J_AMD_INVALID_ARGUMENT, "wrap_index: null operand");
+    hipLaunchKernelGGL(wrap_index_kernel, dim3(grid_for(n)), dim3(256), 0, (hipStream_t)stream_,
+                       index, n, num_nodes, out);
+    return check_hip(hipGetLastError(), "wrap_index");
+}
+
 size_t e3j_amd_order_workspace_bytes(int32_t num_nodes) {
     if (num_nodes < 0) return 0;
     // [sort temp | label a | label b | keys in | keys out | order tmp]
     return align_up(sort_temp_bytes(num_nodes)) + 5 * align_up(sizeof(int32_t) * (size_t)num_nodes) + 256;
 }
 
-int e3j_amd_locality_order(const int32_t *sender, const int32_t *receiver, int64_t num_edges,
-                           int32_t num_nodes, int32_t rounds, int32_t *order, void *workspace,
-                           void *stream_) {
-    if (num_nodes < 0 || num_edges < 0 || rounds < 0 || rounds > 64)
+int e3j_amd_locality_order(const int32_t *other, const int32_t *row_ptr, int32_t num_nodes,
+                           int32_t rounds, int32_t *order, void *workspace, void *stream_) {
+    if (num_nodes < 0 || rounds < 0 || rounds > 64)
         return set_error(E3J_AMD_INVALID_ARGUMENT, "locality_order: bad sizes");
     if (num_nodes == 0) return E3J_AMD_OK;
-    if (order == nullptr || workspace == nullptr || (num_edges > 0 && (!sender || !receiver)))
+    if (order == nullptr || workspace == nullptr || row_ptr == nullptr)
         return set_error(E3J_AMD_INVALID_ARGUMENT, "locality_order: null operand");
     hipStream_t stream = static_cast<hipStream_t>(stream_);
     unsigned char *ws = static_cast<unsigned char *>(workspace);
@@ -135,7 +174,8 @@ int e3j_amd_locality_order(const int32_t *sender, const int32_t *receiver, int64
     uint32_t *keys_in = reinterpret_cast<uint32_t *>(ws + align_up(sort_bytes) + 2 * vec);
     uint32_t *keys_out = reinterpret_cast<uint32_t *>(ws + align_up(sort_bytes) + 3 * vec);
     int32_t *order_tmp = reinterpret_cast<int32_t *>(ws + align_up(sort_bytes) + 4 * vec);
-    const unsigned ngrid = grid_for(num_nodes), egrid = grid_for(num_edges);
+    const unsigned ngrid = grid_for(num_nodes);
+    const unsigned rows_grid = (unsigned)((num_nodes + 255) / 256);
 
     hipLaunchKernelGGL(iota_kernel, dim3(ngrid), dim3(256), 0, stream, lab_a, (int64_t)num_nodes);
     hipLaunchKernelGGL(iota_kernel, dim3(ngrid), dim3(256), 0, stream, order, (int64_t)num_nodes);
@@ -147,11 +187,8 @@ int e3j_amd_locality_order(const int32_t *sender, const int32_t *receiver, int64
     int done = 0;
     for (int level = 1; level <= rounds; level *= 2) {
         for (; done < level; done++) {
-            hipLaunchKernelGGL(copy_i32_kernel, dim3(ngrid), dim3(256), 0, stream, lab_a, lab_b,
-                               (int64_t)num_nodes);
-            if (num_edges > 0)
-                hipLaunchKernelGGL(min_label_kernel, dim3(egrid), dim3(256), 0, stream, sender,
-                                   receiver, num_edges, num_nodes, lab_a, lab_b);
+            hipLaunchKernelGGL(min_label_kernel, dim3(rows_grid), dim3(256), 0, stream, other, row_ptr,
+                               num_nodes, lab_a, lab_b);
             int32_t *t = lab_a; lab_a = lab_b; lab_b = t;
         }
         hipLaunchKernelGGL(gather_kernel, dim3(ngrid), dim3(256), 0, stream, lab_a, order,

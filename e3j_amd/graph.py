@@ -83,22 +83,24 @@ def sort_edges(key: torch.Tensor, other: torch.Tensor, num_nodes: int):
     return perm, other_sorted, row_ptr
 
 
-def locality_order(sender: torch.Tensor, receiver: torch.Tensor, num_nodes: int,
-                   rounds: int = 4) -> torch.Tensor:
+def locality_order(other: torch.Tensor, row_ptr: torch.Tensor, num_nodes: int,
+                   rounds: int = 2) -> torch.Tensor:
     """Processing order of the nodes in which graph neighbours are close together (int32 permutation).
 
-    Kernels that walk rows in this order gather sender rows that the rows running beside them
-    gather too, so those rows are served from cache.  Results do not depend on the order.
+    `(other, row_ptr)`: a CSR adjacency (e.g. senders per receiver-sorted position and
+    `receiver_ptr`).  Kernels that walk rows in this order gather sender rows that the rows
+    running beside them gather too, so those rows are served from cache.  Results do not
+    depend on the order.
     """
-    device = _require_device(sender, receiver)
-    sender, receiver = _as_index(sender), _as_index(receiver)
+    device = _require_device(other, row_ptr)
+    other, row_ptr = _as_index(other), _as_index(row_ptr)
     order = torch.empty(num_nodes, dtype=INDEX_DTYPE, device=device)
     lib = _lib.load()
     ws = torch.empty(max(int(lib.e3j_amd_order_workspace_bytes(num_nodes)), 256), dtype=torch.uint8,
                      device=device)
     with torch.cuda.device(device):
-        _lib.check(lib.e3j_amd_locality_order(sender.data_ptr(), receiver.data_ptr(), sender.numel(),
-                                              num_nodes, int(rounds), order.data_ptr(), ws.data_ptr(),
+        _lib.check(lib.e3j_amd_locality_order(other.data_ptr(), row_ptr.data_ptr(), num_nodes,
+                                              int(rounds), order.data_ptr(), ws.data_ptr(),
                                               _stream_ptr(device)))
     return order
 
@@ -147,8 +149,16 @@ class GraphCSR:
 
 def wrap_global_index(index: torch.Tensor, num_nodes: int) -> torch.Tensor:
     """Reduce modulo `num_nodes`, keeping the sentinel (`src/e3j/ops/convolution.py:39-51`)."""
-    local = torch.where(is_dummy_index(index), index, index % num_nodes)
-    return local.to(INDEX_DTYPE)
+    if index.device.type != "cuda" or index.dtype != INDEX_DTYPE or num_nodes <= 0:
+        # host-side planning and wide index types: plain tensor arithmetic
+        local = torch.where(is_dummy_index(index), index, index % max(num_nodes, 1))
+        return local.to(INDEX_DTYPE)
+    index = index.contiguous()
+    out = torch.empty_like(index)
+    with torch.cuda.device(index.device):
+        _lib.check(_lib.load().e3j_amd_wrap_index(index.data_ptr(), index.numel(), num_nodes,
+                                                  out.data_ptr(), _stream_ptr(index.device)))
+    return out
 
 
 def fold_endpoints(group: torch.Tensor, guard: torch.Tensor, axis_size: int, num_nodes: int):

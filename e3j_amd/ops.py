@@ -155,26 +155,26 @@ def _check_operands(x, y, s, sender, receiver):
         raise TypeError("x, y and s must share one dtype")
 
 
-def _row_order(sender_l: torch.Tensor, receiver_l: torch.Tensor, n: int):
-    """Locality-aware processing order of the rows, or None when switched off."""
+def _row_order(other: torch.Tensor, row_ptr: torch.Tensor, n: int):
+    """Locality-aware processing order of the rows of a CSR, or None when switched off."""
     rounds = config().locality_rounds
-    if rounds <= 0 or n < 2 or sender_l.numel() == 0:
+    if rounds <= 0 or n < 2 or other.numel() == 0:
         return None
-    return locality_order(sender_l, receiver_l, n, rounds)
+    return locality_order(other, row_ptr, n, rounds)
 
 
 def _forward_graph(meta: _Meta, sender: torch.Tensor, receiver: torch.Tensor):
     """CSR used by the forward kernel: `(other, row_ptr, perm, row_order)`."""
     n = meta.num_nodes
     sender_l, receiver_l = wrap_global_index(sender, n), wrap_global_index(receiver, n)
-    order = _row_order(sender_l, receiver_l, n)
     if meta.ordering == GraphOrdering.RECEIVER:
-        return sender_l.contiguous(), csr_row_ptr(receiver_l, n), None, order
-    if meta.ordering == GraphOrdering.SENDER:
+        other, row_ptr, perm = sender_l.contiguous(), csr_row_ptr(receiver_l, n), None
+    elif meta.ordering == GraphOrdering.SENDER:
         # aggregate over reversed edges; y parities are folded into the coefficients
-        return receiver_l.contiguous(), csr_row_ptr(sender_l, n), None, order
-    perm, sender_sorted, row_ptr = sort_edges(receiver_l, sender_l, n)
-    return sender_sorted, row_ptr, perm, order
+        other, row_ptr, perm = receiver_l.contiguous(), csr_row_ptr(sender_l, n), None
+    else:
+        perm, other, row_ptr = sort_edges(receiver_l, sender_l, n)
+    return other, row_ptr, perm, _row_order(other, row_ptr, n)
 
 
 def _raw_forward(meta: _Meta, x, y, s, sender, receiver, graph=None) -> torch.Tensor:
@@ -206,7 +206,6 @@ def _raw_backward(meta: _Meta, x, y, s, dm, sender, receiver, graph=None):
         group_receiver = True
     else:
         sender_l, receiver_l = wrap_global_index(sender, n), wrap_global_index(receiver, n)
-        order = graph[3] if graph is not None else _row_order(sender_l, receiver_l, n)
         if meta.ordering == GraphOrdering.SENDER:
             # already grouped by sender: rows own their dx, no permutation
             group_receiver, other, row_ptr, perm = False, receiver_l.contiguous(), csr_row_ptr(sender_l, n), None
@@ -218,6 +217,7 @@ def _raw_backward(meta: _Meta, x, y, s, dm, sender, receiver, graph=None):
         else:
             perm, other, row_ptr = sort_edges(receiver_l, sender_l, n)
             group_receiver = True
+        order = graph[3] if graph is not None else _row_order(other, row_ptr, n)
     p, table = _fill_params(meta, x, y, s, forward=False, use_signature=group_receiver, row_order=order)
     fn = lib.e3j_amd_convolution_bwd_receiver if group_receiver else lib.e3j_amd_convolution_bwd_sender
     with torch.cuda.device(x.device):

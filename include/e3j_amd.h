@@ -134,16 +134,22 @@ int e3j_amd_sort_edges(const int32_t *key, const int32_t *other, int64_t num_edg
                        int32_t num_nodes, int32_t *perm, int32_t *other_sorted,
                        int32_t *row_ptr, void *workspace, void *stream);
 
+/* e3j_amd_wrap_index: global node ids of a sharded graph to shard-local ids,
+ *   out[i] = index[i] mod num_nodes, the sentinel INT32_MAX kept
+ *   (replaces wrap_global_index, src/e3j/ops/convolution.py:39-51). */
+int e3j_amd_wrap_index(const int32_t *index, int64_t n, int32_t num_nodes, int32_t *out,
+                       void *stream);
+
 /* e3j_amd_locality_order: a processing order of the nodes in which nodes that are close in
  *   the graph are close in the order, from `rounds` sweeps of minimum-label propagation over
- *   the edges (clusters of nodes within `rounds` hops of a local minimum id), ordered
- *   hierarchically.  order (N): a permutation.  workspace: >= e3j_amd_order_workspace_bytes().
+ *   a CSR adjacency (other, row_ptr): clusters of nodes within `rounds` hops of a local
+ *   minimum id, ordered hierarchically.  order (N): a permutation.
+ *   workspace: >= e3j_amd_order_workspace_bytes().
  *   No counterpart in the reference, whose kernels walk the rows in index order
  *   (lib/e3j_ops/cuda/convolution/fwd.cuh:346). */
 size_t e3j_amd_order_workspace_bytes(int32_t num_nodes);
-int e3j_amd_locality_order(const int32_t *sender, const int32_t *receiver, int64_t num_edges,
-                           int32_t num_nodes, int32_t rounds, int32_t *order, void *workspace,
-                           void *stream);
+int e3j_amd_locality_order(const int32_t *other, const int32_t *row_ptr, int32_t num_nodes,
+                           int32_t rounds, int32_t *order, void *workspace, void *stream);
 
 /* XLA-FFI handlers (C ABI of xla/ffi/api/c_api.h): `XLA_FFI_Error* handler(XLA_FFI_CallFrame*)`.
  * Operand order of "convolution"/"convolution_bwd" as in lib/e3j_ops/ffi/e3j_ops.h:457-472,575-594;

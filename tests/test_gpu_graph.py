@@ -64,7 +64,8 @@ def test_locality_order_is_a_permutation_that_groups_neighbours(rounds):
     from e3j_amd import workloads as W
     w = W.config2(0.2)
     n = w.num_nodes
-    order = locality_order(w.sender.cuda(), w.receiver.cuda(), n, rounds).cpu().numpy()
+    ptr = csr_row_ptr(w.receiver.cuda(), n)
+    order = locality_order(w.sender.cuda(), ptr, n, rounds).cpu().numpy()
     assert sorted(order.tolist()) == list(range(n))
     if rounds == 0:
         assert order.tolist() == list(range(n))
@@ -80,5 +81,23 @@ def test_locality_order_is_a_permutation_that_groups_neighbours(rounds):
     # padding endpoints are ignored
     snd2 = snd.copy()
     snd2[::7] = DUMMY_INDEX
-    order2 = locality_order(dev(snd2), w.receiver.cuda(), n, rounds).cpu().numpy()
+    order2 = locality_order(dev(snd2), ptr, n, rounds).cpu().numpy()
     assert sorted(order2.tolist()) == list(range(n))
+
+
+@pytest.mark.parametrize("num_nodes", [1, 7, 1000])
+def test_wrap_global_index_matches_the_tensor_arithmetic(num_nodes):
+    """Global ids of a sharded graph modulo the shard size, sentinel kept
+    (`src/e3j/ops/convolution.py:39-51`); the int32 device path against int64 host arithmetic."""
+    rng = np.random.default_rng(num_nodes)
+    index = rng.integers(0, 5 * num_nodes, size=4099).astype(np.int32)
+    index[rng.random(index.size) < 0.1] = DUMMY_INDEX
+    index[:3] = [0, num_nodes - 1, num_nodes]
+    want = np.where(index == DUMMY_INDEX, index, index % num_nodes)
+    got = wrap_global_index(torch.from_numpy(index).cuda(), num_nodes)
+    assert got.dtype == torch.int32
+    np.testing.assert_array_equal(got.cpu().numpy(), want)
+    # wide indices take the tensor-arithmetic route and agree
+    got64 = wrap_global_index(torch.from_numpy(index.astype(np.int64)).cuda(), num_nodes)
+    np.testing.assert_array_equal(got64.cpu().numpy(), want)
+    assert wrap_global_index(torch.empty(0, dtype=torch.int32, device="cuda"), num_nodes).numel() == 0
