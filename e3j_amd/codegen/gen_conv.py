@@ -281,10 +281,10 @@ def emit_edge_bwd(p: Part) -> list[str]:
             else:
                 lines.append(f"            dy[{k}] = hsum(vmulv(s[{p.sl[l]}], a{k}));")
                 dy_init.add(k)
-        lines.append(f"            if (active) store_vec<C>(ds_row + {l} * K, dsl);")
+        lines.append(f"            if (active) store_stream<C>(ds_row + {l} * K, dsl);")
         lines.append("        }")
     for l in p.zero_paths:  # paths no coefficient touches get exact zeros
-        lines.append(f"        if (active) store_vec<C>(ds_row + {l} * K, vzero<C>());")
+        lines.append(f"        if (active) store_stream<C>(ds_row + {l} * K, vzero<C>());")
     for k in range(t.Y):
         if k not in dy_init:
             lines.append(f"        dy[{k}] = 0.f;")

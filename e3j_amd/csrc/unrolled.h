@@ -90,10 +90,38 @@ __device__ __forceinline__ Vec<4> load_vec<4>(const float *p) {
     r.v[0] = t.x; r.v[1] = t.y; r.v[2] = t.z; r.v[3] = t.w;
     return r;
 }
+typedef float f32x2 __attribute__((ext_vector_type(2)));
+typedef float f32x4 __attribute__((ext_vector_type(4)));
+// Loads and stores of data that is touched once (radial weights, output rows): marked
+// non-temporal so that they do not displace the gathered sender rows from the L2.
+template <int C>
+__device__ __forceinline__ Vec<C> load_stream(const float *p);
+template <>
+__device__ __forceinline__ Vec<1> load_stream<1>(const float *p) {
+    Vec<1> r;
+    r.v[0] = __builtin_nontemporal_load(p);
+    return r;
+}
+template <>
+__device__ __forceinline__ Vec<2> load_stream<2>(const float *p) {
+    const f32x2 t = __builtin_nontemporal_load(reinterpret_cast<const f32x2 *>(p));
+    Vec<2> r;
+    r.v[0] = t.x; r.v[1] = t.y;
+    return r;
+}
+template <>
+__device__ __forceinline__ Vec<4> load_stream<4>(const float *p) {
+    const f32x4 t = __builtin_nontemporal_load(reinterpret_cast<const f32x4 *>(p));
+    Vec<4> r;
+    r.v[0] = t.x; r.v[1] = t.y; r.v[2] = t.z; r.v[3] = t.w;
+    return r;
+}
 template <int C>
 __device__ __forceinline__ void store_vec(float *p, const Vec<C> &a);
 template <>
-__device__ __forceinline__ void store_vec<1>(float *p, const Vec<1> &a) { *p = a.v[0]; }
+__device__ __forceinline__ void store_vec<1>(float *p, const Vec<1> &a) {
+    *p = a.v[0];
+}
 template <>
 __device__ __forceinline__ void store_vec<2>(float *p, const Vec<2> &a) {
     *reinterpret_cast<float2 *>(p) = make_float2(a.v[0], a.v[1]);
@@ -101,6 +129,24 @@ __device__ __forceinline__ void store_vec<2>(float *p, const Vec<2> &a) {
 template <>
 __device__ __forceinline__ void store_vec<4>(float *p, const Vec<4> &a) {
     *reinterpret_cast<float4 *>(p) = make_float4(a.v[0], a.v[1], a.v[2], a.v[3]);
+}
+template <int C>
+__device__ __forceinline__ void store_stream(float *p, const Vec<C> &a);
+template <>
+__device__ __forceinline__ void store_stream<1>(float *p, const Vec<1> &a) {
+    __builtin_nontemporal_store(a.v[0], p);
+}
+template <>
+__device__ __forceinline__ void store_stream<2>(float *p, const Vec<2> &a) {
+    f32x2 t;
+    t.x = a.v[0]; t.y = a.v[1];
+    __builtin_nontemporal_store(t, reinterpret_cast<f32x2 *>(p));
+}
+template <>
+__device__ __forceinline__ void store_stream<4>(float *p, const Vec<4> &a) {
+    f32x4 t;
+    t.x = a.v[0]; t.y = a.v[1]; t.z = a.v[2]; t.w = a.v[3];
+    __builtin_nontemporal_store(t, reinterpret_cast<f32x4 *>(p));
 }
 
 __device__ __forceinline__ int uniform(int v) { return __builtin_amdgcn_readfirstlane(v); }
@@ -227,7 +273,7 @@ __device__ __forceinline__ void unrolled_fwd_part(
 #pragma unroll
         for (int j = 0; j < NX; j++) xn[j] = load_vec<CPL>(xr + Part::kX[j] * K);
 #pragma unroll
-        for (int l = 0; l < NS; l++) sn[l] = load_vec<CPL>(sr + Part::kS[l] * K);
+        for (int l = 0; l < NS; l++) sn[l] = load_stream<CPL>(sr + Part::kS[l] * K);
 #pragma unroll
         for (int k = 0; k < Y; k++) yn[k] = yr[k];
     };
@@ -249,7 +295,7 @@ __device__ __forceinline__ void unrolled_fwd_part(
     if (active) {
         float *orow = out + (int64_t)r * (Z * K) + c0;
 #pragma unroll
-        for (int i = 0; i < NZ; i++) store_vec<CPL>(orow + Part::kZ[i] * K, vmul(acc[i], scale));
+        for (int i = 0; i < NZ; i++) store_stream<CPL>(orow + Part::kZ[i] * K, vmul(acc[i], scale));
     }
 }
 
@@ -314,7 +360,7 @@ __device__ __forceinline__ void unrolled_bwd_part(
         const float *zr = dm + (int64_t)r * (Z * K) + c0;
 #pragma unroll
         for (int i = 0; i < NZ; i++) {
-            dmr[i] = vmul(load_vec<CPL>(zr + Part::kZ[i] * K), scale);
+            dmr[i] = vmul(load_stream<CPL>(zr + Part::kZ[i] * K), scale);
             if (!active) dmr[i] = vzero<CPL>();  // idle lanes must add nothing to dy
         }
     }
@@ -338,7 +384,7 @@ __device__ __forceinline__ void unrolled_bwd_part(
 #pragma unroll
         for (int j = 0; j < NX; j++) xn[j] = load_vec<CPL>(xr + Part::kX[j] * K);
 #pragma unroll
-        for (int l = 0; l < NS; l++) sn[l] = load_vec<CPL>(sr + Part::kS[l] * K);
+        for (int l = 0; l < NS; l++) sn[l] = load_stream<CPL>(sr + Part::kS[l] * K);
 #pragma unroll
         for (int k = 0; k < Y; k++) yn[k] = yr[k];
     };
