@@ -56,6 +56,14 @@ LAUNCH = {
 }
 
 
+#: leading-channels layout: (waves per block, parts) variants; the forward pass is never split.
+LAUNCH_LEADING = {
+    32: dict(fwd=[(4, 1)], bwd=[(4, 1)]),
+    64: dict(fwd=[(4, 1)], bwd=[(4, 2), (4, 1), (4, 3)]),
+    128: dict(fwd=[(4, 1)], bwd=[(4, 2), (4, 1), (4, 3)]),
+}
+
+
 def _f32_bits(v: float) -> int:
     return struct.unpack("<I", struct.pack("<f", float(v)))[0]
 
@@ -191,6 +199,11 @@ def _arr(name: str, values) -> str:
     return f"    static constexpr int {name}[{max(len(values), 1)}] = {{{body}}};"
 
 
+def _mask(indices) -> str:
+    """Bit set of small indices; indices past 63 (no leading-layout kernels then) are dropped."""
+    return hex(sum(1 << i for i in indices if i < 64))
+
+
 def emit_edge_fwd(p: Part) -> list[str]:
     lines = ["    template <int C>",
              "    __device__ static __forceinline__ void edge_fwd(const Vec<C> *x, const float *y,",
@@ -230,12 +243,11 @@ def emit_edge_bwd(p: Part) -> list[str]:
     One product dm_i x_j per (i, j) pair serves both ds and dy.
     """
     t = p.t
-    lines = ["    // dx (this part's x rows) and dy (all Y) are written here; ds rows are stored path by path.",
-             "    template <int C, int K>",
+    lines = ["    // dx (this part's x rows) and dy (all Y) are written here; ds rows go to `ds` path by path.",
+             "    template <int C, typename DsSink>",
              "    __device__ static __forceinline__ void edge_bwd(const Vec<C> *x, const float *y,",
              "                                                     const Vec<C> *s, const Vec<C> *dm,",
-             "                                                     Vec<C> *dx, float *dy, float *ds_row,",
-             "                                                     bool active) {"]
+             "                                                     Vec<C> *dx, float *dy, const DsSink &ds) {"]
     dx_init, dy_init = set(), set()
     for l, rows in p.paths.items():
         ids, defs = Table.path_products(rows)
@@ -281,10 +293,10 @@ def emit_edge_bwd(p: Part) -> list[str]:
             else:
                 lines.append(f"            dy[{k}] = hsum(vmulv(s[{p.sl[l]}], a{k}));")
                 dy_init.add(k)
-        lines.append(f"            if (active) store_stream<C>(ds_row + {l} * K, dsl);")
+        lines.append(f"            ds.template put<{l}>(dsl);")
         lines.append("        }")
     for l in p.zero_paths:  # paths no coefficient touches get exact zeros
-        lines.append(f"        if (active) store_stream<C>(ds_row + {l} * K, vzero<C>());")
+        lines.append(f"        ds.template put<{l}>(vzero<C>());")
     for k in range(t.Y):
         if k not in dy_init:
             lines.append(f"        dy[{k}] = 0.f;")
@@ -297,7 +309,10 @@ def emit_part(struct_name: str, p: Part) -> list[str]:
     out = [f"struct {struct_name} {{",
            f"    static constexpr int X = {t.X}, Y = {t.Y}, S = {t.S}, Z = {t.Z};",
            f"    static constexpr int NX = {len(p.kX)}, NS = {len(p.kS)}, NZ = {len(p.kZ)};",
-           _arr("kX", p.kX), _arr("kS", p.kS), _arr("kZ", p.kZ), ""]
+           _arr("kX", p.kX), _arr("kS", p.kS), _arr("kZ", p.kZ),
+           "    // x coordinates whose dx, and paths whose ds, this part writes (bit per index)",
+           f"    static constexpr unsigned long long kDxMask = {_mask(p.kX)}ull, "
+           f"kDsMask = {_mask(list(p.kS) + list(p.zero_paths))}ull;", ""]
     out += emit_edge_fwd(p)
     out.append("")
     out += emit_edge_bwd(p)
@@ -330,7 +345,9 @@ def emit_signature(sig_id: int, name: str, x_irreps: str, y_irreps: str, out_fil
         "namespace {",
         "",
     ]
-    splits = sorted({v[2] for v in launch["fwd"] + launch["bwd"]})
+    lead = LAUNCH_LEADING[channels] if (t.X <= 64 and t.S <= 64) else None
+    splits = sorted({v[2] for v in launch["fwd"] + launch["bwd"]} |
+                    ({v[1] for v in lead["fwd"] + lead["bwd"]} if lead else set()))
     part_names = {}
     for zs in splits:
         names = []
@@ -339,44 +356,73 @@ def emit_signature(sig_id: int, name: str, x_irreps: str, y_irreps: str, out_fil
             out += emit_part(sname, part)
             names.append(sname)
         part_names[zs] = ", ".join(names)
+    fwd_args = ["    const float *, const float *, const float *, const int32_t *, const int32_t *,",
+                "    const int32_t *, const int32_t *, float *, int, float);"]
+    bwd_args = ["    const float *, const float *, const float *, const float *, const int32_t *,",
+                "    const int32_t *, const int32_t *, const int32_t *, float *, float *, float *, int, float);"]
     out += ["}  // namespace", "", "// both passes: the device pass needs the kernels instantiated"]
     for cpl, wpb, zs in launch["fwd"]:
-        out += [f"template __global__ void unrolled_fwd_kernel<{channels}, {cpl}, {wpb}, {part_names[zs]}>(",
-                "    const float *, const float *, const float *, const int32_t *, const int32_t *,",
-                "    const int32_t *, const int32_t *, float *, int, float);"]
+        out += [f"template __global__ void unrolled_fwd_kernel<{channels}, {cpl}, {wpb}, {part_names[zs]}>("] + fwd_args
     for cpl, wpb, zs in launch["bwd"]:
-        out += [f"template __global__ void unrolled_bwd_kernel<{channels}, {cpl}, {wpb}, {part_names[zs]}>(",
-                "    const float *, const float *, const float *, const float *, const int32_t *,",
-                "    const int32_t *, const int32_t *, const int32_t *, float *, float *, float *, int, float);"]
-    out += ["", "// host pass only: the registry entry holds host function pointers",
+        out += [f"template __global__ void unrolled_bwd_kernel<{channels}, {cpl}, {wpb}, {part_names[zs]}>("] + bwd_args
+    if lead:
+        for wpb, zs in lead["fwd"]:
+            out += [f"template __global__ void unrolled_fwd_leading_kernel<{channels}, {wpb}, {part_names[zs]}>("] + fwd_args
+        for wpb, zs in lead["bwd"]:
+            out += [f"template __global__ void unrolled_bwd_leading_kernel<{channels}, {wpb}, {part_names[zs]}>("] + bwd_args
+
+    fwd_sig = ["(const e3j_amd_conv_params &p, const float *x, const float *y, const float *s,",
+               "                   const int32_t *sender, const int32_t *row_ptr, const int32_t *perm,",
+               "                   float *out, hipStream_t stream) {"]
+    bwd_sig = ["(const e3j_amd_conv_params &p, const float *x, const float *y, const float *s,",
+               "                   const float *dm, const int32_t *sender, const int32_t *row_ptr,",
+               "                   const int32_t *perm, float *dx, float *dy, float *ds, hipStream_t stream) {"]
+
+    def switch(variants, call):
+        body = ["    switch (VARIANT) {"]
+        for n, v in reversed(list(enumerate(variants))):
+            label = f"case {n}:" if n else "default:"
+            body.append(f"        {label} return {call(v)}")
+        return body + ["    }", "}", ""]
+
+    out += ["", "// host pass only: the registry entries hold host function pointers",
             "#if !defined(__HIP_DEVICE_COMPILE__)",
             f"static const float kVal[] = {{{vals}}};",
             f"static const uint8_t kIdx[] = {{{idxs}}};",
-            "",
-            "static int run_fwd(const e3j_amd_conv_params &p, const float *x, const float *y, const float *s,",
-            "                   const int32_t *sender, const int32_t *row_ptr, const int32_t *perm,",
-            "                   float *out, hipStream_t stream) {",
-            "    switch (tuning().fwd_variant) {"]
-    for n, (cpl, wpb, zs) in reversed(list(enumerate(launch["fwd"]))):
-        label = f"case {n}:" if n else "default:"
-        out.append(f"        {label} return launch_unrolled_fwd<{channels}, {cpl}, {wpb}, {part_names[zs]}>("
-                   "p, x, y, s, sender, row_ptr, perm, out, stream);")
-    out += ["    }", "}", "",
-            "static int run_bwd(const e3j_amd_conv_params &p, const float *x, const float *y, const float *s,",
-            "                   const float *dm, const int32_t *sender, const int32_t *row_ptr,",
-            "                   const int32_t *perm, float *dx, float *dy, float *ds, hipStream_t stream) {",
-            "    switch (tuning().bwd_variant) {"]
-    for n, (cpl, wpb, zs) in reversed(list(enumerate(launch["bwd"]))):
-        label = f"case {n}:" if n else "default:"
-        out.append(f"        {label} return launch_unrolled_bwd<{channels}, {cpl}, {wpb}, {t.Y}, {t.X}, "
-                   f"{part_names[zs]}>(p, x, y, s, dm, sender, row_ptr, perm, dx, dy, ds, stream);")
-    out += ["    }", "}", "",
-            f"extern const Signature kSignature_{sig_id} = {{",
+            ""]
+    out += ["static int run_fwd" + fwd_sig[0]] + fwd_sig[1:]
+    out += [ln.replace("VARIANT", "tuning().fwd_variant") for ln in switch(
+        launch["fwd"], lambda v: f"launch_unrolled_fwd<{channels}, {v[0]}, {v[1]}, {part_names[v[2]]}>("
+                                 "p, x, y, s, sender, row_ptr, perm, out, stream);")]
+    out += ["static int run_bwd" + bwd_sig[0]] + bwd_sig[1:]
+    out += [ln.replace("VARIANT", "tuning().bwd_variant") for ln in switch(
+        launch["bwd"], lambda v: f"launch_unrolled_bwd<{channels}, {v[0]}, {v[1]}, {t.Y}, {t.X}, "
+                                 f"{part_names[v[2]]}>(p, x, y, s, dm, sender, row_ptr, perm, dx, dy, ds, stream);")]
+    out += [f"extern const Signature kSignature_{2 * sig_id} = {{",
             f'    "{desc}",',
             f"    {t.X}, {t.Y}, {t.Z}, {t.S}, {len(t.val)}, {channels}, E3J_AMD_LAYOUT_TRAILING, kVal, kIdx,",
             "    &run_fwd, &run_bwd,",
-            "};",
-            "#endif",
+            "};", ""]
+    if lead:
+        out += ["static int run_fwd_leading" + fwd_sig[0]] + fwd_sig[1:]
+        out += [ln.replace("VARIANT", "tuning().fwd_variant") for ln in switch(
+            lead["fwd"], lambda v: f"launch_unrolled_fwd_leading<{channels}, {v[0]}, {part_names[v[1]]}>("
+                                   "p, x, y, s, sender, row_ptr, perm, out, stream);")]
+        out += ["static int run_bwd_leading" + bwd_sig[0]] + bwd_sig[1:]
+        out += [ln.replace("VARIANT", "tuning().bwd_variant") for ln in switch(
+            lead["bwd"], lambda v: f"launch_unrolled_bwd_leading<{channels}, {v[0]}, {t.Y}, {t.X}, "
+                                   f"{part_names[v[1]]}>(p, x, y, s, dm, sender, row_ptr, perm, dx, dy, ds, stream);")]
+        out += [f"extern const Signature kSignature_{2 * sig_id + 1} = {{",
+                f'    "{desc.replace("trailing", "leading")}",',
+                f"    {t.X}, {t.Y}, {t.Z}, {t.S}, {len(t.val)}, {channels}, E3J_AMD_LAYOUT_LEADING, kVal, kIdx,",
+                "    &run_fwd_leading, &run_bwd_leading,",
+                "};"]
+    else:  # no leading-layout kernels: an entry that never matches keeps the numbering regular
+        out += [f"extern const Signature kSignature_{2 * sig_id + 1} = {{",
+                f'    "{desc.replace("trailing", "leading (not built)")}",',
+                "    -1, -1, -1, -1, -1, -1, E3J_AMD_LAYOUT_LEADING, nullptr, nullptr, nullptr, nullptr,",
+                "};"]
+    out += ["#endif",
             "",
             "}  // namespace e3j_amd",
             ""]
@@ -415,7 +461,7 @@ def write_all(out_dir: str, signatures=None) -> list[str]:
         wanted.add(fname)
         _write_if_changed(os.path.join(out_dir, fname), emit_signature(n, name, xi, yi, oi, k))
         paths.append(os.path.join(out_dir, fname))
-    _write_if_changed(os.path.join(out_dir, "registry.hip"), emit_registry(len(signatures)))
+    _write_if_changed(os.path.join(out_dir, "registry.hip"), emit_registry(2 * len(signatures)))
     for stale in os.listdir(out_dir):
         if stale.endswith(".hip") and stale not in wanted:
             os.remove(os.path.join(out_dir, stale))

@@ -4,6 +4,9 @@
 #include <cstdlib>
 #include <cstring>
 
+#include <cstdint>
+#include <initializer_list>
+
 #include "common.h"
 
 namespace e3j_amd {
@@ -67,6 +70,16 @@ int validate(const e3j_amd_conv_params *p, const char *op) {
 
 bool missing(const void *ptr, int64_t count) { return count > 0 && ptr == nullptr; }
 
+// The unrolled kernels of the leading-channels layout move rows in 16-byte pieces.
+bool aligned16(std::initializer_list<const void *> ptrs) {
+    for (const void *ptr : ptrs)
+        if (reinterpret_cast<uintptr_t>(ptr) % 16 != 0) return false;
+    return true;
+}
+bool signature_fits(const e3j_amd_conv_params *p, std::initializer_list<const void *> ptrs) {
+    return p->signature >= 0 && (p->layout == E3J_AMD_LAYOUT_TRAILING || aligned16(ptrs));
+}
+
 int finish(const e3j_amd_conv_params *p, hipStream_t stream, int rc, const char *op) {
     if (rc != E3J_AMD_OK || p->debug <= 0) return rc;
     return check_hip(hipStreamSynchronize(stream), op);
@@ -88,7 +101,8 @@ int run_backward(const e3j_amd_conv_params *p, bool group_is_receiver, const voi
         (p->signature < 0 && missing(coef, p->num_coef)))
         return set_error(E3J_AMD_INVALID_ARGUMENT, std::string(op) + ": null operand");
     if (p->num_nodes == 0) return E3J_AMD_OK;
-    if (p->signature >= 0 && group_is_receiver && signature(p->signature).bwd != nullptr) {
+    if (group_is_receiver && signature_fits(p, {x, s, dm, dx, ds}) &&
+        signature(p->signature).bwd != nullptr) {
         rc = signature(p->signature).bwd(*p, static_cast<const float *>(x),
                                          static_cast<const float *>(y), static_cast<const float *>(s),
                                          static_cast<const float *>(dm), other, row_ptr, edge_perm,
@@ -126,11 +140,15 @@ int e3j_amd_convolution_fwd(const e3j_amd_conv_params *p, const void *coef, cons
         missing(sender, p->num_edges) || missing(y, p->num_edges) || missing(s, p->num_edges) ||
         (p->signature < 0 && missing(coef, p->num_coef)))
         return set_error(E3J_AMD_INVALID_ARGUMENT, "convolution: null operand");
-    if (p->signature >= 0) {
+    if (signature_fits(p, {x, s, out})) {
         rc = signature(p->signature).fwd(*p, static_cast<const float *>(x), static_cast<const float *>(y),
                                          static_cast<const float *>(s), sender, receiver_ptr,
                                          edge_perm, static_cast<float *>(out), stream);
     } else {
+        if (missing(coef, p->num_coef))
+            return set_error(E3J_AMD_INVALID_ARGUMENT,
+                             "convolution: operands are not 16-byte aligned, which runs the "
+                             "table-driven kernel and needs `coef`");
         rc = launch_generic_fwd(*p, coef, x, y, s, sender, receiver_ptr, edge_perm, out, stream);
     }
     return finish(p, stream, rc, "convolution");

@@ -338,6 +338,19 @@ __global__ __launch_bounds__(kWave *WPB) void unrolled_fwd_kernel(
 // ---------------------------------------------------------------------------
 // backward, receiver-grouped: dm rows resident, x gathered, dx scattered by atomics
 // ---------------------------------------------------------------------------
+
+// Where the generated arithmetic puts the ds value of path L (trailing layout: straight
+// into the edge's row of ds).
+template <int CPL, int K>
+struct DsRows {
+    float *row;
+    bool active;
+    template <int L>
+    __device__ __forceinline__ void put(const Vec<CPL> &v) const {
+        if (active) store_stream<CPL>(row + L * K, v);
+    }
+};
+
 template <typename Part, int K, int CPL, bool kAtomicDy>
 __device__ __forceinline__ void unrolled_bwd_part(
     const float *__restrict__ x, const float *__restrict__ y, const float *__restrict__ s,
@@ -407,8 +420,8 @@ __device__ __forceinline__ void unrolled_bwd_part(
 
         V dxe[NX];
         float dye[Red::P];
-        Part::template edge_bwd<CPL, K>(xc, yc, sc, dmr, dxe, dye, ds + ee * (int64_t)(S * K) + c0,
-                                        active);
+        const DsRows<CPL, K> ds_rows{ds + ee * (int64_t)(S * K) + c0, active};
+        Part::template edge_bwd<CPL>(xc, yc, sc, dmr, dxe, dye, ds_rows);
 #pragma unroll
         for (int k = Y; k < Red::P; k++) dye[k] = 0.f;
 
@@ -469,6 +482,405 @@ void unrolled_bwd_kernel(
                                                  num_nodes, scale, r, slice, threadIdx.x);
 }
 
+// ---------------------------------------------------------------------------
+// Leading-channels layout: a row is (channels, dim), so the channels of a wave are one
+// contiguous block of W * dim floats.  The wave moves such a block with coalesced 16-byte
+// accesses and turns it through its private strip of LDS: lane c reads (or writes) the
+// values of its channel there at an odd row stride, which is free of bank conflicts.
+// The arithmetic between the two turns is the same generated code as for the trailing
+// layout.  LDS operations of one wave complete in order, so the strip needs no barrier,
+// only fences that keep the compiler from moving accesses across the turn.
+// ---------------------------------------------------------------------------
+constexpr int odd_stride(int n) { return (n % 2) ? n : n + 1; }
+constexpr int round4(int n) { return (n + 3) / 4 * 4; }
+
+__device__ __forceinline__ void strip_fence() {
+    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+    __builtin_amdgcn_wave_barrier();
+    __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+}
+
+// Position in a strip (rows of ROW values at stride PAD) of element g of the linear block.
+template <int ROW, int PAD>
+__device__ __forceinline__ int strip_index(int g) {
+    return PAD == ROW ? g : g + (g / ROW) * (PAD - ROW);
+}
+
+template <int K, int X, int S, int Z>
+struct LeadingGeometry {
+    static constexpr int W = K < kWave ? K : kWave;  // channels per wave
+    static constexpr int COUNT = K / W;              // waves per row
+    static_assert(K % W == 0 && W % 4 == 0, "channel count must be a multiple of 4 and of 64 above 64");
+    static constexpr int PX = odd_stride(X), PS = odd_stride(S), PZ = odd_stride(Z);
+    static constexpr int XR = round4(W * PX);        // floats; keeps the s strip 16-byte aligned
+    static constexpr int SR = round4(W * PS);
+    static constexpr int REGION = XR + SR > 4 * PZ ? XR + SR : round4(4 * PZ);
+    // out / dm rows pass through the whole strip in groups of GC channels
+    static constexpr int group() {
+        int g = W;
+        while (g > 4 && g * PZ > REGION) g /= 2;
+        return g;
+    }
+    static constexpr int GC = group();
+    static_assert(W % GC == 0 && GC % 4 == 0, "channel groups must tile the wave");
+};
+
+// N floats (N % 4 == 0) at a 16-byte aligned address, dealt to the lanes in 16-byte pieces.
+template <int N>
+struct LinearBlock {
+    static_assert(N % 4 == 0, "blocks are moved in 16-byte pieces");
+    static constexpr int PIECES = N / 4;
+    static constexpr int NV = (PIECES + kWave - 1) / kWave;
+    static constexpr bool EXACT = NV * kWave == PIECES;
+    f32x4 v[NV];
+
+    template <bool kStream>
+    __device__ __forceinline__ void load(const float *src, int lane) {
+        const f32x4 *p = reinterpret_cast<const f32x4 *>(src);
+#pragma unroll
+        for (int i = 0; i < NV; i++) {
+            const int idx = i * kWave + lane;
+            if (EXACT || idx < PIECES) v[i] = kStream ? __builtin_nontemporal_load(p + idx) : p[idx];
+        }
+    }
+    __device__ __forceinline__ void store(float *dst, int lane) const {
+        f32x4 *p = reinterpret_cast<f32x4 *>(dst);
+#pragma unroll
+        for (int i = 0; i < NV; i++) {
+            const int idx = i * kWave + lane;
+            if (EXACT || idx < PIECES) __builtin_nontemporal_store(v[i], p + idx);
+        }
+    }
+    template <int ROW, int PAD>
+    __device__ __forceinline__ void to_strip(float *strip, int lane) const {
+#pragma unroll
+        for (int i = 0; i < NV; i++) {
+            const int idx = i * kWave + lane;
+            if (EXACT || idx < PIECES) {
+                if (PAD == ROW) {
+                    reinterpret_cast<f32x4 *>(strip)[idx] = v[i];
+                } else {
+#pragma unroll
+                    for (int t = 0; t < 4; t++) strip[strip_index<ROW, PAD>(4 * idx + t)] = v[i][t];
+                }
+            }
+        }
+    }
+    template <int ROW, int PAD>
+    __device__ __forceinline__ void from_strip(const float *strip, int lane) {
+#pragma unroll
+        for (int i = 0; i < NV; i++) {
+            const int idx = i * kWave + lane;
+            if (EXACT || idx < PIECES) {
+                if (PAD == ROW) {
+                    v[i] = reinterpret_cast<const f32x4 *>(strip)[idx];
+                } else {
+#pragma unroll
+                    for (int t = 0; t < 4; t++) v[i][t] = strip[strip_index<ROW, PAD>(4 * idx + t)];
+                }
+            }
+        }
+    }
+};
+
+// Bit i of the result: element i * 64 + lane of a linear (rows of ROW) block belongs to a
+// column of `mask`.  Computed once per wave; the per-edge loops then test one bit.
+template <int N, int ROW>
+__device__ __forceinline__ unsigned column_predicate(unsigned long long mask, int lane) {
+    constexpr int STEPS = (N + kWave - 1) / kWave;
+    static_assert(STEPS <= 32, "block too large for a 32-bit predicate");
+    unsigned pred = 0;
+#pragma unroll
+    for (int i = 0; i < STEPS; i++) {
+        const int g = i * kWave + lane;
+        if (g < N && ((mask >> (g % ROW)) & 1ull)) pred |= 1u << i;
+    }
+    return pred;
+}
+
+// forward ---------------------------------------------------------------------
+template <typename Part, int K>
+__device__ __forceinline__ void unrolled_fwd_leading(
+    const float *__restrict__ x, const float *__restrict__ y, const float *__restrict__ s,
+    const int32_t *__restrict__ sender, const int32_t *__restrict__ row_ptr,
+    const int32_t *__restrict__ perm, float *__restrict__ out, int num_nodes, float scale, int r,
+    int slice, int lane, float *strip) {
+    constexpr int NX = Part::NX, NS = Part::NS, NZ = Part::NZ, Y = Part::Y;
+    constexpr int X = Part::X, S = Part::S, Z = Part::Z;
+    static_assert(NZ == Z, "the forward pass of the leading layout is not split into parts");
+    using G = LeadingGeometry<K, X, S, Z>;
+    using V = Vec<1>;
+    constexpr int W = G::W, GC = G::GC;
+    float *strip_x = strip, *strip_s = strip + G::XR;
+
+    const bool active = lane < W;
+    const int cl = active ? lane : 0;  // idle lanes (channel count below 64) mirror channel 0
+    const int64_t ch0 = (int64_t)slice * W;
+
+    V acc[NZ];
+#pragma unroll
+    for (int i = 0; i < NZ; i++) acc[i] = vzero<1>();
+
+    int e = row_ptr[r];
+    const int e1 = row_ptr[r + 1];
+
+    LinearBlock<W * X> xl;
+    LinearBlock<W * S> sl;
+    float yn[Y];
+    bool valid_n = false;
+    auto fetch = [&](int pos) {
+        const int snd = sender[pos];
+        valid_n = (unsigned)snd < (unsigned)num_nodes;
+        const int row = valid_n ? snd : 0;
+        const int64_t ee = perm ? (int64_t)perm[pos] : (int64_t)pos;
+        xl.template load<false>(x + ((int64_t)row * K + ch0) * X, lane);
+        sl.template load<true>(s + (ee * K + ch0) * S, lane);
+        const float *yr = y + ee * Y;
+#pragma unroll
+        for (int k = 0; k < Y; k++) yn[k] = yr[k];
+    };
+    if (e < e1) fetch(e);
+    while (e < e1) {
+        strip_fence();  // the column reads of the previous edge are done
+        xl.template to_strip<X, G::PX>(strip_x, lane);
+        sl.template to_strip<S, G::PS>(strip_s, lane);
+        strip_fence();
+        V xc[NX], sc[NS];
+        float yc[Y];
+#pragma unroll
+        for (int j = 0; j < NX; j++) xc[j].v[0] = strip_x[cl * G::PX + Part::kX[j]];
+#pragma unroll
+        for (int l = 0; l < NS; l++) sc[l].v[0] = strip_s[cl * G::PS + Part::kS[l]];
+#pragma unroll
+        for (int k = 0; k < Y; k++) yc[k] = to_vgpr(yn[k]);
+        const bool valid = valid_n;
+        e++;
+        if (e < e1) fetch(e);
+        if (valid) Part::template edge_fwd<1>(xc, yc, sc, acc);
+    }
+
+    // write-back: GC channels at a time through the whole strip
+    float *orow = out + ((int64_t)r * K + ch0) * Z;
+#pragma unroll
+    for (int q = 0; q < W / GC; q++) {
+        strip_fence();
+        if (active && lane / GC == q) {
+#pragma unroll
+            for (int i = 0; i < NZ; i++) strip[(lane % GC) * G::PZ + Part::kZ[i]] = acc[i].v[0] * scale;
+        }
+        strip_fence();
+        LinearBlock<GC * Z> ol;
+        ol.template from_strip<Z, G::PZ>(strip, lane);
+        ol.store(orow + (int64_t)q * GC * Z, lane);
+    }
+}
+
+template <int K, int WPB, typename Part>
+__global__ __launch_bounds__(kWave *WPB) void unrolled_fwd_leading_kernel(
+    const float *__restrict__ x, const float *__restrict__ y, const float *__restrict__ s,
+    const int32_t *__restrict__ sender, const int32_t *__restrict__ row_ptr,
+    const int32_t *__restrict__ perm, const int32_t *__restrict__ row_order,
+    float *__restrict__ out, int num_nodes, float scale) {
+    using G = LeadingGeometry<K, Part::X, Part::S, Part::Z>;
+    __shared__ __attribute__((aligned(16))) float strips[WPB * G::REGION];
+    const int64_t item = logical_block() * WPB + threadIdx.y;
+    if (item >= (int64_t)num_nodes * G::COUNT) return;
+    const int slice = uniform((int)(item % G::COUNT));
+    const int q = uniform((int)(item / G::COUNT));
+    const int r = row_order ? row_order[q] : q;
+    unrolled_fwd_leading<Part, K>(x, y, s, sender, row_ptr, perm, out, num_nodes, scale, r, slice,
+                                  threadIdx.x, strips + threadIdx.y * G::REGION);
+}
+
+// backward --------------------------------------------------------------------
+// ds values of a lane go to its row of the s strip (whose s values are in registers by then).
+struct DsStrip {
+    float *row;
+    bool active;
+    template <int L>
+    __device__ __forceinline__ void put(const Vec<1> &v) const {
+        if (active) row[L] = v.v[0];
+    }
+};
+
+template <typename Part, int K, bool kShared>
+__device__ __forceinline__ void unrolled_bwd_leading(
+    const float *__restrict__ x, const float *__restrict__ y, const float *__restrict__ s,
+    const float *__restrict__ dm, const int32_t *__restrict__ sender,
+    const int32_t *__restrict__ row_ptr, const int32_t *__restrict__ perm,
+    float *__restrict__ dx, float *__restrict__ dy, float *__restrict__ ds, int num_nodes,
+    float scale, int r, int slice, int lane, float *strip) {
+    constexpr int NX = Part::NX, NS = Part::NS, NZ = Part::NZ, Y = Part::Y;
+    constexpr int X = Part::X, S = Part::S, Z = Part::Z;
+    static_assert(X <= 64 && S <= 64, "part masks hold 64 columns");
+    using G = LeadingGeometry<K, X, S, Z>;
+    using V = Vec<1>;
+    using Red = WaveReduce<Y>;
+    constexpr int W = G::W, GC = G::GC;
+    constexpr int XN = W * X, SN = W * S;
+    float *strip_x = strip, *strip_s = strip + G::XR;
+
+    const bool active = lane < W;
+    const int cl = active ? lane : 0;
+    const int64_t ch0 = (int64_t)slice * W;
+
+    // cotangent rows: GC channels at a time through the whole strip
+    V dmr[NZ];
+    {
+        const float *zr = dm + ((int64_t)r * K + ch0) * Z;
+#pragma unroll
+        for (int i = 0; i < NZ; i++) dmr[i] = vzero<1>();  // idle lanes must add nothing to dy
+#pragma unroll
+        for (int q = 0; q < W / GC; q++) {
+            LinearBlock<GC * Z> zl;
+            zl.template load<!kShared>(zr + (int64_t)q * GC * Z, lane);
+            strip_fence();
+            zl.template to_strip<Z, G::PZ>(strip, lane);
+            strip_fence();
+            if (active && lane / GC == q) {
+#pragma unroll
+                for (int i = 0; i < NZ; i++) dmr[i].v[0] = strip[(lane % GC) * G::PZ + Part::kZ[i]] * scale;
+            }
+        }
+    }
+    // which elements of the linear dx / ds blocks this part owns (all of them when not split)
+    unsigned own_dx = ~0u, own_ds = ~0u;
+    if (kShared) {
+        own_dx = column_predicate<XN, X>(Part::kDxMask, lane);
+        own_ds = column_predicate<SN, S>(Part::kDsMask, lane);
+    }
+
+    int e = row_ptr[r];
+    const int e1 = row_ptr[r + 1];
+
+    LinearBlock<XN> xl;
+    LinearBlock<SN> sl;
+    float yn[Y];
+    bool valid_n = false;
+    int snd_n = 0;
+    int64_t ee_n = 0;
+    auto fetch = [&](int pos) {
+        const int snd = sender[pos];
+        valid_n = (unsigned)snd < (unsigned)num_nodes;
+        snd_n = valid_n ? snd : 0;
+        ee_n = perm ? (int64_t)perm[pos] : (int64_t)pos;
+        xl.template load<false>(x + ((int64_t)snd_n * K + ch0) * X, lane);
+        // the parts of a split signature read the same block one after the other: keep it cached
+        sl.template load<!kShared>(s + (ee_n * K + ch0) * S, lane);
+        const float *yr = y + ee_n * Y;
+#pragma unroll
+        for (int k = 0; k < Y; k++) yn[k] = yr[k];
+    };
+    if (e < e1) fetch(e);
+    while (e < e1) {
+        strip_fence();  // the linear reads of the previous edge are done
+        xl.template to_strip<X, G::PX>(strip_x, lane);
+        sl.template to_strip<S, G::PS>(strip_s, lane);
+        strip_fence();
+        V xc[NX], sc[NS];
+        float yc[Y];
+#pragma unroll
+        for (int j = 0; j < NX; j++) xc[j].v[0] = strip_x[cl * G::PX + Part::kX[j]];
+#pragma unroll
+        for (int l = 0; l < NS; l++) sc[l].v[0] = strip_s[cl * G::PS + Part::kS[l]];
+#pragma unroll
+        for (int k = 0; k < Y; k++) yc[k] = to_vgpr(yn[k]);
+        const bool valid = valid_n;
+        const int snd = snd_n;
+        const int64_t ee = ee_n;
+        e++;
+        if (e < e1) fetch(e);
+        if (!valid) continue;  // padding edge: its dy/ds rows are zero-filled separately
+
+        V dxe[NX];
+        float dye[Red::P];
+        strip_fence();  // every lane holds its x and s values: the rows can take dx and ds
+        const DsStrip ds_strip{strip_s + cl * G::PS, active};
+        Part::template edge_bwd<1>(xc, yc, sc, dmr, dxe, dye, ds_strip);
+#pragma unroll
+        for (int k = Y; k < Red::P; k++) dye[k] = 0.f;
+        if (active) {
+#pragma unroll
+            for (int j = 0; j < NX; j++) strip_x[cl * G::PX + Part::kX[j]] = dxe[j].v[0];
+        }
+        strip_fence();
+
+        float *ds_block = ds + (ee * K + ch0) * S;
+        if (!kShared) {
+            LinearBlock<SN> dl;
+            dl.template from_strip<S, G::PS>(strip_s, lane);
+            dl.store(ds_block, lane);
+        } else {
+#pragma unroll
+            for (int i = 0; i < (SN + kWave - 1) / kWave; i++) {
+                const int g = i * kWave + lane;
+                if ((own_ds >> i) & 1u)
+                    __builtin_nontemporal_store(strip_s[strip_index<S, G::PS>(g)], ds_block + g);
+            }
+        }
+        float *dx_block = dx + ((int64_t)snd * K + ch0) * X;
+#pragma unroll
+        for (int i = 0; i < (XN + kWave - 1) / kWave; i++) {
+            const int g = i * kWave + lane;
+            const bool mine = kShared ? (((own_dx >> i) & 1u) != 0) : (XN % kWave == 0 || g < XN);
+            if (mine) unsafeAtomicAdd(dx_block + g, strip_x[strip_index<X, G::PX>(g)]);
+        }
+
+        const float total = Red::run(dye, lane);
+        const int k = Red::slot(lane);
+        if (lane < 16 && k < Y) {
+            if (kShared || G::COUNT > 1) unsafeAtomicAdd(dy + ee * Y + k, total);  // dy zero-filled by the launcher
+            else dy[ee * Y + k] = total;
+        }
+    }
+}
+
+template <int K, int I>
+__device__ __forceinline__ void dispatch_bwd_leading(int, const float *, const float *, const float *,
+                                                     const float *, const int32_t *, const int32_t *,
+                                                     const int32_t *, float *, float *, float *, int,
+                                                     float, int, int, int, float *) {}
+template <int K, int I, typename Part, typename... Rest>
+__device__ __forceinline__ void dispatch_bwd_leading(int part, const float *x, const float *y,
+                                                     const float *s, const float *dm,
+                                                     const int32_t *sender, const int32_t *row_ptr,
+                                                     const int32_t *perm, float *dx, float *dy,
+                                                     float *ds, int num_nodes, float scale, int r,
+                                                     int slice, int lane, float *strip) {
+    if (part == I)
+        unrolled_bwd_leading<Part, K, (I > 0 || sizeof...(Rest) > 0)>(
+            x, y, s, dm, sender, row_ptr, perm, dx, dy, ds, num_nodes, scale, r, slice, lane, strip);
+    else
+        dispatch_bwd_leading<K, I + 1, Rest...>(part, x, y, s, dm, sender, row_ptr, perm, dx, dy, ds,
+                                                num_nodes, scale, r, slice, lane, strip);
+}
+
+template <typename First, typename...>
+struct FirstOf {
+    using type = First;
+};
+
+template <int K, int WPB, typename... Parts>
+__global__ __launch_bounds__(kWave *WPB) void unrolled_bwd_leading_kernel(
+    const float *__restrict__ x, const float *__restrict__ y, const float *__restrict__ s,
+    const float *__restrict__ dm, const int32_t *__restrict__ sender,
+    const int32_t *__restrict__ row_ptr, const int32_t *__restrict__ perm,
+    const int32_t *__restrict__ row_order, float *__restrict__ dx, float *__restrict__ dy,
+    float *__restrict__ ds, int num_nodes, float scale) {
+    using P0 = typename FirstOf<Parts...>::type;
+    using G = LeadingGeometry<K, P0::X, P0::S, P0::Z>;
+    constexpr int NP = sizeof...(Parts);
+    __shared__ __attribute__((aligned(16))) float strips[WPB * G::REGION];
+    const int64_t item = logical_block() * WPB + threadIdx.y;
+    if (item >= (int64_t)num_nodes * (G::COUNT * NP)) return;
+    const int part = uniform((int)(item % NP));
+    const int slice = uniform((int)((item / NP) % G::COUNT));
+    const int q = uniform((int)(item / (NP * G::COUNT)));
+    const int r = row_order ? row_order[q] : q;
+    dispatch_bwd_leading<K, 0, Parts...>(part, x, y, s, dm, sender, row_ptr, perm, dx, dy, ds, num_nodes,
+                                         scale, r, slice, threadIdx.x, strips + threadIdx.y * G::REGION);
+}
+
 template <int K, int CPL, int WPB, typename... Parts>
 int launch_unrolled_fwd(const e3j_amd_conv_params &p, const float *x, const float *y, const float *s,
                         const int32_t *sender, const int32_t *row_ptr, const int32_t *perm,
@@ -498,6 +910,44 @@ int launch_unrolled_bwd(const e3j_amd_conv_params &p, const float *x, const floa
     const int64_t blocks = padded_grid(((int64_t)p.num_nodes * PER_NODE + WPB - 1) / WPB);
     if (blocks > 0x7fffffffLL) return set_error(E3J_AMD_INVALID_ARGUMENT, "convolution_bwd: grid too large");
     hipLaunchKernelGGL((unrolled_bwd_kernel<K, CPL, WPB, Parts...>), dim3((unsigned)blocks),
+                       dim3(kWave, WPB), 0, stream, x, y, s, dm, sender, row_ptr, perm, p.row_order,
+                       dx, dy, ds, p.num_nodes, p.coef_scale);
+    return check_hip(hipGetLastError(), "convolution backward launch");
+}
+
+
+template <int K, int WPB, typename Part>
+int launch_unrolled_fwd_leading(const e3j_amd_conv_params &p, const float *x, const float *y,
+                                const float *s, const int32_t *sender, const int32_t *row_ptr,
+                                const int32_t *perm, float *out, hipStream_t stream) {
+    using G = LeadingGeometry<K, Part::X, Part::S, Part::Z>;
+    const int64_t blocks = padded_grid(((int64_t)p.num_nodes * G::COUNT + WPB - 1) / WPB);
+    if (blocks > 0x7fffffffLL) return set_error(E3J_AMD_INVALID_ARGUMENT, "convolution: grid too large");
+    hipLaunchKernelGGL((unrolled_fwd_leading_kernel<K, WPB, Part>), dim3((unsigned)blocks),
+                       dim3(kWave, WPB), 0, stream, x, y, s, sender, row_ptr, perm, p.row_order, out,
+                       p.num_nodes, p.coef_scale);
+    return check_hip(hipGetLastError(), "convolution forward launch");
+}
+
+template <int K, int WPB, int Y, int X, typename... Parts>
+int launch_unrolled_bwd_leading(const e3j_amd_conv_params &p, const float *x, const float *y,
+                                const float *s, const float *dm, const int32_t *sender,
+                                const int32_t *row_ptr, const int32_t *perm, float *dx, float *dy,
+                                float *ds, hipStream_t stream) {
+    using P0 = typename FirstOf<Parts...>::type;
+    using G = LeadingGeometry<K, P0::X, P0::S, P0::Z>;
+    constexpr int64_t PER_NODE = (int64_t)G::COUNT * sizeof...(Parts);
+    int rc = launch_fill_zero(dx, sizeof(float) * (size_t)p.num_nodes * X * K, stream);
+    if (rc) return rc;
+    if (PER_NODE > 1) {
+        rc = launch_fill_zero(dy, sizeof(float) * (size_t)p.num_edges * Y, stream);
+        if (rc) return rc;
+    }
+    rc = launch_zero_padding(p, sender, row_ptr, perm, dy, ds, stream);
+    if (rc) return rc;
+    const int64_t blocks = padded_grid(((int64_t)p.num_nodes * PER_NODE + WPB - 1) / WPB);
+    if (blocks > 0x7fffffffLL) return set_error(E3J_AMD_INVALID_ARGUMENT, "convolution_bwd: grid too large");
+    hipLaunchKernelGGL((unrolled_bwd_leading_kernel<K, WPB, Parts...>), dim3((unsigned)blocks),
                        dim3(kWave, WPB), 0, stream, x, y, s, dm, sender, row_ptr, perm, p.row_order,
                        dx, dy, ds, p.num_nodes, p.coef_scale);
     return check_hip(hipGetLastError(), "convolution backward launch");

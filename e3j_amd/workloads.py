@@ -21,28 +21,47 @@ import torch
 
 from .convolution import Convolution
 from .harmonics import Harmonics
+from .options import Layout
 
 
 @dataclasses.dataclass
 class Workload:
     name: str
     module: Convolution
-    x: torch.Tensor         # (N, X, K)
+    x: torch.Tensor         # (N, X, K); (N, K, X) in the leading-channels layout
     y: torch.Tensor         # (E, Y)
-    s: torch.Tensor         # (E, S, K)
-    dm: torch.Tensor        # (N, Z, K)
+    s: torch.Tensor         # (E, S, K); (E, K, S)
+    dm: torch.Tensor        # (N, Z, K); (N, K, Z)
     sender: torch.Tensor    # (E,) int32
     receiver: torch.Tensor  # (E,) int32
     positions: np.ndarray
     box: float
+
+    @property
+    def leading(self) -> bool:
+        return self.module.layout == Layout.LEADING_CHANNELS
+
+    def with_layout(self, layout) -> "Workload":
+        """The same values in the other memory layout (a module of that layout, axes swapped)."""
+        layout = Layout.parse(layout)
+        if layout == self.module.layout:
+            return self
+        m = self.module
+        out_filter = "+".join(dict.fromkeys(f"{ir.l}{'e' if ir.p == 1 else 'o'}" for _, ir in m.target))
+        module = Convolution((m.source[0], m.source[1]), out_filter, graph_ordering=m.graph_ordering,
+                             layout=layout, avg_num_neighbors=m.avg_num_neighbors,
+                             normalization=m.normalization)
+        swap = {f: getattr(self, f).transpose(1, 2).contiguous() for f in ("x", "s", "dm")}
+        return dataclasses.replace(self, module=module, **swap)
 
     def to(self, device) -> "Workload":
         return dataclasses.replace(self, **{f: getattr(self, f).to(device) for f in
                                             ("x", "y", "s", "dm", "sender", "receiver")})
 
     def numpy(self) -> dict:
-        """Host copies of the operands, for the CPU checker."""
-        return {f: getattr(self, f).cpu().numpy() for f in ("x", "y", "s", "dm", "sender", "receiver")}
+        """Host copies of the operands in the trailing-channels layout, for the CPU checker."""
+        w = self.with_layout(Layout.TRAILING_CHANNELS)
+        return {f: getattr(w, f).cpu().numpy() for f in ("x", "y", "s", "dm", "sender", "receiver")}
 
     def table(self):
         """`(idx (nnz, 3), val, mix_idx)` of the module's coefficient table."""
@@ -71,12 +90,13 @@ class Workload:
 
     @property
     def channels(self) -> int:
-        return int(self.x.shape[2])
+        return int(self.x.shape[1 if self.leading else 2])
 
     def algorithmic_bytes(self, sorted_edges: bool = True) -> dict:
         """Compulsory traffic: each operand element read once, each result written once."""
         n, e, k = self.num_nodes, self.num_edges, self.channels
-        X, Y, S, Z = (int(t.shape[1]) for t in (self.x, self.y, self.s, self.dm))
+        d = 2 if self.leading else 1
+        X, Y, S, Z = int(self.x.shape[d]), int(self.y.shape[1]), int(self.s.shape[d]), int(self.dm.shape[d])
         fwd = 4 * (n * X * k + e * Y + e * S * k + n * Z * k) + 4 * (e + n + 1)
         bwd = 4 * (2 * n * X * k + 2 * e * Y + 2 * e * S * k + n * Z * k) + 4 * (2 * e + n + 1)
         if not sorted_edges:

@@ -22,33 +22,41 @@ CASES = {
 
 def _signature_of(w):
     packed = w.module._packed_coef("float32")
-    dims = (int(w.x.shape[1]), int(w.y.shape[1]), w.module.params.num_out, int(w.s.shape[1]))
+    d = 2 if w.leading else 1
+    dims = (int(w.x.shape[d]), int(w.y.shape[1]), w.module.params.num_out, int(w.s.shape[d]))
     return _Table.get(packed, np.float32).signature(dims, w.channels, w.module.layout)
 
 
+def _trailing(t, w):
+    """Node/edge arrays of a workload as (rows, dim, channels) numpy arrays."""
+    return (t.transpose(1, 2) if w.leading else t).cpu().numpy()
+
+
+@pytest.mark.parametrize("layout", ["TRAILING_CHANNELS", "LEADING_CHANNELS"])
 @pytest.mark.parametrize("name", list(CASES))
-def test_unrolled_matches_oracle(name):
-    w = CASES[name]()
+def test_unrolled_matches_oracle(name, layout):
+    w = CASES[name]().with_layout(layout)
     sig, scale = _signature_of(w)
     assert sig >= 0, "benchmark signature must resolve to a built-in unrolled kernel"
     assert scale == 1.0
     d = w.to("cuda")
     m = w.module
     coef = m._packed_coef("float32")
-    out = e3j_amd.convolution(coef, d.x, d.y, d.s, d.sender, d.receiver, m.params, m.graph_ordering)
+    out = e3j_amd.convolution(coef, d.x, d.y, d.s, d.sender, d.receiver, m.params, m.graph_ordering,
+                              layout=m.layout)
     dx, dy, ds = e3j_amd.convolution_bwd(coef, d.x, d.y, d.s, d.sender, d.receiver, d.dm, m.params,
-                                         m.graph_ordering)
+                                         m.graph_ordering, layout=m.layout)
     torch.cuda.synchronize()
     idx, val, mix = w.table()
     a = w.numpy()
     ref, mag = H.forward_reference(idx, val, mix, a["x"], a["y"], a["s"], a["sender"], a["receiver"],
                                    m.params.num_out)
-    H.assert_parity(out.cpu().numpy(), ref, mag, f"{name} out")
+    H.assert_parity(_trailing(out, w), ref, mag, f"{name} out")
     (rx, ry, rs), (mx, my, ms) = H.backward_reference(idx, val, mix, a["x"], a["y"], a["s"],
                                                       a["sender"], a["receiver"], a["dm"])
-    H.assert_parity(dx.cpu().numpy(), rx, mx, f"{name} dx")
+    H.assert_parity(_trailing(dx, w), rx, mx, f"{name} dx")
     H.assert_parity(dy.cpu().numpy(), ry, my, f"{name} dy")
-    H.assert_parity(ds.cpu().numpy(), rs, ms, f"{name} ds")
+    H.assert_parity(_trailing(ds, w), rs, ms, f"{name} ds")
 
 
 def test_scaled_table_uses_unrolled_kernel():
