@@ -38,7 +38,7 @@ HBM_PEAK_GBS = 8000.0
 #: `rocprofv3 --pmc` runs of this script (FETCH_SIZE and WRITE_SIZE, KiB per dispatch), each
 #: scaled by what the same counter reads for a 1 GiB device copy (`--calibrate-copy`):
 #: 2.0 * 10.24e6 KiB fetched + 1.0 * 18.96e6 KiB written.  Only quoted for that workload.
-MEASURED_TRAFFIC_BYTES = {("cfg3", 1.0): {"backward": 2.0 * 10.236e6 * 1024 + 18.959e6 * 1024,
+MEASURED_TRAFFIC_BYTES = {("cfg3", 1.0, "trailing"): {"backward": 2.0 * 10.236e6 * 1024 + 18.959e6 * 1024,
                                           "forward": 2.0 * 9.399e6 * 1024 + 1.584e6 * 1024}}
 
 
@@ -48,6 +48,8 @@ def parse_args():
     ap.add_argument("--steps", type=int, default=20)
     ap.add_argument("--warmup", type=int, default=5)
     ap.add_argument("--config", default="cfg3", choices=["cfg2", "cfg3", "cfg4"])
+    ap.add_argument("--layout", default="trailing", choices=["trailing", "leading"],
+                    help="memory layout of the node and edge arrays (channels last or first)")
     ap.add_argument("--scale", type=float, default=1.0, help="fraction of the configuration's atoms")
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--cpu-seconds", type=float, default=15.0)
@@ -86,7 +88,8 @@ class AbiCalls:
         module = w.module
         packed = module._packed_coef("float32")
         self.table = _Table.get(packed, np.float32)
-        dims = (w.x.shape[1], w.y.shape[1], module.params.num_out, w.s.shape[1])
+        d = 2 if w.leading else 1
+        dims = (w.x.shape[d], w.y.shape[1], module.params.num_out, w.s.shape[d])
         sig, scale = self.table.signature(tuple(int(d) for d in dims), w.channels, module.layout)
         self.signature = sig
         self.params = _lib.ConvParams(
@@ -189,6 +192,7 @@ def main():
     torch.cuda.set_device(device)
 
     w = build_workload(args.config, args.scale, device, args.spatial_sort)
+    w = w.with_layout("LEADING_CHANNELS" if args.layout == "leading" else "TRAILING_CHANNELS")
     module = w.module
     coef = module._packed_coef("float32")
     bytes_ = w.algorithmic_bytes(sorted_edges=module.graph_ordering.value != "NONE")
@@ -198,7 +202,7 @@ def main():
     def step():
         # forward, then the VJP of (x, y, s) for the cotangent dm, as autograd runs them
         out = e3j_amd.convolution(coef, xg, yg, sg, w.sender, w.receiver, module.params,
-                                  module.graph_ordering)
+                                  module.graph_ordering, layout=module.layout)
         grads = torch.autograd.grad(out, (xg, yg, sg), w.dm)
         return out, grads
 
@@ -231,6 +235,7 @@ def main():
     def gbs(nbytes, ms):
         return nbytes / (ms * 1e-3) / 1e9
 
+    measured = {} if args.spatial_sort else MEASURED_TRAFFIC_BYTES.get((args.config, args.scale, args.layout), {})
     bwd_gbs, fwd_gbs = gbs(bytes_["bwd"], bwd_ms), gbs(bytes_["fwd"], fwd_ms)
     both_gbs = gbs(bytes_["fwd_bwd"], fwd_ms + bwd_ms)
     result = {
@@ -249,7 +254,7 @@ def main():
         "config": {
             "workload": f"{args.config}: {w.num_nodes} atoms, {w.num_edges} edges, K={w.channels}, "
                         f"x {module.source[0]}, y {module.source[1]}, out {module.target}, "
-                        f"{module.graph_ordering.value.lower()}-ordered edges, trailing-channels layout, "
+                        f"{module.graph_ordering.value.lower()}-ordered edges, {args.layout}-channels layout, "
                         "forward + VJP (dx, dy, ds)",
             "scale": args.scale,
             "atom_numbering": "space-filling curve" if args.spatial_sort else "random",
@@ -260,10 +265,10 @@ def main():
         "roofline": {
             "bound": "hbm", "kernel": "convolution backward (unrolled_bwd_kernel + dx zero fill)",
             "achieved": bwd_gbs, "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": bwd_gbs / HBM_PEAK_GBS,
-            "traffic": MEASURED_TRAFFIC_BYTES.get((args.config, args.scale if not args.spatial_sort else -1), {}).get("backward"),
+            "traffic": measured.get("backward"),
             "algorithmic_bytes": bytes_["bwd"], "ms": bwd_ms,
             "forward": {"achieved": fwd_gbs, "frac": fwd_gbs / HBM_PEAK_GBS,
-                        "traffic": MEASURED_TRAFFIC_BYTES.get((args.config, args.scale if not args.spatial_sort else -1), {}).get("forward"),
+                        "traffic": measured.get("forward"),
                         "algorithmic_bytes": bytes_["fwd"], "ms": fwd_ms},
             "forward_plus_backward": {"achieved": both_gbs, "frac": both_gbs / HBM_PEAK_GBS,
                                       "algorithmic_bytes": bytes_["fwd_bwd"], "ms": fwd_ms + bwd_ms},

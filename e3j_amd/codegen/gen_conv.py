@@ -56,11 +56,13 @@ LAUNCH = {
 }
 
 
-#: leading-channels layout: (waves per block, parts) variants; the forward pass is never split.
+#: leading-channels layout: (waves per block, parts) variants.  The forward pass is never
+#: split; a backward block is the parts of one (receiver, channel slice), so its wave count
+#: is the part count (the first number is ignored there).
 LAUNCH_LEADING = {
-    32: dict(fwd=[(4, 1)], bwd=[(4, 1)]),
-    64: dict(fwd=[(4, 1)], bwd=[(4, 2), (4, 1), (4, 3)]),
-    128: dict(fwd=[(4, 1)], bwd=[(4, 2), (4, 1), (4, 3)]),
+    32: dict(fwd=[(4, 1)], bwd=[(1, 1)]),
+    64: dict(fwd=[(4, 1)], bwd=[(3, 3), (1, 1), (2, 2), (4, 4)]),
+    128: dict(fwd=[(4, 1)], bwd=[(3, 3), (1, 1), (2, 2), (4, 4)]),
 }
 
 
@@ -369,7 +371,7 @@ def emit_signature(sig_id: int, name: str, x_irreps: str, y_irreps: str, out_fil
         for wpb, zs in lead["fwd"]:
             out += [f"template __global__ void unrolled_fwd_leading_kernel<{channels}, {wpb}, {part_names[zs]}>("] + fwd_args
         for wpb, zs in lead["bwd"]:
-            out += [f"template __global__ void unrolled_bwd_leading_kernel<{channels}, {wpb}, {part_names[zs]}>("] + bwd_args
+            out += [f"template __global__ void unrolled_bwd_leading_kernel<{channels}, {part_names[zs]}>("] + bwd_args
 
     fwd_sig = ["(const e3j_amd_conv_params &p, const float *x, const float *y, const float *s,",
                "                   const int32_t *sender, const int32_t *row_ptr, const int32_t *perm,",
@@ -410,7 +412,7 @@ def emit_signature(sig_id: int, name: str, x_irreps: str, y_irreps: str, out_fil
                                    "p, x, y, s, sender, row_ptr, perm, out, stream);")]
         out += ["static int run_bwd_leading" + bwd_sig[0]] + bwd_sig[1:]
         out += [ln.replace("VARIANT", "tuning().bwd_variant") for ln in switch(
-            lead["bwd"], lambda v: f"launch_unrolled_bwd_leading<{channels}, {v[0]}, {t.Y}, {t.X}, "
+            lead["bwd"], lambda v: f"launch_unrolled_bwd_leading<{channels}, {t.Y}, {t.X}, "
                                    f"{part_names[v[1]]}>(p, x, y, s, dm, sender, row_ptr, perm, dx, dy, ds, stream);")]
         out += [f"extern const Signature kSignature_{2 * sig_id + 1} = {{",
                 f'    "{desc.replace("trailing", "leading")}",',

@@ -525,37 +525,37 @@ struct LeadingGeometry {
     static_assert(W % GC == 0 && GC % 4 == 0, "channel groups must tile the wave");
 };
 
-// N floats (N % 4 == 0) at a 16-byte aligned address, dealt to the lanes in 16-byte pieces.
-template <int N>
+// N floats (N % 4 == 0) at a 16-byte aligned address, dealt to NT threads in 16-byte pieces.
+template <int N, int NT = kWave>
 struct LinearBlock {
     static_assert(N % 4 == 0, "blocks are moved in 16-byte pieces");
     static constexpr int PIECES = N / 4;
-    static constexpr int NV = (PIECES + kWave - 1) / kWave;
-    static constexpr bool EXACT = NV * kWave == PIECES;
+    static constexpr int NV = (PIECES + NT - 1) / NT;
+    static constexpr bool EXACT = NV * NT == PIECES;
     f32x4 v[NV];
 
     template <bool kStream>
-    __device__ __forceinline__ void load(const float *src, int lane) {
+    __device__ __forceinline__ void load(const float *src, int tid) {
         const f32x4 *p = reinterpret_cast<const f32x4 *>(src);
 #pragma unroll
         for (int i = 0; i < NV; i++) {
-            const int idx = i * kWave + lane;
+            const int idx = i * NT + tid;
             if (EXACT || idx < PIECES) v[i] = kStream ? __builtin_nontemporal_load(p + idx) : p[idx];
         }
     }
-    __device__ __forceinline__ void store(float *dst, int lane) const {
+    __device__ __forceinline__ void store(float *dst, int tid) const {
         f32x4 *p = reinterpret_cast<f32x4 *>(dst);
 #pragma unroll
         for (int i = 0; i < NV; i++) {
-            const int idx = i * kWave + lane;
+            const int idx = i * NT + tid;
             if (EXACT || idx < PIECES) __builtin_nontemporal_store(v[i], p + idx);
         }
     }
     template <int ROW, int PAD>
-    __device__ __forceinline__ void to_strip(float *strip, int lane) const {
+    __device__ __forceinline__ void to_strip(float *strip, int tid) const {
 #pragma unroll
         for (int i = 0; i < NV; i++) {
-            const int idx = i * kWave + lane;
+            const int idx = i * NT + tid;
             if (EXACT || idx < PIECES) {
                 if (PAD == ROW) {
                     reinterpret_cast<f32x4 *>(strip)[idx] = v[i];
@@ -567,10 +567,10 @@ struct LinearBlock {
         }
     }
     template <int ROW, int PAD>
-    __device__ __forceinline__ void from_strip(const float *strip, int lane) {
+    __device__ __forceinline__ void from_strip(const float *strip, int tid) {
 #pragma unroll
         for (int i = 0; i < NV; i++) {
-            const int idx = i * kWave + lane;
+            const int idx = i * NT + tid;
             if (EXACT || idx < PIECES) {
                 if (PAD == ROW) {
                     v[i] = reinterpret_cast<const f32x4 *>(strip)[idx];
@@ -583,16 +583,16 @@ struct LinearBlock {
     }
 };
 
-// Bit i of the result: element i * 64 + lane of a linear (rows of ROW) block belongs to a
-// column of `mask`.  Computed once per wave; the per-edge loops then test one bit.
-template <int N, int ROW>
-__device__ __forceinline__ unsigned column_predicate(unsigned long long mask, int lane) {
-    constexpr int STEPS = (N + kWave - 1) / kWave;
+// Bit i of the result: element i * NT + tid of a linear block of N values in rows of ROW
+// lies in a column of `mask`.  Computed once per thread; the per-edge loops test one bit.
+template <int N, int ROW, int NT>
+__device__ __forceinline__ unsigned column_predicate(unsigned long long mask, int tid) {
+    constexpr int STEPS = (N + NT - 1) / NT;
     static_assert(STEPS <= 32, "block too large for a 32-bit predicate");
     unsigned pred = 0;
 #pragma unroll
     for (int i = 0; i < STEPS; i++) {
-        const int g = i * kWave + lane;
+        const int g = i * NT + tid;
         if (g < N && ((mask >> (g % ROW)) & 1ull)) pred |= 1u << i;
     }
     return pred;
@@ -693,7 +693,11 @@ __global__ __launch_bounds__(kWave *WPB) void unrolled_fwd_leading_kernel(
 }
 
 // backward --------------------------------------------------------------------
-// ds values of a lane go to its row of the s strip (whose s values are in registers by then).
+// One block per (receiver, channel slice); its waves are the parts of the signature.  They
+// share the staged x and s blocks of an edge (each thread moves its pieces once), and their
+// ds and dx values meet in a second pair of strips from which the block stores whole ds
+// rows and issues the dx atomics in linear, coalesced order.  All waves of a block walk the
+// same edge segment, so the two block barriers per edge are reached uniformly.
 struct DsStrip {
     float *row;
     bool active;
@@ -703,28 +707,43 @@ struct DsStrip {
     }
 };
 
-template <typename Part, int K, bool kShared>
+template <int K, int X, int S, int Z, int NP>
+struct LeadingBwdGeometry : LeadingGeometry<K, X, S, Z> {
+    using Base = LeadingGeometry<K, X, S, Z>;
+    static constexpr int NT = kWave * NP;
+    static constexpr int IN = Base::XR + Base::SR;  // staged operands, then as much again for results
+    static constexpr int REGION = 2 * IN > 4 * Base::PZ ? 2 * IN : round4(4 * Base::PZ);
+    static constexpr int group() {
+        int g = Base::W;
+        while (g > 4 && g * Base::PZ > REGION) g /= 2;
+        return g;
+    }
+    static constexpr int GC = group();  // channels of dm rows staged at a time
+};
+
+template <typename Part, int K, int NP, unsigned long long kCoveredDx>
 __device__ __forceinline__ void unrolled_bwd_leading(
     const float *__restrict__ x, const float *__restrict__ y, const float *__restrict__ s,
     const float *__restrict__ dm, const int32_t *__restrict__ sender,
     const int32_t *__restrict__ row_ptr, const int32_t *__restrict__ perm,
     float *__restrict__ dx, float *__restrict__ dy, float *__restrict__ ds, int num_nodes,
-    float scale, int r, int slice, int lane, float *strip) {
+    float scale, int r, int slice, int lane, int tid, float *region) {
     constexpr int NX = Part::NX, NS = Part::NS, NZ = Part::NZ, Y = Part::Y;
     constexpr int X = Part::X, S = Part::S, Z = Part::Z;
     static_assert(X <= 64 && S <= 64, "part masks hold 64 columns");
-    using G = LeadingGeometry<K, X, S, Z>;
+    using G = LeadingBwdGeometry<K, X, S, Z, NP>;
     using V = Vec<1>;
     using Red = WaveReduce<Y>;
-    constexpr int W = G::W, GC = G::GC;
+    constexpr int W = G::W, GC = G::GC, NT = G::NT;
     constexpr int XN = W * X, SN = W * S;
-    float *strip_x = strip, *strip_s = strip + G::XR;
+    constexpr bool kAllDx = kCoveredDx == (X == 64 ? ~0ull : ((1ull << X) - 1));
+    float *in_x = region, *in_s = in_x + G::XR, *out_x = in_s + G::SR, *out_s = out_x + G::XR;
 
     const bool active = lane < W;
     const int cl = active ? lane : 0;
     const int64_t ch0 = (int64_t)slice * W;
 
-    // cotangent rows: GC channels at a time through the whole strip
+    // cotangent rows: GC channels at a time through the whole region
     V dmr[NZ];
     {
         const float *zr = dm + ((int64_t)r * K + ch0) * Z;
@@ -732,29 +751,27 @@ __device__ __forceinline__ void unrolled_bwd_leading(
         for (int i = 0; i < NZ; i++) dmr[i] = vzero<1>();  // idle lanes must add nothing to dy
 #pragma unroll
         for (int q = 0; q < W / GC; q++) {
-            LinearBlock<GC * Z> zl;
-            zl.template load<!kShared>(zr + (int64_t)q * GC * Z, lane);
-            strip_fence();
-            zl.template to_strip<Z, G::PZ>(strip, lane);
-            strip_fence();
+            LinearBlock<GC * Z, NT> zl;
+            zl.template load<true>(zr + (int64_t)q * GC * Z, tid);
+            __syncthreads();  // the column reads of the previous group are done
+            zl.template to_strip<Z, G::PZ>(region, tid);
+            __syncthreads();
             if (active && lane / GC == q) {
 #pragma unroll
-                for (int i = 0; i < NZ; i++) dmr[i].v[0] = strip[(lane % GC) * G::PZ + Part::kZ[i]] * scale;
+                for (int i = 0; i < NZ; i++) dmr[i].v[0] = region[(lane % GC) * G::PZ + Part::kZ[i]] * scale;
             }
         }
+        __syncthreads();
     }
-    // which elements of the linear dx / ds blocks this part owns (all of them when not split)
-    unsigned own_dx = ~0u, own_ds = ~0u;
-    if (kShared) {
-        own_dx = column_predicate<XN, X>(Part::kDxMask, lane);
-        own_ds = column_predicate<SN, S>(Part::kDsMask, lane);
-    }
+    // x columns no coefficient touches take no dx (their rows stay zero)
+    unsigned covered = ~0u;
+    if (!kAllDx) covered = column_predicate<XN, X, NT>(kCoveredDx, tid);
 
     int e = row_ptr[r];
     const int e1 = row_ptr[r + 1];
 
-    LinearBlock<XN> xl;
-    LinearBlock<SN> sl;
+    LinearBlock<XN, NT> xl;
+    LinearBlock<SN, NT> sl;
     float yn[Y];
     bool valid_n = false;
     int snd_n = 0;
@@ -764,95 +781,87 @@ __device__ __forceinline__ void unrolled_bwd_leading(
         valid_n = (unsigned)snd < (unsigned)num_nodes;
         snd_n = valid_n ? snd : 0;
         ee_n = perm ? (int64_t)perm[pos] : (int64_t)pos;
-        xl.template load<false>(x + ((int64_t)snd_n * K + ch0) * X, lane);
-        // the parts of a split signature read the same block one after the other: keep it cached
-        sl.template load<!kShared>(s + (ee_n * K + ch0) * S, lane);
+        xl.template load<false>(x + ((int64_t)snd_n * K + ch0) * X, tid);
+        sl.template load<true>(s + (ee_n * K + ch0) * S, tid);
         const float *yr = y + ee_n * Y;
 #pragma unroll
         for (int k = 0; k < Y; k++) yn[k] = yr[k];
     };
     if (e < e1) fetch(e);
     while (e < e1) {
-        strip_fence();  // the linear reads of the previous edge are done
-        xl.template to_strip<X, G::PX>(strip_x, lane);
-        sl.template to_strip<S, G::PS>(strip_s, lane);
-        strip_fence();
+        // (the result strips of the previous edge are still being read by other waves: the
+        // operand strips are separate, and the barrier below orders the next result writes)
+        xl.template to_strip<X, G::PX>(in_x, tid);
+        sl.template to_strip<S, G::PS>(in_s, tid);
+        __syncthreads();
         V xc[NX], sc[NS];
         float yc[Y];
 #pragma unroll
-        for (int j = 0; j < NX; j++) xc[j].v[0] = strip_x[cl * G::PX + Part::kX[j]];
+        for (int j = 0; j < NX; j++) xc[j].v[0] = in_x[cl * G::PX + Part::kX[j]];
 #pragma unroll
-        for (int l = 0; l < NS; l++) sc[l].v[0] = strip_s[cl * G::PS + Part::kS[l]];
+        for (int l = 0; l < NS; l++) sc[l].v[0] = in_s[cl * G::PS + Part::kS[l]];
 #pragma unroll
         for (int k = 0; k < Y; k++) yc[k] = to_vgpr(yn[k]);
-        const bool valid = valid_n;
+        const bool valid = valid_n;  // uniform over the block: every wave looks at the same edge
         const int snd = snd_n;
         const int64_t ee = ee_n;
         e++;
         if (e < e1) fetch(e);
-        if (!valid) continue;  // padding edge: its dy/ds rows are zero-filled separately
 
-        V dxe[NX];
         float dye[Red::P];
-        strip_fence();  // every lane holds its x and s values: the rows can take dx and ds
-        const DsStrip ds_strip{strip_s + cl * G::PS, active};
-        Part::template edge_bwd<1>(xc, yc, sc, dmr, dxe, dye, ds_strip);
+        if (valid) {
+            V dxe[NX];
+            const DsStrip ds_strip{out_s + cl * G::PS, active};
+            Part::template edge_bwd<1>(xc, yc, sc, dmr, dxe, dye, ds_strip);
+            if (active) {
 #pragma unroll
-        for (int k = Y; k < Red::P; k++) dye[k] = 0.f;
-        if (active) {
-#pragma unroll
-            for (int j = 0; j < NX; j++) strip_x[cl * G::PX + Part::kX[j]] = dxe[j].v[0];
-        }
-        strip_fence();
-
-        float *ds_block = ds + (ee * K + ch0) * S;
-        if (!kShared) {
-            LinearBlock<SN> dl;
-            dl.template from_strip<S, G::PS>(strip_s, lane);
-            dl.store(ds_block, lane);
-        } else {
-#pragma unroll
-            for (int i = 0; i < (SN + kWave - 1) / kWave; i++) {
-                const int g = i * kWave + lane;
-                if ((own_ds >> i) & 1u)
-                    __builtin_nontemporal_store(strip_s[strip_index<S, G::PS>(g)], ds_block + g);
+                for (int j = 0; j < NX; j++) out_x[cl * G::PX + Part::kX[j]] = dxe[j].v[0];
             }
         }
+        __syncthreads();  // operands consumed by every wave, results of every wave in place
+        if (!valid) continue;  // padding edge: its dy/ds rows are zero-filled separately
+
+        LinearBlock<SN, NT> dl;
+        dl.template from_strip<S, G::PS>(out_s, tid);
+        dl.store(ds + (ee * K + ch0) * S, tid);
         float *dx_block = dx + ((int64_t)snd * K + ch0) * X;
 #pragma unroll
-        for (int i = 0; i < (XN + kWave - 1) / kWave; i++) {
-            const int g = i * kWave + lane;
-            const bool mine = kShared ? (((own_dx >> i) & 1u) != 0) : (XN % kWave == 0 || g < XN);
-            if (mine) unsafeAtomicAdd(dx_block + g, strip_x[strip_index<X, G::PX>(g)]);
+        for (int i = 0; i < (XN + NT - 1) / NT; i++) {
+            const int g = i * NT + tid;
+            const bool mine = kAllDx ? (XN % NT == 0 || g < XN) : (((covered >> i) & 1u) != 0);
+            if (mine) unsafeAtomicAdd(dx_block + g, out_x[strip_index<X, G::PX>(g)]);
         }
 
+#pragma unroll
+        for (int k = Y; k < Red::P; k++) dye[k] = 0.f;
         const float total = Red::run(dye, lane);
         const int k = Red::slot(lane);
         if (lane < 16 && k < Y) {
-            if (kShared || G::COUNT > 1) unsafeAtomicAdd(dy + ee * Y + k, total);  // dy zero-filled by the launcher
+            if (NP > 1 || G::COUNT > 1) unsafeAtomicAdd(dy + ee * Y + k, total);  // dy zero-filled by the launcher
             else dy[ee * Y + k] = total;
         }
     }
 }
 
-template <int K, int I>
+template <int K, int NP, unsigned long long kCoveredDx, int I>
 __device__ __forceinline__ void dispatch_bwd_leading(int, const float *, const float *, const float *,
                                                      const float *, const int32_t *, const int32_t *,
                                                      const int32_t *, float *, float *, float *, int,
-                                                     float, int, int, int, float *) {}
-template <int K, int I, typename Part, typename... Rest>
+                                                     float, int, int, int, int, float *) {}
+template <int K, int NP, unsigned long long kCoveredDx, int I, typename Part, typename... Rest>
 __device__ __forceinline__ void dispatch_bwd_leading(int part, const float *x, const float *y,
                                                      const float *s, const float *dm,
                                                      const int32_t *sender, const int32_t *row_ptr,
                                                      const int32_t *perm, float *dx, float *dy,
                                                      float *ds, int num_nodes, float scale, int r,
-                                                     int slice, int lane, float *strip) {
+                                                     int slice, int lane, int tid, float *region) {
     if (part == I)
-        unrolled_bwd_leading<Part, K, (I > 0 || sizeof...(Rest) > 0)>(
-            x, y, s, dm, sender, row_ptr, perm, dx, dy, ds, num_nodes, scale, r, slice, lane, strip);
+        unrolled_bwd_leading<Part, K, NP, kCoveredDx>(x, y, s, dm, sender, row_ptr, perm, dx, dy, ds,
+                                                      num_nodes, scale, r, slice, lane, tid, region);
     else
-        dispatch_bwd_leading<K, I + 1, Rest...>(part, x, y, s, dm, sender, row_ptr, perm, dx, dy, ds,
-                                                num_nodes, scale, r, slice, lane, strip);
+        dispatch_bwd_leading<K, NP, kCoveredDx, I + 1, Rest...>(part, x, y, s, dm, sender, row_ptr, perm,
+                                                                dx, dy, ds, num_nodes, scale, r, slice,
+                                                                lane, tid, region);
 }
 
 template <typename First, typename...>
@@ -860,25 +869,27 @@ struct FirstOf {
     using type = First;
 };
 
-template <int K, int WPB, typename... Parts>
-__global__ __launch_bounds__(kWave *WPB) void unrolled_bwd_leading_kernel(
+template <int K, typename... Parts>
+__global__ __launch_bounds__(kWave * sizeof...(Parts)) void unrolled_bwd_leading_kernel(
     const float *__restrict__ x, const float *__restrict__ y, const float *__restrict__ s,
     const float *__restrict__ dm, const int32_t *__restrict__ sender,
     const int32_t *__restrict__ row_ptr, const int32_t *__restrict__ perm,
     const int32_t *__restrict__ row_order, float *__restrict__ dx, float *__restrict__ dy,
     float *__restrict__ ds, int num_nodes, float scale) {
     using P0 = typename FirstOf<Parts...>::type;
-    using G = LeadingGeometry<K, P0::X, P0::S, P0::Z>;
     constexpr int NP = sizeof...(Parts);
-    __shared__ __attribute__((aligned(16))) float strips[WPB * G::REGION];
-    const int64_t item = logical_block() * WPB + threadIdx.y;
-    if (item >= (int64_t)num_nodes * (G::COUNT * NP)) return;
-    const int part = uniform((int)(item % NP));
-    const int slice = uniform((int)((item / NP) % G::COUNT));
-    const int q = uniform((int)(item / (NP * G::COUNT)));
+    using G = LeadingBwdGeometry<K, P0::X, P0::S, P0::Z, NP>;
+    constexpr unsigned long long kCoveredDx = (Parts::kDxMask | ...);
+    __shared__ __attribute__((aligned(16))) float region[G::REGION];
+    const int64_t item = logical_block();
+    if (item >= (int64_t)num_nodes * G::COUNT) return;  // whole block: no barrier is left waiting
+    const int slice = (int)(item % G::COUNT);
+    const int q = (int)(item / G::COUNT);
     const int r = row_order ? row_order[q] : q;
-    dispatch_bwd_leading<K, 0, Parts...>(part, x, y, s, dm, sender, row_ptr, perm, dx, dy, ds, num_nodes,
-                                         scale, r, slice, threadIdx.x, strips + threadIdx.y * G::REGION);
+    const int part = uniform((int)threadIdx.y);
+    dispatch_bwd_leading<K, NP, kCoveredDx, 0, Parts...>(
+        part, x, y, s, dm, sender, row_ptr, perm, dx, dy, ds, num_nodes, scale, r, slice,
+        threadIdx.x, threadIdx.y * kWave + threadIdx.x, region);
 }
 
 template <int K, int CPL, int WPB, typename... Parts>
@@ -929,26 +940,26 @@ int launch_unrolled_fwd_leading(const e3j_amd_conv_params &p, const float *x, co
     return check_hip(hipGetLastError(), "convolution forward launch");
 }
 
-template <int K, int WPB, int Y, int X, typename... Parts>
+template <int K, int Y, int X, typename... Parts>
 int launch_unrolled_bwd_leading(const e3j_amd_conv_params &p, const float *x, const float *y,
                                 const float *s, const float *dm, const int32_t *sender,
                                 const int32_t *row_ptr, const int32_t *perm, float *dx, float *dy,
                                 float *ds, hipStream_t stream) {
     using P0 = typename FirstOf<Parts...>::type;
-    using G = LeadingGeometry<K, P0::X, P0::S, P0::Z>;
-    constexpr int64_t PER_NODE = (int64_t)G::COUNT * sizeof...(Parts);
+    constexpr int NP = sizeof...(Parts);
+    using G = LeadingBwdGeometry<K, P0::X, P0::S, P0::Z, NP>;
     int rc = launch_fill_zero(dx, sizeof(float) * (size_t)p.num_nodes * X * K, stream);
     if (rc) return rc;
-    if (PER_NODE > 1) {
+    if (G::COUNT * NP > 1) {
         rc = launch_fill_zero(dy, sizeof(float) * (size_t)p.num_edges * Y, stream);
         if (rc) return rc;
     }
     rc = launch_zero_padding(p, sender, row_ptr, perm, dy, ds, stream);
     if (rc) return rc;
-    const int64_t blocks = padded_grid(((int64_t)p.num_nodes * PER_NODE + WPB - 1) / WPB);
+    const int64_t blocks = padded_grid((int64_t)p.num_nodes * G::COUNT);
     if (blocks > 0x7fffffffLL) return set_error(E3J_AMD_INVALID_ARGUMENT, "convolution_bwd: grid too large");
-    hipLaunchKernelGGL((unrolled_bwd_leading_kernel<K, WPB, Parts...>), dim3((unsigned)blocks),
-                       dim3(kWave, WPB), 0, stream, x, y, s, dm, sender, row_ptr, perm, p.row_order,
+    hipLaunchKernelGGL((unrolled_bwd_leading_kernel<K, Parts...>), dim3((unsigned)blocks),
+                       dim3(kWave, NP), 0, stream, x, y, s, dm, sender, row_ptr, perm, p.row_order,
                        dx, dy, ds, p.num_nodes, p.coef_scale);
     return check_hip(hipGetLastError(), "convolution backward launch");
 }
