@@ -242,3 +242,115 @@ def config4(scale: float = 1.0, device="cpu") -> Workload:
     dm = _normal((n, Z, 64), 36, device)
     return Workload("cfg4", module, x, y, s, dm, torch.from_numpy(sender).to(device),
                     torch.from_numpy(receiver).to(device), np.zeros((n, 3)), 0.0)
+
+
+class EnergyModel:
+    """Two stacked convolutions with per-degree channel mixing and a scalar energy readout.
+
+    The layer sequence of the end-to-end configuration: positions -> edge vectors ->
+    (spherical harmonics, Bessel radial basis -> MLP -> per-path radial weights) ->
+    Convolution -> Linear mixing, twice, then a linear readout on the `0e` rows summed over
+    the atoms.  Everything but the convolution is plain tensor arithmetic, so the gradient
+    with respect to the positions reaches the fused kernels' VJPs through `y` and `s`
+    (layer 2 also through `x`).  `convolve(layer, x, y, s, sender, receiver)` can be
+    replaced to evaluate the same model with another implementation of the operator.
+    """
+
+    def __init__(self, channels: int = 64, irreps: str = "0e+1o+2e+3o", l_max: int = 3,
+                 num_basis: int = 8, hidden: int = 32, cutoff: float = 5.0,
+                 avg_num_neighbors: float = 30.0, seeds=(43, 44, 45)):
+        y_irreps = "+".join(f"{l}{'e' if l % 2 == 0 else 'o'}" for l in range(l_max + 1))
+        self.layers = [Convolution((irreps, y_irreps), irreps, graph_ordering="RECEIVER",
+                                   avg_num_neighbors=avg_num_neighbors) for _ in range(2)]
+        self.channels, self.cutoff, self.num_basis = channels, float(cutoff), num_basis
+        self.harmonics = Harmonics(l_max, normalization="component")
+        module = self.layers[0]
+        self.num_x, self.num_paths = module.source[0].dim, module.params.num_scalars
+        # (degree block of the output, copies, components) in row order
+        self.blocks = [(mul, 2 * ir.l + 1) for mul, ir in module.target]
+        seed_mlp, seed_mix, seed_read = seeds
+        rng = np.random.default_rng(seed_mlp)
+        self.mlp = [(rng.standard_normal((num_basis, hidden)) / math.sqrt(num_basis),
+                     rng.standard_normal((hidden, self.num_paths * channels)) / math.sqrt(hidden))
+                    for _ in self.layers]
+        rng = np.random.default_rng(seed_mix)
+        self.mix = [[rng.standard_normal((mul, channels, channels)) / math.sqrt(mul * channels)
+                     for mul, _ in self.blocks] for _ in self.layers]
+        self.readout = np.random.default_rng(seed_read).standard_normal(channels) / math.sqrt(channels)
+
+    def _t(self, array, like: torch.Tensor) -> torch.Tensor:
+        return torch.as_tensor(array, dtype=like.dtype, device=like.device)
+
+    def radial_basis(self, r: torch.Tensor) -> torch.Tensor:
+        """Bessel functions `sqrt(2/rc) sin(n pi r / rc) / r` times a smooth cutoff envelope."""
+        n = torch.arange(1, self.num_basis + 1, dtype=r.dtype, device=r.device)
+        u = (r / self.cutoff).clamp(max=1.0)
+        envelope = 1.0 - 10.0 * u ** 3 + 15.0 * u ** 4 - 6.0 * u ** 5
+        bessel = math.sqrt(2.0 / self.cutoff) * torch.sin(n * math.pi * r[:, None] / self.cutoff) / r[:, None]
+        return bessel * envelope[:, None]
+
+    def edge_inputs(self, positions, sender, receiver, shift):
+        vec = positions[sender.long()] - positions[receiver.long()] + shift
+        r = torch.linalg.vector_norm(vec, dim=-1)
+        return self.harmonics(vec / r[:, None]), self.radial_basis(r)
+
+    def convolve(self, layer, x, y, s, sender, receiver):
+        return self.layers[layer](x, y, s, sender, receiver)
+
+    def energy(self, positions, node_features, sender, receiver, shift, convolve=None):
+        convolve = convolve or self.convolve
+        y, basis = self.edge_inputs(positions, sender, receiver, shift)
+        x = node_features
+        for layer, (w1, w2) in enumerate(self.mlp):
+            hidden = torch.nn.functional.silu(basis @ self._t(w1, basis))
+            s = (hidden @ self._t(w2, basis)).reshape(-1, self.num_paths, self.channels)
+            out = convolve(layer, x, y, s, sender, receiver)          # (N, Z, K)
+            rows, mixed = 0, []
+            for (mul, dim), w in zip(self.blocks, self.mix[layer]):
+                block = out[:, rows:rows + mul * dim, :].reshape(-1, mul, dim, self.channels)
+                mixed.append(torch.einsum("numk,ukc->nmc", block, self._t(w, out)))
+                rows += mul * dim
+            x = torch.cat(mixed, dim=1)                                # (N, X, K)
+        return (x[:, 0, :] @ self._t(self.readout, x)).sum()
+
+    def energy_and_forces(self, positions, node_features, sender, receiver, shift, convolve=None):
+        positions = positions.detach().requires_grad_(True)
+        e = self.energy(positions, node_features, sender, receiver, shift, convolve)
+        (grad,) = torch.autograd.grad(e, positions)
+        return e.detach(), -grad
+
+
+@dataclasses.dataclass
+class EnergyWorkload:
+    name: str
+    model: EnergyModel
+    positions: torch.Tensor      # (N, 3) float64
+    node_features: torch.Tensor  # (N, X, K)
+    sender: torch.Tensor
+    receiver: torch.Tensor
+    shift: torch.Tensor          # (E, 3) lattice translation of each edge (minimum image)
+
+    @property
+    def num_edges(self) -> int:
+        return int(self.sender.shape[0])
+
+    def to(self, device, dtype=torch.float32) -> "EnergyWorkload":
+        cast = {f: getattr(self, f).to(device=device, dtype=dtype)
+                for f in ("positions", "node_features", "shift")}
+        return dataclasses.replace(self, sender=self.sender.to(device), receiver=self.receiver.to(device),
+                                   **cast)
+
+
+def config5(scale: float = 1.0) -> EnergyWorkload:
+    """6 000 atoms in a periodic box (~200k edges): energy and forces through two convolutions."""
+    n = max(16, int(6000 * scale))
+    box = periodic_box_length(n, 30.0, 5.0)
+    if box <= 10.0:
+        raise ValueError("the periodic box must be wider than two cutoffs")
+    pos = np.random.default_rng(41).uniform(0.0, box, size=(n, 3))
+    sender, receiver, vec = radius_graph(pos, 5.0, box)
+    shift = vec - (pos[sender] - pos[receiver])
+    model = EnergyModel()
+    x = np.random.default_rng(42).standard_normal((n, model.num_x, model.channels))
+    return EnergyWorkload("cfg5", model, torch.from_numpy(pos), torch.from_numpy(x),
+                          torch.from_numpy(sender), torch.from_numpy(receiver), torch.from_numpy(shift))

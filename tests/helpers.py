@@ -107,3 +107,23 @@ def assert_parity(result, ref64, mag64, what="", rtol=1e-5, atol=1e-6, ulps=16.0
 
 def float32_noise_bound(ref64, mag64, rtol=1e-5, atol=1e-6, ulps=16.0):
     return np.maximum(atol + rtol * np.abs(ref64), ulps * EPS32 * mag64)
+
+
+def dense_convolve(model):
+    """The operator of an `EnergyModel` as a dense einsum with index_add, differentiable by torch
+    on the host: the independent form the end-to-end energy and forces are checked against."""
+    import torch
+
+    def convolve(layer, x, y, s, sender, receiver):
+        m = model.layers[layer]
+        c = m.coef
+        idx = np.asarray(c.idx, dtype=np.int64)
+        Z, X, Y = m.params.num_out, x.shape[1], y.shape[1]
+        dense = torch.zeros((Z, X, Y), dtype=x.dtype)
+        dense.index_put_(tuple(torch.as_tensor(idx[:, :3].T)), torch.as_tensor(np.asarray(c.val), dtype=x.dtype),
+                         accumulate=True)
+        mix = torch.as_tensor(m._mix.mix_indices, dtype=torch.long)
+        weights = torch.einsum("ijk,ek->eij", dense, y)
+        msg = torch.einsum("eij,ejc->eic", weights, x[sender.long()]) * s[:, mix, :]
+        return torch.zeros((x.shape[0], Z, x.shape[2]), dtype=x.dtype).index_add(0, receiver.long(), msg)
+    return convolve

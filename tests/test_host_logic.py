@@ -268,3 +268,24 @@ def test_resolve_val_dtype():
     assert resolve_val_dtype(np.float32) == "float32"
     with pytest.raises(TypeError, match="Cast the operands"):
         resolve_val_dtype(np.int32)
+
+
+def test_energy_model_forces_are_the_energy_gradient():
+    """The end-to-end model on the host with the dense form of the operator: central differences
+    of the energy along a random direction equal -F.direction (pins the reference the GPU
+    energy and forces are compared with)."""
+    import torch
+    from e3j_amd import workloads as W
+    from tests import helpers as H
+    w = W.config5(0.02)
+    host = w.to("cpu", torch.float64)
+    conv = H.dense_convolve(w.model)
+    args = (host.node_features, host.sender, host.receiver, host.shift, conv)
+    _, forces = w.model.energy_and_forces(host.positions, *args)
+    direction = torch.from_numpy(np.random.default_rng(0).standard_normal(tuple(host.positions.shape)))
+    h = 1e-5
+    slope = (w.model.energy(host.positions + h * direction, *args)
+             - w.model.energy(host.positions - h * direction, *args)) / (2 * h)
+    torch.testing.assert_close(slope, -(forces * direction).sum(), rtol=1e-6, atol=1e-8)
+    # translation invariance of a periodic cell: no net force
+    assert float(forces.sum(0).abs().max()) < 1e-12
