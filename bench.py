@@ -34,12 +34,16 @@ if ROOT not in sys.path:
 
 HBM_PEAK_GBS = 8000.0
 
-#: HBM bytes per launch of the backward kernel on the full cfg3 workload, from two
+#: HBM bytes per launch of the convolution kernels on the full cfg3 workload, from two
 #: `rocprofv3 --pmc` runs of this script (FETCH_SIZE and WRITE_SIZE, KiB per dispatch), each
-#: scaled by what the same counter reads for a 1 GiB device copy (`--calibrate-copy`):
-#: 2.0 * 10.24e6 KiB fetched + 1.0 * 18.96e6 KiB written.  Only quoted for that workload.
-MEASURED_TRAFFIC_BYTES = {("cfg3", 1.0, "trailing"): {"backward": 2.0 * 10.236e6 * 1024 + 18.959e6 * 1024,
-                                          "forward": 2.0 * 9.399e6 * 1024 + 1.584e6 * 1024}}
+#: scaled by what the same counter reads for a 1 GiB device copy (`--calibrate-copy`: 2.0 for
+#: FETCH_SIZE, 1.0 for WRITE_SIZE).  Only quoted for the workloads they were measured on.
+MEASURED_TRAFFIC_BYTES = {
+    ("cfg3", 1.0, "trailing"): {"backward": 2.0 * 7.453e6 * 1024 + 18.96e6 * 1024,
+                                "forward": 2.0 * 6.264e6 * 1024 + 1.584e6 * 1024},
+    ("cfg3", 1.0, "leading"): {"backward": 2.0 * 7.404e6 * 1024 + 19.08e6 * 1024,
+                               "forward": 2.0 * 6.259e6 * 1024 + 1.592e6 * 1024},
+}
 
 
 def parse_args():
