@@ -52,7 +52,7 @@ LAUNCH = {
     32: dict(fwd=[(1, 4, 1)], bwd=[(1, 4, 1)]),
     64: dict(fwd=[(1, 4, 1), (1, 4, 2)], bwd=[(1, 4, 2), (1, 4, 1), (1, 4, 3), (1, 4, 4)]),
     128: dict(fwd=[(1, 4, 1), (1, 4, 2), (2, 4, 2), (2, 4, 4)],
-              bwd=[(1, 4, 2), (1, 4, 1), (1, 4, 3), (1, 4, 4), (2, 4, 4)]),
+              bwd=[(2, 4, 3), (1, 4, 1), (1, 4, 3), (1, 4, 4), (2, 4, 4), (1, 4, 2)]),
 }
 
 

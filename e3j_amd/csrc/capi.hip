@@ -26,8 +26,9 @@ int check_hip(hipError_t err, const char *what) {
     return set_error(E3J_AMD_INTERNAL, std::string(what) + ": " + hipGetErrorString(err));
 }
 
-const Tuning &tuning() {
-    static const Tuning t = [] {
+namespace {
+Tuning &mutable_tuning() {
+    static Tuning t = [] {
         Tuning v{0, 0};
         if (const char *e = std::getenv("E3J_AMD_FWD_VARIANT")) v.fwd_variant = std::atoi(e);
         if (const char *e = std::getenv("E3J_AMD_BWD_VARIANT")) v.bwd_variant = std::atoi(e);
@@ -35,6 +36,9 @@ const Tuning &tuning() {
     }();
     return t;
 }
+}  // namespace
+
+const Tuning &tuning() { return mutable_tuning(); }
 
 namespace {
 
@@ -127,6 +131,10 @@ extern "C" {
 const char *e3j_amd_last_error(void) { return g_last_error.c_str(); }
 
 const char *e3j_amd_version(void) { return "e3j_amd 0.1 (gfx950)"; }
+
+void e3j_amd_set_launch_variant(int32_t fwd_variant, int32_t bwd_variant) {
+    mutable_tuning() = Tuning{fwd_variant, bwd_variant};
+}
 
 int e3j_amd_convolution_fwd(const e3j_amd_conv_params *p, const void *coef, const void *x,
                             const void *y, const void *s, const int32_t *sender,

@@ -149,6 +149,29 @@ __device__ __forceinline__ void store_stream<4>(float *p, const Vec<4> &a) {
     __builtin_nontemporal_store(t, reinterpret_cast<f32x4 *>(p));
 }
 
+// Backward: the C channels of a lane lie a wave apart (lane, lane + 64, ...), so each of the C
+// accesses of a wave is one coalesced 256-byte piece of a row and every float atomic request
+// carries 16 values (atomics retire per 64-byte request, whatever it holds).
+template <int C>
+__device__ __forceinline__ Vec<C> load_apart(const float *p) {
+    Vec<C> r;
+#pragma unroll
+    for (int t = 0; t < C; t++) r.v[t] = p[t * kWave];
+    return r;
+}
+template <int C>
+__device__ __forceinline__ Vec<C> load_apart_stream(const float *p) {
+    Vec<C> r;
+#pragma unroll
+    for (int t = 0; t < C; t++) r.v[t] = __builtin_nontemporal_load(p + t * kWave);
+    return r;
+}
+template <int C>
+__device__ __forceinline__ void store_apart_stream(float *p, const Vec<C> &a) {
+#pragma unroll
+    for (int t = 0; t < C; t++) __builtin_nontemporal_store(a.v[t], p + t * kWave);
+}
+
 __device__ __forceinline__ int uniform(int v) { return __builtin_amdgcn_readfirstlane(v); }
 
 // Pin a wave-uniform value (scalar register) into a vector register.  A VALU operation
@@ -347,7 +370,7 @@ struct DsRows {
     bool active;
     template <int L>
     __device__ __forceinline__ void put(const Vec<CPL> &v) const {
-        if (active) store_stream<CPL>(row + L * K, v);
+        if (active) store_apart_stream<CPL>(row + L * K, v);
     }
 };
 
@@ -364,7 +387,8 @@ __device__ __forceinline__ void unrolled_bwd_part(
     using SL = Slice<K, CPL>;
     using Red = WaveReduce<Y>;
 
-    const int c_raw = slice * SL::WIDTH + lane * CPL;
+    static_assert(CPL == 1 || SL::FULL, "several channels per lane need whole slices");
+    const int c_raw = slice * SL::WIDTH + lane;  // further channels of the lane: + 64, + 128, ...
     const bool active = SL::FULL || c_raw < K;
     const int c0 = active ? c_raw : 0;
 
@@ -373,7 +397,7 @@ __device__ __forceinline__ void unrolled_bwd_part(
         const float *zr = dm + (int64_t)r * (Z * K) + c0;
 #pragma unroll
         for (int i = 0; i < NZ; i++) {
-            dmr[i] = vmul(load_stream<CPL>(zr + Part::kZ[i] * K), scale);
+            dmr[i] = vmul(load_apart_stream<CPL>(zr + Part::kZ[i] * K), scale);
             if (!active) dmr[i] = vzero<CPL>();  // idle lanes must add nothing to dy
         }
     }
@@ -395,9 +419,9 @@ __device__ __forceinline__ void unrolled_bwd_part(
         const float *sr = s + ee_n * (int64_t)(S * K) + c0;
         const float *yr = y + ee_n * Y;
 #pragma unroll
-        for (int j = 0; j < NX; j++) xn[j] = load_vec<CPL>(xr + Part::kX[j] * K);
+        for (int j = 0; j < NX; j++) xn[j] = load_apart<CPL>(xr + Part::kX[j] * K);
 #pragma unroll
-        for (int l = 0; l < NS; l++) sn[l] = load_stream<CPL>(sr + Part::kS[l] * K);
+        for (int l = 0; l < NS; l++) sn[l] = load_apart_stream<CPL>(sr + Part::kS[l] * K);
 #pragma unroll
         for (int k = 0; k < Y; k++) yn[k] = yr[k];
     };
@@ -430,7 +454,7 @@ __device__ __forceinline__ void unrolled_bwd_part(
 #pragma unroll
             for (int j = 0; j < NX; j++) {
 #pragma unroll
-                for (int t = 0; t < CPL; t++) unsafeAtomicAdd(dxr + Part::kX[j] * K + t, dxe[j].v[t]);
+                for (int t = 0; t < CPL; t++) unsafeAtomicAdd(dxr + Part::kX[j] * K + t * kWave, dxe[j].v[t]);
             }
         }
         const float total = Red::run(dye, lane);

@@ -117,6 +117,14 @@ int e3j_amd_find_signature(const void *coef_host, int32_t coef_idx_bytes, int32_
                            int32_t num_scalars, int32_t channels, int32_t layout,
                            float *coef_scale);
 
+/* Tuning aid: selects which launch shape (channels per lane, waves per block, parts) of a
+ * signature's kernels later calls use; 0 = default, unknown numbers = default.  The
+ * environment variables E3J_AMD_FWD_VARIANT / E3J_AMD_BWD_VARIANT give the initial values.
+ * Process-wide and not synchronised with running calls.  Results do not depend on it.
+ * No counterpart in the reference, whose launch shape is planned on the host per call
+ * (src/e3j/ops/convolution.py:178-208). */
+void e3j_amd_set_launch_variant(int32_t fwd_variant, int32_t bwd_variant);
+
 /* Number of built-in signatures and a printable description of one. */
 int e3j_amd_num_signatures(void);
 const char *e3j_amd_signature_name(int signature);

@@ -72,3 +72,37 @@ def test_scaled_table_uses_unrolled_kernel():
     out = m(d.x, d.y, d.s, d.sender, d.receiver)
     base = w.module(d.x, d.y, d.s, d.sender, d.receiver)
     torch.testing.assert_close(out, base / 30.0, rtol=2e-6, atol=1e-6)
+
+
+@pytest.mark.parametrize("layout", ["TRAILING_CHANNELS", "LEADING_CHANNELS"])
+@pytest.mark.parametrize("name", ["cfg3", "cfg2"])
+def test_every_launch_variant_gives_the_same_results(name, layout):
+    """The launch shapes of a signature (channels per lane, parts, waves per block) differ in how
+    the work is dealt to waves, not in what is computed: forward bit-identical, backward equal
+    up to the order of the dx / dy atomic sums."""
+    w = CASES[name]().with_layout(layout)
+    d = w.to("cuda")
+    m = w.module
+    coef = m._packed_coef("float32")
+    lib = _lib.load()
+
+    def run():
+        out = e3j_amd.convolution(coef, d.x, d.y, d.s, d.sender, d.receiver, m.params, m.graph_ordering,
+                                  layout=m.layout)
+        grads = e3j_amd.convolution_bwd(coef, d.x, d.y, d.s, d.sender, d.receiver, d.dm, m.params,
+                                        m.graph_ordering, layout=m.layout)
+        torch.cuda.synchronize()
+        return out, grads
+
+    try:
+        lib.e3j_amd_set_launch_variant(0, 0)
+        out0, grads0 = run()
+        for variant in range(1, 8):  # numbers past the last variant fall back to the default
+            lib.e3j_amd_set_launch_variant(variant, variant)
+            out, grads = run()
+            assert torch.equal(out, out0), f"forward variant {variant}"
+            for g, g0, what in zip(grads, grads0, ("dx", "dy", "ds")):
+                scale = float(g0.abs().max())
+                assert float((g - g0).abs().max()) <= 2e-5 * scale, f"backward variant {variant} {what}"
+    finally:
+        lib.e3j_amd_set_launch_variant(0, 0)
