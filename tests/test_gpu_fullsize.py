@@ -17,9 +17,15 @@ def _run(w, ordering=None):
     m = w.module
     coef = m._packed_coef("float32")
     ordering = ordering or m.graph_ordering
-    out = e3j_amd.convolution(coef, w.x, w.y, w.s, w.sender, w.receiver, m.params, ordering)
-    grads = e3j_amd.convolution_bwd(coef, w.x, w.y, w.s, w.sender, w.receiver, w.dm, m.params, ordering)
+    out = e3j_amd.convolution(coef, w.x, w.y, w.s, w.sender, w.receiver, m.params, ordering,
+                              layout=m.layout)
+    grads = e3j_amd.convolution_bwd(coef, w.x, w.y, w.s, w.sender, w.receiver, w.dm, m.params, ordering,
+                                    layout=m.layout)
     return out, grads
+
+
+def _trailing(t, w):
+    return (t.transpose(1, 2) if w.leading and t.dim() == 3 else t).cpu().numpy()
 
 
 def _against_c_oracle(w, out, grads, tag):
@@ -31,17 +37,24 @@ def _against_c_oracle(w, out, grads, tag):
     mag_args = tuple(np.abs(t) for t in args[:3]) + args[3:]
     ref = c_oracle.convolution(idx, val, mix, *args, Z)
     mag = c_oracle.convolution(idx, np.abs(val), mix, *mag_args, Z)
-    H.assert_parity(out.cpu().numpy(), ref.astype(np.float64), 2.0 * mag.astype(np.float64), f"{tag} out", ulps=32.0)
+    H.assert_parity(_trailing(out, w), ref.astype(np.float64), 2.0 * mag.astype(np.float64), f"{tag} out", ulps=32.0)
     refs = c_oracle.convolution_vjp(idx, val, mix, *args, a["dm"])
     mags = c_oracle.convolution_vjp(idx, np.abs(val), mix, *mag_args, np.abs(a["dm"]))
     for g, r, m, name in zip(grads, refs, mags, ("dx", "dy", "ds")):
-        H.assert_parity(g.cpu().numpy(), r.astype(np.float64), 2.0 * m.astype(np.float64), f"{tag} {name}", ulps=32.0)
+        H.assert_parity(_trailing(g, w), r.astype(np.float64), 2.0 * m.astype(np.float64), f"{tag} {name}", ulps=32.0)
 
 
 def test_config1_and_config2_full_size_match_checker():
     for w in (W.config1(device="cuda"), W.config2(device="cuda")):
         out, grads = _run(w)
         _against_c_oracle(w, out, grads, w.name)
+
+
+def test_config2_leading_layout_full_size_matches_checker():
+    """The configuration as the baseline names it: channels before the irreps axis."""
+    w = W.config2(device="cuda").with_layout("LEADING_CHANNELS")
+    out, grads = _run(w)
+    _against_c_oracle(w, out, grads, "cfg2 leading")
 
 
 def test_config4_unsorted_skewed_matches_checker():
@@ -68,6 +81,14 @@ def test_config3_full_size_properties():
     # the forward is bit-reproducible
     again, _ = _run(w)
     assert torch.equal(out, again)
+    # the leading-channels layout gives the same numbers (forward: the same sums in the same order)
+    wl = w.with_layout("LEADING_CHANNELS")
+    out_l, (dx_l, dy_l, ds_l) = _run(wl)
+    assert torch.equal(out_l.transpose(1, 2), out)
+    torch.testing.assert_close(ds_l.transpose(1, 2), ds, rtol=1e-5, atol=1e-6)
+    assert float((dx_l.transpose(1, 2) - dx).abs().max()) <= 2e-5 * float(dx.abs().max())
+    assert float((dy_l - dy).abs().max()) <= 2e-5 * float(dy.abs().max())
+    del wl, out_l, dx_l, dy_l, ds_l
     # a head of the workload agrees with the C checker
     head = w.head(64)
     idx, val, mix = w.table()
