@@ -94,7 +94,7 @@ class AbiCalls:
         self.table = _Table.get(packed, np.float32)
         d = 2 if w.leading else 1
         dims = (w.x.shape[d], w.y.shape[1], module.params.num_out, w.s.shape[d])
-        sig, scale = self.table.signature(tuple(int(d) for d in dims), w.channels, module.layout)
+        sig, scale, _ = self.table.signature(tuple(int(d) for d in dims), w.channels, module.layout)
         self.signature = sig
         self.params = _lib.ConvParams(
             num_nodes=w.num_nodes, num_edges=w.num_edges, num_coef=self.table.num_coef,

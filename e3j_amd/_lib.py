@@ -38,6 +38,7 @@ class ConvParams(ctypes.Structure):
         ("signature", ctypes.c_int32),
         ("coef_scale", ctypes.c_float),
         ("debug", ctypes.c_int32),
+        ("y_flip", ctypes.c_uint32),
         ("row_order", ctypes.c_void_p),
     ]
 
@@ -60,7 +61,8 @@ SYMBOLS = {
     "e3j_amd_convolution_fwd": (ctypes.c_int, [_PARAMS] + [_P] * 9),
     "e3j_amd_convolution_bwd_sender": (ctypes.c_int, [_PARAMS] + [_P] * 12),
     "e3j_amd_convolution_bwd_receiver": (ctypes.c_int, [_PARAMS] + [_P] * 12),
-    "e3j_amd_find_signature": (ctypes.c_int, [_P] + [ctypes.c_int32] * 9 + [ctypes.POINTER(ctypes.c_float)]),
+    "e3j_amd_find_signature": (ctypes.c_int, [_P] + [ctypes.c_int32] * 9 + [ctypes.POINTER(ctypes.c_float),
+                                                                             ctypes.POINTER(ctypes.c_uint32)]),
     "e3j_amd_num_signatures": (ctypes.c_int, []),
     "e3j_amd_signature_name": (ctypes.c_char_p, [ctypes.c_int]),
     "e3j_amd_csr_workspace_bytes": (ctypes.c_size_t, [ctypes.c_int32, ctypes.c_int64]),

@@ -359,9 +359,10 @@ def emit_signature(sig_id: int, name: str, x_irreps: str, y_irreps: str, out_fil
             names.append(sname)
         part_names[zs] = ", ".join(names)
     fwd_args = ["    const float *, const float *, const float *, const int32_t *, const int32_t *,",
-                "    const int32_t *, const int32_t *, float *, int, float);"]
+                "    const int32_t *, const int32_t *, float *, int, float, unsigned);"]
     bwd_args = ["    const float *, const float *, const float *, const float *, const int32_t *,",
-                "    const int32_t *, const int32_t *, const int32_t *, float *, float *, float *, int, float);"]
+                "    const int32_t *, const int32_t *, const int32_t *, float *, float *, float *, int, float,",
+                "    unsigned);"]
     out += ["}  // namespace", "", "// both passes: the device pass needs the kernels instantiated"]
     for cpl, wpb, zs in launch["fwd"]:
         out += [f"template __global__ void unrolled_fwd_kernel<{channels}, {cpl}, {wpb}, {part_names[zs]}>("] + fwd_args

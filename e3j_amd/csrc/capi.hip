@@ -61,6 +61,10 @@ int validate(const e3j_amd_conv_params *p, const char *op) {
     if (p->signature >= num_signatures())
         return set_error(E3J_AMD_INVALID_ARGUMENT,
                          name + ": unknown signature id " + std::to_string(p->signature));
+    if (p->signature < 0 && p->y_flip != 0)
+        return set_error(E3J_AMD_INVALID_ARGUMENT,
+                         name + ": y_flip needs an unrolled kernel (the table-driven kernels take "
+                                "the signs in the table)");
     if (p->signature >= 0) {
         const Signature &sg = signature(p->signature);
         if (p->val_dtype != E3J_AMD_F32 || sg.num_x != p->num_x || sg.num_y != p->num_y ||
@@ -82,6 +86,13 @@ bool aligned16(std::initializer_list<const void *> ptrs) {
 }
 bool signature_fits(const e3j_amd_conv_params *p, std::initializer_list<const void *> ptrs) {
     return p->signature >= 0 && (p->layout == E3J_AMD_LAYOUT_TRAILING || aligned16(ptrs));
+}
+// Falling back to the table-driven kernel is only right when no sign flip was asked for.
+int flip_without_kernel(const e3j_amd_conv_params *p, const char *op) {
+    if (p->y_flip == 0) return E3J_AMD_OK;
+    return set_error(E3J_AMD_INVALID_ARGUMENT,
+                     std::string(op) + ": y_flip needs the unrolled kernel, which these operands "
+                                       "(alignment or grouping) cannot use");
 }
 
 int finish(const e3j_amd_conv_params *p, hipStream_t stream, int rc, const char *op) {
@@ -113,6 +124,7 @@ int run_backward(const e3j_amd_conv_params *p, bool group_is_receiver, const voi
                                          static_cast<float *>(dx), static_cast<float *>(dy),
                                          static_cast<float *>(ds), stream);
     } else {
+        if ((rc = flip_without_kernel(p, op))) return rc;
         if (coef == nullptr && p->num_coef > 0)
             return set_error(E3J_AMD_INVALID_ARGUMENT,
                              std::string(op) + ": this grouping runs the table-driven kernel and needs `coef`");
@@ -153,6 +165,7 @@ int e3j_amd_convolution_fwd(const e3j_amd_conv_params *p, const void *coef, cons
                                          static_cast<const float *>(s), sender, receiver_ptr,
                                          edge_perm, static_cast<float *>(out), stream);
     } else {
+        if ((rc = flip_without_kernel(p, "convolution"))) return rc;
         if (missing(coef, p->num_coef))
             return set_error(E3J_AMD_INVALID_ARGUMENT,
                              "convolution: operands are not 16-byte aligned, which runs the "
@@ -190,27 +203,32 @@ const char *e3j_amd_signature_name(int id) {
 int e3j_amd_find_signature(const void *coef_host, int32_t coef_idx_bytes, int32_t val_dtype,
                            int32_t num_coef, int32_t num_x, int32_t num_y, int32_t num_out,
                            int32_t num_scalars, int32_t channels, int32_t layout,
-                           float *coef_scale) {
+                           float *coef_scale, uint32_t *y_flip) {
     if (coef_scale) *coef_scale = 1.0f;
+    if (y_flip) *y_flip = 0;
     if (coef_host == nullptr || val_dtype != E3J_AMD_F32 || num_coef <= 0) return -1;
     if (coef_idx_bytes != 1 && coef_idx_bytes != 4) return -1;
     const size_t item = coef_idx_bytes == 1 ? sizeof(Coef4D<uint8_t, float>) : sizeof(Coef4D<int32_t, float>);
     const unsigned char *bytes = static_cast<const unsigned char *>(coef_host);
+    const bool signs_allowed = y_flip != nullptr && num_y <= 32;
     for (int id = 0; id < num_signatures(); id++) {
         const Signature &sg = signature(id);
         if (sg.num_coef != num_coef || sg.num_x != num_x || sg.num_y != num_y ||
             sg.num_out != num_out || sg.num_scalars != num_scalars || sg.channels != channels ||
             sg.layout != layout)
             continue;
-        // One uniform positive factor is allowed between the tables; it is taken from
-        // the entry of largest magnitude and every entry must agree to float32 rounding.
+        // One uniform positive factor is allowed between the tables; its magnitude is taken
+        // from the entry of largest magnitude and every entry must agree to float32 rounding.
+        // A negative ratio is a sign flip of that entry's y component, which must then hold
+        // for every entry of the component.
         int big = 0;
         for (int n = 1; n < num_coef; n++)
             if (std::fabs(sg.val[n]) > std::fabs(sg.val[big])) big = n;
         float vbig;
         std::memcpy(&vbig, bytes + big * item, sizeof(float));
-        const double scale = (double)vbig / (double)sg.val[big];
+        const double scale = std::fabs((double)vbig / (double)sg.val[big]);
         bool same = scale > 0.0 && std::isfinite(scale);
+        uint32_t flip = 0, seen = 0;
         for (int n = 0; n < num_coef && same; n++) {
             float v;
             int32_t idx[4];
@@ -219,12 +237,24 @@ int e3j_amd_find_signature(const void *coef_host, int32_t coef_idx_bytes, int32_
                 if (coef_idx_bytes == 1) idx[t] = bytes[n * item + 4 + t];
                 else std::memcpy(&idx[t], bytes + n * item + 4 + 4 * t, 4);
             }
-            const double want = scale * (double)sg.val[n];
-            same = std::fabs((double)v - want) <= 4e-7 * std::fabs(want);
             for (int t = 0; t < 4 && same; t++) same = idx[t] == (int32_t)sg.idx[4 * n + t];
+            if (!same) break;
+            const double want = scale * (double)sg.val[n];
+            const bool plus = std::fabs((double)v - want) <= 4e-7 * std::fabs(want);
+            const bool minus = std::fabs((double)v + want) <= 4e-7 * std::fabs(want);
+            if (plus) {
+                same = !signs_allowed || !((seen >> idx[2]) & 1u) || !((flip >> idx[2]) & 1u);
+            } else if (minus && signs_allowed) {
+                same = !((seen >> idx[2]) & 1u) || ((flip >> idx[2]) & 1u);
+                flip |= 1u << idx[2];
+            } else {
+                same = false;
+            }
+            if (signs_allowed) seen |= 1u << idx[2];
         }
         if (same) {
             if (coef_scale) *coef_scale = (float)scale;
+            if (y_flip) *y_flip = flip;
             return id;
         }
     }

@@ -178,6 +178,12 @@ __device__ __forceinline__ int uniform(int v) { return __builtin_amdgcn_readfirs
 // reads at most one scalar or literal operand, so `literal * y` with y in a scalar
 // register would make the compiler park every coefficient literal in a vector register
 // for the whole kernel; with y in a vector register the literals stay inline.
+// Negate v when bit k of `flip` is set (the parity signs of the y components when a kernel
+// walks the edges of a symmetric graph in the reversed direction).
+__device__ __forceinline__ float flip_sign(float v, unsigned flip, int k) {
+    return __uint_as_float(__float_as_uint(v) ^ (((flip >> k) & 1u) << 31));
+}
+
 __device__ __forceinline__ float to_vgpr(float v) {
     asm volatile("" : "+v"(v));
     return v;
@@ -264,8 +270,7 @@ template <typename Part, int K, int CPL>
 __device__ __forceinline__ void unrolled_fwd_part(
     const float *__restrict__ x, const float *__restrict__ y, const float *__restrict__ s,
     const int32_t *__restrict__ sender, const int32_t *__restrict__ row_ptr,
-    const int32_t *__restrict__ perm, float *__restrict__ out, int num_nodes, float scale,
-    int r, int slice, int lane) {
+    const int32_t *__restrict__ perm, float *__restrict__ out, int num_nodes, float scale, unsigned y_flip, int r, int slice, int lane) {
     constexpr int NX = Part::NX, NS = Part::NS, NZ = Part::NZ, Y = Part::Y;
     constexpr int X = Part::X, S = Part::S, Z = Part::Z;
     using V = Vec<CPL>;
@@ -309,7 +314,7 @@ __device__ __forceinline__ void unrolled_fwd_part(
 #pragma unroll
         for (int l = 0; l < NS; l++) sc[l] = sn[l];
 #pragma unroll
-        for (int k = 0; k < Y; k++) yc[k] = to_vgpr(yn[k]);
+        for (int k = 0; k < Y; k++) yc[k] = to_vgpr(flip_sign(yn[k], y_flip, k));
         const bool valid = valid_n;
         e++;
         if (e < e1) fetch(e);
@@ -325,18 +330,18 @@ __device__ __forceinline__ void unrolled_fwd_part(
 template <int K, int CPL, int I>
 __device__ __forceinline__ void dispatch_fwd(int, const float *, const float *, const float *,
                                              const int32_t *, const int32_t *, const int32_t *,
-                                             float *, int, float, int, int, int) {}
+                                             float *, int, float, unsigned, int, int, int) {}
 template <int K, int CPL, int I, typename Part, typename... Rest>
 __device__ __forceinline__ void dispatch_fwd(int part, const float *x, const float *y, const float *s,
                                              const int32_t *sender, const int32_t *row_ptr,
                                              const int32_t *perm, float *out, int num_nodes,
-                                             float scale, int r, int slice, int lane) {
+                                             float scale, unsigned y_flip, int r, int slice, int lane) {
     if (part == I)
-        unrolled_fwd_part<Part, K, CPL>(x, y, s, sender, row_ptr, perm, out, num_nodes, scale, r,
+        unrolled_fwd_part<Part, K, CPL>(x, y, s, sender, row_ptr, perm, out, num_nodes, scale, y_flip, r,
                                         slice, lane);
     else
         dispatch_fwd<K, CPL, I + 1, Rest...>(part, x, y, s, sender, row_ptr, perm, out, num_nodes,
-                                             scale, r, slice, lane);
+                                             scale, y_flip, r, slice, lane);
 }
 
 // One wave per (receiver, channel slice, part); consecutive waves share a receiver.
@@ -345,7 +350,7 @@ __global__ __launch_bounds__(kWave *WPB) void unrolled_fwd_kernel(
     const float *__restrict__ x, const float *__restrict__ y, const float *__restrict__ s,
     const int32_t *__restrict__ sender, const int32_t *__restrict__ row_ptr,
     const int32_t *__restrict__ perm, const int32_t *__restrict__ row_order,
-    float *__restrict__ out, int num_nodes, float scale) {
+    float *__restrict__ out, int num_nodes, float scale, unsigned y_flip) {
     constexpr int NP = sizeof...(Parts);
     constexpr int CW = Slice<K, CPL>::COUNT;
     const int64_t item = logical_block() * WPB + threadIdx.y;
@@ -354,7 +359,7 @@ __global__ __launch_bounds__(kWave *WPB) void unrolled_fwd_kernel(
     const int slice = uniform((int)((item / NP) % CW));
     const int q = uniform((int)(item / (NP * CW)));
     const int r = row_order ? row_order[q] : q;
-    dispatch_fwd<K, CPL, 0, Parts...>(part, x, y, s, sender, row_ptr, perm, out, num_nodes, scale, r,
+    dispatch_fwd<K, CPL, 0, Parts...>(part, x, y, s, sender, row_ptr, perm, out, num_nodes, scale, y_flip, r,
                                       slice, threadIdx.x);
 }
 
@@ -380,7 +385,7 @@ __device__ __forceinline__ void unrolled_bwd_part(
     const float *__restrict__ dm, const int32_t *__restrict__ sender,
     const int32_t *__restrict__ row_ptr, const int32_t *__restrict__ perm,
     float *__restrict__ dx, float *__restrict__ dy, float *__restrict__ ds, int num_nodes,
-    float scale, int r, int slice, int lane) {
+    float scale, unsigned y_flip, int r, int slice, int lane) {
     constexpr int NX = Part::NX, NS = Part::NS, NZ = Part::NZ, Y = Part::Y;
     constexpr int X = Part::X, S = Part::S, Z = Part::Z;
     using V = Vec<CPL>;
@@ -434,7 +439,7 @@ __device__ __forceinline__ void unrolled_bwd_part(
 #pragma unroll
         for (int l = 0; l < NS; l++) sc[l] = sn[l];
 #pragma unroll
-        for (int k = 0; k < Y; k++) yc[k] = to_vgpr(yn[k]);
+        for (int k = 0; k < Y; k++) yc[k] = to_vgpr(flip_sign(yn[k], y_flip, k));
         const bool valid = valid_n;
         const int snd = snd_n;
         const int64_t ee = ee_n;
@@ -457,8 +462,8 @@ __device__ __forceinline__ void unrolled_bwd_part(
                 for (int t = 0; t < CPL; t++) unsafeAtomicAdd(dxr + Part::kX[j] * K + t * kWave, dxe[j].v[t]);
             }
         }
-        const float total = Red::run(dye, lane);
         const int k = Red::slot(lane);
+        const float total = flip_sign(Red::run(dye, lane), y_flip, k);
         if (lane < 16 && k < Y) {
             if (kAtomicDy) unsafeAtomicAdd(dy + ee * Y + k, total);  // dy zero-filled by the launcher
             else dy[ee * Y + k] = total;
@@ -470,19 +475,19 @@ template <int K, int CPL, bool A, int I>
 __device__ __forceinline__ void dispatch_bwd(int, const float *, const float *, const float *,
                                              const float *, const int32_t *, const int32_t *,
                                              const int32_t *, float *, float *, float *, int, float,
-                                             int, int, int) {}
+                                             unsigned, int, int, int) {}
 template <int K, int CPL, bool A, int I, typename Part, typename... Rest>
 __device__ __forceinline__ void dispatch_bwd(int part, const float *x, const float *y, const float *s,
                                              const float *dm, const int32_t *sender,
                                              const int32_t *row_ptr, const int32_t *perm, float *dx,
-                                             float *dy, float *ds, int num_nodes, float scale, int r,
+                                             float *dy, float *ds, int num_nodes, float scale, unsigned y_flip, int r,
                                              int slice, int lane) {
     if (part == I)
         unrolled_bwd_part<Part, K, CPL, A>(x, y, s, dm, sender, row_ptr, perm, dx, dy, ds, num_nodes,
-                                           scale, r, slice, lane);
+                                           scale, y_flip, r, slice, lane);
     else
         dispatch_bwd<K, CPL, A, I + 1, Rest...>(part, x, y, s, dm, sender, row_ptr, perm, dx, dy, ds,
-                                                num_nodes, scale, r, slice, lane);
+                                                num_nodes, scale, y_flip, r, slice, lane);
 }
 
 template <int K, int CPL, int WPB, typename... Parts>
@@ -492,7 +497,7 @@ void unrolled_bwd_kernel(
     const float *__restrict__ dm, const int32_t *__restrict__ sender,
     const int32_t *__restrict__ row_ptr, const int32_t *__restrict__ perm,
     const int32_t *__restrict__ row_order, float *__restrict__ dx, float *__restrict__ dy,
-    float *__restrict__ ds, int num_nodes, float scale) {
+    float *__restrict__ ds, int num_nodes, float scale, unsigned y_flip) {
     constexpr int NP = sizeof...(Parts);
     constexpr int CW = Slice<K, CPL>::COUNT;
     constexpr bool kAtomicDy = NP * CW > 1;  // several waves add into one dy row
@@ -503,7 +508,7 @@ void unrolled_bwd_kernel(
     const int q = uniform((int)(item / (NP * CW)));
     const int r = row_order ? row_order[q] : q;
     dispatch_bwd<K, CPL, kAtomicDy, 0, Parts...>(part, x, y, s, dm, sender, row_ptr, perm, dx, dy, ds,
-                                                 num_nodes, scale, r, slice, threadIdx.x);
+                                                 num_nodes, scale, y_flip, r, slice, threadIdx.x);
 }
 
 // ---------------------------------------------------------------------------
@@ -627,7 +632,7 @@ template <typename Part, int K>
 __device__ __forceinline__ void unrolled_fwd_leading(
     const float *__restrict__ x, const float *__restrict__ y, const float *__restrict__ s,
     const int32_t *__restrict__ sender, const int32_t *__restrict__ row_ptr,
-    const int32_t *__restrict__ perm, float *__restrict__ out, int num_nodes, float scale, int r,
+    const int32_t *__restrict__ perm, float *__restrict__ out, int num_nodes, float scale, unsigned y_flip, int r,
     int slice, int lane, float *strip) {
     constexpr int NX = Part::NX, NS = Part::NS, NZ = Part::NZ, Y = Part::Y;
     constexpr int X = Part::X, S = Part::S, Z = Part::Z;
@@ -676,7 +681,7 @@ __device__ __forceinline__ void unrolled_fwd_leading(
 #pragma unroll
         for (int l = 0; l < NS; l++) sc[l].v[0] = strip_s[cl * G::PS + Part::kS[l]];
 #pragma unroll
-        for (int k = 0; k < Y; k++) yc[k] = to_vgpr(yn[k]);
+        for (int k = 0; k < Y; k++) yc[k] = to_vgpr(flip_sign(yn[k], y_flip, k));
         const bool valid = valid_n;
         e++;
         if (e < e1) fetch(e);
@@ -704,7 +709,7 @@ __global__ __launch_bounds__(kWave *WPB) void unrolled_fwd_leading_kernel(
     const float *__restrict__ x, const float *__restrict__ y, const float *__restrict__ s,
     const int32_t *__restrict__ sender, const int32_t *__restrict__ row_ptr,
     const int32_t *__restrict__ perm, const int32_t *__restrict__ row_order,
-    float *__restrict__ out, int num_nodes, float scale) {
+    float *__restrict__ out, int num_nodes, float scale, unsigned y_flip) {
     using G = LeadingGeometry<K, Part::X, Part::S, Part::Z>;
     __shared__ __attribute__((aligned(16))) float strips[WPB * G::REGION];
     const int64_t item = logical_block() * WPB + threadIdx.y;
@@ -712,7 +717,7 @@ __global__ __launch_bounds__(kWave *WPB) void unrolled_fwd_leading_kernel(
     const int slice = uniform((int)(item % G::COUNT));
     const int q = uniform((int)(item / G::COUNT));
     const int r = row_order ? row_order[q] : q;
-    unrolled_fwd_leading<Part, K>(x, y, s, sender, row_ptr, perm, out, num_nodes, scale, r, slice,
+    unrolled_fwd_leading<Part, K>(x, y, s, sender, row_ptr, perm, out, num_nodes, scale, y_flip, r, slice,
                                   threadIdx.x, strips + threadIdx.y * G::REGION);
 }
 
@@ -751,7 +756,7 @@ __device__ __forceinline__ void unrolled_bwd_leading(
     const float *__restrict__ dm, const int32_t *__restrict__ sender,
     const int32_t *__restrict__ row_ptr, const int32_t *__restrict__ perm,
     float *__restrict__ dx, float *__restrict__ dy, float *__restrict__ ds, int num_nodes,
-    float scale, int r, int slice, int lane, int tid, float *region) {
+    float scale, unsigned y_flip, int r, int slice, int lane, int tid, float *region) {
     constexpr int NX = Part::NX, NS = Part::NS, NZ = Part::NZ, Y = Part::Y;
     constexpr int X = Part::X, S = Part::S, Z = Part::Z;
     static_assert(X <= 64 && S <= 64, "part masks hold 64 columns");
@@ -825,7 +830,7 @@ __device__ __forceinline__ void unrolled_bwd_leading(
 #pragma unroll
         for (int l = 0; l < NS; l++) sc[l].v[0] = in_s[cl * G::PS + Part::kS[l]];
 #pragma unroll
-        for (int k = 0; k < Y; k++) yc[k] = to_vgpr(yn[k]);
+        for (int k = 0; k < Y; k++) yc[k] = to_vgpr(flip_sign(yn[k], y_flip, k));
         const bool valid = valid_n;  // uniform over the block: every wave looks at the same edge
         const int snd = snd_n;
         const int64_t ee = ee_n;
@@ -858,8 +863,8 @@ __device__ __forceinline__ void unrolled_bwd_leading(
 
 #pragma unroll
         for (int k = Y; k < Red::P; k++) dye[k] = 0.f;
-        const float total = Red::run(dye, lane);
         const int k = Red::slot(lane);
+        const float total = flip_sign(Red::run(dye, lane), y_flip, k);
         if (lane < 16 && k < Y) {
             if (NP > 1 || G::COUNT > 1) unsafeAtomicAdd(dy + ee * Y + k, total);  // dy zero-filled by the launcher
             else dy[ee * Y + k] = total;
@@ -871,20 +876,20 @@ template <int K, int NP, unsigned long long kCoveredDx, int I>
 __device__ __forceinline__ void dispatch_bwd_leading(int, const float *, const float *, const float *,
                                                      const float *, const int32_t *, const int32_t *,
                                                      const int32_t *, float *, float *, float *, int,
-                                                     float, int, int, int, int, float *) {}
+                                                     float, unsigned, int, int, int, int, float *) {}
 template <int K, int NP, unsigned long long kCoveredDx, int I, typename Part, typename... Rest>
 __device__ __forceinline__ void dispatch_bwd_leading(int part, const float *x, const float *y,
                                                      const float *s, const float *dm,
                                                      const int32_t *sender, const int32_t *row_ptr,
                                                      const int32_t *perm, float *dx, float *dy,
-                                                     float *ds, int num_nodes, float scale, int r,
+                                                     float *ds, int num_nodes, float scale, unsigned y_flip, int r,
                                                      int slice, int lane, int tid, float *region) {
     if (part == I)
         unrolled_bwd_leading<Part, K, NP, kCoveredDx>(x, y, s, dm, sender, row_ptr, perm, dx, dy, ds,
-                                                      num_nodes, scale, r, slice, lane, tid, region);
+                                                      num_nodes, scale, y_flip, r, slice, lane, tid, region);
     else
         dispatch_bwd_leading<K, NP, kCoveredDx, I + 1, Rest...>(part, x, y, s, dm, sender, row_ptr, perm,
-                                                                dx, dy, ds, num_nodes, scale, r, slice,
+                                                                dx, dy, ds, num_nodes, scale, y_flip, r, slice,
                                                                 lane, tid, region);
 }
 
@@ -899,7 +904,7 @@ __global__ __launch_bounds__(kWave * sizeof...(Parts)) void unrolled_bwd_leading
     const float *__restrict__ dm, const int32_t *__restrict__ sender,
     const int32_t *__restrict__ row_ptr, const int32_t *__restrict__ perm,
     const int32_t *__restrict__ row_order, float *__restrict__ dx, float *__restrict__ dy,
-    float *__restrict__ ds, int num_nodes, float scale) {
+    float *__restrict__ ds, int num_nodes, float scale, unsigned y_flip) {
     using P0 = typename FirstOf<Parts...>::type;
     constexpr int NP = sizeof...(Parts);
     using G = LeadingBwdGeometry<K, P0::X, P0::S, P0::Z, NP>;
@@ -912,7 +917,7 @@ __global__ __launch_bounds__(kWave * sizeof...(Parts)) void unrolled_bwd_leading
     const int r = row_order ? row_order[q] : q;
     const int part = uniform((int)threadIdx.y);
     dispatch_bwd_leading<K, NP, kCoveredDx, 0, Parts...>(
-        part, x, y, s, dm, sender, row_ptr, perm, dx, dy, ds, num_nodes, scale, r, slice,
+        part, x, y, s, dm, sender, row_ptr, perm, dx, dy, ds, num_nodes, scale, y_flip, r, slice,
         threadIdx.x, threadIdx.y * kWave + threadIdx.x, region);
 }
 
@@ -925,7 +930,7 @@ int launch_unrolled_fwd(const e3j_amd_conv_params &p, const float *x, const floa
     if (blocks > 0x7fffffffLL) return set_error(E3J_AMD_INVALID_ARGUMENT, "convolution: grid too large");
     hipLaunchKernelGGL((unrolled_fwd_kernel<K, CPL, WPB, Parts...>), dim3((unsigned)blocks),
                        dim3(kWave, WPB), 0, stream, x, y, s, sender, row_ptr, perm, p.row_order, out,
-                       p.num_nodes, p.coef_scale);
+                       p.num_nodes, p.coef_scale, p.y_flip);
     return check_hip(hipGetLastError(), "convolution forward launch");
 }
 
@@ -946,7 +951,7 @@ int launch_unrolled_bwd(const e3j_amd_conv_params &p, const float *x, const floa
     if (blocks > 0x7fffffffLL) return set_error(E3J_AMD_INVALID_ARGUMENT, "convolution_bwd: grid too large");
     hipLaunchKernelGGL((unrolled_bwd_kernel<K, CPL, WPB, Parts...>), dim3((unsigned)blocks),
                        dim3(kWave, WPB), 0, stream, x, y, s, dm, sender, row_ptr, perm, p.row_order,
-                       dx, dy, ds, p.num_nodes, p.coef_scale);
+                       dx, dy, ds, p.num_nodes, p.coef_scale, p.y_flip);
     return check_hip(hipGetLastError(), "convolution backward launch");
 }
 
@@ -960,7 +965,7 @@ int launch_unrolled_fwd_leading(const e3j_amd_conv_params &p, const float *x, co
     if (blocks > 0x7fffffffLL) return set_error(E3J_AMD_INVALID_ARGUMENT, "convolution: grid too large");
     hipLaunchKernelGGL((unrolled_fwd_leading_kernel<K, WPB, Part>), dim3((unsigned)blocks),
                        dim3(kWave, WPB), 0, stream, x, y, s, sender, row_ptr, perm, p.row_order, out,
-                       p.num_nodes, p.coef_scale);
+                       p.num_nodes, p.coef_scale, p.y_flip);
     return check_hip(hipGetLastError(), "convolution forward launch");
 }
 
@@ -984,7 +989,7 @@ int launch_unrolled_bwd_leading(const e3j_amd_conv_params &p, const float *x, co
     if (blocks > 0x7fffffffLL) return set_error(E3J_AMD_INVALID_ARGUMENT, "convolution_bwd: grid too large");
     hipLaunchKernelGGL((unrolled_bwd_leading_kernel<K, Parts...>), dim3((unsigned)blocks),
                        dim3(kWave, NP), 0, stream, x, y, s, dm, sender, row_ptr, perm, p.row_order,
-                       dx, dy, ds, p.num_nodes, p.coef_scale);
+                       dx, dy, ds, p.num_nodes, p.coef_scale, p.y_flip);
     return check_hip(hipGetLastError(), "convolution backward launch");
 }
 

@@ -10,7 +10,7 @@
 // the first of the three, sorted for dx with columns (j, i, k, l), is then used.
 // A third target, "convolution_bwd_receiver", takes the forward's receiver CSR:
 //   coef, x, y, s, dm, sender, receiver_ptr, edge_perm -> dx, dy, ds.
-// Attributes: num_nodes, debug (reference); layout, signature, coef_scale,
+// Attributes: num_nodes, debug (reference); layout, signature, coef_scale, y_flip,
 // coef_stacked (optional).  Handlers are re-entrant, allocate nothing and
 // enqueue on the stream XLA hands over; they answer the metadata query.
 
@@ -106,6 +106,7 @@ void *decode_common(XlaCallFrame *f, const char *op, const XlaBuffer *coef, cons
     p.layout = attr<int32_t>(f, "layout", kXlaS32, E3J_AMD_LAYOUT_TRAILING);
     p.signature = attr<int32_t>(f, "signature", kXlaS32, -1);
     p.coef_scale = attr<float>(f, "coef_scale", kXlaF32, 1.0f);
+    p.y_flip = (uint32_t)attr<int32_t>(f, "y_flip", kXlaS32, 0);
     p.num_edges = y->dims[0];
     p.num_y = (int32_t)y->dims[1];
     if (y->rank == 3 && y->dims[2] != 1)

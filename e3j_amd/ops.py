@@ -87,16 +87,20 @@ class _Table:
         return t
 
     def signature(self, dims, channels: int, layout: Layout):
-        """`(id, scale)` of a built-in unrolled kernel, `(-1, 1.0)` if none matches."""
+        """`(id, scale, y_flip)` of a built-in unrolled kernel, `(-1, 1.0, 0)` if none matches.
+
+        `y_flip`: bit mask of the y components whose coefficients carry the opposite sign of
+        the built-in table (the parity signs of the SENDER ordering).
+        """
         key = (dims, channels, layout)
         hit = self._signature.get(key)
         if hit is None:
-            scale = ctypes.c_float(1.0)
+            scale, flip = ctypes.c_float(1.0), ctypes.c_uint32(0)
             val_code = _lib.F32 if self.val_np_dtype == np.float32 else _lib.F64
             sig = _lib.load().e3j_amd_find_signature(
                 self.packed.ctypes.data, self.idx_bytes, val_code, self.num_coef, dims[0], dims[1],
-                dims[2], dims[3], channels, layout.value, ctypes.byref(scale))
-            hit = self._signature[key] = (int(sig), float(scale.value))
+                dims[2], dims[3], channels, layout.value, ctypes.byref(scale), ctypes.byref(flip))
+            hit = self._signature[key] = (int(sig), float(scale.value), int(flip.value))
         return hit
 
 
@@ -119,25 +123,27 @@ def _stream(device) -> int:
     return int(torch.cuda.current_stream(device).cuda_stream)
 
 
-def _fill_params(meta: _Meta, x: torch.Tensor, y: torch.Tensor, s: torch.Tensor, forward: bool,
+def _shape(meta: _Meta, x: torch.Tensor, y: torch.Tensor, s: torch.Tensor):
+    """`((num_x, num_y, num_out, num_scalars), channels)` of a call."""
+    if meta.layout == Layout.TRAILING_CHANNELS:
+        num_x, channels, num_s = x.shape[1], x.shape[2], s.shape[1]
+    else:
+        channels, num_x, num_s = x.shape[1], x.shape[2], s.shape[2]
+    return (int(num_x), int(y.shape[1]), int(meta.params.num_out), int(num_s)), int(channels)
+
+
+def _fill_params(meta: _Meta, x: torch.Tensor, y: torch.Tensor, s: torch.Tensor, table: _Table,
                  use_signature: bool = True, row_order: torch.Tensor | None = None):
     layout = meta.layout
-    if layout == Layout.TRAILING_CHANNELS:
-        num_x, channels = x.shape[1], x.shape[2]
-        num_s = s.shape[1]
-    else:
-        channels, num_x = x.shape[1], x.shape[2]
-        num_s = s.shape[2]
     val_code = _VAL_DTYPES[x.dtype][0]
-    table = meta.signed_table if (forward and meta.signed_table is not None) else meta.table
-    dims = (int(num_x), int(y.shape[1]), int(meta.params.num_out), int(num_s))
-    sig, scale = table.signature(dims, int(channels), layout) if use_signature else (-1, 1.0)
+    dims, channels = _shape(meta, x, y, s)
+    sig, scale, flip = table.signature(dims, channels, layout) if use_signature else (-1, 1.0, 0)
     cfg = config()
     p = _lib.ConvParams(
         num_nodes=int(x.shape[0]), num_edges=int(y.shape[0]), num_coef=table.num_coef,
         num_x=dims[0], num_y=dims[1], num_out=dims[2], num_scalars=dims[3], channels=int(channels),
         layout=layout.value, val_dtype=val_code, coef_idx_bytes=table.idx_bytes,
-        signature=sig, coef_scale=scale, debug=int(cfg.debug_level),
+        signature=sig, coef_scale=scale, debug=int(cfg.debug_level), y_flip=flip,
         row_order=row_order.data_ptr() if row_order is not None else None)
     return p, table
 
@@ -180,7 +186,9 @@ def _forward_graph(meta: _Meta, sender: torch.Tensor, receiver: torch.Tensor):
 def _raw_forward(meta: _Meta, x, y, s, sender, receiver, graph=None) -> torch.Tensor:
     x, y, s = x.contiguous(), y.contiguous(), s.contiguous()
     other, row_ptr, perm, order = graph if graph is not None else _forward_graph(meta, sender, receiver)
-    p, table = _fill_params(meta, x, y, s, forward=True, row_order=order)
+    # SENDER ordering: the table carries the parity signs of y (unrolled kernels take them as
+    # a sign mask on the unsigned built-in table instead)
+    p, table = _fill_params(meta, x, y, s, meta.signed_table or meta.table, row_order=order)
     if meta.layout == Layout.TRAILING_CHANNELS:
         out = torch.empty((x.shape[0], meta.params.num_out, x.shape[2]), dtype=x.dtype, device=x.device)
     else:
@@ -200,10 +208,14 @@ def _raw_backward(meta: _Meta, x, y, s, dm, sender, receiver, graph=None):
     dx, dy, ds = torch.empty_like(x), torch.empty_like(y), torch.empty_like(s)
     lib = _lib.load()
     deterministic = config().deterministic
-    reuse = graph is not None and not deterministic and meta.ordering != GraphOrdering.SENDER
+    table = meta.table
+    # SENDER ordering: the cotangents belong to the edges as given (dy[e], ds[e] come from
+    # dm[receiver(e)]), not to the reversed edges the forward walks, so the backward keeps the
+    # sender rows but gathers dm and owns dx (`src/e3j/ops/convolution.py:413-431`).
+    reuse = graph is not None and (not deterministic or meta.ordering == GraphOrdering.SENDER)
     if reuse:
         other, row_ptr, perm, order = graph
-        group_receiver = True
+        group_receiver = meta.ordering != GraphOrdering.SENDER
     else:
         sender_l, receiver_l = wrap_global_index(sender, n), wrap_global_index(receiver, n)
         if meta.ordering == GraphOrdering.SENDER:
@@ -218,7 +230,7 @@ def _raw_backward(meta: _Meta, x, y, s, dm, sender, receiver, graph=None):
             perm, other, row_ptr = sort_edges(receiver_l, sender_l, n)
             group_receiver = True
         order = graph[3] if graph is not None else _row_order(other, row_ptr, n)
-    p, table = _fill_params(meta, x, y, s, forward=False, use_signature=group_receiver, row_order=order)
+    p, table = _fill_params(meta, x, y, s, table, use_signature=group_receiver, row_order=order)
     fn = lib.e3j_amd_convolution_bwd_receiver if group_receiver else lib.e3j_amd_convolution_bwd_sender
     with torch.cuda.device(x.device):
         _lib.check(fn(ctypes.byref(p), table.device(x.device).data_ptr(), x.data_ptr(), y.data_ptr(),

@@ -63,6 +63,11 @@ typedef struct e3j_amd_conv_params {
     int32_t signature;      /* id from e3j_amd_find_signature, or -1: table-driven kernel */
     float   coef_scale;     /* unrolled kernels: table = coef_scale * built-in table (1 by default) */
     int32_t debug;
+    /* Unrolled kernels: bit k set = the kernel reads -y[:, k] and returns -dy[:, k].  With the
+     * parity signs of y this runs a symmetric graph's edges in the reversed direction (the
+     * SENDER ordering, src/e3j/ops/convolution.py:166-176) on the unsigned built-in table.
+     * Must be 0 for the table-driven kernels, which take the signs in the table. */
+    uint32_t y_flip;
     /* Optional processing order of the CSR rows (device, num_nodes entries, a permutation of
      * 0..num_nodes-1), e.g. from e3j_amd_locality_order; NULL = natural order.  It only
      * changes which rows run together (cache reuse of gathered rows), never the results. */
@@ -109,13 +114,17 @@ int e3j_amd_convolution_bwd_receiver(const e3j_amd_conv_params *p, const void *c
 /* Match a HOST copy of a packed forward table against the tables of the
  * compile-time-unrolled kernels built into the library, up to one uniform
  * positive factor (the 1/avg_num_neighbors the reference folds into the values,
- * src/e3j/core/convolution.py:135-140), which is returned in *coef_scale.
- * Returns the signature id (>= 0) or -1.  Takes the place of the reference's
+ * src/e3j/core/convolution.py:135-140), which is returned in *coef_scale, and, when
+ * y_flip is not NULL, up to one sign per y component (the parity signs the reference folds
+ * into the table for the SENDER ordering, src/e3j/ops/convolution.py:166-176), returned as
+ * a bit mask for e3j_amd_conv_params.y_flip (tables with more than 32 y components match
+ * only without signs).  Returns the signature id (>= 0) or -1.  Takes the place of the reference's
  * trace-time launch planning (src/e3j/ops/convolution.py:178-208). */
 int e3j_amd_find_signature(const void *coef_host, int32_t coef_idx_bytes, int32_t val_dtype,
                            int32_t num_coef, int32_t num_x, int32_t num_y, int32_t num_out,
                            int32_t num_scalars, int32_t channels, int32_t layout,
-                           float *coef_scale);
+                           float *coef_scale,
+                           uint32_t *y_flip);
 
 /* Tuning aid: selects which launch shape (channels per lane, waves per block, parts) of a
  * signature's kernels later calls use; 0 = default, unknown numbers = default.  The

@@ -33,9 +33,9 @@ def test_every_declared_symbol_is_exported():
 def test_params_struct_matches_header():
     header = open(os.path.join(ROOT, "include", "e3j_amd.h")).read()
     body = re.search(r"typedef struct e3j_amd_conv_params \{(.*?)\} e3j_amd_conv_params;", header, re.S).group(1)
-    fields = re.findall(r"^\s*(const int32_t \*|int32_t|int64_t|float)\s*(\w+);", body, re.M)
+    fields = re.findall(r"^\s*(const int32_t \*|uint32_t|int32_t|int64_t|float)\s*(\w+);", body, re.M)
     assert [name for _, name in fields] == [name for name, _ in _lib.ConvParams._fields_]
-    ctype = {"int32_t": C.c_int32, "int64_t": C.c_int64, "float": C.c_float, "const int32_t *": C.c_void_p}
+    ctype = {"int32_t": C.c_int32, "uint32_t": C.c_uint32, "int64_t": C.c_int64, "float": C.c_float, "const int32_t *": C.c_void_p}
     assert [ctype[t] for t, _ in fields] == [t for _, t in _lib.ConvParams._fields_]
 
 
@@ -91,11 +91,11 @@ def test_find_signature_matches_benchmark_tables():
     assert lib.e3j_amd_num_signatures() >= 10
     module = Convolution(("0e+1o+2e+3o", "0e+1o+2e+3o"), "0e+1o+2e+3o", graph_ordering="RECEIVER")
     packed = module._packed_coef("float32")
-    scale = C.c_float(0)
+    scale, flip = C.c_float(0), C.c_uint32(0)
 
-    def find(buf, channels, idx_bytes=1, layout=1):
+    def find(buf, channels, idx_bytes=1, layout=1, signs=False):
         return lib.e3j_amd_find_signature(buf.ctypes.data, idx_bytes, _lib.F32, buf.shape[0], 16, 16, 99, 23,
-                                          channels, layout, C.byref(scale))
+                                          channels, layout, C.byref(scale), C.byref(flip) if signs else None)
     sig = find(packed, 128)
     assert sig >= 0 and scale.value == 1.0
     assert b"K=128" in lib.e3j_amd_signature_name(sig)
@@ -120,6 +120,18 @@ def test_find_signature_matches_benchmark_tables():
     c2 = Coef4D(c.val.copy(), c.idx, "float32", "uint8")
     c2.val[7] *= 1.001
     assert find(c2.pack(), 128) == -1
+    # the parity signs of y folded into the values (SENDER ordering) come back as a bit mask
+    parity = module.y_parity
+    signed = Coef4D(c.val * parity[c.idx[:, 2].astype(np.int64)], c.idx, "float32", "uint8").pack()
+    assert find(signed, 128) == -1                       # not asked for: no match
+    assert find(signed, 128, signs=True) == sig and scale.value == 1.0
+    assert flip.value == sum(1 << k for k in range(16) if parity[k] < 0) == 0b1111111000001110
+    assert find(packed, 128, signs=True) == sig and flip.value == 0
+    # signs that differ within one y component are no parity pattern
+    c3 = Coef4D(c.val.copy(), c.idx, "float32", "uint8")
+    first_k1 = int(np.flatnonzero(c.idx[:, 2] == 1)[0])
+    c3.val[first_k1] *= -1.0
+    assert find(c3.pack(), 128, signs=True) == -1
 
 
 # --- XLA-FFI handlers -----------------------------------------------------------------

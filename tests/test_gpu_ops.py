@@ -133,25 +133,44 @@ def test_double_backward_matches_autograd_of_dense_form():
         torch.testing.assert_close(u, v, rtol=1e-9, atol=1e-9)
 
 
-def test_sender_ordering_on_symmetric_graph():
+@pytest.mark.parametrize("irreps, l_max, K, layout, unrolled", [
+    ("0e+1o", 2, 16, "TRAILING_CHANNELS", False),           # table-driven kernels, signs in the table
+    ("0e+1o", 2, 32, "TRAILING_CHANNELS", True),            # unrolled kernels, signs as a y mask
+    ("0e+1o+2e+3o", 3, 64, "TRAILING_CHANNELS", True),
+    ("0e+1o+2e+3o", 3, 64, "LEADING_CHANNELS", True),
+])
+def test_sender_ordering_on_symmetric_graph(irreps, l_max, K, layout, unrolled):
     """SENDER ordering = RECEIVER ordering on a symmetric graph with y_ba = p y_ab, s_ba = s_ab
     (tests/test_convolution.py:351-456)."""
     rng = np.random.default_rng(6)
-    N, K = 10, 16
+    N = 10
     pos = rng.normal(size=(N, 3))
     pairs = [(a, b) for a in range(N) for b in range(N) if a != b and np.linalg.norm(pos[a] - pos[b]) < 1.6]
     snd = np.array([a for a, b in pairs], dtype=np.int32)
     rcv = np.array([b for a, b in pairs], dtype=np.int32)
-    module_r = Convolution(("0e+1o", "0e+1o+2e"), "0e+1o+2e", graph_ordering="RECEIVER")
-    module_s = Convolution(("0e+1o", "0e+1o+2e"), "0e+1o+2e", graph_ordering="SENDER")
+    y_irreps = "+".join(f"{l}{'e' if l % 2 == 0 else 'o'}" for l in range(l_max + 1))
+    out_irreps = irreps if l_max == 3 else "0e+1o+2e"
+    module_r = Convolution((irreps, y_irreps), out_irreps, graph_ordering="RECEIVER", layout=layout)
+    module_s = Convolution((irreps, y_irreps), out_irreps, graph_ordering="SENDER", layout=layout)
     vec = torch.from_numpy(pos[snd] - pos[rcv])
-    y = Harmonics(2, normalize=True)(vec).float().numpy()
+    y = Harmonics(l_max, normalize=True)(vec).float().numpy()
     dist = np.linalg.norm(pos[snd] - pos[rcv], axis=-1)
     S = module_r.params.num_scalars
+    X = module_r.source[0].dim
     w = rng.normal(size=(S, K)).astype(np.float32)
     s = (np.cos(dist)[:, None, None] * w[None]).astype(np.float32)        # symmetric in (a, b)
-    x = rng.normal(size=(N, 4, K)).astype(np.float32)
+    x = rng.normal(size=(N, X, K)).astype(np.float32)
     dm = rng.normal(size=(N, module_r.target.dim, K)).astype(np.float32)
+    if layout == "LEADING_CHANNELS":
+        s, x, dm = (np.ascontiguousarray(t.transpose(0, 2, 1)) for t in (s, x, dm))
+    # which kernels serve the signed table of the SENDER ordering
+    from e3j_amd.ops import _Table
+    c = module_s.coef
+    signed = e3j_amd.Coef4D(c.val * module_s.y_parity[c.idx[:, 2].astype(np.int64)], c.idx, "float32",
+                            c.idx_dtype).pack()
+    sig, _, flip = _Table.get(signed, np.float32).signature((X, y.shape[1], module_s.target.dim, S), K,
+                                                            module_s.layout)
+    assert (sig >= 0 and flip != 0) == unrolled
 
     def run(module, order):
         xs, ys, ss = dev(x, grad=True), dev(y[order], grad=True), dev(s[order], grad=True)

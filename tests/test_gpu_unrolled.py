@@ -36,7 +36,8 @@ def _trailing(t, w):
 @pytest.mark.parametrize("name", list(CASES))
 def test_unrolled_matches_oracle(name, layout):
     w = CASES[name]().with_layout(layout)
-    sig, scale = _signature_of(w)
+    sig, scale, flip = _signature_of(w)
+    assert flip == 0
     assert sig >= 0, "benchmark signature must resolve to a built-in unrolled kernel"
     assert scale == 1.0
     d = w.to("cuda")
@@ -66,7 +67,7 @@ def test_scaled_table_uses_unrolled_kernel():
                             avg_num_neighbors=30.0)
     packed = m._packed_coef("float32")
     dims = (int(w.x.shape[1]), int(w.y.shape[1]), m.params.num_out, int(w.s.shape[1]))
-    sig, scale = _Table.get(packed, np.float32).signature(dims, w.channels, m.layout)
+    sig, scale, _ = _Table.get(packed, np.float32).signature(dims, w.channels, m.layout)
     assert sig >= 0 and abs(scale - 1.0 / 30.0) < 1e-8
     d = w.to("cuda")
     out = m(d.x, d.y, d.s, d.sender, d.receiver)
@@ -106,3 +107,56 @@ def test_every_launch_variant_gives_the_same_results(name, layout):
                 assert float((g - g0).abs().max()) <= 2e-5 * scale, f"backward variant {variant} {what}"
     finally:
         lib.e3j_amd_set_launch_variant(0, 0)
+
+
+def test_y_flip_mask_equals_negated_components():
+    """`y_flip` through the C ABI: reading -y[:, k] for the masked components and returning
+    -dy[:, k] is the same as handing the kernels the negated columns."""
+    import ctypes
+    from e3j_amd.graph import csr_row_ptr
+    w = CASES["cfg2"]()
+    d = w.to("cuda")
+    m = w.module
+    table = _Table.get(m._packed_coef("float32"), np.float32)
+    sig, scale, _ = _signature_of(w)
+    mask = 0b1111111000001110                               # the odd-parity components up to l = 3
+    signs = torch.tensor([-1.0 if (mask >> k) & 1 else 1.0 for k in range(16)], device="cuda")
+    ptr = csr_row_ptr(d.receiver, w.num_nodes)
+    lib = _lib.load()
+    stream = int(torch.cuda.current_stream().cuda_stream)
+
+    def run(y, flip):
+        p = _lib.ConvParams(num_nodes=w.num_nodes, num_edges=w.num_edges, num_coef=table.num_coef,
+                            num_x=int(d.x.shape[1]), num_y=16, num_out=m.params.num_out,
+                            num_scalars=int(d.s.shape[1]), channels=w.channels, layout=m.layout.value,
+                            val_dtype=_lib.F32, coef_idx_bytes=table.idx_bytes, signature=sig,
+                            coef_scale=scale, debug=0, y_flip=flip, row_order=None)
+        out = torch.empty_like(d.dm)
+        dx, dy, ds = torch.empty_like(d.x), torch.empty_like(y), torch.empty_like(d.s)
+        coef = table.device(d.x.device)
+        _lib.check(lib.e3j_amd_convolution_fwd(ctypes.byref(p), coef.data_ptr(), d.x.data_ptr(), y.data_ptr(),
+                                               d.s.data_ptr(), d.sender.data_ptr(), ptr.data_ptr(), None,
+                                               out.data_ptr(), stream))
+        _lib.check(lib.e3j_amd_convolution_bwd_receiver(
+            ctypes.byref(p), coef.data_ptr(), d.x.data_ptr(), y.data_ptr(), d.s.data_ptr(), d.dm.data_ptr(),
+            d.sender.data_ptr(), ptr.data_ptr(), None, dx.data_ptr(), dy.data_ptr(), ds.data_ptr(), stream))
+        torch.cuda.synchronize()
+        return out, dx, dy, ds
+
+    flipped = run(d.y, mask)
+    negated = run((d.y * signs).contiguous(), 0)
+    assert torch.equal(flipped[0], negated[0])
+    assert torch.equal(flipped[3], negated[3])
+    torch.testing.assert_close(flipped[1], negated[1], rtol=1e-5, atol=1e-5)
+    torch.testing.assert_close(flipped[2], negated[2] * signs, rtol=1e-5, atol=1e-5)
+    # the table-driven kernels refuse the mask instead of ignoring it
+    p = _lib.ConvParams(num_nodes=w.num_nodes, num_edges=w.num_edges, num_coef=table.num_coef,
+                        num_x=int(d.x.shape[1]), num_y=16, num_out=m.params.num_out,
+                        num_scalars=int(d.s.shape[1]), channels=w.channels, layout=m.layout.value,
+                        val_dtype=_lib.F32, coef_idx_bytes=table.idx_bytes, signature=-1,
+                        coef_scale=1.0, debug=0, y_flip=mask, row_order=None)
+    out = torch.empty_like(d.dm)
+    rc = lib.e3j_amd_convolution_fwd(ctypes.byref(p), table.device(d.x.device).data_ptr(), d.x.data_ptr(),
+                                     d.y.data_ptr(), d.s.data_ptr(), d.sender.data_ptr(), ptr.data_ptr(), None,
+                                     out.data_ptr(), stream)
+    assert rc == _lib.INVALID_ARGUMENT and b"y_flip" in lib.e3j_amd_last_error()
