@@ -62,6 +62,8 @@ def parse_args():
     ap.add_argument("--spatial-sort", action="store_true",
                     help="cfg3 only: number the atoms along a space-filling curve instead of at random "
                          "(a secondary figure; the headline keeps the random numbering)")
+    ap.add_argument("--deterministic", action="store_true",
+                    help="time the atomic-free (bit-reproducible) backward instead of the default one")
     ap.add_argument("--calibrate-copy", action="store_true",
                     help="also run a 1 GiB device copy, the known-size kernel that hardware "
                          "traffic counters are scaled by")
@@ -122,6 +124,18 @@ class AbiCalls:
             ctypes.byref(self.params), self.coef.data_ptr(), w.x.data_ptr(), w.y.data_ptr(),
             w.s.data_ptr(), self.other.data_ptr(), self.ptr.data_ptr(),
             self.perm.data_ptr() if self.perm is not None else None, self.out.data_ptr(),
+            self._stream()))
+
+    def backward_ordered(self):
+        w = self.w
+        if not hasattr(self, "workspace"):
+            nbytes = int(self.lib.e3j_amd_convolution_bwd_ordered_workspace_bytes(ctypes.byref(self.params)))
+            self.workspace = self.torch.empty(nbytes, dtype=self.torch.uint8, device=w.x.device)
+        self._lib.check(self.lib.e3j_amd_convolution_bwd_ordered(
+            ctypes.byref(self.params), self.coef.data_ptr(), w.x.data_ptr(), w.y.data_ptr(),
+            w.s.data_ptr(), w.dm.data_ptr(), self.other.data_ptr(), self.ptr.data_ptr(),
+            self.perm.data_ptr() if self.perm is not None else None,
+            self.dx.data_ptr(), self.dy.data_ptr(), self.ds.data_ptr(), self.workspace.data_ptr(),
             self._stream()))
 
     def backward(self):
@@ -219,6 +233,9 @@ def main():
         del src, dst
 
     abi = AbiCalls(w)
+    if args.deterministic:
+        e3j_amd.config(deterministic=True)
+        abi.backward = abi.backward_ordered
     if args.kernel_only:
         def step():  # noqa: F811
             abi.forward()
@@ -267,7 +284,10 @@ def main():
                                if abi.signature >= 0 else "table-driven kernel"),
         },
         "roofline": {
-            "bound": "hbm", "kernel": "convolution backward (unrolled_bwd_kernel + dx zero fill)",
+            "bound": "hbm",
+            "kernel": ("convolution backward, atomic-free (position sort + unrolled_bwd_kernel + fixed-order "
+                       "dx/dy reductions)" if args.deterministic else
+                       "convolution backward (unrolled_bwd_kernel + dx zero fill)"),
             "achieved": bwd_gbs, "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": bwd_gbs / HBM_PEAK_GBS,
             "traffic": measured.get("backward"),
             "algorithmic_bytes": bytes_["bwd"], "ms": bwd_ms,

@@ -61,6 +61,8 @@ SYMBOLS = {
     "e3j_amd_convolution_fwd": (ctypes.c_int, [_PARAMS] + [_P] * 9),
     "e3j_amd_convolution_bwd_sender": (ctypes.c_int, [_PARAMS] + [_P] * 12),
     "e3j_amd_convolution_bwd_receiver": (ctypes.c_int, [_PARAMS] + [_P] * 12),
+    "e3j_amd_convolution_bwd_ordered_workspace_bytes": (ctypes.c_size_t, [_PARAMS]),
+    "e3j_amd_convolution_bwd_ordered": (ctypes.c_int, [_PARAMS] + [_P] * 13),
     "e3j_amd_find_signature": (ctypes.c_int, [_P] + [ctypes.c_int32] * 9 + [ctypes.POINTER(ctypes.c_float),
                                                                              ctypes.POINTER(ctypes.c_uint32)]),
     "e3j_amd_num_signatures": (ctypes.c_int, []),

@@ -367,19 +367,24 @@ def emit_signature(sig_id: int, name: str, x_irreps: str, y_irreps: str, out_fil
     for cpl, wpb, zs in launch["fwd"]:
         out += [f"template __global__ void unrolled_fwd_kernel<{channels}, {cpl}, {wpb}, {part_names[zs]}>("] + fwd_args
     for cpl, wpb, zs in launch["bwd"]:
-        out += [f"template __global__ void unrolled_bwd_kernel<{channels}, {cpl}, {wpb}, {part_names[zs]}>("] + bwd_args
+        for ordered in ("false", "true"):
+            out += [f"template __global__ void unrolled_bwd_kernel<{channels}, {cpl}, {wpb}, {ordered}, "
+                    f"{part_names[zs]}>("] + bwd_args
     if lead:
         for wpb, zs in lead["fwd"]:
             out += [f"template __global__ void unrolled_fwd_leading_kernel<{channels}, {wpb}, {part_names[zs]}>("] + fwd_args
         for wpb, zs in lead["bwd"]:
-            out += [f"template __global__ void unrolled_bwd_leading_kernel<{channels}, {part_names[zs]}>("] + bwd_args
+            for ordered in ("false", "true"):
+                out += [f"template __global__ void unrolled_bwd_leading_kernel<{channels}, {ordered}, "
+                        f"{part_names[zs]}>("] + bwd_args
 
     fwd_sig = ["(const e3j_amd_conv_params &p, const float *x, const float *y, const float *s,",
                "                   const int32_t *sender, const int32_t *row_ptr, const int32_t *perm,",
                "                   float *out, hipStream_t stream) {"]
     bwd_sig = ["(const e3j_amd_conv_params &p, const float *x, const float *y, const float *s,",
                "                   const float *dm, const int32_t *sender, const int32_t *row_ptr,",
-               "                   const int32_t *perm, float *dx, float *dy, float *ds, hipStream_t stream) {"]
+               "                   const int32_t *perm, float *dx, float *dy, float *ds, hipStream_t stream,",
+               "                   OrderedBwd *ordered) {"]
 
     def switch(variants, call):
         body = ["    switch (VARIANT) {"]
@@ -400,7 +405,7 @@ def emit_signature(sig_id: int, name: str, x_irreps: str, y_irreps: str, out_fil
     out += ["static int run_bwd" + bwd_sig[0]] + bwd_sig[1:]
     out += [ln.replace("VARIANT", "tuning().bwd_variant") for ln in switch(
         launch["bwd"], lambda v: f"launch_unrolled_bwd<{channels}, {v[0]}, {v[1]}, {t.Y}, {t.X}, "
-                                 f"{part_names[v[2]]}>(p, x, y, s, dm, sender, row_ptr, perm, dx, dy, ds, stream);")]
+                                 f"{part_names[v[2]]}>(p, x, y, s, dm, sender, row_ptr, perm, dx, dy, ds, stream, ordered);")]
     out += [f"extern const Signature kSignature_{2 * sig_id} = {{",
             f'    "{desc}",',
             f"    {t.X}, {t.Y}, {t.Z}, {t.S}, {len(t.val)}, {channels}, E3J_AMD_LAYOUT_TRAILING, kVal, kIdx,",
@@ -414,7 +419,7 @@ def emit_signature(sig_id: int, name: str, x_irreps: str, y_irreps: str, out_fil
         out += ["static int run_bwd_leading" + bwd_sig[0]] + bwd_sig[1:]
         out += [ln.replace("VARIANT", "tuning().bwd_variant") for ln in switch(
             lead["bwd"], lambda v: f"launch_unrolled_bwd_leading<{channels}, {t.Y}, {t.X}, "
-                                   f"{part_names[v[1]]}>(p, x, y, s, dm, sender, row_ptr, perm, dx, dy, ds, stream);")]
+                                   f"{part_names[v[1]]}>(p, x, y, s, dm, sender, row_ptr, perm, dx, dy, ds, stream, ordered);")]
         out += [f"extern const Signature kSignature_{2 * sig_id + 1} = {{",
                 f'    "{desc.replace("trailing", "leading")}",',
                 f"    {t.X}, {t.Y}, {t.Z}, {t.S}, {len(t.val)}, {channels}, E3J_AMD_LAYOUT_LEADING, kVal, kIdx,",

@@ -122,7 +122,10 @@ int run_backward(const e3j_amd_conv_params *p, bool group_is_receiver, const voi
                                          static_cast<const float *>(y), static_cast<const float *>(s),
                                          static_cast<const float *>(dm), other, row_ptr, edge_perm,
                                          static_cast<float *>(dx), static_cast<float *>(dy),
-                                         static_cast<float *>(ds), stream);
+                                         static_cast<float *>(ds), stream, nullptr);
+        if (rc == E3J_AMD_OK)
+            rc = launch_zero_padding(*p, other, row_ptr, edge_perm, static_cast<float *>(dy),
+                                     static_cast<float *>(ds), stream);
     } else {
         if ((rc = flip_without_kernel(p, op))) return rc;
         if (coef == nullptr && p->num_coef > 0)
@@ -198,6 +201,83 @@ int e3j_amd_num_signatures(void) { return num_signatures(); }
 const char *e3j_amd_signature_name(int id) {
     if (id < 0 || id >= num_signatures()) return "";
     return signature(id).name;
+}
+
+namespace {
+size_t align256(size_t n) { return (n + 255) / 256 * 256; }
+struct OrderedWorkspace {
+    size_t keys, pos, scratch, ptr, csr, u, slots, total;
+    explicit OrderedWorkspace(const e3j_amd_conv_params &p) {
+        const size_t e = (size_t)p.num_edges, n = (size_t)p.num_nodes;
+        size_t at = 0;
+        auto take = [&](size_t bytes) { const size_t here = at; at += align256(bytes); return here; };
+        keys = take(4 * e);
+        pos = take(4 * e);
+        scratch = take(4 * e);
+        ptr = take(4 * (n + 1));
+        csr = take(e3j_amd_csr_workspace_bytes(p.num_nodes, p.num_edges));
+        u = take(4 * e * (size_t)p.num_x * (size_t)p.channels);
+        slots = take(4 * e * (size_t)kMaxDySlots * (size_t)p.num_y);
+        total = at;
+    }
+};
+}  // namespace
+
+size_t e3j_amd_convolution_bwd_ordered_workspace_bytes(const e3j_amd_conv_params *p) {
+    if (p == nullptr || p->num_nodes < 0 || p->num_edges < 0 || p->num_x < 1 || p->num_y < 1 ||
+        p->channels < 1)
+        return 0;
+    return OrderedWorkspace(*p).total + 256;
+}
+
+int e3j_amd_convolution_bwd_ordered(const e3j_amd_conv_params *p, const void *coef, const void *x,
+                                    const void *y, const void *s, const void *dm,
+                                    const int32_t *sender, const int32_t *receiver_ptr,
+                                    const int32_t *edge_perm, void *dx, void *dy, void *ds,
+                                    void *workspace, void *stream_) {
+    (void)coef;
+    const char *op = "convolution_bwd_ordered";
+    int rc = validate(p, op);
+    if (rc) return rc;
+    hipStream_t stream = static_cast<hipStream_t>(stream_);
+    if (p->num_nodes == 0 && p->num_edges == 0) return E3J_AMD_OK;
+    if (missing(x, p->num_nodes) || missing(dm, p->num_nodes) || missing(dx, p->num_nodes) ||
+        receiver_ptr == nullptr || missing(sender, p->num_edges) || missing(y, p->num_edges) ||
+        missing(s, p->num_edges) || missing(dy, p->num_edges) || missing(ds, p->num_edges) ||
+        workspace == nullptr)
+        return set_error(E3J_AMD_INVALID_ARGUMENT, std::string(op) + ": null operand");
+    if (p->num_nodes == 0) return E3J_AMD_OK;
+    if (!signature_fits(p, {x, s, dm, dx, ds}) || signature(p->signature).bwd == nullptr)
+        return set_error(E3J_AMD_UNIMPLEMENTED,
+                         std::string(op) + ": needs a compile-time-unrolled kernel for the table; "
+                                           "e3j_amd_convolution_bwd_sender is the atomic-free "
+                                           "table-driven backward");
+    char *base = static_cast<char *>(workspace);
+    base += (256 - reinterpret_cast<uintptr_t>(base) % 256) % 256;
+    const OrderedWorkspace w(*p);
+    int32_t *keys = reinterpret_cast<int32_t *>(base + w.keys);
+    int32_t *pos = reinterpret_cast<int32_t *>(base + w.pos);
+    int32_t *scratch = reinterpret_cast<int32_t *>(base + w.scratch);
+    int32_t *sender_ptr = reinterpret_cast<int32_t *>(base + w.ptr);
+    // positions grouped by sender, ascending within a sender (stable sort): the summation order
+    rc = launch_live_keys(sender, receiver_ptr, p->num_nodes, p->num_edges, keys, stream);
+    if (rc) return rc;
+    rc = e3j_amd_sort_edges(keys, keys, p->num_edges, p->num_nodes, pos, scratch, sender_ptr,
+                            base + w.csr, stream);
+    if (rc) return rc;
+    OrderedBwd ordered{reinterpret_cast<float *>(base + w.u), reinterpret_cast<float *>(base + w.slots), 0, 0};
+    rc = signature(p->signature).bwd(*p, static_cast<const float *>(x), static_cast<const float *>(y),
+                                     static_cast<const float *>(s), static_cast<const float *>(dm),
+                                     sender, receiver_ptr, edge_perm, static_cast<float *>(dx),
+                                     static_cast<float *>(dy), static_cast<float *>(ds), stream, &ordered);
+    if (rc == E3J_AMD_OK)
+        rc = reduce_ordered_dx(*p, ordered.u, sender_ptr, pos, ordered.covered, static_cast<float *>(dx), stream);
+    if (rc == E3J_AMD_OK && ordered.slots > 1)
+        rc = reduce_ordered_dy(*p, ordered.dy_slots, ordered.slots, edge_perm, static_cast<float *>(dy), stream);
+    if (rc == E3J_AMD_OK)
+        rc = launch_zero_padding(*p, sender, receiver_ptr, edge_perm, static_cast<float *>(dy),
+                                 static_cast<float *>(ds), stream);
+    return finish(p, stream, rc, op);
 }
 
 int e3j_amd_find_signature(const void *coef_host, int32_t coef_idx_bytes, int32_t val_dtype,

@@ -78,6 +78,27 @@ struct Tuning {
 };
 const Tuning &tuning();
 
+// Atomic-free backward of the unrolled kernels: instead of float atomics, a wave stores the dx
+// contribution of every CSR position as one row of `u` and, when several waves share an
+// edge, its dy sums into slot (position, wave) of `dy_slots`; fixed-order reductions follow
+// (`reduce_ordered_dx`, `reduce_ordered_dy`).  The launcher fills in `slots` and `covered`.
+constexpr int kMaxDySlots = 8;
+struct OrderedBwd {
+    float *u;                 // (num_edges, X * K)
+    float *dy_slots;          // (num_edges, slots, Y)
+    int slots;                // waves per edge of the launched variant (1: dy written directly)
+    unsigned long long covered;  // x coordinates some coefficient touches (bit per coordinate)
+};
+// keys[pos] = other[pos] for the positions the kernels visit (inside a CSR row, endpoint in
+// range), INT32_MAX otherwise (graph.hip).
+int launch_live_keys(const int32_t *other, const int32_t *row_ptr, int32_t num_nodes,
+                     int64_t num_edges, int32_t *keys, hipStream_t stream);
+int reduce_ordered_dx(const e3j_amd_conv_params &p, const float *u, const int32_t *sender_ptr,
+                      const int32_t *sender_pos, unsigned long long covered, float *dx,
+                      hipStream_t stream);
+int reduce_ordered_dy(const e3j_amd_conv_params &p, const float *dy_slots, int slots,
+                      const int32_t *perm, float *dy, hipStream_t stream);
+
 // Compile-time-unrolled kernels (generated, sig_*.hip) ----------------------
 struct Signature {
     const char *name;
@@ -91,7 +112,8 @@ struct Signature {
                float *out, hipStream_t stream);
     int (*bwd)(const e3j_amd_conv_params &p, const float *x, const float *y, const float *s,
                const float *dm, const int32_t *sender, const int32_t *receiver_ptr,
-               const int32_t *edge_perm, float *dx, float *dy, float *ds, hipStream_t stream);
+               const int32_t *edge_perm, float *dx, float *dy, float *ds, hipStream_t stream,
+               OrderedBwd *ordered);  // ordered: nullptr = dx (and shared dy) by float atomics
 };
 int num_signatures();
 const Signature &signature(int id);

@@ -317,7 +317,85 @@ int run_bwd(const e3j_amd_conv_params &p, bool group_is_receiver, const void *co
     return check_hip(hipGetLastError(), "convolution backward launch");
 }
 
+// Atomic-free dx: sum the per-position contribution rows of every sender in ascending
+// position order (a fixed order: the result is bit-reproducible).  One wave per (sender,
+// 256-float piece of the row); x coordinates no coefficient touches read as zero.
+__global__ __launch_bounds__(256) void reduce_ordered_dx_kernel(
+    const float *__restrict__ u, const int32_t *__restrict__ sender_ptr,
+    const int32_t *__restrict__ sender_pos, int num_nodes, int row_floats, int num_x,
+    int channels, int trailing, unsigned long long covered, float *__restrict__ dx) {
+    typedef float f32x4 __attribute__((ext_vector_type(4)));
+    const int pieces = (row_floats + 255) / 256;
+    const int64_t item = (int64_t)blockIdx.x * blockDim.y + threadIdx.y;
+    if (item >= (int64_t)num_nodes * pieces) return;
+    const int n = (int)(item / pieces);
+    const int first = ((int)(item % pieces) * kWave + threadIdx.x) * 4;  // first float of the lane
+    if (first >= row_floats) return;
+    f32x4 acc = {0.f, 0.f, 0.f, 0.f};
+    const int t1 = sender_ptr[n + 1];
+    int t = sender_ptr[n];
+    auto row = [&](int at) {
+        return __builtin_nontemporal_load(
+            reinterpret_cast<const f32x4 *>(u + (int64_t)sender_pos[at] * row_floats + first));
+    };
+    for (; t + 8 <= t1; t += 8) {  // eight rows in flight, added in position order
+        f32x4 v[8];
+#pragma unroll
+        for (int q = 0; q < 8; q++) v[q] = row(t + q);
+#pragma unroll
+        for (int q = 0; q < 8; q++) acc += v[q];
+    }
+    for (; t < t1; t++) acc += row(t);
+#pragma unroll
+    for (int q = 0; q < 4; q++) {
+        // trailing layout (X, K): coordinate = index / K; leading (K, X): coordinate = index % X
+        const int coord = trailing ? (first + q) / channels : (first + q) % num_x;
+        if (!((covered >> coord) & 1ull)) acc[q] = 0.f;
+    }
+    *reinterpret_cast<f32x4 *>(dx + (int64_t)n * row_floats + first) = acc;
+}
+
+// dy of every position from the slots its waves filled, in slot order.
+__global__ void reduce_ordered_dy_kernel(const float *__restrict__ dy_slots, int slots, int num_y,
+                                         int64_t num_edges, const int32_t *__restrict__ perm,
+                                         float *__restrict__ dy) {
+    const int64_t stride = (int64_t)gridDim.x * blockDim.x;
+    for (int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; i < num_edges * num_y; i += stride) {
+        const int64_t pos = i / num_y;
+        const int k = (int)(i % num_y);
+        float total = 0.f;
+        for (int q = 0; q < slots; q++) total += dy_slots[(pos * slots + q) * num_y + k];
+        const int64_t ee = perm ? (int64_t)perm[pos] : pos;
+        dy[ee * num_y + k] = total;
+    }
+}
+
 }  // namespace
+
+int reduce_ordered_dx(const e3j_amd_conv_params &p, const float *u, const int32_t *sender_ptr,
+                      const int32_t *sender_pos, unsigned long long covered, float *dx,
+                      hipStream_t stream) {
+    const int row_floats = p.num_x * p.channels;
+    if (row_floats % 4 != 0 || p.num_x > 64)
+        return set_error(E3J_AMD_INVALID_ARGUMENT, "convolution_bwd_ordered: unsupported row shape");
+    if (p.num_nodes == 0) return E3J_AMD_OK;
+    const int pieces = (row_floats + 255) / 256;
+    const int64_t blocks = ((int64_t)p.num_nodes * pieces + 3) / 4;
+    hipLaunchKernelGGL(reduce_ordered_dx_kernel, dim3((unsigned)blocks), dim3(kWave, 4), 0, stream, u,
+                       sender_ptr, sender_pos, p.num_nodes, row_floats, p.num_x, p.channels,
+                       p.layout == E3J_AMD_LAYOUT_TRAILING ? 1 : 0, covered, dx);
+    return check_hip(hipGetLastError(), "ordered dx reduction launch");
+}
+
+int reduce_ordered_dy(const e3j_amd_conv_params &p, const float *dy_slots, int slots,
+                      const int32_t *perm, float *dy, hipStream_t stream) {
+    if (p.num_edges == 0) return E3J_AMD_OK;
+    const int64_t total = p.num_edges * p.num_y;
+    const unsigned blocks = (unsigned)std::min<int64_t>((total + 255) / 256, 8192);
+    hipLaunchKernelGGL(reduce_ordered_dy_kernel, dim3(blocks), dim3(256), 0, stream, dy_slots, slots,
+                       p.num_y, p.num_edges, perm, dy);
+    return check_hip(hipGetLastError(), "ordered dy reduction launch");
+}
 
 int launch_fill_zero(void *ptr, size_t bytes, hipStream_t stream) {
     if (bytes == 0) return E3J_AMD_OK;

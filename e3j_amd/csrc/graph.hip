@@ -115,7 +115,26 @@ __global__ void wrap_index_kernel(const int32_t *__restrict__ index, int64_t n, 
     }
 }
 
+__global__ void live_keys_kernel(const int32_t *__restrict__ other, const int32_t *__restrict__ row_ptr,
+                                 int32_t num_nodes, int64_t num_edges, int32_t *__restrict__ keys) {
+    const int64_t live_end = row_ptr[num_nodes];
+    const int64_t stride = (int64_t)gridDim.x * blockDim.x;
+    for (int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; i < num_edges; i += stride) {
+        const int32_t v = other[i];
+        keys[i] = (i < live_end && (unsigned)v < (unsigned)num_nodes) ? v : INT32_MAX;
+    }
+}
+
 }  // namespace
+
+int launch_live_keys(const int32_t *other, const int32_t *row_ptr, int32_t num_nodes,
+                     int64_t num_edges, int32_t *keys, hipStream_t stream) {
+    if (num_edges == 0) return E3J_AMD_OK;
+    hipLaunchKernelGGL(live_keys_kernel, dim3(grid_for(num_edges)), dim3(256), 0, stream, other, row_ptr,
+                       num_nodes, num_edges, keys);
+    return check_hip(hipGetLastError(), "live keys launch");
+}
+
 }  // namespace e3j_amd
 
 using namespace e3j_amd;

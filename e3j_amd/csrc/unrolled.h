@@ -379,13 +379,15 @@ struct DsRows {
     }
 };
 
-template <typename Part, int K, int CPL, bool kAtomicDy>
+template <typename Part, int K, int CPL, bool kAtomicDy, bool kOrdered>
 __device__ __forceinline__ void unrolled_bwd_part(
     const float *__restrict__ x, const float *__restrict__ y, const float *__restrict__ s,
     const float *__restrict__ dm, const int32_t *__restrict__ sender,
     const int32_t *__restrict__ row_ptr, const int32_t *__restrict__ perm,
     float *__restrict__ dx, float *__restrict__ dy, float *__restrict__ ds, int num_nodes,
-    float scale, unsigned y_flip, int r, int slice, int lane) {
+    float scale, unsigned y_flip, int dy_slot, int dy_slots, int r, int slice, int lane) {
+    // kOrdered: `dx` is the per-position contribution buffer and, when several waves share an
+    // edge, `dy` the slot buffer (no atomics; fixed-order reductions follow)
     constexpr int NX = Part::NX, NS = Part::NS, NZ = Part::NZ, Y = Part::Y;
     constexpr int X = Part::X, S = Part::S, Z = Part::Z;
     using V = Vec<CPL>;
@@ -443,6 +445,7 @@ __device__ __forceinline__ void unrolled_bwd_part(
         const bool valid = valid_n;
         const int snd = snd_n;
         const int64_t ee = ee_n;
+        const int pos = e;
         e++;
         if (e < e1) fetch(e);
         if (!valid) continue;  // padding edge: its dy/ds rows are zero-filled separately
@@ -455,42 +458,52 @@ __device__ __forceinline__ void unrolled_bwd_part(
         for (int k = Y; k < Red::P; k++) dye[k] = 0.f;
 
         if (active) {
-            float *dxr = dx + (int64_t)snd * (X * K) + c0;
+            if (kOrdered) {
+                float *ur = dx + (int64_t)pos * (X * K) + c0;
 #pragma unroll
-            for (int j = 0; j < NX; j++) {
+                for (int j = 0; j < NX; j++) store_apart_stream<CPL>(ur + Part::kX[j] * K, dxe[j]);
+            } else {
+                float *dxr = dx + (int64_t)snd * (X * K) + c0;
 #pragma unroll
-                for (int t = 0; t < CPL; t++) unsafeAtomicAdd(dxr + Part::kX[j] * K + t * kWave, dxe[j].v[t]);
+                for (int j = 0; j < NX; j++) {
+#pragma unroll
+                    for (int t = 0; t < CPL; t++)
+                        unsafeAtomicAdd(dxr + Part::kX[j] * K + t * kWave, dxe[j].v[t]);
+                }
             }
         }
         const int k = Red::slot(lane);
         const float total = flip_sign(Red::run(dye, lane), y_flip, k);
         if (lane < 16 && k < Y) {
-            if (kAtomicDy) unsafeAtomicAdd(dy + ee * Y + k, total);  // dy zero-filled by the launcher
-            else dy[ee * Y + k] = total;
+            if (!kAtomicDy) dy[ee * Y + k] = total;
+            else if (kOrdered) dy[((int64_t)pos * dy_slots + dy_slot) * Y + k] = total;
+            else unsafeAtomicAdd(dy + ee * Y + k, total);  // dy zero-filled by the launcher
         }
     }
 }
 
-template <int K, int CPL, bool A, int I>
+template <int K, int CPL, bool A, bool O, int I>
 __device__ __forceinline__ void dispatch_bwd(int, const float *, const float *, const float *,
                                              const float *, const int32_t *, const int32_t *,
                                              const int32_t *, float *, float *, float *, int, float,
-                                             unsigned, int, int, int) {}
-template <int K, int CPL, bool A, int I, typename Part, typename... Rest>
+                                             unsigned, int, int, int, int, int) {}
+template <int K, int CPL, bool A, bool O, int I, typename Part, typename... Rest>
 __device__ __forceinline__ void dispatch_bwd(int part, const float *x, const float *y, const float *s,
                                              const float *dm, const int32_t *sender,
                                              const int32_t *row_ptr, const int32_t *perm, float *dx,
-                                             float *dy, float *ds, int num_nodes, float scale, unsigned y_flip, int r,
-                                             int slice, int lane) {
+                                             float *dy, float *ds, int num_nodes, float scale,
+                                             unsigned y_flip, int dy_slot, int dy_slots,
+                                             int r, int slice, int lane) {
     if (part == I)
-        unrolled_bwd_part<Part, K, CPL, A>(x, y, s, dm, sender, row_ptr, perm, dx, dy, ds, num_nodes,
-                                           scale, y_flip, r, slice, lane);
+        unrolled_bwd_part<Part, K, CPL, A, O>(x, y, s, dm, sender, row_ptr, perm, dx, dy, ds, num_nodes,
+                                              scale, y_flip, dy_slot, dy_slots, r, slice, lane);
     else
-        dispatch_bwd<K, CPL, A, I + 1, Rest...>(part, x, y, s, dm, sender, row_ptr, perm, dx, dy, ds,
-                                                num_nodes, scale, y_flip, r, slice, lane);
+        dispatch_bwd<K, CPL, A, O, I + 1, Rest...>(part, x, y, s, dm, sender, row_ptr, perm, dx, dy, ds,
+                                                   num_nodes, scale, y_flip, dy_slot, dy_slots, r, slice,
+                                                   lane);
 }
 
-template <int K, int CPL, int WPB, typename... Parts>
+template <int K, int CPL, int WPB, bool kOrdered, typename... Parts>
 __global__ __launch_bounds__(kWave *WPB)
 void unrolled_bwd_kernel(
     const float *__restrict__ x, const float *__restrict__ y, const float *__restrict__ s,
@@ -507,8 +520,10 @@ void unrolled_bwd_kernel(
     const int slice = uniform((int)((item / NP) % CW));
     const int q = uniform((int)(item / (NP * CW)));
     const int r = row_order ? row_order[q] : q;
-    dispatch_bwd<K, CPL, kAtomicDy, 0, Parts...>(part, x, y, s, dm, sender, row_ptr, perm, dx, dy, ds,
-                                                 num_nodes, scale, y_flip, r, slice, threadIdx.x);
+    dispatch_bwd<K, CPL, kAtomicDy, kOrdered, 0, Parts...>(part, x, y, s, dm, sender, row_ptr, perm, dx,
+                                                           dy, ds, num_nodes, scale, y_flip,
+                                                           part * CW + slice, NP * CW, r, slice,
+                                                           threadIdx.x);
 }
 
 // ---------------------------------------------------------------------------
@@ -750,13 +765,13 @@ struct LeadingBwdGeometry : LeadingGeometry<K, X, S, Z> {
     static constexpr int GC = group();  // channels of dm rows staged at a time
 };
 
-template <typename Part, int K, int NP, unsigned long long kCoveredDx>
+template <typename Part, int K, int NP, unsigned long long kCoveredDx, bool kOrdered>
 __device__ __forceinline__ void unrolled_bwd_leading(
     const float *__restrict__ x, const float *__restrict__ y, const float *__restrict__ s,
     const float *__restrict__ dm, const int32_t *__restrict__ sender,
     const int32_t *__restrict__ row_ptr, const int32_t *__restrict__ perm,
     float *__restrict__ dx, float *__restrict__ dy, float *__restrict__ ds, int num_nodes,
-    float scale, unsigned y_flip, int r, int slice, int lane, int tid, float *region) {
+    float scale, unsigned y_flip, int part, int r, int slice, int lane, int tid, float *region) {
     constexpr int NX = Part::NX, NS = Part::NS, NZ = Part::NZ, Y = Part::Y;
     constexpr int X = Part::X, S = Part::S, Z = Part::Z;
     static_assert(X <= 64 && S <= 64, "part masks hold 64 columns");
@@ -834,6 +849,7 @@ __device__ __forceinline__ void unrolled_bwd_leading(
         const bool valid = valid_n;  // uniform over the block: every wave looks at the same edge
         const int snd = snd_n;
         const int64_t ee = ee_n;
+        const int pos = e;
         e++;
         if (e < e1) fetch(e);
 
@@ -853,12 +869,18 @@ __device__ __forceinline__ void unrolled_bwd_leading(
         LinearBlock<SN, NT> dl;
         dl.template from_strip<S, G::PS>(out_s, tid);
         dl.store(ds + (ee * K + ch0) * S, tid);
-        float *dx_block = dx + ((int64_t)snd * K + ch0) * X;
+        if (kOrdered) {  // the contribution of this position as one row of the buffer, no atomics
+            LinearBlock<XN, NT> ul;
+            ul.template from_strip<X, G::PX>(out_x, tid);
+            ul.store(dx + ((int64_t)pos * K + ch0) * X, tid);
+        } else {
+            float *dx_block = dx + ((int64_t)snd * K + ch0) * X;
 #pragma unroll
-        for (int i = 0; i < (XN + NT - 1) / NT; i++) {
-            const int g = i * NT + tid;
-            const bool mine = kAllDx ? (XN % NT == 0 || g < XN) : (((covered >> i) & 1u) != 0);
-            if (mine) unsafeAtomicAdd(dx_block + g, out_x[strip_index<X, G::PX>(g)]);
+            for (int i = 0; i < (XN + NT - 1) / NT; i++) {
+                const int g = i * NT + tid;
+                const bool mine = kAllDx ? (XN % NT == 0 || g < XN) : (((covered >> i) & 1u) != 0);
+                if (mine) unsafeAtomicAdd(dx_block + g, out_x[strip_index<X, G::PX>(g)]);
+            }
         }
 
 #pragma unroll
@@ -866,31 +888,35 @@ __device__ __forceinline__ void unrolled_bwd_leading(
         const int k = Red::slot(lane);
         const float total = flip_sign(Red::run(dye, lane), y_flip, k);
         if (lane < 16 && k < Y) {
-            if (NP > 1 || G::COUNT > 1) unsafeAtomicAdd(dy + ee * Y + k, total);  // dy zero-filled by the launcher
-            else dy[ee * Y + k] = total;
+            constexpr int SLOTS = NP * G::COUNT;
+            if (SLOTS == 1) dy[ee * Y + k] = total;
+            else if (kOrdered) dy[((int64_t)pos * SLOTS + part * G::COUNT + slice) * Y + k] = total;
+            else unsafeAtomicAdd(dy + ee * Y + k, total);  // dy zero-filled by the launcher
         }
     }
 }
 
-template <int K, int NP, unsigned long long kCoveredDx, int I>
+template <int K, int NP, unsigned long long kCoveredDx, bool O, int I>
 __device__ __forceinline__ void dispatch_bwd_leading(int, const float *, const float *, const float *,
                                                      const float *, const int32_t *, const int32_t *,
                                                      const int32_t *, float *, float *, float *, int,
                                                      float, unsigned, int, int, int, int, float *) {}
-template <int K, int NP, unsigned long long kCoveredDx, int I, typename Part, typename... Rest>
+template <int K, int NP, unsigned long long kCoveredDx, bool O, int I, typename Part, typename... Rest>
 __device__ __forceinline__ void dispatch_bwd_leading(int part, const float *x, const float *y,
                                                      const float *s, const float *dm,
                                                      const int32_t *sender, const int32_t *row_ptr,
                                                      const int32_t *perm, float *dx, float *dy,
-                                                     float *ds, int num_nodes, float scale, unsigned y_flip, int r,
-                                                     int slice, int lane, int tid, float *region) {
+                                                     float *ds, int num_nodes, float scale,
+                                                     unsigned y_flip, int r, int slice, int lane,
+                                                     int tid, float *region) {
     if (part == I)
-        unrolled_bwd_leading<Part, K, NP, kCoveredDx>(x, y, s, dm, sender, row_ptr, perm, dx, dy, ds,
-                                                      num_nodes, scale, y_flip, r, slice, lane, tid, region);
+        unrolled_bwd_leading<Part, K, NP, kCoveredDx, O>(x, y, s, dm, sender, row_ptr, perm, dx, dy, ds,
+                                                         num_nodes, scale, y_flip, part, r, slice, lane,
+                                                         tid, region);
     else
-        dispatch_bwd_leading<K, NP, kCoveredDx, I + 1, Rest...>(part, x, y, s, dm, sender, row_ptr, perm,
-                                                                dx, dy, ds, num_nodes, scale, y_flip, r, slice,
-                                                                lane, tid, region);
+        dispatch_bwd_leading<K, NP, kCoveredDx, O, I + 1, Rest...>(part, x, y, s, dm, sender, row_ptr,
+                                                                   perm, dx, dy, ds, num_nodes, scale,
+                                                                   y_flip, r, slice, lane, tid, region);
 }
 
 template <typename First, typename...>
@@ -898,8 +924,12 @@ struct FirstOf {
     using type = First;
 };
 
-template <int K, typename... Parts>
-__global__ __launch_bounds__(kWave * sizeof...(Parts)) void unrolled_bwd_leading_kernel(
+// The second launch bound asks for three resident waves per SIMD when the signature is split
+// in three or more parts (at most 168 vector registers): a few registers above that line cost
+// a third of the occupancy and 35 % of the run time.
+template <int K, bool kOrdered, typename... Parts>
+__global__ __launch_bounds__(kWave * sizeof...(Parts), sizeof...(Parts) >= 3 ? 3 : sizeof...(Parts))
+void unrolled_bwd_leading_kernel(
     const float *__restrict__ x, const float *__restrict__ y, const float *__restrict__ s,
     const float *__restrict__ dm, const int32_t *__restrict__ sender,
     const int32_t *__restrict__ row_ptr, const int32_t *__restrict__ perm,
@@ -916,7 +946,7 @@ __global__ __launch_bounds__(kWave * sizeof...(Parts)) void unrolled_bwd_leading
     const int q = (int)(item / G::COUNT);
     const int r = row_order ? row_order[q] : q;
     const int part = uniform((int)threadIdx.y);
-    dispatch_bwd_leading<K, NP, kCoveredDx, 0, Parts...>(
+    dispatch_bwd_leading<K, NP, kCoveredDx, kOrdered, 0, Parts...>(
         part, x, y, s, dm, sender, row_ptr, perm, dx, dy, ds, num_nodes, scale, y_flip, r, slice,
         threadIdx.x, threadIdx.y * kWave + threadIdx.x, region);
 }
@@ -934,27 +964,45 @@ int launch_unrolled_fwd(const e3j_amd_conv_params &p, const float *x, const floa
     return check_hip(hipGetLastError(), "convolution forward launch");
 }
 
+// Where the backward kernels put dx and dy: float atomics into zero-filled results, or (ordered)
+// the per-position buffers behind `ordered`, which is then told what the variant produced.
+template <int X, int Y, int SLOTS, unsigned long long COVERED>
+int prepare_bwd_targets(const e3j_amd_conv_params &p, OrderedBwd *ordered, int K, float *&dx, float *&dy,
+                        hipStream_t stream) {
+    static_assert(SLOTS <= kMaxDySlots, "more waves per edge than dy slots");
+    if (ordered != nullptr) {
+        ordered->slots = SLOTS;
+        ordered->covered = COVERED;
+        dx = ordered->u;
+        if (SLOTS > 1) dy = ordered->dy_slots;
+        return E3J_AMD_OK;
+    }
+    int rc = launch_fill_zero(dx, sizeof(float) * (size_t)p.num_nodes * X * K, stream);
+    if (rc == E3J_AMD_OK && SLOTS > 1) rc = launch_fill_zero(dy, sizeof(float) * (size_t)p.num_edges * Y, stream);
+    return rc;
+}
+
 template <int K, int CPL, int WPB, int Y, int X, typename... Parts>
 int launch_unrolled_bwd(const e3j_amd_conv_params &p, const float *x, const float *y, const float *s,
                         const float *dm, const int32_t *sender, const int32_t *row_ptr,
-                        const int32_t *perm, float *dx, float *dy, float *ds, hipStream_t stream) {
+                        const int32_t *perm, float *dx, float *dy, float *ds, hipStream_t stream,
+                        OrderedBwd *ordered) {
     constexpr int64_t PER_NODE = (int64_t)Slice<K, CPL>::COUNT * sizeof...(Parts);
-    int rc = launch_fill_zero(dx, sizeof(float) * (size_t)p.num_nodes * X * K, stream);
-    if (rc) return rc;
-    if (PER_NODE > 1) {
-        rc = launch_fill_zero(dy, sizeof(float) * (size_t)p.num_edges * Y, stream);
-        if (rc) return rc;
-    }
-    rc = launch_zero_padding(p, sender, row_ptr, perm, dy, ds, stream);
+    constexpr unsigned long long kCovered = (Parts::kDxMask | ...);
+    int rc = prepare_bwd_targets<X, Y, (int)PER_NODE, kCovered>(p, ordered, K, dx, dy, stream);
     if (rc) return rc;
     const int64_t blocks = padded_grid(((int64_t)p.num_nodes * PER_NODE + WPB - 1) / WPB);
     if (blocks > 0x7fffffffLL) return set_error(E3J_AMD_INVALID_ARGUMENT, "convolution_bwd: grid too large");
-    hipLaunchKernelGGL((unrolled_bwd_kernel<K, CPL, WPB, Parts...>), dim3((unsigned)blocks),
-                       dim3(kWave, WPB), 0, stream, x, y, s, dm, sender, row_ptr, perm, p.row_order,
-                       dx, dy, ds, p.num_nodes, p.coef_scale, p.y_flip);
+    if (ordered != nullptr)
+        hipLaunchKernelGGL((unrolled_bwd_kernel<K, CPL, WPB, true, Parts...>), dim3((unsigned)blocks),
+                           dim3(kWave, WPB), 0, stream, x, y, s, dm, sender, row_ptr, perm, p.row_order,
+                           dx, dy, ds, p.num_nodes, p.coef_scale, p.y_flip);
+    else
+        hipLaunchKernelGGL((unrolled_bwd_kernel<K, CPL, WPB, false, Parts...>), dim3((unsigned)blocks),
+                           dim3(kWave, WPB), 0, stream, x, y, s, dm, sender, row_ptr, perm, p.row_order,
+                           dx, dy, ds, p.num_nodes, p.coef_scale, p.y_flip);
     return check_hip(hipGetLastError(), "convolution backward launch");
 }
-
 
 template <int K, int WPB, typename Part>
 int launch_unrolled_fwd_leading(const e3j_amd_conv_params &p, const float *x, const float *y,
@@ -973,23 +1021,23 @@ template <int K, int Y, int X, typename... Parts>
 int launch_unrolled_bwd_leading(const e3j_amd_conv_params &p, const float *x, const float *y,
                                 const float *s, const float *dm, const int32_t *sender,
                                 const int32_t *row_ptr, const int32_t *perm, float *dx, float *dy,
-                                float *ds, hipStream_t stream) {
+                                float *ds, hipStream_t stream, OrderedBwd *ordered) {
     using P0 = typename FirstOf<Parts...>::type;
     constexpr int NP = sizeof...(Parts);
     using G = LeadingBwdGeometry<K, P0::X, P0::S, P0::Z, NP>;
-    int rc = launch_fill_zero(dx, sizeof(float) * (size_t)p.num_nodes * X * K, stream);
-    if (rc) return rc;
-    if (G::COUNT * NP > 1) {
-        rc = launch_fill_zero(dy, sizeof(float) * (size_t)p.num_edges * Y, stream);
-        if (rc) return rc;
-    }
-    rc = launch_zero_padding(p, sender, row_ptr, perm, dy, ds, stream);
+    constexpr unsigned long long kCovered = (Parts::kDxMask | ...);
+    int rc = prepare_bwd_targets<X, Y, G::COUNT * NP, kCovered>(p, ordered, K, dx, dy, stream);
     if (rc) return rc;
     const int64_t blocks = padded_grid((int64_t)p.num_nodes * G::COUNT);
     if (blocks > 0x7fffffffLL) return set_error(E3J_AMD_INVALID_ARGUMENT, "convolution_bwd: grid too large");
-    hipLaunchKernelGGL((unrolled_bwd_leading_kernel<K, Parts...>), dim3((unsigned)blocks),
-                       dim3(kWave, NP), 0, stream, x, y, s, dm, sender, row_ptr, perm, p.row_order,
-                       dx, dy, ds, p.num_nodes, p.coef_scale, p.y_flip);
+    if (ordered != nullptr)
+        hipLaunchKernelGGL((unrolled_bwd_leading_kernel<K, true, Parts...>), dim3((unsigned)blocks),
+                           dim3(kWave, NP), 0, stream, x, y, s, dm, sender, row_ptr, perm, p.row_order,
+                           dx, dy, ds, p.num_nodes, p.coef_scale, p.y_flip);
+    else
+        hipLaunchKernelGGL((unrolled_bwd_leading_kernel<K, false, Parts...>), dim3((unsigned)blocks),
+                           dim3(kWave, NP), 0, stream, x, y, s, dm, sender, row_ptr, perm, p.row_order,
+                           dx, dy, ds, p.num_nodes, p.coef_scale, p.y_flip);
     return check_hip(hipGetLastError(), "convolution backward launch");
 }
 

@@ -209,19 +209,25 @@ def _raw_backward(meta: _Meta, x, y, s, dm, sender, receiver, graph=None):
     lib = _lib.load()
     deterministic = config().deterministic
     table = meta.table
+    sender_rows = meta.ordering == GraphOrdering.SENDER
+    # deterministic: the atomic-free backward of the unrolled kernels on the forward's own rows
+    # (per-position dx rows summed in a fixed order); tables without such a kernel fall back
+    # to the table-driven kernel on sender rows, which owns dx
+    ordered = (deterministic and not sender_rows
+               and table.signature(*_shape(meta, x, y, s), meta.layout)[0] >= 0)
     # SENDER ordering: the cotangents belong to the edges as given (dy[e], ds[e] come from
     # dm[receiver(e)]), not to the reversed edges the forward walks, so the backward keeps the
     # sender rows but gathers dm and owns dx (`src/e3j/ops/convolution.py:413-431`).
-    reuse = graph is not None and (not deterministic or meta.ordering == GraphOrdering.SENDER)
+    reuse = graph is not None and (not deterministic or ordered or sender_rows)
     if reuse:
         other, row_ptr, perm, order = graph
-        group_receiver = meta.ordering != GraphOrdering.SENDER
+        group_receiver = not sender_rows
     else:
         sender_l, receiver_l = wrap_global_index(sender, n), wrap_global_index(receiver, n)
-        if meta.ordering == GraphOrdering.SENDER:
+        if sender_rows:
             # already grouped by sender: rows own their dx, no permutation
             group_receiver, other, row_ptr, perm = False, receiver_l.contiguous(), csr_row_ptr(sender_l, n), None
-        elif deterministic:
+        elif deterministic and not ordered:
             perm, other, row_ptr = sort_edges(sender_l, receiver_l, n)
             group_receiver = False
         elif meta.ordering == GraphOrdering.RECEIVER:
@@ -231,12 +237,18 @@ def _raw_backward(meta: _Meta, x, y, s, dm, sender, receiver, graph=None):
             group_receiver = True
         order = graph[3] if graph is not None else _row_order(other, row_ptr, n)
     p, table = _fill_params(meta, x, y, s, table, use_signature=group_receiver, row_order=order)
-    fn = lib.e3j_amd_convolution_bwd_receiver if group_receiver else lib.e3j_amd_convolution_bwd_sender
+    args = (ctypes.byref(p), table.device(x.device).data_ptr(), x.data_ptr(), y.data_ptr(),
+            s.data_ptr(), dm.data_ptr(), other.data_ptr(), row_ptr.data_ptr(),
+            perm.data_ptr() if perm is not None else None,
+            dx.data_ptr(), dy.data_ptr(), ds.data_ptr())
     with torch.cuda.device(x.device):
-        _lib.check(fn(ctypes.byref(p), table.device(x.device).data_ptr(), x.data_ptr(), y.data_ptr(),
-                      s.data_ptr(), dm.data_ptr(), other.data_ptr(), row_ptr.data_ptr(),
-                      perm.data_ptr() if perm is not None else None,
-                      dx.data_ptr(), dy.data_ptr(), ds.data_ptr(), _stream(x.device)))
+        if ordered:
+            nbytes = int(lib.e3j_amd_convolution_bwd_ordered_workspace_bytes(ctypes.byref(p)))
+            workspace = torch.empty(nbytes, dtype=torch.uint8, device=x.device)
+            _lib.check(lib.e3j_amd_convolution_bwd_ordered(*args, workspace.data_ptr(), _stream(x.device)))
+        else:
+            fn = lib.e3j_amd_convolution_bwd_receiver if group_receiver else lib.e3j_amd_convolution_bwd_sender
+            _lib.check(fn(*args, _stream(x.device)))
     return dx, dy, ds
 
 

@@ -111,6 +111,22 @@ int e3j_amd_convolution_bwd_receiver(const e3j_amd_conv_params *p, const void *c
                                      const int32_t *edge_perm,
                                      void *dx, void *dy, void *ds, void *stream);
 
+/* The same backward on the forward's receiver CSR without any atomic: every wave stores the dx
+ * contribution of its CSR positions into a buffer, which is then summed per sender in ascending
+ * position order, and dy sums of waves that share an edge are combined in a fixed order.
+ * Bit-reproducible from run to run like the reference's backward
+ * (tests/test_ops/test_convolution_op.py:329-342), at the price of one more pass over
+ * E * num_x * channels floats.  Needs a compile-time-unrolled kernel (p->signature >= 0),
+ * else E3J_AMD_UNIMPLEMENTED.  workspace: device memory, at least
+ * e3j_amd_convolution_bwd_ordered_workspace_bytes(p) bytes (about E * (num_x * channels + 8 * num_y)
+ * floats); contents on entry and exit are irrelevant. */
+size_t e3j_amd_convolution_bwd_ordered_workspace_bytes(const e3j_amd_conv_params *p);
+int e3j_amd_convolution_bwd_ordered(const e3j_amd_conv_params *p, const void *coef, const void *x,
+                                    const void *y, const void *s, const void *dm,
+                                    const int32_t *sender, const int32_t *receiver_ptr,
+                                    const int32_t *edge_perm, void *dx, void *dy, void *ds,
+                                    void *workspace, void *stream);
+
 /* Match a HOST copy of a packed forward table against the tables of the
  * compile-time-unrolled kernels built into the library, up to one uniform
  * positive factor (the 1/avg_num_neighbors the reference folds into the values,

@@ -160,3 +160,70 @@ def test_y_flip_mask_equals_negated_components():
                                      d.y.data_ptr(), d.s.data_ptr(), d.sender.data_ptr(), ptr.data_ptr(), None,
                                      out.data_ptr(), stream)
     assert rc == _lib.INVALID_ARGUMENT and b"y_flip" in lib.e3j_amd_last_error()
+
+
+@pytest.mark.parametrize("layout", ["TRAILING_CHANNELS", "LEADING_CHANNELS"])
+@pytest.mark.parametrize("name", ["cfg1", "cfg2", "cfg3"])
+def test_deterministic_backward_is_bit_reproducible_and_matches(name, layout):
+    """`config(deterministic=True)`: the atomic-free backward of the unrolled kernels (dx rows per
+    position summed in a fixed order).  Bit-identical over repeats like the reference's backward
+    (`tests/test_ops/test_convolution_op.py:329-342`), same values as the oracle, and independent
+    of the launch variant's wave count per edge only through float32 rounding."""
+    w = CASES[name]().with_layout(layout)
+    d = w.to("cuda")
+    m = w.module
+    coef = m._packed_coef("float32")
+    # some padding edges inside the list and an unsorted variant below
+    snd = d.sender.clone()
+    snd[::17] = e3j_amd.DUMMY_INDEX
+    lib = _lib.load()
+
+    def run():
+        g = e3j_amd.convolution_bwd(coef, d.x, d.y, d.s, snd, d.receiver, d.dm, m.params, m.graph_ordering,
+                                    layout=m.layout)
+        torch.cuda.synchronize()
+        return g
+
+    with e3j_amd.config.use(deterministic=True):
+        base = run()
+        for _ in range(4):
+            for a, b in zip(base, run()):
+                assert torch.equal(a, b)
+        try:  # another launch shape: other waves per edge, same sums up to rounding
+            lib.e3j_amd_set_launch_variant(0, 2)
+            other = run()
+        finally:
+            lib.e3j_amd_set_launch_variant(0, 0)
+    atomic = run()
+    for a, b, c, what in zip(base, atomic, other, ("dx", "dy", "ds")):
+        scale = float(a.abs().max())
+        assert float((a - b).abs().max()) <= 2e-5 * scale, what
+        assert float((a - c).abs().max()) <= 2e-5 * scale, what
+    idx, val, mix = w.table()
+    a = w.numpy()
+    a["sender"] = snd.cpu().numpy()
+    (rx, ry, rs), (mx, my, ms) = H.backward_reference(idx, val, mix, a["x"], a["y"], a["s"], a["sender"],
+                                                      a["receiver"], a["dm"])
+    H.assert_parity(_trailing(base[0], w), rx, mx, f"{name} dx")
+    H.assert_parity(base[1].cpu().numpy(), ry, my, f"{name} dy")
+    H.assert_parity(_trailing(base[2], w), rs, ms, f"{name} ds")
+    assert not base[1][::17].any() and not base[2][::17].any()     # padding edges: exact zeros
+
+
+def test_deterministic_backward_on_unsorted_edges():
+    """`GraphOrdering.NONE`: positions are sorted on the device first; the ordered backward then
+    runs on the sorted positions and writes dy/ds through the permutation."""
+    w = CASES["cfg2"]()
+    d = w.to("cuda")
+    m = w.module
+    coef = m._packed_coef("float32")
+    shuffle = torch.randperm(w.num_edges, generator=torch.Generator().manual_seed(3)).cuda()
+    y, s, snd, rcv = d.y[shuffle].contiguous(), d.s[shuffle].contiguous(), d.sender[shuffle], d.receiver[shuffle]
+    with e3j_amd.config.use(deterministic=True):
+        got = e3j_amd.convolution_bwd(coef, d.x, y, s, snd, rcv, d.dm, m.params, "NONE")
+        again = e3j_amd.convolution_bwd(coef, d.x, y, s, snd, rcv, d.dm, m.params, "NONE")
+        want = e3j_amd.convolution_bwd(coef, d.x, d.y, d.s, d.sender, d.receiver, d.dm, m.params, "RECEIVER")
+    for a, b in zip(got, again):
+        assert torch.equal(a, b)
+    assert torch.equal(got[0], want[0])                      # same positions after the stable sort
+    assert torch.equal(got[1], want[1][shuffle]) and torch.equal(got[2], want[2][shuffle])
