@@ -44,8 +44,8 @@ BUILTIN_SIGNATURES = [
     ("l3_l3_to_l3_k128", "0e+1o+2e+3o", "0e+1o+2e+3o", "0e+1o+2e+3o", 128),
 ]
 
-#: launch shapes per channel count: (channels per lane, waves per block, parts) variants for
-#: fwd and bwd.  `parts` splits the paths of the signature over that many waves.  Variant 0
+#: launch shapes per channel count: (channels per lane, waves per block, parts[, resident
+#: waves per SIMD the register allocation must allow]) variants for fwd and bwd.  `parts` splits the paths of the signature over that many waves.  Variant 0
 #: is the default; the others are selected with the environment variables
 #: E3J_AMD_FWD_VARIANT / E3J_AMD_BWD_VARIANT (read once) for tuning runs.
 LAUNCH = {
@@ -364,11 +364,14 @@ def emit_signature(sig_id: int, name: str, x_irreps: str, y_irreps: str, out_fil
                 "    const int32_t *, const int32_t *, const int32_t *, float *, float *, float *, int, float,",
                 "    unsigned);"]
     out += ["}  // namespace", "", "// both passes: the device pass needs the kernels instantiated"]
-    for cpl, wpb, zs in launch["fwd"]:
-        out += [f"template __global__ void unrolled_fwd_kernel<{channels}, {cpl}, {wpb}, {part_names[zs]}>("] + fwd_args
-    for cpl, wpb, zs in launch["bwd"]:
+    for v in launch["fwd"]:
+        cpl, wpb, zs, minw = (*v, 1)[:4]
+        out += [f"template __global__ void unrolled_fwd_kernel<{channels}, {cpl}, {wpb}, {minw}, "
+                f"{part_names[zs]}>("] + fwd_args
+    for v in launch["bwd"]:
+        cpl, wpb, zs, minw = (*v, 1)[:4]
         for ordered in ("false", "true"):
-            out += [f"template __global__ void unrolled_bwd_kernel<{channels}, {cpl}, {wpb}, {ordered}, "
+            out += [f"template __global__ void unrolled_bwd_kernel<{channels}, {cpl}, {wpb}, {minw}, {ordered}, "
                     f"{part_names[zs]}>("] + bwd_args
     if lead:
         for wpb, zs in lead["fwd"]:
@@ -400,11 +403,11 @@ def emit_signature(sig_id: int, name: str, x_irreps: str, y_irreps: str, out_fil
             ""]
     out += ["static int run_fwd" + fwd_sig[0]] + fwd_sig[1:]
     out += [ln.replace("VARIANT", "tuning().fwd_variant") for ln in switch(
-        launch["fwd"], lambda v: f"launch_unrolled_fwd<{channels}, {v[0]}, {v[1]}, {part_names[v[2]]}>("
+        launch["fwd"], lambda v: f"launch_unrolled_fwd<{channels}, {v[0]}, {v[1]}, {(*v, 1)[3]}, {part_names[v[2]]}>("
                                  "p, x, y, s, sender, row_ptr, perm, out, stream);")]
     out += ["static int run_bwd" + bwd_sig[0]] + bwd_sig[1:]
     out += [ln.replace("VARIANT", "tuning().bwd_variant") for ln in switch(
-        launch["bwd"], lambda v: f"launch_unrolled_bwd<{channels}, {v[0]}, {v[1]}, {t.Y}, {t.X}, "
+        launch["bwd"], lambda v: f"launch_unrolled_bwd<{channels}, {v[0]}, {v[1]}, {(*v, 1)[3]}, {t.Y}, {t.X}, "
                                  f"{part_names[v[2]]}>(p, x, y, s, dm, sender, row_ptr, perm, dx, dy, ds, stream, ordered);")]
     out += [f"extern const Signature kSignature_{2 * sig_id} = {{",
             f'    "{desc}",',

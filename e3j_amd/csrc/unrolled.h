@@ -345,8 +345,9 @@ __device__ __forceinline__ void dispatch_fwd(int part, const float *x, const flo
 }
 
 // One wave per (receiver, channel slice, part); consecutive waves share a receiver.
-template <int K, int CPL, int WPB, typename... Parts>
-__global__ __launch_bounds__(kWave *WPB) void unrolled_fwd_kernel(
+// MINW: resident waves per SIMD the register allocation must leave room for (1 = no demand).
+template <int K, int CPL, int WPB, int MINW, typename... Parts>
+__global__ __launch_bounds__(kWave *WPB, MINW) void unrolled_fwd_kernel(
     const float *__restrict__ x, const float *__restrict__ y, const float *__restrict__ s,
     const int32_t *__restrict__ sender, const int32_t *__restrict__ row_ptr,
     const int32_t *__restrict__ perm, const int32_t *__restrict__ row_order,
@@ -503,8 +504,8 @@ __device__ __forceinline__ void dispatch_bwd(int part, const float *x, const flo
                                                    lane);
 }
 
-template <int K, int CPL, int WPB, bool kOrdered, typename... Parts>
-__global__ __launch_bounds__(kWave *WPB)
+template <int K, int CPL, int WPB, int MINW, bool kOrdered, typename... Parts>
+__global__ __launch_bounds__(kWave *WPB, MINW)
 void unrolled_bwd_kernel(
     const float *__restrict__ x, const float *__restrict__ y, const float *__restrict__ s,
     const float *__restrict__ dm, const int32_t *__restrict__ sender,
@@ -951,14 +952,14 @@ void unrolled_bwd_leading_kernel(
         threadIdx.x, threadIdx.y * kWave + threadIdx.x, region);
 }
 
-template <int K, int CPL, int WPB, typename... Parts>
+template <int K, int CPL, int WPB, int MINW, typename... Parts>
 int launch_unrolled_fwd(const e3j_amd_conv_params &p, const float *x, const float *y, const float *s,
                         const int32_t *sender, const int32_t *row_ptr, const int32_t *perm,
                         float *out, hipStream_t stream) {
     constexpr int64_t PER_NODE = (int64_t)Slice<K, CPL>::COUNT * sizeof...(Parts);
     const int64_t blocks = padded_grid(((int64_t)p.num_nodes * PER_NODE + WPB - 1) / WPB);
     if (blocks > 0x7fffffffLL) return set_error(E3J_AMD_INVALID_ARGUMENT, "convolution: grid too large");
-    hipLaunchKernelGGL((unrolled_fwd_kernel<K, CPL, WPB, Parts...>), dim3((unsigned)blocks),
+    hipLaunchKernelGGL((unrolled_fwd_kernel<K, CPL, WPB, MINW, Parts...>), dim3((unsigned)blocks),
                        dim3(kWave, WPB), 0, stream, x, y, s, sender, row_ptr, perm, p.row_order, out,
                        p.num_nodes, p.coef_scale, p.y_flip);
     return check_hip(hipGetLastError(), "convolution forward launch");
@@ -982,7 +983,7 @@ int prepare_bwd_targets(const e3j_amd_conv_params &p, OrderedBwd *ordered, int K
     return rc;
 }
 
-template <int K, int CPL, int WPB, int Y, int X, typename... Parts>
+template <int K, int CPL, int WPB, int MINW, int Y, int X, typename... Parts>
 int launch_unrolled_bwd(const e3j_amd_conv_params &p, const float *x, const float *y, const float *s,
                         const float *dm, const int32_t *sender, const int32_t *row_ptr,
                         const int32_t *perm, float *dx, float *dy, float *ds, hipStream_t stream,
@@ -994,11 +995,11 @@ int launch_unrolled_bwd(const e3j_amd_conv_params &p, const float *x, const floa
     const int64_t blocks = padded_grid(((int64_t)p.num_nodes * PER_NODE + WPB - 1) / WPB);
     if (blocks > 0x7fffffffLL) return set_error(E3J_AMD_INVALID_ARGUMENT, "convolution_bwd: grid too large");
     if (ordered != nullptr)
-        hipLaunchKernelGGL((unrolled_bwd_kernel<K, CPL, WPB, true, Parts...>), dim3((unsigned)blocks),
+        hipLaunchKernelGGL((unrolled_bwd_kernel<K, CPL, WPB, MINW, true, Parts...>), dim3((unsigned)blocks),
                            dim3(kWave, WPB), 0, stream, x, y, s, dm, sender, row_ptr, perm, p.row_order,
                            dx, dy, ds, p.num_nodes, p.coef_scale, p.y_flip);
     else
-        hipLaunchKernelGGL((unrolled_bwd_kernel<K, CPL, WPB, false, Parts...>), dim3((unsigned)blocks),
+        hipLaunchKernelGGL((unrolled_bwd_kernel<K, CPL, WPB, MINW, false, Parts...>), dim3((unsigned)blocks),
                            dim3(kWave, WPB), 0, stream, x, y, s, dm, sender, row_ptr, perm, p.row_order,
                            dx, dy, ds, p.num_nodes, p.coef_scale, p.y_flip);
     return check_hip(hipGetLastError(), "convolution backward launch");
