@@ -39,10 +39,10 @@ HBM_PEAK_GBS = 8000.0
 #: scaled by what the same counter reads for a 1 GiB device copy (`--calibrate-copy`: 2.0 for
 #: FETCH_SIZE, 1.0 for WRITE_SIZE).  Only quoted for the workloads they were measured on.
 MEASURED_TRAFFIC_BYTES = {
-    ("cfg3", 1.0, "trailing"): {"backward": 2.0 * 7.453e6 * 1024 + 18.96e6 * 1024,
-                                "forward": 2.0 * 6.264e6 * 1024 + 1.584e6 * 1024},
-    ("cfg3", 1.0, "leading"): {"backward": 2.0 * 7.404e6 * 1024 + 19.08e6 * 1024,
-                               "forward": 2.0 * 6.259e6 * 1024 + 1.592e6 * 1024},
+    ("cfg3", 1.0, "trailing"): {"backward": 2.0 * 7.47e6 * 1024 + 18.9e6 * 1024,
+                                "forward": 2.0 * 6.263e6 * 1024 + 1.584e6 * 1024},
+    ("cfg3", 1.0, "leading"): {"backward": 2.0 * 7.403e6 * 1024 + 19.08e6 * 1024,
+                               "forward": 2.0 * 6.258e6 * 1024 + 1.592e6 * 1024},
 }
 
 
@@ -256,7 +256,8 @@ def main():
     def gbs(nbytes, ms):
         return nbytes / (ms * 1e-3) / 1e9
 
-    measured = {} if args.spatial_sort else MEASURED_TRAFFIC_BYTES.get((args.config, args.scale, args.layout), {})
+    measured = ({} if args.spatial_sort or args.deterministic else
+                MEASURED_TRAFFIC_BYTES.get((args.config, args.scale, args.layout), {}))
     bwd_gbs, fwd_gbs = gbs(bytes_["bwd"], bwd_ms), gbs(bytes_["fwd"], fwd_ms)
     both_gbs = gbs(bytes_["fwd_bwd"], fwd_ms + bwd_ms)
     result = {

@@ -291,9 +291,9 @@ def emit_edge_bwd(p: Part) -> list[str]:
             else:
                 lines.append(f"            dsl = vfma(a{k}, y[{k}], dsl);")
             if k in dy_init:
-                lines.append(f"            dy[{k}] += hsum(vmulv(s[{p.sl[l]}], a{k}));")
+                lines.append(f"            dy[{k}] = vdot(s[{p.sl[l]}], a{k}, dy[{k}]);")
             else:
-                lines.append(f"            dy[{k}] = hsum(vmulv(s[{p.sl[l]}], a{k}));")
+                lines.append(f"            dy[{k}] = vdot(s[{p.sl[l]}], a{k});")
                 dy_init.add(k)
         lines.append(f"            ds.template put<{l}>(dsl);")
         lines.append("        }")

@@ -60,6 +60,20 @@ __device__ __forceinline__ Vec<C> vfmav(const Vec<C> &a, const Vec<C> &b, const 
     for (int t = 0; t < C; t++) r.v[t] = fmaf(a.v[t], b.v[t], c.v[t]);
     return r;
 }
+// sum over the channels of a lane of a * b (+ c): one fused multiply-add per channel
+template <int C>
+__device__ __forceinline__ float vdot(const Vec<C> &a, const Vec<C> &b, float c) {
+#pragma unroll
+    for (int t = 0; t < C; t++) c = fmaf(a.v[t], b.v[t], c);
+    return c;
+}
+template <int C>
+__device__ __forceinline__ float vdot(const Vec<C> &a, const Vec<C> &b) {
+    float c = a.v[0] * b.v[0];
+#pragma unroll
+    for (int t = 1; t < C; t++) c = fmaf(a.v[t], b.v[t], c);
+    return c;
+}
 template <int C>
 __device__ __forceinline__ float hsum(const Vec<C> &a) {
     float r = a.v[0];
