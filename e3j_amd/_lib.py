@@ -72,6 +72,8 @@ SYMBOLS = {
     "e3j_amd_sort_edges": (ctypes.c_int, [_P, _P, ctypes.c_int64, ctypes.c_int32, _P, _P, _P, _P, _P]),
     "e3j_amd_order_workspace_bytes": (ctypes.c_size_t, [ctypes.c_int32]),
     "e3j_amd_set_launch_variant": (None, [ctypes.c_int32, ctypes.c_int32]),
+    "e3j_amd_harmonics": (ctypes.c_int, [_P, ctypes.c_int64] + [ctypes.c_int32] * 4 + [_P, _P]),
+    "e3j_amd_harmonics_bwd": (ctypes.c_int, [_P, _P, ctypes.c_int64] + [ctypes.c_int32] * 4 + [_P, _P]),
     "e3j_amd_wrap_index": (ctypes.c_int, [_P, ctypes.c_int64, ctypes.c_int32, _P, _P]),
     "e3j_amd_locality_order": (ctypes.c_int, [_P, _P, ctypes.c_int32, ctypes.c_int32, _P, _P, _P]),
     "e3j_amd_xla_convolution": (_P, [_P]),

@@ -25,6 +25,50 @@ import torch
 
 from .spaces import O3Space, harmonics_space
 
+_NORMALIZATIONS = {"integral": 0, "component": 1, "norm": 2}
+_KERNEL_MAX_DEGREE = 6
+
+
+class _HarmonicsKernel(torch.autograd.Function):
+    """Degrees 0..l_max of GPU vectors through the HIP kernels (forward and VJP in one launch each)."""
+
+    @staticmethod
+    def forward(ctx, vec, module):
+        from . import _lib
+        flat = vec.reshape(-1, 3).contiguous()
+        l_max = max(module.degrees)
+        out = torch.empty((flat.shape[0], (l_max + 1) ** 2), dtype=flat.dtype, device=flat.device)
+        code = _lib.F32 if flat.dtype == torch.float32 else _lib.F64
+        with torch.cuda.device(flat.device):
+            _lib.check(_lib.load().e3j_amd_harmonics(
+                flat.data_ptr(), flat.shape[0], l_max, int(module.normalize),
+                _NORMALIZATIONS[module.normalization], code, out.data_ptr(),
+                int(torch.cuda.current_stream(flat.device).cuda_stream)))
+        ctx.module = module
+        ctx.save_for_backward(vec)
+        return out.reshape(*vec.shape[:-1], out.shape[-1])
+
+    @staticmethod
+    def backward(ctx, dout):
+        from . import _lib
+        (vec,) = ctx.saved_tensors
+        module = ctx.module
+        if torch.is_grad_enabled():
+            # a higher derivative is wanted: differentiate the tensor-operation form instead
+            with torch.enable_grad():
+                (grad,) = torch.autograd.grad(module._evaluate(vec), vec, dout, create_graph=True)
+            return grad, None
+        flat = vec.reshape(-1, 3).contiguous()
+        dflat = dout.reshape(flat.shape[0], -1).contiguous()
+        dvec = torch.empty_like(flat)
+        code = _lib.F32 if flat.dtype == torch.float32 else _lib.F64
+        with torch.cuda.device(flat.device):
+            _lib.check(_lib.load().e3j_amd_harmonics_bwd(
+                flat.data_ptr(), dflat.data_ptr(), flat.shape[0], max(module.degrees),
+                int(module.normalize), _NORMALIZATIONS[module.normalization], code, dvec.data_ptr(),
+                int(torch.cuda.current_stream(flat.device).cuda_stream)))
+        return dvec.reshape(vec.shape), None
+
 
 def _normalization_factor(l: int, normalization: str) -> float:
     if normalization == "integral":
@@ -48,6 +92,19 @@ class Harmonics:
             _normalization_factor(l, normalization)
 
     def __call__(self, r: torch.Tensor) -> torch.Tensor:
+        """Harmonics of the vectors `r (..., 3)`: `(..., dim)`.
+
+        Vectors in GPU memory and a target made of the degrees 0..l_max run the HIP kernels;
+        anything else (host tensors, other targets, degrees above 6, half precision) is
+        evaluated with tensor operations.
+        """
+        full = self.degrees == list(range(len(self.degrees)))
+        if (r.is_cuda and full and self.degrees[-1] <= _KERNEL_MAX_DEGREE and r.shape[-1] == 3
+                and r.dtype in (torch.float32, torch.float64)):
+            return _HarmonicsKernel.apply(r, self)
+        return self._evaluate(r)
+
+    def _evaluate(self, r: torch.Tensor) -> torch.Tensor:
         if self.normalize:
             norm = torch.linalg.vector_norm(r, dim=-1, keepdim=True)
             r = r / torch.where(norm > 0, norm, torch.ones_like(norm))

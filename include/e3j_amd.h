@@ -184,6 +184,19 @@ size_t e3j_amd_order_workspace_bytes(int32_t num_nodes);
 int e3j_amd_locality_order(const int32_t *other, const int32_t *row_ptr, int32_t num_nodes,
                            int32_t rounds, int32_t *order, void *workspace, void *stream);
 
+/* Edge featurisation next to the convolution: real spherical harmonics of `num` vectors
+ * (num, 3) for the degrees 0..l_max (l_max <= 6), out (num, (l_max + 1)^2), and the
+ * vector-Jacobian product dvec (num, 3) for a cotangent dout of that shape.  Order, harmonic
+ * frame and normalisations of the reference's Harmonics module
+ * (src/e3j/core/harmonics.py:25-42,92-101; src/e3j/utils/spherical_harmonics.py:33-38,66-75):
+ * normalization 0 "integral", 1 "component", 2 "norm"; normalize != 0 projects the vectors
+ * on the unit sphere first (zero vectors are left as they are).  val_dtype: E3J_AMD_F32/F64. */
+int e3j_amd_harmonics(const void *vec, int64_t num, int32_t l_max, int32_t normalize,
+                      int32_t normalization, int32_t val_dtype, void *out, void *stream);
+int e3j_amd_harmonics_bwd(const void *vec, const void *dout, int64_t num, int32_t l_max,
+                          int32_t normalize, int32_t normalization, int32_t val_dtype, void *dvec,
+                          void *stream);
+
 /* XLA-FFI handlers (C ABI of xla/ffi/api/c_api.h): `XLA_FFI_Error* handler(XLA_FFI_CallFrame*)`.
  * Operand order of "convolution"/"convolution_bwd" as in lib/e3j_ops/ffi/e3j_ops.h:457-472,575-594;
  * attrs: num_nodes, debug (reference) + layout, signature (optional). */
