@@ -54,6 +54,8 @@ def parse_args():
     ap.add_argument("--config", default="cfg3", choices=["cfg2", "cfg3", "cfg4"])
     ap.add_argument("--layout", default="trailing", choices=["trailing", "leading"],
                     help="memory layout of the node and edge arrays (channels last or first)")
+    ap.add_argument("--channels", type=int, default=None,
+                    help="channel count of cfg3 (default 128; kernels are built for 32, 64, 128, 256)")
     ap.add_argument("--scale", type=float, default=1.0, help="fraction of the configuration's atoms")
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--cpu-seconds", type=float, default=15.0)
@@ -70,13 +72,13 @@ def parse_args():
     return ap.parse_args()
 
 
-def build_workload(name: str, scale: float, device, spatial_sort: bool = False):
+def build_workload(name: str, scale: float, device, spatial_sort: bool = False, channels=None):
     from e3j_amd import workloads as W
     if name == "cfg2":
         return W.config2(scale, device=device)
     if name == "cfg4":
         return W.config4(scale, device=device)
-    return W.config3(scale, device=device, spatial_sort=spatial_sort)
+    return W.config3(scale, device=device, spatial_sort=spatial_sort, **({"channels": channels} if channels else {}))
 
 
 class AbiCalls:
@@ -209,7 +211,7 @@ def main():
     device = torch.device("cuda:0")
     torch.cuda.set_device(device)
 
-    w = build_workload(args.config, args.scale, device, args.spatial_sort)
+    w = build_workload(args.config, args.scale, device, args.spatial_sort, args.channels)
     w = w.with_layout("LEADING_CHANNELS" if args.layout == "leading" else "TRAILING_CHANNELS")
     module = w.module
     coef = module._packed_coef("float32")
@@ -256,7 +258,7 @@ def main():
     def gbs(nbytes, ms):
         return nbytes / (ms * 1e-3) / 1e9
 
-    measured = ({} if args.spatial_sort or args.deterministic else
+    measured = ({} if args.spatial_sort or args.deterministic or args.channels not in (None, 128) else
                 MEASURED_TRAFFIC_BYTES.get((args.config, args.scale, args.layout), {}))
     bwd_gbs, fwd_gbs = gbs(bytes_["bwd"], bwd_ms), gbs(bytes_["fwd"], fwd_ms)
     both_gbs = gbs(bytes_["fwd_bwd"], fwd_ms + bwd_ms)

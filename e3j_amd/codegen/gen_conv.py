@@ -33,26 +33,29 @@ from ..options import Layout
 from ..scalar_mixing import ScalarMixing
 from ..tensor_product import TensorProduct
 
-#: Signatures compiled into the library: (name, x irreps, y irreps, output filter, channels).
-#: They are the irreps/channel combinations of the benchmark configurations
-#: (SQRT_DIM_OUT normalisation, the default of `Convolution`).
-BUILTIN_SIGNATURES = [
-    ("l1_l2_to_l2_k32", "0e+1o", "0e+1o+2e", "0e+1o+2e", 32),
-    ("l2_l3_to_l2_k64", "0e+1o+2e", "0e+1o+2e+3o", "0e+1o+2e", 64),
-    ("l2_l3_to_l3_k64", "0e+1o+2e", "0e+1o+2e+3o", "0e+1o+2e+3o", 64),
-    ("l3_l3_to_l3_k64", "0e+1o+2e+3o", "0e+1o+2e+3o", "0e+1o+2e+3o", 64),
-    ("l3_l3_to_l3_k128", "0e+1o+2e+3o", "0e+1o+2e+3o", "0e+1o+2e+3o", 128),
+#: Tables compiled into the library: (name, x irreps, y irreps, output filter), the irreps
+#: combinations of the benchmark configurations (SQRT_DIM_OUT normalisation, the default of
+#: `Convolution`), each for the power-of-two channel counts the reference's fused kernel is
+#: used with (`tests/test_convolution.py:245-246`: multiples of 32).
+BUILTIN_TABLES = [
+    ("l1_l2_to_l2", "0e+1o", "0e+1o+2e", "0e+1o+2e", (32, 64, 128)),
+    ("l2_l3_to_l2", "0e+1o+2e", "0e+1o+2e+3o", "0e+1o+2e", (32, 64, 128)),
+    ("l2_l3_to_l3", "0e+1o+2e", "0e+1o+2e+3o", "0e+1o+2e+3o", (64, 128)),
+    ("l3_l3_to_l3", "0e+1o+2e+3o", "0e+1o+2e+3o", "0e+1o+2e+3o", (32, 64, 128, 256)),
 ]
+#: (name, x irreps, y irreps, output filter, channels) of every compiled signature
+BUILTIN_SIGNATURES = [(f"{name}_k{k}", xi, yi, oi, k) for name, xi, yi, oi, ks in BUILTIN_TABLES for k in ks]
 
 #: launch shapes per channel count: (channels per lane, waves per block, parts[, resident
 #: waves per SIMD the register allocation must allow]) variants for fwd and bwd.  `parts` splits the paths of the signature over that many waves.  Variant 0
 #: is the default; the others are selected with the environment variables
 #: E3J_AMD_FWD_VARIANT / E3J_AMD_BWD_VARIANT (read once) for tuning runs.
 LAUNCH = {
-    32: dict(fwd=[(1, 4, 1)], bwd=[(1, 4, 1)]),
+    32: dict(fwd=[(1, 4, 1)], bwd=[(1, 4, 2), (1, 4, 1)]),
     64: dict(fwd=[(1, 4, 1), (1, 4, 2)], bwd=[(1, 4, 2), (1, 4, 1), (1, 4, 3), (1, 4, 4)]),
     128: dict(fwd=[(1, 4, 1), (1, 4, 2), (2, 4, 2), (2, 4, 4)],
               bwd=[(2, 4, 3), (1, 4, 1), (1, 4, 3), (1, 4, 4), (2, 4, 4), (1, 4, 2)]),
+    256: dict(fwd=[(1, 4, 1), (1, 4, 2)], bwd=[(2, 4, 3), (1, 4, 2), (1, 4, 3)]),
 }
 
 
@@ -60,9 +63,10 @@ LAUNCH = {
 #: split; a backward block is the parts of one (receiver, channel slice), so its wave count
 #: is the part count (the first number is ignored there).
 LAUNCH_LEADING = {
-    32: dict(fwd=[(4, 1)], bwd=[(1, 1)]),
+    32: dict(fwd=[(4, 1)], bwd=[(2, 2), (1, 1)]),
     64: dict(fwd=[(4, 1)], bwd=[(3, 3), (1, 1), (2, 2), (4, 4)]),
     128: dict(fwd=[(4, 1)], bwd=[(3, 3), (1, 1), (2, 2), (4, 4)]),
+    256: dict(fwd=[(4, 1)], bwd=[(3, 3), (2, 2)]),
 }
 
 

@@ -217,7 +217,7 @@ struct OrderedWorkspace {
         ptr = take(4 * (n + 1));
         csr = take(e3j_amd_csr_workspace_bytes(p.num_nodes, p.num_edges));
         u = take(4 * e * (size_t)p.num_x * (size_t)p.channels);
-        slots = take(4 * e * (size_t)kMaxDySlots * (size_t)p.num_y);
+        slots = take(4 * e * (size_t)max_dy_slots(p.channels) * (size_t)p.num_y);
         total = at;
     }
 };

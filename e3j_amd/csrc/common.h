@@ -82,7 +82,12 @@ const Tuning &tuning();
 // contribution of every CSR position as one row of `u` and, when several waves share an
 // edge, its dy sums into slot (position, wave) of `dy_slots`; fixed-order reductions follow
 // (`reduce_ordered_dx`, `reduce_ordered_dy`).  The launcher fills in `slots` and `covered`.
-constexpr int kMaxDySlots = 8;
+constexpr int kMaxDySlots = 16;
+// upper bound for a channel count: at most four parts times the 64-channel slices
+inline int max_dy_slots(int channels) {
+    const int slots = 4 * ((channels + 63) / 64);
+    return slots < kMaxDySlots ? slots : kMaxDySlots;
+}
 struct OrderedBwd {
     float *u;                 // (num_edges, X * K)
     float *dy_slots;          // (num_edges, slots, Y)

@@ -7,12 +7,17 @@
 // register-resident accumulation over a receiver's edge segment, the single
 // row write-back, the channel reduction of dy and the float atomics of dx.
 //
-// Mapping (trailing-channels layout): one 64-lane wavefront owns one receiver
-// and a slice of 64*CPL consecutive channels; a lane owns CPL consecutive
-// channels, so every row access is one fully coalesced 256*CPL-byte load.
+// Mapping (trailing-channels layout): one 64-lane wavefront owns one receiver,
+// a slice of 64*CPL channels and one part of the signature's paths; a lane owns
+// CPL channels (consecutive in the forward, a wave apart in the backward), so
+// every row access is a fully coalesced load of whole 256-byte row pieces.
 // Waves never communicate (no LDS, no barrier): a block is only a bundle of
 // WPB independent waves.  Everything indexed by the edge is wave-uniform
 // (scalar registers / scalar loads).
+//
+// Mapping (leading-channels layout): the same arithmetic between two 90-degree
+// turns of contiguous (channels, dim) blocks through LDS strips; see the
+// section further down.
 #ifndef E3J_AMD_CSRC_UNROLLED_H_
 #define E3J_AMD_CSRC_UNROLLED_H_
 

@@ -200,10 +200,10 @@ def config1(scale: float = 1.0, device="cpu") -> Workload:
                          box=20.0 * scale ** (1.0 / 3.0), periodic=False, device=device)
 
 
-def config2(scale: float = 1.0, out_irreps: str = "0e+1o+2e", device="cpu") -> Workload:
+def config2(scale: float = 1.0, out_irreps: str = "0e+1o+2e", channels: int = 64, device="cpu") -> Workload:
     """5 000 atoms, ~30 neighbours (~150k edges), 64 channels, 0e+1o+2e x lmax 3."""
     n = max(8, int(5000 * scale))
-    return make_workload("cfg2", n, "0e+1o+2e", 3, out_irreps, 64, (11, 12, 13, 14), device=device)
+    return make_workload("cfg2", n, "0e+1o+2e", 3, out_irreps, channels, (11, 12, 13, 14), device=device)
 
 
 def config3(scale: float = 1.0, channels: int = 128, device="cpu", spatial_sort: bool = False) -> Workload:

@@ -118,8 +118,8 @@ int e3j_amd_convolution_bwd_receiver(const e3j_amd_conv_params *p, const void *c
  * (tests/test_ops/test_convolution_op.py:329-342), at the price of one more pass over
  * E * num_x * channels floats.  Needs a compile-time-unrolled kernel (p->signature >= 0),
  * else E3J_AMD_UNIMPLEMENTED.  workspace: device memory, at least
- * e3j_amd_convolution_bwd_ordered_workspace_bytes(p) bytes (about E * (num_x * channels + 8 * num_y)
- * floats); contents on entry and exit are irrelevant. */
+ * e3j_amd_convolution_bwd_ordered_workspace_bytes(p) bytes (about E * (num_x * channels +
+ * channels / 16 * num_y) floats); contents on entry and exit are irrelevant. */
 size_t e3j_amd_convolution_bwd_ordered_workspace_bytes(const e3j_amd_conv_params *p);
 int e3j_amd_convolution_bwd_ordered(const e3j_amd_conv_params *p, const void *coef, const void *x,
                                     const void *y, const void *s, const void *dm,

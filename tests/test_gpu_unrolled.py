@@ -12,6 +12,10 @@ from tests import helpers as H
 pytestmark = pytest.mark.gpu
 
 CASES = {
+    "cfg3_k32": lambda: W.config3(0.006, channels=32),
+    "cfg3_k256": lambda: W.config3(0.003, channels=256),
+    "cfg2_k32": lambda: W.config2(0.04, channels=32),
+    "cfg2_k128": lambda: W.config2(0.03, channels=128),
     "cfg1": lambda: W.config1(0.2),
     "cfg2": lambda: W.config2(0.04),
     "cfg2_out3": lambda: W.config2(0.04, out_irreps="0e+1o+2e+3o"),
