@@ -71,6 +71,7 @@ SYMBOLS = {
     "e3j_amd_csr_row_ptr": (ctypes.c_int, [_P, ctypes.c_int64, ctypes.c_int32, _P, _P, _P]),
     "e3j_amd_sort_edges": (ctypes.c_int, [_P, _P, ctypes.c_int64, ctypes.c_int32, _P, _P, _P, _P, _P]),
     "e3j_amd_order_workspace_bytes": (ctypes.c_size_t, [ctypes.c_int32]),
+    "e3j_amd_register_signature": (ctypes.c_int, [_P]),
     "e3j_amd_set_launch_variant": (None, [ctypes.c_int32, ctypes.c_int32]),
     "e3j_amd_harmonics": (ctypes.c_int, [_P, ctypes.c_int64] + [ctypes.c_int32] * 4 + [_P, _P]),
     "e3j_amd_harmonics_bwd": (ctypes.c_int, [_P, _P, ctypes.c_int64] + [ctypes.c_int32] * 4 + [_P, _P]),
@@ -93,7 +94,8 @@ def load() -> ctypes.CDLL:
         raise ImportError(
             f"{LIB_PATH} is missing: build it with `python -m e3j_amd.build` "
             "(hipcc, gfx950). e3j_amd has no fallback implementation.")
-    lib = ctypes.CDLL(LIB_PATH)
+    # global symbols: signature libraries compiled at run time resolve against this one
+    lib = ctypes.CDLL(LIB_PATH, mode=ctypes.RTLD_GLOBAL)
     for name, (restype, argtypes) in SYMBOLS.items():
         fn = getattr(lib, name)  # AttributeError if the export is missing
         fn.restype = restype

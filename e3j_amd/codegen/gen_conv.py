@@ -337,21 +337,54 @@ def build_table(x_irreps, y_irreps, out_filter):
 def emit_signature(sig_id: int, name: str, x_irreps: str, y_irreps: str, out_filter: str,
                    channels: int) -> str:
     t, tp = build_table(x_irreps, y_irreps, out_filter)
-    launch = LAUNCH[channels]
-    vals = ", ".join(_lit(v) for v in t.val)
-    idxs = ", ".join(str(int(a)) for row in t.idx for a in row)
     desc = (f"{name}: x {tp.source[0]} | y {tp.source[1]} -> {tp.target}, "
             f"K={channels}, trailing, nnz={len(t.val)}")
+    return emit_table_source(t, name, desc, channels, symbols=(f"kSignature_{2 * sig_id}",
+                                                                 f"kSignature_{2 * sig_id + 1}"))
+
+
+def plugin_launch(channels: int):
+    """Launch shapes of a signature compiled at run time: the default variant of each pass."""
+    if channels % 128 == 0:
+        trailing = dict(fwd=[(1, 4, 1)], bwd=[(2, 4, 3)])
+    elif channels % 64 == 0:
+        trailing = dict(fwd=[(1, 4, 1)], bwd=[(1, 4, 2)])
+    else:
+        trailing = dict(fwd=[(1, 4, 1)], bwd=[(1, 4, 2)])
+    width = min(channels, 64)
+    leading = None
+    if channels % width == 0 and width >= 4 and (width & (width - 1)) == 0:  # power-of-two wave width
+        parts = 3 if channels >= 64 else 2
+        leading = dict(fwd=[(4, 1)], bwd=[(parts, parts)])
+    return trailing, leading
+
+
+def supports(t: "Table", channels: int) -> bool:
+    """Whether the kernel templates can take this table (register-resident dy sums, bit masks)."""
+    return t.Y <= 16 and t.X <= 64 and t.S <= 64 and t.Z <= 255 and channels >= 1
+
+
+def emit_table_source(t: "Table", name: str, desc: str, channels: int, symbols, include='"../unrolled.h"',
+                      launch=None, lead="builtin", plugin: bool = False) -> str:
+    """HIP source of the kernels and registry entries of one table at one channel count.
+
+    `symbols`: names of the trailing- and leading-layout `Signature` objects.  `plugin` adds
+    the C accessor a run-time compiled library is loaded through.
+    """
+    launch = LAUNCH[channels] if launch is None else launch
+    vals = ", ".join(_lit(v) for v in t.val)
+    idxs = ", ".join(str(int(a)) for row in t.idx for a in row)
     out = [
         "// GENERATED by e3j_amd/codegen/gen_conv.py -- do not edit.",
         f"// {desc}",
-        '#include "../unrolled.h"',
+        f"#include {include}",
         "",
         "namespace e3j_amd {",
         "namespace {",
         "",
     ]
-    lead = LAUNCH_LEADING[channels] if (t.X <= 64 and t.S <= 64) else None
+    if lead == "builtin":
+        lead = LAUNCH_LEADING[channels] if (t.X <= 64 and t.S <= 64) else None
     splits = sorted({v[2] for v in launch["fwd"] + launch["bwd"]} |
                     ({v[1] for v in lead["fwd"] + lead["bwd"]} if lead else set()))
     part_names = {}
@@ -413,7 +446,7 @@ def emit_signature(sig_id: int, name: str, x_irreps: str, y_irreps: str, out_fil
     out += [ln.replace("VARIANT", "tuning().bwd_variant") for ln in switch(
         launch["bwd"], lambda v: f"launch_unrolled_bwd<{channels}, {v[0]}, {v[1]}, {(*v, 1)[3]}, {t.Y}, {t.X}, "
                                  f"{part_names[v[2]]}>(p, x, y, s, dm, sender, row_ptr, perm, dx, dy, ds, stream, ordered);")]
-    out += [f"extern const Signature kSignature_{2 * sig_id} = {{",
+    out += [f"extern const Signature {symbols[0]} = {{",
             f'    "{desc}",',
             f"    {t.X}, {t.Y}, {t.Z}, {t.S}, {len(t.val)}, {channels}, E3J_AMD_LAYOUT_TRAILING, kVal, kIdx,",
             "    &run_fwd, &run_bwd,",
@@ -427,16 +460,22 @@ def emit_signature(sig_id: int, name: str, x_irreps: str, y_irreps: str, out_fil
         out += [ln.replace("VARIANT", "tuning().bwd_variant") for ln in switch(
             lead["bwd"], lambda v: f"launch_unrolled_bwd_leading<{channels}, {t.Y}, {t.X}, "
                                    f"{part_names[v[1]]}>(p, x, y, s, dm, sender, row_ptr, perm, dx, dy, ds, stream, ordered);")]
-        out += [f"extern const Signature kSignature_{2 * sig_id + 1} = {{",
+        out += [f"extern const Signature {symbols[1]} = {{",
                 f'    "{desc.replace("trailing", "leading")}",',
                 f"    {t.X}, {t.Y}, {t.Z}, {t.S}, {len(t.val)}, {channels}, E3J_AMD_LAYOUT_LEADING, kVal, kIdx,",
                 "    &run_fwd_leading, &run_bwd_leading,",
                 "};"]
     else:  # no leading-layout kernels: an entry that never matches keeps the numbering regular
-        out += [f"extern const Signature kSignature_{2 * sig_id + 1} = {{",
+        out += [f"extern const Signature {symbols[1]} = {{",
                 f'    "{desc.replace("trailing", "leading (not built)")}",',
                 "    -1, -1, -1, -1, -1, -1, E3J_AMD_LAYOUT_LEADING, nullptr, nullptr, nullptr, nullptr,",
                 "};"]
+    if plugin:
+        out += ["",
+                "// entry point of a run-time compiled signature library: 0 trailing, 1 leading layout",
+                'extern "C" const void *e3j_amd_plugin_signature(int which) {',
+                f"    return which == 0 ? &{symbols[0]} : which == 1 ? &{symbols[1]} : nullptr;",
+                "}"]
     out += ["#endif",
             "",
             "}  // namespace e3j_amd",
@@ -449,8 +488,8 @@ def emit_registry(count: int) -> str:
            '#include "../common.h"', "", "namespace e3j_amd {", ""]
     for n in range(count):
         out.append(f"extern const Signature kSignature_{n};")
-    out += ["", f"int num_signatures() {{ return {count}; }}", "",
-            "const Signature &signature(int id) {",
+    out += ["", f"int num_builtin_signatures() {{ return {count}; }}", "",
+            "const Signature &builtin_signature(int id) {",
             "    static const Signature *const table[] = {" +
             ", ".join(f"&kSignature_{n}" for n in range(count)) + (", " if count else "") + "nullptr};",
             "    return *table[id];", "}", "", "}  // namespace e3j_amd", ""]

@@ -5,7 +5,9 @@
 #include <cstring>
 
 #include <cstdint>
+#include <deque>
 #include <initializer_list>
+#include <mutex>
 
 #include "common.h"
 
@@ -39,6 +41,24 @@ Tuning &mutable_tuning() {
 }  // namespace
 
 const Tuning &tuning() { return mutable_tuning(); }
+
+// Signatures registered at run time live behind the built-in ones.  The list only grows and
+// a deque never moves its elements, so ids and references stay valid.
+namespace {
+std::mutex g_registry_mutex;
+std::deque<const Signature *> g_registered;
+}  // namespace
+
+int num_signatures() {
+    std::lock_guard<std::mutex> lock(g_registry_mutex);
+    return num_builtin_signatures() + (int)g_registered.size();
+}
+
+const Signature &signature(int id) {
+    if (id < num_builtin_signatures()) return builtin_signature(id);
+    std::lock_guard<std::mutex> lock(g_registry_mutex);
+    return *g_registered[id - num_builtin_signatures()];
+}
 
 namespace {
 
@@ -146,6 +166,18 @@ extern "C" {
 const char *e3j_amd_last_error(void) { return g_last_error.c_str(); }
 
 const char *e3j_amd_version(void) { return "e3j_amd 0.1 (gfx950)"; }
+
+int e3j_amd_register_signature(const void *entry) {
+    const Signature *sg = static_cast<const Signature *>(entry);
+    if (sg == nullptr || sg->fwd == nullptr || sg->bwd == nullptr || sg->val == nullptr ||
+        sg->idx == nullptr || sg->num_coef <= 0) {
+        set_error(E3J_AMD_INVALID_ARGUMENT, "register_signature: incomplete entry");
+        return -1;
+    }
+    std::lock_guard<std::mutex> lock(g_registry_mutex);
+    g_registered.push_back(sg);
+    return num_builtin_signatures() + (int)g_registered.size() - 1;
+}
 
 void e3j_amd_set_launch_variant(int32_t fwd_variant, int32_t bwd_variant) {
     mutable_tuning() = Tuning{fwd_variant, bwd_variant};

@@ -120,6 +120,9 @@ struct Signature {
                const int32_t *edge_perm, float *dx, float *dy, float *ds, hipStream_t stream,
                OrderedBwd *ordered);  // ordered: nullptr = dx (and shared dy) by float atomics
 };
+// built-in signatures (generated/registry.hip), then the ones registered at run time (capi.hip)
+int num_builtin_signatures();
+const Signature &builtin_signature(int id);
 int num_signatures();
 const Signature &signature(int id);
 

@@ -92,15 +92,26 @@ class _Table:
         `y_flip`: bit mask of the y components whose coefficients carry the opposite sign of
         the built-in table (the parity signs of the SENDER ordering).
         """
-        key = (dims, channels, layout)
+        jit = config().jit
+        key = (dims, channels, layout, jit)
         hit = self._signature.get(key)
         if hit is None:
             scale, flip = ctypes.c_float(1.0), ctypes.c_uint32(0)
             val_code = _lib.F32 if self.val_np_dtype == np.float32 else _lib.F64
-            sig = _lib.load().e3j_amd_find_signature(
-                self.packed.ctypes.data, self.idx_bytes, val_code, self.num_coef, dims[0], dims[1],
-                dims[2], dims[3], channels, layout.value, ctypes.byref(scale), ctypes.byref(flip))
-            hit = self._signature[key] = (int(sig), float(scale.value), int(flip.value))
+
+            def find():
+                return int(_lib.load().e3j_amd_find_signature(
+                    self.packed.ctypes.data, self.idx_bytes, val_code, self.num_coef, dims[0], dims[1],
+                    dims[2], dims[3], channels, layout.value, ctypes.byref(scale), ctypes.byref(flip)))
+
+            sig = find()
+            if sig < 0 and jit and self.val_np_dtype == np.float32 and self.num_coef > 0:
+                # not built in: generate and compile the kernels of this table, then look again
+                from . import jit as _jit
+                c = self.unpack()
+                if _jit.register(c.val, c.idx.astype(np.int64), dims, channels):
+                    sig = find()
+            hit = self._signature[key] = (sig, float(scale.value), int(flip.value))
         return hit
 
 

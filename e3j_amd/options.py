@@ -86,6 +86,10 @@ class Config:
     #: sweeps of label propagation behind the locality-aware row order of the kernels
     #: (0 = rows are processed in index order).
     locality_rounds: int = 2
+    #: compile unrolled kernels at run time for coefficient tables the library was not built
+    #: for (needs hipcc; about half a minute per new table, cached on disk); off: such tables
+    #: run the table-driven kernels.
+    jit: bool = False
 
 
 class _ConfigHolder:
@@ -96,6 +100,7 @@ class _ConfigHolder:
             debug_level=int(os.environ.get("E3J_AMD_DEBUG", "0")),
             deterministic=os.environ.get("E3J_AMD_DETERMINISTIC", "0") not in ("0", ""),
             locality_rounds=int(os.environ.get("E3J_AMD_LOCALITY_ROUNDS", "2")),
+            jit=os.environ.get("E3J_AMD_JIT", "0") not in ("0", ""),
         )
 
     def __call__(self, **updates) -> Config:

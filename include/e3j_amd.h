@@ -150,7 +150,15 @@ int e3j_amd_find_signature(const void *coef_host, int32_t coef_idx_bytes, int32_
  * (src/e3j/ops/convolution.py:178-208). */
 void e3j_amd_set_launch_variant(int32_t fwd_variant, int32_t bwd_variant);
 
-/* Number of built-in signatures and a printable description of one. */
+/* Adds a signature compiled at run time (e3j_amd/jit.py generates the kernels of a table
+ * the library was not built for, compiles them against this library and hands over the entry
+ * its plugin exports).  Returns the new signature id, which e3j_amd_find_signature reports
+ * from then on, or -1.  The entry must stay loaded for the life of the process.  Counterpart
+ * of the trace-time unrolling of the reference's Pallas kernels
+ * (src/e3j/pallas_ops/convolution/mosaic_gpu/fwd.py:162-177). */
+int e3j_amd_register_signature(const void *entry);
+
+/* Number of signatures (built-in and registered) and a printable description of one. */
 int e3j_amd_num_signatures(void);
 const char *e3j_amd_signature_name(int signature);
 

@@ -1,0 +1,86 @@
+"""Kernels generated and compiled at run time for tables the library was not built for
+(`config(jit=True)`), against the CPU oracle."""
+
+import numpy as np
+import pytest
+import torch
+
+import e3j_amd
+from e3j_amd import ConvolutionParams, convolution, convolution_bwd
+from e3j_amd.ops import _Table
+from tests import helpers as H
+
+pytestmark = pytest.mark.gpu
+
+
+def dev(a):
+    return torch.from_numpy(np.ascontiguousarray(a)).cuda()
+
+
+def _random_case(seed, N, E, X, Y, Z, S, K, nnz):
+    rng = np.random.default_rng(seed)
+    idx, val, mix = H.random_table(rng, nnz, X, Y, Z, S)
+    snd, rcv = H.random_graph(rng, N, E)
+    x, y, s, dm = H.random_operands(rng, N, E, X, Y, S, K, Z)
+    return dict(idx=idx, val=val, mix=mix, snd=snd, rcv=rcv, x=x, y=y, s=s, dm=dm,
+                coef=H.pack_table(idx, val, mix), params=ConvolutionParams(num_out=Z, num_scalars=S))
+
+
+@pytest.mark.parametrize("layout", ["TRAILING_CHANNELS", "LEADING_CHANNELS"])
+@pytest.mark.parametrize("case", [
+    dict(seed=1, N=40, E=600, X=5, Y=6, Z=7, S=4, K=64, nnz=60),     # whole waves
+    dict(seed=2, N=30, E=400, X=3, Y=9, Z=10, S=5, K=48, nnz=80),    # idle lanes; leading: table-driven
+    dict(seed=3, N=25, E=300, X=6, Y=4, Z=12, S=6, K=128, nnz=100),  # two channels per lane backward
+])
+def test_random_tables_run_on_generated_kernels(case, layout):
+    p = _random_case(**case)
+    leading = layout == "LEADING_CHANNELS"
+    t = (lambda a: np.ascontiguousarray(a.transpose(0, 2, 1))) if leading else (lambda a: a)
+    back = (lambda g: g.transpose(1, 2)) if leading else (lambda g: g)
+    x, y, s, dm = dev(t(p["x"])), dev(p["y"]), dev(t(p["s"])), dev(t(p["dm"]))
+    snd, rcv = dev(p["snd"]), dev(p["rcv"])
+    dims = (case["X"], case["Y"], case["Z"], case["S"])
+    table = _Table.get(p["coef"], np.float32)
+    with e3j_amd.config.use(jit=True):  # (a registered table stays registered for the process)
+        sig = table.signature(dims, case["K"], e3j_amd.Layout.parse(layout))[0]
+        assert (sig >= 0) == (not leading or case["K"] % 64 == 0)
+        out = convolution(p["coef"], x, y, s, snd, rcv, p["params"], layout=layout)
+        grads = convolution_bwd(p["coef"], x, y, s, snd, rcv, dm, p["params"], layout=layout)
+        with e3j_amd.config.use(jit=True, deterministic=True):
+            ordered = convolution_bwd(p["coef"], x, y, s, snd, rcv, dm, p["params"], layout=layout)
+    ref, mag = H.forward_reference(p["idx"], p["val"], p["mix"], p["x"], p["y"], p["s"], p["snd"], p["rcv"],
+                                   case["Z"])
+    H.assert_parity(back(out).cpu().numpy(), ref, mag, "out")
+    refs, mags = H.backward_reference(p["idx"], p["val"], p["mix"], p["x"], p["y"], p["s"], p["snd"], p["rcv"],
+                                      p["dm"])
+    for g, o, r, m, name in zip(grads, ordered, refs, mags, ("dx", "dy", "ds")):
+        for got in (g, o):
+            got = back(got) if got.dim() == 3 else got
+            H.assert_parity(got.cpu().numpy(), r, m, name)
+
+
+def test_module_with_irreps_outside_the_built_in_tables():
+    """x = 0e+1o+2e, y up to l = 2, out up to l = 2, 64 channels: generated on first use, then
+    the same numbers as the table-driven kernels."""
+    m = e3j_amd.Convolution(("0e+1o+2e", "0e+1o+2e"), "0e+1o+2e", graph_ordering="RECEIVER")
+    rng = np.random.default_rng(5)
+    N, E, K = 50, 900, 64
+    snd, rcv = H.random_graph(rng, N, E)
+    x = dev(rng.standard_normal((N, m.source[0].dim, K)).astype(np.float32)).requires_grad_(True)
+    y = dev(rng.standard_normal((E, m.source[1].dim)).astype(np.float32)).requires_grad_(True)
+    s = dev(rng.standard_normal((E, m.params.num_scalars, K)).astype(np.float32)).requires_grad_(True)
+    dm = dev(rng.standard_normal((N, m.target.dim, K)).astype(np.float32))
+
+    def run():
+        out = m(x, y, s, dev(snd), dev(rcv))
+        return (out,) + torch.autograd.grad(out, (x, y, s), dm)
+
+    with e3j_amd.config.use(jit=False):
+        slow = run()
+    with e3j_amd.config.use(jit=True):
+        packed = m._packed_coef("float32")
+        dims = (m.source[0].dim, m.source[1].dim, m.target.dim, m.params.num_scalars)
+        assert _Table.get(packed, np.float32).signature(dims, K, m.layout)[0] >= 0
+        fast = run()
+    for a, b in zip(slow, fast):
+        assert float((a - b).detach().abs().max()) <= 2e-5 * float(a.detach().abs().max())

@@ -289,3 +289,31 @@ def test_energy_model_forces_are_the_energy_gradient():
     torch.testing.assert_close(slope, -(forces * direction).sum(), rtol=1e-6, atol=1e-8)
     # translation invariance of a periodic cell: no net force
     assert float(forces.sum(0).abs().max()) < 1e-12
+
+
+def test_run_time_signature_compiles_and_registers():
+    """A table the library was not built for: the generator's output compiles against the
+    installed kernel templates, loads next to the library and is found by the signature
+    lookup (hipcc cross-compiles, so this runs without a GPU)."""
+    import ctypes
+    from e3j_amd import _lib, jit
+    module = Convolution(("0e+1o", "0e+1o"), "0e+1o", graph_ordering="RECEIVER")
+    c = module.coef
+    dims = (4, 4, module.params.num_out, module.params.num_scalars)
+    lib = _lib.load()
+    packed = module._packed_coef("float32")
+    scale, flip = ctypes.c_float(0), ctypes.c_uint32(0)
+
+    def find(channels, layout):
+        return lib.e3j_amd_find_signature(packed.ctypes.data, 1, _lib.F32, packed.shape[0], *dims, channels,
+                                          layout, ctypes.byref(scale), ctypes.byref(flip))
+    ids = jit.register(np.asarray(c.val, np.float32), np.asarray(c.idx, np.int64), dims, 64)
+    assert len(ids) == 2 and ids == jit.register(np.asarray(c.val, np.float32), np.asarray(c.idx, np.int64), dims, 64)
+    assert find(64, 1) == ids[0] and find(64, 0) == ids[1] and scale.value == 1.0
+    assert b"run-time table" in lib.e3j_amd_signature_name(ids[0])
+    assert find(128, 1) == -1                                     # another channel count: not built
+    # 25 y components exceed the register-resident dy sums of the templates: served table-driven
+    big = Convolution(("0e+1o", "0e+1o+2e+3o+4e"), "0e+1o", graph_ordering="RECEIVER")
+    cb = big.coef
+    assert jit.register(np.asarray(cb.val, np.float32), np.asarray(cb.idx, np.int64),
+                        (4, 25, big.params.num_out, big.params.num_scalars), 64) == []
