@@ -80,6 +80,7 @@ SYMBOLS = {
     "e3j_amd_xla_convolution": (_P, [_P]),
     "e3j_amd_xla_convolution_bwd": (_P, [_P]),
     "e3j_amd_xla_convolution_bwd_receiver": (_P, [_P]),
+    "e3j_amd_xla_convolution_bwd_ordered": (_P, [_P]),
 }
 
 _lib = None

@@ -9,7 +9,9 @@
 // (3, nnz, numel) / (3*nnz, numel) flagged by the attribute coef_stacked = 1;
 // the first of the three, sorted for dx with columns (j, i, k, l), is then used.
 // A third target, "convolution_bwd_receiver", takes the forward's receiver CSR:
-//   coef, x, y, s, dm, sender, receiver_ptr, edge_perm -> dx, dy, ds.
+//   coef, x, y, s, dm, sender, receiver_ptr, edge_perm -> dx, dy, ds;
+// a fourth, "convolution_bwd_ordered", the same operands and a scratch buffer as a fourth
+// result (the atomic-free, bit-reproducible backward).
 // Attributes: num_nodes, debug (reference); layout, signature, coef_scale, y_flip,
 // coef_stacked (optional).  Handlers are re-entrant, allocate nothing and
 // enqueue on the stream XLA hands over; they answer the metadata query.
@@ -58,6 +60,16 @@ const XlaBuffer *ret(const XlaCallFrame *f, int64_t i) {
     if (i >= f->rets.size || f->rets.types[i] != kXlaRetBuffer) return nullptr;
     return static_cast<const XlaBuffer *>(f->rets.rets[i]);
 }
+size_t dtype_bytes(int32_t dtype) {
+    switch (dtype) {
+        case kXlaU8: return 1;
+        case kXlaF16: return 2;
+        case kXlaS32: case kXlaF32: return 4;
+        case kXlaS64: case kXlaF64: return 8;
+        default: return 1;  // unknown element types are counted as bytes
+    }
+}
+
 int64_t count(const XlaBuffer *b) {
     int64_t n = 1;
     for (int64_t d = 0; d < b->rank; d++) n *= b->dims[d];
@@ -149,13 +161,19 @@ void *decode_common(XlaCallFrame *f, const char *op, const XlaBuffer *coef, cons
 
 bool is_s32_vector(const XlaBuffer *b) { return b && b->dtype == kXlaS32 && b->rank == 1; }
 
-void *backward_handler(XlaCallFrame *f, bool group_is_receiver) {
-    const char *op = group_is_receiver ? "convolution_bwd_receiver" : "convolution_bwd";
+enum class Backward { kSenderRows, kReceiverRows, kReceiverRowsOrdered };
+
+void *backward_handler(XlaCallFrame *f, Backward mode) {
+    const bool group_is_receiver = mode != Backward::kSenderRows;
+    const bool ordered = mode == Backward::kReceiverRowsOrdered;
+    const char *op = ordered ? "convolution_bwd_ordered"
+                             : group_is_receiver ? "convolution_bwd_receiver" : "convolution_bwd";
     if (answer_metadata(f)) return nullptr;
     if (f->stage != kXlaStageExecute) return nullptr;
-    if (f->args.size < 8 || f->rets.size != 3)
+    if (f->args.size < 8 || f->rets.size != (ordered ? 4 : 3))
         return make_error(f, E3J_AMD_INVALID_ARGUMENT,
-                          std::string(op) + ": expected 8 or 9 operands and 3 results");
+                          std::string(op) + (ordered ? ": expected 8 operands and 4 results (dx, dy, ds, workspace)"
+                                                     : ": expected 8 or 9 operands and 3 results"));
     const XlaBuffer *coef = arg(f, 0), *x = arg(f, 1), *y = arg(f, 2), *s = arg(f, 3), *dm = arg(f, 4);
     const XlaBuffer *other = arg(f, 5), *row_ptr = arg(f, 6), *perm = arg(f, 7);
     const XlaBuffer *dx = ret(f, 0), *dy = ret(f, 1), *ds = ret(f, 2);
@@ -172,6 +190,21 @@ void *backward_handler(XlaCallFrame *f, bool group_is_receiver) {
     const int64_t numel = coef->dims[coef->rank - 1];
     d.p.num_coef = (int32_t)(count(coef) / numel / (stacked ? 3 : 1));
     const int32_t *perm_ptr = count(perm) ? static_cast<const int32_t *>(perm->data) : nullptr;
+    if (ordered) {
+        // the scratch of the atomic-free backward travels as a fourth result buffer (any dtype)
+        const XlaBuffer *workspace = ret(f, 3);
+        if (!workspace || workspace->data == nullptr ||
+            (size_t)count(workspace) * dtype_bytes(workspace->dtype) <
+                e3j_amd_convolution_bwd_ordered_workspace_bytes(&d.p))
+            return make_error(f, E3J_AMD_INVALID_ARGUMENT,
+                              std::string(op) + ": the workspace result is smaller than "
+                                                "e3j_amd_convolution_bwd_ordered_workspace_bytes");
+        const int rc = e3j_amd_convolution_bwd_ordered(
+            &d.p, coef->data, x->data, y->data, s->data, dm->data, static_cast<const int32_t *>(other->data),
+            static_cast<const int32_t *>(row_ptr->data), perm_ptr, dx->data, dy->data, ds->data,
+            workspace->data, d.stream);
+        return status_to_error(f, rc);
+    }
     const int rc = run_backward(&d.p, group_is_receiver, coef->data, x->data, y->data, s->data, dm->data,
                                 static_cast<const int32_t *>(other->data),
                                 static_cast<const int32_t *>(row_ptr->data), perm_ptr, dx->data,
@@ -213,11 +246,15 @@ void *e3j_amd_xla_convolution(void *call_frame) {
 }
 
 void *e3j_amd_xla_convolution_bwd(void *call_frame) {
-    return backward_handler(static_cast<XlaCallFrame *>(call_frame), false);
+    return backward_handler(static_cast<XlaCallFrame *>(call_frame), Backward::kSenderRows);
 }
 
 void *e3j_amd_xla_convolution_bwd_receiver(void *call_frame) {
-    return backward_handler(static_cast<XlaCallFrame *>(call_frame), true);
+    return backward_handler(static_cast<XlaCallFrame *>(call_frame), Backward::kReceiverRows);
+}
+
+void *e3j_amd_xla_convolution_bwd_ordered(void *call_frame) {
+    return backward_handler(static_cast<XlaCallFrame *>(call_frame), Backward::kReceiverRowsOrdered);
 }
 
 }  // extern "C"

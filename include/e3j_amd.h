@@ -211,6 +211,7 @@ int e3j_amd_harmonics_bwd(const void *vec, const void *dout, int64_t num, int32_
 void *e3j_amd_xla_convolution(void *call_frame);
 void *e3j_amd_xla_convolution_bwd(void *call_frame);
 void *e3j_amd_xla_convolution_bwd_receiver(void *call_frame);
+void *e3j_amd_xla_convolution_bwd_ordered(void *call_frame);
 
 #ifdef __cplusplus
 }

@@ -94,3 +94,53 @@ def test_forward_and_both_backward_targets():
     assert lib.e3j_amd_xla_convolution_bwd_receiver(C.addressof(frame)) is None, xla.errors
     check(dx, dy, ds, "receiver grouping")
     del empty, keep
+
+
+def test_ordered_backward_target_with_a_signature_and_scratch_result():
+    """"convolution_bwd_ordered": the forward CSR, attributes `signature`/`coef_scale` from the
+    host-side lookup, and the scratch of the atomic-free backward as a fourth result."""
+    from e3j_amd import workloads as W
+    from e3j_amd.ops import _Table
+    w = W.config2(0.04)
+    m = w.module
+    packed = m._packed_coef("float32")
+    dims = (int(w.x.shape[1]), int(w.y.shape[1]), m.params.num_out, int(w.s.shape[1]))
+    sig, scale, _ = _Table.get(packed, np.float32).signature(dims, w.channels, m.layout)
+    assert sig >= 0
+    lib = _lib.load()
+    xla = FakeXla(stream=torch.cuda.current_stream().cuda_stream)
+    d = w.to("cuda")
+    n = w.num_nodes
+    ptr = dev(O.receiver_ptr(d.receiver.cpu().numpy(), n))
+    p = _lib.ConvParams(num_nodes=n, num_edges=w.num_edges, num_coef=packed.shape[0], num_x=dims[0],
+                        num_y=dims[1], num_out=dims[2], num_scalars=dims[3], channels=w.channels,
+                        layout=m.layout.value, val_dtype=_lib.F32, coef_idx_bytes=1, signature=sig,
+                        coef_scale=scale, debug=0, y_flip=0, row_order=None)
+    nbytes = int(lib.e3j_amd_convolution_bwd_ordered_workspace_bytes(C.byref(p)))
+    attrs = {"num_nodes": (S32, C.c_int32(n)), "debug": (S32, C.c_int32(0)),
+             "signature": (S32, C.c_int32(sig)), "coef_scale": (F32, C.c_float(scale))}
+    operands = [_buf(xla, dev(packed), U8), _buf(xla, d.x, F32), _buf(xla, d.y, F32), _buf(xla, d.s, F32),
+                _buf(xla, d.dm, F32), _buf(xla, d.sender, S32), _buf(xla, ptr, S32), xla.buffer(S32, 0, (0,))]
+
+    def run(workspace_bytes):
+        dx, dy, ds = (torch.full_like(t, float("nan")) for t in (d.x, d.y, d.s))
+        workspace = torch.empty(workspace_bytes, dtype=torch.uint8, device="cuda")
+        frame = xla.frame(operands, [_buf(xla, dx, F32), _buf(xla, dy, F32), _buf(xla, ds, F32),
+                                     _buf(xla, workspace, U8)], dict(attrs))
+        err = lib.e3j_amd_xla_convolution_bwd_ordered(C.addressof(frame))
+        torch.cuda.synchronize()
+        return err, (dx, dy, ds)
+
+    err, first = run(nbytes)
+    assert err is None, xla.errors
+    err, second = run(nbytes)
+    assert err is None
+    for a, b in zip(first, second):
+        assert torch.equal(a, b)                               # bit-reproducible
+    idx, val, mix = w.table()
+    a = w.numpy()
+    refs, mags = H.backward_reference(idx, val, mix, a["x"], a["y"], a["s"], a["sender"], a["receiver"], a["dm"])
+    for g, r, mg, name in zip(first, refs, mags, ("dx", "dy", "ds")):
+        H.assert_parity(g.cpu().numpy(), r, mg, f"ordered {name}")
+    err, _ = run(nbytes // 2)                                  # a scratch result that is too small
+    assert err is not None and "workspace" in xla.errors[-1][1]
