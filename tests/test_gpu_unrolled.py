@@ -231,3 +231,60 @@ def test_deterministic_backward_on_unsorted_edges():
         assert torch.equal(a, b)
     assert torch.equal(got[0], want[0])                      # same positions after the stable sort
     assert torch.equal(got[1], want[1][shuffle]) and torch.equal(got[2], want[2][shuffle])
+
+
+def test_kernel_entry_points_replay_from_a_captured_graph():
+    """The forward and backward entry points only enqueue kernels on the stream they are given
+    (zero fills included: no memset nodes), so a caller can record them into a HIP graph and
+    replay it.  Each replay, with other work and new operand values in between, must equal the
+    eager result of the same operands."""
+    import ctypes
+    from e3j_amd.graph import csr_row_ptr, locality_order
+    w = CASES["cfg2"]()
+    d = w.to("cuda")
+    m = w.module
+    table = _Table.get(m._packed_coef("float32"), np.float32)
+    sig, scale, _ = _signature_of(w)
+    ptr = csr_row_ptr(d.receiver, w.num_nodes)
+    order = locality_order(d.sender, ptr, w.num_nodes, 2)
+    lib = _lib.load()
+    p = _lib.ConvParams(num_nodes=w.num_nodes, num_edges=w.num_edges, num_coef=table.num_coef,
+                        num_x=int(d.x.shape[1]), num_y=16, num_out=m.params.num_out,
+                        num_scalars=int(d.s.shape[1]), channels=w.channels, layout=m.layout.value,
+                        val_dtype=_lib.F32, coef_idx_bytes=table.idx_bytes, signature=sig,
+                        coef_scale=scale, debug=0, y_flip=0, row_order=order.data_ptr())
+    coef = table.device(d.x.device)
+    x, y, s, dm = d.x.clone(), d.y.clone(), d.s.clone(), d.dm.clone()
+    out = torch.empty_like(dm)
+    dx, dy, ds = torch.empty_like(x), torch.empty_like(y), torch.empty_like(s)
+
+    def launch(stream):
+        _lib.check(lib.e3j_amd_convolution_fwd(ctypes.byref(p), coef.data_ptr(), x.data_ptr(), y.data_ptr(),
+                                               s.data_ptr(), d.sender.data_ptr(), ptr.data_ptr(), None,
+                                               out.data_ptr(), stream))
+        _lib.check(lib.e3j_amd_convolution_bwd_receiver(
+            ctypes.byref(p), coef.data_ptr(), x.data_ptr(), y.data_ptr(), s.data_ptr(), dm.data_ptr(),
+            d.sender.data_ptr(), ptr.data_ptr(), None, dx.data_ptr(), dy.data_ptr(), ds.data_ptr(), stream))
+
+    side = torch.cuda.Stream()
+    side.wait_stream(torch.cuda.current_stream())
+    with torch.cuda.stream(side):
+        launch(side.cuda_stream)                      # warm-up outside the capture
+    torch.cuda.current_stream().wait_stream(side)
+    torch.cuda.synchronize()
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph, stream=side):
+        launch(side.cuda_stream)
+    for trial in range(3):
+        gen = torch.Generator(device="cuda").manual_seed(100 + trial)
+        for t in (x, y, s, dm):
+            t.copy_(torch.randn(t.shape, device="cuda", generator=gen))
+        (x.sum() + s.sum()).item()                    # unrelated eager work and a synchronisation
+        graph.replay()
+        torch.cuda.synchronize()
+        replayed = [t.clone() for t in (out, dx, dy, ds)]
+        launch(torch.cuda.current_stream().cuda_stream)
+        torch.cuda.synchronize()
+        assert torch.equal(replayed[0], out) and torch.equal(replayed[3], ds), trial
+        for a, b in ((replayed[1], dx), (replayed[2], dy)):       # atomics: equal up to summation order
+            assert float((a - b).abs().max()) <= 2e-5 * float(b.abs().max()), trial
