@@ -220,16 +220,22 @@ def _raw_backward(meta: _Meta, x, y, s, dm, sender, receiver, graph=None):
     lib = _lib.load()
     deterministic = config().deterministic
     table = meta.table
-    sender_rows = meta.ordering == GraphOrdering.SENDER
-    # deterministic: the atomic-free backward of the unrolled kernels on the forward's own rows
-    # (per-position dx rows summed in a fixed order); tables without such a kernel fall back
-    # to the table-driven kernel on sender rows, which owns dx
-    ordered = (deterministic and not sender_rows
-               and table.signature(*_shape(meta, x, y, s), meta.layout)[0] >= 0)
+    has_kernel = table.signature(*_shape(meta, x, y, s), meta.layout)[0] >= 0
     # SENDER ordering: the cotangents belong to the edges as given (dy[e], ds[e] come from
-    # dm[receiver(e)]), not to the reversed edges the forward walks, so the backward keeps the
-    # sender rows but gathers dm and owns dx (`src/e3j/ops/convolution.py:413-431`).
-    reuse = graph is not None and (not deterministic or ordered or sender_rows)
+    # dm[receiver(e)]), not to the reversed edges the forward walks
+    # (`src/e3j/ops/convolution.py:413-431`).  With an unrolled kernel for the table the edges
+    # are sorted by receiver on the device and the receiver-grouped backward runs on them
+    # (results land on the edges' own rows through the permutation); otherwise the
+    # table-driven kernel keeps the sender rows, gathers dm and owns dx.
+    sender_rows = meta.ordering == GraphOrdering.SENDER and not has_kernel
+    resort = meta.ordering in (GraphOrdering.NONE, GraphOrdering.SENDER) and not sender_rows
+    # deterministic: the atomic-free backward of the unrolled kernels on receiver rows
+    # (per-position dx rows summed in a fixed order); tables without such a kernel fall back
+    # to the table-driven kernel on sender rows
+    ordered = deterministic and has_kernel
+    forward_rows = meta.ordering != GraphOrdering.SENDER   # the forward's rows are receivers
+    reuse = graph is not None and (
+        (forward_rows and (not deterministic or ordered)) or sender_rows)
     if reuse:
         other, row_ptr, perm, order = graph
         group_receiver = not sender_rows
@@ -241,12 +247,12 @@ def _raw_backward(meta: _Meta, x, y, s, dm, sender, receiver, graph=None):
         elif deterministic and not ordered:
             perm, other, row_ptr = sort_edges(sender_l, receiver_l, n)
             group_receiver = False
-        elif meta.ordering == GraphOrdering.RECEIVER:
-            group_receiver, other, row_ptr, perm = True, sender_l.contiguous(), csr_row_ptr(receiver_l, n), None
-        else:
+        elif resort:
             perm, other, row_ptr = sort_edges(receiver_l, sender_l, n)
             group_receiver = True
-        order = graph[3] if graph is not None else _row_order(other, row_ptr, n)
+        else:
+            group_receiver, other, row_ptr, perm = True, sender_l.contiguous(), csr_row_ptr(receiver_l, n), None
+        order = (graph[3] if graph is not None and forward_rows else _row_order(other, row_ptr, n))
     p, table = _fill_params(meta, x, y, s, table, use_signature=group_receiver, row_order=order)
     args = (ctypes.byref(p), table.device(x.device).data_ptr(), x.data_ptr(), y.data_ptr(),
             s.data_ptr(), dm.data_ptr(), other.data_ptr(), row_ptr.data_ptr(),
