@@ -219,8 +219,12 @@ def main():
 
     xg, yg, sg = (t.detach().requires_grad_(True) for t in (w.x, w.y, w.s))
 
+    from e3j_amd.ops import clear_graph_cache
+
     def step():
-        # forward, then the VJP of (x, y, s) for the cotangent dm, as autograd runs them
+        # forward, then the VJP of (x, y, s) for the cotangent dm, as autograd runs them; the
+        # adjacency is prepared anew in every step (no reuse between steps)
+        clear_graph_cache()
         out = e3j_amd.convolution(coef, xg, yg, sg, w.sender, w.receiver, module.params,
                                   module.graph_ordering, layout=module.layout)
         grads = torch.autograd.grad(out, (xg, yg, sg), w.dm)

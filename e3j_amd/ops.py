@@ -18,6 +18,7 @@ from __future__ import annotations
 import ctypes
 import dataclasses
 import warnings
+import weakref
 
 import numpy as np
 import torch
@@ -180,8 +181,38 @@ def _row_order(other: torch.Tensor, row_ptr: torch.Tensor, n: int):
     return locality_order(other, row_ptr, n, rounds)
 
 
+#: adjacencies prepared for the index tensors seen last (the layers of a model, and the steps
+#: between two neighbour-list rebuilds, pass the same tensors): keyed by the identity and the
+#: in-place version of both tensors, dropped when either tensor dies.
+_GRAPH_CACHE: dict = {}
+_GRAPH_CACHE_SIZE = 8
+
+
+def clear_graph_cache() -> None:
+    """Forget the prepared adjacencies (the next call prepares its graph again)."""
+    _GRAPH_CACHE.clear()
+
+
 def _forward_graph(meta: _Meta, sender: torch.Tensor, receiver: torch.Tensor):
-    """CSR used by the forward kernel: `(other, row_ptr, perm, row_order)`."""
+    """CSR used by the forward kernel: `(other, row_ptr, perm, row_order)`, prepared once per
+    pair of index tensors."""
+    key = (id(sender), id(receiver), sender._version, receiver._version, meta.num_nodes,
+           meta.ordering, config().locality_rounds)
+    hit = _GRAPH_CACHE.get(key)
+    if hit is not None and hit[0]() is sender and hit[1]() is receiver:
+        return hit[2]
+    graph = _prepare_graph(meta, sender, receiver)
+    if len(_GRAPH_CACHE) >= _GRAPH_CACHE_SIZE:
+        _GRAPH_CACHE.pop(next(iter(_GRAPH_CACHE)))
+
+    def evict(_, key=key):
+        _GRAPH_CACHE.pop(key, None)
+
+    _GRAPH_CACHE[key] = (weakref.ref(sender, evict), weakref.ref(receiver, evict), graph)
+    return graph
+
+
+def _prepare_graph(meta: _Meta, sender: torch.Tensor, receiver: torch.Tensor):
     n = meta.num_nodes
     sender_l, receiver_l = wrap_global_index(sender, n), wrap_global_index(receiver, n)
     if meta.ordering == GraphOrdering.RECEIVER:

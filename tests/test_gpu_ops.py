@@ -285,3 +285,25 @@ def test_operator_errors():
         convolution(p["coef"], x, y, s, snd, rcv, p["params"], GraphOrdering.SENDER)
     with pytest.raises(TypeError, match="Cast the operands"):
         convolution(p["coef"], x.half(), y.half(), s.half(), snd, rcv, p["params"])
+
+
+def test_prepared_graph_is_reused_per_index_tensor_pair_and_follows_in_place_changes():
+    from e3j_amd import ops
+    p = _problem(8, N=20, E=200, K=16)
+    x, y, s = (dev(p[k]) for k in ("x", "y", "s"))
+    snd, rcv = dev(p["snd"]), dev(p["rcv"])
+    ops.clear_graph_cache()
+    first = convolution(p["coef"], x, y, s, snd, rcv, p["params"])
+    assert len(ops._GRAPH_CACHE) == 1
+    again = convolution(p["coef"], x, y, s, snd, rcv, p["params"])
+    assert len(ops._GRAPH_CACHE) == 1 and torch.equal(first, again)
+    # an in-place change of the senders must not be served from the cache
+    snd[:] = torch.roll(snd, 1)
+    changed = convolution(p["coef"], x, y, s, snd, rcv, p["params"])
+    ref, mag = H.forward_reference(p["idx"], p["val"], p["mix"], p["x"], p["y"], p["s"],
+                                   np.roll(p["snd"], 1), p["rcv"], p["params"].num_out)
+    H.assert_parity(changed.cpu().numpy(), ref, mag, "after in-place change")
+    del snd, rcv
+    import gc
+    gc.collect()
+    assert len(ops._GRAPH_CACHE) == 0                      # entries die with their tensors
