@@ -9,7 +9,7 @@ and fails if `e3j_amd/lib/libe3j_amd.so` has not been built.
 from .coef import Coef, Coef4D, resolve_val_dtype
 from .convolution import Convolution
 from .graph import DUMMY_INDEX, GraphCSR
-from .ops import (ConvolutionBatchingWarning, ConvolutionParams, CUDAConvolutionParams,
+from .ops import (ConvolutionBatchingWarning, ConvolutionParams, CUDAConvolutionParams, TableDrivenKernelWarning,
                   convolution, convolution_batched, convolution_bwd)
 from .options import Config, GraphOrdering, Layout, TensorProductNormalization, config
 from .scalar_mixing import ScalarMixing
@@ -20,6 +20,7 @@ Space = O3Space
 
 __all__ = [
     "Coef", "Coef4D", "Config", "Convolution", "ConvolutionBatchingWarning", "ConvolutionParams",
+    "TableDrivenKernelWarning",
     "CUDAConvolutionParams", "DUMMY_INDEX", "GraphCSR", "GraphOrdering", "Layout", "O3Irrep",
     "O3Space", "ScalarMixing", "Space", "TensorProduct", "TensorProductNormalization", "config",
     "convolution", "convolution_batched", "convolution_bwd", "resolve_val_dtype",

@@ -46,6 +46,12 @@ class ConvolutionBatchingWarning(UserWarning):
     """Emitted when the convolution is batched over graph adjacencies."""
 
 
+class TableDrivenKernelWarning(UserWarning):
+    """Emitted once per coefficient table that runs the table-driven kernels (no built-in
+    unrolled kernel and run-time compilation switched off): they are an order of magnitude
+    slower than the unrolled ones."""
+
+
 _VAL_DTYPES = {torch.float32: (_lib.F32, np.float32), torch.float64: (_lib.F64, np.float64)}
 
 
@@ -112,6 +118,13 @@ class _Table:
                 c = self.unpack()
                 if _jit.register(c.val, c.idx.astype(np.int64), dims, channels):
                     sig = find()
+            if sig < 0 and not jit and self.val_np_dtype == np.float32:
+                warnings.warn(
+                    f"no unrolled kernel is built for this coefficient table (x {dims[0]}, y {dims[1]}, "
+                    f"out {dims[2]}, paths {dims[3]}, {channels} channels, {layout.name.lower()}): the "
+                    "table-driven kernels serve it, an order of magnitude slower; config(jit=True) "
+                    "(or E3J_AMD_JIT=1) compiles unrolled kernels for it with hipcc on first use",
+                    TableDrivenKernelWarning, stacklevel=3)
             hit = self._signature[key] = (sig, float(scale.value), int(flip.value))
         return hit
 

@@ -10,6 +10,8 @@ if ROOT not in sys.path:
 
 def pytest_configure(config):
     config.addinivalue_line("markers", "gpu: needs an MI355X (runs the HIP kernels)")
+    # the random tables of the tests are meant to run the table-driven kernels
+    config.addinivalue_line("filterwarnings", "ignore::e3j_amd.ops.TableDrivenKernelWarning")
 
 
 def pytest_collection_modifyitems(config, items):

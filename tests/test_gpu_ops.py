@@ -307,3 +307,15 @@ def test_prepared_graph_is_reused_per_index_tensor_pair_and_follows_in_place_cha
     import gc
     gc.collect()
     assert len(ops._GRAPH_CACHE) == 0                      # entries die with their tensors
+
+
+def test_tables_without_an_unrolled_kernel_warn_once():
+    p = _problem(9, N=10, E=60, K=8)
+    x, y, s = (dev(p[k]) for k in ("x", "y", "s"))
+    snd, rcv = dev(p["snd"]), dev(p["rcv"])
+    with warnings.catch_warnings(record=True) as seen:
+        warnings.simplefilter("always")
+        convolution(p["coef"], x, y, s, snd, rcv, p["params"])
+        convolution(p["coef"], x, y, s, snd, rcv, p["params"])
+    hits = [w for w in seen if issubclass(w.category, e3j_amd.TableDrivenKernelWarning)]
+    assert len(hits) == 1 and "jit" in str(hits[0].message)
