@@ -288,3 +288,46 @@ def test_kernel_entry_points_replay_from_a_captured_graph():
         assert torch.equal(replayed[0], out) and torch.equal(replayed[3], ds), trial
         for a, b in ((replayed[1], dx), (replayed[2], dy)):       # atomics: equal up to summation order
             assert float((a - b).abs().max()) <= 2e-5 * float(b.abs().max()), trial
+
+
+@pytest.mark.parametrize("layout", ["TRAILING_CHANNELS", "LEADING_CHANNELS"])
+def test_padding_edges_with_poisoned_features_never_reach_the_results(layout):
+    """Padding edges (sender and/or receiver = INT32_MAX) may carry NaN/Inf features; nodes
+    without live edges and the padding rows of dy/ds must come out as exact zeros and no NaN may
+    leak into a neighbouring row (`tests/test_pallas_mosaic_gpu_convolution.py:1530-1563`,
+    `tests/test_convolution_jax_transforms.py:229-306`), here on the unrolled kernels."""
+    w = CASES["cfg2"]().with_layout(layout)
+    d = w.to("cuda")
+    m = w.module
+    coef = m._packed_coef("float32")
+    E, n = w.num_edges, w.num_nodes
+    snd, rcv = d.sender.clone(), d.receiver.clone()
+    y, s = d.y.clone(), d.s.clone()
+    tail = E - 40                                  # the last receivers' edges become padding
+    rcv[tail:] = e3j_amd.DUMMY_INDEX
+    snd[tail + 20:] = e3j_amd.DUMMY_INDEX          # half of them with a padding sender as well
+    inside = torch.arange(5, tail, 23, device="cuda")   # sender-only padding inside live rows
+    snd[inside] = e3j_amd.DUMMY_INDEX
+    poisoned = torch.cat([inside, torch.arange(tail, E, device="cuda")])
+    y[poisoned] = float("nan")
+    s[poisoned] = float("inf")
+    out = e3j_amd.convolution(coef, d.x, y, s, snd, rcv, m.params, m.graph_ordering, layout=m.layout)
+    dx, dy, ds = e3j_amd.convolution_bwd(coef, d.x, y, s, snd, rcv, d.dm, m.params, m.graph_ordering,
+                                         layout=m.layout)
+    with e3j_amd.config.use(deterministic=True):
+        dx2, dy2, ds2 = e3j_amd.convolution_bwd(coef, d.x, y, s, snd, rcv, d.dm, m.params, m.graph_ordering,
+                                                layout=m.layout)
+    for t in (out, dx, dy, ds, dx2, dy2, ds2):
+        assert torch.isfinite(t).all()
+    for g in (dy, ds, dy2, ds2):
+        assert not g[poisoned].any()
+    # same as the graph without those edges
+    keep = torch.ones(E, dtype=torch.bool, device="cuda")
+    keep[poisoned] = False
+    ref = e3j_amd.convolution(coef, d.x, d.y[keep].contiguous(), d.s[keep].contiguous(), d.sender[keep],
+                              d.receiver[keep], m.params, m.graph_ordering, layout=m.layout)
+    assert torch.equal(out, ref)
+    last_rows = d.receiver[tail:].unique()
+    emptied = [int(r) for r in last_rows if not bool((d.receiver[:tail] == r).any())]
+    for r in emptied:
+        assert not out[r].any()
