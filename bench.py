@@ -66,6 +66,10 @@ def parse_args():
                          "(a secondary figure; the headline keeps the random numbering)")
     ap.add_argument("--deterministic", action="store_true",
                     help="time the atomic-free (bit-reproducible) backward instead of the default one")
+    ap.add_argument("--access-floor", action="store_true",
+                    help="cfg3, 128 channels, trailing layout only: also time kernels that perform the "
+                         "memory accesses of the two passes without their arithmetic (reported under "
+                         "roofline.access_floor)")
     ap.add_argument("--calibrate-copy", action="store_true",
                     help="also run a 1 GiB device copy, the known-size kernel that hardware "
                          "traffic counters are scaled by")
@@ -147,6 +151,48 @@ class AbiCalls:
             w.s.data_ptr(), w.dm.data_ptr(), self.other.data_ptr(), self.ptr.data_ptr(),
             self.perm.data_ptr() if self.perm is not None else None,
             self.dx.data_ptr(), self.dy.data_ptr(), self.ds.data_ptr(), self._stream()))
+
+
+#: access patterns of `--access-floor`: name -> mask of e3j_amd/csrc/probe/access_pattern.hip
+#: (1 read s, 2 gather x, 4 write ds, 8 dx atomics, 16 write out, 32 read dm)
+ACCESS_PATTERNS = {
+    "read_s": 1,
+    "read_s+gather_x": 3,
+    "forward: read_s+gather_x+write_out": 19,
+    "write_ds": 4,
+    "read_s+write_ds": 5,
+    "read_s+write_ds+gather_x": 7,
+    "read_s+write_ds+gather_x+read_dm": 39,
+    "dx_atomics": 8,
+    "read_s+write_ds+gather_x+dx_atomics": 15,
+    "backward: read_s+write_ds+gather_x+dx_atomics+read_dm": 47,
+}
+
+
+def access_floor(torch, abi, steps: int) -> dict:
+    """Milliseconds of the passes' memory accesses without their arithmetic (a separate probe
+    library; the y reads, dy writes and zero fills of the real passes, under 2 % of their bytes,
+    are left out)."""
+    from e3j_amd import build as lib_build
+    if not os.path.exists(lib_build.PROBE_LIB_PATH):
+        raise RuntimeError(f"{lib_build.PROBE_LIB_PATH} is missing: run `python -m e3j_amd.build`")
+    probe = ctypes.CDLL(lib_build.PROBE_LIB_PATH)
+    fn = probe.e3j_amd_probe_access_pattern
+    fn.restype = ctypes.c_int
+    fn.argtypes = [ctypes.c_uint] + [ctypes.c_int] * 4 + [ctypes.c_void_p] * 9 + [ctypes.c_int] + [ctypes.c_void_p] * 2
+    w, p = abi.w, abi.params
+    sink = torch.zeros(1, dtype=torch.float32, device=w.x.device)
+    order = abi.order.data_ptr() if abi.order is not None else None
+    result = {}
+    for name, mask in ACCESS_PATTERNS.items():
+        def run():
+            rc = fn(mask, p.num_x, p.num_scalars, p.num_out, p.channels, w.x.data_ptr(), w.s.data_ptr(),
+                    w.dm.data_ptr(), abi.other.data_ptr(), abi.ptr.data_ptr(), order, abi.ds.data_ptr(),
+                    abi.dx.data_ptr(), abi.out.data_ptr(), w.num_nodes, sink.data_ptr(), abi._stream())
+            if rc != 0:
+                raise RuntimeError("the access-pattern probe covers cfg3 with 128 channels, trailing layout, only")
+        result[name] = round(time_events(torch, run, steps, 1), 4)
+    return result
 
 
 def time_events(torch, fn, steps: int, warmup: int) -> float:
@@ -305,6 +351,11 @@ def main():
                                       "algorithmic_bytes": bytes_["fwd_bwd"], "ms": fwd_ms + bwd_ms},
         },
     }
+    if args.access_floor:
+        if args.layout != "trailing" or abi.perm is not None:
+            print("--access-floor covers the receiver-sorted trailing layout only", file=sys.stderr)
+            return 2
+        result["roofline"]["access_floor"] = {"unit": "ms", **access_floor(torch, abi, args.steps)}
     if not args.no_cpu_baseline:
         result["cpu_baseline"] = cpu_baseline(w, args.cpu_seconds)
     print(json.dumps(result))

@@ -1,0 +1,140 @@
+// Measurement aid, not part of the operator library: kernels that perform the memory accesses
+// of the convolution passes (trailing-channels layout, one wave per receiver and slice of 64
+// channels, next edge prefetched) without their arithmetic.  The time such a kernel takes is what
+// the memory system needs for the access pattern alone; `bench.py --access-floor` runs them on
+// the operands of the benchmark workload and reports the times beside those of the real kernels.
+// Built into its own library (libe3j_amd_probe.so); nothing in the operators links against it.
+#include <hip/hip_runtime.h>
+
+#include <cstdint>
+
+namespace {
+
+constexpr unsigned kReadS = 1u;     // stream the S rows of s of every edge (non-temporal loads)
+constexpr unsigned kGatherX = 2u;   // gather the X rows of x[sender]
+constexpr unsigned kWriteDs = 4u;   // stream out S rows of ds per edge (non-temporal stores)
+constexpr unsigned kAtomicDx = 8u;  // X float-atomic row pieces into dx[sender]
+constexpr unsigned kWriteOut = 16u; // Z output rows per receiver (non-temporal stores)
+constexpr unsigned kReadDm = 32u;   // Z rows of dm per receiver (non-temporal loads)
+
+template <unsigned M, int NS, int NX, int NZ, int K>
+__global__ __launch_bounds__(256) void access_pattern_kernel(
+    const float *__restrict__ x, const float *__restrict__ s, const float *__restrict__ dm,
+    const int32_t *__restrict__ sender, const int32_t *__restrict__ row_ptr,
+    const int32_t *__restrict__ row_order, float *__restrict__ ds, float *__restrict__ dx,
+    float *__restrict__ out, int num_nodes, float *__restrict__ sink) {
+    constexpr int SLICES = K / 64;
+    // the work list is walked as the operator kernels walk it: every XCD (workgroups are dealt
+    // to the 8 XCDs round-robin) takes one contiguous eighth, rows in the caller's row order
+    const unsigned per_xcd = gridDim.x / 8;
+    const int64_t block = (int64_t)(blockIdx.x % 8) * per_xcd + blockIdx.x / 8;
+    const int64_t item = block * 4 + threadIdx.y;
+    if (item >= (int64_t)num_nodes * SLICES) return;
+    const int slice = (int)(item % SLICES), q = (int)(item / SLICES);
+    const int r = row_order ? row_order[q] : q;
+    const int c0 = slice * 64 + threadIdx.x;
+    float acc = 0.f;
+    if (M & kReadDm) {
+        const float *zr = dm + (int64_t)r * (NZ * K) + c0;
+#pragma unroll
+        for (int i = 0; i < NZ; i++) acc += __builtin_nontemporal_load(zr + i * K);
+    }
+    int e = row_ptr[r];
+    const int e1 = row_ptr[r + 1];
+    float sn[NS], xn[NX];
+    int snd_n = 0;
+    auto fetch = [&](int pos) {
+        if (M & kReadS) {
+            const float *sr = s + (int64_t)pos * (NS * K) + c0;
+#pragma unroll
+            for (int l = 0; l < NS; l++) sn[l] = __builtin_nontemporal_load(sr + l * K);
+        }
+        if (M & (kGatherX | kAtomicDx)) {
+            const int snd = sender[pos];
+            snd_n = (unsigned)snd < (unsigned)num_nodes ? snd : 0;
+        }
+        if (M & kGatherX) {
+            const float *xr = x + (int64_t)snd_n * (NX * K) + c0;
+#pragma unroll
+            for (int j = 0; j < NX; j++) xn[j] = xr[j * K];
+        }
+    };
+    if (e < e1) fetch(e);
+    while (e < e1) {
+        float sc[NS], xc[NX];
+#pragma unroll
+        for (int l = 0; l < NS; l++) sc[l] = (M & kReadS) ? sn[l] : 1.f;
+#pragma unroll
+        for (int j = 0; j < NX; j++) xc[j] = (M & kGatherX) ? xn[j] : 1.f;
+        const int snd = snd_n;
+        const int pos = e;
+        e++;
+        if (e < e1) fetch(e);
+        if (M & kWriteDs) {
+            float *dr = ds + (int64_t)pos * (NS * K) + c0;
+#pragma unroll
+            for (int l = 0; l < NS; l++) __builtin_nontemporal_store(sc[l] + xc[l % NX], dr + l * K);
+        } else {
+#pragma unroll
+            for (int l = 0; l < NS; l++) acc += sc[l];
+        }
+        if (M & kAtomicDx) {
+            float *dxr = dx + (int64_t)snd * (NX * K) + c0;
+#pragma unroll
+            for (int j = 0; j < NX; j++) unsafeAtomicAdd(dxr + j * K, xc[j] + sc[j % NS]);
+        } else {
+#pragma unroll
+            for (int j = 0; j < NX; j++) acc += xc[j];
+        }
+    }
+    if (M & kWriteOut) {
+        float *orow = out + (int64_t)r * (NZ * K) + c0;
+#pragma unroll
+        for (int i = 0; i < NZ; i++) __builtin_nontemporal_store(acc + (float)i, orow + i * K);
+    } else if (acc == 1.2345e30f) {
+        *sink = acc;  // never true for finite operands; keeps the loads alive
+    }
+}
+
+template <unsigned M>
+void launch(const float *x, const float *s, const float *dm, const int32_t *sender, const int32_t *row_ptr,
+            const int32_t *row_order, float *ds, float *dx, float *out, int num_nodes, float *sink,
+            hipStream_t stream) {
+    constexpr int K = 128;
+    const int blocks = ((num_nodes * (K / 64) + 3) / 4 + 7) / 8 * 8;
+    hipLaunchKernelGGL((access_pattern_kernel<M, 23, 16, 99, K>), dim3(blocks), dim3(64, 4), 0, stream, x, s, dm,
+                       sender, row_ptr, row_order, ds, dx, out, num_nodes, sink);
+}
+
+}  // namespace
+
+// Runs the access pattern `mask` (bits: 1 read s, 2 gather x, 4 write ds, 8 dx atomics, 16 write
+// out, 32 read dm) once on `stream`.  Shapes are those of the 128-channel l<=3 benchmark
+// workload only: s, ds (E, 23, 128); x, dx (N, 16, 128); dm, out (N, 99, 128); row_ptr (N + 1);
+// row_order (N) or null for rows in index order.
+// Buffers of accesses that the mask leaves out may be null; `sink` is one float of scratch.
+// Returns 0, or -1 for a mask that has no instantiation or shapes other than the above.
+extern "C" int e3j_amd_probe_access_pattern(unsigned mask, int num_x, int num_scalars, int num_out, int channels,
+                                            const float *x, const float *s, const float *dm,
+                                            const int32_t *sender, const int32_t *row_ptr,
+                                            const int32_t *row_order, float *ds, float *dx, float *out,
+                                            int num_nodes, float *sink, hipStream_t stream) {
+    if (num_x != 16 || num_scalars != 23 || num_out != 99 || channels != 128 || num_nodes <= 0) return -1;
+#define E3J_PROBE_CASE(M) \
+    case (M): launch<(M)>(x, s, dm, sender, row_ptr, row_order, ds, dx, out, num_nodes, sink, stream); break;
+    switch (mask) {
+        E3J_PROBE_CASE(kReadS)
+        E3J_PROBE_CASE(kReadS | kGatherX)
+        E3J_PROBE_CASE(kReadS | kGatherX | kWriteOut)
+        E3J_PROBE_CASE(kReadS | kWriteDs)
+        E3J_PROBE_CASE(kReadS | kWriteDs | kGatherX)
+        E3J_PROBE_CASE(kReadS | kWriteDs | kGatherX | kAtomicDx)
+        E3J_PROBE_CASE(kReadS | kWriteDs | kGatherX | kAtomicDx | kReadDm)
+        E3J_PROBE_CASE(kReadS | kWriteDs | kGatherX | kReadDm)
+        E3J_PROBE_CASE(kAtomicDx)
+        E3J_PROBE_CASE(kWriteDs)
+        default: return -1;
+    }
+#undef E3J_PROBE_CASE
+    return hipGetLastError() == hipSuccess ? 0 : -1;
+}
