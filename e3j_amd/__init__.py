@@ -1,7 +1,8 @@
 """MI355X-native fused equivariant message-passing convolution.
 
 Public names follow the reference package for this path: `Convolution`,
-`convolution`, `convolution_bwd`, `GraphCSR`, `Coef4D`, `O3Space`, `config`.
+`convolution`, `convolution_bwd`, `tensor_product`, `tensor_product_bwd`, `GraphCSR`,
+`Coef4D`, `O3Space`, `config`.
 Importing the package does not load the kernel library; the first operator call does,
 and fails if `e3j_amd/lib/libe3j_amd.so` has not been built.
 """
@@ -11,10 +12,11 @@ from .convolution import Convolution
 from .graph import DUMMY_INDEX, GraphCSR
 from .ops import (ConvolutionBatchingWarning, ConvolutionParams, CUDAConvolutionParams, TableDrivenKernelWarning,
                   convolution, convolution_batched, convolution_bwd)
-from .options import Config, GraphOrdering, Layout, TensorProductNormalization, config
+from .options import Config, GraphOrdering, Layout, MixingMode, TensorProductNormalization, config
 from .scalar_mixing import ScalarMixing
 from .spaces import O3Irrep, O3Space
 from .tensor_product import TensorProduct
+from .tp_ops import CUDATensorProductParams, TensorProductParams, tensor_product, tensor_product_bwd
 
 Space = O3Space
 
@@ -24,4 +26,5 @@ __all__ = [
     "CUDAConvolutionParams", "DUMMY_INDEX", "GraphCSR", "GraphOrdering", "Layout", "O3Irrep",
     "O3Space", "ScalarMixing", "Space", "TensorProduct", "TensorProductNormalization", "config",
     "convolution", "convolution_batched", "convolution_bwd", "resolve_val_dtype",
+    "CUDATensorProductParams", "MixingMode", "TensorProductParams", "tensor_product", "tensor_product_bwd",
 ]

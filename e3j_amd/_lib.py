@@ -43,6 +43,29 @@ class ConvParams(ctypes.Structure):
     ]
 
 
+MODE_OUTER, MODE_INNER, MODE_MAP = 0, 1, 2
+
+
+class TpParams(ctypes.Structure):
+    """`e3j_amd_tp_params`."""
+
+    _fields_ = [
+        ("num_rows", ctypes.c_int64),
+        ("num_coef", ctypes.c_int32),
+        ("num_x", ctypes.c_int32),
+        ("num_y", ctypes.c_int32),
+        ("num_out", ctypes.c_int32),
+        ("channels_x", ctypes.c_int32),
+        ("channels_y", ctypes.c_int32),
+        ("mode", ctypes.c_int32),
+        ("layout", ctypes.c_int32),
+        ("val_dtype", ctypes.c_int32),
+        ("coef_idx_bytes", ctypes.c_int32),
+        ("coef_sorted", ctypes.c_int32),
+        ("debug", ctypes.c_int32),
+    ]
+
+
 class E3jAmdError(RuntimeError):
     """Failure reported by the kernel library; `.code` is the status code."""
 
@@ -53,6 +76,7 @@ class E3jAmdError(RuntimeError):
 
 _P = ctypes.c_void_p
 _PARAMS = ctypes.POINTER(ConvParams)
+_TP_PARAMS = ctypes.POINTER(TpParams)
 
 #: name -> (restype, argtypes): every symbol `include/e3j_amd.h` declares.
 SYMBOLS = {
@@ -77,6 +101,8 @@ SYMBOLS = {
     "e3j_amd_harmonics_bwd": (ctypes.c_int, [_P, _P, ctypes.c_int64] + [ctypes.c_int32] * 4 + [_P, _P]),
     "e3j_amd_wrap_index": (ctypes.c_int, [_P, ctypes.c_int64, ctypes.c_int32, _P, _P]),
     "e3j_amd_locality_order": (ctypes.c_int, [_P, _P, ctypes.c_int32, ctypes.c_int32, _P, _P, _P]),
+    "e3j_amd_tensor_product_fwd": (ctypes.c_int, [_TP_PARAMS] + [_P] * 5),
+    "e3j_amd_tensor_product_bwd": (ctypes.c_int, [_TP_PARAMS] + [_P] * 7),
     "e3j_amd_xla_convolution": (_P, [_P]),
     "e3j_amd_xla_convolution_bwd": (_P, [_P]),
     "e3j_amd_xla_convolution_bwd_receiver": (_P, [_P]),

@@ -56,6 +56,19 @@ class GraphOrdering(_ParsedEnum):
     NONE = "NONE"
 
 
+class MixingMode(_ParsedEnum):
+    """How a bilinear product mixes the channel axes (`src/e3j/utils/options.py:154-168`).
+
+    OUTER: `u, v -> (u, v)` (also broadcasts an operand without channel axis); INNER:
+    `v, v -> 1`; MAP: `v, v -> v`.  The integer values are the ones the reference hands to
+    its FFI.
+    """
+
+    OUTER = 0
+    INNER = 1
+    MAP = 2
+
+
 class TensorProductNormalization(_ParsedEnum):
     """Scaling of the stacked Clebsch-Gordan blocks (`src/e3j/utils/options.py:171-180`)."""
 

@@ -1,10 +1,10 @@
-"""Host-side construction of the stacked Clebsch-Gordan coefficient table.
+"""The stacked Clebsch-Gordan coefficient table and its row-wise evaluation.
 
-Only the parts of the reference's `TensorProduct` that the fused convolution
-consumes are here: selection rules, block stacking and the canonical sort of
-output blocks (`src/e3j/core/tensor_product.py:169-274`,
-`src/e3j/core/permutation.py:55-74`).  Evaluating a stand-alone tensor
-product is a different operator and is not part of this package.
+Host side: selection rules, block stacking and the canonical sort of output blocks
+(`src/e3j/core/tensor_product.py:169-274`, `src/e3j/core/permutation.py:55-74`), which
+the fused convolution consumes.  Calling a `TensorProduct` evaluates the bilinear map
+row by row with the fused HIP kernels of `e3j_amd.tp_ops`
+(`src/e3j/core/tensor_product.py:322-343,404-420`).
 """
 
 from __future__ import annotations
@@ -14,7 +14,7 @@ import itertools
 import numpy as np
 
 from .clebsch_gordan import clebsch_gordan
-from .options import Layout, TensorProductNormalization, config as _config
+from .options import Layout, MixingMode, TensorProductNormalization, config as _config
 from .sparse import SparseCOO, sparse_coo
 from .spaces import O3Space
 
@@ -39,13 +39,14 @@ class TensorProduct:
     r"""Coefficients of the bilinear map `z_i = \sum_{jk} c_{ijk} x_j y_k`."""
 
     def __init__(self, source, target=None, coef: SparseCOO | None = None, sort: bool = True,
-                 config=None, layout=Layout.LEADING_CHANNELS,
+                 config=None, layout=Layout.LEADING_CHANNELS, mode=MixingMode.OUTER,
                  normalization=TensorProductNormalization.NONE):
         if len(source) != 2:
             raise TypeError("TensorProduct expects a binary tuple as source argument.")
         self.source = tuple(O3Space(s) for s in source)
         self.config = _config.snapshot(config)
         self.layout = Layout.parse(layout)
+        self.mode = MixingMode.parse(mode)
         self.normalization = TensorProductNormalization.parse(normalization)
         infer = coef is None
         if target is None:
@@ -93,8 +94,27 @@ class TensorProduct:
         idx = self.indices.astype(np.int64)
         idx = np.concatenate((sigma_inv[idx[:, 0]][:, None], idx[:, 1:]), axis=-1)
         return TensorProduct(self.source, target, coef=sparse_coo(self.values, idx, self.shape),
-                             sort=False, config=self.config, layout=self.layout,
+                             sort=False, config=self.config, layout=self.layout, mode=self.mode,
                              normalization=self.normalization)
+
+    # --- evaluation ------------------------------------------------------
+    def packed_coef(self, val_dtype="float32") -> np.ndarray:
+        """The table in the operator's wire format (`src/e3j/core/tensor_product.py:340-343`)."""
+        from .coef import Coef
+        idx = self.indices
+        return Coef(self.values, idx, val_dtype=val_dtype, idx_dtype=idx.dtype).pack()
+
+    def __call__(self, x, y):
+        """Evaluate the bilinear map on GPU tensors with the fused HIP kernels (the
+        counterpart of the reference's `FUSED_CUDA` branch,
+        `src/e3j/core/tensor_product.py:322-343`); there is no other evaluation strategy."""
+        import torch
+        from .coef import resolve_val_dtype
+        from .tp_ops import TensorProductParams, tensor_product
+        dtype = torch.result_type(x, y)
+        val_dtype = resolve_val_dtype(str(dtype).replace("torch.", ""))
+        params = TensorProductParams(num_out=self.target.dim, mode=self.mode, layout=self.layout)
+        return tensor_product(self.packed_coef(val_dtype), x.to(dtype), y.to(dtype), params)
 
     @staticmethod
     def clebsch_gordan(target, source_1, source_2,

@@ -1,0 +1,275 @@
+"""The fused row-wise tensor product operators: `tensor_product` and `tensor_product_bwd`.
+
+Same signatures, argument meaning and errors as the reference's primitives
+(`src/e3j/ops/tensor_product.py:50-145,276-326`), with tensors in GPU memory and the
+HIP library of this package behind them.  `tensor_product` is differentiable in
+`(x, y)` to any reverse-mode order: its backward is `tensor_product_bwd`, whose own
+backward is one `tensor_product_bwd` and two `tensor_product` calls
+(`src/e3j/ops/tensor_product.py:571-591`).
+
+Extensions over the reference's operator: any channel count (no power-of-two rule in
+the trailing layout), MAP mode served directly in the leading layout, and a fused
+backward in both layouts (the reference falls back to two forward products in the
+leading layout).
+"""
+
+from __future__ import annotations
+
+import ctypes
+import dataclasses
+
+import numpy as np
+import torch
+
+from . import _lib
+from .coef import Coef
+from .options import Layout, MixingMode, config
+
+_VAL_DTYPES = {torch.float32: (_lib.F32, np.float32), torch.float64: (_lib.F64, np.float64)}
+
+
+@dataclasses.dataclass
+class TensorProductParams:
+    """Static description of the operator (`src/e3j/ops/tensor_product.py:41-45`)."""
+
+    num_out: int
+    mode: str | MixingMode = MixingMode.OUTER
+    layout: str | Layout = Layout.LEADING_CHANNELS
+
+
+#: name used by code written against the reference
+CUDATensorProductParams = TensorProductParams
+
+
+def _is_sorted(first_column: np.ndarray) -> bool:
+    return bool(np.all(np.diff(first_column.astype(np.int64)) >= 0))
+
+
+class _Table:
+    """A packed rank-3 coefficient table, its two transposes and their device copies."""
+
+    _cache: dict = {}
+
+    def __init__(self, packed: np.ndarray, val_np_dtype):
+        self.packed = np.ascontiguousarray(packed)
+        self.idx_bytes = self.packed.dtype.itemsize
+        self.val_np_dtype = np.dtype(val_np_dtype)
+        self.num_coef = int(self.packed.shape[0])
+        c = Coef.unpack(self.packed, self.val_np_dtype)
+        self.sorted = _is_sorted(c.idx[:, 0]) if self.num_coef else True
+        # dx and dy tables: columns (j, i, k) and (k, i, j), stable-sorted by the new first
+        # column (src/e3j/ops/tensor_product.py:331-338); always sorted, whatever the input
+        self.packed_bwd = np.ascontiguousarray(np.stack(
+            [c.transpose((1, 0, 2)).pack(), c.transpose((2, 0, 1)).pack()]))
+        self._device = {}
+
+    @classmethod
+    def get(cls, coef, val_np_dtype) -> "_Table":
+        if isinstance(coef, torch.Tensor):
+            raise TypeError("`coef` must be concrete: it is read on the host.")
+        packed = np.asarray(coef)
+        if packed.dtype not in (np.dtype(np.uint8), np.dtype(np.int32)):
+            raise TypeError(f"unsupported coefficient index dtype {packed.dtype}")
+        key = (packed.dtype.str, packed.shape, packed.tobytes(), np.dtype(val_np_dtype).str)
+        table = cls._cache.get(key)
+        if table is None:
+            if len(cls._cache) > 256:
+                cls._cache.clear()
+            table = cls._cache[key] = cls(packed, val_np_dtype)
+        return table
+
+    def device(self, device: torch.device, backward: bool = False) -> torch.Tensor:
+        key = (device, backward)
+        t = self._device.get(key)
+        if t is None:
+            host = self.packed_bwd if backward else self.packed
+            t = torch.from_numpy(host.view(np.uint8).reshape(-1).copy()).to(device)
+            self._device[key] = t
+        return t
+
+
+@dataclasses.dataclass
+class _Meta:
+    """Everything static about one call."""
+
+    table: _Table
+    num_out: int
+    mode: MixingMode
+    layout: Layout
+    has_cx: bool
+    has_cy: bool
+
+    def dims(self, t: torch.Tensor, has_c: bool):
+        """`(dim, channels)` of an operand."""
+        if not has_c:
+            return int(t.shape[1]), 1
+        if self.layout == Layout.TRAILING_CHANNELS:
+            return int(t.shape[1]), int(t.shape[2])
+        return int(t.shape[2]), int(t.shape[1])
+
+    def out_shape(self, rows: int, cx: int, cy: int):
+        if self.mode == MixingMode.INNER:
+            chans = []
+        elif self.mode == MixingMode.MAP:
+            chans = [cx]
+        else:
+            chans = ([cx] if self.has_cx else []) + ([cy] if self.has_cy else [])
+        if self.layout == Layout.TRAILING_CHANNELS:
+            return (rows, self.num_out, *chans)
+        return (rows, *chans, self.num_out)
+
+
+def _stream(device) -> int:
+    return int(torch.cuda.current_stream(device).cuda_stream)
+
+
+def _params(meta: _Meta, x: torch.Tensor, y: torch.Tensor, backward: bool) -> _lib.TpParams:
+    num_x, cx = meta.dims(x, meta.has_cx)
+    num_y, cy = meta.dims(y, meta.has_cy)
+    return _lib.TpParams(
+        num_rows=int(x.shape[0]), num_coef=meta.table.num_coef, num_x=num_x, num_y=num_y,
+        num_out=meta.num_out, channels_x=cx, channels_y=cy, mode=meta.mode.value, layout=meta.layout.value,
+        val_dtype=_VAL_DTYPES[x.dtype][0], coef_idx_bytes=meta.table.idx_bytes,
+        coef_sorted=1 if (backward or meta.table.sorted) else 0, debug=int(config().debug_level))
+
+
+def _raw_forward(meta: _Meta, x: torch.Tensor, y: torch.Tensor) -> torch.Tensor:
+    x, y = x.contiguous(), y.contiguous()
+    p = _params(meta, x, y, backward=False)
+    z = torch.empty(meta.out_shape(int(x.shape[0]), p.channels_x, p.channels_y), dtype=x.dtype, device=x.device)
+    lib = _lib.load()
+    with torch.cuda.device(x.device):
+        _lib.check(lib.e3j_amd_tensor_product_fwd(
+            ctypes.byref(p), meta.table.device(x.device).data_ptr(), x.data_ptr(), y.data_ptr(), z.data_ptr(),
+            _stream(x.device)))
+    return z
+
+
+def _raw_backward(meta: _Meta, x: torch.Tensor, y: torch.Tensor, dz: torch.Tensor):
+    x, y, dz = x.contiguous(), y.contiguous(), dz.contiguous()
+    p = _params(meta, x, y, backward=True)
+    if tuple(dz.shape) != meta.out_shape(int(x.shape[0]), p.channels_x, p.channels_y):
+        raise ValueError(f"cotangent shape {tuple(dz.shape)} does not match the output of the product")
+    dx, dy = torch.empty_like(x), torch.empty_like(y)
+    lib = _lib.load()
+    with torch.cuda.device(x.device):
+        _lib.check(lib.e3j_amd_tensor_product_bwd(
+            ctypes.byref(p), meta.table.device(x.device, backward=True).data_ptr(), x.data_ptr(), y.data_ptr(),
+            dz.data_ptr(), dx.data_ptr(), dy.data_ptr(), _stream(x.device)))
+    return dx, dy
+
+
+def _sum(*terms):
+    terms = [t for t in terms if t is not None]
+    if not terms:
+        return None
+    total = terms[0]
+    for t in terms[1:]:
+        total = total + t
+    return total
+
+
+class _TensorProduct(torch.autograd.Function):
+    @staticmethod
+    def forward(ctx, x, y, meta):
+        ctx.meta = meta
+        ctx.save_for_backward(x, y)
+        return _raw_forward(meta, x, y)
+
+    @staticmethod
+    def backward(ctx, dz):
+        x, y = ctx.saved_tensors
+        meta = ctx.meta
+        if meta.mode == MixingMode.OUTER and meta.has_cx and meta.has_cy:
+            raise NotImplementedError("Cannot backpropagate through 'OUTER' tensor product "
+                                      "with channel axes on both inputs.")
+        dx, dy = _TensorProductBwd.apply(x, y, dz, meta)
+        return dx, dy, None
+
+
+class _TensorProductBwd(torch.autograd.Function):
+    @staticmethod
+    def forward(ctx, x, y, dz, meta):
+        ctx.meta = meta
+        ctx.save_for_backward(x, y, dz)
+        return _raw_backward(meta, x, y, dz)
+
+    @staticmethod
+    def backward(ctx, ddx, ddy):
+        # (dx, dy) is bilinear in (dz, y) and (dz, x): cotangents of x, y through one backward
+        # product in (ddx, ddy), of dz through two forward products
+        # (src/e3j/ops/tensor_product.py:576-591)
+        x, y, dz = ctx.saved_tensors
+        meta = ctx.meta
+        ddx = torch.zeros_like(x) if ddx is None else ddx
+        ddy = torch.zeros_like(y) if ddy is None else ddy
+        gx = gy = gdz = None
+        if ctx.needs_input_grad[0] or ctx.needs_input_grad[1]:
+            gx, gy = _TensorProductBwd.apply(ddx, ddy, dz, meta)
+        if ctx.needs_input_grad[2]:
+            gdz = _sum(_TensorProduct.apply(x, ddy, meta), _TensorProduct.apply(ddx, y, meta))
+        return gx, gy, gdz, None
+
+
+def _check(x: torch.Tensor, y: torch.Tensor):
+    for name, t in (("x", x), ("y", y)):
+        if not isinstance(t, torch.Tensor):
+            raise TypeError(f"`{name}` must be a torch tensor")
+        if t.ndim not in (2, 3):
+            raise ValueError(f"Expected {name} rank 2 or 3, got {tuple(t.shape)}")
+    if x.dtype != y.dtype:
+        raise TypeError(f"x and y must share a dtype, got {x.dtype} and {y.dtype}")
+    if x.dtype not in _VAL_DTYPES:
+        raise NotImplementedError(f"the HIP tensor product runs in float32 or float64, got {x.dtype}")
+    if not x.is_cuda or x.device != y.device:
+        raise ValueError("x and y must live on the same GPU: the tensor product has no CPU path")
+    if x.shape[0] != y.shape[0]:
+        raise ValueError(f"x and y must have as many rows, got {x.shape[0]} and {y.shape[0]}")
+
+
+def _make_meta(coef, x, y, params: TensorProductParams) -> _Meta:
+    layout = Layout.parse(params.layout)
+    mode = MixingMode.parse(params.mode)
+    has_cx, has_cy = x.ndim > 2, y.ndim > 2
+    meta = _Meta(table=_Table.get(coef, _VAL_DTYPES[x.dtype][1]), num_out=int(params.num_out), mode=mode,
+                 layout=layout, has_cx=has_cx, has_cy=has_cy)
+    _, cx = meta.dims(x, has_cx)
+    _, cy = meta.dims(y, has_cy)
+    if mode != MixingMode.OUTER:
+        if not (has_cx and has_cy):
+            raise ValueError(f"{mode.name} mode requires channel dims on both x and y")
+        if cx != cy:
+            raise ValueError("MAP and INNER modes require same number of LHS and RHS channels. "
+                             f"Got ({cx, cy}).")
+    return meta
+
+
+def tensor_product(coef, x: torch.Tensor, y: torch.Tensor, params: TensorProductParams) -> torch.Tensor:
+    """Contraction of the sparse 3-D coefficient table with `x` and `y`, row by row.
+
+    Args:
+        coef: packed `Coef` table `(val, i, j, k)` (host numpy array, opaque index dtype).
+        x: `(rows, num_x, channels_x)` or `(rows, num_x)` [leading layout: `(rows, channels_x, num_x)`].
+        y: `(rows, num_y, channels_y)` or `(rows, num_y)` [leading: `(rows, channels_y, num_y)`].
+        params: `TensorProductParams(num_out, mode, layout)`.
+
+    Returns `(rows, num_out, *channels_z)` [leading: `(rows, *channels_z, num_out)`] with
+    `channels_z` = the channel axes of x then y (OUTER), none (INNER), the shared one (MAP).
+    """
+    _check(x, y)
+    meta = _make_meta(coef, x, y, params)
+    return _TensorProduct.apply(x, y, meta)
+
+
+def tensor_product_bwd(coef, x: torch.Tensor, y: torch.Tensor, ct_z: torch.Tensor, params: TensorProductParams):
+    """Cotangents `(ct_x, ct_y)` of `tensor_product` for the output cotangent `ct_z`; the
+    cotangent is read by one call for both results."""
+    _check(x, y)
+    meta = _make_meta(coef, x, y, params)
+    if meta.mode == MixingMode.OUTER and meta.has_cx and meta.has_cy:
+        raise NotImplementedError("The `tensor_product_bwd` handler requires either LHS or RHS to have one "
+                                  f"channel for now, got ({meta.dims(x, True)[1], meta.dims(y, True)[1]}).")
+    return _TensorProductBwd.apply(x, y, ct_z, meta)
+
+
+tensor_product.Params = TensorProductParams

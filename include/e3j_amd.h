@@ -205,6 +205,51 @@ int e3j_amd_harmonics_bwd(const void *vec, const void *dout, int64_t num, int32_
                           int32_t normalize, int32_t normalization, int32_t val_dtype, void *dvec,
                           void *stream);
 
+/* Row-wise sparse tensor product, the edge-wise sibling of the convolution (no gather, no
+ * scatter): z[r] = sum_n val_n x[r, j_n] (*) y[r, k_n] -> z[r, i_n].  Operands and sizes of the
+ * reference's "tensor_product" / "tensor_product_bwd" targets (lib/e3j_ops/ffi/e3j_ops.h:124-253,
+ * :258-372; Params of lib/e3j_ops/cuda/tensor_product.cuh:58-95) minus `coef_ranges`.
+ * Channel modes (src/e3j/utils/options.py:154-168):
+ *   OUTER z[r, i, cx, cy] = x[r, j, cx] y[r, k, cy]; an operand without channel axis has channels 1
+ *   INNER z[r, i]         = sum_c x[r, j, c] y[r, k, c]
+ *   MAP   z[r, i, c]      = x[r, j, c] y[r, k, c]
+ * TRAILING layout: x (R, X, Cx), y (R, Y, Cy), z (R, Z, Cx, Cy) / (R, Z) / (R, Z, C);
+ * LEADING layout: x (R, Cx, X), y (R, Cy, Y), z (R, Cx, Cy, Z) / (R, Z) / (R, C, Z).
+ * `coef` is the packed table {val; i; j; k} of lib/e3j_ops/cuda/tensor_product.cuh:98-111 in
+ * device memory (8, 16, 16, 32 bytes per entry for uint8/float32, int32/float32,
+ * uint8/float64, int32/float64).  Any channel count is accepted (the reference requires powers
+ * of two in the trailing layout, e3j_ops.h:168-185). */
+enum { E3J_AMD_MODE_OUTER = 0, E3J_AMD_MODE_INNER = 1, E3J_AMD_MODE_MAP = 2 };
+typedef struct e3j_amd_tp_params {
+    int64_t num_rows;
+    int32_t num_coef;
+    int32_t num_x;
+    int32_t num_y;
+    int32_t num_out;
+    int32_t channels_x;
+    int32_t channels_y;
+    int32_t mode;           /* E3J_AMD_MODE_* of the forward pass */
+    int32_t layout;         /* E3J_AMD_LAYOUT_* */
+    int32_t val_dtype;      /* E3J_AMD_F32 / E3J_AMD_F64 */
+    int32_t coef_idx_bytes; /* 1 or 4 */
+    /* != 0: entries with equal output index are contiguous and the output indices ascend (the
+     * order sparse_coo and Coef.transpose produce, src/e3j/utils/sparse.py:76-126,
+     * src/e3j/ops/coef.py:174-184); every output coordinate is then written once.  0: any
+     * order; the result is zero-filled first and runs are added. */
+    int32_t coef_sorted;
+    int32_t debug;
+} e3j_amd_tp_params;
+int e3j_amd_tensor_product_fwd(const e3j_amd_tp_params *p, const void *coef, const void *x, const void *y,
+                               void *z, void *stream);
+/* Cotangents dx (shape of x) and dy (shape of y) for the output cotangent dz.  `coef_bwd` holds
+ * two tables of num_coef entries each, the forward table with its index columns permuted to
+ * (j, i, k) and to (k, i, j) and sorted by the new first column
+ * (src/e3j/ops/tensor_product.py:331-338); `p` describes the forward pass.  Coordinates of x or y
+ * that no coefficient touches get zeros.  OUTER mode needs channels_x == 1 or channels_y == 1
+ * (as the reference, src/e3j/ops/tensor_product.py:322-326); both layouts are served. */
+int e3j_amd_tensor_product_bwd(const e3j_amd_tp_params *p, const void *coef_bwd, const void *x, const void *y,
+                               const void *dz, void *dx, void *dy, void *stream);
+
 /* XLA-FFI handlers (C ABI of xla/ffi/api/c_api.h): `XLA_FFI_Error* handler(XLA_FFI_CallFrame*)`.
  * Operand order of "convolution"/"convolution_bwd" as in lib/e3j_ops/ffi/e3j_ops.h:457-472,575-594;
  * attrs: num_nodes, debug (reference) + layout, signature (optional). */

@@ -52,6 +52,32 @@ def test_params_struct_matches_header():
     assert [ctype[t] for t, _ in fields] == [t for _, t in _lib.ConvParams._fields_]
 
 
+def test_tensor_product_params_struct_matches_header():
+    header = open(os.path.join(ROOT, "include", "e3j_amd.h")).read()
+    body = re.search(r"typedef struct e3j_amd_tp_params \{(.*?)\} e3j_amd_tp_params;", header, re.S).group(1)
+    fields = re.findall(r"^\s*(int32_t|int64_t)\s*(\w+);", body, re.M)
+    assert [name for _, name in fields] == [name for name, _ in _lib.TpParams._fields_]
+    ctype = {"int32_t": C.c_int32, "int64_t": C.c_int64}
+    assert [ctype[t] for t, _ in fields] == [t for _, t in _lib.TpParams._fields_]
+    modes = re.search(r"E3J_AMD_MODE_OUTER = (\d), E3J_AMD_MODE_INNER = (\d), E3J_AMD_MODE_MAP = (\d)", header)
+    assert tuple(map(int, modes.groups())) == (_lib.MODE_OUTER, _lib.MODE_INNER, _lib.MODE_MAP)
+
+
+def test_tensor_product_argument_errors_need_no_launch():
+    lib = _lib.load()
+    assert lib.e3j_amd_tensor_product_fwd(None, None, None, None, None, None) == _lib.INVALID_ARGUMENT
+    assert "null params" in lib.e3j_amd_last_error().decode()
+    p = _lib.TpParams(num_rows=0, num_coef=0, num_x=1, num_y=1, num_out=1, channels_x=1, channels_y=1,
+                      mode=_lib.MODE_OUTER, layout=_lib.LAYOUT_LEADING, val_dtype=_lib.F32, coef_idx_bytes=1)
+    assert lib.e3j_amd_tensor_product_fwd(C.byref(p), None, None, None, None, None) == _lib.OK   # no rows: a no-op
+    p.num_rows = 3
+    assert lib.e3j_amd_tensor_product_fwd(C.byref(p), None, None, None, None, None) == _lib.INVALID_ARGUMENT
+    assert "null operand" in lib.e3j_amd_last_error().decode()
+    p.mode = 9
+    assert lib.e3j_amd_tensor_product_bwd(C.byref(p), *[None] * 7) == _lib.INVALID_ARGUMENT
+    assert "unknown mode" in lib.e3j_amd_last_error().decode()
+
+
 @pytest.mark.parametrize("kw, code, needle", [
     (dict(layout=7), _lib.INVALID_ARGUMENT, "unknown layout"),
     (dict(channels=0), _lib.INVALID_ARGUMENT, "must be >= 1"),

@@ -1,0 +1,257 @@
+"""Row-wise tensor product on the GPU against the CPU checker: the grid of the reference's op
+tests (`tests/test_ops/test_tensor_product_op.py`: modes x channel counts x layouts, random
+table of 530 entries over 42 x 25 coordinates) plus dtypes, index widths, unsorted tables,
+uncovered coordinates, autograd to second order and the module-level call."""
+
+import ctypes
+
+import numpy as np
+import pytest
+import torch
+
+import e3j_amd
+from e3j_amd import TensorProduct, _lib
+from e3j_amd.coef import Coef
+from e3j_amd.tp_ops import TensorProductParams
+from oracle import tp_oracle as T
+from tests import helpers as H
+
+pytestmark = pytest.mark.gpu
+
+DEV = "cuda:0"
+MODES = ("OUTER", "INNER", "MAP")
+LAYOUTS = ("LEADING_CHANNELS", "TRAILING_CHANNELS")
+NUM_X, NUM_Y, NUM_OUT, NNZ = 42, 25, 30, 530
+
+
+def _table(seed=1234, nnz=NNZ, dims=(NUM_OUT, NUM_X, NUM_Y)):
+    idx, val, _ = H.random_table(np.random.default_rng(seed), nnz, dims[1], dims[2], dims[0], 3)
+    return idx, val.astype(np.float64)
+
+
+def _operands(rng, mode, layout, channels, rows=100, dims=(NUM_X, NUM_Y), dtype=np.float32, has=(True, True)):
+    tr = layout == "TRAILING_CHANNELS"
+    def make(dim, has_c):
+        if not has_c:
+            return rng.normal(size=(rows, dim)).astype(dtype)
+        return rng.normal(size=(rows, dim, channels) if tr else (rows, channels, dim)).astype(dtype)
+    if mode != "OUTER":
+        has = (True, True)
+    return make(dims[0], has[0]), make(dims[1], has[1])
+
+
+def _check_forward(idx, val, x, y, num_out, mode, layout, idx_dtype="int32", what=""):
+    coef = Coef(val, idx, str(x.dtype), idx_dtype).pack()
+    p = TensorProductParams(num_out=num_out, mode=mode, layout=layout)
+    z = e3j_amd.tensor_product(coef, torch.from_numpy(x).to(DEV), torch.from_numpy(y).to(DEV), p).cpu().numpy()
+    x64, y64 = x.astype(np.float64), y.astype(np.float64)
+    val_r = val.astype(x.dtype).astype(np.float64)    # the kernel sees the table rounded to the value dtype
+    ref = T.tensor_product_unfused(idx, val_r, x64, y64, num_out, mode, layout)
+    mag = T.tensor_product_unfused(idx, np.abs(val_r), np.abs(x64), np.abs(y64), num_out, mode, layout)
+    if x.dtype == np.float64:
+        np.testing.assert_allclose(z, ref, rtol=1e-12, atol=1e-12 * max(1.0, float(mag.max())))
+    else:
+        H.assert_parity(z, ref, mag, f"{what} z")
+    return z
+
+
+def _check_backward(idx, val, x, y, num_out, mode, layout, rng, idx_dtype="int32", what=""):
+    coef = Coef(val, idx, str(x.dtype), idx_dtype).pack()
+    p = TensorProductParams(num_out=num_out, mode=mode, layout=layout)
+    xt = torch.from_numpy(x).to(DEV).requires_grad_(True)
+    yt = torch.from_numpy(y).to(DEV).requires_grad_(True)
+    z = e3j_amd.tensor_product(coef, xt, yt, p)
+    dz = rng.normal(size=tuple(z.shape)).astype(x.dtype)
+    dx, dy = torch.autograd.grad(z, (xt, yt), torch.from_numpy(dz).to(DEV))
+    x64, y64, dz64 = (a.astype(np.float64) for a in (x, y, dz))
+    val_r = val.astype(x.dtype).astype(np.float64)
+    rdx, rdy = T.tensor_product_vjp(idx, val_r, x64, y64, dz64, mode, layout)
+    mdx, mdy = T.tensor_product_vjp(idx, np.abs(val_r), np.abs(x64), np.abs(y64), np.abs(dz64), mode, layout)
+    for got, ref, mag, name in ((dx, rdx, mdx, "dx"), (dy, rdy, mdy, "dy")):
+        got = got.cpu().numpy()
+        if x.dtype == np.float64:
+            np.testing.assert_allclose(got, ref, rtol=1e-12, atol=1e-12 * max(1.0, float(mag.max())))
+        else:
+            H.assert_parity(got, ref, mag, f"{what} {name}", ulps=32.0)
+
+
+@pytest.mark.parametrize("channels", [1, 2, 16, 32, 64, 128, 512])
+@pytest.mark.parametrize("mode", MODES)
+@pytest.mark.parametrize("layout", LAYOUTS)
+def test_forward_and_backward_grid(channels, mode, layout):
+    rng = np.random.default_rng(channels)
+    idx, val = _table()
+    x, y = _operands(rng, mode, layout, channels, has=(True, False))
+    _check_forward(idx, val, x, y, NUM_OUT, mode, layout, what=f"{mode} {layout} C={channels}")
+    _check_backward(idx, val, x, y, NUM_OUT, mode, layout, rng, what=f"{mode} {layout} C={channels}")
+
+
+@pytest.mark.parametrize("has", [(False, True), (False, False), (True, True)])
+@pytest.mark.parametrize("layout", LAYOUTS)
+def test_outer_mode_channel_axes(has, layout):
+    rng = np.random.default_rng(7)
+    idx, val = _table()
+    x, y = _operands(rng, "OUTER", layout, 8, rows=37, has=has)
+    if has == (True, True):    # different channel counts on the two sides
+        tr = layout == "TRAILING_CHANNELS"
+        y = rng.normal(size=(37, NUM_Y, 3) if tr else (37, 3, NUM_Y)).astype(np.float32)
+    _check_forward(idx, val, x, y, NUM_OUT, "OUTER", layout, what=f"OUTER {has}")
+    if has != (True, True):
+        _check_backward(idx, val, x, y, NUM_OUT, "OUTER", layout, rng, what=f"OUTER {has}")
+    else:
+        coef = Coef(val, idx, "float32", "int32").pack()
+        p = TensorProductParams(num_out=NUM_OUT, mode="OUTER", layout=layout)
+        xt = torch.from_numpy(x).to(DEV).requires_grad_(True)
+        z = e3j_amd.tensor_product(coef, xt, torch.from_numpy(y).to(DEV), p)
+        with pytest.raises(NotImplementedError, match="channel axes on both inputs"):
+            z.sum().backward()
+        with pytest.raises(NotImplementedError, match="one channel"):
+            e3j_amd.tensor_product_bwd(coef, xt, torch.from_numpy(y).to(DEV), z.detach(), p)
+
+
+@pytest.mark.parametrize("dtype", [np.float32, np.float64])
+@pytest.mark.parametrize("idx_dtype", ["uint8", "int32"])
+@pytest.mark.parametrize("mode", MODES)
+def test_dtypes_and_index_widths(dtype, idx_dtype, mode):
+    rng = np.random.default_rng(11)
+    idx, val = _table()
+    for layout in LAYOUTS:
+        x, y = _operands(rng, mode, layout, 24, rows=33, dtype=dtype, has=(True, False))
+        _check_forward(idx, val, x, y, NUM_OUT, mode, layout, idx_dtype, what=f"{mode} {dtype.__name__} {idx_dtype}")
+        _check_backward(idx, val, x, y, NUM_OUT, mode, layout, rng, idx_dtype)
+
+
+@pytest.mark.parametrize("mode", MODES)
+def test_clebsch_gordan_table_through_the_module(mode):
+    """`TensorProduct.__call__` on the full l <= 2 product (nnz 357) against the dense contraction."""
+    rng = np.random.default_rng(12)
+    for layout in LAYOUTS:
+        tp = TensorProduct(("0e+1o+2e", "0e+1o+2e"), None, layout=layout, mode=mode)
+        Z, X, Y = tp.shape
+        x, y = _operands(rng, mode, layout, 64, rows=50, dims=(X, Y), has=(True, False))
+        z = tp(torch.from_numpy(x).to(DEV), torch.from_numpy(y).to(DEV)).cpu().numpy()
+        idx, val = np.asarray(tp.indices, dtype=np.int64), np.asarray(tp.values, dtype=np.float64)
+        ref = T.tensor_product_unfused(idx, val, x.astype(np.float64), y.astype(np.float64), Z, mode, layout)
+        mag = T.tensor_product_unfused(idx, np.abs(val), np.abs(x).astype(np.float64), np.abs(y).astype(np.float64),
+                                       Z, mode, layout)
+        H.assert_parity(z, ref, mag, f"module {mode} {layout}")
+
+
+@pytest.mark.parametrize("mode", MODES)
+@pytest.mark.parametrize("layout", LAYOUTS)
+def test_unsorted_table_and_uncovered_coordinates(mode, layout):
+    """Entries in any order give the same result; output coordinates (and, in the backward pass,
+    input coordinates) that no entry touches are exact zeros, never stale memory
+    (`tests/test_ops/test_zero_gap_rows.py:15-26`)."""
+    rng = np.random.default_rng(13)
+    idx, val = _table(nnz=200)
+    keep = (idx[:, 0] != 3) & (idx[:, 0] != NUM_OUT - 1) & (idx[:, 1] != 5) & (idx[:, 2] != 0)
+    idx, val = idx[keep], val[keep]
+    x, y = _operands(rng, mode, layout, 16, rows=21, has=(True, False))
+    z_sorted = _check_forward(idx, val, x, y, NUM_OUT, mode, layout, what="gaps")
+    tr = layout == "TRAILING_CHANNELS"
+    zi = np.moveaxis(z_sorted, 1, -1) if tr and z_sorted.ndim > 2 else z_sorted
+    assert np.all(zi[..., 3] == 0) and np.all(zi[..., NUM_OUT - 1] == 0)
+    shuffle = rng.permutation(len(val))
+    z_any = _check_forward(idx[shuffle], val[shuffle], x, y, NUM_OUT, mode, layout, what="shuffled")
+    np.testing.assert_allclose(z_any, z_sorted, rtol=1e-5, atol=1e-5)
+    # backward: poison the results first, the gaps must come back as zeros
+    coef = Coef(val[shuffle], idx[shuffle], "float32", "int32").pack()
+    p = TensorProductParams(num_out=NUM_OUT, mode=mode, layout=layout)
+    xt, yt = torch.from_numpy(x).to(DEV), torch.from_numpy(y).to(DEV)
+    dz = torch.randn(tuple(z_sorted.shape), device=DEV)
+    poison = [torch.full_like(xt, float("nan")), torch.full_like(yt, float("nan"))]
+    torch.cuda.synchronize()
+    del poison          # the allocator hands these blocks to the results of the next call
+    dx, dy = e3j_amd.tensor_product_bwd(coef, xt, yt, dz, p)
+    dxi = dx.movedim(1, -1) if tr and dx.ndim > 2 else dx
+    dyi = dy.movedim(1, -1) if tr and dy.ndim > 2 else dy
+    assert torch.all(dxi[..., 5] == 0) and torch.all(dyi[..., 0] == 0)
+    assert torch.isfinite(dx).all() and torch.isfinite(dy).all()
+    _check_backward(idx[shuffle], val[shuffle], x, y, NUM_OUT, mode, layout, rng, what="shuffled")
+
+
+def _dense_torch(idx, val, num_out, dims, mode, layout, has):
+    dense = torch.zeros((num_out,) + dims, dtype=torch.float64, device=DEV)
+    dense.index_put_(tuple(torch.as_tensor(np.asarray(idx).T.astype(np.int64), device=DEV)),
+                     torch.as_tensor(val, dtype=torch.float64, device=DEV), accumulate=True)
+    tr = layout == "TRAILING_CHANNELS"
+
+    def f(x, y):
+        xl = x.transpose(1, 2) if tr and x.ndim == 3 else x
+        yl = y.transpose(1, 2) if tr and y.ndim == 3 else y
+        if mode == "MAP":
+            z = torch.einsum("ijk,rcj,rck->rci", dense, xl, yl)
+        elif mode == "INNER":
+            z = torch.einsum("ijk,rcj,rck->ri", dense, xl, yl)
+        else:
+            sx = "raj" if has[0] else "rj"
+            sy = "rbk" if has[1] else "rk"
+            so = "r" + ("a" if has[0] else "") + ("b" if has[1] else "") + "i"
+            z = torch.einsum(f"ijk,{sx},{sy}->{so}", dense, xl, yl)
+        return z.movedim(-1, 1) if tr and z.ndim > 2 else z
+    return f
+
+
+@pytest.mark.parametrize("mode,has", [("MAP", (True, True)), ("INNER", (True, True)), ("OUTER", (True, False)),
+                                      ("OUTER", (False, True))])
+@pytest.mark.parametrize("layout", LAYOUTS)
+def test_second_order_gradients_against_dense_autograd(mode, has, layout):
+    rng = np.random.default_rng(14)
+    idx, val = _table(nnz=90, dims=(9, 6, 5))
+    x, y = _operands(rng, mode, layout, 4, rows=6, dims=(6, 5), dtype=np.float64, has=has)
+    coef = Coef(val, idx, "float64", "int32").pack()
+    p = TensorProductParams(num_out=9, mode=mode, layout=layout)
+    dense = _dense_torch(idx, val, 9, (6, 5), mode, layout, has)
+
+    def run(fn):
+        xt = torch.from_numpy(x).to(DEV).requires_grad_(True)
+        yt = torch.from_numpy(y).to(DEV).requires_grad_(True)
+        z = fn(xt, yt)
+        g = torch.Generator(device="cpu").manual_seed(0)
+        dz = torch.randn(tuple(z.shape), generator=g, dtype=torch.float64).to(DEV).requires_grad_(True)
+        dx, dy = torch.autograd.grad(z, (xt, yt), dz, create_graph=True)
+        wx = torch.randn(tuple(dx.shape), generator=g, dtype=torch.float64).to(DEV)
+        wy = torch.randn(tuple(dy.shape), generator=g, dtype=torch.float64).to(DEV)
+        second = torch.autograd.grad((dx * wx).sum() + (dy * wy).sum(), (xt, yt, dz))
+        return [z, dx, dy, *second]
+
+    for a, b in zip(run(lambda u, v: e3j_amd.tensor_product(coef, u, v, p)), run(dense)):
+        torch.testing.assert_close(a, b, rtol=1e-11, atol=1e-11)
+
+
+def test_no_rows_and_repeatability():
+    idx, val = _table()
+    coef = Coef(val, idx, "float32", "uint8").pack()
+    p = TensorProductParams(num_out=NUM_OUT, mode="MAP", layout="TRAILING_CHANNELS")
+    z = e3j_amd.tensor_product(coef, torch.zeros(0, NUM_X, 8, device=DEV), torch.zeros(0, NUM_Y, 8, device=DEV), p)
+    assert tuple(z.shape) == (0, NUM_OUT, 8)
+    x, y = torch.randn(64, NUM_X, 32, device=DEV), torch.randn(64, NUM_Y, 32, device=DEV)
+    a = e3j_amd.tensor_product(coef, x, y, p)
+    b = e3j_amd.tensor_product(coef, x, y, p)
+    assert torch.equal(a, b)
+
+
+def test_c_abi_errors():
+    lib = _lib.load()
+    stream = int(torch.cuda.current_stream().cuda_stream)
+    buf = torch.zeros(4096, device=DEV)
+    def params(**kw):
+        base = dict(num_rows=2, num_coef=3, num_x=4, num_y=3, num_out=5, channels_x=8, channels_y=8,
+                    mode=_lib.MODE_MAP, layout=_lib.LAYOUT_TRAILING, val_dtype=_lib.F32, coef_idx_bytes=4,
+                    coef_sorted=1, debug=0)
+        base.update(kw)
+        return _lib.TpParams(**base)
+    def fwd(p):
+        return lib.e3j_amd_tensor_product_fwd(ctypes.byref(p), buf.data_ptr(), buf.data_ptr(), buf.data_ptr(),
+                                              buf.data_ptr(), stream)
+    assert lib.e3j_amd_tensor_product_fwd(None, None, None, None, None, None) == _lib.INVALID_ARGUMENT
+    assert fwd(params(mode=7)) == _lib.INVALID_ARGUMENT and b"unknown mode" in lib.e3j_amd_last_error()
+    assert fwd(params(channels_y=4)) == _lib.INVALID_ARGUMENT and b"same number" in lib.e3j_amd_last_error()
+    assert fwd(params(coef_idx_bytes=2)) == _lib.INVALID_ARGUMENT and b"dtype pair" in lib.e3j_amd_last_error()
+    assert fwd(params(layout=5)) == _lib.INVALID_ARGUMENT
+    assert fwd(params(mode=_lib.MODE_INNER, num_out=400, val_dtype=_lib.F64)) == _lib.UNIMPLEMENTED
+    p = params(mode=_lib.MODE_OUTER, channels_y=2)
+    rc = lib.e3j_amd_tensor_product_bwd(ctypes.byref(p), *[buf.data_ptr()] * 6, stream)
+    assert rc == _lib.UNIMPLEMENTED and b"one channel" in lib.e3j_amd_last_error()
+    torch.cuda.synchronize()
