@@ -63,6 +63,8 @@ class TpParams(ctypes.Structure):
         ("coef_idx_bytes", ctypes.c_int32),
         ("coef_sorted", ctypes.c_int32),
         ("debug", ctypes.c_int32),
+        ("signature", ctypes.c_int32),
+        ("coef_scale", ctypes.c_float),
     ]
 
 
@@ -103,6 +105,9 @@ SYMBOLS = {
     "e3j_amd_locality_order": (ctypes.c_int, [_P, _P, ctypes.c_int32, ctypes.c_int32, _P, _P, _P]),
     "e3j_amd_tensor_product_fwd": (ctypes.c_int, [_TP_PARAMS] + [_P] * 5),
     "e3j_amd_tensor_product_bwd": (ctypes.c_int, [_TP_PARAMS] + [_P] * 7),
+    "e3j_amd_tp_find_signature": (ctypes.c_int, [_P] + [ctypes.c_int32] * 8 + [ctypes.POINTER(ctypes.c_float)]),
+    "e3j_amd_tp_num_signatures": (ctypes.c_int, []),
+    "e3j_amd_tp_signature_name": (ctypes.c_char_p, [ctypes.c_int]),
     "e3j_amd_xla_convolution": (_P, [_P]),
     "e3j_amd_xla_convolution_bwd": (_P, [_P]),
     "e3j_amd_xla_convolution_bwd_receiver": (_P, [_P]),

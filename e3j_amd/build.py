@@ -55,8 +55,9 @@ def build(regenerate: bool = True, jobs: int | None = None, verbose: bool = True
     os.makedirs(OBJ_DIR, exist_ok=True)
     os.makedirs(GENERATED, exist_ok=True)
     if regenerate:
-        from .codegen import gen_conv
+        from .codegen import gen_conv, gen_tp
         gen_conv.write_all(GENERATED)
+        gen_tp.write_all(GENERATED)
     srcs = sources()
     extra = ["-save-temps=obj"] if save_temps else []
     jobs = jobs or min(8, os.cpu_count() or 1)

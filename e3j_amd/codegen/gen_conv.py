@@ -517,7 +517,7 @@ def write_all(out_dir: str, signatures=None) -> list[str]:
         paths.append(os.path.join(out_dir, fname))
     _write_if_changed(os.path.join(out_dir, "registry.hip"), emit_registry(2 * len(signatures)))
     for stale in os.listdir(out_dir):
-        if stale.endswith(".hip") and stale not in wanted:
+        if stale.startswith("sig_") and stale.endswith(".hip") and stale not in wanted:
             os.remove(os.path.join(out_dir, stale))
     return paths
 

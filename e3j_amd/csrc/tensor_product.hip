@@ -12,7 +12,10 @@
 // indexes dynamically; coefficients are wave-uniform and travel through scalar loads.  Runs
 // of equal output index are summed in a register and stored once.
 
-#include "common.h"
+#include <cmath>
+#include <cstring>
+
+#include "tp_unrolled.h"
 
 namespace e3j_amd {
 namespace {
@@ -218,6 +221,17 @@ int validate_tp(const e3j_amd_tp_params *p, const char *op) {
     if ((p->val_dtype != E3J_AMD_F32 && p->val_dtype != E3J_AMD_F64) ||
         (p->coef_idx_bytes != 1 && p->coef_idx_bytes != 4))
         return set_error(E3J_AMD_INVALID_ARGUMENT, name + ": unsupported (IDX, VAL) dtype pair");
+    if (p->signature >= num_tp_signatures())
+        return set_error(E3J_AMD_INVALID_ARGUMENT, name + ": unknown signature id " + std::to_string(p->signature));
+    if (p->signature >= 0) {
+        const TpSignature &sg = tp_signature(p->signature);
+        const bool mode_ok = sg.uniform_y ? (p->mode == E3J_AMD_MODE_OUTER && p->channels_y == 1)
+                                          : (p->mode == E3J_AMD_MODE_MAP && p->channels_y == sg.channels);
+        if (!mode_ok || p->val_dtype != E3J_AMD_F32 || p->layout != E3J_AMD_LAYOUT_TRAILING ||
+            sg.num_x != p->num_x || sg.num_y != p->num_y || sg.num_out != p->num_out || sg.channels != p->channels_x)
+            return set_error(E3J_AMD_INVALID_ARGUMENT,
+                             name + ": operands do not match signature " + sg.name);
+    }
     return E3J_AMD_OK;
 }
 
@@ -238,8 +252,13 @@ extern "C" int e3j_amd_tensor_product_fwd(const e3j_amd_tp_params *p, const void
     hipStream_t stream = static_cast<hipStream_t>(stream_ptr);
     if (int rc = validate_tp(p, "tensor_product")) return rc;
     if (absent(x, p->num_rows) || absent(y, p->num_rows) || absent(z, p->num_rows) ||
-        absent(coef, (int64_t)p->num_coef * p->num_rows))
+        (p->signature < 0 && absent(coef, (int64_t)p->num_coef * p->num_rows)))
         return set_error(E3J_AMD_INVALID_ARGUMENT, "tensor_product: null operand");
+    if (p->signature >= 0) {
+        const int rc = tp_signature(p->signature).fwd(p->num_rows, p->coef_scale, static_cast<const float *>(x),
+                                                      static_cast<const float *>(y), static_cast<float *>(z), stream);
+        return finish_tp(p, stream, rc, "tensor_product");
+    }
     const int rc = launch_product(p, p->mode, coef, x, p->num_x, p->channels_x, y, p->num_y, p->channels_y, z,
                                   p->num_out, stream);
     return finish_tp(p, stream, rc, "tensor_product");
@@ -255,8 +274,14 @@ extern "C" int e3j_amd_tensor_product_bwd(const e3j_amd_tp_params *p, const void
                          "tensor_product_bwd: OUTER mode requires either LHS or RHS to have one channel, got (" +
                              std::to_string(p->channels_x) + ", " + std::to_string(p->channels_y) + ")");
     if (absent(x, p->num_rows) || absent(y, p->num_rows) || absent(dz, p->num_rows) || absent(dx, p->num_rows) ||
-        absent(dy, p->num_rows) || absent(coef_bwd, (int64_t)p->num_coef * p->num_rows))
+        absent(dy, p->num_rows) || (p->signature < 0 && absent(coef_bwd, (int64_t)p->num_coef * p->num_rows)))
         return set_error(E3J_AMD_INVALID_ARGUMENT, "tensor_product_bwd: null operand");
+    if (p->signature >= 0) {
+        const int rc = tp_signature(p->signature).bwd(
+            p->num_rows, p->coef_scale, static_cast<const float *>(x), static_cast<const float *>(y),
+            static_cast<const float *>(dz), static_cast<float *>(dx), static_cast<float *>(dy), stream);
+        return finish_tp(p, stream, rc, "tensor_product_bwd");
+    }
     // dx = product(table (j; i, k); dz, y), dy = product(table (k; i, j); dz, x).  The channel
     // mode of each half follows from where the channel axis of the forward pass went
     // (src/e3j/ops/tensor_product.py:503-529): u,u->u gives MAP twice; u,u->1 gives 1,u->u twice;
@@ -277,4 +302,52 @@ extern "C" int e3j_amd_tensor_product_bwd(const e3j_amd_tp_params *p, const void
     if (rc == E3J_AMD_OK)
         rc = launch_product(p, mode_y, coef_y, dz, p->num_out, cz, x, p->num_x, cx, dy, p->num_y, stream);
     return finish_tp(p, stream, rc, "tensor_product_bwd");
+}
+
+extern "C" int e3j_amd_tp_num_signatures(void) { return num_tp_signatures(); }
+
+extern "C" const char *e3j_amd_tp_signature_name(int id) {
+    return (id >= 0 && id < num_tp_signatures()) ? tp_signature(id).name : "";
+}
+
+extern "C" int e3j_amd_tp_find_signature(const void *coef_host, int32_t coef_idx_bytes, int32_t val_dtype,
+                                         int32_t num_coef, int32_t num_x, int32_t num_y, int32_t num_out,
+                                         int32_t channels, int32_t uniform_y, float *coef_scale) {
+    if (coef_scale) *coef_scale = 1.0f;
+    if (coef_host == nullptr || val_dtype != E3J_AMD_F32 || num_coef <= 0) return -1;
+    if (coef_idx_bytes != 1 && coef_idx_bytes != 4) return -1;
+    const size_t item = coef_idx_bytes == 1 ? sizeof(Coef3<uint8_t, float>) : sizeof(Coef3<int32_t, float>);
+    const unsigned char *bytes = static_cast<const unsigned char *>(coef_host);
+    for (int id = 0; id < num_tp_signatures(); id++) {
+        const TpSignature &sg = tp_signature(id);
+        if (sg.num_coef != num_coef || sg.num_x != num_x || sg.num_y != num_y || sg.num_out != num_out ||
+            sg.channels != channels || sg.uniform_y != (uniform_y != 0))
+            continue;
+        // one uniform positive factor is allowed between the tables, taken from the entry of
+        // largest magnitude; every entry must agree with it to float32 rounding
+        int big = 0;
+        for (int n = 1; n < num_coef; n++)
+            if (std::fabs(sg.val[n]) > std::fabs(sg.val[big])) big = n;
+        float vbig;
+        std::memcpy(&vbig, bytes + big * item, sizeof(float));
+        const double scale = (double)vbig / (double)sg.val[big];
+        bool same = scale > 0.0 && std::isfinite(scale);
+        for (int n = 0; n < num_coef && same; n++) {
+            float v;
+            std::memcpy(&v, bytes + n * item, sizeof(float));
+            for (int t = 0; t < 3 && same; t++) {
+                int32_t index;
+                if (coef_idx_bytes == 1) index = bytes[n * item + 4 + t];
+                else std::memcpy(&index, bytes + n * item + 4 + 4 * t, 4);
+                same = index == (int32_t)sg.idx[3 * n + t];
+            }
+            const double want = scale * (double)sg.val[n];
+            same = same && std::fabs((double)v - want) <= 4e-7 * std::fabs(want);
+        }
+        if (same) {
+            if (coef_scale) *coef_scale = (float)scale;
+            return id;
+        }
+    }
+    return -1;
 }

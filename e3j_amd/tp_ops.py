@@ -62,6 +62,21 @@ class _Table:
         self.packed_bwd = np.ascontiguousarray(np.stack(
             [c.transpose((1, 0, 2)).pack(), c.transpose((2, 0, 1)).pack()]))
         self._device = {}
+        self._signature = {}
+
+    def signature(self, num_x: int, num_y: int, num_out: int, channels: int, uniform_y: bool):
+        """`(id, scale)` of a built-in unrolled kernel, `(-1, 1.0)` if none matches."""
+        key = (num_x, num_y, num_out, channels, uniform_y)
+        hit = self._signature.get(key)
+        if hit is None:
+            scale = ctypes.c_float(1.0)
+            sig = -1
+            if self.val_np_dtype == np.float32 and self.num_coef > 0:
+                sig = int(_lib.load().e3j_amd_tp_find_signature(
+                    self.packed.ctypes.data, self.idx_bytes, _lib.F32, self.num_coef, num_x, num_y, num_out,
+                    channels, int(uniform_y), ctypes.byref(scale)))
+            hit = self._signature[key] = (sig, float(scale.value))
+        return hit
 
     @classmethod
     def get(cls, coef, val_np_dtype) -> "_Table":
@@ -126,7 +141,15 @@ def _stream(device) -> int:
 def _params(meta: _Meta, x: torch.Tensor, y: torch.Tensor, backward: bool) -> _lib.TpParams:
     num_x, cx = meta.dims(x, meta.has_cx)
     num_y, cy = meta.dims(y, meta.has_cy)
+    # unrolled kernels: trailing layout, float32, MAP or OUTER with a channel-free y
+    sig, scale = -1, 1.0
+    if meta.layout == Layout.TRAILING_CHANNELS and x.dtype == torch.float32 and cx % 64 == 0:
+        if meta.mode == MixingMode.MAP:
+            sig, scale = meta.table.signature(num_x, num_y, meta.num_out, cx, False)
+        elif meta.mode == MixingMode.OUTER and cy == 1:
+            sig, scale = meta.table.signature(num_x, num_y, meta.num_out, cx, True)
     return _lib.TpParams(
+        signature=sig, coef_scale=scale,
         num_rows=int(x.shape[0]), num_coef=meta.table.num_coef, num_x=num_x, num_y=num_y,
         num_out=meta.num_out, channels_x=cx, channels_y=cy, mode=meta.mode.value, layout=meta.layout.value,
         val_dtype=_VAL_DTYPES[x.dtype][0], coef_idx_bytes=meta.table.idx_bytes,

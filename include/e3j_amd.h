@@ -238,6 +238,8 @@ typedef struct e3j_amd_tp_params {
      * order; the result is zero-filled first and runs are added. */
     int32_t coef_sorted;
     int32_t debug;
+    int32_t signature;      /* id from e3j_amd_tp_find_signature, or -1: table-driven kernel */
+    float   coef_scale;     /* unrolled kernels: table = coef_scale * built-in table */
 } e3j_amd_tp_params;
 int e3j_amd_tensor_product_fwd(const e3j_amd_tp_params *p, const void *coef, const void *x, const void *y,
                                void *z, void *stream);
@@ -249,6 +251,20 @@ int e3j_amd_tensor_product_fwd(const e3j_amd_tp_params *p, const void *coef, con
  * (as the reference, src/e3j/ops/tensor_product.py:322-326); both layouts are served. */
 int e3j_amd_tensor_product_bwd(const e3j_amd_tp_params *p, const void *coef_bwd, const void *x, const void *y,
                                const void *dz, void *dx, void *dy, void *stream);
+
+/* Compile-time-unrolled kernels of the tensor product exist for built-in Clebsch-Gordan tables in
+ * the trailing layout, float32, channel counts that are multiples of 64, and two channel modes:
+ * MAP (uniform_y = 0) and OUTER with channels_y == 1 (uniform_y = 1).  The lookup compares a
+ * packed forward table in HOST memory with the built-in ones (same entries in the same order, up
+ * to one positive factor returned in *coef_scale) and returns an id for
+ * e3j_amd_tp_params.signature, or -1.  With a signature the `coef` / `coef_bwd` operands of the
+ * two entry points above are not read and may be NULL.  No counterpart in the reference, whose
+ * kernels are table-driven only. */
+int e3j_amd_tp_find_signature(const void *coef_host, int32_t coef_idx_bytes, int32_t val_dtype,
+                              int32_t num_coef, int32_t num_x, int32_t num_y, int32_t num_out,
+                              int32_t channels, int32_t uniform_y, float *coef_scale);
+int e3j_amd_tp_num_signatures(void);
+const char *e3j_amd_tp_signature_name(int id);
 
 /* XLA-FFI handlers (C ABI of xla/ffi/api/c_api.h): `XLA_FFI_Error* handler(XLA_FFI_CallFrame*)`.
  * Operand order of "convolution"/"convolution_bwd" as in lib/e3j_ops/ffi/e3j_ops.h:457-472,575-594;

@@ -55,9 +55,9 @@ def test_params_struct_matches_header():
 def test_tensor_product_params_struct_matches_header():
     header = open(os.path.join(ROOT, "include", "e3j_amd.h")).read()
     body = re.search(r"typedef struct e3j_amd_tp_params \{(.*?)\} e3j_amd_tp_params;", header, re.S).group(1)
-    fields = re.findall(r"^\s*(int32_t|int64_t)\s*(\w+);", body, re.M)
+    fields = re.findall(r"^\s*(int32_t|int64_t|float)\s*(\w+);", body, re.M)
     assert [name for _, name in fields] == [name for name, _ in _lib.TpParams._fields_]
-    ctype = {"int32_t": C.c_int32, "int64_t": C.c_int64}
+    ctype = {"int32_t": C.c_int32, "int64_t": C.c_int64, "float": C.c_float}
     assert [ctype[t] for t, _ in fields] == [t for _, t in _lib.TpParams._fields_]
     modes = re.search(r"E3J_AMD_MODE_OUTER = (\d), E3J_AMD_MODE_INNER = (\d), E3J_AMD_MODE_MAP = (\d)", header)
     assert tuple(map(int, modes.groups())) == (_lib.MODE_OUTER, _lib.MODE_INNER, _lib.MODE_MAP)
@@ -68,7 +68,8 @@ def test_tensor_product_argument_errors_need_no_launch():
     assert lib.e3j_amd_tensor_product_fwd(None, None, None, None, None, None) == _lib.INVALID_ARGUMENT
     assert "null params" in lib.e3j_amd_last_error().decode()
     p = _lib.TpParams(num_rows=0, num_coef=0, num_x=1, num_y=1, num_out=1, channels_x=1, channels_y=1,
-                      mode=_lib.MODE_OUTER, layout=_lib.LAYOUT_LEADING, val_dtype=_lib.F32, coef_idx_bytes=1)
+                      mode=_lib.MODE_OUTER, layout=_lib.LAYOUT_LEADING, val_dtype=_lib.F32, coef_idx_bytes=1,
+                      signature=-1, coef_scale=1.0)
     assert lib.e3j_amd_tensor_product_fwd(C.byref(p), None, None, None, None, None) == _lib.OK   # no rows: a no-op
     p.num_rows = 3
     assert lib.e3j_amd_tensor_product_fwd(C.byref(p), None, None, None, None, None) == _lib.INVALID_ARGUMENT
@@ -76,6 +77,40 @@ def test_tensor_product_argument_errors_need_no_launch():
     p.mode = 9
     assert lib.e3j_amd_tensor_product_bwd(C.byref(p), *[None] * 7) == _lib.INVALID_ARGUMENT
     assert "unknown mode" in lib.e3j_amd_last_error().decode()
+    p.mode, p.signature = _lib.MODE_OUTER, 10_000
+    assert lib.e3j_amd_tensor_product_fwd(C.byref(p), None, None, None, None, None) == _lib.INVALID_ARGUMENT
+    assert "unknown signature" in lib.e3j_amd_last_error().decode()
+    p.signature = 0      # a built-in kernel: trailing layout, 64 channels, MAP
+    assert lib.e3j_amd_tensor_product_fwd(C.byref(p), None, None, None, None, None) == _lib.INVALID_ARGUMENT
+    assert "do not match signature" in lib.e3j_amd_last_error().decode()
+
+
+def test_tensor_product_signature_lookup():
+    from e3j_amd import TensorProduct
+    lib = _lib.load()
+    assert lib.e3j_amd_tp_num_signatures() >= 8
+    tp = TensorProduct(("0e+1o+2e+3o", "0e+1o+2e+3o"), "0e+1o+2e+3o")
+    packed = tp.packed_coef("float32")
+    Z, X, Y = tp.shape
+    scale = C.c_float(0)
+
+    def find(buf, channels, uniform, idx_bytes=None):
+        return lib.e3j_amd_tp_find_signature(buf.ctypes.data, idx_bytes or buf.dtype.itemsize, _lib.F32, buf.shape[0],
+                                             X, Y, Z, channels, uniform, C.byref(scale))
+    a, b = find(packed, 128, 0), find(packed, 128, 1)
+    assert a >= 0 and b >= 0 and a != b and scale.value == 1.0
+    assert b"K=128" in lib.e3j_amd_tp_signature_name(a) and b"MAP" in lib.e3j_amd_tp_signature_name(a)
+    assert b"without channel axis" in lib.e3j_amd_tp_signature_name(b)
+    assert find(packed, 64, 0) >= 0 and find(packed, 96, 0) == -1 and find(packed, 32, 0) == -1
+    from e3j_amd.coef import Coef
+    c = Coef.unpack(packed, np.float32)
+    assert find(Coef(3.0 * c.val, c.idx, "float32", "int32").pack(), 128, 0) == a and abs(scale.value - 3.0) < 1e-6
+    bent = c.val.copy()
+    bent[5] *= 1.001
+    assert find(Coef(bent, c.idx, "float32", "int32").pack(), 128, 0) == -1
+    assert find(Coef(-c.val, c.idx, "float32", "int32").pack(), 128, 0) == -1
+    other = TensorProduct(("0e+1o+2e+3o", "0e+1o+2e+3o"), "0e+1o+2e+3o", normalization="SQRT_DIM_OUT")
+    assert find(other.packed_coef("float32"), 128, 0) == -1     # one factor per path is not one factor
 
 
 @pytest.mark.parametrize("kw, code, needle", [

@@ -239,7 +239,7 @@ def test_c_abi_errors():
     def params(**kw):
         base = dict(num_rows=2, num_coef=3, num_x=4, num_y=3, num_out=5, channels_x=8, channels_y=8,
                     mode=_lib.MODE_MAP, layout=_lib.LAYOUT_TRAILING, val_dtype=_lib.F32, coef_idx_bytes=4,
-                    coef_sorted=1, debug=0)
+                    coef_sorted=1, debug=0, signature=-1, coef_scale=1.0)
         base.update(kw)
         return _lib.TpParams(**base)
     def fwd(p):
@@ -255,3 +255,69 @@ def test_c_abi_errors():
     rc = lib.e3j_amd_tensor_product_bwd(ctypes.byref(p), *[buf.data_ptr()] * 6, stream)
     assert rc == _lib.UNIMPLEMENTED and b"one channel" in lib.e3j_amd_last_error()
     torch.cuda.synchronize()
+
+
+# ---------------------------------------------------------------------------
+# compile-time-unrolled kernels (built-in Clebsch-Gordan tables, trailing layout)
+# ---------------------------------------------------------------------------
+BUILTIN = [("0e+1o+2e", "0e+1o+2e", None), ("0e+1o+2e", "0e+1o+2e+3o", "0e+1o+2e+3o"),
+           ("0e+1o+2e+3o", "0e+1o+2e+3o", "0e+1o+2e+3o")]
+
+
+@pytest.mark.parametrize("spaces", BUILTIN, ids=["l2_l2_full", "l2_l3_to_l3", "l3_l3_to_l3"])
+@pytest.mark.parametrize("channels", [64, 128])
+@pytest.mark.parametrize("mode", ["MAP", "OUTER"])
+def test_unrolled_kernels_against_the_checker(spaces, channels, mode):
+    from e3j_amd.tp_ops import _Table
+    rng = np.random.default_rng(21)
+    tp = TensorProduct(spaces[:2], spaces[2], layout="TRAILING_CHANNELS", mode=mode)
+    Z, X, Y = tp.shape
+    idx, val = np.asarray(tp.indices, dtype=np.int64), 1.5 * np.asarray(tp.values, dtype=np.float64)
+    table = _Table.get(Coef(val, idx, "float32", "uint8").pack(), np.float32)
+    sig, scale = table.signature(X, Y, Z, channels, mode == "OUTER")
+    assert sig >= 0 and abs(scale - 1.5) < 1e-6, "a built-in unrolled kernel must serve this table"
+    x, y = _operands(rng, mode, "TRAILING_CHANNELS", channels, rows=77, dims=(X, Y), has=(True, False))
+    _check_forward(idx, val, x, y, Z, mode, "TRAILING_CHANNELS", "uint8", what=f"unrolled {mode} K={channels}")
+    _check_backward(idx, val, x, y, Z, mode, "TRAILING_CHANNELS", rng, "uint8", what=f"unrolled {mode} K={channels}")
+
+
+@pytest.mark.parametrize("mode", ["MAP", "OUTER"])
+def test_unrolled_and_table_driven_kernels_agree_through_the_c_abi(mode):
+    lib = _lib.load()
+    tp = TensorProduct(("0e+1o+2e+3o", "0e+1o+2e+3o"), "0e+1o+2e+3o", layout="TRAILING_CHANNELS", mode=mode)
+    Z, X, Y = tp.shape
+    K, R = 128, 301
+    packed = tp.packed_coef("float32")
+    from e3j_amd.tp_ops import _Table
+    table = _Table.get(packed, np.float32)
+    uniform = mode == "OUTER"
+    sig, scale = table.signature(X, Y, Z, K, uniform)
+    assert sig >= 0
+    g = torch.Generator(device="cpu").manual_seed(3)
+    x = torch.randn(R, X, K, generator=g).to(DEV)
+    y = (torch.randn(R, Y, generator=g) if uniform else torch.randn(R, Y, K, generator=g)).to(DEV)
+    dz = torch.randn(R, Z, K, generator=g).to(DEV)
+    stream = int(torch.cuda.current_stream().cuda_stream)
+    results = []
+    for signature in (sig, -1):
+        p = _lib.TpParams(num_rows=R, num_coef=table.num_coef, num_x=X, num_y=Y, num_out=Z, channels_x=K,
+                          channels_y=1 if uniform else K, mode=_lib.MODE_OUTER if uniform else _lib.MODE_MAP,
+                          layout=_lib.LAYOUT_TRAILING, val_dtype=_lib.F32, coef_idx_bytes=table.idx_bytes,
+                          coef_sorted=1, debug=1, signature=signature, coef_scale=scale)
+        z = torch.full((R, Z, K), float("nan"), device=DEV)
+        dx, dy = torch.full_like(x, float("nan")), torch.full_like(y, float("nan"))
+        coef = None if signature >= 0 else table.device(x.device).data_ptr()
+        coef_bwd = None if signature >= 0 else table.device(x.device, backward=True).data_ptr()
+        _lib.check(lib.e3j_amd_tensor_product_fwd(ctypes.byref(p), coef, x.data_ptr(), y.data_ptr(), z.data_ptr(), stream))
+        _lib.check(lib.e3j_amd_tensor_product_bwd(ctypes.byref(p), coef_bwd, x.data_ptr(), y.data_ptr(), dz.data_ptr(),
+                                                  dx.data_ptr(), dy.data_ptr(), stream))
+        results.append((z, dx, dy))
+    for a, b, name in zip(results[0], results[1], ("z", "dx", "dy")):
+        assert torch.isfinite(a).all(), name
+        torch.testing.assert_close(a, b, rtol=2e-5, atol=2e-5, msg=lambda m, name=name: f"{name}: {m}")
+    # repeatable to the bit (no atomics anywhere)
+    z2 = torch.empty_like(results[0][0])
+    p.signature = sig
+    _lib.check(lib.e3j_amd_tensor_product_fwd(ctypes.byref(p), None, x.data_ptr(), y.data_ptr(), z2.data_ptr(), stream))
+    torch.cuda.synchronize()
+    assert torch.equal(z2, results[0][0])
