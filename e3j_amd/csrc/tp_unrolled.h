@@ -103,27 +103,36 @@ __global__ __launch_bounds__(kWave * WPB) void tp_unrolled_bwd_map_kernel(
     for (int k = 0; k < Y; k++) __builtin_nontemporal_store(dyv[k], dyr + k * K);
 }
 
-// Uniform-y backward: one wave per row walks the channel slices; dy (rows, Y) is the channel
-// sum, reduced over the wave once per row.
-template <typename Sig, int K, int WPB>
-__global__ __launch_bounds__(kWave * WPB) void tp_unrolled_bwd_uniform_kernel(
+// Uniform-y backward: a wave per (row, slice); dy (rows, Y) is the channel sum: every wave
+// reduces its 64 channels, the slices of a row sit in one block and meet in LDS, and the
+// first of them stores the row (fixed order, no atomics).
+template <int K>
+struct TpUniformGeometry {
+    static constexpr int SL = K / kWave;              // waves per row
+    static constexpr int RPB = SL >= 4 ? 1 : 4 / SL;  // rows per block
+    static constexpr int WPB = SL * RPB;
+};
+
+template <typename Sig, int K>
+__global__ __launch_bounds__(kWave * TpUniformGeometry<K>::WPB) void tp_unrolled_bwd_uniform_kernel(
     const float *__restrict__ x, const float *__restrict__ y, const float *__restrict__ dz,
     float *__restrict__ dx, float *__restrict__ dy, int64_t rows, float scale) {
-    constexpr int X = Sig::X, Y = Sig::Y, Z = Sig::Z, SL = K / kWave;
+    constexpr int X = Sig::X, Y = Sig::Y, Z = Sig::Z;
+    using G = TpUniformGeometry<K>;
     using Red = WaveReduce<Y>;
-    const int64_t r = tp_uniform((int64_t)blockIdx.x * WPB + threadIdx.y);
-    if (r >= rows) return;
-    const int lane = threadIdx.x;
-    float yv[Y], dyv[Red::P];
-    const float *yr = y + r * Y;
+    __shared__ float partial[G::WPB][Red::P];
+    const int wave = threadIdx.y, lane = threadIdx.x;
+    const int slice = wave % G::SL;
+    const int64_t r = tp_uniform((int64_t)blockIdx.x * G::RPB + wave / G::SL);
+    const bool valid = r < rows;  // uniform per wave; every wave reaches the barrier
+    if (valid) {
+        float yv[Y], dyv[Red::P], xv[X], dxv[X];
+        const float *yr = y + r * Y;
 #pragma unroll
-    for (int k = 0; k < Y; k++) yv[k] = to_vgpr(yr[k]);
+        for (int k = 0; k < Y; k++) yv[k] = to_vgpr(yr[k]);
 #pragma unroll
-    for (int k = 0; k < Red::P; k++) dyv[k] = 0.f;
-#pragma unroll 1
-    for (int slice = 0; slice < SL; slice++) {
+        for (int k = 0; k < Red::P; k++) dyv[k] = 0.f;
         const int c0 = slice * kWave + lane;
-        float xv[X], dxv[X];
         const float *xr = x + r * (X * K) + c0;
 #pragma unroll
         for (int j = 0; j < X; j++) { xv[j] = __builtin_nontemporal_load(xr + j * K); dxv[j] = 0.f; }
@@ -131,10 +140,16 @@ __global__ __launch_bounds__(kWave * WPB) void tp_unrolled_bwd_uniform_kernel(
         float *dxr = dx + r * (X * K) + c0;
 #pragma unroll
         for (int j = 0; j < X; j++) __builtin_nontemporal_store(dxv[j], dxr + j * K);
+        const float total = Red::run(dyv, lane);
+        if (lane < 16) partial[wave][Red::slot(lane)] = total;
     }
-    const int k = Red::slot(lane);
-    const float total = Red::run(dyv, lane);
-    if (lane < 16 && k < Y) dy[r * Y + k] = total;
+    __syncthreads();
+    if (valid && slice == 0 && lane < Y) {
+        float total = partial[wave][lane];
+#pragma unroll
+        for (int s2 = 1; s2 < G::SL; s2++) total += partial[wave + s2][lane];
+        dy[r * Y + lane] = total;
+    }
 }
 
 inline int tp_grid(int64_t items, int wpb, unsigned *blocks) {
@@ -163,8 +178,9 @@ int launch_tp_unrolled_bwd(int64_t rows, float scale, const float *x, const floa
     if (rows == 0) return E3J_AMD_OK;
     unsigned blocks;
     if (kUniformY) {
-        if (int rc = tp_grid(rows, WPB, &blocks)) return rc;
-        hipLaunchKernelGGL((tp_unrolled_bwd_uniform_kernel<Sig, K, WPB>), dim3(blocks), dim3(kWave, WPB), 0, stream,
+        using G = TpUniformGeometry<K>;
+        if (int rc = tp_grid(rows, G::RPB, &blocks)) return rc;
+        hipLaunchKernelGGL((tp_unrolled_bwd_uniform_kernel<Sig, K>), dim3(blocks), dim3(kWave, G::WPB), 0, stream,
                            x, y, dz, dx, dy, rows, scale);
     } else {
         if (int rc = tp_grid(rows * (K / kWave), WPB, &blocks)) return rc;
