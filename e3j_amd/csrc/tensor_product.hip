@@ -14,6 +14,7 @@
 
 #include <cmath>
 #include <cstring>
+#include <initializer_list>
 
 #include "tp_unrolled.h"
 
@@ -226,9 +227,13 @@ int validate_tp(const e3j_amd_tp_params *p, const char *op) {
     if (p->signature >= 0) {
         const TpSignature &sg = tp_signature(p->signature);
         const bool mode_ok = sg.uniform_y ? (p->mode == E3J_AMD_MODE_OUTER && p->channels_y == 1)
-                                          : (p->mode == E3J_AMD_MODE_MAP && p->channels_y == sg.channels);
-        if (!mode_ok || p->val_dtype != E3J_AMD_F32 || p->layout != E3J_AMD_LAYOUT_TRAILING ||
-            sg.num_x != p->num_x || sg.num_y != p->num_y || sg.num_out != p->num_out || sg.channels != p->channels_x)
+                                          : (p->mode == E3J_AMD_MODE_MAP && p->channels_y == p->channels_x);
+        const bool channels_ok = sg.layout == E3J_AMD_LAYOUT_TRAILING
+                                     ? sg.channels == p->channels_x
+                                     : (tp_leading_channels_ok(p->channels_x, sg.uniform_y != 0) &&
+                                        p->num_rows * p->channels_x >= kWave);
+        if (!mode_ok || !channels_ok || p->val_dtype != E3J_AMD_F32 || p->layout != sg.layout ||
+            sg.num_x != p->num_x || sg.num_y != p->num_y || sg.num_out != p->num_out)
             return set_error(E3J_AMD_INVALID_ARGUMENT,
                              name + ": operands do not match signature " + sg.name);
     }
@@ -236,6 +241,16 @@ int validate_tp(const e3j_amd_tp_params *p, const char *op) {
 }
 
 bool absent(const void *ptr, int64_t count) { return count > 0 && ptr == nullptr; }
+
+// The unrolled kernels of the leading layout move columns in 16-byte pieces.
+const char *const kUnaligned = "tensor_product: the unrolled kernels of the leading layout need 16-byte "
+                               "aligned operands (pass signature -1 for the table-driven kernels)";
+bool pieces_aligned(const e3j_amd_tp_params *p, std::initializer_list<const void *> ptrs) {
+    if (p->layout != E3J_AMD_LAYOUT_LEADING) return true;
+    for (const void *ptr : ptrs)
+        if (reinterpret_cast<uintptr_t>(ptr) % 16 != 0) return false;
+    return true;
+}
 
 int finish_tp(const e3j_amd_tp_params *p, hipStream_t stream, int rc, const char *op) {
     if (rc != E3J_AMD_OK || p->debug <= 0) return rc;
@@ -255,8 +270,10 @@ extern "C" int e3j_amd_tensor_product_fwd(const e3j_amd_tp_params *p, const void
         (p->signature < 0 && absent(coef, (int64_t)p->num_coef * p->num_rows)))
         return set_error(E3J_AMD_INVALID_ARGUMENT, "tensor_product: null operand");
     if (p->signature >= 0) {
-        const int rc = tp_signature(p->signature).fwd(p->num_rows, p->coef_scale, static_cast<const float *>(x),
-                                                      static_cast<const float *>(y), static_cast<float *>(z), stream);
+        if (!pieces_aligned(p, {x, y, z})) return set_error(E3J_AMD_INVALID_ARGUMENT, kUnaligned);
+        const int rc = tp_signature(p->signature).fwd(p->num_rows, p->channels_x, p->coef_scale,
+                                                      static_cast<const float *>(x), static_cast<const float *>(y),
+                                                      static_cast<float *>(z), stream);
         return finish_tp(p, stream, rc, "tensor_product");
     }
     const int rc = launch_product(p, p->mode, coef, x, p->num_x, p->channels_x, y, p->num_y, p->channels_y, z,
@@ -277,8 +294,9 @@ extern "C" int e3j_amd_tensor_product_bwd(const e3j_amd_tp_params *p, const void
         absent(dy, p->num_rows) || (p->signature < 0 && absent(coef_bwd, (int64_t)p->num_coef * p->num_rows)))
         return set_error(E3J_AMD_INVALID_ARGUMENT, "tensor_product_bwd: null operand");
     if (p->signature >= 0) {
+        if (!pieces_aligned(p, {x, y, dz, dx, dy})) return set_error(E3J_AMD_INVALID_ARGUMENT, kUnaligned);
         const int rc = tp_signature(p->signature).bwd(
-            p->num_rows, p->coef_scale, static_cast<const float *>(x), static_cast<const float *>(y),
+            p->num_rows, p->channels_x, p->coef_scale, static_cast<const float *>(x), static_cast<const float *>(y),
             static_cast<const float *>(dz), static_cast<float *>(dx), static_cast<float *>(dy), stream);
         return finish_tp(p, stream, rc, "tensor_product_bwd");
     }
@@ -312,7 +330,8 @@ extern "C" const char *e3j_amd_tp_signature_name(int id) {
 
 extern "C" int e3j_amd_tp_find_signature(const void *coef_host, int32_t coef_idx_bytes, int32_t val_dtype,
                                          int32_t num_coef, int32_t num_x, int32_t num_y, int32_t num_out,
-                                         int32_t channels, int32_t uniform_y, float *coef_scale) {
+                                         int32_t channels, int32_t uniform_y, int32_t layout,
+                                         float *coef_scale) {
     if (coef_scale) *coef_scale = 1.0f;
     if (coef_host == nullptr || val_dtype != E3J_AMD_F32 || num_coef <= 0) return -1;
     if (coef_idx_bytes != 1 && coef_idx_bytes != 4) return -1;
@@ -321,7 +340,10 @@ extern "C" int e3j_amd_tp_find_signature(const void *coef_host, int32_t coef_idx
     for (int id = 0; id < num_tp_signatures(); id++) {
         const TpSignature &sg = tp_signature(id);
         if (sg.num_coef != num_coef || sg.num_x != num_x || sg.num_y != num_y || sg.num_out != num_out ||
-            sg.channels != channels || sg.uniform_y != (uniform_y != 0))
+            sg.layout != layout || sg.uniform_y != (uniform_y != 0))
+            continue;
+        if (sg.layout == E3J_AMD_LAYOUT_TRAILING ? sg.channels != channels
+                                                 : !tp_leading_channels_ok(channels, uniform_y != 0))
             continue;
         // one uniform positive factor is allowed between the tables, taken from the entry of
         // largest magnitude; every entry must agree with it to float32 rounding

@@ -1,5 +1,6 @@
-// Kernel templates of the compile-time-unrolled row-wise tensor product (gfx950, float32,
-// trailing-channels layout, channel counts that are multiples of 64).
+// Kernel templates of the compile-time-unrolled row-wise tensor product (gfx950, float32):
+// trailing-channels layout for channel counts that are multiples of 64 (first part), and
+// leading-channels layout (second part).
 //
 // A generated `Sig` type supplies the straight-line Clebsch-Gordan arithmetic of one table
 // (`fwd`, `bwd`); the templates supply the wave <-> (row, 64-channel slice) mapping and the
@@ -20,14 +21,23 @@ namespace e3j_amd {
 struct TpSignature {
     const char *name;
     int32_t num_x, num_y, num_out, num_coef;
-    int32_t channels;
+    int32_t channels;     // trailing layout: the channel count the kernels were built for;
+                          // leading layout: 0, the kernels take the channel count at run time
     int32_t uniform_y;    // 1: y has no channel axis (OUTER); 0: MAP
+    int32_t layout;
     const float *val;     // (num_coef) table values as float32
     const uint8_t *idx;   // (num_coef, 3) i, j, k
-    int (*fwd)(int64_t rows, float scale, const float *x, const float *y, float *z, hipStream_t stream);
-    int (*bwd)(int64_t rows, float scale, const float *x, const float *y, const float *dz, float *dx,
-               float *dy, hipStream_t stream);
+    int (*fwd)(int64_t rows, int channels, float scale, const float *x, const float *y, float *z,
+               hipStream_t stream);
+    int (*bwd)(int64_t rows, int channels, float scale, const float *x, const float *y, const float *dz,
+               float *dx, float *dy, hipStream_t stream);
 };
+// channel counts the leading-layout kernels take: MAP any multiple of 4 (16-byte pieces) with at
+// least 64 columns in all; uniform y: forward the same, backward whole waves per row that fit a block
+inline bool tp_leading_channels_ok(int channels, bool uniform_y) {
+    if (channels < 4 || channels % 4 != 0) return false;
+    return !uniform_y || channels == 64 || channels == 128 || channels == 256;
+}
 int num_tp_signatures();
 const TpSignature &tp_signature(int id);
 
@@ -160,7 +170,7 @@ inline int tp_grid(int64_t items, int wpb, unsigned *blocks) {
 }
 
 template <typename Sig, int K, bool kUniformY>
-int launch_tp_unrolled_fwd(int64_t rows, float scale, const float *x, const float *y, float *z,
+int launch_tp_unrolled_fwd(int64_t rows, int, float scale, const float *x, const float *y, float *z,
                            hipStream_t stream) {
     constexpr int WPB = 4;
     if (rows == 0) return E3J_AMD_OK;
@@ -172,7 +182,7 @@ int launch_tp_unrolled_fwd(int64_t rows, float scale, const float *x, const floa
 }
 
 template <typename Sig, int K, bool kUniformY>
-int launch_tp_unrolled_bwd(int64_t rows, float scale, const float *x, const float *y, const float *dz,
+int launch_tp_unrolled_bwd(int64_t rows, int, float scale, const float *x, const float *y, const float *dz,
                            float *dx, float *dy, hipStream_t stream) {
     constexpr int WPB = 4;
     if (rows == 0) return E3J_AMD_OK;
@@ -188,6 +198,235 @@ int launch_tp_unrolled_bwd(int64_t rows, float scale, const float *x, const floa
                            x, y, dz, dx, dy, rows, scale);
     }
     return check_hip(hipGetLastError(), "tensor_product_bwd (unrolled) launch");
+}
+
+// ---------------------------------------------------------------------------
+// Leading-channels layout: x (R, K, X), y (R, K, Y) or (R, Y), z (R, K, Z).  The columns
+// (r, c) are consecutive blocks of X (Y, Z) floats, so a wave takes 64 consecutive columns
+// whatever the channel count: it moves their contiguous block with coalesced 16-byte
+// accesses and turns it through its strip of LDS (odd row stride: conflict-free column
+// access), runs the same generated arithmetic on registers, and turns the results back.
+// The last tile is moved back to end at the last column; the columns it shares with the
+// tile before receive the same values from both.
+// ---------------------------------------------------------------------------
+template <int X, int Y, int Z>
+struct TpLeadingGeometry {
+    static constexpr int PX = odd_stride(X), PY = odd_stride(Y), PZ = odd_stride(Z);
+    static constexpr int XR = round4(kWave * PX), YR = round4(kWave * PY);
+    static constexpr int GC = 16;  // columns of z / dz that pass through the strip at a time
+    static constexpr int ZR = round4(GC * PZ);
+    static constexpr int REGION = XR + YR > ZR ? XR + YR : ZR;
+};
+
+template <int Z>
+struct RegStore {
+    float *v;
+    template <int I>
+    __device__ __forceinline__ void put(float a) const { v[I] = a; }
+};
+template <int Z>
+struct RegLoad {
+    const float *v;
+    template <int I>
+    __device__ __forceinline__ float get() const { return v[I]; }
+};
+
+__device__ __forceinline__ int64_t tp_tile_start(int64_t tile, int64_t cols) {
+    const int64_t c = tile * kWave;
+    return c + kWave <= cols ? c : cols - kWave;
+}
+
+// columns of this wave into registers (x scaled); y from its strip, or per row when uniform
+template <typename Sig, bool kUniformY>
+__device__ __forceinline__ void tp_leading_operands(const float *__restrict__ x, const float *__restrict__ y,
+                                                    int64_t col0, int K, float scale, float *strip, int lane,
+                                                    float *xv, float *yv) {
+    using G = TpLeadingGeometry<Sig::X, Sig::Y, Sig::Z>;
+    float *strip_x = strip, *strip_y = strip + G::XR;
+    LinearBlock<kWave * Sig::X> xl;
+    xl.template load<true>(x + col0 * Sig::X, lane);
+    xl.template to_strip<Sig::X, G::PX>(strip_x, lane);
+    if (!kUniformY) {
+        LinearBlock<kWave * Sig::Y> yl;
+        yl.template load<true>(y + col0 * Sig::Y, lane);
+        yl.template to_strip<Sig::Y, G::PY>(strip_y, lane);
+    }
+    strip_fence();
+#pragma unroll
+    for (int j = 0; j < Sig::X; j++) xv[j] = strip_x[lane * G::PX + j] * scale;
+    if (kUniformY) {
+        const float *yr = y + ((col0 + lane) / K) * Sig::Y;
+#pragma unroll
+        for (int k = 0; k < Sig::Y; k++) yv[k] = yr[k];
+    } else {
+#pragma unroll
+        for (int k = 0; k < Sig::Y; k++) yv[k] = strip_y[lane * G::PY + k];
+    }
+}
+
+template <typename Sig, int WPB, bool kUniformY>
+__global__ __launch_bounds__(kWave * WPB) void tp_unrolled_fwd_leading_kernel(
+    const float *__restrict__ x, const float *__restrict__ y, float *__restrict__ z, int64_t cols, int K,
+    float scale) {
+    constexpr int Z = Sig::Z;
+    using G = TpLeadingGeometry<Sig::X, Sig::Y, Z>;
+    __shared__ __attribute__((aligned(16))) float strips[WPB * G::REGION];
+    float *strip = strips + threadIdx.y * G::REGION;
+    const int lane = threadIdx.x;
+    const int64_t tile = tp_uniform((int64_t)blockIdx.x * WPB + threadIdx.y);
+    if (tile >= (cols + kWave - 1) / kWave) return;  // uniform per wave; no block barrier below
+    const int64_t col0 = tp_tile_start(tile, cols);
+    float xv[Sig::X], yv[Sig::Y], zv[Z];
+    tp_leading_operands<Sig, kUniformY>(x, y, col0, K, scale, strip, lane, xv, yv);
+    Sig::fwd(xv, yv, RegStore<Z>{zv});
+#pragma unroll
+    for (int q = 0; q < kWave / G::GC; q++) {
+        strip_fence();  // the reads of the strip so far are done
+        if (lane / G::GC == q) {
+#pragma unroll
+            for (int i = 0; i < Z; i++) strip[(lane % G::GC) * G::PZ + i] = zv[i];
+        }
+        strip_fence();
+        LinearBlock<G::GC * Z> ol;
+        ol.template from_strip<Z, G::PZ>(strip, lane);
+        ol.store(z + (col0 + q * G::GC) * Z, lane);
+    }
+}
+
+// cotangent columns of this wave into registers (scaled), 16 columns at a time through the strip
+template <typename Sig>
+__device__ __forceinline__ void tp_leading_cotangent(const float *__restrict__ dz, int64_t col0, float scale,
+                                                     float *strip, int lane, float *dzv) {
+    constexpr int Z = Sig::Z;
+    using G = TpLeadingGeometry<Sig::X, Sig::Y, Z>;
+#pragma unroll
+    for (int q = 0; q < kWave / G::GC; q++) {
+        LinearBlock<G::GC * Z> dl;
+        dl.template load<true>(dz + (col0 + q * G::GC) * Z, lane);
+        strip_fence();
+        dl.template to_strip<Z, G::PZ>(strip, lane);
+        strip_fence();
+        if (lane / G::GC == q) {
+#pragma unroll
+            for (int i = 0; i < Z; i++) dzv[i] = strip[(lane % G::GC) * G::PZ + i] * scale;
+        }
+    }
+}
+
+template <typename Sig, int WPB>
+__global__ __launch_bounds__(kWave * WPB) void tp_unrolled_bwd_map_leading_kernel(
+    const float *__restrict__ x, const float *__restrict__ y, const float *__restrict__ dz,
+    float *__restrict__ dx, float *__restrict__ dy, int64_t cols, int K, float scale) {
+    constexpr int X = Sig::X, Y = Sig::Y, Z = Sig::Z;
+    using G = TpLeadingGeometry<X, Y, Z>;
+    __shared__ __attribute__((aligned(16))) float strips[WPB * G::REGION];
+    float *strip = strips + threadIdx.y * G::REGION;
+    const int lane = threadIdx.x;
+    const int64_t tile = tp_uniform((int64_t)blockIdx.x * WPB + threadIdx.y);
+    if (tile >= (cols + kWave - 1) / kWave) return;
+    const int64_t col0 = tp_tile_start(tile, cols);
+    float xv[X], yv[Y], dzv[Z], dxv[X], dyv[Y];
+    tp_leading_operands<Sig, false>(x, y, col0, K, 1.f, strip, lane, xv, yv);
+    tp_leading_cotangent<Sig>(dz, col0, scale, strip, lane, dzv);
+#pragma unroll
+    for (int j = 0; j < X; j++) dxv[j] = 0.f;
+#pragma unroll
+    for (int k = 0; k < Y; k++) dyv[k] = 0.f;
+    Sig::bwd(xv, yv, RegLoad<Z>{dzv}, dxv, dyv);
+    float *strip_x = strip, *strip_y = strip + G::XR;
+    strip_fence();
+#pragma unroll
+    for (int j = 0; j < X; j++) strip_x[lane * G::PX + j] = dxv[j];
+#pragma unroll
+    for (int k = 0; k < Y; k++) strip_y[lane * G::PY + k] = dyv[k];
+    strip_fence();
+    LinearBlock<kWave * X> xl;
+    xl.template from_strip<X, G::PX>(strip_x, lane);
+    xl.store(dx + col0 * X, lane);
+    LinearBlock<kWave * Y> yl;
+    yl.template from_strip<Y, G::PY>(strip_y, lane);
+    yl.store(dy + col0 * Y, lane);
+}
+
+// Uniform y, K = 64 * SL with SL in {1, 2, 4}: the SL tiles of a row sit in one block; each
+// wave reduces its 64 channels and the first wave of the row adds the partial sums in a fixed order.
+template <typename Sig, int WPB>
+__global__ __launch_bounds__(kWave * WPB) void tp_unrolled_bwd_uniform_leading_kernel(
+    const float *__restrict__ x, const float *__restrict__ y, const float *__restrict__ dz,
+    float *__restrict__ dx, float *__restrict__ dy, int64_t rows, int K, float scale) {
+    constexpr int X = Sig::X, Y = Sig::Y, Z = Sig::Z;
+    using G = TpLeadingGeometry<X, Y, Z>;
+    using Red = WaveReduce<Y>;
+    __shared__ __attribute__((aligned(16))) float strips[WPB * G::REGION];
+    __shared__ float partial[WPB][Red::P];
+    float *strip = strips + threadIdx.y * G::REGION;
+    const int lane = threadIdx.x, wave = threadIdx.y;
+    const int sl = K / kWave, rpb = WPB / sl;
+    const int slice = wave % sl;
+    const int64_t r = tp_uniform((int64_t)blockIdx.x * rpb + wave / sl);
+    const bool valid = r < rows;  // uniform per wave; every wave reaches the barrier
+    if (valid) {
+        const int64_t col0 = r * K + (int64_t)slice * kWave;
+        float xv[X], yv[Y], dzv[Z], dxv[X], dyv[Red::P];
+        tp_leading_operands<Sig, true>(x, y, col0, K, 1.f, strip, lane, xv, yv);
+        tp_leading_cotangent<Sig>(dz, col0, scale, strip, lane, dzv);
+#pragma unroll
+        for (int j = 0; j < X; j++) dxv[j] = 0.f;
+#pragma unroll
+        for (int k = 0; k < Red::P; k++) dyv[k] = 0.f;
+        Sig::bwd(xv, yv, RegLoad<Z>{dzv}, dxv, dyv);
+        strip_fence();
+#pragma unroll
+        for (int j = 0; j < X; j++) strip[lane * G::PX + j] = dxv[j];
+        strip_fence();
+        LinearBlock<kWave * X> xl;
+        xl.template from_strip<X, G::PX>(strip, lane);
+        xl.store(dx + col0 * X, lane);
+        const float total = Red::run(dyv, lane);
+        if (lane < 16) partial[wave][Red::slot(lane)] = total;
+    }
+    __syncthreads();
+    if (valid && slice == 0 && lane < Y) {
+        float total = partial[wave][lane];
+        for (int s2 = 1; s2 < sl; s2++) total += partial[wave + s2][lane];
+        dy[r * Y + lane] = total;
+    }
+}
+
+template <typename Sig, bool kUniformY>
+int launch_tp_unrolled_fwd_leading(int64_t rows, int channels, float scale, const float *x, const float *y,
+                                   float *z, hipStream_t stream) {
+    constexpr int WPB = 4;
+    const int64_t cols = rows * channels;
+    if (cols < kWave || !tp_leading_channels_ok(channels, false))
+        return set_error(E3J_AMD_INVALID_ARGUMENT, "tensor_product: the leading-layout kernels need a channel "
+                                                   "count that is a multiple of 4 and at least 64 columns");
+    unsigned blocks;
+    if (int rc = tp_grid((cols + kWave - 1) / kWave, WPB, &blocks)) return rc;
+    hipLaunchKernelGGL((tp_unrolled_fwd_leading_kernel<Sig, WPB, kUniformY>), dim3(blocks), dim3(kWave, WPB), 0,
+                       stream, x, y, z, cols, channels, scale);
+    return check_hip(hipGetLastError(), "tensor_product (unrolled, leading) launch");
+}
+
+template <typename Sig, bool kUniformY>
+int launch_tp_unrolled_bwd_leading(int64_t rows, int channels, float scale, const float *x, const float *y,
+                                   const float *dz, float *dx, float *dy, hipStream_t stream) {
+    constexpr int WPB = 4;
+    const int64_t cols = rows * channels;
+    if (cols < kWave || !tp_leading_channels_ok(channels, kUniformY))
+        return set_error(E3J_AMD_INVALID_ARGUMENT, "tensor_product_bwd: channel count outside the "
+                                                   "leading-layout kernels");
+    unsigned blocks;
+    if (kUniformY) {
+        if (int rc = tp_grid(rows, WPB / (channels / kWave), &blocks)) return rc;
+        hipLaunchKernelGGL((tp_unrolled_bwd_uniform_leading_kernel<Sig, WPB>), dim3(blocks), dim3(kWave, WPB), 0,
+                           stream, x, y, dz, dx, dy, rows, channels, scale);
+    } else {
+        if (int rc = tp_grid((cols + kWave - 1) / kWave, WPB, &blocks)) return rc;
+        hipLaunchKernelGGL((tp_unrolled_bwd_map_leading_kernel<Sig, WPB>), dim3(blocks), dim3(kWave, WPB), 0,
+                           stream, x, y, dz, dx, dy, cols, channels, scale);
+    }
+    return check_hip(hipGetLastError(), "tensor_product_bwd (unrolled, leading) launch");
 }
 
 }  // namespace e3j_amd

@@ -88,20 +88,26 @@ def test_tensor_product_argument_errors_need_no_launch():
 def test_tensor_product_signature_lookup():
     from e3j_amd import TensorProduct
     lib = _lib.load()
-    assert lib.e3j_amd_tp_num_signatures() >= 8
+    assert lib.e3j_amd_tp_num_signatures() >= 12
     tp = TensorProduct(("0e+1o+2e+3o", "0e+1o+2e+3o"), "0e+1o+2e+3o")
     packed = tp.packed_coef("float32")
     Z, X, Y = tp.shape
     scale = C.c_float(0)
 
-    def find(buf, channels, uniform, idx_bytes=None):
-        return lib.e3j_amd_tp_find_signature(buf.ctypes.data, idx_bytes or buf.dtype.itemsize, _lib.F32, buf.shape[0],
-                                             X, Y, Z, channels, uniform, C.byref(scale))
+    def find(buf, channels, uniform, layout=_lib.LAYOUT_TRAILING):
+        return lib.e3j_amd_tp_find_signature(buf.ctypes.data, buf.dtype.itemsize, _lib.F32, buf.shape[0],
+                                             X, Y, Z, channels, uniform, layout, C.byref(scale))
     a, b = find(packed, 128, 0), find(packed, 128, 1)
     assert a >= 0 and b >= 0 and a != b and scale.value == 1.0
     assert b"K=128" in lib.e3j_amd_tp_signature_name(a) and b"MAP" in lib.e3j_amd_tp_signature_name(a)
     assert b"without channel axis" in lib.e3j_amd_tp_signature_name(b)
     assert find(packed, 64, 0) >= 0 and find(packed, 96, 0) == -1 and find(packed, 32, 0) == -1
+    # leading layout: one kernel for every multiple of 4 channels (MAP); whole waves per row (uniform y)
+    lead = find(packed, 100, 0, _lib.LAYOUT_LEADING)
+    assert lead >= 0 and lead == find(packed, 4, 0, _lib.LAYOUT_LEADING) and lead not in (a, b)
+    assert b"leading" in lib.e3j_amd_tp_signature_name(lead)
+    assert find(packed, 6, 0, _lib.LAYOUT_LEADING) == -1
+    assert find(packed, 128, 1, _lib.LAYOUT_LEADING) >= 0 and find(packed, 100, 1, _lib.LAYOUT_LEADING) == -1
     from e3j_amd.coef import Coef
     c = Coef.unpack(packed, np.float32)
     assert find(Coef(3.0 * c.val, c.idx, "float32", "int32").pack(), 128, 0) == a and abs(scale.value - 3.0) < 1e-6

@@ -321,3 +321,33 @@ def test_unrolled_and_table_driven_kernels_agree_through_the_c_abi(mode):
     _lib.check(lib.e3j_amd_tensor_product_fwd(ctypes.byref(p), None, x.data_ptr(), y.data_ptr(), z2.data_ptr(), stream))
     torch.cuda.synchronize()
     assert torch.equal(z2, results[0][0])
+
+
+@pytest.mark.parametrize("spaces", BUILTIN, ids=["l2_l2_full", "l2_l3_to_l3", "l3_l3_to_l3"])
+@pytest.mark.parametrize("mode,channels", [("MAP", 4), ("MAP", 12), ("MAP", 64), ("MAP", 100), ("MAP", 128),
+                                           ("OUTER", 64), ("OUTER", 128), ("OUTER", 256)])
+def test_unrolled_leading_kernels_against_the_checker(spaces, mode, channels):
+    from e3j_amd.options import Layout
+    from e3j_amd.tp_ops import _Table
+    rng = np.random.default_rng(22)
+    tp = TensorProduct(spaces[:2], spaces[2], layout="LEADING_CHANNELS", mode=mode)
+    Z, X, Y = tp.shape
+    idx, val = np.asarray(tp.indices, dtype=np.int64), 0.5 * np.asarray(tp.values, dtype=np.float64)
+    table = _Table.get(Coef(val, idx, "float32", "uint8").pack(), np.float32)
+    sig, scale = table.signature(X, Y, Z, channels, mode == "OUTER", Layout.LEADING_CHANNELS)
+    assert sig >= 0 and abs(scale - 0.5) < 1e-6, "a built-in unrolled kernel must serve this table"
+    rows = 77 if channels >= 64 else 53      # 53 * 4 = 212 and 53 * 12 = 636 columns: a moved-back last tile
+    x, y = _operands(rng, mode, "LEADING_CHANNELS", channels, rows=rows, dims=(X, Y), has=(True, False))
+    _check_forward(idx, val, x, y, Z, mode, "LEADING_CHANNELS", "uint8", what=f"leading {mode} K={channels}")
+    _check_backward(idx, val, x, y, Z, mode, "LEADING_CHANNELS", rng, "uint8", what=f"leading {mode} K={channels}")
+
+
+def test_leading_kernels_fall_back_below_one_tile():
+    """Fewer than 64 columns in all: the table-driven kernels serve the call."""
+    rng = np.random.default_rng(23)
+    tp = TensorProduct(("0e+1o+2e", "0e+1o+2e"), None, layout="LEADING_CHANNELS", mode="MAP")
+    Z, X, Y = tp.shape
+    idx, val = np.asarray(tp.indices, dtype=np.int64), np.asarray(tp.values, dtype=np.float64)
+    x, y = _operands(rng, "MAP", "LEADING_CHANNELS", 4, rows=9, dims=(X, Y))
+    _check_forward(idx, val, x, y, Z, "MAP", "LEADING_CHANNELS", "uint8", what="small leading")
+    _check_backward(idx, val, x, y, Z, "MAP", "LEADING_CHANNELS", rng, "uint8", what="small leading")
