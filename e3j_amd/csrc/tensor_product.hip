@@ -226,11 +226,12 @@ int validate_tp(const e3j_amd_tp_params *p, const char *op) {
         return set_error(E3J_AMD_INVALID_ARGUMENT, name + ": unknown signature id " + std::to_string(p->signature));
     if (p->signature >= 0) {
         const TpSignature &sg = tp_signature(p->signature);
-        const bool mode_ok = sg.uniform_y ? (p->mode == E3J_AMD_MODE_OUTER && p->channels_y == 1)
-                                          : (p->mode == E3J_AMD_MODE_MAP && p->channels_y == p->channels_x);
+        const bool mode_ok = sg.uniform_y == 1 ? (p->mode == E3J_AMD_MODE_OUTER && p->channels_y == 1)
+                           : sg.uniform_y == 2 ? (p->mode == E3J_AMD_MODE_INNER && p->channels_y == p->channels_x)
+                                               : (p->mode == E3J_AMD_MODE_MAP && p->channels_y == p->channels_x);
         const bool channels_ok = sg.layout == E3J_AMD_LAYOUT_TRAILING
                                      ? sg.channels == p->channels_x
-                                     : (tp_leading_channels_ok(p->channels_x, sg.uniform_y != 0) &&
+                                     : (tp_leading_channels_ok(p->channels_x, sg.uniform_y) &&
                                         p->num_rows * p->channels_x >= kWave);
         if (!mode_ok || !channels_ok || p->val_dtype != E3J_AMD_F32 || p->layout != sg.layout ||
             sg.num_x != p->num_x || sg.num_y != p->num_y || sg.num_out != p->num_out)
@@ -330,7 +331,7 @@ extern "C" const char *e3j_amd_tp_signature_name(int id) {
 
 extern "C" int e3j_amd_tp_find_signature(const void *coef_host, int32_t coef_idx_bytes, int32_t val_dtype,
                                          int32_t num_coef, int32_t num_x, int32_t num_y, int32_t num_out,
-                                         int32_t channels, int32_t uniform_y, int32_t layout,
+                                         int32_t channels, int32_t kind, int32_t layout,
                                          float *coef_scale) {
     if (coef_scale) *coef_scale = 1.0f;
     if (coef_host == nullptr || val_dtype != E3J_AMD_F32 || num_coef <= 0) return -1;
@@ -340,10 +341,10 @@ extern "C" int e3j_amd_tp_find_signature(const void *coef_host, int32_t coef_idx
     for (int id = 0; id < num_tp_signatures(); id++) {
         const TpSignature &sg = tp_signature(id);
         if (sg.num_coef != num_coef || sg.num_x != num_x || sg.num_y != num_y || sg.num_out != num_out ||
-            sg.layout != layout || sg.uniform_y != (uniform_y != 0))
+            sg.layout != layout || sg.uniform_y != kind)
             continue;
         if (sg.layout == E3J_AMD_LAYOUT_TRAILING ? sg.channels != channels
-                                                 : !tp_leading_channels_ok(channels, uniform_y != 0))
+                                                 : !tp_leading_channels_ok(channels, kind))
             continue;
         // one uniform positive factor is allowed between the tables, taken from the entry of
         // largest magnitude; every entry must agree with it to float32 rounding

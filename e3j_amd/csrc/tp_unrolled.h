@@ -23,7 +23,7 @@ struct TpSignature {
     int32_t num_x, num_y, num_out, num_coef;
     int32_t channels;     // trailing layout: the channel count the kernels were built for;
                           // leading layout: 0, the kernels take the channel count at run time
-    int32_t uniform_y;    // 1: y has no channel axis (OUTER); 0: MAP
+    int32_t uniform_y;    // channel mode: 0 MAP; 1 OUTER with a y without channel axis; 2 INNER
     int32_t layout;
     const float *val;     // (num_coef) table values as float32
     const uint8_t *idx;   // (num_coef, 3) i, j, k
@@ -33,10 +33,10 @@ struct TpSignature {
                float *dx, float *dy, hipStream_t stream);
 };
 // channel counts the leading-layout kernels take: MAP any multiple of 4 (16-byte pieces) with at
-// least 64 columns in all; uniform y: forward the same, backward whole waves per row that fit a block
-inline bool tp_leading_channels_ok(int channels, bool uniform_y) {
+// least 64 columns in all; uniform y and INNER (channel sums): whole waves per row that fit a block
+inline bool tp_leading_channels_ok(int channels, int kind) {
     if (channels < 4 || channels % 4 != 0) return false;
-    return !uniform_y || channels == 64 || channels == 128 || channels == 256;
+    return kind == 0 || channels == 64 || channels == 128 || channels == 256;
 }
 int num_tp_signatures();
 const TpSignature &tp_signature(int id);
@@ -54,6 +54,20 @@ struct RowLoad {
     float scale;
     template <int I>
     __device__ __forceinline__ float get() const { return __builtin_nontemporal_load(p + I * K) * scale; }
+};
+
+// Coordinates kept in registers (results of `fwd`, cotangents for `bwd`).
+template <int Z>
+struct RegStore {
+    float *v;
+    template <int I>
+    __device__ __forceinline__ void put(float a) const { v[I] = a; }
+};
+template <int Z>
+struct RegLoad {
+    const float *v;
+    template <int I>
+    __device__ __forceinline__ float get() const { return v[I]; }
 };
 
 __device__ __forceinline__ int64_t tp_uniform(int64_t v) {
@@ -162,6 +176,91 @@ __global__ __launch_bounds__(kWave * TpUniformGeometry<K>::WPB) void tp_unrolled
     }
 }
 
+// INNER mode, z[r, i] = sum over the channels: a wave per (row, slice) runs the MAP arithmetic
+// on registers, reduces its 64 channels sixteen coordinates at a time, and the slices of a row
+// meet in LDS as in the uniform-y backward.  Its backward is the MAP backward with a
+// wave-uniform cotangent (scalar loads).
+template <int Z>
+struct UniformLoad {
+    const float *p;
+    float scale;
+    template <int I>
+    __device__ __forceinline__ float get() const { return p[I] * scale; }
+};
+
+// sums of zv[0..Z) over the lanes of the wave into out[0..Z) (LDS, one row per wave)
+template <int Z>
+__device__ __forceinline__ void tp_reduce_columns(const float *zv, float *out, int lane) {
+    using Red = WaveReduce<16>;
+#pragma unroll
+    for (int base = 0; base < Z; base += 16) {
+        float part[16];
+#pragma unroll
+        for (int t = 0; t < 16; t++) part[t] = base + t < Z ? zv[base + t] : 0.f;
+        const float total = Red::run(part, lane);
+        const int slot = base + Red::slot(lane);
+        if (lane < 16 && slot < Z) out[slot] = total;
+    }
+}
+
+template <typename Sig, int K>
+__global__ __launch_bounds__(kWave * TpUniformGeometry<K>::WPB) void tp_unrolled_fwd_inner_kernel(
+    const float *__restrict__ x, const float *__restrict__ y, float *__restrict__ z, int64_t rows, float scale) {
+    constexpr int X = Sig::X, Y = Sig::Y, Z = Sig::Z;
+    using G = TpUniformGeometry<K>;
+    __shared__ float partial[G::WPB][Z];
+    const int wave = threadIdx.y, lane = threadIdx.x;
+    const int slice = wave % G::SL;
+    const int64_t r = tp_uniform((int64_t)blockIdx.x * G::RPB + wave / G::SL);
+    const bool valid = r < rows;  // uniform per wave; every wave reaches the barrier
+    if (valid) {
+        const int c0 = slice * kWave + lane;
+        float xv[X], yv[Y], zv[Z];
+        const float *xr = x + r * (X * K) + c0;
+        const float *yr = y + r * (Y * K) + c0;
+#pragma unroll
+        for (int j = 0; j < X; j++) xv[j] = __builtin_nontemporal_load(xr + j * K) * scale;
+#pragma unroll
+        for (int k = 0; k < Y; k++) yv[k] = __builtin_nontemporal_load(yr + k * K);
+        Sig::fwd(xv, yv, RegStore<Z>{zv});
+        tp_reduce_columns<Z>(zv, partial[wave], lane);
+    }
+    __syncthreads();
+    if (valid && slice == 0) {
+        for (int i = lane; i < Z; i += kWave) {
+            float total = partial[wave][i];
+#pragma unroll
+            for (int s2 = 1; s2 < G::SL; s2++) total += partial[wave + s2][i];
+            z[r * Z + i] = total;
+        }
+    }
+}
+
+template <typename Sig, int K, int WPB>
+__global__ __launch_bounds__(kWave * WPB) void tp_unrolled_bwd_inner_kernel(
+    const float *__restrict__ x, const float *__restrict__ y, const float *__restrict__ dz,
+    float *__restrict__ dx, float *__restrict__ dy, int64_t rows, float scale) {
+    constexpr int X = Sig::X, Y = Sig::Y, Z = Sig::Z, SL = K / kWave;
+    const int64_t item = tp_uniform((int64_t)blockIdx.x * WPB + threadIdx.y);
+    if (item >= rows * SL) return;
+    const int64_t r = item / SL;
+    const int c0 = (int)(item % SL) * kWave + threadIdx.x;
+    float xv[X], yv[Y], dxv[X], dyv[Y];
+    const float *xr = x + r * (X * K) + c0;
+    const float *yr = y + r * (Y * K) + c0;
+#pragma unroll
+    for (int j = 0; j < X; j++) { xv[j] = __builtin_nontemporal_load(xr + j * K); dxv[j] = 0.f; }
+#pragma unroll
+    for (int k = 0; k < Y; k++) { yv[k] = __builtin_nontemporal_load(yr + k * K); dyv[k] = 0.f; }
+    Sig::bwd(xv, yv, UniformLoad<Z>{dz + r * Z, scale}, dxv, dyv);
+    float *dxr = dx + r * (X * K) + c0;
+    float *dyr = dy + r * (Y * K) + c0;
+#pragma unroll
+    for (int j = 0; j < X; j++) __builtin_nontemporal_store(dxv[j], dxr + j * K);
+#pragma unroll
+    for (int k = 0; k < Y; k++) __builtin_nontemporal_store(dyv[k], dyr + k * K);
+}
+
 inline int tp_grid(int64_t items, int wpb, unsigned *blocks) {
     const int64_t b = (items + wpb - 1) / wpb;
     if (b > 0x7fffffffLL) return set_error(E3J_AMD_INVALID_ARGUMENT, "tensor_product: too many rows for one launch");
@@ -169,25 +268,37 @@ inline int tp_grid(int64_t items, int wpb, unsigned *blocks) {
     return E3J_AMD_OK;
 }
 
-template <typename Sig, int K, bool kUniformY>
+// kKind: 0 MAP, 1 OUTER with a channel-free y, 2 INNER
+template <typename Sig, int K, int kKind>
 int launch_tp_unrolled_fwd(int64_t rows, int, float scale, const float *x, const float *y, float *z,
                            hipStream_t stream) {
     constexpr int WPB = 4;
     if (rows == 0) return E3J_AMD_OK;
     unsigned blocks;
-    if (int rc = tp_grid(rows * (K / kWave), WPB, &blocks)) return rc;
-    hipLaunchKernelGGL((tp_unrolled_fwd_kernel<Sig, K, WPB, kUniformY>), dim3(blocks), dim3(kWave, WPB), 0, stream,
-                       x, y, z, rows, scale);
+    if (kKind == 2) {
+        using G = TpUniformGeometry<K>;
+        if (int rc = tp_grid(rows, G::RPB, &blocks)) return rc;
+        hipLaunchKernelGGL((tp_unrolled_fwd_inner_kernel<Sig, K>), dim3(blocks), dim3(kWave, G::WPB), 0, stream,
+                           x, y, z, rows, scale);
+    } else {
+        if (int rc = tp_grid(rows * (K / kWave), WPB, &blocks)) return rc;
+        hipLaunchKernelGGL((tp_unrolled_fwd_kernel<Sig, K, WPB, kKind == 1>), dim3(blocks), dim3(kWave, WPB), 0,
+                           stream, x, y, z, rows, scale);
+    }
     return check_hip(hipGetLastError(), "tensor_product (unrolled) launch");
 }
 
-template <typename Sig, int K, bool kUniformY>
+template <typename Sig, int K, int kKind>
 int launch_tp_unrolled_bwd(int64_t rows, int, float scale, const float *x, const float *y, const float *dz,
                            float *dx, float *dy, hipStream_t stream) {
     constexpr int WPB = 4;
     if (rows == 0) return E3J_AMD_OK;
     unsigned blocks;
-    if (kUniformY) {
+    if (kKind == 2) {
+        if (int rc = tp_grid(rows * (K / kWave), WPB, &blocks)) return rc;
+        hipLaunchKernelGGL((tp_unrolled_bwd_inner_kernel<Sig, K, WPB>), dim3(blocks), dim3(kWave, WPB), 0, stream,
+                           x, y, dz, dx, dy, rows, scale);
+    } else if (kKind == 1) {
         using G = TpUniformGeometry<K>;
         if (int rc = tp_grid(rows, G::RPB, &blocks)) return rc;
         hipLaunchKernelGGL((tp_unrolled_bwd_uniform_kernel<Sig, K>), dim3(blocks), dim3(kWave, G::WPB), 0, stream,
@@ -216,19 +327,6 @@ struct TpLeadingGeometry {
     static constexpr int GC = 16;  // columns of z / dz that pass through the strip at a time
     static constexpr int ZR = round4(GC * PZ);
     static constexpr int REGION = XR + YR > ZR ? XR + YR : ZR;
-};
-
-template <int Z>
-struct RegStore {
-    float *v;
-    template <int I>
-    __device__ __forceinline__ void put(float a) const { v[I] = a; }
-};
-template <int Z>
-struct RegLoad {
-    const float *v;
-    template <int I>
-    __device__ __forceinline__ float get() const { return v[I]; }
 };
 
 __device__ __forceinline__ int64_t tp_tile_start(int64_t tile, int64_t cols) {
@@ -313,7 +411,8 @@ __device__ __forceinline__ void tp_leading_cotangent(const float *__restrict__ d
     }
 }
 
-template <typename Sig, int WPB>
+// kInner: the cotangent is (rows, Z), one row per column's row (INNER mode)
+template <typename Sig, int WPB, bool kInner>
 __global__ __launch_bounds__(kWave * WPB) void tp_unrolled_bwd_map_leading_kernel(
     const float *__restrict__ x, const float *__restrict__ y, const float *__restrict__ dz,
     float *__restrict__ dx, float *__restrict__ dy, int64_t cols, int K, float scale) {
@@ -327,7 +426,13 @@ __global__ __launch_bounds__(kWave * WPB) void tp_unrolled_bwd_map_leading_kerne
     const int64_t col0 = tp_tile_start(tile, cols);
     float xv[X], yv[Y], dzv[Z], dxv[X], dyv[Y];
     tp_leading_operands<Sig, false>(x, y, col0, K, 1.f, strip, lane, xv, yv);
-    tp_leading_cotangent<Sig>(dz, col0, scale, strip, lane, dzv);
+    if (kInner) {
+        const float *zr = dz + ((col0 + lane) / K) * Z;
+#pragma unroll
+        for (int i = 0; i < Z; i++) dzv[i] = zr[i] * scale;
+    } else {
+        tp_leading_cotangent<Sig>(dz, col0, scale, strip, lane, dzv);
+    }
 #pragma unroll
     for (int j = 0; j < X; j++) dxv[j] = 0.f;
 #pragma unroll
@@ -393,38 +498,77 @@ __global__ __launch_bounds__(kWave * WPB) void tp_unrolled_bwd_uniform_leading_k
     }
 }
 
-template <typename Sig, bool kUniformY>
+// INNER forward, K = 64 * SL with SL in {1, 2, 4}: as the uniform-y backward, the tiles of a
+// row sit in one block and their channel sums meet in LDS.
+template <typename Sig, int WPB>
+__global__ __launch_bounds__(kWave * WPB) void tp_unrolled_fwd_inner_leading_kernel(
+    const float *__restrict__ x, const float *__restrict__ y, float *__restrict__ z, int64_t rows, int K,
+    float scale) {
+    constexpr int X = Sig::X, Y = Sig::Y, Z = Sig::Z;
+    using G = TpLeadingGeometry<X, Y, Z>;
+    __shared__ __attribute__((aligned(16))) float strips[WPB * G::REGION];
+    __shared__ float partial[WPB][Z];
+    float *strip = strips + threadIdx.y * G::REGION;
+    const int lane = threadIdx.x, wave = threadIdx.y;
+    const int sl = K / kWave, rpb = WPB / sl;
+    const int slice = wave % sl;
+    const int64_t r = tp_uniform((int64_t)blockIdx.x * rpb + wave / sl);
+    const bool valid = r < rows;  // uniform per wave; every wave reaches the barrier
+    if (valid) {
+        float xv[X], yv[Y], zv[Z];
+        tp_leading_operands<Sig, false>(x, y, r * K + (int64_t)slice * kWave, K, scale, strip, lane, xv, yv);
+        Sig::fwd(xv, yv, RegStore<Z>{zv});
+        tp_reduce_columns<Z>(zv, partial[wave], lane);
+    }
+    __syncthreads();
+    if (valid && slice == 0) {
+        for (int i = lane; i < Z; i += kWave) {
+            float total = partial[wave][i];
+            for (int s2 = 1; s2 < sl; s2++) total += partial[wave + s2][i];
+            z[r * Z + i] = total;
+        }
+    }
+}
+
+template <typename Sig, int kKind>
 int launch_tp_unrolled_fwd_leading(int64_t rows, int channels, float scale, const float *x, const float *y,
                                    float *z, hipStream_t stream) {
     constexpr int WPB = 4;
     const int64_t cols = rows * channels;
-    if (cols < kWave || !tp_leading_channels_ok(channels, false))
-        return set_error(E3J_AMD_INVALID_ARGUMENT, "tensor_product: the leading-layout kernels need a channel "
-                                                   "count that is a multiple of 4 and at least 64 columns");
+    if (cols < kWave || !tp_leading_channels_ok(channels, kKind))
+        return set_error(E3J_AMD_INVALID_ARGUMENT, "tensor_product: channel count outside the leading-layout "
+                                                   "kernels (a multiple of 4, at least 64 columns in all; "
+                                                   "64, 128 or 256 where channels are summed)");
     unsigned blocks;
-    if (int rc = tp_grid((cols + kWave - 1) / kWave, WPB, &blocks)) return rc;
-    hipLaunchKernelGGL((tp_unrolled_fwd_leading_kernel<Sig, WPB, kUniformY>), dim3(blocks), dim3(kWave, WPB), 0,
-                       stream, x, y, z, cols, channels, scale);
+    if (kKind == 2) {
+        if (int rc = tp_grid(rows, WPB / (channels / kWave), &blocks)) return rc;
+        hipLaunchKernelGGL((tp_unrolled_fwd_inner_leading_kernel<Sig, WPB>), dim3(blocks), dim3(kWave, WPB), 0,
+                           stream, x, y, z, rows, channels, scale);
+    } else {
+        if (int rc = tp_grid((cols + kWave - 1) / kWave, WPB, &blocks)) return rc;
+        hipLaunchKernelGGL((tp_unrolled_fwd_leading_kernel<Sig, WPB, kKind == 1>), dim3(blocks), dim3(kWave, WPB), 0,
+                           stream, x, y, z, cols, channels, scale);
+    }
     return check_hip(hipGetLastError(), "tensor_product (unrolled, leading) launch");
 }
 
-template <typename Sig, bool kUniformY>
+template <typename Sig, int kKind>
 int launch_tp_unrolled_bwd_leading(int64_t rows, int channels, float scale, const float *x, const float *y,
                                    const float *dz, float *dx, float *dy, hipStream_t stream) {
     constexpr int WPB = 4;
     const int64_t cols = rows * channels;
-    if (cols < kWave || !tp_leading_channels_ok(channels, kUniformY))
+    if (cols < kWave || !tp_leading_channels_ok(channels, kKind))
         return set_error(E3J_AMD_INVALID_ARGUMENT, "tensor_product_bwd: channel count outside the "
                                                    "leading-layout kernels");
     unsigned blocks;
-    if (kUniformY) {
+    if (kKind == 1) {
         if (int rc = tp_grid(rows, WPB / (channels / kWave), &blocks)) return rc;
         hipLaunchKernelGGL((tp_unrolled_bwd_uniform_leading_kernel<Sig, WPB>), dim3(blocks), dim3(kWave, WPB), 0,
                            stream, x, y, dz, dx, dy, rows, channels, scale);
     } else {
         if (int rc = tp_grid((cols + kWave - 1) / kWave, WPB, &blocks)) return rc;
-        hipLaunchKernelGGL((tp_unrolled_bwd_map_leading_kernel<Sig, WPB>), dim3(blocks), dim3(kWave, WPB), 0,
-                           stream, x, y, dz, dx, dy, cols, channels, scale);
+        hipLaunchKernelGGL((tp_unrolled_bwd_map_leading_kernel<Sig, WPB, kKind == 2>), dim3(blocks),
+                           dim3(kWave, WPB), 0, stream, x, y, dz, dx, dy, cols, channels, scale);
     }
     return check_hip(hipGetLastError(), "tensor_product_bwd (unrolled, leading) launch");
 }

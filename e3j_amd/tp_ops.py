@@ -64,10 +64,12 @@ class _Table:
         self._device = {}
         self._signature = {}
 
-    def signature(self, num_x: int, num_y: int, num_out: int, channels: int, uniform_y: bool,
+    def signature(self, num_x: int, num_y: int, num_out: int, channels: int, kind: int,
                   layout: Layout = Layout.TRAILING_CHANNELS):
-        """`(id, scale)` of a built-in unrolled kernel, `(-1, 1.0)` if none matches."""
-        key = (num_x, num_y, num_out, channels, uniform_y, layout)
+        """`(id, scale)` of a built-in unrolled kernel, `(-1, 1.0)` if none matches.  `kind`: 0 MAP,
+        1 OUTER with a channel-free y, 2 INNER."""
+        kind = int(kind)
+        key = (num_x, num_y, num_out, channels, kind, layout)
         hit = self._signature.get(key)
         if hit is None:
             scale = ctypes.c_float(1.0)
@@ -75,7 +77,7 @@ class _Table:
             if self.val_np_dtype == np.float32 and self.num_coef > 0:
                 sig = int(_lib.load().e3j_amd_tp_find_signature(
                     self.packed.ctypes.data, self.idx_bytes, _lib.F32, self.num_coef, num_x, num_y, num_out,
-                    channels, int(uniform_y), layout.value, ctypes.byref(scale)))
+                    channels, kind, layout.value, ctypes.byref(scale)))
             hit = self._signature[key] = (sig, float(scale.value))
         return hit
 
@@ -142,16 +144,18 @@ def _stream(device) -> int:
 def _params(meta: _Meta, x: torch.Tensor, y: torch.Tensor, backward: bool, dz=None) -> _lib.TpParams:
     num_x, cx = meta.dims(x, meta.has_cx)
     num_y, cy = meta.dims(y, meta.has_cy)
-    # unrolled kernels: float32, MAP or OUTER with a channel-free y; the leading-layout ones
+    # unrolled kernels: float32, MAP, OUTER with a channel-free y, or INNER; the leading-layout ones
     # need 64 columns in all and 16-byte aligned operands
     sig, scale = -1, 1.0
     usable = x.dtype == torch.float32 and (
         meta.layout == Layout.TRAILING_CHANNELS or
         (int(x.shape[0]) * cx >= 64 and all(t.data_ptr() % 16 == 0 for t in (x, y, dz) if t is not None)))
     if usable and meta.mode == MixingMode.MAP:
-        sig, scale = meta.table.signature(num_x, num_y, meta.num_out, cx, False, meta.layout)
+        sig, scale = meta.table.signature(num_x, num_y, meta.num_out, cx, 0, meta.layout)
     elif usable and meta.mode == MixingMode.OUTER and cy == 1 and cx > 1:
-        sig, scale = meta.table.signature(num_x, num_y, meta.num_out, cx, True, meta.layout)
+        sig, scale = meta.table.signature(num_x, num_y, meta.num_out, cx, 1, meta.layout)
+    elif usable and meta.mode == MixingMode.INNER:
+        sig, scale = meta.table.signature(num_x, num_y, meta.num_out, cx, 2, meta.layout)
     return _lib.TpParams(
         signature=sig, coef_scale=scale,
         num_rows=int(x.shape[0]), num_coef=meta.table.num_coef, num_x=num_x, num_y=num_y,

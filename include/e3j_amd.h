@@ -253,10 +253,10 @@ int e3j_amd_tensor_product_bwd(const e3j_amd_tp_params *p, const void *coef_bwd,
                                const void *dz, void *dx, void *dy, void *stream);
 
 /* Compile-time-unrolled kernels of the tensor product exist for built-in Clebsch-Gordan tables,
- * float32 and two channel modes, MAP (uniform_y = 0) and OUTER with channels_y == 1
- * (uniform_y = 1): in the trailing layout for the channel counts they were built for (64, 128),
- * in the leading layout for any multiple of 4 channels (uniform_y: 64, 128 or 256), operands
- * 16-byte aligned and num_rows * channels >= 64.  The lookup compares a
+ * float32 and three channel modes, `kind` 0 MAP, 1 OUTER with channels_y == 1, 2 INNER: in the
+ * trailing layout for the channel counts they were built for (64, 128), in the leading layout
+ * for any multiple of 4 channels (kinds 1 and 2, which sum over the channels: 64, 128 or 256),
+ * operands 16-byte aligned and num_rows * channels >= 64.  The lookup compares a
  * packed forward table in HOST memory with the built-in ones (same entries in the same order, up
  * to one positive factor returned in *coef_scale) and returns an id for
  * e3j_amd_tp_params.signature, or -1.  With a signature the `coef` / `coef_bwd` operands of the
@@ -264,7 +264,7 @@ int e3j_amd_tensor_product_bwd(const e3j_amd_tp_params *p, const void *coef_bwd,
  * kernels are table-driven only. */
 int e3j_amd_tp_find_signature(const void *coef_host, int32_t coef_idx_bytes, int32_t val_dtype,
                               int32_t num_coef, int32_t num_x, int32_t num_y, int32_t num_out,
-                              int32_t channels, int32_t uniform_y, int32_t layout, float *coef_scale);
+                              int32_t channels, int32_t kind, int32_t layout, float *coef_scale);
 int e3j_amd_tp_num_signatures(void);
 const char *e3j_amd_tp_signature_name(int id);
 

@@ -88,7 +88,7 @@ def test_tensor_product_argument_errors_need_no_launch():
 def test_tensor_product_signature_lookup():
     from e3j_amd import TensorProduct
     lib = _lib.load()
-    assert lib.e3j_amd_tp_num_signatures() >= 12
+    assert lib.e3j_amd_tp_num_signatures() >= 27
     tp = TensorProduct(("0e+1o+2e+3o", "0e+1o+2e+3o"), "0e+1o+2e+3o")
     packed = tp.packed_coef("float32")
     Z, X, Y = tp.shape
@@ -101,6 +101,7 @@ def test_tensor_product_signature_lookup():
     assert a >= 0 and b >= 0 and a != b and scale.value == 1.0
     assert b"K=128" in lib.e3j_amd_tp_signature_name(a) and b"MAP" in lib.e3j_amd_tp_signature_name(a)
     assert b"without channel axis" in lib.e3j_amd_tp_signature_name(b)
+    assert find(packed, 128, 2) >= 0 and b"INNER" in lib.e3j_amd_tp_signature_name(find(packed, 128, 2))
     assert find(packed, 64, 0) >= 0 and find(packed, 96, 0) == -1 and find(packed, 32, 0) == -1
     # leading layout: one kernel for every multiple of 4 channels (MAP); whole waves per row (uniform y)
     lead = find(packed, 100, 0, _lib.LAYOUT_LEADING)
