@@ -112,6 +112,8 @@ SYMBOLS = {
     "e3j_amd_xla_convolution_bwd": (_P, [_P]),
     "e3j_amd_xla_convolution_bwd_receiver": (_P, [_P]),
     "e3j_amd_xla_convolution_bwd_ordered": (_P, [_P]),
+    "e3j_amd_xla_tensor_product": (_P, [_P]),
+    "e3j_amd_xla_tensor_product_bwd": (_P, [_P]),
 }
 
 _lib = None

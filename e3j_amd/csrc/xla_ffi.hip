@@ -15,6 +15,11 @@
 // Attributes: num_nodes, debug (reference); layout, signature, coef_scale, y_flip,
 // coef_stacked (optional).  Handlers are re-entrant, allocate nothing and
 // enqueue on the stream XLA hands over; they answer the metadata query.
+//
+// The row-wise tensor product (lib/e3j_ops/ffi/e3j_ops.h:124-253,258-372):
+//   "tensor_product":      coef, x, y [, coef_ranges] -> z;  attrs num_out, mode, layout, debug
+//   "tensor_product_bwd":  coef (2, nnz, numel), x, y, dz [, coef_ranges] -> dx, dy;  attrs mode, layout, debug
+// plus the optional attributes signature, coef_scale and coef_sorted (default 1).
 
 #include <cstring>
 
@@ -212,6 +217,55 @@ void *backward_handler(XlaCallFrame *f, Backward mode) {
     return status_to_error(f, rc);
 }
 
+// Sizes of the tensor product from the buffer shapes (lib/e3j_ops/ffi/e3j_ops.h:146-187,285-309).
+void *decode_tensor_product(XlaCallFrame *f, const char *op, const XlaBuffer *coef, const XlaBuffer *x,
+                            const XlaBuffer *y, e3j_amd_tp_params *p, hipStream_t *stream) {
+    const std::string name(op);
+    if (!coef || !x || !y) return make_error(f, E3J_AMD_INVALID_ARGUMENT, name + ": missing or non-buffer operand");
+    if (x->rank < 2 || x->rank > 3 || y->rank < 2 || y->rank > 3 || coef->rank < 2)
+        return make_error(f, E3J_AMD_INVALID_ARGUMENT, name + ": operand rank");
+    std::memset(p, 0, sizeof(*p));
+    bool has_mode = false, has_layout = false;
+    p->mode = attr<int32_t>(f, "mode", kXlaS32, 0, &has_mode);
+    p->layout = attr<int32_t>(f, "layout", kXlaS32, 0, &has_layout);
+    if (!has_mode || !has_layout)
+        return make_error(f, E3J_AMD_INVALID_ARGUMENT, name + ": attributes mode and layout (i32) are required");
+    p->debug = attr<int32_t>(f, "debug", kXlaS32, 0);
+    p->signature = attr<int32_t>(f, "signature", kXlaS32, -1);
+    p->coef_scale = attr<float>(f, "coef_scale", kXlaF32, 1.0f);
+    p->coef_sorted = attr<int32_t>(f, "coef_sorted", kXlaS32, 1);
+    const bool leading = p->layout == E3J_AMD_LAYOUT_LEADING;
+    p->num_rows = x->dims[0];
+    p->num_x = (int32_t)(x->rank == 3 && !leading ? x->dims[1] : x->dims[x->rank - 1]);
+    p->num_y = (int32_t)(y->rank == 3 && !leading ? y->dims[1] : y->dims[y->rank - 1]);
+    p->channels_x = (int32_t)(x->rank == 3 ? (leading ? x->dims[1] : x->dims[2]) : 1);
+    p->channels_y = (int32_t)(y->rank == 3 ? (leading ? y->dims[1] : y->dims[2]) : 1);
+    if (y->dims[0] != p->num_rows)
+        return make_error(f, E3J_AMD_INVALID_ARGUMENT, name + ": x and y must have as many rows");
+    if (coef->dtype == kXlaU8) p->coef_idx_bytes = 1;
+    else if (coef->dtype == kXlaS32) p->coef_idx_bytes = 4;
+    else return make_error(f, E3J_AMD_INVALID_ARGUMENT, "unsupported (IDX, VAL) dtype pair");
+    if (x->dtype == kXlaF32) p->val_dtype = E3J_AMD_F32;
+    else if (x->dtype == kXlaF64) p->val_dtype = E3J_AMD_F64;
+    else return make_error(f, E3J_AMD_INVALID_ARGUMENT, "unsupported (IDX, VAL) dtype pair");
+    if (y->dtype != x->dtype)
+        return make_error(f, E3J_AMD_INVALID_ARGUMENT, name + ": value operands must share one dtype");
+    XlaStreamGetArgs sg;
+    sg.struct_size = sizeof(XlaStreamGetArgs);
+    sg.extension_start = nullptr;
+    sg.ctx = f->ctx;
+    sg.stream = nullptr;
+    if (void *err = f->api->stream_get(&sg)) return err;
+    *stream = static_cast<hipStream_t>(sg.stream);
+    return nullptr;
+}
+
+int64_t tp_out_count(const e3j_amd_tp_params &p) {
+    const int64_t chans = p.mode == E3J_AMD_MODE_OUTER ? (int64_t)p.channels_x * p.channels_y
+                        : p.mode == E3J_AMD_MODE_INNER ? 1 : p.channels_x;
+    return p.num_rows * p.num_out * chans;
+}
+
 }  // namespace
 }  // namespace e3j_amd
 
@@ -243,6 +297,51 @@ void *e3j_amd_xla_convolution(void *call_frame) {
                                            static_cast<const int32_t *>(row_ptr->data), perm_ptr,
                                            out->data, d.stream);
     return status_to_error(f, rc);
+}
+
+void *e3j_amd_xla_tensor_product(void *call_frame) {
+    XlaCallFrame *f = static_cast<XlaCallFrame *>(call_frame);
+    if (answer_metadata(f)) return nullptr;
+    if (f->stage != kXlaStageExecute) return nullptr;
+    if (f->args.size < 3 || f->args.size > 4 || f->rets.size != 1)
+        return make_error(f, E3J_AMD_INVALID_ARGUMENT, "tensor_product: expected 3 or 4 operands and 1 result");
+    const XlaBuffer *coef = arg(f, 0), *x = arg(f, 1), *y = arg(f, 2), *z = ret(f, 0);
+    e3j_amd_tp_params p;
+    hipStream_t stream;
+    if (void *err = decode_tensor_product(f, "tensor_product", coef, x, y, &p, &stream)) return err;
+    bool has_out = false;
+    p.num_out = attr<int32_t>(f, "num_out", kXlaS32, 0, &has_out);
+    if (!has_out) return make_error(f, E3J_AMD_INVALID_ARGUMENT, "tensor_product: attribute num_out (i32) is required");
+    p.num_coef = (int32_t)coef->dims[0];
+    if (!z || z->dtype != x->dtype || count(z) != tp_out_count(p))
+        return make_error(f, E3J_AMD_INVALID_ARGUMENT, "tensor_product: result shape or dtype");
+    return status_to_error(f, e3j_amd_tensor_product_fwd(&p, coef->data, x->data, y->data, z->data, stream));
+}
+
+void *e3j_amd_xla_tensor_product_bwd(void *call_frame) {
+    XlaCallFrame *f = static_cast<XlaCallFrame *>(call_frame);
+    if (answer_metadata(f)) return nullptr;
+    if (f->stage != kXlaStageExecute) return nullptr;
+    if (f->args.size < 4 || f->args.size > 5 || f->rets.size != 2)
+        return make_error(f, E3J_AMD_INVALID_ARGUMENT, "tensor_product_bwd: expected 4 or 5 operands and 2 results");
+    const XlaBuffer *coef = arg(f, 0), *x = arg(f, 1), *y = arg(f, 2), *dz = arg(f, 3);
+    const XlaBuffer *dx = ret(f, 0), *dy = ret(f, 1);
+    e3j_amd_tp_params p;
+    hipStream_t stream;
+    if (void *err = decode_tensor_product(f, "tensor_product_bwd", coef, x, y, &p, &stream)) return err;
+    if (!dz || dz->rank < 2 || dz->dtype != x->dtype)
+        return make_error(f, E3J_AMD_INVALID_ARGUMENT, "tensor_product_bwd: cotangent operand");
+    // the two transposed tables arrive stacked; sizes as the reference takes them (e3j_ops.h:279-283,298-300)
+    const int64_t numel = coef->dims[coef->rank - 1];
+    p.num_coef = (int32_t)(count(coef) / (2 * numel));
+    const bool leading = p.layout == E3J_AMD_LAYOUT_LEADING;
+    p.num_out = (int32_t)(dz->rank == 2 || leading ? dz->dims[dz->rank - 1] : dz->dims[1]);
+    if (dz->dims[0] != p.num_rows || count(dz) != tp_out_count(p))
+        return make_error(f, E3J_AMD_INVALID_ARGUMENT, "tensor_product_bwd: cotangent shape");
+    if (!dx || !dy || count(dx) != count(x) || count(dy) != count(y) || dx->dtype != x->dtype || dy->dtype != x->dtype)
+        return make_error(f, E3J_AMD_INVALID_ARGUMENT, "tensor_product_bwd: result shapes");
+    return status_to_error(f, e3j_amd_tensor_product_bwd(&p, coef->data, x->data, y->data, dz->data, dx->data,
+                                                         dy->data, stream));
 }
 
 void *e3j_amd_xla_convolution_bwd(void *call_frame) {

@@ -275,6 +275,11 @@ void *e3j_amd_xla_convolution(void *call_frame);
 void *e3j_amd_xla_convolution_bwd(void *call_frame);
 void *e3j_amd_xla_convolution_bwd_receiver(void *call_frame);
 void *e3j_amd_xla_convolution_bwd_ordered(void *call_frame);
+/* "tensor_product" / "tensor_product_bwd" (lib/e3j_ops/ffi/e3j_ops.h:238-253,358-372): operands coef,
+ * x, y [, coef_ranges] -> z and coef (two stacked tables), x, y, dz [, coef_ranges] -> dx, dy; attrs
+ * num_out (forward), mode, layout, debug (reference) + signature, coef_scale, coef_sorted (optional). */
+void *e3j_amd_xla_tensor_product(void *call_frame);
+void *e3j_amd_xla_tensor_product_bwd(void *call_frame);
 
 #ifdef __cplusplus
 }

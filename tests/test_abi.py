@@ -220,13 +220,51 @@ def test_find_signature_matches_benchmark_tables():
 def test_xla_metadata_query():
     lib = _lib.load()
     for handler in (lib.e3j_amd_xla_convolution, lib.e3j_amd_xla_convolution_bwd,
-                    lib.e3j_amd_xla_convolution_bwd_receiver):
+                    lib.e3j_amd_xla_convolution_bwd_receiver, lib.e3j_amd_xla_convolution_bwd_ordered,
+                    lib.e3j_amd_xla_tensor_product, lib.e3j_amd_xla_tensor_product_bwd):
         xla = FakeXla()
         frame, md = xla.metadata_frame()
         assert handler(C.addressof(frame)) is None
         assert (md.api_version.major_version, md.api_version.minor_version) == (0, 2)
         assert md.traits == 0 and md.state_type_id == 0
         assert not xla.errors
+
+
+def test_xla_tensor_product_decoding_errors():
+    """Operand and attribute checks of the tensor-product handlers (host addresses, no launch)."""
+    lib = _lib.load()
+    xla = FakeXla()
+    host = np.zeros(4096, dtype=np.float32)
+    coef = xla.buffer(S32, host.ctypes.data, (5, 4))
+    x = xla.buffer(F32, host.ctypes.data, (3, 4, 8))
+    y = xla.buffer(F32, host.ctypes.data, (3, 2, 8))
+    z = xla.buffer(F32, host.ctypes.data, (3, 6, 8))
+    i32 = lambda v: (S32, C.c_int32(v))  # noqa: E731
+    full = {"num_out": i32(6), "mode": i32(2), "layout": i32(1), "debug": i32(0)}
+
+    def run(args, rets, attrs, handler=lib.e3j_amd_xla_tensor_product):
+        frame = xla.frame(args, rets, attrs)
+        assert handler(C.addressof(frame)) is not None
+        return xla.errors[-1]
+
+    assert "3 or 4 operands" in run([coef, x], [z], full)[1]
+    assert "mode and layout" in run([coef, x, y], [z], {"num_out": i32(6)})[1]
+    assert "as many rows" in run([coef, x, xla.buffer(F32, host.ctypes.data, (4, 2, 8))], [z], full)[1]
+    code, msg = run([xla.buffer(F64, host.ctypes.data, (5, 4)), x, y], [z], full)
+    assert code == ERR_INVALID_ARGUMENT and "dtype pair" in msg
+    assert "share one dtype" in run([coef, x, xla.buffer(F64, host.ctypes.data, (3, 2, 8))], [z], full)[1]
+    assert "result shape" in run([coef, x, y], [xla.buffer(F32, host.ctypes.data, (3, 5, 8))], full)[1]
+    assert "same number" in run([coef, x, xla.buffer(F32, host.ctypes.data, (3, 2, 4))],
+                                [z], full)[1]                       # MAP with 8 and 4 channels
+    back = {k: v for k, v in full.items() if k != "num_out"}
+    stacked = xla.buffer(S32, host.ctypes.data, (2, 5, 4))
+    dz_bad = xla.buffer(F32, host.ctypes.data, (3, 6, 4))
+    assert "cotangent shape" in run([stacked, x, y, dz_bad], [x, y], back, lib.e3j_amd_xla_tensor_product_bwd)[1]
+    assert "2 results" in run([stacked, x, y, z], [x], back, lib.e3j_amd_xla_tensor_product_bwd)[1]
+    outer = dict(back, mode=i32(0))
+    dz_outer = xla.buffer(F32, host.ctypes.data, (3, 6, 8, 8))
+    code, msg = run([stacked, x, y, dz_outer], [x, y], outer, lib.e3j_amd_xla_tensor_product_bwd)
+    assert code == ERR_UNIMPLEMENTED and "one channel" in msg
 
 
 def _conv_frame(xla, *, x_dtype=F32, coef_dtype=U8, y_dims=(6, 3), n_attr=4, drop=None, channels=8):

@@ -144,3 +144,60 @@ def test_ordered_backward_target_with_a_signature_and_scratch_result():
         H.assert_parity(g.cpu().numpy(), r, mg, f"ordered {name}")
     err, _ = run(nbytes // 2)                                  # a scratch result that is too small
     assert err is not None and "workspace" in xla.errors[-1][1]
+
+
+@pytest.mark.parametrize("mode,layout", [(2, 1), (0, 1), (1, 0), (2, 0)])
+def test_tensor_product_targets(mode, layout):
+    """"tensor_product" and "tensor_product_bwd" with the reference's operand order and attributes
+    (MAP / OUTER with a channel-free y / INNER; trailing and leading layouts)."""
+    from e3j_amd.coef import Coef
+    from oracle import tp_oracle as T
+    rng = np.random.default_rng(31)
+    R, X, Y, Z, K, nnz = 40, 6, 5, 9, 16, 70
+    idx, val, _ = H.random_table(rng, nnz, X, Y, Z, 3)
+    name = {0: "OUTER", 1: "INNER", 2: "MAP"}[mode]
+    lay = "TRAILING_CHANNELS" if layout == 1 else "LEADING_CHANNELS"
+    x = rng.normal(size=(R, X, K) if layout == 1 else (R, K, X)).astype(np.float32)
+    y = (rng.normal(size=(R, Y)) if mode == 0 else
+         rng.normal(size=(R, Y, K) if layout == 1 else (R, K, Y))).astype(np.float32)
+    ref = T.tensor_product_unfused(idx, val, x.astype(np.float64), y.astype(np.float64), Z, name, lay)
+    mag = T.tensor_product_unfused(idx, np.abs(val), np.abs(x).astype(np.float64), np.abs(y).astype(np.float64),
+                                   Z, name, lay)
+    lib = _lib.load()
+    xla = FakeXla(stream=torch.cuda.current_stream().cuda_stream)
+    c = Coef(val, idx, "float32", "int32")
+    coef = dev(c.pack())
+    xd, yd = dev(x), dev(y)
+    z = torch.full(ref.shape, float("nan"), device="cuda")
+    ranges = dev(np.zeros((0,), dtype=np.int32))
+    attrs = {"num_out": (S32, C.c_int32(Z)), "mode": (S32, C.c_int32(mode)), "layout": (S32, C.c_int32(layout)),
+             "debug": (S32, C.c_int32(1))}
+    frame = xla.frame([_buf(xla, coef, S32), _buf(xla, xd, F32), _buf(xla, yd, F32), _buf(xla, ranges, S32)],
+                      [_buf(xla, z, F32)], attrs)
+    assert lib.e3j_amd_xla_tensor_product(C.addressof(frame)) is None, xla.errors
+    torch.cuda.synchronize()
+    H.assert_parity(z.cpu().numpy(), ref, mag, "xla tensor_product")
+
+    dz = rng.normal(size=ref.shape).astype(np.float32)
+    rdx, rdy = T.tensor_product_vjp(idx, val, x.astype(np.float64), y.astype(np.float64), dz.astype(np.float64), name, lay)
+    mdx, mdy = T.tensor_product_vjp(idx, np.abs(val), np.abs(x).astype(np.float64), np.abs(y).astype(np.float64),
+                                    np.abs(dz).astype(np.float64), name, lay)
+    stacked = dev(np.stack([c.transpose((1, 0, 2)).pack(), c.transpose((2, 0, 1)).pack()]))
+    dx, dy = torch.full_like(xd, float("nan")), torch.full_like(yd, float("nan"))
+    attrs_b = {k: v for k, v in attrs.items() if k != "num_out"}
+    frame_b = xla.frame([_buf(xla, stacked, S32), _buf(xla, xd, F32), _buf(xla, yd, F32), _buf(xla, dev(dz), F32),
+                         _buf(xla, ranges, S32)], [_buf(xla, dx, F32), _buf(xla, dy, F32)], attrs_b)
+    assert lib.e3j_amd_xla_tensor_product_bwd(C.addressof(frame_b)) is None, xla.errors
+    torch.cuda.synchronize()
+    H.assert_parity(dx.cpu().numpy(), rdx, mdx, "xla dx", ulps=32.0)
+    H.assert_parity(dy.cpu().numpy(), rdy, mdy, "xla dy", ulps=32.0)
+
+    # decoding errors come back as XLA errors, nothing is launched
+    bad = xla.frame([_buf(xla, coef, S32), _buf(xla, xd, F32), _buf(xla, yd, F32)], [_buf(xla, z, F32)],
+                    {k: v for k, v in attrs.items() if k != "num_out"})
+    assert lib.e3j_amd_xla_tensor_product(C.addressof(bad)) is not None
+    assert "num_out" in xla.errors[-1][1]
+    wrong = torch.zeros(3, device="cuda")
+    bad = xla.frame([_buf(xla, coef, S32), _buf(xla, xd, F32), _buf(xla, yd, F32)], [_buf(xla, wrong, F32)], attrs)
+    assert lib.e3j_amd_xla_tensor_product(C.addressof(bad)) is not None
+    assert "result shape" in xla.errors[-1][1]
