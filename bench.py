@@ -70,6 +70,12 @@ def parse_args():
                     help="cfg3, 128 channels, trailing layout only: also time kernels that perform the "
                          "memory accesses of the two passes without their arithmetic (reported under "
                          "roofline.access_floor)")
+    ap.add_argument("--op", default="convolution", choices=["convolution", "tensor_product"],
+                    help="convolution: the headline benchmark; tensor_product: a secondary figure, the "
+                         "row-wise product on the same table (0e+1o+2e+3o squared, l <= 3, 128 channels)")
+    ap.add_argument("--mode", default="MAP", choices=["MAP", "OUTER", "INNER"],
+                    help="--op tensor_product: channel mode (OUTER: y without channel axis)")
+    ap.add_argument("--rows", type=int, default=1 << 18, help="--op tensor_product: number of rows")
     ap.add_argument("--calibrate-copy", action="store_true",
                     help="also run a 1 GiB device copy, the known-size kernel that hardware "
                          "traffic counters are scaled by")
@@ -241,6 +247,105 @@ def cpu_baseline(w, seconds: float) -> dict:
                       f"({edges} edges) of the same workload, {t:.1f} s"}
 
 
+def calibrate_copy(torch, device) -> None:
+    """A 1 GiB device copy: the kernel of known size that the traffic counters are scaled by."""
+    src = torch.empty(1 << 28, dtype=torch.float32, device=device).normal_()
+    dst = torch.empty_like(src)
+    for _ in range(3):
+        dst.copy_(src)
+    torch.cuda.synchronize()
+    del src, dst
+
+
+def bench_tensor_product(args, torch, device) -> int:
+    """Secondary figure: the row-wise tensor product (forward + VJP) on the benchmark's table."""
+    import numpy as np
+    import e3j_amd
+    from e3j_amd import TensorProduct
+    from e3j_amd.tp_ops import TensorProductParams, _make_meta, _params, _raw_backward, _raw_forward
+    if args.calibrate_copy:
+        calibrate_copy(torch, device)
+    layout = "LEADING_CHANNELS" if args.layout == "leading" else "TRAILING_CHANNELS"
+    trailing = layout == "TRAILING_CHANNELS"
+    K, R = args.channels or 128, args.rows
+    tp = TensorProduct(("0e+1o+2e+3o", "0e+1o+2e+3o"), "0e+1o+2e+3o", layout=layout, mode=args.mode)
+    Z, X, Y = tp.shape
+    coef = tp.packed_coef("float32")
+    params = TensorProductParams(num_out=Z, mode=args.mode, layout=layout)
+    g = torch.Generator(device=device).manual_seed(0)
+    x = torch.randn((R, X, K) if trailing else (R, K, X), device=device, generator=g)
+    has_cy = args.mode != "OUTER"
+    y = torch.randn(((R, Y, K) if trailing else (R, K, Y)) if has_cy else (R, Y), device=device, generator=g)
+    meta = _make_meta(coef, x, y, params)
+    z = _raw_forward(meta, x, y)
+    dz = torch.randn(tuple(z.shape), device=device, generator=g)
+    signature = _params(meta, x, y, backward=False).signature
+    xg, yg = x.detach().requires_grad_(True), y.detach().requires_grad_(True)
+
+    def step():
+        out = e3j_amd.tensor_product(coef, xg, yg, params)
+        return torch.autograd.grad(out, (xg, yg), dz)
+
+    for _ in range(args.warmup):
+        step()
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for _ in range(args.steps):
+        step()
+    torch.cuda.synchronize()
+    ms_per_step = (time.perf_counter() - t0) * 1e3 / args.steps
+    fwd_ms = time_events(torch, lambda: _raw_forward(meta, x, y), args.steps, 2)
+    bwd_ms = time_events(torch, lambda: _raw_backward(meta, x, y, dz), args.steps, 2)
+    fwd_bytes = 4 * (x.numel() + y.numel() + z.numel())
+    bwd_bytes = 4 * (2 * x.numel() + 2 * y.numel() + z.numel())
+
+    def gbs(nbytes, ms):
+        return nbytes / (ms * 1e-3) / 1e9
+
+    result = {
+        "metric": "rows/sec fused TensorProduct fwd+VJP fp32; achieved HBM GB/s vs peak",
+        "value": R / (ms_per_step * 1e-3), "unit": "rows/s", "n_gpus": 1, "steps": args.steps,
+        "warmup": args.warmup, "ms_per_step": ms_per_step, "higher_is_better": True, "scaling": "weak",
+        "vs_baseline": None, "dtype": "f32", "data": "synthetic",
+        "config": {"workload": f"row-wise tensor product 0e+1o+2e+3o (x) 0e+1o+2e+3o -> l <= 3 ({len(tp.values)} "
+                               f"coefficients, {Z} output coordinates), {R} rows, {K} channels, mode {args.mode}, "
+                               f"{args.layout}-channels layout, forward + VJP (dx, dy)",
+                   "signature": signature,
+                   "signature_name": (_lib_name(signature) if signature >= 0 else "table-driven kernel")},
+        "roofline": {"bound": "hbm", "kernel": "tensor product backward (dz read once for dx and dy)",
+                     "achieved": gbs(bwd_bytes, bwd_ms), "peak": HBM_PEAK_GBS, "unit": "GB/s",
+                     "frac": gbs(bwd_bytes, bwd_ms) / HBM_PEAK_GBS, "traffic": None,
+                     "algorithmic_bytes": bwd_bytes, "ms": bwd_ms,
+                     "forward": {"achieved": gbs(fwd_bytes, fwd_ms), "frac": gbs(fwd_bytes, fwd_ms) / HBM_PEAK_GBS,
+                                 "algorithmic_bytes": fwd_bytes, "ms": fwd_ms},
+                     "forward_plus_backward": {"achieved": gbs(fwd_bytes + bwd_bytes, fwd_ms + bwd_ms),
+                                               "frac": gbs(fwd_bytes + bwd_bytes, fwd_ms + bwd_ms) / HBM_PEAK_GBS,
+                                               "algorithmic_bytes": fwd_bytes + bwd_bytes, "ms": fwd_ms + bwd_ms}},
+    }
+    if not args.no_cpu_baseline:
+        from oracle import tp_oracle
+        idx, val = np.asarray(tp.indices, dtype=np.int64), np.asarray(tp.values, dtype=np.float32)
+        rows = 2048
+        xs, ys, dzs = (t[:rows].cpu().numpy() for t in (x, y, dz))
+        t0 = time.perf_counter()
+        reps = 0
+        while time.perf_counter() - t0 < args.cpu_seconds:
+            tp_oracle.tensor_product_unfused(idx, val, xs, ys, Z, args.mode, layout)
+            tp_oracle.tensor_product_vjp(idx, val, xs, ys, dzs, args.mode, layout)
+            reps += 1
+        elapsed = time.perf_counter() - t0
+        result["cpu_baseline"] = {"value": rows * reps / elapsed, "unit": "rows/s", "cores": 1, "kind": "port",
+                                  "sample": f"forward + VJP of the numpy restatement on the first {rows} rows, "
+                                            f"{reps} repetitions, {elapsed:.1f} s"}
+    print(json.dumps(result))
+    return 0
+
+
+def _lib_name(signature: int) -> str:
+    from e3j_amd import _lib
+    return _lib.load().e3j_amd_tp_signature_name(signature).decode()
+
+
 def main():
     args = parse_args()
     if args.gpus != 1:
@@ -256,6 +361,8 @@ def main():
     _lib.load()  # fail loudly when the HIP library is missing
     device = torch.device("cuda:0")
     torch.cuda.set_device(device)
+    if args.op == "tensor_product":
+        return bench_tensor_product(args, torch, device)
 
     w = build_workload(args.config, args.scale, device, args.spatial_sort, args.channels)
     w = w.with_layout("LEADING_CHANNELS" if args.layout == "leading" else "TRAILING_CHANNELS")
@@ -277,12 +384,7 @@ def main():
         return out, grads
 
     if args.calibrate_copy:
-        src = torch.empty(1 << 28, dtype=torch.float32, device=device).normal_()
-        dst = torch.empty_like(src)
-        for _ in range(3):
-            dst.copy_(src)
-        torch.cuda.synchronize()
-        del src, dst
+        calibrate_copy(torch, device)
 
     abi = AbiCalls(w)
     if args.deterministic:
