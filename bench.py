@@ -247,6 +247,13 @@ def cpu_baseline(w, seconds: float) -> dict:
                       f"({edges} edges) of the same workload, {t:.1f} s"}
 
 
+#: the same for `--op tensor_product` (MAP, trailing layout, 262 144 rows, 128 channels)
+MEASURED_TP_TRAFFIC_BYTES = {
+    ("MAP", "trailing", 1 << 18, 128): {"forward": 2.0 * 2.097e6 * 1024 + 1.299e7 * 1024,
+                                        "backward": 2.0 * 8.585e6 * 1024 + 4.194e6 * 1024},
+}
+
+
 def calibrate_copy(torch, device) -> None:
     """A 1 GiB device copy: the kernel of known size that the traffic counters are scaled by."""
     src = torch.empty(1 << 28, dtype=torch.float32, device=device).normal_()
@@ -302,6 +309,7 @@ def bench_tensor_product(args, torch, device) -> int:
     def gbs(nbytes, ms):
         return nbytes / (ms * 1e-3) / 1e9
 
+    measured = MEASURED_TP_TRAFFIC_BYTES.get((args.mode, args.layout, R, K), {})
     result = {
         "metric": "rows/sec fused TensorProduct fwd+VJP fp32; achieved HBM GB/s vs peak",
         "value": R / (ms_per_step * 1e-3), "unit": "rows/s", "n_gpus": 1, "steps": args.steps,
@@ -314,9 +322,10 @@ def bench_tensor_product(args, torch, device) -> int:
                    "signature_name": (_lib_name(signature) if signature >= 0 else "table-driven kernel")},
         "roofline": {"bound": "hbm", "kernel": "tensor product backward (dz read once for dx and dy)",
                      "achieved": gbs(bwd_bytes, bwd_ms), "peak": HBM_PEAK_GBS, "unit": "GB/s",
-                     "frac": gbs(bwd_bytes, bwd_ms) / HBM_PEAK_GBS, "traffic": None,
+                     "frac": gbs(bwd_bytes, bwd_ms) / HBM_PEAK_GBS, "traffic": measured.get("backward"),
                      "algorithmic_bytes": bwd_bytes, "ms": bwd_ms,
                      "forward": {"achieved": gbs(fwd_bytes, fwd_ms), "frac": gbs(fwd_bytes, fwd_ms) / HBM_PEAK_GBS,
+                                 "traffic": measured.get("forward"),
                                  "algorithmic_bytes": fwd_bytes, "ms": fwd_ms},
                      "forward_plus_backward": {"achieved": gbs(fwd_bytes + bwd_bytes, fwd_ms + bwd_ms),
                                                "frac": gbs(fwd_bytes + bwd_bytes, fwd_ms + bwd_ms) / HBM_PEAK_GBS,
