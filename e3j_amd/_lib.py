@@ -107,6 +107,7 @@ SYMBOLS = {
     "e3j_amd_tensor_product_bwd": (ctypes.c_int, [_TP_PARAMS] + [_P] * 7),
     "e3j_amd_tp_find_signature": (ctypes.c_int, [_P] + [ctypes.c_int32] * 9 + [ctypes.POINTER(ctypes.c_float)]),
     "e3j_amd_tp_num_signatures": (ctypes.c_int, []),
+    "e3j_amd_tp_register_signature": (ctypes.c_int, [_P]),
     "e3j_amd_tp_signature_name": (ctypes.c_char_p, [ctypes.c_int]),
     "e3j_amd_xla_convolution": (_P, [_P]),
     "e3j_amd_xla_convolution_bwd": (_P, [_P]),

@@ -14,11 +14,32 @@
 
 #include <cmath>
 #include <cstring>
+#include <deque>
 #include <initializer_list>
+#include <mutex>
 
 #include "tp_unrolled.h"
 
 namespace e3j_amd {
+
+// Signatures registered at run time live behind the built-in ones.  The list only grows and a
+// deque never moves its elements, so ids and references stay valid.
+namespace {
+std::mutex g_tp_registry_mutex;
+std::deque<const TpSignature *> g_tp_registered;
+}  // namespace
+
+int num_tp_signatures() {
+    std::lock_guard<std::mutex> lock(g_tp_registry_mutex);
+    return num_builtin_tp_signatures() + (int)g_tp_registered.size();
+}
+
+const TpSignature &tp_signature(int id) {
+    if (id < num_builtin_tp_signatures()) return builtin_tp_signature(id);
+    std::lock_guard<std::mutex> lock(g_tp_registry_mutex);
+    return *g_tp_registered[id - num_builtin_tp_signatures()];
+}
+
 namespace {
 
 // Packed (val, i, j, k) entry: field order and padding of
@@ -324,6 +345,18 @@ extern "C" int e3j_amd_tensor_product_bwd(const e3j_amd_tp_params *p, const void
 }
 
 extern "C" int e3j_amd_tp_num_signatures(void) { return num_tp_signatures(); }
+
+extern "C" int e3j_amd_tp_register_signature(const void *entry) {
+    const TpSignature *sg = static_cast<const TpSignature *>(entry);
+    if (sg == nullptr || sg->fwd == nullptr || sg->bwd == nullptr || sg->val == nullptr || sg->idx == nullptr ||
+        sg->num_coef <= 0 || sg->uniform_y < 0 || sg->uniform_y > 2) {
+        set_error(E3J_AMD_INVALID_ARGUMENT, "tp_register_signature: incomplete entry");
+        return -1;
+    }
+    std::lock_guard<std::mutex> lock(g_tp_registry_mutex);
+    g_tp_registered.push_back(sg);
+    return num_builtin_tp_signatures() + (int)g_tp_registered.size() - 1;
+}
 
 extern "C" const char *e3j_amd_tp_signature_name(int id) {
     return (id >= 0 && id < num_tp_signatures()) ? tp_signature(id).name : "";

@@ -38,6 +38,9 @@ inline bool tp_leading_channels_ok(int channels, int kind) {
     if (channels < 4 || channels % 4 != 0) return false;
     return kind == 0 || channels == 64 || channels == 128 || channels == 256;
 }
+// built-in signatures (generated/tp_registry.hip), then the ones registered at run time
+int num_builtin_tp_signatures();
+const TpSignature &builtin_tp_signature(int id);
 int num_tp_signatures();
 const TpSignature &tp_signature(int id);
 

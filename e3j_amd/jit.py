@@ -24,7 +24,7 @@ import numpy as np
 
 from . import _lib
 from . import build as _build
-from .codegen import gen_conv
+from .codegen import gen_conv, gen_tp
 
 #: where compiled signature libraries are kept (in-tree by default, so that they travel with it)
 CACHE_DIR = os.environ.get("E3J_AMD_JIT_CACHE", os.path.join(_build.HERE, "lib", "jit"))
@@ -119,6 +119,80 @@ def register(val, idx4, dims, channels: int) -> list[int]:
             entry = plugin.e3j_amd_plugin_signature(which)
             if entry:
                 sig = main.e3j_amd_register_signature(entry)
+                if sig >= 0:
+                    ids.append(int(sig))
+        _loaded[key] = (plugin, ids)
+        return ids
+
+
+# ---------------------------------------------------------------------------
+# row-wise tensor product
+# ---------------------------------------------------------------------------
+def _tp_key(val: np.ndarray, idx: np.ndarray, shape, channels: int) -> str:
+    h = hashlib.sha256()
+    h.update(b"tensor_product")
+    h.update(np.ascontiguousarray(val, dtype=np.float32).tobytes())
+    h.update(np.ascontiguousarray(idx, dtype=np.int64).tobytes())
+    h.update(repr((tuple(int(d) for d in shape), int(channels))).encode())
+    for path in (gen_tp.__file__, os.path.join(_build.CSRC, "tp_unrolled.h"),
+                 os.path.join(_build.CSRC, "unrolled.h"), os.path.join(_build.CSRC, "common.h")):
+        with open(path, "rb") as fh:
+            h.update(fh.read())
+    return h.hexdigest()[:20]
+
+
+def tp_signature_library(val, idx, shape, channels: int, build: bool = True) -> str | None:
+    """Path of the compiled tensor-product library of a table `(val; i, j, k)` with dense shape
+    `(num_out, num_x, num_y)`: trailing-layout kernels for `channels` (a multiple of 64), or the
+    leading-layout kernels (any channel count) for `channels` 0.  None when the kernel templates
+    cannot take the table."""
+    num_out, num_x, num_y = (int(d) for d in shape)
+    idx = np.asarray(idx)
+    if not gen_tp.supports(num_x, num_y, num_out, channels or 64) or idx.max(initial=0) > 255 or not len(val):
+        return None
+    key = _tp_key(val, idx, shape, channels)
+    path = os.path.join(CACHE_DIR, key, "signature.so")
+    if not os.path.exists(path):
+        if not build:
+            return None
+        name = f"jit_{key}"
+        where = f"K={channels}, trailing" if channels else "leading"
+        desc = f"{name}: run-time table (x {num_x}, y {num_y}, out {num_out}), {where}, nnz={len(val)}"
+        symbols = tuple(f"kTp_{key}_{t}" for t in range(3))
+        source = gen_tp.emit_source(name, desc, np.asarray(val, dtype=np.float32), idx, (num_out, num_x, num_y),
+                                    channels, symbols, include='"tp_unrolled.h"', plugin=True)
+        _compile(source, path)
+    return path
+
+
+def register_tp(val, idx, shape, channels: int) -> list[int]:
+    """Compile (or find in the cache) and register the tensor-product kernels of a table (MAP,
+    channel-free y, INNER); `channels` 0 = the leading layout.  Ids of the new signatures, empty
+    when the table cannot be served."""
+    key = _tp_key(val, idx, shape, channels)
+    with _lock:
+        if key in _loaded:
+            return _loaded[key][1]
+        if key in _failed:
+            return []
+        try:
+            path = tp_signature_library(val, idx, shape, channels)
+        except (RuntimeError, OSError) as err:
+            warnings.warn(f"e3j_amd: no run-time kernels for this table ({err}); "
+                          "the table-driven kernels serve it", RuntimeWarning)
+            path = None
+        if path is None:
+            _failed.add(key)
+            return []
+        main = _lib.load()
+        plugin = ctypes.CDLL(path, mode=ctypes.RTLD_LOCAL)
+        plugin.e3j_amd_tp_plugin_signature.restype = ctypes.c_void_p
+        plugin.e3j_amd_tp_plugin_signature.argtypes = [ctypes.c_int]
+        ids = []
+        for which in range(3):
+            entry = plugin.e3j_amd_tp_plugin_signature(which)
+            if entry:
+                sig = main.e3j_amd_tp_register_signature(entry)
                 if sig >= 0:
                     ids.append(int(sig))
         _loaded[key] = (plugin, ids)

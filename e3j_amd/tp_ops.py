@@ -69,15 +69,27 @@ class _Table:
         """`(id, scale)` of a built-in unrolled kernel, `(-1, 1.0)` if none matches.  `kind`: 0 MAP,
         1 OUTER with a channel-free y, 2 INNER."""
         kind = int(kind)
-        key = (num_x, num_y, num_out, channels, kind, layout)
+        key = (num_x, num_y, num_out, channels, kind, layout, config().jit)
         hit = self._signature.get(key)
         if hit is None:
             scale = ctypes.c_float(1.0)
             sig = -1
-            if self.val_np_dtype == np.float32 and self.num_coef > 0:
-                sig = int(_lib.load().e3j_amd_tp_find_signature(
+
+            def find():
+                return int(_lib.load().e3j_amd_tp_find_signature(
                     self.packed.ctypes.data, self.idx_bytes, _lib.F32, self.num_coef, num_x, num_y, num_out,
                     channels, kind, layout.value, ctypes.byref(scale)))
+
+            if self.val_np_dtype == np.float32 and self.num_coef > 0:
+                sig = find()
+                if sig < 0 and config().jit:
+                    # not built in: generate and compile the kernels of this table, then look again
+                    from . import jit as _jit
+                    c = Coef.unpack(self.packed, self.val_np_dtype)
+                    trailing = layout == Layout.TRAILING_CHANNELS
+                    if (channels % 64 == 0 or not trailing) and _jit.register_tp(
+                            c.val, c.idx.astype(np.int64), (num_out, num_x, num_y), channels if trailing else 0):
+                        sig = find()
             hit = self._signature[key] = (sig, float(scale.value))
         return hit
 

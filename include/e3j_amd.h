@@ -267,6 +267,10 @@ int e3j_amd_tp_find_signature(const void *coef_host, int32_t coef_idx_bytes, int
                               int32_t channels, int32_t kind, int32_t layout, float *coef_scale);
 int e3j_amd_tp_num_signatures(void);
 const char *e3j_amd_tp_signature_name(int id);
+/* Adds the kernels of one table compiled at run time (an entry produced by the generator of this
+ * library, `e3j_amd/codegen/gen_tp.py`, living in a shared library that stays loaded); returns
+ * its id or -1.  The counterpart of e3j_amd_register_signature for the tensor product. */
+int e3j_amd_tp_register_signature(const void *entry);
 
 /* XLA-FFI handlers (C ABI of xla/ffi/api/c_api.h): `XLA_FFI_Error* handler(XLA_FFI_CallFrame*)`.
  * Operand order of "convolution"/"convolution_bwd" as in lib/e3j_ops/ffi/e3j_ops.h:457-472,575-594;

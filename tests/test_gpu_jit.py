@@ -84,3 +84,40 @@ def test_module_with_irreps_outside_the_built_in_tables():
         fast = run()
     for a, b in zip(slow, fast):
         assert float((a - b).detach().abs().max()) <= 2e-5 * float(a.detach().abs().max())
+
+
+@pytest.mark.parametrize("layout,channels", [("TRAILING_CHANNELS", 64), ("TRAILING_CHANNELS", 128),
+                                             ("LEADING_CHANNELS", 12), ("LEADING_CHANNELS", 128)])
+@pytest.mark.parametrize("mode", ["MAP", "OUTER", "INNER"])
+def test_tensor_product_tables_run_on_generated_kernels(mode, layout, channels):
+    from e3j_amd.coef import Coef
+    from e3j_amd.tp_ops import TensorProductParams, _Table as TpTable
+    from oracle import tp_oracle as T
+    if layout == "LEADING_CHANNELS" and channels == 12 and mode != "MAP":
+        pytest.skip("channel sums in the leading layout need whole waves per row")
+    rng = np.random.default_rng(5)
+    X, Y, Z, nnz, R = 5, 6, 11, 70, 90
+    idx, val, _ = H.random_table(rng, nnz, X, Y, Z, 3)
+    coef = Coef(val, idx, "float32", "uint8").pack()
+    tr = layout == "TRAILING_CHANNELS"
+    x = rng.normal(size=(R, X, channels) if tr else (R, channels, X)).astype(np.float32)
+    y = (rng.normal(size=(R, Y)) if mode == "OUTER" else
+         rng.normal(size=(R, Y, channels) if tr else (R, channels, Y))).astype(np.float32)
+    kind = {"MAP": 0, "OUTER": 1, "INNER": 2}[mode]
+    p = TensorProductParams(num_out=Z, mode=mode, layout=layout)
+    with e3j_amd.config.use(jit=True):
+        sig = TpTable.get(coef, np.float32).signature(X, Y, Z, channels, kind, e3j_amd.Layout.parse(layout))[0]
+        assert sig >= 0, "the table must run on kernels compiled for it"
+        xt, yt = dev(x).requires_grad_(True), dev(y).requires_grad_(True)
+        z = e3j_amd.tensor_product(coef, xt, yt, p)
+        dz = rng.normal(size=tuple(z.shape)).astype(np.float32)
+        dx, dy = torch.autograd.grad(z, (xt, yt), dev(dz))
+    f64 = lambda a: a.astype(np.float64)  # noqa: E731
+    val_r = val.astype(np.float32).astype(np.float64)
+    ref = T.tensor_product_unfused(idx, val_r, f64(x), f64(y), Z, mode, layout)
+    mag = T.tensor_product_unfused(idx, np.abs(val_r), np.abs(f64(x)), np.abs(f64(y)), Z, mode, layout)
+    H.assert_parity(z.detach().cpu().numpy(), ref, mag, "z")
+    rdx, rdy = T.tensor_product_vjp(idx, val_r, f64(x), f64(y), f64(dz), mode, layout)
+    mdx, mdy = T.tensor_product_vjp(idx, np.abs(val_r), np.abs(f64(x)), np.abs(f64(y)), np.abs(f64(dz)), mode, layout)
+    H.assert_parity(dx.cpu().numpy(), rdx, mdx, "dx", ulps=32.0)
+    H.assert_parity(dy.cpu().numpy(), rdy, mdy, "dy", ulps=32.0)

@@ -317,3 +317,30 @@ def test_run_time_signature_compiles_and_registers():
     cb = big.coef
     assert jit.register(np.asarray(cb.val, np.float32), np.asarray(cb.idx, np.int64),
                         (4, 25, big.params.num_out, big.params.num_scalars), 64) == []
+
+
+def test_run_time_tensor_product_signature_compiles_and_registers():
+    """The tensor-product generator's output for a table outside the built-in ones compiles,
+    loads and is found by the lookup, in both layouts (no GPU needed)."""
+    import ctypes
+    from e3j_amd import TensorProduct, _lib, jit
+    tp = TensorProduct(("0e+1o", "0e+1o"), None)
+    val, idx = np.asarray(tp.values, np.float32), np.asarray(tp.indices, np.int64)
+    Z, X, Y = tp.shape
+    lib = _lib.load()
+    packed = tp.packed_coef("float32")
+    scale = ctypes.c_float(0)
+
+    def find(channels, kind, layout):
+        return lib.e3j_amd_tp_find_signature(packed.ctypes.data, packed.dtype.itemsize, _lib.F32, packed.shape[0],
+                                             X, Y, Z, channels, kind, layout, ctypes.byref(scale))
+    assert find(64, 0, 1) == -1
+    ids = jit.register_tp(val, idx, tp.shape, 64)
+    assert len(ids) == 3 and ids == jit.register_tp(val, idx, tp.shape, 64)
+    assert [find(64, kind, 1) for kind in (0, 1, 2)] == ids and scale.value == 1.0
+    assert b"run-time table" in lib.e3j_amd_tp_signature_name(ids[0])
+    assert find(128, 0, 1) == -1 and find(64, 0, 0) == -1       # other channel count / layout: not built
+    lead = jit.register_tp(val, idx, tp.shape, 0)               # leading layout: any multiple of 4 channels
+    assert len(lead) == 3 and find(20, 0, 0) == lead[0] and find(128, 2, 0) == lead[2]
+    big = TensorProduct(("0e+1o", "0e+1o+2e+3o+4e"), "0e+1o")   # 25 y components: outside the templates
+    assert jit.register_tp(np.asarray(big.values, np.float32), np.asarray(big.indices, np.int64), big.shape, 64) == []
