@@ -16,7 +16,8 @@ from .options import Config, GraphOrdering, Layout, MixingMode, TensorProductNor
 from .scalar_mixing import ScalarMixing
 from .spaces import O3Irrep, O3Space
 from .tensor_product import TensorProduct
-from .tp_ops import CUDATensorProductParams, TensorProductParams, tensor_product, tensor_product_bwd
+from .tp_ops import (CUDATensorProductParams, TensorProductParams, tensor_product, tensor_product_batched,
+                     tensor_product_bwd)
 
 Space = O3Space
 
@@ -26,5 +27,5 @@ __all__ = [
     "CUDAConvolutionParams", "DUMMY_INDEX", "GraphCSR", "GraphOrdering", "Layout", "O3Irrep",
     "O3Space", "ScalarMixing", "Space", "TensorProduct", "TensorProductNormalization", "config",
     "convolution", "convolution_batched", "convolution_bwd", "resolve_val_dtype",
-    "CUDATensorProductParams", "MixingMode", "TensorProductParams", "tensor_product", "tensor_product_bwd",
+    "CUDATensorProductParams", "MixingMode", "TensorProductParams", "tensor_product", "tensor_product_batched", "tensor_product_bwd",
 ]

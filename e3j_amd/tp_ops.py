@@ -315,4 +315,24 @@ def tensor_product_bwd(coef, x: torch.Tensor, y: torch.Tensor, ct_z: torch.Tenso
     return _TensorProductBwd.apply(x, y, ct_z, meta)
 
 
+def tensor_product_batched(coef, x: torch.Tensor, y: torch.Tensor, params: TensorProductParams,
+                            x_batched: bool = True, y_batched: bool = True) -> torch.Tensor:
+    """Batch on a leading axis, folded into the rows: the counterpart of the reference's batching
+    rule (`src/e3j/ops/tensor_product.py:251-268`).  An operand that is not batched is broadcast
+    over the batch (the asymmetric pattern a Jacobian produces)."""
+    if not (x_batched or y_batched):
+        return tensor_product(coef, x, y, params)
+    batch = x.shape[0] if x_batched else y.shape[0]
+    if not x_batched:
+        x = x.unsqueeze(0).expand((batch,) + tuple(x.shape))
+    if not y_batched:
+        y = y.unsqueeze(0).expand((batch,) + tuple(y.shape))
+    if x.shape[0] != y.shape[0] or x.shape[1] != y.shape[1]:
+        raise ValueError(f"batched operands disagree: x {tuple(x.shape)}, y {tuple(y.shape)}")
+    rows = x.shape[1]
+    out = tensor_product(coef, x.reshape((batch * rows,) + tuple(x.shape[2:])),
+                         y.reshape((batch * rows,) + tuple(y.shape[2:])), params)
+    return out.reshape((batch, rows) + tuple(out.shape[1:]))
+
+
 tensor_product.Params = TensorProductParams

@@ -97,3 +97,41 @@ def test_config3_full_size_properties():
                                w.module.params.num_out)
     got = out[:64].cpu().numpy()
     assert np.abs(got - ref[:64]).max() <= 2e-5 * np.abs(ref[:64]).max()
+
+
+@pytest.mark.parametrize("mode,layout", [("MAP", "TRAILING_CHANNELS"), ("OUTER", "TRAILING_CHANNELS"),
+                                         ("INNER", "TRAILING_CHANNELS"), ("MAP", "LEADING_CHANNELS")])
+def test_tensor_product_benchmark_size_properties(mode, layout):
+    """The row-wise tensor product at the size `bench.py --op tensor_product` runs (262 144 rows,
+    128 channels, l <= 3 table), through properties that do not depend on the size: the Euler
+    identity of a bilinear form <dz, z> = <dx, x> = <dy, y>, linearity in x, bit-identical
+    repetition, and a head of rows against the CPU checker."""
+    from e3j_amd import TensorProduct
+    from e3j_amd.tp_ops import TensorProductParams
+    from oracle import tp_oracle as T
+    R, K = 1 << 18, 128
+    tr = layout == "TRAILING_CHANNELS"
+    tp = TensorProduct(("0e+1o+2e+3o", "0e+1o+2e+3o"), "0e+1o+2e+3o", layout=layout, mode=mode)
+    Z, X, Y = tp.shape
+    coef = tp.packed_coef("float32")
+    p = TensorProductParams(num_out=Z, mode=mode, layout=layout)
+    g = torch.Generator(device="cuda").manual_seed(1)
+    x = torch.randn((R, X, K) if tr else (R, K, X), device="cuda", generator=g)
+    y = torch.randn(((R, Y, K) if tr else (R, K, Y)) if mode != "OUTER" else (R, Y), device="cuda", generator=g)
+    z = e3j_amd.tensor_product(coef, x, y, p)
+    assert torch.equal(z, e3j_amd.tensor_product(coef, x, y, p))
+    dz = torch.randn(tuple(z.shape), device="cuda", generator=g)
+    dx, dy = e3j_amd.tensor_product_bwd(coef, x, y, dz, p)
+    dot = lambda a, b: float((a.double() * b.double()).sum())  # noqa: E731
+    ref = dot(dz, z)
+    scale = float((dz.double().abs() * z.double().abs()).sum())
+    assert abs(dot(dx, x) - ref) <= 1e-6 * scale and abs(dot(dy, y) - ref) <= 1e-6 * scale
+    x2 = torch.randn(tuple(x.shape), device="cuda", generator=g)
+    lin = e3j_amd.tensor_product(coef, x + 2.0 * x2, y, p) - (z + 2.0 * e3j_amd.tensor_product(coef, x2, y, p))
+    assert float(lin.abs().max()) <= 2e-5 * float(z.abs().max())
+    head = 64
+    idx, val = np.asarray(tp.indices, dtype=np.int64), np.asarray(tp.values, dtype=np.float64)
+    xs, ys = x[:head].cpu().numpy().astype(np.float64), y[:head].cpu().numpy().astype(np.float64)
+    want = T.tensor_product_unfused(idx, val, xs, ys, Z, mode, layout)
+    mag = T.tensor_product_unfused(idx, np.abs(val), np.abs(xs), np.abs(ys), Z, mode, layout)
+    H.assert_parity(z[:head].cpu().numpy(), want, mag, f"head {mode} {layout}")

@@ -356,3 +356,19 @@ def test_leading_kernels_fall_back_below_one_tile():
     x, y = _operands(rng, "MAP", "LEADING_CHANNELS", 4, rows=9, dims=(X, Y))
     _check_forward(idx, val, x, y, Z, "MAP", "LEADING_CHANNELS", "uint8", what="small leading")
     _check_backward(idx, val, x, y, Z, "MAP", "LEADING_CHANNELS", rng, "uint8", what="small leading")
+
+
+def test_batched_call_folds_the_batch_into_rows():
+    rng = np.random.default_rng(24)
+    idx, val = _table(nnz=120, dims=(9, 6, 5))
+    coef = Coef(val, idx, "float32", "uint8").pack()
+    p = TensorProductParams(num_out=9, mode="OUTER", layout="TRAILING_CHANNELS")
+    x = torch.from_numpy(rng.normal(size=(3, 17, 6, 8)).astype(np.float32)).to(DEV)
+    y = torch.from_numpy(rng.normal(size=(3, 17, 5)).astype(np.float32)).to(DEV)
+    z = e3j_amd.tensor_product_batched(coef, x, y, p)
+    assert tuple(z.shape) == (3, 17, 9, 8)
+    for b in range(3):
+        assert torch.equal(z[b], e3j_amd.tensor_product(coef, x[b], y[b], p))
+    shared = e3j_amd.tensor_product_batched(coef, x, y[0], p, y_batched=False)   # y broadcast over the batch
+    for b in range(3):
+        assert torch.equal(shared[b], e3j_amd.tensor_product(coef, x[b], y[0], p))
