@@ -361,7 +361,7 @@ def plugin_launch(channels: int):
 
 def supports(t: "Table", channels: int) -> bool:
     """Whether the kernel templates can take this table (register-resident dy sums, bit masks)."""
-    return t.Y <= 16 and t.X <= 64 and t.S <= 64 and t.Z <= 255 and channels >= 1
+    return t.Y <= 64 and t.X <= 64 and t.S <= 64 and t.Z <= 255 and channels >= 1
 
 
 def emit_table_source(t: "Table", name: str, desc: str, channels: int, symbols, include='"../unrolled.h"',

@@ -146,7 +146,7 @@ __global__ __launch_bounds__(kWave * TpUniformGeometry<K>::WPB) void tp_unrolled
     float *__restrict__ dx, float *__restrict__ dy, int64_t rows, float scale) {
     constexpr int X = Sig::X, Y = Sig::Y, Z = Sig::Z;
     using G = TpUniformGeometry<K>;
-    using Red = WaveReduce<Y>;
+    using Red = WaveReduceBlocks<Y>;
     __shared__ float partial[G::WPB][Red::P];
     const int wave = threadIdx.y, lane = threadIdx.x;
     const int slice = wave % G::SL;
@@ -167,8 +167,8 @@ __global__ __launch_bounds__(kWave * TpUniformGeometry<K>::WPB) void tp_unrolled
         float *dxr = dx + r * (X * K) + c0;
 #pragma unroll
         for (int j = 0; j < X; j++) __builtin_nontemporal_store(dxv[j], dxr + j * K);
-        const float total = Red::run(dyv, lane);
-        if (lane < 16) partial[wave][Red::slot(lane)] = total;
+        float *mine = partial[wave];
+        Red::run(dyv, lane, [&](int k, float total) { mine[k] = total; });
     }
     __syncthreads();
     if (valid && slice == 0 && lane < Y) {
@@ -194,16 +194,11 @@ struct UniformLoad {
 // sums of zv[0..Z) over the lanes of the wave into out[0..Z) (LDS, one row per wave)
 template <int Z>
 __device__ __forceinline__ void tp_reduce_columns(const float *zv, float *out, int lane) {
-    using Red = WaveReduce<16>;
+    using Red = WaveReduceBlocks<Z>;
+    float padded[Red::P];
 #pragma unroll
-    for (int base = 0; base < Z; base += 16) {
-        float part[16];
-#pragma unroll
-        for (int t = 0; t < 16; t++) part[t] = base + t < Z ? zv[base + t] : 0.f;
-        const float total = Red::run(part, lane);
-        const int slot = base + Red::slot(lane);
-        if (lane < 16 && slot < Z) out[slot] = total;
-    }
+    for (int t = 0; t < Red::P; t++) padded[t] = t < Z ? zv[t] : 0.f;
+    Red::run(padded, lane, [&](int i, float total) { out[i] = total; });
 }
 
 template <typename Sig, int K>
@@ -464,7 +459,7 @@ __global__ __launch_bounds__(kWave * WPB) void tp_unrolled_bwd_uniform_leading_k
     float *__restrict__ dx, float *__restrict__ dy, int64_t rows, int K, float scale) {
     constexpr int X = Sig::X, Y = Sig::Y, Z = Sig::Z;
     using G = TpLeadingGeometry<X, Y, Z>;
-    using Red = WaveReduce<Y>;
+    using Red = WaveReduceBlocks<Y>;
     __shared__ __attribute__((aligned(16))) float strips[WPB * G::REGION];
     __shared__ float partial[WPB][Red::P];
     float *strip = strips + threadIdx.y * G::REGION;
@@ -490,8 +485,8 @@ __global__ __launch_bounds__(kWave * WPB) void tp_unrolled_bwd_uniform_leading_k
         LinearBlock<kWave * X> xl;
         xl.template from_strip<X, G::PX>(strip, lane);
         xl.store(dx + col0 * X, lane);
-        const float total = Red::run(dyv, lane);
-        if (lane < 16) partial[wave][Red::slot(lane)] = total;
+        float *mine = partial[wave];
+        Red::run(dyv, lane, [&](int k, float total) { mine[k] = total; });
     }
     __syncthreads();
     if (valid && slice == 0 && lane < Y) {

@@ -200,6 +200,7 @@ __device__ __forceinline__ int uniform(int v) { return __builtin_amdgcn_readfirs
 // Negate v when bit k of `flip` is set (the parity signs of the y components when a kernel
 // walks the edges of a symmetric graph in the reversed direction).
 __device__ __forceinline__ float flip_sign(float v, unsigned flip, int k) {
+    if (k >= 32) return v;  // the mask covers 32 components; tables with more carry their signs
     return __uint_as_float(__float_as_uint(v) ^ (((flip >> k) & 1u) << 31));
 }
 
@@ -249,6 +250,26 @@ struct WaveReduce {
         v[0] += __shfl_xor(v[0], 16, kWave);
         v[0] += __shfl_xor(v[0], 32, kWave);
         return v[0];
+    }
+};
+
+// Any number of values: sixteen at a time.  `sink(k, total)` is called on the lanes 0..15 of the
+// wave for the values k they hold (k < NV); `v` must be padded to a multiple of 16.
+template <int NV>
+struct WaveReduceBlocks {
+    static constexpr int P = (NV + 15) / 16 * 16;
+    template <typename Sink>
+    __device__ static __forceinline__ void run(float (&v)[P], int lane, const Sink &sink) {
+        using Red = WaveReduce<16>;
+#pragma unroll
+        for (int base = 0; base < P; base += 16) {
+            float part[16];
+#pragma unroll
+            for (int t = 0; t < 16; t++) part[t] = v[base + t];
+            const float total = Red::run(part, lane);
+            const int k = base + Red::slot(lane);
+            if (lane < 16 && k < NV) sink(k, total);
+        }
     }
 };
 
@@ -412,7 +433,7 @@ __device__ __forceinline__ void unrolled_bwd_part(
     constexpr int X = Part::X, S = Part::S, Z = Part::Z;
     using V = Vec<CPL>;
     using SL = Slice<K, CPL>;
-    using Red = WaveReduce<Y>;
+    using Red = WaveReduceBlocks<Y>;
 
     static_assert(CPL == 1 || SL::FULL, "several channels per lane need whole slices");
     const int c_raw = slice * SL::WIDTH + lane;  // further channels of the lane: + 64, + 128, ...
@@ -492,13 +513,12 @@ __device__ __forceinline__ void unrolled_bwd_part(
                 }
             }
         }
-        const int k = Red::slot(lane);
-        const float total = flip_sign(Red::run(dye, lane), y_flip, k);
-        if (lane < 16 && k < Y) {
+        Red::run(dye, lane, [&](int k, float sum) {
+            const float total = flip_sign(sum, y_flip, k);
             if (!kAtomicDy) dy[ee * Y + k] = total;
             else if (kOrdered) dy[((int64_t)pos * dy_slots + dy_slot) * Y + k] = total;
             else unsafeAtomicAdd(dy + ee * Y + k, total);  // dy zero-filled by the launcher
-        }
+        });
     }
 }
 
@@ -797,7 +817,7 @@ __device__ __forceinline__ void unrolled_bwd_leading(
     static_assert(X <= 64 && S <= 64, "part masks hold 64 columns");
     using G = LeadingBwdGeometry<K, X, S, Z, NP>;
     using V = Vec<1>;
-    using Red = WaveReduce<Y>;
+    using Red = WaveReduceBlocks<Y>;
     constexpr int W = G::W, GC = G::GC, NT = G::NT;
     constexpr int XN = W * X, SN = W * S;
     constexpr bool kAllDx = kCoveredDx == (X == 64 ? ~0ull : ((1ull << X) - 1));
@@ -905,14 +925,13 @@ __device__ __forceinline__ void unrolled_bwd_leading(
 
 #pragma unroll
         for (int k = Y; k < Red::P; k++) dye[k] = 0.f;
-        const int k = Red::slot(lane);
-        const float total = flip_sign(Red::run(dye, lane), y_flip, k);
-        if (lane < 16 && k < Y) {
+        Red::run(dye, lane, [&](int k, float sum) {
             constexpr int SLOTS = NP * G::COUNT;
+            const float total = flip_sign(sum, y_flip, k);
             if (SLOTS == 1) dy[ee * Y + k] = total;
             else if (kOrdered) dy[((int64_t)pos * SLOTS + part * G::COUNT + slice) * Y + k] = total;
             else unsafeAtomicAdd(dy + ee * Y + k, total);  // dy zero-filled by the launcher
-        }
+        });
     }
 }
 

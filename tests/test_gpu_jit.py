@@ -31,6 +31,7 @@ def _random_case(seed, N, E, X, Y, Z, S, K, nnz):
     dict(seed=1, N=40, E=600, X=5, Y=6, Z=7, S=4, K=64, nnz=60),     # whole waves
     dict(seed=2, N=30, E=400, X=3, Y=9, Z=10, S=5, K=48, nnz=80),    # idle lanes; leading: table-driven
     dict(seed=3, N=25, E=300, X=6, Y=4, Z=12, S=6, K=128, nnz=100),  # two channels per lane backward
+    dict(seed=4, N=20, E=250, X=4, Y=25, Z=9, S=5, K=64, nnz=150),   # harmonics up to l = 4: 25 y components
 ])
 def test_random_tables_run_on_generated_kernels(case, layout):
     p = _random_case(**case)
@@ -96,7 +97,7 @@ def test_tensor_product_tables_run_on_generated_kernels(mode, layout, channels):
     if layout == "LEADING_CHANNELS" and channels == 12 and mode != "MAP":
         pytest.skip("channel sums in the leading layout need whole waves per row")
     rng = np.random.default_rng(5)
-    X, Y, Z, nnz, R = 5, 6, 11, 70, 90
+    X, Y, Z, nnz, R = (5, 6, 11, 70, 90) if channels != 128 else (5, 20, 11, 120, 90)   # 20 y components at 128
     idx, val, _ = H.random_table(rng, nnz, X, Y, Z, 3)
     coef = Coef(val, idx, "float32", "uint8").pack()
     tr = layout == "TRAILING_CHANNELS"

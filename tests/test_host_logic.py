@@ -12,6 +12,7 @@ from e3j_amd.clebsch_gordan import (change_basis_real_to_complex, clebsch_gordan
 from e3j_amd.coef import Coef, Coef4D, resolve_val_dtype
 from e3j_amd.sparse import narrow_index_dtype, sparse_coo
 from e3j_amd.tensor_product import block_sort_permutation
+from tests import helpers as H
 
 
 # --- spaces ------------------------------------------------------------------
@@ -312,11 +313,16 @@ def test_run_time_signature_compiles_and_registers():
     assert find(64, 1) == ids[0] and find(64, 0) == ids[1] and scale.value == 1.0
     assert b"run-time table" in lib.e3j_amd_signature_name(ids[0])
     assert find(128, 1) == -1                                     # another channel count: not built
-    # 25 y components exceed the register-resident dy sums of the templates: served table-driven
+    # 25 y components (harmonics up to l = 4): the dy sums are reduced sixteen at a time
     big = Convolution(("0e+1o", "0e+1o+2e+3o+4e"), "0e+1o", graph_ordering="RECEIVER")
     cb = big.coef
-    assert jit.register(np.asarray(cb.val, np.float32), np.asarray(cb.idx, np.int64),
-                        (4, 25, big.params.num_out, big.params.num_scalars), 64) == []
+    assert len(jit.register(np.asarray(cb.val, np.float32), np.asarray(cb.idx, np.int64),
+                            (4, 25, big.params.num_out, big.params.num_scalars), 64)) == 2
+    # more than 255 output coordinates: outside the templates, served table-driven
+    rng = np.random.default_rng(0)
+    idx, val, mix = H.random_table(rng, 400, 4, 5, 300, 7)
+    idx4 = np.concatenate([idx, mix[idx[:, 0]][:, None]], axis=1).astype(np.int64)
+    assert jit.register(np.asarray(val, np.float32), idx4, (4, 5, 300, 7), 64) == []
 
 
 def test_run_time_tensor_product_signature_compiles_and_registers():
@@ -342,5 +348,8 @@ def test_run_time_tensor_product_signature_compiles_and_registers():
     assert find(128, 0, 1) == -1 and find(64, 0, 0) == -1       # other channel count / layout: not built
     lead = jit.register_tp(val, idx, tp.shape, 0)               # leading layout: any multiple of 4 channels
     assert len(lead) == 3 and find(20, 0, 0) == lead[0] and find(128, 2, 0) == lead[2]
-    big = TensorProduct(("0e+1o", "0e+1o+2e+3o+4e"), "0e+1o")   # 25 y components: outside the templates
-    assert jit.register_tp(np.asarray(big.values, np.float32), np.asarray(big.indices, np.int64), big.shape, 64) == []
+    big = TensorProduct(("0e+1o", "0e+1o+2e+3o+4e"), "0e+1o")   # 25 y components: sums reduced 16 at a time
+    assert len(jit.register_tp(np.asarray(big.values, np.float32), np.asarray(big.indices, np.int64),
+                               big.shape, 64)) == 3
+    idx, val, _ = H.random_table(np.random.default_rng(0), 400, 4, 5, 300, 7)   # 300 outputs: outside the templates
+    assert jit.register_tp(np.asarray(val, np.float32), idx.astype(np.int64), (300, 4, 5), 64) == []
