@@ -212,12 +212,34 @@ def _sum(*terms):
     return total
 
 
+def _lead(t: torch.Tensor, dim, batch: int) -> torch.Tensor:
+    """Batch axis first; an operand that is not batched is broadcast over the batch."""
+    if dim is None:
+        return t.unsqueeze(0).expand((batch,) + tuple(t.shape))
+    return t.movedim(dim, 0)
+
+
+def _fold(t: torch.Tensor) -> torch.Tensor:
+    return t.reshape((t.shape[0] * t.shape[1],) + tuple(t.shape[2:]))
+
+
+def _unfold(t: torch.Tensor, batch: int) -> torch.Tensor:
+    return t.reshape((batch, t.shape[0] // batch) + tuple(t.shape[1:]))
+
+
 class _TensorProduct(torch.autograd.Function):
+    """Differentiable to any reverse-mode order; composes with `torch.func` transforms (the
+    batching rule folds the batch into the rows, `src/e3j/ops/tensor_product.py:251-268`)."""
+
     @staticmethod
-    def forward(ctx, x, y, meta):
+    def forward(x, y, meta):
+        return _raw_forward(meta, x, y)
+
+    @staticmethod
+    def setup_context(ctx, inputs, output):
+        x, y, meta = inputs
         ctx.meta = meta
         ctx.save_for_backward(x, y)
-        return _raw_forward(meta, x, y)
 
     @staticmethod
     def backward(ctx, dz):
@@ -229,13 +251,23 @@ class _TensorProduct(torch.autograd.Function):
         dx, dy = _TensorProductBwd.apply(x, y, dz, meta)
         return dx, dy, None
 
+    @staticmethod
+    def vmap(info, in_dims, x, y, meta):
+        batch = info.batch_size
+        out = _TensorProduct.apply(_fold(_lead(x, in_dims[0], batch)), _fold(_lead(y, in_dims[1], batch)), meta)
+        return _unfold(out, batch), 0
+
 
 class _TensorProductBwd(torch.autograd.Function):
     @staticmethod
-    def forward(ctx, x, y, dz, meta):
+    def forward(x, y, dz, meta):
+        return _raw_backward(meta, x, y, dz)
+
+    @staticmethod
+    def setup_context(ctx, inputs, output):
+        x, y, dz, meta = inputs
         ctx.meta = meta
         ctx.save_for_backward(x, y, dz)
-        return _raw_backward(meta, x, y, dz)
 
     @staticmethod
     def backward(ctx, ddx, ddy):
@@ -252,6 +284,13 @@ class _TensorProductBwd(torch.autograd.Function):
         if ctx.needs_input_grad[2]:
             gdz = _sum(_TensorProduct.apply(x, ddy, meta), _TensorProduct.apply(ddx, y, meta))
         return gx, gy, gdz, None
+
+    @staticmethod
+    def vmap(info, in_dims, x, y, dz, meta):
+        batch = info.batch_size
+        dx, dy = _TensorProductBwd.apply(_fold(_lead(x, in_dims[0], batch)), _fold(_lead(y, in_dims[1], batch)),
+                                         _fold(_lead(dz, in_dims[2], batch)), meta)
+        return (_unfold(dx, batch), _unfold(dy, batch)), (0, 0)
 
 
 def _check(x: torch.Tensor, y: torch.Tensor):

@@ -372,3 +372,30 @@ def test_batched_call_folds_the_batch_into_rows():
     shared = e3j_amd.tensor_product_batched(coef, x, y[0], p, y_batched=False)   # y broadcast over the batch
     for b in range(3):
         assert torch.equal(shared[b], e3j_amd.tensor_product(coef, x[b], y[0], p))
+
+
+def test_torch_func_transforms():
+    """vmap over either operand, Jacobians and Hessian-vector products through `torch.func`, as the
+    reference's transform tests do with jax (`tests/test_ops/test_tensor_product_jax_transforms.py`)."""
+    from torch.func import grad, jacrev, vmap
+    rng = np.random.default_rng(25)
+    idx, val = _table(nnz=90, dims=(9, 6, 5))
+    coef = Coef(val, idx, "float64", "int32").pack()
+    p = TensorProductParams(num_out=9, mode="MAP", layout="TRAILING_CHANNELS")
+    dense = _dense_torch(idx, val, 9, (6, 5), "MAP", "TRAILING_CHANNELS", (True, True))
+    f = lambda a, b: e3j_amd.tensor_product(coef, a, b, p)  # noqa: E731
+    x = torch.from_numpy(rng.normal(size=(3, 7, 6, 4))).to(DEV)
+    y = torch.from_numpy(rng.normal(size=(3, 7, 5, 4))).to(DEV)
+    torch.testing.assert_close(vmap(f)(x, y), torch.stack([dense(x[b], y[b]) for b in range(3)]))
+    torch.testing.assert_close(vmap(f, in_dims=(0, None))(x, y[0]), torch.stack([dense(x[b], y[0]) for b in range(3)]))
+    torch.testing.assert_close(vmap(f, in_dims=(None, 0))(x[0], y), torch.stack([dense(x[0], y[b]) for b in range(3)]))
+    # Jacobian of a small product with respect to x (a vmap over the backward operator)
+    xs, ys = x[0, :2], y[0, :2]
+    torch.testing.assert_close(jacrev(f)(xs, ys), jacrev(dense)(xs, ys))
+    # gradient of a scalar of the gradient (second order through the transforms)
+    w = torch.from_numpy(rng.normal(size=(7, 9, 4))).to(DEV)
+    energy = lambda fn: (lambda a, b: (fn(a, b) * w).sum())  # noqa: E731
+    second = lambda fn: grad(lambda a, b: (grad(energy(fn))(a, b) ** 2).sum(), argnums=1)  # noqa: E731
+    torch.testing.assert_close(second(f)(x[0], y[0]), second(dense)(x[0], y[0]))
+    with pytest.raises(RuntimeError):   # forward-mode differentiation is not defined for the operator
+        torch.func.jvp(f, (x[0], y[0]), (x[0], y[0]))
