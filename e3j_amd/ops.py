@@ -206,14 +206,16 @@ def clear_graph_cache() -> None:
     _GRAPH_CACHE.clear()
 
 
-def _forward_graph(meta: _Meta, sender: torch.Tensor, receiver: torch.Tensor):
+def _forward_graph(meta: _Meta, sender: torch.Tensor, receiver: torch.Tensor, build: bool = True):
     """CSR used by the forward kernel: `(other, row_ptr, perm, row_order)`, prepared once per
-    pair of index tensors."""
+    pair of index tensors (`build` off: only looked up, None when it is not there)."""
     key = (id(sender), id(receiver), sender._version, receiver._version, meta.num_nodes,
            meta.ordering, config().locality_rounds)
     hit = _GRAPH_CACHE.get(key)
     if hit is not None and hit[0]() is sender and hit[1]() is receiver:
         return hit[2]
+    if not build:
+        return None
     graph = _prepare_graph(meta, sender, receiver)
     if len(_GRAPH_CACHE) >= _GRAPH_CACHE_SIZE:
         _GRAPH_CACHE.pop(next(iter(_GRAPH_CACHE)))
@@ -323,35 +325,92 @@ def _sum(*terms):
     return total
 
 
+def _lead(t: torch.Tensor, dim, batch: int) -> torch.Tensor:
+    """Batch axis first; an operand that is not batched is broadcast over the batch."""
+    if dim is None:
+        return t.unsqueeze(0).expand((batch,) + tuple(t.shape))
+    return t.movedim(dim, 0)
+
+
+def _fold_rows(t: torch.Tensor) -> torch.Tensor:
+    return t.reshape((t.shape[0] * t.shape[1],) + tuple(t.shape[2:]))
+
+
+def _unfold_rows(t: torch.Tensor, batch: int) -> torch.Tensor:
+    return t.reshape((batch, t.shape[0] // batch) + tuple(t.shape[1:]))
+
+
+def _fold_graphs(meta: _Meta, sender, receiver, dims, batch: int):
+    """Endpoints of `batch` graphs as one disjoint graph (`src/e3j/ops/convolution.py:54-78,271-308`);
+    returns the folded endpoints and the meta of the folded problem."""
+    if dims[0] is not None or dims[1] is not None:
+        warnings.warn("Convolution is being batched over graph adjacency. Batch graphs into a "
+                      "single, disconnected graph upstream or silence this warning by filtering "
+                      "`ConvolutionBatchingWarning`.", ConvolutionBatchingWarning, stacklevel=3)
+    snd = _lead(sender, dims[0], batch).to(torch.int64)
+    rcv = _lead(receiver, dims[1], batch).to(torch.int64)
+    if meta.ordering == GraphOrdering.SENDER:
+        snd_f, rcv_f = fold_endpoints(snd, rcv, batch, meta.num_nodes)
+    else:
+        rcv_f, snd_f = fold_endpoints(rcv, snd, batch, meta.num_nodes)
+    return snd_f, rcv_f, dataclasses.replace(meta, num_nodes=batch * meta.num_nodes)
+
+
 class _Convolution(torch.autograd.Function):
+    """Differentiable in (x, y, s) to any reverse-mode order; composes with `torch.func`
+    transforms (the batching rule folds the graphs of a batch into one disjoint graph)."""
+
     @staticmethod
-    def forward(ctx, x, y, s, sender, receiver, meta, graph=None):
-        ctx.meta = meta
-        ctx.save_for_backward(x, y, s, sender, receiver)
-        # the adjacency prepared here also serves the backward of this call
-        ctx.graph = graph if graph is not None else _forward_graph(meta, sender, receiver)
-        return _raw_forward(meta, x, y, s, sender, receiver, ctx.graph)
+    def forward(x, y, s, sender, receiver, meta, graph):
+        if graph is None:
+            graph = _forward_graph(meta, sender, receiver)
+        return _raw_forward(meta, x, y, s, sender, receiver, graph)
+
+    @staticmethod
+    def setup_context(ctx, inputs, output):
+        x, y, s, sender, receiver, meta, graph = inputs
+        ctx.meta, ctx.graph = meta, graph
+        # the index tensors themselves (not copies): the adjacency prepared for them by the
+        # forward pass is found again by their identity
+        ctx.index = (sender, receiver)
+        ctx.save_for_backward(x, y, s)
 
     @staticmethod
     def backward(ctx, dm):
-        x, y, s, sender, receiver = ctx.saved_tensors
+        x, y, s = ctx.saved_tensors
+        sender, receiver = ctx.index
         dx, dy, ds = _ConvolutionBwd.apply(x, y, s, dm, sender, receiver, ctx.meta, ctx.graph)
         return dx, dy, ds, None, None, None, None
+
+    @staticmethod
+    def vmap(info, in_dims, x, y, s, sender, receiver, meta, graph):
+        batch = info.batch_size
+        snd, rcv, folded = _fold_graphs(meta, sender, receiver, in_dims[3:5], batch)
+        out = _Convolution.apply(_fold_rows(_lead(x, in_dims[0], batch)), _fold_rows(_lead(y, in_dims[1], batch)),
+                                 _fold_rows(_lead(s, in_dims[2], batch)), snd, rcv, folded, None)
+        return _unfold_rows(out, batch), 0
 
 
 class _ConvolutionBwd(torch.autograd.Function):
     @staticmethod
-    def forward(ctx, x, y, s, dm, sender, receiver, meta, graph=None):
-        ctx.meta = meta
-        ctx.graph = graph
-        ctx.save_for_backward(x, y, s, dm, sender, receiver)
+    def forward(x, y, s, dm, sender, receiver, meta, graph):
+        if graph is None:  # the adjacency the forward pass prepared for these index tensors
+            graph = _forward_graph(meta, sender, receiver, build=False)
         return _raw_backward(meta, x, y, s, dm, sender, receiver, graph)
+
+    @staticmethod
+    def setup_context(ctx, inputs, output):
+        x, y, s, dm, sender, receiver, meta, graph = inputs
+        ctx.meta, ctx.graph = meta, graph
+        ctx.index = (sender, receiver)
+        ctx.save_for_backward(x, y, s, dm)
 
     @staticmethod
     def backward(ctx, ddx, ddy, dds):
         # (Dx, Dy, Ds, Ddm) from (Ddx, Ddy, Dds): the trilinear form's second variation
         # (`src/e3j/ops/convolution.py:535-562`).
-        x, y, s, dm, sender, receiver = ctx.saved_tensors
+        x, y, s, dm = ctx.saved_tensors
+        sender, receiver = ctx.index
         meta = ctx.meta
 
         graph = ctx.graph
@@ -379,6 +438,15 @@ class _ConvolutionBwd(torch.autograd.Function):
             d_x.append(gx)
             d_y.append(gy)
         return _sum(*d_x), _sum(*d_y), _sum(*d_s), _sum(*d_dm), None, None, None, None
+
+    @staticmethod
+    def vmap(info, in_dims, x, y, s, dm, sender, receiver, meta, graph):
+        batch = info.batch_size
+        snd, rcv, folded = _fold_graphs(meta, sender, receiver, in_dims[4:6], batch)
+        dx, dy, ds = _ConvolutionBwd.apply(
+            _fold_rows(_lead(x, in_dims[0], batch)), _fold_rows(_lead(y, in_dims[1], batch)),
+            _fold_rows(_lead(s, in_dims[2], batch)), _fold_rows(_lead(dm, in_dims[3], batch)), snd, rcv, folded, None)
+        return (_unfold_rows(dx, batch), _unfold_rows(dy, batch), _unfold_rows(ds, batch)), (0, 0, 0)
 
 
 def _make_meta(coef, x, y, s, params, graph_ordering, y_parity, layout) -> _Meta:
@@ -438,7 +506,7 @@ def convolution(coef, x, y, s, sender, receiver, params: ConvolutionParams,
     y_in_shape = tuple(y.shape)
     x3, y2, s3, squeeze = _canonical(x, y, s, layout)
     meta = _make_meta(coef, x3, y2, s3, params, graph_ordering, y_parity, layout)
-    out = _Convolution.apply(x3, y2, s3, sender, receiver, meta)
+    out = _Convolution.apply(x3, y2, s3, sender, receiver, meta, None)
     del y_in_shape
     if squeeze:
         out = out.squeeze(-1 if layout == Layout.TRAILING_CHANNELS else 1)
@@ -455,7 +523,7 @@ def convolution_bwd(coef, x, y, s, sender, receiver, dm, params: ConvolutionPara
     x3, y2, s3, squeeze = _canonical(x, y, s, layout)
     dm3 = dm.unsqueeze(-1 if layout == Layout.TRAILING_CHANNELS else 1) if squeeze else dm
     meta = _make_meta(coef, x3, y2, s3, params, graph_ordering, y_parity, layout)
-    dx, dy, ds = _ConvolutionBwd.apply(x3, y2, s3, dm3, sender, receiver, meta)
+    dx, dy, ds = _ConvolutionBwd.apply(x3, y2, s3, dm3, sender, receiver, meta, None)
     if squeeze:
         axis = -1 if layout == Layout.TRAILING_CHANNELS else 1
         dx = dx.squeeze(axis)

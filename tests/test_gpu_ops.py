@@ -319,3 +319,65 @@ def test_tables_without_an_unrolled_kernel_warn_once():
         convolution(p["coef"], x, y, s, snd, rcv, p["params"])
     hits = [w for w in seen if issubclass(w.category, e3j_amd.TableDrivenKernelWarning)]
     assert len(hits) == 1 and "jit" in str(hits[0].message)
+
+
+def test_third_order_gradients_match_autograd_of_dense_form():
+    """Differentiable to any reverse-mode order
+    (tests/test_ops/test_convolution_jax_transforms.py:713-767)."""
+    p = _problem(15, N=5, E=14, K=2, X=3, Y=4, Z=5, S=3, nnz=30, dtype=np.float64)
+    snd, rcv = dev(p["snd"]), dev(p["rcv"])
+
+    def third(fn):
+        x, y, s = (dev(p[k], grad=True) for k in ("x", "y", "s"))
+        out = fn(x, y, s)
+        g1 = torch.autograd.grad((out ** 2).sum(), (x, y, s), create_graph=True)
+        g2 = torch.autograd.grad(sum((g ** 2).sum() for g in g1), (x, y, s), create_graph=True)
+        return torch.autograd.grad(sum((g ** 2).sum() for g in g2), (x, y, s))
+
+    ours = third(lambda x, y, s: convolution(p["coef"], x, y, s, snd, rcv, p["params"]))
+    theirs = third(lambda x, y, s: _dense_reference(p, x, y, s))
+    for u, v in zip(ours, theirs):
+        torch.testing.assert_close(u, v, rtol=1e-8, atol=1e-8 * float(v.abs().max()))
+
+
+def test_torch_func_transforms():
+    """vmap (operands batched, graph shared or batched), Jacobians, Hessian-vector products and
+    per-sample gradients through `torch.func`; forward mode raises
+    (tests/test_ops/test_convolution_jax_transforms.py:108-196,622-711,770-788,843-900)."""
+    from torch.func import grad, jacrev, vmap
+    p = _problem(16, N=6, E=20, K=4, dtype=np.float64)
+    snd, rcv = dev(p["snd"]), dev(p["rcv"])
+    f = lambda x, y, s: convolution(p["coef"], x, y, s, snd, rcv, p["params"])  # noqa: E731
+    dense = lambda x, y, s: _dense_reference(p, x, y, s)  # noqa: E731
+    rng = np.random.default_rng(17)
+    B = 3
+    xb, yb, sb = (dev(rng.normal(size=(B,) + p[k].shape)) for k in ("x", "y", "s"))
+    want = torch.stack([dense(xb[b], yb[b], sb[b]) for b in range(B)])
+    torch.testing.assert_close(vmap(f)(xb, yb, sb), want)
+    # only x batched: the other operands are broadcast over the batch
+    torch.testing.assert_close(vmap(f, in_dims=(0, None, None))(xb, yb[0], sb[0]),
+                               torch.stack([dense(xb[b], yb[0], sb[0]) for b in range(B)]))
+    # a graph per batch entry: folded into one disjoint graph, with the reference's warning
+    graphs = [H.random_graph(rng, 6, 20) for _ in range(B)]
+    snd_b = dev(np.stack([g[0] for g in graphs]))
+    rcv_b = dev(np.stack([g[1] for g in graphs]))
+    g_fn = lambda x, y, s, a, b: convolution(p["coef"], x, y, s, a, b, p["params"])  # noqa: E731
+    with pytest.warns(e3j_amd.ConvolutionBatchingWarning):
+        got = vmap(g_fn)(xb, yb, sb, snd_b, rcv_b)
+    for b in range(B):
+        q = dict(p, snd=graphs[b][0], rcv=graphs[b][1])
+        torch.testing.assert_close(got[b], _dense_reference(q, xb[b], yb[b], sb[b]))
+    # per-sample gradients and a Jacobian (vmap over the backward operator)
+    w = dev(rng.normal(size=p["dm"].shape))
+    energy = lambda fn: (lambda x, y, s: (fn(x, y, s) * w).sum())  # noqa: E731
+    ours = vmap(grad(energy(f), argnums=(0, 1, 2)))(xb, yb, sb)
+    theirs = vmap(grad(energy(dense), argnums=(0, 1, 2)))(xb, yb, sb)
+    for u, v in zip(ours, theirs):
+        torch.testing.assert_close(u, v)
+    x0, y0, s0 = xb[0], yb[0], sb[0]
+    torch.testing.assert_close(jacrev(f, argnums=1)(x0, y0, s0), jacrev(dense, argnums=1)(x0, y0, s0))
+    # Hessian-vector product under vmap
+    hvp = lambda fn: (lambda x, y, s: grad(lambda a: (grad(energy(fn))(a, y, s) * x).sum())(x))  # noqa: E731
+    torch.testing.assert_close(vmap(hvp(f))(xb, yb, sb), vmap(hvp(dense))(xb, yb, sb))
+    with pytest.raises(RuntimeError):   # forward-mode differentiation is not defined for the operator
+        torch.func.jvp(f, (x0, y0, s0), (x0, y0, s0))
