@@ -33,7 +33,7 @@ class _HarmonicsKernel(torch.autograd.Function):
     """Degrees 0..l_max of GPU vectors through the HIP kernels (forward and VJP in one launch each)."""
 
     @staticmethod
-    def forward(ctx, vec, module):
+    def forward(vec, module):
         from . import _lib
         flat = vec.reshape(-1, 3).contiguous()
         l_max = max(module.degrees)
@@ -44,9 +44,18 @@ class _HarmonicsKernel(torch.autograd.Function):
                 flat.data_ptr(), flat.shape[0], l_max, int(module.normalize),
                 _NORMALIZATIONS[module.normalization], code, out.data_ptr(),
                 int(torch.cuda.current_stream(flat.device).cuda_stream)))
+        return out.reshape(*vec.shape[:-1], out.shape[-1])
+
+    @staticmethod
+    def setup_context(ctx, inputs, output):
+        vec, module = inputs
         ctx.module = module
         ctx.save_for_backward(vec)
-        return out.reshape(*vec.shape[:-1], out.shape[-1])
+
+    @staticmethod
+    def vmap(info, in_dims, vec, module):
+        # any number of leading axes is a list of vectors: the batch axis is one more of them
+        return _HarmonicsKernel.apply(vec.movedim(in_dims[0], 0), module), 0
 
     @staticmethod
     def backward(ctx, dout):

@@ -75,3 +75,19 @@ def test_abi_errors():
     assert lib.e3j_amd_harmonics(v.data_ptr(), 4, 2, 0, 5, _lib.F32, out.data_ptr(), None) == _lib.INVALID_ARGUMENT
     assert lib.e3j_amd_harmonics(None, 4, 2, 0, 1, _lib.F32, out.data_ptr(), None) == _lib.INVALID_ARGUMENT
     assert lib.e3j_amd_harmonics(None, 0, 2, 0, 1, _lib.F32, None, None) == _lib.OK
+
+
+def test_torch_func_transforms():
+    """vmap over a batch of vector lists and second derivatives through `torch.func`."""
+    from torch.func import grad, vmap
+    from e3j_amd.harmonics import Harmonics
+    h = Harmonics(3, normalize=True)
+    g = torch.Generator().manual_seed(3)
+    r = torch.randn(4, 11, 3, generator=g, dtype=torch.float64).cuda()
+    torch.testing.assert_close(vmap(h)(r), torch.stack([h._evaluate(r[b]) for b in range(4)]))
+    w = torch.randn(11, 16, generator=g, dtype=torch.float64).cuda()
+    energy = lambda fn: (lambda v: (fn(v) * w).sum())  # noqa: E731
+    torch.testing.assert_close(grad(energy(h))(r[0]), grad(energy(h._evaluate))(r[0]))
+    second = lambda fn: grad(lambda v: (grad(energy(fn))(v) ** 2).sum())  # noqa: E731
+    torch.testing.assert_close(second(h)(r[0]), second(h._evaluate)(r[0]))
+    torch.testing.assert_close(vmap(grad(energy(h)))(r), vmap(grad(energy(h._evaluate)))(r))
