@@ -316,7 +316,9 @@ int launch_tp_unrolled_bwd(int64_t rows, int, float scale, const float *x, const
 // accesses and turns it through its strip of LDS (odd row stride: conflict-free column
 // access), runs the same generated arithmetic on registers, and turns the results back.
 // The last tile is moved back to end at the last column; the columns it shares with the
-// tile before receive the same values from both.
+// tile before receive the same values from both.  The register budgets in the launch bounds
+// (resident waves per SIMD) are the measured optima: a fourth wave pays for the uniform-y
+// forward and a third for the MAP backward despite a few spilled registers, nowhere else.
 // ---------------------------------------------------------------------------
 template <int X, int Y, int Z>
 struct TpLeadingGeometry {
@@ -361,7 +363,7 @@ __device__ __forceinline__ void tp_leading_operands(const float *__restrict__ x,
 }
 
 template <typename Sig, int WPB, bool kUniformY>
-__global__ __launch_bounds__(kWave * WPB) void tp_unrolled_fwd_leading_kernel(
+__global__ __launch_bounds__(kWave * WPB, kUniformY ? 4 : 1) void tp_unrolled_fwd_leading_kernel(
     const float *__restrict__ x, const float *__restrict__ y, float *__restrict__ z, int64_t cols, int K,
     float scale) {
     constexpr int Z = Sig::Z;
@@ -411,7 +413,7 @@ __device__ __forceinline__ void tp_leading_cotangent(const float *__restrict__ d
 
 // kInner: the cotangent is (rows, Z), one row per column's row (INNER mode)
 template <typename Sig, int WPB, bool kInner>
-__global__ __launch_bounds__(kWave * WPB) void tp_unrolled_bwd_map_leading_kernel(
+__global__ __launch_bounds__(kWave * WPB, kInner ? 1 : 3) void tp_unrolled_bwd_map_leading_kernel(
     const float *__restrict__ x, const float *__restrict__ y, const float *__restrict__ dz,
     float *__restrict__ dx, float *__restrict__ dy, int64_t cols, int K, float scale) {
     constexpr int X = Sig::X, Y = Sig::Y, Z = Sig::Z;
