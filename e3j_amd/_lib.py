@@ -17,7 +17,7 @@ LIB_PATH = os.environ.get("E3J_AMD_LIBRARY") or os.path.join(_HERE, "lib", "libe
 
 OK, INVALID_ARGUMENT, UNIMPLEMENTED, INTERNAL = 0, 1, 2, 3
 LAYOUT_LEADING, LAYOUT_TRAILING = 0, 1
-F32, F64 = 0, 1
+F32, F64, F16 = 0, 1, 2
 
 
 class ConvParams(ctypes.Structure):

@@ -86,9 +86,6 @@ class Convolution:
         dtype = torch.promote_types(torch.promote_types(node_features.dtype, edge_features.dtype),
                                     edge_scalars.dtype)
         val_dtype = resolve_val_dtype(_NP_OF_TORCH.get(dtype, "int64"))
-        if val_dtype == "float16":
-            raise TypeError("Fused ops support value dtypes ('float32', 'float64'), got 'float16'. "
-                            "Cast the operands.")
         node_features = node_features.to(dtype)
         edge_features = edge_features.to(dtype)
         edge_scalars = edge_scalars.to(dtype)

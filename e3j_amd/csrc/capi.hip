@@ -72,7 +72,7 @@ int validate(const e3j_amd_conv_params *p, const char *op) {
                          name + ": num_x, num_y, num_out, num_scalars and channels must be >= 1");
     if (p->layout != E3J_AMD_LAYOUT_LEADING && p->layout != E3J_AMD_LAYOUT_TRAILING)
         return set_error(E3J_AMD_INVALID_ARGUMENT, name + ": unknown layout " + std::to_string(p->layout));
-    if (p->val_dtype != E3J_AMD_F32 && p->val_dtype != E3J_AMD_F64)
+    if (p->val_dtype != E3J_AMD_F32 && p->val_dtype != E3J_AMD_F64 && p->val_dtype != E3J_AMD_F16)
         return set_error(E3J_AMD_INVALID_ARGUMENT, name + ": unsupported (IDX, VAL) dtype pair");
     if (p->coef_idx_bytes != 1 && p->coef_idx_bytes != 4)
         return set_error(E3J_AMD_INVALID_ARGUMENT, name + ": unsupported (IDX, VAL) dtype pair");

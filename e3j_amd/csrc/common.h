@@ -20,6 +20,9 @@ template <> struct CoefAlign<uint8_t, float>  { static constexpr int value = 8; 
 template <> struct CoefAlign<int32_t, float>  { static constexpr int value = 32; };
 template <> struct CoefAlign<uint8_t, double> { static constexpr int value = 16; };
 template <> struct CoefAlign<int32_t, double> { static constexpr int value = 32; };
+typedef _Float16 half_t;  // float16 values: arithmetic in half precision
+template <> struct CoefAlign<uint8_t, half_t>  { static constexpr int value = 8; };
+template <> struct CoefAlign<int32_t, half_t>  { static constexpr int value = 32; };
 
 template <typename Idx, typename Val>
 struct alignas(CoefAlign<Idx, Val>::value) Coef4D {
@@ -30,6 +33,25 @@ static_assert(sizeof(Coef4D<uint8_t, float>) == 8, "packed size");
 static_assert(sizeof(Coef4D<int32_t, float>) == 32, "packed size");
 static_assert(sizeof(Coef4D<uint8_t, double>) == 16, "packed size");
 static_assert(sizeof(Coef4D<int32_t, double>) == 32, "packed size");
+static_assert(sizeof(Coef4D<uint8_t, half_t>) == 8, "packed size");
+static_assert(sizeof(Coef4D<int32_t, half_t>) == 32, "packed size");
+
+// Sum over the 64 lanes of a wave (half values travel as float).
+template <typename Val>
+__device__ inline Val wave_sum(Val v) {
+#pragma unroll
+    for (int off = kWave / 2; off > 0; off >>= 1) v += __shfl_xor(v, off, kWave);
+    return v;
+}
+template <>
+__device__ inline half_t wave_sum<half_t>(half_t v) {
+#pragma unroll
+    for (int off = kWave / 2; off > 0; off >>= 1) v += (half_t)__shfl_xor((float)v, off, kWave);
+    return v;
+}
+inline size_t val_bytes(int val_dtype) {
+    return val_dtype == E3J_AMD_F64 ? 8 : val_dtype == E3J_AMD_F16 ? 2 : 4;
+}
 
 // Element strides of a (rows, dim, channels) operand in either layout.
 struct RowLayout {

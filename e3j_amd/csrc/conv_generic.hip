@@ -14,17 +14,12 @@
 // skipped by a bounds check on the gathered endpoint, dy/ds of padding edges
 // written as zeros, dx rows zero-filled before accumulation.
 
+#include <type_traits>
+
 #include "common.h"
 
 namespace e3j_amd {
 namespace {
-
-template <typename Val>
-__device__ inline Val wave_sum(Val v) {
-#pragma unroll
-    for (int off = kWave / 2; off > 0; off >>= 1) v += __shfl_xor(v, off, kWave);
-    return v;
-}
 
 template <typename Idx, typename Val>
 __global__ void generic_fwd_kernel(const Coef4D<Idx, Val> *__restrict__ coef, int num_coef,
@@ -167,7 +162,7 @@ __global__ void generic_bwd_kernel(const Coef4D<Idx, Val> *__restrict__ coef, in
                 for (int l = 0; l < S; l++) dsrow[(int64_t)l * ls.dim] = dsc[l * kWave];
                 Val *dxrow = dx + (int64_t)xnode * lx.row + (int64_t)c * lx.chan;
                 for (int j = 0; j < X; j++) {
-                    if (kGroupIsReceiver) unsafeAtomicAdd(dxrow + (int64_t)j * lx.dim, dxc[j * kWave]);
+                    if constexpr (kGroupIsReceiver) unsafeAtomicAdd(dxrow + (int64_t)j * lx.dim, dxc[j * kWave]);
                     else dxrow[(int64_t)j * lx.dim] += dxc[j * kWave];
                 }
             }
@@ -311,8 +306,17 @@ int run_bwd(const e3j_amd_conv_params &p, bool group_is_receiver, const void *co
                            static_cast<Val *>(ds), p.num_nodes, p.channels, p.num_x,              \
                            p.num_scalars, p.num_out, nchunks, cols_ji ? 1 : 0);                   \
     } while (0)
-    if (group_is_receiver) E3J_LAUNCH_BWD(true);
-    else E3J_LAUNCH_BWD(false);
+    if constexpr (std::is_same<Val, half_t>::value) {
+        // no float atomics on half values: rows must own their dx (sender-grouped)
+        if (group_is_receiver)
+            return set_error(E3J_AMD_UNIMPLEMENTED,
+                             "convolution_bwd: float16 runs the sender-grouped backward only (dx by "
+                             "float atomics has no half-precision form)");
+        E3J_LAUNCH_BWD(false);
+    } else {
+        if (group_is_receiver) E3J_LAUNCH_BWD(true);
+        else E3J_LAUNCH_BWD(false);
+    }
 #undef E3J_LAUNCH_BWD
     return check_hip(hipGetLastError(), "convolution backward launch");
 }
@@ -418,6 +422,8 @@ int launch_zero_padding(const e3j_amd_conv_params &p, const int32_t *other, cons
     if (p.val_dtype == E3J_AMD_F32 && p.coef_idx_bytes == 4) return CALL(int32_t, float);   \
     if (p.val_dtype == E3J_AMD_F64 && p.coef_idx_bytes == 1) return CALL(uint8_t, double);  \
     if (p.val_dtype == E3J_AMD_F64 && p.coef_idx_bytes == 4) return CALL(int32_t, double);  \
+    if (p.val_dtype == E3J_AMD_F16 && p.coef_idx_bytes == 1) return CALL(uint8_t, half_t);  \
+    if (p.val_dtype == E3J_AMD_F16 && p.coef_idx_bytes == 4) return CALL(int32_t, half_t);  \
     return set_error(E3J_AMD_INVALID_ARGUMENT, "unsupported (IDX, VAL) dtype pair")
 
 int launch_generic_fwd(const e3j_amd_conv_params &p, const void *coef, const void *x, const void *y,

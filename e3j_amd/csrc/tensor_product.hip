@@ -49,6 +49,8 @@ template <> struct Coef3Align<uint8_t, float>  { static constexpr int value = 8;
 template <> struct Coef3Align<int32_t, float>  { static constexpr int value = 16; };
 template <> struct Coef3Align<uint8_t, double> { static constexpr int value = 16; };
 template <> struct Coef3Align<int32_t, double> { static constexpr int value = 32; };
+template <> struct Coef3Align<uint8_t, half_t> { static constexpr int value = 8; };
+template <> struct Coef3Align<int32_t, half_t> { static constexpr int value = 16; };
 template <typename Idx, typename Val>
 struct alignas(Coef3Align<Idx, Val>::value) Coef3 {
     Val val;
@@ -58,6 +60,8 @@ static_assert(sizeof(Coef3<uint8_t, float>) == 8, "packed size");
 static_assert(sizeof(Coef3<int32_t, float>) == 16, "packed size");
 static_assert(sizeof(Coef3<uint8_t, double>) == 16, "packed size");
 static_assert(sizeof(Coef3<int32_t, double>) == 32, "packed size");
+static_assert(sizeof(Coef3<uint8_t, half_t>) == 8, "packed size");
+static_assert(sizeof(Coef3<int32_t, half_t>) == 16, "packed size");
 
 // One operand or the result: base pointer strides and channel count.
 struct Side {
@@ -120,13 +124,6 @@ __global__ void tp_columns_kernel(const Coef3<Idx, Val> *__restrict__ coef, int 
         for (; next_row < sz.dim; next_row++) zr[(int64_t)next_row * sz.l.dim] = Val(0);
 }
 
-template <typename Val>
-__device__ inline Val wave_total(Val v) {
-#pragma unroll
-    for (int off = kWave / 2; off > 0; off >>= 1) v += __shfl_xor(v, off, kWave);
-    return v;
-}
-
 // INNER: a wave per row; lanes walk the channels in chunks of 64 and keep one partial sum per
 // output coordinate in their LDS column; the channel sum is a wave reduction per coordinate.
 template <typename Idx, typename Val>
@@ -156,7 +153,7 @@ __global__ void tp_inner_kernel(const Coef3<Idx, Val> *__restrict__ coef, int nu
     }
     Val *zr = z + r * num_out;
     for (int i = 0; i < num_out; i++) {
-        const Val total = wave_total(zs[i * kWave]);
+        const Val total = wave_sum(zs[i * kWave]);
         if (lane == 0) zr[i] = total;
     }
 }
@@ -218,6 +215,9 @@ int launch_product(const e3j_amd_tp_params *p, int mode, const void *coef, const
     const Side so = make_side(p->layout, dim_out, out_channels(mode, ch_a, ch_b));
     const bool sorted = p->coef_sorted != 0;
     const bool u8 = p->coef_idx_bytes == 1;
+    if (p->val_dtype == E3J_AMD_F16)
+        return u8 ? launch_typed<uint8_t, half_t>(mode, sorted, coef, p->num_coef, a, sa, b, sb, out, so, p->num_rows, stream)
+                  : launch_typed<int32_t, half_t>(mode, sorted, coef, p->num_coef, a, sa, b, sb, out, so, p->num_rows, stream);
     if (p->val_dtype == E3J_AMD_F32)
         return u8 ? launch_typed<uint8_t, float>(mode, sorted, coef, p->num_coef, a, sa, b, sb, out, so, p->num_rows, stream)
                   : launch_typed<int32_t, float>(mode, sorted, coef, p->num_coef, a, sa, b, sb, out, so, p->num_rows, stream);
@@ -240,7 +240,7 @@ int validate_tp(const e3j_amd_tp_params *p, const char *op) {
         return set_error(E3J_AMD_INVALID_ARGUMENT,
                          name + ": MAP and INNER modes require same number of LHS and RHS channels, got (" +
                              std::to_string(p->channels_x) + ", " + std::to_string(p->channels_y) + ")");
-    if ((p->val_dtype != E3J_AMD_F32 && p->val_dtype != E3J_AMD_F64) ||
+    if ((p->val_dtype != E3J_AMD_F32 && p->val_dtype != E3J_AMD_F64 && p->val_dtype != E3J_AMD_F16) ||
         (p->coef_idx_bytes != 1 && p->coef_idx_bytes != 4))
         return set_error(E3J_AMD_INVALID_ARGUMENT, name + ": unsupported (IDX, VAL) dtype pair");
     if (p->signature >= num_tp_signatures())
@@ -334,8 +334,8 @@ extern "C" int e3j_amd_tensor_product_bwd(const e3j_amd_tp_params *p, const void
     else if (cx > 1) { mode_x = E3J_AMD_MODE_OUTER; mode_y = E3J_AMD_MODE_INNER; }
     else if (cy > 1) { mode_x = E3J_AMD_MODE_INNER; mode_y = E3J_AMD_MODE_OUTER; }
     else mode_x = mode_y = E3J_AMD_MODE_OUTER;
-    const size_t item = p->coef_idx_bytes == 1 ? (p->val_dtype == E3J_AMD_F32 ? 8 : 16)
-                                               : (p->val_dtype == E3J_AMD_F32 ? 16 : 32);
+    const size_t item = p->coef_idx_bytes == 1 ? (p->val_dtype == E3J_AMD_F64 ? 16 : 8)
+                                               : (p->val_dtype == E3J_AMD_F64 ? 32 : 16);
     const void *coef_x = coef_bwd;
     const void *coef_y = static_cast<const unsigned char *>(coef_bwd) + item * (size_t)p->num_coef;
     int rc = launch_product(p, mode_x, coef_x, dz, p->num_out, cz, y, p->num_y, cy, dx, p->num_x, stream);

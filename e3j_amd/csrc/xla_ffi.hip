@@ -150,6 +150,7 @@ void *decode_common(XlaCallFrame *f, const char *op, const XlaBuffer *coef, cons
     else return make_error(f, E3J_AMD_INVALID_ARGUMENT, "unsupported (IDX, VAL) dtype pair");
     if (x->dtype == kXlaF32) p.val_dtype = E3J_AMD_F32;
     else if (x->dtype == kXlaF64) p.val_dtype = E3J_AMD_F64;
+    else if (x->dtype == kXlaF16) p.val_dtype = E3J_AMD_F16;
     else return make_error(f, E3J_AMD_INVALID_ARGUMENT, "unsupported (IDX, VAL) dtype pair");
     if (y->dtype != x->dtype || s->dtype != x->dtype || node_rows->dtype != x->dtype)
         return make_error(f, E3J_AMD_INVALID_ARGUMENT, name + ": value operands must share one dtype");
@@ -247,6 +248,7 @@ void *decode_tensor_product(XlaCallFrame *f, const char *op, const XlaBuffer *co
     else return make_error(f, E3J_AMD_INVALID_ARGUMENT, "unsupported (IDX, VAL) dtype pair");
     if (x->dtype == kXlaF32) p->val_dtype = E3J_AMD_F32;
     else if (x->dtype == kXlaF64) p->val_dtype = E3J_AMD_F64;
+    else if (x->dtype == kXlaF16) p->val_dtype = E3J_AMD_F16;
     else return make_error(f, E3J_AMD_INVALID_ARGUMENT, "unsupported (IDX, VAL) dtype pair");
     if (y->dtype != x->dtype)
         return make_error(f, E3J_AMD_INVALID_ARGUMENT, name + ": value operands must share one dtype");

@@ -52,7 +52,8 @@ class TableDrivenKernelWarning(UserWarning):
     slower than the unrolled ones."""
 
 
-_VAL_DTYPES = {torch.float32: (_lib.F32, np.float32), torch.float64: (_lib.F64, np.float64)}
+_VAL_DTYPES = {torch.float32: (_lib.F32, np.float32), torch.float64: (_lib.F64, np.float64),
+               torch.float16: (_lib.F16, np.float16)}
 
 
 class _Table:
@@ -180,7 +181,7 @@ def _check_operands(x, y, s, sender, receiver):
         if t.device.type != "cuda":
             raise RuntimeError(f"`{name}` must live in GPU memory; e3j_amd has no CPU implementation")
     if x.dtype not in _VAL_DTYPES:
-        raise TypeError(f"Fused ops support value dtypes ('float32', 'float64'), got {x.dtype}. "
+        raise TypeError(f"Fused ops support value dtypes ('float16', 'float32', 'float64'), got {x.dtype}. "
                         "Cast the operands.")
     if y.dtype != x.dtype or s.dtype != x.dtype:
         raise TypeError("x, y and s must share one dtype")
@@ -264,7 +265,8 @@ def _raw_backward(meta: _Meta, x, y, s, dm, sender, receiver, graph=None):
     n = meta.num_nodes
     dx, dy, ds = torch.empty_like(x), torch.empty_like(y), torch.empty_like(s)
     lib = _lib.load()
-    deterministic = config().deterministic
+    # float16: dx by float atomics has no half-precision form, rows must own their dx
+    deterministic = config().deterministic or x.dtype == torch.float16
     table = meta.table
     has_kernel = table.signature(*_shape(meta, x, y, s), meta.layout)[0] >= 0
     # SENDER ordering: the cotangents belong to the edges as given (dy[e], ds[e] come from

@@ -25,7 +25,8 @@ from . import _lib
 from .coef import Coef
 from .options import Layout, MixingMode, config
 
-_VAL_DTYPES = {torch.float32: (_lib.F32, np.float32), torch.float64: (_lib.F64, np.float64)}
+_VAL_DTYPES = {torch.float32: (_lib.F32, np.float32), torch.float64: (_lib.F64, np.float64),
+               torch.float16: (_lib.F16, np.float16)}
 
 
 @dataclasses.dataclass
@@ -302,7 +303,7 @@ def _check(x: torch.Tensor, y: torch.Tensor):
     if x.dtype != y.dtype:
         raise TypeError(f"x and y must share a dtype, got {x.dtype} and {y.dtype}")
     if x.dtype not in _VAL_DTYPES:
-        raise NotImplementedError(f"the HIP tensor product runs in float32 or float64, got {x.dtype}")
+        raise NotImplementedError(f"the HIP tensor product runs in float16, float32 or float64, got {x.dtype}")
     if not x.is_cuda or x.device != y.device:
         raise ValueError("x and y must live on the same GPU: the tensor product has no CPU path")
     if x.shape[0] != y.shape[0]:

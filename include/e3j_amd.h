@@ -9,7 +9,8 @@
  * a compile-time-unrolled kernel.
  *
  * Conventions
- *  - Values are float32 (or float64 on the table-driven kernels); indices int32.
+ *  - Values are float32 (or float64 / float16 on the table-driven kernels; float16 computes in
+ *    half precision with fused multiply-adds, lib/e3j_ops/cuda/utils.cuh:108-112); indices int32.
  *  - TRAILING layout: x (N, X, K), s (E, S, K), out/dm (N, Z, K).
  *    LEADING  layout: x (N, K, X), s (E, K, S), out/dm (N, K, Z).  y is (E, Y).
  *  - A CSR adjacency groups edge positions by one endpoint: `row_ptr` (N+1)
@@ -45,7 +46,7 @@ enum {
 };
 
 enum { E3J_AMD_LAYOUT_LEADING = 0, E3J_AMD_LAYOUT_TRAILING = 1 }; /* src/e3j/utils/options.py:144-145 */
-enum { E3J_AMD_F32 = 0, E3J_AMD_F64 = 1 };
+enum { E3J_AMD_F32 = 0, E3J_AMD_F64 = 1, E3J_AMD_F16 = 2 };
 
 /* Problem sizes, the counterpart of convolution::Params (lib/e3j_ops/cuda/convolution.cuh:46-60). */
 typedef struct e3j_amd_conv_params {
@@ -58,7 +59,7 @@ typedef struct e3j_amd_conv_params {
     int32_t num_scalars;
     int32_t channels;
     int32_t layout;         /* E3J_AMD_LAYOUT_* */
-    int32_t val_dtype;      /* E3J_AMD_F32 / E3J_AMD_F64 */
+    int32_t val_dtype;      /* E3J_AMD_F32 / E3J_AMD_F64 / E3J_AMD_F16 */
     int32_t coef_idx_bytes; /* 1 or 4 */
     int32_t signature;      /* id from e3j_amd_find_signature, or -1: table-driven kernel */
     float   coef_scale;     /* unrolled kernels: table = coef_scale * built-in table (1 by default) */
@@ -216,8 +217,8 @@ int e3j_amd_harmonics_bwd(const void *vec, const void *dout, int64_t num, int32_
  * TRAILING layout: x (R, X, Cx), y (R, Y, Cy), z (R, Z, Cx, Cy) / (R, Z) / (R, Z, C);
  * LEADING layout: x (R, Cx, X), y (R, Cy, Y), z (R, Cx, Cy, Z) / (R, Z) / (R, C, Z).
  * `coef` is the packed table {val; i; j; k} of lib/e3j_ops/cuda/tensor_product.cuh:98-111 in
- * device memory (8, 16, 16, 32 bytes per entry for uint8/float32, int32/float32,
- * uint8/float64, int32/float64).  Any channel count is accepted (the reference requires powers
+ * device memory (8, 16, 16, 32, 8, 16 bytes per entry for uint8/float32, int32/float32,
+ * uint8/float64, int32/float64, uint8/float16, int32/float16).  Any channel count is accepted (the reference requires powers
  * of two in the trailing layout, e3j_ops.h:168-185). */
 enum { E3J_AMD_MODE_OUTER = 0, E3J_AMD_MODE_INNER = 1, E3J_AMD_MODE_MAP = 2 };
 typedef struct e3j_amd_tp_params {
@@ -230,7 +231,7 @@ typedef struct e3j_amd_tp_params {
     int32_t channels_y;
     int32_t mode;           /* E3J_AMD_MODE_* of the forward pass */
     int32_t layout;         /* E3J_AMD_LAYOUT_* */
-    int32_t val_dtype;      /* E3J_AMD_F32 / E3J_AMD_F64 */
+    int32_t val_dtype;      /* E3J_AMD_F32 / E3J_AMD_F64 / E3J_AMD_F16 */
     int32_t coef_idx_bytes; /* 1 or 4 */
     /* != 0: entries with equal output index are contiguous and the output indices ascend (the
      * order sparse_coo and Coef.transpose produce, src/e3j/utils/sparse.py:76-126,

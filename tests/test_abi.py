@@ -280,7 +280,7 @@ def _conv_frame(xla, *, x_dtype=F32, coef_dtype=U8, y_dims=(6, 3), n_attr=4, dro
 
 
 @pytest.mark.parametrize("kw, code, needle", [
-    (dict(x_dtype=10), ERR_INVALID_ARGUMENT, "unsupported (IDX, VAL) dtype pair"),
+    (dict(x_dtype=16), ERR_INVALID_ARGUMENT, "unsupported (IDX, VAL) dtype pair"),    # BF16
     (dict(coef_dtype=F32), ERR_INVALID_ARGUMENT, "unsupported (IDX, VAL) dtype pair"),
     (dict(y_dims=(6, 3, 2)), ERR_UNIMPLEMENTED, "RHS y should have only one channel"),
     (dict(n_attr=5), ERR_INVALID_ARGUMENT, "num_nodes rows"),

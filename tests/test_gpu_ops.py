@@ -284,7 +284,7 @@ def test_operator_errors():
     with pytest.raises(ValueError, match="y_parity"):
         convolution(p["coef"], x, y, s, snd, rcv, p["params"], GraphOrdering.SENDER)
     with pytest.raises(TypeError, match="Cast the operands"):
-        convolution(p["coef"], x.half(), y.half(), s.half(), snd, rcv, p["params"])
+        convolution(p["coef"], x.bfloat16(), y.bfloat16(), s.bfloat16(), snd, rcv, p["params"])
 
 
 def test_prepared_graph_is_reused_per_index_tensor_pair_and_follows_in_place_changes():
@@ -381,3 +381,32 @@ def test_torch_func_transforms():
     torch.testing.assert_close(vmap(hvp(f))(xb, yb, sb), vmap(hvp(dense))(xb, yb, sb))
     with pytest.raises(RuntimeError):   # forward-mode differentiation is not defined for the operator
         torch.func.jvp(f, (x0, y0, s0), (x0, y0, s0))
+
+
+@pytest.mark.parametrize("layout", ["TRAILING_CHANNELS", "LEADING_CHANNELS"])
+@pytest.mark.parametrize("ordering", ["RECEIVER", "NONE"])
+def test_float16_operands(layout, ordering):
+    """float16 values run the table-driven kernels in half precision
+    (tests/test_ops/test_dtype.py:253-330): parity with the float64 checker on the rounded
+    operands, within the rounding of a half-precision running sum."""
+    p = _problem(18, N=15, E=90, K=24, nnz=50, sort_by="receiver" if ordering == "RECEIVER" else None)
+    half = {k: p[k].astype(np.float16) for k in ("x", "y", "s", "dm")}
+    val16 = p["val"].astype(np.float16)
+    coef = H.pack_table(p["idx"], val16, p["mix"], val_dtype=np.float16)
+    lead = layout == "LEADING_CHANNELS"
+    t = (lambda a: np.ascontiguousarray(a.transpose(0, 2, 1))) if lead else (lambda a: a)
+    back = (lambda g: g.transpose(1, 2)) if lead else (lambda g: g)
+    x, y, s = dev(t(half["x"]), grad=True), dev(half["y"], grad=True), dev(t(half["s"]), grad=True)
+    out = convolution(coef, x, y, s, dev(p["snd"]), dev(p["rcv"]), p["params"], ordering, layout=layout)
+    assert out.dtype == torch.float16
+    grads = torch.autograd.grad(out, (x, y, s), dev(t(half["dm"])))
+    f64 = {k: v.astype(np.float64) for k, v in half.items()}
+    ref, mag = H.forward_reference(p["idx"], val16.astype(np.float64), p["mix"], f64["x"], f64["y"], f64["s"],
+                                   p["snd"], p["rcv"], p["params"].num_out)
+    refs, mags = H.backward_reference(p["idx"], val16.astype(np.float64), p["mix"], f64["x"], f64["y"], f64["s"],
+                                      p["snd"], p["rcv"], f64["dm"])
+    eps = 2.0 ** -10
+    for got, r, m, name in [(out, ref, mag, "out")] + list(zip(grads, refs, mags, ("dx", "dy", "ds"))):
+        got = back(got) if got.dim() == 3 else got
+        err = np.abs(got.detach().float().cpu().numpy().astype(np.float64) - r)
+        assert np.all(err <= 6 * eps * m + 1e-3), f"{name}: {err.max()} against magnitude {m.max()}"

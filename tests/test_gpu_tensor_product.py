@@ -399,3 +399,33 @@ def test_torch_func_transforms():
     torch.testing.assert_close(second(f)(x[0], y[0]), second(dense)(x[0], y[0]))
     with pytest.raises(RuntimeError):   # forward-mode differentiation is not defined for the operator
         torch.func.jvp(f, (x[0], y[0]), (x[0], y[0]))
+
+
+@pytest.mark.parametrize("mode", MODES)
+@pytest.mark.parametrize("layout", LAYOUTS)
+@pytest.mark.parametrize("idx_dtype", ["uint8", "int32"])
+def test_float16_operands(mode, layout, idx_dtype):
+    """float16 values run the table-driven kernels in half precision, both layouts (the
+    reference serves float16 in the trailing layout only, tests/test_ops/test_dtype.py:136-190):
+    parity with the float64 checker on the rounded operands within half-precision rounding."""
+    rng = np.random.default_rng(26)
+    idx, val = _table(nnz=200)
+    val16 = val.astype(np.float16)
+    x, y = _operands(rng, mode, layout, 16, rows=40, dtype=np.float16, has=(True, False))
+    coef = Coef(val16, idx, "float16", idx_dtype).pack()
+    p = TensorProductParams(num_out=NUM_OUT, mode=mode, layout=layout)
+    xt, yt = torch.from_numpy(x).to(DEV).requires_grad_(True), torch.from_numpy(y).to(DEV).requires_grad_(True)
+    z = e3j_amd.tensor_product(coef, xt, yt, p)
+    assert z.dtype == torch.float16
+    dz = rng.normal(size=tuple(z.shape)).astype(np.float16)
+    dx, dy = torch.autograd.grad(z, (xt, yt), torch.from_numpy(dz).to(DEV))
+    f64 = lambda a: a.astype(np.float64)  # noqa: E731
+    v = f64(val16)
+    ref = T.tensor_product_unfused(idx, v, f64(x), f64(y), NUM_OUT, mode, layout)
+    mag = T.tensor_product_unfused(idx, np.abs(v), np.abs(f64(x)), np.abs(f64(y)), NUM_OUT, mode, layout)
+    rdx, rdy = T.tensor_product_vjp(idx, v, f64(x), f64(y), f64(dz), mode, layout)
+    mdx, mdy = T.tensor_product_vjp(idx, np.abs(v), np.abs(f64(x)), np.abs(f64(y)), np.abs(f64(dz)), mode, layout)
+    eps = 2.0 ** -10
+    for got, r, m, name in ((z, ref, mag, "z"), (dx, rdx, mdx, "dx"), (dy, rdy, mdy, "dy")):
+        err = np.abs(got.detach().float().cpu().numpy().astype(np.float64) - r)
+        assert np.all(err <= 8 * eps * m + 1e-3), f"{name}: {err.max()} against magnitude {m.max()}"

@@ -168,8 +168,8 @@ def test_operator_argument_errors_need_no_gpu():
         e3j_amd.tensor_product(coef, torch.zeros(3), y, p)
     with pytest.raises(TypeError, match="share a dtype"):
         e3j_amd.tensor_product(coef, x.double(), y, p)
-    with pytest.raises(NotImplementedError, match="float32 or float64"):
-        e3j_amd.tensor_product(coef, x.half(), y.half(), p)
+    with pytest.raises(NotImplementedError, match="float16, float32 or float64"):
+        e3j_amd.tensor_product(coef, x.bfloat16(), y.bfloat16(), p)
     assert e3j_amd.CUDATensorProductParams is TensorProductParams
     assert e3j_amd.MixingMode.parse("map") is e3j_amd.MixingMode.MAP
     assert [m.value for m in e3j_amd.MixingMode] == [0, 1, 2]   # the integers the FFI carries
