@@ -218,9 +218,10 @@ __device__ __forceinline__ float to_vgpr(float v) {
 // mask (never a register-array select, which the compiler would lower to a chain of
 // compares), and two cross-row exchanges finish the sum.  On return every lane holds
 // in v[0] the total of value `slot(lane)`.
-template <int NV>
+template <int NV, int LANES = kWave>
 struct WaveReduce {
     static_assert(NV >= 1 && NV <= 16, "at most 16 values");
+    static_assert(LANES == 16 || LANES == 32 || LANES == 64, "sums run over groups of 16, 32 or 64 lanes");
     static constexpr int P = 16;  // values are padded to 16 by the caller
     __device__ static __forceinline__ int slot(int lane) {
         return ((lane & 1) << 3) | ((lane & 2) << 1) | ((lane & 4) >> 1) | ((lane & 8) >> 3);
@@ -247,20 +248,21 @@ struct WaveReduce {
         level<0x4E, 8>(v, (lane & 2) ? ~0u : 0u);    // quad_perm [2,3,0,1]
         level<0x124, 4>(v, (lane & 4) ? ~0u : 0u);   // row_ror:4 (the source lane differs in bit 2)
         level<0x128, 2>(v, (lane & 8) ? ~0u : 0u);   // row_ror:8 (= xor 8)
-        v[0] += __shfl_xor(v[0], 16, kWave);
-        v[0] += __shfl_xor(v[0], 32, kWave);
+        if (LANES > 16) v[0] += __shfl_xor(v[0], 16, kWave);
+        if (LANES > 32) v[0] += __shfl_xor(v[0], 32, kWave);
         return v[0];
     }
 };
 
-// Any number of values: sixteen at a time.  `sink(k, total)` is called on the lanes 0..15 of the
-// wave for the values k they hold (k < NV); `v` must be padded to a multiple of 16.
-template <int NV>
+// Any number of values: sixteen at a time.  `sink(k, total)` is called on the first 16 lanes of
+// every group of LANES lanes for the values k they hold (k < NV); `v` must be padded to a
+// multiple of 16.
+template <int NV, int LANES = kWave>
 struct WaveReduceBlocks {
     static constexpr int P = (NV + 15) / 16 * 16;
     template <typename Sink>
     __device__ static __forceinline__ void run(float (&v)[P], int lane, const Sink &sink) {
-        using Red = WaveReduce<16>;
+        using Red = WaveReduce<16, LANES>;
 #pragma unroll
         for (int base = 0; base < P; base += 16) {
             float part[16];
@@ -268,7 +270,7 @@ struct WaveReduceBlocks {
             for (int t = 0; t < 16; t++) part[t] = v[base + t];
             const float total = Red::run(part, lane);
             const int k = base + Red::slot(lane);
-            if (lane < 16 && k < NV) sink(k, total);
+            if (lane % LANES < 16 && k < NV) sink(k, total);
         }
     }
 };
@@ -300,6 +302,9 @@ struct Slice {
     static constexpr int WIDTH = kWave * CPL;                 // channels per wave
     static constexpr int COUNT = (K + WIDTH - 1) / WIDTH;     // waves per row
     static constexpr bool FULL = (K % WIDTH) == 0;            // no idle lanes
+    // Fewer channels than lanes (16 or 32, one per lane): the wave walks SUB edges of its row
+    // side by side, one per group of K lanes, instead of idling the lanes past K.
+    static constexpr int SUB = (CPL == 1 && (K == 16 || K == 32)) ? kWave / K : 1;
     static_assert(K % CPL == 0, "channels must be a multiple of the per-lane vector width");
 };
 
@@ -315,9 +320,11 @@ __device__ __forceinline__ void unrolled_fwd_part(
     constexpr int X = Part::X, S = Part::S, Z = Part::Z;
     using V = Vec<CPL>;
     using SL = Slice<K, CPL>;
+    constexpr int SUB = SL::SUB;
 
-    const int c_raw = slice * SL::WIDTH + lane * CPL;
-    const bool active = SL::FULL || c_raw < K;
+    const int sub = SUB > 1 ? lane / K : 0;  // which of the SUB edges walked side by side
+    const int c_raw = SUB > 1 ? lane % K : slice * SL::WIDTH + lane * CPL;
+    const bool active = SL::FULL || SUB > 1 || c_raw < K;
     const int c0 = active ? c_raw : 0;  // idle lanes read channel 0 and never store
 
     V acc[NZ];
@@ -330,9 +337,13 @@ __device__ __forceinline__ void unrolled_fwd_part(
     V xn[NX], sn[NS];
     float yn[Y];
     bool valid_n = false;
-    auto fetch = [&](int pos) {
+    auto fetch = [&](int base) {
+        // SUB > 1: the group's own position; past the end of the row it re-reads the last
+        // position and contributes nothing
+        const bool inside = SUB == 1 || base + sub < e1;
+        const int pos = SUB == 1 ? base : (inside ? base + sub : e1 - 1);
         const int snd = sender[pos];
-        valid_n = (unsigned)snd < (unsigned)num_nodes;
+        valid_n = inside && (unsigned)snd < (unsigned)num_nodes;
         const int row = valid_n ? snd : 0;
         const int64_t ee = perm ? (int64_t)perm[pos] : (int64_t)pos;
         const float *xr = x + (int64_t)row * (X * K) + c0;
@@ -356,11 +367,18 @@ __device__ __forceinline__ void unrolled_fwd_part(
 #pragma unroll
         for (int k = 0; k < Y; k++) yc[k] = to_vgpr(flip_sign(yn[k], y_flip, k));
         const bool valid = valid_n;
-        e++;
+        e += SUB;
         if (e < e1) fetch(e);
         if (valid) Part::template edge_fwd<CPL>(xc, yc, sc, acc);
     }
-    if (active) {
+    if (SUB > 1) {  // the groups hold partial sums over their edges: add them up
+#pragma unroll
+        for (int i = 0; i < NZ; i++) {
+#pragma unroll
+            for (int off = K; off < kWave; off *= 2) acc[i].v[0] += __shfl_xor(acc[i].v[0], off, kWave);
+        }
+    }
+    if (active && sub == 0) {
         float *orow = out + (int64_t)r * (Z * K) + c0;
 #pragma unroll
         for (int i = 0; i < NZ; i++) store_stream<CPL>(orow + Part::kZ[i] * K, vmul(acc[i], scale));
@@ -433,11 +451,13 @@ __device__ __forceinline__ void unrolled_bwd_part(
     constexpr int X = Part::X, S = Part::S, Z = Part::Z;
     using V = Vec<CPL>;
     using SL = Slice<K, CPL>;
-    using Red = WaveReduceBlocks<Y>;
+    constexpr int SUB = SL::SUB;  // edges of the row walked side by side (channel counts below 64)
+    using Red = WaveReduceBlocks<Y, kWave / SUB>;
 
     static_assert(CPL == 1 || SL::FULL, "several channels per lane need whole slices");
-    const int c_raw = slice * SL::WIDTH + lane;  // further channels of the lane: + 64, + 128, ...
-    const bool active = SL::FULL || c_raw < K;
+    const int sub = SUB > 1 ? lane / K : 0;
+    const int c_raw = SUB > 1 ? lane % K : slice * SL::WIDTH + lane;  // further channels of the lane: + 64, + 128, ...
+    const bool active = SL::FULL || SUB > 1 || c_raw < K;
     const int c0 = active ? c_raw : 0;
 
     V dmr[NZ];
@@ -456,11 +476,16 @@ __device__ __forceinline__ void unrolled_bwd_part(
     V xn[NX], sn[NS];
     float yn[Y];
     bool valid_n = false;
-    int snd_n = 0;
+    int snd_n = 0, pos_n = 0;
     int64_t ee_n = 0;
-    auto fetch = [&](int pos) {
+    auto fetch = [&](int base) {
+        // SUB > 1: the group's own position; past the end of the row it re-reads the last
+        // position and does nothing with it
+        const bool inside = SUB == 1 || base + sub < e1;
+        const int pos = SUB == 1 ? base : (inside ? base + sub : e1 - 1);
+        pos_n = pos;
         const int snd = sender[pos];
-        valid_n = (unsigned)snd < (unsigned)num_nodes;
+        valid_n = inside && (unsigned)snd < (unsigned)num_nodes;
         snd_n = valid_n ? snd : 0;
         ee_n = perm ? (int64_t)perm[pos] : (int64_t)pos;
         const float *xr = x + (int64_t)snd_n * (X * K) + c0;
@@ -486,8 +511,8 @@ __device__ __forceinline__ void unrolled_bwd_part(
         const bool valid = valid_n;
         const int snd = snd_n;
         const int64_t ee = ee_n;
-        const int pos = e;
-        e++;
+        const int pos = pos_n;
+        e += SUB;
         if (e < e1) fetch(e);
         if (!valid) continue;  // padding edge: its dy/ds rows are zero-filled separately
 

@@ -32,6 +32,8 @@ def _random_case(seed, N, E, X, Y, Z, S, K, nnz):
     dict(seed=2, N=30, E=400, X=3, Y=9, Z=10, S=5, K=48, nnz=80),    # idle lanes; leading: table-driven
     dict(seed=3, N=25, E=300, X=6, Y=4, Z=12, S=6, K=128, nnz=100),  # two channels per lane backward
     dict(seed=4, N=20, E=250, X=4, Y=25, Z=9, S=5, K=64, nnz=150),   # harmonics up to l = 4: 25 y components
+    dict(seed=5, N=30, E=500, X=5, Y=6, Z=8, S=4, K=32, nnz=70),     # two edges of a row side by side
+    dict(seed=6, N=30, E=500, X=5, Y=6, Z=8, S=4, K=16, nnz=70),     # four edges side by side
 ])
 def test_random_tables_run_on_generated_kernels(case, layout):
     p = _random_case(**case)
@@ -44,7 +46,8 @@ def test_random_tables_run_on_generated_kernels(case, layout):
     table = _Table.get(p["coef"], np.float32)
     with e3j_amd.config.use(jit=True):  # (a registered table stays registered for the process)
         sig = table.signature(dims, case["K"], e3j_amd.Layout.parse(layout))[0]
-        assert (sig >= 0) == (not leading or case["K"] % 64 == 0)
+        # leading layout: whole waves, or a power-of-two channel count below 64
+        assert (sig >= 0) == (not leading or case["K"] % 64 == 0 or case["K"] in (16, 32))
         out = convolution(p["coef"], x, y, s, snd, rcv, p["params"], layout=layout)
         grads = convolution_bwd(p["coef"], x, y, s, snd, rcv, dm, p["params"], layout=layout)
         with e3j_amd.config.use(jit=True, deterministic=True):
