@@ -174,6 +174,7 @@ int launch_typed(int mode, bool sorted, const void *coef, int num_coef, const vo
         int waves = (int)(kMaxLds / per_wave);
         waves = waves > 4 ? 4 : waves;
         const int64_t blocks = (num_rows + waves - 1) / waves;
+        if (blocks > 0x7fffffffLL) return set_error(E3J_AMD_INVALID_ARGUMENT, "tensor_product: too many rows");
         hipLaunchKernelGGL((tp_inner_kernel<Idx, Val>), dim3((unsigned)blocks), dim3(kWave, waves),
                            per_wave * waves, stream, static_cast<const C *>(coef), num_coef,
                            static_cast<const Val *>(x), sx, static_cast<const Val *>(y), sy,
