@@ -1,6 +1,6 @@
 // Kernel templates of the compile-time-unrolled row-wise tensor product (gfx950, float32):
-// trailing-channels layout for channel counts that are multiples of 64 (first part), and
-// leading-channels layout (second part).
+// trailing-channels layout for channel counts that are multiples of 64, or 16 or 32 (first
+// part), and leading-channels layout (second part).
 //
 // A generated `Sig` type supplies the straight-line Clebsch-Gordan arithmetic of one table
 // (`fwd`, `bwd`); the templates supply the wave <-> (row, 64-channel slice) mapping and the
@@ -48,8 +48,11 @@ const TpSignature &tp_signature(int id);
 template <int K>
 struct RowStore {
     float *p;
+    bool on;  // lanes past the last row store nothing
     template <int I>
-    __device__ __forceinline__ void put(float v) const { __builtin_nontemporal_store(v, p + I * K); }
+    __device__ __forceinline__ void put(float v) const {
+        if (on) __builtin_nontemporal_store(v, p + I * K);
+    }
 };
 template <int K>
 struct RowLoad {
@@ -79,15 +82,40 @@ __device__ __forceinline__ int64_t tp_uniform(int64_t v) {
     return (int64_t)(((unsigned long long)hi << 32) | lo);
 }
 
+// Which row and channel a lane works on.  Whole waves per row for K >= 64; for 16 or 32
+// channels the wave takes 64 / K consecutive rows side by side, one per group of K lanes.
+template <int K>
+struct TpTile {
+    static constexpr int SUB = (K == 16 || K == 32) ? kWave / K : 1;
+    static constexpr int SL = K >= kWave ? K / kWave : 1;
+    static_assert(SUB > 1 || K % kWave == 0, "64-channel slices, or 16 / 32 channels");
+    int64_t r;  // row (clamped to the last one on lanes past the end)
+    int c0;     // channel
+    bool on;    // the lane has a row
+    __device__ __forceinline__ TpTile(int64_t item, int lane, int64_t rows) {
+        if (SUB > 1) {
+            const int64_t rr = item * SUB + lane / K;
+            on = rr < rows;
+            r = on ? rr : rows - 1;
+            c0 = lane % K;
+        } else {
+            r = item / SL;
+            c0 = (int)(item % SL) * kWave + lane;
+            on = true;
+        }
+    }
+    __host__ __device__ static int64_t items(int64_t rows) { return SUB > 1 ? (rows + SUB - 1) / SUB : rows * SL; }
+};
+
 template <typename Sig, int K, int WPB, bool kUniformY>
 __global__ __launch_bounds__(kWave * WPB) void tp_unrolled_fwd_kernel(
     const float *__restrict__ x, const float *__restrict__ y, float *__restrict__ z, int64_t rows, float scale) {
-    constexpr int X = Sig::X, Y = Sig::Y, Z = Sig::Z, SL = K / kWave;
-    static_assert(K % kWave == 0, "whole 64-channel slices");
+    constexpr int X = Sig::X, Y = Sig::Y, Z = Sig::Z;
     const int64_t item = tp_uniform((int64_t)blockIdx.x * WPB + threadIdx.y);
-    if (item >= rows * SL) return;
-    const int64_t r = item / SL;
-    const int c0 = (int)(item % SL) * kWave + threadIdx.x;
+    if (item >= TpTile<K>::items(rows)) return;
+    const TpTile<K> t(item, threadIdx.x, rows);
+    const int64_t r = t.r;
+    const int c0 = t.c0;
     float xv[X], yv[Y];
     const float *xr = x + r * (X * K) + c0;
 #pragma unroll
@@ -101,7 +129,7 @@ __global__ __launch_bounds__(kWave * WPB) void tp_unrolled_fwd_kernel(
 #pragma unroll
         for (int k = 0; k < Y; k++) yv[k] = __builtin_nontemporal_load(yr + k * K);
     }
-    Sig::fwd(xv, yv, RowStore<K>{z + r * (Z * K) + c0});
+    Sig::fwd(xv, yv, RowStore<K>{z + r * (Z * K) + c0, t.on});
 }
 
 // MAP backward: dz is read once for both cotangents.
@@ -109,11 +137,12 @@ template <typename Sig, int K, int WPB>
 __global__ __launch_bounds__(kWave * WPB) void tp_unrolled_bwd_map_kernel(
     const float *__restrict__ x, const float *__restrict__ y, const float *__restrict__ dz,
     float *__restrict__ dx, float *__restrict__ dy, int64_t rows, float scale) {
-    constexpr int X = Sig::X, Y = Sig::Y, Z = Sig::Z, SL = K / kWave;
+    constexpr int X = Sig::X, Y = Sig::Y, Z = Sig::Z;
     const int64_t item = tp_uniform((int64_t)blockIdx.x * WPB + threadIdx.y);
-    if (item >= rows * SL) return;
-    const int64_t r = item / SL;
-    const int c0 = (int)(item % SL) * kWave + threadIdx.x;
+    if (item >= TpTile<K>::items(rows)) return;
+    const TpTile<K> t(item, threadIdx.x, rows);
+    const int64_t r = t.r;
+    const int c0 = t.c0;
     float xv[X], yv[Y], dxv[X], dyv[Y];
     const float *xr = x + r * (X * K) + c0;
     const float *yr = y + r * (Y * K) + c0;
@@ -122,6 +151,7 @@ __global__ __launch_bounds__(kWave * WPB) void tp_unrolled_bwd_map_kernel(
 #pragma unroll
     for (int k = 0; k < Y; k++) { yv[k] = __builtin_nontemporal_load(yr + k * K); dyv[k] = 0.f; }
     Sig::bwd(xv, yv, RowLoad<K>{dz + r * (Z * K) + c0, scale}, dxv, dyv);
+    if (!t.on) return;
     float *dxr = dx + r * (X * K) + c0;
     float *dyr = dy + r * (Y * K) + c0;
 #pragma unroll
@@ -135,8 +165,8 @@ __global__ __launch_bounds__(kWave * WPB) void tp_unrolled_bwd_map_kernel(
 // first of them stores the row (fixed order, no atomics).
 template <int K>
 struct TpUniformGeometry {
-    static constexpr int SL = K / kWave;              // waves per row
-    static constexpr int RPB = SL >= 4 ? 1 : 4 / SL;  // rows per block
+    static constexpr int SL = K >= kWave ? K / kWave : 1;  // waves per row
+    static constexpr int RPB = SL >= 4 ? 1 : 4 / SL;       // rows per block
     static constexpr int WPB = SL * RPB;
 };
 
@@ -238,11 +268,12 @@ template <typename Sig, int K, int WPB>
 __global__ __launch_bounds__(kWave * WPB) void tp_unrolled_bwd_inner_kernel(
     const float *__restrict__ x, const float *__restrict__ y, const float *__restrict__ dz,
     float *__restrict__ dx, float *__restrict__ dy, int64_t rows, float scale) {
-    constexpr int X = Sig::X, Y = Sig::Y, Z = Sig::Z, SL = K / kWave;
+    constexpr int X = Sig::X, Y = Sig::Y, Z = Sig::Z;
     const int64_t item = tp_uniform((int64_t)blockIdx.x * WPB + threadIdx.y);
-    if (item >= rows * SL) return;
-    const int64_t r = item / SL;
-    const int c0 = (int)(item % SL) * kWave + threadIdx.x;
+    if (item >= TpTile<K>::items(rows)) return;
+    const TpTile<K> t(item, threadIdx.x, rows);
+    const int64_t r = t.r;
+    const int c0 = t.c0;
     float xv[X], yv[Y], dxv[X], dyv[Y];
     const float *xr = x + r * (X * K) + c0;
     const float *yr = y + r * (Y * K) + c0;
@@ -251,12 +282,71 @@ __global__ __launch_bounds__(kWave * WPB) void tp_unrolled_bwd_inner_kernel(
 #pragma unroll
     for (int k = 0; k < Y; k++) { yv[k] = __builtin_nontemporal_load(yr + k * K); dyv[k] = 0.f; }
     Sig::bwd(xv, yv, UniformLoad<Z>{dz + r * Z, scale}, dxv, dyv);
+    if (!t.on) return;
     float *dxr = dx + r * (X * K) + c0;
     float *dyr = dy + r * (Y * K) + c0;
 #pragma unroll
     for (int j = 0; j < X; j++) __builtin_nontemporal_store(dxv[j], dxr + j * K);
 #pragma unroll
     for (int k = 0; k < Y; k++) __builtin_nontemporal_store(dyv[k], dyr + k * K);
+}
+
+// 16 or 32 channels, kinds that sum over the channels: the groups of K lanes reduce on their
+// own and store their own row; no slices to combine.
+template <typename Sig, int K, int WPB>
+__global__ __launch_bounds__(kWave * WPB) void tp_unrolled_bwd_uniform_narrow_kernel(
+    const float *__restrict__ x, const float *__restrict__ y, const float *__restrict__ dz,
+    float *__restrict__ dx, float *__restrict__ dy, int64_t rows, float scale) {
+    constexpr int X = Sig::X, Y = Sig::Y, Z = Sig::Z;
+    using Red = WaveReduceBlocks<Y, K>;
+    const int64_t item = tp_uniform((int64_t)blockIdx.x * WPB + threadIdx.y);
+    if (item >= TpTile<K>::items(rows)) return;
+    const int lane = threadIdx.x;
+    const TpTile<K> t(item, lane, rows);
+    const int64_t r = t.r;
+    float yv[Y], dyv[Red::P], xv[X], dxv[X];
+    const float *yr = y + r * Y;
+#pragma unroll
+    for (int k = 0; k < Y; k++) yv[k] = yr[k];
+#pragma unroll
+    for (int k = 0; k < Red::P; k++) dyv[k] = 0.f;
+    const float *xr = x + r * (X * K) + t.c0;
+#pragma unroll
+    for (int j = 0; j < X; j++) { xv[j] = __builtin_nontemporal_load(xr + j * K); dxv[j] = 0.f; }
+    Sig::bwd(xv, yv, RowLoad<K>{dz + r * (Z * K) + t.c0, scale}, dxv, dyv);
+    if (t.on) {
+        float *dxr = dx + r * (X * K) + t.c0;
+#pragma unroll
+        for (int j = 0; j < X; j++) __builtin_nontemporal_store(dxv[j], dxr + j * K);
+    }
+    const bool on = t.on;
+    float *dyr = dy + r * Y;
+    Red::run(dyv, lane, [&](int k, float total) { if (on) dyr[k] = total; });
+}
+
+template <typename Sig, int K, int WPB>
+__global__ __launch_bounds__(kWave * WPB) void tp_unrolled_fwd_inner_narrow_kernel(
+    const float *__restrict__ x, const float *__restrict__ y, float *__restrict__ z, int64_t rows, float scale) {
+    constexpr int X = Sig::X, Y = Sig::Y, Z = Sig::Z;
+    using Red = WaveReduceBlocks<Z, K>;
+    const int64_t item = tp_uniform((int64_t)blockIdx.x * WPB + threadIdx.y);
+    if (item >= TpTile<K>::items(rows)) return;
+    const int lane = threadIdx.x;
+    const TpTile<K> t(item, lane, rows);
+    const int64_t r = t.r;
+    float xv[X], yv[Y], zv[Red::P];
+    const float *xr = x + r * (X * K) + t.c0;
+    const float *yr = y + r * (Y * K) + t.c0;
+#pragma unroll
+    for (int j = 0; j < X; j++) xv[j] = __builtin_nontemporal_load(xr + j * K) * scale;
+#pragma unroll
+    for (int k = 0; k < Y; k++) yv[k] = __builtin_nontemporal_load(yr + k * K);
+#pragma unroll
+    for (int i = Z; i < Red::P; i++) zv[i] = 0.f;
+    Sig::fwd(xv, yv, RegStore<Z>{zv});
+    const bool on = t.on;
+    float *zr = z + r * Z;
+    Red::run(zv, lane, [&](int i, float total) { if (on) zr[i] = total; });
 }
 
 inline int tp_grid(int64_t items, int wpb, unsigned *blocks) {
@@ -273,13 +363,17 @@ int launch_tp_unrolled_fwd(int64_t rows, int, float scale, const float *x, const
     constexpr int WPB = 4;
     if (rows == 0) return E3J_AMD_OK;
     unsigned blocks;
-    if (kKind == 2) {
+    if constexpr (kKind == 2 && TpTile<K>::SUB > 1) {
+        if (int rc = tp_grid(TpTile<K>::items(rows), WPB, &blocks)) return rc;
+        hipLaunchKernelGGL((tp_unrolled_fwd_inner_narrow_kernel<Sig, K, WPB>), dim3(blocks), dim3(kWave, WPB), 0,
+                           stream, x, y, z, rows, scale);
+    } else if constexpr (kKind == 2) {
         using G = TpUniformGeometry<K>;
         if (int rc = tp_grid(rows, G::RPB, &blocks)) return rc;
         hipLaunchKernelGGL((tp_unrolled_fwd_inner_kernel<Sig, K>), dim3(blocks), dim3(kWave, G::WPB), 0, stream,
                            x, y, z, rows, scale);
     } else {
-        if (int rc = tp_grid(rows * (K / kWave), WPB, &blocks)) return rc;
+        if (int rc = tp_grid(TpTile<K>::items(rows), WPB, &blocks)) return rc;
         hipLaunchKernelGGL((tp_unrolled_fwd_kernel<Sig, K, WPB, kKind == 1>), dim3(blocks), dim3(kWave, WPB), 0,
                            stream, x, y, z, rows, scale);
     }
@@ -292,17 +386,21 @@ int launch_tp_unrolled_bwd(int64_t rows, int, float scale, const float *x, const
     constexpr int WPB = 4;
     if (rows == 0) return E3J_AMD_OK;
     unsigned blocks;
-    if (kKind == 2) {
-        if (int rc = tp_grid(rows * (K / kWave), WPB, &blocks)) return rc;
+    if constexpr (kKind == 2) {
+        if (int rc = tp_grid(TpTile<K>::items(rows), WPB, &blocks)) return rc;
         hipLaunchKernelGGL((tp_unrolled_bwd_inner_kernel<Sig, K, WPB>), dim3(blocks), dim3(kWave, WPB), 0, stream,
                            x, y, dz, dx, dy, rows, scale);
-    } else if (kKind == 1) {
+    } else if constexpr (kKind == 1 && TpTile<K>::SUB > 1) {
+        if (int rc = tp_grid(TpTile<K>::items(rows), WPB, &blocks)) return rc;
+        hipLaunchKernelGGL((tp_unrolled_bwd_uniform_narrow_kernel<Sig, K, WPB>), dim3(blocks), dim3(kWave, WPB), 0,
+                           stream, x, y, dz, dx, dy, rows, scale);
+    } else if constexpr (kKind == 1) {
         using G = TpUniformGeometry<K>;
         if (int rc = tp_grid(rows, G::RPB, &blocks)) return rc;
         hipLaunchKernelGGL((tp_unrolled_bwd_uniform_kernel<Sig, K>), dim3(blocks), dim3(kWave, G::WPB), 0, stream,
                            x, y, dz, dx, dy, rows, scale);
     } else {
-        if (int rc = tp_grid(rows * (K / kWave), WPB, &blocks)) return rc;
+        if (int rc = tp_grid(TpTile<K>::items(rows), WPB, &blocks)) return rc;
         hipLaunchKernelGGL((tp_unrolled_bwd_map_kernel<Sig, K, WPB>), dim3(blocks), dim3(kWave, WPB), 0, stream,
                            x, y, dz, dx, dy, rows, scale);
     }

@@ -88,7 +88,7 @@ class _Table:
                     from . import jit as _jit
                     c = Coef.unpack(self.packed, self.val_np_dtype)
                     trailing = layout == Layout.TRAILING_CHANNELS
-                    if (channels % 64 == 0 or not trailing) and _jit.register_tp(
+                    if (channels % 64 == 0 or channels in (16, 32) or not trailing) and _jit.register_tp(
                             c.val, c.idx.astype(np.int64), (num_out, num_x, num_y), channels if trailing else 0):
                         sig = find()
             hit = self._signature[key] = (sig, float(scale.value))

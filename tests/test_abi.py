@@ -102,7 +102,8 @@ def test_tensor_product_signature_lookup():
     assert b"K=128" in lib.e3j_amd_tp_signature_name(a) and b"MAP" in lib.e3j_amd_tp_signature_name(a)
     assert b"without channel axis" in lib.e3j_amd_tp_signature_name(b)
     assert find(packed, 128, 2) >= 0 and b"INNER" in lib.e3j_amd_tp_signature_name(find(packed, 128, 2))
-    assert find(packed, 64, 0) >= 0 and find(packed, 96, 0) == -1 and find(packed, 32, 0) == -1
+    assert find(packed, 64, 0) >= 0 and find(packed, 96, 0) == -1 and find(packed, 16, 0) == -1
+    assert b"K=32" in lib.e3j_amd_tp_signature_name(find(packed, 32, 2))   # two rows side by side in a wave
     # leading layout: one kernel for every multiple of 4 channels (MAP); whole waves per row (uniform y)
     lead = find(packed, 100, 0, _lib.LAYOUT_LEADING)
     assert lead >= 0 and lead == find(packed, 4, 0, _lib.LAYOUT_LEADING) and lead not in (a, b)
