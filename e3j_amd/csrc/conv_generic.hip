@@ -21,7 +21,98 @@
 namespace e3j_amd {
 namespace {
 
+// Value of lane `src` (a wave-uniform number) of a per-lane variable, as a wave-uniform value.
+template <typename T>
+__device__ __forceinline__ T lane_pick(T v, int src) {
+    if constexpr (sizeof(T) == 2) {
+        const uint32_t w = __builtin_amdgcn_readlane((uint32_t)__builtin_bit_cast(uint16_t, v), src);
+        return __builtin_bit_cast(T, (uint16_t)w);
+    } else {
+        static_assert(sizeof(T) % 4 == 0, "whole registers");
+        uint32_t w[sizeof(T) / 4];
+        __builtin_memcpy(w, &v, sizeof(T));
+#pragma unroll
+        for (int q = 0; q < (int)(sizeof(T) / 4); q++) w[q] = __builtin_amdgcn_readlane(w[q], src);
+        __builtin_memcpy(&v, w, sizeof(T));
+        return v;
+    }
+}
+
+template <typename Val>
+struct CoefFields {  // one table entry, wave-uniform
+    int i, j, k, l;
+    Val val;
+};
+
+// Sixty-four consecutive entries of the table, one per lane (one coalesced vector load), handed
+// out one at a time as wave-uniform values through lane reads: the coefficient stream costs
+// no scalar-memory round trip per entry.
 template <typename Idx, typename Val>
+struct CoefChunk {
+    Val val;
+    uint32_t w[sizeof(Idx) == 1 ? 1 : 4];
+
+    __device__ __forceinline__ void load(const Coef4D<Idx, Val> *__restrict__ coef, int n0, int num_coef, int lane) {
+        int n = n0 + lane;
+        if (n >= num_coef) n = num_coef - 1;
+        const Coef4D<Idx, Val> c = coef[n];
+        val = c.val;
+        if constexpr (sizeof(Idx) == 1) {
+            w[0] = (uint32_t)c.i | ((uint32_t)c.j << 8) | ((uint32_t)c.k << 16) | ((uint32_t)c.l << 24);
+        } else {
+            w[0] = (uint32_t)c.i; w[1] = (uint32_t)c.j; w[2] = (uint32_t)c.k; w[3] = (uint32_t)c.l;
+        }
+    }
+    __device__ __forceinline__ CoefFields<Val> pick(int u) const {
+        CoefFields<Val> f;
+        f.val = lane_pick(val, u);
+        if constexpr (sizeof(Idx) == 1) {
+            const uint32_t a = __builtin_amdgcn_readlane(w[0], u);
+            f.i = (int)(a & 255u); f.j = (int)((a >> 8) & 255u); f.k = (int)((a >> 16) & 255u); f.l = (int)(a >> 24);
+        } else {
+            f.i = (int)__builtin_amdgcn_readlane(w[0], u); f.j = (int)__builtin_amdgcn_readlane(w[1], u);
+            f.k = (int)__builtin_amdgcn_readlane(w[2], u); f.l = (int)__builtin_amdgcn_readlane(w[3], u);
+        }
+        return f;
+    }
+};
+
+// A strided row of global memory into a lane-private LDS column, sixteen loads in flight.
+// `row` must be readable on every lane (lanes past the last channel pass the last channel's
+// row); lanes that are not `active` store zeros.
+template <typename Val>
+__device__ __forceinline__ void stage_column(Val *col, const Val *row, int64_t stride, int n, bool active) {
+    constexpr int B = 16;
+    for (int j0 = 0; j0 < n; j0 += B) {
+        Val t[B];
+#pragma unroll
+        for (int v = 0; v < B; v++) {
+            const int j = j0 + v < n ? j0 + v : n - 1;
+            t[v] = row[(int64_t)j * stride];
+        }
+#pragma unroll
+        for (int v = 0; v < B; v++) {
+            const int j = j0 + v < n ? j0 + v : n - 1;  // the tail rewrites the last element
+            col[j * kWave] = active ? t[v] : Val(0);
+        }
+    }
+}
+
+// y of one edge for the coefficient loop: up to 64 components sit in one register (lane k
+// holds y[k]) and are read as wave-uniform values; longer y rows are read from memory.
+template <typename Val, bool kYLane>
+struct EdgeY {
+    Val reg;
+    const Val *row;
+    __device__ __forceinline__ EdgeY(const Val *ye, int num_y, int lane) : reg(Val(0)), row(ye) {
+        if (kYLane && lane < num_y) reg = ye[lane];
+    }
+    __device__ __forceinline__ Val operator[](int k) const { return kYLane ? lane_pick(reg, k) : row[k]; }
+};
+
+constexpr int kCoefBatch = 8;  // table entries whose LDS reads are issued together
+
+template <typename Idx, typename Val, bool kYLane>
 __global__ void generic_fwd_kernel(const Coef4D<Idx, Val> *__restrict__ coef, int num_coef,
                                    const Val *__restrict__ x, RowLayout lx,
                                    const Val *__restrict__ y, int num_y,
@@ -41,35 +132,56 @@ __global__ void generic_fwd_kernel(const Coef4D<Idx, Val> *__restrict__ coef, in
     const int r = row_order ? row_order[q] : q;
     const int c = (int)(item % nchunks) * kWave + lane;
     const bool active = c < channels;
+    const int cr = active ? c : channels - 1;  // channel whose rows an idle lane reads
 
     Val *acc = reinterpret_cast<Val *>(smem_raw) + (size_t)wave * (Z + X + S) * kWave + lane;
     Val *xs = acc + (size_t)Z * kWave;
     Val *ss = xs + (size_t)X * kWave;
     for (int i = 0; i < Z; i++) acc[i * kWave] = Val(0);
 
+    CoefChunk<Idx, Val> next;
+    if (num_coef > 0) next.load(coef, 0, num_coef, lane);
+
     const int e0 = row_ptr[r], e1 = row_ptr[r + 1];
     for (int e = e0; e < e1; e++) {
         const int snd = other[e];
         if ((unsigned)snd >= (unsigned)num_nodes) continue;  // padding edge
         const int64_t ee = perm ? (int64_t)perm[e] : (int64_t)e;
-        const Val *xrow = x + (int64_t)snd * lx.row + (int64_t)c * lx.chan;
-        const Val *srow = s + ee * ls.row + (int64_t)c * ls.chan;
-        for (int j = 0; j < X; j++) xs[j * kWave] = active ? xrow[(int64_t)j * lx.dim] : Val(0);
-        for (int l = 0; l < S; l++) ss[l * kWave] = active ? srow[(int64_t)l * ls.dim] : Val(0);
-        const Val *ye = y + ee * num_y;
+        stage_column(xs, x + (int64_t)snd * lx.row + (int64_t)cr * lx.chan, lx.dim, X, active);
+        stage_column(ss, s + ee * ls.row + (int64_t)cr * ls.chan, ls.dim, S, active);
+        const EdgeY<Val, kYLane> ye(y + ee * num_y, num_y, lane);
 
+        // runs of equal (output coordinate, path): the old accumulator and the path's scalar
+        // are read when the run starts, so that its end is one LDS write
         int cur_i = -1, cur_l = 0;
-        Val msg = Val(0);
-        for (int n = 0; n < num_coef; n++) {
-            const Coef4D<Idx, Val> cf = coef[n];
-            const int ci = (int)cf.i, cl = (int)cf.l;
-            if (ci != cur_i || cl != cur_l) {
-                if (cur_i >= 0) acc[cur_i * kWave] += ss[cur_l * kWave] * msg;
-                cur_i = ci; cur_l = cl; msg = Val(0);
+        Val msg = Val(0), before = Val(0), scalar = Val(0);
+        for (int n0 = 0; n0 < num_coef; n0 += kWave) {
+            const CoefChunk<Idx, Val> chunk = next;
+            next.load(coef, n0 + kWave < num_coef ? n0 + kWave : 0, num_coef, lane);
+            const int nn = num_coef - n0 < kWave ? num_coef - n0 : kWave;
+            for (int u = 0; u < nn; u += kCoefBatch) {
+                CoefFields<Val> cf[kCoefBatch];
+                Val xv[kCoefBatch], yv[kCoefBatch];
+#pragma unroll
+                for (int v = 0; v < kCoefBatch; v++) {
+                    cf[v] = chunk.pick(u + v < nn ? u + v : nn - 1);
+                    xv[v] = xs[cf[v].j * kWave];
+                    yv[v] = ye[cf[v].k];
+                }
+#pragma unroll
+                for (int v = 0; v < kCoefBatch; v++) {
+                    if (u + v >= nn) break;
+                    if (cf[v].i != cur_i || cf[v].l != cur_l) {
+                        if (cur_i >= 0) acc[cur_i * kWave] = before + scalar * msg;
+                        cur_i = cf[v].i; cur_l = cf[v].l; msg = Val(0);
+                        before = acc[cur_i * kWave];
+                        scalar = ss[cur_l * kWave];
+                    }
+                    msg += (xv[v] * yv[v]) * cf[v].val;
+                }
             }
-            msg += (xs[(int)cf.j * kWave] * ye[(int)cf.k]) * cf.val;
         }
-        if (cur_i >= 0) acc[cur_i * kWave] += ss[cur_l * kWave] * msg;
+        if (cur_i >= 0) acc[cur_i * kWave] = before + scalar * msg;
     }
     if (active) {
         Val *orow = out + (int64_t)r * lo.row + (int64_t)c * lo.chan;
@@ -80,7 +192,7 @@ __global__ void generic_fwd_kernel(const Coef4D<Idx, Val> *__restrict__ coef, in
 // kGroupIsReceiver: rows are receivers (dm row fixed, x gathered, dx scattered with
 // atomics into a zero-filled buffer).  Otherwise rows are senders (x row fixed, dm
 // gathered, dx accumulated in place by the owning wave).
-template <typename Idx, typename Val, bool kGroupIsReceiver>
+template <typename Idx, typename Val, bool kGroupIsReceiver, bool kYLane>
 __global__ void generic_bwd_kernel(const Coef4D<Idx, Val> *__restrict__ coef, int num_coef,
                                    const Val *__restrict__ x, RowLayout lx,
                                    const Val *__restrict__ y, int num_y,
@@ -118,6 +230,9 @@ __global__ void generic_bwd_kernel(const Coef4D<Idx, Val> *__restrict__ coef, in
         }
     }
 
+    CoefChunk<Idx, Val> next;
+    if (num_coef > 0) next.load(coef, 0, num_coef, lane);
+
     const int e0 = row_ptr[g], e1 = row_ptr[g + 1];
     for (int e = e0; e < e1; e++) {
         const int o = other[e];
@@ -125,37 +240,47 @@ __global__ void generic_bwd_kernel(const Coef4D<Idx, Val> *__restrict__ coef, in
         const int64_t ee = perm ? (int64_t)perm[e] : (int64_t)e;
         const int xnode = kGroupIsReceiver ? o : g;
         const int znode = kGroupIsReceiver ? g : o;
-        const Val *ye = y + ee * num_y;
+        const EdgeY<Val, kYLane> ye(y + ee * num_y, num_y, lane);
         for (int k = 0; k < num_y; k++) dyc[k * kWave] = Val(0);
 
         for (int q = 0; q < nchunks; q++) {
             const int c = q * kWave + lane;
             const bool active = c < channels;
-            const Val *xrow = x + (int64_t)xnode * lx.row + (int64_t)c * lx.chan;
-            const Val *zrow = dm + (int64_t)znode * lo.row + (int64_t)c * lo.chan;
-            const Val *srow = s + ee * ls.row + (int64_t)c * ls.chan;
-            for (int i = 0; i < Z; i++) zc[i * kWave] = active ? zrow[(int64_t)i * lo.dim] : Val(0);
-            for (int j = 0; j < X; j++) {
-                xc[j * kWave] = active ? xrow[(int64_t)j * lx.dim] : Val(0);
-                dxc[j * kWave] = Val(0);
-            }
-            for (int l = 0; l < S; l++) {
-                sc[l * kWave] = active ? srow[(int64_t)l * ls.dim] : Val(0);
-                dsc[l * kWave] = Val(0);
-            }
-            for (int n = 0; n < num_coef; n++) {
-                const Coef4D<Idx, Val> cf = coef[n];
-                // cols_ji: the table's first two columns hold (x, output) coordinates, as in the
-                // dx-transposed copy the reference passes (src/e3j/ops/convolution.py:367).
-                const int ci = cols_ji ? (int)cf.j : (int)cf.i, cj = cols_ji ? (int)cf.i : (int)cf.j;
-                const int ck = (int)cf.k, cl = (int)cf.l;
-                const Val dz = zc[ci * kWave];
-                const Val xv = xc[cj * kWave];
-                const Val gz = dz * sc[cl * kWave];
-                const Val t = cf.val * ye[ck];
-                dxc[cj * kWave] += t * gz;
-                dsc[cl * kWave] += (t * dz) * xv;
-                dyc[ck * kWave] += (cf.val * gz) * xv;
+            const int cr = active ? c : channels - 1;  // channel whose rows an idle lane reads
+            stage_column(zc, dm + (int64_t)znode * lo.row + (int64_t)cr * lo.chan, lo.dim, Z, active);
+            stage_column(xc, x + (int64_t)xnode * lx.row + (int64_t)cr * lx.chan, lx.dim, X, active);
+            stage_column(sc, s + ee * ls.row + (int64_t)cr * ls.chan, ls.dim, S, active);
+            for (int j = 0; j < X; j++) dxc[j * kWave] = Val(0);
+            for (int l = 0; l < S; l++) dsc[l * kWave] = Val(0);
+            for (int n0 = 0; n0 < num_coef; n0 += kWave) {
+                const CoefChunk<Idx, Val> chunk = next;
+                next.load(coef, n0 + kWave < num_coef ? n0 + kWave : 0, num_coef, lane);
+                const int nn = num_coef - n0 < kWave ? num_coef - n0 : kWave;
+                for (int u = 0; u < nn; u += kCoefBatch) {
+                    CoefFields<Val> cf[kCoefBatch];
+                    Val dz[kCoefBatch], xv[kCoefBatch], sv[kCoefBatch], yv[kCoefBatch];
+#pragma unroll
+                    for (int v = 0; v < kCoefBatch; v++) {
+                        cf[v] = chunk.pick(u + v < nn ? u + v : nn - 1);
+                        // cols_ji: the table's first two columns hold (x, output) coordinates, as in
+                        // the dx-transposed copy the reference passes (src/e3j/ops/convolution.py:367).
+                        if (cols_ji) { const int t = cf[v].i; cf[v].i = cf[v].j; cf[v].j = t; }
+                        dz[v] = zc[cf[v].i * kWave];
+                        xv[v] = xc[cf[v].j * kWave];
+                        sv[v] = sc[cf[v].l * kWave];
+                        yv[v] = ye[cf[v].k];
+                    }
+#pragma unroll
+                    for (int v = 0; v < kCoefBatch; v++) {
+                        if (u + v >= nn) break;
+                        const Val gz = dz[v] * sv[v];
+                        const Val t = cf[v].val * yv[v];
+                        // (LDS float adds retire far slower than a read, an add and a write)
+                        dxc[cf[v].j * kWave] += t * gz;
+                        dsc[cf[v].l * kWave] += (t * dz[v]) * xv[v];
+                        dyc[cf[v].k * kWave] += (cf[v].val * gz) * xv[v];
+                    }
+                }
             }
             if (active) {
                 Val *dsrow = ds + ee * ls.row + (int64_t)c * ls.chan;
@@ -230,7 +355,8 @@ int run_fwd(const e3j_amd_conv_params &p, const void *coef, const void *x, const
                          " exceeds the LDS capacity of the table-driven kernel");
     const int waves = pick_waves(per_wave, 64 * 1024);
     const size_t lds = per_wave * waves;
-    auto kernel = generic_fwd_kernel<Idx, Val>;
+    // y rows of up to 64 components travel in a register of the wave
+    auto kernel = p.num_y <= kWave ? generic_fwd_kernel<Idx, Val, true> : generic_fwd_kernel<Idx, Val, false>;
     if (lds > 64 * 1024) {
         int rc = check_hip(hipFuncSetAttribute(reinterpret_cast<const void *>(kernel),
                                                hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds),
@@ -289,7 +415,8 @@ int run_bwd(const e3j_amd_conv_params &p, bool group_is_receiver, const void *co
     if (rc) return rc;
 #define E3J_LAUNCH_BWD(FLAG)                                                                      \
     do {                                                                                          \
-        auto kernel = generic_bwd_kernel<Idx, Val, FLAG>;                                         \
+        auto kernel = p.num_y <= kWave ? generic_bwd_kernel<Idx, Val, FLAG, true>                 \
+                                       : generic_bwd_kernel<Idx, Val, FLAG, false>;               \
         if (lds > 64 * 1024) {                                                                    \
             rc = check_hip(hipFuncSetAttribute(reinterpret_cast<const void *>(kernel),            \
                                                hipFuncAttributeMaxDynamicSharedMemorySize,        \
