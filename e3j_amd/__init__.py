@@ -1,8 +1,8 @@
 """MI355X-native fused equivariant message-passing convolution.
 
 Public names follow the reference package for this path: `Convolution`,
-`convolution`, `convolution_bwd`, `tensor_product`, `tensor_product_bwd`, `GraphCSR`,
-`Coef4D`, `O3Space`, `config`.
+`convolution`, `convolution_bwd`, `TensorProduct`, `tensor_product`, `tensor_product_bwd`,
+`Harmonics`, `GraphCSR`, `Coef4D`, `O3Space`, `config`.
 Importing the package does not load the kernel library; the first operator call does,
 and fails if `e3j_amd/lib/libe3j_amd.so` has not been built.
 """
@@ -10,6 +10,7 @@ and fails if `e3j_amd/lib/libe3j_amd.so` has not been built.
 from .coef import Coef, Coef4D, resolve_val_dtype
 from .convolution import Convolution
 from .graph import DUMMY_INDEX, GraphCSR
+from .harmonics import Harmonics
 from .ops import (ConvolutionBatchingWarning, ConvolutionParams, CUDAConvolutionParams, TableDrivenKernelWarning,
                   convolution, convolution_batched, convolution_bwd)
 from .options import Config, GraphOrdering, Layout, MixingMode, TensorProductNormalization, config
@@ -24,7 +25,7 @@ Space = O3Space
 __all__ = [
     "Coef", "Coef4D", "Config", "Convolution", "ConvolutionBatchingWarning", "ConvolutionParams",
     "TableDrivenKernelWarning",
-    "CUDAConvolutionParams", "DUMMY_INDEX", "GraphCSR", "GraphOrdering", "Layout", "O3Irrep",
+    "CUDAConvolutionParams", "DUMMY_INDEX", "GraphCSR", "GraphOrdering", "Harmonics", "Layout", "O3Irrep",
     "O3Space", "ScalarMixing", "Space", "TensorProduct", "TensorProductNormalization", "config",
     "convolution", "convolution_batched", "convolution_bwd", "resolve_val_dtype",
     "CUDATensorProductParams", "MixingMode", "TensorProductParams", "tensor_product", "tensor_product_batched", "tensor_product_bwd",
