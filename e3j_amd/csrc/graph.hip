@@ -67,6 +67,40 @@ __global__ void copy_i32_kernel(const int32_t *__restrict__ src, int32_t *__rest
     for (int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; i < n; i += stride) dst[i] = src[i];
 }
 
+// Rows with more than twice the mean number of edges ("long rows"): flag per list position.
+__global__ void long_row_flags_kernel(const int32_t *__restrict__ order, const int32_t *__restrict__ row_ptr,
+                                      int num_nodes, int32_t *__restrict__ flags) {
+    const int i = blockIdx.x * blockDim.x + threadIdx.x;
+    if (i >= num_nodes) return;
+    const int r = order[i];
+    const int64_t degree = row_ptr[r + 1] - row_ptr[r];
+    flags[i] = degree * num_nodes > 2 * (int64_t)row_ptr[num_nodes] ? 1 : 0;
+}
+
+// The kernels hand one contiguous eighth of the row list to each XCD and every XCD walks its
+// eighth front to back.  Long rows started late leave the machine waiting for a few waves at
+// the end, so they are dealt to the fronts of the eighths: eighth p takes the p-th eighth of the
+// long rows, then the p-th eighth of the others, both in list order.  `rank` is the
+// inclusive prefix sum of `flags`.  Without long rows the list is unchanged.
+__global__ void deal_long_rows_kernel(const int32_t *__restrict__ order, const int32_t *__restrict__ flags,
+                                      const int32_t *__restrict__ rank, int num_nodes,
+                                      int32_t *__restrict__ dealt) {
+    const int i = blockIdx.x * blockDim.x + threadIdx.x;
+    if (i >= num_nodes) return;
+    constexpr int64_t kParts = 8;
+    const int64_t num_long = rank[num_nodes - 1], num_short = num_nodes - num_long;
+    const bool is_long = flags[i] != 0;
+    const int64_t mine = is_long ? rank[i] - 1 : i - rank[i];  // position among the rows of its kind
+    const int64_t kind = is_long ? num_long : num_short;
+    int64_t part = 0;
+    while (part < kParts - 1 && (part + 1) * kind / kParts <= mine) part++;
+    const int64_t start = part * num_long / kParts + part * num_short / kParts;
+    const int64_t longs_here = (part + 1) * num_long / kParts - part * num_long / kParts;
+    const int64_t at = is_long ? start + (mine - part * num_long / kParts)
+                               : start + longs_here + (mine - part * num_short / kParts);
+    dealt[at] = order[i];
+}
+
 size_t align_up(size_t v, size_t a = 256) { return (v + a - 1) / a * a; }
 
 unsigned grid_for(int64_t n) { return (unsigned)std::max<int64_t>(1, std::min<int64_t>((n + 255) / 256, 4096)); }
@@ -172,8 +206,9 @@ int e3j_amd_wrap_index(const int32_t *index, int64_t n, int32_t num_nodes, int32
 
 size_t e3j_amd_order_workspace_bytes(int32_t num_nodes) {
     if (num_nodes < 0) return 0;
-    // [sort temp | label a | label b | keys in | keys out | order tmp]
-    return align_up(sort_temp_bytes(num_nodes)) + 5 * align_up(sizeof(int32_t) * (size_t)num_nodes) + 256;
+    // [sort / scan temp | label a | label b | keys in | keys out | order tmp]
+    return align_up(std::max(sort_temp_bytes(num_nodes), scan_temp_bytes(num_nodes))) +
+           5 * align_up(sizeof(int32_t) * (size_t)num_nodes) + 256;
 }
 
 int e3j_amd_locality_order(const int32_t *other, const int32_t *row_ptr, int32_t num_nodes,
@@ -185,7 +220,7 @@ int e3j_amd_locality_order(const int32_t *other, const int32_t *row_ptr, int32_t
         return set_error(E3J_AMD_INVALID_ARGUMENT, "locality_order: null operand");
     hipStream_t stream = static_cast<hipStream_t>(stream_);
     unsigned char *ws = static_cast<unsigned char *>(workspace);
-    const size_t sort_bytes = sort_temp_bytes(num_nodes);
+    const size_t sort_bytes = std::max(sort_temp_bytes(num_nodes), scan_temp_bytes(num_nodes));
     const size_t vec = align_up(sizeof(int32_t) * (size_t)num_nodes);
     void *sort_temp = ws;
     int32_t *lab_a = reinterpret_cast<int32_t *>(ws + align_up(sort_bytes));
@@ -222,6 +257,20 @@ int e3j_amd_locality_order(const int32_t *other, const int32_t *row_ptr, int32_t
         hipLaunchKernelGGL(copy_i32_kernel, dim3(ngrid), dim3(256), 0, stream, order_tmp, order,
                            (int64_t)num_nodes);
     }
+    // long rows to the fronts of the eighths of the list
+    int32_t *flags = reinterpret_cast<int32_t *>(keys_in), *rank = reinterpret_cast<int32_t *>(keys_out);
+    hipLaunchKernelGGL(long_row_flags_kernel, dim3(rows_grid), dim3(256), 0, stream, order, row_ptr, num_nodes,
+                       flags);
+    rc = check_hip(hipGetLastError(), "locality_order flags");
+    if (rc) return rc;
+    size_t scan_bytes = sort_bytes;
+    rc = check_hip(hipcub::DeviceScan::InclusiveSum(sort_temp, scan_bytes, flags, rank, num_nodes, stream),
+                   "locality_order scan");
+    if (rc) return rc;
+    hipLaunchKernelGGL(deal_long_rows_kernel, dim3(rows_grid), dim3(256), 0, stream, order, flags, rank,
+                       num_nodes, order_tmp);
+    hipLaunchKernelGGL(copy_i32_kernel, dim3(ngrid), dim3(256), 0, stream, order_tmp, order,
+                       (int64_t)num_nodes);
     return check_hip(hipGetLastError(), "locality_order");
 }
 

@@ -85,6 +85,31 @@ def test_locality_order_is_a_permutation_that_groups_neighbours(rounds):
     assert sorted(order2.tolist()) == list(range(n))
 
 
+@pytest.mark.parametrize("num_nodes", [5, 64, 1003])
+def test_long_rows_are_dealt_to_the_fronts_of_the_eighths_of_the_row_list(num_nodes):
+    """Rows with more than twice the mean number of edges start first on every XCD: eighth p of
+    the list holds the p-th eighth of the long rows, then the p-th eighth of the others."""
+    rng = np.random.default_rng(num_nodes)
+    degree = np.where(rng.random(num_nodes) < 0.1, 40, 4)
+    degree[0] = 40
+    receiver = np.repeat(np.arange(num_nodes), degree).astype(np.int32)
+    sender = rng.integers(0, num_nodes, receiver.size).astype(np.int32)
+    ptr = csr_row_ptr(dev(receiver), num_nodes)
+    order = locality_order(dev(sender), ptr, num_nodes, 0).cpu().numpy()   # no sweeps: index order, then the deal
+    assert sorted(order.tolist()) == list(range(num_nodes))
+    long_row = degree * num_nodes > 2 * degree.sum()
+    longs, shorts = np.flatnonzero(long_row), np.flatnonzero(~long_row)
+    want = []
+    for p in range(8):
+        want += longs[p * len(longs) // 8:(p + 1) * len(longs) // 8].tolist()
+        want += shorts[p * len(shorts) // 8:(p + 1) * len(shorts) // 8].tolist()
+    assert order.tolist() == want
+    # a graph without long rows keeps its list
+    even = np.repeat(np.arange(num_nodes), 3).astype(np.int32)
+    same = locality_order(dev(sender[:even.size] % num_nodes), csr_row_ptr(dev(even), num_nodes), num_nodes, 0)
+    assert same.cpu().tolist() == list(range(num_nodes))
+
+
 @pytest.mark.parametrize("num_nodes", [1, 7, 1000])
 def test_wrap_global_index_matches_the_tensor_arithmetic(num_nodes):
     """Global ids of a sharded graph modulo the shard size, sentinel kept
