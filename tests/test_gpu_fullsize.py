@@ -99,6 +99,32 @@ def test_config3_full_size_properties():
     assert np.abs(got - ref[:64]).max() <= 2e-5 * np.abs(ref[:64]).max()
 
 
+def _dot(a, b, chunk=1 << 16):
+    """<a, b> in float64 without a float64 copy of the operands."""
+    return sum(float((a[i:i + chunk].double() * b[i:i + chunk].double()).sum()) for i in range(0, a.shape[0], chunk))
+
+
+def test_radial_weights_beyond_two_to_32_elements():
+    """51 200 atoms, ~1.5 M edges, 128 channels: `s` and `ds` hold more than 2^32 elements each
+    (18 GB), so the rows of the last receivers sit behind offsets no 32-bit index reaches.  Their
+    edges, passed again as a problem of their own (small offsets), must give the same bits."""
+    import dataclasses
+    w = W.config3(1.6, device="cuda")
+    assert w.s.numel() > 2 ** 32
+    out, (dx, dy, ds) = _run(w)
+    total = _dot(out, w.dm)
+    for a, g, name in ((w.x, dx, "x"), (w.y, dy, "y"), (w.s, ds, "s")):
+        assert abs(_dot(a, g) - total) <= 2e-5 * abs(total), name
+    first = w.num_nodes - 200
+    e0 = int((w.receiver < first).sum())
+    assert e0 * w.s.shape[1] * w.s.shape[2] > 2 ** 32
+    tail = dataclasses.replace(w, s=w.s[e0:], y=w.y[e0:], sender=w.sender[e0:], receiver=w.receiver[e0:])
+    out_t, (_, dy_t, ds_t) = _run(tail)
+    assert torch.equal(out_t[first:], out[first:]) and not bool(out_t[:first].any())
+    assert torch.equal(ds_t, ds[e0:])
+    torch.testing.assert_close(dy_t, dy[e0:], rtol=1e-5, atol=1e-6)   # (summed over waves by float atomics)
+
+
 @pytest.mark.parametrize("mode,layout", [("MAP", "TRAILING_CHANNELS"), ("OUTER", "TRAILING_CHANNELS"),
                                          ("INNER", "TRAILING_CHANNELS"), ("MAP", "LEADING_CHANNELS")])
 def test_tensor_product_benchmark_size_properties(mode, layout):
