@@ -51,7 +51,9 @@ def parse_args():
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=20)
     ap.add_argument("--warmup", type=int, default=5)
-    ap.add_argument("--config", default="cfg3", choices=["cfg2", "cfg3", "cfg4"])
+    ap.add_argument("--config", default="cfg3", choices=["cfg2", "cfg3", "cfg4", "cfg5"],
+                    help="cfg3: the headline workload; cfg2 / cfg4: the other single-convolution "
+                         "configurations; cfg5: a secondary figure, energy and forces of the two-layer model")
     ap.add_argument("--layout", default="trailing", choices=["trailing", "leading"],
                     help="memory layout of the node and edge arrays (channels last or first)")
     ap.add_argument("--channels", type=int, default=None,
@@ -264,6 +266,68 @@ def calibrate_copy(torch, device) -> None:
     del src, dst
 
 
+def bench_energy(args, torch, device) -> int:
+    """Secondary figure: energy and forces of the two-layer model (positions -> harmonics and
+    radial weights -> two convolutions with channel mixing -> scalar energy; forces by autograd
+    through the kernels' VJPs).  The roofline entry is the backward kernel of one of its layers."""
+    from e3j_amd import workloads as W
+    wl = W.config5(args.scale)
+    d = wl.to(device, torch.float32)
+    model = wl.model
+
+    def step():
+        return model.energy_and_forces(d.positions, d.node_features, d.sender, d.receiver, d.shift)
+
+    for _ in range(args.warmup):
+        step()
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for _ in range(args.steps):
+        step()
+    torch.cuda.synchronize()
+    ms_per_step = (time.perf_counter() - t0) * 1e3 / args.steps
+
+    # one layer's convolution on the model's own operands, through the C ABI
+    with torch.no_grad():
+        y, basis = model.edge_inputs(d.positions, d.sender, d.receiver, d.shift)
+        w1, w2 = (torch.as_tensor(a, dtype=torch.float32, device=device) for a in model.mlp[0])
+        s = (torch.nn.functional.silu(basis @ w1) @ w2).reshape(-1, model.num_paths, model.channels).contiguous()
+    layer = model.layers[0]
+    dm = torch.randn((d.node_features.shape[0], layer.target.dim, model.channels), device=device,
+                     generator=torch.Generator(device=device).manual_seed(0))
+    w = W.Workload("cfg5 layer", layer, d.node_features.contiguous(), y.contiguous(), s, dm, d.sender, d.receiver,
+                   wl.positions.numpy(), 0.0)
+    abi = AbiCalls(w)
+    fwd_ms = time_events(torch, abi.forward, args.steps, 2)
+    bwd_ms = time_events(torch, abi.backward, args.steps, 2)
+    bytes_ = w.algorithmic_bytes()
+
+    def gbs(nbytes, ms):
+        return nbytes / (ms * 1e-3) / 1e9
+
+    result = {
+        "metric": "edges/sec energy + forces, two fused Convolution layers, fp32",
+        "value": wl.num_edges / (ms_per_step * 1e-3), "unit": "edges/s", "n_gpus": 1, "steps": args.steps,
+        "warmup": args.warmup, "ms_per_step": ms_per_step, "higher_is_better": True, "scaling": "weak",
+        "vs_baseline": None, "dtype": "f32", "data": "synthetic",
+        "config": {"workload": f"cfg5: {d.positions.shape[0]} atoms in a periodic box, {wl.num_edges} edges, two "
+                               f"convolutions ({model.channels} channels, 0e+1o+2e+3o, l <= 3) with channel mixing, "
+                               "radial weights from an MLP over 8 Bessel functions, scalar energy, forces by "
+                               "autograd with respect to the positions",
+                   "scale": args.scale, "signature": abi.signature},
+        "roofline": {"bound": "hbm", "kernel": "convolution backward of one layer (unrolled_bwd_kernel + dx zero fill)",
+                     "achieved": gbs(bytes_["bwd"], bwd_ms), "peak": HBM_PEAK_GBS, "unit": "GB/s",
+                     "frac": gbs(bytes_["bwd"], bwd_ms) / HBM_PEAK_GBS, "traffic": None,
+                     "algorithmic_bytes": bytes_["bwd"], "ms": bwd_ms,
+                     "forward": {"achieved": gbs(bytes_["fwd"], fwd_ms), "frac": gbs(bytes_["fwd"], fwd_ms) / HBM_PEAK_GBS,
+                                 "traffic": None, "algorithmic_bytes": bytes_["fwd"], "ms": fwd_ms},
+                     "convolution_kernels_ms_per_step": 2 * (fwd_ms + bwd_ms)},
+        "cpu_baseline": None,
+    }
+    print(json.dumps(result))
+    return 0
+
+
 def bench_tensor_product(args, torch, device) -> int:
     """Secondary figure: the row-wise tensor product (forward + VJP) on the benchmark's table."""
     import numpy as np
@@ -372,6 +436,8 @@ def main():
     torch.cuda.set_device(device)
     if args.op == "tensor_product":
         return bench_tensor_product(args, torch, device)
+    if args.config == "cfg5":
+        return bench_energy(args, torch, device)
 
     w = build_workload(args.config, args.scale, device, args.spatial_sort, args.channels)
     w = w.with_layout("LEADING_CHANNELS" if args.layout == "leading" else "TRAILING_CHANNELS")
