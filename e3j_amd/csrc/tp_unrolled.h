@@ -596,6 +596,78 @@ __global__ __launch_bounds__(kWave * WPB) void tp_unrolled_bwd_uniform_leading_k
     }
 }
 
+// The same with the cotangent tile resident in LDS (64 columns x Z floats per wave) and read
+// where the arithmetic needs it, instead of Z more registers per lane: three times the resident
+// waves.  Two waves per block (25 KB each at Z = 99), so rows of at most 128 channels.
+template <int X, int Y, int Z, int WPB>
+struct TpCotangentTile {
+    using G = TpLeadingGeometry<X, Y, Z>;
+    static constexpr int TILE = round4(kWave * G::PZ);
+    static constexpr int REGION = TILE > G::REGION ? TILE : G::REGION;
+    static constexpr bool FITS = WPB * REGION * sizeof(float) <= 60 * 1024;  // static LDS of a block
+};
+
+template <int Z>
+struct StripLoad {
+    const float *column;
+    float scale;
+    template <int I>
+    __device__ __forceinline__ float get() const { return column[I] * scale; }
+};
+
+template <typename Sig, int WPB>
+__global__ __launch_bounds__(kWave * WPB) void tp_unrolled_bwd_uniform_leading_lds_kernel(
+    const float *__restrict__ x, const float *__restrict__ y, const float *__restrict__ dz,
+    float *__restrict__ dx, float *__restrict__ dy, int64_t rows, int K, float scale) {
+    constexpr int X = Sig::X, Y = Sig::Y, Z = Sig::Z;
+    using G = TpLeadingGeometry<X, Y, Z>;
+    using Red = WaveReduceBlocks<Y>;
+    using T = TpCotangentTile<X, Y, Z, WPB>;
+    constexpr int REGION = T::REGION;
+    if constexpr (!T::FITS) return;  // (never launched: the launcher takes the register form)
+    __shared__ __attribute__((aligned(16))) float strips[T::FITS ? WPB * REGION : 4];
+    __shared__ float partial[WPB][Red::P];
+    float *strip = strips + threadIdx.y * REGION;
+    const int lane = threadIdx.x, wave = threadIdx.y;
+    const int sl = K / kWave, rpb = WPB / sl;
+    const int slice = wave % sl;
+    const int64_t r = tp_uniform((int64_t)blockIdx.x * rpb + wave / sl);
+    const bool valid = r < rows;  // uniform per wave; every wave reaches the barrier
+    if (valid) {
+        const int64_t col0 = r * K + (int64_t)slice * kWave;
+        float xv[X], yv[Y], dxv[X], dyv[Red::P];
+        tp_leading_operands<Sig, true>(x, y, col0, K, 1.f, strip, lane, xv, yv);
+        strip_fence();  // the operand columns are in registers: the strip takes the cotangent tile
+#pragma unroll
+        for (int q = 0; q < kWave / G::GC; q++) {
+            LinearBlock<G::GC * Z> dl;
+            dl.template load<true>(dz + (col0 + q * G::GC) * Z, lane);
+            dl.template to_strip<Z, G::PZ>(strip + q * G::GC * G::PZ, lane);
+        }
+        strip_fence();
+#pragma unroll
+        for (int j = 0; j < X; j++) dxv[j] = 0.f;
+#pragma unroll
+        for (int k = 0; k < Red::P; k++) dyv[k] = 0.f;
+        Sig::bwd(xv, yv, StripLoad<Z>{strip + lane * G::PZ, scale}, dxv, dyv);
+        strip_fence();
+#pragma unroll
+        for (int j = 0; j < X; j++) strip[lane * G::PX + j] = dxv[j];
+        strip_fence();
+        LinearBlock<kWave * X> xl;
+        xl.template from_strip<X, G::PX>(strip, lane);
+        xl.store(dx + col0 * X, lane);
+        float *mine = partial[wave];
+        Red::run(dyv, lane, [&](int k, float total) { mine[k] = total; });
+    }
+    __syncthreads();
+    if (valid && slice == 0 && lane < Y) {
+        float total = partial[wave][lane];
+        for (int s2 = 1; s2 < sl; s2++) total += partial[wave + s2][lane];
+        dy[r * Y + lane] = total;
+    }
+}
+
 // INNER forward, K = 64 * SL with SL in {1, 2, 4}: as the uniform-y backward, the tiles of a
 // row sit in one block and their channel sums meet in LDS.
 template <typename Sig, int WPB>
@@ -659,7 +731,12 @@ int launch_tp_unrolled_bwd_leading(int64_t rows, int channels, float scale, cons
         return set_error(E3J_AMD_INVALID_ARGUMENT, "tensor_product_bwd: channel count outside the "
                                                    "leading-layout kernels");
     unsigned blocks;
-    if (kKind == 1) {
+    constexpr int PAIR = 2;  // waves per block of the kernel that keeps the cotangent tile in LDS
+    if (kKind == 1 && channels <= PAIR * kWave && TpCotangentTile<Sig::X, Sig::Y, Sig::Z, PAIR>::FITS) {
+        if (int rc = tp_grid(rows, PAIR / (channels / kWave), &blocks)) return rc;
+        hipLaunchKernelGGL((tp_unrolled_bwd_uniform_leading_lds_kernel<Sig, PAIR>), dim3(blocks),
+                           dim3(kWave, PAIR), 0, stream, x, y, dz, dx, dy, rows, channels, scale);
+    } else if (kKind == 1) {
         if (int rc = tp_grid(rows, WPB / (channels / kWave), &blocks)) return rc;
         hipLaunchKernelGGL((tp_unrolled_bwd_uniform_leading_kernel<Sig, WPB>), dim3(blocks), dim3(kWave, WPB), 0,
                            stream, x, y, dz, dx, dy, rows, channels, scale);
