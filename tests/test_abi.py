@@ -63,6 +63,33 @@ def test_tensor_product_params_struct_matches_header():
     assert tuple(map(int, modes.groups())) == (_lib.MODE_OUTER, _lib.MODE_INNER, _lib.MODE_MAP)
 
 
+def test_header_is_plain_c_and_ctypes_mirrors_its_layout(tmp_path):
+    """The header compiles as strict C99 (what a cgo / JNI / FFI binding would include), and the
+    compiler's sizes and field offsets of both parameter structs are those of the ctypes mirrors."""
+    import shutil
+    import subprocess
+    if shutil.which("gcc") is None:
+        pytest.skip("no C compiler")
+    fields = {"e3j_amd_conv_params": _lib.ConvParams, "e3j_amd_tp_params": _lib.TpParams}
+    lines = ['#include <stdio.h>', '#include <stddef.h>', f'#include "{os.path.join(ROOT, "include", "e3j_amd.h")}"',
+             'int main(void) {']
+    for struct, mirror in fields.items():
+        lines.append(f'    printf("{struct} %zu\\n", sizeof({struct}));')
+        for name, _ in mirror._fields_:
+            lines.append(f'    printf("{struct}.{name} %zu\\n", offsetof({struct}, {name}));')
+    lines += ['    return 0;', '}']
+    src = tmp_path / "layout.c"
+    src.write_text("\n".join(lines))
+    exe = tmp_path / "layout"
+    subprocess.run(["gcc", "-std=c99", "-pedantic", "-Wall", "-Wextra", "-Werror", str(src), "-o", str(exe)], check=True)
+    got = dict(line.split() for line in subprocess.run([str(exe)], check=True, capture_output=True,
+                                                       text=True).stdout.splitlines())
+    for struct, mirror in fields.items():
+        assert int(got[struct]) == C.sizeof(mirror)
+        for name, _ in mirror._fields_:
+            assert int(got[f"{struct}.{name}"]) == getattr(mirror, name).offset, (struct, name)
+
+
 def test_tensor_product_argument_errors_need_no_launch():
     lib = _lib.load()
     assert lib.e3j_amd_tensor_product_fwd(None, None, None, None, None, None) == _lib.INVALID_ARGUMENT
