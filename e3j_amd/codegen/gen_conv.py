@@ -29,7 +29,6 @@ from collections import OrderedDict
 
 import numpy as np
 
-from ..options import Layout
 from ..scalar_mixing import ScalarMixing
 from ..tensor_product import TensorProduct
 

@@ -11,7 +11,6 @@ helpers is plain tensor arithmetic.
 
 from __future__ import annotations
 
-import ctypes
 
 import numpy as np
 import torch

@@ -25,7 +25,7 @@ import torch
 
 from . import _lib
 from .coef import Coef4D
-from .graph import (DUMMY_INDEX, INDEX_DTYPE, csr_row_ptr, fold_endpoints, locality_order,
+from .graph import (csr_row_ptr, fold_endpoints, locality_order,
                     sort_edges, wrap_global_index)
 from .options import GraphOrdering, Layout, config
 
