@@ -277,9 +277,15 @@ class EnergyModel:
         self.mix = [[rng.standard_normal((mul, channels, channels)) / math.sqrt(mul * channels)
                      for mul, _ in self.blocks] for _ in self.layers]
         self.readout = np.random.default_rng(seed_read).standard_normal(channels) / math.sqrt(channels)
+        self._weights: dict = {}
 
     def _t(self, array, like: torch.Tensor) -> torch.Tensor:
-        return torch.as_tensor(array, dtype=like.dtype, device=like.device)
+        """A weight array as a tensor beside `like`; uploaded once per dtype and device."""
+        key = (id(array), like.dtype, like.device)
+        hit = self._weights.get(key)
+        if hit is None:
+            hit = self._weights[key] = torch.as_tensor(array, dtype=like.dtype, device=like.device)
+        return hit
 
     def radial_basis(self, r: torch.Tensor) -> torch.Tensor:
         """Bessel functions `sqrt(2/rc) sin(n pi r / rc) / r` times a smooth cutoff envelope."""
