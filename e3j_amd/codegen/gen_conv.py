@@ -41,6 +41,8 @@ BUILTIN_TABLES = [
     ("l2_l3_to_l2", "0e+1o+2e", "0e+1o+2e+3o", "0e+1o+2e", (32, 64, 128)),
     ("l2_l3_to_l3", "0e+1o+2e", "0e+1o+2e+3o", "0e+1o+2e+3o", (64, 128)),
     ("l3_l3_to_l3", "0e+1o+2e+3o", "0e+1o+2e+3o", "0e+1o+2e+3o", (32, 64, 128, 256)),
+    # scalar node features times the harmonics: the first layer of a model whose input is invariant
+    ("l0_l3_to_l3", "0e", "0e+1o+2e+3o", "0e+1o+2e+3o", (64, 128, 256)),
 ]
 #: (name, x irreps, y irreps, output filter, channels) of every compiled signature
 BUILTIN_SIGNATURES = [(f"{name}_k{k}", xi, yi, oi, k) for name, xi, yi, oi, ks in BUILTIN_TABLES for k in ks]

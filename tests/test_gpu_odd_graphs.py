@@ -16,7 +16,8 @@ pytestmark = pytest.mark.gpu
 TABLES = [(("0e+1o", "0e+1o+2e"), "0e+1o+2e", (32, 64, 128)),
           (("0e+1o+2e", "0e+1o+2e+3o"), "0e+1o+2e", (32, 64, 128)),
           (("0e+1o+2e", "0e+1o+2e+3o"), "0e+1o+2e+3o", (64, 128)),
-          (("0e+1o+2e+3o", "0e+1o+2e+3o"), "0e+1o+2e+3o", (32, 64, 128, 256))]
+          (("0e+1o+2e+3o", "0e+1o+2e+3o"), "0e+1o+2e+3o", (32, 64, 128, 256)),
+          (("0e", "0e+1o+2e+3o"), "0e+1o+2e+3o", (64, 128, 256))]
 
 
 def _degrees(rng, kind, n):
@@ -33,10 +34,10 @@ def _degrees(rng, kind, n):
     return rng.integers(0, 2, n)
 
 
-@pytest.mark.parametrize("case", range(40))
+@pytest.mark.parametrize("case", range(50))
 def test_odd_graph(case):
     rng = np.random.default_rng(7000 + case)
-    src, tgt, channel_counts = TABLES[case % 4]
+    src, tgt, channel_counts = TABLES[case % len(TABLES)]
     K = int(rng.choice(channel_counts))
     ordering = ("RECEIVER", "NONE")[case % 2]
     layout = ("TRAILING_CHANNELS", "LEADING_CHANNELS")[(case // 2) % 2]

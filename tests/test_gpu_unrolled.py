@@ -21,6 +21,9 @@ CASES = {
     "cfg2_out3": lambda: W.config2(0.04, out_irreps="0e+1o+2e+3o"),
     "cfg3_k64": lambda: W.config3(0.006, channels=64),
     "cfg3": lambda: W.config3(0.006),
+    # scalar node features (one x coordinate, four paths)
+    "scalars_k64": lambda: W.make_workload("scalars", 200, "0e", 3, "0e+1o+2e+3o", 64, (51, 52, 53, 54)),
+    "scalars_k256": lambda: W.make_workload("scalars", 120, "0e", 3, "0e+1o+2e+3o", 256, (55, 56, 57, 58)),
 }
 
 
