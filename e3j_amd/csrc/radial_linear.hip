@@ -1,0 +1,268 @@
+// Last layer of the radial network that produces the per-edge, per-path weights of the
+// convolution: s (E, N) = h (E, H) W (H, N) with N = paths * channels, float32, and the two
+// products of its backward pass.  The one dense contraction next to the convolution: it runs
+// on the matrix cores (v_mfma_f32_32x32x2_f32, plain float32 arithmetic).  H is small (8..128), so
+// every pass is bound by the E * N stream it writes (forward) or reads (backward); the tiling
+// keeps that stream at whole 128-byte lines and everything else (h, W) in registers or LDS.
+//
+// Register layout of one 32x32x2 product D += A B on a 64-lane wave (g = lane / 32, c = lane % 32):
+// a lane supplies A[c][g] and B[g][c] and holds D[8 * (v / 4) + 4 * g + v % 4][c] in element v of
+// its sixteen accumulators.  Which two inner indices a product takes is free as long as A and
+// B agree: product j of a lane half takes the inner index g * (inner / 2) + j, so the operands of a
+// lane are contiguous in memory.
+
+#include "common.h"
+
+namespace e3j_amd {
+namespace {
+
+typedef float f32x4 __attribute__((ext_vector_type(4)));
+typedef float f32x16 __attribute__((ext_vector_type(16)));
+
+constexpr int kTile = 32;        // rows and columns of a matrix-core tile
+constexpr int kWaves = 4;        // waves per block
+
+// s = h W.  A block takes kWaves * R * 32 consecutive edges, keeps their rows of h in registers
+// as A operands and walks the columns of W in tiles of 32 that all its waves share through LDS
+// (double buffered: the next tile is fetched while the current one is multiplied).
+template <int H, int R>
+__global__ __launch_bounds__(kWave * kWaves) void radial_linear_fwd_kernel(
+    const float *__restrict__ h, const float *__restrict__ w, float *__restrict__ s, int64_t num_edges, int n) {
+    constexpr int HH = H / 2;                        // inner indices per lane half
+    constexpr int PIECES = H * kTile / 4;            // 16-byte pieces of a W tile
+    constexpr int PER_THREAD = (PIECES + kWave * kWaves - 1) / (kWave * kWaves);
+    static_assert(H % 8 == 0 && H <= 128, "inner size: a multiple of 8 up to 128");
+    __shared__ __attribute__((aligned(16))) float tile[2][H * kTile];
+    const int tid = threadIdx.x, lane = tid % kWave, wave = tid / kWave;
+    const int g = lane / kTile, c = lane % kTile;
+    const int64_t e0 = ((int64_t)blockIdx.x * kWaves + wave) * (kTile * R);
+
+    float a[R][HH];
+#pragma unroll
+    for (int r = 0; r < R; r++) {
+        int64_t row = e0 + r * kTile + c;
+        if (row >= num_edges) row = num_edges - 1;  // rows past the end are computed and not stored
+        const f32x4 *p = reinterpret_cast<const f32x4 *>(h + row * H + g * HH);
+#pragma unroll
+        for (int q = 0; q < HH / 4; q++) {
+            const f32x4 v = __builtin_nontemporal_load(p + q);
+            a[r][4 * q] = v.x; a[r][4 * q + 1] = v.y; a[r][4 * q + 2] = v.z; a[r][4 * q + 3] = v.w;
+        }
+    }
+
+    f32x4 staged[PER_THREAD];
+    auto fetch = [&](int t) {  // columns [32 t, 32 t + 32) of W into registers
+#pragma unroll
+        for (int i = 0; i < PER_THREAD; i++) {
+            const int piece = i * kWave * kWaves + tid;
+            if (PIECES % (kWave * kWaves) == 0 || piece < PIECES)
+                staged[i] = *reinterpret_cast<const f32x4 *>(w + (int64_t)(piece / 8) * n + t * kTile + (piece % 8) * 4);
+        }
+    };
+    auto commit = [&](int buf) {
+#pragma unroll
+        for (int i = 0; i < PER_THREAD; i++) {
+            const int piece = i * kWave * kWaves + tid;
+            if (PIECES % (kWave * kWaves) == 0 || piece < PIECES)
+                *reinterpret_cast<f32x4 *>(&tile[buf][piece * 4]) = staged[i];
+        }
+    };
+    const int tiles = n / kTile;
+    fetch(0);
+    commit(0);
+    __syncthreads();
+    for (int t = 0; t < tiles; t++) {
+        if (t + 1 < tiles) fetch(t + 1);
+        float b[HH];
+#pragma unroll
+        for (int j = 0; j < HH; j++) b[j] = tile[t & 1][(g * HH + j) * kTile + c];
+        f32x16 d[R];
+#pragma unroll
+        for (int r = 0; r < R; r++) d[r] = f32x16{0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+        for (int j = 0; j < HH; j++) {  // the R row tiles side by side: independent accumulator chains
+#pragma unroll
+            for (int r = 0; r < R; r++) d[r] = __builtin_amdgcn_mfma_f32_32x32x2f32(a[r][j], b[j], d[r], 0, 0, 0);
+        }
+#pragma unroll
+        for (int r = 0; r < R; r++) {
+            float *out = s + (e0 + r * kTile + 4 * g) * n + t * kTile + c;
+#pragma unroll
+            for (int v = 0; v < 16; v++) {
+                const int row = 8 * (v / 4) + v % 4;
+                if (e0 + r * kTile + 4 * g + row < num_edges) __builtin_nontemporal_store(d[r][v], out + (int64_t)row * n);
+            }
+        }
+        if (t + 1 < tiles) commit((t + 1) & 1);
+        __syncthreads();
+    }
+}
+
+// Inner sizes of 64 and more: at the float32 rate of the matrix cores (64 flop per cycle and
+// SIMD) the products themselves would take longer than the stream, so they run at the bfloat16
+// rate (16 times that) on operands split three ways: x = x1 + x2 + x3 with x1 the upper 8
+// mantissa bits, x2 the next 8 and x3 the last 8 (each a bfloat16, the sum exact), and
+// x y = x1 y1 + (x1 y2 + x2 y1) + (x1 y3 + x2 y2 + x3 y1) + O(2^-24 x y): six products whose
+// partial products are exact and whose sum is kept in float32 accumulators, i.e. the accuracy
+// of a float32 product at 6/16 of its cost.
+typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
+typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
+
+struct Split3 {
+    bf16x8 term[3];
+};
+
+// eight floats into their three bfloat16 parts (truncation keeps every part exact)
+__device__ __forceinline__ Split3 split3(const float (&x)[8]) {
+    Split3 out;
+    float rest[8];
+#pragma unroll
+    for (int m = 0; m < 8; m++) rest[m] = x[m];
+#pragma unroll
+    for (int t = 0; t < 3; t++) {
+        u32x4 packed;
+#pragma unroll
+        for (int m = 0; m < 8; m += 2) {
+            const uint32_t lo = __float_as_uint(rest[m]) & 0xffff0000u, hi = __float_as_uint(rest[m + 1]) & 0xffff0000u;
+            packed[m / 2] = (lo >> 16) | hi;
+            rest[m] -= __uint_as_float(lo);
+            rest[m + 1] -= __uint_as_float(hi);
+        }
+        out.term[t] = __builtin_bit_cast(bf16x8, packed);
+    }
+    return out;
+}
+
+// One 32x32x16 product takes sixteen inner indices; a lane (g, c) supplies eight of them for
+// row (A) or column (B) c: block q of the inner dimension gives it the indices 16 q + 8 g + m.
+template <int H, int R>
+__global__ __launch_bounds__(kWave * kWaves) void radial_linear_fwd_split_kernel(
+    const float *__restrict__ h, const float *__restrict__ w, float *__restrict__ s, int64_t num_edges, int n) {
+    constexpr int Q = H / 16;                         // inner blocks
+    constexpr int SLOTS = 2 * Q * kTile;              // (q, g, c) operand slots of a W tile: 8 values each
+    constexpr int PER_THREAD = (SLOTS + kWave * kWaves - 1) / (kWave * kWaves);
+    static_assert(H % 16 == 0, "whole inner blocks");
+    __shared__ __attribute__((aligned(16))) bf16x8 tile[2][3][SLOTS];
+    const int tid = threadIdx.x, lane = tid % kWave, wave = tid / kWave;
+    const int g = lane / kTile, c = lane % kTile;
+    const int64_t e0 = ((int64_t)blockIdx.x * kWaves + wave) * (kTile * R);
+
+    Split3 a[R][Q];
+#pragma unroll
+    for (int r = 0; r < R; r++) {
+        int64_t row = e0 + r * kTile + c;
+        if (row >= num_edges) row = num_edges - 1;  // rows past the end are computed and not stored
+#pragma unroll
+        for (int q = 0; q < Q; q++) {
+            const f32x4 *p = reinterpret_cast<const f32x4 *>(h + row * H + q * 16 + g * 8);
+            const f32x4 v0 = __builtin_nontemporal_load(p), v1 = __builtin_nontemporal_load(p + 1);
+            const float x[8] = {v0.x, v0.y, v0.z, v0.w, v1.x, v1.y, v1.z, v1.w};
+            a[r][q] = split3(x);
+        }
+    }
+
+    // a thread stages whole operand slots: eight consecutive inner indices of one column
+    float staged[PER_THREAD][8];
+    auto fetch = [&](int t) {
+#pragma unroll
+        for (int i = 0; i < PER_THREAD; i++) {
+            const int slot = i * kWave * kWaves + tid;
+            if (SLOTS % (kWave * kWaves) == 0 || slot < SLOTS) {
+                const float *col = w + (int64_t)((slot / kTile) * 8) * n + t * kTile + slot % kTile;
+#pragma unroll
+                for (int m = 0; m < 8; m++) staged[i][m] = col[(int64_t)m * n];
+            }
+        }
+    };
+    auto commit = [&](int buf) {
+#pragma unroll
+        for (int i = 0; i < PER_THREAD; i++) {
+            const int slot = i * kWave * kWaves + tid;
+            if (SLOTS % (kWave * kWaves) == 0 || slot < SLOTS) {
+                const Split3 parts = split3(staged[i]);
+#pragma unroll
+                for (int t = 0; t < 3; t++) tile[buf][t][slot] = parts.term[t];
+            }
+        }
+    };
+    const int tiles = n / kTile;
+    fetch(0);
+    commit(0);
+    __syncthreads();
+    for (int t = 0; t < tiles; t++) {
+        if (t + 1 < tiles) fetch(t + 1);
+        f32x16 d[R];
+#pragma unroll
+        for (int r = 0; r < R; r++) d[r] = f32x16{0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+        for (int q = 0; q < Q; q++) {
+            bf16x8 b[3];
+#pragma unroll
+            for (int tb = 0; tb < 3; tb++) b[tb] = tile[t & 1][tb][(q * 2 + g) * kTile + c];
+            // smallest partial products first
+            constexpr int kPairs[6][2] = {{0, 2}, {1, 1}, {2, 0}, {0, 1}, {1, 0}, {0, 0}};
+#pragma unroll
+            for (int u = 0; u < 6; u++) {
+#pragma unroll
+                for (int r = 0; r < R; r++)
+                    d[r] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a[r][q].term[kPairs[u][0]], b[kPairs[u][1]], d[r], 0, 0, 0);
+            }
+        }
+#pragma unroll
+        for (int r = 0; r < R; r++) {
+            float *out = s + (e0 + r * kTile + 4 * g) * n + t * kTile + c;
+#pragma unroll
+            for (int v = 0; v < 16; v++) {
+                const int row = 8 * (v / 4) + v % 4;
+                if (e0 + r * kTile + 4 * g + row < num_edges) __builtin_nontemporal_store(d[r][v], out + (int64_t)row * n);
+            }
+        }
+        if (t + 1 < tiles) commit((t + 1) & 1);
+        __syncthreads();
+    }
+}
+
+template <int H>
+int launch_fwd(const float *h, const float *w, float *s, int64_t num_edges, int n, hipStream_t stream) {
+    constexpr int R = H >= 128 ? 1 : 2;  // row tiles per wave (their A operands stay in registers)
+    const int64_t per_block = (int64_t)kWaves * R * kTile;
+    const int64_t blocks = (num_edges + per_block - 1) / per_block;
+    if (blocks > 0x7fffffffLL) return set_error(E3J_AMD_INVALID_ARGUMENT, "radial_linear: too many edges");
+    if constexpr (H >= 64)  // float32 matrix-core rate would bound these; the split form is bound by the stream
+        hipLaunchKernelGGL((radial_linear_fwd_split_kernel<H, R>), dim3((unsigned)blocks), dim3(kWave * kWaves), 0,
+                           stream, h, w, s, num_edges, n);
+    else
+        hipLaunchKernelGGL((radial_linear_fwd_kernel<H, R>), dim3((unsigned)blocks), dim3(kWave * kWaves), 0, stream,
+                           h, w, s, num_edges, n);
+    return check_hip(hipGetLastError(), "radial_linear launch");
+}
+
+int check_shapes(const char *what, int64_t num_edges, int32_t inner, int32_t n) {
+    if (num_edges < 0 || inner <= 0 || n <= 0)
+        return set_error(E3J_AMD_INVALID_ARGUMENT, std::string(what) + ": bad sizes");
+    if (n % kTile != 0)
+        return set_error(E3J_AMD_UNIMPLEMENTED, std::string(what) + ": paths * channels must be a multiple of 32");
+    if (inner != 8 && inner != 16 && inner != 32 && inner != 64 && inner != 128)
+        return set_error(E3J_AMD_UNIMPLEMENTED, std::string(what) + ": hidden size must be 8, 16, 32, 64 or 128");
+    return E3J_AMD_OK;
+}
+
+}  // namespace
+
+extern "C" int e3j_amd_radial_linear_fwd(const float *h, const float *w, float *s, int64_t num_edges,
+                                         int32_t inner, int32_t n, void *stream_) {
+    if (int rc = check_shapes("radial_linear", num_edges, inner, n)) return rc;
+    if (num_edges == 0) return E3J_AMD_OK;
+    if (h == nullptr || w == nullptr || s == nullptr)
+        return set_error(E3J_AMD_INVALID_ARGUMENT, "radial_linear: null operand");
+    hipStream_t stream = static_cast<hipStream_t>(stream_);
+    switch (inner) {
+        case 8: return launch_fwd<8>(h, w, s, num_edges, n, stream);
+        case 16: return launch_fwd<16>(h, w, s, num_edges, n, stream);
+        case 32: return launch_fwd<32>(h, w, s, num_edges, n, stream);
+        case 64: return launch_fwd<64>(h, w, s, num_edges, n, stream);
+        default: return launch_fwd<128>(h, w, s, num_edges, n, stream);
+    }
+}
+
+}  // namespace e3j_amd

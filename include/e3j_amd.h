@@ -206,6 +206,15 @@ int e3j_amd_harmonics_bwd(const void *vec, const void *dout, int64_t num, int32_
                           int32_t normalize, int32_t normalization, int32_t val_dtype, void *dvec,
                           void *stream);
 
+/* Last layer of the radial network that produces the convolution's per-edge, per-path weights:
+ * s (num_edges, n) = h (num_edges, inner) w (inner, n), n = paths * channels, float32, row-major,
+ * on the matrix cores.  inner: 8, 16, 32, 64 or 128; n: a multiple of 32.  No counterpart in the
+ * reference, which leaves the radial network to the caller (edge_scalars of
+ * src/e3j/core/convolution.py:342-350 arrive ready-made); it is the dense contraction next to the
+ * convolution, and the operand the convolution reads most. */
+int e3j_amd_radial_linear_fwd(const float *h, const float *w, float *s, int64_t num_edges,
+                              int32_t inner, int32_t n, void *stream);
+
 /* Row-wise sparse tensor product, the edge-wise sibling of the convolution (no gather, no
  * scatter): z[r] = sum_n val_n x[r, j_n] (*) y[r, k_n] -> z[r, i_n].  Operands and sizes of the
  * reference's "tensor_product" / "tensor_product_bwd" targets (lib/e3j_ops/ffi/e3j_ops.h:124-253,
