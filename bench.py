@@ -72,7 +72,8 @@ def parse_args():
                     help="cfg3, 128 channels, trailing layout only: also time kernels that perform the "
                          "memory accesses of the two passes without their arithmetic (reported under "
                          "roofline.access_floor)")
-    ap.add_argument("--op", default="convolution", choices=["convolution", "tensor_product"],
+    ap.add_argument("--inner", type=int, default=64, help="--op radial_linear: hidden size of the radial network")
+    ap.add_argument("--op", default="convolution", choices=["convolution", "tensor_product", "radial_linear"],
                     help="convolution: the headline benchmark; tensor_product: a secondary figure, the "
                          "row-wise product on the same table (0e+1o+2e+3o squared, l <= 3, 128 channels)")
     ap.add_argument("--mode", default="MAP", choices=["MAP", "OUTER", "INNER"],
@@ -328,6 +329,41 @@ def bench_energy(args, torch, device) -> int:
     return 0
 
 
+def bench_radial_linear(args, torch, device) -> int:
+    """Secondary figure: the last layer of the radial network, s = h W on the matrix cores, at the
+    edge count and paths * channels of the headline workload; beside it the library product."""
+    from e3j_amd.radial import radial_linear
+    edges, n, inner = int(959970 * args.scale), 23 * (args.channels or 128), args.inner
+    g = torch.Generator(device=device).manual_seed(0)
+    h = torch.randn(edges, inner, device=device, generator=g)
+    w = torch.randn(inner, n, device=device, generator=g)
+    out = torch.empty(edges, n, device=device)
+    ms = time_events(torch, lambda: radial_linear(h, w), args.steps, args.warmup)
+    lib_ms = time_events(torch, lambda: torch.matmul(h, w, out=out), args.steps, args.warmup)
+    nbytes = 4 * (edges * n + edges * inner + inner * n)
+    flops = 2.0 * edges * inner * n
+    split = inner >= 64   # three-way bfloat16 split: six matrix-core products per float32 product
+    result = {
+        "metric": "edges/sec radial network last layer (s = h W) fp32", "value": edges / (ms * 1e-3),
+        "unit": "edges/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup, "ms_per_step": ms,
+        "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": "f32", "data": "synthetic",
+        "config": {"workload": f"s ({edges}, {n}) = h ({edges}, {inner}) W ({inner}, {n}), float32"
+                               + (", operands split three ways on the bfloat16 matrix cores" if split else
+                                  ", float32 matrix-core products")},
+        "roofline": {"bound": "hbm", "kernel": "radial_linear_fwd" + ("_split" if split else "") + "_kernel",
+                     "achieved": nbytes / (ms * 1e-3) / 1e9, "peak": HBM_PEAK_GBS, "unit": "GB/s",
+                     "frac": nbytes / (ms * 1e-3) / 1e9 / HBM_PEAK_GBS, "traffic": None, "algorithmic_bytes": nbytes,
+                     "ms": ms,
+                     "matrix_cores": {"flop": flops, "products_per_float32_product": 6 if split else 1,
+                                      "achieved_tflops": flops * (6 if split else 1) / (ms * 1e-3) / 1e12,
+                                      "peak_tflops": 2500.0 if split else 157.3},
+                     "library_product_ms": lib_ms},
+        "cpu_baseline": None,
+    }
+    print(json.dumps(result))
+    return 0
+
+
 def bench_tensor_product(args, torch, device) -> int:
     """Secondary figure: the row-wise tensor product (forward + VJP) on the benchmark's table."""
     import numpy as np
@@ -436,6 +472,8 @@ def main():
     torch.cuda.set_device(device)
     if args.op == "tensor_product":
         return bench_tensor_product(args, torch, device)
+    if args.op == "radial_linear":
+        return bench_radial_linear(args, torch, device)
     if args.config == "cfg5":
         return bench_energy(args, torch, device)
 

@@ -2,7 +2,8 @@
 
 Public names follow the reference package for this path: `Convolution`,
 `convolution`, `convolution_bwd`, `TensorProduct`, `tensor_product`, `tensor_product_bwd`,
-`Harmonics`, `GraphCSR`, `Coef4D`, `O3Space`, `config`.
+`Harmonics`, `GraphCSR`, `Coef4D`, `O3Space`, `config`; `radial_linear` (the radial network's last
+layer) has no counterpart there.
 Importing the package does not load the kernel library; the first operator call does,
 and fails if `e3j_amd/lib/libe3j_amd.so` has not been built.
 """
@@ -14,6 +15,7 @@ from .harmonics import Harmonics
 from .ops import (ConvolutionBatchingWarning, ConvolutionParams, CUDAConvolutionParams, TableDrivenKernelWarning,
                   convolution, convolution_batched, convolution_bwd)
 from .options import Config, GraphOrdering, Layout, MixingMode, TensorProductNormalization, config
+from .radial import radial_linear
 from .scalar_mixing import ScalarMixing
 from .spaces import O3Irrep, O3Space
 from .tensor_product import TensorProduct
@@ -27,6 +29,6 @@ __all__ = [
     "TableDrivenKernelWarning",
     "CUDAConvolutionParams", "DUMMY_INDEX", "GraphCSR", "GraphOrdering", "Harmonics", "Layout", "O3Irrep",
     "O3Space", "ScalarMixing", "Space", "TensorProduct", "TensorProductNormalization", "config",
-    "convolution", "convolution_batched", "convolution_bwd", "resolve_val_dtype",
+    "convolution", "convolution_batched", "convolution_bwd", "radial_linear", "resolve_val_dtype",
     "CUDATensorProductParams", "MixingMode", "TensorProductParams", "tensor_product", "tensor_product_batched", "tensor_product_bwd",
 ]

@@ -3,7 +3,8 @@
 The per-edge, per-path weights `s (E, paths * channels)` are the operand the convolution reads
 most; the layer that writes them is a product with a small inner size (the hidden width of the
 radial network), bound by the stream it writes.  `radial_linear` runs it as one HIP kernel
-(`csrc/radial_linear.hip`); its backward uses the library products `ds @ w.T` and `h.T @ ds`.
+(`csrc/radial_linear.hip`); the products of its backward, `ds @ w.T` and `h.T @ ds`, read the
+stream along the contracted index and are left to the library.
 """
 
 from __future__ import annotations

@@ -22,6 +22,7 @@ import torch
 from .convolution import Convolution
 from .harmonics import Harmonics
 from .options import Layout
+from .radial import radial_linear, supported as radial_supported
 
 
 @dataclasses.dataclass
@@ -309,7 +310,10 @@ class EnergyModel:
         x = node_features
         for layer, (w1, w2) in enumerate(self.mlp):
             hidden = torch.nn.functional.silu(basis @ self._t(w1, basis))
-            s = (hidden @ self._t(w2, basis)).reshape(-1, self.num_paths, self.channels)
+            last = self._t(w2, basis)
+            # the weights of every path and channel: the matrix-core kernel where it applies
+            s = radial_linear(hidden, last) if radial_supported(hidden, last) else hidden @ last
+            s = s.reshape(-1, self.num_paths, self.channels)
             out = convolve(layer, x, y, s, sender, receiver)          # (N, Z, K)
             rows, mixed = 0, []
             for (mul, dim), w in zip(self.blocks, self.mix[layer]):
