@@ -1,11 +1,12 @@
 // Last layer of the radial network that produces the per-edge, per-path weights of the
-// convolution: s (E, N) = h (E, H) W (H, N) with N = paths * channels, float32.  The one dense
-// contraction next to the convolution: it runs on the matrix cores.  H is small (8..128), so the
-// pass is bound by the E * N stream it writes; the tiling keeps that stream at whole 128-byte
-// lines and everything else (h, W) in registers or LDS.  (The products of the backward pass,
-// ds W^T and h^T ds, read that stream with the contracted index along the rows, which the
-// operand layout below can only take through a transposition in LDS; they are left to the
-// library, which reads it at 3.3 to 5.8 TB/s.)
+// convolution: s (E, N) = h (E, H) W (H, N) with N = paths * channels, float32, and the weight
+// gradient of its backward pass, dW = h^T ds.  The one dense contraction next to the
+// convolution: it runs on the matrix cores.  H is small (8..128), so each pass is bound by the
+// E * N stream it writes or reads; the tilings keep that stream at whole 128-byte lines and
+// everything else (h, W) in registers or LDS.  (The other product of the backward pass, ds W^T,
+// reads that stream with the contracted index along the rows, which the operand layout below can
+// only take through a transposition in LDS; it is left to the library, which reads it at 3.3 to
+// 5.8 TB/s.)
 //
 // Register layout of one 32x32x2 product D += A B on a 64-lane wave (g = lane / 32, c = lane % 32):
 // a lane supplies A[c][g] and B[g][c] and holds D[8 * (v / 4) + 4 * g + v % 4][c] in element v of
@@ -239,6 +240,272 @@ int launch_fwd(const float *h, const float *w, float *s, int64_t num_edges, int 
     return check_hip(hipGetLastError(), "radial_linear launch");
 }
 
+// dW (H, n) = h^T ds, the contraction running over the edges.  Both operands are read the way the
+// matrix cores want them: a lane (g, c) supplies A[c][k] = h[edge k][row tile * 32 + c] and
+// B[k][c] = ds[edge k][column tile * 32 + c], so consecutive lanes read consecutive addresses.
+// A block takes a slab of kSlab columns (kColTiles column tiles per wave) and one of `groups`
+// ranges of the edges, keeps its part of dW in the accumulators and stores it as one slice of
+// `partial (groups, H, n)`; a second kernel adds the slices in a fixed order.  The rows of h of a
+// chunk of 64 edges (one contiguous block) are shared by the waves through LDS (double buffered).
+// ds is read once; h once per slab (from the L2).
+constexpr int kColTiles = 2;
+constexpr int kSlab = kTile * kColTiles * kWaves;
+
+template <int H>
+__global__ __launch_bounds__(kWave * kWaves) void radial_linear_bwd_weight_kernel(
+    const float *__restrict__ h, const float *__restrict__ ds, float *__restrict__ partial, int64_t num_edges,
+    int n, int groups) {
+    constexpr int RT = (H + kTile - 1) / kTile;  // row tiles of dW
+    constexpr int HP = RT * kTile;               // rows padded to whole tiles (inner sizes 8, 16)
+    constexpr int CHUNK = 64;                    // edges per step: 32 per lane half
+    constexpr int HALF = CHUNK / 2;
+    constexpr int PIECES = CHUNK * H / 4;        // 16-byte pieces of a chunk of h
+    constexpr int PER_THREAD = (PIECES + kWave * kWaves - 1) / (kWave * kWaves);
+    __shared__ __attribute__((aligned(16))) float rows[2][CHUNK * HP];
+    const int tid = threadIdx.x, lane = tid % kWave, wave = tid / kWave;
+    const int g = lane / kTile, c = lane % kTile;
+    const int slabs = (n + kSlab - 1) / kSlab;
+    const int slab = blockIdx.x % slabs, group = blockIdx.x / slabs;
+    const int col0 = slab * kSlab + wave * (kTile * kColTiles);  // first column of this wave
+    const int64_t per_group = ((num_edges + groups - 1) / groups + CHUNK - 1) / CHUNK * CHUNK;
+    const int64_t first = (int64_t)group * per_group;
+    const int64_t last = first + per_group < num_edges ? first + per_group : num_edges;
+    if (HP != H) {  // rows past the inner size multiply zeros
+        for (int i = tid; i < 2 * CHUNK * HP; i += kWave * kWaves) (&rows[0][0])[i] = 0.f;
+        __syncthreads();
+    }
+
+    f32x16 d[kColTiles][RT];
+#pragma unroll
+    for (int t = 0; t < kColTiles; t++)
+#pragma unroll
+        for (int rt = 0; rt < RT; rt++)
+            d[t][rt] = f32x16{0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
+    bool col_ok[kColTiles];                      // (n is a multiple of 32: whole tiles are in or out)
+    const float *dcol[kColTiles];
+#pragma unroll
+    for (int t = 0; t < kColTiles; t++) {
+        col_ok[t] = col0 + t * kTile < n;
+        dcol[t] = ds + (col_ok[t] ? col0 + t * kTile + c : 0);
+    }
+
+    f32x4 staged[PER_THREAD];
+    auto fetch = [&](int64_t e0) {  // rows [e0, e0 + 64) of h: edges past the range read as zeros
+#pragma unroll
+        for (int i = 0; i < PER_THREAD; i++) {
+            const int piece = i * kWave * kWaves + tid;
+            if (PIECES % (kWave * kWaves) == 0 || piece < PIECES) {
+                const int64_t e = e0 + piece * 4 / H;
+                staged[i] = e < last ? *reinterpret_cast<const f32x4 *>(h + e0 * H + (int64_t)piece * 4)
+                                     : f32x4{0.f, 0.f, 0.f, 0.f};
+            }
+        }
+    };
+    auto commit = [&](int buf) {
+#pragma unroll
+        for (int i = 0; i < PER_THREAD; i++) {
+            const int piece = i * kWave * kWaves + tid;
+            if (PIECES % (kWave * kWaves) == 0 || piece < PIECES) {
+                const int at = piece * 4;
+                *reinterpret_cast<f32x4 *>(&rows[buf][(at / H) * HP + at % H]) = staged[i];
+            }
+        }
+    };
+    if (first < last) {
+        fetch(first);
+        commit(0);
+    }
+    __syncthreads();
+    int buf = 0;
+    for (int64_t e0 = first; e0 < last; e0 += CHUNK, buf ^= 1) {
+        const bool more = e0 + CHUNK < last;
+        if (more) fetch(e0 + CHUNK);
+        float b[kColTiles][HALF];
+#pragma unroll
+        for (int j = 0; j < HALF; j++) {
+            const int64_t e = e0 + g * HALF + j;
+            const bool in = e < last;            // edges past the range multiply zeros
+            const int64_t ee = in ? e : last - 1;
+#pragma unroll
+            for (int t = 0; t < kColTiles; t++) b[t][j] = in ? __builtin_nontemporal_load(dcol[t] + ee * n) : 0.f;
+        }
+#pragma unroll
+        for (int j = 0; j < HALF; j++) {
+#pragma unroll
+            for (int rt = 0; rt < RT; rt++) {
+                const float a = rows[buf][(g * HALF + j) * HP + rt * kTile + c];
+#pragma unroll
+                for (int t = 0; t < kColTiles; t++)
+                    d[t][rt] = __builtin_amdgcn_mfma_f32_32x32x2f32(a, b[t][j], d[t][rt], 0, 0, 0);
+            }
+        }
+        if (more) commit(buf ^ 1);
+        __syncthreads();
+    }
+#pragma unroll
+    for (int t = 0; t < kColTiles; t++) {
+        if (!col_ok[t]) continue;
+        float *out = partial + (int64_t)group * H * n + col0 + t * kTile + c;
+#pragma unroll
+        for (int rt = 0; rt < RT; rt++) {
+#pragma unroll
+            for (int v = 0; v < 16; v++) {
+                const int row = rt * kTile + 8 * (v / 4) + 4 * g + v % 4;
+                if (row < H) out[(int64_t)row * n] = d[t][rt][v];
+            }
+        }
+    }
+}
+
+// The same from inner size 64 on, at the bfloat16 rate with both operands split three ways (see
+// the forward kernel): h when a chunk is staged (an operand slot = eight consecutive edges of one
+// row of dW), ds in registers as it arrives.
+template <int H>
+__global__ __launch_bounds__(kWave * kWaves) void radial_linear_bwd_weight_split_kernel(
+    const float *__restrict__ h, const float *__restrict__ ds, float *__restrict__ partial, int64_t num_edges,
+    int n, int groups) {
+    constexpr int RT = H / kTile;                // row tiles of dW
+    constexpr int CHUNK = 64, Q = CHUNK / 16;    // edges per step; inner blocks of 16 edges
+    constexpr int SLOTS = 2 * Q * H;             // (q, g, row) operand slots of a chunk of h
+    constexpr int PER_THREAD = SLOTS / (kWave * kWaves);
+    static_assert(H % kTile == 0 && SLOTS % (kWave * kWaves) == 0, "whole tiles, whole rounds of slots");
+    __shared__ __attribute__((aligned(16))) bf16x8 rows[2][3][SLOTS];
+    const int tid = threadIdx.x, lane = tid % kWave, wave = tid / kWave;
+    const int g = lane / kTile, c = lane % kTile;
+    const int slabs = (n + kSlab - 1) / kSlab;
+    const int slab = blockIdx.x % slabs, group = blockIdx.x / slabs;
+    const int col0 = slab * kSlab + wave * (kTile * kColTiles);
+    const int64_t per_group = ((num_edges + groups - 1) / groups + CHUNK - 1) / CHUNK * CHUNK;
+    const int64_t first = (int64_t)group * per_group;
+    const int64_t last = first + per_group < num_edges ? first + per_group : num_edges;
+
+    f32x16 d[kColTiles][RT];
+#pragma unroll
+    for (int t = 0; t < kColTiles; t++)
+#pragma unroll
+        for (int rt = 0; rt < RT; rt++)
+            d[t][rt] = f32x16{0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
+    bool col_ok[kColTiles];
+    const float *dcol[kColTiles];
+#pragma unroll
+    for (int t = 0; t < kColTiles; t++) {
+        col_ok[t] = col0 + t * kTile < n;
+        dcol[t] = ds + (col_ok[t] ? col0 + t * kTile + c : 0);
+    }
+
+    float staged[PER_THREAD][8];
+    auto fetch = [&](int64_t e0) {  // slot (q, g, row): h[e0 + 16 q + 8 g + m][row], m < 8
+#pragma unroll
+        for (int i = 0; i < PER_THREAD; i++) {
+            const int slot = i * kWave * kWaves + tid;
+            const int64_t e = e0 + (slot / H) * 8;
+#pragma unroll
+            for (int m = 0; m < 8; m++) staged[i][m] = e + m < last ? h[(e + m) * H + slot % H] : 0.f;
+        }
+    };
+    auto commit = [&](int buf) {
+#pragma unroll
+        for (int i = 0; i < PER_THREAD; i++) {
+            const Split3 parts = split3(staged[i]);
+#pragma unroll
+            for (int t = 0; t < 3; t++) rows[buf][t][i * kWave * kWaves + tid] = parts.term[t];
+        }
+    };
+    if (first < last) {
+        fetch(first);
+        commit(0);
+    }
+    __syncthreads();
+    // the eight ds values of a lane for the block of 16 edges at `e`: loaded one block ahead
+    float xn[kColTiles][8];
+    auto load_ds = [&](int64_t e) {
+#pragma unroll
+        for (int t = 0; t < kColTiles; t++)
+#pragma unroll
+            for (int m = 0; m < 8; m++) {
+                const int64_t em = e + g * 8 + m;
+                xn[t][m] = em < last ? __builtin_nontemporal_load(dcol[t] + em * n) : 0.f;
+            }
+    };
+    if (first < last) load_ds(first);
+    int buf = 0;
+    for (int64_t e0 = first; e0 < last; e0 += CHUNK, buf ^= 1) {
+        const bool more = e0 + CHUNK < last;
+        if (more) fetch(e0 + CHUNK);
+#pragma unroll 1
+        for (int q = 0; q < Q; q++) {  // (not unrolled: the split operands of one block fill the registers)
+            Split3 b[kColTiles];
+#pragma unroll
+            for (int t = 0; t < kColTiles; t++) b[t] = split3(xn[t]);
+            if (e0 + (q + 1) * 16 < last) load_ds(e0 + (q + 1) * 16);
+            constexpr int kPairs[6][2] = {{0, 2}, {1, 1}, {2, 0}, {0, 1}, {1, 0}, {0, 0}};
+#pragma unroll
+            for (int rt = 0; rt < RT; rt++) {
+                bf16x8 a[3];
+#pragma unroll
+                for (int ta = 0; ta < 3; ta++) a[ta] = rows[buf][ta][(q * 2 + g) * H + rt * kTile + c];
+#pragma unroll
+                for (int u = 0; u < 6; u++) {
+#pragma unroll
+                    for (int t = 0; t < kColTiles; t++)
+                        d[t][rt] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a[kPairs[u][0]], b[t].term[kPairs[u][1]],
+                                                                           d[t][rt], 0, 0, 0);
+                }
+            }
+        }
+        if (more) commit(buf ^ 1);
+        __syncthreads();
+    }
+#pragma unroll
+    for (int t = 0; t < kColTiles; t++) {
+        if (!col_ok[t]) continue;
+        float *out = partial + (int64_t)group * H * n + col0 + t * kTile + c;
+#pragma unroll
+        for (int rt = 0; rt < RT; rt++) {
+#pragma unroll
+            for (int v = 0; v < 16; v++) out[(int64_t)(rt * kTile + 8 * (v / 4) + 4 * g + v % 4) * n] = d[t][rt][v];
+        }
+    }
+}
+
+__global__ void radial_linear_sum_groups_kernel(const float *__restrict__ partial, float *__restrict__ dw,
+                                                int64_t count, int groups) {
+    const int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+    if (i >= count) return;
+    float total = 0.f;
+    for (int q = 0; q < groups; q++) total += partial[(int64_t)q * count + i];
+    dw[i] = total;
+}
+
+// ranges of the edges: enough blocks to fill the machine several times over, at most 128 slices
+int weight_groups(int64_t num_edges, int n) {
+    const int slabs = (n + kSlab - 1) / kSlab;
+    int64_t groups = (2048 + slabs - 1) / slabs;
+    const int64_t most = (num_edges + 63) / 64;
+    if (groups > most) groups = most;
+    if (groups > 128) groups = 128;
+    return groups < 1 ? 1 : (int)groups;
+}
+
+template <int H>
+int launch_bwd_weight(const float *h, const float *ds, float *dw, float *partial, int64_t num_edges, int n,
+                      hipStream_t stream) {
+    const int groups = weight_groups(num_edges, n);
+    const int slabs = (n + kSlab - 1) / kSlab;
+    if constexpr (H >= 64)
+        hipLaunchKernelGGL((radial_linear_bwd_weight_split_kernel<H>), dim3((unsigned)(slabs * groups)),
+                           dim3(kWave * kWaves), 0, stream, h, ds, partial, num_edges, n, groups);
+    else
+        hipLaunchKernelGGL((radial_linear_bwd_weight_kernel<H>), dim3((unsigned)(slabs * groups)),
+                           dim3(kWave * kWaves), 0, stream, h, ds, partial, num_edges, n, groups);
+    int rc = check_hip(hipGetLastError(), "radial_linear_bwd_weight launch");
+    if (rc) return rc;
+    const int64_t count = (int64_t)H * n;
+    hipLaunchKernelGGL(radial_linear_sum_groups_kernel, dim3((unsigned)((count + 255) / 256)), dim3(256), 0, stream,
+                       partial, dw, count, groups);
+    return check_hip(hipGetLastError(), "radial_linear_bwd_weight reduction launch");
+}
+
 int check_shapes(const char *what, int64_t num_edges, int32_t inner, int32_t n) {
     if (num_edges < 0 || inner <= 0 || n <= 0)
         return set_error(E3J_AMD_INVALID_ARGUMENT, std::string(what) + ": bad sizes");
@@ -264,6 +531,29 @@ extern "C" int e3j_amd_radial_linear_fwd(const float *h, const float *w, float *
         case 32: return launch_fwd<32>(h, w, s, num_edges, n, stream);
         case 64: return launch_fwd<64>(h, w, s, num_edges, n, stream);
         default: return launch_fwd<128>(h, w, s, num_edges, n, stream);
+    }
+}
+
+extern "C" size_t e3j_amd_radial_linear_bwd_weight_workspace_bytes(int64_t num_edges, int32_t inner, int32_t n) {
+    if (num_edges <= 0 || inner <= 0 || n <= 0) return 0;
+    return sizeof(float) * (size_t)weight_groups(num_edges, n) * inner * n;
+}
+
+extern "C" int e3j_amd_radial_linear_bwd_weight(const float *h, const float *ds, float *dw, void *workspace,
+                                                int64_t num_edges, int32_t inner, int32_t n, void *stream_) {
+    if (int rc = check_shapes("radial_linear_bwd_weight", num_edges, inner, n)) return rc;
+    if (dw == nullptr) return set_error(E3J_AMD_INVALID_ARGUMENT, "radial_linear_bwd_weight: null operand");
+    hipStream_t stream = static_cast<hipStream_t>(stream_);
+    if (num_edges == 0) return launch_fill_zero(dw, sizeof(float) * (size_t)inner * n, stream);
+    if (h == nullptr || ds == nullptr || workspace == nullptr)
+        return set_error(E3J_AMD_INVALID_ARGUMENT, "radial_linear_bwd_weight: null operand");
+    float *partial = static_cast<float *>(workspace);
+    switch (inner) {
+        case 8: return launch_bwd_weight<8>(h, ds, dw, partial, num_edges, n, stream);
+        case 16: return launch_bwd_weight<16>(h, ds, dw, partial, num_edges, n, stream);
+        case 32: return launch_bwd_weight<32>(h, ds, dw, partial, num_edges, n, stream);
+        case 64: return launch_bwd_weight<64>(h, ds, dw, partial, num_edges, n, stream);
+        default: return launch_bwd_weight<128>(h, ds, dw, partial, num_edges, n, stream);
     }
 }
 

@@ -3,8 +3,9 @@
 The per-edge, per-path weights `s (E, paths * channels)` are the operand the convolution reads
 most; the layer that writes them is a product with a small inner size (the hidden width of the
 radial network), bound by the stream it writes.  `radial_linear` runs it as one HIP kernel
-(`csrc/radial_linear.hip`); the products of its backward, `ds @ w.T` and `h.T @ ds`, read the
-stream along the contracted index and are left to the library.
+(`csrc/radial_linear.hip`), and so does `dw = h.T @ ds` of its backward (the contraction runs over
+the edges: both operands arrive coalesced); `dh = ds @ w.T` reads the stream along the contracted
+index and is left to the library.
 """
 
 from __future__ import annotations
@@ -42,8 +43,26 @@ class _RadialLinear(torch.autograd.Function):
     def backward(ctx, ds):
         h, w = ctx.saved_tensors
         dh = ds @ w.t() if ctx.needs_input_grad[0] else None
-        dw = h.t() @ ds if ctx.needs_input_grad[1] else None
+        dw = _weight_gradient(h, ds) if ctx.needs_input_grad[1] else None
         return dh, dw
+
+
+def _weight_gradient(h: torch.Tensor, ds: torch.Tensor) -> torch.Tensor:
+    """`h.T @ ds` on the matrix cores (the library product when autograd records the backward,
+    e.g. for a second derivative, or for tensors the kernel does not take)."""
+    if torch.is_grad_enabled() and (h.requires_grad or ds.requires_grad) or ds.dtype != torch.float32:
+        return h.t() @ ds
+    lib = _lib.load()
+    h, ds = h.contiguous(), ds.contiguous()
+    edges, inner, n = int(h.shape[0]), int(h.shape[1]), int(ds.shape[1])
+    dw = torch.empty((inner, n), dtype=h.dtype, device=h.device)
+    ws = torch.empty(max(int(lib.e3j_amd_radial_linear_bwd_weight_workspace_bytes(edges, inner, n)), 4),
+                     dtype=torch.uint8, device=h.device)
+    with torch.cuda.device(h.device):
+        _lib.check(lib.e3j_amd_radial_linear_bwd_weight(
+            h.data_ptr(), ds.data_ptr(), dw.data_ptr(), ws.data_ptr(), edges, inner, n,
+            torch.cuda.current_stream(h.device).cuda_stream))
+    return dw
 
 
 def radial_linear(h: torch.Tensor, w: torch.Tensor) -> torch.Tensor:

@@ -214,6 +214,12 @@ int e3j_amd_harmonics_bwd(const void *vec, const void *dout, int64_t num, int32_
  * convolution, and the operand the convolution reads most. */
 int e3j_amd_radial_linear_fwd(const float *h, const float *w, float *s, int64_t num_edges,
                               int32_t inner, int32_t n, void *stream);
+/* Its backward with respect to the weights: dw (inner, n) = h^T ds, ds (num_edges, n) read once,
+ * summed over the edges in a fixed order (bit-reproducible).  workspace: device memory of
+ * e3j_amd_radial_linear_bwd_weight_workspace_bytes(num_edges, inner, n) bytes. */
+size_t e3j_amd_radial_linear_bwd_weight_workspace_bytes(int64_t num_edges, int32_t inner, int32_t n);
+int e3j_amd_radial_linear_bwd_weight(const float *h, const float *ds, float *dw, void *workspace,
+                                     int64_t num_edges, int32_t inner, int32_t n, void *stream);
 
 /* Row-wise sparse tensor product, the edge-wise sibling of the convolution (no gather, no
  * scatter): z[r] = sum_n val_n x[r, j_n] (*) y[r, k_n] -> z[r, i_n].  Operands and sizes of the

@@ -50,3 +50,30 @@ def test_gradients_and_errors():
     lib = _lib.load()
     assert lib.e3j_amd_radial_linear_fwd(None, None, None, 4, 24, 64, None) == _lib.UNIMPLEMENTED
     assert lib.e3j_amd_radial_linear_fwd(None, None, None, 4, 32, 64, None) == _lib.INVALID_ARGUMENT
+
+
+@pytest.mark.parametrize("inner", [8, 16, 32, 64, 128])
+@pytest.mark.parametrize("edges,n", [(1, 32), (70, 128), (4099, 1472), (20001, 96)])
+def test_weight_gradient_matches_the_float64_product_and_repeats(inner, edges, n):
+    g = torch.Generator(device="cuda").manual_seed(inner * 31 + edges)
+    h = torch.randn(edges, inner, device="cuda", generator=g)
+    w = torch.randn(inner, n, device="cuda", generator=g, requires_grad=True)
+    ds = torch.randn(edges, n, device="cuda", generator=g)
+    (dw,) = torch.autograd.grad(radial_linear(h, w), (w,), ds)
+    want = h.double().t() @ ds.double()
+    bound = 1e-6 + 1e-5 * want.abs() + 16 * 2.0 ** -24 * (h.double().abs().t() @ ds.double().abs())
+    assert dw.shape == (inner, n)
+    assert bool(((dw.double() - want).abs() <= bound).all())
+    (again,) = torch.autograd.grad(radial_linear(h, w), (w,), ds)
+    assert torch.equal(dw, again)   # fixed summation order over the edges
+
+
+def test_second_derivative_goes_through_the_library_products():
+    g = torch.Generator(device="cuda").manual_seed(9)
+    h = torch.randn(50, 16, device="cuda", generator=g, requires_grad=True)
+    w = torch.randn(16, 64, device="cuda", generator=g, requires_grad=True)
+    ds = torch.randn(50, 64, device="cuda", generator=g, requires_grad=True)
+    dh, dw = torch.autograd.grad(radial_linear(h, w), (h, w), ds, create_graph=True)
+    (dds,) = torch.autograd.grad((dh.sum() + dw.sum()), (ds,))
+    want = (torch.ones_like(dh) @ w + h @ torch.ones_like(dw)).detach()
+    torch.testing.assert_close(dds, want, rtol=1e-5, atol=1e-5)
