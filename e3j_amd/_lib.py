@@ -102,6 +102,7 @@ SYMBOLS = {
     "e3j_amd_harmonics": (ctypes.c_int, [_P, ctypes.c_int64] + [ctypes.c_int32] * 4 + [_P, _P]),
     "e3j_amd_harmonics_bwd": (ctypes.c_int, [_P, _P, ctypes.c_int64] + [ctypes.c_int32] * 4 + [_P, _P]),
     "e3j_amd_radial_linear_fwd": (ctypes.c_int, [_P, _P, _P, ctypes.c_int64, ctypes.c_int32, ctypes.c_int32, _P]),
+    "e3j_amd_radial_linear_bwd_input": (ctypes.c_int, [_P, _P, _P, ctypes.c_int64, ctypes.c_int32, ctypes.c_int32, _P]),
     "e3j_amd_radial_linear_bwd_weight_workspace_bytes": (ctypes.c_size_t, [ctypes.c_int64, ctypes.c_int32, ctypes.c_int32]),
     "e3j_amd_radial_linear_bwd_weight": (ctypes.c_int, [_P, _P, _P, _P, ctypes.c_int64, ctypes.c_int32, ctypes.c_int32, _P]),
     "e3j_amd_wrap_index": (ctypes.c_int, [_P, ctypes.c_int64, ctypes.c_int32, _P, _P]),

@@ -1,12 +1,9 @@
 // Last layer of the radial network that produces the per-edge, per-path weights of the
-// convolution: s (E, N) = h (E, H) W (H, N) with N = paths * channels, float32, and the weight
-// gradient of its backward pass, dW = h^T ds.  The one dense contraction next to the
-// convolution: it runs on the matrix cores.  H is small (8..128), so each pass is bound by the
-// E * N stream it writes or reads; the tilings keep that stream at whole 128-byte lines and
-// everything else (h, W) in registers or LDS.  (The other product of the backward pass, ds W^T,
-// reads that stream with the contracted index along the rows, which the operand layout below can
-// only take through a transposition in LDS; it is left to the library, which reads it at 3.3 to
-// 5.8 TB/s.)
+// convolution: s (E, N) = h (E, H) W (H, N) with N = paths * channels, float32, and the two
+// products of its backward pass, dW = h^T ds and (from H = 64 on) dh = ds W^T.  The one dense
+// contraction next to the convolution: it runs on the matrix cores.  H is small (8..128), so each
+// pass is bound by the E * N stream it writes or reads; the tilings keep that stream at whole
+// 128-byte lines and everything else (h, W) in registers or LDS.
 //
 // Register layout of one 32x32x2 product D += A B on a 64-lane wave (g = lane / 32, c = lane % 32):
 // a lane supplies A[c][g] and B[g][c] and holds D[8 * (v / 4) + 4 * g + v % 4][c] in element v of
@@ -506,6 +503,149 @@ int launch_bwd_weight(const float *h, const float *ds, float *dw, float *partial
     return check_hip(hipGetLastError(), "radial_linear_bwd_weight reduction launch");
 }
 
+// dh (E, H) = ds W^T for inner sizes of 64 and more, with W^T passed as wt (n, H).  The
+// contraction runs along the rows of ds, so a lane (which stands for an edge in the operand
+// layout) would read its own row; instead a wave loads its tile of 32 R edges x 32 n the coalesced
+// way (a row piece of 128 bytes per 8 lanes), splits it three ways and writes the parts to its
+// private piece of LDS in operand order, from where every lane fetches its slots with 16-byte
+// reads.  The rows of wt of the same 32 n, one contiguous block, are split and shared by the
+// waves of the block.  ds is read once.
+typedef uint32_t u32x2 __attribute__((ext_vector_type(2)));
+
+template <int H, int R>
+__global__ __launch_bounds__(kWave * kWaves) void radial_linear_bwd_input_split_kernel(
+    const float *__restrict__ ds, const float *__restrict__ wt, float *__restrict__ dh, int64_t num_edges, int n) {
+    constexpr int CT = H / kTile;                 // column tiles of dh
+    constexpr int CHUNK = 32, Q = CHUNK / 16;     // n per step; inner blocks of 16
+    constexpr int ROWS = R * kTile;               // edges of a wave
+    constexpr int A_SLOTS = 2 * Q * ROWS;         // (q, g, edge) operand slots of a wave's tile
+    constexpr int A_PIECES = ROWS * CHUNK / 4 / kWave;  // 16-byte pieces of the tile per lane
+    constexpr int B_SLOTS = 2 * Q * H;            // (q, g, column) operand slots of the wt chunk
+    constexpr int B_PER_THREAD = (B_SLOTS + kWave * kWaves - 1) / (kWave * kWaves);
+    __shared__ __attribute__((aligned(16))) bf16x8 a_tile[kWaves][3][A_SLOTS];
+    __shared__ __attribute__((aligned(16))) bf16x8 b_tile[3][B_SLOTS];
+    const int tid = threadIdx.x, lane = tid % kWave, wave = tid / kWave;
+    const int g = lane / kTile, c = lane % kTile;
+    const int64_t e0 = ((int64_t)blockIdx.x * kWaves + wave) * ROWS;
+
+    // a lane moves A_PIECES pieces of 16 bytes of the tile: piece p = 64 i + lane is n-quad p % 8 of edge p / 8
+    const float *src[A_PIECES];
+    int half_slot[A_PIECES];  // where the piece goes: 8-byte half (p % 2) of slot (q, g, edge)
+#pragma unroll
+    for (int i = 0; i < A_PIECES; i++) {
+        const int p = i * kWave + lane, edge = p / 8, quad = p % 8;
+        int64_t row = e0 + edge;
+        if (row >= num_edges) row = num_edges - 1;  // rows past the end are computed and not stored
+        src[i] = ds + row * n + quad * 4;
+        half_slot[i] = (((quad / 4) * 2 + (quad / 2) % 2) * ROWS + edge) * 2 + quad % 2;
+    }
+    f32x16 d[R][CT];
+#pragma unroll
+    for (int r = 0; r < R; r++)
+#pragma unroll
+        for (int ct = 0; ct < CT; ct++)
+            d[r][ct] = f32x16{0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
+
+    f32x4 a_next[A_PIECES];
+    float b_next[B_PER_THREAD][8];
+    auto fetch = [&](int t) {
+#pragma unroll
+        for (int i = 0; i < A_PIECES; i++)
+            a_next[i] = __builtin_nontemporal_load(reinterpret_cast<const f32x4 *>(src[i] + t * CHUNK));
+#pragma unroll
+        for (int i = 0; i < B_PER_THREAD; i++) {  // slot (q, g, column): wt[32 t + 16 q + 8 g + m][column]
+            const int slot = i * kWave * kWaves + tid;
+            if (B_SLOTS % (kWave * kWaves) == 0 || slot < B_SLOTS) {
+                const float *col = wt + ((int64_t)t * CHUNK + (slot / H) * 8) * H + slot % H;
+#pragma unroll
+                for (int m = 0; m < 8; m++) b_next[i][m] = col[m * H];
+            }
+        }
+    };
+    auto commit = [&]() {
+        u32x2 *halves[3] = {reinterpret_cast<u32x2 *>(a_tile[wave][0]), reinterpret_cast<u32x2 *>(a_tile[wave][1]),
+                            reinterpret_cast<u32x2 *>(a_tile[wave][2])};
+#pragma unroll
+        for (int i = 0; i < A_PIECES; i++) {
+            float rest[4] = {a_next[i].x, a_next[i].y, a_next[i].z, a_next[i].w};
+#pragma unroll
+            for (int t = 0; t < 3; t++) {  // the three parts of four values: see split3
+                u32x2 packed;
+#pragma unroll
+                for (int m = 0; m < 4; m += 2) {
+                    const uint32_t lo = __float_as_uint(rest[m]) & 0xffff0000u, hi = __float_as_uint(rest[m + 1]) & 0xffff0000u;
+                    packed[m / 2] = (lo >> 16) | hi;
+                    rest[m] -= __uint_as_float(lo);
+                    rest[m + 1] -= __uint_as_float(hi);
+                }
+                halves[t][half_slot[i]] = packed;
+            }
+        }
+#pragma unroll
+        for (int i = 0; i < B_PER_THREAD; i++) {
+            const int slot = i * kWave * kWaves + tid;
+            if (B_SLOTS % (kWave * kWaves) == 0 || slot < B_SLOTS) {
+                const Split3 parts = split3(b_next[i]);
+#pragma unroll
+                for (int t = 0; t < 3; t++) b_tile[t][slot] = parts.term[t];
+            }
+        }
+    };
+    const int chunks = n / CHUNK;
+    fetch(0);
+    for (int t = 0; t < chunks; t++) {
+        commit();
+        if (t + 1 < chunks) fetch(t + 1);
+        __syncthreads();
+        constexpr int kPairs[6][2] = {{0, 2}, {1, 1}, {2, 0}, {0, 1}, {1, 0}, {0, 0}};
+#pragma unroll
+        for (int q = 0; q < Q; q++) {
+            bf16x8 a[R][3];
+#pragma unroll
+            for (int r = 0; r < R; r++)
+#pragma unroll
+                for (int ta = 0; ta < 3; ta++) a[r][ta] = a_tile[wave][ta][(q * 2 + g) * ROWS + r * kTile + c];
+#pragma unroll
+            for (int ct = 0; ct < CT; ct++) {
+                bf16x8 b[3];
+#pragma unroll
+                for (int tb = 0; tb < 3; tb++) b[tb] = b_tile[tb][(q * 2 + g) * H + ct * kTile + c];
+#pragma unroll
+                for (int u = 0; u < 6; u++) {
+#pragma unroll
+                    for (int r = 0; r < R; r++)
+                        d[r][ct] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a[r][kPairs[u][0]], b[kPairs[u][1]], d[r][ct],
+                                                                           0, 0, 0);
+                }
+            }
+        }
+        __syncthreads();  // every wave is done with the shared rows of wt before they are replaced
+    }
+#pragma unroll
+    for (int r = 0; r < R; r++) {
+#pragma unroll
+        for (int ct = 0; ct < CT; ct++) {
+            float *out = dh + (e0 + r * kTile + 4 * g) * H + ct * kTile + c;
+#pragma unroll
+            for (int v = 0; v < 16; v++) {
+                const int row = 8 * (v / 4) + v % 4;
+                if (e0 + r * kTile + 4 * g + row < num_edges) out[(int64_t)row * H] = d[r][ct][v];
+            }
+        }
+    }
+}
+
+template <int H>
+int launch_bwd_input(const float *ds, const float *wt, float *dh, int64_t num_edges, int n, hipStream_t stream) {
+    constexpr int R = H >= 128 ? 1 : 2;  // row tiles per wave
+    const int64_t per_block = (int64_t)kWaves * R * kTile;
+    const int64_t blocks = (num_edges + per_block - 1) / per_block;
+    if (blocks > 0x7fffffffLL) return set_error(E3J_AMD_INVALID_ARGUMENT, "radial_linear_bwd_input: too many edges");
+    hipLaunchKernelGGL((radial_linear_bwd_input_split_kernel<H, R>), dim3((unsigned)blocks), dim3(kWave * kWaves), 0,
+                       stream, ds, wt, dh, num_edges, n);
+    return check_hip(hipGetLastError(), "radial_linear_bwd_input launch");
+}
+
 int check_shapes(const char *what, int64_t num_edges, int32_t inner, int32_t n) {
     if (num_edges < 0 || inner <= 0 || n <= 0)
         return set_error(E3J_AMD_INVALID_ARGUMENT, std::string(what) + ": bad sizes");
@@ -555,6 +695,20 @@ extern "C" int e3j_amd_radial_linear_bwd_weight(const float *h, const float *ds,
         case 64: return launch_bwd_weight<64>(h, ds, dw, partial, num_edges, n, stream);
         default: return launch_bwd_weight<128>(h, ds, dw, partial, num_edges, n, stream);
     }
+}
+
+extern "C" int e3j_amd_radial_linear_bwd_input(const float *ds, const float *wt, float *dh, int64_t num_edges,
+                                               int32_t inner, int32_t n, void *stream_) {
+    if (int rc = check_shapes("radial_linear_bwd_input", num_edges, inner, n)) return rc;
+    if (inner < 64)
+        return set_error(E3J_AMD_UNIMPLEMENTED, "radial_linear_bwd_input: hidden sizes below 64 are left to the "
+                                                "library product, which reads ds near the rate of the memory");
+    if (num_edges == 0) return E3J_AMD_OK;
+    if (ds == nullptr || wt == nullptr || dh == nullptr)
+        return set_error(E3J_AMD_INVALID_ARGUMENT, "radial_linear_bwd_input: null operand");
+    hipStream_t stream = static_cast<hipStream_t>(stream_);
+    return inner == 64 ? launch_bwd_input<64>(ds, wt, dh, num_edges, n, stream)
+                       : launch_bwd_input<128>(ds, wt, dh, num_edges, n, stream);
 }
 
 }  // namespace e3j_amd

@@ -4,8 +4,8 @@ The per-edge, per-path weights `s (E, paths * channels)` are the operand the con
 most; the layer that writes them is a product with a small inner size (the hidden width of the
 radial network), bound by the stream it writes.  `radial_linear` runs it as one HIP kernel
 (`csrc/radial_linear.hip`), and so does `dw = h.T @ ds` of its backward (the contraction runs over
-the edges: both operands arrive coalesced); `dh = ds @ w.T` reads the stream along the contracted
-index and is left to the library.
+the edges: both operands arrive coalesced) and, from inner size 64 on, `dh = ds @ w.T` (the stream
+transposed through LDS); below that the library product already reads `ds` near the rate of the memory.
 """
 
 from __future__ import annotations
@@ -42,9 +42,24 @@ class _RadialLinear(torch.autograd.Function):
     @staticmethod
     def backward(ctx, ds):
         h, w = ctx.saved_tensors
-        dh = ds @ w.t() if ctx.needs_input_grad[0] else None
+        dh = _input_gradient(ds, w) if ctx.needs_input_grad[0] else None
         dw = _weight_gradient(h, ds) if ctx.needs_input_grad[1] else None
         return dh, dw
+
+
+def _input_gradient(ds: torch.Tensor, w: torch.Tensor) -> torch.Tensor:
+    """`ds @ w.T`: from inner size 64 on the kernel that transposes `ds` through LDS; below, and when
+    autograd records the backward, the library product (which reads `ds` near the rate of the memory)."""
+    if (int(w.shape[0]) < 64 or ds.dtype != torch.float32
+            or torch.is_grad_enabled() and (ds.requires_grad or w.requires_grad)):
+        return ds @ w.t()
+    ds, wt = ds.contiguous(), w.t().contiguous()
+    dh = torch.empty((ds.shape[0], w.shape[0]), dtype=ds.dtype, device=ds.device)
+    with torch.cuda.device(ds.device):
+        _lib.check(_lib.load().e3j_amd_radial_linear_bwd_input(
+            ds.data_ptr(), wt.data_ptr(), dh.data_ptr(), int(ds.shape[0]), int(w.shape[0]), int(w.shape[1]),
+            torch.cuda.current_stream(ds.device).cuda_stream))
+    return dh
 
 
 def _weight_gradient(h: torch.Tensor, ds: torch.Tensor) -> torch.Tensor:

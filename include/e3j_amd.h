@@ -214,6 +214,11 @@ int e3j_amd_harmonics_bwd(const void *vec, const void *dout, int64_t num, int32_
  * convolution, and the operand the convolution reads most. */
 int e3j_amd_radial_linear_fwd(const float *h, const float *w, float *s, int64_t num_edges,
                               int32_t inner, int32_t n, void *stream);
+/* Its backward with respect to h for inner sizes of 64 and 128: dh (num_edges, inner) = ds w^T, with
+ * the weights passed transposed, wt (n, inner) row-major; ds is read once.  Smaller inner sizes
+ * return E3J_AMD_UNIMPLEMENTED: the library product already reads ds near the rate of the memory. */
+int e3j_amd_radial_linear_bwd_input(const float *ds, const float *wt, float *dh, int64_t num_edges,
+                                    int32_t inner, int32_t n, void *stream);
 /* Its backward with respect to the weights: dw (inner, n) = h^T ds, ds (num_edges, n) read once,
  * summed over the edges in a fixed order (bit-reproducible).  workspace: device memory of
  * e3j_amd_radial_linear_bwd_weight_workspace_bytes(num_edges, inner, n) bytes. */

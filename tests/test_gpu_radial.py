@@ -77,3 +77,23 @@ def test_second_derivative_goes_through_the_library_products():
     (dds,) = torch.autograd.grad((dh.sum() + dw.sum()), (ds,))
     want = (torch.ones_like(dh) @ w + h @ torch.ones_like(dw)).detach()
     torch.testing.assert_close(dds, want, rtol=1e-5, atol=1e-5)
+
+
+@pytest.mark.parametrize("inner", [32, 64, 128])
+@pytest.mark.parametrize("edges,n", [(1, 32), (33, 64), (257, 1472), (1000, 2944)])
+def test_input_gradient_matches_the_float64_product(inner, edges, n):
+    g = torch.Generator(device="cuda").manual_seed(inner * 77 + edges)
+    h = torch.randn(edges, inner, device="cuda", generator=g, requires_grad=True)
+    w = torch.randn(inner, n, device="cuda", generator=g)
+    ds = torch.randn(edges, n, device="cuda", generator=g)
+    (dh,) = torch.autograd.grad(radial_linear(h, w), (h,), ds)
+    want = ds.double() @ w.double().t()
+    bound = 1e-6 + 1e-5 * want.abs() + 16 * 2.0 ** -24 * (ds.double().abs() @ w.double().abs().t())
+    assert dh.shape == (edges, inner)
+    assert bool(((dh.double() - want).abs() <= bound).all())
+    # one-hot cotangent rows pick rows of w^T exactly (integers split exactly)
+    wi = torch.arange(inner * n, device="cuda", dtype=torch.float32).reshape(inner, n) % 4093
+    pick = torch.zeros(edges, n, device="cuda")
+    pick[torch.arange(edges), (torch.arange(edges) * 7) % n] = 1.0
+    (picked,) = torch.autograd.grad(radial_linear(h, wi), (h,), pick)
+    assert torch.equal(picked, wi.t()[(torch.arange(edges, device="cuda") * 7) % n])
