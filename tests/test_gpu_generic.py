@@ -106,6 +106,25 @@ def test_random_table_fwd_bwd(channels, grouping):
     check_all(idx, val, mix, x, y, s, dm, snd, rcv, Z, res, tag=f"K={channels} {grouping}")
 
 
+@pytest.mark.parametrize("dtype", [np.float32, np.float64])
+@pytest.mark.parametrize("grouping", ["receiver", "sender"])
+def test_more_than_64_harmonics_components(dtype, grouping):
+    """Up to 64 y components travel in one register of the wave; longer rows (here 81, the
+    harmonics up to l = 8) are read from memory, and a table longer than one 64-entry load."""
+    rng = np.random.default_rng(81)
+    N, E, X, Y, Z, S, K, nnz = 7, 30, 4, 81, 12, 5, 40, 300
+    idx, val, mix = H.random_table(rng, nnz, X, Y, Z, S)
+    assert idx[:, 2].max() >= 64
+    snd, rcv = H.random_graph(rng, N, E)
+    x, y, s, dm = H.random_operands(rng, N, E, X, Y, S, K, Z, dtype=dtype)
+    out, dx, dy, ds = run_abi(idx, val, mix, x, y, s, dm, snd, rcv, Z, dtype=dtype, grouping=grouping)
+    ref, mag = H.forward_reference(idx, val, mix, x, y, s, snd, rcv, Z)
+    (rx, ry, rs), (mx, my, ms) = H.backward_reference(idx, val, mix, x, y, s, snd, rcv, dm)
+    tol = dict(rtol=1e-5, atol=1e-6) if dtype == np.float32 else dict(rtol=1e-12, atol=1e-12, ulps=0.0)
+    for got, r, m, name in ((out, ref, mag, "out"), (dx, rx, mx, "dx"), (dy, ry, my, "dy"), (ds, rs, ms, "ds")):
+        H.assert_parity(got, r, m, f"{name} Y=81 {np.dtype(dtype).name} {grouping}", **tol)
+
+
 # ---------------------------------------------------------------------------
 # layouts, dtypes, index widths
 # ---------------------------------------------------------------------------
