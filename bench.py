@@ -129,6 +129,12 @@ class AbiCalls:
         self.params.row_order = self.order.data_ptr() if self.order is not None else None
         self.out = torch.empty_like(w.dm)
         self.dx, self.dy, self.ds = torch.empty_like(w.x), torch.empty_like(w.y), torch.empty_like(w.s)
+        # the default backward of the operators: tiles of receivers when the signature has such a kernel
+        self.schedule = None
+        tile_rows = min(int(config().tile_rows), int(self.lib.e3j_amd_tile_rows(sig))) if sig >= 0 else 0
+        if tile_rows >= 2:
+            from e3j_amd.graph import TileSchedule
+            self.schedule = TileSchedule(self.other, self.ptr, self.perm, self.order, w.num_nodes, tile_rows)
 
     def _stream(self):
         return int(self.torch.cuda.current_stream().cuda_stream)
@@ -154,6 +160,18 @@ class AbiCalls:
             self._stream()))
 
     def backward(self):
+        """The backward the operators run by default."""
+        if self.schedule is None:
+            return self.backward_receiver()
+        w = self.w
+        self._lib.check(self.lib.e3j_amd_convolution_bwd_tiled(
+            ctypes.byref(self.params), w.x.data_ptr(), w.y.data_ptr(), w.s.data_ptr(), w.dm.data_ptr(),
+            self.other.data_ptr(), self.ptr.data_ptr(), self.perm.data_ptr() if self.perm is not None else None,
+            ctypes.byref(self.schedule.struct), self.dx.data_ptr(), self.dy.data_ptr(), self.ds.data_ptr(),
+            self._stream()))
+
+    def backward_receiver(self):
+        """One wave per (receiver, slice, part), one set of dx atomics per edge."""
         w = self.w
         self._lib.check(self.lib.e3j_amd_convolution_bwd_receiver(
             ctypes.byref(self.params), self.coef.data_ptr(), w.x.data_ptr(), w.y.data_ptr(),

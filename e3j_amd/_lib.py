@@ -46,6 +46,19 @@ class ConvParams(ctypes.Structure):
 MODE_OUTER, MODE_INNER, MODE_MAP = 0, 1, 2
 
 
+class TileSchedule(ctypes.Structure):
+    """`e3j_amd_tile_schedule`."""
+
+    _fields_ = [
+        ("tile_rows", ctypes.c_int32),
+        ("num_work", ctypes.c_int32),
+        ("work", ctypes.c_void_p),
+        ("sender", ctypes.c_void_p),
+        ("edge", ctypes.c_void_p),
+        ("local", ctypes.c_void_p),
+    ]
+
+
 class TpParams(ctypes.Structure):
     """`e3j_amd_tp_params`."""
 
@@ -89,6 +102,12 @@ SYMBOLS = {
     "e3j_amd_convolution_bwd_receiver": (ctypes.c_int, [_PARAMS] + [_P] * 12),
     "e3j_amd_convolution_bwd_ordered_workspace_bytes": (ctypes.c_size_t, [_PARAMS]),
     "e3j_amd_convolution_bwd_ordered": (ctypes.c_int, [_PARAMS] + [_P] * 13),
+    "e3j_amd_tile_rows": (ctypes.c_int32, [ctypes.c_int32]),
+    "e3j_amd_tile_schedule_num_work": (ctypes.c_int64, [ctypes.c_int32, ctypes.c_int64, ctypes.c_int32, ctypes.c_int32]),
+    "e3j_amd_tile_schedule_workspace_bytes": (ctypes.c_size_t, [ctypes.c_int32, ctypes.c_int64, ctypes.c_int32]),
+    "e3j_amd_tile_schedule_build": (ctypes.c_int, [_P] * 4 + [ctypes.c_int32, ctypes.c_int64, ctypes.c_int32,
+                                                              ctypes.c_int32] + [_P] * 6),
+    "e3j_amd_convolution_bwd_tiled": (ctypes.c_int, [_PARAMS] + [_P] * 7 + [ctypes.POINTER(TileSchedule)] + [_P] * 4),
     "e3j_amd_find_signature": (ctypes.c_int, [_P] + [ctypes.c_int32] * 9 + [ctypes.POINTER(ctypes.c_float),
                                                                              ctypes.POINTER(ctypes.c_uint32)]),
     "e3j_amd_num_signatures": (ctypes.c_int, []),

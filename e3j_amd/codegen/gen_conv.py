@@ -53,11 +53,16 @@ BUILTIN_SIGNATURES = [(f"{name}_k{k}", xi, yi, oi, k) for name, xi, yi, oi, ks i
 #: E3J_AMD_FWD_VARIANT / E3J_AMD_BWD_VARIANT (read once) for tuning runs.
 LAUNCH = {
     32: dict(fwd=[(1, 4, 1)], bwd=[(1, 4, 2), (1, 4, 1)]),
-    64: dict(fwd=[(1, 4, 1), (1, 4, 2)], bwd=[(1, 4, 2), (1, 4, 1), (1, 4, 3), (1, 4, 4)]),
+    64: dict(fwd=[(1, 4, 1), (1, 4, 2)], bwd=[(1, 4, 2), (1, 4, 1), (1, 4, 3), (1, 4, 4)],
+             bwd_tile=[(1, 16, 4), (1, 16, 3), (1, 8, 4), (1, 12, 4)]),
     128: dict(fwd=[(1, 4, 1), (1, 4, 2), (2, 4, 2), (2, 4, 4)],
-              bwd=[(2, 4, 3), (1, 4, 1), (1, 4, 3), (1, 4, 4), (2, 4, 4), (1, 4, 2)]),
-    256: dict(fwd=[(1, 4, 1), (1, 4, 2)], bwd=[(2, 4, 3), (1, 4, 2), (1, 4, 3)]),
+              bwd=[(2, 4, 3), (1, 4, 1), (1, 4, 3), (1, 4, 4), (2, 4, 4), (1, 4, 2)],
+              bwd_tile=[(1, 16, 4), (1, 16, 3), (2, 8, 4), (2, 8, 3), (1, 8, 4), (1, 12, 4)]),
+    256: dict(fwd=[(1, 4, 1), (1, 4, 2)], bwd=[(2, 4, 3), (1, 4, 2), (1, 4, 3)],
+              bwd_tile=[(1, 16, 4), (2, 8, 4)]),
 }
+#: `bwd_tile`: variants of the backward over tiles of receivers (trailing layout, at least 64
+#: channels): a block of `waves per block` waves shares the dm rows of a tile in LDS.
 
 
 #: leading-channels layout: (waves per block, parts) variants.  The forward pass is never
@@ -251,9 +256,10 @@ def emit_edge_bwd(p: Part) -> list[str]:
     """
     t = p.t
     lines = ["    // dx (this part's x rows) and dy (all Y) are written here; ds rows go to `ds` path by path.",
-             "    template <int C, typename DsSink>",
+             "    // `dm`: anything indexable by the part's local output row (registers or LDS).",
+             "    template <int C, typename Dm, typename DsSink>",
              "    __device__ static __forceinline__ void edge_bwd(const Vec<C> *x, const float *y,",
-             "                                                     const Vec<C> *s, const Vec<C> *dm,",
+             "                                                     const Vec<C> *s, const Dm &dm,",
              "                                                     Vec<C> *dx, float *dy, const DsSink &ds) {"]
     dx_init, dy_init = set(), set()
     for l, rows in p.paths.items():
@@ -267,7 +273,8 @@ def emit_edge_bwd(p: Part) -> list[str]:
         for i, cols in rows.items():
             zi = p.zi[i]
             lines.append("            {")
-            lines.append(f"                const Vec<C> g = vmulv(dm[{zi}], s[{p.sl[l]}]);")
+            lines.append(f"                const Vec<C> dmi = dm[{zi}];")
+            lines.append(f"                const Vec<C> g = vmulv(dmi, s[{p.sl[l]}]);")
             for j, terms in cols.items():
                 xj = p.xj[j]
                 expr, bare = Table.weight_expr(terms, ids)
@@ -279,7 +286,7 @@ def emit_edge_bwd(p: Part) -> list[str]:
                 else:
                     lines.append(f"                dx[{xj}] = vmul(g, {expr});")
                     dx_init.add(j)
-                lines.append(f"                {{ const Vec<C> pr = vmulv(dm[{zi}], x[{xj}]);")
+                lines.append(f"                {{ const Vec<C> pr = vmulv(dmi, x[{xj}]);")
                 for c, k in terms:
                     if k in a_init:
                         lines.append(f"                  a{k} = vfma(pr, {_lit(c)}, a{k});")
@@ -347,9 +354,9 @@ def emit_signature(sig_id: int, name: str, x_irreps: str, y_irreps: str, out_fil
 def plugin_launch(channels: int):
     """Launch shapes of a signature compiled at run time: the default variant of each pass."""
     if channels % 128 == 0:
-        trailing = dict(fwd=[(1, 4, 1)], bwd=[(2, 4, 3)])
+        trailing = dict(fwd=[(1, 4, 1)], bwd=[(2, 4, 3)], bwd_tile=[LAUNCH[128]["bwd_tile"][0]])
     elif channels % 64 == 0:
-        trailing = dict(fwd=[(1, 4, 1)], bwd=[(1, 4, 2)])
+        trailing = dict(fwd=[(1, 4, 1)], bwd=[(1, 4, 2)], bwd_tile=[LAUNCH[64]["bwd_tile"][0]])
     else:
         trailing = dict(fwd=[(1, 4, 1)], bwd=[(1, 4, 2)])
     width = min(channels, 64)
@@ -386,7 +393,8 @@ def emit_table_source(t: "Table", name: str, desc: str, channels: int, symbols, 
     ]
     if lead == "builtin":
         lead = LAUNCH_LEADING[channels] if (t.X <= 64 and t.S <= 64) else None
-    splits = sorted({v[2] for v in launch["fwd"] + launch["bwd"]} |
+    tile = launch.get("bwd_tile", [])
+    splits = sorted({v[2] for v in launch["fwd"] + launch["bwd"] + tile} |
                     ({v[1] for v in lead["fwd"] + lead["bwd"]} if lead else set()))
     part_names = {}
     for zs in splits:
@@ -411,6 +419,13 @@ def emit_table_source(t: "Table", name: str, desc: str, channels: int, symbols, 
         for ordered in ("false", "true"):
             out += [f"template __global__ void unrolled_bwd_kernel<{channels}, {cpl}, {wpb}, {minw}, {ordered}, "
                     f"{part_names[zs]}>("] + bwd_args
+    tile_args = ["    const float *, const float *, const float *, const float *, const int32_t *,",
+                 "    const int32_t *, const int32_t *, const int32_t *, const int32_t *, float *, float *, float *,",
+                 "    int, int, int, float, unsigned, unsigned);"]
+    for v in tile:
+        cpl, wpb, zs, minw = (*v, 1)[:4]
+        out += [f"template __global__ void unrolled_bwd_tile_kernel<{channels}, {cpl}, {wpb}, {minw}, "
+                f"{part_names[zs]}>("] + tile_args
     if lead:
         for wpb, zs in lead["fwd"]:
             out += [f"template __global__ void unrolled_fwd_leading_kernel<{channels}, {wpb}, {part_names[zs]}>("] + fwd_args
@@ -447,10 +462,21 @@ def emit_table_source(t: "Table", name: str, desc: str, channels: int, symbols, 
     out += [ln.replace("VARIANT", "tuning().bwd_variant") for ln in switch(
         launch["bwd"], lambda v: f"launch_unrolled_bwd<{channels}, {v[0]}, {v[1]}, {(*v, 1)[3]}, {t.Y}, {t.X}, "
                                  f"{part_names[v[2]]}>(p, x, y, s, dm, sender, row_ptr, perm, dx, dy, ds, stream, ordered);")]
+    if tile:
+        out += ["static int run_bwd_tiled(const e3j_amd_conv_params &p, const float *x, const float *y,",
+                "                         const float *s, const float *dm, const e3j_amd_tile_schedule &schedule,",
+                "                         float *dx, float *dy, float *ds, hipStream_t stream) {"]
+        out += [ln.replace("VARIANT", "tuning().bwd_variant") for ln in switch(
+            tile, lambda v: f"launch_unrolled_bwd_tile<{channels}, {v[0]}, {v[1]}, {(*v, 1)[3]}, {t.Y}, {t.X}, "
+                            f"{part_names[v[2]]}>(p, x, y, s, dm, schedule, dx, dy, ds, stream);")]
+        out += ["static int run_tile_row_bytes() {"]
+        out += [ln.replace("VARIANT", "tuning().bwd_variant") for ln in switch(
+            tile, lambda v: f"tile_row_bytes<{v[0]}, {part_names[v[2]]}>();")]
+    tiled = "&run_bwd_tiled, &run_tile_row_bytes" if tile else "nullptr, nullptr"
     out += [f"extern const Signature {symbols[0]} = {{",
             f'    "{desc}",',
             f"    {t.X}, {t.Y}, {t.Z}, {t.S}, {len(t.val)}, {channels}, E3J_AMD_LAYOUT_TRAILING, kVal, kIdx,",
-            "    &run_fwd, &run_bwd,",
+            f"    &run_fwd, &run_bwd, {tiled},",
             "};", ""]
     if lead:
         out += ["static int run_fwd_leading" + fwd_sig[0]] + fwd_sig[1:]
@@ -464,12 +490,12 @@ def emit_table_source(t: "Table", name: str, desc: str, channels: int, symbols, 
         out += [f"extern const Signature {symbols[1]} = {{",
                 f'    "{desc.replace("trailing", "leading")}",',
                 f"    {t.X}, {t.Y}, {t.Z}, {t.S}, {len(t.val)}, {channels}, E3J_AMD_LAYOUT_LEADING, kVal, kIdx,",
-                "    &run_fwd_leading, &run_bwd_leading,",
+                "    &run_fwd_leading, &run_bwd_leading, nullptr, nullptr,",
                 "};"]
     else:  # no leading-layout kernels: an entry that never matches keeps the numbering regular
         out += [f"extern const Signature {symbols[1]} = {{",
                 f'    "{desc.replace("trailing", "leading (not built)")}",',
-                "    -1, -1, -1, -1, -1, -1, E3J_AMD_LAYOUT_LEADING, nullptr, nullptr, nullptr, nullptr,",
+                "    -1, -1, -1, -1, -1, -1, E3J_AMD_LAYOUT_LEADING, nullptr, nullptr, nullptr, nullptr, nullptr, nullptr,",
                 "};"]
     if plugin:
         out += ["",

@@ -31,7 +31,8 @@ int check_hip(hipError_t err, const char *what) {
 namespace {
 Tuning &mutable_tuning() {
     static Tuning t = [] {
-        Tuning v{0, 0};
+        Tuning v{0, 0, 0};
+        if (const char *e = std::getenv("E3J_AMD_TILE_DEBUG")) v.tile_debug = std::atoi(e);
         if (const char *e = std::getenv("E3J_AMD_FWD_VARIANT")) v.fwd_variant = std::atoi(e);
         if (const char *e = std::getenv("E3J_AMD_BWD_VARIANT")) v.bwd_variant = std::atoi(e);
         return v;
@@ -180,7 +181,7 @@ int e3j_amd_register_signature(const void *entry) {
 }
 
 void e3j_amd_set_launch_variant(int32_t fwd_variant, int32_t bwd_variant) {
-    mutable_tuning() = Tuning{fwd_variant, bwd_variant};
+    mutable_tuning() = Tuning{fwd_variant, bwd_variant, mutable_tuning().tile_debug};
 }
 
 int e3j_amd_convolution_fwd(const e3j_amd_conv_params *p, const void *coef, const void *x,
@@ -306,6 +307,49 @@ int e3j_amd_convolution_bwd_ordered(const e3j_amd_conv_params *p, const void *co
         rc = reduce_ordered_dx(*p, ordered.u, sender_ptr, pos, ordered.covered, static_cast<float *>(dx), stream);
     if (rc == E3J_AMD_OK && ordered.slots > 1)
         rc = reduce_ordered_dy(*p, ordered.dy_slots, ordered.slots, edge_perm, static_cast<float *>(dy), stream);
+    if (rc == E3J_AMD_OK)
+        rc = launch_zero_padding(*p, sender, receiver_ptr, edge_perm, static_cast<float *>(dy),
+                                 static_cast<float *>(ds), stream);
+    return finish(p, stream, rc, op);
+}
+
+int32_t e3j_amd_tile_rows(int32_t sig) {
+    if (sig < 0 || sig >= num_signatures()) return 0;
+    const Signature &sg = signature(sig);
+    if (sg.bwd_tiled == nullptr || sg.tile_row_bytes == nullptr) return 0;
+    const int bytes = sg.tile_row_bytes();
+    return bytes > 0 ? (int32_t)(160 * 1024 / bytes) : 0;
+}
+
+int e3j_amd_convolution_bwd_tiled(const e3j_amd_conv_params *p, const void *x, const void *y,
+                                  const void *s, const void *dm, const int32_t *sender,
+                                  const int32_t *receiver_ptr, const int32_t *edge_perm,
+                                  const e3j_amd_tile_schedule *schedule, void *dx, void *dy, void *ds,
+                                  void *stream_) {
+    const char *op = "convolution_bwd_tiled";
+    int rc = validate(p, op);
+    if (rc) return rc;
+    hipStream_t stream = static_cast<hipStream_t>(stream_);
+    if (p->num_nodes == 0 && p->num_edges == 0) return E3J_AMD_OK;
+    if (missing(x, p->num_nodes) || missing(dm, p->num_nodes) || missing(dx, p->num_nodes) ||
+        receiver_ptr == nullptr || missing(sender, p->num_edges) || missing(y, p->num_edges) ||
+        missing(s, p->num_edges) || missing(dy, p->num_edges) || missing(ds, p->num_edges) ||
+        schedule == nullptr)
+        return set_error(E3J_AMD_INVALID_ARGUMENT, std::string(op) + ": null operand");
+    if (p->num_nodes == 0) return E3J_AMD_OK;
+    if (p->signature < 0 || signature(p->signature).bwd_tiled == nullptr)
+        return set_error(E3J_AMD_UNIMPLEMENTED,
+                         std::string(op) + ": needs a compile-time-unrolled kernel of the trailing layout "
+                                           "with at least 64 channels; e3j_amd_convolution_bwd_receiver "
+                                           "serves the other cases");
+    if (schedule->num_work < 0 || (schedule->num_work > 0 && schedule->work == nullptr) ||
+        missing(schedule->sender, p->num_edges) || missing(schedule->edge, p->num_edges) ||
+        missing(schedule->local, p->num_edges))
+        return set_error(E3J_AMD_INVALID_ARGUMENT, std::string(op) + ": incomplete schedule");
+    rc = signature(p->signature).bwd_tiled(*p, static_cast<const float *>(x), static_cast<const float *>(y),
+                                           static_cast<const float *>(s), static_cast<const float *>(dm),
+                                           *schedule, static_cast<float *>(dx), static_cast<float *>(dy),
+                                           static_cast<float *>(ds), stream);
     if (rc == E3J_AMD_OK)
         rc = launch_zero_padding(*p, sender, receiver_ptr, edge_perm, static_cast<float *>(dy),
                                  static_cast<float *>(ds), stream);

@@ -97,6 +97,7 @@ int launch_zero_padding(const e3j_amd_conv_params &p, const int32_t *other, cons
 struct Tuning {
     int fwd_variant;
     int bwd_variant;
+    int tile_debug;
 };
 const Tuning &tuning();
 
@@ -141,6 +142,11 @@ struct Signature {
                const float *dm, const int32_t *sender, const int32_t *receiver_ptr,
                const int32_t *edge_perm, float *dx, float *dy, float *ds, hipStream_t stream,
                OrderedBwd *ordered);  // ordered: nullptr = dx (and shared dy) by float atomics
+    // backward over tiles of receivers (nullptr: none) and the LDS bytes it needs per tile row
+    int (*bwd_tiled)(const e3j_amd_conv_params &p, const float *x, const float *y, const float *s,
+                     const float *dm, const e3j_amd_tile_schedule &schedule, float *dx, float *dy,
+                     float *ds, hipStream_t stream);
+    int (*tile_row_bytes)();
 };
 // built-in signatures (generated/registry.hip), then the ones registered at run time (capi.hip)
 int num_builtin_signatures();

@@ -159,6 +159,122 @@ __global__ void live_keys_kernel(const int32_t *__restrict__ other, const int32_
     }
 }
 
+
+// ---- schedule of the backward over tiles of receivers ---------------------------------------
+// Tiles are `tile_rows` consecutive entries of the row order.  Every CSR position gets the key
+// (tile, sender) with padding senders after the live ones; a radix sort of the positions by that
+// key lists each tile's edges in sender order.
+
+__global__ void tile_rank_kernel(const int32_t *__restrict__ row_order, int num_nodes,
+                                 int32_t *__restrict__ rank) {
+    const int q = blockIdx.x * blockDim.x + threadIdx.x;
+    if (q >= num_nodes) return;
+    rank[row_order ? row_order[q] : q] = q;
+}
+
+// counts[t + 1] = positions of tile t; pieces[t + 1] = work descriptors it is cut into
+__global__ void tile_count_kernel(const int32_t *__restrict__ row_order, const int32_t *__restrict__ row_ptr,
+                                  int num_nodes, int tile_rows, int num_tiles, int max_work_edges,
+                                  int32_t *__restrict__ counts, int32_t *__restrict__ pieces) {
+    const int t = blockIdx.x * blockDim.x + threadIdx.x;
+    if (t == 0) counts[0] = pieces[0] = 0;
+    if (t >= num_tiles) return;
+    int total = 0;
+    for (int q = t * tile_rows; q < (t + 1) * tile_rows && q < num_nodes; q++) {
+        const int r = row_order ? row_order[q] : q;
+        total += row_ptr[r + 1] - row_ptr[r];
+    }
+    counts[t + 1] = total;
+    pieces[t + 1] = total == 0 ? 1 : (total + max_work_edges - 1) / max_work_edges;
+}
+
+__global__ void tile_keys_kernel(const int32_t *__restrict__ other, const int32_t *__restrict__ row_ptr,
+                                 const int32_t *__restrict__ rank, int num_nodes, int64_t num_edges,
+                                 int tile_rows, int sender_bits, uint64_t sentinel, uint64_t *__restrict__ keys,
+                                 int32_t *__restrict__ vals, int32_t *__restrict__ local) {
+    const int64_t live_end = row_ptr[num_nodes];
+    const int64_t stride = (int64_t)gridDim.x * blockDim.x;
+    for (int64_t pos = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; pos < num_edges; pos += stride) {
+        vals[pos] = (int32_t)pos;
+        if (pos >= live_end) {  // past the last row: belongs to no tile
+            keys[pos] = sentinel;
+            local[pos] = 0;
+            continue;
+        }
+        // the row of the position: last r with row_ptr[r] <= pos (empty rows share their start)
+        int lo = 0, hi = num_nodes;  // invariant: row_ptr[lo] <= pos < row_ptr[hi]
+        while (hi - lo > 1) {
+            const int mid = (lo + hi) >> 1;
+            if (row_ptr[mid] <= pos) lo = mid; else hi = mid;
+        }
+        const int q = rank[lo];
+        const int32_t snd = other[pos];
+        const uint64_t sk = (unsigned)snd < (unsigned)num_nodes ? (uint64_t)snd : (uint64_t)num_nodes;
+        keys[pos] = ((uint64_t)(q / tile_rows) << sender_bits) | sk;
+        local[pos] = q % tile_rows;
+    }
+}
+
+__global__ void tile_entries_kernel(const uint64_t *__restrict__ keys, const int32_t *__restrict__ vals,
+                                    const int32_t *__restrict__ local, const int32_t *__restrict__ perm,
+                                    int num_nodes, int64_t num_edges, int sender_bits, uint64_t sentinel,
+                                    int32_t *__restrict__ t_sender, int32_t *__restrict__ t_edge,
+                                    int32_t *__restrict__ t_local) {
+    const int64_t stride = (int64_t)gridDim.x * blockDim.x;
+    for (int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; i < num_edges; i += stride) {
+        const uint64_t key = keys[i];
+        const int32_t pos = vals[i];
+        if (key == sentinel) {
+            t_sender[i] = -1; t_edge[i] = 0; t_local[i] = 0;
+            continue;
+        }
+        const uint64_t sk = key & ((1ull << sender_bits) - 1);
+        t_sender[i] = sk == (uint64_t)num_nodes ? -1 : (int32_t)sk;
+        t_edge[i] = perm ? perm[pos] : pos;
+        t_local[i] = local[pos];
+    }
+}
+
+// descriptors (tile, begin, end, 0); `starts` / `first_piece`: inclusive prefix sums, entry 0 = 0
+__global__ void tile_work_kernel(const int32_t *__restrict__ starts, const int32_t *__restrict__ first_piece,
+                                 int num_tiles, int max_work_edges, int32_t *__restrict__ work) {
+    const int t = blockIdx.x * blockDim.x + threadIdx.x;
+    if (t >= num_tiles) return;
+    const int begin = starts[t], end = starts[t + 1];
+    int w = first_piece[t];
+    for (int b = begin; b < end; b += max_work_edges, w++) {
+        work[4 * w] = t;
+        work[4 * w + 1] = b;
+        work[4 * w + 2] = b + max_work_edges < end ? b + max_work_edges : end;
+        work[4 * w + 3] = 0;
+    }
+}
+
+size_t sort64_temp_bytes(int64_t num_edges) {
+    size_t bytes = 0;
+    hipcub::DeviceRadixSort::SortPairs(nullptr, bytes, (const uint64_t *)nullptr, (uint64_t *)nullptr,
+                                       (const int32_t *)nullptr, (int32_t *)nullptr, (int)num_edges);
+    return bytes;
+}
+
+struct TileWorkspace {
+    size_t temp, temp_bytes, keys_in, keys_out, vals_in, vals_out, local, rank, counts, pieces, total;
+    TileWorkspace(int32_t num_nodes, int64_t num_edges, int32_t tile_rows) {
+        const size_t e = (size_t)num_edges, n = (size_t)num_nodes;
+        const size_t tiles = (n + (size_t)tile_rows - 1) / (size_t)tile_rows;
+        size_t at = 0;
+        auto take = [&](size_t bytes) { const size_t here = at; at += align_up(bytes); return here; };
+        temp_bytes = std::max(sort64_temp_bytes(num_edges), scan_temp_bytes((int32_t)tiles));
+        temp = take(temp_bytes);
+        keys_in = take(8 * e); keys_out = take(8 * e);
+        vals_in = take(4 * e); vals_out = take(4 * e);
+        local = take(4 * e);
+        rank = take(4 * n);
+        counts = take(4 * (tiles + 1)); pieces = take(4 * (tiles + 1));
+        total = at;
+    }
+};
+
 }  // namespace
 
 int launch_live_keys(const int32_t *other, const int32_t *row_ptr, int32_t num_nodes,
@@ -272,6 +388,87 @@ int e3j_amd_locality_order(const int32_t *other, const int32_t *row_ptr, int32_t
     hipLaunchKernelGGL(copy_i32_kernel, dim3(ngrid), dim3(256), 0, stream, order_tmp, order,
                        (int64_t)num_nodes);
     return check_hip(hipGetLastError(), "locality_order");
+}
+
+int64_t e3j_amd_tile_schedule_num_work(int32_t num_nodes, int64_t num_edges, int32_t tile_rows,
+                                       int32_t max_work_edges) {
+    if (num_nodes < 0 || num_edges < 0 || tile_rows < 1 || max_work_edges < 1) return 0;
+    const int64_t tiles = ((int64_t)num_nodes + tile_rows - 1) / tile_rows;
+    return tiles + num_edges / max_work_edges;  // sum over tiles of max(1, ceil(count / max)) at most
+}
+
+size_t e3j_amd_tile_schedule_workspace_bytes(int32_t num_nodes, int64_t num_edges, int32_t tile_rows) {
+    if (num_nodes < 0 || num_edges < 0 || tile_rows < 1) return 0;
+    return TileWorkspace(num_nodes, num_edges, tile_rows).total + 256;
+}
+
+int e3j_amd_tile_schedule_build(const int32_t *other, const int32_t *row_ptr, const int32_t *edge_perm,
+                                const int32_t *row_order, int32_t num_nodes, int64_t num_edges,
+                                int32_t tile_rows, int32_t max_work_edges, int32_t *work,
+                                int32_t *t_sender, int32_t *t_edge, int32_t *t_local, void *workspace,
+                                void *stream_) {
+    if (num_nodes < 0 || num_edges < 0 || num_edges > 0x7fffffffLL || tile_rows < 1 || max_work_edges < 1)
+        return set_error(E3J_AMD_INVALID_ARGUMENT, "tile_schedule_build: bad sizes");
+    if (num_nodes == 0) return E3J_AMD_OK;
+    if (row_ptr == nullptr || work == nullptr || workspace == nullptr ||
+        (num_edges > 0 && (other == nullptr || t_sender == nullptr || t_edge == nullptr || t_local == nullptr)))
+        return set_error(E3J_AMD_INVALID_ARGUMENT, "tile_schedule_build: null operand");
+    hipStream_t stream = static_cast<hipStream_t>(stream_);
+    unsigned char *ws = static_cast<unsigned char *>(workspace);
+    ws += (256 - reinterpret_cast<uintptr_t>(ws) % 256) % 256;
+    const TileWorkspace w(num_nodes, num_edges, tile_rows);
+    uint64_t *keys_in = reinterpret_cast<uint64_t *>(ws + w.keys_in);
+    uint64_t *keys_out = reinterpret_cast<uint64_t *>(ws + w.keys_out);
+    int32_t *vals_in = reinterpret_cast<int32_t *>(ws + w.vals_in);
+    int32_t *vals_out = reinterpret_cast<int32_t *>(ws + w.vals_out);
+    int32_t *local = reinterpret_cast<int32_t *>(ws + w.local);
+    int32_t *rank = reinterpret_cast<int32_t *>(ws + w.rank);
+    int32_t *counts = reinterpret_cast<int32_t *>(ws + w.counts);
+    int32_t *pieces = reinterpret_cast<int32_t *>(ws + w.pieces);
+    const int num_tiles = (num_nodes + tile_rows - 1) / tile_rows;
+    const int64_t num_work = e3j_amd_tile_schedule_num_work(num_nodes, num_edges, tile_rows, max_work_edges);
+    const unsigned rows_grid = (unsigned)((num_nodes + 255) / 256);
+    const unsigned tiles_grid = (unsigned)((num_tiles + 255) / 256);
+
+    int rc = launch_fill_zero(work, sizeof(int32_t) * 4 * (size_t)num_work, stream);
+    if (rc) return rc;
+    hipLaunchKernelGGL(tile_rank_kernel, dim3(rows_grid), dim3(256), 0, stream, row_order, num_nodes, rank);
+    hipLaunchKernelGGL(tile_count_kernel, dim3(tiles_grid), dim3(256), 0, stream, row_order, row_ptr, num_nodes,
+                       tile_rows, num_tiles, max_work_edges, counts, pieces);
+    rc = check_hip(hipGetLastError(), "tile schedule counts");
+    if (rc) return rc;
+    size_t temp_bytes = w.temp_bytes;
+    rc = check_hip(hipcub::DeviceScan::InclusiveSum(ws + w.temp, temp_bytes, counts, counts, num_tiles + 1, stream),
+                   "tile schedule scan");
+    if (rc) return rc;
+    temp_bytes = w.temp_bytes;
+    rc = check_hip(hipcub::DeviceScan::InclusiveSum(ws + w.temp, temp_bytes, pieces, pieces, num_tiles + 1, stream),
+                   "tile schedule scan");
+    if (rc) return rc;
+    hipLaunchKernelGGL(tile_work_kernel, dim3(tiles_grid), dim3(256), 0, stream, counts, pieces, num_tiles,
+                       max_work_edges, work);
+    rc = check_hip(hipGetLastError(), "tile schedule work");
+    if (rc || num_edges == 0) return rc;
+
+    // key = tile << sender_bits | sender, padding senders as num_nodes; sentinel above every live key
+    int sender_bits = 1;
+    while (((uint64_t)num_nodes >> sender_bits) != 0) sender_bits++;
+    const uint64_t sentinel = (uint64_t)num_tiles << sender_bits;
+    int end_bit = sender_bits + 1;
+    while (end_bit < 64 && (sentinel >> end_bit) != 0) end_bit++;
+    const int begin_bit = (tuning().tile_debug & 4) ? sender_bits : 0;
+    hipLaunchKernelGGL(tile_keys_kernel, dim3(grid_for(num_edges)), dim3(256), 0, stream, other, row_ptr, rank,
+                       num_nodes, num_edges, tile_rows, sender_bits, sentinel, keys_in, vals_in, local);
+    rc = check_hip(hipGetLastError(), "tile schedule keys");
+    if (rc) return rc;
+    temp_bytes = w.temp_bytes;
+    rc = check_hip(hipcub::DeviceRadixSort::SortPairs(ws + w.temp, temp_bytes, keys_in, keys_out, vals_in, vals_out,
+                                                      (int)num_edges, begin_bit, end_bit, stream),
+                   "tile schedule sort");
+    if (rc) return rc;
+    hipLaunchKernelGGL(tile_entries_kernel, dim3(grid_for(num_edges)), dim3(256), 0, stream, keys_out, vals_out,
+                       local, edge_perm, num_nodes, num_edges, sender_bits, sentinel, t_sender, t_edge, t_local);
+    return check_hip(hipGetLastError(), "tile schedule entries");
 }
 
 int e3j_amd_sort_edges(const int32_t *key, const int32_t *other, int64_t num_edges,

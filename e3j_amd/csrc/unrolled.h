@@ -21,6 +21,8 @@
 #ifndef E3J_AMD_CSRC_UNROLLED_H_
 #define E3J_AMD_CSRC_UNROLLED_H_
 
+#include <initializer_list>
+
 #include "common.h"
 
 namespace e3j_amd {
@@ -592,6 +594,213 @@ void unrolled_bwd_kernel(
 }
 
 // ---------------------------------------------------------------------------
+// backward over tiles of receivers: dm rows of the tile resident in LDS, the tile's edges
+// walked in sender order, dx summed in registers over the edges that share a sender
+// ---------------------------------------------------------------------------
+// Float atomics retire per 64-byte request at a fixed rate that bounds the receiver-grouped
+// backward above.  Neighbouring receivers share most of their senders, so a block takes a
+// tile of receivers that are consecutive in the row order (one part of the signature, one
+// channel slice), keeps their dm rows in LDS, and walks the tile's edges sorted by sender
+// (the schedule of `e3j_amd_tile_schedule_build`).  Its waves split that list at sender
+// boundaries; a wave sums the dx contributions of the consecutive edges of one sender in
+// registers and issues one set of atomics per (tile, sender) instead of one per edge, and
+// gathers the sender's x row once.  dm is indexed from LDS by the edge's receiver, which
+// also frees the registers the resident dm rows took.  ds and dy belong to the edge and
+// are written as in the kernel above.  One barrier per block (after the tile is staged).
+
+// The dm rows of one receiver of the tile as the generated arithmetic indexes them.
+template <int CPL>
+struct DmTile {
+    const float *row;  // LDS: this lane's CPL values of the receiver's first staged row
+    __device__ __forceinline__ Vec<CPL> operator[](int i) const {
+        return load_vec<CPL>(row + i * (kWave * CPL));
+    }
+};
+
+template <typename Part, int K, int CPL, bool kAtomicDy>
+__device__ __forceinline__ void unrolled_bwd_tile_part(
+    const float *__restrict__ x, const float *__restrict__ y, const float *__restrict__ s,
+    const float *__restrict__ dm, const int32_t *__restrict__ t_sender,
+    const int32_t *__restrict__ t_edge, const int32_t *__restrict__ t_local,
+    const int32_t *__restrict__ row_order, float *__restrict__ dx, float *__restrict__ dy,
+    float *__restrict__ ds, int num_nodes, float scale, unsigned y_flip, int tile, int tile_rows,
+    int begin, int end, int slice, float *tile_lds, unsigned dbg) {
+    constexpr int NX = Part::NX, NS = Part::NS, NZ = Part::NZ, Y = Part::Y;
+    constexpr int X = Part::X, S = Part::S, Z = Part::Z;
+    using V = Vec<CPL>;
+    using SL = Slice<K, CPL>;
+    using Red = WaveReduceBlocks<Y, kWave>;
+    constexpr int WIDTH = SL::WIDTH;
+    static_assert(SL::SUB == 1, "the tile kernel takes whole waves of channels");
+    static_assert(CPL == 1 || SL::FULL, "several channels per lane need whole slices");
+
+    const int lane = threadIdx.x;
+    const int wave = uniform(threadIdx.y), nw = blockDim.y;
+    const int c_raw = slice * WIDTH + lane;  // further channels of the lane: + 64, + 128, ...
+    const bool active = SL::FULL || c_raw < K;
+    const int c0 = active ? c_raw : 0;
+
+    // stage the dm rows of the tile's receivers (scaled): row (t, i) at (t * NZ + i) * WIDTH
+    {
+        const int first = tile * tile_rows;
+        const int rows = num_nodes - first < tile_rows ? num_nodes - first : tile_rows;
+        for (int t = wave; t < rows; t += nw) {
+            const int r = row_order ? row_order[first + t] : first + t;
+            const float *zr = dm + (int64_t)r * (Z * K) + c0;
+            float *dst = tile_lds + t * (NZ * WIDTH) + lane * CPL;
+            V v[NZ];
+#pragma unroll
+            for (int i = 0; i < NZ; i++) v[i] = load_apart_stream<CPL>(zr + Part::kZ[i] * K);
+#pragma unroll
+            for (int i = 0; i < NZ; i++)  // idle lanes must add nothing to dy
+                store_vec<CPL>(dst + i * WIDTH, active ? vmul(v[i], scale) : vzero<CPL>());
+        }
+    }
+    __syncthreads();
+
+    // this wave's share of the list, cut at sender boundaries
+    auto boundary = [&](int p) {
+        if (p <= begin) return begin;
+        while (p < end && t_sender[p] == t_sender[p - 1]) p++;
+        return p;
+    };
+    const int n = end - begin;
+    const int lo = boundary(begin + (int)((int64_t)n * wave / nw));
+    const int hi = boundary(begin + (int)((int64_t)n * (wave + 1) / nw));
+
+    V xc[NX], xn[NX], sn[NS], acc[NX];
+    float yn[Y];
+    bool valid_n = false, newx_n = false;
+    int snd_n = 0, loc_n = 0;
+    int64_t ee_n = 0;
+    // `held`: the sender whose x row the registers will hold when the fetched edge is computed
+    auto fetch = [&](int pos, int held) {
+        const int snd = t_sender[pos];
+        valid_n = (unsigned)snd < (unsigned)num_nodes;
+        snd_n = snd;
+        ee_n = t_edge[pos];
+        loc_n = t_local[pos];
+        newx_n = valid_n && snd != held;
+        if (newx_n) {
+            const float *xr = x + (int64_t)snd * (X * K) + c0;
+#pragma unroll
+            for (int j = 0; j < NX; j++) xn[j] = load_apart<CPL>(xr + Part::kX[j] * K);
+        }
+        const float *sr = s + ee_n * (int64_t)(S * K) + c0;
+        const float *yr = y + ee_n * Y;
+#pragma unroll
+        for (int l = 0; l < NS; l++) sn[l] = load_apart_stream<CPL>(sr + Part::kS[l] * K);
+#pragma unroll
+        for (int k = 0; k < Y; k++) yn[k] = yr[k];
+    };
+    auto flush = [&](int snd) {
+        if (!active || (dbg & 1u)) return;
+        float *dxr = dx + (int64_t)snd * (X * K) + c0;
+#pragma unroll
+        for (int j = 0; j < NX; j++) {
+#pragma unroll
+            for (int t = 0; t < CPL; t++) unsafeAtomicAdd(dxr + Part::kX[j] * K + t * kWave, acc[j].v[t]);
+        }
+    };
+
+    int held = -1, run = -1;
+    if (lo < hi) fetch(lo, held);
+    for (int pos = lo; pos < hi; pos++) {
+        V sc[NS];
+        float yc[Y];
+        if (newx_n) {
+#pragma unroll
+            for (int j = 0; j < NX; j++) xc[j] = xn[j];
+            held = snd_n;
+        }
+#pragma unroll
+        for (int l = 0; l < NS; l++) sc[l] = sn[l];
+#pragma unroll
+        for (int k = 0; k < Y; k++) yc[k] = to_vgpr(flip_sign(yn[k], y_flip, k));
+        const bool valid = valid_n;
+        const int snd = snd_n, loc = loc_n;
+        const int64_t ee = ee_n;
+        if (pos + 1 < hi) fetch(pos + 1, held);
+        if (!valid) continue;  // padding edge: its dy/ds rows are zero-filled separately
+
+        if (snd != run) {
+            if (run >= 0) flush(run);
+            run = snd;
+#pragma unroll
+            for (int j = 0; j < NX; j++) acc[j] = vzero<CPL>();
+        }
+        V dxe[NX];
+        float dye[Red::P];
+        const DsRows<CPL, K> ds_rows{ds + ee * (int64_t)(S * K) + c0, active && !(dbg & 2u)};
+        const DmTile<CPL> dm_rows{tile_lds + loc * (NZ * WIDTH) + lane * CPL};
+        Part::template edge_bwd<CPL>(xc, yc, sc, dm_rows, dxe, dye, ds_rows);
+#pragma unroll
+        for (int j = 0; j < NX; j++) {
+#pragma unroll
+            for (int t = 0; t < CPL; t++) acc[j].v[t] += dxe[j].v[t];
+        }
+#pragma unroll
+        for (int k = Y; k < Red::P; k++) dye[k] = 0.f;
+        Red::run(dye, lane, [&](int k, float sum) {
+            const float total = flip_sign(sum, y_flip, k);
+            if (dbg & 8u) return;
+            if (!kAtomicDy) dy[ee * Y + k] = total;
+            else unsafeAtomicAdd(dy + ee * Y + k, total);  // dy zero-filled by the launcher
+        });
+    }
+    if (run >= 0) flush(run);
+}
+
+template <int K, int CPL, bool A, int I>
+__device__ __forceinline__ void dispatch_bwd_tile(int, const float *, const float *, const float *,
+                                                  const float *, const int32_t *, const int32_t *,
+                                                  const int32_t *, const int32_t *, float *, float *,
+                                                  float *, int, float, unsigned, int, int, int, int, int,
+                                                  float *, unsigned) {}
+template <int K, int CPL, bool A, int I, typename Part, typename... Rest>
+__device__ __forceinline__ void dispatch_bwd_tile(int part, const float *x, const float *y, const float *s,
+                                                  const float *dm, const int32_t *t_sender,
+                                                  const int32_t *t_edge, const int32_t *t_local,
+                                                  const int32_t *row_order, float *dx, float *dy,
+                                                  float *ds, int num_nodes, float scale, unsigned y_flip,
+                                                  int tile, int tile_rows, int begin, int end, int slice,
+                                                  float *tile_lds, unsigned dbg) {
+    if (part == I)
+        unrolled_bwd_tile_part<Part, K, CPL, A>(x, y, s, dm, t_sender, t_edge, t_local, row_order, dx, dy,
+                                                ds, num_nodes, scale, y_flip, tile, tile_rows, begin, end,
+                                                slice, tile_lds, dbg);
+    else
+        dispatch_bwd_tile<K, CPL, A, I + 1, Rest...>(part, x, y, s, dm, t_sender, t_edge, t_local,
+                                                     row_order, dx, dy, ds, num_nodes, scale, y_flip,
+                                                     tile, tile_rows, begin, end, slice, tile_lds, dbg);
+}
+
+// One block per (work item, channel slice, part); a work item is a piece of one tile's edge list.
+template <int K, int CPL, int WPB, int MINW, typename... Parts>
+__global__ __launch_bounds__(kWave *WPB, MINW) void unrolled_bwd_tile_kernel(
+    const float *__restrict__ x, const float *__restrict__ y, const float *__restrict__ s,
+    const float *__restrict__ dm, const int32_t *__restrict__ work,
+    const int32_t *__restrict__ t_sender, const int32_t *__restrict__ t_edge,
+    const int32_t *__restrict__ t_local, const int32_t *__restrict__ row_order,
+    float *__restrict__ dx, float *__restrict__ dy, float *__restrict__ ds, int num_nodes,
+    int tile_rows, int num_work, float scale, unsigned y_flip, unsigned dbg) {
+    extern __shared__ __attribute__((aligned(16))) float tile_lds[];
+    constexpr int NP = sizeof...(Parts);
+    constexpr int CW = Slice<K, CPL>::COUNT;
+    constexpr bool kAtomicDy = NP * CW > 1;  // several waves add into one dy row
+    const int64_t item = logical_block();
+    if (item >= (int64_t)num_work * (CW * NP)) return;  // whole block: no barrier is left waiting
+    const int part = (int)(item % NP);
+    const int slice = (int)((item / NP) % CW);
+    const int64_t w = item / (NP * CW);
+    const int tile = work[4 * w], begin = work[4 * w + 1], end = work[4 * w + 2];
+    if (begin >= end) return;  // unused descriptor or a tile without edges (uniform over the block)
+    dispatch_bwd_tile<K, CPL, kAtomicDy, 0, Parts...>(part, x, y, s, dm, t_sender, t_edge, t_local,
+                                                      row_order, dx, dy, ds, num_nodes, scale, y_flip,
+                                                      tile, tile_rows, begin, end, slice, tile_lds, dbg);
+}
+
+// ---------------------------------------------------------------------------
 // Leading-channels layout: a row is (channels, dim), so the channels of a wave are one
 // contiguous block of W * dim floats.  The wave moves such a block with coalesced 16-byte
 // accesses and turns it through its private strip of LDS: lane c reads (or writes) the
@@ -1066,6 +1275,46 @@ int launch_unrolled_bwd(const e3j_amd_conv_params &p, const float *x, const floa
                            dim3(kWave, WPB), 0, stream, x, y, s, dm, sender, row_ptr, perm, p.row_order,
                            dx, dy, ds, p.num_nodes, p.coef_scale, p.y_flip);
     return check_hip(hipGetLastError(), "convolution backward launch");
+}
+
+constexpr int max_of(std::initializer_list<int> v) {
+    int m = 0;
+    for (int a : v) m = a > m ? a : m;
+    return m;
+}
+constexpr size_t kMaxTileLds = 160 * 1024;  // LDS of a CU, all of which one block may take
+
+// LDS bytes per receiver of a tile (the part with the most dm rows decides).
+template <int CPL, typename... Parts>
+constexpr int tile_row_bytes() {
+    return max_of({Parts::NZ...}) * kWave * CPL * (int)sizeof(float);
+}
+
+template <int K, int CPL, int WPB, int MINW, int Y, int X, typename... Parts>
+int launch_unrolled_bwd_tile(const e3j_amd_conv_params &p, const float *x, const float *y, const float *s,
+                             const float *dm, const e3j_amd_tile_schedule &sch, float *dx, float *dy,
+                             float *ds, hipStream_t stream) {
+    constexpr int64_t PER_WORK = (int64_t)Slice<K, CPL>::COUNT * sizeof...(Parts);
+    constexpr unsigned long long kCovered = (Parts::kDxMask | ...);
+    const size_t lds = (size_t)tile_row_bytes<CPL, Parts...>() * (size_t)sch.tile_rows;
+    if (sch.tile_rows < 1 || lds > kMaxTileLds)
+        return set_error(E3J_AMD_INVALID_ARGUMENT,
+                         "convolution_bwd_tiled: the schedule's tiles hold more receivers than fit the LDS "
+                         "(e3j_amd_tile_rows gives the limit)");
+    int rc = prepare_bwd_targets<X, Y, (int)PER_WORK, kCovered>(p, nullptr, K, dx, dy, stream);
+    if (rc) return rc;
+    const int64_t blocks = padded_grid((int64_t)sch.num_work * PER_WORK);
+    if (blocks > 0x7fffffffLL) return set_error(E3J_AMD_INVALID_ARGUMENT, "convolution_bwd_tiled: grid too large");
+    if (blocks == 0) return E3J_AMD_OK;
+    auto kernel = unrolled_bwd_tile_kernel<K, CPL, WPB, MINW, Parts...>;
+    rc = check_hip(hipFuncSetAttribute(reinterpret_cast<const void *>(kernel),
+                                       hipFuncAttributeMaxDynamicSharedMemorySize, (int)kMaxTileLds),
+                   "hipFuncSetAttribute(bwd_tiled)");
+    if (rc) return rc;
+    hipLaunchKernelGGL(kernel, dim3((unsigned)blocks), dim3(kWave, WPB), lds, stream, x, y, s, dm, sch.work,
+                       sch.sender, sch.edge, sch.local, p.row_order, dx, dy, ds, p.num_nodes, sch.tile_rows,
+                       sch.num_work, p.coef_scale, p.y_flip, (unsigned)tuning().tile_debug);
+    return check_hip(hipGetLastError(), "convolution backward (tiled) launch");
 }
 
 template <int K, int WPB, typename Part>

@@ -104,6 +104,43 @@ def locality_order(other: torch.Tensor, row_ptr: torch.Tensor, num_nodes: int,
     return order
 
 
+#: edge positions per work item of the tiled backward: longer tile lists (hub rows) are cut
+#: into pieces of this many positions, each taken by a workgroup of its own
+MAX_WORK_EDGES = 2048
+
+
+class TileSchedule:
+    """Schedule of the backward over tiles of receivers (`e3j_amd_tile_schedule`).
+
+    The edge positions of every tile of `tile_rows` receivers (consecutive in `row_order`),
+    sorted by sender, and the work descriptors that hand them to the workgroups.  Built on
+    the device; holds the buffers the C struct points to.
+    """
+
+    def __init__(self, other: torch.Tensor, row_ptr: torch.Tensor, perm, row_order, num_nodes: int,
+                 tile_rows: int, max_work_edges: int = MAX_WORK_EDGES):
+        device = _require_device(other, row_ptr)
+        lib = _lib.load()
+        num_edges = int(other.numel())
+        self.tile_rows = int(tile_rows)
+        self.num_work = int(lib.e3j_amd_tile_schedule_num_work(num_nodes, num_edges, tile_rows, max_work_edges))
+        self.work = torch.empty((max(self.num_work, 1), 4), dtype=INDEX_DTYPE, device=device)
+        self.sender = torch.empty(num_edges, dtype=INDEX_DTYPE, device=device)
+        self.edge = torch.empty(num_edges, dtype=INDEX_DTYPE, device=device)
+        self.local = torch.empty(num_edges, dtype=INDEX_DTYPE, device=device)
+        nbytes = int(lib.e3j_amd_tile_schedule_workspace_bytes(num_nodes, num_edges, tile_rows))
+        ws = torch.empty(max(nbytes, 256), dtype=torch.uint8, device=device)
+        with torch.cuda.device(device):
+            _lib.check(lib.e3j_amd_tile_schedule_build(
+                other.data_ptr(), row_ptr.data_ptr(), perm.data_ptr() if perm is not None else None,
+                row_order.data_ptr() if row_order is not None else None, num_nodes, num_edges,
+                self.tile_rows, int(max_work_edges), self.work.data_ptr(), self.sender.data_ptr(),
+                self.edge.data_ptr(), self.local.data_ptr(), ws.data_ptr(), _stream_ptr(device)))
+        self.struct = _lib.TileSchedule(
+            tile_rows=self.tile_rows, num_work=self.num_work, work=self.work.data_ptr(),
+            sender=self.sender.data_ptr(), edge=self.edge.data_ptr(), local=self.local.data_ptr())
+
+
 class GraphCSR:
     """Edges grouped by receiver (`src/e3j/data/graph.py:38-73`)."""
 

@@ -25,7 +25,7 @@ import torch
 
 from . import _lib
 from .coef import Coef4D
-from .graph import (csr_row_ptr, fold_endpoints, locality_order,
+from .graph import (TileSchedule, csr_row_ptr, fold_endpoints, locality_order,
                     sort_edges, wrap_global_index)
 from .options import GraphOrdering, Layout, config
 
@@ -228,6 +228,29 @@ def _forward_graph(meta: _Meta, sender: torch.Tensor, receiver: torch.Tensor, bu
     return graph
 
 
+class _Graph:
+    """A prepared adjacency: CSR (`other`, `row_ptr`), optional permutation of the edge rows,
+    row order and, built on first use, the schedules of the tiled backward."""
+
+    def __init__(self, other, row_ptr, perm, order, num_nodes: int):
+        self.other, self.row_ptr, self.perm, self.order = other, row_ptr, perm, order
+        self.num_nodes = int(num_nodes)
+        self._schedules = {}
+
+    def __iter__(self):
+        return iter((self.other, self.row_ptr, self.perm, self.order))
+
+    def __getitem__(self, i):
+        return (self.other, self.row_ptr, self.perm, self.order)[i]
+
+    def schedule(self, tile_rows: int) -> TileSchedule:
+        hit = self._schedules.get(tile_rows)
+        if hit is None:
+            hit = self._schedules[tile_rows] = TileSchedule(self.other, self.row_ptr, self.perm, self.order,
+                                                            self.num_nodes, tile_rows)
+        return hit
+
+
 def _prepare_graph(meta: _Meta, sender: torch.Tensor, receiver: torch.Tensor):
     n = meta.num_nodes
     sender_l, receiver_l = wrap_global_index(sender, n), wrap_global_index(receiver, n)
@@ -238,7 +261,7 @@ def _prepare_graph(meta: _Meta, sender: torch.Tensor, receiver: torch.Tensor):
         other, row_ptr, perm = receiver_l.contiguous(), csr_row_ptr(sender_l, n), None
     else:
         perm, other, row_ptr = sort_edges(receiver_l, sender_l, n)
-    return other, row_ptr, perm, _row_order(other, row_ptr, n)
+    return _Graph(other, row_ptr, perm, _row_order(other, row_ptr, n), n)
 
 
 def _raw_forward(meta: _Meta, x, y, s, sender, receiver, graph=None) -> torch.Tensor:
@@ -284,9 +307,12 @@ def _raw_backward(meta: _Meta, x, y, s, dm, sender, receiver, graph=None):
     forward_rows = meta.ordering != GraphOrdering.SENDER   # the forward's rows are receivers
     reuse = graph is not None and (
         (forward_rows and (not deterministic or ordered)) or sender_rows)
+    prepared = None  # the receiver-grouped adjacency as an object that keeps tile schedules
     if reuse:
         other, row_ptr, perm, order = graph
         group_receiver = not sender_rows
+        if isinstance(graph, _Graph) and group_receiver:
+            prepared = graph
     else:
         sender_l, receiver_l = wrap_global_index(sender, n), wrap_global_index(receiver, n)
         if sender_rows:
@@ -306,8 +332,20 @@ def _raw_backward(meta: _Meta, x, y, s, dm, sender, receiver, graph=None):
             s.data_ptr(), dm.data_ptr(), other.data_ptr(), row_ptr.data_ptr(),
             perm.data_ptr() if perm is not None else None,
             dx.data_ptr(), dy.data_ptr(), ds.data_ptr())
+    # tiles of receivers whose dm rows fit the LDS of a workgroup: dx summed per (tile, sender)
+    tile_rows = 0
+    if group_receiver and not ordered and p.signature >= 0 and y.shape[0] > 0:
+        tile_rows = min(int(config().tile_rows), int(lib.e3j_amd_tile_rows(p.signature)))
     with torch.cuda.device(x.device):
-        if ordered:
+        if tile_rows >= 2:
+            if prepared is None:
+                prepared = _Graph(other, row_ptr, perm, order, n)
+            schedule = prepared.schedule(tile_rows)
+            _lib.check(lib.e3j_amd_convolution_bwd_tiled(
+                ctypes.byref(p), x.data_ptr(), y.data_ptr(), s.data_ptr(), dm.data_ptr(), other.data_ptr(),
+                row_ptr.data_ptr(), perm.data_ptr() if perm is not None else None,
+                ctypes.byref(schedule.struct), dx.data_ptr(), dy.data_ptr(), ds.data_ptr(), _stream(x.device)))
+        elif ordered:
             nbytes = int(lib.e3j_amd_convolution_bwd_ordered_workspace_bytes(ctypes.byref(p)))
             workspace = torch.empty(nbytes, dtype=torch.uint8, device=x.device)
             _lib.check(lib.e3j_amd_convolution_bwd_ordered(*args, workspace.data_ptr(), _stream(x.device)))

@@ -128,6 +128,49 @@ int e3j_amd_convolution_bwd_ordered(const e3j_amd_conv_params *p, const void *co
                                     const int32_t *edge_perm, void *dx, void *dy, void *ds,
                                     void *workspace, void *stream);
 
+/* The receiver-grouped backward over tiles of receivers.  Neighbouring receivers share most of
+ * their senders; a workgroup takes `tile_rows` receivers that are consecutive in the row order,
+ * keeps their dm rows in LDS and walks the tile's edges sorted by sender, so that the dx
+ * contributions of one sender are summed on chip and leave as one set of float atomics per
+ * (tile, sender) instead of one per edge.  Same results as e3j_amd_convolution_bwd_receiver up
+ * to the summation order of dx.  Needs a compile-time-unrolled kernel of the trailing layout with
+ * at least 64 channels (else E3J_AMD_UNIMPLEMENTED) and a schedule built for the same adjacency,
+ * edge_perm and p->row_order.  No counterpart in the reference; prior art for grouping the
+ * backward by receivers with dx added into a zero-filled buffer:
+ * src/e3j/pallas_ops/convolution/mosaic_gpu/bwd.py:336-457.
+ *
+ * Schedule: the edge positions of every tile sorted by sender (padding edges last), as three
+ * parallel arrays, and work descriptors (tile, begin, end, 0) that cut the tiles' lists into
+ * pieces of at most `max_work_edges` positions (long rows are thereby shared by several
+ * workgroups).  All pointers are device memory owned by the caller. */
+typedef struct e3j_amd_tile_schedule {
+    int32_t tile_rows;     /* receivers per tile */
+    int32_t num_work;      /* entries of `work` (an upper bound; unused entries have begin == end) */
+    const int32_t *work;   /* (num_work, 4) */
+    const int32_t *sender; /* (E) sender of the position, -1 for a padding edge */
+    const int32_t *edge;   /* (E) row of y / s / dy / ds */
+    const int32_t *local;  /* (E) index of the position's receiver within its tile */
+} e3j_amd_tile_schedule;
+/* Largest `tile_rows` the tiled backward of a signature takes (its LDS holds the dm rows of a
+ * tile), 0 if the signature has no tiled backward. */
+int32_t e3j_amd_tile_rows(int32_t signature);
+/* Number of work descriptors to provide for a graph (upper bound used by the builder). */
+int64_t e3j_amd_tile_schedule_num_work(int32_t num_nodes, int64_t num_edges, int32_t tile_rows,
+                                       int32_t max_work_edges);
+size_t e3j_amd_tile_schedule_workspace_bytes(int32_t num_nodes, int64_t num_edges, int32_t tile_rows);
+/* Builds the schedule of a receiver-grouped CSR (sender per position, receiver_ptr), optional
+ * edge_perm and optional row order, into work (num_work, 4), t_sender, t_edge, t_local (E each). */
+int e3j_amd_tile_schedule_build(const int32_t *sender, const int32_t *receiver_ptr,
+                                const int32_t *edge_perm, const int32_t *row_order,
+                                int32_t num_nodes, int64_t num_edges, int32_t tile_rows,
+                                int32_t max_work_edges, int32_t *work, int32_t *t_sender,
+                                int32_t *t_edge, int32_t *t_local, void *workspace, void *stream);
+int e3j_amd_convolution_bwd_tiled(const e3j_amd_conv_params *p, const void *x, const void *y,
+                                  const void *s, const void *dm, const int32_t *sender,
+                                  const int32_t *receiver_ptr, const int32_t *edge_perm,
+                                  const e3j_amd_tile_schedule *schedule, void *dx, void *dy, void *ds,
+                                  void *stream);
+
 /* Match a HOST copy of a packed forward table against the tables of the
  * compile-time-unrolled kernels built into the library, up to one uniform
  * positive factor (the 1/avg_num_neighbors the reference folds into the values,
