@@ -54,12 +54,12 @@ BUILTIN_SIGNATURES = [(f"{name}_k{k}", xi, yi, oi, k) for name, xi, yi, oi, ks i
 LAUNCH = {
     32: dict(fwd=[(1, 4, 1)], bwd=[(1, 4, 2), (1, 4, 1)]),
     64: dict(fwd=[(1, 4, 1), (1, 4, 2)], bwd=[(1, 4, 2), (1, 4, 1), (1, 4, 3), (1, 4, 4)],
-             bwd_tile=[(1, 16, 4), (1, 16, 3), (1, 8, 4), (1, 12, 4)]),
+             bwd_tile=[(1, 8, 3), (1, 8, 4), (1, 16, 4)]),
     128: dict(fwd=[(1, 4, 1), (1, 4, 2), (2, 4, 2), (2, 4, 4)],
               bwd=[(2, 4, 3), (1, 4, 1), (1, 4, 3), (1, 4, 4), (2, 4, 4), (1, 4, 2)],
-              bwd_tile=[(1, 16, 4), (1, 16, 3), (2, 8, 4), (2, 8, 3), (1, 8, 4), (1, 12, 4)]),
+              bwd_tile=[(2, 8, 3), (2, 8, 4), (1, 8, 4), (1, 16, 4)]),
     256: dict(fwd=[(1, 4, 1), (1, 4, 2)], bwd=[(2, 4, 3), (1, 4, 2), (1, 4, 3)],
-              bwd_tile=[(1, 16, 4), (2, 8, 4)]),
+              bwd_tile=[(2, 8, 3), (1, 8, 4)]),
 }
 #: `bwd_tile`: variants of the backward over tiles of receivers (trailing layout, at least 64
 #: channels): a block of `waves per block` waves shares the dm rows of a tile in LDS.
@@ -421,7 +421,7 @@ def emit_table_source(t: "Table", name: str, desc: str, channels: int, symbols, 
                     f"{part_names[zs]}>("] + bwd_args
     tile_args = ["    const float *, const float *, const float *, const float *, const int32_t *,",
                  "    const int32_t *, const int32_t *, const int32_t *, const int32_t *, float *, float *, float *,",
-                 "    int, int, int, float, unsigned, unsigned);"]
+                 "    int, int, int, float, unsigned);"]
     for v in tile:
         cpl, wpb, zs, minw = (*v, 1)[:4]
         out += [f"template __global__ void unrolled_bwd_tile_kernel<{channels}, {cpl}, {wpb}, {minw}, "

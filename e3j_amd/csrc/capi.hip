@@ -31,8 +31,7 @@ int check_hip(hipError_t err, const char *what) {
 namespace {
 Tuning &mutable_tuning() {
     static Tuning t = [] {
-        Tuning v{0, 0, 0};
-        if (const char *e = std::getenv("E3J_AMD_TILE_DEBUG")) v.tile_debug = std::atoi(e);
+        Tuning v{0, 0};
         if (const char *e = std::getenv("E3J_AMD_FWD_VARIANT")) v.fwd_variant = std::atoi(e);
         if (const char *e = std::getenv("E3J_AMD_BWD_VARIANT")) v.bwd_variant = std::atoi(e);
         return v;
@@ -181,7 +180,7 @@ int e3j_amd_register_signature(const void *entry) {
 }
 
 void e3j_amd_set_launch_variant(int32_t fwd_variant, int32_t bwd_variant) {
-    mutable_tuning() = Tuning{fwd_variant, bwd_variant, mutable_tuning().tile_debug};
+    mutable_tuning() = Tuning{fwd_variant, bwd_variant};
 }
 
 int e3j_amd_convolution_fwd(const e3j_amd_conv_params *p, const void *coef, const void *x,

@@ -97,7 +97,6 @@ int launch_zero_padding(const e3j_amd_conv_params &p, const int32_t *other, cons
 struct Tuning {
     int fwd_variant;
     int bwd_variant;
-    int tile_debug;
 };
 const Tuning &tuning();
 

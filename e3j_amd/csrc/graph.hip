@@ -8,6 +8,8 @@
 
 #include <hipcub/hipcub.hpp>
 
+#include <mutex>
+
 #include "common.h"
 
 namespace e3j_amd {
@@ -456,14 +458,13 @@ int e3j_amd_tile_schedule_build(const int32_t *other, const int32_t *row_ptr, co
     const uint64_t sentinel = (uint64_t)num_tiles << sender_bits;
     int end_bit = sender_bits + 1;
     while (end_bit < 64 && (sentinel >> end_bit) != 0) end_bit++;
-    const int begin_bit = (tuning().tile_debug & 4) ? sender_bits : 0;
     hipLaunchKernelGGL(tile_keys_kernel, dim3(grid_for(num_edges)), dim3(256), 0, stream, other, row_ptr, rank,
                        num_nodes, num_edges, tile_rows, sender_bits, sentinel, keys_in, vals_in, local);
     rc = check_hip(hipGetLastError(), "tile schedule keys");
     if (rc) return rc;
     temp_bytes = w.temp_bytes;
     rc = check_hip(hipcub::DeviceRadixSort::SortPairs(ws + w.temp, temp_bytes, keys_in, keys_out, vals_in, vals_out,
-                                                      (int)num_edges, begin_bit, end_bit, stream),
+                                                      (int)num_edges, 0, end_bit, stream),
                    "tile schedule sort");
     if (rc) return rc;
     hipLaunchKernelGGL(tile_entries_kernel, dim3(grid_for(num_edges)), dim3(256), 0, stream, keys_out, vals_out,

@@ -624,7 +624,7 @@ __device__ __forceinline__ void unrolled_bwd_tile_part(
     const int32_t *__restrict__ t_edge, const int32_t *__restrict__ t_local,
     const int32_t *__restrict__ row_order, float *__restrict__ dx, float *__restrict__ dy,
     float *__restrict__ ds, int num_nodes, float scale, unsigned y_flip, int tile, int tile_rows,
-    int begin, int end, int slice, float *tile_lds, unsigned dbg) {
+    int begin, int end, int slice, float *tile_lds) {
     constexpr int NX = Part::NX, NS = Part::NS, NZ = Part::NZ, Y = Part::Y;
     constexpr int X = Part::X, S = Part::S, Z = Part::Z;
     using V = Vec<CPL>;
@@ -639,6 +639,66 @@ __device__ __forceinline__ void unrolled_bwd_tile_part(
     const int c_raw = slice * WIDTH + lane;  // further channels of the lane: + 64, + 128, ...
     const bool active = SL::FULL || c_raw < K;
     const int c0 = active ? c_raw : 0;
+
+    // this wave's share of the list, cut at sender boundaries
+    auto boundary = [&](int p) {
+        if (p <= begin) return begin;
+        while (p < end && t_sender[p] == t_sender[p - 1]) p++;
+        return p;
+    };
+    const int n = end - begin;
+    const int lo = boundary(begin + (int)((int64_t)n * wave / nw));
+    const int hi = boundary(begin + (int)((int64_t)n * (wave + 1) / nw));
+
+    V xc[NX], xn[NX], sn[NS], acc[NX];
+    float yn[Y];
+    bool valid_n = false, newx_n = false;
+    int snd_n = 0, loc_n = 0;
+    int64_t ee_n = 0;
+    // `held`: the sender whose x row the registers will hold when the fetched edge is computed
+    // The indices of a position are read two positions ahead (scalar registers), so that the
+    // loads of the next edge never wait for them.
+    int snd_a = 0, ee_a = 0, loc_a = 0;
+    auto read_indices = [&](int pos) {
+        snd_a = t_sender[pos];
+        ee_a = t_edge[pos];
+        loc_a = t_local[pos];
+    };
+    auto fetch = [&](int held) {  // the edge whose indices were read last
+        const int snd = snd_a;
+        valid_n = (unsigned)snd < (unsigned)num_nodes;
+        snd_n = snd;
+        ee_n = ee_a;
+        loc_n = loc_a;
+        newx_n = valid_n && snd != held;
+        if (newx_n) {
+            const float *xr = x + (int64_t)snd * (X * K) + c0;
+#pragma unroll
+            for (int j = 0; j < NX; j++) xn[j] = load_apart<CPL>(xr + Part::kX[j] * K);
+        }
+        const float *sr = s + ee_n * (int64_t)(S * K) + c0;
+        const float *yr = y + ee_n * Y;
+#pragma unroll
+        for (int l = 0; l < NS; l++) sn[l] = load_apart_stream<CPL>(sr + Part::kS[l] * K);
+#pragma unroll
+        for (int k = 0; k < Y; k++) yn[k] = yr[k];
+    };
+    auto flush = [&](int snd) {
+        if (!active) return;
+        float *dxr = dx + (int64_t)snd * (X * K) + c0;
+#pragma unroll
+        for (int j = 0; j < NX; j++) {
+#pragma unroll
+            for (int t = 0; t < CPL; t++) unsafeAtomicAdd(dxr + Part::kX[j] * K + t * kWave, acc[j].v[t]);
+        }
+    };
+
+    int held = -1, run = -1;
+    if (lo < hi) {
+        read_indices(lo);
+        fetch(held);
+        if (lo + 1 < hi) read_indices(lo + 1);
+    }
 
     // stage the dm rows of the tile's receivers (scaled): row (t, i) at (t * NZ + i) * WIDTH
     {
@@ -658,53 +718,7 @@ __device__ __forceinline__ void unrolled_bwd_tile_part(
     }
     __syncthreads();
 
-    // this wave's share of the list, cut at sender boundaries
-    auto boundary = [&](int p) {
-        if (p <= begin) return begin;
-        while (p < end && t_sender[p] == t_sender[p - 1]) p++;
-        return p;
-    };
-    const int n = end - begin;
-    const int lo = boundary(begin + (int)((int64_t)n * wave / nw));
-    const int hi = boundary(begin + (int)((int64_t)n * (wave + 1) / nw));
 
-    V xc[NX], xn[NX], sn[NS], acc[NX];
-    float yn[Y];
-    bool valid_n = false, newx_n = false;
-    int snd_n = 0, loc_n = 0;
-    int64_t ee_n = 0;
-    // `held`: the sender whose x row the registers will hold when the fetched edge is computed
-    auto fetch = [&](int pos, int held) {
-        const int snd = t_sender[pos];
-        valid_n = (unsigned)snd < (unsigned)num_nodes;
-        snd_n = snd;
-        ee_n = t_edge[pos];
-        loc_n = t_local[pos];
-        newx_n = valid_n && snd != held;
-        if (newx_n) {
-            const float *xr = x + (int64_t)snd * (X * K) + c0;
-#pragma unroll
-            for (int j = 0; j < NX; j++) xn[j] = load_apart<CPL>(xr + Part::kX[j] * K);
-        }
-        const float *sr = s + ee_n * (int64_t)(S * K) + c0;
-        const float *yr = y + ee_n * Y;
-#pragma unroll
-        for (int l = 0; l < NS; l++) sn[l] = load_apart_stream<CPL>(sr + Part::kS[l] * K);
-#pragma unroll
-        for (int k = 0; k < Y; k++) yn[k] = yr[k];
-    };
-    auto flush = [&](int snd) {
-        if (!active || (dbg & 1u)) return;
-        float *dxr = dx + (int64_t)snd * (X * K) + c0;
-#pragma unroll
-        for (int j = 0; j < NX; j++) {
-#pragma unroll
-            for (int t = 0; t < CPL; t++) unsafeAtomicAdd(dxr + Part::kX[j] * K + t * kWave, acc[j].v[t]);
-        }
-    };
-
-    int held = -1, run = -1;
-    if (lo < hi) fetch(lo, held);
     for (int pos = lo; pos < hi; pos++) {
         V sc[NS];
         float yc[Y];
@@ -720,7 +734,10 @@ __device__ __forceinline__ void unrolled_bwd_tile_part(
         const bool valid = valid_n;
         const int snd = snd_n, loc = loc_n;
         const int64_t ee = ee_n;
-        if (pos + 1 < hi) fetch(pos + 1, held);
+        if (pos + 1 < hi) {
+            fetch(held);
+            if (pos + 2 < hi) read_indices(pos + 2);
+        }
         if (!valid) continue;  // padding edge: its dy/ds rows are zero-filled separately
 
         if (snd != run) {
@@ -731,7 +748,7 @@ __device__ __forceinline__ void unrolled_bwd_tile_part(
         }
         V dxe[NX];
         float dye[Red::P];
-        const DsRows<CPL, K> ds_rows{ds + ee * (int64_t)(S * K) + c0, active && !(dbg & 2u)};
+        const DsRows<CPL, K> ds_rows{ds + ee * (int64_t)(S * K) + c0, active};
         const DmTile<CPL> dm_rows{tile_lds + loc * (NZ * WIDTH) + lane * CPL};
         Part::template edge_bwd<CPL>(xc, yc, sc, dm_rows, dxe, dye, ds_rows);
 #pragma unroll
@@ -743,7 +760,6 @@ __device__ __forceinline__ void unrolled_bwd_tile_part(
         for (int k = Y; k < Red::P; k++) dye[k] = 0.f;
         Red::run(dye, lane, [&](int k, float sum) {
             const float total = flip_sign(sum, y_flip, k);
-            if (dbg & 8u) return;
             if (!kAtomicDy) dy[ee * Y + k] = total;
             else unsafeAtomicAdd(dy + ee * Y + k, total);  // dy zero-filled by the launcher
         });
@@ -756,7 +772,7 @@ __device__ __forceinline__ void dispatch_bwd_tile(int, const float *, const floa
                                                   const float *, const int32_t *, const int32_t *,
                                                   const int32_t *, const int32_t *, float *, float *,
                                                   float *, int, float, unsigned, int, int, int, int, int,
-                                                  float *, unsigned) {}
+                                                  float *) {}
 template <int K, int CPL, bool A, int I, typename Part, typename... Rest>
 __device__ __forceinline__ void dispatch_bwd_tile(int part, const float *x, const float *y, const float *s,
                                                   const float *dm, const int32_t *t_sender,
@@ -764,15 +780,15 @@ __device__ __forceinline__ void dispatch_bwd_tile(int part, const float *x, cons
                                                   const int32_t *row_order, float *dx, float *dy,
                                                   float *ds, int num_nodes, float scale, unsigned y_flip,
                                                   int tile, int tile_rows, int begin, int end, int slice,
-                                                  float *tile_lds, unsigned dbg) {
+                                                  float *tile_lds) {
     if (part == I)
         unrolled_bwd_tile_part<Part, K, CPL, A>(x, y, s, dm, t_sender, t_edge, t_local, row_order, dx, dy,
                                                 ds, num_nodes, scale, y_flip, tile, tile_rows, begin, end,
-                                                slice, tile_lds, dbg);
+                                                slice, tile_lds);
     else
         dispatch_bwd_tile<K, CPL, A, I + 1, Rest...>(part, x, y, s, dm, t_sender, t_edge, t_local,
                                                      row_order, dx, dy, ds, num_nodes, scale, y_flip,
-                                                     tile, tile_rows, begin, end, slice, tile_lds, dbg);
+                                                     tile, tile_rows, begin, end, slice, tile_lds);
 }
 
 // One block per (work item, channel slice, part); a work item is a piece of one tile's edge list.
@@ -783,7 +799,7 @@ __global__ __launch_bounds__(kWave *WPB, MINW) void unrolled_bwd_tile_kernel(
     const int32_t *__restrict__ t_sender, const int32_t *__restrict__ t_edge,
     const int32_t *__restrict__ t_local, const int32_t *__restrict__ row_order,
     float *__restrict__ dx, float *__restrict__ dy, float *__restrict__ ds, int num_nodes,
-    int tile_rows, int num_work, float scale, unsigned y_flip, unsigned dbg) {
+    int tile_rows, int num_work, float scale, unsigned y_flip) {
     extern __shared__ __attribute__((aligned(16))) float tile_lds[];
     constexpr int NP = sizeof...(Parts);
     constexpr int CW = Slice<K, CPL>::COUNT;
@@ -797,7 +813,7 @@ __global__ __launch_bounds__(kWave *WPB, MINW) void unrolled_bwd_tile_kernel(
     if (begin >= end) return;  // unused descriptor or a tile without edges (uniform over the block)
     dispatch_bwd_tile<K, CPL, kAtomicDy, 0, Parts...>(part, x, y, s, dm, t_sender, t_edge, t_local,
                                                       row_order, dx, dy, ds, num_nodes, scale, y_flip,
-                                                      tile, tile_rows, begin, end, slice, tile_lds, dbg);
+                                                      tile, tile_rows, begin, end, slice, tile_lds);
 }
 
 // ---------------------------------------------------------------------------
@@ -1313,7 +1329,7 @@ int launch_unrolled_bwd_tile(const e3j_amd_conv_params &p, const float *x, const
     if (rc) return rc;
     hipLaunchKernelGGL(kernel, dim3((unsigned)blocks), dim3(kWave, WPB), lds, stream, x, y, s, dm, sch.work,
                        sch.sender, sch.edge, sch.local, p.row_order, dx, dy, ds, p.num_nodes, sch.tile_rows,
-                       sch.num_work, p.coef_scale, p.y_flip, (unsigned)tuning().tile_debug);
+                       sch.num_work, p.coef_scale, p.y_flip);
     return check_hip(hipGetLastError(), "convolution backward (tiled) launch");
 }
 
