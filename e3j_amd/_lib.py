@@ -114,6 +114,8 @@ SYMBOLS = {
     "e3j_amd_signature_name": (ctypes.c_char_p, [ctypes.c_int]),
     "e3j_amd_csr_workspace_bytes": (ctypes.c_size_t, [ctypes.c_int32, ctypes.c_int64]),
     "e3j_amd_csr_row_ptr": (ctypes.c_int, [_P, ctypes.c_int64, ctypes.c_int32, _P, _P, _P]),
+    "e3j_amd_csr_row_ptr_static_max_nodes": (ctypes.c_int32, []),
+    "e3j_amd_csr_row_ptr_static": (ctypes.c_int, [_P, ctypes.c_int64, ctypes.c_int32, _P, _P]),
     "e3j_amd_sort_edges": (ctypes.c_int, [_P, _P, ctypes.c_int64, ctypes.c_int32, _P, _P, _P, _P, _P]),
     "e3j_amd_order_workspace_bytes": (ctypes.c_size_t, [ctypes.c_int32]),
     "e3j_amd_register_signature": (ctypes.c_int, [_P]),

@@ -310,6 +310,65 @@ int e3j_amd_csr_row_ptr(const int32_t *key, int64_t num_edges, int32_t num_nodes
                         static_cast<hipStream_t>(stream_));
 }
 
+// ---- row pointers without a workspace argument ------------------------------------------------
+// The scan of e3j_amd_csr_row_ptr needs a few KB of temporary storage.  Callers that cannot
+// allocate (code under graph capture, serving loops) get it from this array instead: device
+// memory of the library's code object, one copy per GPU, held until the process ends.
+constexpr size_t kStaticScratchBytes = 256 * 1024;
+static __device__ __align__(256) unsigned char scratch[kStaticScratchBytes];
+
+namespace {
+constexpr int kMaxDevices = 64;
+std::mutex g_scratch_mutex;
+void *g_scratch_ptr[kMaxDevices];  // address of `scratch` on each device, looked up once
+// The device address of the array on the current device (the array's name is only a host-side
+// handle of the symbol).
+int static_scratch(void **ptr) {
+    int device = 0;
+    int rc = check_hip(hipGetDevice(&device), "csr_row_ptr_static: hipGetDevice");
+    if (rc) return rc;
+    if (device < 0 || device >= kMaxDevices)
+        return set_error(E3J_AMD_INVALID_ARGUMENT, "csr_row_ptr_static: device index out of range");
+    std::lock_guard<std::mutex> lock(g_scratch_mutex);
+    if (g_scratch_ptr[device] == nullptr) {
+        void *address = nullptr;
+        rc = check_hip(hipGetSymbolAddress(&address, HIP_SYMBOL(scratch)), "csr_row_ptr_static: hipGetSymbolAddress");
+        if (rc) return rc;
+        g_scratch_ptr[device] = address;
+    }
+    *ptr = g_scratch_ptr[device];
+    return E3J_AMD_OK;
+}
+}  // namespace
+
+int32_t e3j_amd_csr_row_ptr_static_max_nodes(void) {
+    // the scan's temporary storage grows with the number of entries; largest count that fits
+    int32_t lo = 0, hi = INT32_MAX - 1;
+    while (lo < hi) {
+        const int32_t mid = lo + (hi - lo + 1) / 2;
+        if (scan_temp_bytes(mid) <= kStaticScratchBytes) lo = mid; else hi = mid - 1;
+    }
+    return lo;
+}
+
+int e3j_amd_csr_row_ptr_static(const int32_t *key, int64_t num_edges, int32_t num_nodes, int32_t *row_ptr,
+                               void *stream_) {
+    if (num_nodes < 0 || num_edges < 0 || num_edges > 0x7fffffffLL)
+        return set_error(E3J_AMD_INVALID_ARGUMENT, "csr_row_ptr_static: bad sizes");
+    if (row_ptr == nullptr || (num_edges > 0 && key == nullptr))
+        return set_error(E3J_AMD_INVALID_ARGUMENT, "csr_row_ptr_static: null operand");
+    const size_t need = scan_temp_bytes(num_nodes);
+    if (need > kStaticScratchBytes)
+        return set_error(E3J_AMD_INVALID_ARGUMENT,
+                         "csr_row_ptr_static: " + std::to_string(num_nodes) + " nodes need " + std::to_string(need) +
+                             " bytes of scan storage, the built-in scratch holds " +
+                             std::to_string(kStaticScratchBytes) + " (use e3j_amd_csr_row_ptr with a workspace)");
+    void *temp = nullptr;
+    int rc = static_scratch(&temp);
+    if (rc) return rc;
+    return row_ptr_impl(key, num_edges, num_nodes, row_ptr, temp, need, static_cast<hipStream_t>(stream_));
+}
+
 int e3j_amd_wrap_index(const int32_t *index, int64_t n, int32_t num_nodes, int32_t *out,
                        void *stream_) {
     if (n < 0 || num_nodes <= 0)

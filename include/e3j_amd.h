@@ -213,6 +213,16 @@ const char *e3j_amd_signature_name(int signature);
 size_t e3j_amd_csr_workspace_bytes(int32_t num_nodes, int64_t num_edges);
 int e3j_amd_csr_row_ptr(const int32_t *key, int64_t num_edges, int32_t num_nodes,
                         int32_t *row_ptr, void *workspace, void *stream);
+/* e3j_amd_csr_row_ptr_static: the same row pointers for callers that cannot allocate or bring a
+ *   workspace (code under HIP graph capture, serving loops, harnesses that forbid hipMalloc).  The
+ *   scan's temporary storage lives in a 256 KiB device array inside the library (one copy per GPU,
+ *   held until the process ends); the call allocates nothing.  num_nodes above
+ *   e3j_amd_csr_row_ptr_static_max_nodes() is refused with E3J_AMD_INVALID_ARGUMENT.  Every call
+ *   on a GPU uses that GPU's one array: calls that overlap on one GPU (different streams or
+ *   threads) race; calls on one stream are ordered.  No counterpart in the reference. */
+int32_t e3j_amd_csr_row_ptr_static_max_nodes(void);
+int e3j_amd_csr_row_ptr_static(const int32_t *key, int64_t num_edges, int32_t num_nodes,
+                               int32_t *row_ptr, void *stream);
 /* e3j_amd_sort_edges: stable counting sort of edge positions by key (out-of-range
  *   keys last): perm (E), other_sorted = other[perm] (E), row_ptr (N+1). */
 int e3j_amd_sort_edges(const int32_t *key, const int32_t *other, int64_t num_edges,
