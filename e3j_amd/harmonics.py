@@ -11,10 +11,11 @@ degree-1 block is proportional to `(x, y, z)` of the input
 The reference builds explicit polynomials with ladder operators; here the same
 functions come from the recurrences of the associated Legendre polynomials and
 of `(X + iY)^m`, written with tensor operations so they run on the GPU and are
-differentiable with respect to the positions.  The values are pinned by the
-closed forms of degrees 0-2, the addition theorem and the Clebsch-Gordan
-coupling of this package, not by the reference's third-party comparison
-(`tests/test_harmonics.py:178-182`), which needs e3nn.
+differentiable with respect to the positions.  The test-suite checks the values against
+an independent restatement (scipy's harmonics and the textbook polynomials, themselves
+pinned by the closed forms of degrees 0-2, the addition theorem and the unit norm on the
+sphere), not by the reference's third-party comparison (`tests/test_harmonics.py:178-182`),
+which needs e3nn.
 """
 
 from __future__ import annotations

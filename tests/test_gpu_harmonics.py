@@ -1,6 +1,6 @@
-"""The spherical-harmonics kernels against the tensor-operation form of the same functions
-(which the CPU suite pins with closed forms, the addition theorem and the Clebsch-Gordan
-coupling)."""
+"""The spherical-harmonics kernels against the CPU checker `oracle/sh_oracle.py` (values from
+scipy's harmonics and, to degree 3, the textbook polynomials; cotangents from float64 central
+differences), and against the package's tensor-operation form of the same functions."""
 
 import numpy as np
 import pytest
@@ -8,6 +8,7 @@ import torch
 
 from e3j_amd import _lib
 from e3j_amd.harmonics import Harmonics
+from oracle import sh_oracle
 
 pytestmark = pytest.mark.gpu
 
@@ -15,6 +16,30 @@ pytestmark = pytest.mark.gpu
 def _vectors(n, dtype, seed=0):
     v = np.random.default_rng(seed).standard_normal((n, 3)) * 1.7
     return torch.from_numpy(v).to(dtype).cuda()
+
+
+@pytest.mark.parametrize("dtype, tol", [(torch.float64, 1e-11), (torch.float32, 2e-6)])
+@pytest.mark.parametrize("normalize", [False, True])
+@pytest.mark.parametrize("normalization", ["component", "integral", "norm"])
+def test_kernel_matches_checker(normalization, normalize, dtype, tol):
+    """`e3j_amd_harmonics` against the scipy-based checker (and the polynomial table to degree 3);
+    `e3j_amd_harmonics_bwd` against float64 central differences of the checker."""
+    for l_max in range(7):
+        h = Harmonics(l_max, normalize=normalize, normalization=normalization)
+        v = _vectors(400, dtype, seed=10 + l_max).requires_grad_(True)
+        got = h(v)
+        host = v.detach().cpu().numpy().astype(np.float64)
+        want = sh_oracle.harmonics_scipy(host, l_max, normalize, normalization)
+        scale = np.abs(want).max()
+        assert np.abs(got.detach().cpu().numpy() - want).max() <= tol * scale, (l_max, "values")
+        if l_max <= 3:
+            table = sh_oracle.harmonics_polynomial(host, l_max, normalize, normalization)
+            assert np.abs(got.detach().cpu().numpy() - table).max() <= tol * scale, (l_max, "polynomial table")
+        dout = np.random.default_rng(11).standard_normal(want.shape)
+        (g,) = torch.autograd.grad(got, v, torch.from_numpy(dout).to(dtype).cuda())
+        fd = sh_oracle.harmonics_vjp_fd(host, dout, l_max, normalize, normalization)
+        bound = max(4 * tol, 2e-6) * (np.abs(fd).max() + 1e-30)   # the differences carry 1e-6 of their own
+        assert np.abs(g.cpu().numpy() - fd).max() <= bound, (l_max, "gradient")
 
 
 @pytest.mark.parametrize("dtype, tol", [(torch.float64, 1e-12), (torch.float32, 2e-6)])
