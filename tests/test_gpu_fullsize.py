@@ -161,3 +161,34 @@ def test_tensor_product_benchmark_size_properties(mode, layout):
     want = T.tensor_product_unfused(idx, val, xs, ys, Z, mode, layout)
     mag = T.tensor_product_unfused(idx, np.abs(val), np.abs(xs), np.abs(ys), Z, mode, layout)
     H.assert_parity(z[:head].cpu().numpy(), want, mag, f"head {mode} {layout}")
+
+
+@pytest.mark.parametrize("layout", ["TRAILING_CHANNELS", "LEADING_CHANNELS"])
+def test_sender_ordering_on_the_symmetric_config2_graph_matches_checker(layout):
+    """SENDER ordering (`src/e3j/ops/convolution.py:166-176,413-425`) at the size of config 2: the
+    radius graph is symmetric, y of a reversed edge is the parity image of y, and the radial
+    weights are made symmetric; edges sorted by sender.  Forward and all three cotangents
+    against the CPU checker, which knows nothing of orderings."""
+    w = W.config2()
+    n = w.num_nodes
+    snd, rcv = w.sender.numpy().astype(np.int64), w.receiver.numpy().astype(np.int64)
+    key, rev_key = snd * n + rcv, rcv * n + snd
+    by_key = np.argsort(key)
+    rev = by_key[np.searchsorted(key[by_key], rev_key)]
+    assert np.array_equal(key[rev], rev_key), "every edge has its reverse"
+    m = e3j_amd.Convolution((w.module.source[0], w.module.source[1]), "0e+1o+2e", graph_ordering="SENDER")
+    parity = torch.as_tensor(np.asarray(m.y_parity, dtype=np.float32))
+    torch.testing.assert_close(w.y[rev], w.y * parity[None, :], rtol=1e-5, atol=1e-5)
+    s = 0.5 * (w.s + w.s[rev])                                    # s_ba = s_ab
+    y = 0.5 * (w.y + w.y[rev] * parity[None, :])                  # y_ba = p y_ab to the last bit
+    order = torch.as_tensor(np.argsort(snd, kind="stable"))
+    base = W.Workload("cfg2 by sender", m, w.x, y[order], s[order], w.dm, w.sender[order], w.receiver[order],
+                      w.positions, w.box)
+    ws = base.with_layout(layout).to("cuda")
+    m = ws.module
+    assert m.graph_ordering.value == "SENDER" and m.layout.name == layout
+    xs, ys, ss = (t.clone().requires_grad_(True) for t in (ws.x, ws.y, ws.s))
+    out = m(xs, ys, ss, ws.sender, ws.receiver)
+    grads = torch.autograd.grad(out, (xs, ys, ss), ws.dm)
+    torch.cuda.synchronize()
+    _against_c_oracle(ws, out.detach(), grads, f"cfg2 SENDER {layout}")
