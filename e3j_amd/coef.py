@@ -50,18 +50,22 @@ class Coef:
 
     @classmethod
     def _numpy_dtype(cls, val_t, idx_t) -> np.dtype:
+        """The entry as a numpy record: the value first, the indices behind it at the first
+        multiple of the index size, the record padded to a power of two (the `alignas` of
+        `lib/e3j_ops/cuda/convolution.cuh:31-44`)."""
         val_t, idx_t = np.dtype(val_t), np.dtype(idx_t)
-        fields = [("val", val_t)] + [(name, idx_t) for name in cls.index_names]
-        dt = np.dtype(fields, align=True)
-        target = next_pow2(val_t.itemsize + cls.rank * idx_t.itemsize)
-        if dt.itemsize < target:
-            dt = np.dtype({
-                "names": list(dt.names),
-                "formats": [dt.fields[n][0] for n in dt.names],
-                "offsets": [dt.fields[n][1] for n in dt.names],
-                "itemsize": target,
-            })
-        return dt
+        step = idx_t.itemsize
+        first_index = -(-val_t.itemsize // step) * step
+        offsets = {"val": 0}
+        for n, name in enumerate(cls.index_names):
+            offsets[name] = first_index + n * step
+        names = ["val", *cls.index_names]
+        return np.dtype({
+            "names": names,
+            "formats": [val_t] + [idx_t] * cls.rank,
+            "offsets": [offsets[n] for n in names],
+            "itemsize": next_pow2(val_t.itemsize + cls.rank * step),
+        })
 
     @property
     def dtype(self) -> np.dtype:
@@ -90,26 +94,23 @@ class Coef:
         return packed.view(idx_t).reshape(-1, numel)
 
     def transpose(self, argnums):
-        """Permute index columns, stable-sort by the new first column (`src/e3j/ops/coef.py:174-184`)."""
-        idx = self.idx.T
-        sigma = np.argsort(idx[argnums[0]], kind="stable")
-        new_idx = np.stack([idx[a][sigma] for a in argnums]).T
-        return type(self)(self.val[sigma], new_idx, self.val_dtype, self.idx_dtype)
+        """The table with its index columns reordered to `argnums` and its entries grouped by the
+        new leading column, earlier entries first within a group (behaviour of
+        `src/e3j/ops/coef.py:174-184`)."""
+        columns = self.idx[:, list(argnums)]
+        order = np.argsort(columns[:, 0], kind="stable")
+        return type(self)(self.val[order], columns[order], self.val_dtype, self.idx_dtype)
 
     @classmethod
     def unpack(cls, data, val_dtype):
-        data = np.asarray(data)
-        idx_t = data.dtype["i"] if data.dtype.fields is not None else data.dtype
-        val_t = np.dtype(val_dtype)
-        coef_t = cls._numpy_dtype(val_t, idx_t)
-        numel = coef_t.itemsize // idx_t.itemsize
-        numval = -(-val_t.itemsize // idx_t.itemsize)
-        flat = np.ascontiguousarray(data).view(idx_t).reshape(-1, numel)
-        val_slots = np.ascontiguousarray(flat[:, :numval])
-        val = val_slots.view(val_t).reshape(flat.shape[0], -1)[:, 0] if flat.shape[0] else \
-            np.zeros((0,), dtype=val_t)
-        idx = flat[:, numval:numval + cls.rank]
-        return cls(val, idx, val_t, idx_t)
+        """Inverse of `pack` / `pack_numpy`: read the records back through the record dtype."""
+        data = np.ascontiguousarray(data)
+        idx_t = data.dtype if data.dtype.fields is None else data.dtype["i"]
+        record = cls._numpy_dtype(val_dtype, idx_t)
+        table = data.view(np.uint8).reshape(-1).view(record) if data.size else np.zeros(0, dtype=record)
+        idx = np.stack([table[name] for name in cls.index_names], axis=1) if len(table) else \
+            np.zeros((0, cls.rank), dtype=idx_t)
+        return cls(np.array(table["val"]), idx, np.dtype(val_dtype), idx_t)
 
 
 class Coef4D(Coef):

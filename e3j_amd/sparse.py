@@ -35,26 +35,31 @@ class SparseCOO:
 
 
 def sparse_coo(values, indices, shape, coalesce: bool = True, dtype=np.float32) -> SparseCOO:
-    """Build a `SparseCOO`, coalesced by default (`src/e3j/utils/sparse.py:76-126`)."""
+    """Build a `SparseCOO`; coalesced by default: entries in lexicographic order of their
+    coordinates, repeated coordinates merged by summation, entries that sum to exactly zero
+    removed (behaviour of `src/e3j/utils/sparse.py:76-126`)."""
     shape = tuple(int(n) for n in shape)
-    values = np.asarray(values).astype(dtype)
-    indices = np.asarray(indices, dtype=np.int64)
-    if indices.ndim != 2 or indices.shape[1] != len(shape):
-        raise ValueError(f"Expected indices of shape (nnz, {len(shape)}) for shape {shape}, "
-                         f"got {indices.shape}.")
-    if indices.shape[0] != values.shape[0]:
-        raise ValueError(f"Got {values.shape[0]} values for {indices.shape[0]} indices.")
-    if indices.size and ((indices < 0).any() or (indices >= np.asarray(shape)).any()):
+    coords = np.asarray(indices, dtype=np.int64)
+    vals = np.asarray(values).astype(dtype)
+    rank = len(shape)
+    if coords.ndim != 2 or coords.shape[1] != rank:
+        raise ValueError(f"indices must be (nnz, {rank}) for a rank-{rank} array of shape {shape}; got {coords.shape}")
+    if len(vals) != len(coords):
+        raise ValueError(f"{len(vals)} values do not pair with {len(coords)} coordinate rows")
+    limits = np.asarray(shape, dtype=np.int64).reshape(1, rank)
+    if coords.size and not ((coords >= 0) & (coords < limits)).all():
         raise ValueError(f"Out of bounds indices for shape {shape}.")
-    if coalesce and indices.shape[0]:
-        keys = np.ravel_multi_index(tuple(indices.T), shape)
-        order = np.argsort(keys, kind="stable")
-        keys = keys[order]
-        first = np.ones(keys.shape[0], dtype=bool)
-        np.not_equal(keys[1:], keys[:-1], out=first[1:])
-        summed = np.zeros(int(first.sum()), dtype=values.dtype)
-        np.add.at(summed, np.cumsum(first) - 1, values[order])
-        indices = indices[order[first]]
-        keep = summed != 0
-        indices, values = indices[keep], summed[keep]
-    return SparseCOO(values, indices.astype(narrow_index_dtype(shape)), shape)
+    if coalesce and len(coords):
+        # row-major linear position of every entry; np.unique returns the distinct positions in
+        # ascending order (= lexicographic order of the coordinates) and, per entry, which of
+        # them it falls on, so one weighted histogram merges the duplicates
+        strides = np.concatenate([np.cumprod(limits[0, :0:-1])[::-1], [1]]).astype(np.int64)
+        linear = coords @ strides
+        distinct, slot = np.unique(linear, return_inverse=True)
+        merged = np.zeros(len(distinct), dtype=np.float64)
+        np.add.at(merged, slot.reshape(-1), vals.astype(np.float64))
+        merged = merged.astype(vals.dtype)
+        alive = np.flatnonzero(merged)
+        coords = np.stack(np.unravel_index(distinct[alive], shape), axis=1).astype(np.int64)
+        vals = merged[alive]
+    return SparseCOO(vals, coords.astype(narrow_index_dtype(shape)), shape)

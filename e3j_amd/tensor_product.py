@@ -9,7 +9,6 @@ row by row with the fused HIP kernels of `e3j_amd.tp_ops`
 
 from __future__ import annotations
 
-import itertools
 
 import numpy as np
 
@@ -126,28 +125,30 @@ class TensorProduct:
         """
         target, in1, in2 = O3Space(target), O3Space(source_1), O3Space(source_2)
         normalization = TensorProductNormalization.parse(normalization)
-        keep = {(ir.l, ir.p) for _, ir in target}
-        values, indices, begin_out = [], [], 0
-        for ((m1, ir1), s1), ((m2, ir2), s2) in itertools.product(
-                zip(in1, in1.slices()), zip(in2, in2.slices())):
-            k1, k2 = np.mgrid[:m1, :m2].reshape(2, -1)
-            for _, ir0 in ir1 * ir2:
-                if (ir0.l, ir0.p) not in keep:
-                    continue
-                dense = clebsch_gordan(ir0.l, ir1.l, ir2.l)
-                nz = np.nonzero(dense)
-                data = dense[nz]
-                if normalization == TensorProductNormalization.SQRT_DIM_OUT:
-                    data = data * np.sqrt(2 * ir0.l + 1)
-                block_idx = np.stack(nz, axis=-1)
-                values.append(np.tile(data, m1 * m2))
-                offset = np.array([begin_out, s1.start, s2.start])
-                dims = np.array([ir0.dim, ir1.dim, ir2.dim])
-                mul_grid = np.stack((k1 * m2 + k2, k1, k2), axis=-1)
-                offsets = offset + mul_grid * dims
-                indices.append((block_idx[None, :] + offsets[:, None]).reshape(-1, 3))
-                begin_out += m1 * m2 * ir0.dim
+        wanted = {(ir.l, ir.p) for _, ir in target}
+        scaled = normalization == TensorProductNormalization.SQRT_DIM_OUT
         shape = (target.dim, in1.dim, in2.dim)
-        if not values:
+        rows, vals = [], []
+        out_at = 0   # first output coordinate of the next path
+        for (mul_x, ir_x), at_x in zip(in1, in1.slices()):
+            for (mul_y, ir_y), at_y in zip(in2, in2.slices()):
+                for _, ir_o in ir_x * ir_y:
+                    if (ir_o.l, ir_o.p) not in wanted:
+                        continue
+                    block = clebsch_gordan(ir_o.l, ir_x.l, ir_y.l)
+                    if scaled:
+                        block = block * np.sqrt(2 * ir_o.l + 1)
+                    i, j, k = np.nonzero(block)
+                    # every pair of copies (a of x, b of y) gets its own copy a * mul_y + b of
+                    # the output irrep, all with the same block
+                    for a in range(mul_x):
+                        for b in range(mul_y):
+                            copy = a * mul_y + b
+                            rows.append(np.stack([out_at + copy * ir_o.dim + i,
+                                                  at_x.start + a * ir_x.dim + j,
+                                                  at_y.start + b * ir_y.dim + k], axis=1))
+                            vals.append(block[i, j, k])
+                    out_at += mul_x * mul_y * ir_o.dim
+        if not rows:
             return sparse_coo(np.zeros((0,)), np.zeros((0, 3), dtype=np.int64), shape)
-        return sparse_coo(np.concatenate(values), np.concatenate(indices, axis=0), shape)
+        return sparse_coo(np.concatenate(vals), np.concatenate(rows, axis=0), shape)
