@@ -69,7 +69,7 @@ def parse_args():
     ap.add_argument("--deterministic", action="store_true",
                     help="time the atomic-free (bit-reproducible) backward instead of the default one")
     ap.add_argument("--access-floor", action="store_true",
-                    help="cfg3, 128 channels, trailing layout only: also time kernels that perform the "
+                    help="trailing layout, built-in tables at 64/128/256 channels: also time kernels that perform the "
                          "memory accesses of the two passes without their arithmetic (reported under "
                          "roofline.access_floor)")
     ap.add_argument("--inner", type=int, default=64, help="--op radial_linear: hidden size of the radial network")
@@ -217,7 +217,7 @@ def access_floor(torch, abi, steps: int) -> dict:
                     w.dm.data_ptr(), abi.other.data_ptr(), abi.ptr.data_ptr(), order, abi.ds.data_ptr(),
                     abi.dx.data_ptr(), abi.out.data_ptr(), w.num_nodes, sink.data_ptr(), abi._stream())
             if rc != 0:
-                raise RuntimeError("the access-pattern probe covers cfg3 with 128 channels, trailing layout, only")
+                raise RuntimeError("the access-pattern probe has no instantiation for these operand sizes (built-in tables, 64/128/256 channels, trailing layout)")
         result[name] = round(time_events(torch, run, steps, 1), 4)
     return result
 

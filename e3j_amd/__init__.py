@@ -13,7 +13,8 @@ from .convolution import Convolution
 from .graph import DUMMY_INDEX, GraphCSR
 from .harmonics import Harmonics
 from .ops import (ConvolutionBatchingWarning, ConvolutionParams, CUDAConvolutionParams, TableDrivenKernelWarning,
-                  convolution, convolution_batched, convolution_bwd)
+                  PreparedGraph, clear_graph_cache, convolution, convolution_batched, convolution_bwd,
+                  prepare_graph)
 from .options import Config, GraphOrdering, Layout, MixingMode, TensorProductNormalization, config
 from .radial import radial_linear
 from .scalar_mixing import ScalarMixing
@@ -30,5 +31,6 @@ __all__ = [
     "CUDAConvolutionParams", "DUMMY_INDEX", "GraphCSR", "GraphOrdering", "Harmonics", "Layout", "O3Irrep",
     "O3Space", "ScalarMixing", "Space", "TensorProduct", "TensorProductNormalization", "config",
     "convolution", "convolution_batched", "convolution_bwd", "radial_linear", "resolve_val_dtype",
+    "PreparedGraph", "prepare_graph", "clear_graph_cache",
     "CUDATensorProductParams", "MixingMode", "TensorProductParams", "tensor_product", "tensor_product_batched", "tensor_product_bwd",
 ]

@@ -455,22 +455,22 @@ def emit_table_source(t: "Table", name: str, desc: str, channels: int, symbols, 
             f"static const uint8_t kIdx[] = {{{idxs}}};",
             ""]
     out += ["static int run_fwd" + fwd_sig[0]] + fwd_sig[1:]
-    out += [ln.replace("VARIANT", "tuning().fwd_variant") for ln in switch(
+    out += [ln.replace("VARIANT", "tuning().fwd_variant.load(std::memory_order_relaxed)") for ln in switch(
         launch["fwd"], lambda v: f"launch_unrolled_fwd<{channels}, {v[0]}, {v[1]}, {(*v, 1)[3]}, {part_names[v[2]]}>("
                                  "p, x, y, s, sender, row_ptr, perm, out, stream);")]
     out += ["static int run_bwd" + bwd_sig[0]] + bwd_sig[1:]
-    out += [ln.replace("VARIANT", "tuning().bwd_variant") for ln in switch(
+    out += [ln.replace("VARIANT", "tuning().bwd_variant.load(std::memory_order_relaxed)") for ln in switch(
         launch["bwd"], lambda v: f"launch_unrolled_bwd<{channels}, {v[0]}, {v[1]}, {(*v, 1)[3]}, {t.Y}, {t.X}, "
                                  f"{part_names[v[2]]}>(p, x, y, s, dm, sender, row_ptr, perm, dx, dy, ds, stream, ordered);")]
     if tile:
         out += ["static int run_bwd_tiled(const e3j_amd_conv_params &p, const float *x, const float *y,",
                 "                         const float *s, const float *dm, const e3j_amd_tile_schedule &schedule,",
                 "                         float *dx, float *dy, float *ds, hipStream_t stream) {"]
-        out += [ln.replace("VARIANT", "tuning().bwd_variant") for ln in switch(
+        out += [ln.replace("VARIANT", "tuning().bwd_variant.load(std::memory_order_relaxed)") for ln in switch(
             tile, lambda v: f"launch_unrolled_bwd_tile<{channels}, {v[0]}, {v[1]}, {(*v, 1)[3]}, {t.Y}, {t.X}, "
                             f"{part_names[v[2]]}>(p, x, y, s, dm, schedule, dx, dy, ds, stream);")]
         out += ["static int run_tile_row_bytes() {"]
-        out += [ln.replace("VARIANT", "tuning().bwd_variant") for ln in switch(
+        out += [ln.replace("VARIANT", "tuning().bwd_variant.load(std::memory_order_relaxed)") for ln in switch(
             tile, lambda v: f"tile_row_bytes<{v[0]}, {part_names[v[2]]}>();")]
     tiled = "&run_bwd_tiled, &run_tile_row_bytes" if tile else "nullptr, nullptr"
     out += [f"extern const Signature {symbols[0]} = {{",
@@ -480,11 +480,11 @@ def emit_table_source(t: "Table", name: str, desc: str, channels: int, symbols, 
             "};", ""]
     if lead:
         out += ["static int run_fwd_leading" + fwd_sig[0]] + fwd_sig[1:]
-        out += [ln.replace("VARIANT", "tuning().fwd_variant") for ln in switch(
+        out += [ln.replace("VARIANT", "tuning().fwd_variant.load(std::memory_order_relaxed)") for ln in switch(
             lead["fwd"], lambda v: f"launch_unrolled_fwd_leading<{channels}, {v[0]}, {part_names[v[1]]}>("
                                    "p, x, y, s, sender, row_ptr, perm, out, stream);")]
         out += ["static int run_bwd_leading" + bwd_sig[0]] + bwd_sig[1:]
-        out += [ln.replace("VARIANT", "tuning().bwd_variant") for ln in switch(
+        out += [ln.replace("VARIANT", "tuning().bwd_variant.load(std::memory_order_relaxed)") for ln in switch(
             lead["bwd"], lambda v: f"launch_unrolled_bwd_leading<{channels}, {t.Y}, {t.X}, "
                                    f"{part_names[v[1]]}>(p, x, y, s, dm, sender, row_ptr, perm, dx, dy, ds, stream, ordered);")]
         out += [f"extern const Signature {symbols[1]} = {{",

@@ -80,9 +80,10 @@ class Convolution:
             c = self.coef
             packed = self._packed[val_dtype] = Coef4D(c.val, c.idx, val_dtype=val_dtype,
                                                       idx_dtype=c.idx_dtype).pack()
+            packed.setflags(write=False)   # frozen: the operators may key their caches on its identity
         return packed
 
-    def _fused_eval(self, node_features, edge_features, edge_scalars, senders, receivers):
+    def _fused_eval(self, node_features, edge_features, edge_scalars, senders, receivers, graph=None):
         dtype = torch.promote_types(torch.promote_types(node_features.dtype, edge_features.dtype),
                                     edge_scalars.dtype)
         val_dtype = resolve_val_dtype(_NP_OF_TORCH.get(dtype, "int64"))
@@ -92,18 +93,22 @@ class Convolution:
         y_parity = self.y_parity if self.graph_ordering == GraphOrdering.SENDER else None
         return convolution(self._packed_coef(val_dtype), node_features, edge_features, edge_scalars,
                            senders, receivers, self.params, self.graph_ordering, y_parity,
-                           layout=self.layout)
+                           layout=self.layout, graph=graph)
 
     def __call__(self, node_features, edge_features, edge_scalars, senders, receivers,
-                 node_mask=None):
+                 node_mask=None, graph=None):
         """Sum of messages on receiver nodes.
 
         node_features `(num_nodes, num_x, channels)`, edge_features `(num_edges, num_y)`,
         edge_scalars `(num_edges, num_scalars, channels)` (leading layout: channels before
         the irreps axis); `node_mask` marks real nodes, padding nodes lie at the tail.
+        `graph`: optional `prepare_graph` handle of `(senders, receivers)` in this module's
+        ordering (not together with `node_mask`, which changes the edges).
         """
+        if node_mask is not None and graph is not None:
+            raise ValueError("`graph` was prepared for the unmasked edges; pass either `node_mask` or `graph`")
         if node_mask is not None:
             senders, receivers = GraphCSR.mask_edges(senders, receivers, node_mask)
         if self.config.convolution == ConvolutionImpl.FUSED_HIP:
-            return self._fused_eval(node_features, edge_features, edge_scalars, senders, receivers)
+            return self._fused_eval(node_features, edge_features, edge_scalars, senders, receivers, graph)
         raise RuntimeError("Unknown convolution implementation.")

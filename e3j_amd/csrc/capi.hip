@@ -30,12 +30,13 @@ int check_hip(hipError_t err, const char *what) {
 
 namespace {
 Tuning &mutable_tuning() {
-    static Tuning t = [] {
-        Tuning v{0, 0};
-        if (const char *e = std::getenv("E3J_AMD_FWD_VARIANT")) v.fwd_variant = std::atoi(e);
-        if (const char *e = std::getenv("E3J_AMD_BWD_VARIANT")) v.bwd_variant = std::atoi(e);
-        return v;
+    static Tuning t;
+    static const bool from_environment = [] {
+        if (const char *e = std::getenv("E3J_AMD_FWD_VARIANT")) t.fwd_variant.store(std::atoi(e));
+        if (const char *e = std::getenv("E3J_AMD_BWD_VARIANT")) t.bwd_variant.store(std::atoi(e));
+        return true;
     }();
+    (void)from_environment;
     return t;
 }
 }  // namespace
@@ -98,14 +99,16 @@ int validate(const e3j_amd_conv_params *p, const char *op) {
 
 bool missing(const void *ptr, int64_t count) { return count > 0 && ptr == nullptr; }
 
-// The unrolled kernels of the leading-channels layout move rows in 16-byte pieces.
+// The unrolled kernels move rows in pieces of up to 16 bytes (whole blocks in the leading layout,
+// several channels per lane and the fixed-order dx reduction in the trailing one): operands that
+// are not 16-byte aligned (a view at an odd element offset) take the table-driven kernels.
 bool aligned16(std::initializer_list<const void *> ptrs) {
     for (const void *ptr : ptrs)
         if (reinterpret_cast<uintptr_t>(ptr) % 16 != 0) return false;
     return true;
 }
 bool signature_fits(const e3j_amd_conv_params *p, std::initializer_list<const void *> ptrs) {
-    return p->signature >= 0 && (p->layout == E3J_AMD_LAYOUT_TRAILING || aligned16(ptrs));
+    return p->signature >= 0 && aligned16(ptrs);
 }
 // Falling back to the table-driven kernel is only right when no sign flip was asked for.
 int flip_without_kernel(const e3j_amd_conv_params *p, const char *op) {
@@ -180,7 +183,8 @@ int e3j_amd_register_signature(const void *entry) {
 }
 
 void e3j_amd_set_launch_variant(int32_t fwd_variant, int32_t bwd_variant) {
-    mutable_tuning() = Tuning{fwd_variant, bwd_variant};
+    mutable_tuning().fwd_variant.store(fwd_variant, std::memory_order_relaxed);
+    mutable_tuning().bwd_variant.store(bwd_variant, std::memory_order_relaxed);
 }
 
 int e3j_amd_convolution_fwd(const e3j_amd_conv_params *p, const void *coef, const void *x,
@@ -279,6 +283,8 @@ int e3j_amd_convolution_bwd_ordered(const e3j_amd_conv_params *p, const void *co
         workspace == nullptr)
         return set_error(E3J_AMD_INVALID_ARGUMENT, std::string(op) + ": null operand");
     if (p->num_nodes == 0) return E3J_AMD_OK;
+    if (p->signature >= 0 && !aligned16({x, s, dm, dx, ds, workspace}))
+        return set_error(E3J_AMD_INVALID_ARGUMENT, std::string(op) + ": operands must be 16-byte aligned");
     if (!signature_fits(p, {x, s, dm, dx, ds}) || signature(p->signature).bwd == nullptr)
         return set_error(E3J_AMD_UNIMPLEMENTED,
                          std::string(op) + ": needs a compile-time-unrolled kernel for the table; "
@@ -341,6 +347,8 @@ int e3j_amd_convolution_bwd_tiled(const e3j_amd_conv_params *p, const void *x, c
                          std::string(op) + ": needs a compile-time-unrolled kernel of the trailing layout "
                                            "with at least 64 channels; e3j_amd_convolution_bwd_receiver "
                                            "serves the other cases");
+    if (!aligned16({x, s, dm, dx, ds}))
+        return set_error(E3J_AMD_INVALID_ARGUMENT, std::string(op) + ": operands must be 16-byte aligned");
     if (schedule->num_work < 0 || (schedule->num_work > 0 && schedule->work == nullptr) ||
         missing(schedule->sender, p->num_edges) || missing(schedule->edge, p->num_edges) ||
         missing(schedule->local, p->num_edges))

@@ -5,6 +5,7 @@
 #include <hip/hip_runtime.h>
 #include <stdint.h>
 
+#include <atomic>
 #include <string>
 
 #include "../../include/e3j_amd.h"
@@ -94,9 +95,11 @@ int launch_zero_padding(const e3j_amd_conv_params &p, const int32_t *other, cons
 
 // Launch-shape variants of the unrolled kernels, from E3J_AMD_FWD_VARIANT /
 // E3J_AMD_BWD_VARIANT (read once; 0 = default).  For tuning runs.
+// The two numbers are read by every launch and may be set from another thread: relaxed atomics
+// (a launch sees the old or the new shape, never a torn value).
 struct Tuning {
-    int fwd_variant;
-    int bwd_variant;
+    std::atomic<int> fwd_variant{0};
+    std::atomic<int> bwd_variant{0};
 };
 const Tuning &tuning();
 

@@ -96,32 +96,21 @@ __global__ __launch_bounds__(256) void access_pattern_kernel(
     }
 }
 
-template <unsigned M>
+template <unsigned M, int NS, int NX, int NZ, int K>
 void launch(const float *x, const float *s, const float *dm, const int32_t *sender, const int32_t *row_ptr,
             const int32_t *row_order, float *ds, float *dx, float *out, int num_nodes, float *sink,
             hipStream_t stream) {
-    constexpr int K = 128;
     const int blocks = ((num_nodes * (K / 64) + 3) / 4 + 7) / 8 * 8;
-    hipLaunchKernelGGL((access_pattern_kernel<M, 23, 16, 99, K>), dim3(blocks), dim3(64, 4), 0, stream, x, s, dm,
+    hipLaunchKernelGGL((access_pattern_kernel<M, NS, NX, NZ, K>), dim3(blocks), dim3(64, 4), 0, stream, x, s, dm,
                        sender, row_ptr, row_order, ds, dx, out, num_nodes, sink);
 }
 
-}  // namespace
-
-// Runs the access pattern `mask` (bits: 1 read s, 2 gather x, 4 write ds, 8 dx atomics, 16 write
-// out, 32 read dm) once on `stream`.  Shapes are those of the 128-channel l<=3 benchmark
-// workload only: s, ds (E, 23, 128); x, dx (N, 16, 128); dm, out (N, 99, 128); row_ptr (N + 1);
-// row_order (N) or null for rows in index order.
-// Buffers of accesses that the mask leaves out may be null; `sink` is one float of scratch.
-// Returns 0, or -1 for a mask that has no instantiation or shapes other than the above.
-extern "C" int e3j_amd_probe_access_pattern(unsigned mask, int num_x, int num_scalars, int num_out, int channels,
-                                            const float *x, const float *s, const float *dm,
-                                            const int32_t *sender, const int32_t *row_ptr,
-                                            const int32_t *row_order, float *ds, float *dx, float *out,
-                                            int num_nodes, float *sink, hipStream_t stream) {
-    if (num_x != 16 || num_scalars != 23 || num_out != 99 || channels != 128 || num_nodes <= 0) return -1;
+template <int NS, int NX, int NZ, int K>
+int run_mask(unsigned mask, const float *x, const float *s, const float *dm, const int32_t *sender,
+             const int32_t *row_ptr, const int32_t *row_order, float *ds, float *dx, float *out, int num_nodes,
+             float *sink, hipStream_t stream) {
 #define E3J_PROBE_CASE(M) \
-    case (M): launch<(M)>(x, s, dm, sender, row_ptr, row_order, ds, dx, out, num_nodes, sink, stream); break;
+    case (M): launch<(M), NS, NX, NZ, K>(x, s, dm, sender, row_ptr, row_order, ds, dx, out, num_nodes, sink, stream); break;
     switch (mask) {
         E3J_PROBE_CASE(kReadS)
         E3J_PROBE_CASE(kReadS | kGatherX)
@@ -137,4 +126,45 @@ extern "C" int e3j_amd_probe_access_pattern(unsigned mask, int num_x, int num_sc
     }
 #undef E3J_PROBE_CASE
     return hipGetLastError() == hipSuccess ? 0 : -1;
+}
+
+template <int NS, int NX, int NZ>
+int run_channels(int channels, unsigned mask, const float *x, const float *s, const float *dm,
+                 const int32_t *sender, const int32_t *row_ptr, const int32_t *row_order, float *ds, float *dx,
+                 float *out, int num_nodes, float *sink, hipStream_t stream) {
+    switch (channels) {
+        case 64: return run_mask<NS, NX, NZ, 64>(mask, x, s, dm, sender, row_ptr, row_order, ds, dx, out, num_nodes, sink, stream);
+        case 128: return run_mask<NS, NX, NZ, 128>(mask, x, s, dm, sender, row_ptr, row_order, ds, dx, out, num_nodes, sink, stream);
+        case 256: return run_mask<NS, NX, NZ, 256>(mask, x, s, dm, sender, row_ptr, row_order, ds, dx, out, num_nodes, sink, stream);
+        default: return -1;
+    }
+}
+
+}  // namespace
+
+// Runs the access pattern `mask` (bits: 1 read s, 2 gather x, 4 write ds, 8 dx atomics, 16 write
+// out, 32 read dm) once on `stream` for operands of the trailing-channels layout: s, ds
+// (E, num_scalars, channels); x, dx (N, num_x, channels); dm, out (N, num_out, channels); row_ptr
+// (N + 1); row_order (N) or null for rows in index order.  The sizes are those of the operands at
+// hand: instantiations exist for the (paths, x, output) dimensions of the tables the library
+// has unrolled kernels for, at 64, 128 and 256 channels.
+// Buffers of accesses that the mask leaves out may be null; `sink` is one float of scratch.
+// Returns 0, or -1 for a mask or a shape without an instantiation.
+extern "C" int e3j_amd_probe_access_pattern(unsigned mask, int num_x, int num_scalars, int num_out, int channels,
+                                            const float *x, const float *s, const float *dm,
+                                            const int32_t *sender, const int32_t *row_ptr,
+                                            const int32_t *row_order, float *ds, float *dx, float *out,
+                                            int num_nodes, float *sink, hipStream_t stream) {
+    if (num_nodes <= 0) return -1;
+#define E3J_PROBE_SHAPE(NS, NX, NZ)                                                                      \
+    if (num_scalars == NS && num_x == NX && num_out == NZ)                                               \
+        return run_channels<NS, NX, NZ>(channels, mask, x, s, dm, sender, row_ptr, row_order, ds, dx, out, \
+                                        num_nodes, sink, stream);
+    E3J_PROBE_SHAPE(23, 16, 99)  // 0e+1o+2e+3o x l<=3 -> l<=3
+    E3J_PROBE_SHAPE(17, 9, 71)   // 0e+1o+2e x l<=3 -> l<=3
+    E3J_PROBE_SHAPE(13, 9, 43)   // 0e+1o+2e x l<=3 -> l<=2
+    E3J_PROBE_SHAPE(7, 4, 21)    // 0e+1o x l<=2 -> l<=2
+    E3J_PROBE_SHAPE(4, 1, 16)    // 0e x l<=3 -> l<=3
+#undef E3J_PROBE_SHAPE
+    return -1;
 }

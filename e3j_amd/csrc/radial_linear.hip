@@ -11,6 +11,8 @@
 // B agree: product j of a lane half takes the inner index g * (inner / 2) + j, so the operands of a
 // lane are contiguous in memory.
 
+#include <initializer_list>
+
 #include "common.h"
 
 namespace e3j_amd {
@@ -646,6 +648,14 @@ int launch_bwd_input(const float *ds, const float *wt, float *dh, int64_t num_ed
     return check_hip(hipGetLastError(), "radial_linear_bwd_input launch");
 }
 
+// The kernels move rows of the operands in 16-byte pieces.
+int check_aligned(const char *what, std::initializer_list<const void *> ptrs) {
+    for (const void *ptr : ptrs)
+        if (reinterpret_cast<uintptr_t>(ptr) % 16 != 0)
+            return set_error(E3J_AMD_INVALID_ARGUMENT, std::string(what) + ": operands must be 16-byte aligned");
+    return E3J_AMD_OK;
+}
+
 int check_shapes(const char *what, int64_t num_edges, int32_t inner, int32_t n) {
     if (num_edges < 0 || inner <= 0 || n <= 0)
         return set_error(E3J_AMD_INVALID_ARGUMENT, std::string(what) + ": bad sizes");
@@ -664,6 +674,7 @@ extern "C" int e3j_amd_radial_linear_fwd(const float *h, const float *w, float *
     if (num_edges == 0) return E3J_AMD_OK;
     if (h == nullptr || w == nullptr || s == nullptr)
         return set_error(E3J_AMD_INVALID_ARGUMENT, "radial_linear: null operand");
+    if (int rc = check_aligned("radial_linear", {h, w, s})) return rc;
     hipStream_t stream = static_cast<hipStream_t>(stream_);
     switch (inner) {
         case 8: return launch_fwd<8>(h, w, s, num_edges, n, stream);
@@ -687,6 +698,7 @@ extern "C" int e3j_amd_radial_linear_bwd_weight(const float *h, const float *ds,
     if (num_edges == 0) return launch_fill_zero(dw, sizeof(float) * (size_t)inner * n, stream);
     if (h == nullptr || ds == nullptr || workspace == nullptr)
         return set_error(E3J_AMD_INVALID_ARGUMENT, "radial_linear_bwd_weight: null operand");
+    if (int rc = check_aligned("radial_linear_bwd_weight", {h, ds, dw, workspace})) return rc;
     float *partial = static_cast<float *>(workspace);
     switch (inner) {
         case 8: return launch_bwd_weight<8>(h, ds, dw, partial, num_edges, n, stream);
@@ -706,6 +718,7 @@ extern "C" int e3j_amd_radial_linear_bwd_input(const float *ds, const float *wt,
     if (num_edges == 0) return E3J_AMD_OK;
     if (ds == nullptr || wt == nullptr || dh == nullptr)
         return set_error(E3J_AMD_INVALID_ARGUMENT, "radial_linear_bwd_input: null operand");
+    if (int rc = check_aligned("radial_linear_bwd_input", {ds, wt, dh})) return rc;
     hipStream_t stream = static_cast<hipStream_t>(stream_);
     return inner == 64 ? launch_bwd_input<64>(ds, wt, dh, num_edges, n, stream)
                        : launch_bwd_input<128>(ds, wt, dh, num_edges, n, stream);

@@ -68,21 +68,47 @@ class _Table:
         self.num_coef = int(self.packed.shape[0])
         self._device = {}
         self._signature = {}
+        self._signed = {}
+
+    #: tables by the identity of the packed array (a module hands over the same array on every
+    #: call): the bytes of a table are hashed once, not per call
+    _by_identity: dict = {}
 
     @classmethod
     def get(cls, coef, val_np_dtype) -> "_Table":
         if isinstance(coef, torch.Tensor):
             raise TypeError("`coef` must be concrete: it is read on the host.")
+        val_key = np.dtype(val_np_dtype).str
+        seen = cls._by_identity.get((id(coef), val_key))
+        if seen is not None and seen[0]() is coef:
+            return seen[1]
         packed = np.asarray(coef)
         if packed.dtype not in (np.dtype(np.uint8), np.dtype(np.int32)):
             raise TypeError(f"unsupported coefficient index dtype {packed.dtype}")
-        key = (packed.dtype.str, packed.shape, packed.tobytes(), np.dtype(val_np_dtype).str)
+        key = (packed.dtype.str, packed.shape, packed.tobytes(), val_key)
         table = cls._cache.get(key)
         if table is None:
             if len(cls._cache) > 256:
                 cls._cache.clear()
             table = cls._cache[key] = cls(packed, val_np_dtype)
+        if isinstance(coef, np.ndarray) and not coef.flags.writeable:
+            # only arrays that cannot change under the cache (modules freeze their packed tables)
+            ident = (id(coef), val_key)
+            if len(cls._by_identity) > 256:
+                cls._by_identity.clear()
+            cls._by_identity[ident] = (weakref.ref(coef, lambda _, k=ident: cls._by_identity.pop(k, None)), table)
         return table
+
+    def signed(self, y_parity) -> "_Table":
+        """The table with the parity signs of y folded in (SENDER ordering), built once per parity."""
+        key = np.asarray(y_parity, dtype=np.float64).tobytes()
+        hit = self._signed.get(key)
+        if hit is None:
+            c = self.unpack()
+            signs = np.asarray(y_parity, dtype=c.val.dtype)[c.idx[:, 2].astype(np.int64)]
+            hit = self._signed[key] = _Table.get(Coef4D(c.val * signs, c.idx, c.val_dtype, c.idx_dtype).pack(),
+                                                 self.val_np_dtype)
+        return hit
 
     def unpack(self) -> Coef4D:
         return Coef4D.unpack(self.packed, self.val_np_dtype)
@@ -195,47 +221,50 @@ def _row_order(other: torch.Tensor, row_ptr: torch.Tensor, n: int):
     return locality_order(other, row_ptr, n, rounds)
 
 
-#: adjacencies prepared for the index tensors seen last (the layers of a model, and the steps
-#: between two neighbour-list rebuilds, pass the same tensors): keyed by the identity and the
-#: in-place version of both tensors, dropped when either tensor dies.
+#: Opt-in (`config(graph_cache=True)`): adjacencies prepared for the index tensors seen last, keyed by
+#: the identity and the in-place version counter of both tensors, dropped when either tensor dies.
+#: The version counter only sees writes that go through torch: a buffer rewritten through its raw
+#: pointer, a DLPack / numpy view or `.data` keeps its version and would get the adjacency of its
+#: old contents.  Callers that reuse an adjacency should hold a `prepare_graph` handle instead.
 _GRAPH_CACHE: dict = {}
 _GRAPH_CACHE_SIZE = 8
 
 
 def clear_graph_cache() -> None:
-    """Forget the prepared adjacencies (the next call prepares its graph again)."""
+    """Forget the cached adjacencies (only filled under `config(graph_cache=True)`)."""
     _GRAPH_CACHE.clear()
 
 
-def _forward_graph(meta: _Meta, sender: torch.Tensor, receiver: torch.Tensor, build: bool = True):
-    """CSR used by the forward kernel: `(other, row_ptr, perm, row_order)`, prepared once per
-    pair of index tensors (`build` off: only looked up, None when it is not there)."""
-    key = (id(sender), id(receiver), sender._version, receiver._version, meta.num_nodes,
-           meta.ordering, config().locality_rounds)
-    hit = _GRAPH_CACHE.get(key)
-    if hit is not None and hit[0]() is sender and hit[1]() is receiver:
-        return hit[2]
-    if not build:
-        return None
-    graph = _prepare_graph(meta, sender, receiver)
-    if len(_GRAPH_CACHE) >= _GRAPH_CACHE_SIZE:
-        _GRAPH_CACHE.pop(next(iter(_GRAPH_CACHE)))
-
-    def evict(_, key=key):
-        _GRAPH_CACHE.pop(key, None)
-
-    _GRAPH_CACHE[key] = (weakref.ref(sender, evict), weakref.ref(receiver, evict), graph)
-    return graph
-
-
-class _Graph:
+class PreparedGraph:
     """A prepared adjacency: CSR (`other`, `row_ptr`), optional permutation of the edge rows,
-    row order and, built on first use, the schedules of the tiled backward."""
+    row order and, built on first use, the schedules of the tiled backward.
 
-    def __init__(self, other, row_ptr, perm, order, num_nodes: int):
+    Returned by `prepare_graph`; valid for as long as the contents of the index tensors it was
+    built from do not change.  It remembers the stream it was prepared on and makes any other
+    stream that uses it wait for the preparation.
+    """
+
+    def __init__(self, other, row_ptr, perm, order, num_nodes: int, ordering=None):
         self.other, self.row_ptr, self.perm, self.order = other, row_ptr, perm, order
         self.num_nodes = int(num_nodes)
+        self.ordering = ordering
         self._schedules = {}
+        self._mark()
+
+    def _mark(self):
+        self.stream = torch.cuda.current_stream(self.row_ptr.device)
+        self.event = torch.cuda.Event()
+        self.event.record(self.stream)
+
+    def ready(self):
+        """Order the current stream after the kernels that prepared this adjacency."""
+        current = torch.cuda.current_stream(self.row_ptr.device)
+        if current != self.stream:
+            current.wait_event(self.event)
+
+    @property
+    def num_edges(self) -> int:
+        return int(self.other.numel())
 
     def __iter__(self):
         return iter((self.other, self.row_ptr, self.perm, self.order))
@@ -246,27 +275,78 @@ class _Graph:
     def schedule(self, tile_rows: int) -> TileSchedule:
         hit = self._schedules.get(tile_rows)
         if hit is None:
+            self.ready()
             hit = self._schedules[tile_rows] = TileSchedule(self.other, self.row_ptr, self.perm, self.order,
                                                             self.num_nodes, tile_rows)
+            self._mark()
         return hit
 
 
-def _prepare_graph(meta: _Meta, sender: torch.Tensor, receiver: torch.Tensor):
-    n = meta.num_nodes
+_Graph = PreparedGraph
+
+
+def prepare_graph(sender: torch.Tensor, receiver: torch.Tensor, num_nodes: int,
+                  graph_ordering=GraphOrdering.RECEIVER) -> PreparedGraph:
+    """Prepare the adjacency of `(sender, receiver)` once, for every call that passes it as `graph=`.
+
+    The counterpart of the reference's per-call `GraphCSR` (`src/e3j/ops/convolution.py:227,426-431`)
+    for callers whose graph outlives one call: the layers of a model, the steps between two
+    neighbour-list rebuilds.  Build a new handle whenever the contents of the index tensors change.
+    """
+    ordering = GraphOrdering.parse(graph_ordering)
+    return _prepare_graph(ordering, int(num_nodes), sender, receiver)
+
+
+def _check_graph(graph: PreparedGraph, meta: "_Meta", num_edges: int) -> None:
+    if graph.num_nodes != meta.num_nodes or graph.num_edges != num_edges:
+        raise ValueError(f"`graph` was prepared for {graph.num_nodes} nodes and {graph.num_edges} edges; the "
+                         f"operands have {meta.num_nodes} and {num_edges}")
+    if graph.ordering is not None and graph.ordering != meta.ordering:
+        raise ValueError(f"`graph` was prepared for {graph.ordering.name} ordering, the call asks for "
+                         f"{meta.ordering.name}")
+
+
+def _forward_graph(meta: _Meta, sender: torch.Tensor, receiver: torch.Tensor, build: bool = True):
+    """Adjacency used by the forward kernel.  Without the opt-in cache it is prepared on every call
+    (`build` off: None, the caller prepares what it needs)."""
+    if not config().graph_cache:
+        return _prepare_graph(meta.ordering, meta.num_nodes, sender, receiver) if build else None
+    key = (id(sender), id(receiver), sender._version, receiver._version, meta.num_nodes,
+           meta.ordering, config().locality_rounds)
+    hit = _GRAPH_CACHE.get(key)
+    if hit is not None and hit[0]() is sender and hit[1]() is receiver:
+        return hit[2]
+    if not build:
+        return None
+    graph = _prepare_graph(meta.ordering, meta.num_nodes, sender, receiver)
+    if len(_GRAPH_CACHE) >= _GRAPH_CACHE_SIZE:
+        _GRAPH_CACHE.pop(next(iter(_GRAPH_CACHE)))
+
+    def evict(_, key=key):
+        _GRAPH_CACHE.pop(key, None)
+
+    _GRAPH_CACHE[key] = (weakref.ref(sender, evict), weakref.ref(receiver, evict), graph)
+    return graph
+
+
+def _prepare_graph(ordering: GraphOrdering, n: int, sender: torch.Tensor, receiver: torch.Tensor) -> PreparedGraph:
     sender_l, receiver_l = wrap_global_index(sender, n), wrap_global_index(receiver, n)
-    if meta.ordering == GraphOrdering.RECEIVER:
+    if ordering == GraphOrdering.RECEIVER:
         other, row_ptr, perm = sender_l.contiguous(), csr_row_ptr(receiver_l, n), None
-    elif meta.ordering == GraphOrdering.SENDER:
+    elif ordering == GraphOrdering.SENDER:
         # aggregate over reversed edges; y parities are folded into the coefficients
         other, row_ptr, perm = receiver_l.contiguous(), csr_row_ptr(sender_l, n), None
     else:
         perm, other, row_ptr = sort_edges(receiver_l, sender_l, n)
-    return _Graph(other, row_ptr, perm, _row_order(other, row_ptr, n), n)
+    return PreparedGraph(other, row_ptr, perm, _row_order(other, row_ptr, n), n, ordering)
 
 
 def _raw_forward(meta: _Meta, x, y, s, sender, receiver, graph=None) -> torch.Tensor:
     x, y, s = x.contiguous(), y.contiguous(), s.contiguous()
-    other, row_ptr, perm, order = graph if graph is not None else _forward_graph(meta, sender, receiver)
+    if graph is None:
+        graph = _forward_graph(meta, sender, receiver)
+    graph.ready()
+    other, row_ptr, perm, order = graph
     # SENDER ordering: the table carries the parity signs of y (unrolled kernels take them as
     # a sign mask on the unsigned built-in table instead)
     p, table = _fill_params(meta, x, y, s, meta.signed_table or meta.table, row_order=order)
@@ -308,6 +388,8 @@ def _raw_backward(meta: _Meta, x, y, s, dm, sender, receiver, graph=None):
     reuse = graph is not None and (
         (forward_rows and (not deterministic or ordered)) or sender_rows)
     prepared = None  # the receiver-grouped adjacency as an object that keeps tile schedules
+    if graph is not None:
+        graph.ready()
     if reuse:
         other, row_ptr, perm, order = graph
         group_receiver = not sender_rows
@@ -339,7 +421,7 @@ def _raw_backward(meta: _Meta, x, y, s, dm, sender, receiver, graph=None):
     with torch.cuda.device(x.device):
         if tile_rows >= 2:
             if prepared is None:
-                prepared = _Graph(other, row_ptr, perm, order, n)
+                prepared = PreparedGraph(other, row_ptr, perm, order, n)
             schedule = prepared.schedule(tile_rows)
             _lib.check(lib.e3j_amd_convolution_bwd_tiled(
                 ctypes.byref(p), x.data_ptr(), y.data_ptr(), s.data_ptr(), dm.data_ptr(), other.data_ptr(),
@@ -498,9 +580,7 @@ def _make_meta(coef, x, y, s, params, graph_ordering, y_parity, layout) -> _Meta
     if ordering == GraphOrdering.SENDER:
         if y_parity is None:
             raise ValueError("SENDER graph ordering requires `y_parity`.")
-        c = table.unpack()
-        signs = np.asarray(y_parity, dtype=c.val.dtype)[c.idx[:, 2].astype(np.int64)]
-        signed = _Table.get(Coef4D(c.val * signs, c.idx, c.val_dtype, c.idx_dtype).pack(), val_np)
+        signed = table.signed(y_parity)
     return _Meta(table=table, signed_table=signed, params=params, ordering=ordering, layout=layout,
                  y_parity=None if y_parity is None else np.asarray(y_parity),
                  num_nodes=int(x.shape[0]), squeeze_channels=False, y_shape=tuple(y.shape))
@@ -528,7 +608,7 @@ def _canonical(x, y, s, layout: Layout):
 
 def convolution(coef, x, y, s, sender, receiver, params: ConvolutionParams,
                 graph_ordering=GraphOrdering.RECEIVER, y_parity=None, *,
-                layout=Layout.TRAILING_CHANNELS) -> torch.Tensor:
+                layout=Layout.TRAILING_CHANNELS, graph: PreparedGraph | None = None) -> torch.Tensor:
     """`out[r] = sum_{e: recv(e)=r} (x[send(e)] (x) y[e]) . s[e]` with the fused HIP kernels.
 
     Args:
@@ -540,14 +620,18 @@ def convolution(coef, x, y, s, sender, receiver, params: ConvolutionParams,
             Sorted by receiver (RECEIVER) or sender (SENDER), or in any order (NONE).
         params: `ConvolutionParams(num_out, num_scalars)`.
         y_parity: per-`y`-component parity, required under SENDER ordering.
+        graph: optional handle from `prepare_graph(sender, receiver, num_nodes, graph_ordering)`; the
+            adjacency is then not prepared again (forward and backward).
     """
     _check_operands(x, y, s, sender, receiver)
     layout = Layout.parse(layout)
-    y_in_shape = tuple(y.shape)
     x3, y2, s3, squeeze = _canonical(x, y, s, layout)
     meta = _make_meta(coef, x3, y2, s3, params, graph_ordering, y_parity, layout)
-    out = _Convolution.apply(x3, y2, s3, sender, receiver, meta, None)
-    del y_in_shape
+    if graph is not None:
+        _check_graph(graph, meta, int(y2.shape[0]))
+    else:  # prepared here, so that the backward pass finds it in its context
+        graph = _forward_graph(meta, sender, receiver)
+    out = _Convolution.apply(x3, y2, s3, sender, receiver, meta, graph)
     if squeeze:
         out = out.squeeze(-1 if layout == Layout.TRAILING_CHANNELS else 1)
     return out
@@ -555,7 +639,7 @@ def convolution(coef, x, y, s, sender, receiver, params: ConvolutionParams,
 
 def convolution_bwd(coef, x, y, s, sender, receiver, dm, params: ConvolutionParams,
                     graph_ordering=GraphOrdering.RECEIVER, y_parity=None, *,
-                    layout=Layout.TRAILING_CHANNELS):
+                    layout=Layout.TRAILING_CHANNELS, graph: PreparedGraph | None = None):
     """Cotangents `(dx, dy, ds)` of `convolution` for the output cotangent `dm`."""
     _check_operands(x, y, s, sender, receiver)
     layout = Layout.parse(layout)
@@ -563,7 +647,9 @@ def convolution_bwd(coef, x, y, s, sender, receiver, dm, params: ConvolutionPara
     x3, y2, s3, squeeze = _canonical(x, y, s, layout)
     dm3 = dm.unsqueeze(-1 if layout == Layout.TRAILING_CHANNELS else 1) if squeeze else dm
     meta = _make_meta(coef, x3, y2, s3, params, graph_ordering, y_parity, layout)
-    dx, dy, ds = _ConvolutionBwd.apply(x3, y2, s3, dm3, sender, receiver, meta, None)
+    if graph is not None:
+        _check_graph(graph, meta, int(y2.shape[0]))
+    dx, dy, ds = _ConvolutionBwd.apply(x3, y2, s3, dm3, sender, receiver, meta, graph)
     if squeeze:
         axis = -1 if layout == Layout.TRAILING_CHANNELS else 1
         dx = dx.squeeze(axis)

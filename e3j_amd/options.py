@@ -99,6 +99,11 @@ class Config:
     #: sweeps of label propagation behind the locality-aware row order of the kernels
     #: (0 = rows are processed in index order).
     locality_rounds: int = 2
+    #: keep the adjacencies prepared for the index tensors seen last and reuse them when the same
+    #: tensors (identity and in-place version) come again.  Off by default: a buffer rewritten behind
+    #: torch's back (raw pointer, DLPack, `.data`) would get a stale adjacency; `prepare_graph`
+    #: handles are the explicit way to reuse one.
+    graph_cache: bool = False
     #: receivers per tile of the backward that sums dx per (tile, sender) on chip before the float
     #: atomics and shares long rows between workgroups (trailing layout, unrolled kernels, at least
     #: 64 channels; capped by what the LDS holds); 0 or 1 = one wave per receiver and one set of
@@ -119,6 +124,7 @@ class _ConfigHolder:
             deterministic=os.environ.get("E3J_AMD_DETERMINISTIC", "0") not in ("0", ""),
             locality_rounds=int(os.environ.get("E3J_AMD_LOCALITY_ROUNDS", "2")),
             tile_rows=int(os.environ.get("E3J_AMD_TILE_ROWS", "0")),
+            graph_cache=os.environ.get("E3J_AMD_GRAPH_CACHE", "0") not in ("0", ""),
             jit=os.environ.get("E3J_AMD_JIT", "0") not in ("0", ""),
         )
 

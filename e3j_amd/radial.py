@@ -24,10 +24,16 @@ def supported(h: torch.Tensor, w: torch.Tensor) -> bool:
             and int(w.shape[1]) % 32 == 0)
 
 
+def _aligned(t: torch.Tensor) -> torch.Tensor:
+    """Contiguous and 16-byte aligned (a contiguous view at an odd element offset is copied)."""
+    t = t.contiguous()
+    return t if t.data_ptr() % 16 == 0 else t.clone()
+
+
 class _RadialLinear(torch.autograd.Function):
     @staticmethod
     def forward(h, w):
-        h, w = h.contiguous(), w.contiguous()
+        h, w = _aligned(h), _aligned(w)
         s = torch.empty((h.shape[0], w.shape[1]), dtype=h.dtype, device=h.device)
         with torch.cuda.device(h.device):
             _lib.check(_lib.load().e3j_amd_radial_linear_fwd(
@@ -53,7 +59,7 @@ def _input_gradient(ds: torch.Tensor, w: torch.Tensor) -> torch.Tensor:
     if (int(w.shape[0]) < 64 or ds.dtype != torch.float32
             or torch.is_grad_enabled() and (ds.requires_grad or w.requires_grad)):
         return ds @ w.t()
-    ds, wt = ds.contiguous(), w.t().contiguous()
+    ds, wt = _aligned(ds), w.t().contiguous()
     dh = torch.empty((ds.shape[0], w.shape[0]), dtype=ds.dtype, device=ds.device)
     with torch.cuda.device(ds.device):
         _lib.check(_lib.load().e3j_amd_radial_linear_bwd_input(
@@ -68,7 +74,7 @@ def _weight_gradient(h: torch.Tensor, ds: torch.Tensor) -> torch.Tensor:
     if torch.is_grad_enabled() and (h.requires_grad or ds.requires_grad) or ds.dtype != torch.float32:
         return h.t() @ ds
     lib = _lib.load()
-    h, ds = h.contiguous(), ds.contiguous()
+    h, ds = _aligned(h), _aligned(ds)
     edges, inner, n = int(h.shape[0]), int(h.shape[1]), int(ds.shape[1])
     dw = torch.empty((inner, n), dtype=h.dtype, device=h.device)
     ws = torch.empty(max(int(lib.e3j_amd_radial_linear_bwd_weight_workspace_bytes(edges, inner, n)), 4),

@@ -302,10 +302,17 @@ class EnergyModel:
         return self.harmonics(vec / r[:, None]), self.radial_basis(r)
 
     def convolve(self, layer, x, y, s, sender, receiver):
-        return self.layers[layer](x, y, s, sender, receiver)
+        # one adjacency for all layers of a step
+        held = getattr(self, "_prepared", None)
+        if x.is_cuda and (held is None or held[0] is not sender or held[1] is not receiver):
+            from .ops import prepare_graph
+            held = self._prepared = (sender, receiver, prepare_graph(sender, receiver, x.shape[0],
+                                                                     self.layers[layer].graph_ordering))
+        return self.layers[layer](x, y, s, sender, receiver, graph=held[2] if x.is_cuda else None)
 
     def energy(self, positions, node_features, sender, receiver, shift, convolve=None):
         convolve = convolve or self.convolve
+        self._prepared = None   # the neighbour list may have been rewritten in place since the last step
         y, basis = self.edge_inputs(positions, sender, receiver, shift)
         x = node_features
         for layer, (w1, w2) in enumerate(self.mlp):

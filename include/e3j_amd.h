@@ -26,6 +26,11 @@
  *    synchronised before returning so device faults surface at the call
  *    (lib/e3j_ops/cuda/convolution/launch_fwd.cuh:255-263).
  *  - Rows of nodes without live edges are written as exact zeros.
+ *  - Alignment: any element-aligned pointer is accepted by the forward and the two grouped
+ *    backwards; the compile-time-unrolled kernels are used when x, s, out / dm, dx and ds are
+ *    16-byte aligned (true of whole allocations), otherwise the table-driven kernels run (which
+ *    then need `coef`).  The ordered and tiled backwards and e3j_amd_radial_linear_* require
+ *    16-byte aligned operands and return E3J_AMD_INVALID_ARGUMENT otherwise.
  */
 #ifndef E3J_AMD_H_
 #define E3J_AMD_H_
@@ -189,7 +194,8 @@ int e3j_amd_find_signature(const void *coef_host, int32_t coef_idx_bytes, int32_
 /* Tuning aid: selects which launch shape (channels per lane, waves per block, parts) of a
  * signature's kernels later calls use; 0 = default, unknown numbers = default.  The
  * environment variables E3J_AMD_FWD_VARIANT / E3J_AMD_BWD_VARIANT give the initial values.
- * Process-wide and not synchronised with running calls.  Results do not depend on it.
+ * Process-wide; may be called from any thread while other threads launch (each launch reads the
+ * numbers once, atomically, and uses the old or the new shape).  Results do not depend on it.
  * No counterpart in the reference, whose launch shape is planned on the host per call
  * (src/e3j/ops/convolution.py:178-208). */
 void e3j_amd_set_launch_variant(int32_t fwd_variant, int32_t bwd_variant);

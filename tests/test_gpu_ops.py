@@ -287,26 +287,81 @@ def test_operator_errors():
         convolution(p["coef"], x.bfloat16(), y.bfloat16(), s.bfloat16(), snd, rcv, p["params"])
 
 
-def test_prepared_graph_is_reused_per_index_tensor_pair_and_follows_in_place_changes():
+def test_opt_in_cache_reuses_per_index_tensor_pair_and_follows_in_place_changes():
+    import e3j_amd
     from e3j_amd import ops
     p = _problem(8, N=20, E=200, K=16)
     x, y, s = (dev(p[k]) for k in ("x", "y", "s"))
     snd, rcv = dev(p["snd"]), dev(p["rcv"])
     ops.clear_graph_cache()
-    first = convolution(p["coef"], x, y, s, snd, rcv, p["params"])
-    assert len(ops._GRAPH_CACHE) == 1
-    again = convolution(p["coef"], x, y, s, snd, rcv, p["params"])
-    assert len(ops._GRAPH_CACHE) == 1 and torch.equal(first, again)
-    # an in-place change of the senders must not be served from the cache
-    snd[:] = torch.roll(snd, 1)
-    changed = convolution(p["coef"], x, y, s, snd, rcv, p["params"])
-    ref, mag = H.forward_reference(p["idx"], p["val"], p["mix"], p["x"], p["y"], p["s"],
-                                   np.roll(p["snd"], 1), p["rcv"], p["params"].num_out)
-    H.assert_parity(changed.cpu().numpy(), ref, mag, "after in-place change")
-    del snd, rcv
-    import gc
-    gc.collect()
-    assert len(ops._GRAPH_CACHE) == 0                      # entries die with their tensors
+    convolution(p["coef"], x, y, s, snd, rcv, p["params"])
+    assert len(ops._GRAPH_CACHE) == 0                      # off unless asked for
+    with e3j_amd.config.use(graph_cache=True):
+        first = convolution(p["coef"], x, y, s, snd, rcv, p["params"])
+        assert len(ops._GRAPH_CACHE) == 1
+        again = convolution(p["coef"], x, y, s, snd, rcv, p["params"])
+        assert len(ops._GRAPH_CACHE) == 1 and torch.equal(first, again)
+        # an in-place change of the senders through torch must not be served from the cache
+        snd[:] = torch.roll(snd, 1)
+        changed = convolution(p["coef"], x, y, s, snd, rcv, p["params"])
+        ref, mag = H.forward_reference(p["idx"], p["val"], p["mix"], p["x"], p["y"], p["s"],
+                                       np.roll(p["snd"], 1), p["rcv"], p["params"].num_out)
+        H.assert_parity(changed.cpu().numpy(), ref, mag, "after in-place change")
+        del snd, rcv
+        import gc
+        gc.collect()
+        assert len(ops._GRAPH_CACHE) == 0                  # entries die with their tensors
+
+
+def test_index_buffer_rewritten_behind_the_version_counter():
+    """A neighbour list rewritten through `.data` (or a raw pointer) keeps its version counter: the
+    default path prepares the adjacency on every call and follows the new contents; a
+    `prepare_graph` handle is rebuilt by its owner."""
+    from e3j_amd import prepare_graph
+    p = _problem(9, N=24, E=240, K=16)
+    x, y, s = (dev(p[k], grad=True) for k in ("x", "y", "s"))
+    snd, rcv = dev(p["snd"]), dev(p["rcv"])
+    dm = dev(p["dm"])
+
+    def check(out, grads, senders, what):
+        ref, mag = H.forward_reference(p["idx"], p["val"], p["mix"], p["x"], p["y"], p["s"], senders, p["rcv"],
+                                       p["params"].num_out)
+        H.assert_parity(out.detach().cpu().numpy(), ref, mag, what + " out")
+        refs, mags = H.backward_reference(p["idx"], p["val"], p["mix"], p["x"], p["y"], p["s"], senders, p["rcv"],
+                                          p["dm"])
+        for g, r, m, name in zip(grads, refs, mags, ("dx", "dy", "ds")):
+            H.assert_parity(g.cpu().numpy(), r, m, f"{what} {name}")
+
+    out = convolution(p["coef"], x, y, s, snd, rcv, p["params"])
+    check(out, torch.autograd.grad(out, (x, y, s), dm), p["snd"], "before")
+    version = snd._version
+    rolled = np.roll(p["snd"], 3)
+    snd.data.copy_(torch.as_tensor(rolled))                # rewritten behind the version counter
+    assert snd._version == version
+    out = convolution(p["coef"], x, y, s, snd, rcv, p["params"])
+    check(out, torch.autograd.grad(out, (x, y, s), dm), rolled, "after the rewrite")
+    # the explicit handle: one preparation for forward and backward of several calls
+    handle = prepare_graph(snd, rcv, 24)
+    for _ in range(2):
+        out = convolution(p["coef"], x, y, s, snd, rcv, p["params"], graph=handle)
+        check(out, torch.autograd.grad(out, (x, y, s), dm), rolled, "with a handle")
+    with pytest.raises(ValueError, match="prepared for"):
+        convolution(p["coef"], x, y, s, snd[:-1], rcv[:-1], p["params"], graph=handle)
+
+
+def test_prepared_graph_used_on_another_stream_waits_for_its_preparation():
+    from e3j_amd import prepare_graph
+    p = _problem(10, N=2000, E=60000, K=16)
+    x, y, s = (dev(p[k]) for k in ("x", "y", "s"))
+    snd, rcv = dev(p["snd"]), dev(p["rcv"])
+    want = convolution(p["coef"], x, y, s, snd, rcv, p["params"])
+    torch.cuda.synchronize()
+    side = torch.cuda.Stream()
+    handle = prepare_graph(snd, rcv, 2000)                 # prepared on the current stream, not waited for
+    with torch.cuda.stream(side):
+        got = convolution(p["coef"], x, y, s, snd, rcv, p["params"], graph=handle)
+    side.synchronize()
+    assert torch.equal(got, want)
 
 
 def test_tables_without_an_unrolled_kernel_warn_once():

@@ -334,3 +334,38 @@ def test_padding_edges_with_poisoned_features_never_reach_the_results(layout):
     emptied = [int(r) for r in last_rows if not bool((d.receiver[:tail] == r).any())]
     for r in emptied:
         assert not out[r].any()
+
+
+def test_views_at_odd_element_offsets_are_served():
+    """Operands that are only 4-byte aligned (contiguous views one element into an allocation)
+    are outside what the unrolled kernels' 16-byte row pieces take: the operators serve them
+    with the table-driven kernels, with the same results."""
+    w = CASES["cfg2"]()
+    d = w.to("cuda")
+    m = w.module
+    coef = m._packed_coef("float32")
+
+    def shifted(t):
+        flat = torch.empty(t.numel() + 1, dtype=t.dtype, device=t.device)
+        view = flat[1:].view(t.shape)
+        view.copy_(t)
+        assert view.data_ptr() % 16 == 4 and view.is_contiguous()
+        return view
+
+    want = e3j_amd.convolution(coef, d.x, d.y, d.s, d.sender, d.receiver, m.params, m.graph_ordering)
+    want_g = e3j_amd.convolution_bwd(coef, d.x, d.y, d.s, d.sender, d.receiver, d.dm, m.params, m.graph_ordering)
+    got = e3j_amd.convolution(coef, shifted(d.x), d.y, shifted(d.s), d.sender, d.receiver, m.params, m.graph_ordering)
+    got_g = e3j_amd.convolution_bwd(coef, shifted(d.x), d.y, shifted(d.s), d.sender, d.receiver, shifted(d.dm),
+                                    m.params, m.graph_ordering)
+    torch.testing.assert_close(got, want, rtol=2e-5, atol=2e-5)
+    for a, b in zip(got_g, want_g):
+        torch.testing.assert_close(a, b, rtol=2e-5, atol=2e-5 * float(b.abs().max()))
+    # the entry points that have no table-driven form refuse such operands
+    from e3j_amd.radial import radial_linear
+    h = torch.randn(256, 32, device="cuda")
+    wt = torch.randn(32, 64, device="cuda")
+    torch.testing.assert_close(radial_linear(shifted(h), wt), h @ wt, rtol=1e-5, atol=1e-5)
+    s_out = torch.empty(256 * 64 + 1, device="cuda")
+    rc = _lib.load().e3j_amd_radial_linear_fwd(shifted(h).data_ptr(), wt.data_ptr(), s_out.data_ptr(), 256, 32, 64,
+                                               int(torch.cuda.current_stream().cuda_stream))
+    assert rc == _lib.INVALID_ARGUMENT and b"16-byte" in _lib.load().e3j_amd_last_error()
