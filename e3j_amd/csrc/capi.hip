@@ -7,7 +7,9 @@
 #include <cstdint>
 #include <deque>
 #include <initializer_list>
+#include <algorithm>
 #include <mutex>
+#include <vector>
 
 #include "common.h"
 
@@ -158,6 +160,91 @@ int run_backward(const e3j_amd_conv_params *p, bool group_is_receiver, const voi
                                 dx, dy, ds, stream, coef_cols_ji);
     }
     return finish(p, stream, rc, op);
+}
+
+// ---- table lookup ---------------------------------------------------------------------------
+std::vector<TableEntry> unpack_entries(const void *packed, int32_t coef_idx_bytes, int32_t num_coef,
+                                       bool columns_ji) {
+    const size_t item = coef_idx_bytes == 1 ? sizeof(Coef4D<uint8_t, float>) : sizeof(Coef4D<int32_t, float>);
+    const unsigned char *bytes = static_cast<const unsigned char *>(packed);
+    std::vector<TableEntry> entries((size_t)num_coef);
+    for (int n = 0; n < num_coef; n++) {
+        TableEntry &e = entries[n];
+        std::memcpy(&e.val, bytes + n * item, sizeof(float));
+        for (int t = 0; t < 4; t++) {
+            if (coef_idx_bytes == 1) e.idx[t] = bytes[n * item + 4 + t];
+            else std::memcpy(&e.idx[t], bytes + n * item + 4 + 4 * t, 4);
+        }
+        if (columns_ji) std::swap(e.idx[0], e.idx[1]);  // (j, i, k, l) of a dx table -> (i, j, k, l)
+    }
+    return entries;
+}
+
+namespace {
+bool entry_less(const TableEntry &a, const TableEntry &b) {
+    for (int t = 0; t < 4; t++)
+        if (a.idx[t] != b.idx[t]) return a.idx[t] < b.idx[t];
+    return false;
+}
+}  // namespace
+
+// The tables are compared as sets of entries (both sorted by their coordinates): the reference
+// permutes the rows of a table when it balances them over warps (src/e3j/ops/convolution.py:178-208).
+int match_signature(std::vector<TableEntry> entries, int32_t num_x, int32_t num_y, int32_t num_out,
+                    int32_t num_scalars, int32_t channels, int32_t layout, float *coef_scale,
+                    uint32_t *y_flip) {
+    if (coef_scale) *coef_scale = 1.0f;
+    if (y_flip) *y_flip = 0;
+    const int num_coef = (int)entries.size();
+    if (num_coef == 0) return -1;
+    std::stable_sort(entries.begin(), entries.end(), entry_less);
+    const bool signs_allowed = y_flip != nullptr && num_y <= 32;
+    std::vector<TableEntry> own((size_t)num_coef);
+    for (int id = 0; id < num_signatures(); id++) {
+        const Signature &sg = signature(id);
+        if (sg.num_coef != num_coef || sg.num_x != num_x || sg.num_y != num_y ||
+            sg.num_out != num_out || sg.num_scalars != num_scalars || sg.channels != channels ||
+            sg.layout != layout)
+            continue;
+        for (int n = 0; n < num_coef; n++) {
+            own[n].val = sg.val[n];
+            for (int t = 0; t < 4; t++) own[n].idx[t] = sg.idx[4 * n + t];
+        }
+        std::stable_sort(own.begin(), own.end(), entry_less);
+        // One uniform positive factor is allowed between the tables; its magnitude is taken
+        // from the entry of largest magnitude and every entry must agree to float32 rounding.
+        // A negative ratio is a sign flip of that entry's y component, which must then hold
+        // for every entry of the component.
+        int big = 0;
+        for (int n = 1; n < num_coef; n++)
+            if (std::fabs(own[n].val) > std::fabs(own[big].val)) big = n;
+        const double scale = std::fabs((double)entries[big].val / (double)own[big].val);
+        bool same = scale > 0.0 && std::isfinite(scale);
+        uint32_t flip = 0, seen = 0;
+        for (int n = 0; n < num_coef && same; n++) {
+            const int32_t *idx = entries[n].idx;
+            for (int t = 0; t < 4 && same; t++) same = idx[t] == own[n].idx[t];
+            if (!same) break;
+            const double v = entries[n].val, want = scale * (double)own[n].val;
+            const bool plus = std::fabs(v - want) <= 4e-7 * std::fabs(want);
+            const bool minus = std::fabs(v + want) <= 4e-7 * std::fabs(want);
+            if (plus) {
+                same = !signs_allowed || !((seen >> idx[2]) & 1u) || !((flip >> idx[2]) & 1u);
+            } else if (minus && signs_allowed) {
+                same = !((seen >> idx[2]) & 1u) || ((flip >> idx[2]) & 1u);
+                flip |= 1u << idx[2];
+            } else {
+                same = false;
+            }
+            if (signs_allowed) seen |= 1u << idx[2];
+        }
+        if (same) {
+            if (coef_scale) *coef_scale = (float)scale;
+            if (y_flip) *y_flip = flip;
+            return id;
+        }
+    }
+    return -1;
 }
 
 }  // namespace e3j_amd
@@ -371,57 +458,8 @@ int e3j_amd_find_signature(const void *coef_host, int32_t coef_idx_bytes, int32_
     if (y_flip) *y_flip = 0;
     if (coef_host == nullptr || val_dtype != E3J_AMD_F32 || num_coef <= 0) return -1;
     if (coef_idx_bytes != 1 && coef_idx_bytes != 4) return -1;
-    const size_t item = coef_idx_bytes == 1 ? sizeof(Coef4D<uint8_t, float>) : sizeof(Coef4D<int32_t, float>);
-    const unsigned char *bytes = static_cast<const unsigned char *>(coef_host);
-    const bool signs_allowed = y_flip != nullptr && num_y <= 32;
-    for (int id = 0; id < num_signatures(); id++) {
-        const Signature &sg = signature(id);
-        if (sg.num_coef != num_coef || sg.num_x != num_x || sg.num_y != num_y ||
-            sg.num_out != num_out || sg.num_scalars != num_scalars || sg.channels != channels ||
-            sg.layout != layout)
-            continue;
-        // One uniform positive factor is allowed between the tables; its magnitude is taken
-        // from the entry of largest magnitude and every entry must agree to float32 rounding.
-        // A negative ratio is a sign flip of that entry's y component, which must then hold
-        // for every entry of the component.
-        int big = 0;
-        for (int n = 1; n < num_coef; n++)
-            if (std::fabs(sg.val[n]) > std::fabs(sg.val[big])) big = n;
-        float vbig;
-        std::memcpy(&vbig, bytes + big * item, sizeof(float));
-        const double scale = std::fabs((double)vbig / (double)sg.val[big]);
-        bool same = scale > 0.0 && std::isfinite(scale);
-        uint32_t flip = 0, seen = 0;
-        for (int n = 0; n < num_coef && same; n++) {
-            float v;
-            int32_t idx[4];
-            std::memcpy(&v, bytes + n * item, sizeof(float));
-            for (int t = 0; t < 4; t++) {
-                if (coef_idx_bytes == 1) idx[t] = bytes[n * item + 4 + t];
-                else std::memcpy(&idx[t], bytes + n * item + 4 + 4 * t, 4);
-            }
-            for (int t = 0; t < 4 && same; t++) same = idx[t] == (int32_t)sg.idx[4 * n + t];
-            if (!same) break;
-            const double want = scale * (double)sg.val[n];
-            const bool plus = std::fabs((double)v - want) <= 4e-7 * std::fabs(want);
-            const bool minus = std::fabs((double)v + want) <= 4e-7 * std::fabs(want);
-            if (plus) {
-                same = !signs_allowed || !((seen >> idx[2]) & 1u) || !((flip >> idx[2]) & 1u);
-            } else if (minus && signs_allowed) {
-                same = !((seen >> idx[2]) & 1u) || ((flip >> idx[2]) & 1u);
-                flip |= 1u << idx[2];
-            } else {
-                same = false;
-            }
-            if (signs_allowed) seen |= 1u << idx[2];
-        }
-        if (same) {
-            if (coef_scale) *coef_scale = (float)scale;
-            if (y_flip) *y_flip = flip;
-            return id;
-        }
-    }
-    return -1;
+    const std::vector<TableEntry> entries = unpack_entries(coef_host, coef_idx_bytes, num_coef, false);
+    return match_signature(entries, num_x, num_y, num_out, num_scalars, channels, layout, coef_scale, y_flip);
 }
 
 }  // extern "C"

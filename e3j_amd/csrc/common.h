@@ -7,6 +7,7 @@
 
 #include <atomic>
 #include <string>
+#include <vector>
 
 #include "../../include/e3j_amd.h"
 
@@ -123,6 +124,11 @@ struct OrderedBwd {
 // range), INT32_MAX otherwise (graph.hip).
 int launch_live_keys(const int32_t *other, const int32_t *row_ptr, int32_t num_nodes,
                      int64_t num_edges, int32_t *keys, hipStream_t stream);
+// rows[pos] = CSR row of every position (INT32_MAX past the last row); out[i] = inner[outer[i]]
+// (inner null: identity) (graph.hip).
+int launch_expand_rows(const int32_t *row_ptr, int32_t num_nodes, int64_t num_edges, int32_t *rows,
+                       hipStream_t stream);
+int launch_compose_perm(const int32_t *outer, const int32_t *inner, int64_t n, int32_t *out, hipStream_t stream);
 int reduce_ordered_dx(const e3j_amd_conv_params &p, const float *u, const int32_t *sender_ptr,
                       const int32_t *sender_pos, unsigned long long covered, float *dx,
                       hipStream_t stream);
@@ -151,6 +157,17 @@ struct Signature {
     int (*tile_row_bytes)();
 };
 // built-in signatures (generated/registry.hip), then the ones registered at run time (capi.hip)
+// A table entry on the host, and the lookup of a table among the signatures (capi.hip): the
+// tables are compared as sets of entries, up to one positive factor and one sign per y component.
+struct TableEntry {
+    float val;
+    int32_t idx[4];  // i, j, k, l
+};
+std::vector<TableEntry> unpack_entries(const void *packed_host, int32_t coef_idx_bytes, int32_t num_coef,
+                                       bool columns_ji);
+int match_signature(std::vector<TableEntry> entries, int32_t num_x, int32_t num_y, int32_t num_out,
+                    int32_t num_scalars, int32_t channels, int32_t layout, float *coef_scale,
+                    uint32_t *y_flip);
 int num_builtin_signatures();
 const Signature &builtin_signature(int id);
 int num_signatures();

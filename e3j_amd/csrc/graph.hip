@@ -277,6 +277,30 @@ struct TileWorkspace {
     }
 };
 
+
+// rows[pos] = the CSR row that holds position pos; INT32_MAX past the last row
+__global__ void expand_rows_kernel(const int32_t *__restrict__ row_ptr, int num_nodes, int64_t num_edges,
+                                   int32_t *__restrict__ rows) {
+    const int64_t live_end = row_ptr[num_nodes];
+    const int64_t stride = (int64_t)gridDim.x * blockDim.x;
+    for (int64_t pos = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; pos < num_edges; pos += stride) {
+        if (pos >= live_end) { rows[pos] = INT32_MAX; continue; }
+        int lo = 0, hi = num_nodes;  // row_ptr[lo] <= pos < row_ptr[hi]
+        while (hi - lo > 1) {
+            const int mid = (lo + hi) >> 1;
+            if (row_ptr[mid] <= pos) lo = mid; else hi = mid;
+        }
+        rows[pos] = lo;
+    }
+}
+
+__global__ void compose_perm_kernel(const int32_t *__restrict__ outer, const int32_t *__restrict__ inner,
+                                    int64_t n, int32_t *__restrict__ out) {
+    const int64_t stride = (int64_t)gridDim.x * blockDim.x;
+    for (int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; i < n; i += stride)
+        out[i] = inner ? inner[outer[i]] : outer[i];
+}
+
 }  // namespace
 
 int launch_live_keys(const int32_t *other, const int32_t *row_ptr, int32_t num_nodes,
@@ -285,6 +309,20 @@ int launch_live_keys(const int32_t *other, const int32_t *row_ptr, int32_t num_n
     hipLaunchKernelGGL(live_keys_kernel, dim3(grid_for(num_edges)), dim3(256), 0, stream, other, row_ptr,
                        num_nodes, num_edges, keys);
     return check_hip(hipGetLastError(), "live keys launch");
+}
+
+int launch_expand_rows(const int32_t *row_ptr, int32_t num_nodes, int64_t num_edges, int32_t *rows,
+                       hipStream_t stream) {
+    if (num_edges == 0) return E3J_AMD_OK;
+    hipLaunchKernelGGL(expand_rows_kernel, dim3(grid_for(num_edges)), dim3(256), 0, stream, row_ptr, num_nodes,
+                       num_edges, rows);
+    return check_hip(hipGetLastError(), "expand rows launch");
+}
+
+int launch_compose_perm(const int32_t *outer, const int32_t *inner, int64_t n, int32_t *out, hipStream_t stream) {
+    if (n == 0) return E3J_AMD_OK;
+    hipLaunchKernelGGL(compose_perm_kernel, dim3(grid_for(n)), dim3(256), 0, stream, outer, inner, n, out);
+    return check_hip(hipGetLastError(), "compose permutation launch");
 }
 
 }  // namespace e3j_amd

@@ -13,8 +13,11 @@
 // a fourth, "convolution_bwd_ordered", the same operands and a scratch buffer as a fourth
 // result (the atomic-free, bit-reproducible backward).
 // Attributes: num_nodes, debug (reference); layout, signature, coef_scale, y_flip,
-// coef_stacked (optional).  Handlers are re-entrant, allocate nothing and
-// enqueue on the stream XLA hands over; they answer the metadata query.
+// coef_stacked (optional).  Without `signature` the handler finds the kernels of the table the
+// frame carries (see TableResolver).  Handlers are re-entrant (the only shared state is that
+// lookup, behind a mutex), allocate nothing themselves ("convolution_bwd" borrows scratch from the
+// runtime through XLA_FFI_DeviceMemory_Allocate when it runs the unrolled kernels) and enqueue
+// on the stream XLA hands over; they answer the metadata query.
 //
 // The row-wise tensor product (lib/e3j_ops/ffi/e3j_ops.h:124-253,258-372):
 //   "tensor_product":      coef, x, y [, coef_ranges] -> z;  attrs num_out, mode, layout, debug
@@ -22,6 +25,10 @@
 // plus the optional attributes signature, coef_scale and coef_sorted (default 1).
 
 #include <cstring>
+#include <map>
+#include <mutex>
+#include <tuple>
+#include <vector>
 
 #include "common.h"
 #include "xla_ffi_abi.h"
@@ -100,6 +107,106 @@ T attr(const XlaCallFrame *f, const char *name, int32_t dtype, T fallback, bool 
     return fallback;
 }
 
+// ---- which unrolled kernels serve the table of a frame ----------------------------------------
+// The reference's frames carry the coefficient table as a device buffer and no kernel id
+// (src/e3j/ops/convolution.py:229-242,433-452).  The handler reads the table back (a few KB) on a
+// stream of its own, which waits for nothing of the caller's work, and looks it up among the
+// signatures; the answer is remembered under the table's bytes.  Under stream capture nothing
+// may be read back: the answer a previous call found for the same device buffer and shape is
+// used, and an unknown table runs the table-driven kernels.
+struct ResolvedTable {
+    int32_t signature = -1;
+    float scale = 1.0f;
+    uint32_t flip = 0;
+};
+
+class TableResolver {
+  public:
+    ResolvedTable resolve(const void *device_table, int32_t num_coef, int32_t idx_bytes, bool columns_ji,
+                          const e3j_amd_conv_params &p, hipStream_t caller_stream) {
+        ResolvedTable none;
+        if (p.val_dtype != E3J_AMD_F32 || num_coef <= 0 || device_table == nullptr) return none;
+        const size_t item = idx_bytes == 1 ? sizeof(Coef4D<uint8_t, float>) : sizeof(Coef4D<int32_t, float>);
+        const size_t bytes = item * (size_t)num_coef;
+        const Shape shape{num_coef, idx_bytes, columns_ji ? 1 : 0, p.num_x, p.num_y, p.num_out, p.num_scalars,
+                          p.channels, p.layout};
+        std::lock_guard<std::mutex> lock(mutex_);
+        hipStreamCaptureStatus capture = hipStreamCaptureStatusNone;
+        if (hipStreamIsCapturing(caller_stream, &capture) != hipSuccess) {
+            (void)hipGetLastError();
+            return none;
+        }
+        if (capture != hipStreamCaptureStatusNone) {
+            auto seen = by_pointer_.find(std::make_pair(device_table, shape));
+            return seen == by_pointer_.end() ? none : seen->second;
+        }
+        int device = 0;
+        if (hipGetDevice(&device) != hipSuccess) return none;
+        hipStream_t &side = side_streams_[device];
+        if (side == nullptr && hipStreamCreateWithFlags(&side, hipStreamNonBlocking) != hipSuccess) {
+            side = nullptr;
+            (void)hipGetLastError();
+            return none;
+        }
+        std::vector<unsigned char> host(bytes);
+        if (hipMemcpyAsync(host.data(), device_table, bytes, hipMemcpyDeviceToHost, side) != hipSuccess ||
+            hipStreamSynchronize(side) != hipSuccess) {
+            (void)hipGetLastError();
+            return none;
+        }
+        ResolvedTable &entry = by_content_[std::make_pair(shape, host)];
+        if (!entry_known_(entry)) {
+            const std::vector<TableEntry> entries = unpack_entries(host.data(), idx_bytes, num_coef, columns_ji);
+            entry.signature = match_signature(entries, p.num_x, p.num_y, p.num_out, p.num_scalars, p.channels,
+                                              p.layout, &entry.scale, &entry.flip);
+            if (entry.signature < 0) entry.signature = kNoKernel;
+        }
+        ResolvedTable found = entry;
+        if (found.signature == kNoKernel) found = none;
+        if (by_pointer_.size() > 4096) by_pointer_.clear();
+        by_pointer_[std::make_pair(device_table, shape)] = found;
+        return found;
+    }
+
+  private:
+    using Shape = std::tuple<int32_t, int32_t, int32_t, int32_t, int32_t, int32_t, int32_t, int32_t, int32_t>;
+    static constexpr int32_t kNoKernel = -2;  // looked up, nothing matches (a fresh entry holds -1)
+    static bool entry_known_(const ResolvedTable &e) { return e.signature != -1; }
+    std::mutex mutex_;
+    std::map<int, hipStream_t> side_streams_;
+    std::map<std::pair<Shape, std::vector<unsigned char>>, ResolvedTable> by_content_;
+    std::map<std::pair<const void *, Shape>, ResolvedTable> by_pointer_;
+};
+
+TableResolver &resolver() {
+    static TableResolver r;
+    return r;
+}
+
+// Uses the id the frame names, or finds the kernels of the table the frame carries.
+void *choose_kernels(XlaCallFrame *f, const char *op, const XlaBuffer *coef, bool columns_ji,
+                     e3j_amd_conv_params *p, hipStream_t stream) {
+    bool named = false;
+    (void)attr<int32_t>(f, "signature", kXlaS32, -1, &named);
+    if (named) {
+        // an id chosen by the host: at least the table sizes must agree with the operand
+        if (p->signature >= 0 && p->signature < e3j_amd_num_signatures() &&
+            signature(p->signature).num_coef != p->num_coef)
+            return make_error(f, E3J_AMD_INVALID_ARGUMENT,
+                              std::string(op) + ": attribute signature names kernels of a table with " +
+                                  std::to_string(signature(p->signature).num_coef) + " entries, the coef operand has " +
+                                  std::to_string(p->num_coef));
+        return nullptr;
+    }
+    const ResolvedTable found = resolver().resolve(coef->data, p->num_coef, p->coef_idx_bytes, columns_ji, *p, stream);
+    if (found.signature >= 0) {
+        p->signature = found.signature;
+        p->coef_scale = found.scale;
+        p->y_flip = found.flip;
+    }
+    return nullptr;
+}
+
 struct Decoded {
     e3j_amd_conv_params p;
     hipStream_t stream;
@@ -169,6 +276,70 @@ bool is_s32_vector(const XlaBuffer *b) { return b && b->dtype == kXlaS32 && b->r
 
 enum class Backward { kSenderRows, kReceiverRows, kReceiverRowsOrdered };
 
+size_t align256(size_t n) { return (n + 255) / 256 * 256; }
+
+// "convolution_bwd" as the reference sends it (receiver_t per position of the sender-grouped
+// adjacency, sender_ptr, edge_perm) on the receiver-grouped unrolled kernels: positions are
+// sorted by receiver (stable), which gives sender per position, receiver_ptr and, composed with
+// edge_perm, the row of y / s / dy / ds of every position.  `done` is left false when the
+// runtime hands out no scratch memory.
+void *backward_on_receiver_rows(XlaCallFrame *f, const char *op, Decoded *d, const XlaBuffer *coef, bool stacked,
+                                const XlaBuffer *x, const XlaBuffer *y, const XlaBuffer *s, const XlaBuffer *dm,
+                                const XlaBuffer *receiver_t, const XlaBuffer *sender_ptr, const int32_t *perm,
+                                const XlaBuffer *dx, const XlaBuffer *dy, const XlaBuffer *ds, bool *done) {
+    *done = false;
+    const XlaApi *api = f->api;
+    if (api->struct_size < offsetof(XlaApi, device_memory_free) + sizeof(void *) ||
+        api->device_memory_allocate == nullptr || api->device_memory_free == nullptr)
+        return nullptr;
+    const e3j_amd_conv_params &p = d->p;
+    const size_t e = (size_t)p.num_edges, n = (size_t)p.num_nodes;
+    const size_t vec = align256(4 * e);
+    const size_t csr = align256(e3j_amd_csr_workspace_bytes(p.num_nodes, p.num_edges));
+    const size_t total = 4 * vec + align256(4 * (n + 1)) + csr;
+    XlaDeviceMemoryAllocateArgs get;
+    get.struct_size = sizeof(get);
+    get.extension_start = nullptr;
+    get.ctx = f->ctx;
+    get.size = total;
+    get.alignment = 256;
+    get.data = nullptr;
+    if (void *err = api->device_memory_allocate(&get)) {
+        (void)err;  // ownership of the error object stays with the runtime's bookkeeping
+        return nullptr;
+    }
+    if (get.data == nullptr) return nullptr;
+    unsigned char *base = static_cast<unsigned char *>(get.data);
+    int32_t *senders = reinterpret_cast<int32_t *>(base);
+    int32_t *by_receiver = reinterpret_cast<int32_t *>(base + vec);
+    int32_t *sender_sorted = reinterpret_cast<int32_t *>(base + 2 * vec);
+    int32_t *edge_rows = reinterpret_cast<int32_t *>(base + 3 * vec);
+    int32_t *receiver_ptr = reinterpret_cast<int32_t *>(base + 4 * vec);
+    void *workspace = base + 4 * vec + align256(4 * (n + 1));
+    hipStream_t stream = d->stream;
+    int rc = launch_expand_rows(static_cast<const int32_t *>(sender_ptr->data), p.num_nodes, p.num_edges, senders,
+                                stream);
+    if (rc == E3J_AMD_OK)
+        rc = e3j_amd_sort_edges(static_cast<const int32_t *>(receiver_t->data), senders, p.num_edges, p.num_nodes,
+                                by_receiver, sender_sorted, receiver_ptr, workspace, stream);
+    if (rc == E3J_AMD_OK) rc = launch_compose_perm(by_receiver, perm, p.num_edges, edge_rows, stream);
+    if (rc == E3J_AMD_OK)
+        rc = run_backward(&p, true, coef->data, x->data, y->data, s->data, dm->data, sender_sorted, receiver_ptr,
+                          edge_rows, dx->data, dy->data, ds->data, stream, stacked);
+    // the runtime's allocator orders the reuse of the block after the work enqueued on this stream
+    XlaDeviceMemoryFreeArgs give;
+    give.struct_size = sizeof(give);
+    give.extension_start = nullptr;
+    give.ctx = f->ctx;
+    give.size = total;
+    give.data = get.data;
+    void *free_err = api->device_memory_free(&give);
+    *done = true;
+    if (rc != E3J_AMD_OK) return status_to_error(f, rc);
+    return free_err;
+    (void)op;
+}
+
 void *backward_handler(XlaCallFrame *f, Backward mode) {
     const bool group_is_receiver = mode != Backward::kSenderRows;
     const bool ordered = mode == Backward::kReceiverRowsOrdered;
@@ -196,6 +367,16 @@ void *backward_handler(XlaCallFrame *f, Backward mode) {
     const int64_t numel = coef->dims[coef->rank - 1];
     d.p.num_coef = (int32_t)(count(coef) / numel / (stacked ? 3 : 1));
     const int32_t *perm_ptr = count(perm) ? static_cast<const int32_t *>(perm->data) : nullptr;
+    if (void *err = choose_kernels(f, op, coef, stacked != 0, &d.p, d.stream)) return err;
+    if (mode == Backward::kSenderRows && d.p.signature >= 0) {
+        // The reference's operands: the adjacency grouped by sender.  The unrolled backward walks
+        // receiver rows, so the receiver CSR is rebuilt on the device in scratch memory of the
+        // runtime; without such memory the table-driven kernel keeps the sender rows.
+        bool done = false;
+        void *err = backward_on_receiver_rows(f, op, &d, coef, stacked != 0, x, y, s, dm, other, row_ptr, perm_ptr,
+                                              dx, dy, ds, &done);
+        if (err != nullptr || done) return err;
+    }
     if (ordered) {
         // the scratch of the atomic-free backward travels as a fourth result buffer (any dtype)
         const XlaBuffer *workspace = ret(f, 3);
@@ -293,6 +474,7 @@ void *e3j_amd_xla_convolution(void *call_frame) {
         (perm && count(perm) != 0 && count(perm) != d.p.num_edges))
         return make_error(f, E3J_AMD_INVALID_ARGUMENT, "convolution: adjacency operand sizes");
     d.p.num_coef = (int32_t)coef->dims[0];
+    if (void *err = choose_kernels(f, "convolution", coef, false, &d.p, d.stream)) return err;
     const int32_t *perm_ptr = (perm && count(perm)) ? static_cast<const int32_t *>(perm->data) : nullptr;
     const int rc = e3j_amd_convolution_fwd(&d.p, coef->data, x->data, y->data, s->data,
                                            static_cast<const int32_t *>(sender->data),

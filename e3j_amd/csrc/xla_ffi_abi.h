@@ -2,7 +2,7 @@
 // this library: only the structures a handler touches, in the field order the
 // ABI fixes (OpenXLA xla/ffi/api/c_api.h; the copy the reference vendors is
 // lib/e3j_ops/xla/ffi/api/c_api.h:52-56,96-101,150-155,228-236,277-286,
-// 403-454,577-583,722-739,749-773).  Function-table slots that this library
+// 403-454,577-583,595-620,722-739,749-773).  Function-table slots that this library
 // never calls are typed as opaque pointers.
 #ifndef E3J_AMD_CSRC_XLA_FFI_ABI_H_
 #define E3J_AMD_CSRC_XLA_FFI_ABI_H_
@@ -107,6 +107,23 @@ struct XlaStreamGetArgs {
     void *stream;  // out
 };
 
+struct XlaDeviceMemoryAllocateArgs {
+    size_t struct_size;
+    XlaExtensionBase *extension_start;
+    void *ctx;
+    size_t size;
+    size_t alignment;
+    void *data;  // out
+};
+
+struct XlaDeviceMemoryFreeArgs {
+    size_t struct_size;
+    XlaExtensionBase *extension_start;
+    void *ctx;
+    size_t size;
+    void *data;
+};
+
 struct XlaMetadata {
     size_t struct_size;
     XlaApiVersion api_version;
@@ -129,9 +146,14 @@ struct XlaApi {
     void *error_destroy;
     void *handler_register;
     void *(*stream_get)(XlaStreamGetArgs *);
-    // type_register, execution_context_get, state_set, state_get, device_memory_allocate,
-    // device_memory_free, thread_pool_schedule, thread_pool_num_threads, future_create,
-    // future_set_available, future_set_error, run_id_get, device_ordinal_get follow; unused.
+    void *type_register;
+    void *execution_context_get;
+    void *state_set;
+    void *state_get;
+    void *(*device_memory_allocate)(XlaDeviceMemoryAllocateArgs *);
+    void *(*device_memory_free)(XlaDeviceMemoryFreeArgs *);
+    // thread_pool_schedule, thread_pool_num_threads, future_create, future_set_available,
+    // future_set_error, run_id_get, device_ordinal_get follow; unused.
 };
 
 }  // extern "C"

@@ -586,6 +586,10 @@ def _make_meta(coef, x, y, s, params, graph_ordering, y_parity, layout) -> _Meta
                  num_nodes=int(x.shape[0]), squeeze_channels=False, y_shape=tuple(y.shape))
 
 
+def _under_transform() -> bool:
+    return torch._C._functorch.peek_interpreter_stack() is not None
+
+
 def _canonical(x, y, s, layout: Layout):
     """Add the channel axis of a 2-D `x`/`s`, drop a unit channel axis of `y`."""
     squeeze = x.ndim == 2
@@ -629,7 +633,10 @@ def convolution(coef, x, y, s, sender, receiver, params: ConvolutionParams,
     meta = _make_meta(coef, x3, y2, s3, params, graph_ordering, y_parity, layout)
     if graph is not None:
         _check_graph(graph, meta, int(y2.shape[0]))
-    else:  # prepared here, so that the backward pass finds it in its context
+    elif not _under_transform():
+        # prepared here, so that the backward pass finds it in its context; under a torch.func
+        # transform the operator prepares it itself, on the plain tensors the transform hands it
+        # (the batching rule first folds batched index tensors into one graph)
         graph = _forward_graph(meta, sender, receiver)
     out = _Convolution.apply(x3, y2, s3, sender, receiver, meta, graph)
     if squeeze:

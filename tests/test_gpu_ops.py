@@ -346,7 +346,7 @@ def test_index_buffer_rewritten_behind_the_version_counter():
         out = convolution(p["coef"], x, y, s, snd, rcv, p["params"], graph=handle)
         check(out, torch.autograd.grad(out, (x, y, s), dm), rolled, "with a handle")
     with pytest.raises(ValueError, match="prepared for"):
-        convolution(p["coef"], x, y, s, snd[:-1], rcv[:-1], p["params"], graph=handle)
+        convolution(p["coef"], x, y[:-1], s[:-1], snd[:-1], rcv[:-1], p["params"], graph=handle)
 
 
 def test_prepared_graph_used_on_another_stream_waits_for_its_preparation():

@@ -201,3 +201,160 @@ def test_tensor_product_targets(mode, layout):
     bad = xla.frame([_buf(xla, coef, S32), _buf(xla, xd, F32), _buf(xla, yd, F32)], [_buf(xla, wrong, F32)], attrs)
     assert lib.e3j_amd_xla_tensor_product(C.addressof(bad)) is not None
     assert "result shape" in xla.errors[-1][1]
+
+
+def _time_ms(fn, reps=20):
+    for _ in range(3):
+        fn()
+    torch.cuda.synchronize()
+    start, stop = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    start.record()
+    for _ in range(reps):
+        fn()
+    stop.record()
+    torch.cuda.synchronize()
+    return start.elapsed_time(stop) / reps
+
+
+def test_reference_frames_run_the_unrolled_kernels():
+    """Exactly the operands and attributes the reference sends (`src/e3j/ops/convolution.py:229-242`:
+    coef, x, y, s, sender, receiver_ptr, coef_ranges + num_nodes, debug; `:433-452`: the stack of
+    three transposed tables, x, y, s, dm, sender_t, receiver_ptr_t, perm, coef_ranges + num_nodes,
+    debug), at the size of config 2, with the table's rows in a permuted order as the reference's
+    balancing leaves them: parity against the CPU checker, and the time of the unrolled kernels
+    (within 1.3x of the direct C-ABI launches), not of the table-driven ones."""
+    from e3j_amd import workloads as W
+    from e3j_amd.graph import csr_row_ptr
+    from e3j_amd.ops import _Table
+    from oracle import c_oracle
+    w = W.config2()
+    m = w.module
+    packed = m._packed_coef("float32")
+    dims = (int(w.x.shape[1]), int(w.y.shape[1]), m.params.num_out, int(w.s.shape[1]))
+    sig, scale, _ = _Table.get(packed, np.float32).signature(dims, w.channels, m.layout)
+    assert sig >= 0
+    lib = _lib.load()
+    d = w.to("cuda")
+    n, e = w.num_nodes, w.num_edges
+    rng = np.random.default_rng(3)
+    c = Coef4D.unpack(packed, np.float32)
+    shuffled = Coef4D(c.val, c.idx, "float32", c.idx_dtype)
+    order = rng.permutation(len(c.val))
+    shuffled = Coef4D(c.val[order], c.idx[order], "float32", c.idx_dtype)
+    stacked = np.stack([shuffled.transpose(a).pack() for a in ((1, 0, 2, 3), (2, 0, 1, 3), (3, 0, 2, 1))])
+    snd, rcv = w.sender.numpy(), w.receiver.numpy()
+    perm, recv_t, sptr = O.transpose_graph(snd, rcv, n)
+    ptr = csr_row_ptr(d.receiver, n)
+    ranges = dev(np.array([len(c.val)], dtype=np.int32))
+    torch.cuda.synchronize()
+
+    xla = FakeXla(stream=torch.cuda.current_stream().cuda_stream)
+    xla.allocate = lambda nbytes: torch.empty(nbytes, dtype=torch.uint8, device="cuda")
+    attrs = lambda: {"num_nodes": (S32, C.c_int32(n)), "debug": (S32, C.c_int32(0))}  # noqa: E731
+    out = torch.full_like(d.dm, float("nan"))
+    fwd = xla.frame([_buf(xla, dev(shuffled.pack()), U8), _buf(xla, d.x, F32), _buf(xla, d.y, F32),
+                     _buf(xla, d.s, F32), _buf(xla, d.sender, S32), _buf(xla, ptr, S32), _buf(xla, ranges, S32)],
+                    [_buf(xla, out, F32)], attrs())
+    dx, dy, ds = (torch.full_like(t, float("nan")) for t in (d.x, d.y, d.s))
+    bwd = xla.frame([_buf(xla, dev(stacked), U8), _buf(xla, d.x, F32), _buf(xla, d.y, F32), _buf(xla, d.s, F32),
+                     _buf(xla, d.dm, F32), _buf(xla, dev(recv_t.astype(np.int32)), S32), _buf(xla, dev(sptr), S32),
+                     _buf(xla, dev(perm), S32), _buf(xla, ranges, S32)],
+                    [_buf(xla, dx, F32), _buf(xla, dy, F32), _buf(xla, ds, F32)], attrs())
+    torch.cuda.synchronize()
+    assert lib.e3j_amd_xla_convolution(C.addressof(fwd)) is None, xla.errors
+    assert lib.e3j_amd_xla_convolution_bwd(C.addressof(bwd)) is None, xla.errors
+    torch.cuda.synchronize()
+    assert xla.allocations == 1 and not xla.scratch            # scratch borrowed once and handed back
+
+    idx, val, mix = w.table()
+    a = w.numpy()
+    args = (a["x"], a["y"], a["s"], a["sender"], a["receiver"])
+    mag_args = tuple(np.abs(t) for t in args[:3]) + args[3:]
+    ref = c_oracle.convolution(idx, val, mix, *args, dims[2])
+    mag = c_oracle.convolution(idx, np.abs(val), mix, *mag_args, dims[2])
+    H.assert_parity(out.cpu().numpy(), ref.astype(np.float64), 2.0 * mag.astype(np.float64), "reference frame out",
+                    ulps=32.0)
+    refs = c_oracle.convolution_vjp(idx, val, mix, *args, a["dm"])
+    mags = c_oracle.convolution_vjp(idx, np.abs(val), mix, *mag_args, np.abs(a["dm"]))
+    for g, r, mg, name in zip((dx, dy, ds), refs, mags, ("dx", "dy", "ds")):
+        H.assert_parity(g.cpu().numpy(), r.astype(np.float64), 2.0 * mg.astype(np.float64), f"reference frame {name}",
+                        ulps=32.0)
+
+    # the direct launches of the same kernels through the C ABI
+    p = _lib.ConvParams(num_nodes=n, num_edges=e, num_coef=packed.shape[0], num_x=dims[0], num_y=dims[1],
+                        num_out=dims[2], num_scalars=dims[3], channels=w.channels, layout=m.layout.value,
+                        val_dtype=_lib.F32, coef_idx_bytes=1, signature=sig, coef_scale=scale, debug=0, y_flip=0,
+                        row_order=None)
+    stream = int(torch.cuda.current_stream().cuda_stream)
+
+    def direct_fwd():
+        _lib.check(lib.e3j_amd_convolution_fwd(C.byref(p), None, d.x.data_ptr(), d.y.data_ptr(), d.s.data_ptr(),
+                                               d.sender.data_ptr(), ptr.data_ptr(), None, out.data_ptr(), stream))
+
+    def direct_bwd():
+        _lib.check(lib.e3j_amd_convolution_bwd_receiver(
+            C.byref(p), None, d.x.data_ptr(), d.y.data_ptr(), d.s.data_ptr(), d.dm.data_ptr(), d.sender.data_ptr(),
+            ptr.data_ptr(), None, dx.data_ptr(), dy.data_ptr(), ds.data_ptr(), stream))
+
+    t_direct = _time_ms(direct_fwd), _time_ms(direct_bwd)
+    t_frames = (_time_ms(lambda: lib.e3j_amd_xla_convolution(C.addressof(fwd))),
+                _time_ms(lambda: lib.e3j_amd_xla_convolution_bwd(C.addressof(bwd))))
+    print(f"direct fwd/bwd {t_direct[0]:.3f}/{t_direct[1]:.3f} ms, reference frames {t_frames[0]:.3f}/{t_frames[1]:.3f} ms")
+    assert t_frames[0] <= 1.3 * t_direct[0] + 0.02, (t_frames, t_direct)
+    assert sum(t_frames) <= 1.3 * sum(t_direct) + 0.03, (t_frames, t_direct)
+
+    # without scratch from the runtime the backward keeps the sender rows (table-driven), same results
+    xla.allocate = None
+    dx2, dy2, ds2 = (torch.full_like(t, float("nan")) for t in (d.x, d.y, d.s))
+    bwd2 = xla.frame(bwd_operands(bwd), [_buf(xla, dx2, F32), _buf(xla, dy2, F32), _buf(xla, ds2, F32)], attrs())
+    assert lib.e3j_amd_xla_convolution_bwd(C.addressof(bwd2)) is None, xla.errors
+    torch.cuda.synchronize()
+    for g, g0, name in zip((dx2, dy2, ds2), (dx, dy, ds), ("dx", "dy", "ds")):
+        assert float((g - g0).abs().max()) <= 3e-5 * float(g0.abs().max()), name
+
+    # a `signature` attribute that names kernels of another table size is refused
+    bad = dict(attrs())
+    bad["signature"] = (S32, C.c_int32(0))
+    frame = xla.frame(bwd_operands(fwd), [_buf(xla, out, F32)], bad)
+    if lib.e3j_amd_signature_name(0) and sig != 0:
+        err = lib.e3j_amd_xla_convolution(C.addressof(frame))
+        assert err is not None and ("entries" in xla.errors[-1][1] or "match" in xla.errors[-1][1])
+
+
+def bwd_operands(frame):
+    """The argument buffers of a frame, to build another frame over them."""
+    from tests.xla_frame import Buffer
+    n = frame.args.size
+    return [C.cast(frame.args.args[i], C.POINTER(Buffer)).contents for i in range(n)]
+
+
+def test_reference_forward_frame_under_graph_capture_uses_what_an_earlier_call_found():
+    """Nothing can be read back while a stream is captured: the handler then uses the kernels an
+    earlier call found for the same table buffer; replays give the eager result."""
+    from e3j_amd import workloads as W
+    from e3j_amd.graph import csr_row_ptr
+    w = W.config2(0.05)
+    d = w.to("cuda")
+    n = w.num_nodes
+    lib = _lib.load()
+    packed = dev(w.module._packed_coef("float32"))
+    ptr = csr_row_ptr(d.receiver, n)
+    ranges = dev(np.array([1], dtype=np.int32))
+    xla = FakeXla(stream=torch.cuda.current_stream().cuda_stream)
+    out = torch.zeros_like(d.dm)
+    frame = xla.frame([_buf(xla, packed, U8), _buf(xla, d.x, F32), _buf(xla, d.y, F32), _buf(xla, d.s, F32),
+                       _buf(xla, d.sender, S32), _buf(xla, ptr, S32), _buf(xla, ranges, S32)],
+                      [_buf(xla, out, F32)], {"num_nodes": (S32, C.c_int32(n)), "debug": (S32, C.c_int32(0))})
+    torch.cuda.synchronize()
+    assert lib.e3j_amd_xla_convolution(C.addressof(frame)) is None, xla.errors
+    torch.cuda.synchronize()
+    eager = out.clone()
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph):
+        xla.stream = torch.cuda.current_stream().cuda_stream
+        assert lib.e3j_amd_xla_convolution(C.addressof(frame)) is None, xla.errors
+    for _ in range(3):
+        out.zero_()
+        graph.replay()
+        torch.cuda.synchronize()
+        assert torch.equal(out, eager)

@@ -55,7 +55,16 @@ PAIRS = [
       ("error_get_message", "XLA_FFI_Error_GetMessage", "error_get_message"),
       ("error_destroy", "XLA_FFI_Error_Destroy", "error_destroy"),
       ("handler_register", "XLA_FFI_Handler_Register", "handler_register"),
-      ("stream_get", "XLA_FFI_Stream_Get", "stream_get")]),
+      ("stream_get", "XLA_FFI_Stream_Get", "stream_get"),
+      ("type_register", "XLA_FFI_Type_Register", "type_register"),
+      ("execution_context_get", "XLA_FFI_ExecutionContext_Get", "execution_context_get"),
+      ("state_set", "XLA_FFI_State_Set", "state_set"), ("state_get", "XLA_FFI_State_Get", "state_get"),
+      ("device_memory_allocate", "XLA_FFI_DeviceMemory_Allocate", "device_memory_allocate"),
+      ("device_memory_free", "XLA_FFI_DeviceMemory_Free", "device_memory_free")]),
+    ("XlaDeviceMemoryAllocateArgs", "XLA_FFI_DeviceMemory_Allocate_Args", F.DeviceMemoryAllocateArgs,
+     [("struct_size",) * 3, ("extension_start",) * 3, ("ctx",) * 3, ("size",) * 3, ("alignment",) * 3, ("data",) * 3]),
+    ("XlaDeviceMemoryFreeArgs", "XLA_FFI_DeviceMemory_Free_Args", F.DeviceMemoryFreeArgs,
+     [("struct_size",) * 3, ("extension_start",) * 3, ("ctx",) * 3, ("size",) * 3, ("data",) * 3]),
 ]
 #: constants of xla_ffi_abi.h and the enumerators they restate
 CONSTANTS = [

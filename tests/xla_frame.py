@@ -62,12 +62,29 @@ ERROR_CREATE = C.CFUNCTYPE(C.c_void_p, C.POINTER(ErrorCreateArgs))
 STREAM_GET = C.CFUNCTYPE(C.c_void_p, C.POINTER(StreamGetArgs))
 
 
+class DeviceMemoryAllocateArgs(C.Structure):
+    _fields_ = [("struct_size", C.c_size_t), ("extension_start", C.c_void_p), ("ctx", C.c_void_p),
+                ("size", C.c_size_t), ("alignment", C.c_size_t), ("data", C.c_void_p)]
+
+
+class DeviceMemoryFreeArgs(C.Structure):
+    _fields_ = [("struct_size", C.c_size_t), ("extension_start", C.c_void_p), ("ctx", C.c_void_p),
+                ("size", C.c_size_t), ("data", C.c_void_p)]
+
+
+DEVICE_ALLOCATE = C.CFUNCTYPE(C.c_void_p, C.POINTER(DeviceMemoryAllocateArgs))
+DEVICE_FREE = C.CFUNCTYPE(C.c_void_p, C.POINTER(DeviceMemoryFreeArgs))
+
+
 class Api(C.Structure):
     _fields_ = [("struct_size", C.c_size_t), ("extension_start", C.c_void_p),
                 ("api_version", ApiVersion), ("internal_api", C.c_void_p),
                 ("error_create", ERROR_CREATE), ("error_get_message", C.c_void_p),
                 ("error_destroy", C.c_void_p), ("handler_register", C.c_void_p),
-                ("stream_get", STREAM_GET)] + [(f"unused{n}", C.c_void_p) for n in range(13)]
+                ("stream_get", STREAM_GET), ("type_register", C.c_void_p),
+                ("execution_context_get", C.c_void_p), ("state_set", C.c_void_p), ("state_get", C.c_void_p),
+                ("device_memory_allocate", DEVICE_ALLOCATE), ("device_memory_free", DEVICE_FREE)] + \
+               [(f"unused{n}", C.c_void_p) for n in range(7)]
 
 
 class CallFrame(C.Structure):
@@ -101,8 +118,32 @@ class FakeXla:
             args.contents.stream = self.stream
             return None
 
-        self._cb = (ERROR_CREATE(error_create), STREAM_GET(stream_get))
-        self.api = Api(struct_size=C.sizeof(Api), error_create=self._cb[0], stream_get=self._cb[1])
+        #: device scratch handed out through the allocation callbacks: address -> buffer; `allocate`
+        #: is a callable `(nbytes) -> object with data_ptr()` (None: the runtime has no memory to give)
+        self.allocate = None
+        self.scratch = {}
+        self.allocations = 0
+
+        def device_allocate(args):
+            if self.allocate is None:
+                return 0xA110C
+            buf = self.allocate(int(args.contents.size) + int(args.contents.alignment))
+            base = buf.data_ptr()
+            align = max(int(args.contents.alignment), 1)
+            aligned = (base + align - 1) // align * align
+            self.scratch[aligned] = buf
+            self.allocations += 1
+            args.contents.data = aligned
+            return None
+
+        def device_free(args):
+            self.scratch.pop(args.contents.data)   # KeyError: freed what was never handed out
+            return None
+
+        self._cb = (ERROR_CREATE(error_create), STREAM_GET(stream_get), DEVICE_ALLOCATE(device_allocate),
+                    DEVICE_FREE(device_free))
+        self.api = Api(struct_size=C.sizeof(Api), error_create=self._cb[0], stream_get=self._cb[1],
+                       device_memory_allocate=self._cb[2], device_memory_free=self._cb[3])
         self.api.api_version = ApiVersion(C.sizeof(ApiVersion), None, 0, 2)
 
     def buffer(self, dtype: int, data_ptr: int, dims) -> Buffer:
