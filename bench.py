@@ -34,16 +34,78 @@ if ROOT not in sys.path:
 
 HBM_PEAK_GBS = 8000.0
 
-#: HBM bytes per launch of the convolution kernels on the full cfg3 workload, from two
-#: `rocprofv3 --pmc` runs of this script (FETCH_SIZE and WRITE_SIZE, KiB per dispatch), each
-#: scaled by what the same counter reads for a 1 GiB device copy (`--calibrate-copy`: 2.0 for
-#: FETCH_SIZE, 1.0 for WRITE_SIZE).  Only quoted for the workloads they were measured on.
-MEASURED_TRAFFIC_BYTES = {
-    ("cfg3", 1.0, "trailing"): {"backward": 2.0 * 7.47e6 * 1024 + 18.9e6 * 1024,
-                                "forward": 2.0 * 6.263e6 * 1024 + 1.584e6 * 1024},
-    ("cfg3", 1.0, "leading"): {"backward": 2.0 * 7.403e6 * 1024 + 19.08e6 * 1024,
-                               "forward": 2.0 * 6.258e6 * 1024 + 1.592e6 * 1024},
-}
+#: HBM bytes per launch come from `profiles/traffic.json`: two `rocprofv3 --pmc` runs of this
+#: script (FETCH_SIZE and WRITE_SIZE, KiB per dispatch), each scaled by what the same counter reads
+#: for a 1 GiB device copy (`--calibrate-copy`), written by `python bench.py --write-traffic ...`
+#: together with a hash of the kernel sources.  A figure is only quoted while the sources it was
+#: measured on are the ones in the tree.
+TRAFFIC_FILE = os.path.join(ROOT, "profiles", "traffic.json")
+KERNEL_SOURCES = ("e3j_amd/csrc/unrolled.h", "e3j_amd/csrc/common.h", "e3j_amd/csrc/tp_unrolled.h",
+                  "e3j_amd/codegen/gen_conv.py", "e3j_amd/codegen/gen_tp.py")
+
+
+def kernel_source_hash() -> str:
+    import hashlib
+    h = hashlib.sha256()
+    for rel in KERNEL_SOURCES:
+        with open(os.path.join(ROOT, rel), "rb") as fh:
+            h.update(rel.encode() + b"\0" + fh.read())
+    return h.hexdigest()[:16]
+
+
+def measured_traffic(key: str) -> dict:
+    """`{"forward": bytes, "backward": bytes}` for a workload key, {} when there is no measurement of
+    the kernels as they are now."""
+    try:
+        with open(TRAFFIC_FILE) as fh:
+            table = json.load(fh)
+    except (OSError, ValueError):
+        return {}
+    if table.get("kernel_source_hash") != kernel_source_hash():
+        return {}
+    return table.get("workloads", {}).get(key, {})
+
+
+def write_traffic(paths, out_path: str, key: str, kernels: dict) -> int:
+    """Summarise rocprofv3 counter CSVs (FETCH_SIZE / WRITE_SIZE runs of one bench command) into
+    `profiles/traffic.json` under `key`.  `kernels`: pass name -> substring of the kernel name."""
+    import csv
+    sums = {}
+    for path in paths:
+        with open(path) as fh:
+            for row in csv.DictReader(fh):
+                name, counter = row["Kernel_Name"], row["Counter_Name"]
+                which = next((k for k, sub in kernels.items() if sub in name), None)
+                if "copyBuffer" in name or "copy" in name.lower() and which is None:
+                    which = "copy"
+                if which is not None and counter in ("FETCH_SIZE", "WRITE_SIZE"):
+                    sums.setdefault((which, counter), []).append(float(row["Counter_Value"]))
+    copy_fetch = max(sums.get(("copy", "FETCH_SIZE"), [0.0]))
+    copy_write = max(sums.get(("copy", "WRITE_SIZE"), [0.0]))
+    gib_kib = float(1 << 20)
+    fetch_scale = gib_kib / copy_fetch if copy_fetch else 2.0
+    write_scale = gib_kib / copy_write if copy_write else 1.0
+    entry = {"fetch_scale": round(fetch_scale, 3), "write_scale": round(write_scale, 3)}
+    for which in kernels:
+        f = sums.get((which, "FETCH_SIZE"), [])
+        w = sums.get((which, "WRITE_SIZE"), [])
+        if f and w:
+            fetch, write = sum(f) / len(f), sum(w) / len(w)
+            entry[which] = (fetch_scale * fetch + write_scale * write) * 1024.0
+            entry[which + "_counters_KiB"] = {"FETCH_SIZE": fetch, "WRITE_SIZE": write}
+    try:
+        with open(out_path) as fh:
+            table = json.load(fh)
+    except (OSError, ValueError):
+        table = {}
+    if table.get("kernel_source_hash") != kernel_source_hash():
+        table = {"kernel_source_hash": kernel_source_hash(), "workloads": {}}
+    table["workloads"][key] = entry
+    with open(out_path, "w") as fh:
+        json.dump(table, fh, indent=1, sort_keys=True)
+        fh.write("\n")
+    print(json.dumps({key: entry}))
+    return 0
 
 
 def parse_args():
@@ -60,6 +122,8 @@ def parse_args():
                     help="channel count of cfg3 (default 128; kernels are built for 32, 64, 128, 256)")
     ap.add_argument("--scale", type=float, default=1.0, help="fraction of the configuration's atoms")
     ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--no-layouts", action="store_true",
+                    help="skip the leading-channels sub-record of the default run")
     ap.add_argument("--cpu-seconds", type=float, default=15.0)
     ap.add_argument("--kernel-only", action="store_true",
                     help="time the C-ABI launches only (no operator-level step)")
@@ -79,6 +143,12 @@ def parse_args():
     ap.add_argument("--mode", default="MAP", choices=["MAP", "OUTER", "INNER"],
                     help="--op tensor_product: channel mode (OUTER: y without channel axis)")
     ap.add_argument("--rows", type=int, default=1 << 18, help="--op tensor_product: number of rows")
+    ap.add_argument("--write-traffic", nargs="+", metavar="CSV",
+                    help="no GPU work: summarise rocprofv3 counter CSVs (FETCH_SIZE and WRITE_SIZE runs of this "
+                         "script with --calibrate-copy) into profiles/traffic.json for --config/--layout/--scale")
+    ap.add_argument("--tile-rows", type=int, default=None,
+                    help="receivers per tile of the tiled backward (default: the library's setting, 0 = one "
+                         "wave per receiver)")
     ap.add_argument("--calibrate-copy", action="store_true",
                     help="also run a 1 GiB device copy, the known-size kernel that hardware "
                          "traffic counters are scaled by")
@@ -222,8 +292,9 @@ def access_floor(torch, abi, steps: int) -> dict:
     return result
 
 
-def time_events(torch, fn, steps: int, warmup: int) -> float:
-    """Average milliseconds of `fn` from HIP events recorded on the launch stream."""
+def time_events(torch, fn, steps: int, warmup: int, stats: dict | None = None) -> float:
+    """Average milliseconds of `fn` from HIP events recorded on the launch stream (`stats`, if given,
+    also receives the median and the minimum)."""
     for _ in range(warmup):
         fn()
     torch.cuda.synchronize()
@@ -234,7 +305,10 @@ def time_events(torch, fn, steps: int, warmup: int) -> float:
         fn()
         b.record()
     torch.cuda.synchronize()
-    return sum(a.elapsed_time(b) for a, b in zip(starts, stops)) / steps
+    times = sorted(a.elapsed_time(b) for a, b in zip(starts, stops))
+    if stats is not None:
+        stats.update(ms_median=times[len(times) // 2], ms_min=times[0])
+    return sum(times) / steps
 
 
 def cpu_baseline(w, seconds: float) -> dict:
@@ -473,12 +547,21 @@ def _lib_name(signature: int) -> str:
     return _lib.load().e3j_amd_tp_signature_name(signature).decode()
 
 
+def traffic_key(args) -> str:
+    return f"{args.config}/{args.scale}/{args.layout}/k{args.channels or 'default'}"
+
+
 def main():
     args = parse_args()
     if args.gpus != 1:
         print("bench.py measures one GPU: this build has no multi-GPU path (run with --gpus 1)",
               file=sys.stderr)
         return 2
+    if args.write_traffic:
+        key = traffic_key(args)
+        names = ({"forward": "unrolled_fwd_leading", "backward": "unrolled_bwd_leading"} if args.layout == "leading"
+                 else {"forward": "unrolled_fwd_kernel", "backward": "unrolled_bwd_kernel"})
+        return write_traffic(args.write_traffic, TRAFFIC_FILE, key, names)
     import torch
     if not torch.cuda.is_available():
         print("bench.py needs an MI355X: no GPU is visible", file=sys.stderr)
@@ -486,6 +569,8 @@ def main():
     import e3j_amd
     from e3j_amd import _lib
     _lib.load()  # fail loudly when the HIP library is missing
+    if args.tile_rows is not None:
+        e3j_amd.config(tile_rows=args.tile_rows)
     device = torch.device("cuda:0")
     torch.cuda.set_device(device)
     if args.op == "tensor_product":
@@ -535,14 +620,22 @@ def main():
     torch.cuda.synchronize()
     ms_per_step = (time.perf_counter() - t0) * 1e3 / args.steps
 
-    fwd_ms = time_events(torch, abi.forward, args.steps, 2)
-    bwd_ms = time_events(torch, abi.backward, args.steps, 2)
+    fwd_stats, bwd_stats = {}, {}
+    fwd_ms = time_events(torch, abi.forward, args.steps, 2, fwd_stats)
+    bwd_ms = time_events(torch, abi.backward, args.steps, 2, bwd_stats)
+
+    # graph preparation of one step (row pointers, row order; the reference pays its bincount, cumsum
+    # and argsort inside the operator too): part of `ms_per_step`, reported on its own as well
+    from e3j_amd.ops import prepare_graph
+    prep_stats = {}
+    prep_ms = time_events(torch, lambda: prepare_graph(w.sender, w.receiver, w.num_nodes, module.graph_ordering),
+                          args.steps, 2, prep_stats)
 
     def gbs(nbytes, ms):
         return nbytes / (ms * 1e-3) / 1e9
 
-    measured = ({} if args.spatial_sort or args.deterministic or args.channels not in (None, 128) else
-                MEASURED_TRAFFIC_BYTES.get((args.config, args.scale, args.layout), {}))
+    tiled = abi.schedule is not None and not args.deterministic
+    measured = ({} if args.spatial_sort or args.deterministic or tiled else measured_traffic(traffic_key(args)))
     bwd_gbs, fwd_gbs = gbs(bytes_["bwd"], bwd_ms), gbs(bytes_["fwd"], fwd_ms)
     both_gbs = gbs(bytes_["fwd_bwd"], fwd_ms + bwd_ms)
     result = {
@@ -573,17 +666,34 @@ def main():
             "bound": "hbm",
             "kernel": ("convolution backward, atomic-free (position sort + unrolled_bwd_kernel + fixed-order "
                        "dx/dy reductions)" if args.deterministic else
-                       "convolution backward (unrolled_bwd_kernel + dx zero fill)"),
+                       "convolution backward over tiles of receivers (unrolled_bwd_tile_kernel + dx zero fill)"
+                       if tiled else "convolution backward (unrolled_bwd_kernel + dx zero fill)"),
             "achieved": bwd_gbs, "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": bwd_gbs / HBM_PEAK_GBS,
             "traffic": measured.get("backward"),
-            "algorithmic_bytes": bytes_["bwd"], "ms": bwd_ms,
+            "algorithmic_bytes": bytes_["bwd"], "ms": bwd_ms, **bwd_stats,
             "forward": {"achieved": fwd_gbs, "frac": fwd_gbs / HBM_PEAK_GBS,
                         "traffic": measured.get("forward"),
-                        "algorithmic_bytes": bytes_["fwd"], "ms": fwd_ms},
+                        "algorithmic_bytes": bytes_["fwd"], "ms": fwd_ms, **fwd_stats},
             "forward_plus_backward": {"achieved": both_gbs, "frac": both_gbs / HBM_PEAK_GBS,
                                       "algorithmic_bytes": bytes_["fwd_bwd"], "ms": fwd_ms + bwd_ms},
+            "graph_preparation": {"ms": prep_ms, **prep_stats,
+                                  "what": "index wrap, row pointers, row order (per step; included in ms_per_step)"},
         },
     }
+    if args.layout == "trailing" and not args.kernel_only and not args.no_layouts and args.config in ("cfg2", "cfg3"):
+        # the same workload in the leading-channels layout (the configurations name both), kernels only
+        del abi
+        wl = w.with_layout("LEADING_CHANNELS")
+        lead = AbiCalls(wl)
+        ls_f, ls_b = {}, {}
+        lf = time_events(torch, lead.forward, args.steps, 2, ls_f)
+        lb = time_events(torch, lead.backward, args.steps, 2, ls_b)
+        result["layouts"] = {"leading": {
+            "forward": {"ms": lf, **ls_f, "frac": gbs(bytes_["fwd"], lf) / HBM_PEAK_GBS},
+            "backward": {"ms": lb, **ls_b, "frac": gbs(bytes_["bwd"], lb) / HBM_PEAK_GBS},
+            "forward_plus_backward": {"ms": lf + lb, "frac": gbs(bytes_["fwd_bwd"], lf + lb) / HBM_PEAK_GBS}}}
+        del lead, wl
+        abi = AbiCalls(w)
     if args.access_floor:
         if args.layout != "trailing" or abi.perm is not None:
             print("--access-floor covers the receiver-sorted trailing layout only", file=sys.stderr)
