@@ -195,6 +195,18 @@ __device__ __forceinline__ void store_apart_stream(float *p, const Vec<C> &a) {
 
 __device__ __forceinline__ int uniform(int v) { return __builtin_amdgcn_readfirstlane(v); }
 
+// s_waitcnt operand on gfx9: vmcnt(0), the other counters left alone (expcnt 7, lgkmcnt 15).
+constexpr int kWaitVmcnt0 = 0x0F70;
+
+// One int32 at a wave-uniform address through the scalar data path, waited for on the spot.  For
+// loads inside small search loops, which the compiler otherwise issues as vector loads whose wait
+// (vmcnt is one in-order counter) would also wait for every store and atomic issued before.
+__device__ __forceinline__ int load_uniform(const int32_t *p) {
+    int v;
+    asm volatile("s_load_dword %0, %1, 0x0\n\ts_waitcnt lgkmcnt(0)" : "=s"(v) : "s"(p));
+    return __builtin_amdgcn_readfirstlane(v);  // tells the compiler what the register class says
+}
+
 // Pin a wave-uniform value (scalar register) into a vector register.  A VALU operation
 // reads at most one scalar or literal operand, so `literal * y` with y in a scalar
 // register would make the compiler park every coefficient literal in a vector register
@@ -486,10 +498,11 @@ __device__ __forceinline__ void unrolled_bwd_part(
         const bool inside = SUB == 1 || base + sub < e1;
         const int pos = SUB == 1 ? base : (inside ? base + sub : e1 - 1);
         pos_n = pos;
-        const int snd = sender[pos];
+        // (explicit scalar loads where the position is wave-uniform: see load_uniform)
+        const int snd = SUB == 1 ? load_uniform(sender + pos) : sender[pos];
         valid_n = inside && (unsigned)snd < (unsigned)num_nodes;
         snd_n = valid_n ? snd : 0;
-        ee_n = perm ? (int64_t)perm[pos] : (int64_t)pos;
+        ee_n = perm ? (int64_t)(SUB == 1 ? load_uniform(perm + pos) : perm[pos]) : (int64_t)pos;
         const float *xr = x + (int64_t)snd_n * (X * K) + c0;
         const float *sr = s + ee_n * (int64_t)(S * K) + c0;
         const float *yr = y + ee_n * Y;
@@ -500,7 +513,21 @@ __device__ __forceinline__ void unrolled_bwd_part(
 #pragma unroll
         for (int k = 0; k < Y; k++) yn[k] = yr[k];
     };
+    // Padding edges (their dy/ds rows are zero-filled separately) are stepped over while looking
+    // for the next edge, on wave-uniform values, so that the body below is one straight line
+    // from the loads of the next edge to the stores and atomics of this one: the wait for those
+    // loads at the top of the next turn then leaves the younger stores and atomics in flight.
+    // (A branch around the body would make that wait a wait for everything, every edge.)
+    auto next_edge = [&](int p) {
+        if (SUB == 1)
+            while (p < e1 && !((unsigned)load_uniform(sender + p) < (unsigned)num_nodes)) p++;
+        return p;
+    };
+    e = next_edge(e);
     if (e < e1) fetch(e);
+    // The first edge's operands are waited for here, before the loop: the loop is then entered
+    // with nothing in flight, and the waits inside it are exact counts of what one turn issues.
+    __builtin_amdgcn_s_waitcnt(kWaitVmcnt0);
     while (e < e1) {
         V xc[NX], sc[NS];
         float yc[Y];
@@ -514,9 +541,9 @@ __device__ __forceinline__ void unrolled_bwd_part(
         const int snd = snd_n;
         const int64_t ee = ee_n;
         const int pos = pos_n;
-        e += SUB;
+        e = next_edge(e + SUB);
         if (e < e1) fetch(e);
-        if (!valid) continue;  // padding edge: its dy/ds rows are zero-filled separately
+        if (SUB > 1 && !valid) continue;  // (side-by-side edges: per group of lanes)
 
         V dxe[NX];
         float dye[Red::P];
@@ -643,12 +670,15 @@ __device__ __forceinline__ void unrolled_bwd_tile_part(
     // this wave's share of the list, cut at sender boundaries
     auto boundary = [&](int p) {
         if (p <= begin) return begin;
-        while (p < end && t_sender[p] == t_sender[p - 1]) p++;
+        while (p < end && load_uniform(t_sender + p) == load_uniform(t_sender + p - 1)) p++;
         return p;
     };
     const int n = end - begin;
     const int lo = boundary(begin + (int)((int64_t)n * wave / nw));
-    const int hi = boundary(begin + (int)((int64_t)n * (wave + 1) / nw));
+    int hi = boundary(begin + (int)((int64_t)n * (wave + 1) / nw));
+    // padding edges (their dy/ds rows are zero-filled separately) are the tail of a tile's list:
+    // the loop below never sees one, so its body is one straight line (see the kernel above)
+    while (hi > lo && !((unsigned)load_uniform(t_sender + hi - 1) < (unsigned)num_nodes)) hi--;
 
     V xc[NX], xn[NX], sn[NS], acc[NX];
     float yn[Y];
@@ -660,13 +690,17 @@ __device__ __forceinline__ void unrolled_bwd_tile_part(
     // loads of the next edge never wait for them.
     int snd_a = 0, ee_a = 0, loc_a = 0;
     auto read_indices = [&](int pos) {
-        snd_a = t_sender[pos];
-        ee_a = t_edge[pos];
-        loc_a = t_local[pos];
+        asm volatile("s_load_dword %0, %3, 0x0\n\ts_load_dword %1, %4, 0x0\n\ts_load_dword %2, %5, 0x0\n\t"
+                     "s_waitcnt lgkmcnt(0)"
+                     : "=&s"(snd_a), "=&s"(ee_a), "=&s"(loc_a)
+                     : "s"(t_sender + pos), "s"(t_edge + pos), "s"(t_local + pos));
+        snd_a = uniform(snd_a);
+        ee_a = uniform(ee_a);
+        loc_a = uniform(loc_a);
     };
     auto fetch = [&](int held) {  // the edge whose indices were read last
         const int snd = snd_a;
-        valid_n = (unsigned)snd < (unsigned)num_nodes;
+        valid_n = true;  // (padding entries are cut off the range)
         snd_n = snd;
         ee_n = ee_a;
         loc_n = loc_a;
@@ -717,7 +751,8 @@ __device__ __forceinline__ void unrolled_bwd_tile_part(
         }
     }
     __syncthreads();
-
+    // entered with nothing in flight: the waits inside the loop are exact counts of one turn
+    __builtin_amdgcn_s_waitcnt(kWaitVmcnt0);
 
     for (int pos = lo; pos < hi; pos++) {
         V sc[NS];
@@ -738,7 +773,7 @@ __device__ __forceinline__ void unrolled_bwd_tile_part(
             fetch(held);
             if (pos + 2 < hi) read_indices(pos + 2);
         }
-        if (!valid) continue;  // padding edge: its dy/ds rows are zero-filled separately
+        (void)valid;
 
         if (snd != run) {
             if (run >= 0) flush(run);
