@@ -103,6 +103,7 @@ SYMBOLS = {
     "e3j_amd_convolution_bwd_ordered_workspace_bytes": (ctypes.c_size_t, [_PARAMS]),
     "e3j_amd_convolution_bwd_ordered": (ctypes.c_int, [_PARAMS] + [_P] * 13),
     "e3j_amd_tile_rows": (ctypes.c_int32, [ctypes.c_int32]),
+    "e3j_amd_tile_rows_default": (ctypes.c_int32, [ctypes.c_int32]),
     "e3j_amd_tile_schedule_num_work": (ctypes.c_int64, [ctypes.c_int32, ctypes.c_int64, ctypes.c_int32, ctypes.c_int32]),
     "e3j_amd_tile_schedule_workspace_bytes": (ctypes.c_size_t, [ctypes.c_int32, ctypes.c_int64, ctypes.c_int32]),
     "e3j_amd_tile_schedule_build": (ctypes.c_int, [_P] * 4 + [ctypes.c_int32, ctypes.c_int64, ctypes.c_int32,

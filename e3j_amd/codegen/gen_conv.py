@@ -57,12 +57,14 @@ LAUNCH = {
              bwd_tile=[(1, 8, 3), (1, 8, 4), (1, 16, 4)]),
     128: dict(fwd=[(1, 4, 1), (1, 4, 2), (2, 4, 2), (2, 4, 4)],
               bwd=[(2, 4, 3), (1, 4, 1), (1, 4, 3), (1, 4, 4), (2, 4, 4), (1, 4, 2)],
-              bwd_tile=[(2, 8, 3), (2, 8, 4), (1, 8, 4), (1, 16, 4)]),
+              bwd_tile=[(2, 4, 3, 3, 2), (2, 8, 3, 1, 8), (2, 12, 3, 3, 8), (2, 4, 3, 2, 4), (1, 8, 4, 1, 8)]),
     256: dict(fwd=[(1, 4, 1), (1, 4, 2)], bwd=[(2, 4, 3), (1, 4, 2), (1, 4, 3)],
               bwd_tile=[(2, 8, 3), (1, 8, 4)]),
 }
 #: `bwd_tile`: variants of the backward over tiles of receivers (trailing layout, at least 64
-#: channels): a block of `waves per block` waves shares the dm rows of a tile in LDS.
+#: channels): a block of `waves per block` waves shares the dm rows of a tile in LDS.  A fifth
+#: number is the receivers per tile the variant is tuned for (8 if absent): few enough that the
+#: LDS of a CU holds the tiles of as many blocks as its wave slots take.
 
 
 #: leading-channels layout: (waves per block, parts) variants.  The forward pass is never
@@ -257,7 +259,9 @@ def emit_edge_bwd(p: Part) -> list[str]:
     t = p.t
     lines = ["    // dx (this part's x rows) and dy (all Y) are written here; ds rows go to `ds` path by path.",
              "    // `dm`: anything indexable by the part's local output row (registers or LDS).",
-             "    template <int C, typename Dm, typename DsSink>",
+             "    // kAcc: dx holds running sums the edge's contributions are added to (else it is overwritten).",
+             "    // kPin: each row's dx sums are computed where the row is (see `pin`); for dm rows read from LDS.",
+             "    template <int C, bool kAcc = false, bool kPin = false, typename Dm, typename DsSink>",
              "    __device__ static __forceinline__ void edge_bwd(const Vec<C> *x, const float *y,",
              "                                                     const Vec<C> *s, const Dm &dm,",
              "                                                     Vec<C> *dx, float *dy, const DsSink &ds) {"]
@@ -284,7 +288,7 @@ def emit_edge_bwd(p: Part) -> list[str]:
                 if j in dx_init:
                     lines.append(f"                dx[{xj}] = vfma(g, {expr}, dx[{xj}]);")
                 else:
-                    lines.append(f"                dx[{xj}] = vmul(g, {expr});")
+                    lines.append(f"                dx[{xj}] = kAcc ? vfma(g, {expr}, dx[{xj}]) : vmul(g, {expr});")
                     dx_init.add(j)
                 lines.append(f"                {{ const Vec<C> pr = vmulv(dmi, x[{xj}]);")
                 for c, k in terms:
@@ -295,6 +299,7 @@ def emit_edge_bwd(p: Part) -> list[str]:
                         a_init.add(k)
                 lines.append("                }")
             lines.append("            }")
+            lines.append("            if (kPin) { " + " ".join(f"pin(dx[{p.xj[j]}]);" for j in cols) + " }")
         first = True
         for k in ks:
             if first:
@@ -472,7 +477,10 @@ def emit_table_source(t: "Table", name: str, desc: str, channels: int, symbols, 
         out += ["static int run_tile_row_bytes() {"]
         out += [ln.replace("VARIANT", "tuning().bwd_variant.load(std::memory_order_relaxed)") for ln in switch(
             tile, lambda v: f"tile_row_bytes<{v[0]}, {part_names[v[2]]}>();")]
-    tiled = "&run_bwd_tiled, &run_tile_row_bytes" if tile else "nullptr, nullptr"
+        out += ["static int run_tile_rows_default() {"]
+        out += [ln.replace("VARIANT", "tuning().bwd_variant.load(std::memory_order_relaxed)") for ln in switch(
+            tile, lambda v: f"{v[4] if len(v) > 4 else 8};")]
+    tiled = "&run_bwd_tiled, &run_tile_row_bytes, &run_tile_rows_default" if tile else "nullptr, nullptr, nullptr"
     out += [f"extern const Signature {symbols[0]} = {{",
             f'    "{desc}",',
             f"    {t.X}, {t.Y}, {t.Z}, {t.S}, {len(t.val)}, {channels}, E3J_AMD_LAYOUT_TRAILING, kVal, kIdx,",

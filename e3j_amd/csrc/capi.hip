@@ -413,6 +413,13 @@ int32_t e3j_amd_tile_rows(int32_t sig) {
     return bytes > 0 ? (int32_t)(160 * 1024 / bytes) : 0;
 }
 
+int32_t e3j_amd_tile_rows_default(int32_t sig) {
+    const int32_t limit = e3j_amd_tile_rows(sig);
+    if (limit <= 0) return 0;
+    const int32_t want = signature(sig).tile_rows_default ? signature(sig).tile_rows_default() : limit;
+    return want < 1 ? 1 : want > limit ? limit : want;
+}
+
 int e3j_amd_convolution_bwd_tiled(const e3j_amd_conv_params *p, const void *x, const void *y,
                                   const void *s, const void *dm, const int32_t *sender,
                                   const int32_t *receiver_ptr, const int32_t *edge_perm,

@@ -155,6 +155,7 @@ struct Signature {
                      const float *dm, const e3j_amd_tile_schedule &schedule, float *dx, float *dy,
                      float *ds, hipStream_t stream);
     int (*tile_row_bytes)();
+    int (*tile_rows_default)();  // receivers per tile the launch variant is tuned for
 };
 // built-in signatures (generated/registry.hip), then the ones registered at run time (capi.hip)
 // A table entry on the host, and the lookup of a table among the signatures (capi.hip): the

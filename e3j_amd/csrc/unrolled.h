@@ -39,6 +39,15 @@ __device__ __forceinline__ Vec<C> vzero() {
     for (int t = 0; t < C; t++) r.v[t] = 0.f;
     return r;
 }
+// Fixes the point in the instruction stream where `a` is computed: the value is an operand of
+// an (empty) statement the compiler keeps in program order.  Without it the instruction
+// selector emits a sum at its last use, and the operands of every term stay in registers
+// until then.
+template <int C>
+__device__ __forceinline__ void pin(Vec<C> &a) {
+#pragma unroll
+    for (int t = 0; t < C; t++) asm volatile("" : "+v"(a.v[t]));
+}
 template <int C>
 __device__ __forceinline__ Vec<C> vmul(const Vec<C> &a, float w) {
     Vec<C> r;
@@ -781,16 +790,10 @@ __device__ __forceinline__ void unrolled_bwd_tile_part(
 #pragma unroll
             for (int j = 0; j < NX; j++) acc[j] = vzero<CPL>();
         }
-        V dxe[NX];
         float dye[Red::P];
         const DsRows<CPL, K> ds_rows{ds + ee * (int64_t)(S * K) + c0, active};
         const DmTile<CPL> dm_rows{tile_lds + loc * (NZ * WIDTH) + lane * CPL};
-        Part::template edge_bwd<CPL>(xc, yc, sc, dm_rows, dxe, dye, ds_rows);
-#pragma unroll
-        for (int j = 0; j < NX; j++) {
-#pragma unroll
-            for (int t = 0; t < CPL; t++) acc[j].v[t] += dxe[j].v[t];
-        }
+        Part::template edge_bwd<CPL, true, true>(xc, yc, sc, dm_rows, acc, dye, ds_rows);  // adds to the run's sums
 #pragma unroll
         for (int k = Y; k < Red::P; k++) dye[k] = 0.f;
         Red::run(dye, lane, [&](int k, float sum) {

@@ -416,10 +416,10 @@ def _raw_backward(meta: _Meta, x, y, s, dm, sender, receiver, graph=None):
             dx.data_ptr(), dy.data_ptr(), ds.data_ptr())
     # tiles of receivers whose dm rows fit the LDS of a workgroup: dx summed per (tile, sender)
     tile_rows = 0
-    if group_receiver and not ordered and p.signature >= 0 and y.shape[0] > 0:
-        tile_rows = min(int(config().tile_rows), int(lib.e3j_amd_tile_rows(p.signature)))
+    if group_receiver and not ordered and y.shape[0] > 0 and p.layout == _lib.LAYOUT_TRAILING:
+        tile_rows = _tile_rows(p.signature)
     with torch.cuda.device(x.device):
-        if tile_rows >= 2:
+        if tile_rows >= 1:
             if prepared is None:
                 prepared = PreparedGraph(other, row_ptr, perm, order, n)
             schedule = prepared.schedule(tile_rows)
@@ -435,6 +435,18 @@ def _raw_backward(meta: _Meta, x, y, s, dm, sender, receiver, graph=None):
             fn = lib.e3j_amd_convolution_bwd_receiver if group_receiver else lib.e3j_amd_convolution_bwd_sender
             _lib.check(fn(*args, _stream(x.device)))
     return dx, dy, ds
+
+
+def _tile_rows(signature: int) -> int:
+    """Receivers per tile of the tiled backward for a compiled signature under the current
+    configuration; 0: the one-wave-per-receiver backward runs."""
+    want = int(config().tile_rows)
+    if signature < 0 or want == 0:
+        return 0
+    lib = _lib.load()
+    if want < 0:
+        return int(lib.e3j_amd_tile_rows_default(signature))
+    return min(want, int(lib.e3j_amd_tile_rows(signature)))
 
 
 def _sum(*terms):

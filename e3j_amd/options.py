@@ -106,9 +106,9 @@ class Config:
     graph_cache: bool = False
     #: receivers per tile of the backward that sums dx per (tile, sender) on chip before the float
     #: atomics and shares long rows between workgroups (trailing layout, unrolled kernels, at least
-    #: 64 channels; capped by what the LDS holds); 0 or 1 = one wave per receiver and one set of
-    #: atomics per edge (the default: as fast on graphs without long rows, and no schedule to build).
-    tile_rows: int = 0
+    #: 64 channels; capped by what the LDS holds).  -1: the size the kernel of the signature is
+    #: tuned for; 0: one wave per receiver and one set of atomics per edge (no schedule to build).
+    tile_rows: int = -1
     #: compile unrolled kernels at run time for coefficient tables the library was not built
     #: for (needs hipcc; about half a minute per new table, cached on disk); off: such tables
     #: run the table-driven kernels.
@@ -123,7 +123,7 @@ class _ConfigHolder:
             debug_level=int(os.environ.get("E3J_AMD_DEBUG", "0")),
             deterministic=os.environ.get("E3J_AMD_DETERMINISTIC", "0") not in ("0", ""),
             locality_rounds=int(os.environ.get("E3J_AMD_LOCALITY_ROUNDS", "2")),
-            tile_rows=int(os.environ.get("E3J_AMD_TILE_ROWS", "0")),
+            tile_rows=int(os.environ.get("E3J_AMD_TILE_ROWS", "-1")),
             graph_cache=os.environ.get("E3J_AMD_GRAPH_CACHE", "0") not in ("0", ""),
             jit=os.environ.get("E3J_AMD_JIT", "0") not in ("0", ""),
         )

@@ -159,6 +159,9 @@ typedef struct e3j_amd_tile_schedule {
 /* Largest `tile_rows` the tiled backward of a signature takes (its LDS holds the dm rows of a
  * tile), 0 if the signature has no tiled backward. */
 int32_t e3j_amd_tile_rows(int32_t signature);
+/* The `tile_rows` the tiled backward of a signature is tuned for (leaves room in the LDS for the
+ * number of workgroups per CU its launch shape wants), 0 if the signature has no tiled backward. */
+int32_t e3j_amd_tile_rows_default(int32_t signature);
 /* Number of work descriptors to provide for a graph (upper bound used by the builder). */
 int64_t e3j_amd_tile_schedule_num_work(int32_t num_nodes, int64_t num_edges, int32_t tile_rows,
                                        int32_t max_work_edges);
