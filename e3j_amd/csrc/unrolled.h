@@ -22,6 +22,7 @@
 #define E3J_AMD_CSRC_UNROLLED_H_
 
 #include <initializer_list>
+#include <type_traits>
 
 #include "common.h"
 
@@ -864,12 +865,30 @@ __global__ __launch_bounds__(kWave *WPB, MINW) void unrolled_bwd_tile_kernel(
 // only fences that keep the compiler from moving accesses across the turn.
 // ---------------------------------------------------------------------------
 constexpr int odd_stride(int n) { return (n % 2) ? n : n + 1; }
+
+// f(std::integral_constant<int, I>) for I = FIRST .. LAST - 1
+template <int FIRST, int LAST, typename F>
+__device__ __forceinline__ void static_for(F &&f) {
+    if constexpr (FIRST < LAST) {
+        f(std::integral_constant<int, FIRST>{});
+        static_for<FIRST + 1, LAST>(f);
+    }
+}
 constexpr int round4(int n) { return (n + 3) / 4 * 4; }
 
 __device__ __forceinline__ void strip_fence() {
     __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
     __builtin_amdgcn_wave_barrier();
     __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+}
+
+// Block barrier that orders LDS accesses only.  `__syncthreads()` also waits for every global
+// load, store and atomic of the wave (its fence covers all address spaces), which would drain
+// the next edge's prefetch and the previous edge's stores at each barrier of the edge loop.
+__device__ __forceinline__ void lds_barrier() {
+    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup", "local");
+    __builtin_amdgcn_s_barrier();
+    __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "workgroup", "local");
 }
 
 // Position in a strip (rows of ROW values at stride PAD) of element g of the linear block.
@@ -951,6 +970,70 @@ struct LinearBlock {
                     for (int t = 0; t < 4; t++) v[i][t] = strip[strip_index<ROW, PAD>(4 * idx + t)];
                 }
             }
+        }
+    }
+
+    // The same moves for a wave whose first thread index BASE is a compile-time constant (thread
+    // = BASE + lane).  Whether a step's pieces exist is then known per wave when the code is
+    // generated, and the global accesses of the loop are issued unconditionally: a step that
+    // only part of the wave owns clamps the other lanes to the wave's last piece (they load it
+    // again, and store the same values to the same place again).  With no global access under a
+    // condition the compiler's wait counts stay exact.
+    template <int BASE, int I>
+    static constexpr int step_kind() {  // 0: no lane owns a piece, 1: every lane, 2: the first lanes
+        return I * NT + BASE >= PIECES ? 0 : I * NT + BASE + kWave - 1 < PIECES ? 1 : 2;
+    }
+    template <int BASE, int I>
+    __device__ static __forceinline__ int piece(int lane) {
+        const int idx = I * NT + BASE + lane;
+        return step_kind<BASE, I>() == 2 && idx >= PIECES ? PIECES - 1 : idx;
+    }
+    template <int BASE, bool kStream, int I = 0>
+    __device__ __forceinline__ void load_at(const float *src, int lane) {
+        if constexpr (I < NV) {
+            if constexpr (step_kind<BASE, I>() != 0) {
+                const f32x4 *p = reinterpret_cast<const f32x4 *>(src) + piece<BASE, I>(lane);
+                v[I] = kStream ? __builtin_nontemporal_load(p) : *p;
+            }
+            load_at<BASE, kStream, I + 1>(src, lane);
+        }
+    }
+    template <int BASE, int I = 0>
+    __device__ __forceinline__ void store_at(float *dst, int lane) const {
+        if constexpr (I < NV) {
+            if constexpr (step_kind<BASE, I>() != 0)
+                __builtin_nontemporal_store(v[I], reinterpret_cast<f32x4 *>(dst) + piece<BASE, I>(lane));
+            store_at<BASE, I + 1>(dst, lane);
+        }
+    }
+    template <int BASE, int ROW, int PAD, int I = 0>
+    __device__ __forceinline__ void to_strip_at(float *strip, int lane) const {
+        if constexpr (I < NV) {
+            if constexpr (step_kind<BASE, I>() != 0) {
+                const int idx = piece<BASE, I>(lane);  // clamped lanes rewrite the last piece with its own values
+                if (PAD == ROW) {
+                    reinterpret_cast<f32x4 *>(strip)[idx] = v[I];
+                } else {
+#pragma unroll
+                    for (int t = 0; t < 4; t++) strip[strip_index<ROW, PAD>(4 * idx + t)] = v[I][t];
+                }
+            }
+            to_strip_at<BASE, ROW, PAD, I + 1>(strip, lane);
+        }
+    }
+    template <int BASE, int ROW, int PAD, int I = 0>
+    __device__ __forceinline__ void from_strip_at(const float *strip, int lane) {
+        if constexpr (I < NV) {
+            if constexpr (step_kind<BASE, I>() != 0) {
+                const int idx = piece<BASE, I>(lane);
+                if (PAD == ROW) {
+                    v[I] = reinterpret_cast<const f32x4 *>(strip)[idx];
+                } else {
+#pragma unroll
+                    for (int t = 0; t < 4; t++) v[I][t] = strip[strip_index<ROW, PAD>(4 * idx + t)];
+                }
+            }
+            from_strip_at<BASE, ROW, PAD, I + 1>(strip, lane);
         }
     }
 };
@@ -1093,13 +1176,15 @@ struct LeadingBwdGeometry : LeadingGeometry<K, X, S, Z> {
     static constexpr int GC = group();  // channels of dm rows staged at a time
 };
 
-template <typename Part, int K, int NP, unsigned long long kCoveredDx, bool kOrdered>
+template <typename Part, int K, int NP, int PART, unsigned long long kCoveredDx, bool kOrdered>
 __device__ __forceinline__ void unrolled_bwd_leading(
     const float *__restrict__ x, const float *__restrict__ y, const float *__restrict__ s,
     const float *__restrict__ dm, const int32_t *__restrict__ sender,
     const int32_t *__restrict__ row_ptr, const int32_t *__restrict__ perm,
     float *__restrict__ dx, float *__restrict__ dy, float *__restrict__ ds, int num_nodes,
-    float scale, unsigned y_flip, int part, int r, int slice, int lane, int tid, float *region) {
+    float scale, unsigned y_flip, int r, int slice, int lane, int tid, float *region) {
+    // PART: this wave's index in the block (tid = PART * 64 + lane), a constant of the generated code
+    constexpr int part = PART, BASE = PART * kWave;
     constexpr int NX = Part::NX, NS = Part::NS, NZ = Part::NZ, Y = Part::Y;
     constexpr int X = Part::X, S = Part::S, Z = Part::Z;
     static_assert(X <= 64 && S <= 64, "part masks hold 64 columns");
@@ -1145,27 +1230,32 @@ __device__ __forceinline__ void unrolled_bwd_leading(
     LinearBlock<XN, NT> xl;
     LinearBlock<SN, NT> sl;
     float yn[Y];
-    bool valid_n = false;
     int snd_n = 0;
     int64_t ee_n = 0;
+    // Padding edges (their dy/ds rows are zero-filled separately) are stepped over here, so the
+    // loop body is one straight line and its waits are exact counts (see the trailing kernel).
+    auto next_edge = [&](int p) {
+        while (p < e1 && !((unsigned)load_uniform(sender + p) < (unsigned)num_nodes)) p++;
+        return p;
+    };
     auto fetch = [&](int pos) {
-        const int snd = sender[pos];
-        valid_n = (unsigned)snd < (unsigned)num_nodes;
-        snd_n = valid_n ? snd : 0;
-        ee_n = perm ? (int64_t)perm[pos] : (int64_t)pos;
-        xl.template load<false>(x + ((int64_t)snd_n * K + ch0) * X, tid);
-        sl.template load<true>(s + (ee_n * K + ch0) * S, tid);
+        snd_n = load_uniform(sender + pos);
+        ee_n = perm ? (int64_t)load_uniform(perm + pos) : (int64_t)pos;
+        xl.template load_at<BASE, false>(x + ((int64_t)snd_n * K + ch0) * X, lane);
+        sl.template load_at<BASE, true>(s + (ee_n * K + ch0) * S, lane);
         const float *yr = y + ee_n * Y;
 #pragma unroll
         for (int k = 0; k < Y; k++) yn[k] = yr[k];
     };
+    e = next_edge(e);
     if (e < e1) fetch(e);
+    __builtin_amdgcn_s_waitcnt(kWaitVmcnt0);  // entered with nothing in flight
     while (e < e1) {
         // (the result strips of the previous edge are still being read by other waves: the
         // operand strips are separate, and the barrier below orders the next result writes)
-        xl.template to_strip<X, G::PX>(in_x, tid);
-        sl.template to_strip<S, G::PS>(in_s, tid);
-        __syncthreads();
+        xl.template to_strip_at<BASE, X, G::PX>(in_x, lane);
+        sl.template to_strip_at<BASE, S, G::PS>(in_s, lane);
+        lds_barrier();
         V xc[NX], sc[NS];
         float yc[Y];
 #pragma unroll
@@ -1174,15 +1264,14 @@ __device__ __forceinline__ void unrolled_bwd_leading(
         for (int l = 0; l < NS; l++) sc[l].v[0] = in_s[cl * G::PS + Part::kS[l]];
 #pragma unroll
         for (int k = 0; k < Y; k++) yc[k] = to_vgpr(flip_sign(yn[k], y_flip, k));
-        const bool valid = valid_n;  // uniform over the block: every wave looks at the same edge
         const int snd = snd_n;
         const int64_t ee = ee_n;
         const int pos = e;
-        e++;
+        e = next_edge(e + 1);
         if (e < e1) fetch(e);
 
         float dye[Red::P];
-        if (valid) {
+        {
             V dxe[NX];
             const DsStrip ds_strip{out_s + cl * G::PS, active};
             Part::template edge_bwd<1>(xc, yc, sc, dmr, dxe, dye, ds_strip);
@@ -1191,24 +1280,27 @@ __device__ __forceinline__ void unrolled_bwd_leading(
                 for (int j = 0; j < NX; j++) out_x[cl * G::PX + Part::kX[j]] = dxe[j].v[0];
             }
         }
-        __syncthreads();  // operands consumed by every wave, results of every wave in place
-        if (!valid) continue;  // padding edge: its dy/ds rows are zero-filled separately
+        lds_barrier();  // operands consumed by every wave, results of every wave in place
 
         LinearBlock<SN, NT> dl;
-        dl.template from_strip<S, G::PS>(out_s, tid);
-        dl.store(ds + (ee * K + ch0) * S, tid);
+        dl.template from_strip_at<BASE, S, G::PS>(out_s, lane);
+        dl.template store_at<BASE>(ds + (ee * K + ch0) * S, lane);
         if (kOrdered) {  // the contribution of this position as one row of the buffer, no atomics
             LinearBlock<XN, NT> ul;
-            ul.template from_strip<X, G::PX>(out_x, tid);
-            ul.store(dx + ((int64_t)pos * K + ch0) * X, tid);
+            ul.template from_strip_at<BASE, X, G::PX>(out_x, lane);
+            ul.template store_at<BASE>(dx + ((int64_t)pos * K + ch0) * X, lane);
         } else {
             float *dx_block = dx + ((int64_t)snd * K + ch0) * X;
-#pragma unroll
-            for (int i = 0; i < (XN + NT - 1) / NT; i++) {
-                const int g = i * NT + tid;
-                const bool mine = kAllDx ? (XN % NT == 0 || g < XN) : (((covered >> i) & 1u) != 0);
-                if (mine) unsafeAtomicAdd(dx_block + g, out_x[strip_index<X, G::PX>(g)]);
-            }
+            static_for<0, (XN + NT - 1) / NT>([&](auto step) {
+                constexpr int i = decltype(step)::value, first = i * NT + BASE;
+                // does this wave own elements in this step: none, all (no condition left), some
+                constexpr int kind = first >= XN ? 0 : first + kWave - 1 < XN ? 1 : 2;
+                if constexpr (kind != 0) {
+                    const int g = first + lane;
+                    const bool mine = kAllDx ? (kind == 1 || g < XN) : (((covered >> i) & 1u) != 0);
+                    if (mine) unsafeAtomicAdd(dx_block + g, out_x[strip_index<X, G::PX>(g)]);
+                }
+            });
         }
 
 #pragma unroll
@@ -1237,9 +1329,9 @@ __device__ __forceinline__ void dispatch_bwd_leading(int part, const float *x, c
                                                      unsigned y_flip, int r, int slice, int lane,
                                                      int tid, float *region) {
     if (part == I)
-        unrolled_bwd_leading<Part, K, NP, kCoveredDx, O>(x, y, s, dm, sender, row_ptr, perm, dx, dy, ds,
-                                                         num_nodes, scale, y_flip, part, r, slice, lane,
-                                                         tid, region);
+        unrolled_bwd_leading<Part, K, NP, I, kCoveredDx, O>(x, y, s, dm, sender, row_ptr, perm, dx, dy, ds,
+                                                            num_nodes, scale, y_flip, r, slice, lane, tid,
+                                                            region);
     else
         dispatch_bwd_leading<K, NP, kCoveredDx, O, I + 1, Rest...>(part, x, y, s, dm, sender, row_ptr,
                                                                    perm, dx, dy, ds, num_nodes, scale,

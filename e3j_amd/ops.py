@@ -416,7 +416,8 @@ def _raw_backward(meta: _Meta, x, y, s, dm, sender, receiver, graph=None):
             dx.data_ptr(), dy.data_ptr(), ds.data_ptr())
     # tiles of receivers whose dm rows fit the LDS of a workgroup: dx summed per (tile, sender)
     tile_rows = 0
-    if group_receiver and not ordered and y.shape[0] > 0 and p.layout == _lib.LAYOUT_TRAILING:
+    aligned = all(t.data_ptr() % 16 == 0 for t in (x, y, s, dm, dx, dy, ds))  # what the unrolled kernels take
+    if group_receiver and not ordered and y.shape[0] > 0 and p.layout == _lib.LAYOUT_TRAILING and aligned:
         tile_rows = _tile_rows(p.signature)
     with torch.cuda.device(x.device):
         if tile_rows >= 1:
