@@ -40,6 +40,10 @@ class ConvParams(ctypes.Structure):
         ("debug", ctypes.c_int32),
         ("y_flip", ctypes.c_uint32),
         ("row_order", ctypes.c_void_p),
+        ("row_cap", ctypes.c_int32),
+        ("row_piece", ctypes.c_int32),
+        ("max_segments", ctypes.c_int32),
+        ("segments", ctypes.c_void_p),
     ]
 
 
@@ -102,6 +106,9 @@ SYMBOLS = {
     "e3j_amd_convolution_bwd_receiver": (ctypes.c_int, [_PARAMS] + [_P] * 12),
     "e3j_amd_convolution_bwd_ordered_workspace_bytes": (ctypes.c_size_t, [_PARAMS]),
     "e3j_amd_convolution_bwd_ordered": (ctypes.c_int, [_PARAMS] + [_P] * 13),
+    "e3j_amd_row_segments_max": (ctypes.c_int64, [ctypes.c_int64, ctypes.c_int32]),
+    "e3j_amd_row_segments_build": (ctypes.c_int, [ctypes.c_void_p, ctypes.c_int32, ctypes.c_int32, ctypes.c_int32,
+                                                  ctypes.c_int32, ctypes.c_void_p, ctypes.c_void_p]),
     "e3j_amd_tile_rows": (ctypes.c_int32, [ctypes.c_int32]),
     "e3j_amd_tile_rows_default": (ctypes.c_int32, [ctypes.c_int32]),
     "e3j_amd_tile_schedule_num_work": (ctypes.c_int64, [ctypes.c_int32, ctypes.c_int64, ctypes.c_int32, ctypes.c_int32]),

@@ -415,10 +415,11 @@ def emit_table_source(t: "Table", name: str, desc: str, channels: int, symbols, 
                 "    const int32_t *, const int32_t *, const int32_t *, float *, float *, float *, int, float,",
                 "    unsigned);"]
     out += ["}  // namespace", "", "// both passes: the device pass needs the kernels instantiated"]
+    fwd_args_trailing = [fwd_args[0], fwd_args[1].replace("unsigned);", "unsigned, int, int, const int32_t *, int);")]
     for v in launch["fwd"]:
         cpl, wpb, zs, minw = (*v, 1)[:4]
         out += [f"template __global__ void unrolled_fwd_kernel<{channels}, {cpl}, {wpb}, {minw}, "
-                f"{part_names[zs]}>("] + fwd_args
+                f"{part_names[zs]}>("] + fwd_args_trailing
     for v in launch["bwd"]:
         cpl, wpb, zs, minw = (*v, 1)[:4]
         for ordered in ("false", "true"):

@@ -286,6 +286,13 @@ int e3j_amd_convolution_fwd(const e3j_amd_conv_params *p, const void *coef, cons
         missing(sender, p->num_edges) || missing(y, p->num_edges) || missing(s, p->num_edges) ||
         (p->signature < 0 && missing(coef, p->num_coef)))
         return set_error(E3J_AMD_INVALID_ARGUMENT, "convolution: null operand");
+    const bool split_rows = p->row_cap > 0 || p->segments != nullptr;
+    if (p->row_cap < 0 || p->max_segments < 0 || p->row_piece < 0 || p->row_piece > p->row_cap)
+        return set_error(E3J_AMD_INVALID_ARGUMENT, "convolution: row_cap / row_piece / max_segments");
+    if (split_rows && !(signature_fits(p, {x, s, out}) && p->layout == E3J_AMD_LAYOUT_TRAILING))
+        return set_error(E3J_AMD_UNIMPLEMENTED,
+                         "convolution: row_cap / segments are taken by the unrolled kernels of the "
+                         "trailing layout only (16-byte aligned operands)");
     if (signature_fits(p, {x, s, out})) {
         rc = signature(p->signature).fwd(*p, static_cast<const float *>(x), static_cast<const float *>(y),
                                          static_cast<const float *>(s), sender, receiver_ptr,

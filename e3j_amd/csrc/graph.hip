@@ -51,13 +51,18 @@ __global__ void gather_kernel(const int32_t *__restrict__ src, const int32_t *__
 
 // One sweep of minimum-label propagation over a CSR adjacency:
 // next[n] = min(cur[n], cur[m] for every m in row n).  One thread per row, no atomics.
+// A row is read up to kLabelRowCap positions: the labels only steer which rows run together,
+// and a thread that walked a hub's whole row would outlast the rest of the sweep many times.
+constexpr int kLabelRowCap = 128;
 __global__ void min_label_kernel(const int32_t *__restrict__ other,
                                  const int32_t *__restrict__ row_ptr, int num_nodes,
                                  const int32_t *__restrict__ cur, int32_t *__restrict__ next) {
     const int n = blockIdx.x * blockDim.x + threadIdx.x;
     if (n >= num_nodes) return;
     int best = cur[n];
-    for (int e = row_ptr[n]; e < row_ptr[n + 1]; e++) {
+    const int begin = row_ptr[n];
+    const int end = min(row_ptr[n + 1], begin + kLabelRowCap);
+    for (int e = begin; e < end; e++) {
         const int m = other[e];
         if ((unsigned)m < (unsigned)num_nodes) best = min(best, cur[m]);
     }
@@ -237,7 +242,8 @@ __global__ void tile_entries_kernel(const uint64_t *__restrict__ keys, const int
     }
 }
 
-// descriptors (tile, begin, end, 0); `starts` / `first_piece`: inclusive prefix sums, entry 0 = 0
+// descriptors (tile, begin, end, 0), the first num_used of the num_work entries, num_used in the
+// fourth field of descriptor 0; `starts` / `first_piece`: inclusive prefix sums, entry 0 = 0
 __global__ void tile_work_kernel(const int32_t *__restrict__ starts, const int32_t *__restrict__ first_piece,
                                  int num_tiles, int max_work_edges, int32_t *__restrict__ work) {
     const int t = blockIdx.x * blockDim.x + threadIdx.x;
@@ -250,6 +256,8 @@ __global__ void tile_work_kernel(const int32_t *__restrict__ starts, const int32
         work[4 * w + 2] = b + max_work_edges < end ? b + max_work_edges : end;
         work[4 * w + 3] = 0;
     }
+    // the number of descriptors in use, for the kernel to deal them evenly to the XCDs
+    if (t == 0) work[3] = first_piece[num_tiles];
 }
 
 size_t sort64_temp_bytes(int64_t num_edges) {
@@ -405,6 +413,44 @@ int e3j_amd_csr_row_ptr_static(const int32_t *key, int64_t num_edges, int32_t nu
     int rc = static_scratch(&temp);
     if (rc) return rc;
     return row_ptr_impl(key, num_edges, num_nodes, row_ptr, temp, need, static_cast<hipStream_t>(stream_));
+}
+
+// Pieces of the rows longer than `cap`, past their first `cap` positions: a row reserves its
+// pieces with one atomic on the count (the order of the list is free).
+__global__ void row_segments_kernel(const int32_t *__restrict__ row_ptr, int num_nodes, int cap, int piece,
+                                    int max_segments, int32_t *__restrict__ segments) {
+    const int r = blockIdx.x * blockDim.x + threadIdx.x;
+    if (r >= num_nodes) return;
+    const int begin = row_ptr[r], end = row_ptr[r + 1];
+    if (end - begin <= cap) return;
+    const int extra = (end - begin - 1) / piece;  // pieces after the first
+    const int at = atomicAdd(segments, extra);
+    for (int k = 0; k < extra && at + k < max_segments; k++) {
+        const int b = begin + (k + 1) * piece;
+        int32_t *seg = segments + 4 + 3 * (at + k);
+        seg[0] = r;
+        seg[1] = b;
+        seg[2] = b + piece < end ? b + piece : end;
+    }
+}
+
+int64_t e3j_amd_row_segments_max(int64_t num_edges, int32_t row_piece) {
+    if (num_edges <= 0 || row_piece <= 0) return 0;
+    return num_edges / row_piece;  // a piece after the first follows row_piece positions of its row
+}
+
+int e3j_amd_row_segments_build(const int32_t *receiver_ptr, int32_t num_nodes, int32_t row_cap,
+                               int32_t row_piece, int32_t max_segments, int32_t *segments, void *stream_) {
+    if (num_nodes < 0 || row_piece <= 0 || row_cap < row_piece || max_segments < 0)
+        return set_error(E3J_AMD_INVALID_ARGUMENT, "row_segments_build: bad sizes");
+    if (segments == nullptr || (num_nodes > 0 && receiver_ptr == nullptr))
+        return set_error(E3J_AMD_INVALID_ARGUMENT, "row_segments_build: null operand");
+    hipStream_t stream = static_cast<hipStream_t>(stream_);
+    int rc = launch_fill_zero(segments, sizeof(int32_t) * 4, stream);
+    if (rc || num_nodes == 0) return rc;
+    hipLaunchKernelGGL(row_segments_kernel, dim3(grid_for(num_nodes)), dim3(256), 0, stream, receiver_ptr,
+                       num_nodes, row_cap, row_piece, max_segments, segments);
+    return check_hip(hipGetLastError(), "row_segments_build");
 }
 
 int e3j_amd_wrap_index(const int32_t *index, int64_t n, int32_t num_nodes, int32_t *out,

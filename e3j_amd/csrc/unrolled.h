@@ -339,7 +339,10 @@ template <typename Part, int K, int CPL>
 __device__ __forceinline__ void unrolled_fwd_part(
     const float *__restrict__ x, const float *__restrict__ y, const float *__restrict__ s,
     const int32_t *__restrict__ sender, const int32_t *__restrict__ row_ptr,
-    const int32_t *__restrict__ perm, float *__restrict__ out, int num_nodes, float scale, unsigned y_flip, int r, int slice, int lane) {
+    const int32_t *__restrict__ perm, float *__restrict__ out, int num_nodes, float scale, unsigned y_flip, int r, int slice, int lane,
+    int e, int e1, bool add) {
+    // [e, e1): the positions of row r this wave sums; add: into `out` by float atomics (one of
+    // several waves that share a long row) instead of storing the row
     constexpr int NX = Part::NX, NS = Part::NS, NZ = Part::NZ, Y = Part::Y;
     constexpr int X = Part::X, S = Part::S, Z = Part::Z;
     using V = Vec<CPL>;
@@ -354,9 +357,6 @@ __device__ __forceinline__ void unrolled_fwd_part(
     V acc[NZ];
 #pragma unroll
     for (int i = 0; i < NZ; i++) acc[i] = vzero<CPL>();
-
-    int e = row_ptr[r];
-    const int e1 = row_ptr[r + 1];
 
     V xn[NX], sn[NS];
     float yn[Y];
@@ -404,26 +404,37 @@ __device__ __forceinline__ void unrolled_fwd_part(
     }
     if (active && sub == 0) {
         float *orow = out + (int64_t)r * (Z * K) + c0;
+        if (!add) {
 #pragma unroll
-        for (int i = 0; i < NZ; i++) store_stream<CPL>(orow + Part::kZ[i] * K, vmul(acc[i], scale));
+            for (int i = 0; i < NZ; i++) store_stream<CPL>(orow + Part::kZ[i] * K, vmul(acc[i], scale));
+        } else {
+#pragma unroll
+            for (int i = 0; i < NZ; i++) {
+#pragma unroll
+                for (int t = 0; t < CPL; t++)
+                    unsafeAtomicAdd(orow + Part::kZ[i] * K + t, acc[i].v[t] * scale);
+            }
+        }
     }
 }
 
 template <int K, int CPL, int I>
 __device__ __forceinline__ void dispatch_fwd(int, const float *, const float *, const float *,
                                              const int32_t *, const int32_t *, const int32_t *,
-                                             float *, int, float, unsigned, int, int, int) {}
+                                             float *, int, float, unsigned, int, int, int, int, int,
+                                             bool) {}
 template <int K, int CPL, int I, typename Part, typename... Rest>
 __device__ __forceinline__ void dispatch_fwd(int part, const float *x, const float *y, const float *s,
                                              const int32_t *sender, const int32_t *row_ptr,
                                              const int32_t *perm, float *out, int num_nodes,
-                                             float scale, unsigned y_flip, int r, int slice, int lane) {
+                                             float scale, unsigned y_flip, int r, int slice, int lane,
+                                             int e, int e1, bool add) {
     if (part == I)
         unrolled_fwd_part<Part, K, CPL>(x, y, s, sender, row_ptr, perm, out, num_nodes, scale, y_flip, r,
-                                        slice, lane);
+                                        slice, lane, e, e1, add);
     else
         dispatch_fwd<K, CPL, I + 1, Rest...>(part, x, y, s, sender, row_ptr, perm, out, num_nodes,
-                                             scale, y_flip, r, slice, lane);
+                                             scale, y_flip, r, slice, lane, e, e1, add);
 }
 
 // One wave per (receiver, channel slice, part); consecutive waves share a receiver.
@@ -433,17 +444,34 @@ __global__ __launch_bounds__(kWave *WPB, MINW) void unrolled_fwd_kernel(
     const float *__restrict__ x, const float *__restrict__ y, const float *__restrict__ s,
     const int32_t *__restrict__ sender, const int32_t *__restrict__ row_ptr,
     const int32_t *__restrict__ perm, const int32_t *__restrict__ row_order,
-    float *__restrict__ out, int num_nodes, float scale, unsigned y_flip) {
+    float *__restrict__ out, int num_nodes, float scale, unsigned y_flip, int row_cap, int row_piece,
+    const int32_t *__restrict__ segments, int max_segments) {
+    // segments == nullptr: one item per row; a row longer than row_cap (> 0) is cut after
+    // row_piece positions.
+    // Otherwise the items are the listed pieces of long rows (count in segments[0], then
+    // (row, begin, end) from segments[4] on), whose sums are added to `out`.
     constexpr int NP = sizeof...(Parts);
     constexpr int CW = Slice<K, CPL>::COUNT;
     const int64_t item = logical_block() * WPB + threadIdx.y;
-    if (item >= (int64_t)num_nodes * (CW * NP)) return;
+    const int rows = segments ? min(segments[0], max_segments) : num_nodes;
+    if (item >= (int64_t)rows * (CW * NP)) return;
     const int part = uniform((int)(item % NP));
     const int slice = uniform((int)((item / NP) % CW));
     const int q = uniform((int)(item / (NP * CW)));
-    const int r = row_order ? row_order[q] : q;
-    dispatch_fwd<K, CPL, 0, Parts...>(part, x, y, s, sender, row_ptr, perm, out, num_nodes, scale, y_flip, r,
-                                      slice, threadIdx.x);
+    int r, e, e1;
+    if (segments) {
+        r = segments[4 + 3 * q];
+        e = segments[5 + 3 * q];
+        e1 = segments[6 + 3 * q];
+    } else {
+        r = row_order ? row_order[q] : q;
+        e = row_ptr[r];
+        e1 = row_ptr[r + 1];
+        if (row_cap > 0 && e1 - e > row_cap) e1 = e + row_piece;
+    }
+    dispatch_fwd<K, CPL, 0, Parts...>(part, x, y, s, sender, row_ptr, perm, out, num_nodes, scale, y_flip,
+                                      uniform(r), slice, threadIdx.x, uniform(e), uniform(e1),
+                                      segments != nullptr);
 }
 
 // ---------------------------------------------------------------------------
@@ -843,8 +871,14 @@ __global__ __launch_bounds__(kWave *WPB, MINW) void unrolled_bwd_tile_kernel(
     constexpr int NP = sizeof...(Parts);
     constexpr int CW = Slice<K, CPL>::COUNT;
     constexpr bool kAtomicDy = NP * CW > 1;  // several waves add into one dy row
-    const int64_t item = logical_block();
-    if (item >= (int64_t)num_work * (CW * NP)) return;  // whole block: no barrier is left waiting
+    // The grid covers all num_work descriptors, of which the first work[3] are in use: those are
+    // dealt to the XCDs in contiguous eighths (see logical_block), the surplus blocks leave.
+    const int used = min(work[3], num_work);
+    const int64_t items = (int64_t)used * (CW * NP);
+    const int64_t per_xcd = (items + kXcds - 1) / kXcds;
+    if ((int64_t)(blockIdx.x / kXcds) >= per_xcd) return;  // whole block: no barrier is left waiting
+    const int64_t item = (int64_t)(blockIdx.x % kXcds) * per_xcd + blockIdx.x / kXcds;
+    if (item >= items) return;
     const int part = (int)(item % NP);
     const int slice = (int)((item / NP) % CW);
     const int64_t w = item / (NP * CW);
@@ -1375,11 +1409,14 @@ int launch_unrolled_fwd(const e3j_amd_conv_params &p, const float *x, const floa
                         const int32_t *sender, const int32_t *row_ptr, const int32_t *perm,
                         float *out, hipStream_t stream) {
     constexpr int64_t PER_NODE = (int64_t)Slice<K, CPL>::COUNT * sizeof...(Parts);
-    const int64_t blocks = padded_grid(((int64_t)p.num_nodes * PER_NODE + WPB - 1) / WPB);
+    const int64_t items = p.segments ? (int64_t)p.max_segments : (int64_t)p.num_nodes;
+    const int64_t blocks = padded_grid((items * PER_NODE + WPB - 1) / WPB);
     if (blocks > 0x7fffffffLL) return set_error(E3J_AMD_INVALID_ARGUMENT, "convolution: grid too large");
+    if (blocks == 0) return E3J_AMD_OK;
     hipLaunchKernelGGL((unrolled_fwd_kernel<K, CPL, WPB, MINW, Parts...>), dim3((unsigned)blocks),
                        dim3(kWave, WPB), 0, stream, x, y, s, sender, row_ptr, perm, p.row_order, out,
-                       p.num_nodes, p.coef_scale, p.y_flip);
+                       p.num_nodes, p.coef_scale, p.y_flip, p.row_cap,
+                       p.row_piece > 0 ? p.row_piece : p.row_cap, p.segments, p.max_segments);
     return check_hip(hipGetLastError(), "convolution forward launch");
 }
 

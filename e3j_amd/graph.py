@@ -106,7 +106,41 @@ def locality_order(other: torch.Tensor, row_ptr: torch.Tensor, num_nodes: int,
 
 #: edge positions per work item of the tiled backward: longer tile lists (hub rows) are cut
 #: into pieces of this many positions, each taken by a workgroup of its own
-MAX_WORK_EDGES = 2048
+MAX_WORK_EDGES = 256
+
+
+#: smallest row length above which the forward pass shares a row between waves, and the
+#: positions per wave of a shared row
+MIN_ROW_CAP = 64
+ROW_PIECE = 64
+
+
+def row_cap_for(num_nodes: int, num_edges: int) -> int:
+    """Row length above which the forward pass shares a row between waves: twice the mean
+    degree (at least 64), which no row of a radius graph of even density reaches."""
+    mean = num_edges / max(num_nodes, 1)
+    return max(MIN_ROW_CAP, int(2 * mean))
+
+
+class RowSegments:
+    """The pieces of long rows for the second call of the forward pass
+    (`e3j_amd_row_segments_build`).  `count`: pieces to launch, the bound `num_edges // row_piece`
+    (the list's own count, which the kernel reads on the device, is never read back: the
+    surplus workgroups of the second call leave at once, which costs less than a wait)."""
+
+    def __init__(self, row_ptr: torch.Tensor, num_nodes: int, num_edges: int, row_cap: int,
+                 row_piece: int = ROW_PIECE):
+        device = _require_device(row_ptr)
+        lib = _lib.load()
+        self.row_cap = int(row_cap)
+        self.row_piece = min(int(row_piece), self.row_cap)
+        self.max_segments = int(lib.e3j_amd_row_segments_max(int(num_edges), self.row_piece))
+        self.buffer = torch.empty(4 + 3 * self.max_segments, dtype=INDEX_DTYPE, device=device)
+        with torch.cuda.device(device):
+            _lib.check(lib.e3j_amd_row_segments_build(
+                row_ptr.data_ptr(), int(num_nodes), self.row_cap, self.row_piece, self.max_segments,
+                self.buffer.data_ptr(), _stream_ptr(device)))
+        self.count = self.max_segments
 
 
 class TileSchedule:

@@ -25,8 +25,8 @@ import torch
 
 from . import _lib
 from .coef import Coef4D
-from .graph import (TileSchedule, csr_row_ptr, fold_endpoints, locality_order,
-                    sort_edges, wrap_global_index)
+from .graph import (RowSegments, TileSchedule, csr_row_ptr, fold_endpoints, locality_order,
+                    row_cap_for, sort_edges, wrap_global_index)
 from .options import GraphOrdering, Layout, config
 
 
@@ -249,6 +249,7 @@ class PreparedGraph:
         self.num_nodes = int(num_nodes)
         self.ordering = ordering
         self._schedules = {}
+        self._segments = {}
         self._mark()
 
     def _mark(self):
@@ -278,6 +279,16 @@ class PreparedGraph:
             self.ready()
             hit = self._schedules[tile_rows] = TileSchedule(self.other, self.row_ptr, self.perm, self.order,
                                                             self.num_nodes, tile_rows)
+            self._mark()
+        return hit
+
+
+    def segments(self, row_cap: int) -> RowSegments:
+        """The pieces of the rows longer than `row_cap` (second call of the forward pass)."""
+        hit = self._segments.get(row_cap)
+        if hit is None:
+            self.ready()
+            hit = self._segments[row_cap] = RowSegments(self.row_ptr, self.num_nodes, self.num_edges, row_cap)
             self._mark()
         return hit
 
@@ -354,11 +365,27 @@ def _raw_forward(meta: _Meta, x, y, s, sender, receiver, graph=None) -> torch.Te
         out = torch.empty((x.shape[0], meta.params.num_out, x.shape[2]), dtype=x.dtype, device=x.device)
     else:
         out = torch.empty((x.shape[0], x.shape[1], meta.params.num_out), dtype=x.dtype, device=x.device)
+    # Rows much longer than the mean are shared between waves: the first call cuts every row at
+    # `cap` positions, a second call adds the remaining pieces (unrolled kernels of the trailing
+    # layout; off in deterministic mode, where a row's sum must not depend on an order of atomics)
+    cap = 0
+    if (p.signature >= 0 and meta.layout == Layout.TRAILING_CHANNELS and not config().deterministic
+            and isinstance(graph, PreparedGraph) and y.shape[0] > 0
+            and all(t.data_ptr() % 16 == 0 for t in (x, s, out))):
+        want = int(config().row_cap)
+        cap = row_cap_for(x.shape[0], y.shape[0]) if want < 0 else want
+    lib = _lib.load()
     with torch.cuda.device(x.device):
-        _lib.check(_lib.load().e3j_amd_convolution_fwd(
-            ctypes.byref(p), table.device(x.device).data_ptr(), x.data_ptr(), y.data_ptr(), s.data_ptr(),
-            other.data_ptr(), row_ptr.data_ptr(), perm.data_ptr() if perm is not None else None,
-            out.data_ptr(), _stream(x.device)))
+        args = (table.device(x.device).data_ptr(), x.data_ptr(), y.data_ptr(), s.data_ptr(),
+                other.data_ptr(), row_ptr.data_ptr(), perm.data_ptr() if perm is not None else None,
+                out.data_ptr(), _stream(x.device))
+        pieces = graph.segments(cap) if cap > 0 else None
+        if pieces is not None:
+            p.row_cap, p.row_piece = cap, pieces.row_piece
+        _lib.check(lib.e3j_amd_convolution_fwd(ctypes.byref(p), *args))
+        if pieces is not None and pieces.count > 0:
+            p.segments, p.max_segments = pieces.buffer.data_ptr(), pieces.count
+            _lib.check(lib.e3j_amd_convolution_fwd(ctypes.byref(p), *args))
     return out
 
 

@@ -109,6 +109,10 @@ class Config:
     #: 64 channels; capped by what the LDS holds).  -1: the size the kernel of the signature is
     #: tuned for; 0: one wave per receiver and one set of atomics per edge (no schedule to build).
     tile_rows: int = -1
+    #: positions of a row one wave of the forward pass sums; longer rows are shared between waves
+    #: (their sums then come from float atomics).  -1: twice the mean row length, at least 64;
+    #: 0: never share a row.
+    row_cap: int = -1
     #: compile unrolled kernels at run time for coefficient tables the library was not built
     #: for (needs hipcc; about half a minute per new table, cached on disk); off: such tables
     #: run the table-driven kernels.
@@ -124,6 +128,7 @@ class _ConfigHolder:
             deterministic=os.environ.get("E3J_AMD_DETERMINISTIC", "0") not in ("0", ""),
             locality_rounds=int(os.environ.get("E3J_AMD_LOCALITY_ROUNDS", "2")),
             tile_rows=int(os.environ.get("E3J_AMD_TILE_ROWS", "-1")),
+            row_cap=int(os.environ.get("E3J_AMD_ROW_CAP", "-1")),
             graph_cache=os.environ.get("E3J_AMD_GRAPH_CACHE", "0") not in ("0", ""),
             jit=os.environ.get("E3J_AMD_JIT", "0") not in ("0", ""),
         )

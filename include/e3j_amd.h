@@ -78,6 +78,20 @@ typedef struct e3j_amd_conv_params {
      * 0..num_nodes-1), e.g. from e3j_amd_locality_order; NULL = natural order.  It only
      * changes which rows run together (cache reuse of gathered rows), never the results. */
     const int32_t *row_order;
+    /* Long rows of the forward pass (unrolled kernels, trailing layout; anything else answers
+     * E3J_AMD_UNIMPLEMENTED when one of these is set).  One wave sums a row edge by edge, so a
+     * receiver with very many edges would hold one wave for the whole launch.  With row_cap > 0
+     * the wave of a row longer than row_cap sums only its first row_piece edges (row_piece <=
+     * row_cap; 0 means row_cap).  The rest of every such row is listed in `segments`, in
+     * pieces of row_piece edges (e3j_amd_row_segments_build), and summed by a second call of
+     * e3j_amd_convolution_fwd with `segments` set, which ADDS to `out` with float atomics (so it
+     * runs after the first call, on the same stream, and the sum of a split row depends on the
+     * order of the additions).  segments: device, int32: [0] = number of pieces n (at most
+     * max_segments are run), [4 + 3 i ...] = (row, first position, end position) of piece i. */
+    int32_t row_cap;
+    int32_t row_piece;
+    int32_t max_segments;
+    const int32_t *segments;
 } e3j_amd_conv_params;
 
 /* Message of the last failure on the calling thread ("" if none). */
@@ -151,11 +165,23 @@ int e3j_amd_convolution_bwd_ordered(const e3j_amd_conv_params *p, const void *co
 typedef struct e3j_amd_tile_schedule {
     int32_t tile_rows;     /* receivers per tile */
     int32_t num_work;      /* entries of `work` (an upper bound; unused entries have begin == end) */
-    const int32_t *work;   /* (num_work, 4) */
+    const int32_t *work;   /* (num_work, 4): (tile, begin, end, 0), the entries in use first; the
+                              fourth field of entry 0 holds their number */
     const int32_t *sender; /* (E) sender of the position, -1 for a padding edge */
     const int32_t *edge;   /* (E) row of y / s / dy / ds */
     const int32_t *local;  /* (E) index of the position's receiver within its tile */
 } e3j_amd_tile_schedule;
+/* The list of pieces for e3j_amd_conv_params.segments: every row of the CSR longer than row_cap
+ * is cut into pieces of at most row_piece positions (1 <= row_piece <= row_cap), and all but the
+ * first are listed (the forward pass with p->row_cap / row_piece set sums the first).
+ * `segments` holds 4 + 3 * max_segments int32; e3j_amd_row_segments_max bounds the number of
+ * pieces for any graph with that many edges.  One small kernel after a 16-byte fill; no workspace.  No counterpart in the
+ * reference, whose forward kernel also walks the edges of a receiver one after another in one
+ * block (lib/e3j_ops/cuda/convolution/fwd.cuh:346-363). */
+int64_t e3j_amd_row_segments_max(int64_t num_edges, int32_t row_piece);
+int e3j_amd_row_segments_build(const int32_t *receiver_ptr, int32_t num_nodes, int32_t row_cap,
+                               int32_t row_piece, int32_t max_segments, int32_t *segments,
+                               void *stream);
 /* Largest `tile_rows` the tiled backward of a signature takes (its LDS holds the dm rows of a
  * tile), 0 if the signature has no tiled backward. */
 int32_t e3j_amd_tile_rows(int32_t signature);

@@ -1,0 +1,167 @@
+"""Receivers with very many edges: the forward pass shares a long row between waves (the row
+cut at `row_cap` positions, the rest as listed pieces added with float atomics), the tiled
+backward cuts a tile's edge list into work pieces.  Checked against the CPU oracle on a star
+(one receiver takes every edge), on a graph that mixes long rows, ordinary rows, empty rows and
+padding edges, and for run time against a graph of the same size with uniform degrees."""
+
+import ctypes
+import zlib
+
+import numpy as np
+import pytest
+import torch
+
+import e3j_amd
+from e3j_amd import _lib, workloads as W
+from e3j_amd.graph import RowSegments, csr_row_ptr, row_cap_for
+from e3j_amd.ops import convolution
+from tests import helpers as H
+
+pytestmark = pytest.mark.gpu
+
+DUMMY = int(np.iinfo(np.int32).max)
+
+
+def _workload(kind: str, n: int, e: int, seed: int, channels: int = 128):
+    """cfg3's operator (x, y 0e..3o -> 0e..3o) on a graph of `n` nodes and about `e` edges."""
+    rng = np.random.default_rng(seed)
+    base = W.config3(0.0003, channels=channels)
+    if kind == "star":
+        receiver = np.full(e, n // 3)
+        sender = rng.integers(0, n, e)
+    elif kind == "uniform":
+        receiver = np.sort(rng.integers(0, n, e))
+        sender = rng.integers(0, n, e)
+    else:  # mixed: three long rows of different lengths (one an exact multiple of the cap),
+        # ordinary rows, empty rows, padding edges inside long rows and behind the last row
+        long_rows = [(5, 64 * 9), (n // 2, 700), (n - 1, 65)]
+        receiver = np.concatenate([np.full(m, r) for r, m in long_rows] + [rng.integers(0, n // 4, e)])
+        receiver = np.sort(receiver)
+        sender = rng.integers(0, n, receiver.shape[0])
+        sender[rng.random(sender.shape[0]) < 0.1] = DUMMY
+        receiver = np.concatenate([receiver, np.full(30, DUMMY)])
+        sender = np.concatenate([sender, rng.integers(0, n, 30)])
+    e = receiver.shape[0]
+    f32 = lambda a: torch.as_tensor(a.astype(np.float32))
+    x = f32(rng.normal(size=(n,) + tuple(base.x.shape[1:])))
+    dm = f32(rng.normal(size=(n,) + tuple(base.dm.shape[1:])))
+    y = f32(rng.normal(size=(e, base.y.shape[1])))
+    s = f32(rng.normal(size=(e,) + tuple(base.s.shape[1:])) * 0.2)
+    return W.Workload(kind, base.module, x, y, s, dm, torch.as_tensor(sender.astype(np.int32)),
+                      torch.as_tensor(receiver.astype(np.int32)), np.zeros((n, 3)), 0.0)
+
+
+def _check(w, what):
+    d = w.to("cuda")
+    x, y, s = (t.clone().requires_grad_(True) for t in (d.x, d.y, d.s))
+    out = convolution(w.module._packed_coef("float32"), x, y, s, d.sender, d.receiver, w.module.params)
+    dx, dy, ds = torch.autograd.grad(out, (x, y, s), d.dm)
+    idx, val, mix = w.table()
+    a = w.numpy()
+    ref, mag = H.forward_reference(idx, val, mix, a["x"], a["y"], a["s"], a["sender"], a["receiver"],
+                                   w.module.params.num_out)
+    H.assert_parity(out.detach().cpu().numpy(), ref, mag, f"{what} out")
+    refs, mags = H.backward_reference(idx, val, mix, a["x"], a["y"], a["s"], a["sender"], a["receiver"], a["dm"])
+    for g, r, m, name in zip((dx, dy, ds), refs, mags, ("dx", "dy", "ds")):
+        H.assert_parity(g.cpu().numpy(), r, m, f"{what} {name}")
+
+
+def test_segment_list_matches_a_host_restatement():
+    rng = np.random.default_rng(3)
+    n, cap, piece = 500, 100, 64
+    degree = rng.integers(0, 40, n)
+    degree[[7, 100, 499]] = [100, 101, 1000]   # not longer than the cap: left whole
+    degree[250] = 128
+    ptr = np.concatenate([[0], np.cumsum(degree)]).astype(np.int32)
+    seg = RowSegments(torch.as_tensor(ptr).cuda(), n, int(ptr[-1]), cap, piece)
+    torch.cuda.synchronize()
+    buf = seg.buffer.cpu().numpy()
+    count = int(buf[0])
+    want = set()
+    for r in range(n):
+        if degree[r] > cap:
+            for b in range(ptr[r] + piece, ptr[r + 1], piece):
+                want.add((r, b, min(b + piece, ptr[r + 1])))
+    assert len(want) == 1 + 15 + 1
+    assert count == len(want) <= seg.max_segments == int(ptr[-1]) // piece
+    got = {tuple(int(v) for v in buf[4 + 3 * i: 7 + 3 * i]) for i in range(count)}
+    assert got == want
+
+
+@pytest.mark.parametrize("kind,n,e", [("star", 600, 50000), ("mixed", 400, 3000)])
+def test_long_rows_match_oracle(kind, n, e):
+    w = _workload(kind, n, e, zlib.crc32(kind.encode()))
+    assert row_cap_for(n, w.num_edges) < 600
+    _check(w, kind)
+
+
+def test_long_rows_with_row_sharing_off_and_in_deterministic_mode():
+    """`row_cap=0` keeps one wave per row; deterministic mode never shares a row (and gives the
+    same bits twice)."""
+    w = _workload("mixed", 300, 2000, 11)
+    with e3j_amd.config.use(row_cap=0):
+        _check(w, "row_cap=0")
+    d = w.to("cuda")
+    with e3j_amd.config.use(deterministic=True):
+        _check(w, "deterministic")
+        outs = [convolution(w.module._packed_coef("float32"), d.x, d.y, d.s, d.sender, d.receiver, w.module.params)
+                for _ in range(2)]
+    assert torch.equal(outs[0], outs[1])
+
+
+def test_leading_layout_refuses_row_pieces():
+    w = W.config3(0.002).with_layout("LEADING_CHANNELS").to("cuda")
+    from e3j_amd.ops import _Table
+    table = _Table.get(w.module._packed_coef("float32"), np.float32)
+    dims = (int(w.x.shape[2]), int(w.y.shape[1]), w.module.params.num_out, int(w.s.shape[2]))
+    sig, scale, _ = table.signature(dims, w.channels, w.module.layout)
+    assert sig >= 0
+    p = _lib.ConvParams(
+        num_nodes=w.num_nodes, num_edges=w.num_edges, num_coef=table.num_coef, num_x=dims[0], num_y=dims[1],
+        num_out=dims[2], num_scalars=dims[3], channels=w.channels, layout=_lib.LAYOUT_LEADING,
+        val_dtype=_lib.F32, coef_idx_bytes=table.idx_bytes, signature=sig, coef_scale=scale, debug=0,
+        y_flip=0, row_order=None, row_cap=64, row_piece=64)
+    ptr = csr_row_ptr(w.receiver, w.num_nodes)
+    out = torch.empty_like(w.dm)
+    with pytest.raises(_lib.E3jAmdError) as err:
+        _lib.check(_lib.load().e3j_amd_convolution_fwd(
+            ctypes.byref(p), table.device(w.x.device).data_ptr(), w.x.data_ptr(), w.y.data_ptr(), w.s.data_ptr(),
+            w.sender.data_ptr(), ptr.data_ptr(), None, out.data_ptr(),
+            int(torch.cuda.current_stream().cuda_stream)))
+    assert err.value.code == _lib.UNIMPLEMENTED
+
+
+def _time(fn, reps=7):
+    fn()
+    torch.cuda.synchronize()
+    times = []
+    for _ in range(reps):
+        a, b = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        a.record()
+        fn()
+        b.record()
+        torch.cuda.synchronize()
+        times.append(a.elapsed_time(b))
+    return float(np.median(times))
+
+
+def test_star_graph_runs_within_twice_the_uniform_graph():
+    """One receiver with 50 000 edges against 50 000 edges spread evenly over the same nodes:
+    forward and backward through the operator (graph preparation included on both sides)."""
+    n, e = 600, 50000
+    times = {}
+    for kind in ("uniform", "star"):
+        d = _workload(kind, n, e, 5).to("cuda")
+        coef = d.module._packed_coef("float32")
+        x, y, s = (t.clone().requires_grad_(True) for t in (d.x, d.y, d.s))
+
+        def forward():
+            return convolution(coef, x, y, s, d.sender, d.receiver, d.module.params)
+
+        def both():
+            torch.autograd.grad(forward(), (x, y, s), d.dm)
+
+        times[kind] = (_time(forward), _time(both))
+    print("forward, forward+backward ms:", times)
+    assert times["star"][0] <= 2.0 * times["uniform"][0], times
+    assert times["star"][1] <= 2.0 * times["uniform"][1], times
