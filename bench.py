@@ -253,7 +253,8 @@ class AbiCalls:
 
 
 #: access patterns of `--access-floor`: name -> mask of e3j_amd/csrc/probe/access_pattern.hip
-#: (1 read s, 2 gather x, 4 write ds, 8 dx atomics, 16 write out, 32 read dm)
+#: (1 read s, 2 gather x, 4 write ds, 8 dx atomics, 16 write out, 32 read dm, 64 the atomics of
+#: every second position only)
 ACCESS_PATTERNS = {
     "read_s": 1,
     "read_s+gather_x": 3,
@@ -265,6 +266,8 @@ ACCESS_PATTERNS = {
     "dx_atomics": 8,
     "read_s+write_ds+gather_x+dx_atomics": 15,
     "backward: read_s+write_ds+gather_x+dx_atomics+read_dm": 47,
+    "half_of_the_dx_atomics": 72,
+    "backward with half of the dx atomics": 111,
 }
 
 
@@ -549,8 +552,11 @@ def _lib_name(signature: int) -> str:
     return _lib.load().e3j_amd_tp_signature_name(signature).decode()
 
 
-def traffic_key(args) -> str:
-    return f"{args.config}/{args.scale}/{args.layout}/k{args.channels or 'default'}"
+def traffic_key(args, tiled=None) -> str:
+    """Key of a measurement: workload, layout and which backward kernel ran."""
+    if tiled is None:  # what the library does by default for the trailing layout
+        tiled = args.layout == "trailing" and args.tile_rows != 0 and not args.deterministic
+    return f"{args.config}/{args.scale}/{args.layout}/k{args.channels or 'default'}" + ("/tiled" if tiled else "")
 
 
 def main():
@@ -562,7 +568,8 @@ def main():
     if args.write_traffic:
         key = traffic_key(args)
         names = ({"forward": "unrolled_fwd_leading", "backward": "unrolled_bwd_leading"} if args.layout == "leading"
-                 else {"forward": "unrolled_fwd_kernel", "backward": "unrolled_bwd_kernel"})
+                 else {"forward": "unrolled_fwd_kernel",
+                       "backward": "unrolled_bwd_tile_kernel" if key.endswith("/tiled") else "unrolled_bwd_kernel"})
         return write_traffic(args.write_traffic, TRAFFIC_FILE, key, names)
     import torch
     if not torch.cuda.is_available():
@@ -640,7 +647,7 @@ def main():
         return nbytes / (ms * 1e-3) / 1e9
 
     tiled = abi.schedule is not None and not args.deterministic
-    measured = ({} if args.spatial_sort or args.deterministic or tiled else measured_traffic(traffic_key(args)))
+    measured = ({} if args.spatial_sort or args.deterministic else measured_traffic(traffic_key(args, tiled)))
     bwd_gbs, fwd_gbs = gbs(bytes_["bwd"], bwd_ms), gbs(bytes_["fwd"], fwd_ms)
     both_gbs = gbs(bytes_["fwd_bwd"], fwd_ms + bwd_ms)
     result = {

@@ -16,6 +16,8 @@ constexpr unsigned kWriteDs = 4u;   // stream out S rows of ds per edge (non-tem
 constexpr unsigned kAtomicDx = 8u;  // X float-atomic row pieces into dx[sender]
 constexpr unsigned kWriteOut = 16u; // Z output rows per receiver (non-temporal stores)
 constexpr unsigned kReadDm = 32u;   // Z rows of dm per receiver (non-temporal loads)
+constexpr unsigned kHalfDx = 64u;   // with kAtomicDx: the atomics of every second position only (the
+                                    // request count of a backward that sums half of its dx on chip)
 
 template <unsigned M, int NS, int NX, int NZ, int K>
 __global__ __launch_bounds__(256) void access_pattern_kernel(
@@ -78,7 +80,7 @@ __global__ __launch_bounds__(256) void access_pattern_kernel(
 #pragma unroll
             for (int l = 0; l < NS; l++) acc += sc[l];
         }
-        if (M & kAtomicDx) {
+        if ((M & kAtomicDx) && (!(M & kHalfDx) || !(pos & 1))) {
             float *dxr = dx + (int64_t)snd * (NX * K) + c0;
 #pragma unroll
             for (int j = 0; j < NX; j++) unsafeAtomicAdd(dxr + j * K, xc[j] + sc[j % NS]);
@@ -121,6 +123,8 @@ int run_mask(unsigned mask, const float *x, const float *s, const float *dm, con
         E3J_PROBE_CASE(kReadS | kWriteDs | kGatherX | kAtomicDx | kReadDm)
         E3J_PROBE_CASE(kReadS | kWriteDs | kGatherX | kReadDm)
         E3J_PROBE_CASE(kAtomicDx)
+        E3J_PROBE_CASE(kAtomicDx | kHalfDx)
+        E3J_PROBE_CASE(kReadS | kWriteDs | kGatherX | kAtomicDx | kReadDm | kHalfDx)
         E3J_PROBE_CASE(kWriteDs)
         default: return -1;
     }
@@ -143,7 +147,7 @@ int run_channels(int channels, unsigned mask, const float *x, const float *s, co
 }  // namespace
 
 // Runs the access pattern `mask` (bits: 1 read s, 2 gather x, 4 write ds, 8 dx atomics, 16 write
-// out, 32 read dm) once on `stream` for operands of the trailing-channels layout: s, ds
+// out, 32 read dm, 64 only every second position's atomics) once on `stream` for operands of the trailing-channels layout: s, ds
 // (E, num_scalars, channels); x, dx (N, num_x, channels); dm, out (N, num_out, channels); row_ptr
 // (N + 1); row_order (N) or null for rows in index order.  The sizes are those of the operands at
 // hand: instantiations exist for the (paths, x, output) dimensions of the tables the library
