@@ -136,6 +136,10 @@ def parse_args():
                     help="trailing layout, built-in tables at 64/128/256 channels: also time kernels that perform the "
                          "memory accesses of the two passes without their arithmetic (reported under "
                          "roofline.access_floor)")
+    ap.add_argument("--tile-sharing", action="store_true",
+                    help="also count, on the host, the dx atomic requests a backward over tiles of T receivers "
+                         "issues (distinct (tile, sender) pairs) for T = 2..32, with the library's row order and "
+                         "with rows along a space-filling curve of the atoms (reported under roofline.tile_sharing)")
     ap.add_argument("--inner", type=int, default=64, help="--op radial_linear: hidden size of the radial network")
     ap.add_argument("--op", default="convolution", choices=["convolution", "tensor_product", "radial_linear"],
                     help="convolution: the headline benchmark; tensor_product: a secondary figure, the "
@@ -269,6 +273,29 @@ ACCESS_PATTERNS = {
     "half_of_the_dx_atomics": 72,
     "backward with half of the dx atomics": 111,
 }
+
+
+def tile_sharing(abi, w) -> dict:
+    """Share of the per-edge dx atomic requests left when the contributions of one sender are summed
+    within a tile of T receivers that are consecutive in the row order: distinct (tile, sender)
+    pairs over live edges.  Host arithmetic on the benchmark's graph; two row orders."""
+    import numpy as np
+    from e3j_amd.workloads import morton_order
+    n = w.num_nodes
+    ptr = abi.ptr.cpu().numpy().astype(np.int64)
+    snd = abi.other.cpu().numpy().astype(np.int64)[:ptr[n]]
+    rcv = np.repeat(np.arange(n), np.diff(ptr))
+    live = (snd >= 0) & (snd < n)
+    snd, rcv = snd[live], rcv[live]
+    orders = {"locality_order": (abi.order.cpu().numpy() if abi.order is not None else np.arange(n)),
+              "space_filling_curve": morton_order(np.asarray(w.positions), float(w.box))}
+    out = {}
+    for name, order in orders.items():
+        rank = np.empty(n, np.int64)
+        rank[order] = np.arange(n)
+        out[name] = {str(t): round(len(np.unique((rank[rcv] // t) * n + snd)) / max(len(snd), 1), 4)
+                     for t in (1, 2, 4, 8, 16, 32)}
+    return out
 
 
 def access_floor(torch, abi, steps: int) -> dict:
@@ -707,6 +734,8 @@ def main():
             "forward_plus_backward": {"ms": lf + lb, "frac": gbs(bytes_["fwd_bwd"], lf + lb) / HBM_PEAK_GBS}}}
         del lead, wl
         abi = AbiCalls(w)
+    if args.tile_sharing:
+        result["roofline"]["tile_sharing"] = tile_sharing(abi, w)
     if args.access_floor:
         if args.layout != "trailing" or abi.perm is not None:
             print("--access-floor covers the receiver-sorted trailing layout only", file=sys.stderr)

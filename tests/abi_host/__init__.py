@@ -18,3 +18,12 @@ def build() -> str:
            "-Wl,-rpath,$ORIGIN", f"-Wl,-rpath,{ROCM}/lib"]
     subprocess.run(cmd, check=True)
     return BINARY
+
+
+def binary() -> str:
+    """The built program; compiled again when the header or the source is newer than it (a
+    program built against an older layout of the parameter structs would pass garbage)."""
+    sources = (os.path.join(ROOT, "include", "e3j_amd.h"), os.path.join(HERE, "conv_host.c"))
+    if not os.path.exists(BINARY) or any(os.path.getmtime(s) > os.path.getmtime(BINARY) for s in sources):
+        return build()
+    return BINARY

@@ -65,12 +65,13 @@ def test_tensor_product_params_struct_matches_header():
 
 def test_header_is_plain_c_and_ctypes_mirrors_its_layout(tmp_path):
     """The header compiles as strict C99 (what a cgo / JNI / FFI binding would include), and the
-    compiler's sizes and field offsets of both parameter structs are those of the ctypes mirrors."""
+    compiler's sizes and field offsets of the parameter structs are those of the ctypes mirrors."""
     import shutil
     import subprocess
     if shutil.which("gcc") is None:
         pytest.skip("no C compiler")
-    fields = {"e3j_amd_conv_params": _lib.ConvParams, "e3j_amd_tp_params": _lib.TpParams}
+    fields = {"e3j_amd_conv_params": _lib.ConvParams, "e3j_amd_tp_params": _lib.TpParams,
+              "e3j_amd_tile_schedule": _lib.TileSchedule}
     lines = ['#include <stdio.h>', '#include <stddef.h>', f'#include "{os.path.join(ROOT, "include", "e3j_amd.h")}"',
              'int main(void) {']
     for struct, mirror in fields.items():

@@ -18,7 +18,7 @@ pytestmark = pytest.mark.gpu
 
 
 def _run_host(tmp_path, coef, x, y, s, dm, sender, receiver, dims, layout):
-    binary = abi_host.BINARY if os.path.exists(abi_host.BINARY) else abi_host.build()
+    binary = abi_host.binary()
     N, E, K, X, Y, Z, S = dims
     problem, result = tmp_path / "problem.bin", tmp_path / "result.bin"
     with open(problem, "wb") as f:

@@ -1,8 +1,9 @@
 """Receivers with very many edges: the forward pass shares a long row between waves (the row
 cut at `row_cap` positions, the rest as listed pieces added with float atomics), the tiled
 backward cuts a tile's edge list into work pieces.  Checked against the CPU oracle on a star
-(one receiver takes every edge), on a graph that mixes long rows, ordinary rows, empty rows and
-padding edges, and for run time against a graph of the same size with uniform degrees."""
+(one receiver takes every edge; 15 000 edges, what the numpy oracle finishes in half a minute), on
+a graph that mixes long rows, ordinary rows, empty rows and padding edges, and for run time, at
+50 000 edges, against a graph of the same size with uniform degrees."""
 
 import ctypes
 import zlib
@@ -88,7 +89,7 @@ def test_segment_list_matches_a_host_restatement():
     assert got == want
 
 
-@pytest.mark.parametrize("kind,n,e", [("star", 600, 50000), ("mixed", 400, 3000)])
+@pytest.mark.parametrize("kind,n,e", [("star", 300, 15000), ("mixed", 400, 3000)])
 def test_long_rows_match_oracle(kind, n, e):
     w = _workload(kind, n, e, zlib.crc32(kind.encode()))
     assert row_cap_for(n, w.num_edges) < 600
