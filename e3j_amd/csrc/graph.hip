@@ -195,9 +195,11 @@ __global__ void tile_count_kernel(const int32_t *__restrict__ row_order, const i
     pieces[t + 1] = total == 0 ? 1 : (total + max_work_edges - 1) / max_work_edges;
 }
 
+// KeyT: 32-bit keys when (tile, sender) fits them, which halves the key bytes the sort moves
+template <typename KeyT>
 __global__ void tile_keys_kernel(const int32_t *__restrict__ other, const int32_t *__restrict__ row_ptr,
                                  const int32_t *__restrict__ rank, int num_nodes, int64_t num_edges,
-                                 int tile_rows, int sender_bits, uint64_t sentinel, uint64_t *__restrict__ keys,
+                                 int tile_rows, int sender_bits, KeyT sentinel, KeyT *__restrict__ keys,
                                  int32_t *__restrict__ vals, int32_t *__restrict__ local) {
     const int64_t live_end = row_ptr[num_nodes];
     const int64_t stride = (int64_t)gridDim.x * blockDim.x;
@@ -216,27 +218,28 @@ __global__ void tile_keys_kernel(const int32_t *__restrict__ other, const int32_
         }
         const int q = rank[lo];
         const int32_t snd = other[pos];
-        const uint64_t sk = (unsigned)snd < (unsigned)num_nodes ? (uint64_t)snd : (uint64_t)num_nodes;
-        keys[pos] = ((uint64_t)(q / tile_rows) << sender_bits) | sk;
+        const KeyT sk = (unsigned)snd < (unsigned)num_nodes ? (KeyT)snd : (KeyT)num_nodes;
+        keys[pos] = ((KeyT)(q / tile_rows) << sender_bits) | sk;
         local[pos] = q % tile_rows;
     }
 }
 
-__global__ void tile_entries_kernel(const uint64_t *__restrict__ keys, const int32_t *__restrict__ vals,
+template <typename KeyT>
+__global__ void tile_entries_kernel(const KeyT *__restrict__ keys, const int32_t *__restrict__ vals,
                                     const int32_t *__restrict__ local, const int32_t *__restrict__ perm,
-                                    int num_nodes, int64_t num_edges, int sender_bits, uint64_t sentinel,
+                                    int num_nodes, int64_t num_edges, int sender_bits, KeyT sentinel,
                                     int32_t *__restrict__ t_sender, int32_t *__restrict__ t_edge,
                                     int32_t *__restrict__ t_local) {
     const int64_t stride = (int64_t)gridDim.x * blockDim.x;
     for (int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; i < num_edges; i += stride) {
-        const uint64_t key = keys[i];
+        const KeyT key = keys[i];
         const int32_t pos = vals[i];
         if (key == sentinel) {
             t_sender[i] = -1; t_edge[i] = 0; t_local[i] = 0;
             continue;
         }
-        const uint64_t sk = key & ((1ull << sender_bits) - 1);
-        t_sender[i] = sk == (uint64_t)num_nodes ? -1 : (int32_t)sk;
+        const KeyT sk = key & (((KeyT)1 << sender_bits) - 1);
+        t_sender[i] = sk == (KeyT)num_nodes ? -1 : (int32_t)sk;
         t_edge[i] = perm ? perm[pos] : pos;
         t_local[i] = local[pos];
     }
@@ -267,6 +270,28 @@ size_t sort64_temp_bytes(int64_t num_edges) {
     return bytes;
 }
 
+// keys -> sorted positions -> the schedule's three lists
+template <typename KeyT>
+int tile_lists(const int32_t *other, const int32_t *row_ptr, const int32_t *edge_perm, const int32_t *rank,
+               int32_t num_nodes, int64_t num_edges, int32_t tile_rows, int sender_bits, uint64_t sentinel,
+               int end_bit, void *keys_in_, void *keys_out_, int32_t *vals_in, int32_t *vals_out, int32_t *local,
+               void *temp, size_t temp_bytes, int32_t *t_sender, int32_t *t_edge, int32_t *t_local,
+               hipStream_t stream) {
+    KeyT *keys_in = static_cast<KeyT *>(keys_in_), *keys_out = static_cast<KeyT *>(keys_out_);
+    hipLaunchKernelGGL(tile_keys_kernel<KeyT>, dim3(grid_for(num_edges)), dim3(256), 0, stream, other, row_ptr,
+                       rank, num_nodes, num_edges, tile_rows, sender_bits, (KeyT)sentinel, keys_in, vals_in, local);
+    int rc = check_hip(hipGetLastError(), "tile schedule keys");
+    if (rc) return rc;
+    rc = check_hip(hipcub::DeviceRadixSort::SortPairs(temp, temp_bytes, keys_in, keys_out, vals_in, vals_out,
+                                                      (int)num_edges, 0, end_bit, stream),
+                   "tile schedule sort");
+    if (rc) return rc;
+    hipLaunchKernelGGL(tile_entries_kernel<KeyT>, dim3(grid_for(num_edges)), dim3(256), 0, stream, keys_out,
+                       vals_out, local, edge_perm, num_nodes, num_edges, sender_bits, (KeyT)sentinel, t_sender,
+                       t_edge, t_local);
+    return check_hip(hipGetLastError(), "tile schedule entries");
+}
+
 struct TileWorkspace {
     size_t temp, temp_bytes, keys_in, keys_out, vals_in, vals_out, local, rank, counts, pieces, total;
     TileWorkspace(int32_t num_nodes, int64_t num_edges, int32_t tile_rows) {
@@ -274,7 +299,8 @@ struct TileWorkspace {
         const size_t tiles = (n + (size_t)tile_rows - 1) / (size_t)tile_rows;
         size_t at = 0;
         auto take = [&](size_t bytes) { const size_t here = at; at += align_up(bytes); return here; };
-        temp_bytes = std::max(sort64_temp_bytes(num_edges), scan_temp_bytes((int32_t)tiles));
+        temp_bytes = std::max({sort64_temp_bytes(num_edges), sort_temp_bytes(num_edges),
+                               scan_temp_bytes((int32_t)tiles)});
         temp = take(temp_bytes);
         keys_in = take(8 * e); keys_out = take(8 * e);
         vals_in = take(4 * e); vals_out = take(4 * e);
@@ -500,6 +526,8 @@ int e3j_amd_locality_order(const int32_t *other, const int32_t *row_ptr, int32_t
     // refined from the finest level to the coarsest with stable sorts, so the coarsest clusters
     // are contiguous and, inside them, the finer ones.
     int done = 0;
+    int label_bits = 1;  // labels are node ids: the sort passes stop at their highest bit
+    while (label_bits < 32 && ((int64_t)1 << label_bits) < (int64_t)num_nodes) label_bits++;
     for (int level = 1; level <= rounds; level *= 2) {
         for (; done < level; done++) {
             hipLaunchKernelGGL(min_label_kernel, dim3(rows_grid), dim3(256), 0, stream, other, row_ptr,
@@ -512,7 +540,7 @@ int e3j_amd_locality_order(const int32_t *other, const int32_t *row_ptr, int32_t
         if (rc) return rc;
         size_t temp_bytes = sort_bytes;
         rc = check_hip(hipcub::DeviceRadixSort::SortPairs(sort_temp, temp_bytes, keys_in, keys_out, order,
-                                                          order_tmp, (int)num_nodes, 0, 32, stream),
+                                                          order_tmp, (int)num_nodes, 0, label_bits, stream),
                        "locality_order sort");
         if (rc) return rc;
         hipLaunchKernelGGL(copy_i32_kernel, dim3(ngrid), dim3(256), 0, stream, order_tmp, order,
@@ -601,18 +629,13 @@ int e3j_amd_tile_schedule_build(const int32_t *other, const int32_t *row_ptr, co
     const uint64_t sentinel = (uint64_t)num_tiles << sender_bits;
     int end_bit = sender_bits + 1;
     while (end_bit < 64 && (sentinel >> end_bit) != 0) end_bit++;
-    hipLaunchKernelGGL(tile_keys_kernel, dim3(grid_for(num_edges)), dim3(256), 0, stream, other, row_ptr, rank,
-                       num_nodes, num_edges, tile_rows, sender_bits, sentinel, keys_in, vals_in, local);
-    rc = check_hip(hipGetLastError(), "tile schedule keys");
-    if (rc) return rc;
-    temp_bytes = w.temp_bytes;
-    rc = check_hip(hipcub::DeviceRadixSort::SortPairs(ws + w.temp, temp_bytes, keys_in, keys_out, vals_in, vals_out,
-                                                      (int)num_edges, 0, end_bit, stream),
-                   "tile schedule sort");
-    if (rc) return rc;
-    hipLaunchKernelGGL(tile_entries_kernel, dim3(grid_for(num_edges)), dim3(256), 0, stream, keys_out, vals_out,
-                       local, edge_perm, num_nodes, num_edges, sender_bits, sentinel, t_sender, t_edge, t_local);
-    return check_hip(hipGetLastError(), "tile schedule entries");
+    if (end_bit <= 32)
+        return tile_lists<uint32_t>(other, row_ptr, edge_perm, rank, num_nodes, num_edges, tile_rows, sender_bits,
+                                    sentinel, end_bit, keys_in, keys_out, vals_in, vals_out, local, ws + w.temp,
+                                    w.temp_bytes, t_sender, t_edge, t_local, stream);
+    return tile_lists<uint64_t>(other, row_ptr, edge_perm, rank, num_nodes, num_edges, tile_rows, sender_bits,
+                                sentinel, end_bit, keys_in, keys_out, vals_in, vals_out, local, ws + w.temp,
+                                w.temp_bytes, t_sender, t_edge, t_local, stream);
 }
 
 int e3j_amd_sort_edges(const int32_t *key, const int32_t *other, int64_t num_edges,
