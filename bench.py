@@ -200,6 +200,9 @@ class AbiCalls:
             self.ptr = csr_row_ptr(w.receiver, w.num_nodes)
         rounds = config().locality_rounds
         self.order = locality_order(self.other, self.ptr, w.num_nodes, rounds) if rounds > 0 else None
+        if self.order is not None and config().pair_rows:   # as the operators do
+            from e3j_amd.graph import pair_rows
+            self.order = pair_rows(self.other, self.ptr, w.num_nodes, self.order)
         self.params.row_order = self.order.data_ptr() if self.order is not None else None
         self.out = torch.empty_like(w.dm)
         self.dx, self.dy, self.ds = torch.empty_like(w.x), torch.empty_like(w.y), torch.empty_like(w.s)

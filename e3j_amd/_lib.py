@@ -109,6 +109,8 @@ SYMBOLS = {
     "e3j_amd_row_segments_max": (ctypes.c_int64, [ctypes.c_int64, ctypes.c_int32]),
     "e3j_amd_row_segments_build": (ctypes.c_int, [ctypes.c_void_p, ctypes.c_int32, ctypes.c_int32, ctypes.c_int32,
                                                   ctypes.c_int32, ctypes.c_void_p, ctypes.c_void_p]),
+    "e3j_amd_pair_rows_workspace_bytes": (ctypes.c_size_t, [ctypes.c_int32, ctypes.c_int64]),
+    "e3j_amd_pair_rows": (ctypes.c_int, [_P, _P, ctypes.c_int32, ctypes.c_int64, _P, _P, _P, _P]),
     "e3j_amd_tile_rows": (ctypes.c_int32, [ctypes.c_int32]),
     "e3j_amd_tile_rows_default": (ctypes.c_int32, [ctypes.c_int32]),
     "e3j_amd_tile_schedule_num_work": (ctypes.c_int64, [ctypes.c_int32, ctypes.c_int64, ctypes.c_int32, ctypes.c_int32]),

@@ -335,6 +335,141 @@ __global__ void compose_perm_kernel(const int32_t *__restrict__ outer, const int
         out[i] = inner ? inner[outer[i]] : outer[i];
 }
 
+// Pieces of the rows longer than `cap`, past their first `cap` positions: a row reserves its
+// pieces with one atomic on the count (the order of the list is free).
+__global__ void row_segments_kernel(const int32_t *__restrict__ row_ptr, int num_nodes, int cap, int piece,
+                                    int max_segments, int32_t *__restrict__ segments) {
+    const int r = blockIdx.x * blockDim.x + threadIdx.x;
+    if (r >= num_nodes) return;
+    const int begin = row_ptr[r], end = row_ptr[r + 1];
+    if (end - begin <= cap) return;
+    const int extra = (end - begin - 1) / piece;  // pieces after the first
+    const int at = atomicAdd(segments, extra);
+    for (int k = 0; k < extra && at + k < max_segments; k++) {
+        const int b = begin + (k + 1) * piece;
+        int32_t *seg = segments + 4 + 3 * (at + k);
+        seg[0] = r;
+        seg[1] = b;
+        seg[2] = b + piece < end ? b + piece : end;
+    }
+}
+
+// ---- pairing of rows for the backward over tiles of two receivers ------------------------------
+// Two rows that share most of their senders should sit in one tile: the tile then issues one set
+// of dx atomics for every shared sender.  Every row picks, among the rows it has an edge from,
+// the one with which it has the most senders in common; rows that pick each other are paired, the
+// rest pick again among the rows still free (a few rounds of this greedy matching pair most rows
+// of a radius graph).  Pairs are then listed first, in the order their earlier member had, each
+// pair on an even and the following odd position; the unpaired rows follow in their old order.
+constexpr int kPairMaxDegree = 128;  // rows with more edges (or none) stay unpaired
+constexpr int kPairSlots = 256;      // hash slots per wave for the senders of its row
+constexpr int kPairRounds = 4;
+
+__device__ __forceinline__ unsigned pair_hash(int v) { return ((unsigned)v * 2654435761u) >> 24; }
+
+// common[pos] = number of senders that the row of position pos and the row other[pos] share
+// (-1: no candidate).  One wave per row; its senders go into a hash set in LDS, then every lane
+// walks the row of one neighbour and counts hits.
+__global__ __launch_bounds__(256) void pair_common_kernel(const int32_t *__restrict__ other,
+                                                          const int32_t *__restrict__ row_ptr, int num_nodes,
+                                                          int32_t *__restrict__ common) {
+    __shared__ int32_t slots_all[4][kPairSlots];
+    const int wave = threadIdx.x / 64, lane = threadIdx.x % 64;
+    const int i = blockIdx.x * 4 + wave;
+    if (i >= num_nodes) return;
+    int32_t *slots = slots_all[wave];
+    const int begin = row_ptr[i], deg = row_ptr[i + 1] - begin;
+    if (deg < 1) return;
+    if (deg > kPairMaxDegree) {
+        for (int q = lane; q < deg; q += 64) common[begin + q] = -1;
+        return;
+    }
+    for (int t = lane; t < kPairSlots; t += 64) slots[t] = -1;
+    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+    __builtin_amdgcn_wave_barrier();
+    for (int q = lane; q < deg; q += 64) {
+        const int v = other[begin + q];
+        if ((unsigned)v >= (unsigned)num_nodes) continue;
+        unsigned h = pair_hash(v);
+        for (int probe = 0; probe < kPairSlots; probe++) {
+            const int old = atomicCAS(&slots[h], -1, v);
+            if (old == -1 || old == v) break;
+            h = (h + 1) % kPairSlots;
+        }
+    }
+    __builtin_amdgcn_fence(__ATOMIC_ACQ_REL, "wavefront");
+    __builtin_amdgcn_wave_barrier();
+    for (int q = lane; q < deg; q += 64) {
+        const int p = other[begin + q];
+        int count = -1;
+        if ((unsigned)p < (unsigned)num_nodes && p != i) {
+            const int pb = row_ptr[p], pd = row_ptr[p + 1] - pb;
+            if (pd >= 1 && pd <= kPairMaxDegree) {
+                count = 0;
+                for (int t = 0; t < pd; t++) {
+                    const int v = other[pb + t];
+                    if ((unsigned)v >= (unsigned)num_nodes) continue;
+                    unsigned h = pair_hash(v);
+                    for (int probe = 0; probe < kPairSlots; probe++) {
+                        const int held = slots[h];
+                        if (held == v) { count++; break; }
+                        if (held == -1) break;
+                        h = (h + 1) % kPairSlots;
+                    }
+                }
+            }
+        }
+        common[begin + q] = count;
+    }
+}
+
+// best[i] = the free row with the most senders in common with free row i (smaller id on ties), -1 if none
+__global__ void pair_best_kernel(const int32_t *__restrict__ other, const int32_t *__restrict__ row_ptr,
+                                 const int32_t *__restrict__ common, const int32_t *__restrict__ partner,
+                                 int num_nodes, int32_t *__restrict__ best) {
+    const int i = blockIdx.x * blockDim.x + threadIdx.x;
+    if (i >= num_nodes) return;
+    int pick = -1, most = -1;
+    const int begin = row_ptr[i], deg = row_ptr[i + 1] - begin;
+    if (partner[i] < 0 && deg >= 1 && deg <= kPairMaxDegree) {
+        for (int q = 0; q < deg; q++) {
+            const int c = common[begin + q];
+            if (c < 0) continue;
+            const int p = other[begin + q];
+            if (partner[p] >= 0) continue;
+            if (c > most || (c == most && p < pick)) { most = c; pick = p; }
+        }
+    }
+    best[i] = pick;
+}
+
+__global__ void pair_match_kernel(const int32_t *__restrict__ best, int num_nodes, int32_t *__restrict__ partner) {
+    const int i = blockIdx.x * blockDim.x + threadIdx.x;
+    if (i >= num_nodes) return;
+    const int p = best[i];
+    if (p >= 0 && best[p] == i) partner[i] = p;  // (the thread of row p writes partner[p] = i)
+}
+
+__global__ void pair_keys_kernel(const int32_t *__restrict__ partner, const int32_t *__restrict__ rank,
+                                 int num_nodes, uint32_t *__restrict__ keys, int32_t *__restrict__ vals) {
+    const int i = blockIdx.x * blockDim.x + threadIdx.x;
+    if (i >= num_nodes) return;
+    const int p = partner[i];
+    const unsigned mine = rank ? rank[i] : i;
+    vals[i] = i;
+    if (p < 0) {
+        keys[i] = 2u * (unsigned)num_nodes + mine;
+    } else {
+        const unsigned theirs = rank ? rank[p] : p;
+        keys[i] = 2u * (mine < theirs ? mine : theirs) + (mine > theirs ? 1u : 0u);
+    }
+}
+
+__global__ void fill_i32_kernel(int32_t *__restrict__ out, int64_t n, int32_t value) {
+    const int64_t stride = (int64_t)gridDim.x * blockDim.x;
+    for (int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; i < n; i += stride) out[i] = value;
+}
+
 }  // namespace
 
 int launch_live_keys(const int32_t *other, const int32_t *row_ptr, int32_t num_nodes,
@@ -441,25 +576,6 @@ int e3j_amd_csr_row_ptr_static(const int32_t *key, int64_t num_edges, int32_t nu
     return row_ptr_impl(key, num_edges, num_nodes, row_ptr, temp, need, static_cast<hipStream_t>(stream_));
 }
 
-// Pieces of the rows longer than `cap`, past their first `cap` positions: a row reserves its
-// pieces with one atomic on the count (the order of the list is free).
-__global__ void row_segments_kernel(const int32_t *__restrict__ row_ptr, int num_nodes, int cap, int piece,
-                                    int max_segments, int32_t *__restrict__ segments) {
-    const int r = blockIdx.x * blockDim.x + threadIdx.x;
-    if (r >= num_nodes) return;
-    const int begin = row_ptr[r], end = row_ptr[r + 1];
-    if (end - begin <= cap) return;
-    const int extra = (end - begin - 1) / piece;  // pieces after the first
-    const int at = atomicAdd(segments, extra);
-    for (int k = 0; k < extra && at + k < max_segments; k++) {
-        const int b = begin + (k + 1) * piece;
-        int32_t *seg = segments + 4 + 3 * (at + k);
-        seg[0] = r;
-        seg[1] = b;
-        seg[2] = b + piece < end ? b + piece : end;
-    }
-}
-
 int64_t e3j_amd_row_segments_max(int64_t num_edges, int32_t row_piece) {
     if (num_edges <= 0 || row_piece <= 0) return 0;
     return num_edges / row_piece;  // a piece after the first follows row_piece positions of its row
@@ -489,6 +605,72 @@ int e3j_amd_wrap_index(const int32_t *index, int64_t n, int32_t num_nodes, int32
     hipLaunchKernelGGL(wrap_index_kernel, dim3(grid_for(n)), dim3(256), 0, (hipStream_t)stream_,
                        index, n, num_nodes, out);
     return check_hip(hipGetLastError(), "wrap_index");
+}
+
+namespace {
+struct PairWorkspace {
+    size_t temp, temp_bytes, common, best, partner, rank, keys_in, keys_out, vals_in, total;
+    PairWorkspace(int32_t num_nodes, int64_t num_edges) {
+        const size_t n = (size_t)num_nodes, e = (size_t)num_edges;
+        size_t at = 0;
+        auto take = [&](size_t bytes) { const size_t here = at; at += align_up(bytes); return here; };
+        temp_bytes = sort_temp_bytes(num_nodes);
+        temp = take(temp_bytes);
+        common = take(4 * e);
+        best = take(4 * n); partner = take(4 * n); rank = take(4 * n);
+        keys_in = take(4 * n); keys_out = take(4 * n); vals_in = take(4 * n);
+        total = at + 256;
+    }
+};
+}  // namespace
+
+size_t e3j_amd_pair_rows_workspace_bytes(int32_t num_nodes, int64_t num_edges) {
+    if (num_nodes < 0 || num_edges < 0) return 0;
+    return PairWorkspace(num_nodes, num_edges).total;
+}
+
+int e3j_amd_pair_rows(const int32_t *other, const int32_t *row_ptr, int32_t num_nodes, int64_t num_edges,
+                      const int32_t *order_in, int32_t *order_out, void *workspace, void *stream_) {
+    if (num_nodes < 0 || num_edges < 0 || num_edges > 0x7fffffffLL || num_nodes > 0x3fffffff)
+        return set_error(E3J_AMD_INVALID_ARGUMENT, "pair_rows: bad sizes");
+    if (num_nodes == 0) return E3J_AMD_OK;
+    if (order_out == nullptr || workspace == nullptr || row_ptr == nullptr || (num_edges > 0 && other == nullptr))
+        return set_error(E3J_AMD_INVALID_ARGUMENT, "pair_rows: null operand");
+    hipStream_t stream = static_cast<hipStream_t>(stream_);
+    unsigned char *ws = static_cast<unsigned char *>(workspace);
+    const PairWorkspace w(num_nodes, num_edges);
+    int32_t *common = reinterpret_cast<int32_t *>(ws + w.common);
+    int32_t *best = reinterpret_cast<int32_t *>(ws + w.best);
+    int32_t *partner = reinterpret_cast<int32_t *>(ws + w.partner);
+    int32_t *rank = reinterpret_cast<int32_t *>(ws + w.rank);
+    uint32_t *keys_in = reinterpret_cast<uint32_t *>(ws + w.keys_in);
+    uint32_t *keys_out = reinterpret_cast<uint32_t *>(ws + w.keys_out);
+    int32_t *vals_in = reinterpret_cast<int32_t *>(ws + w.vals_in);
+    const unsigned rows_grid = (unsigned)((num_nodes + 255) / 256);
+
+    hipLaunchKernelGGL(fill_i32_kernel, dim3(grid_for(num_nodes)), dim3(256), 0, stream, partner,
+                       (int64_t)num_nodes, -1);
+    hipLaunchKernelGGL(pair_common_kernel, dim3((unsigned)((num_nodes + 3) / 4)), dim3(256), 0, stream, other,
+                       row_ptr, num_nodes, common);
+    int rc = check_hip(hipGetLastError(), "pair_rows common");
+    if (rc) return rc;
+    for (int round = 0; round < kPairRounds; round++) {
+        hipLaunchKernelGGL(pair_best_kernel, dim3(rows_grid), dim3(256), 0, stream, other, row_ptr, common, partner,
+                           num_nodes, best);
+        hipLaunchKernelGGL(pair_match_kernel, dim3(rows_grid), dim3(256), 0, stream, best, num_nodes, partner);
+    }
+    if (order_in != nullptr)
+        hipLaunchKernelGGL(tile_rank_kernel, dim3(rows_grid), dim3(256), 0, stream, order_in, num_nodes, rank);
+    hipLaunchKernelGGL(pair_keys_kernel, dim3(rows_grid), dim3(256), 0, stream, partner,
+                       order_in != nullptr ? rank : nullptr, num_nodes, keys_in, vals_in);
+    rc = check_hip(hipGetLastError(), "pair_rows keys");
+    if (rc) return rc;
+    int key_bits = 2;  // keys are below 3 * num_nodes
+    while (key_bits < 32 && ((uint64_t)1 << key_bits) < 3ull * (uint64_t)num_nodes) key_bits++;
+    size_t temp_bytes = w.temp_bytes;
+    return check_hip(hipcub::DeviceRadixSort::SortPairs(ws + w.temp, temp_bytes, keys_in, keys_out, vals_in,
+                                                        order_out, (int)num_nodes, 0, key_bits, stream),
+                     "pair_rows sort");
 }
 
 size_t e3j_amd_order_workspace_bytes(int32_t num_nodes) {

@@ -104,6 +104,25 @@ def locality_order(other: torch.Tensor, row_ptr: torch.Tensor, num_nodes: int,
     return order
 
 
+def pair_rows(other: torch.Tensor, row_ptr: torch.Tensor, num_nodes: int,
+              order: torch.Tensor | None = None) -> torch.Tensor:
+    """`order` (or the index order) rearranged so that rows sharing most of their senders sit side
+    by side on positions 2q, 2q + 1: the tiles of the backward over two receivers per tile
+    (`e3j_amd_pair_rows`).  Results do not depend on it."""
+    device = _require_device(other, row_ptr)
+    other, row_ptr = _as_index(other), _as_index(row_ptr)
+    lib = _lib.load()
+    num_edges = int(other.numel())
+    out = torch.empty(num_nodes, dtype=INDEX_DTYPE, device=device)
+    ws = torch.empty(max(int(lib.e3j_amd_pair_rows_workspace_bytes(num_nodes, num_edges)), 256),
+                     dtype=torch.uint8, device=device)
+    with torch.cuda.device(device):
+        _lib.check(lib.e3j_amd_pair_rows(other.data_ptr(), row_ptr.data_ptr(), num_nodes, num_edges,
+                                         order.data_ptr() if order is not None else None, out.data_ptr(),
+                                         ws.data_ptr(), _stream_ptr(device)))
+    return out
+
+
 #: edge positions per work item of the tiled backward: longer tile lists (hub rows) are cut
 #: into pieces of this many positions, each taken by a workgroup of its own
 MAX_WORK_EDGES = 256

@@ -26,7 +26,7 @@ import torch
 from . import _lib
 from .coef import Coef4D
 from .graph import (RowSegments, TileSchedule, csr_row_ptr, fold_endpoints, locality_order,
-                    row_cap_for, sort_edges, wrap_global_index)
+                    pair_rows, row_cap_for, sort_edges, wrap_global_index)
 from .options import GraphOrdering, Layout, config
 
 
@@ -218,7 +218,10 @@ def _row_order(other: torch.Tensor, row_ptr: torch.Tensor, n: int):
     rounds = config().locality_rounds
     if rounds <= 0 or n < 2 or other.numel() == 0:
         return None
-    return locality_order(other, row_ptr, n, rounds)
+    order = locality_order(other, row_ptr, n, rounds)
+    if config().pair_rows:
+        order = pair_rows(other, row_ptr, n, order)
+    return order
 
 
 #: Opt-in (`config(graph_cache=True)`): adjacencies prepared for the index tensors seen last, keyed by

@@ -109,6 +109,11 @@ class Config:
     #: 64 channels; capped by what the LDS holds).  -1: the size the kernel of the signature is
     #: tuned for; 0: one wave per receiver and one set of atomics per edge (no schedule to build).
     tile_rows: int = -1
+    #: put rows that share most of their senders side by side in the row order, so that the tiles
+    #: of the default backward (two receivers at K = 128) sum more dx contributions on chip: 19 %
+    #: fewer atomic requests and a 2 % faster backward at 1M edges, for 0.28 ms more graph
+    #: preparation; worth it for a graph that serves many calls (`prepare_graph`), off by default
+    pair_rows: bool = False
     #: positions of a row one wave of the forward pass sums; longer rows are shared between waves
     #: (their sums then come from float atomics).  -1: twice the mean row length, at least 64;
     #: 0: never share a row.
@@ -129,6 +134,7 @@ class _ConfigHolder:
             locality_rounds=int(os.environ.get("E3J_AMD_LOCALITY_ROUNDS", "2")),
             tile_rows=int(os.environ.get("E3J_AMD_TILE_ROWS", "-1")),
             row_cap=int(os.environ.get("E3J_AMD_ROW_CAP", "-1")),
+            pair_rows=os.environ.get("E3J_AMD_PAIR_ROWS", "0") not in ("0", ""),
             graph_cache=os.environ.get("E3J_AMD_GRAPH_CACHE", "0") not in ("0", ""),
             jit=os.environ.get("E3J_AMD_JIT", "0") not in ("0", ""),
         )

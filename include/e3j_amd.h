@@ -281,6 +281,19 @@ size_t e3j_amd_order_workspace_bytes(int32_t num_nodes);
 int e3j_amd_locality_order(const int32_t *other, const int32_t *row_ptr, int32_t num_nodes,
                            int32_t rounds, int32_t *order, void *workspace, void *stream);
 
+/* e3j_amd_pair_rows: reorders a processing order for the backward over tiles of two receivers.
+ *   Rows that share most of their senders are put side by side (greedy matching over a few
+ *   rounds: rows that pick each other as the row with the most senders in common are paired),
+ *   pairs first, each on an even and the next odd position, in the order their earlier member
+ *   had in order_in (NULL: index order); unpaired rows (also those without edges or with more
+ *   than 128) follow in their old order.  order_out (N): a permutation; must not alias order_in.
+ *   Results of the convolution do not depend on it; the tiled backward issues one set of dx
+ *   atomics per sender a pair shares.  workspace: >= e3j_amd_pair_rows_workspace_bytes().
+ *   No counterpart in the reference. */
+size_t e3j_amd_pair_rows_workspace_bytes(int32_t num_nodes, int64_t num_edges);
+int e3j_amd_pair_rows(const int32_t *other, const int32_t *row_ptr, int32_t num_nodes, int64_t num_edges,
+                      const int32_t *order_in, int32_t *order_out, void *workspace, void *stream);
+
 /* Edge featurisation next to the convolution: real spherical harmonics of `num` vectors
  * (num, 3) for the degrees 0..l_max (l_max <= 6), out (num, (l_max + 1)^2), and the
  * vector-Jacobian product dvec (num, 3) for a cotangent dout of that shape.  Order, harmonic
