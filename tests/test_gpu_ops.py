@@ -79,6 +79,29 @@ def test_convolution_bwd_direct_and_deterministic_bits():
     _check(p, out, base)
 
 
+@pytest.mark.parametrize("channels", [32, 128])
+def test_fifty_runs_give_the_same_bits(channels):
+    """The reference's determinism checks (`tests/test_ops/test_convolution_op.py:322-342`: 50
+    repeats of the forward and of the gradient, zero tolerance).  The forward is bit-reproducible
+    as it stands; the gradient under `config(deterministic=True)` (the default backward adds dx
+    with float atomics, in an order that varies)."""
+    p = _problem(12, N=200, E=6000, K=channels)
+    x, y, s = (dev(p[k], grad=True) for k in ("x", "y", "s"))
+    snd, rcv, dm = dev(p["snd"]), dev(p["rcv"]), dev(p["dm"])
+    base = convolution(p["coef"], x, y, s, snd, rcv, p["params"])
+    for _ in range(50):
+        assert torch.equal(base, convolution(p["coef"], x, y, s, snd, rcv, p["params"]))
+    with e3j_amd.config.use(deterministic=True):
+        def grads():
+            out = convolution(p["coef"], x, y, s, snd, rcv, p["params"])
+            return torch.autograd.grad(out, (x, y, s), dm)
+        first = grads()
+        for _ in range(50):
+            for a, b in zip(first, grads()):
+                assert torch.equal(a, b)
+    _check(p, base.detach(), first)
+
+
 def test_two_dimensional_x_means_one_channel():
     p = _problem(3, K=1)
     x, y, s = dev(p["x"][:, :, 0], grad=True), dev(p["y"], grad=True), dev(p["s"], grad=True)
