@@ -194,6 +194,20 @@ def test_graph_entry_point_errors():
     assert lib.e3j_amd_csr_row_ptr(None, -1, 4, None, None, None) == _lib.INVALID_ARGUMENT
     assert lib.e3j_amd_sort_edges(None, None, 4, 4, None, None, None, None, None) == _lib.INVALID_ARGUMENT
     assert lib.e3j_amd_csr_workspace_bytes(1000, 100000) > 0
+    # the row order, the tile schedule and the pieces of long rows
+    assert lib.e3j_amd_pair_rows(None, None, 4, 8, None, None, None, None) == _lib.INVALID_ARGUMENT
+    assert "null operand" in lib.e3j_amd_last_error().decode()
+    assert lib.e3j_amd_pair_rows(None, None, -1, 8, None, None, None, None) == _lib.INVALID_ARGUMENT
+    assert lib.e3j_amd_pair_rows(None, None, 0, 0, None, None, None, None) == _lib.OK
+    assert lib.e3j_amd_pair_rows_workspace_bytes(1000, 30000) > 4 * 30000
+    assert lib.e3j_amd_row_segments_max(1000, 64) == 15 and lib.e3j_amd_row_segments_max(1000, 0) == 0
+    assert lib.e3j_amd_row_segments_build(None, 4, 64, 64, 10, None, None) == _lib.INVALID_ARGUMENT
+    assert lib.e3j_amd_row_segments_build(None, 4, 32, 64, 10, None, None) == _lib.INVALID_ARGUMENT   # piece > cap
+    assert lib.e3j_amd_tile_rows(-1) == 0 and lib.e3j_amd_tile_rows_default(10_000) == 0
+    p = _params(row_cap=-1)
+    assert lib.e3j_amd_convolution_fwd(C.byref(p), *([C.c_void_p(64)] * 6), None, C.c_void_p(64), None) \
+        == _lib.INVALID_ARGUMENT
+    assert "row_cap" in lib.e3j_amd_last_error().decode()
 
 
 def test_find_signature_matches_benchmark_tables():
