@@ -168,9 +168,8 @@ __global__ void live_keys_kernel(const int32_t *__restrict__ other, const int32_
 
 
 // ---- schedule of the backward over tiles of receivers ---------------------------------------
-// Tiles are `tile_rows` consecutive entries of the row order.  Every CSR position gets the key
-// (tile, sender) with padding senders after the live ones; a radix sort of the positions by that
-// key lists each tile's edges in sender order.
+// Tiles are `tile_rows` consecutive entries of the row order.  A scan of the tiles' position
+// counts places each tile's list; one wave per tile then writes the list, sorted by sender.
 
 __global__ void tile_rank_kernel(const int32_t *__restrict__ row_order, int num_nodes,
                                  int32_t *__restrict__ rank) {
@@ -195,53 +194,107 @@ __global__ void tile_count_kernel(const int32_t *__restrict__ row_order, const i
     pieces[t + 1] = total == 0 ? 1 : (total + max_work_edges - 1) / max_work_edges;
 }
 
-// KeyT: 32-bit keys when (tile, sender) fits them, which halves the key bytes the sort moves
-template <typename KeyT>
-__global__ void tile_keys_kernel(const int32_t *__restrict__ other, const int32_t *__restrict__ row_ptr,
-                                 const int32_t *__restrict__ rank, int num_nodes, int64_t num_edges,
-                                 int tile_rows, int sender_bits, KeyT sentinel, KeyT *__restrict__ keys,
-                                 int32_t *__restrict__ vals, int32_t *__restrict__ local) {
-    const int64_t live_end = row_ptr[num_nodes];
-    const int64_t stride = (int64_t)gridDim.x * blockDim.x;
-    for (int64_t pos = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; pos < num_edges; pos += stride) {
-        vals[pos] = (int32_t)pos;
-        if (pos >= live_end) {  // past the last row: belongs to no tile
-            keys[pos] = sentinel;
-            local[pos] = 0;
-            continue;
+// The three lists of one tile, by one wave: the tile's positions (its rows in tile order, each
+// row's positions ascending) are keyed by (sender, position), padding senders after the live
+// ones, and sorted in LDS with a bitonic network when the tile has at most kTileSortLimit of
+// them.  Longer tiles (hub rows) are not sorted by sender, only split into live positions first
+// and padding positions last, which is all the kernel needs for correctness (it sums runs of
+// equal senders wherever they occur); a hub's senders are mostly distinct anyway.
+constexpr int kTileSortLimit = 512;
+__global__ __launch_bounds__(256) void tile_lists_kernel(
+    const int32_t *__restrict__ other, const int32_t *__restrict__ row_ptr, const int32_t *__restrict__ perm,
+    const int32_t *__restrict__ row_order, const int32_t *__restrict__ starts, int num_nodes, int tile_rows,
+    int num_tiles, int32_t *__restrict__ t_sender, int32_t *__restrict__ t_edge, int32_t *__restrict__ t_local) {
+    __shared__ uint64_t keys_all[4][kTileSortLimit];
+    __shared__ uint16_t local_all[4][kTileSortLimit];
+    const int wave = threadIdx.x / 64, lane = threadIdx.x % 64;
+    const int t = blockIdx.x * 4 + wave;
+    if (t >= num_tiles) return;
+    uint64_t *keys = keys_all[wave];
+    uint16_t *locals = local_all[wave];
+    const int begin = starts[t], m = starts[t + 1] - begin;
+    if (m == 0) return;
+    const int first = t * tile_rows;
+    const int rows = num_nodes - first < tile_rows ? num_nodes - first : tile_rows;
+    if (m <= kTileSortLimit) {
+        int filled = 0;
+        for (int i = 0; i < rows; i++) {
+            const int r = row_order ? row_order[first + i] : first + i;
+            const int b = row_ptr[r], d = row_ptr[r + 1] - b;
+            for (int q = lane; q < d; q += 64) {
+                const int snd = other[b + q];
+                const uint64_t sk = (unsigned)snd < (unsigned)num_nodes ? (uint64_t)snd : (uint64_t)num_nodes;
+                // (sender, position) orders the list; the row the position came from travels beside it
+                keys[filled + q] = (sk << 32) | (uint64_t)(uint32_t)(b + q);
+                locals[filled + q] = (uint16_t)i;
+            }
+            filled += d;
         }
-        // the row of the position: last r with row_ptr[r] <= pos (empty rows share their start)
-        int lo = 0, hi = num_nodes;  // invariant: row_ptr[lo] <= pos < row_ptr[hi]
-        while (hi - lo > 1) {
-            const int mid = (lo + hi) >> 1;
-            if (row_ptr[mid] <= pos) lo = mid; else hi = mid;
+        int padded = 64;
+        while (padded < m) padded *= 2;
+        for (int q = m + lane; q < padded; q += 64) { keys[q] = ~0ull; locals[q] = 0; }
+        __builtin_amdgcn_fence(__ATOMIC_ACQ_REL, "wavefront");
+        __builtin_amdgcn_wave_barrier();
+        for (int k = 2; k <= padded; k *= 2) {
+            for (int j = k / 2; j > 0; j /= 2) {
+                for (int q = lane; q < padded; q += 64) {
+                    const int partner = q ^ j;
+                    if (partner > q) {
+                        const uint64_t a = keys[q], c = keys[partner];
+                        const bool ascending = (q & k) == 0;
+                        if ((a > c) == ascending) {
+                            keys[q] = c; keys[partner] = a;
+                            const uint16_t la = locals[q];
+                            locals[q] = locals[partner]; locals[partner] = la;
+                        }
+                    }
+                }
+                __builtin_amdgcn_fence(__ATOMIC_ACQ_REL, "wavefront");
+                __builtin_amdgcn_wave_barrier();
+            }
         }
-        const int q = rank[lo];
-        const int32_t snd = other[pos];
-        const KeyT sk = (unsigned)snd < (unsigned)num_nodes ? (KeyT)snd : (KeyT)num_nodes;
-        keys[pos] = ((KeyT)(q / tile_rows) << sender_bits) | sk;
-        local[pos] = q % tile_rows;
+        for (int q = lane; q < m; q += 64) {
+            const uint64_t key = keys[q];
+            const int pos = (int)(uint32_t)key;
+            const uint64_t sk = key >> 32;
+            t_sender[begin + q] = sk == (uint64_t)num_nodes ? -1 : (int32_t)sk;
+            t_edge[begin + q] = perm ? perm[pos] : pos;
+            t_local[begin + q] = locals[q];
+        }
+        return;
+    }
+    // a long tile: live positions in tile order, then the padding positions
+    int at = begin;
+    for (int pass = 0; pass < 2; pass++) {
+        for (int i = 0; i < rows; i++) {
+            const int r = row_order ? row_order[first + i] : first + i;
+            const int b = row_ptr[r], d = row_ptr[r + 1] - b;
+            for (int q0 = 0; q0 < d; q0 += 64) {
+                const int q = q0 + lane;
+                const int snd = q < d ? other[b + q] : -1;
+                const bool live = (unsigned)snd < (unsigned)num_nodes;
+                const bool mine = q < d && (live == (pass == 0));
+                const unsigned long long mask = __ballot(mine);
+                if (mine) {
+                    const int slot = at + __popcll(mask & ((1ull << lane) - 1ull));
+                    t_sender[slot] = live ? snd : -1;
+                    t_edge[slot] = perm ? perm[b + q] : b + q;
+                    t_local[slot] = i;
+                }
+                at += __popcll(mask);
+            }
+        }
     }
 }
 
-template <typename KeyT>
-__global__ void tile_entries_kernel(const KeyT *__restrict__ keys, const int32_t *__restrict__ vals,
-                                    const int32_t *__restrict__ local, const int32_t *__restrict__ perm,
-                                    int num_nodes, int64_t num_edges, int sender_bits, KeyT sentinel,
-                                    int32_t *__restrict__ t_sender, int32_t *__restrict__ t_edge,
-                                    int32_t *__restrict__ t_local) {
+// entries of the lists past the last row (padding positions that belong to no tile)
+__global__ void tile_tail_kernel(const int32_t *__restrict__ row_ptr, int num_nodes, int64_t num_edges,
+                                 int32_t *__restrict__ t_sender, int32_t *__restrict__ t_edge,
+                                 int32_t *__restrict__ t_local) {
+    const int64_t live_end = row_ptr[num_nodes];
     const int64_t stride = (int64_t)gridDim.x * blockDim.x;
-    for (int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; i < num_edges; i += stride) {
-        const KeyT key = keys[i];
-        const int32_t pos = vals[i];
-        if (key == sentinel) {
-            t_sender[i] = -1; t_edge[i] = 0; t_local[i] = 0;
-            continue;
-        }
-        const KeyT sk = key & (((KeyT)1 << sender_bits) - 1);
-        t_sender[i] = sk == (KeyT)num_nodes ? -1 : (int32_t)sk;
-        t_edge[i] = perm ? perm[pos] : pos;
-        t_local[i] = local[pos];
+    for (int64_t i = live_end + (int64_t)blockIdx.x * blockDim.x + threadIdx.x; i < num_edges; i += stride) {
+        t_sender[i] = -1; t_edge[i] = 0; t_local[i] = 0;
     }
 }
 
@@ -263,49 +316,15 @@ __global__ void tile_work_kernel(const int32_t *__restrict__ starts, const int32
     if (t == 0) work[3] = first_piece[num_tiles];
 }
 
-size_t sort64_temp_bytes(int64_t num_edges) {
-    size_t bytes = 0;
-    hipcub::DeviceRadixSort::SortPairs(nullptr, bytes, (const uint64_t *)nullptr, (uint64_t *)nullptr,
-                                       (const int32_t *)nullptr, (int32_t *)nullptr, (int)num_edges);
-    return bytes;
-}
-
-// keys -> sorted positions -> the schedule's three lists
-template <typename KeyT>
-int tile_lists(const int32_t *other, const int32_t *row_ptr, const int32_t *edge_perm, const int32_t *rank,
-               int32_t num_nodes, int64_t num_edges, int32_t tile_rows, int sender_bits, uint64_t sentinel,
-               int end_bit, void *keys_in_, void *keys_out_, int32_t *vals_in, int32_t *vals_out, int32_t *local,
-               void *temp, size_t temp_bytes, int32_t *t_sender, int32_t *t_edge, int32_t *t_local,
-               hipStream_t stream) {
-    KeyT *keys_in = static_cast<KeyT *>(keys_in_), *keys_out = static_cast<KeyT *>(keys_out_);
-    hipLaunchKernelGGL(tile_keys_kernel<KeyT>, dim3(grid_for(num_edges)), dim3(256), 0, stream, other, row_ptr,
-                       rank, num_nodes, num_edges, tile_rows, sender_bits, (KeyT)sentinel, keys_in, vals_in, local);
-    int rc = check_hip(hipGetLastError(), "tile schedule keys");
-    if (rc) return rc;
-    rc = check_hip(hipcub::DeviceRadixSort::SortPairs(temp, temp_bytes, keys_in, keys_out, vals_in, vals_out,
-                                                      (int)num_edges, 0, end_bit, stream),
-                   "tile schedule sort");
-    if (rc) return rc;
-    hipLaunchKernelGGL(tile_entries_kernel<KeyT>, dim3(grid_for(num_edges)), dim3(256), 0, stream, keys_out,
-                       vals_out, local, edge_perm, num_nodes, num_edges, sender_bits, (KeyT)sentinel, t_sender,
-                       t_edge, t_local);
-    return check_hip(hipGetLastError(), "tile schedule entries");
-}
-
 struct TileWorkspace {
-    size_t temp, temp_bytes, keys_in, keys_out, vals_in, vals_out, local, rank, counts, pieces, total;
-    TileWorkspace(int32_t num_nodes, int64_t num_edges, int32_t tile_rows) {
-        const size_t e = (size_t)num_edges, n = (size_t)num_nodes;
+    size_t temp, temp_bytes, counts, pieces, total;
+    TileWorkspace(int32_t num_nodes, int32_t tile_rows) {
+        const size_t n = (size_t)num_nodes;
         const size_t tiles = (n + (size_t)tile_rows - 1) / (size_t)tile_rows;
         size_t at = 0;
         auto take = [&](size_t bytes) { const size_t here = at; at += align_up(bytes); return here; };
-        temp_bytes = std::max({sort64_temp_bytes(num_edges), sort_temp_bytes(num_edges),
-                               scan_temp_bytes((int32_t)tiles)});
+        temp_bytes = scan_temp_bytes((int32_t)tiles + 1);
         temp = take(temp_bytes);
-        keys_in = take(8 * e); keys_out = take(8 * e);
-        vals_in = take(4 * e); vals_out = take(4 * e);
-        local = take(4 * e);
-        rank = take(4 * n);
         counts = take(4 * (tiles + 1)); pieces = take(4 * (tiles + 1));
         total = at;
     }
@@ -754,7 +773,8 @@ int64_t e3j_amd_tile_schedule_num_work(int32_t num_nodes, int64_t num_edges, int
 
 size_t e3j_amd_tile_schedule_workspace_bytes(int32_t num_nodes, int64_t num_edges, int32_t tile_rows) {
     if (num_nodes < 0 || num_edges < 0 || tile_rows < 1) return 0;
-    return TileWorkspace(num_nodes, num_edges, tile_rows).total + 256;
+    (void)num_edges;
+    return TileWorkspace(num_nodes, tile_rows).total + 256;
 }
 
 int e3j_amd_tile_schedule_build(const int32_t *other, const int32_t *row_ptr, const int32_t *edge_perm,
@@ -762,7 +782,8 @@ int e3j_amd_tile_schedule_build(const int32_t *other, const int32_t *row_ptr, co
                                 int32_t tile_rows, int32_t max_work_edges, int32_t *work,
                                 int32_t *t_sender, int32_t *t_edge, int32_t *t_local, void *workspace,
                                 void *stream_) {
-    if (num_nodes < 0 || num_edges < 0 || num_edges > 0x7fffffffLL || tile_rows < 1 || max_work_edges < 1)
+    if (num_nodes < 0 || num_edges < 0 || num_edges > 0x7fffffffLL || tile_rows < 1 || tile_rows > 65535 ||
+        max_work_edges < 1)
         return set_error(E3J_AMD_INVALID_ARGUMENT, "tile_schedule_build: bad sizes");
     if (num_nodes == 0) return E3J_AMD_OK;
     if (row_ptr == nullptr || work == nullptr || workspace == nullptr ||
@@ -771,23 +792,15 @@ int e3j_amd_tile_schedule_build(const int32_t *other, const int32_t *row_ptr, co
     hipStream_t stream = static_cast<hipStream_t>(stream_);
     unsigned char *ws = static_cast<unsigned char *>(workspace);
     ws += (256 - reinterpret_cast<uintptr_t>(ws) % 256) % 256;
-    const TileWorkspace w(num_nodes, num_edges, tile_rows);
-    uint64_t *keys_in = reinterpret_cast<uint64_t *>(ws + w.keys_in);
-    uint64_t *keys_out = reinterpret_cast<uint64_t *>(ws + w.keys_out);
-    int32_t *vals_in = reinterpret_cast<int32_t *>(ws + w.vals_in);
-    int32_t *vals_out = reinterpret_cast<int32_t *>(ws + w.vals_out);
-    int32_t *local = reinterpret_cast<int32_t *>(ws + w.local);
-    int32_t *rank = reinterpret_cast<int32_t *>(ws + w.rank);
+    const TileWorkspace w(num_nodes, tile_rows);
     int32_t *counts = reinterpret_cast<int32_t *>(ws + w.counts);
     int32_t *pieces = reinterpret_cast<int32_t *>(ws + w.pieces);
     const int num_tiles = (num_nodes + tile_rows - 1) / tile_rows;
     const int64_t num_work = e3j_amd_tile_schedule_num_work(num_nodes, num_edges, tile_rows, max_work_edges);
-    const unsigned rows_grid = (unsigned)((num_nodes + 255) / 256);
     const unsigned tiles_grid = (unsigned)((num_tiles + 255) / 256);
 
     int rc = launch_fill_zero(work, sizeof(int32_t) * 4 * (size_t)num_work, stream);
     if (rc) return rc;
-    hipLaunchKernelGGL(tile_rank_kernel, dim3(rows_grid), dim3(256), 0, stream, row_order, num_nodes, rank);
     hipLaunchKernelGGL(tile_count_kernel, dim3(tiles_grid), dim3(256), 0, stream, row_order, row_ptr, num_nodes,
                        tile_rows, num_tiles, max_work_edges, counts, pieces);
     rc = check_hip(hipGetLastError(), "tile schedule counts");
@@ -804,20 +817,12 @@ int e3j_amd_tile_schedule_build(const int32_t *other, const int32_t *row_ptr, co
                        max_work_edges, work);
     rc = check_hip(hipGetLastError(), "tile schedule work");
     if (rc || num_edges == 0) return rc;
-
-    // key = tile << sender_bits | sender, padding senders as num_nodes; sentinel above every live key
-    int sender_bits = 1;
-    while (((uint64_t)num_nodes >> sender_bits) != 0) sender_bits++;
-    const uint64_t sentinel = (uint64_t)num_tiles << sender_bits;
-    int end_bit = sender_bits + 1;
-    while (end_bit < 64 && (sentinel >> end_bit) != 0) end_bit++;
-    if (end_bit <= 32)
-        return tile_lists<uint32_t>(other, row_ptr, edge_perm, rank, num_nodes, num_edges, tile_rows, sender_bits,
-                                    sentinel, end_bit, keys_in, keys_out, vals_in, vals_out, local, ws + w.temp,
-                                    w.temp_bytes, t_sender, t_edge, t_local, stream);
-    return tile_lists<uint64_t>(other, row_ptr, edge_perm, rank, num_nodes, num_edges, tile_rows, sender_bits,
-                                sentinel, end_bit, keys_in, keys_out, vals_in, vals_out, local, ws + w.temp,
-                                w.temp_bytes, t_sender, t_edge, t_local, stream);
+    // the lists: one wave per tile sorts its positions by sender in LDS
+    hipLaunchKernelGGL(tile_lists_kernel, dim3((unsigned)((num_tiles + 3) / 4)), dim3(256), 0, stream, other, row_ptr,
+                       edge_perm, row_order, counts, num_nodes, tile_rows, num_tiles, t_sender, t_edge, t_local);
+    hipLaunchKernelGGL(tile_tail_kernel, dim3(64), dim3(256), 0, stream, row_ptr, num_nodes, num_edges, t_sender,
+                       t_edge, t_local);
+    return check_hip(hipGetLastError(), "tile schedule lists");
 }
 
 int e3j_amd_sort_edges(const int32_t *key, const int32_t *other, int64_t num_edges,

@@ -158,7 +158,9 @@ int e3j_amd_convolution_bwd_ordered(const e3j_amd_conv_params *p, const void *co
  * backward by receivers with dx added into a zero-filled buffer:
  * src/e3j/pallas_ops/convolution/mosaic_gpu/bwd.py:336-457.
  *
- * Schedule: the edge positions of every tile sorted by sender (padding edges last), as three
+ * Schedule: the edge positions of every tile sorted by sender (padding edges last; a tile of
+ * more than 512 positions lists its live positions in row order, unsorted, then its padding
+ * positions: the kernel only needs equal senders side by side to sum them), as three
  * parallel arrays, and work descriptors (tile, begin, end, 0) that cut the tiles' lists into
  * pieces of at most `max_work_edges` positions (long rows are thereby shared by several
  * workgroups).  All pointers are device memory owned by the caller. */

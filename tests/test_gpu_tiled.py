@@ -60,7 +60,8 @@ def _run_receiver(d, p, other, ptr, perm):
 
 def _check_schedule(sch, other, ptr, perm, order, n, tile_rows, max_work):
     """The schedule is what a host restatement builds: per tile the positions sorted by
-    (sender, position), padding senders last; descriptors tile every tile's list."""
+    (sender, position), padding senders last (tiles of more than 512 positions: live positions
+    in tile order, then the padding ones); descriptors tile every tile's list."""
     other, ptr = other.cpu().numpy(), ptr.cpu().numpy().astype(np.int64)
     order = np.arange(n) if order is None else order.cpu().numpy()
     perm = None if perm is None else perm.cpu().numpy()
@@ -73,8 +74,11 @@ def _check_schedule(sch, other, ptr, perm, order, n, tile_rows, max_work):
         local = np.concatenate([np.full(ptr[r + 1] - ptr[r], i) for i, r in enumerate(rows)] + [np.zeros(0, np.int64)])
         s = other[pos].astype(np.int64)
         key = np.where((s >= 0) & (s < n), s, n)
-        o = np.lexsort((pos, key))
         m = len(pos)
+        if m <= 512:
+            o = np.lexsort((pos, key))
+        else:   # a long tile: live positions in tile order, padding positions behind them
+            o = np.concatenate([np.nonzero(key < n)[0], np.nonzero(key == n)[0]])
         want_snd = np.where(key[o] == n, -1, key[o])
         assert np.array_equal(snd[at:at + m], want_snd), f"tile {t}: senders"
         assert np.array_equal(edge[at:at + m], pos[o] if perm is None else perm[pos[o]]), f"tile {t}: edge rows"
