@@ -54,19 +54,36 @@ __global__ void gather_kernel(const int32_t *__restrict__ src, const int32_t *__
 // A row is read up to kLabelRowCap positions: the labels only steer which rows run together,
 // and a thread that walked a hub's whole row would outlast the rest of the sweep many times.
 constexpr int kLabelRowCap = 128;
+constexpr int kLabelLanes = 4;  // lanes that share a row (its gathers then run four at a time)
 __global__ void min_label_kernel(const int32_t *__restrict__ other,
                                  const int32_t *__restrict__ row_ptr, int num_nodes,
                                  const int32_t *__restrict__ cur, int32_t *__restrict__ next) {
-    const int n = blockIdx.x * blockDim.x + threadIdx.x;
-    if (n >= num_nodes) return;
-    int best = cur[n];
-    const int begin = row_ptr[n];
-    const int end = min(row_ptr[n + 1], begin + kLabelRowCap);
-    for (int e = begin; e < end; e++) {
-        const int m = other[e];
-        if ((unsigned)m < (unsigned)num_nodes) best = min(best, cur[m]);
+    const int t = blockIdx.x * blockDim.x + threadIdx.x;
+    const int n = t / kLabelLanes, part = t % kLabelLanes;
+    const bool inside = n < num_nodes;  // (no early exit: the lanes of a group exchange below)
+    int best = inside ? cur[n] : 0;
+    if (inside) {
+        const int begin = row_ptr[n];
+        const int end = min(row_ptr[n + 1], begin + kLabelRowCap);
+        for (int e = begin + part; e < end; e += kLabelLanes) {
+            const int m = other[e];
+            if ((unsigned)m < (unsigned)num_nodes) best = min(best, cur[m]);
+        }
     }
-    next[n] = best;
+#pragma unroll
+    for (int off = 1; off < kLabelLanes; off *= 2) best = min(best, __shfl_xor(best, off, kWave));
+    if (inside && part == 0) next[n] = best;
+}
+
+// key = (label after the second sweep, label after the first): one sort lists the coarse clusters
+// and, inside them, the fine ones
+__global__ void two_level_keys_kernel(const int32_t *__restrict__ coarse, const int32_t *__restrict__ fine,
+                                      int num_nodes, int bits, uint32_t *__restrict__ keys,
+                                      int32_t *__restrict__ vals) {
+    const int i = blockIdx.x * blockDim.x + threadIdx.x;
+    if (i >= num_nodes) return;
+    keys[i] = ((uint32_t)coarse[i] << bits) | (uint32_t)fine[i];
+    vals[i] = i;
 }
 
 __global__ void copy_i32_kernel(const int32_t *__restrict__ src, int32_t *__restrict__ dst, int64_t n) {
@@ -729,9 +746,27 @@ int e3j_amd_locality_order(const int32_t *other, const int32_t *row_ptr, int32_t
     int done = 0;
     int label_bits = 1;  // labels are node ids: the sort passes stop at their highest bit
     while (label_bits < 32 && ((int64_t)1 << label_bits) < (int64_t)num_nodes) label_bits++;
+    const unsigned label_grid = (unsigned)(((int64_t)num_nodes * kLabelLanes + 255) / 256);
+    if (rounds == 2 && 2 * label_bits <= 32) {
+        // the two levels in one sort: same order as the two stable sorts below, half the passes
+        hipLaunchKernelGGL(min_label_kernel, dim3(label_grid), dim3(256), 0, stream, other, row_ptr, num_nodes,
+                           lab_a, lab_b);
+        hipLaunchKernelGGL(min_label_kernel, dim3(label_grid), dim3(256), 0, stream, other, row_ptr, num_nodes,
+                           lab_b, lab_a);
+        hipLaunchKernelGGL(two_level_keys_kernel, dim3(rows_grid), dim3(256), 0, stream, lab_a, lab_b, num_nodes,
+                           label_bits, keys_in, order_tmp);
+        rc = check_hip(hipGetLastError(), "locality_order sweeps");
+        if (rc) return rc;
+        size_t temp_bytes = sort_bytes;
+        rc = check_hip(hipcub::DeviceRadixSort::SortPairs(sort_temp, temp_bytes, keys_in, keys_out, order_tmp, order,
+                                                          (int)num_nodes, 0, 2 * label_bits, stream),
+                       "locality_order sort");
+        if (rc) return rc;
+        rounds = 0;  // done: skip the level loop
+    }
     for (int level = 1; level <= rounds; level *= 2) {
         for (; done < level; done++) {
-            hipLaunchKernelGGL(min_label_kernel, dim3(rows_grid), dim3(256), 0, stream, other, row_ptr,
+            hipLaunchKernelGGL(min_label_kernel, dim3(label_grid), dim3(256), 0, stream, other, row_ptr,
                                num_nodes, lab_a, lab_b);
             int32_t *t = lab_a; lab_a = lab_b; lab_b = t;
         }
