@@ -61,13 +61,14 @@ __global__ void min_label_kernel(const int32_t *__restrict__ other,
     const int t = blockIdx.x * blockDim.x + threadIdx.x;
     const int n = t / kLabelLanes, part = t % kLabelLanes;
     const bool inside = n < num_nodes;  // (no early exit: the lanes of a group exchange below)
-    int best = inside ? cur[n] : 0;
+    // cur == nullptr: every node still carries its own id (the first sweep)
+    int best = inside ? (cur ? cur[n] : n) : 0;
     if (inside) {
         const int begin = row_ptr[n];
         const int end = min(row_ptr[n + 1], begin + kLabelRowCap);
         for (int e = begin + part; e < end; e += kLabelLanes) {
             const int m = other[e];
-            if ((unsigned)m < (unsigned)num_nodes) best = min(best, cur[m]);
+            if ((unsigned)m < (unsigned)num_nodes) best = min(best, cur ? cur[m] : m);
         }
     }
 #pragma unroll
@@ -195,20 +196,26 @@ __global__ void tile_rank_kernel(const int32_t *__restrict__ row_order, int num_
     rank[row_order ? row_order[q] : q] = q;
 }
 
-// counts[t + 1] = positions of tile t; pieces[t + 1] = work descriptors it is cut into
+// Per tile, two numbers that one prefix sum carries side by side in a 64-bit word: the positions
+// of the tile (high half) and the work descriptors it is cut into (low half); both totals stay
+// below 2^31, so the low half never carries into the high one.
+__device__ inline int tile_start(uint64_t packed) { return (int)(packed >> 32); }
+__device__ inline int tile_first_piece(uint64_t packed) { return (int)(uint32_t)packed; }
+
+// packed[t + 1] = (positions of tile t, descriptors of tile t); packed[0] = 0
 __global__ void tile_count_kernel(const int32_t *__restrict__ row_order, const int32_t *__restrict__ row_ptr,
                                   int num_nodes, int tile_rows, int num_tiles, int max_work_edges,
-                                  int32_t *__restrict__ counts, int32_t *__restrict__ pieces) {
+                                  uint64_t *__restrict__ packed) {
     const int t = blockIdx.x * blockDim.x + threadIdx.x;
-    if (t == 0) counts[0] = pieces[0] = 0;
+    if (t == 0) packed[0] = 0;
     if (t >= num_tiles) return;
     int total = 0;
     for (int q = t * tile_rows; q < (t + 1) * tile_rows && q < num_nodes; q++) {
         const int r = row_order ? row_order[q] : q;
         total += row_ptr[r + 1] - row_ptr[r];
     }
-    counts[t + 1] = total;
-    pieces[t + 1] = total == 0 ? 1 : (total + max_work_edges - 1) / max_work_edges;
+    const int pieces = total == 0 ? 1 : (total + max_work_edges - 1) / max_work_edges;
+    packed[t + 1] = ((uint64_t)total << 32) | (uint64_t)pieces;
 }
 
 // The three lists of one tile, by one wave: the tile's positions (its rows in tile order, each
@@ -217,19 +224,29 @@ __global__ void tile_count_kernel(const int32_t *__restrict__ row_order, const i
 // them.  Longer tiles (hub rows) are not sorted by sender, only split into live positions first
 // and padding positions last, which is all the kernel needs for correctness (it sums runs of
 // equal senders wherever they occur); a hub's senders are mostly distinct anyway.
+// The entries past the last row (padding positions that belong to no tile) are filled by all
+// threads of the grid before they turn to their tiles.
 constexpr int kTileSortLimit = 512;
 __global__ __launch_bounds__(256) void tile_lists_kernel(
     const int32_t *__restrict__ other, const int32_t *__restrict__ row_ptr, const int32_t *__restrict__ perm,
-    const int32_t *__restrict__ row_order, const int32_t *__restrict__ starts, int num_nodes, int tile_rows,
-    int num_tiles, int32_t *__restrict__ t_sender, int32_t *__restrict__ t_edge, int32_t *__restrict__ t_local) {
+    const int32_t *__restrict__ row_order, const uint64_t *__restrict__ packed, int num_nodes, int64_t num_edges,
+    int tile_rows, int num_tiles, int32_t *__restrict__ t_sender, int32_t *__restrict__ t_edge,
+    int32_t *__restrict__ t_local) {
     __shared__ uint64_t keys_all[4][kTileSortLimit];
     __shared__ uint16_t local_all[4][kTileSortLimit];
+    {
+        const int64_t stride = (int64_t)gridDim.x * blockDim.x;
+        for (int64_t i = (int64_t)row_ptr[num_nodes] + (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+             i < num_edges; i += stride) {
+            t_sender[i] = -1; t_edge[i] = 0; t_local[i] = 0;
+        }
+    }
     const int wave = threadIdx.x / 64, lane = threadIdx.x % 64;
     const int t = blockIdx.x * 4 + wave;
     if (t >= num_tiles) return;
     uint64_t *keys = keys_all[wave];
     uint16_t *locals = local_all[wave];
-    const int begin = starts[t], m = starts[t + 1] - begin;
+    const int begin = tile_start(packed[t]), m = tile_start(packed[t + 1]) - begin;
     if (m == 0) return;
     const int first = t * tile_rows;
     const int rows = num_nodes - first < tile_rows ? num_nodes - first : tile_rows;
@@ -304,45 +321,45 @@ __global__ __launch_bounds__(256) void tile_lists_kernel(
     }
 }
 
-// entries of the lists past the last row (padding positions that belong to no tile)
-__global__ void tile_tail_kernel(const int32_t *__restrict__ row_ptr, int num_nodes, int64_t num_edges,
-                                 int32_t *__restrict__ t_sender, int32_t *__restrict__ t_edge,
-                                 int32_t *__restrict__ t_local) {
-    const int64_t live_end = row_ptr[num_nodes];
-    const int64_t stride = (int64_t)gridDim.x * blockDim.x;
-    for (int64_t i = live_end + (int64_t)blockIdx.x * blockDim.x + threadIdx.x; i < num_edges; i += stride) {
-        t_sender[i] = -1; t_edge[i] = 0; t_local[i] = 0;
-    }
-}
-
-// descriptors (tile, begin, end, 0), the first num_used of the num_work entries, num_used in the
-// fourth field of descriptor 0; `starts` / `first_piece`: inclusive prefix sums, entry 0 = 0
-__global__ void tile_work_kernel(const int32_t *__restrict__ starts, const int32_t *__restrict__ first_piece,
-                                 int num_tiles, int max_work_edges, int32_t *__restrict__ work) {
+// descriptors (tile, begin, end, 0), the first num_used of the num_work entries (a tile without
+// positions takes one, with begin == end; the entries behind the used ones are not written),
+// num_used in the fourth field of descriptor 0; `packed`: inclusive prefix sums, entry 0 = 0
+__global__ void tile_work_kernel(const uint64_t *__restrict__ packed, int num_tiles, int max_work_edges,
+                                 int32_t *__restrict__ work) {
     const int t = blockIdx.x * blockDim.x + threadIdx.x;
     if (t >= num_tiles) return;
-    const int begin = starts[t], end = starts[t + 1];
-    int w = first_piece[t];
+    const int begin = tile_start(packed[t]), end = tile_start(packed[t + 1]);
+    int w = tile_first_piece(packed[t]);
+    if (begin == end) {
+        work[4 * w] = t; work[4 * w + 1] = begin; work[4 * w + 2] = begin; work[4 * w + 3] = 0;
+    }
     for (int b = begin; b < end; b += max_work_edges, w++) {
         work[4 * w] = t;
         work[4 * w + 1] = b;
         work[4 * w + 2] = b + max_work_edges < end ? b + max_work_edges : end;
         work[4 * w + 3] = 0;
     }
-    // the number of descriptors in use, for the kernel to deal them evenly to the XCDs
-    if (t == 0) work[3] = first_piece[num_tiles];
+    // the number of descriptors in use, for the kernel to deal them evenly to the XCDs (the
+    // thread of tile 0 wrote descriptor 0 just above)
+    if (t == 0) work[3] = tile_first_piece(packed[num_tiles]);
+}
+
+size_t scan64_temp_bytes(int32_t n) {
+    size_t bytes = 0;
+    hipcub::DeviceScan::InclusiveSum(nullptr, bytes, (uint64_t *)nullptr, (uint64_t *)nullptr, (int)std::max(n, 1));
+    return bytes;
 }
 
 struct TileWorkspace {
-    size_t temp, temp_bytes, counts, pieces, total;
+    size_t temp, temp_bytes, packed, total;
     TileWorkspace(int32_t num_nodes, int32_t tile_rows) {
         const size_t n = (size_t)num_nodes;
         const size_t tiles = (n + (size_t)tile_rows - 1) / (size_t)tile_rows;
         size_t at = 0;
         auto take = [&](size_t bytes) { const size_t here = at; at += align_up(bytes); return here; };
-        temp_bytes = scan_temp_bytes((int32_t)tiles + 1);
+        temp_bytes = scan64_temp_bytes((int32_t)tiles + 1);
         temp = take(temp_bytes);
-        counts = take(4 * (tiles + 1)); pieces = take(4 * (tiles + 1));
+        packed = take(8 * (tiles + 1));
         total = at;
     }
 };
@@ -736,10 +753,8 @@ int e3j_amd_locality_order(const int32_t *other, const int32_t *row_ptr, int32_t
     const unsigned ngrid = grid_for(num_nodes);
     const unsigned rows_grid = (unsigned)((num_nodes + 255) / 256);
 
-    hipLaunchKernelGGL(iota_kernel, dim3(ngrid), dim3(256), 0, stream, lab_a, (int64_t)num_nodes);
-    hipLaunchKernelGGL(iota_kernel, dim3(ngrid), dim3(256), 0, stream, order, (int64_t)num_nodes);
-    int rc = check_hip(hipGetLastError(), "locality_order init");
-    if (rc) return rc;
+    int rc = E3J_AMD_OK;
+    const int32_t *listed = order;  // where the order stands before the long rows are dealt
     // Levels: after 1, 2, 4, 8, ... sweeps the labels name ever larger clusters.  The order is
     // refined from the finest level to the coarsest with stable sorts, so the coarsest clusters
     // are contiguous and, inside them, the finer ones.
@@ -747,22 +762,29 @@ int e3j_amd_locality_order(const int32_t *other, const int32_t *row_ptr, int32_t
     int label_bits = 1;  // labels are node ids: the sort passes stop at their highest bit
     while (label_bits < 32 && ((int64_t)1 << label_bits) < (int64_t)num_nodes) label_bits++;
     const unsigned label_grid = (unsigned)(((int64_t)num_nodes * kLabelLanes + 255) / 256);
-    if (rounds == 2 && 2 * label_bits <= 32) {
+    const bool two_levels = rounds == 2 && 2 * label_bits <= 32;
+    if (two_levels) {
         // the two levels in one sort: same order as the two stable sorts below, half the passes
         hipLaunchKernelGGL(min_label_kernel, dim3(label_grid), dim3(256), 0, stream, other, row_ptr, num_nodes,
-                           lab_a, lab_b);
+                           static_cast<const int32_t *>(nullptr), lab_b);
         hipLaunchKernelGGL(min_label_kernel, dim3(label_grid), dim3(256), 0, stream, other, row_ptr, num_nodes,
                            lab_b, lab_a);
         hipLaunchKernelGGL(two_level_keys_kernel, dim3(rows_grid), dim3(256), 0, stream, lab_a, lab_b, num_nodes,
-                           label_bits, keys_in, order_tmp);
+                           label_bits, keys_in, order);
         rc = check_hip(hipGetLastError(), "locality_order sweeps");
         if (rc) return rc;
         size_t temp_bytes = sort_bytes;
-        rc = check_hip(hipcub::DeviceRadixSort::SortPairs(sort_temp, temp_bytes, keys_in, keys_out, order_tmp, order,
+        rc = check_hip(hipcub::DeviceRadixSort::SortPairs(sort_temp, temp_bytes, keys_in, keys_out, order, order_tmp,
                                                           (int)num_nodes, 0, 2 * label_bits, stream),
                        "locality_order sort");
         if (rc) return rc;
+        listed = order_tmp;
         rounds = 0;  // done: skip the level loop
+    } else {
+        hipLaunchKernelGGL(iota_kernel, dim3(ngrid), dim3(256), 0, stream, lab_a, (int64_t)num_nodes);
+        hipLaunchKernelGGL(iota_kernel, dim3(ngrid), dim3(256), 0, stream, order, (int64_t)num_nodes);
+        rc = check_hip(hipGetLastError(), "locality_order init");
+        if (rc) return rc;
     }
     for (int level = 1; level <= rounds; level *= 2) {
         for (; done < level; done++) {
@@ -784,7 +806,7 @@ int e3j_amd_locality_order(const int32_t *other, const int32_t *row_ptr, int32_t
     }
     // long rows to the fronts of the eighths of the list
     int32_t *flags = reinterpret_cast<int32_t *>(keys_in), *rank = reinterpret_cast<int32_t *>(keys_out);
-    hipLaunchKernelGGL(long_row_flags_kernel, dim3(rows_grid), dim3(256), 0, stream, order, row_ptr, num_nodes,
+    hipLaunchKernelGGL(long_row_flags_kernel, dim3(rows_grid), dim3(256), 0, stream, listed, row_ptr, num_nodes,
                        flags);
     rc = check_hip(hipGetLastError(), "locality_order flags");
     if (rc) return rc;
@@ -792,10 +814,15 @@ int e3j_amd_locality_order(const int32_t *other, const int32_t *row_ptr, int32_t
     rc = check_hip(hipcub::DeviceScan::InclusiveSum(sort_temp, scan_bytes, flags, rank, num_nodes, stream),
                    "locality_order scan");
     if (rc) return rc;
-    hipLaunchKernelGGL(deal_long_rows_kernel, dim3(rows_grid), dim3(256), 0, stream, order, flags, rank,
-                       num_nodes, order_tmp);
-    hipLaunchKernelGGL(copy_i32_kernel, dim3(ngrid), dim3(256), 0, stream, order_tmp, order,
-                       (int64_t)num_nodes);
+    if (listed == order_tmp) {  // dealt straight into the result
+        hipLaunchKernelGGL(deal_long_rows_kernel, dim3(rows_grid), dim3(256), 0, stream, listed, flags, rank,
+                           num_nodes, order);
+    } else {
+        hipLaunchKernelGGL(deal_long_rows_kernel, dim3(rows_grid), dim3(256), 0, stream, listed, flags, rank,
+                           num_nodes, order_tmp);
+        hipLaunchKernelGGL(copy_i32_kernel, dim3(ngrid), dim3(256), 0, stream, order_tmp, order,
+                           (int64_t)num_nodes);
+    }
     return check_hip(hipGetLastError(), "locality_order");
 }
 
@@ -828,35 +855,26 @@ int e3j_amd_tile_schedule_build(const int32_t *other, const int32_t *row_ptr, co
     unsigned char *ws = static_cast<unsigned char *>(workspace);
     ws += (256 - reinterpret_cast<uintptr_t>(ws) % 256) % 256;
     const TileWorkspace w(num_nodes, tile_rows);
-    int32_t *counts = reinterpret_cast<int32_t *>(ws + w.counts);
-    int32_t *pieces = reinterpret_cast<int32_t *>(ws + w.pieces);
+    uint64_t *packed = reinterpret_cast<uint64_t *>(ws + w.packed);
     const int num_tiles = (num_nodes + tile_rows - 1) / tile_rows;
-    const int64_t num_work = e3j_amd_tile_schedule_num_work(num_nodes, num_edges, tile_rows, max_work_edges);
     const unsigned tiles_grid = (unsigned)((num_tiles + 255) / 256);
 
-    int rc = launch_fill_zero(work, sizeof(int32_t) * 4 * (size_t)num_work, stream);
-    if (rc) return rc;
     hipLaunchKernelGGL(tile_count_kernel, dim3(tiles_grid), dim3(256), 0, stream, row_order, row_ptr, num_nodes,
-                       tile_rows, num_tiles, max_work_edges, counts, pieces);
-    rc = check_hip(hipGetLastError(), "tile schedule counts");
+                       tile_rows, num_tiles, max_work_edges, packed);
+    int rc = check_hip(hipGetLastError(), "tile schedule counts");
     if (rc) return rc;
     size_t temp_bytes = w.temp_bytes;
-    rc = check_hip(hipcub::DeviceScan::InclusiveSum(ws + w.temp, temp_bytes, counts, counts, num_tiles + 1, stream),
+    rc = check_hip(hipcub::DeviceScan::InclusiveSum(ws + w.temp, temp_bytes, packed, packed, num_tiles + 1, stream),
                    "tile schedule scan");
     if (rc) return rc;
-    temp_bytes = w.temp_bytes;
-    rc = check_hip(hipcub::DeviceScan::InclusiveSum(ws + w.temp, temp_bytes, pieces, pieces, num_tiles + 1, stream),
-                   "tile schedule scan");
-    if (rc) return rc;
-    hipLaunchKernelGGL(tile_work_kernel, dim3(tiles_grid), dim3(256), 0, stream, counts, pieces, num_tiles,
-                       max_work_edges, work);
+    hipLaunchKernelGGL(tile_work_kernel, dim3(tiles_grid), dim3(256), 0, stream, packed, num_tiles, max_work_edges,
+                       work);
     rc = check_hip(hipGetLastError(), "tile schedule work");
     if (rc || num_edges == 0) return rc;
     // the lists: one wave per tile sorts its positions by sender in LDS
     hipLaunchKernelGGL(tile_lists_kernel, dim3((unsigned)((num_tiles + 3) / 4)), dim3(256), 0, stream, other, row_ptr,
-                       edge_perm, row_order, counts, num_nodes, tile_rows, num_tiles, t_sender, t_edge, t_local);
-    hipLaunchKernelGGL(tile_tail_kernel, dim3(64), dim3(256), 0, stream, row_ptr, num_nodes, num_edges, t_sender,
-                       t_edge, t_local);
+                       edge_perm, row_order, packed, num_nodes, num_edges, tile_rows, num_tiles, t_sender, t_edge,
+                       t_local);
     return check_hip(hipGetLastError(), "tile schedule lists");
 }
 

@@ -166,9 +166,10 @@ int e3j_amd_convolution_bwd_ordered(const e3j_amd_conv_params *p, const void *co
  * workgroups).  All pointers are device memory owned by the caller. */
 typedef struct e3j_amd_tile_schedule {
     int32_t tile_rows;     /* receivers per tile */
-    int32_t num_work;      /* entries of `work` (an upper bound; unused entries have begin == end) */
-    const int32_t *work;   /* (num_work, 4): (tile, begin, end, 0), the entries in use first; the
-                              fourth field of entry 0 holds their number */
+    int32_t num_work;      /* entries of `work` (an upper bound of the entries in use) */
+    const int32_t *work;   /* (num_work, 4): (tile, begin, end, 0), the entries in use first (a tile
+                              without positions takes one with begin == end); the fourth field of
+                              entry 0 holds their number, the entries behind them are not read */
     const int32_t *sender; /* (E) sender of the position, -1 for a padding edge */
     const int32_t *edge;   /* (E) row of y / s / dy / ds */
     const int32_t *local;  /* (E) index of the position's receiver within its tile */

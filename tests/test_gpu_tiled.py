@@ -67,6 +67,9 @@ def _check_schedule(sch, other, ptr, perm, order, n, tile_rows, max_work):
     perm = None if perm is None else perm.cpu().numpy()
     snd, edge, loc = sch.sender.cpu().numpy(), sch.edge.cpu().numpy(), sch.local.cpu().numpy()
     work = sch.work.cpu().numpy()[:sch.num_work]
+    used = int(work[0, 3])
+    assert (n + tile_rows - 1) // tile_rows <= used <= sch.num_work
+    work = work[:used]          # the entries behind the used ones are not written
     at, covered = 0, []
     for t in range((n + tile_rows - 1) // tile_rows):
         rows = order[t * tile_rows:(t + 1) * tile_rows]
