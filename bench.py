@@ -125,6 +125,9 @@ def parse_args():
     ap.add_argument("--no-layouts", action="store_true",
                     help="skip the leading-channels sub-record of the default run")
     ap.add_argument("--cpu-seconds", type=float, default=15.0)
+    ap.add_argument("--table-driven", action="store_true",
+                    help="with --kernel-only: time the table-driven kernels (signature -1) instead of the "
+                         "unrolled ones; E3J_AMD_TABLE_PLANS=0 selects their form without a plan")
     ap.add_argument("--kernel-only", action="store_true",
                     help="time the C-ABI launches only (no operator-level step)")
     ap.add_argument("--spatial-sort", action="store_true",
@@ -171,7 +174,7 @@ def build_workload(name: str, scale: float, device, spatial_sort: bool = False, 
 class AbiCalls:
     """Direct launches through the C ABI with a prebuilt receiver CSR (kernel timing)."""
 
-    def __init__(self, w):
+    def __init__(self, w, table_driven=False):
         import numpy as np
         import torch
         from e3j_amd import _lib
@@ -186,6 +189,8 @@ class AbiCalls:
         d = 2 if w.leading else 1
         dims = (w.x.shape[d], w.y.shape[1], module.params.num_out, w.s.shape[d])
         sig, scale, _ = self.table.signature(tuple(int(d) for d in dims), w.channels, module.layout)
+        if table_driven:   # the kernels that read the table at run time, as for a table without a signature
+            sig, scale = -1, 1.0
         self.signature = sig
         self.params = _lib.ConvParams(
             num_nodes=w.num_nodes, num_edges=w.num_edges, num_coef=self.table.num_coef,
@@ -641,7 +646,7 @@ def main():
     if args.calibrate_copy:
         calibrate_copy(torch, device)
 
-    abi = AbiCalls(w)
+    abi = AbiCalls(w, table_driven=args.table_driven)
     if args.deterministic:
         e3j_amd.config(deterministic=True)
         abi.backward = abi.backward_ordered

@@ -130,6 +130,9 @@ SYMBOLS = {
     "e3j_amd_order_workspace_bytes": (ctypes.c_size_t, [ctypes.c_int32]),
     "e3j_amd_register_signature": (ctypes.c_int, [_P]),
     "e3j_amd_set_launch_variant": (None, [ctypes.c_int32, ctypes.c_int32]),
+    "e3j_amd_set_table_plans": (None, [ctypes.c_int32]),
+    "e3j_amd_table_plan_status": (ctypes.c_int, [ctypes.POINTER(ConvParams), ctypes.c_void_p, ctypes.c_int32,
+                                                 ctypes.POINTER(ctypes.c_int32), ctypes.c_void_p]),
     "e3j_amd_harmonics": (ctypes.c_int, [_P, ctypes.c_int64] + [ctypes.c_int32] * 4 + [_P, _P]),
     "e3j_amd_harmonics_bwd": (ctypes.c_int, [_P, _P, ctypes.c_int64] + [ctypes.c_int32] * 4 + [_P, _P]),
     "e3j_amd_radial_linear_fwd": (ctypes.c_int, [_P, _P, _P, ctypes.c_int64, ctypes.c_int32, ctypes.c_int32, _P]),

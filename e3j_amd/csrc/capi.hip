@@ -45,6 +45,14 @@ Tuning &mutable_tuning() {
 
 const Tuning &tuning() { return mutable_tuning(); }
 
+std::atomic<int> &table_plans() {
+    static std::atomic<int> on{[] {
+        const char *e = std::getenv("E3J_AMD_TABLE_PLANS");
+        return e == nullptr || std::atoi(e) != 0 ? 1 : 0;
+    }()};
+    return on;
+}
+
 // Signatures registered at run time live behind the built-in ones.  The list only grows and
 // a deque never moves its elements, so ids and references stay valid.
 namespace {
@@ -268,6 +276,8 @@ int e3j_amd_register_signature(const void *entry) {
     g_registered.push_back(sg);
     return num_builtin_signatures() + (int)g_registered.size() - 1;
 }
+
+void e3j_amd_set_table_plans(int32_t on) { table_plans().store(on ? 1 : 0, std::memory_order_relaxed); }
 
 void e3j_amd_set_launch_variant(int32_t fwd_variant, int32_t bwd_variant) {
     mutable_tuning().fwd_variant.store(fwd_variant, std::memory_order_relaxed);

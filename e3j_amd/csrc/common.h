@@ -90,6 +90,21 @@ int launch_generic_bwd(const e3j_amd_conv_params &p, bool group_is_receiver, con
                        void *dx, void *dy, void *ds, hipStream_t stream,
                        bool coef_cols_ji = false);
 int launch_fill_zero(void *ptr, size_t bytes, hipStream_t stream);
+// Table-driven kernels over a plan of the table (conv_planned.hip): float32 tables within the
+// plan's limits.  The plan is built on the device; its first word says whether the table could
+// be taken, and the kernels with and without plan both look at it.
+bool plan_takes(const e3j_amd_conv_params &p);
+size_t plan_bytes(const e3j_amd_conv_params &p);
+int launch_plan_build(const e3j_amd_conv_params &p, const void *coef, bool cols_ji, int32_t *plan,
+                      hipStream_t stream);
+int launch_planned_fwd(const e3j_amd_conv_params &p, const int32_t *plan, const void *x, const void *y,
+                       const void *s, const int32_t *other, const int32_t *row_ptr, const int32_t *perm,
+                       void *out, hipStream_t stream);
+int launch_planned_bwd(const e3j_amd_conv_params &p, bool group_is_receiver, const int32_t *plan, const void *x,
+                       const void *y, const void *s, const void *dm, const int32_t *other,
+                       const int32_t *row_ptr, const int32_t *perm, void *dx, void *dy, void *ds,
+                       hipStream_t stream);
+std::atomic<int> &table_plans();  // 1: plan the tables that can be planned (default); 0: never
 // Zero the dy/ds rows of padding edges (float32 operands).
 int launch_zero_padding(const e3j_amd_conv_params &p, const int32_t *other, const int32_t *row_ptr,
                         const int32_t *perm, float *dy, float *ds, hipStream_t stream);

@@ -122,8 +122,10 @@ __global__ void generic_fwd_kernel(const Coef4D<Idx, Val> *__restrict__ coef, in
                                    const int32_t *__restrict__ perm,
                                    const int32_t *__restrict__ row_order,
                                    Val *__restrict__ out, RowLayout lo,
-                                   int num_nodes, int channels, int X, int S, int Z, int nchunks) {
+                                   int num_nodes, int channels, int X, int S, int Z, int nchunks,
+                                   const int32_t *__restrict__ served) {
     extern __shared__ __align__(16) unsigned char smem_raw[];
+    if (served && *served) return;  // the kernel over the table's plan has taken the call
     const int lane = threadIdx.x;
     const int wave = threadIdx.y;
     const int64_t item = (int64_t)blockIdx.x * blockDim.y + wave;
@@ -204,8 +206,9 @@ __global__ void generic_bwd_kernel(const Coef4D<Idx, Val> *__restrict__ coef, in
                                    const int32_t *__restrict__ row_order,
                                    Val *__restrict__ dx, Val *__restrict__ dy, Val *__restrict__ ds,
                                    int num_nodes, int channels, int X, int S, int Z, int nchunks,
-                                   int cols_ji) {
+                                   int cols_ji, const int32_t *__restrict__ served) {
     extern __shared__ __align__(16) unsigned char smem_raw[];
+    if (served && *served) return;  // the kernel over the table's plan has taken the call
     const int lane = threadIdx.x;
     const int wave = threadIdx.y;
     const int64_t item = (int64_t)blockIdx.x * blockDim.y + wave;
@@ -346,8 +349,12 @@ int pick_waves(size_t per_wave_bytes, size_t budget) {
 template <typename Idx, typename Val>
 int run_fwd(const e3j_amd_conv_params &p, const void *coef, const void *x, const void *y,
             const void *s, const int32_t *other, const int32_t *row_ptr, const int32_t *perm,
-            void *out, hipStream_t stream) {
+            void *out, hipStream_t stream, const int32_t *plan) {
     const int nchunks = (p.channels + kWave - 1) / kWave;
+    if (plan) {  // runs if the plan took the table; the kernel below runs if it did not
+        int rc = launch_planned_fwd(p, plan, x, y, s, other, row_ptr, perm, out, stream);
+        if (rc) return rc;
+    }
     const size_t per_wave = (size_t)(p.num_out + p.num_x + p.num_scalars) * kWave * sizeof(Val);
     if (per_wave > kMaxLds)
         return set_error(E3J_AMD_UNIMPLEMENTED, "convolution: num_out + num_x + num_scalars = " +
@@ -373,7 +380,7 @@ int run_fwd(const e3j_amd_conv_params &p, const void *coef, const void *x, const
                        static_cast<const Val *>(s), make_layout(p.layout, p.num_scalars, p.channels),
                        other, row_ptr, perm, p.row_order,
                        static_cast<Val *>(out), make_layout(p.layout, p.num_out, p.channels),
-                       p.num_nodes, p.channels, p.num_x, p.num_scalars, p.num_out, nchunks);
+                       p.num_nodes, p.channels, p.num_x, p.num_scalars, p.num_out, nchunks, plan);
     return check_hip(hipGetLastError(), "convolution forward launch");
 }
 
@@ -392,7 +399,7 @@ template <typename Idx, typename Val>
 int run_bwd(const e3j_amd_conv_params &p, bool group_is_receiver, const void *coef, const void *x,
             const void *y, const void *s, const void *dm, const int32_t *other,
             const int32_t *row_ptr, const int32_t *perm, void *dx, void *dy, void *ds,
-            hipStream_t stream, bool cols_ji) {
+            hipStream_t stream, bool cols_ji, const int32_t *plan) {
     const int nchunks = (p.channels + kWave - 1) / kWave;
     const size_t per_wave =
         (size_t)(p.num_out + 2 * p.num_x + 2 * p.num_scalars + p.num_y) * kWave * sizeof(Val);
@@ -411,8 +418,16 @@ int run_bwd(const e3j_amd_conv_params &p, bool group_is_receiver, const void *co
         rc = launch_fill_zero(dx, (size_t)p.num_nodes * p.num_x * p.channels * sizeof(Val), stream);
         if (rc) return rc;
     }
+    if (plan && group_is_receiver && nchunks > 1) {  // the waves of an edge add their dy parts
+        rc = launch_fill_zero(dy, (size_t)p.num_edges * p.num_y * sizeof(Val), stream);
+        if (rc) return rc;
+    }
     rc = zero_padding<Val>(p, other, row_ptr, perm, static_cast<Val *>(dy), static_cast<Val *>(ds), stream);
     if (rc) return rc;
+    if (plan) {  // runs if the plan took the table; the kernel below runs if it did not
+        rc = launch_planned_bwd(p, group_is_receiver, plan, x, y, s, dm, other, row_ptr, perm, dx, dy, ds, stream);
+        if (rc) return rc;
+    }
 #define E3J_LAUNCH_BWD(FLAG)                                                                      \
     do {                                                                                          \
         auto kernel = p.num_y <= kWave ? generic_bwd_kernel<Idx, Val, FLAG, true>                 \
@@ -431,7 +446,7 @@ int run_bwd(const e3j_amd_conv_params &p, bool group_is_receiver, const void *co
                            other, row_ptr, perm, p.row_order, static_cast<Val *>(dx),             \
                            static_cast<Val *>(dy),                                               \
                            static_cast<Val *>(ds), p.num_nodes, p.channels, p.num_x,              \
-                           p.num_scalars, p.num_out, nchunks, cols_ji ? 1 : 0);                   \
+                           p.num_scalars, p.num_out, nchunks, cols_ji ? 1 : 0, plan);             \
     } while (0)
     if constexpr (std::is_same<Val, half_t>::value) {
         // no float atomics on half values: rows must own their dx (sender-grouped)
@@ -544,6 +559,30 @@ int launch_zero_padding(const e3j_amd_conv_params &p, const int32_t *other, cons
     return zero_padding<float>(p, other, row_ptr, perm, dy, ds, stream);
 }
 
+// The plan of a table the planned kernels can take (conv_planned.hip), in memory of the stream's
+// pool for the length of the call; none when the sizes are outside the plan's limits, when
+// planning is switched off, or when the pool gives nothing (a stream under capture).
+struct PlanScratch {
+    int32_t *plan = nullptr;
+    hipStream_t stream;
+    int rc = E3J_AMD_OK;
+    PlanScratch(const e3j_amd_conv_params &p, const void *coef, bool cols_ji, hipStream_t st) : stream(st) {
+        if (!plan_takes(p) || !table_plans().load(std::memory_order_relaxed)) return;
+        void *mem = nullptr;
+        if (hipMallocAsync(&mem, plan_bytes(p), stream) != hipSuccess) {
+            (void)hipGetLastError();
+            return;
+        }
+        plan = static_cast<int32_t *>(mem);
+        rc = launch_plan_build(p, coef, cols_ji, plan, stream);
+    }
+    ~PlanScratch() {
+        if (plan) (void)hipFreeAsync(plan, stream);
+    }
+    PlanScratch(const PlanScratch &) = delete;
+    PlanScratch &operator=(const PlanScratch &) = delete;
+};
+
 #define E3J_DISPATCH(CALL)                                                                  \
     if (p.val_dtype == E3J_AMD_F32 && p.coef_idx_bytes == 1) return CALL(uint8_t, float);   \
     if (p.val_dtype == E3J_AMD_F32 && p.coef_idx_bytes == 4) return CALL(int32_t, float);   \
@@ -556,7 +595,10 @@ int launch_zero_padding(const e3j_amd_conv_params &p, const int32_t *other, cons
 int launch_generic_fwd(const e3j_amd_conv_params &p, const void *coef, const void *x, const void *y,
                        const void *s, const int32_t *other, const int32_t *row_ptr,
                        const int32_t *edge_perm, void *out, hipStream_t stream) {
-#define E3J_FWD(I, V) run_fwd<I, V>(p, coef, x, y, s, other, row_ptr, edge_perm, out, stream)
+    const PlanScratch scratch(p, coef, false, stream);
+    if (scratch.rc) return scratch.rc;
+    const int32_t *plan = scratch.plan;
+#define E3J_FWD(I, V) run_fwd<I, V>(p, coef, x, y, s, other, row_ptr, edge_perm, out, stream, plan)
     E3J_DISPATCH(E3J_FWD);
 #undef E3J_FWD
 }
@@ -565,9 +607,12 @@ int launch_generic_bwd(const e3j_amd_conv_params &p, bool group_is_receiver, con
                        const void *x, const void *y, const void *s, const void *dm,
                        const int32_t *other, const int32_t *row_ptr, const int32_t *edge_perm,
                        void *dx, void *dy, void *ds, hipStream_t stream, bool coef_cols_ji) {
+    const PlanScratch scratch(p, coef, coef_cols_ji, stream);
+    if (scratch.rc) return scratch.rc;
+    const int32_t *plan = scratch.plan;
 #define E3J_BWD(I, V)                                                                            \
     run_bwd<I, V>(p, group_is_receiver, coef, x, y, s, dm, other, row_ptr, edge_perm, dx, dy, ds, \
-                  stream, coef_cols_ji)
+                  stream, coef_cols_ji, plan)
     E3J_DISPATCH(E3J_BWD);
 #undef E3J_BWD
 }

@@ -232,6 +232,30 @@ int e3j_amd_find_signature(const void *coef_host, int32_t coef_idx_bytes, int32_
  * (src/e3j/ops/convolution.py:178-208). */
 void e3j_amd_set_launch_variant(int32_t fwd_variant, int32_t bwd_variant);
 
+/* The table-driven kernels (calls with signature < 0, and calls whose operands an unrolled kernel
+ * cannot take) come in two forms.  For a float32 table in which every output coordinate uses one
+ * scalar, with at most 128 output coordinates, 16 x coordinates, 64 y components, 1024 scalars and
+ * 8192 entries, the call first turns the table into a plan on the device (one small kernel; the
+ * plan lives in memory of the stream's pool, hipMallocAsync, for the length of the call) and runs
+ * kernels that keep x and the accumulators in registers; any other table, float64 and float16
+ * run the kernels that index LDS columns by the table's coordinates.  Whether a table fits is
+ * decided on the device, without a read-back.  on = 0 switches the planned form off for later
+ * calls (process-wide, atomic; initial value from E3J_AMD_TABLE_PLANS, default 1); a stream under
+ * graph capture, where the pool gives no memory, gets the LDS-column kernels as well.  Results
+ * agree to rounding (the planned form sums per output coordinate in a different order).
+ * No counterpart in the reference, which has one table-driven kernel
+ * (lib/e3j_ops/cuda/convolution/fwd.cuh:88-153). */
+void e3j_amd_set_table_plans(int32_t on);
+/* Whether the planned form takes a table, and what its plan looks like: builds the plan of the
+ * device-resident table `coef` (the operand of the convolution calls; coef_cols_ji as for the
+ * backward entry points), waits for it and writes status[0] = 1 if the planned kernels take the
+ * table (0: sizes beyond the limits, or an output coordinate with two scalars), status[1] = its
+ * non-empty (output coordinate, x coordinate) cells, status[2] = the (16 output coordinates x 4 x
+ * coordinates) blocks the loops visit, status[3] = scalars no entry uses.  Allocates and
+ * synchronises: for tests and set-up code, not for the hot path. */
+int e3j_amd_table_plan_status(const e3j_amd_conv_params *p, const void *coef, int32_t coef_cols_ji,
+                              int32_t *status, void *stream);
+
 /* Adds a signature compiled at run time (e3j_amd/jit.py generates the kernels of a table
  * the library was not built for, compiles them against this library and hands over the entry
  * its plugin exports).  Returns the new signature id, which e3j_amd_find_signature reports
