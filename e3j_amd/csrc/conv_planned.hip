@@ -257,7 +257,10 @@ __device__ __forceinline__ void stage_table(const int32_t *__restrict__ plan, co
     for (int t = tid; t < num_cells; t += threads) tab[t] = plan[L.cells + t];
     for (int t = tid; t < 2 * num_coef; t += threads) tab[pairs + t] = plan[L.pairs + t];
     int32_t *dense = tab + table_words(num_coef);
-    for (int t = tid; t < dense_cells; t += threads) dense[t] = plan[L.first + t] | (plan[L.count + t] << 11);
+    for (int t = tid; t < dense_cells; t += threads) {
+        const int cnt = plan[L.count + t];  // (an empty cell behind the last entry has first = 2048: dropped)
+        dense[t] = cnt > 0 ? plan[L.first + t] | (cnt << 11) : 0;
+    }
     __syncthreads();
 }
 

@@ -1,0 +1,233 @@
+"""The two forms of the table-driven kernels through the C ABI (signature -1): over a plan of the
+table that one workgroup builds on the device (float32 tables in which every output coordinate
+uses one scalar, within the plan's size limits), and over LDS columns indexed by the table's
+coordinates (everything else).  Which form a table gets is checked through
+`e3j_amd_table_plan_status`; both forms are compared with the CPU oracle and with each other."""
+
+import ctypes
+
+import numpy as np
+import pytest
+import torch
+
+from e3j_amd import _lib, workloads as W
+from oracle import conv_oracle as O
+from tests import helpers as H
+from tests.test_gpu_generic import _dev, _params, check_all, run_abi
+
+pytestmark = pytest.mark.gpu
+
+
+@pytest.fixture
+def plans_off():
+    lib = _lib.load()
+    lib.e3j_amd_set_table_plans(0)
+    yield
+    lib.e3j_amd_set_table_plans(1)
+
+
+def _status(packed, X, Y, Z, S, K=8, cols_ji=0, val=_lib.F32):
+    """(taken, cells, blocks, unused scalars) of the plan of a packed table."""
+    coef_d = _dev(packed.view(np.uint8).reshape(-1))
+    p = _params(4, 4, len(packed), X, Y, Z, S, K, 1, val, packed.dtype.itemsize)
+    status = (ctypes.c_int32 * 4)()
+    _lib.check(_lib.load().e3j_amd_table_plan_status(ctypes.byref(p), coef_d.data_ptr(), cols_ji, status,
+                                                    torch.cuda.current_stream().cuda_stream))
+    return tuple(int(v) for v in status)
+
+
+def test_plan_of_the_l3_table():
+    """cfg3's table: 353 entries on 311 (output, x) cells; the output coordinates sorted by the
+    x coordinates of their paths leave 14 of the 28 blocks of 16 outputs x 4 x coordinates."""
+    w = W.config3(0.002)
+    idx, val, mix = w.table()
+    packed = H.pack_table(idx, val, mix)
+    i, j = np.asarray(idx)[:, 0], np.asarray(idx)[:, 1]
+    cells = len(set(zip(i.tolist(), j.tolist())))
+    taken, got_cells, blocks, unused = _status(packed, 16, 16, 99, 23)
+    assert (taken, got_cells, unused) == (1, cells, 0) and cells == 311
+    assert blocks == 14
+
+
+def test_tables_the_plan_does_not_take():
+    rng = np.random.default_rng(0)
+    idx, val, mix = H.random_table(rng, 60, 5, 7, 6, 4)
+    assert _status(H.pack_table(idx, val, mix), 5, 7, 6, 4)[0] == 1
+    # an output coordinate with two scalars
+    other_mix = (np.asarray(mix) + 1) % 4
+    both = np.concatenate([H.pack_table(idx, val, mix, idx_dtype=np.uint8),
+                           H.pack_table(idx[:5], val[:5], other_mix, idx_dtype=np.uint8)])
+    assert _status(both, 5, 7, 6, 4)[0] == 0
+    # sizes beyond the limits: x coordinates, y components, output coordinates, float64
+    big = H.random_table(rng, 300, 17, 7, 6, 4)
+    assert _status(H.pack_table(*big), 17, 7, 6, 4)[0] == 0
+    big = H.random_table(rng, 300, 5, 65, 6, 4)
+    assert _status(H.pack_table(*big), 5, 65, 6, 4)[0] == 0
+    big = H.random_table(rng, 300, 5, 7, 129, 4)
+    assert _status(H.pack_table(*big), 5, 7, 129, 4)[0] == 0
+    assert _status(H.pack_table(idx, val, mix, val_dtype=np.float64), 5, 7, 6, 4, val=_lib.F64)[0] == 0
+
+
+def test_a_table_with_two_scalars_on_one_output_runs_the_column_kernels():
+    """Not plannable; the result is still the sum of the two tables' results (the contraction is
+    linear in the table)."""
+    rng = np.random.default_rng(1)
+    N, E, X, Y, Z, S, K = 9, 40, 5, 7, 6, 4, 24
+    idx, val, mix = H.random_table(rng, 60, X, Y, Z, S)
+    mix2 = (np.asarray(mix) + 1) % S
+    sub = slice(0, 25)
+    packed = np.concatenate([H.pack_table(idx, val, mix, idx_dtype=np.uint8),
+                             H.pack_table(idx[sub], val[sub], mix2, idx_dtype=np.uint8)])
+    snd, rcv = H.random_graph(rng, N, E)
+    x, y, s, dm = H.random_operands(rng, N, E, X, Y, S, K, Z)
+    lib = _lib.load()
+    coef_d = _dev(packed.view(np.uint8).reshape(-1))
+    xd, yd, sd, dmd = _dev(x), _dev(y), _dev(s), _dev(dm)
+    other, ptr_d = _dev(snd.astype(np.int32)), _dev(O.receiver_ptr(rcv, N))
+    p = _params(N, E, len(packed), X, Y, Z, S, K, 1, _lib.F32, packed.dtype.itemsize)
+    out = torch.full((N, Z, K), float("nan"), device="cuda")
+    dx, dy, ds = (torch.full_like(t, float("nan")) for t in (xd, yd, sd))
+    stream = torch.cuda.current_stream().cuda_stream
+    _lib.check(lib.e3j_amd_convolution_fwd(ctypes.byref(p), coef_d.data_ptr(), xd.data_ptr(), yd.data_ptr(),
+                                           sd.data_ptr(), other.data_ptr(), ptr_d.data_ptr(), None,
+                                           out.data_ptr(), stream))
+    _lib.check(lib.e3j_amd_convolution_bwd_receiver(
+        ctypes.byref(p), coef_d.data_ptr(), xd.data_ptr(), yd.data_ptr(), sd.data_ptr(), dmd.data_ptr(),
+        other.data_ptr(), ptr_d.data_ptr(), None, dx.data_ptr(), dy.data_ptr(), ds.data_ptr(), stream))
+    torch.cuda.synchronize()
+    ref = mag = 0
+    grads, mags = [0, 0, 0], [0, 0, 0]
+    for ti, tv, tm in ((idx, val, mix), (idx[sub], val[sub], mix2)):
+        r, m = H.forward_reference(ti, tv, tm, x, y, s, snd, rcv, Z)
+        ref, mag = ref + r, mag + m
+        g, gm = H.backward_reference(ti, tv, tm, x, y, s, snd, rcv, dm)
+        grads = [a + b for a, b in zip(grads, g)]
+        mags = [a + b for a, b in zip(mags, gm)]
+    H.assert_parity(out.cpu().numpy(), ref, mag, "two scalars out")
+    for got, r, m, name in zip((dx, dy, ds), grads, mags, ("dx", "dy", "ds")):
+        H.assert_parity(got.cpu().numpy(), r, m, f"two scalars {name}")
+
+
+# shapes: (X, Y, Z, S, nnz): one block, several blocks with a partial last one, the largest plan
+SHAPES = [(3, 4, 5, 2, 30), (9, 16, 35, 11, 260), (16, 16, 99, 23, 353), (16, 64, 128, 64, 2048)]
+
+
+@pytest.mark.parametrize("grouping", ["receiver", "sender"])
+@pytest.mark.parametrize("channels", [1, 64, 70, 130])
+@pytest.mark.parametrize("X, Y, Z, S, nnz", SHAPES)
+def test_planned_kernels_match_oracle(X, Y, Z, S, nnz, channels, grouping):
+    rng = np.random.default_rng(X * 1000 + channels)
+    idx, val, mix = H.random_table(rng, nnz, X, Y, Z, S)
+    assert _status(H.pack_table(idx, val, mix), X, Y, Z, S)[0] == 1
+    N, E = 7, 30
+    snd, rcv = H.random_graph(rng, N, E)
+    x, y, s, dm = H.random_operands(rng, N, E, X, Y, S, channels, Z)
+    res = run_abi(idx, val, mix, x, y, s, dm, snd, rcv, Z, grouping=grouping)
+    check_all(idx, val, mix, x, y, s, dm, snd, rcv, Z, res, tag=f"{(X, Y, Z, S)} K={channels} {grouping}")
+
+
+def test_l3_table_with_padding_edges_and_permutation():
+    """cfg3's table (7 blocks x 4 groups, 14 visited) on unsorted edges with padding among them."""
+    w = W.config3(0.002)
+    idx, val, mix = w.table()
+    rng = np.random.default_rng(33)
+    N, E, K = 12, 90, 128
+    snd, rcv = H.random_graph(rng, N, E, sort_by=None)
+    snd[rng.random(E) < 0.1] = O.DUMMY_INDEX
+    x, y, s, dm = H.random_operands(rng, N, E, 16, 16, 23, K, 99)
+    perm = np.argsort(rcv, kind="stable").astype(np.int32)
+    out, dx, dy, ds = run_abi(idx, val, mix, x, y, s, dm, snd, rcv, 99, perm=perm)
+    live = snd != O.DUMMY_INDEX
+    assert not dy[~live].any() and not ds[~live].any()
+    ref, mag = H.forward_reference(idx, val, mix, x, y[live], s[live], snd[live], rcv[live], 99)
+    H.assert_parity(out, ref, mag, "out")
+    refs, mags = H.backward_reference(idx, val, mix, x, y[live], s[live], snd[live], rcv[live], dm)
+    H.assert_parity(dx, refs[0], mags[0], "dx")
+    H.assert_parity(dy[live], refs[1], mags[1], "dy")
+    H.assert_parity(ds[live], refs[2], mags[2], "ds")
+
+
+def test_leading_layout_and_wide_indices():
+    rng = np.random.default_rng(44)
+    N, E, X, Y, Z, S, K, nnz = 9, 40, 9, 9, 20, 6, 40, 120
+    idx, val, mix = H.random_table(rng, nnz, X, Y, Z, S)
+    snd, rcv = H.random_graph(rng, N, E)
+    x, y, s, dm = H.random_operands(rng, N, E, X, Y, S, K, Z)
+    xl, sl, dml = (a.swapaxes(1, 2).copy() for a in (x, s, dm))
+    res = run_abi(idx, val, mix, xl, y, sl, dml, snd, rcv, Z, leading=True, idx_dtype=np.int32)
+    check_all(idx, val, mix, xl, y, sl, dml, snd, rcv, Z, res, leading=True, tag="leading int32")
+
+
+def test_both_forms_agree_and_the_column_form_still_runs(plans_off):
+    """With planning switched off the same calls run the LDS-column kernels: same results to rounding."""
+    rng = np.random.default_rng(55)
+    N, E, X, Y, Z, S, K, nnz = 9, 60, 9, 16, 35, 11, 96, 260
+    idx, val, mix = H.random_table(rng, nnz, X, Y, Z, S)
+    snd, rcv = H.random_graph(rng, N, E)
+    x, y, s, dm = H.random_operands(rng, N, E, X, Y, S, K, Z)
+    columns = run_abi(idx, val, mix, x, y, s, dm, snd, rcv, Z)
+    check_all(idx, val, mix, x, y, s, dm, snd, rcv, Z, columns, tag="columns")
+    _lib.load().e3j_amd_set_table_plans(1)
+    planned = run_abi(idx, val, mix, x, y, s, dm, snd, rcv, Z)
+    for a, b, name in zip(planned, columns, ("out", "dx", "dy", "ds")):
+        np.testing.assert_allclose(a, b, rtol=2e-5, atol=2e-5, err_msg=name)
+
+
+def test_sender_grouped_backward_gives_the_same_bits_every_time():
+    """The sender-grouped form owns dx and dy (no float atomics in global memory); the dy row of a
+    wave is summed in LDS in a fixed order."""
+    rng = np.random.default_rng(66)
+    N, E, X, Y, Z, S, K, nnz = 64, 2000, 16, 16, 99, 23, 128, 353
+    idx, val, mix = H.random_table(rng, nnz, X, Y, Z, S)
+    snd, rcv = H.random_graph(rng, N, E)
+    x, y, s, dm = H.random_operands(rng, N, E, X, Y, S, K, Z)
+    base = run_abi(idx, val, mix, x, y, s, dm, snd, rcv, Z, grouping="sender")
+    for _ in range(10):
+        again = run_abi(idx, val, mix, x, y, s, dm, snd, rcv, Z, grouping="sender")
+        for a, b in zip(base, again):
+            assert np.array_equal(a, b)
+
+
+def test_planned_kernels_at_120k_edges():
+    """cfg3 at an eighth of its size (4 000 atoms, 120k edges, K = 128, l <= 3): the planned
+    forward and backward against the column kernels' 9.1 ms and 24 ms on the same inputs."""
+    import time
+
+    w = W.config3(0.125).to("cuda")
+    idx, val, mix = w.table()
+    packed = H.pack_table(idx, val, mix)
+    coef_d = _dev(packed.view(np.uint8).reshape(-1))
+    lib = _lib.load()
+    p = _params(w.num_nodes, w.num_edges, len(packed), 16, 16, 99, 23, 128, 1, _lib.F32, packed.dtype.itemsize,
+                debug=0)
+    from e3j_amd.graph import csr_row_ptr
+    ptr = csr_row_ptr(w.receiver, w.num_nodes)
+    out = torch.empty_like(w.dm)
+    dx, dy, ds = torch.empty_like(w.x), torch.empty_like(w.y), torch.empty_like(w.s)
+    stream = torch.cuda.current_stream().cuda_stream
+
+    def fwd():
+        _lib.check(lib.e3j_amd_convolution_fwd(ctypes.byref(p), coef_d.data_ptr(), w.x.data_ptr(), w.y.data_ptr(),
+                                               w.s.data_ptr(), w.sender.data_ptr(), ptr.data_ptr(), None,
+                                               out.data_ptr(), stream))
+
+    def bwd():
+        _lib.check(lib.e3j_amd_convolution_bwd_receiver(
+            ctypes.byref(p), coef_d.data_ptr(), w.x.data_ptr(), w.y.data_ptr(), w.s.data_ptr(), w.dm.data_ptr(),
+            w.sender.data_ptr(), ptr.data_ptr(), None, dx.data_ptr(), dy.data_ptr(), ds.data_ptr(), stream))
+
+    times = {}
+    for name, fn in (("fwd", fwd), ("bwd", bwd)):
+        fn()
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        for _ in range(5):
+            fn()
+        torch.cuda.synchronize()
+        times[name] = (time.perf_counter() - t0) / 5 * 1e3
+    print("planned kernels, ms:", times)
+    assert times["fwd"] < 4.5 and times["bwd"] < 12.0, times
+    # and they agree with the unrolled kernels of the same table on the same inputs
+    from e3j_amd.ops import convolution
+    ref = convolution(w.module._packed_coef("float32"), w.x, w.y, w.s, w.sender, w.receiver, w.module.params)
+    torch.testing.assert_close(out, ref, rtol=2e-4, atol=2e-4)
