@@ -1,6 +1,6 @@
 // Table-driven convolution kernels over a plan of the table (float32; any table whose output
 // coordinates each use one scalar, up to 128 output coordinates, 16 x coordinates, 64 y
-// components).
+// components, 64 scalars, 2048 entries).
 //
 // The contraction out[i] += c * x[j] * y[k] * s[l] (lib/e3j_ops/cuda/convolution/fwd.cuh:88-153)
 // is regrouped per edge as out[i] += s[l(i)] * sum_j M[i][j] * x[j] with the channel-independent
@@ -20,7 +20,10 @@
 // forward's partial sums, dx[j] += M[i][j] * s[l(i)] * dm[i], and for dy the per-channel products
 // x[j] * s * dm[i] of a block of 64 cells are summed over the 64 channels with a transposing
 // butterfly (lane t ends with the total of cell t), multiplied with the cell's coefficients and
-// added into the wave's dy row in LDS.
+// added into the wave's dy row in LDS.  Per edge a wave first copies the edge's scalar rows into its
+// LDS strip (the loops read them by the slot's scalar, a number of the plan) and gathers the x row
+// into registers; the table part of the plan sits in the workgroup's LDS, the per-slot numbers in
+// two vector registers of every wave that are read lane by lane.
 //
 // Tables the plan cannot take (an output coordinate with two different scalars, sizes beyond the
 // limits) run the kernels of conv_generic.hip: eligibility is a flag in the plan that both
@@ -28,12 +31,6 @@
 
 #include "common.h"
 
-#ifndef E3J_ADDR_MODE
-#define E3J_ADDR_MODE 1
-#endif
-#ifndef E3J_LBYTES
-#define E3J_LBYTES 0
-#endif
 
 namespace e3j_amd {
 namespace {
@@ -55,12 +52,12 @@ struct PlanLayout {  // offsets in 32-bit words
     // cell (slot * 16 + j); cells: the non-empty cells packed as cell | first << 11 | count << 22;
     // pairs: (coefficient bits, k) of the entries, cell by cell; coef, k, t, cell_list: working arrays
     // of the builder; zero_l: scalars no entry uses
-    // slot_l8, slot_row8: the same as bytes, four slots to a word, 255 = none
-    int slot_row, slot_l, slot_l8, slot_row8, first, count, cell_list, cells, pairs, coef, k, t, zero_l, words;
+    // slot_lw: 64 * scalar of the slot (the word offset of its row in a wave's LDS copy of s), 0 if none
+    int slot_row, slot_l, slot_lw, first, count, cell_list, cells, pairs, coef, k, t, zero_l, words;
     PlanLayout(int num_coef, int num_scalars) {
         int at = kHeaderWords;
         auto take = [&](int n) { const int here = at; at += (n + 3) / 4 * 4; return here; };
-        slot_row = take(kSlots); slot_l = take(kSlots); slot_l8 = take(kSlots / 4); slot_row8 = take(kSlots / 4);
+        slot_row = take(kSlots); slot_l = take(kSlots); slot_lw = take(kSlots);
         first = take(kCells); count = take(kCells); cell_list = take(kCells); cells = take(kCells);
         pairs = take(2 * num_coef);
         coef = take(num_coef); k = take(num_coef); t = take(num_coef);
@@ -75,14 +72,6 @@ __host__ __device__ inline int table_words(int num_coef) {
     return ((cells + 1) / 2 * 2 + 2 * num_coef + 3) / 4 * 4;
 }
 
-__device__ __forceinline__ int wave_max_int(int v) {
-#pragma unroll
-    for (int off = kWave / 2; off > 0; off >>= 1) {
-        const int o = __shfl_xor(v, off, kWave);
-        v = o > v ? o : v;
-    }
-    return v;
-}
 
 template <typename Idx>
 __device__ inline void decode(const Coef4D<Idx, float> &c, int cols_ji, int &i, int &j, int &k, int &l) {
@@ -211,15 +200,9 @@ __global__ __launch_bounds__(kBuildThreads) void plan_build_kernel(
         if (cnt > kPlanMaxRun) eligible = 0;
         if (cnt > 0) atomicMax(&max_run, cnt);
     }
-    for (int w = tid; w < kSlots / 4; w += kBuildThreads) {
-        unsigned lw = 0, rw = 0;
-        for (int q = 0; q < 4; q++) {
-            const int l = plan[L.slot_l + 4 * w + q], row = plan[L.slot_row + 4 * w + q];
-            lw |= (unsigned)(l < 0 ? 255 : l) << (8 * q);
-            rw |= (unsigned)(row < 0 ? 255 : row) << (8 * q);
-        }
-        plan[L.slot_l8 + w] = (int)lw;
-        plan[L.slot_row8 + w] = (int)rw;
+    for (int q = tid; q < kSlots; q += kBuildThreads) {
+        const int l = plan[L.slot_l + q];
+        plan[L.slot_lw + q] = l < 0 ? 0 : l * kWave;
     }
     __syncthreads();
     // the forms the kernels stage in LDS
@@ -245,7 +228,6 @@ __device__ __forceinline__ void wave_lds_sync() {
 }
 
 typedef float f32x4 __attribute__((ext_vector_type(4)));
-constexpr int kAhead = 32;  // scalar rows of the next edge a wave holds in registers
 
 // The table part of the plan in LDS, shared by the waves of a workgroup: the packed cells, then
 // (coefficient, k) pairs.  Every thread of the workgroup calls this (it holds a barrier).
@@ -265,6 +247,7 @@ __device__ __forceinline__ void stage_table(const int32_t *__restrict__ plan, co
 }
 
 // M of one edge: lane q takes the cells q, q + 64, ... of the staged list; lane k of `yreg` holds y[k].
+// `most`: the longest entry list of a cell (lanes with shorter lists add zeros).
 template <int XG>
 __device__ __forceinline__ void build_edge_matrix(const int32_t *tab, int num_cells, int most, float yreg, float *M,
                                                   int lane) {
@@ -288,29 +271,55 @@ __device__ __forceinline__ void build_edge_matrix(const int32_t *tab, int num_ce
     }
 }
 
+// Per-slot numbers of the plan, kept by a wave in two vector registers (lane t of register k
+// holds the number of slot 64 k + t) and read as wave-uniform values with lane reads.
+struct SlotWords {
+    int lo, hi;
+    __device__ __forceinline__ SlotWords(const int32_t *__restrict__ words, int lane)
+        : lo(words[lane]), hi(words[kWave + lane]) {}
+    __device__ __forceinline__ int operator[](int slot) const {
+        return __builtin_amdgcn_readlane(slot < kWave ? lo : hi, slot % kWave);
+    }
+};
+
 __device__ __forceinline__ int next_live(const int32_t *__restrict__ other, int e, int e1, int num_nodes) {
     while (e < e1 && (unsigned)other[e] >= (unsigned)num_nodes) e++;  // padding edges are stepped over
     return e;
 }
 
-// A row of an operand: `base` is wave-uniform, the lanes differ by a 32-bit offset, so that the
-// load takes a scalar base and one offset register.
-__device__ __forceinline__ const float *row_at(const float *base, int64_t row_stride, int row) {
-    return base + (int64_t)row * row_stride;
-}
-// element `lane_off + row * stride` behind a wave-uniform base: one scalar base, one 32-bit offset
-__device__ __forceinline__ float load_row(const float *base, unsigned lane_off, unsigned stride, int row) {
-#if E3J_ADDR_MODE == 0
-    return (base + lane_off)[(int64_t)row * stride];   // per-lane pointer, 64-bit row offset
-#elif E3J_ADDR_MODE == 1
-    return (base + (int64_t)row * stride)[lane_off];   // scalar row pointer, lane offset
-#else
-    return base[lane_off + (unsigned)row * stride];
-#endif
-}
-// slot byte q of a packed word array held in scalar registers
-#define E3J_SLOT_BYTE(words, slot) (((words)[(slot) / 4] >> (8 * ((slot) % 4))) & 255u)
+// Rows of an operand behind a wave-uniform base: the lanes keep one 32-bit byte offset that
+// moves from row to row by the row stride, so that a load takes a scalar base, one offset
+// register and one vector addition.
+struct RowCursor {
+    const char *base;   // wave-uniform
+    unsigned at;        // byte offset of the lane's element in the current row
+    unsigned step;      // bytes between rows
+    __device__ __forceinline__ RowCursor(const float *row0, unsigned lane_elems, unsigned stride_elems)
+        : base(reinterpret_cast<const char *>(row0)), at(4u * lane_elems), step(4u * stride_elems) {}
+    __device__ __forceinline__ float next() {
+        const float v = *reinterpret_cast<const float *>(base + at);
+        at += step;
+        return v;
+    }
+    __device__ __forceinline__ float row(unsigned r) const {  // r wave-uniform
+        return *reinterpret_cast<const float *>(base + (at + r * step));
+    }
+};
 
+// The scalar rows of one edge into the wave's LDS copy, eight loads in flight.
+__device__ __forceinline__ void stage_scalars(const float *srow0, unsigned soff, unsigned sdim, int S, float *sbuf,
+                                              int lane) {
+    RowCursor cur(srow0, soff, sdim);
+    for (int t0 = 0; t0 < S; t0 += 8) {
+        float v[8];
+#pragma unroll
+        for (int t = 0; t < 8; t++) v[t] = cur.row((unsigned)(t0 + t < S ? t0 + t : S - 1));  // (clamped: straight-line)
+#pragma unroll
+        for (int t = 0; t < 8; t++) sbuf[(t0 + t < S ? t0 + t : S - 1) * kWave + lane] = v[t];
+    }
+}
+
+// Forward: a wave takes (row, 64 channels) and holds NB * 16 accumulators.
 template <int NB, int XG>
 __global__ __launch_bounds__(256, 2) void planned_fwd_kernel(
     const int32_t *__restrict__ plan, PlanLayout L, const float *__restrict__ x, RowLayout lx,
@@ -321,9 +330,8 @@ __global__ __launch_bounds__(256, 2) void planned_fwd_kernel(
     extern __shared__ __align__(16) float planned_lds[];
     if (plan[kEligible] == 0) return;  // (the whole grid) the table-driven kernel without a plan runs instead
     constexpr int kStrip = NB * 16 * XG * 4;
-    const int lane = threadIdx.x, wave = __builtin_amdgcn_readfirstlane((int)threadIdx.y);  // (wave-uniform: in scalar registers)
+    const int lane = threadIdx.x, wave = __builtin_amdgcn_readfirstlane((int)threadIdx.y);
     const int num_cells = plan[kNumCells];
-    const unsigned chunk_mask = (unsigned)plan[kChunkMask];
     const int max_run = plan[kMaxRun];
     int32_t *tab = reinterpret_cast<int32_t *>(planned_lds);
     float *M = planned_lds + table_words(num_coef) + wave * (kStrip + S * kWave);
@@ -338,45 +346,29 @@ __global__ __launch_bounds__(256, 2) void planned_fwd_kernel(
     const bool active = c < channels;
     const int cr = active ? c : channels - 1;  // channel whose rows an idle lane reads
     const unsigned xoff = (unsigned)cr * (unsigned)lx.chan, soff = (unsigned)cr * (unsigned)ls.chan;
-    unsigned lbytes[NB * 4];  // the scalar of every slot, a byte each
-#pragma unroll
-    for (int w = 0; w < NB * 4; w++) lbytes[w] = (unsigned)plan[L.slot_l8 + w];
-
+    const unsigned chunk_mask = (unsigned)plan[kChunkMask];
+    const SlotWords slot_lw(plan + L.slot_lw, lane);
     float acc[NB * 16];
 #pragma unroll
     for (int t = 0; t < NB * 16; t++) acc[t] = 0.f;
 
     const int e1 = row_ptr[r + 1];
-    int e = next_live(other, row_ptr[r], e1, num_nodes);
-    // operands of the edge after the one in work, loaded while that one is computed
-    float yn = 0.f, xn[XG * 4], sn[kAhead];
-    int64_t een = 0;
-    auto issue = [&](int at) {
-        const int snd = other[at];
-        een = perm ? (int64_t)perm[at] : (int64_t)at;
-        yn = lane < num_y ? y[een * num_y + lane] : 0.f;
-        const float *xbase = x + (int64_t)snd * lx.row;
-#pragma unroll
-        for (int j = 0; j < XG * 4; j++) xn[j] = load_row(xbase, xoff, (unsigned)lx.dim, j < X ? j : X - 1);  // (clamped, not skipped: straight-line loads)
-        const float *sbase = s + een * ls.row;
-#pragma unroll
-        for (int t = 0; t < kAhead; t++) sn[t] = load_row(sbase, soff, (unsigned)ls.dim, t < S ? t : S - 1);
-    };
-    if (e < e1) issue(e);
-    while (e < e1) {
-        const float ycur = yn;
-        const int64_t ee = een;
-        float xv[XG * 4];
-#pragma unroll
-        for (int j = 0; j < XG * 4; j++) xv[j] = j < X ? xn[j] : 0.f;
+    for (int e = next_live(other, row_ptr[r], e1, num_nodes); e < e1; e = next_live(other, e + 1, e1, num_nodes)) {
+        const int snd = other[e];
+        const int64_t ee = perm ? (int64_t)perm[e] : (int64_t)e;
+        const float yreg = lane < num_y ? y[ee * num_y + lane] : 0.f;
         wave_lds_sync();  // the reads of the edge before are behind the writes below
+        stage_scalars(s + ee * ls.row, soff, (unsigned)ls.dim, S, sbuf, lane);
+        float xv[XG * 4];
+        {
+            const RowCursor xc(x + (int64_t)snd * lx.row, xoff, (unsigned)lx.dim);
 #pragma unroll
-        for (int t = 0; t < kAhead; t++) sbuf[(t < S ? t : S - 1) * kWave + lane] = sn[t];
-        for (int t = kAhead; t < S; t++)  // (rows past the ones held ahead: read now)
-            sbuf[t * kWave + lane] = load_row(s + ee * ls.row, soff, (unsigned)ls.dim, t);
-        const int en = next_live(other, e + 1, e1, num_nodes);
-        if (en < e1) issue(en);
-        build_edge_matrix<XG>(tab, num_cells, max_run, ycur, M, lane);
+            for (int j = 0; j < XG * 4; j++) {
+                xv[j] = xc.row((unsigned)(j < X ? j : X - 1));
+                if (j >= X) xv[j] = 0.f;
+            }
+        }
+        build_edge_matrix<XG>(tab, num_cells, max_run, yreg, M, lane);
         wave_lds_sync();
 #pragma unroll
         for (int b = 0; b < NB; b++) {
@@ -384,13 +376,7 @@ __global__ __launch_bounds__(256, 2) void planned_fwd_kernel(
             float sv[16], T[16];
 #pragma unroll
             for (int u = 0; u < 16; u++) {
-                // (a slot without entries reads row 0 of s; its output row is written as zero below)
-#if E3J_LBYTES
-                const unsigned l = E3J_SLOT_BYTE(lbytes, b * 16 + u);
-#else
-                const unsigned l = (unsigned)plan[L.slot_l + b * 16 + u] & 255u;
-#endif
-                sv[u] = sbuf[(l == 255u ? 0u : l) * kWave + lane];
+                sv[u] = sbuf[slot_lw[b * 16 + u] + lane];
                 T[u] = 0.f;
             }
 #pragma unroll
@@ -408,37 +394,52 @@ __global__ __launch_bounds__(256, 2) void planned_fwd_kernel(
 #pragma unroll
             for (int u = 0; u < 16; u++) acc[b * 16 + u] = __builtin_fmaf(sv[u], T[u], acc[b * 16 + u]);
         }
-        e = en;
     }
-    if (active) {
+    {
+        const SlotWords slot_row(plan + L.slot_row, lane), slot_l(plan + L.slot_l, lane);
         float *obase = out + (int64_t)r * lo.row;
         const unsigned ooff = (unsigned)c * (unsigned)lo.chan;
 #pragma unroll
         for (int t = 0; t < NB * 16; t++) {
-            const unsigned row = ((unsigned)plan[L.slot_row8 + t / 4] >> (8 * (t % 4))) & 255u;
-            const unsigned l = E3J_SLOT_BYTE(lbytes, t);
-            if (row != 255u) (obase + (int64_t)row * lo.dim)[ooff] = l == 255u ? 0.f : acc[t];
+            const int row = slot_row[t];
+            // (a slot whose output coordinate no entry touches has read row 0 of s: it stores zero)
+            if (row >= 0 && active) obase[ooff + (unsigned)row * (unsigned)lo.dim] = slot_l[t] < 0 ? 0.f : acc[t];
         }
     }
 }
 
-// v[t] (t < 32) summed over the 64 lanes, the total of v[t] left in lanes t and t + 32.  Five
-// halving steps inside each half of the wave (lanes whose bit N is clear keep the lower half of
-// the values and hand the upper half to their partner), then the two halves are added.
-template <int N>  // N pairs (p, p + N) are left; partner lanes differ in bit N
+// The channel sums of 64 per-lane products, left one to a lane: v[t] (t < 32) of one wave is summed
+// over the lanes of each half of the wave with five halving steps (lanes whose bit N is clear keep
+// the lower half of the values and take their partner's partial sums of them; the partners are a
+// row swap for N = 16 and DPP lane permutations inside rows of 16 below that), which leaves the
+// partial sum of v[t % 32] over the lane's half in lane t; two such arrays are then finished with
+// one swap of wave halves, lanes 0..31 getting the totals of the first, 32..63 of the second.
+template <int N, int CTRL>  // N pairs (p, p + N) are left; partner lanes differ in bit N
 __device__ __forceinline__ void transpose_sum_step(float (&v)[32], int lane) {
     const bool upper = (lane & N) != 0;
 #pragma unroll
     for (int p = 0; p < N; p++) {
         const float keep = upper ? v[p + N] : v[p];
         const float send = upper ? v[p] : v[p + N];
-        v[p] = keep + __shfl_xor(send, N, kWave);
+        v[p] = keep + __int_as_float(__builtin_amdgcn_update_dpp(0, __float_as_int(send), CTRL, 0xf, 0xf, true));
     }
 }
-__device__ __forceinline__ float transpose_sum(float (&v)[32], int lane) {
-    transpose_sum_step<16>(v, lane); transpose_sum_step<8>(v, lane); transpose_sum_step<4>(v, lane);
-    transpose_sum_step<2>(v, lane); transpose_sum_step<1>(v, lane);
-    return v[0] + __shfl_xor(v[0], 32, kWave);
+__device__ __forceinline__ float transpose_sum_half(float (&v)[32], int lane) {
+#pragma unroll
+    for (int p = 0; p < 16; p++) {  // rows 1 and 3 of v[p] change places with rows 0 and 2 of v[p + 16]
+        const auto r = __builtin_amdgcn_permlane16_swap(__float_as_uint(v[p]), __float_as_uint(v[p + 16]), false, false);
+        v[p] = __uint_as_float(r[0]) + __uint_as_float(r[1]);
+    }
+    transpose_sum_step<8, 0x140>(v, lane);  // row_mirror: lane ^ 15
+    transpose_sum_step<4, 0x141>(v, lane);  // row_half_mirror: lane ^ 7
+    transpose_sum_step<2, 0x4E>(v, lane);   // quad_perm [2, 3, 0, 1]: lane ^ 2
+    transpose_sum_step<1, 0xB1>(v, lane);   // quad_perm [1, 0, 3, 2]: lane ^ 1
+    return v[0];
+}
+// lanes 0..31: first.lower + first.upper, lanes 32..63: second.lower + second.upper
+__device__ __forceinline__ float join_halves(float first, float second) {
+    const auto r = __builtin_amdgcn_permlane32_swap(__float_as_uint(first), __float_as_uint(second), false, false);
+    return __uint_as_float(r[0]) + __uint_as_float(r[1]);
 }
 
 enum DyMode { kDyStore = 0, kDyAdd = 1, kDyAtomic = 2 };
@@ -455,7 +456,7 @@ __global__ __launch_bounds__(256, 2) void planned_bwd_kernel(
     extern __shared__ __align__(16) float planned_lds[];
     if (plan[kEligible] == 0) return;
     constexpr int kStrip = NB * 16 * XG * 4;
-    const int lane = threadIdx.x, wave = __builtin_amdgcn_readfirstlane((int)threadIdx.y);  // (wave-uniform: in scalar registers)
+    const int lane = threadIdx.x, wave = __builtin_amdgcn_readfirstlane((int)threadIdx.y);
     const int num_cells = plan[kNumCells];
     const unsigned chunk_mask = (unsigned)plan[kChunkMask];
     const int max_run = plan[kMaxRun];
@@ -478,6 +479,7 @@ __global__ __launch_bounds__(256, 2) void planned_bwd_kernel(
     const int chunk0 = group_is_receiver ? (int)(item % nchunks) : 0;
     const int chunk1 = group_is_receiver ? chunk0 + 1 : nchunks;
     const int e0 = row_ptr[g], e1 = row_ptr[g + 1];
+    const SlotWords slot_l(plan + L.slot_l, lane), slot_row(plan + L.slot_row, lane);
 
     for (int chunk = chunk0; chunk < chunk1; chunk++) {
         const int c = chunk * kWave + lane;
@@ -490,44 +492,29 @@ __global__ __launch_bounds__(256, 2) void planned_bwd_kernel(
         float dxa[XG * 4];
 #pragma unroll
         for (int j = 0; j < XG * 4; j++) dxa[j] = 0.f;
-        int e = next_live(other, e0, e1, num_nodes);
-        float yn = 0.f, xn[XG * 4], sn[kAhead];
-        int64_t een = 0;
-        int on = 0;
-        auto issue = [&](int at) {
-            on = other[at];
-            een = perm ? (int64_t)perm[at] : (int64_t)at;
-            yn = lane < num_y ? y[een * num_y + lane] : 0.f;
-            const float *xbase = x + (int64_t)(group_is_receiver ? on : g) * lx.row;
-#pragma unroll
-            for (int j = 0; j < XG * 4; j++) xn[j] = load_row(xbase, xoff, (unsigned)lx.dim, j < X ? j : X - 1);  // (clamped, not skipped: straight-line loads)
-            const float *sbase = s + een * ls.row;
-#pragma unroll
-            for (int t = 0; t < kAhead; t++) sn[t] = load_row(sbase, soff, (unsigned)ls.dim, t < S ? t : S - 1);
-        };
-        if (e < e1) issue(e);
-        while (e < e1) {
-            const float ycur = yn;
-            const int64_t ee = een;
-            const int o = on;
+        for (int e = next_live(other, e0, e1, num_nodes); e < e1; e = next_live(other, e + 1, e1, num_nodes)) {
+            const int o = other[e];
+            const int64_t ee = perm ? (int64_t)perm[e] : (int64_t)e;
             const int xnode = group_is_receiver ? o : g;
             const int znode = group_is_receiver ? g : o;
+            const float yreg = lane < num_y ? y[ee * num_y + lane] : 0.f;
+            wave_lds_sync();
+            stage_scalars(s + ee * ls.row, soff, (unsigned)ls.dim, S, sbuf, lane);
             float xv[XG * 4];
+            {
+                const RowCursor xc(x + (int64_t)xnode * lx.row, xoff, (unsigned)lx.dim);
 #pragma unroll
-            for (int j = 0; j < XG * 4; j++) xv[j] = (j < X && active) ? xn[j] : 0.f;  // (idle lanes add nothing to dy)
+                for (int j = 0; j < XG * 4; j++) {
+                    xv[j] = xc.row((unsigned)(j < X ? j : X - 1));
+                    if (j >= X || !active) xv[j] = 0.f;  // (idle lanes add nothing to dy)
+                }
+            }
+            build_edge_matrix<XG>(tab, num_cells, max_run, yreg, M, lane);
             wave_lds_sync();
-#pragma unroll
-            for (int t = 0; t < kAhead; t++) sbuf[(t < S ? t : S - 1) * kWave + lane] = sn[t];
-            for (int t = kAhead; t < S; t++)
-                sbuf[t * kWave + lane] = load_row(s + ee * ls.row, soff, (unsigned)ls.dim, t);
-            const int en = next_live(other, e + 1, e1, num_nodes);
-            if (en < e1) issue(en);
-            build_edge_matrix<XG>(tab, num_cells, max_run, ycur, M, lane);
-            wave_lds_sync();
-            const float *zbase = dm + (int64_t)znode * lo.row;
-            float *dsbase = ds + ee * ls.row;
-            const unsigned dsoff = (unsigned)c * (unsigned)ls.chan;
-            unsigned cur_l = 255u;
+            const RowCursor zc(dm + (int64_t)znode * lo.row, zoff, (unsigned)lo.dim);
+            char *dsbytes = reinterpret_cast<char *>(ds + ee * ls.row);
+            const unsigned dsat = 4u * (unsigned)c * (unsigned)ls.chan, dsstep = 4u * (unsigned)ls.dim;
+            int cur_l = -1;
             float dsa = 0.f;
 #pragma unroll
             for (int b = 0; b < NB; b++) {
@@ -535,12 +522,11 @@ __global__ __launch_bounds__(256, 2) void planned_bwd_kernel(
                 float sd[16], dz[16], T[16];
 #pragma unroll
                 for (int u = 0; u < 16; u++) {
-                    const unsigned l = (unsigned)plan[L.slot_l + b * 16 + u] & 255u;  // (255: none)
-                    const unsigned row = (unsigned)plan[L.slot_row + b * 16 + u] & 255u;
-                    const float sv = sbuf[(l == 255u ? 0u : l) * kWave + lane];
-                    dz[u] = load_row(zbase, zoff, (unsigned)lo.dim, row == 255u ? 0 : (int)row);
-                    if (l == 255u || !active) dz[u] = 0.f;  // (wave-uniform or per lane: a select)
-                    sd[u] = l == 255u ? 0.f : sv * dz[u];
+                    const int l = slot_l[b * 16 + u], row = slot_row[b * 16 + u];  // (-1: none)
+                    const float sv = sbuf[(l < 0 ? 0 : l) * kWave + lane];
+                    dz[u] = zc.row((unsigned)(row < 0 ? 0 : row));
+                    if (l < 0) dz[u] = 0.f;
+                    sd[u] = sv * dz[u];
                     T[u] = 0.f;
                 }
 #pragma unroll
@@ -548,7 +534,7 @@ __global__ __launch_bounds__(256, 2) void planned_bwd_kernel(
                     if (!((chunk_mask >> (b * XG + gx)) & 1u)) continue;
                     // lane t ends with the channel sum of cell (slot 16 b + t / 4, x coordinate 4 gx + t % 4):
                     // the slots in two halves of eight, the first for lanes 0..31, the second for the rest
-                    float total = 0.f;
+                    float part[2];
 #pragma unroll
                     for (int half = 0; half < 2; half++) {
                         float G[32];
@@ -567,9 +553,9 @@ __global__ __launch_bounds__(256, 2) void planned_bwd_kernel(
 #pragma unroll
                             for (int jj = 0; jj < 4; jj++) G[uu * 4 + jj] = sd[u] * xv[4 * gx + jj];
                         }
-                        const float both = transpose_sum(G, lane);
-                        if ((lane >> 5) == half) total = both;
+                        part[half] = transpose_sum_half(G, lane);
                     }
+                    const float total = join_halves(part[0], part[1]);
                     const int where = dense[(b * 16 + lane / 4) * kPlanX + 4 * gx + lane % 4];
                     const int first = where & 2047, cnt = where >> 11;
                     for (int rr = 0; rr < cnt; rr++)
@@ -579,18 +565,20 @@ __global__ __launch_bounds__(256, 2) void planned_bwd_kernel(
                 // ds: the slots of one scalar are adjacent; a scalar's sum is stored when the next begins
 #pragma unroll
                 for (int u = 0; u < 16; u++) {
-                    const unsigned l = (unsigned)plan[L.slot_l + b * 16 + u] & 255u;
+                    const int l = slot_l[b * 16 + u];
                     if (l != cur_l) {
-                        if (cur_l != 255u && active) (dsbase + (int64_t)cur_l * ls.dim)[dsoff] = dsa;
+                        if (cur_l >= 0 && active)
+                            *reinterpret_cast<float *>(dsbytes + (dsat + (unsigned)cur_l * dsstep)) = dsa;
                         cur_l = l;
                         dsa = 0.f;
                     }
                     dsa = __builtin_fmaf(dz[u], T[u], dsa);
                 }
             }
-            if (cur_l != 255u && active) (dsbase + (int64_t)cur_l * ls.dim)[dsoff] = dsa;
+            if (cur_l >= 0 && active) *reinterpret_cast<float *>(dsbytes + (dsat + (unsigned)cur_l * dsstep)) = dsa;
             if (active)
-                for (int z = 0; z < num_zero_l; z++) (dsbase + (int64_t)plan[L.zero_l + z] * ls.dim)[dsoff] = 0.f;
+                for (int z = 0; z < num_zero_l; z++)
+                    *reinterpret_cast<float *>(dsbytes + (dsat + (unsigned)plan[L.zero_l + z] * dsstep)) = 0.f;
             wave_lds_sync();
             if (lane < num_y) {
                 const float v = dyl[lane];
@@ -602,21 +590,22 @@ __global__ __launch_bounds__(256, 2) void planned_bwd_kernel(
             }
             if (group_is_receiver) {
                 if (active) {
-                    float *dxbase = dx + (int64_t)xnode * lx.row;
+                    char *dxbytes = reinterpret_cast<char *>(dx + (int64_t)xnode * lx.row);
 #pragma unroll
                     for (int j = 0; j < XG * 4; j++)
-                        if (j < X) unsafeAtomicAdd(dxbase + (int64_t)j * lx.dim + xoff, dxa[j]);
+                        if (j < X)
+                            unsafeAtomicAdd(reinterpret_cast<float *>(dxbytes + 4u * (xoff + (unsigned)j * (unsigned)lx.dim)),
+                                            dxa[j]);
                 }
 #pragma unroll
                 for (int j = 0; j < XG * 4; j++) dxa[j] = 0.f;
             }
-            e = en;
         }
         if (!group_is_receiver && active) {
             float *dxbase = dx + (int64_t)g * lx.row;
 #pragma unroll
             for (int j = 0; j < XG * 4; j++)
-                if (j < X) (dxbase + (int64_t)j * lx.dim)[xoff] = dxa[j];
+                if (j < X) dxbase[xoff + (unsigned)j * (unsigned)lx.dim] = dxa[j];
         }
     }
 }
@@ -628,11 +617,7 @@ typedef void (*BwdKernel)(const int32_t *, PlanLayout, const float *, RowLayout,
                           RowLayout, const float *, RowLayout, const int32_t *, const int32_t *, const int32_t *,
                           const int32_t *, float *, float *, float *, int, int, int, int, int, int, int);
 
-#ifdef E3J_PLANNED_ONE_SHAPE  // (a compile-time experiment: only the 7 x 4 shape)
-#define E3J_ROW(K, NB) {K<7, 4>, K<7, 4>, K<7, 4>, K<7, 4>}
-#else
 #define E3J_ROW(K, NB) {K<NB, 1>, K<NB, 2>, K<NB, 3>, K<NB, 4>}
-#endif
 #define E3J_TABLE(K) {E3J_ROW(K, 1), E3J_ROW(K, 2), E3J_ROW(K, 3), E3J_ROW(K, 4), \
                       E3J_ROW(K, 5), E3J_ROW(K, 6), E3J_ROW(K, 7), E3J_ROW(K, 8)}
 const FwdKernel kFwd[8][4] = E3J_TABLE(planned_fwd_kernel);
