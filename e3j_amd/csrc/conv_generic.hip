@@ -561,13 +561,20 @@ int launch_zero_padding(const e3j_amd_conv_params &p, const int32_t *other, cons
 
 // The plan of a table the planned kernels can take (conv_planned.hip), in memory of the stream's
 // pool for the length of the call; none when the sizes are outside the plan's limits, when
-// planning is switched off, or when the pool gives nothing (a stream under capture).
+// planning is switched off, when the stream is being captured into a graph (the call then
+// allocates nothing) or when the pool gives nothing.
 struct PlanScratch {
     int32_t *plan = nullptr;
     hipStream_t stream;
     int rc = E3J_AMD_OK;
     PlanScratch(const e3j_amd_conv_params &p, const void *coef, bool cols_ji, hipStream_t st) : stream(st) {
         if (!plan_takes(p) || !table_plans().load(std::memory_order_relaxed)) return;
+        hipStreamCaptureStatus capture = hipStreamCaptureStatusNone;
+        if (hipStreamIsCapturing(stream, &capture) != hipSuccess) {
+            (void)hipGetLastError();
+            return;
+        }
+        if (capture != hipStreamCaptureStatusNone) return;
         void *mem = nullptr;
         if (hipMallocAsync(&mem, plan_bytes(p), stream) != hipSuccess) {
             (void)hipGetLastError();

@@ -240,8 +240,8 @@ void e3j_amd_set_launch_variant(int32_t fwd_variant, int32_t bwd_variant);
  * kernels that keep x and the accumulators in registers; any other table, float64 and float16
  * run the kernels that index LDS columns by the table's coordinates.  Whether a table fits is
  * decided on the device, without a read-back.  on = 0 switches the planned form off for later
- * calls (process-wide, atomic; initial value from E3J_AMD_TABLE_PLANS, default 1); a stream under
- * graph capture, where the pool gives no memory, gets the LDS-column kernels as well.  Results
+ * calls (process-wide, atomic; initial value from E3J_AMD_TABLE_PLANS, default 1); a call on a
+ * stream that is being captured into a graph allocates nothing and runs the LDS-column kernels.  Results
  * agree to rounding (the planned form sums per output coordinate in a different order).
  * No counterpart in the reference, which has one table-driven kernel
  * (lib/e3j_ops/cuda/convolution/fwd.cuh:88-153). */
