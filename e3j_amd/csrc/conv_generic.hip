@@ -401,6 +401,11 @@ int run_bwd(const e3j_amd_conv_params &p, bool group_is_receiver, const void *co
             const int32_t *row_ptr, const int32_t *perm, void *dx, void *dy, void *ds,
             hipStream_t stream, bool cols_ji, const int32_t *plan) {
     const int nchunks = (p.channels + kWave - 1) / kWave;
+    if (std::is_same<Val, half_t>::value && group_is_receiver)
+        // no float atomics on half values: rows must own their dx (sender-grouped)
+        return set_error(E3J_AMD_UNIMPLEMENTED,
+                         "convolution_bwd: float16 runs the sender-grouped backward only (dx by "
+                         "float atomics has no half-precision form)");
     const size_t per_wave =
         (size_t)(p.num_out + 2 * p.num_x + 2 * p.num_scalars + p.num_y) * kWave * sizeof(Val);
     if (per_wave > kMaxLds)
@@ -449,11 +454,6 @@ int run_bwd(const e3j_amd_conv_params &p, bool group_is_receiver, const void *co
                            p.num_scalars, p.num_out, nchunks, cols_ji ? 1 : 0, plan);             \
     } while (0)
     if constexpr (std::is_same<Val, half_t>::value) {
-        // no float atomics on half values: rows must own their dx (sender-grouped)
-        if (group_is_receiver)
-            return set_error(E3J_AMD_UNIMPLEMENTED,
-                             "convolution_bwd: float16 runs the sender-grouped backward only (dx by "
-                             "float atomics has no half-precision form)");
         E3J_LAUNCH_BWD(false);
     } else {
         if (group_is_receiver) E3J_LAUNCH_BWD(true);

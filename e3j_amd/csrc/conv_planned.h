@@ -1,0 +1,734 @@
+// Table-driven convolution kernels over a plan of the table (float32; any table whose output
+// coordinates each use one scalar, up to 128 output coordinates, 16 x coordinates, 64 y
+// components, 64 scalars, 2048 entries).
+//
+// The contraction out[i] += c * x[j] * y[k] * s[l] (lib/e3j_ops/cuda/convolution/fwd.cuh:88-153)
+// is regrouped per edge as out[i] += s[l(i)] * sum_j M[i][j] * x[j] with the channel-independent
+// matrix M[i][j] = sum_k c_ijk * y[k].  A wave builds M once per edge in its strip of LDS (the
+// lanes share the table's non-empty cells), and then every lane (one channel) runs loops over
+// i and j whose bounds are compile-time numbers, so that x, the accumulators and the partial
+// sums sit in registers under constant indices; M is read as wave-uniform 16-byte LDS
+// broadcasts.  What depends on the table is data: the plan, built on the device by one
+// workgroup per call (no read-back, no compiler at run time):
+//   * the output coordinates in the order the loops visit them ("slots": sorted by the x
+//     coordinates their path touches, then by scalar, so that rows of one scalar are adjacent
+//     and blocks of 16 slots touch few groups of 4 x coordinates),
+//   * a bit per (block of 16 slots, group of 4 x coordinates) that has a coefficient at all: the
+//     loops skip the others with a wave-uniform branch,
+//   * the non-empty cells (slot, j) with their (coefficient, k) lists in table order.
+// The backward pass (lib/e3j_ops/cuda/convolution/bwd.cuh:116-321) uses the same M: ds from the
+// forward's partial sums, dx[j] += M[i][j] * s[l(i)] * dm[i], and for dy the per-channel products
+// x[j] * s * dm[i] of a block of 64 cells are summed over the 64 channels with a transposing
+// butterfly (lane t ends with the total of cell t), multiplied with the cell's coefficients and
+// added into the wave's dy row in LDS.  Per edge a wave first copies the edge's scalar rows into its
+// LDS strip (the loops read them by the slot's scalar, a number of the plan) and gathers the x row
+// into registers; the table part of the plan sits in the workgroup's LDS, the per-slot numbers in
+// two vector registers of every wave that are read lane by lane.
+//
+// Tables the plan cannot take (an output coordinate with two different scalars, sizes beyond the
+// limits) run the kernels of conv_generic.hip: eligibility is a flag in the plan that both
+// kernels read, so the host never waits for the device.
+
+#ifndef E3J_AMD_CSRC_CONV_PLANNED_H_
+#define E3J_AMD_CSRC_CONV_PLANNED_H_
+
+#include <type_traits>
+
+#include "common.h"
+
+
+namespace e3j_amd {
+namespace {
+
+constexpr int kSlots = 128;     // output coordinates a plan holds (8 blocks of 16)
+constexpr int kPlanX = 16;      // x coordinates (4 groups of 4)
+constexpr int kCells = kSlots * kPlanX;
+constexpr int kPlanMaxY = 64;
+constexpr int kPlanMaxS = 64;       // scalars (their rows of one edge sit in the wave's LDS)
+constexpr int kPlanMaxCoef = 2048;  // entries (the table sits in the workgroup's LDS; 11-bit fields)
+constexpr int kPlanMaxRun = 255;    // entries of one cell
+constexpr int kBuildThreads = 256;
+
+// header words
+enum { kEligible = 0, kNumCells = 1, kChunkMask = 2, kNumZeroL = 3, kMaxRun = 4, kHeaderWords = 8 };
+
+struct PlanLayout {  // offsets in 32-bit words
+    // slot_row, slot_l: output coordinate and scalar of a slot; first, count: the entries of a dense
+    // cell (slot * 16 + j); cells: the non-empty cells packed as cell | first << 11 | count << 22;
+    // pairs: (coefficient bits, k) of the entries, cell by cell; coef, k, t, cell_list: working arrays
+    // of the builder; zero_l: scalars no entry uses
+    // slot_lw: 64 * scalar of the slot (the word offset of its row in a wave's LDS copy of s), 0 if none
+    int slot_row, slot_l, slot_lw, first, count, cell_list, cells, pairs, coef, k, t, zero_l, words;
+    PlanLayout(int num_coef, int num_scalars) {
+        int at = kHeaderWords;
+        auto take = [&](int n) { const int here = at; at += (n + 3) / 4 * 4; return here; };
+        slot_row = take(kSlots); slot_l = take(kSlots); slot_lw = take(kSlots);
+        first = take(kCells); count = take(kCells); cell_list = take(kCells); cells = take(kCells);
+        pairs = take(2 * num_coef);
+        coef = take(num_coef); k = take(num_coef); t = take(num_coef);
+        zero_l = take(num_scalars);
+        words = at;
+    }
+};
+
+// words of LDS the staged table takes (cells, then pairs from an even word on)
+__host__ __device__ inline int table_words(int num_coef) {
+    const int cells = num_coef < kCells ? num_coef : kCells;
+    return ((cells + 1) / 2 * 2 + 2 * num_coef + 3) / 4 * 4;
+}
+
+
+template <typename Idx, typename Val>
+__device__ inline void decode(const Coef4D<Idx, Val> &c, int cols_ji, int &i, int &j, int &k, int &l) {
+    i = (int)c.i; j = (int)c.j; k = (int)c.k; l = (int)c.l;
+    if (cols_ji) { const int t = i; i = j; j = t; }
+}
+
+// One workgroup turns the table into the plan.
+template <typename Idx, typename Val>
+__global__ __launch_bounds__(kBuildThreads) void plan_build_kernel(
+    const Coef4D<Idx, Val> *__restrict__ coef, int num_coef, int X, int Y, int Z, int S, int xg, int cols_ji,
+    int32_t *__restrict__ plan, PlanLayout L) {
+    __shared__ int lmin[kSlots], lmax[kSlots], support[kSlots], slot_of_row[kSlots];
+    __shared__ int path_support[kPlanMaxS], referenced[kPlanMaxS];
+    __shared__ int eligible, chunk_mask, num_cells, num_zero_l, max_run;
+    __shared__ int scan[kBuildThreads];
+    const int tid = threadIdx.x;
+    if (tid == 0) { eligible = 1; chunk_mask = 0; num_cells = 0; num_zero_l = 0; max_run = 0; }
+    for (int i = tid; i < kSlots; i += kBuildThreads) { lmin[i] = 0x7fffffff; lmax[i] = -1; support[i] = 0; }
+    for (int l = tid; l < S; l += kBuildThreads) { path_support[l] = 0; referenced[l] = 0; }
+    for (int c = tid; c < kCells; c += kBuildThreads) plan[L.count + c] = 0;
+    __syncthreads();
+    // rows: the scalars and the groups of x coordinates their entries use
+    for (int n = tid; n < num_coef; n += kBuildThreads) {
+        int i, j, k, l;
+        decode(coef[n], cols_ji, i, j, k, l);
+        if ((unsigned)i >= (unsigned)Z || (unsigned)j >= (unsigned)X || (unsigned)k >= (unsigned)Y ||
+            (unsigned)l >= (unsigned)S) { eligible = 0; continue; }
+        atomicMin(&lmin[i], l); atomicMax(&lmax[i], l); atomicOr(&support[i], 1 << (j >> 2));
+    }
+    __syncthreads();
+    for (int i = tid; i < Z; i += kBuildThreads) {
+        if (lmax[i] < 0) continue;
+        if (lmin[i] != lmax[i]) { eligible = 0; continue; }
+        atomicOr(&path_support[lmax[i]], support[i]);
+        referenced[lmax[i]] = 1;
+    }
+    __syncthreads();
+    // slots: rows sorted by (support of the row's scalar, scalar, row); rows without entries last
+    auto key = [&](int i) {
+        return lmax[i] < 0 ? (1 << 30) | i : (path_support[lmax[i]] << 24) | (lmax[i] << 8) | i;
+    };
+    for (int i = tid; i < kSlots; i += kBuildThreads) { plan[L.slot_row + i] = -1; plan[L.slot_l + i] = -1; }
+    __syncthreads();
+    for (int i = tid; i < Z; i += kBuildThreads) {
+        const int mine = key(i);
+        int rank = 0;
+        for (int o = 0; o < Z; o++) rank += key(o) < mine ? 1 : 0;
+        slot_of_row[i] = rank;
+        plan[L.slot_row + rank] = i;
+        plan[L.slot_l + rank] = lmax[i];
+    }
+    if (tid == 0) {  // scalars no row uses: their ds rows are zeros
+        for (int l = 0; l < S; l++)
+            if (!referenced[l]) plan[L.zero_l + num_zero_l++] = l;
+    }
+    __syncthreads();
+    if (!eligible) {
+        if (tid == 0) plan[kEligible] = 0;
+        return;  // (uniform: `eligible` is shared and was last written before the barrier)
+    }
+    // cells: entry counts, then their places (an exclusive scan over the dense cell array)
+    for (int n = tid; n < num_coef; n += kBuildThreads) {
+        int i, j, k, l;
+        decode(coef[n], cols_ji, i, j, k, l);
+        atomicAdd(&plan[L.count + slot_of_row[i] * kPlanX + j], 1);
+    }
+    __syncthreads();
+    constexpr int kPer = kCells / kBuildThreads;  // consecutive cells per thread
+    int sum = 0, live = 0;
+    for (int q = 0; q < kPer; q++) {
+        const int c = plan[L.count + tid * kPer + q];
+        sum += c; live += c > 0 ? 1 : 0;
+    }
+    // two scans with one buffer: entries (low 16 bits hold up to 8192) and live cells (high bits)
+    scan[tid] = sum | (live << 16);
+    __syncthreads();
+    for (int off = 1; off < kBuildThreads; off *= 2) {
+        const int add = tid >= off ? scan[tid - off] : 0;
+        __syncthreads();
+        scan[tid] += add;
+        __syncthreads();
+    }
+    {
+        const int before = tid ? scan[tid - 1] : 0;
+        int at = before & 0xffff, cell_at = before >> 16;
+        for (int q = 0; q < kPer; q++) {
+            const int cell = tid * kPer + q;
+            const int c = plan[L.count + cell];
+            plan[L.first + cell] = at;
+            at += c;
+            if (c > 0) {
+                plan[L.cell_list + cell_at++] = cell;
+                atomicOr(&chunk_mask, 1 << ((cell / kPlanX / 16) * xg + (cell % kPlanX) / 4));
+            }
+        }
+        if (tid == kBuildThreads - 1) num_cells = scan[tid] >> 16;
+    }
+    __syncthreads();
+    // entries to their cells; table order inside a cell (a fixed summation order)
+    for (int c = tid; c < kCells; c += kBuildThreads) plan[L.count + c] = 0;
+    __syncthreads();
+    for (int n = tid; n < num_coef; n += kBuildThreads) {
+        int i, j, k, l;
+        decode(coef[n], cols_ji, i, j, k, l);
+        const int cell = slot_of_row[i] * kPlanX + j;
+        const int at = plan[L.first + cell] + atomicAdd(&plan[L.count + cell], 1);
+        plan[L.coef + at] = __float_as_int((float)coef[n].val);
+        plan[L.k + at] = k;
+        plan[L.t + at] = n;
+    }
+    __syncthreads();
+    for (int cell = tid; cell < kCells; cell += kBuildThreads) {
+        const int first = plan[L.first + cell], cnt = plan[L.count + cell];
+        for (int a = 1; a < cnt; a++) {  // insertion sort by table position
+            const int t = plan[L.t + first + a], cf = plan[L.coef + first + a], kk = plan[L.k + first + a];
+            int b = a - 1;
+            while (b >= 0 && plan[L.t + first + b] > t) {
+                plan[L.t + first + b + 1] = plan[L.t + first + b];
+                plan[L.coef + first + b + 1] = plan[L.coef + first + b];
+                plan[L.k + first + b + 1] = plan[L.k + first + b];
+                b--;
+            }
+            plan[L.t + first + b + 1] = t; plan[L.coef + first + b + 1] = cf; plan[L.k + first + b + 1] = kk;
+        }
+        if (cnt > kPlanMaxRun) eligible = 0;
+        if (cnt > 0) atomicMax(&max_run, cnt);
+    }
+    for (int q = tid; q < kSlots; q += kBuildThreads) {
+        const int l = plan[L.slot_l + q];
+        plan[L.slot_lw + q] = l < 0 ? 0 : l * kWave;
+    }
+    __syncthreads();
+    // the forms the kernels stage in LDS
+    for (int q = tid; q < num_cells; q += kBuildThreads) {
+        const int cell = plan[L.cell_list + q];
+        plan[L.cells + q] = cell | (plan[L.first + cell] << 11) | (plan[L.count + cell] << 22);
+    }
+    for (int n = tid; n < num_coef; n += kBuildThreads) {
+        plan[L.pairs + 2 * n] = plan[L.coef + n];
+        plan[L.pairs + 2 * n + 1] = plan[L.k + n];
+    }
+    if (tid == 0) {
+        plan[kEligible] = eligible; plan[kNumCells] = num_cells; plan[kChunkMask] = chunk_mask;
+        plan[kNumZeroL] = num_zero_l; plan[kMaxRun] = max_run;
+    }
+}
+
+// LDS traffic between the lanes of one wave: its LDS operations complete in program order, so
+// only the compiler has to be kept from moving accesses across this point.
+__device__ __forceinline__ void wave_lds_sync() {
+    __builtin_amdgcn_fence(__ATOMIC_ACQ_REL, "wavefront");
+    __builtin_amdgcn_wave_barrier();
+}
+
+typedef float f32x4 __attribute__((ext_vector_type(4)));
+
+// The table part of the plan in LDS, shared by the waves of a workgroup: the packed cells, then
+// (coefficient, k) pairs.  Every thread of the workgroup calls this (it holds a barrier).
+// `dense` (backward): first | count << 11 of the first `dense_cells` dense cells behind them.
+__device__ __forceinline__ void stage_table(const int32_t *__restrict__ plan, const PlanLayout &L, int num_cells,
+                                            int num_coef, int32_t *tab, int dense_cells = 0) {
+    const int tid = threadIdx.y * kWave + threadIdx.x, threads = blockDim.y * kWave;
+    const int pairs = (num_cells + 1) & ~1;  // the pairs start at an even word
+    for (int t = tid; t < num_cells; t += threads) tab[t] = plan[L.cells + t];
+    for (int t = tid; t < 2 * num_coef; t += threads) tab[pairs + t] = plan[L.pairs + t];
+    int32_t *dense = tab + table_words(num_coef);
+    for (int t = tid; t < dense_cells; t += threads) {
+        const int cnt = plan[L.count + t];  // (an empty cell behind the last entry has first = 2048: dropped)
+        dense[t] = cnt > 0 ? plan[L.first + t] | (cnt << 11) : 0;
+    }
+    __syncthreads();
+}
+
+// M of one edge: lane q takes the cells q, q + 64, ... of the staged list; lane k of `yreg` holds y[k].
+// `most`: the longest entry list of a cell (lanes with shorter lists add zeros).
+template <int XG>
+__device__ __forceinline__ void build_edge_matrix(const int32_t *tab, int num_cells, int most, float yreg, float *M,
+                                                  int lane) {
+    const int pairs = (num_cells + 1) & ~1;
+    for (int q0 = 0; q0 < num_cells; q0 += kWave) {  // (all lanes run the same trips: the lane reads below are shuffles)
+        const int q = q0 + lane;
+        const unsigned w = (unsigned)tab[q < num_cells ? q : 0];
+        const int cell = (int)(w & 2047u), first = (int)((w >> 11) & 2047u);
+        const int cnt = q < num_cells ? (int)(w >> 22) : 0;
+        float sum = 0.f;
+        for (int r = 0; r < most; r++) {
+            const int at = r < cnt ? first + r : first;
+            const int kk = tab[pairs + 2 * at + 1];
+            const float cf = r < cnt ? __int_as_float(tab[pairs + 2 * at]) : 0.f;
+            sum += cf * __shfl(yreg, kk, kWave);
+        }
+        if (cnt > 0) {
+            const int slot = cell / kPlanX, j = cell % kPlanX;
+            M[(slot * XG + (j >> 2)) * 4 + (j & 3)] = sum;
+        }
+    }
+}
+
+// Per-slot numbers of the plan, kept by a wave in two vector registers (lane t of register k
+// holds the number of slot 64 k + t) and read as wave-uniform values with lane reads.
+struct SlotWords {
+    int lo, hi;
+    __device__ __forceinline__ SlotWords(const int32_t *__restrict__ words, int lane)
+        : lo(words[lane]), hi(words[kWave + lane]) {}
+    __device__ __forceinline__ int operator[](int slot) const {
+        return __builtin_amdgcn_readlane(slot < kWave ? lo : hi, slot % kWave);
+    }
+};
+
+__device__ __forceinline__ int next_live(const int32_t *__restrict__ other, int e, int e1, int num_nodes) {
+    while (e < e1 && (unsigned)other[e] >= (unsigned)num_nodes) e++;  // padding edges are stepped over
+    return e;
+}
+
+// Rows of an operand behind a wave-uniform base: the lanes keep one 32-bit byte offset that
+// moves from row to row by the row stride, so that a load takes a scalar base, one offset
+// register and one vector addition.
+// Values are held in memory as Val (float, or half: converted on the way in and out) and
+// computed in float.
+template <typename Val>
+struct RowCursor {
+    const char *base;   // wave-uniform
+    unsigned at;        // byte offset of the lane's element in row 0
+    unsigned step;      // bytes between rows
+    __device__ __forceinline__ RowCursor(const Val *row0, unsigned lane_elems, unsigned stride_elems)
+        : base(reinterpret_cast<const char *>(row0)), at((unsigned)sizeof(Val) * lane_elems),
+          step((unsigned)sizeof(Val) * stride_elems) {}
+    __device__ __forceinline__ float row(unsigned r) const {  // r wave-uniform
+        return (float)*reinterpret_cast<const Val *>(base + (at + r * step));
+    }
+};
+// the lane's element of row r of an output operand (same addressing)
+template <typename Val>
+__device__ __forceinline__ Val *element_at(Val *row0, unsigned lane_elems, unsigned stride_elems, unsigned r) {
+    return reinterpret_cast<Val *>(reinterpret_cast<char *>(row0) +
+                                   (unsigned)sizeof(Val) * (lane_elems + r * stride_elems));
+}
+
+// The scalar rows of one edge into the wave's LDS copy, eight loads in flight.
+template <typename Val>
+__device__ __forceinline__ void stage_scalars(const Val *srow0, unsigned soff, unsigned sdim, int S, float *sbuf,
+                                              int lane) {
+    const RowCursor<Val> cur(srow0, soff, sdim);
+    for (int t0 = 0; t0 < S; t0 += 8) {
+        float v[8];
+#pragma unroll
+        for (int t = 0; t < 8; t++) v[t] = cur.row((unsigned)(t0 + t < S ? t0 + t : S - 1));  // (clamped: straight-line)
+#pragma unroll
+        for (int t = 0; t < 8; t++) sbuf[(t0 + t < S ? t0 + t : S - 1) * kWave + lane] = v[t];
+    }
+}
+
+// Forward: a wave takes (row, 64 channels) and holds NB * 16 accumulators.
+template <typename Val, int NB, int XG>
+__global__ __launch_bounds__(256, 2) void planned_fwd_kernel(
+    const int32_t *__restrict__ plan, PlanLayout L, const Val *__restrict__ x, RowLayout lx,
+    const Val *__restrict__ y, int num_y, const Val *__restrict__ s, RowLayout ls,
+    const int32_t *__restrict__ other, const int32_t *__restrict__ row_ptr, const int32_t *__restrict__ perm,
+    const int32_t *__restrict__ row_order, Val *__restrict__ out, RowLayout lo, int num_nodes, int channels,
+    int X, int S, int num_coef, int nchunks) {
+    extern __shared__ __align__(16) float planned_lds[];
+    if (plan[kEligible] == 0) return;  // (the whole grid) the table-driven kernel without a plan runs instead
+    constexpr int kStrip = NB * 16 * XG * 4;
+    const int lane = threadIdx.x, wave = __builtin_amdgcn_readfirstlane((int)threadIdx.y);
+    const int num_cells = plan[kNumCells];
+    const int max_run = plan[kMaxRun];
+    int32_t *tab = reinterpret_cast<int32_t *>(planned_lds);
+    float *M = planned_lds + table_words(num_coef) + wave * (kStrip + S * kWave);
+    float *sbuf = M + kStrip;
+    for (int t = lane; t < kStrip; t += kWave) M[t] = 0.f;
+    stage_table(plan, L, num_cells, num_coef, tab);
+    const int64_t item = (int64_t)blockIdx.x * blockDim.y + wave;
+    if (item >= (int64_t)num_nodes * nchunks) return;  // uniform per wave; no workgroup barrier below
+    const int q = (int)(item / nchunks);
+    const int r = row_order ? row_order[q] : q;
+    const int c = (int)(item % nchunks) * kWave + lane;
+    const bool active = c < channels;
+    const int cr = active ? c : channels - 1;  // channel whose rows an idle lane reads
+    const unsigned xoff = (unsigned)cr * (unsigned)lx.chan, soff = (unsigned)cr * (unsigned)ls.chan;
+    const unsigned chunk_mask = (unsigned)plan[kChunkMask];
+    const SlotWords slot_lw(plan + L.slot_lw, lane);
+    float acc[NB * 16];
+#pragma unroll
+    for (int t = 0; t < NB * 16; t++) acc[t] = 0.f;
+
+    const int e1 = row_ptr[r + 1];
+    for (int e = next_live(other, row_ptr[r], e1, num_nodes); e < e1; e = next_live(other, e + 1, e1, num_nodes)) {
+        const int snd = other[e];
+        const int64_t ee = perm ? (int64_t)perm[e] : (int64_t)e;
+        const float yreg = lane < num_y ? (float)y[ee * num_y + lane] : 0.f;
+        wave_lds_sync();  // the reads of the edge before are behind the writes below
+        stage_scalars(s + ee * ls.row, soff, (unsigned)ls.dim, S, sbuf, lane);
+        float xv[XG * 4];
+        {
+            const RowCursor<Val> xc(x + (int64_t)snd * lx.row, xoff, (unsigned)lx.dim);
+#pragma unroll
+            for (int j = 0; j < XG * 4; j++) {
+                xv[j] = xc.row((unsigned)(j < X ? j : X - 1));
+                if (j >= X) xv[j] = 0.f;
+            }
+        }
+        build_edge_matrix<XG>(tab, num_cells, max_run, yreg, M, lane);
+        wave_lds_sync();
+#pragma unroll
+        for (int b = 0; b < NB; b++) {
+            if (((chunk_mask >> (b * XG)) & ((1u << XG) - 1u)) == 0) continue;  // no coefficient in the block
+            float sv[16], T[16];
+#pragma unroll
+            for (int u = 0; u < 16; u++) {
+                sv[u] = sbuf[slot_lw[b * 16 + u] + lane];
+                T[u] = 0.f;
+            }
+#pragma unroll
+            for (int g = 0; g < XG; g++) {
+                if (!((chunk_mask >> (b * XG + g)) & 1u)) continue;
+#pragma unroll
+                for (int u = 0; u < 16; u++) {
+                    const f32x4 m = *reinterpret_cast<const f32x4 *>(&M[((b * 16 + u) * XG + g) * 4]);
+                    T[u] = __builtin_fmaf(m.x, xv[4 * g], T[u]);
+                    T[u] = __builtin_fmaf(m.y, xv[4 * g + 1], T[u]);
+                    T[u] = __builtin_fmaf(m.z, xv[4 * g + 2], T[u]);
+                    T[u] = __builtin_fmaf(m.w, xv[4 * g + 3], T[u]);
+                }
+            }
+#pragma unroll
+            for (int u = 0; u < 16; u++) acc[b * 16 + u] = __builtin_fmaf(sv[u], T[u], acc[b * 16 + u]);
+        }
+    }
+    {
+        const SlotWords slot_row(plan + L.slot_row, lane), slot_l(plan + L.slot_l, lane);
+        Val *obase = out + (int64_t)r * lo.row;
+        const unsigned ooff = (unsigned)c * (unsigned)lo.chan;
+#pragma unroll
+        for (int t = 0; t < NB * 16; t++) {
+            const int row = slot_row[t];
+            // (a slot whose output coordinate no entry touches has read row 0 of s: it stores zero)
+            if (row >= 0 && active)
+                *element_at(obase, ooff, (unsigned)lo.dim, (unsigned)row) = (Val)(slot_l[t] < 0 ? 0.f : acc[t]);
+        }
+    }
+}
+
+// The channel sums of 64 per-lane products, left one to a lane: v[t] (t < 32) of one wave is summed
+// over the lanes of each half of the wave with five halving steps (lanes whose bit N is clear keep
+// the lower half of the values and take their partner's partial sums of them; the partners are a
+// row swap for N = 16 and DPP lane permutations inside rows of 16 below that), which leaves the
+// partial sum of v[t % 32] over the lane's half in lane t; two such arrays are then finished with
+// one swap of wave halves, lanes 0..31 getting the totals of the first, 32..63 of the second.
+template <int N, int CTRL>  // N pairs (p, p + N) are left; partner lanes differ in bit N
+__device__ __forceinline__ void transpose_sum_step(float (&v)[32], int lane) {
+    const bool upper = (lane & N) != 0;
+#pragma unroll
+    for (int p = 0; p < N; p++) {
+        const float keep = upper ? v[p + N] : v[p];
+        const float send = upper ? v[p] : v[p + N];
+        v[p] = keep + __int_as_float(__builtin_amdgcn_update_dpp(0, __float_as_int(send), CTRL, 0xf, 0xf, true));
+    }
+}
+__device__ __forceinline__ float transpose_sum_half(float (&v)[32], int lane) {
+#pragma unroll
+    for (int p = 0; p < 16; p++) {  // rows 1 and 3 of v[p] change places with rows 0 and 2 of v[p + 16]
+        const auto r = __builtin_amdgcn_permlane16_swap(__float_as_uint(v[p]), __float_as_uint(v[p + 16]), false, false);
+        v[p] = __uint_as_float(r[0]) + __uint_as_float(r[1]);
+    }
+    transpose_sum_step<8, 0x140>(v, lane);  // row_mirror: lane ^ 15
+    transpose_sum_step<4, 0x141>(v, lane);  // row_half_mirror: lane ^ 7
+    transpose_sum_step<2, 0x4E>(v, lane);   // quad_perm [2, 3, 0, 1]: lane ^ 2
+    transpose_sum_step<1, 0xB1>(v, lane);   // quad_perm [1, 0, 3, 2]: lane ^ 1
+    return v[0];
+}
+// lanes 0..31: first.lower + first.upper, lanes 32..63: second.lower + second.upper
+__device__ __forceinline__ float join_halves(float first, float second) {
+    const auto r = __builtin_amdgcn_permlane32_swap(__float_as_uint(first), __float_as_uint(second), false, false);
+    return __uint_as_float(r[0]) + __uint_as_float(r[1]);
+}
+
+enum DyMode { kDyStore = 0, kDyAdd = 1, kDyAtomic = 2 };
+
+template <typename Val, int NB, int XG>
+__global__ __launch_bounds__(256, 2) void planned_bwd_kernel(
+    const int32_t *__restrict__ plan, PlanLayout L, const Val *__restrict__ x, RowLayout lx,
+    const Val *__restrict__ y, int num_y, const Val *__restrict__ s, RowLayout ls,
+    const Val *__restrict__ dm, RowLayout lo, const int32_t *__restrict__ other,
+    const int32_t *__restrict__ row_ptr, const int32_t *__restrict__ perm,
+    const int32_t *__restrict__ row_order, Val *__restrict__ dx, Val *__restrict__ dy,
+    Val *__restrict__ ds, int num_nodes, int channels, int X, int S, int num_coef, int nchunks,
+    int group_is_receiver) {
+    extern __shared__ __align__(16) float planned_lds[];
+    if (plan[kEligible] == 0) return;
+    constexpr int kStrip = NB * 16 * XG * 4;
+    const int lane = threadIdx.x, wave = __builtin_amdgcn_readfirstlane((int)threadIdx.y);
+    const int num_cells = plan[kNumCells];
+    const unsigned chunk_mask = (unsigned)plan[kChunkMask];
+    const int max_run = plan[kMaxRun];
+    const int num_zero_l = plan[kNumZeroL];
+    int32_t *tab = reinterpret_cast<int32_t *>(planned_lds);
+    const int32_t *dense = tab + table_words(num_coef);
+    float *M = planned_lds + table_words(num_coef) + NB * 256 + wave * (kStrip + kPlanMaxY + S * kWave);
+    float *dyl = M + kStrip;
+    float *sbuf = dyl + kPlanMaxY;
+    for (int t = lane; t < kStrip + kPlanMaxY; t += kWave) M[t] = 0.f;
+    stage_table(plan, L, num_cells, num_coef, tab, NB * 256);
+    const int pairs = (num_cells + 1) & ~1;
+    const int64_t item = (int64_t)blockIdx.x * blockDim.y + wave;
+    // receiver rows: a wave per (row, 64 channels), dx by float atomics, dy shared between the
+    // waves of an edge; sender rows: a wave per row walks the channel chunks and owns dx and dy
+    const int64_t items = group_is_receiver ? (int64_t)num_nodes * nchunks : (int64_t)num_nodes;
+    if (item >= items) return;
+    const int qrow = (int)(group_is_receiver ? item / nchunks : item);
+    const int g = row_order ? row_order[qrow] : qrow;
+    const int chunk0 = group_is_receiver ? (int)(item % nchunks) : 0;
+    const int chunk1 = group_is_receiver ? chunk0 + 1 : nchunks;
+    const int e0 = row_ptr[g], e1 = row_ptr[g + 1];
+    const SlotWords slot_l(plan + L.slot_l, lane), slot_row(plan + L.slot_row, lane);
+
+    for (int chunk = chunk0; chunk < chunk1; chunk++) {
+        const int c = chunk * kWave + lane;
+        const bool active = c < channels;
+        const int cr = active ? c : channels - 1;
+        const unsigned xoff = (unsigned)cr * (unsigned)lx.chan, soff = (unsigned)cr * (unsigned)ls.chan;
+        const unsigned zoff = (unsigned)cr * (unsigned)lo.chan;
+        const int dy_mode = group_is_receiver ? (nchunks > 1 ? kDyAtomic : kDyStore)
+                                              : (chunk == 0 ? kDyStore : kDyAdd);
+        float dxa[XG * 4];
+#pragma unroll
+        for (int j = 0; j < XG * 4; j++) dxa[j] = 0.f;
+        for (int e = next_live(other, e0, e1, num_nodes); e < e1; e = next_live(other, e + 1, e1, num_nodes)) {
+            const int o = other[e];
+            const int64_t ee = perm ? (int64_t)perm[e] : (int64_t)e;
+            const int xnode = group_is_receiver ? o : g;
+            const int znode = group_is_receiver ? g : o;
+            const float yreg = lane < num_y ? (float)y[ee * num_y + lane] : 0.f;
+            wave_lds_sync();
+            stage_scalars(s + ee * ls.row, soff, (unsigned)ls.dim, S, sbuf, lane);
+            float xv[XG * 4];
+            {
+                const RowCursor<Val> xc(x + (int64_t)xnode * lx.row, xoff, (unsigned)lx.dim);
+#pragma unroll
+                for (int j = 0; j < XG * 4; j++) {
+                    xv[j] = xc.row((unsigned)(j < X ? j : X - 1));
+                    if (j >= X || !active) xv[j] = 0.f;  // (idle lanes add nothing to dy)
+                }
+            }
+            build_edge_matrix<XG>(tab, num_cells, max_run, yreg, M, lane);
+            wave_lds_sync();
+            const RowCursor<Val> zc(dm + (int64_t)znode * lo.row, zoff, (unsigned)lo.dim);
+            Val *dsrow0 = ds + ee * ls.row;
+            const unsigned dsoff = (unsigned)c * (unsigned)ls.chan;
+            int cur_l = -1;
+            float dsa = 0.f;
+#pragma unroll
+            for (int b = 0; b < NB; b++) {
+                if (((chunk_mask >> (b * XG)) & ((1u << XG) - 1u)) == 0) continue;
+                float sd[16], dz[16], T[16];
+#pragma unroll
+                for (int u = 0; u < 16; u++) {
+                    const int l = slot_l[b * 16 + u], row = slot_row[b * 16 + u];  // (-1: none)
+                    const float sv = sbuf[(l < 0 ? 0 : l) * kWave + lane];
+                    dz[u] = zc.row((unsigned)(row < 0 ? 0 : row));
+                    if (l < 0) dz[u] = 0.f;
+                    sd[u] = sv * dz[u];
+                    T[u] = 0.f;
+                }
+#pragma unroll
+                for (int gx = 0; gx < XG; gx++) {
+                    if (!((chunk_mask >> (b * XG + gx)) & 1u)) continue;
+                    // lane t ends with the channel sum of cell (slot 16 b + t / 4, x coordinate 4 gx + t % 4):
+                    // the slots in two halves of eight, the first for lanes 0..31, the second for the rest
+                    float part[2];
+#pragma unroll
+                    for (int half = 0; half < 2; half++) {
+                        float G[32];
+#pragma unroll
+                        for (int uu = 0; uu < 8; uu++) {
+                            const int u = half * 8 + uu;
+                            const f32x4 m = *reinterpret_cast<const f32x4 *>(&M[((b * 16 + u) * XG + gx) * 4]);
+                            T[u] = __builtin_fmaf(m.x, xv[4 * gx], T[u]);
+                            T[u] = __builtin_fmaf(m.y, xv[4 * gx + 1], T[u]);
+                            T[u] = __builtin_fmaf(m.z, xv[4 * gx + 2], T[u]);
+                            T[u] = __builtin_fmaf(m.w, xv[4 * gx + 3], T[u]);
+                            dxa[4 * gx] = __builtin_fmaf(m.x, sd[u], dxa[4 * gx]);
+                            dxa[4 * gx + 1] = __builtin_fmaf(m.y, sd[u], dxa[4 * gx + 1]);
+                            dxa[4 * gx + 2] = __builtin_fmaf(m.z, sd[u], dxa[4 * gx + 2]);
+                            dxa[4 * gx + 3] = __builtin_fmaf(m.w, sd[u], dxa[4 * gx + 3]);
+#pragma unroll
+                            for (int jj = 0; jj < 4; jj++) G[uu * 4 + jj] = sd[u] * xv[4 * gx + jj];
+                        }
+                        part[half] = transpose_sum_half(G, lane);
+                    }
+                    const float total = join_halves(part[0], part[1]);
+                    const int where = dense[(b * 16 + lane / 4) * kPlanX + 4 * gx + lane % 4];
+                    const int first = where & 2047, cnt = where >> 11;
+                    for (int rr = 0; rr < cnt; rr++)
+                        atomicAdd(&dyl[tab[pairs + 2 * (first + rr) + 1]],
+                                  __int_as_float(tab[pairs + 2 * (first + rr)]) * total);
+                }
+                // ds: the slots of one scalar are adjacent; a scalar's sum is stored when the next begins
+#pragma unroll
+                for (int u = 0; u < 16; u++) {
+                    const int l = slot_l[b * 16 + u];
+                    if (l != cur_l) {
+                        if (cur_l >= 0 && active) *element_at(dsrow0, dsoff, (unsigned)ls.dim, (unsigned)cur_l) = (Val)dsa;
+                        cur_l = l;
+                        dsa = 0.f;
+                    }
+                    dsa = __builtin_fmaf(dz[u], T[u], dsa);
+                }
+            }
+            if (cur_l >= 0 && active) *element_at(dsrow0, dsoff, (unsigned)ls.dim, (unsigned)cur_l) = (Val)dsa;
+            if (active)
+                for (int z = 0; z < num_zero_l; z++)
+                    *element_at(dsrow0, dsoff, (unsigned)ls.dim, (unsigned)plan[L.zero_l + z]) = Val(0);
+            wave_lds_sync();
+            if (lane < num_y) {
+                const float v = dyl[lane];
+                dyl[lane] = 0.f;
+                Val *at = dy + ee * num_y + lane;
+                if (dy_mode == kDyStore) *at = (Val)v;
+                else if (dy_mode == kDyAdd) *at = (Val)((float)*at + v);
+                else if constexpr (std::is_same<Val, float>::value) unsafeAtomicAdd(at, v);
+            }
+            if (group_is_receiver) {
+                if constexpr (std::is_same<Val, float>::value) {  // (half values have no float atomics: sender rows only)
+                    if (active) {
+                        Val *dxrow0 = dx + (int64_t)xnode * lx.row;
+#pragma unroll
+                        for (int j = 0; j < XG * 4; j++)
+                            if (j < X) unsafeAtomicAdd(element_at(dxrow0, xoff, (unsigned)lx.dim, (unsigned)j), dxa[j]);
+                    }
+                }
+#pragma unroll
+                for (int j = 0; j < XG * 4; j++) dxa[j] = 0.f;
+            }
+        }
+        if (!group_is_receiver && active) {
+            Val *dxrow0 = dx + (int64_t)g * lx.row;
+#pragma unroll
+            for (int j = 0; j < XG * 4; j++)
+                if (j < X) *element_at(dxrow0, xoff, (unsigned)lx.dim, (unsigned)j) = (Val)dxa[j];
+        }
+    }
+}
+
+constexpr int kWavesPerBlock = 4;
+
+#define E3J_ROW(K, NB) {K<Val, NB, 1>, K<Val, NB, 2>, K<Val, NB, 3>, K<Val, NB, 4>}
+#define E3J_TABLE(K) {E3J_ROW(K, 1), E3J_ROW(K, 2), E3J_ROW(K, 3), E3J_ROW(K, 4), \
+                      E3J_ROW(K, 5), E3J_ROW(K, 6), E3J_ROW(K, 7), E3J_ROW(K, 8)}
+
+template <typename Val>
+int launch_plan_build_t(const e3j_amd_conv_params &p, const void *coef, bool cols_ji, int32_t *plan,
+                        hipStream_t stream) {
+    const PlanLayout L(p.num_coef, p.num_scalars);
+    const int xg = (p.num_x + 3) / 4;
+    if (p.coef_idx_bytes == 1)
+        hipLaunchKernelGGL((plan_build_kernel<uint8_t, Val>), dim3(1), dim3(kBuildThreads), 0, stream,
+                           static_cast<const Coef4D<uint8_t, Val> *>(coef), p.num_coef, p.num_x, p.num_y,
+                           p.num_out, p.num_scalars, xg, cols_ji ? 1 : 0, plan, L);
+    else
+        hipLaunchKernelGGL((plan_build_kernel<int32_t, Val>), dim3(1), dim3(kBuildThreads), 0, stream,
+                           static_cast<const Coef4D<int32_t, Val> *>(coef), p.num_coef, p.num_x, p.num_y,
+                           p.num_out, p.num_scalars, xg, cols_ji ? 1 : 0, plan, L);
+    return check_hip(hipGetLastError(), "convolution plan launch");
+}
+
+template <typename Val>
+int launch_planned_fwd_t(const e3j_amd_conv_params &p, const int32_t *plan, const void *x, const void *y,
+                         const void *s, const int32_t *other, const int32_t *row_ptr, const int32_t *perm,
+                         void *out, hipStream_t stream) {
+    typedef void (*Kernel)(const int32_t *, PlanLayout, const Val *, RowLayout, const Val *, int, const Val *,
+                           RowLayout, const int32_t *, const int32_t *, const int32_t *, const int32_t *, Val *,
+                           RowLayout, int, int, int, int, int, int);
+    static const Kernel kernels[8][4] = E3J_TABLE(planned_fwd_kernel);
+    const int nb = (p.num_out + 15) / 16, xg = (p.num_x + 3) / 4;
+    const int nchunks = (p.channels + kWave - 1) / kWave;
+    const int64_t items = (int64_t)p.num_nodes * nchunks;
+    const int64_t blocks = (items + kWavesPerBlock - 1) / kWavesPerBlock;
+    if (blocks > 0x7fffffffLL) return set_error(E3J_AMD_INVALID_ARGUMENT, "convolution: grid too large");
+    const size_t lds = sizeof(float) * ((size_t)table_words(p.num_coef) +
+                                        (size_t)kWavesPerBlock * (nb * 16 * xg * 4 + p.num_scalars * kWave));
+    if (lds > 64 * 1024) {
+        const int rc = check_hip(hipFuncSetAttribute(reinterpret_cast<const void *>(kernels[nb - 1][xg - 1]),
+                                                     hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds),
+                                 "hipFuncSetAttribute(planned fwd)");
+        if (rc) return rc;
+    }
+    hipLaunchKernelGGL(kernels[nb - 1][xg - 1], dim3((unsigned)blocks), dim3(kWave, kWavesPerBlock), lds, stream, plan,
+                       PlanLayout(p.num_coef, p.num_scalars), static_cast<const Val *>(x),
+                       make_layout(p.layout, p.num_x, p.channels), static_cast<const Val *>(y), p.num_y,
+                       static_cast<const Val *>(s), make_layout(p.layout, p.num_scalars, p.channels), other,
+                       row_ptr, perm, p.row_order, static_cast<Val *>(out),
+                       make_layout(p.layout, p.num_out, p.channels), p.num_nodes, p.channels, p.num_x,
+                       p.num_scalars, p.num_coef, nchunks);
+    return check_hip(hipGetLastError(), "convolution forward launch (planned)");
+}
+
+template <typename Val>
+int launch_planned_bwd_t(const e3j_amd_conv_params &p, bool group_is_receiver, const int32_t *plan, const void *x,
+                         const void *y, const void *s, const void *dm, const int32_t *other,
+                         const int32_t *row_ptr, const int32_t *perm, void *dx, void *dy, void *ds,
+                         hipStream_t stream) {
+    typedef void (*Kernel)(const int32_t *, PlanLayout, const Val *, RowLayout, const Val *, int, const Val *,
+                           RowLayout, const Val *, RowLayout, const int32_t *, const int32_t *, const int32_t *,
+                           const int32_t *, Val *, Val *, Val *, int, int, int, int, int, int, int);
+    static const Kernel kernels[8][4] = E3J_TABLE(planned_bwd_kernel);
+    const int nb = (p.num_out + 15) / 16, xg = (p.num_x + 3) / 4;
+    const int nchunks = (p.channels + kWave - 1) / kWave;
+    const int64_t items = group_is_receiver ? (int64_t)p.num_nodes * nchunks : (int64_t)p.num_nodes;
+    const int64_t blocks = (items + kWavesPerBlock - 1) / kWavesPerBlock;
+    if (blocks > 0x7fffffffLL) return set_error(E3J_AMD_INVALID_ARGUMENT, "convolution_bwd: grid too large");
+    const size_t lds = sizeof(float) * ((size_t)table_words(p.num_coef) + (size_t)nb * 256 +
+                                        (size_t)kWavesPerBlock * (nb * 16 * xg * 4 + kPlanMaxY + p.num_scalars * kWave));
+    if (lds > 64 * 1024) {
+        const int rc = check_hip(hipFuncSetAttribute(reinterpret_cast<const void *>(kernels[nb - 1][xg - 1]),
+                                                     hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds),
+                                 "hipFuncSetAttribute(planned bwd)");
+        if (rc) return rc;
+    }
+    hipLaunchKernelGGL(kernels[nb - 1][xg - 1], dim3((unsigned)blocks), dim3(kWave, kWavesPerBlock), lds, stream, plan,
+                       PlanLayout(p.num_coef, p.num_scalars), static_cast<const Val *>(x),
+                       make_layout(p.layout, p.num_x, p.channels), static_cast<const Val *>(y), p.num_y,
+                       static_cast<const Val *>(s), make_layout(p.layout, p.num_scalars, p.channels),
+                       static_cast<const Val *>(dm), make_layout(p.layout, p.num_out, p.channels), other,
+                       row_ptr, perm, p.row_order, static_cast<Val *>(dx), static_cast<Val *>(dy),
+                       static_cast<Val *>(ds), p.num_nodes, p.channels, p.num_x, p.num_scalars, p.num_coef, nchunks,
+                       group_is_receiver ? 1 : 0);
+    return check_hip(hipGetLastError(), "convolution backward launch (planned)");
+}
+#undef E3J_TABLE
+#undef E3J_ROW
+
+// whether the sizes of a call fit a plan (the value type is the caller's question)
+inline bool plan_sizes_fit(const e3j_amd_conv_params &p) {
+    return p.num_out >= 1 && p.num_out <= kSlots && p.num_x >= 1 && p.num_x <= kPlanX && p.num_y >= 1 &&
+           p.num_y <= kPlanMaxY && p.num_scalars >= 1 && p.num_scalars <= kPlanMaxS && p.num_coef >= 1 &&
+           p.num_coef <= kPlanMaxCoef && p.channels >= 1;
+}
+inline size_t plan_words(const e3j_amd_conv_params &p) { return (size_t)PlanLayout(p.num_coef, p.num_scalars).words; }
+
+}  // namespace
+
+// The float16 instantiations are compiled in a unit of their own (conv_planned_f16.hip).
+int launch_plan_build_f16(const e3j_amd_conv_params &p, const void *coef, bool cols_ji, int32_t *plan,
+                          hipStream_t stream);
+int launch_planned_fwd_f16(const e3j_amd_conv_params &p, const int32_t *plan, const void *x, const void *y,
+                           const void *s, const int32_t *other, const int32_t *row_ptr, const int32_t *perm,
+                           void *out, hipStream_t stream);
+int launch_planned_bwd_f16(const e3j_amd_conv_params &p, bool group_is_receiver, const int32_t *plan, const void *x,
+                           const void *y, const void *s, const void *dm, const int32_t *other,
+                           const int32_t *row_ptr, const int32_t *perm, void *dx, void *dy, void *ds,
+                           hipStream_t stream);
+
+}  // namespace e3j_amd
+#endif

@@ -233,12 +233,13 @@ int e3j_amd_find_signature(const void *coef_host, int32_t coef_idx_bytes, int32_
 void e3j_amd_set_launch_variant(int32_t fwd_variant, int32_t bwd_variant);
 
 /* The table-driven kernels (calls with signature < 0, and calls whose operands an unrolled kernel
- * cannot take) come in two forms.  For a float32 table in which every output coordinate uses one
+ * cannot take) come in two forms.  For a float32 or float16 table (float16: values held as half,
+ * arithmetic in float; the sender-grouped backward only) in which every output coordinate uses one
  * scalar, with at most 128 output coordinates, 16 x coordinates, 64 y components, 1024 scalars and
  * 8192 entries, the call first turns the table into a plan on the device (one small kernel; the
  * plan lives in memory of the stream's pool, hipMallocAsync, for the length of the call) and runs
- * kernels that keep x and the accumulators in registers; any other table, float64 and float16
- * run the kernels that index LDS columns by the table's coordinates.  Whether a table fits is
+ * kernels that keep x and the accumulators in registers; any other table and float64 run the
+ * kernels that index LDS columns by the table's coordinates (float16 there: arithmetic in half).  Whether a table fits is
  * decided on the device, without a read-back.  on = 0 switches the planned form off for later
  * calls (process-wide, atomic; initial value from E3J_AMD_TABLE_PLANS, default 1); a call on a
  * stream that is being captured into a graph allocates nothing and runs the LDS-column kernels.  Results

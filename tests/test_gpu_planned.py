@@ -1,6 +1,6 @@
 """The two forms of the table-driven kernels through the C ABI (signature -1): over a plan of the
-table that one workgroup builds on the device (float32 tables in which every output coordinate
-uses one scalar, within the plan's size limits), and over LDS columns indexed by the table's
+table that one workgroup builds on the device (float32 and float16 tables in which every output
+coordinate uses one scalar, within the plan's size limits), and over LDS columns indexed by the table's
 coordinates (everything else).  Which form a table gets is checked through
 `e3j_amd_table_plan_status`; both forms are compared with the CPU oracle and with each other."""
 
@@ -66,6 +66,9 @@ def test_tables_the_plan_does_not_take():
     big = H.random_table(rng, 300, 5, 7, 129, 4)
     assert _status(H.pack_table(*big), 5, 7, 129, 4)[0] == 0
     assert _status(H.pack_table(idx, val, mix, val_dtype=np.float64), 5, 7, 6, 4, val=_lib.F64)[0] == 0
+    # float16 tables are planned (values held as half, computed in float)
+    assert _status(H.pack_table(idx, val.astype(np.float16), mix, val_dtype=np.float16), 5, 7, 6, 4,
+                   val=_lib.F16)[0] == 1
 
 
 def test_a_table_with_two_scalars_on_one_output_runs_the_column_kernels():
@@ -171,6 +174,40 @@ def test_both_forms_agree_and_the_column_form_still_runs(plans_off):
     planned = run_abi(idx, val, mix, x, y, s, dm, snd, rcv, Z)
     for a, b, name in zip(planned, columns, ("out", "dx", "dy", "ds")):
         np.testing.assert_allclose(a, b, rtol=2e-5, atol=2e-5, err_msg=name)
+
+
+@pytest.mark.parametrize("plans", [1, 0])
+def test_float16_through_the_operator_in_both_forms(plans):
+    """float16 operands with cfg3's table (7 blocks of outputs): the planned kernels hold the values
+    as half and compute in float, the column kernels compute in half; both within half-precision
+    rounding of the float64 checker on the rounded operands (forward, and the sender-grouped
+    backward that float16 takes)."""
+    from e3j_amd.ops import convolution
+    w = W.config3(0.002)
+    idx, val, mix = w.table()
+    rng = np.random.default_rng(77)
+    N, E, K = 12, 70, 128
+    snd, rcv = H.random_graph(rng, N, E)
+    x, y, s, dm = (a.astype(np.float16) for a in H.random_operands(rng, N, E, 16, 16, 23, K, 99))
+    val16 = np.asarray(val).astype(np.float16)
+    coef = H.pack_table(idx, val16, mix, val_dtype=np.float16)
+    lib = _lib.load()
+    lib.e3j_amd_set_table_plans(plans)
+    try:
+        xd, yd, sd = (_dev(a).requires_grad_(True) for a in (x, y, s))
+        out = convolution(coef, xd, yd, sd, _dev(snd.astype(np.int32)), _dev(rcv.astype(np.int32)), w.module.params)
+        grads = torch.autograd.grad(out, (xd, yd, sd), _dev(dm))
+        torch.cuda.synchronize()
+    finally:
+        lib.e3j_amd_set_table_plans(1)
+    assert out.dtype == torch.float16
+    f64 = [a.astype(np.float64) for a in (x, y, s, dm)]
+    ref, mag = H.forward_reference(idx, val16.astype(np.float64), mix, f64[0], f64[1], f64[2], snd, rcv, 99)
+    refs, mags = H.backward_reference(idx, val16.astype(np.float64), mix, f64[0], f64[1], f64[2], snd, rcv, f64[3])
+    eps = 2.0 ** -10
+    for got, r, m, name in [(out, ref, mag, "out")] + list(zip(grads, refs, mags, ("dx", "dy", "ds"))):
+        err = np.abs(got.detach().float().cpu().numpy().astype(np.float64) - r)
+        assert np.all(err <= 6 * eps * m + 1e-3), f"{name} (plans={plans}): {err.max()} against magnitude {m.max()}"
 
 
 def test_sender_grouped_backward_gives_the_same_bits_every_time():
