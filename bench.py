@@ -742,6 +742,20 @@ def main():
             "forward_plus_backward": {"ms": lf + lb, "frac": gbs(bytes_["fwd_bwd"], lf + lb) / HBM_PEAK_GBS}}}
         del lead, wl
         abi = AbiCalls(w)
+    if (args.layout == "trailing" and not args.kernel_only and not args.no_layouts and args.config == "cfg3"
+            and args.scale == 1.0 and not args.table_driven):
+        # the kernels that read the table at run time (a table without built-in kernels on a host
+        # without hipcc), at an eighth of the workload, beside the unrolled kernels on the same inputs
+        small = build_workload(args.config, 0.125, device, channels=args.channels)
+        record = {"workload": f"{args.config} x 0.125: {small.num_nodes} atoms, {small.num_edges} edges, "
+                              f"K={small.channels}", "unit": "ms"}
+        for name, flag in (("table_driven", True), ("unrolled", False)):
+            calls = AbiCalls(small, table_driven=flag)
+            record[name] = {"forward": time_events(torch, calls.forward, args.steps, 2),
+                            "backward": time_events(torch, calls.backward, args.steps, 2)}
+            del calls
+        result["table_driven"] = record
+        del small
     if args.tile_sharing:
         result["roofline"]["tile_sharing"] = tile_sharing(abi, w)
     if args.access_floor:

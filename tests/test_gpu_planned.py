@@ -268,3 +268,52 @@ def test_planned_kernels_at_120k_edges():
     from e3j_amd.ops import convolution
     ref = convolution(w.module._packed_coef("float32"), w.x, w.y, w.s, w.sender, w.receiver, w.module.params)
     torch.testing.assert_close(out, ref, rtol=2e-4, atol=2e-4)
+
+
+def test_a_call_recorded_into_a_graph_allocates_nothing_and_replays():
+    """On a stream that is being captured the table-driven call takes no plan memory from the pool:
+    it records the LDS-column kernels, and the replays agree with eager calls (which plan the table)
+    to rounding, with other work and new operand values in between."""
+    w = W.config3(0.002)
+    idx, val, mix = w.table()
+    rng = np.random.default_rng(88)
+    N, E, K = 40, 600, 64
+    snd, rcv = H.random_graph(rng, N, E)
+    packed = H.pack_table(idx, val, mix)
+    coef_d = _dev(packed.view(np.uint8).reshape(-1))
+    x, y, s, dm = (_dev(a) for a in H.random_operands(rng, N, E, 16, 16, 23, K, 99))
+    other, ptr_d = _dev(snd.astype(np.int32)), _dev(O.receiver_ptr(rcv, N))
+    p = _params(N, E, len(packed), 16, 16, 99, 23, K, 1, _lib.F32, packed.dtype.itemsize, debug=0)
+    out = torch.empty((N, 99, K), device="cuda")
+    dx, dy, ds = torch.empty_like(x), torch.empty_like(y), torch.empty_like(s)
+    lib = _lib.load()
+
+    def launch(stream):
+        _lib.check(lib.e3j_amd_convolution_fwd(ctypes.byref(p), coef_d.data_ptr(), x.data_ptr(), y.data_ptr(),
+                                               s.data_ptr(), other.data_ptr(), ptr_d.data_ptr(), None,
+                                               out.data_ptr(), stream))
+        _lib.check(lib.e3j_amd_convolution_bwd_receiver(
+            ctypes.byref(p), coef_d.data_ptr(), x.data_ptr(), y.data_ptr(), s.data_ptr(), dm.data_ptr(),
+            other.data_ptr(), ptr_d.data_ptr(), None, dx.data_ptr(), dy.data_ptr(), ds.data_ptr(), stream))
+
+    side = torch.cuda.Stream()
+    side.wait_stream(torch.cuda.current_stream())
+    with torch.cuda.stream(side):
+        launch(side.cuda_stream)                      # warm-up outside the capture
+    torch.cuda.current_stream().wait_stream(side)
+    torch.cuda.synchronize()
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph, stream=side):
+        launch(side.cuda_stream)
+    for trial in range(3):
+        gen = torch.Generator(device="cuda").manual_seed(200 + trial)
+        for t in (x, y, s, dm):
+            t.copy_(torch.randn(t.shape, device="cuda", generator=gen))
+        (x.sum() + s.sum()).item()                    # unrelated eager work and a synchronisation
+        graph.replay()
+        torch.cuda.synchronize()
+        replayed = [t.clone() for t in (out, dx, dy, ds)]
+        launch(torch.cuda.current_stream().cuda_stream)
+        torch.cuda.synchronize()
+        for a, b, name in zip(replayed, (out, dx, dy, ds), ("out", "dx", "dy", "ds")):
+            assert float((a - b).abs().max()) <= 5e-5 * float(b.abs().max()), (trial, name)
