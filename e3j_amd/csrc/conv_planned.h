@@ -287,8 +287,12 @@ struct SlotWords {
     }
 };
 
+// A value every lane of the wave holds alike, moved to a scalar register (the compiler cannot
+// know that a vector load of a wave-uniform address gives a wave-uniform value).
+__device__ __forceinline__ int uni(int v) { return __builtin_amdgcn_readfirstlane(v); }
+
 __device__ __forceinline__ int next_live(const int32_t *__restrict__ other, int e, int e1, int num_nodes) {
-    while (e < e1 && (unsigned)other[e] >= (unsigned)num_nodes) e++;  // padding edges are stepped over
+    while (e < e1 && (unsigned)uni(other[e]) >= (unsigned)num_nodes) e++;  // padding edges are stepped over
     return e;
 }
 
@@ -352,7 +356,7 @@ __global__ __launch_bounds__(256, 2) void planned_fwd_kernel(
     const int64_t item = (int64_t)blockIdx.x * blockDim.y + wave;
     if (item >= (int64_t)num_nodes * nchunks) return;  // uniform per wave; no workgroup barrier below
     const int q = (int)(item / nchunks);
-    const int r = row_order ? row_order[q] : q;
+    const int r = row_order ? uni(row_order[q]) : q;
     const int c = (int)(item % nchunks) * kWave + lane;
     const bool active = c < channels;
     const int cr = active ? c : channels - 1;  // channel whose rows an idle lane reads
@@ -363,10 +367,10 @@ __global__ __launch_bounds__(256, 2) void planned_fwd_kernel(
 #pragma unroll
     for (int t = 0; t < NB * 16; t++) acc[t] = 0.f;
 
-    const int e1 = row_ptr[r + 1];
-    for (int e = next_live(other, row_ptr[r], e1, num_nodes); e < e1; e = next_live(other, e + 1, e1, num_nodes)) {
-        const int snd = other[e];
-        const int64_t ee = perm ? (int64_t)perm[e] : (int64_t)e;
+    const int e1 = uni(row_ptr[r + 1]);
+    for (int e = next_live(other, uni(row_ptr[r]), e1, num_nodes); e < e1; e = next_live(other, e + 1, e1, num_nodes)) {
+        const int snd = uni(other[e]);
+        const int64_t ee = perm ? (int64_t)uni(perm[e]) : (int64_t)e;
         const float yreg = lane < num_y ? (float)y[ee * num_y + lane] : 0.f;
         wave_lds_sync();  // the reads of the edge before are behind the writes below
         stage_scalars(s + ee * ls.row, soff, (unsigned)ls.dim, S, sbuf, lane);
@@ -487,10 +491,10 @@ __global__ __launch_bounds__(256, 2) void planned_bwd_kernel(
     const int64_t items = group_is_receiver ? (int64_t)num_nodes * nchunks : (int64_t)num_nodes;
     if (item >= items) return;
     const int qrow = (int)(group_is_receiver ? item / nchunks : item);
-    const int g = row_order ? row_order[qrow] : qrow;
+    const int g = row_order ? uni(row_order[qrow]) : qrow;
     const int chunk0 = group_is_receiver ? (int)(item % nchunks) : 0;
     const int chunk1 = group_is_receiver ? chunk0 + 1 : nchunks;
-    const int e0 = row_ptr[g], e1 = row_ptr[g + 1];
+    const int e0 = uni(row_ptr[g]), e1 = uni(row_ptr[g + 1]);
     const SlotWords slot_l(plan + L.slot_l, lane), slot_row(plan + L.slot_row, lane);
 
     for (int chunk = chunk0; chunk < chunk1; chunk++) {
@@ -505,8 +509,8 @@ __global__ __launch_bounds__(256, 2) void planned_bwd_kernel(
 #pragma unroll
         for (int j = 0; j < XG * 4; j++) dxa[j] = 0.f;
         for (int e = next_live(other, e0, e1, num_nodes); e < e1; e = next_live(other, e + 1, e1, num_nodes)) {
-            const int o = other[e];
-            const int64_t ee = perm ? (int64_t)perm[e] : (int64_t)e;
+            const int o = uni(other[e]);
+            const int64_t ee = perm ? (int64_t)uni(perm[e]) : (int64_t)e;
             const int xnode = group_is_receiver ? o : g;
             const int znode = group_is_receiver ? g : o;
             const float yreg = lane < num_y ? (float)y[ee * num_y + lane] : 0.f;
