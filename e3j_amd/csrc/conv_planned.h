@@ -625,7 +625,7 @@ __global__ __launch_bounds__(256, 2) void planned_bwd_kernel(
     }
 }
 
-constexpr int kWavesPerBlock = 4;
+constexpr int kWavesPerBlock = 2;  // (120k edges, K = 128, l <= 3: forward 2.12 ms, backward 5.17 ms; four: 2.27 and 5.33; one: 2.10 and 6.07)
 
 #define E3J_ROW(K, NB) {K<Val, NB, 1>, K<Val, NB, 2>, K<Val, NB, 3>, K<Val, NB, 4>}
 #define E3J_TABLE(K) {E3J_ROW(K, 1), E3J_ROW(K, 2), E3J_ROW(K, 3), E3J_ROW(K, 4), \
