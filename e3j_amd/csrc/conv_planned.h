@@ -276,6 +276,63 @@ __device__ __forceinline__ void build_edge_matrix(const int32_t *tab, int num_ce
     }
 }
 
+// The same with the lane's first kHeld cells of the list held in registers for all edges (their
+// list words do not change from edge to edge) and their entry chains interleaved: the LDS round
+// trips of the chains overlap instead of following each other.
+constexpr int kHeld = 6;  // 384 cells
+struct HeldCells {
+    unsigned w[kHeld];
+    __device__ __forceinline__ HeldCells(const int32_t *tab, int num_cells, int lane) {
+#pragma unroll
+        for (int it = 0; it < kHeld; it++) w[it] = it * kWave + lane < num_cells ? (unsigned)tab[it * kWave + lane] : 0u;
+    }
+};
+template <int XG>
+__device__ __forceinline__ void build_edge_matrix(const int32_t *tab, const HeldCells &held, int num_cells, int most,
+                                                  float yreg, float *M, int lane) {
+    const int pairs = (num_cells + 1) & ~1;
+    float sum[kHeld];
+#pragma unroll
+    for (int it = 0; it < kHeld; it++) sum[it] = 0.f;
+    for (int r = 0; r < most; r++) {
+#pragma unroll
+        for (int it = 0; it < kHeld; it++) {
+            if (it * kWave >= num_cells) break;  // (wave-uniform)
+            const int first = (int)((held.w[it] >> 11) & 2047u), cnt = (int)(held.w[it] >> 22);
+            const int at = r < cnt ? first + r : first;
+            const int kk = tab[pairs + 2 * at + 1];
+            const float cf = r < cnt ? __int_as_float(tab[pairs + 2 * at]) : 0.f;
+            sum[it] += cf * __shfl(yreg, kk, kWave);
+        }
+    }
+#pragma unroll
+    for (int it = 0; it < kHeld; it++) {
+        if (it * kWave >= num_cells) break;
+        if ((held.w[it] >> 22) > 0) {
+            const int cell = (int)(held.w[it] & 2047u);
+            const int slot = cell / kPlanX, j = cell % kPlanX;
+            M[(slot * XG + (j >> 2)) * 4 + (j & 3)] = sum[it];
+        }
+    }
+    for (int q0 = kHeld * kWave; q0 < num_cells; q0 += kWave) {  // cells past the held ones, one at a time
+        const int q = q0 + lane;
+        const unsigned w = (unsigned)tab[q < num_cells ? q : 0];
+        const int cell = (int)(w & 2047u), first = (int)((w >> 11) & 2047u);
+        const int cnt = q < num_cells ? (int)(w >> 22) : 0;
+        float one = 0.f;
+        for (int r = 0; r < most; r++) {
+            const int at = r < cnt ? first + r : first;
+            const int kk = tab[pairs + 2 * at + 1];
+            const float cf = r < cnt ? __int_as_float(tab[pairs + 2 * at]) : 0.f;
+            one += cf * __shfl(yreg, kk, kWave);
+        }
+        if (cnt > 0) {
+            const int slot = cell / kPlanX, j = cell % kPlanX;
+            M[(slot * XG + (j >> 2)) * 4 + (j & 3)] = one;
+        }
+    }
+}
+
 // Per-slot numbers of the plan, kept by a wave in two vector registers (lane t of register k
 // holds the number of slot 64 k + t) and read as wave-uniform values with lane reads.
 struct SlotWords {
@@ -363,6 +420,7 @@ __global__ __launch_bounds__(256, 2) void planned_fwd_kernel(
     const unsigned xoff = (unsigned)cr * (unsigned)lx.chan, soff = (unsigned)cr * (unsigned)ls.chan;
     const unsigned chunk_mask = (unsigned)plan[kChunkMask];
     const SlotWords slot_lw(plan + L.slot_lw, lane);
+    const HeldCells held(tab, num_cells, lane);
     float acc[NB * 16];
 #pragma unroll
     for (int t = 0; t < NB * 16; t++) acc[t] = 0.f;
@@ -383,7 +441,7 @@ __global__ __launch_bounds__(256, 2) void planned_fwd_kernel(
                 if (j >= X) xv[j] = 0.f;
             }
         }
-        build_edge_matrix<XG>(tab, num_cells, max_run, yreg, M, lane);
+        build_edge_matrix<XG>(tab, held, num_cells, max_run, yreg, M, lane);
         wave_lds_sync();
 #pragma unroll
         for (int b = 0; b < NB; b++) {
