@@ -12,6 +12,7 @@
 #include <vector>
 
 #include "common.h"
+#include "row_pieces.h"
 
 namespace e3j_amd {
 
@@ -303,7 +304,27 @@ int e3j_amd_convolution_fwd(const e3j_amd_conv_params *p, const void *coef, cons
         return set_error(E3J_AMD_UNIMPLEMENTED,
                          "convolution: row_cap / segments are taken by the unrolled kernels of the "
                          "trailing layout only (16-byte aligned operands)");
-    if (signature_fits(p, {x, s, out})) {
+    if (signature_fits(p, {x, s, out}) && p->segments != nullptr && p->partials != nullptr) {
+        // the pieces of long rows in a fixed order: every piece sums into a scratch row of its own
+        // (the launch names the piece's number as its row), then the rows of a receiver's pieces
+        // are added to its output row one after another
+        const int64_t row_floats = (int64_t)p->num_out * p->channels;
+        if (reinterpret_cast<uintptr_t>(p->partials) % 16 != 0)
+            return set_error(E3J_AMD_INVALID_ARGUMENT, "convolution: partials must be 16-byte aligned");
+        rc = launch_prepare_partials(p->segments, p->max_segments, row_floats, p->partials, stream);
+        if (rc == E3J_AMD_OK) {
+            e3j_amd_conv_params numbered = *p;
+            numbered.segments = row_partials_list(p->partials, p->max_segments, row_floats);
+            numbered.partials = nullptr;
+            rc = signature(p->signature).fwd(numbered, static_cast<const float *>(x), static_cast<const float *>(y),
+                                             static_cast<const float *>(s), sender, receiver_ptr, edge_perm,
+                                             p->partials, stream);
+        }
+        if (rc == E3J_AMD_OK)
+            rc = launch_combine_pieces(p->segments, receiver_ptr, p->max_segments,
+                                       p->row_piece > 0 ? p->row_piece : p->row_cap, row_floats, p->partials,
+                                       static_cast<float *>(out), stream);
+    } else if (signature_fits(p, {x, s, out})) {
         rc = signature(p->signature).fwd(*p, static_cast<const float *>(x), static_cast<const float *>(y),
                                          static_cast<const float *>(s), sender, receiver_ptr,
                                          edge_perm, static_cast<float *>(out), stream);
@@ -334,6 +355,11 @@ int e3j_amd_convolution_bwd_receiver(const e3j_amd_conv_params *p, const void *c
                                      void *stream) {
     return run_backward(p, true, coef, x, y, s, dm, sender, receiver_ptr, edge_perm, dx, dy, ds,
                         static_cast<hipStream_t>(stream), false);
+}
+
+size_t e3j_amd_row_partials_bytes(int64_t max_segments, int32_t num_out, int32_t channels) {
+    if (num_out <= 0 || channels <= 0) return 0;
+    return row_partials_bytes(max_segments, (int64_t)num_out * channels);
 }
 
 int e3j_amd_num_signatures(void) { return num_signatures(); }

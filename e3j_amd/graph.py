@@ -141,18 +141,32 @@ def row_cap_for(num_nodes: int, num_edges: int) -> int:
     return max(MIN_ROW_CAP, int(2 * mean))
 
 
+#: bytes of scratch the fixed-order sums of long rows may take (a row of the output per piece):
+#: larger graphs get longer pieces instead of more of them
+PARTIALS_BUDGET = 256 << 20
+
+
+def row_piece_for(num_edges: int, row_floats: int, row_piece: int = ROW_PIECE) -> int:
+    """Positions per piece such that a scratch row for every possible piece (`num_edges //
+    piece` of them, `row_floats` floats each) stays within `PARTIALS_BUDGET`."""
+    need = -(-int(num_edges) * int(row_floats) * 4 // PARTIALS_BUDGET)
+    return max(int(row_piece), need)
+
+
 class RowSegments:
     """The pieces of long rows for the second call of the forward pass
     (`e3j_amd_row_segments_build`).  `count`: pieces to launch, the bound `num_edges // row_piece`
     (the list's own count, which the kernel reads on the device, is never read back: the
-    surplus workgroups of the second call leave at once, which costs less than a wait)."""
+    surplus workgroups of the second call leave at once, which costs less than a wait).
+    `partials(num_out, channels)`: the scratch of the fixed-order sums (`e3j_amd_conv_params.partials`)."""
 
     def __init__(self, row_ptr: torch.Tensor, num_nodes: int, num_edges: int, row_cap: int,
                  row_piece: int = ROW_PIECE):
         device = _require_device(row_ptr)
         lib = _lib.load()
-        self.row_cap = int(row_cap)
+        self.row_cap = max(int(row_cap), int(row_piece)) if row_piece > ROW_PIECE else int(row_cap)
         self.row_piece = min(int(row_piece), self.row_cap)
+        self._partials = {}
         self.max_segments = int(lib.e3j_amd_row_segments_max(int(num_edges), self.row_piece))
         self.buffer = torch.empty(4 + 3 * self.max_segments, dtype=INDEX_DTYPE, device=device)
         with torch.cuda.device(device):
@@ -160,6 +174,14 @@ class RowSegments:
                 row_ptr.data_ptr(), int(num_nodes), self.row_cap, self.row_piece, self.max_segments,
                 self.buffer.data_ptr(), _stream_ptr(device)))
         self.count = self.max_segments
+
+    def partials(self, num_out: int, channels: int) -> torch.Tensor:
+        key = (int(num_out), int(channels))
+        hit = self._partials.get(key)
+        if hit is None:
+            nbytes = int(_lib.load().e3j_amd_row_partials_bytes(self.max_segments, *key))
+            hit = self._partials[key] = torch.empty(max(nbytes, 16), dtype=torch.uint8, device=self.buffer.device)
+        return hit
 
 
 class TileSchedule:

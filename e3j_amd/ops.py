@@ -26,7 +26,7 @@ import torch
 from . import _lib
 from .coef import Coef4D
 from .graph import (RowSegments, TileSchedule, csr_row_ptr, fold_endpoints, locality_order,
-                    pair_rows, row_cap_for, sort_edges, wrap_global_index)
+                    pair_rows, row_cap_for, row_piece_for, sort_edges, wrap_global_index, ROW_PIECE)
 from .options import GraphOrdering, Layout, config
 
 
@@ -286,12 +286,14 @@ class PreparedGraph:
         return hit
 
 
-    def segments(self, row_cap: int) -> RowSegments:
-        """The pieces of the rows longer than `row_cap` (second call of the forward pass)."""
-        hit = self._segments.get(row_cap)
+    def segments(self, row_cap: int, row_piece: int = ROW_PIECE) -> RowSegments:
+        """The pieces of the rows longer than `row_cap` (second call of the forward pass), of
+        `row_piece` positions each."""
+        key = (int(row_cap), int(row_piece))
+        hit = self._segments.get(key)
         if hit is None:
             self.ready()
-            hit = self._segments[row_cap] = RowSegments(self.row_ptr, self.num_nodes, self.num_edges, row_cap)
+            hit = self._segments[key] = RowSegments(self.row_ptr, self.num_nodes, self.num_edges, *key)
             self._mark()
         return hit
 
@@ -369,10 +371,13 @@ def _raw_forward(meta: _Meta, x, y, s, sender, receiver, graph=None) -> torch.Te
     else:
         out = torch.empty((x.shape[0], x.shape[1], meta.params.num_out), dtype=x.dtype, device=x.device)
     # Rows much longer than the mean are shared between waves: the first call cuts every row at
-    # `cap` positions, a second call adds the remaining pieces (unrolled kernels of the trailing
-    # layout; off in deterministic mode, where a row's sum must not depend on an order of atomics)
+    # `cap` positions, a second call sums the remaining pieces, each into a scratch row, and adds
+    # them to their output rows in a fixed order (unrolled kernels of the trailing layout): the
+    # result is the same bits in every run, as for a row that one wave sums
     cap = 0
-    if (p.signature >= 0 and meta.layout == Layout.TRAILING_CHANNELS and not config().deterministic
+    fixed_order = bool(config().fixed_order_rows)
+    if (p.signature >= 0 and meta.layout == Layout.TRAILING_CHANNELS
+            and (fixed_order or not config().deterministic)
             and isinstance(graph, PreparedGraph) and y.shape[0] > 0
             and all(t.data_ptr() % 16 == 0 for t in (x, s, out))):
         want = int(config().row_cap)
@@ -382,12 +387,16 @@ def _raw_forward(meta: _Meta, x, y, s, sender, receiver, graph=None) -> torch.Te
         args = (table.device(x.device).data_ptr(), x.data_ptr(), y.data_ptr(), s.data_ptr(),
                 other.data_ptr(), row_ptr.data_ptr(), perm.data_ptr() if perm is not None else None,
                 out.data_ptr(), _stream(x.device))
-        pieces = graph.segments(cap) if cap > 0 else None
-        if pieces is not None:
-            p.row_cap, p.row_piece = cap, pieces.row_piece
+        pieces = None
+        if cap > 0:
+            row_floats = int(out.shape[1]) * int(out.shape[2])
+            pieces = graph.segments(cap, row_piece_for(int(y.shape[0]), row_floats) if fixed_order else ROW_PIECE)
+            p.row_cap, p.row_piece = pieces.row_cap, pieces.row_piece
         _lib.check(lib.e3j_amd_convolution_fwd(ctypes.byref(p), *args))
         if pieces is not None and pieces.count > 0:
             p.segments, p.max_segments = pieces.buffer.data_ptr(), pieces.count
+            if fixed_order:
+                p.partials = pieces.partials(int(out.shape[1]), int(out.shape[2])).data_ptr()
             _lib.check(lib.e3j_amd_convolution_fwd(ctypes.byref(p), *args))
     return out
 

@@ -118,6 +118,11 @@ class Config:
     #: (their sums then come from float atomics).  -1: twice the mean row length, at least 64;
     #: 0: never share a row.
     row_cap: int = -1
+    #: add the pieces of a shared row to its output row in a fixed order (a scratch row per piece,
+    #: up to 256 MB per prepared graph; the forward then gives the same bits in every run, as the
+    #: reference's does); off: the pieces are added with float atomics (no scratch, and about 0.1 ms
+    #: less for a hub of 50 000 edges)
+    fixed_order_rows: bool = True
     #: compile unrolled kernels at run time for coefficient tables the library was not built
     #: for (needs hipcc; about half a minute per new table, cached on disk); off: such tables
     #: run the table-driven kernels.
@@ -134,6 +139,7 @@ class _ConfigHolder:
             locality_rounds=int(os.environ.get("E3J_AMD_LOCALITY_ROUNDS", "2")),
             tile_rows=int(os.environ.get("E3J_AMD_TILE_ROWS", "-1")),
             row_cap=int(os.environ.get("E3J_AMD_ROW_CAP", "-1")),
+            fixed_order_rows=os.environ.get("E3J_AMD_FIXED_ORDER_ROWS", "1") not in ("0", ""),
             pair_rows=os.environ.get("E3J_AMD_PAIR_ROWS", "0") not in ("0", ""),
             graph_cache=os.environ.get("E3J_AMD_GRAPH_CACHE", "0") not in ("0", ""),
             jit=os.environ.get("E3J_AMD_JIT", "0") not in ("0", ""),

@@ -87,11 +87,17 @@ typedef struct e3j_amd_conv_params {
      * e3j_amd_convolution_fwd with `segments` set, which ADDS to `out` with float atomics (so it
      * runs after the first call, on the same stream, and the sum of a split row depends on the
      * order of the additions).  segments: device, int32: [0] = number of pieces n (at most
-     * max_segments are run), [4 + 3 i ...] = (row, first position, end position) of piece i. */
+     * max_segments are run), [4 + 3 i ...] = (row, first position, end position) of piece i.
+     * partials (optional, with `segments`): device scratch of e3j_amd_row_partials_bytes bytes,
+     * 16-byte aligned.  The second call then sums every piece into a scratch row of its own and
+     * adds the rows of a receiver's pieces to its output row one after another, in the order of
+     * their positions: the result is the same bits in every run (the list must keep the pieces of
+     * one row adjacent and in position order, as e3j_amd_row_segments_build writes it). */
     int32_t row_cap;
     int32_t row_piece;
     int32_t max_segments;
     const int32_t *segments;
+    float *partials;
 } e3j_amd_conv_params;
 
 /* Message of the last failure on the calling thread ("" if none). */
@@ -182,6 +188,9 @@ typedef struct e3j_amd_tile_schedule {
  * reference, whose forward kernel also walks the edges of a receiver one after another in one
  * block (lib/e3j_ops/cuda/convolution/fwd.cuh:346-363). */
 int64_t e3j_amd_row_segments_max(int64_t num_edges, int32_t row_piece);
+/* Bytes of e3j_amd_conv_params.partials for a list of up to max_segments pieces: a row of
+ * num_out * channels floats per piece and a numbered copy of the list. */
+size_t e3j_amd_row_partials_bytes(int64_t max_segments, int32_t num_out, int32_t channels);
 int e3j_amd_row_segments_build(const int32_t *receiver_ptr, int32_t num_nodes, int32_t row_cap,
                                int32_t row_piece, int32_t max_segments, int32_t *segments,
                                void *stream);
