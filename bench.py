@@ -711,7 +711,9 @@ def main():
         },
         "roofline": {
             "bound": "hbm",
-            "kernel": ("convolution backward, atomic-free (position sort + unrolled_bwd_kernel + fixed-order "
+            "kernel": ("convolution backward, table-driven (plan_build_kernel + planned_bwd_kernel + dx zero fill)"
+                       if abi.signature < 0 else
+                       "convolution backward, atomic-free (position sort + unrolled_bwd_kernel + fixed-order "
                        "dx/dy reductions)" if args.deterministic else
                        "convolution backward over tiles of receivers (unrolled_bwd_tile_kernel + dx zero fill)"
                        if tiled else "convolution backward (unrolled_bwd_kernel + dx zero fill)"),
