@@ -3,6 +3,9 @@
 from __future__ import annotations
 
 
+import collections
+import hashlib
+
 import numpy as np
 
 from oracle import conv_oracle as O
@@ -71,20 +74,55 @@ def pack_table(idx, val, mix_idx, val_dtype=np.float32, idx_dtype=None):
 # ---------------------------------------------------------------------------
 # parity criterion
 # ---------------------------------------------------------------------------
+# The float64 references of a test are remembered by the content of their operands: tests that
+# run one workload through several launch shapes, layouts or tile sizes compute them once.
+_REFERENCES: "collections.OrderedDict[bytes, tuple]" = collections.OrderedDict()
+_REFERENCE_BUDGET = 3 << 30  # bytes of results kept
+
+
+def _nbytes(v):
+    return sum(_nbytes(t) for t in v) if isinstance(v, tuple) else int(np.asarray(v).nbytes)
+
+
+def _remembered(tag, arrays, extra, compute):
+    h = hashlib.blake2b(repr((tag, extra)).encode(), digest_size=16)
+    for a in arrays:
+        a = np.ascontiguousarray(a)
+        h.update(repr((a.dtype.str, a.shape)).encode())
+        h.update(a.view(np.uint8).reshape(-1).data)
+    key = h.digest()
+    if key in _REFERENCES:
+        _REFERENCES.move_to_end(key)
+        return _REFERENCES[key]
+    value = compute()
+    _REFERENCES[key] = value
+    while len(_REFERENCES) > 1 and sum(_nbytes(v) for v in _REFERENCES.values()) > _REFERENCE_BUDGET:
+        _REFERENCES.popitem(last=False)
+    return value
+
+
 def forward_reference(idx, val, mix, x, y, s, snd, rcv, num_out, leading=False):
-    """float64 value and the sum of absolute terms of every output element."""
-    ref = O.convolution_unfused(idx, val, mix, x, y, s, snd, rcv, num_out, leading=leading,
-                                dtype=np.float64)
-    mag = O.convolution_unfused(idx, np.abs(val), mix, np.abs(x), np.abs(y), np.abs(s), snd, rcv,
-                                num_out, leading=leading, dtype=np.float64)
-    return ref, mag
+    """float64 value and the sum of absolute terms of every output element (read-only arrays)."""
+    def compute():
+        ref = O.convolution_unfused(idx, val, mix, x, y, s, snd, rcv, num_out, leading=leading,
+                                    dtype=np.float64)
+        mag = O.convolution_unfused(idx, np.abs(val), mix, np.abs(x), np.abs(y), np.abs(s), snd, rcv,
+                                    num_out, leading=leading, dtype=np.float64)
+        for a in (ref, mag):
+            a.setflags(write=False)
+        return ref, mag
+    return _remembered("forward", (idx, val, mix, x, y, s, snd, rcv), (int(num_out), bool(leading)), compute)
 
 
 def backward_reference(idx, val, mix, x, y, s, snd, rcv, dm, leading=False):
-    ref = O.convolution_vjp(idx, val, mix, x, y, s, snd, rcv, dm, leading=leading, dtype=np.float64)
-    mag = O.convolution_vjp(idx, np.abs(val), mix, np.abs(x), np.abs(y), np.abs(s), snd, rcv,
-                            np.abs(dm), leading=leading, dtype=np.float64)
-    return ref, mag
+    def compute():
+        ref = O.convolution_vjp(idx, val, mix, x, y, s, snd, rcv, dm, leading=leading, dtype=np.float64)
+        mag = O.convolution_vjp(idx, np.abs(val), mix, np.abs(x), np.abs(y), np.abs(s), snd, rcv,
+                                np.abs(dm), leading=leading, dtype=np.float64)
+        for a in tuple(ref) + tuple(mag):
+            a.setflags(write=False)
+        return tuple(ref), tuple(mag)
+    return _remembered("backward", (idx, val, mix, x, y, s, snd, rcv, dm), (bool(leading),), compute)
 
 
 def assert_parity(result, ref64, mag64, what="", rtol=1e-5, atol=1e-6, ulps=16.0):

@@ -120,7 +120,8 @@ def _odd_graph(rng, n, kind):
 @pytest.mark.parametrize("tile_rows,max_work", [(16, 2048), (1, 2048), (5, 7), (16, 64), (3, 1)])
 @pytest.mark.parametrize("kind", ["cfg3", "cfg3_k64", "cfg2_k256ish", "hubs", "padding", "one_sender", "unsorted"])
 def test_tiled_backward_matches_oracle(kind, tile_rows, max_work):
-    rng = np.random.default_rng(zlib.crc32(f"{kind}/{tile_rows}".encode()))
+    # (the large cases keep one problem for every tile shape: their float64 reference is computed once)
+    rng = np.random.default_rng(zlib.crc32((kind if kind == "unsorted" else f"{kind}/{tile_rows}").encode()))
     if kind == "cfg3":
         w = W.config3(0.006)
     elif kind == "cfg3_k64":
