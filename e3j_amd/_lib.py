@@ -45,6 +45,7 @@ class ConvParams(ctypes.Structure):
         ("max_segments", ctypes.c_int32),
         ("segments", ctypes.c_void_p),
         ("partials", ctypes.c_void_p),
+        ("table_plan", ctypes.c_void_p),
     ]
 
 
@@ -133,6 +134,7 @@ SYMBOLS = {
     "e3j_amd_set_launch_variant": (None, [ctypes.c_int32, ctypes.c_int32]),
     "e3j_amd_set_table_plans": (None, [ctypes.c_int32]),
     "e3j_amd_row_partials_bytes": (ctypes.c_size_t, [ctypes.c_int64, ctypes.c_int32, ctypes.c_int32]),
+    "e3j_amd_table_plan_bytes": (ctypes.c_size_t, [ctypes.POINTER(ConvParams)]),
     "e3j_amd_table_plan_status": (ctypes.c_int, [ctypes.POINTER(ConvParams), ctypes.c_void_p, ctypes.c_int32,
                                                  ctypes.POINTER(ctypes.c_int32), ctypes.c_void_p]),
     "e3j_amd_harmonics": (ctypes.c_int, [_P, ctypes.c_int64] + [ctypes.c_int32] * 4 + [_P, _P]),

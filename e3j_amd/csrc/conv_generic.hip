@@ -559,16 +559,27 @@ int launch_zero_padding(const e3j_amd_conv_params &p, const int32_t *other, cons
     return zero_padding<float>(p, other, row_ptr, perm, dy, ds, stream);
 }
 
-// The plan of a table the planned kernels can take (conv_planned.hip), in memory of the stream's
-// pool for the length of the call; none when the sizes are outside the plan's limits, when
-// planning is switched off, when the stream is being captured into a graph (the call then
-// allocates nothing) or when the pool gives nothing.
+// The plan of a table the planned kernels can take (conv_planned.hip): in the caller's memory
+// (e3j_amd_conv_params.table_plan) or, without it, in memory of the stream's pool for the length
+// of the call; none when the sizes are outside the plan's limits, when planning is switched off,
+// and, for pool memory, when the stream is being captured into a graph (the call then allocates
+// nothing) or when the pool gives nothing.
 struct PlanScratch {
     int32_t *plan = nullptr;
+    bool pooled = false;  // plan memory taken from the stream's pool (given back when the call returns)
     hipStream_t stream;
     int rc = E3J_AMD_OK;
     PlanScratch(const e3j_amd_conv_params &p, const void *coef, bool cols_ji, hipStream_t st) : stream(st) {
         if (!plan_takes(p) || !table_plans().load(std::memory_order_relaxed)) return;
+        if (p.table_plan != nullptr) {  // the caller's memory: nothing allocated, fine under capture
+            if (reinterpret_cast<uintptr_t>(p.table_plan) % alignof(int32_t) != 0) {
+                rc = set_error(E3J_AMD_INVALID_ARGUMENT, "convolution: table_plan must be 4-byte aligned");
+                return;
+            }
+            plan = p.table_plan;
+            rc = launch_plan_build(p, coef, cols_ji, plan, stream);
+            return;
+        }
         hipStreamCaptureStatus capture = hipStreamCaptureStatusNone;
         if (hipStreamIsCapturing(stream, &capture) != hipSuccess) {
             (void)hipGetLastError();
@@ -581,10 +592,11 @@ struct PlanScratch {
             return;
         }
         plan = static_cast<int32_t *>(mem);
+        pooled = true;
         rc = launch_plan_build(p, coef, cols_ji, plan, stream);
     }
     ~PlanScratch() {
-        if (plan) (void)hipFreeAsync(plan, stream);
+        if (pooled) (void)hipFreeAsync(plan, stream);
     }
     PlanScratch(const PlanScratch &) = delete;
     PlanScratch &operator=(const PlanScratch &) = delete;

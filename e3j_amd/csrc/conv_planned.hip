@@ -62,3 +62,8 @@ extern "C" int e3j_amd_table_plan_status(const e3j_amd_conv_params *p, const voi
     status[3] = header[kNumZeroL];
     return E3J_AMD_OK;
 }
+
+extern "C" size_t e3j_amd_table_plan_bytes(const e3j_amd_conv_params *p) {
+    using namespace e3j_amd;
+    return (p != nullptr && plan_takes(*p)) ? plan_bytes(*p) : 0;
+}

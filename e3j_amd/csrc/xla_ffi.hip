@@ -16,7 +16,9 @@
 // coef_stacked (optional).  Without `signature` the handler finds the kernels of the table the
 // frame carries (see TableResolver).  Handlers are re-entrant (the only shared state is that
 // lookup, behind a mutex), allocate nothing themselves ("convolution_bwd" borrows scratch from the
-// runtime through XLA_FFI_DeviceMemory_Allocate when it runs the unrolled kernels) and enqueue
+// runtime through XLA_FFI_DeviceMemory_Allocate when it runs the unrolled kernels, and so does a
+// table-driven call for the plan of its table; a runtime without such memory leaves the latter to
+// the stream's pool) and enqueue
 // on the stream XLA hands over; they answer the metadata query.
 //
 // The row-wise tensor product (lib/e3j_ops/ffi/e3j_ops.h:124-253,258-372):
@@ -278,6 +280,50 @@ enum class Backward { kSenderRows, kReceiverRows, kReceiverRowsOrdered };
 
 size_t align256(size_t n) { return (n + 255) / 256 * 256; }
 
+// Scratch memory of the runtime for the length of a handler call (XLA_FFI_DeviceMemory_Allocate /
+// _Free; the runtime's allocator orders the reuse of the block after the work enqueued on the
+// call's stream).  `data` stays null when the runtime offers none or nothing is asked for.
+struct RuntimeScratch {
+    XlaCallFrame *frame;
+    void *data = nullptr;
+    size_t size;
+    RuntimeScratch(XlaCallFrame *f, size_t bytes) : frame(f), size(bytes) {
+        const XlaApi *api = f->api;
+        if (bytes == 0 || api->struct_size < offsetof(XlaApi, device_memory_free) + sizeof(void *) ||
+            api->device_memory_allocate == nullptr || api->device_memory_free == nullptr)
+            return;
+        XlaDeviceMemoryAllocateArgs get;
+        get.struct_size = sizeof(get);
+        get.extension_start = nullptr;
+        get.ctx = f->ctx;
+        get.size = bytes;
+        get.alignment = 256;
+        get.data = nullptr;
+        if (api->device_memory_allocate(&get) == nullptr) data = get.data;
+    }
+    ~RuntimeScratch() {
+        if (data == nullptr) return;
+        XlaDeviceMemoryFreeArgs give;
+        give.struct_size = sizeof(give);
+        give.extension_start = nullptr;
+        give.ctx = frame->ctx;
+        give.size = size;
+        give.data = data;
+        (void)frame->api->device_memory_free(&give);
+    }
+    RuntimeScratch(const RuntimeScratch &) = delete;
+    RuntimeScratch &operator=(const RuntimeScratch &) = delete;
+};
+
+// The plan of a table-driven call in the runtime's memory: the library then allocates nothing and
+// the planned kernels also run while the runtime records the stream into a graph.
+struct TablePlanMemory : RuntimeScratch {
+    TablePlanMemory(XlaCallFrame *f, e3j_amd_conv_params *p)
+        : RuntimeScratch(f, p->signature < 0 ? e3j_amd_table_plan_bytes(p) : 0) {
+        p->table_plan = static_cast<int32_t *>(data);
+    }
+};
+
 // "convolution_bwd" as the reference sends it (receiver_t per position of the sender-grouped
 // adjacency, sender_ptr, edge_perm) on the receiver-grouped unrolled kernels: positions are
 // sorted by receiver (stable), which gives sender per position, receiver_ptr and, composed with
@@ -392,6 +438,7 @@ void *backward_handler(XlaCallFrame *f, Backward mode) {
             workspace->data, d.stream);
         return status_to_error(f, rc);
     }
+    const TablePlanMemory plan(f, &d.p);
     const int rc = run_backward(&d.p, group_is_receiver, coef->data, x->data, y->data, s->data, dm->data,
                                 static_cast<const int32_t *>(other->data),
                                 static_cast<const int32_t *>(row_ptr->data), perm_ptr, dx->data,
@@ -476,6 +523,7 @@ void *e3j_amd_xla_convolution(void *call_frame) {
     d.p.num_coef = (int32_t)coef->dims[0];
     if (void *err = choose_kernels(f, "convolution", coef, false, &d.p, d.stream)) return err;
     const int32_t *perm_ptr = (perm && count(perm)) ? static_cast<const int32_t *>(perm->data) : nullptr;
+    const TablePlanMemory plan(f, &d.p);
     const int rc = e3j_amd_convolution_fwd(&d.p, coef->data, x->data, y->data, s->data,
                                            static_cast<const int32_t *>(sender->data),
                                            static_cast<const int32_t *>(row_ptr->data), perm_ptr,

@@ -200,6 +200,19 @@ def _fill_params(meta: _Meta, x: torch.Tensor, y: torch.Tensor, s: torch.Tensor,
     return p, table
 
 
+def _table_plan(p, device) -> torch.Tensor | None:
+    """Memory for the plan of a table-driven call (the caller keeps it until the call is enqueued):
+    with it the library allocates nothing, also while the stream is captured into a graph."""
+    if p.signature >= 0:
+        return None
+    nbytes = int(_lib.load().e3j_amd_table_plan_bytes(ctypes.byref(p)))
+    if nbytes == 0:
+        return None
+    plan = torch.empty((nbytes + 3) // 4, dtype=torch.int32, device=device)
+    p.table_plan = plan.data_ptr()
+    return plan
+
+
 def _check_operands(x, y, s, sender, receiver):
     for name, t in (("x", x), ("y", y), ("s", s), ("sender", sender), ("receiver", receiver)):
         if not isinstance(t, torch.Tensor):
@@ -384,6 +397,7 @@ def _raw_forward(meta: _Meta, x, y, s, sender, receiver, graph=None) -> torch.Te
         cap = row_cap_for(x.shape[0], y.shape[0]) if want < 0 else want
     lib = _lib.load()
     with torch.cuda.device(x.device):
+        plan = _table_plan(p, x.device)  # noqa: F841 (kept alive until the call is enqueued)
         args = (table.device(x.device).data_ptr(), x.data_ptr(), y.data_ptr(), s.data_ptr(),
                 other.data_ptr(), row_ptr.data_ptr(), perm.data_ptr() if perm is not None else None,
                 out.data_ptr(), _stream(x.device))
@@ -459,6 +473,7 @@ def _raw_backward(meta: _Meta, x, y, s, dm, sender, receiver, graph=None):
     if group_receiver and not ordered and y.shape[0] > 0 and p.layout == _lib.LAYOUT_TRAILING and aligned:
         tile_rows = _tile_rows(p.signature)
     with torch.cuda.device(x.device):
+        plan = _table_plan(p, x.device)  # noqa: F841 (kept alive until the call is enqueued)
         if tile_rows >= 1:
             if prepared is None:
                 prepared = PreparedGraph(other, row_ptr, perm, order, n)

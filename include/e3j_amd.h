@@ -98,6 +98,12 @@ typedef struct e3j_amd_conv_params {
     int32_t max_segments;
     const int32_t *segments;
     float *partials;
+    /* Table-driven kernels: optional device memory of e3j_amd_table_plan_bytes bytes for the plan
+     * of the table (see e3j_amd_set_table_plans), 4-byte aligned.  The call writes the plan there
+     * and reads it back on the same stream (calls that share the memory must not overlap).  With
+     * it the call allocates nothing and the planned kernels also run on a stream that is being
+     * captured into a graph; NULL: memory from the stream's pool, and none under capture. */
+    int32_t *table_plan;
 } e3j_amd_conv_params;
 
 /* Message of the last failure on the calling thread ("" if none). */
@@ -250,8 +256,10 @@ void e3j_amd_set_launch_variant(int32_t fwd_variant, int32_t bwd_variant);
  * kernels that keep x and the accumulators in registers; any other table and float64 run the
  * kernels that index LDS columns by the table's coordinates (float16 there: arithmetic in half).  Whether a table fits is
  * decided on the device, without a read-back.  on = 0 switches the planned form off for later
- * calls (process-wide, atomic; initial value from E3J_AMD_TABLE_PLANS, default 1); a call on a
- * stream that is being captured into a graph allocates nothing and runs the LDS-column kernels.  Results
+ * calls (process-wide, atomic; initial value from E3J_AMD_TABLE_PLANS, default 1).  The plan (a few
+ * KB) lives in e3j_amd_conv_params.table_plan when the caller brings that memory, else in memory of
+ * the stream's pool for the length of the call; without the caller's memory a call on a stream that
+ * is being captured into a graph allocates nothing and runs the LDS-column kernels.  Results
  * agree to rounding (the planned form sums per output coordinate in a different order).
  * No counterpart in the reference, which has one table-driven kernel
  * (lib/e3j_ops/cuda/convolution/fwd.cuh:88-153). */
@@ -265,6 +273,10 @@ void e3j_amd_set_table_plans(int32_t on);
  * synchronises: for tests and set-up code, not for the hot path. */
 int e3j_amd_table_plan_status(const e3j_amd_conv_params *p, const void *coef, int32_t coef_cols_ji,
                               int32_t *status, void *stream);
+/* Bytes of e3j_amd_conv_params.table_plan for the sizes in `p` (num_coef, num_scalars and the
+ * dimensions); 0 when the planned form does not take these sizes or this value type (nothing to
+ * bring then). */
+size_t e3j_amd_table_plan_bytes(const e3j_amd_conv_params *p);
 
 /* Adds a signature compiled at run time (e3j_amd/jit.py generates the kernels of a table
  * the library was not built for, compiles them against this library and hands over the entry

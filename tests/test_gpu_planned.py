@@ -317,3 +317,83 @@ def test_a_call_recorded_into_a_graph_allocates_nothing_and_replays():
         torch.cuda.synchronize()
         for a, b, name in zip(replayed, (out, dx, dy, ds), ("out", "dx", "dy", "ds")):
             assert float((a - b).abs().max()) <= 5e-5 * float(b.abs().max()), (trial, name)
+
+
+def test_plan_memory_of_the_caller_serves_eager_calls_and_graph_capture():
+    """With `table_plan` memory from the caller the call takes nothing from the stream's pool and a
+    captured call records the planned kernels: the forward of every replay has the bits of an eager
+    planned call (the LDS-column kernels round differently), the backward agrees to the order of its
+    dx atomics; the size comes from `e3j_amd_table_plan_bytes`, which answers 0 for what the plan
+    does not take."""
+    w = W.config3(0.002)
+    idx, val, mix = w.table()
+    rng = np.random.default_rng(91)
+    N, E, K = 40, 600, 64
+    snd, rcv = H.random_graph(rng, N, E)
+    packed = H.pack_table(idx, val, mix)
+    coef_d = _dev(packed.view(np.uint8).reshape(-1))
+    x, y, s, dm = (_dev(a) for a in H.random_operands(rng, N, E, 16, 16, 23, K, 99))
+    other, ptr_d = _dev(snd.astype(np.int32)), _dev(O.receiver_ptr(rcv, N))
+    lib = _lib.load()
+    p = _params(N, E, len(packed), 16, 16, 99, 23, K, 1, _lib.F32, packed.dtype.itemsize, debug=0)
+    nbytes = int(lib.e3j_amd_table_plan_bytes(ctypes.byref(p)))
+    assert 0 < nbytes < (1 << 20) and nbytes % 4 == 0
+    wide = _params(N, E, len(packed), 16, 16, 99, 23, K, 1, _lib.F64, packed.dtype.itemsize, debug=0)
+    assert int(lib.e3j_amd_table_plan_bytes(ctypes.byref(wide))) == 0          # float64: LDS columns
+    big = _params(N, E, len(packed), 17, 16, 99, 23, K, 1, _lib.F32, packed.dtype.itemsize, debug=0)
+    assert int(lib.e3j_amd_table_plan_bytes(ctypes.byref(big))) == 0           # 17 x coordinates
+    plan = torch.full((nbytes // 4,), -1, dtype=torch.int32, device="cuda")
+    out = torch.empty((N, 99, K), device="cuda")
+    dx, dy, ds = torch.empty_like(x), torch.empty_like(y), torch.empty_like(s)
+
+    def launch(params, stream):
+        _lib.check(lib.e3j_amd_convolution_fwd(ctypes.byref(params), coef_d.data_ptr(), x.data_ptr(), y.data_ptr(),
+                                               s.data_ptr(), other.data_ptr(), ptr_d.data_ptr(), None,
+                                               out.data_ptr(), stream))
+        _lib.check(lib.e3j_amd_convolution_bwd_receiver(
+            ctypes.byref(params), coef_d.data_ptr(), x.data_ptr(), y.data_ptr(), s.data_ptr(), dm.data_ptr(),
+            other.data_ptr(), ptr_d.data_ptr(), None, dx.data_ptr(), dy.data_ptr(), ds.data_ptr(), stream))
+
+    def results():
+        torch.cuda.synchronize()
+        return [t.clone() for t in (out, dx, dy, ds)]
+
+    current = torch.cuda.current_stream().cuda_stream
+    launch(p, current)
+    pooled = results()                               # plan memory from the stream's pool
+    lib.e3j_amd_set_table_plans(0)
+    try:
+        launch(p, current)
+        columns = results()
+    finally:
+        lib.e3j_amd_set_table_plans(1)
+    assert not torch.equal(pooled[0], columns[0]), "the two forms round differently on this problem"
+    p.table_plan = plan.data_ptr()
+    launch(p, current)
+    own = results()
+    assert int(plan[0].item()) == 1                  # the plan was written to the caller's memory
+    assert torch.equal(own[0], pooled[0]) and torch.equal(own[3], pooled[3])
+    p.table_plan = plan.data_ptr() + 2
+    with pytest.raises(_lib.E3jAmdError, match="aligned"):
+        launch(p, current)
+    p.table_plan = plan.data_ptr()
+
+    side = torch.cuda.Stream()
+    side.wait_stream(torch.cuda.current_stream())
+    torch.cuda.synchronize()
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph, stream=side):
+        launch(p, side.cuda_stream)
+    for trial in range(3):
+        gen = torch.Generator(device="cuda").manual_seed(300 + trial)
+        for t in (x, y, s, dm):
+            t.copy_(torch.randn(t.shape, device="cuda", generator=gen))
+        (x.sum() + s.sum()).item()                   # unrelated eager work and a synchronisation
+        graph.replay()
+        replayed = results()
+        launch(p, torch.cuda.current_stream().cuda_stream)
+        eager = results()
+        assert torch.equal(replayed[0], eager[0]), trial         # forward: the planned kernels' bits
+        assert torch.equal(replayed[3], eager[3]), trial         # ds belongs to the edge alone
+        for a, b, name in zip(replayed[1:3], eager[1:3], ("dx", "dy")):
+            assert float((a - b).abs().max()) <= 5e-5 * float(b.abs().max()), (trial, name)

@@ -93,6 +93,24 @@ def test_forward_and_both_backward_targets():
                       [_buf(xla, dx, F32), _buf(xla, dy, F32), _buf(xla, ds, F32)], attrs())
     assert lib.e3j_amd_xla_convolution_bwd_receiver(C.addressof(frame)) is None, xla.errors
     check(dx, dy, ds, "receiver grouping")
+
+    # a runtime that hands out scratch: the plan of the table lives there for the length of a call
+    xla.allocate = lambda nbytes: torch.empty(nbytes, dtype=torch.uint8, device="cuda")
+    dx, dy, ds = (torch.full_like(t, float("nan")) for t in (xd, yd, sd))
+    frame = xla.frame([_buf(xla, coef, U8), _buf(xla, xd, F32), _buf(xla, yd, F32), _buf(xla, sd, F32),
+                       _buf(xla, dmd, F32), _buf(xla, dev(snd), S32), _buf(xla, ptr, S32),
+                       xla.buffer(S32, 0, (0,))],
+                      [_buf(xla, dx, F32), _buf(xla, dy, F32), _buf(xla, ds, F32)], attrs())
+    assert lib.e3j_amd_xla_convolution_bwd_receiver(C.addressof(frame)) is None, xla.errors
+    check(dx, dy, ds, "receiver grouping, plan in the runtime's scratch")
+    out2 = torch.full_like(out, float("nan"))
+    frame = xla.frame([_buf(xla, coef, U8), _buf(xla, xd, F32), _buf(xla, yd, F32), _buf(xla, sd, F32),
+                       _buf(xla, dev(snd), S32), _buf(xla, ptr, S32), _buf(xla, ranges, S32)],
+                      [_buf(xla, out2, F32)], attrs())
+    assert lib.e3j_amd_xla_convolution(C.addressof(frame)) is None, xla.errors
+    torch.cuda.synchronize()
+    H.assert_parity(out2.cpu().numpy(), ref, mag, "xla out, plan in the runtime's scratch")
+    assert xla.allocations == 2 and not xla.scratch   # borrowed once per call and handed back
     del empty, keep
 
 
