@@ -34,13 +34,17 @@ _loaded = {}   # key -> (ctypes.CDLL kept alive, [signature ids])
 _failed = set()
 
 
+# the parameter structs the compiled kernels read
+_PUBLIC_HEADER = os.path.join(os.path.dirname(os.path.dirname(os.path.abspath(__file__))), "include", "e3j_amd.h")
+
+
 def _key(val: np.ndarray, idx4: np.ndarray, dims, channels: int) -> str:
     h = hashlib.sha256()
     h.update(np.ascontiguousarray(val, dtype=np.float32).tobytes())
     h.update(np.ascontiguousarray(idx4, dtype=np.int64).tobytes())
     h.update(repr((tuple(int(d) for d in dims), int(channels))).encode())
     for path in (gen_conv.__file__, os.path.join(_build.CSRC, "unrolled.h"),
-                 os.path.join(_build.CSRC, "common.h")):
+                 os.path.join(_build.CSRC, "common.h"), _PUBLIC_HEADER):
         with open(path, "rb") as fh:      # kernels of another version of the templates are stale
             h.update(fh.read())
     return h.hexdigest()[:20]
@@ -135,7 +139,8 @@ def _tp_key(val: np.ndarray, idx: np.ndarray, shape, channels: int) -> str:
     h.update(np.ascontiguousarray(idx, dtype=np.int64).tobytes())
     h.update(repr((tuple(int(d) for d in shape), int(channels))).encode())
     for path in (gen_tp.__file__, os.path.join(_build.CSRC, "tp_unrolled.h"),
-                 os.path.join(_build.CSRC, "unrolled.h"), os.path.join(_build.CSRC, "common.h")):
+                 os.path.join(_build.CSRC, "unrolled.h"), os.path.join(_build.CSRC, "common.h"),
+                 _PUBLIC_HEADER):
         with open(path, "rb") as fh:
             h.update(fh.read())
     return h.hexdigest()[:20]
