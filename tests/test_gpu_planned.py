@@ -129,6 +129,49 @@ def test_planned_kernels_match_oracle(X, Y, Z, S, nnz, channels, grouping):
     check_all(idx, val, mix, x, y, s, dm, snd, rcv, Z, res, tag=f"{(X, Y, Z, S)} K={channels} {grouping}")
 
 
+@pytest.mark.parametrize("seed", range(24))
+def test_seeded_random_tables_and_graphs(seed):
+    """Random sizes within the plan's limits, tables with holes (output coordinates and scalars no
+    entry uses), graphs with empty rows, a hub, padding edges and unsorted edges behind a
+    permutation, both layouts, both index widths, both groupings: the planned kernels against the
+    CPU oracle."""
+    rng = np.random.default_rng(7000 + seed)
+    X, Y, Z = int(rng.integers(1, 17)), int(rng.integers(1, 65)), int(rng.integers(1, 129))
+    S = int(rng.integers(1, min(Z, 64) + 1))
+    nnz = int(rng.integers(max(X, Y, Z), min(2048, 6 * max(X, Y, Z)) + 1))
+    K = int(rng.choice([1, 3, 32, 64, 65, 128, 200]))
+    N, E = int(rng.integers(1, 30)), int(rng.integers(0, 400))
+    idx, val, mix = H.random_table(rng, nnz, X, Y, Z, S)
+    if rng.random() < 0.4 and len(val) > 4:
+        keep = rng.random(len(val)) < 0.7
+        keep[0] = True
+        idx, val = idx[keep], val[keep]
+    idx_dtype = np.int32 if rng.random() < 0.3 else None
+    assert _status(H.pack_table(idx, val, mix, idx_dtype=idx_dtype), X, Y, Z, S)[0] == 1
+    snd, rcv = H.random_graph(rng, N, E) if E else (np.zeros(0, np.int32), np.zeros(0, np.int32))
+    grouping = "receiver" if rng.random() < 0.6 else "sender"
+    if E and rng.random() < 0.5:                                   # a hub takes most of the edges
+        rcv = rcv.copy()
+        rcv[rng.random(E) < 0.6] = int(rng.integers(0, N))
+        order = np.argsort(rcv, kind="stable")
+        snd, rcv = snd[order], rcv[order]
+    if E and grouping == "receiver" and rng.random() < 0.3:        # padding edges
+        snd = snd.copy()
+        snd[rng.random(E) < 0.2] = O.DUMMY_INDEX
+    perm = None
+    if E and grouping == "receiver" and rng.random() < 0.3:        # unsorted edges behind a permutation
+        shuffle = rng.permutation(E)
+        snd, rcv = snd[shuffle], rcv[shuffle]
+        perm = np.argsort(rcv, kind="stable").astype(np.int32)
+    x, y, s, dm = H.random_operands(rng, N, E, X, Y, S, K, Z)
+    leading = bool(rng.random() < 0.3)
+    args = [np.ascontiguousarray(a.swapaxes(1, 2)) if leading else a for a in (x, s, dm)]
+    res = run_abi(idx, val, mix, args[0], y, args[1], args[2], snd, rcv, Z, leading=leading, grouping=grouping,
+                  idx_dtype=idx_dtype, perm=perm)
+    check_all(idx, val, mix, args[0], y, args[1], args[2], snd, rcv, Z, res, leading=leading,
+              tag=f"seed {seed}: {(X, Y, Z, S)} nnz={len(val)} K={K} N={N} E={E} {grouping} leading={leading}")
+
+
 def test_l3_table_with_padding_edges_and_permutation():
     """cfg3's table (7 blocks x 4 groups, 14 visited) on unsorted edges with padding among them."""
     w = W.config3(0.002)
