@@ -13,8 +13,8 @@
 //   * the output coordinates in the order the loops visit them ("slots": sorted by the x
 //     coordinates their path touches, then by scalar, so that rows of one scalar are adjacent
 //     and blocks of 16 slots touch few groups of 4 x coordinates),
-//   * a bit per (block of 16 slots, group of 4 x coordinates) that has a coefficient at all: the
-//     loops skip the others with a wave-uniform branch,
+//   * a bit per (block of 16 slots, group of 4 x coordinates) that has a coefficient at all, and
+//     inside those a bit per half of 8 slots: the loops skip the others with wave-uniform branches,
 //   * the non-empty cells (slot, j) with their (coefficient, k) lists in table order.
 // The backward pass (lib/e3j_ops/cuda/convolution/bwd.cuh:116-321) uses the same M: ds from the
 // forward's partial sums, dx[j] += M[i][j] * s[l(i)] * dm[i], and for dy the per-channel products
@@ -50,7 +50,16 @@ constexpr int kPlanMaxRun = 255;    // entries of one cell
 constexpr int kBuildThreads = 256;
 
 // header words
-enum { kEligible = 0, kNumCells = 1, kChunkMask = 2, kNumZeroL = 3, kMaxRun = 4, kHeaderWords = 8 };
+enum { kEligible = 0, kNumCells = 1, kChunkMask = 2, kNumZeroL = 3, kMaxRun = 4, kHalfMask0 = 5, kHalfMask1 = 6,
+       kHeaderWords = 8 };
+
+// bit of (block b of 16 slots, group g of 4 x coordinates, half of 8 slots) in the 64-bit mask of halves
+// that hold a coefficient (two header words)
+template <int XG>
+__device__ __forceinline__ bool half_live(unsigned mask0, unsigned mask1, int b, int g, int half) {
+    const int bit = (b * XG + g) * 2 + half;
+    return (((bit < 32 ? mask0 >> bit : mask1 >> (bit - 32))) & 1u) != 0;
+}
 
 struct PlanLayout {  // offsets in 32-bit words
     // slot_row, slot_l: output coordinate and scalar of a slot; first, count: the entries of a dense
@@ -91,10 +100,10 @@ __global__ __launch_bounds__(kBuildThreads) void plan_build_kernel(
     int32_t *__restrict__ plan, PlanLayout L) {
     __shared__ int lmin[kSlots], lmax[kSlots], support[kSlots], slot_of_row[kSlots];
     __shared__ int path_support[kPlanMaxS], referenced[kPlanMaxS];
-    __shared__ int eligible, chunk_mask, num_cells, num_zero_l, max_run;
+    __shared__ int eligible, chunk_mask, half_mask[2], num_cells, num_zero_l, max_run;
     __shared__ int scan[kBuildThreads];
     const int tid = threadIdx.x;
-    if (tid == 0) { eligible = 1; chunk_mask = 0; num_cells = 0; num_zero_l = 0; max_run = 0; }
+    if (tid == 0) { eligible = 1; chunk_mask = 0; half_mask[0] = half_mask[1] = 0; num_cells = 0; num_zero_l = 0; max_run = 0; }
     for (int i = tid; i < kSlots; i += kBuildThreads) { lmin[i] = 0x7fffffff; lmax[i] = -1; support[i] = 0; }
     for (int l = tid; l < S; l += kBuildThreads) { path_support[l] = 0; referenced[l] = 0; }
     for (int c = tid; c < kCells; c += kBuildThreads) plan[L.count + c] = 0;
@@ -170,7 +179,10 @@ __global__ __launch_bounds__(kBuildThreads) void plan_build_kernel(
             at += c;
             if (c > 0) {
                 plan[L.cell_list + cell_at++] = cell;
-                atomicOr(&chunk_mask, 1 << ((cell / kPlanX / 16) * xg + (cell % kPlanX) / 4));
+                const int chunk = (cell / kPlanX / 16) * xg + (cell % kPlanX) / 4;
+                const int half = 2 * chunk + (cell / kPlanX) % 16 / 8;
+                atomicOr(&chunk_mask, 1 << chunk);
+                atomicOr(&half_mask[half >> 5], 1 << (half & 31));
             }
         }
         if (tid == kBuildThreads - 1) num_cells = scan[tid] >> 16;
@@ -222,6 +234,7 @@ __global__ __launch_bounds__(kBuildThreads) void plan_build_kernel(
     if (tid == 0) {
         plan[kEligible] = eligible; plan[kNumCells] = num_cells; plan[kChunkMask] = chunk_mask;
         plan[kNumZeroL] = num_zero_l; plan[kMaxRun] = max_run;
+        plan[kHalfMask0] = half_mask[0]; plan[kHalfMask1] = half_mask[1];
     }
 }
 
@@ -419,6 +432,7 @@ __global__ __launch_bounds__(256, 2) void planned_fwd_kernel(
     const int cr = active ? c : channels - 1;  // channel whose rows an idle lane reads
     const unsigned xoff = (unsigned)cr * (unsigned)lx.chan, soff = (unsigned)cr * (unsigned)ls.chan;
     const unsigned chunk_mask = (unsigned)plan[kChunkMask];
+    const unsigned half0 = (unsigned)plan[kHalfMask0], half1 = (unsigned)plan[kHalfMask1];
     const SlotWords slot_lw(plan + L.slot_lw, lane);
     const HeldCells held(tab, num_cells, lane);
     float acc[NB * 16];
@@ -456,12 +470,17 @@ __global__ __launch_bounds__(256, 2) void planned_fwd_kernel(
             for (int g = 0; g < XG; g++) {
                 if (!((chunk_mask >> (b * XG + g)) & 1u)) continue;
 #pragma unroll
-                for (int u = 0; u < 16; u++) {
-                    const f32x4 m = *reinterpret_cast<const f32x4 *>(&M[((b * 16 + u) * XG + g) * 4]);
-                    T[u] = __builtin_fmaf(m.x, xv[4 * g], T[u]);
-                    T[u] = __builtin_fmaf(m.y, xv[4 * g + 1], T[u]);
-                    T[u] = __builtin_fmaf(m.z, xv[4 * g + 2], T[u]);
-                    T[u] = __builtin_fmaf(m.w, xv[4 * g + 3], T[u]);
+                for (int half = 0; half < 2; half++) {
+                    if (!half_live<XG>(half0, half1, b, g, half)) continue;  // eight slots without a coefficient here
+#pragma unroll
+                    for (int uu = 0; uu < 8; uu++) {
+                        const int u = half * 8 + uu;
+                        const f32x4 m = *reinterpret_cast<const f32x4 *>(&M[((b * 16 + u) * XG + g) * 4]);
+                        T[u] = __builtin_fmaf(m.x, xv[4 * g], T[u]);
+                        T[u] = __builtin_fmaf(m.y, xv[4 * g + 1], T[u]);
+                        T[u] = __builtin_fmaf(m.z, xv[4 * g + 2], T[u]);
+                        T[u] = __builtin_fmaf(m.w, xv[4 * g + 3], T[u]);
+                    }
                 }
             }
 #pragma unroll
@@ -533,6 +552,7 @@ __global__ __launch_bounds__(256, 2) void planned_bwd_kernel(
     const int lane = threadIdx.x, wave = __builtin_amdgcn_readfirstlane((int)threadIdx.y);
     const int num_cells = plan[kNumCells];
     const unsigned chunk_mask = (unsigned)plan[kChunkMask];
+    const unsigned half0 = (unsigned)plan[kHalfMask0], half1 = (unsigned)plan[kHalfMask1];
     const int max_run = plan[kMaxRun];
     const int num_zero_l = plan[kNumZeroL];
     int32_t *tab = reinterpret_cast<int32_t *>(planned_lds);
@@ -611,6 +631,10 @@ __global__ __launch_bounds__(256, 2) void planned_bwd_kernel(
                     float part[2];
 #pragma unroll
                     for (int half = 0; half < 2; half++) {
+                        if (!half_live<XG>(half0, half1, b, gx, half)) {  // eight slots without a coefficient here
+                            part[half] = 0.f;
+                            continue;
+                        }
                         float G[32];
 #pragma unroll
                         for (int uu = 0; uu < 8; uu++) {
@@ -683,7 +707,7 @@ __global__ __launch_bounds__(256, 2) void planned_bwd_kernel(
     }
 }
 
-constexpr int kWavesPerBlock = 2;  // (120k edges, K = 128, l <= 3: forward 2.12 ms, backward 5.17 ms; four: 2.27 and 5.33; one: 2.10 and 6.07)
+constexpr int kWavesPerBlock = 2;  // (120k edges, K = 128, l <= 3, before the skip of empty halves: forward 2.12 ms, backward 5.17 ms; four: 2.27 and 5.33; one: 2.10 and 6.07)
 
 #define E3J_ROW(K, NB) {K<Val, NB, 1>, K<Val, NB, 2>, K<Val, NB, 3>, K<Val, NB, 4>}
 #define E3J_TABLE(K) {E3J_ROW(K, 1), E3J_ROW(K, 2), E3J_ROW(K, 3), E3J_ROW(K, 4), \
