@@ -126,8 +126,8 @@ def parse_args():
                     help="skip the leading-channels sub-record of the default run")
     ap.add_argument("--cpu-seconds", type=float, default=15.0)
     ap.add_argument("--table-driven", action="store_true",
-                    help="with --kernel-only: time the table-driven kernels (signature -1) instead of the "
-                         "unrolled ones; E3J_AMD_TABLE_PLANS=0 selects their form without a plan")
+                    help="time the table-driven kernels (signature -1) through the C ABI instead of the unrolled "
+                         "ones (implies --kernel-only); E3J_AMD_TABLE_PLANS=0 selects their form without a plan")
     ap.add_argument("--kernel-only", action="store_true",
                     help="time the C-ABI launches only (no operator-level step)")
     ap.add_argument("--spatial-sort", action="store_true",
@@ -646,6 +646,8 @@ def main():
     if args.calibrate_copy:
         calibrate_copy(torch, device)
 
+    if args.table_driven:
+        args.kernel_only = True   # the operators resolve the table to its unrolled kernels
     abi = AbiCalls(w, table_driven=args.table_driven)
     if args.deterministic:
         e3j_amd.config(deterministic=True)
