@@ -36,8 +36,9 @@ HBM_PEAK_GBS = 8000.0
 
 #: HBM bytes per launch come from `profiles/traffic.json`: two `rocprofv3 --pmc` runs of this
 #: script (FETCH_SIZE and WRITE_SIZE, KiB per dispatch), each scaled by what the same counter reads
-#: for a 1 GiB device copy (`--calibrate-copy`), written by `python bench.py --write-traffic ...`
-#: together with a hash of the kernel sources.  A figure is only quoted while the sources it was
+#: for a 1 GiB device copy (FETCH_SIZE counts half of the bytes read, factor 2.0; WRITE_SIZE all of
+#: the bytes written, factor 1.0; a copy kernel found in the CSVs overrides the two factors), written
+#: by `python bench.py --write-traffic ...` together with a hash of the kernel sources.  A figure is only quoted while the sources it was
 #: measured on are the ones in the tree.
 TRAFFIC_FILE = os.path.join(ROOT, "profiles", "traffic.json")
 KERNEL_SOURCES = ("e3j_amd/csrc/unrolled.h", "e3j_amd/csrc/common.h", "e3j_amd/csrc/tp_unrolled.h",
@@ -130,19 +131,8 @@ def parse_args():
                          "ones (implies --kernel-only); E3J_AMD_TABLE_PLANS=0 selects their form without a plan")
     ap.add_argument("--kernel-only", action="store_true",
                     help="time the C-ABI launches only (no operator-level step)")
-    ap.add_argument("--spatial-sort", action="store_true",
-                    help="cfg3 only: number the atoms along a space-filling curve instead of at random "
-                         "(a secondary figure; the headline keeps the random numbering)")
     ap.add_argument("--deterministic", action="store_true",
                     help="time the atomic-free (bit-reproducible) backward instead of the default one")
-    ap.add_argument("--access-floor", action="store_true",
-                    help="trailing layout, built-in tables at 64/128/256 channels: also time kernels that perform the "
-                         "memory accesses of the two passes without their arithmetic (reported under "
-                         "roofline.access_floor)")
-    ap.add_argument("--tile-sharing", action="store_true",
-                    help="also count, on the host, the dx atomic requests a backward over tiles of T receivers "
-                         "issues (distinct (tile, sender) pairs) for T = 2..32, with the library's row order and "
-                         "with rows along a space-filling curve of the atoms (reported under roofline.tile_sharing)")
     ap.add_argument("--inner", type=int, default=64, help="--op radial_linear: hidden size of the radial network")
     ap.add_argument("--op", default="convolution", choices=["convolution", "tensor_product", "radial_linear"],
                     help="convolution: the headline benchmark; tensor_product: a secondary figure, the "
@@ -152,23 +142,17 @@ def parse_args():
     ap.add_argument("--rows", type=int, default=1 << 18, help="--op tensor_product: number of rows")
     ap.add_argument("--write-traffic", nargs="+", metavar="CSV",
                     help="no GPU work: summarise rocprofv3 counter CSVs (FETCH_SIZE and WRITE_SIZE runs of this "
-                         "script with --calibrate-copy) into profiles/traffic.json for --config/--layout/--scale")
-    ap.add_argument("--tile-rows", type=int, default=None,
-                    help="receivers per tile of the tiled backward (default: the library's setting, 0 = one "
-                         "wave per receiver)")
-    ap.add_argument("--calibrate-copy", action="store_true",
-                    help="also run a 1 GiB device copy, the known-size kernel that hardware "
-                         "traffic counters are scaled by")
+                         "script) into profiles/traffic.json for --config/--layout/--scale")
     return ap.parse_args()
 
 
-def build_workload(name: str, scale: float, device, spatial_sort: bool = False, channels=None):
+def build_workload(name: str, scale: float, device, channels=None):
     from e3j_amd import workloads as W
     if name == "cfg2":
         return W.config2(scale, device=device)
     if name == "cfg4":
         return W.config4(scale, device=device)
-    return W.config3(scale, device=device, spatial_sort=spatial_sort, **({"channels": channels} if channels else {}))
+    return W.config3(scale, device=device, **({"channels": channels} if channels else {}))
 
 
 class AbiCalls:
@@ -264,74 +248,6 @@ class AbiCalls:
             self.dx.data_ptr(), self.dy.data_ptr(), self.ds.data_ptr(), self._stream()))
 
 
-#: access patterns of `--access-floor`: name -> mask of e3j_amd/csrc/probe/access_pattern.hip
-#: (1 read s, 2 gather x, 4 write ds, 8 dx atomics, 16 write out, 32 read dm, 64 the atomics of
-#: every second position only)
-ACCESS_PATTERNS = {
-    "read_s": 1,
-    "read_s+gather_x": 3,
-    "forward: read_s+gather_x+write_out": 19,
-    "write_ds": 4,
-    "read_s+write_ds": 5,
-    "read_s+write_ds+gather_x": 7,
-    "read_s+write_ds+gather_x+read_dm": 39,
-    "dx_atomics": 8,
-    "read_s+write_ds+gather_x+dx_atomics": 15,
-    "backward: read_s+write_ds+gather_x+dx_atomics+read_dm": 47,
-    "half_of_the_dx_atomics": 72,
-    "backward with half of the dx atomics": 111,
-}
-
-
-def tile_sharing(abi, w) -> dict:
-    """Share of the per-edge dx atomic requests left when the contributions of one sender are summed
-    within a tile of T receivers that are consecutive in the row order: distinct (tile, sender)
-    pairs over live edges.  Host arithmetic on the benchmark's graph; two row orders."""
-    import numpy as np
-    from e3j_amd.workloads import morton_order
-    n = w.num_nodes
-    ptr = abi.ptr.cpu().numpy().astype(np.int64)
-    snd = abi.other.cpu().numpy().astype(np.int64)[:ptr[n]]
-    rcv = np.repeat(np.arange(n), np.diff(ptr))
-    live = (snd >= 0) & (snd < n)
-    snd, rcv = snd[live], rcv[live]
-    orders = {"locality_order": (abi.order.cpu().numpy() if abi.order is not None else np.arange(n)),
-              "space_filling_curve": morton_order(np.asarray(w.positions), float(w.box))}
-    out = {}
-    for name, order in orders.items():
-        rank = np.empty(n, np.int64)
-        rank[order] = np.arange(n)
-        out[name] = {str(t): round(len(np.unique((rank[rcv] // t) * n + snd)) / max(len(snd), 1), 4)
-                     for t in (1, 2, 4, 8, 16, 32)}
-    return out
-
-
-def access_floor(torch, abi, steps: int) -> dict:
-    """Milliseconds of the passes' memory accesses without their arithmetic (a separate probe
-    library; the y reads, dy writes and zero fills of the real passes, under 2 % of their bytes,
-    are left out)."""
-    from e3j_amd import build as lib_build
-    if not os.path.exists(lib_build.PROBE_LIB_PATH):
-        raise RuntimeError(f"{lib_build.PROBE_LIB_PATH} is missing: run `python -m e3j_amd.build`")
-    probe = ctypes.CDLL(lib_build.PROBE_LIB_PATH)
-    fn = probe.e3j_amd_probe_access_pattern
-    fn.restype = ctypes.c_int
-    fn.argtypes = [ctypes.c_uint] + [ctypes.c_int] * 4 + [ctypes.c_void_p] * 9 + [ctypes.c_int] + [ctypes.c_void_p] * 2
-    w, p = abi.w, abi.params
-    sink = torch.zeros(1, dtype=torch.float32, device=w.x.device)
-    order = abi.order.data_ptr() if abi.order is not None else None
-    result = {}
-    for name, mask in ACCESS_PATTERNS.items():
-        def run():
-            rc = fn(mask, p.num_x, p.num_scalars, p.num_out, p.channels, w.x.data_ptr(), w.s.data_ptr(),
-                    w.dm.data_ptr(), abi.other.data_ptr(), abi.ptr.data_ptr(), order, abi.ds.data_ptr(),
-                    abi.dx.data_ptr(), abi.out.data_ptr(), w.num_nodes, sink.data_ptr(), abi._stream())
-            if rc != 0:
-                raise RuntimeError("the access-pattern probe has no instantiation for these operand sizes (built-in tables, 64/128/256 channels, trailing layout)")
-        result[name] = round(time_events(torch, run, steps, 1), 4)
-    return result
-
-
 def time_events(torch, fn, steps: int, warmup: int, stats: dict | None = None) -> float:
     """Average milliseconds of `fn` from HIP events recorded on the launch stream (`stats`, if given,
     also receives the median and the minimum)."""
@@ -387,16 +303,6 @@ MEASURED_TP_TRAFFIC_BYTES = {
     ("MAP", "trailing", 1 << 18, 128): {"forward": 2.0 * 2.097e6 * 1024 + 1.299e7 * 1024,
                                         "backward": 2.0 * 8.585e6 * 1024 + 4.194e6 * 1024},
 }
-
-
-def calibrate_copy(torch, device) -> None:
-    """A 1 GiB device copy: the kernel of known size that the traffic counters are scaled by."""
-    src = torch.empty(1 << 28, dtype=torch.float32, device=device).normal_()
-    dst = torch.empty_like(src)
-    for _ in range(3):
-        dst.copy_(src)
-    torch.cuda.synchronize()
-    del src, dst
 
 
 def bench_energy(args, torch, device) -> int:
@@ -502,8 +408,6 @@ def bench_tensor_product(args, torch, device) -> int:
     import e3j_amd
     from e3j_amd import TensorProduct
     from e3j_amd.tp_ops import TensorProductParams, _make_meta, _params, _raw_backward, _raw_forward
-    if args.calibrate_copy:
-        calibrate_copy(torch, device)
     layout = "LEADING_CHANNELS" if args.layout == "leading" else "TRAILING_CHANNELS"
     trailing = layout == "TRAILING_CHANNELS"
     K, R = args.channels or 128, args.rows
@@ -590,7 +494,7 @@ def _lib_name(signature: int) -> str:
 def traffic_key(args, tiled=None) -> str:
     """Key of a measurement: workload, layout and which backward kernel ran."""
     if tiled is None:  # what the library does by default for the trailing layout
-        tiled = args.layout == "trailing" and args.tile_rows != 0 and not args.deterministic
+        tiled = args.layout == "trailing" and not args.deterministic
     return f"{args.config}/{args.scale}/{args.layout}/k{args.channels or 'default'}" + ("/tiled" if tiled else "")
 
 
@@ -613,8 +517,6 @@ def main():
     import e3j_amd
     from e3j_amd import _lib
     _lib.load()  # fail loudly when the HIP library is missing
-    if args.tile_rows is not None:
-        e3j_amd.config(tile_rows=args.tile_rows)
     device = torch.device("cuda:0")
     torch.cuda.set_device(device)
     if args.op == "tensor_product":
@@ -624,7 +526,7 @@ def main():
     if args.config == "cfg5":
         return bench_energy(args, torch, device)
 
-    w = build_workload(args.config, args.scale, device, args.spatial_sort, args.channels)
+    w = build_workload(args.config, args.scale, device, args.channels)
     w = w.with_layout("LEADING_CHANNELS" if args.layout == "leading" else "TRAILING_CHANNELS")
     module = w.module
     coef = module._packed_coef("float32")
@@ -642,9 +544,6 @@ def main():
                                   module.graph_ordering, layout=module.layout)
         grads = torch.autograd.grad(out, (xg, yg, sg), w.dm)
         return out, grads
-
-    if args.calibrate_copy:
-        calibrate_copy(torch, device)
 
     if args.table_driven:
         args.kernel_only = True   # the operators resolve the table to its unrolled kernels
@@ -684,7 +583,7 @@ def main():
         return nbytes / (ms * 1e-3) / 1e9
 
     tiled = abi.schedule is not None and not args.deterministic
-    measured = ({} if args.spatial_sort or args.deterministic else measured_traffic(traffic_key(args, tiled)))
+    measured = {} if args.deterministic else measured_traffic(traffic_key(args, tiled))
     bwd_gbs, fwd_gbs = gbs(bytes_["bwd"], bwd_ms), gbs(bytes_["fwd"], fwd_ms)
     both_gbs = gbs(bytes_["fwd_bwd"], fwd_ms + bwd_ms)
     result = {
@@ -706,7 +605,7 @@ def main():
                         f"{module.graph_ordering.value.lower()}-ordered edges, {args.layout}-channels layout, "
                         "forward + VJP (dx, dy, ds)",
             "scale": args.scale,
-            "atom_numbering": "space-filling curve" if args.spatial_sort else "random",
+            "atom_numbering": "random",
             "signature": abi.signature,
             "signature_name": (_lib.load().e3j_amd_signature_name(abi.signature).decode()
                                if abi.signature >= 0 else "table-driven kernel"),
@@ -760,13 +659,6 @@ def main():
             del calls
         result["table_driven"] = record
         del small
-    if args.tile_sharing:
-        result["roofline"]["tile_sharing"] = tile_sharing(abi, w)
-    if args.access_floor:
-        if args.layout != "trailing" or abi.perm is not None:
-            print("--access-floor covers the receiver-sorted trailing layout only", file=sys.stderr)
-            return 2
-        result["roofline"]["access_floor"] = {"unit": "ms", **access_floor(torch, abi, args.steps)}
     if not args.no_cpu_baseline:
         result["cpu_baseline"] = cpu_baseline(w, args.cpu_seconds)
     print(json.dumps(result))

@@ -131,7 +131,6 @@ SYMBOLS = {
     "e3j_amd_sort_edges": (ctypes.c_int, [_P, _P, ctypes.c_int64, ctypes.c_int32, _P, _P, _P, _P, _P]),
     "e3j_amd_order_workspace_bytes": (ctypes.c_size_t, [ctypes.c_int32]),
     "e3j_amd_register_signature": (ctypes.c_int, [_P]),
-    "e3j_amd_set_launch_variant": (None, [ctypes.c_int32, ctypes.c_int32]),
     "e3j_amd_set_table_plans": (None, [ctypes.c_int32]),
     "e3j_amd_row_partials_bytes": (ctypes.c_size_t, [ctypes.c_int64, ctypes.c_int32, ctypes.c_int32]),
     "e3j_amd_table_plan_bytes": (ctypes.c_size_t, [ctypes.POINTER(ConvParams)]),
@@ -159,6 +158,11 @@ SYMBOLS = {
     "e3j_amd_xla_tensor_product_bwd": (_P, [_P]),
 }
 
+#: exported for the in-tree tests only, declared in `csrc/tuning_api.h`, not in the public header
+INTERNAL_SYMBOLS = {
+    "e3j_amd_set_launch_variant": (None, [ctypes.c_int32, ctypes.c_int32]),
+}
+
 _lib = None
 
 
@@ -173,7 +177,7 @@ def load() -> ctypes.CDLL:
             "(hipcc, gfx950). e3j_amd has no fallback implementation.")
     # global symbols: signature libraries compiled at run time resolve against this one
     lib = ctypes.CDLL(LIB_PATH, mode=ctypes.RTLD_GLOBAL)
-    for name, (restype, argtypes) in SYMBOLS.items():
+    for name, (restype, argtypes) in {**SYMBOLS, **INTERNAL_SYMBOLS}.items():
         fn = getattr(lib, name)  # AttributeError if the export is missing
         fn.restype = restype
         fn.argtypes = argtypes

@@ -21,10 +21,6 @@ CSRC = os.path.join(HERE, "csrc")
 GENERATED = os.path.join(CSRC, "generated")
 OBJ_DIR = os.path.join(HERE, "lib", "obj")
 LIB_PATH = os.path.join(HERE, "lib", "libe3j_amd.so")
-#: measurement aid of `bench.py --access-floor` (memory accesses of the passes without their
-#: arithmetic); a library of its own, the operators never load it
-PROBE_SOURCE = os.path.join(CSRC, "probe", "access_pattern.hip")
-PROBE_LIB_PATH = os.path.join(HERE, "lib", "libe3j_amd_probe.so")
 
 HIPCC = os.environ.get("HIPCC", shutil.which("hipcc") or "/opt/rocm/bin/hipcc")
 ARCH = "gfx950"
@@ -72,19 +68,7 @@ def build(regenerate: bool = True, jobs: int | None = None, verbose: bool = True
     os.replace(LIB_PATH + ".tmp", LIB_PATH)
     if verbose:
         print(f"[e3j_amd.build] wrote {LIB_PATH}", flush=True)
-    build_probe(verbose)
     return LIB_PATH
-
-
-def build_probe(verbose: bool = True) -> str:
-    cmd = [HIPCC, *COMMON_FLAGS, "-shared", PROBE_SOURCE, "-o", PROBE_LIB_PATH + ".tmp"]
-    proc = subprocess.run(cmd, capture_output=True, text=True)
-    if proc.returncode != 0:
-        raise RuntimeError(f"hipcc failed for {PROBE_SOURCE}:\n{proc.stdout}\n{proc.stderr}")
-    os.replace(PROBE_LIB_PATH + ".tmp", PROBE_LIB_PATH)
-    if verbose:
-        print(f"[e3j_amd.build] wrote {PROBE_LIB_PATH}", flush=True)
-    return PROBE_LIB_PATH
 
 
 if __name__ == "__main__":

@@ -12,6 +12,7 @@
 #include <vector>
 
 #include "common.h"
+#include "tuning_api.h"
 #include "row_pieces.h"
 
 namespace e3j_amd {

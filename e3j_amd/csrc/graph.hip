@@ -562,7 +562,7 @@ size_t e3j_amd_csr_workspace_bytes(int32_t num_nodes, int64_t num_edges) {
 
 int e3j_amd_csr_row_ptr(const int32_t *key, int64_t num_edges, int32_t num_nodes, int32_t *row_ptr,
                         void *workspace, void *stream_) {
-    if (num_nodes < 0 || num_edges < 0 || num_edges > 0x7fffffffLL)
+    if (num_nodes < 0 || num_nodes >= INT32_MAX || num_edges < 0 || num_edges > 0x7fffffffLL)
         return set_error(E3J_AMD_INVALID_ARGUMENT, "csr_row_ptr: bad sizes");
     if (row_ptr == nullptr || workspace == nullptr || (num_edges > 0 && key == nullptr))
         return set_error(E3J_AMD_INVALID_ARGUMENT, "csr_row_ptr: null operand");
@@ -613,7 +613,8 @@ int32_t e3j_amd_csr_row_ptr_static_max_nodes(void) {
 
 int e3j_amd_csr_row_ptr_static(const int32_t *key, int64_t num_edges, int32_t num_nodes, int32_t *row_ptr,
                                void *stream_) {
-    if (num_nodes < 0 || num_edges < 0 || num_edges > 0x7fffffffLL)
+    // (num_nodes + 1 entries are scanned: INT32_MAX nodes would overflow the count)
+    if (num_nodes < 0 || num_nodes >= INT32_MAX || num_edges < 0 || num_edges > 0x7fffffffLL)
         return set_error(E3J_AMD_INVALID_ARGUMENT, "csr_row_ptr_static: bad sizes");
     if (row_ptr == nullptr || (num_edges > 0 && key == nullptr))
         return set_error(E3J_AMD_INVALID_ARGUMENT, "csr_row_ptr_static: null operand");

@@ -14,8 +14,9 @@
 // result (the atomic-free, bit-reproducible backward).
 // Attributes: num_nodes, debug (reference); layout, signature, coef_scale, y_flip,
 // coef_stacked (optional).  Without `signature` the handler finds the kernels of the table the
-// frame carries (see TableResolver).  Handlers are re-entrant (the only shared state is that
-// lookup, behind a mutex), allocate nothing themselves ("convolution_bwd" borrows scratch from the
+// frame carries (see TableResolver: a read-back of the table and a host wait per call; frames that
+// name `signature` wait for nothing).  Handlers are re-entrant (the only shared state is the map
+// of tables already looked up, behind a mutex), allocate nothing themselves ("convolution_bwd" borrows scratch from the
 // runtime through XLA_FFI_DeviceMemory_Allocate when it runs the unrolled kernels, and so does a
 // table-driven call for the plan of its table; a runtime without such memory leaves the latter to
 // the stream's pool) and enqueue
@@ -111,11 +112,15 @@ T attr(const XlaCallFrame *f, const char *name, int32_t dtype, T fallback, bool 
 
 // ---- which unrolled kernels serve the table of a frame ----------------------------------------
 // The reference's frames carry the coefficient table as a device buffer and no kernel id
-// (src/e3j/ops/convolution.py:229-242,433-452).  The handler reads the table back (a few KB) on a
-// stream of its own, which waits for nothing of the caller's work, and looks it up among the
-// signatures; the answer is remembered under the table's bytes.  Under stream capture nothing
-// may be read back: the answer a previous call found for the same device buffer and shape is
-// used, and an unknown table runs the table-driven kernels.
+// (src/e3j/ops/convolution.py:229-242,433-452).  The handler reads the table back (a few KB) and
+// looks it up among the signatures; the answer is remembered under the table's BYTES, never under
+// its address (a buffer can be rewritten or reused for a table of the same shape with another
+// scale or other signs).  The read runs on a stream of the calling thread that first waits for the
+// work already enqueued on the caller's stream (an event), so a table still being written there is
+// read after that write; the host waits for the copy.  Frames that carry the attributes
+// `signature`, `coef_scale` and `y_flip` skip all of this: that is the path without a host wait.
+// Under stream capture nothing can be read back, and nothing is assumed about the buffer: such a
+// frame runs the table-driven kernels, which read the table on the device at every replay.
 struct ResolvedTable {
     int32_t signature = -1;
     float scale = 1.0f;
@@ -132,52 +137,62 @@ class TableResolver {
         const size_t bytes = item * (size_t)num_coef;
         const Shape shape{num_coef, idx_bytes, columns_ji ? 1 : 0, p.num_x, p.num_y, p.num_out, p.num_scalars,
                           p.channels, p.layout};
-        std::lock_guard<std::mutex> lock(mutex_);
         hipStreamCaptureStatus capture = hipStreamCaptureStatusNone;
         if (hipStreamIsCapturing(caller_stream, &capture) != hipSuccess) {
             (void)hipGetLastError();
             return none;
         }
-        if (capture != hipStreamCaptureStatusNone) {
-            auto seen = by_pointer_.find(std::make_pair(device_table, shape));
-            return seen == by_pointer_.end() ? none : seen->second;
-        }
+        if (capture != hipStreamCaptureStatusNone) return none;
         int device = 0;
         if (hipGetDevice(&device) != hipSuccess) return none;
-        hipStream_t &side = side_streams_[device];
-        if (side == nullptr && hipStreamCreateWithFlags(&side, hipStreamNonBlocking) != hipSuccess) {
-            side = nullptr;
-            (void)hipGetLastError();
-            return none;
+        // per thread and device: concurrent handler calls do not share a stream or an event
+        thread_local std::map<int, ReadBack> read_backs;
+        ReadBack &rb = read_backs[device];
+        if (rb.stream == nullptr) {
+            if (hipStreamCreateWithFlags(&rb.stream, hipStreamNonBlocking) != hipSuccess ||
+                hipEventCreateWithFlags(&rb.after_caller, hipEventDisableTiming) != hipSuccess) {
+                rb = ReadBack{};
+                (void)hipGetLastError();
+                return none;
+            }
         }
         std::vector<unsigned char> host(bytes);
-        if (hipMemcpyAsync(host.data(), device_table, bytes, hipMemcpyDeviceToHost, side) != hipSuccess ||
-            hipStreamSynchronize(side) != hipSuccess) {
+        if (hipEventRecord(rb.after_caller, caller_stream) != hipSuccess ||
+            hipStreamWaitEvent(rb.stream, rb.after_caller, 0) != hipSuccess ||
+            hipMemcpyAsync(host.data(), device_table, bytes, hipMemcpyDeviceToHost, rb.stream) != hipSuccess ||
+            hipStreamSynchronize(rb.stream) != hipSuccess) {
             (void)hipGetLastError();
             return none;
         }
-        ResolvedTable &entry = by_content_[std::make_pair(shape, host)];
-        if (!entry_known_(entry)) {
-            const std::vector<TableEntry> entries = unpack_entries(host.data(), idx_bytes, num_coef, columns_ji);
-            entry.signature = match_signature(entries, p.num_x, p.num_y, p.num_out, p.num_scalars, p.channels,
-                                              p.layout, &entry.scale, &entry.flip);
-            if (entry.signature < 0) entry.signature = kNoKernel;
+        auto key = std::make_pair(shape, std::move(host));
+        {
+            std::lock_guard<std::mutex> lock(mutex_);
+            auto seen = by_content_.find(key);
+            if (seen != by_content_.end()) return seen->second.signature == kNoKernel ? none : seen->second;
         }
-        ResolvedTable found = entry;
-        if (found.signature == kNoKernel) found = none;
-        if (by_pointer_.size() > 4096) by_pointer_.clear();
-        by_pointer_[std::make_pair(device_table, shape)] = found;
-        return found;
+        // the lookup itself runs without the lock (two threads may do the same one; both find the same)
+        ResolvedTable entry;
+        const std::vector<TableEntry> entries = unpack_entries(key.second.data(), idx_bytes, num_coef, columns_ji);
+        entry.signature = match_signature(entries, p.num_x, p.num_y, p.num_out, p.num_scalars, p.channels,
+                                          p.layout, &entry.scale, &entry.flip);
+        if (entry.signature < 0) entry.signature = kNoKernel;
+        {
+            std::lock_guard<std::mutex> lock(mutex_);
+            if (by_content_.size() > 1024) by_content_.clear();
+            by_content_[std::move(key)] = entry;
+        }
+        return entry.signature == kNoKernel ? none : entry;
     }
 
   private:
     using Shape = std::tuple<int32_t, int32_t, int32_t, int32_t, int32_t, int32_t, int32_t, int32_t, int32_t>;
-    static constexpr int32_t kNoKernel = -2;  // looked up, nothing matches (a fresh entry holds -1)
-    static bool entry_known_(const ResolvedTable &e) { return e.signature != -1; }
-    std::mutex mutex_;
-    std::map<int, hipStream_t> side_streams_;
+    struct ReadBack {
+        hipStream_t stream = nullptr;
+        hipEvent_t after_caller = nullptr;
+    };
+    static constexpr int32_t kNoKernel = -2;  // looked up, nothing matches
+    std::mutex mutex_;  // guards by_content_ only
     std::map<std::pair<Shape, std::vector<unsigned char>>, ResolvedTable> by_content_;
-    std::map<std::pair<const void *, Shape>, ResolvedTable> by_pointer_;
 };
 
 TableResolver &resolver() {

@@ -9,6 +9,7 @@ stored as float32 (the canonical value dtype of the reference without x64).
 from __future__ import annotations
 
 import dataclasses
+import math
 
 import numpy as np
 
@@ -50,16 +51,19 @@ def sparse_coo(values, indices, shape, coalesce: bool = True, dtype=np.float32) 
     if coords.size and not ((coords >= 0) & (coords < limits)).all():
         raise ValueError(f"Out of bounds indices for shape {shape}.")
     if coalesce and len(coords):
-        # row-major linear position of every entry; np.unique returns the distinct positions in
-        # ascending order (= lexicographic order of the coordinates) and, per entry, which of
-        # them it falls on, so one weighted histogram merges the duplicates
-        strides = np.concatenate([np.cumprod(limits[0, :0:-1])[::-1], [1]]).astype(np.int64)
-        linear = coords @ strides
-        distinct, slot = np.unique(linear, return_inverse=True)
-        merged = np.zeros(len(distinct), dtype=np.float64)
-        np.add.at(merged, slot.reshape(-1), vals.astype(np.float64))
-        merged = merged.astype(vals.dtype)
-        alive = np.flatnonzero(merged)
-        coords = np.stack(np.unravel_index(distinct[alive], shape), axis=1).astype(np.int64)
-        vals = merged[alive]
+        # The distinct coordinates in lexicographic order and, per entry, which of them it falls
+        # on.  Duplicates are added in the value dtype, one after another in the order the
+        # entries were given (`np.add.at` is unbuffered), and an entry is dropped when that sum is
+        # exactly zero in the value dtype: the arithmetic of `src/e3j/utils/sparse.py:116-124`.
+        if math.prod(shape) <= np.iinfo(np.int64).max:
+            # row-major linear positions: ascending positions = lexicographic coordinates
+            strides = np.concatenate([np.cumprod(limits[0, :0:-1])[::-1], [1]]).astype(np.int64)
+            distinct, slot = np.unique(coords @ strides, return_inverse=True)
+            distinct = np.stack(np.unravel_index(distinct, shape), axis=1).astype(np.int64)
+        else:  # the linear position would overflow: compare coordinate rows
+            distinct, slot = np.unique(coords, axis=0, return_inverse=True)
+        merged = np.zeros(len(distinct), dtype=vals.dtype)
+        np.add.at(merged, slot.reshape(-1), vals)
+        alive = merged != 0
+        coords, vals = distinct[alive], merged[alive]
     return SparseCOO(vals, coords.astype(narrow_index_dtype(shape)), shape)

@@ -238,20 +238,11 @@ int e3j_amd_find_signature(const void *coef_host, int32_t coef_idx_bytes, int32_
                            float *coef_scale,
                            uint32_t *y_flip);
 
-/* Tuning aid: selects which launch shape (channels per lane, waves per block, parts) of a
- * signature's kernels later calls use; 0 = default, unknown numbers = default.  The
- * environment variables E3J_AMD_FWD_VARIANT / E3J_AMD_BWD_VARIANT give the initial values.
- * Process-wide; may be called from any thread while other threads launch (each launch reads the
- * numbers once, atomically, and uses the old or the new shape).  Results do not depend on it.
- * No counterpart in the reference, whose launch shape is planned on the host per call
- * (src/e3j/ops/convolution.py:178-208). */
-void e3j_amd_set_launch_variant(int32_t fwd_variant, int32_t bwd_variant);
-
 /* The table-driven kernels (calls with signature < 0, and calls whose operands an unrolled kernel
  * cannot take) come in two forms.  For a float32 or float16 table (float16: values held as half,
  * arithmetic in float; the sender-grouped backward only) in which every output coordinate uses one
- * scalar, with at most 128 output coordinates, 16 x coordinates, 64 y components, 1024 scalars and
- * 8192 entries, the call first turns the table into a plan on the device (one small kernel; the
+ * scalar, with at most 128 output coordinates, 16 x coordinates, 64 y components, 64 scalars and
+ * 2048 entries, the call first turns the table into a plan on the device (one small kernel; the
  * plan lives in memory of the stream's pool, hipMallocAsync, for the length of the call) and runs
  * kernels that keep x and the accumulators in registers; any other table and float64 run the
  * kernels that index LDS columns by the table's coordinates (float16 there: arithmetic in half).  Whether a table fits is

@@ -30,19 +30,6 @@ def test_every_declared_symbol_is_exported():
     assert lib.e3j_amd_version().startswith(b"e3j_amd")
 
 
-def test_probe_library_is_separate_and_refuses_other_shapes():
-    """The access-pattern probe of the benchmark is a library of its own; the operator
-    library does not export it, and it refuses shapes it has no kernel for (no launch)."""
-    from e3j_amd import build as lib_build
-    assert os.path.exists(lib_build.PROBE_LIB_PATH), "run `python -m e3j_amd.build` first"
-    probe = C.CDLL(lib_build.PROBE_LIB_PATH)
-    fn = probe.e3j_amd_probe_access_pattern
-    fn.restype = C.c_int
-    fn.argtypes = [C.c_uint] + [C.c_int] * 4 + [C.c_void_p] * 9 + [C.c_int] + [C.c_void_p] * 2
-    assert fn(1, 9, 13, 43, 64, *[None] * 9, 10, None, None) == -1
-    assert not hasattr(_lib.load(), "e3j_amd_probe_access_pattern")
-
-
 def test_params_struct_matches_header():
     header = open(os.path.join(ROOT, "include", "e3j_amd.h")).read()
     body = re.search(r"typedef struct e3j_amd_conv_params \{(.*?)\} e3j_amd_conv_params;", header, re.S).group(1)

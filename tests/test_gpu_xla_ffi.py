@@ -346,16 +346,14 @@ def bwd_operands(frame):
     return [C.cast(frame.args.args[i], C.POINTER(Buffer)).contents for i in range(n)]
 
 
-def test_reference_forward_frame_under_graph_capture_uses_what_an_earlier_call_found():
-    """Nothing can be read back while a stream is captured: the handler then uses the kernels an
-    earlier call found for the same table buffer; replays give the eager result."""
+def _reference_forward_frame(scale=0.05):
     from e3j_amd import workloads as W
     from e3j_amd.graph import csr_row_ptr
-    w = W.config2(0.05)
+    w = W.config2(scale)
     d = w.to("cuda")
     n = w.num_nodes
-    lib = _lib.load()
-    packed = dev(w.module._packed_coef("float32"))
+    table = w.module._packed_coef("float32")
+    packed = dev(table)
     ptr = csr_row_ptr(d.receiver, n)
     ranges = dev(np.array([1], dtype=np.int32))
     xla = FakeXla(stream=torch.cuda.current_stream().cuda_stream)
@@ -363,10 +361,65 @@ def test_reference_forward_frame_under_graph_capture_uses_what_an_earlier_call_f
     frame = xla.frame([_buf(xla, packed, U8), _buf(xla, d.x, F32), _buf(xla, d.y, F32), _buf(xla, d.s, F32),
                        _buf(xla, d.sender, S32), _buf(xla, ptr, S32), _buf(xla, ranges, S32)],
                       [_buf(xla, out, F32)], {"num_nodes": (S32, C.c_int32(n)), "debug": (S32, C.c_int32(0))})
+    keep = (w, d, ptr, ranges)
+    return xla, frame, table, packed, out, keep
+
+
+def _rescaled(table: np.ndarray, factor: float) -> np.ndarray:
+    """The packed table (uint8 rows of {float32 val; 4 x uint8 index}) with every value times `factor`."""
+    t = table.copy()
+    vals = t[:, :4].copy().view(np.float32) * np.float32(factor)
+    t[:, :4] = vals.view(np.uint8).reshape(-1, 4)
+    return t
+
+
+def test_reference_forward_frame_follows_a_table_rewritten_in_place():
+    """The kernels of a frame without `signature` are found from the table's bytes at every call,
+    never from its address: the same device buffer rewritten with a rescaled table (same shape, as
+    the reference's signed and unsigned tables have) gives the rescaled result, also when the
+    rewrite is still in flight on the caller's stream when the handler is called."""
+    lib = _lib.load()
+    xla, frame, table, packed, out, keep = _reference_forward_frame()
+    torch.cuda.synchronize()
+    assert lib.e3j_amd_xla_convolution(C.addressof(frame)) is None, xla.errors
+    torch.cuda.synchronize()
+    first = out.clone()
+    assert float(first.abs().max()) > 0
+    # rewritten on the caller's stream, handler called without waiting for it
+    staged = torch.as_tensor(_rescaled(table, -2.5)).pin_memory()
+    filler = torch.empty(1 << 26, device="cuda")
+    for _ in range(4):
+        filler.normal_()           # work ahead of the rewrite on the same stream
+    packed.copy_(staged, non_blocking=True)
+    assert lib.e3j_amd_xla_convolution(C.addressof(frame)) is None, xla.errors
+    torch.cuda.synchronize()
+    assert float((out + 2.5 * first).abs().max()) <= 2e-5 * float(first.abs().max()) * 2.5
+    # and a table no signature matches (one value changed) runs the table-driven kernels: same contract
+    odd = table.copy()
+    v = odd[0, :4].copy().view(np.float32) * np.float32(1.5)
+    odd[0, :4] = v.view(np.uint8)
+    packed.copy_(torch.as_tensor(odd))
+    assert lib.e3j_amd_xla_convolution(C.addressof(frame)) is None, xla.errors
+    torch.cuda.synchronize()
+    assert float((out - first).abs().max()) > 0
+
+
+def test_reference_forward_frame_under_graph_capture_reads_the_table_at_every_replay():
+    """Nothing can be read back while a stream is captured, and nothing is assumed about the table
+    buffer: a frame without `signature` records the table-driven kernels, which read the table on
+    the device.  Replays give the eager result; after the table buffer is rewritten in place with
+    a rescaled table, the replays give the rescaled result.  A frame that names `signature`,
+    `coef_scale` and `y_flip` records the unrolled kernels."""
+    from e3j_amd.ops import _Table
+    lib = _lib.load()
+    xla, frame, table, packed, out, keep = _reference_forward_frame()
+    xla.allocate = lambda nbytes: torch.empty(nbytes, dtype=torch.uint8, device="cuda")
+    w = keep[0]
     torch.cuda.synchronize()
     assert lib.e3j_amd_xla_convolution(C.addressof(frame)) is None, xla.errors
     torch.cuda.synchronize()
     eager = out.clone()
+    tol = 2e-5 * float(eager.abs().max())
     graph = torch.cuda.CUDAGraph()
     with torch.cuda.graph(graph):
         xla.stream = torch.cuda.current_stream().cuda_stream
@@ -375,4 +428,31 @@ def test_reference_forward_frame_under_graph_capture_uses_what_an_earlier_call_f
         out.zero_()
         graph.replay()
         torch.cuda.synchronize()
-        assert torch.equal(out, eager)
+        assert float((out - eager).abs().max()) <= tol
+    packed.copy_(torch.as_tensor(_rescaled(table, 3.0)))
+    for _ in range(2):
+        out.zero_()
+        torch.cuda.synchronize()
+        graph.replay()
+        torch.cuda.synchronize()
+        assert float((out - 3.0 * eager).abs().max()) <= 3.0 * tol
+    packed.copy_(torch.as_tensor(table))
+
+    # the path without a host wait: the frame names the kernels itself
+    m = w.module
+    dims = (int(w.x.shape[1]), int(w.y.shape[1]), m.params.num_out, int(w.s.shape[1]))
+    sig, scale, flip = _Table.get(table, np.float32).signature(dims, w.channels, m.layout)
+    assert sig >= 0
+    named = xla.frame(bwd_operands(frame), [_buf(xla, out, F32)],
+                      {"num_nodes": (S32, C.c_int32(w.num_nodes)), "debug": (S32, C.c_int32(0)),
+                       "signature": (S32, C.c_int32(sig)), "coef_scale": (F32, C.c_float(scale)),
+                       "y_flip": (S32, C.c_int32(flip))})
+    graph2 = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph2):
+        xla.stream = torch.cuda.current_stream().cuda_stream
+        assert lib.e3j_amd_xla_convolution(C.addressof(named)) is None, xla.errors
+    for _ in range(2):
+        out.zero_()
+        graph2.replay()
+        torch.cuda.synchronize()
+        assert torch.equal(out, eager)   # the eager call resolved to the same unrolled kernels

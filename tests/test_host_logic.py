@@ -195,6 +195,41 @@ def test_sparse_coo_coalesce():
         sparse_coo([1.0], [[2, 0]], (2, 2))
 
 
+def test_sparse_coo_sums_duplicates_in_the_value_dtype():
+    """Duplicates are added one after another in float32 and dropped when that sum is exactly zero
+    (`src/e3j/utils/sparse.py:116-124`): 1e8 + 1 - 1e8 is 0 in float32 and 1 in float64."""
+    vals = [1e8, 2.5, 1.0, -1e8, 0.1, 0.2, 0.3]
+    idx = [[3, 1], [0, 2], [3, 1], [3, 1], [1, 1], [1, 1], [1, 1]]
+    c = sparse_coo(vals, idx, (4, 3))
+    assert c.data.dtype == np.float32
+    assert c.indices.tolist() == [[0, 2], [1, 1]]          # (3, 1) cancels in float32
+    want = np.float32(0.1) + np.float32(0.2)                 # left to right, rounded at every step
+    want = np.float32(want + np.float32(0.3))
+    assert c.data.tobytes() == np.array([2.5, want], np.float32).tobytes()
+    # literal restatement of the rule on random duplicates: sort stably, add runs sequentially
+    rng = np.random.default_rng(5)
+    idx = rng.integers(0, 4, size=(200, 3))
+    vals = rng.normal(size=200).astype(np.float32)
+    c = sparse_coo(vals, idx, (4, 4, 4))
+    sums = {}
+    for v, row in zip(vals, map(tuple, idx.tolist())):
+        sums[row] = np.float32(sums.get(row, np.float32(0)) + v)
+    rows = sorted(r for r, v in sums.items() if v != 0)
+    assert c.indices.tolist() == [list(r) for r in rows]
+    assert c.data.tobytes() == np.array([sums[r] for r in rows], np.float32).tobytes()
+
+
+def test_sparse_coo_shapes_beyond_int64_positions():
+    """A shape whose number of elements does not fit int64 is coalesced by comparing coordinate
+    rows (the reference switches to a lexicographic sort there, `src/e3j/utils/sparse.py:104-113`)."""
+    big = 2 ** 31 - 1
+    idx = [[5, 1, big - 1], [0, 7, 3], [5, 1, big - 1], [0, 7, 2]]
+    c = sparse_coo([1.0, 2.0, 3.0, 4.0], idx, (big, big, big))
+    assert c.indices.dtype == np.int32
+    assert c.indices.tolist() == [[0, 7, 2], [0, 7, 3], [5, 1, big - 1]]
+    assert c.data.tolist() == [4.0, 2.0, 4.0]
+
+
 def test_mix_indices():
     assert ScalarMixing("2x0e + 1x1o + 1x2e").mix_indices.tolist() == [0, 1, 2, 2, 2, 3, 3, 3, 3, 3]
 

@@ -51,6 +51,62 @@ def test_static_row_ptr_matches_workspace_version_twice():
         outputs.append(out)
 
 
+def test_static_row_ptr_allocates_nothing_and_replays_from_a_graph():
+    """What the entry point is for: the two calls are recorded into a HIP graph (a capture fails on
+    any allocation or synchronisation inside the recorded calls) and the graph is replayed on rewritten
+    inputs, with eager work between the replays; the device's free memory does not move across
+    the eager calls either."""
+    rng = np.random.default_rng(11)
+    cases = [(50_000, 600_000), (700, 2_000)]
+    keys = [torch.empty(e, dtype=torch.int32, device="cuda") for _, e in cases]
+    outs = [torch.empty(n + 1, dtype=torch.int32, device="cuda") for n, _ in cases]
+
+    def fresh_keys():
+        host = []
+        for (n, e), key in zip(cases, keys):
+            k = np.sort(rng.integers(0, n, size=e)).astype(np.int32)
+            k[rng.random(e) < 0.02] = np.iinfo(np.int32).max
+            key.copy_(torch.as_tensor(k))
+            host.append(k)
+        return host
+
+    def expected(host):
+        return [np.concatenate([[0], np.cumsum(np.bincount(k[k < n], minlength=n))]) for (n, _), k in zip(cases, host)]
+
+    host = fresh_keys()
+    for (n, _), key, out in zip(cases, keys, outs):   # warm-up: looks up the scratch address once
+        _static(key, n, out)
+    torch.cuda.synchronize()
+    free_before = torch.cuda.mem_get_info()[0]
+    for (n, _), key, out in zip(cases, keys, outs):
+        _static(key, n, out)
+    torch.cuda.synchronize()
+    assert torch.cuda.mem_get_info()[0] == free_before, "the static entry point changed the device's free memory"
+    for out, want in zip(outs, expected(host)):
+        assert np.array_equal(out.cpu().numpy(), want)
+
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph):
+        for (n, _), key, out in zip(cases, keys, outs):
+            _static(key, n, out)
+    for _ in range(3):
+        host = fresh_keys()
+        for out in outs:
+            out.fill_(-7)
+        torch.cuda.synchronize()
+        graph.replay()
+        torch.cuda.synchronize()
+        for out, want in zip(outs, expected(host)):
+            assert np.array_equal(out.cpu().numpy(), want)
+
+
+def test_static_row_ptr_refuses_bad_node_counts():
+    key = torch.zeros(4, dtype=torch.int32, device="cuda")
+    out = torch.empty(8, dtype=torch.int32, device="cuda")
+    with pytest.raises(_lib.E3jAmdError, match="bad sizes"):
+        _static(key, np.iinfo(np.int32).max, out)
+
+
 def test_static_row_ptr_refuses_sizes_beyond_its_scratch():
     lib = _lib.load()
     limit = int(lib.e3j_amd_csr_row_ptr_static_max_nodes())
