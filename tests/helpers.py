@@ -128,18 +128,21 @@ def backward_reference(idx, val, mix, x, y, s, snd, rcv, dm, leading=False):
 def assert_parity(result, ref64, mag64, what="", rtol=1e-5, atol=1e-6, ulps=16.0):
     """|result - ref| <= atol + rtol*|ref| elementwise (1e-5 relative / 1e-6 absolute);
     an element outside that must lie within `ulps` float32 roundings of the sum of the
-    absolute values of its terms - the float32 summation-order allowance."""
+    absolute values of its terms - the float32 summation-order allowance.
+    Returns the share of the elements that needed that allowance."""
     result = np.asarray(result, dtype=np.float64)
     assert result.shape == ref64.shape, f"{what}: shape {result.shape} != {ref64.shape}"
     assert np.isfinite(result).all(), f"{what}: non-finite values"
     err = np.abs(result - ref64)
-    ok = (err <= atol + rtol * np.abs(ref64)) | (err <= ulps * EPS32 * mag64)
+    in_band = err <= atol + rtol * np.abs(ref64)
+    ok = in_band | (err <= ulps * EPS32 * mag64)
     if not ok.all():
         bad = np.argwhere(~ok)[0]
         t = tuple(bad)
         raise AssertionError(
             f"{what}: {int((~ok).sum())} of {ok.size} elements out of tolerance; first at {t}: "
             f"got {result[t]!r}, want {ref64[t]!r}, err {err[t]:.3e}, term magnitude {mag64[t]:.3e}")
+    return 1.0 - float(in_band.mean()) if in_band.size else 0.0
 
 
 def float32_noise_bound(ref64, mag64, rtol=1e-5, atol=1e-6, ulps=16.0):

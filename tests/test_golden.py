@@ -1,6 +1,9 @@
 """The committed golden fixtures (`tests/golden/*.npz`, written by `tests/golden/make_fixtures.py`):
 the CPU checkers must reproduce them (guards the oracle, the table construction and the
-fixtures against drift), and the HIP kernels must match them to the parity criterion."""
+fixtures against drift), and the HIP kernels must match them to the parity criterion.
+Only `strip` holds values the reference itself holds (its closed-form known-answer case,
+`lib/e3j_ops/tests/test_convolution.cpp:128-183`); `l3_k64`, `padding` and `unsorted_skewed` were
+written by this repository's own oracle and are regression pins, as the test names say."""
 
 import os
 
@@ -32,7 +35,7 @@ def magnitudes(g):
 
 
 @pytest.mark.parametrize("name", CASES)
-def test_numpy_oracle_reproduces_fixture(name):
+def test_numpy_oracle_reproduces_its_own_regression_fixture(name):
     g = load(name)
     tol = dict(rtol=1e-6, atol=1e-6) if g["out"].dtype == np.float32 else dict(rtol=1e-12, atol=1e-12)
     out = O.convolution_unfused(g["idx"], g["val"], g["mix"], g["x"], g["y"], g["s"], g["sender"],
@@ -45,7 +48,7 @@ def test_numpy_oracle_reproduces_fixture(name):
 
 
 @pytest.mark.parametrize("name", ["strip", "l3_k64", "padding"])
-def test_c_checker_matches_fixture(name):
+def test_c_checker_matches_regression_fixture(name):
     """The float32 C restatement of the reference's CPU loops (receiver-sorted cases)."""
     g = load(name)
     mag = magnitudes(g)
@@ -58,7 +61,7 @@ def test_c_checker_matches_fixture(name):
         H.assert_parity(got, g[key].astype(np.float64), mag[key], f"{name} {key}")
 
 
-def test_strip_fixture_is_the_closed_form():
+def test_strip_fixture_is_the_reference_held_closed_form():
     """out[r, 2t+a, c] = (a+1) * 12 * sum over the row's edges of s[e, t]
     (`lib/e3j_ops/tests/test_convolution.cpp:122-207`), exact in float32."""
     g = load("strip")
@@ -75,7 +78,7 @@ def test_strip_fixture_is_the_closed_form():
 @pytest.mark.gpu
 @pytest.mark.parametrize("layout", ["TRAILING_CHANNELS", "LEADING_CHANNELS"])
 @pytest.mark.parametrize("name", CASES)
-def test_hip_kernels_match_fixture(name, layout):
+def test_hip_kernels_match_regression_fixture(name, layout):
     import torch
     import e3j_amd
     g = load(name)

@@ -224,3 +224,26 @@ def test_c_oracle_handles_unsorted_edges():
     a = c_oracle.convolution(idx, val, mix, x, y[order], s[order], snd[order], rcv[order], Z)
     ref, mag = H.forward_reference(idx, val, mix, x, y, s, snd, rcv, Z)
     H.assert_parity(a, ref, mag, "unsorted")
+
+
+def test_c_checker_in_float64_is_the_numpy_restatement():
+    """The C loops compiled for double (the exact reference of the full-size GPU tests) against the
+    numpy restatement in float64, forward and VJP, with padding edges and an unsorted edge list."""
+    from oracle import c_oracle
+    rng = np.random.default_rng(21)
+    idx, val, mix = H.random_table(rng, 60, 6, 5, 11, 4)
+    snd, rcv = H.random_graph(rng, 30, 200, sort_by=None)
+    snd[::17] = np.iinfo(np.int32).max
+    rcv[5::23] = np.iinfo(np.int32).max
+    x, y, s, dm = H.random_operands(rng, 30, 200, 6, 5, 4, 12, 11)
+    got = c_oracle.convolution(idx, val, mix, x, y, s, snd, rcv, 11, dtype=np.float64)
+    want = O.convolution_unfused(idx, val, mix, x, y, s, snd, rcv, 11, dtype=np.float64)
+    assert got.dtype == np.float64
+    np.testing.assert_allclose(got, want, rtol=1e-13, atol=1e-13)
+    grads = c_oracle.convolution_vjp(idx, val, mix, x, y, s, snd, rcv, dm, dtype=np.float64)
+    wants = O.convolution_vjp(idx, val, mix, x, y, s, snd, rcv, dm, dtype=np.float64)
+    for g, w_ in zip(grads, wants):
+        np.testing.assert_allclose(g, w_, rtol=1e-13, atol=1e-12)
+    # and the float32 build differs from it by float32 rounding only
+    low = c_oracle.convolution(idx, val, mix, x, y, s, snd, rcv, 11)
+    assert low.dtype == np.float32 and np.abs(low - want).max() <= 1e-5 * np.abs(want).max()
