@@ -158,7 +158,7 @@ def build_workload(name: str, scale: float, device, channels=None):
 class AbiCalls:
     """Direct launches through the C ABI with a prebuilt receiver CSR (kernel timing)."""
 
-    def __init__(self, w, table_driven=False):
+    def __init__(self, w, table_driven=False, paired=False):
         import numpy as np
         import torch
         from e3j_amd import _lib
@@ -189,7 +189,7 @@ class AbiCalls:
             self.ptr = csr_row_ptr(w.receiver, w.num_nodes)
         rounds = config().locality_rounds
         self.order = locality_order(self.other, self.ptr, w.num_nodes, rounds) if rounds > 0 else None
-        if self.order is not None and config().pair_rows:   # as the operators do
+        if self.order is not None and (paired or config().pair_rows is True):   # as the operators do
             from e3j_amd.graph import pair_rows
             self.order = pair_rows(self.other, self.ptr, w.num_nodes, self.order)
         self.params.row_order = self.order.data_ptr() if self.order is not None else None
@@ -631,6 +631,35 @@ def main():
                                           "included in ms_per_step)"},
         },
     }
+    if not args.kernel_only and not args.table_driven and not args.deterministic:
+        # the same step for a caller that holds the adjacency across calls (the layers of a model, the
+        # steps between two neighbour-list rebuilds): prepared once, outside the timed region, with rows
+        # that share senders paired (the default of `prepare_graph`); `value` above prepares per step
+        handle = prepare_graph(w.sender, w.receiver, w.num_nodes, module.graph_ordering)
+
+        def held_step():
+            out = e3j_amd.convolution(coef, xg, yg, sg, w.sender, w.receiver, module.params,
+                                      module.graph_ordering, layout=module.layout, graph=handle)
+            return torch.autograd.grad(out, (xg, yg, sg), w.dm)
+
+        for _ in range(args.warmup):
+            held_step()
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        for _ in range(args.steps):
+            held_step()
+        torch.cuda.synchronize()
+        held_ms = (time.perf_counter() - t0) * 1e3 / args.steps
+        paired = AbiCalls(w, paired=True)
+        pb_stats = {}
+        pb = time_events(torch, paired.backward, args.steps, 2, pb_stats)
+        result["prepared_graph"] = {
+            "what": "forward + VJP through the operators with a prepare_graph handle built once "
+                    "(row pairing on): no graph preparation inside the step",
+            "ms_per_step": held_ms, "value": w.num_edges / (held_ms * 1e-3), "unit": "edges/s",
+            "frac": gbs(bytes_["fwd_bwd"], held_ms) / HBM_PEAK_GBS,
+            "backward": {"ms": pb, **pb_stats, "frac": gbs(bytes_["bwd"], pb) / HBM_PEAK_GBS}}
+        del handle, paired
     if args.layout == "trailing" and not args.kernel_only and not args.no_layouts and args.config in ("cfg2", "cfg3"):
         # the same workload in the leading-channels layout (the configurations name both), kernels only
         del abi

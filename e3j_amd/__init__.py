@@ -2,14 +2,17 @@
 
 Public names follow the reference package for this path: `Convolution`,
 `convolution`, `convolution_bwd`, `TensorProduct`, `tensor_product`, `tensor_product_bwd`,
-`Harmonics`, `GraphCSR`, `Coef4D`, `O3Space`, `config`; `radial_linear` (the radial network's last
-layer) has no counterpart there.
+`Harmonics`, `GraphCSR`, `Coef4D`, `O3Space`, `config`; `edge_features` (positions to harmonics and
+hidden radial layers in one launch), `radial_linear` (the radial network's last layer) and `ChannelMix`
+(the per-degree mixing after a convolution) have no counterpart there.
 Importing the package does not load the kernel library; the first operator call does,
 and fails if `e3j_amd/lib/libe3j_amd.so` has not been built.
 """
 
+from .channel_mix import ChannelMix
 from .coef import Coef, Coef4D, resolve_val_dtype
 from .convolution import Convolution
+from .edge_features import edge_features
 from .graph import DUMMY_INDEX, GraphCSR
 from .harmonics import Harmonics
 from .ops import (ConvolutionBatchingWarning, ConvolutionParams, CUDAConvolutionParams, TableDrivenKernelWarning,
@@ -31,6 +34,7 @@ __all__ = [
     "CUDAConvolutionParams", "DUMMY_INDEX", "GraphCSR", "GraphOrdering", "Harmonics", "Layout", "O3Irrep",
     "O3Space", "ScalarMixing", "Space", "TensorProduct", "TensorProductNormalization", "config",
     "convolution", "convolution_batched", "convolution_bwd", "radial_linear", "resolve_val_dtype",
+    "edge_features", "ChannelMix",
     "PreparedGraph", "prepare_graph", "clear_graph_cache",
     "CUDATensorProductParams", "MixingMode", "TensorProductParams", "tensor_product", "tensor_product_batched", "tensor_product_bwd",
 ]

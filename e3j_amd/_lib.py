@@ -87,6 +87,22 @@ class TpParams(ctypes.Structure):
     ]
 
 
+class EdgeFeaturesParams(ctypes.Structure):
+    """`e3j_amd_edge_features_params`."""
+
+    _fields_ = [
+        ("num_edges", ctypes.c_int64),
+        ("num_nodes", ctypes.c_int32),
+        ("l_max", ctypes.c_int32),
+        ("normalization", ctypes.c_int32),
+        ("num_basis", ctypes.c_int32),
+        ("hidden", ctypes.c_int32),
+        ("layers", ctypes.c_int32),
+        ("cutoff", ctypes.c_float),
+        ("val_dtype", ctypes.c_int32),
+    ]
+
+
 class E3jAmdError(RuntimeError):
     """Failure reported by the kernel library; `.code` is the status code."""
 
@@ -138,6 +154,10 @@ SYMBOLS = {
                                                  ctypes.POINTER(ctypes.c_int32), ctypes.c_void_p]),
     "e3j_amd_harmonics": (ctypes.c_int, [_P, ctypes.c_int64] + [ctypes.c_int32] * 4 + [_P, _P]),
     "e3j_amd_harmonics_bwd": (ctypes.c_int, [_P, _P, ctypes.c_int64] + [ctypes.c_int32] * 4 + [_P, _P]),
+    "e3j_amd_edge_features_fwd": (ctypes.c_int, [ctypes.POINTER(EdgeFeaturesParams)] + [_P] * 9),
+    "e3j_amd_edge_features_bwd": (ctypes.c_int, [ctypes.POINTER(EdgeFeaturesParams)] + [_P] * 10),
+    "e3j_amd_rows_regroup": (ctypes.c_int, [_P, _P, ctypes.c_int64, ctypes.c_int32, ctypes.c_int32, _P, _P,
+                                            ctypes.c_int32, ctypes.c_int32, _P]),
     "e3j_amd_radial_linear_fwd": (ctypes.c_int, [_P, _P, _P, ctypes.c_int64, ctypes.c_int32, ctypes.c_int32, _P]),
     "e3j_amd_radial_linear_bwd_input": (ctypes.c_int, [_P, _P, _P, ctypes.c_int64, ctypes.c_int32, ctypes.c_int32, _P]),
     "e3j_amd_radial_linear_bwd_weight_workspace_bytes": (ctypes.c_size_t, [ctypes.c_int64, ctypes.c_int32, ctypes.c_int32]),

@@ -111,9 +111,10 @@ class Config:
     tile_rows: int = -1
     #: put rows that share most of their senders side by side in the row order, so that the tiles
     #: of the default backward (two receivers at K = 128) sum more dx contributions on chip: 19 %
-    #: fewer atomic requests and a 2 % faster backward at 1M edges, for 0.28 ms more graph
-    #: preparation; worth it for a graph that serves many calls (`prepare_graph`), off by default
-    pair_rows: bool = False
+    #: fewer atomic requests and a 2-3 % faster backward at 1M edges, for 0.28 ms more graph
+    #: preparation.  "prepared" (default): only for the handles of `prepare_graph`, whose adjacency
+    #: serves many calls; True: also for the adjacency an operator call prepares for itself; False: never
+    pair_rows: object = "prepared"
     #: positions of a row one wave of the forward pass sums; longer rows are shared between waves
     #: (their sums then come from float atomics).  -1: twice the mean row length, at least 64;
     #: 0: never share a row.
@@ -140,7 +141,8 @@ class _ConfigHolder:
             tile_rows=int(os.environ.get("E3J_AMD_TILE_ROWS", "-1")),
             row_cap=int(os.environ.get("E3J_AMD_ROW_CAP", "-1")),
             fixed_order_rows=os.environ.get("E3J_AMD_FIXED_ORDER_ROWS", "1") not in ("0", ""),
-            pair_rows=os.environ.get("E3J_AMD_PAIR_ROWS", "0") not in ("0", ""),
+            pair_rows={"0": False, "": False, "1": True}.get(os.environ.get("E3J_AMD_PAIR_ROWS", "prepared"),
+                                                             "prepared"),
             graph_cache=os.environ.get("E3J_AMD_GRAPH_CACHE", "0") not in ("0", ""),
             jit=os.environ.get("E3J_AMD_JIT", "0") not in ("0", ""),
         )

@@ -19,7 +19,9 @@ import math
 import numpy as np
 import torch
 
+from .channel_mix import ChannelMix
 from .convolution import Convolution
+from .edge_features import edge_features
 from .harmonics import Harmonics
 from .options import Layout
 from .radial import radial_linear, supported as radial_supported
@@ -306,22 +308,40 @@ class EnergyModel:
         held = getattr(self, "_prepared", None)
         if x.is_cuda and (held is None or held[0] is not sender or held[1] is not receiver):
             from .ops import prepare_graph
+            # (rebuilt for every step here: pairing the rows would not pay for itself)
             held = self._prepared = (sender, receiver, prepare_graph(sender, receiver, x.shape[0],
-                                                                     self.layers[layer].graph_ordering))
+                                                                     self.layers[layer].graph_ordering,
+                                                                     pair_rows=False))
         return self.layers[layer](x, y, s, sender, receiver, graph=held[2] if x.is_cuda else None)
 
     def energy(self, positions, node_features, sender, receiver, shift, convolve=None):
+        """Scalar energy.  On the GPU (and with the library's own convolution) the steps around the
+        convolutions are kernels of the library as well: one launch from positions to harmonics and
+        hidden radial layers (`edge_features`), the matrix-core product for the radial weights
+        (`radial_linear`), one regrouping launch either side of the mixing products (`ChannelMix`).
+        Anywhere else (host tensors, a replaced `convolve`) the same formulas run as tensor
+        operations: that form is what the tests differentiate on the host."""
+        kernels = positions.is_cuda and convolve is None
         convolve = convolve or self.convolve
         self._prepared = None   # the neighbour list may have been rewritten in place since the last step
-        y, basis = self.edge_inputs(positions, sender, receiver, shift)
+        if kernels:
+            w1 = self._stacked_w1(positions)
+            y, hidden_layers = edge_features(positions, sender, receiver, shift, w1, max(self.harmonics.degrees),
+                                             self.cutoff, self.harmonics.normalization)
+            hidden_layers = hidden_layers.unbind(0)
+        else:
+            y, basis = self.edge_inputs(positions, sender, receiver, shift)
         x = node_features
         for layer, (w1, w2) in enumerate(self.mlp):
-            hidden = torch.nn.functional.silu(basis @ self._t(w1, basis))
-            last = self._t(w2, basis)
+            hidden = hidden_layers[layer] if kernels else torch.nn.functional.silu(basis @ self._t(w1, basis))
+            last = self._t(w2, hidden)
             # the weights of every path and channel: the matrix-core kernel where it applies
             s = radial_linear(hidden, last) if radial_supported(hidden, last) else hidden @ last
             s = s.reshape(-1, self.num_paths, self.channels)
             out = convolve(layer, x, y, s, sender, receiver)          # (N, Z, K)
+            if kernels:
+                x = self._mixer(layer)(out)
+                continue
             rows, mixed = 0, []
             for (mul, dim), w in zip(self.blocks, self.mix[layer]):
                 block = out[:, rows:rows + mul * dim, :].reshape(-1, mul, dim, self.channels)
@@ -329,6 +349,22 @@ class EnergyModel:
                 rows += mul * dim
             x = torch.cat(mixed, dim=1)                                # (N, X, K)
         return (x[:, 0, :] @ self._t(self.readout, x)).sum()
+
+    def _stacked_w1(self, like: torch.Tensor) -> torch.Tensor:
+        """First layers of the radial networks of all convolution layers, `(layers, num_basis, hidden)`."""
+        key = ("w1", like.dtype, like.device)
+        hit = self._weights.get(key)
+        if hit is None:
+            hit = self._weights[key] = torch.as_tensor(np.stack([w1 for w1, _ in self.mlp]), dtype=like.dtype,
+                                                       device=like.device)
+        return hit
+
+    def _mixer(self, layer: int) -> ChannelMix:
+        key = ("mixer", layer)
+        hit = self._weights.get(key)
+        if hit is None:
+            hit = self._weights[key] = ChannelMix(self.blocks, self.channels, self.mix[layer])
+        return hit
 
     def energy_and_forces(self, positions, node_features, sender, receiver, shift, convolve=None):
         positions = positions.detach().requires_grad_(True)

@@ -347,6 +347,52 @@ int e3j_amd_harmonics_bwd(const void *vec, const void *dout, int64_t num, int32_
                           int32_t normalize, int32_t normalization, int32_t val_dtype, void *dvec,
                           void *stream);
 
+/* Edge featurisation from atom positions in one launch (the producer of the convolution's operands
+ * y and, through e3j_amd_radial_linear_fwd, s): per edge e the vector
+ * positions[sender[e]] - positions[receiver[e]] (+ shift[e], the lattice translation of a periodic
+ * cell; NULL: none), then
+ *   y (num_edges, (l_max + 1)^2)          harmonics of its direction, as e3j_amd_harmonics with normalize = 1
+ *   basis (num_edges, num_basis)          sqrt(2 / cutoff) sin(n pi r / cutoff) / r, n = 1..num_basis, times the
+ *                                         envelope 1 - 10 t^3 + 15 t^4 - 6 t^5, t = min(r / cutoff, 1)   (NULL: not written)
+ *   h (layers, num_edges, hidden)         silu(basis w1[layer]), w1 (layers, num_basis, hidden): the hidden layer
+ *                                         of the radial network of each convolution layer (NULL or hidden = 0: none)
+ * An edge with an endpoint outside [0, num_nodes) or of zero length gets zeros.  The backward entry
+ * point recomputes the chain from the positions and writes dpositions (num_nodes, 3) (zero-filled by
+ * the call, contributions added with float atomics) for the cotangents dy, dbasis, dh (each may be NULL).
+ * No counterpart in the reference, whose callers build these arrays with separate XLA ops
+ * (Harmonics: src/e3j/core/harmonics.py:45-101; edge_scalars of src/e3j/core/convolution.py:342-350
+ * arrive ready-made). */
+typedef struct e3j_amd_edge_features_params {
+    int64_t num_edges;
+    int32_t num_nodes;
+    int32_t l_max;          /* <= 6 */
+    int32_t normalization;  /* 0 integral, 1 component, 2 norm */
+    int32_t num_basis;      /* 1..16 */
+    int32_t hidden;         /* width of the hidden layer, 0: none */
+    int32_t layers;         /* hidden layers evaluated side by side */
+    float   cutoff;
+    int32_t val_dtype;      /* E3J_AMD_F32 / E3J_AMD_F64 */
+} e3j_amd_edge_features_params;
+int e3j_amd_edge_features_fwd(const e3j_amd_edge_features_params *p, const void *positions,
+                              const int32_t *sender, const int32_t *receiver, const void *shift,
+                              const void *w1, void *y, void *basis, void *h, void *stream);
+int e3j_amd_edge_features_bwd(const e3j_amd_edge_features_params *p, const void *positions,
+                              const int32_t *sender, const int32_t *receiver, const void *shift,
+                              const void *w1, const void *dy, const void *dbasis, const void *dh,
+                              void *dpositions, void *stream);
+
+/* Regroups node rows around the per-degree channel mixing that follows a convolution: element
+ * (n, i, k) of a plain array (num_nodes, rows, channels) sits at row_base[i] + n * row_stride[i] + k of
+ * the regrouped array (row_base, row_stride: device, `rows` int64 each, multiples of 4 floats / 2
+ * doubles).  to_plain = 0 copies plain -> regrouped, 1 regrouped -> plain; every row moves in
+ * 16-byte pieces, one launch.  With row_base / row_stride describing A_l[(n, m), (u, k)] per output
+ * degree, the mixing x'[n, m, :] = sum_u out[n, base_l + u dim_l + m, :] W_l[u] becomes one matrix
+ * product per degree, and its backward writes every cotangent row once.  No counterpart in the
+ * reference (an einsum per degree under XLA, src/e3j/core/linear.py). */
+int e3j_amd_rows_regroup(const void *src, void *dst, int64_t num_nodes, int32_t rows, int32_t channels,
+                         const int64_t *row_base, const int64_t *row_stride, int32_t to_plain,
+                         int32_t val_dtype, void *stream);
+
 /* Last layer of the radial network that produces the convolution's per-edge, per-path weights:
  * s (num_edges, n) = h (num_edges, inner) w (inner, n), n = paths * channels, float32, row-major,
  * on the matrix cores.  inner: 8, 16, 32, 64 or 128; n: a multiple of 32.  No counterpart in the

@@ -344,3 +344,22 @@ def test_missing_library_fails_loudly(monkeypatch, tmp_path):
     monkeypatch.setattr(_lib, "LIB_PATH", str(tmp_path / "absent.so"))
     with pytest.raises(ImportError, match="no fallback"):
         _lib.load()
+
+
+def test_edge_features_and_regroup_validate_before_launching():
+    lib = _lib.load()
+    p = _lib.EdgeFeaturesParams(num_edges=4, num_nodes=3, l_max=7, normalization=1, num_basis=8, hidden=4, layers=1,
+                                cutoff=5.0, val_dtype=0)
+    assert lib.e3j_amd_edge_features_fwd(C.byref(p), *[None] * 9) == _lib.UNIMPLEMENTED      # degree 7
+    p.l_max, p.num_basis = 3, 17
+    assert lib.e3j_amd_edge_features_fwd(C.byref(p), *[None] * 9) == _lib.UNIMPLEMENTED      # 17 basis functions
+    p.num_basis, p.cutoff = 8, 0.0
+    assert lib.e3j_amd_edge_features_bwd(C.byref(p), *[None] * 10) == _lib.INVALID_ARGUMENT
+    p.cutoff, p.normalization = 5.0, 9
+    assert lib.e3j_amd_edge_features_fwd(C.byref(p), *[None] * 9) == _lib.INVALID_ARGUMENT
+    p.normalization = 1
+    assert lib.e3j_amd_edge_features_fwd(C.byref(p), *[None] * 9) == _lib.INVALID_ARGUMENT   # null y
+    assert lib.e3j_amd_edge_features_fwd(None, *[None] * 9) == _lib.INVALID_ARGUMENT
+    assert lib.e3j_amd_rows_regroup(None, None, 3, 4, 8, None, None, 0, 0, None) == _lib.INVALID_ARGUMENT
+    assert lib.e3j_amd_rows_regroup(None, None, 0, 4, 8, None, None, 0, 0, None) == _lib.OK
+    assert lib.e3j_amd_rows_regroup(None, None, -1, 4, 8, None, None, 0, 0, None) == _lib.INVALID_ARGUMENT
