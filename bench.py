@@ -81,11 +81,13 @@ def write_traffic(paths, out_path: str, key: str, kernels: dict) -> int:
                     which = "copy"
                 if which is not None and counter in ("FETCH_SIZE", "WRITE_SIZE"):
                     sums.setdefault((which, counter), []).append(float(row["Counter_Value"]))
+    # a device copy of 1 GiB in the same run, if there is one, recalibrates the two factors (the small
+    # uploads of the script are copy kernels too: anything below a quarter of a GiB is not a calibration)
+    gib_kib = float(1 << 20)
     copy_fetch = max(sums.get(("copy", "FETCH_SIZE"), [0.0]))
     copy_write = max(sums.get(("copy", "WRITE_SIZE"), [0.0]))
-    gib_kib = float(1 << 20)
-    fetch_scale = gib_kib / copy_fetch if copy_fetch else 2.0
-    write_scale = gib_kib / copy_write if copy_write else 1.0
+    fetch_scale = gib_kib / copy_fetch if copy_fetch >= gib_kib / 4 else 2.0
+    write_scale = gib_kib / copy_write if copy_write >= gib_kib / 4 else 1.0
     entry = {"fetch_scale": round(fetch_scale, 3), "write_scale": round(write_scale, 3)}
     for which in kernels:
         f = sums.get((which, "FETCH_SIZE"), [])
