@@ -432,6 +432,11 @@ def emit_table_source(t: "Table", name: str, desc: str, channels: int, symbols, 
         cpl, wpb, zs, minw = (*v, 1)[:4]
         out += [f"template __global__ void unrolled_bwd_tile_kernel<{channels}, {cpl}, {wpb}, {minw}, "
                 f"{part_names[zs]}>("] + tile_args
+    # sender-grouped backward: the finest split of the paths (parts run one after another in a wave)
+    sender_split = max(v[2] for v in launch["bwd"] + tile)
+    sender_minw = 2
+    out += [f"template __global__ void unrolled_bwd_sender_kernel<{channels}, 4, {sender_minw}, "
+            f"{part_names[sender_split]}>("] + bwd_args
     if lead:
         for wpb, zs in lead["fwd"]:
             out += [f"template __global__ void unrolled_fwd_leading_kernel<{channels}, {wpb}, {part_names[zs]}>("] + fwd_args
@@ -481,11 +486,17 @@ def emit_table_source(t: "Table", name: str, desc: str, channels: int, symbols, 
         out += ["static int run_tile_rows_default() {"]
         out += [ln.replace("VARIANT", "tuning().bwd_variant.load(std::memory_order_relaxed)") for ln in switch(
             tile, lambda v: f"{v[4] if len(v) > 4 else 8};")]
+    out += ["static int run_bwd_sender(const e3j_amd_conv_params &p, const float *x, const float *y, const float *s,",
+            "                          const float *dm, const int32_t *receiver_t, const int32_t *row_ptr,",
+            "                          const int32_t *perm, float *dx, float *dy, float *ds, hipStream_t stream) {",
+            f"    return launch_unrolled_bwd_sender<{channels}, 4, {sender_minw}, {t.Y}, {part_names[sender_split]}>(",
+            "        p, x, y, s, dm, receiver_t, row_ptr, perm, dx, dy, ds, stream);",
+            "}", ""]
     tiled = "&run_bwd_tiled, &run_tile_row_bytes, &run_tile_rows_default" if tile else "nullptr, nullptr, nullptr"
     out += [f"extern const Signature {symbols[0]} = {{",
             f'    "{desc}",',
             f"    {t.X}, {t.Y}, {t.Z}, {t.S}, {len(t.val)}, {channels}, E3J_AMD_LAYOUT_TRAILING, kVal, kIdx,",
-            f"    &run_fwd, &run_bwd, {tiled},",
+            f"    &run_fwd, &run_bwd, {tiled}, &run_bwd_sender,",
             "};", ""]
     if lead:
         out += ["static int run_fwd_leading" + fwd_sig[0]] + fwd_sig[1:]

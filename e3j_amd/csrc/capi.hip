@@ -161,6 +161,16 @@ int run_backward(const e3j_amd_conv_params *p, bool group_is_receiver, const voi
         if (rc == E3J_AMD_OK)
             rc = launch_zero_padding(*p, other, row_ptr, edge_perm, static_cast<float *>(dy),
                                      static_cast<float *>(ds), stream);
+    } else if (!group_is_receiver && p->layout == E3J_AMD_LAYOUT_TRAILING && signature_fits(p, {x, s, dm, dx, ds}) &&
+               signature(p->signature).bwd_sender != nullptr) {
+        // the reference's grouping on the unrolled kernels: rows own their dx (no atomics)
+        rc = signature(p->signature).bwd_sender(*p, static_cast<const float *>(x), static_cast<const float *>(y),
+                                                static_cast<const float *>(s), static_cast<const float *>(dm),
+                                                other, row_ptr, edge_perm, static_cast<float *>(dx),
+                                                static_cast<float *>(dy), static_cast<float *>(ds), stream);
+        if (rc == E3J_AMD_OK)
+            rc = launch_zero_padding(*p, other, row_ptr, edge_perm, static_cast<float *>(dy),
+                                     static_cast<float *>(ds), stream);
     } else {
         if ((rc = flip_without_kernel(p, op))) return rc;
         if (coef == nullptr && p->num_coef > 0)

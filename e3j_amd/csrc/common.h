@@ -171,6 +171,11 @@ struct Signature {
                      float *ds, hipStream_t stream);
     int (*tile_row_bytes)();
     int (*tile_rows_default)();  // receivers per tile the launch variant is tuned for
+    // backward on the sender-grouped adjacency (receiver per position, row pointer by sender): dx
+    // owned by the rows, no atomics on it (nullptr: none, the table-driven kernel serves that grouping)
+    int (*bwd_sender)(const e3j_amd_conv_params &p, const float *x, const float *y, const float *s,
+                      const float *dm, const int32_t *receiver_t, const int32_t *sender_ptr,
+                      const int32_t *edge_perm, float *dx, float *dy, float *ds, hipStream_t stream);
 };
 // built-in signatures (generated/registry.hip), then the ones registered at run time (capi.hip)
 // A table entry on the host, and the lookup of a table among the signatures (capi.hip): the

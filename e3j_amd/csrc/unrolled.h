@@ -332,6 +332,11 @@ struct Slice {
     static_assert(K % CPL == 0, "channels must be a multiple of the per-lane vector width");
 };
 
+template <typename First, typename...>
+struct FirstOfParts {
+    using type = First;
+};
+
 // ---------------------------------------------------------------------------
 // forward
 // ---------------------------------------------------------------------------
@@ -656,6 +661,115 @@ void unrolled_bwd_kernel(
                                                            dy, ds, num_nodes, scale, y_flip,
                                                            part * CW + slice, NP * CW, r, slice,
                                                            threadIdx.x);
+}
+
+// ---------------------------------------------------------------------------
+// backward, sender-grouped (the operands of the reference's "convolution_bwd"): the rows of the
+// adjacency are senders.  A wave owns (sender, 64 channels): the sender's x row stays in
+// registers, the dx sums of the row are kept in registers and stored once (no atomics, the
+// same bits in every run), and the dm rows of every edge's receiver are gathered.  All parts
+// of the signature run one after another in the wave (their dm rows are loaded per edge
+// anyway), so an edge's dy is complete in the wave: stored directly at 64 channels and below,
+// added by the K / 64 waves of an edge above (two addends at 128 channels: still the same
+// bits in every run).  The gather of dm (Z rows per edge where the receiver-grouped kernels
+// gather X) makes this the slower grouping; it needs no schedule, no workspace and no sort.
+// ---------------------------------------------------------------------------
+template <int K>
+struct DsRowsScaled {  // one channel per lane: the edge's row of ds, values times `scale`
+    float *row;
+    bool active;
+    float scale;
+    template <int L>
+    __device__ __forceinline__ void put(const Vec<1> &v) const {
+        if (active) __builtin_nontemporal_store(v.v[0] * scale, row + L * K);
+    }
+};
+
+template <typename Part, int K>
+__device__ __forceinline__ void bwd_sender_stage(const Vec<1> *x_all, const float *yc, const float *sr,
+                                                 const float *zr, Vec<1> *dx_all, float *dy_all,
+                                                 const DsRowsScaled<K> &ds_rows, bool active) {
+    constexpr int NX = Part::NX, NS = Part::NS, NZ = Part::NZ, Y = Part::Y;
+    using V = Vec<1>;
+    V xl[NX], dxl[NX], sl[NS], dml[NZ];
+#pragma unroll
+    for (int i = 0; i < NZ; i++) {
+        dml[i] = load_vec<1>(zr + Part::kZ[i] * K);
+        if (!active) dml[i] = vzero<1>();  // idle lanes must add nothing to dy
+    }
+#pragma unroll
+    for (int l = 0; l < NS; l++) sl[l] = load_stream<1>(sr + Part::kS[l] * K);
+#pragma unroll
+    for (int j = 0; j < NX; j++) {
+        xl[j] = x_all[Part::kX[j]];
+        dxl[j] = dx_all[Part::kX[j]];
+    }
+    float dyp[Y];
+    Part::template edge_bwd<1, true, false>(xl, yc, sl, dml, dxl, dyp, ds_rows);
+#pragma unroll
+    for (int j = 0; j < NX; j++) dx_all[Part::kX[j]] = dxl[j];
+#pragma unroll
+    for (int k = 0; k < Y; k++) dy_all[k] += dyp[k];
+}
+
+template <int K, int WPB, int MINW, typename... Parts>
+__global__ __launch_bounds__(kWave *WPB, MINW) void unrolled_bwd_sender_kernel(
+    const float *__restrict__ x, const float *__restrict__ y, const float *__restrict__ s,
+    const float *__restrict__ dm, const int32_t *__restrict__ receiver_t,
+    const int32_t *__restrict__ row_ptr, const int32_t *__restrict__ perm,
+    const int32_t *__restrict__ row_order, float *__restrict__ dx, float *__restrict__ dy,
+    float *__restrict__ ds, int num_nodes, float scale, unsigned y_flip) {
+    using P0 = typename FirstOfParts<Parts...>::type;
+    constexpr int X = P0::X, Y = P0::Y, S = P0::S, Z = P0::Z;
+    using SL = Slice<K, 1>;
+    using V = Vec<1>;
+    using Red = WaveReduceBlocks<Y, kWave>;
+    constexpr int CW = SL::COUNT;
+    const int64_t item = logical_block() * WPB + threadIdx.y;
+    if (item >= (int64_t)num_nodes * CW) return;
+    const int slice = uniform((int)(item % CW));
+    const int q = uniform((int)(item / CW));
+    const int r = uniform(row_order ? row_order[q] : q);
+    const int lane = threadIdx.x;
+    const int c_raw = slice * SL::WIDTH + lane;
+    const bool active = SL::FULL || c_raw < K;
+    const int c0 = active ? c_raw : 0;
+
+    V xr[X], acc[X];
+    {
+        const float *xp = x + (int64_t)r * (X * K) + c0;
+#pragma unroll
+        for (int j = 0; j < X; j++) {
+            xr[j] = load_vec<1>(xp + j * K);
+            acc[j] = vzero<1>();
+        }
+    }
+    const int e1 = row_ptr[r + 1];
+    for (int pos = row_ptr[r]; pos < e1; pos++) {
+        const int rcv = uniform(receiver_t[pos]);
+        if (!((unsigned)rcv < (unsigned)num_nodes)) continue;  // padding edge: dy / ds zero-filled separately
+        const int64_t ee = perm ? (int64_t)uniform(perm[pos]) : (int64_t)pos;
+        const float *yr = y + ee * Y;
+        float yc[Y], dye[Red::P];
+#pragma unroll
+        for (int k = 0; k < Y; k++) yc[k] = to_vgpr(flip_sign(yr[k], y_flip, k));
+#pragma unroll
+        for (int k = 0; k < Red::P; k++) dye[k] = 0.f;
+        const DsRowsScaled<K> ds_rows{ds + ee * (int64_t)(S * K) + c0, active, scale};
+        const float *sr = s + ee * (int64_t)(S * K) + c0;
+        const float *zr = dm + (int64_t)rcv * (Z * K) + c0;
+        (bwd_sender_stage<Parts, K>(xr, yc, sr, zr, acc, dye, ds_rows, active), ...);
+        Red::run(dye, lane, [&](int k, float sum) {
+            const float total = flip_sign(sum * scale, y_flip, k);
+            if (CW == 1) dy[ee * Y + k] = total;
+            else unsafeAtomicAdd(dy + ee * Y + k, total);  // dy zero-filled by the launcher
+        });
+    }
+    if (active) {  // the row's dx, written once; coordinates no coefficient touches get zeros
+        float *dxp = dx + (int64_t)r * (X * K) + c0;
+#pragma unroll
+        for (int j = 0; j < X; j++) dxp[j * K] = acc[j].v[0] * scale;
+    }
 }
 
 // ---------------------------------------------------------------------------
@@ -1458,6 +1572,24 @@ int launch_unrolled_bwd(const e3j_amd_conv_params &p, const float *x, const floa
                            dim3(kWave, WPB), 0, stream, x, y, s, dm, sender, row_ptr, perm, p.row_order,
                            dx, dy, ds, p.num_nodes, p.coef_scale, p.y_flip);
     return check_hip(hipGetLastError(), "convolution backward launch");
+}
+
+template <int K, int WPB, int MINW, int Y, typename... Parts>
+int launch_unrolled_bwd_sender(const e3j_amd_conv_params &p, const float *x, const float *y, const float *s,
+                               const float *dm, const int32_t *receiver_t, const int32_t *row_ptr,
+                               const int32_t *perm, float *dx, float *dy, float *ds, hipStream_t stream) {
+    constexpr int CW = Slice<K, 1>::COUNT;
+    if (CW > 1) {  // several waves add into one dy row
+        const int rc = launch_fill_zero(dy, sizeof(float) * (size_t)p.num_edges * Y, stream);
+        if (rc) return rc;
+    }
+    const int64_t blocks = padded_grid(((int64_t)p.num_nodes * CW + WPB - 1) / WPB);
+    if (blocks > 0x7fffffffLL) return set_error(E3J_AMD_INVALID_ARGUMENT, "convolution_bwd: grid too large");
+    if (blocks == 0) return E3J_AMD_OK;
+    hipLaunchKernelGGL((unrolled_bwd_sender_kernel<K, WPB, MINW, Parts...>), dim3((unsigned)blocks),
+                       dim3(kWave, WPB), 0, stream, x, y, s, dm, receiver_t, row_ptr, perm, p.row_order, dx, dy,
+                       ds, p.num_nodes, p.coef_scale, p.y_flip);
+    return check_hip(hipGetLastError(), "convolution backward (sender rows) launch");
 }
 
 constexpr int max_of(std::initializer_list<int> v) {

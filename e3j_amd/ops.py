@@ -443,12 +443,18 @@ def _raw_backward(meta: _Meta, x, y, s, dm, sender, receiver, graph=None):
     # are sorted by receiver on the device and the receiver-grouped backward runs on them
     # (results land on the edges' own rows through the permutation); otherwise the
     # table-driven kernel keeps the sender rows, gathers dm and owns dx.
-    sender_rows = meta.ordering == GraphOrdering.SENDER and not has_kernel
+    # deterministic, with an unrolled kernel: in the trailing layout up to 128 channels the
+    # sender-grouped unrolled backward (rows own their dx, an edge's dy comes from at most two waves:
+    # the same bits in every run, no workspace); otherwise the atomic-free backward on receiver rows
+    # (per-position dx rows in a workspace, summed in a fixed order); tables without a kernel fall
+    # back to the table-driven kernel on sender rows
+    channels = _shape(meta, x, y, s)[1]
+    sender_kernel = (deterministic and has_kernel and meta.layout == Layout.TRAILING_CHANNELS and channels <= 128
+                     and x.dtype == torch.float32
+                     and all(t.data_ptr() % 16 == 0 for t in (x, y, s, dm, dx, dy, ds)))
+    sender_rows = meta.ordering == GraphOrdering.SENDER and (not has_kernel or sender_kernel)
     resort = meta.ordering in (GraphOrdering.NONE, GraphOrdering.SENDER) and not sender_rows
-    # deterministic: the atomic-free backward of the unrolled kernels on receiver rows
-    # (per-position dx rows summed in a fixed order); tables without such a kernel fall back
-    # to the table-driven kernel on sender rows
-    ordered = deterministic and has_kernel
+    ordered = deterministic and has_kernel and not sender_kernel
     forward_rows = meta.ordering != GraphOrdering.SENDER   # the forward's rows are receivers
     reuse = graph is not None and (
         (forward_rows and (not deterministic or ordered)) or sender_rows)
@@ -466,7 +472,14 @@ def _raw_backward(meta: _Meta, x, y, s, dm, sender, receiver, graph=None):
             # already grouped by sender: rows own their dx, no permutation
             group_receiver, other, row_ptr, perm = False, receiver_l.contiguous(), csr_row_ptr(sender_l, n), None
         elif deterministic and not ordered:
-            perm, other, row_ptr = sort_edges(sender_l, receiver_l, n)
+            if meta.ordering == GraphOrdering.NONE:
+                # by receiver first (stable), then by sender (stable): the order in which a sender's
+                # contributions are summed then does not depend on the order the edges came in
+                by_rcv, snd_sorted, _ = sort_edges(receiver_l, sender_l, n)
+                perm2, other, row_ptr = sort_edges(snd_sorted, receiver_l[by_rcv.long()].contiguous(), n)
+                perm = by_rcv[perm2.long()].contiguous()
+            else:
+                perm, other, row_ptr = sort_edges(sender_l, receiver_l, n)
             group_receiver = False
         elif resort:
             perm, other, row_ptr = sort_edges(receiver_l, sender_l, n)
@@ -474,7 +487,7 @@ def _raw_backward(meta: _Meta, x, y, s, dm, sender, receiver, graph=None):
         else:
             group_receiver, other, row_ptr, perm = True, sender_l.contiguous(), csr_row_ptr(receiver_l, n), None
         order = (graph[3] if graph is not None and forward_rows else _row_order(other, row_ptr, n))
-    p, table = _fill_params(meta, x, y, s, table, use_signature=group_receiver, row_order=order)
+    p, table = _fill_params(meta, x, y, s, table, use_signature=group_receiver or sender_kernel, row_order=order)
     args = (ctypes.byref(p), table.device(x.device).data_ptr(), x.data_ptr(), y.data_ptr(),
             s.data_ptr(), dm.data_ptr(), other.data_ptr(), row_ptr.data_ptr(),
             perm.data_ptr() if perm is not None else None,

@@ -126,7 +126,13 @@ int e3j_amd_convolution_fwd(const e3j_amd_conv_params *p, const void *coef,
  * position, sender_ptr = row pointer by sender, edge_perm = position -> original
  * edge (NULL under SENDER ordering).  `coef` is the FORWARD table (i, j, k, l);
  * the reference's three transposed copies are not needed.  dx is accumulated
- * row-locally without atomics: results are bit-reproducible run to run. */
+ * row-locally without atomics: results are bit-reproducible run to run.
+ * With p->signature >= 0 (trailing layout, float32, 16-byte aligned operands) the
+ * compile-time-unrolled kernels serve this grouping too: a wave per (sender, 64 channels)
+ * keeps the sender's x row and its dx sums in registers and gathers the dm rows of the
+ * receivers; `coef` is then not read.  dy of an edge is added by channels / 64 waves: the
+ * same bits in every run up to 128 channels (two addends), equal up to the order of four
+ * additions at 256.  Other operands run the table-driven kernel, which owns dx and dy. */
 int e3j_amd_convolution_bwd_sender(const e3j_amd_conv_params *p, const void *coef,
                                    const void *x, const void *y, const void *s, const void *dm,
                                    const int32_t *receiver_t, const int32_t *sender_ptr,

@@ -375,3 +375,74 @@ def test_views_at_odd_element_offsets_are_served():
     rc = _lib.load().e3j_amd_radial_linear_fwd(shifted(h).data_ptr(), wt.data_ptr(), s_out.data_ptr(), 256, 32, 64,
                                                int(torch.cuda.current_stream().cuda_stream))
     assert rc == _lib.INVALID_ARGUMENT and b"16-byte" in _lib.load().e3j_amd_last_error()
+
+
+@pytest.mark.parametrize("name", ["cfg3", "cfg3_k64", "cfg2", "cfg2_k32", "cfg3_k256", "scalars_k64"])
+def test_sender_grouped_backward_on_the_unrolled_kernels(name):
+    """`e3j_amd_convolution_bwd_sender` with a signature: the reference's grouping (rows are senders,
+    `lib/e3j_ops/ffi/e3j_ops.h:575-594`) on the unrolled kernels.  Against the oracle, with padding
+    edges and through an edge permutation; dx (and dy up to 128 channels) the same bits in every run;
+    a scaled table and a sign mask behave as on the receiver-grouped kernels."""
+    import ctypes as C
+    from oracle import conv_oracle as O
+    w = CASES[name]()
+    sig, scale, _ = _signature_of(w)
+    assert sig >= 0
+    a = w.numpy()
+    n, e = w.num_nodes, w.num_edges
+    rng = np.random.default_rng(17)
+    snd, rcv = a["sender"].copy(), a["receiver"].copy()
+    pad = rng.choice(e, size=max(e // 50, 2), replace=False)
+    snd[pad[::2]] = np.iinfo(np.int32).max        # padding edges of both kinds
+    rcv[pad[1::2]] = np.iinfo(np.int32).max
+    perm, recv_t, sptr = O.transpose_graph(snd, rcv, n)   # positions grouped by sender
+    m = w.module
+    dims = (int(w.x.shape[1]), int(w.y.shape[1]), m.params.num_out, int(w.s.shape[1]))
+    lib = _lib.load()
+    dev = lambda t: torch.as_tensor(np.ascontiguousarray(t)).cuda()  # noqa: E731
+    x, y, s, dm = (dev(a[k]) for k in ("x", "y", "s", "dm"))
+    recv_d, sptr_d, perm_d = dev(recv_t.astype(np.int32)), dev(sptr.astype(np.int32)), dev(perm.astype(np.int32))
+    idx, val, mix = w.table()
+    (rx, ry, rs), (mx, my, ms) = H.backward_reference(idx, val, mix, a["x"], a["y"], a["s"], snd, rcv, a["dm"])
+
+    def run(coef_scale=1.0, y_flip=0):
+        p = _lib.ConvParams(num_nodes=n, num_edges=e, num_coef=len(val), num_x=dims[0], num_y=dims[1],
+                            num_out=dims[2], num_scalars=dims[3], channels=w.channels, layout=_lib.LAYOUT_TRAILING,
+                            val_dtype=_lib.F32, coef_idx_bytes=1, signature=sig, coef_scale=coef_scale * scale,
+                            debug=0, y_flip=y_flip, row_order=None)
+        dx, dy, ds = (torch.full_like(t, float("nan")) for t in (x, y, s))
+        _lib.check(lib.e3j_amd_convolution_bwd_sender(
+            C.byref(p), None, x.data_ptr(), y.data_ptr(), s.data_ptr(), dm.data_ptr(), recv_d.data_ptr(),
+            sptr_d.data_ptr(), perm_d.data_ptr(), dx.data_ptr(), dy.data_ptr(), ds.data_ptr(),
+            int(torch.cuda.current_stream().cuda_stream)))
+        torch.cuda.synchronize()
+        return dx, dy, ds
+
+    dx, dy, ds = run()
+    H.assert_parity(dx.cpu().numpy(), rx, mx, f"{name} dx")
+    H.assert_parity(dy.cpu().numpy(), ry, my, f"{name} dy")
+    H.assert_parity(ds.cpu().numpy(), rs, ms, f"{name} ds")
+    dead = (snd >= n) | (rcv >= n)
+    assert not dy.cpu().numpy()[dead].any() and not ds.cpu().numpy()[dead].any()      # exact zeros
+    dx2, dy2, ds2 = run()
+    assert torch.equal(dx, dx2) and torch.equal(ds, ds2)
+    if w.channels <= 128:
+        assert torch.equal(dy, dy2)
+    # a uniformly scaled table
+    dx3, dy3, ds3 = run(coef_scale=0.25)
+    for g, g0 in ((dx3, dx), (dy3, dy), (ds3, ds)):
+        assert float((g - 0.25 * g0).abs().max()) <= 2e-6 * float(g0.abs().max())
+    # the sign mask on y: as if y[:, k] were negated, with dy[:, k] returned negated
+    mask = 0b1010
+    signs = torch.ones(dims[1], device="cuda")
+    signs[1], signs[3] = -1.0, -1.0
+    dx4, dy4, ds4 = run(y_flip=mask)
+    y_keep = y.clone()
+    y.mul_(signs)
+    dx5, dy5, ds5 = run()
+    y.copy_(y_keep)
+    assert torch.equal(dx4, dx5) and torch.equal(ds4, ds5)
+    if w.channels <= 128:
+        assert torch.equal(dy4, dy5 * signs)
+    else:   # four waves add into a dy row: equal up to the order of those additions
+        assert float((dy4 - dy5 * signs).abs().max()) <= 1e-5 * float(dy5.abs().max())
