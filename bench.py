@@ -37,8 +37,8 @@ HBM_PEAK_GBS = 8000.0
 #: HBM bytes per launch come from `profiles/traffic.json`: two `rocprofv3 --pmc` runs of this
 #: script (FETCH_SIZE and WRITE_SIZE, KiB per dispatch), each scaled by what the same counter reads
 #: for a 1 GiB device copy (FETCH_SIZE counts half of the bytes read, factor 2.0; WRITE_SIZE all of
-#: the bytes written, factor 1.0; a copy kernel found in the CSVs overrides the two factors), written
-#: by `python bench.py --write-traffic ...` together with a hash of the kernel sources.  A figure is only quoted while the sources it was
+#: the bytes written, factor 1.0), written by `python bench.py --write-traffic ...` together with a
+#: hash of the kernel sources.  A figure is only quoted while the sources it was
 #: measured on are the ones in the tree.
 TRAFFIC_FILE = os.path.join(ROOT, "profiles", "traffic.json")
 KERNEL_SOURCES = ("e3j_amd/csrc/unrolled.h", "e3j_amd/csrc/common.h", "e3j_amd/csrc/tp_unrolled.h",
@@ -77,17 +77,11 @@ def write_traffic(paths, out_path: str, key: str, kernels: dict) -> int:
             for row in csv.DictReader(fh):
                 name, counter = row["Kernel_Name"], row["Counter_Name"]
                 which = next((k for k, sub in kernels.items() if sub in name), None)
-                if "copyBuffer" in name or "copy" in name.lower() and which is None:
-                    which = "copy"
                 if which is not None and counter in ("FETCH_SIZE", "WRITE_SIZE"):
                     sums.setdefault((which, counter), []).append(float(row["Counter_Value"]))
-    # a device copy of 1 GiB in the same run, if there is one, recalibrates the two factors (the small
-    # uploads of the script are copy kernels too: anything below a quarter of a GiB is not a calibration)
-    gib_kib = float(1 << 20)
-    copy_fetch = max(sums.get(("copy", "FETCH_SIZE"), [0.0]))
-    copy_write = max(sums.get(("copy", "WRITE_SIZE"), [0.0]))
-    fetch_scale = gib_kib / copy_fetch if copy_fetch >= gib_kib / 4 else 2.0
-    write_scale = gib_kib / copy_write if copy_write >= gib_kib / 4 else 1.0
+    # FETCH_SIZE counts half of the bytes read and WRITE_SIZE all of the bytes written: what the two
+    # counters read for a 1 GiB device copy on this GPU (524 300 and 1 048 576 KiB)
+    fetch_scale, write_scale = 2.0, 1.0
     entry = {"fetch_scale": round(fetch_scale, 3), "write_scale": round(write_scale, 3)}
     for which in kernels:
         f = sums.get((which, "FETCH_SIZE"), [])
