@@ -178,6 +178,17 @@ class AbiCalls:
             channels=w.channels, layout=module.layout.value, val_dtype=_lib.F32,
             coef_idx_bytes=self.table.idx_bytes, signature=sig, coef_scale=scale, debug=0)
         self.coef = self.table.device(w.x.device)
+        if table_driven:   # the plan of the table built once, as the operators do on a table's first call
+            nbytes = int(self.lib.e3j_amd_table_plan_bytes(ctypes.byref(self.params)))
+            if nbytes:
+                self.plan = torch.empty((nbytes + 3) // 4, dtype=torch.int32, device=w.x.device)
+                self.params.table_plan = self.plan.data_ptr()
+                status = (ctypes.c_int32 * 4)()
+                _lib.check(self.lib.e3j_amd_table_plan_status(ctypes.byref(self.params), self.coef.data_ptr(), 0,
+                                                              status, int(torch.cuda.current_stream().cuda_stream)))
+                if not status[0]:
+                    self.params.table_plan = None
+                self.params.table_plan_state = _lib.PLAN_READY if status[0] else _lib.PLAN_NONE
         if module.graph_ordering.value == "NONE":
             self.perm, self.other, self.ptr = sort_edges(w.receiver, w.sender, w.num_nodes)
         else:

@@ -18,6 +18,7 @@ LIB_PATH = os.environ.get("E3J_AMD_LIBRARY") or os.path.join(_HERE, "lib", "libe
 OK, INVALID_ARGUMENT, UNIMPLEMENTED, INTERNAL = 0, 1, 2, 3
 LAYOUT_LEADING, LAYOUT_TRAILING = 0, 1
 F32, F64, F16 = 0, 1, 2
+PLAN_BUILD, PLAN_READY, PLAN_NONE = 0, 1, 2
 
 
 class ConvParams(ctypes.Structure):
@@ -46,6 +47,7 @@ class ConvParams(ctypes.Structure):
         ("segments", ctypes.c_void_p),
         ("partials", ctypes.c_void_p),
         ("table_plan", ctypes.c_void_p),
+        ("table_plan_state", ctypes.c_int32),
     ]
 
 

@@ -349,17 +349,19 @@ int pick_waves(size_t per_wave_bytes, size_t budget) {
 template <typename Idx, typename Val>
 int run_fwd(const e3j_amd_conv_params &p, const void *coef, const void *x, const void *y,
             const void *s, const int32_t *other, const int32_t *row_ptr, const int32_t *perm,
-            void *out, hipStream_t stream, const int32_t *plan) {
+            void *out, hipStream_t stream, const int32_t *plan, bool plan_only) {
     const int nchunks = (p.channels + kWave - 1) / kWave;
+    if (plan && plan_only)  // a plan the caller vouches for: the planned kernel alone
+        return launch_planned_fwd(p, plan, x, y, s, other, row_ptr, perm, out, stream);
+    const size_t per_wave = (size_t)(p.num_out + p.num_x + p.num_scalars) * kWave * sizeof(Val);
+    if (per_wave > kMaxLds)  // (before anything is launched)
+        return set_error(E3J_AMD_UNIMPLEMENTED, "convolution: num_out + num_x + num_scalars = " +
+                         std::to_string(p.num_out + p.num_x + p.num_scalars) +
+                         " exceeds the LDS capacity of the table-driven kernel");
     if (plan) {  // runs if the plan took the table; the kernel below runs if it did not
         int rc = launch_planned_fwd(p, plan, x, y, s, other, row_ptr, perm, out, stream);
         if (rc) return rc;
     }
-    const size_t per_wave = (size_t)(p.num_out + p.num_x + p.num_scalars) * kWave * sizeof(Val);
-    if (per_wave > kMaxLds)
-        return set_error(E3J_AMD_UNIMPLEMENTED, "convolution: num_out + num_x + num_scalars = " +
-                         std::to_string(p.num_out + p.num_x + p.num_scalars) +
-                         " exceeds the LDS capacity of the table-driven kernel");
     const int waves = pick_waves(per_wave, 64 * 1024);
     const size_t lds = per_wave * waves;
     // y rows of up to 64 components travel in a register of the wave
@@ -399,7 +401,7 @@ template <typename Idx, typename Val>
 int run_bwd(const e3j_amd_conv_params &p, bool group_is_receiver, const void *coef, const void *x,
             const void *y, const void *s, const void *dm, const int32_t *other,
             const int32_t *row_ptr, const int32_t *perm, void *dx, void *dy, void *ds,
-            hipStream_t stream, bool cols_ji, const int32_t *plan) {
+            hipStream_t stream, bool cols_ji, const int32_t *plan, bool plan_only) {
     const int nchunks = (p.channels + kWave - 1) / kWave;
     if (std::is_same<Val, half_t>::value && group_is_receiver)
         // no float atomics on half values: rows must own their dx (sender-grouped)
@@ -408,7 +410,7 @@ int run_bwd(const e3j_amd_conv_params &p, bool group_is_receiver, const void *co
                          "float atomics has no half-precision form)");
     const size_t per_wave =
         (size_t)(p.num_out + 2 * p.num_x + 2 * p.num_scalars + p.num_y) * kWave * sizeof(Val);
-    if (per_wave > kMaxLds)
+    if (per_wave > kMaxLds && !(plan && plan_only))
         return set_error(E3J_AMD_UNIMPLEMENTED,
                          "convolution_bwd: irreps dimensions exceed the LDS capacity of the "
                          "table-driven kernel");
@@ -431,7 +433,7 @@ int run_bwd(const e3j_amd_conv_params &p, bool group_is_receiver, const void *co
     if (rc) return rc;
     if (plan) {  // runs if the plan took the table; the kernel below runs if it did not
         rc = launch_planned_bwd(p, group_is_receiver, plan, x, y, s, dm, other, row_ptr, perm, dx, dy, ds, stream);
-        if (rc) return rc;
+        if (rc || plan_only) return rc;  // (a plan the caller vouches for: the planned kernel alone)
     }
 #define E3J_LAUNCH_BWD(FLAG)                                                                      \
     do {                                                                                          \
@@ -567,10 +569,26 @@ int launch_zero_padding(const e3j_amd_conv_params &p, const int32_t *other, cons
 struct PlanScratch {
     int32_t *plan = nullptr;
     bool pooled = false;  // plan memory taken from the stream's pool (given back when the call returns)
+    bool ready = false;   // the caller vouches for a plan built earlier that takes the table: no other kernel runs
     hipStream_t stream;
     int rc = E3J_AMD_OK;
     PlanScratch(const e3j_amd_conv_params &p, const void *coef, bool cols_ji, hipStream_t st) : stream(st) {
+        if (p.table_plan_state == E3J_AMD_PLAN_NONE) return;
+        if (p.table_plan_state != E3J_AMD_PLAN_BUILD && p.table_plan_state != E3J_AMD_PLAN_READY) {
+            rc = set_error(E3J_AMD_INVALID_ARGUMENT, "convolution: unknown table_plan_state");
+            return;
+        }
         if (!plan_takes(p) || !table_plans().load(std::memory_order_relaxed)) return;
+        if (p.table_plan_state == E3J_AMD_PLAN_READY) {
+            if (p.table_plan == nullptr || reinterpret_cast<uintptr_t>(p.table_plan) % alignof(int32_t) != 0) {
+                rc = set_error(E3J_AMD_INVALID_ARGUMENT,
+                               "convolution: table_plan_state says the plan is ready, table_plan holds none");
+                return;
+            }
+            plan = p.table_plan;
+            ready = true;
+            return;
+        }
         if (p.table_plan != nullptr) {  // the caller's memory: nothing allocated, fine under capture
             if (reinterpret_cast<uintptr_t>(p.table_plan) % alignof(int32_t) != 0) {
                 rc = set_error(E3J_AMD_INVALID_ARGUMENT, "convolution: table_plan must be 4-byte aligned");
@@ -617,7 +635,7 @@ int launch_generic_fwd(const e3j_amd_conv_params &p, const void *coef, const voi
     const PlanScratch scratch(p, coef, false, stream);
     if (scratch.rc) return scratch.rc;
     const int32_t *plan = scratch.plan;
-#define E3J_FWD(I, V) run_fwd<I, V>(p, coef, x, y, s, other, row_ptr, edge_perm, out, stream, plan)
+#define E3J_FWD(I, V) run_fwd<I, V>(p, coef, x, y, s, other, row_ptr, edge_perm, out, stream, plan, scratch.ready)
     E3J_DISPATCH(E3J_FWD);
 #undef E3J_FWD
 }
@@ -631,7 +649,7 @@ int launch_generic_bwd(const e3j_amd_conv_params &p, bool group_is_receiver, con
     const int32_t *plan = scratch.plan;
 #define E3J_BWD(I, V)                                                                            \
     run_bwd<I, V>(p, group_is_receiver, coef, x, y, s, dm, other, row_ptr, edge_perm, dx, dy, ds, \
-                  stream, coef_cols_ji, plan)
+                  stream, coef_cols_ji, plan, scratch.ready)
     E3J_DISPATCH(E3J_BWD);
 #undef E3J_BWD
 }

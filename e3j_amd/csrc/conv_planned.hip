@@ -46,15 +46,19 @@ extern "C" int e3j_amd_table_plan_status(const e3j_amd_conv_params *p, const voi
     status[0] = status[1] = status[2] = status[3] = 0;
     if (!plan_takes(*p)) return E3J_AMD_OK;
     hipStream_t stream = static_cast<hipStream_t>(stream_);
-    void *mem = nullptr;
-    int rc = check_hip(hipMalloc(&mem, plan_bytes(*p)), "table_plan_status: hipMalloc");
+    void *mem = p->table_plan;  // the caller's memory: the plan is built there and stays
+    const bool own = mem == nullptr;
+    int rc = E3J_AMD_OK;
+    if (own) rc = check_hip(hipMalloc(&mem, plan_bytes(*p)), "table_plan_status: hipMalloc");
+    else if (reinterpret_cast<uintptr_t>(mem) % alignof(int32_t) != 0)
+        rc = set_error(E3J_AMD_INVALID_ARGUMENT, "table_plan_status: table_plan must be 4-byte aligned");
     if (rc) return rc;
     rc = launch_plan_build(*p, coef, coef_cols_ji != 0, static_cast<int32_t *>(mem), stream);
     int32_t header[kHeaderWords] = {0};
     if (!rc) rc = check_hip(hipMemcpyAsync(header, mem, sizeof(header), hipMemcpyDeviceToHost, stream),
                             "table_plan_status: copy");
     if (!rc) rc = check_hip(hipStreamSynchronize(stream), "table_plan_status: synchronize");
-    (void)hipFree(mem);
+    if (own) (void)hipFree(mem);
     if (rc) return rc;
     status[0] = header[kEligible];
     status[1] = header[kNumCells];

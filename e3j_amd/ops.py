@@ -69,6 +69,7 @@ class _Table:
         self._device = {}
         self._signature = {}
         self._signed = {}
+        self._plans = {}   # (device, value dtype, sizes) -> (plan of the table-driven kernels, taken)
 
     #: tables by the identity of the packed array (a module hands over the same array on every
     #: call): the bytes of a table are hashed once, not per call
@@ -200,16 +201,34 @@ def _fill_params(meta: _Meta, x: torch.Tensor, y: torch.Tensor, s: torch.Tensor,
     return p, table
 
 
-def _table_plan(p, device) -> torch.Tensor | None:
-    """Memory for the plan of a table-driven call (the caller keeps it until the call is enqueued):
-    with it the library allocates nothing, also while the stream is captured into a graph."""
+def _table_plan(p, table, device) -> torch.Tensor | None:
+    """The plan of a table-driven call.  Outside a graph capture it is built once per (table, sizes,
+    device) by the status call, which also says whether the planned kernels take the table: later
+    calls launch that kernel alone (`PLAN_READY`) or skip planning (`PLAN_NONE`).  While the stream is
+    captured (the status call synchronises) a table not seen before gets memory for a plan built
+    inside the call, which the caller keeps until the call is enqueued: the library then allocates
+    nothing."""
     if p.signature >= 0:
         return None
-    nbytes = int(_lib.load().e3j_amd_table_plan_bytes(ctypes.byref(p)))
+    lib = _lib.load()
+    nbytes = int(lib.e3j_amd_table_plan_bytes(ctypes.byref(p)))
     if nbytes == 0:
+        p.table_plan_state = _lib.PLAN_NONE
         return None
-    plan = torch.empty((nbytes + 3) // 4, dtype=torch.int32, device=device)
-    p.table_plan = plan.data_ptr()
+    key = (device, int(p.val_dtype), p.num_x, p.num_y, p.num_out, p.num_scalars)
+    hit = table._plans.get(key)
+    if hit is None:
+        plan = torch.empty((nbytes + 3) // 4, dtype=torch.int32, device=device)
+        p.table_plan = plan.data_ptr()
+        if torch.cuda.is_current_stream_capturing():
+            return plan
+        status = (ctypes.c_int32 * 4)()
+        _lib.check(lib.e3j_amd_table_plan_status(ctypes.byref(p), table.device(device).data_ptr(), 0, status,
+                                                 _stream(device)))
+        hit = table._plans[key] = (plan, bool(status[0]))
+    plan, taken = hit
+    p.table_plan = plan.data_ptr() if taken else None
+    p.table_plan_state = _lib.PLAN_READY if taken else _lib.PLAN_NONE
     return plan
 
 
@@ -409,7 +428,7 @@ def _raw_forward(meta: _Meta, x, y, s, sender, receiver, graph=None) -> torch.Te
         cap = row_cap_for(x.shape[0], y.shape[0]) if want < 0 else want
     lib = _lib.load()
     with torch.cuda.device(x.device):
-        plan = _table_plan(p, x.device)  # noqa: F841 (kept alive until the call is enqueued)
+        plan = _table_plan(p, table, x.device)  # noqa: F841 (kept alive until the call is enqueued)
         args = (table.device(x.device).data_ptr(), x.data_ptr(), y.data_ptr(), s.data_ptr(),
                 other.data_ptr(), row_ptr.data_ptr(), perm.data_ptr() if perm is not None else None,
                 out.data_ptr(), _stream(x.device))
@@ -498,7 +517,7 @@ def _raw_backward(meta: _Meta, x, y, s, dm, sender, receiver, graph=None):
     if group_receiver and not ordered and y.shape[0] > 0 and p.layout == _lib.LAYOUT_TRAILING and aligned:
         tile_rows = _tile_rows(p.signature)
     with torch.cuda.device(x.device):
-        plan = _table_plan(p, x.device)  # noqa: F841 (kept alive until the call is enqueued)
+        plan = _table_plan(p, table, x.device)  # noqa: F841 (kept alive until the call is enqueued)
         if tile_rows >= 1:
             if prepared is None:
                 prepared = PreparedGraph(other, row_ptr, perm, order, n)

@@ -104,7 +104,16 @@ typedef struct e3j_amd_conv_params {
      * it the call allocates nothing and the planned kernels also run on a stream that is being
      * captured into a graph; NULL: memory from the stream's pool, and none under capture. */
     int32_t *table_plan;
+    /* E3J_AMD_PLAN_BUILD (0): the call builds the plan of its table (into table_plan, or into pool
+     * memory) and launches both forms of the table-driven kernels, of which the one the plan's flag
+     * names runs.  E3J_AMD_PLAN_READY: table_plan holds the plan of this very table (same `coef`
+     * contents and column order, same sizes), built by e3j_amd_table_plan_status with table_plan set,
+     * which reported that the planned kernels take the table: nothing is built and only the planned
+     * kernel is launched; the plan is only read, so calls on any stream may share it.
+     * E3J_AMD_PLAN_NONE: the call does not plan (a table the status call reported as not taken). */
+    int32_t table_plan_state;
 } e3j_amd_conv_params;
+enum { E3J_AMD_PLAN_BUILD = 0, E3J_AMD_PLAN_READY = 1, E3J_AMD_PLAN_NONE = 2 };
 
 /* Message of the last failure on the calling thread ("" if none). */
 const char *e3j_amd_last_error(void);
@@ -266,8 +275,10 @@ void e3j_amd_set_table_plans(int32_t on);
  * backward entry points), waits for it and writes status[0] = 1 if the planned kernels take the
  * table (0: sizes beyond the limits, or an output coordinate with two scalars), status[1] = its
  * non-empty (output coordinate, x coordinate) cells, status[2] = the (16 output coordinates x 4 x
- * coordinates) blocks the loops visit, status[3] = scalars no entry uses.  Allocates and
- * synchronises: for tests and set-up code, not for the hot path. */
+ * coordinates) blocks the loops visit, status[3] = scalars no entry uses.  With p->table_plan set the
+ * plan is built in that memory and stays there: later calls with table_plan_state =
+ * E3J_AMD_PLAN_READY (if status[0] is 1) use it without building it again.  Synchronises (and
+ * allocates when p->table_plan is NULL): for tests and set-up code, not for the hot path. */
 int e3j_amd_table_plan_status(const e3j_amd_conv_params *p, const void *coef, int32_t coef_cols_ji,
                               int32_t *status, void *stream);
 /* Bytes of e3j_amd_conv_params.table_plan for the sizes in `p` (num_coef, num_scalars and the

@@ -24,8 +24,11 @@ def _params(n, e, nnz, X, Y, Z, S, K, layout, val, idx_bytes, debug=1):
 
 
 def run_abi(idx, val, mix, x, y, s, dm, snd, rcv, Z, *, leading=False, dtype=np.float32,
-            idx_dtype=None, grouping="receiver", perm=None):
-    """Forward and backward through the C ABI on receiver-sorted (or permuted) edges."""
+            idx_dtype=None, grouping="receiver", perm=None, plan=None):
+    """Forward and backward through the C ABI on receiver-sorted (or permuted) edges.
+
+    `plan`: None, the calls plan their table themselves; "ready", the plan is built once by the status
+    call and the calls are told so; "none", the calls are told not to plan."""
     lib = _lib.load()
     n, e = x.shape[0], y.shape[0]
     X, S = (x.shape[2], s.shape[2]) if leading else (x.shape[1], s.shape[1])
@@ -45,6 +48,16 @@ def run_abi(idx, val, mix, x, y, s, dm, snd, rcv, Z, *, leading=False, dtype=np.
     out = torch.full((n,) + ((K, Z) if leading else (Z, K)), float("nan"),
                      dtype=xd.dtype, device="cuda")
     stream = torch.cuda.current_stream().cuda_stream
+    if plan == "ready":
+        plan_d = torch.empty(max(int(lib.e3j_amd_table_plan_bytes(ctypes.byref(p))), 4) // 4, dtype=torch.int32,
+                             device="cuda")
+        p.table_plan = plan_d.data_ptr()
+        status = (ctypes.c_int32 * 4)()
+        _lib.check(lib.e3j_amd_table_plan_status(ctypes.byref(p), coef_d.data_ptr(), 0, status, stream))
+        assert status[0] == 1, "the planned kernels do not take this table"
+        p.table_plan_state = _lib.PLAN_READY
+    elif plan == "none":
+        p.table_plan_state = _lib.PLAN_NONE
     _lib.check(lib.e3j_amd_convolution_fwd(ctypes.byref(p), coef_d.data_ptr(), xd.data_ptr(),
                                            yd.data_ptr(), sd.data_ptr(), other.data_ptr(),
                                            ptr_d.data_ptr(),

@@ -219,6 +219,79 @@ def test_both_forms_agree_and_the_column_form_still_runs(plans_off):
         np.testing.assert_allclose(a, b, rtol=2e-5, atol=2e-5, err_msg=name)
 
 
+@pytest.mark.parametrize("grouping", ["receiver", "sender"])
+def test_a_plan_built_once_serves_later_calls(grouping):
+    """`table_plan_state`: with a plan built by the status call and declared ready, the calls launch
+    the planned kernel alone, on the same plan contents as a call that builds it: the same bits (the
+    sender-grouped backward has no atomics; for the receiver-grouped one dx is compared to rounding).
+    Told not to plan, the calls run the column kernels; an unknown state and a ready state without a
+    plan are refused before anything is launched."""
+    rng = np.random.default_rng(91)
+    N, E, X, Y, Z, S, K, nnz = 40, 700, 9, 16, 35, 11, 96, 260
+    idx, val, mix = H.random_table(rng, nnz, X, Y, Z, S)
+    snd, rcv = H.random_graph(rng, N, E)
+    x, y, s, dm = H.random_operands(rng, N, E, X, Y, S, K, Z)
+    built = run_abi(idx, val, mix, x, y, s, dm, snd, rcv, Z, grouping=grouping)
+    ready = run_abi(idx, val, mix, x, y, s, dm, snd, rcv, Z, grouping=grouping, plan="ready")
+    check_all(idx, val, mix, x, y, s, dm, snd, rcv, Z, ready, tag="ready plan")
+    for a, b, name in zip(ready, built, ("out", "dx", "dy", "ds")):
+        if name == "dx" and grouping == "receiver":
+            np.testing.assert_allclose(a, b, rtol=2e-5, atol=2e-5, err_msg=name)
+        else:
+            assert np.array_equal(a, b), name
+    columns = run_abi(idx, val, mix, x, y, s, dm, snd, rcv, Z, grouping=grouping, plan="none")
+    check_all(idx, val, mix, x, y, s, dm, snd, rcv, Z, columns, tag="not planned")
+    p = _params(N, E, nnz, X, Y, Z, S, K, 1, _lib.F32, 4)
+    lib = _lib.load()
+    some = _dev(np.zeros(4096, np.float32))
+    for state, plan_ptr, message in ((7, None, "table_plan_state"), (_lib.PLAN_READY, None, "holds none")):
+        p.table_plan_state, p.table_plan = state, plan_ptr
+        with pytest.raises(_lib.E3jAmdError, match=message):
+            _lib.check(lib.e3j_amd_convolution_fwd(ctypes.byref(p), some.data_ptr(), some.data_ptr(), some.data_ptr(),
+                                                   some.data_ptr(), some.data_ptr(), some.data_ptr(), None,
+                                                   some.data_ptr(), torch.cuda.current_stream().cuda_stream))
+
+
+def test_the_operator_plans_a_table_once(monkeypatch):
+    """The operators build the plan of a table on the first table-driven call and reuse it: later calls
+    carry the ready state (one status call per table, sizes and device), and give the first call's bits."""
+    from e3j_amd import ops
+    from e3j_amd.ops import convolution
+    w = W.config3(0.002)
+    idx, val, mix = w.table()
+    coef = H.pack_table(idx, np.asarray(val) * 1.25, mix)   # no unrolled kernel has these values
+    rng = np.random.default_rng(5)
+    N, E, K = 30, 400, 96
+    snd, rcv = H.random_graph(rng, N, E)
+    x, y, s, _ = H.random_operands(rng, N, E, 16, 16, 23, K, 99)
+    calls, states = [], []
+    lib = _lib.load()
+    real_status, real_fwd = lib.e3j_amd_table_plan_status, lib.e3j_amd_convolution_fwd
+
+    class Spy:
+        def __getattr__(self, name):
+            return getattr(lib, name)
+
+        def e3j_amd_table_plan_status(self, *a):
+            calls.append(1)
+            return real_status(*a)
+
+        def e3j_amd_convolution_fwd(self, p, *a):
+            states.append(int(p._obj.table_plan_state))
+            return real_fwd(p, *a)
+
+    monkeypatch.setattr(ops._lib, "load", lambda: Spy())
+    args = (_dev(x), _dev(y), _dev(s), _dev(snd.astype(np.int32)), _dev(rcv.astype(np.int32)), w.module.params)
+    with pytest.warns(ops.TableDrivenKernelWarning):
+        first = convolution(coef, *args)
+    second = convolution(coef, *args)
+    torch.cuda.synchronize()
+    assert len(calls) == 1 and states == [_lib.PLAN_READY, _lib.PLAN_READY]
+    assert torch.equal(first, second)
+    ref, mag = H.forward_reference(idx, np.asarray(val) * 1.25, mix, x, y, s, snd, rcv, 99)
+    H.assert_parity(first.cpu().numpy(), ref, mag, "operator on a cached plan")
+
+
 @pytest.mark.parametrize("plans", [1, 0])
 def test_float16_through_the_operator_in_both_forms(plans):
     """float16 operands with cfg3's table (7 blocks of outputs): the planned kernels hold the values
