@@ -429,10 +429,15 @@ void *backward_handler(XlaCallFrame *f, Backward mode) {
     d.p.num_coef = (int32_t)(count(coef) / numel / (stacked ? 3 : 1));
     const int32_t *perm_ptr = count(perm) ? static_cast<const int32_t *>(perm->data) : nullptr;
     if (void *err = choose_kernels(f, op, coef, stacked != 0, &d.p, d.stream)) return err;
-    if (mode == Backward::kSenderRows && d.p.signature >= 0) {
-        // The reference's operands: the adjacency grouped by sender.  The unrolled backward walks
-        // receiver rows, so the receiver CSR is rebuilt on the device in scratch memory of the
-        // runtime; without such memory the table-driven kernel keeps the sender rows.
+    // The reference's operands: the adjacency grouped by sender.  The unrolled kernels of that
+    // grouping (trailing layout; a row owns its dx) pay a gather of dm rows per edge: faster than
+    // a rebuild of the receiver rows (a dozen small launches) plus the receiver-grouped kernel on
+    // graphs below about a quarter of a million edges (150k edges, 64 channels: 0.36 against
+    // 0.44 ms), slower above (960k edges, 64 channels: 4.07 against 3.62 + 0.2 ms).  Large graphs
+    // therefore get their receiver CSR rebuilt in scratch memory of the runtime; without such
+    // memory run_backward keeps the sender rows (unrolled in the trailing layout, else table-driven).
+    const bool small_graph = d.p.layout == E3J_AMD_LAYOUT_TRAILING && d.p.num_edges < (1 << 18);
+    if (mode == Backward::kSenderRows && d.p.signature >= 0 && !small_graph) {
         bool done = false;
         void *err = backward_on_receiver_rows(f, op, &d, coef, stacked != 0, x, y, s, dm, other, row_ptr, perm_ptr,
                                               dx, dy, ds, &done);

@@ -234,18 +234,23 @@ def _time_ms(fn, reps=20):
     return start.elapsed_time(stop) / reps
 
 
-def test_reference_frames_run_the_unrolled_kernels():
+@pytest.mark.parametrize("size", ["config 2", "288k edges"])
+def test_reference_frames_run_the_unrolled_kernels(size):
     """Exactly the operands and attributes the reference sends (`src/e3j/ops/convolution.py:229-242`:
     coef, x, y, s, sender, receiver_ptr, coef_ranges + num_nodes, debug; `:433-452`: the stack of
     three transposed tables, x, y, s, dm, sender_t, receiver_ptr_t, perm, coef_ranges + num_nodes,
-    debug), at the size of config 2, with the table's rows in a permuted order as the reference's
+    debug), with the table's rows in a permuted order as the reference's
     balancing leaves them: parity against the CPU checker, and the time of the unrolled kernels
-    (within 1.3x of the direct C-ABI launches), not of the table-driven ones."""
+    (within 1.3x of the direct C-ABI launches), not of the table-driven ones.  At the size of
+    config 2 the backward frame runs the sender-grouped unrolled kernels on the operands as they are
+    (nothing borrowed from the runtime); above a quarter of a million edges it rebuilds the receiver rows
+    in scratch memory of the runtime and runs the receiver-grouped kernels."""
     from e3j_amd import workloads as W
     from e3j_amd.graph import csr_row_ptr
     from e3j_amd.ops import _Table
     from oracle import c_oracle
-    w = W.config2()
+    w = W.config2() if size == "config 2" else W.config3(0.3)
+    assert (w.num_edges < (1 << 18)) == (size == "config 2")
     m = w.module
     packed = m._packed_coef("float32")
     dims = (int(w.x.shape[1]), int(w.y.shape[1]), m.params.num_out, int(w.s.shape[1]))
@@ -282,7 +287,8 @@ def test_reference_frames_run_the_unrolled_kernels():
     assert lib.e3j_amd_xla_convolution(C.addressof(fwd)) is None, xla.errors
     assert lib.e3j_amd_xla_convolution_bwd(C.addressof(bwd)) is None, xla.errors
     torch.cuda.synchronize()
-    assert xla.allocations == 1 and not xla.scratch            # scratch borrowed once and handed back
+    # the rebuilt receiver rows: scratch borrowed once and handed back; the small graph borrows nothing
+    assert xla.allocations == (0 if size == "config 2" else 1) and not xla.scratch
 
     idx, val, mix = w.table()
     a = w.numpy()
@@ -321,7 +327,7 @@ def test_reference_frames_run_the_unrolled_kernels():
     assert t_frames[0] <= 1.3 * t_direct[0] + 0.02, (t_frames, t_direct)
     assert sum(t_frames) <= 1.3 * sum(t_direct) + 0.03, (t_frames, t_direct)
 
-    # without scratch from the runtime the backward keeps the sender rows (table-driven), same results
+    # without scratch from the runtime the backward keeps the sender rows (their unrolled kernels), same results
     xla.allocate = None
     dx2, dy2, ds2 = (torch.full_like(t, float("nan")) for t in (d.x, d.y, d.s))
     bwd2 = xla.frame(bwd_operands(bwd), [_buf(xla, dx2, F32), _buf(xla, dy2, F32), _buf(xla, ds2, F32)], attrs())
