@@ -581,7 +581,8 @@ def main():
     from e3j_amd.ops import prepare_graph
     prep_stats = {}
     def prepare():
-        g = prepare_graph(w.sender, w.receiver, w.num_nodes, module.graph_ordering)
+        # as inside an operator call: without the row pairing that handles built once get by default
+        g = prepare_graph(w.sender, w.receiver, w.num_nodes, module.graph_ordering, pair_rows=False)
         if abi.schedule is not None:
             g.schedule(abi.tile_rows)
     prep_ms = time_events(torch, prepare, args.steps, 2, prep_stats)
