@@ -19,6 +19,7 @@ OK, INVALID_ARGUMENT, UNIMPLEMENTED, INTERNAL = 0, 1, 2, 3
 LAYOUT_LEADING, LAYOUT_TRAILING = 0, 1
 F32, F64, F16 = 0, 1, 2
 PLAN_BUILD, PLAN_READY, PLAN_NONE = 0, 1, 2
+F64_CLASSES = 64
 
 
 class ConvParams(ctypes.Structure):
@@ -48,6 +49,7 @@ class ConvParams(ctypes.Structure):
         ("partials", ctypes.c_void_p),
         ("table_plan", ctypes.c_void_p),
         ("table_plan_state", ctypes.c_int32),
+        ("coef_classes", ctypes.c_void_p),
     ]
 
 
@@ -140,6 +142,8 @@ SYMBOLS = {
     "e3j_amd_convolution_bwd_tiled": (ctypes.c_int, [_PARAMS] + [_P] * 7 + [ctypes.POINTER(TileSchedule)] + [_P] * 4),
     "e3j_amd_find_signature": (ctypes.c_int, [_P] + [ctypes.c_int32] * 9 + [ctypes.POINTER(ctypes.c_float),
                                                                              ctypes.POINTER(ctypes.c_uint32)]),
+    "e3j_amd_find_signature_f64": (ctypes.c_int, [_P] + [ctypes.c_int32] * 8 + [ctypes.POINTER(ctypes.c_double),
+                                                                                 ctypes.POINTER(ctypes.c_uint32)]),
     "e3j_amd_num_signatures": (ctypes.c_int, []),
     "e3j_amd_signature_name": (ctypes.c_char_p, [ctypes.c_int]),
     "e3j_amd_csr_workspace_bytes": (ctypes.c_size_t, [ctypes.c_int32, ctypes.c_int64]),

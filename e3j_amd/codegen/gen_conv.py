@@ -61,6 +61,11 @@ LAUNCH = {
     256: dict(fwd=[(1, 4, 1), (1, 4, 2)], bwd=[(2, 4, 3), (1, 4, 2), (1, 4, 3)],
               bwd_tile=[(2, 8, 3), (1, 8, 4)]),
 }
+#: parts of the float64 kernels: (forward, backward).  A double takes the registers of two channels
+#: of a float kernel, so these are the splits the two-channel float kernels use.
+F64_SPLIT = (3, 4)
+#: the float64 kernels take one coefficient per class of equal magnitude as a kernel argument
+F64_MAX_CLASSES = 64
 #: `bwd_tile`: variants of the backward over tiles of receivers (trailing layout, at least 64
 #: channels): a block of `waves per block` waves shares the dm rows of a tile in LDS.  A fifth
 #: number is the receivers per tile the variant is tuned for (8 if absent): few enough that the
@@ -114,9 +119,23 @@ class Table:
                 raise ValueError("an output coordinate must map to one scalar")
             rows = self.paths.setdefault(int(l), OrderedDict())
             rows.setdefault(int(i), OrderedDict()).setdefault(int(j), []).append((float(v), int(k)))
+        # Classes of equal magnitude, in the order of their first entry: the float64 kernels read
+        # one value per class from a kernel argument instead of carrying the values as literals,
+        # so that they serve every table of this structure to float64 accuracy.
+        self.classes = OrderedDict()
+        for v in self.val:
+            if v != 0:
+                self.classes.setdefault(_f32_bits(abs(float(v))), len(self.classes))
+        self.class_of = [self.classes[_f32_bits(abs(float(v)))] if v != 0 else 255 for v in self.val]
 
-    @staticmethod
-    def path_products(rows):
+    def lit(self, c: float, f64: bool) -> str:
+        """Coefficient `c` in generated code: a float literal, or (float64 kernels) the value of
+        its class in the kernel's coefficient argument `cf`, under the sign of `c`."""
+        if not f64:
+            return _lit(c)
+        return ("-" if c < 0 else "") + f"cf[{self.classes[_f32_bits(abs(float(c)))]}]"
+
+    def path_products(self, rows, f64: bool = False):
         """Distinct `(|c|, k)` of one path -> local product id, and their definitions."""
         ids = OrderedDict()
         for cols in rows.values():
@@ -126,7 +145,7 @@ class Table:
         defs = []
         for (bits, k), m in ids.items():
             c = struct.unpack("<f", struct.pack("<I", bits))[0]
-            defs.append(f"            const float p{m} = {_lit(c)} * y[{k}];")
+            defs.append(f"            const {'double' if f64 else 'float'} p{m} = {self.lit(c, f64)} * y[{k}];")
         return ids, defs
 
     @staticmethod
@@ -218,12 +237,19 @@ def _mask(indices) -> str:
     return hex(sum(1 << i for i in indices if i < 64))
 
 
-def emit_edge_fwd(p: Part) -> list[str]:
-    lines = ["    template <int C>",
-             "    __device__ static __forceinline__ void edge_fwd(const Vec<C> *x, const float *y,",
-             "                                                     const Vec<C> *s, Vec<C> *acc) {"]
+def emit_edge_fwd(p: Part, f64: bool = False) -> list[str]:
+    """`f64`: the float64 form (`edge_fwd_f64`): one double per lane, coefficients from `cf`."""
+    V, R = ("Vec<1, double>", "double") if f64 else ("Vec<C>", "float")
+    if f64:
+        lines = ["    __device__ static __forceinline__ void edge_fwd_f64(const Vec<1, double> *x, const double *y,",
+                 "                                                         const Vec<1, double> *s, Vec<1, double> *acc,",
+                 "                                                         const double *cf) {"]
+    else:
+        lines = ["    template <int C>",
+                 "    __device__ static __forceinline__ void edge_fwd(const Vec<C> *x, const float *y,",
+                 "                                                     const Vec<C> *s, Vec<C> *acc) {"]
     for l, rows in p.paths.items():
-        ids, defs = Table.path_products(rows)
+        ids, defs = p.t.path_products(rows, f64)
         lines.append(f"        {{  // path {l}: rows {min(rows)}..{max(rows)}")
         lines += defs
         for i, cols in rows.items():
@@ -232,10 +258,10 @@ def emit_edge_fwd(p: Part) -> list[str]:
             for j, terms in cols.items():
                 expr, bare = Table.weight_expr(terms, ids)
                 if not bare:
-                    lines.append(f"                const float w{j} = {expr};")
+                    lines.append(f"                const {R} w{j} = {expr};")
                     expr = f"w{j}"
                 if first:
-                    lines.append(f"                Vec<C> m = vmul(x[{p.xj[j]}], {expr});")
+                    lines.append(f"                {V} m = vmul(x[{p.xj[j]}], {expr});")
                     first = False
                 else:
                     lines.append(f"                m = vfma(x[{p.xj[j]}], {expr}, m);")
@@ -246,7 +272,7 @@ def emit_edge_fwd(p: Part) -> list[str]:
     return lines
 
 
-def emit_edge_bwd(p: Part) -> list[str]:
+def emit_edge_bwd(p: Part, f64: bool = False) -> list[str]:
     """Backward of one edge for the paths of a part.
 
     Per path l (rows i, x columns j, y components k):
@@ -257,45 +283,54 @@ def emit_edge_bwd(p: Part) -> list[str]:
     One product dm_i x_j per (i, j) pair serves both ds and dy.
     """
     t = p.t
-    lines = ["    // dx (this part's x rows) and dy (all Y) are written here; ds rows go to `ds` path by path.",
-             "    // `dm`: anything indexable by the part's local output row (registers or LDS).",
-             "    // kAcc: dx holds running sums the edge's contributions are added to (else it is overwritten).",
-             "    // kPin: each row's dx sums are computed where the row is (see `pin`); for dm rows read from LDS.",
-             "    template <int C, bool kAcc = false, bool kPin = false, typename Dm, typename DsSink>",
-             "    __device__ static __forceinline__ void edge_bwd(const Vec<C> *x, const float *y,",
-             "                                                     const Vec<C> *s, const Dm &dm,",
-             "                                                     Vec<C> *dx, float *dy, const DsSink &ds) {"]
+    V, R = ("Vec<1, double>", "double") if f64 else ("Vec<C>", "float")
+    if f64:
+        lines = ["    // the float64 form of edge_bwd: one double per lane, coefficients from `cf`",
+                 "    template <bool kAcc = false, bool kPin = false, typename Dm, typename DsSink>",
+                 "    __device__ static __forceinline__ void edge_bwd_f64(const Vec<1, double> *x, const double *y,",
+                 "                                                         const Vec<1, double> *s, const Dm &dm,",
+                 "                                                         Vec<1, double> *dx, double *dy, const DsSink &ds,",
+                 "                                                         const double *cf) {"]
+    else:
+        lines = ["    // dx (this part's x rows) and dy (all Y) are written here; ds rows go to `ds` path by path.",
+                 "    // `dm`: anything indexable by the part's local output row (registers or LDS).",
+                 "    // kAcc: dx holds running sums the edge's contributions are added to (else it is overwritten).",
+                 "    // kPin: each row's dx sums are computed where the row is (see `pin`); for dm rows read from LDS.",
+                 "    template <int C, bool kAcc = false, bool kPin = false, typename Dm, typename DsSink>",
+                 "    __device__ static __forceinline__ void edge_bwd(const Vec<C> *x, const float *y,",
+                 "                                                     const Vec<C> *s, const Dm &dm,",
+                 "                                                     Vec<C> *dx, float *dy, const DsSink &ds) {"]
     dx_init, dy_init = set(), set()
     for l, rows in p.paths.items():
-        ids, defs = Table.path_products(rows)
+        ids, defs = t.path_products(rows, f64)
         ks = sorted({k for cols in rows.values() for terms in cols.values() for _, k in terms})
         lines.append(f"        {{  // path {l}: rows {min(rows)}..{max(rows)}, y components {ks[0]}..{ks[-1]}")
         lines += defs
         a_init = set()
         for k in ks:
-            lines.append(f"            Vec<C> a{k};")
+            lines.append(f"            {V} a{k};")
         for i, cols in rows.items():
             zi = p.zi[i]
             lines.append("            {")
-            lines.append(f"                const Vec<C> dmi = dm[{zi}];")
-            lines.append(f"                const Vec<C> g = vmulv(dmi, s[{p.sl[l]}]);")
+            lines.append(f"                const {V} dmi = dm[{zi}];")
+            lines.append(f"                const {V} g = vmulv(dmi, s[{p.sl[l]}]);")
             for j, terms in cols.items():
                 xj = p.xj[j]
                 expr, bare = Table.weight_expr(terms, ids)
                 if not bare:
-                    lines.append(f"                const float w{j} = {expr};")
+                    lines.append(f"                const {R} w{j} = {expr};")
                     expr = f"w{j}"
                 if j in dx_init:
                     lines.append(f"                dx[{xj}] = vfma(g, {expr}, dx[{xj}]);")
                 else:
                     lines.append(f"                dx[{xj}] = kAcc ? vfma(g, {expr}, dx[{xj}]) : vmul(g, {expr});")
                     dx_init.add(j)
-                lines.append(f"                {{ const Vec<C> pr = vmulv(dmi, x[{xj}]);")
+                lines.append(f"                {{ const {V} pr = vmulv(dmi, x[{xj}]);")
                 for c, k in terms:
                     if k in a_init:
-                        lines.append(f"                  a{k} = vfma(pr, {_lit(c)}, a{k});")
+                        lines.append(f"                  a{k} = vfma(pr, {t.lit(c, f64)}, a{k});")
                     else:
-                        lines.append(f"                  a{k} = vmul(pr, {_lit(c)});")
+                        lines.append(f"                  a{k} = vmul(pr, {t.lit(c, f64)});")
                         a_init.add(k)
                 lines.append("                }")
             lines.append("            }")
@@ -303,7 +338,7 @@ def emit_edge_bwd(p: Part) -> list[str]:
         first = True
         for k in ks:
             if first:
-                lines.append(f"            Vec<C> dsl = vmul(a{k}, y[{k}]);")
+                lines.append(f"            {V} dsl = vmul(a{k}, y[{k}]);")
                 first = False
             else:
                 lines.append(f"            dsl = vfma(a{k}, y[{k}], dsl);")
@@ -315,15 +350,16 @@ def emit_edge_bwd(p: Part) -> list[str]:
         lines.append(f"            ds.template put<{l}>(dsl);")
         lines.append("        }")
     for l in p.zero_paths:  # paths no coefficient touches get exact zeros
-        lines.append(f"        ds.template put<{l}>(vzero<C>());")
+        lines.append(f"        ds.template put<{l}>({'vzero<1, double>()' if f64 else 'vzero<C>()'});")
     for k in range(t.Y):
         if k not in dy_init:
-            lines.append(f"        dy[{k}] = 0.f;")
+            lines.append(f"        dy[{k}] = {'0.0' if f64 else '0.f'};")
     lines.append("    }")
     return lines
 
 
-def emit_part(struct_name: str, p: Part) -> list[str]:
+def emit_part(struct_name: str, p: Part, f64: bool = False) -> list[str]:
+    """`f64`: also the float64 forms of the arithmetic (for the parts the float64 kernels use)."""
     t = p.t
     out = [f"struct {struct_name} {{",
            f"    static constexpr int X = {t.X}, Y = {t.Y}, S = {t.S}, Z = {t.Z};",
@@ -335,6 +371,11 @@ def emit_part(struct_name: str, p: Part) -> list[str]:
     out += emit_edge_fwd(p)
     out.append("")
     out += emit_edge_bwd(p)
+    if f64:
+        out.append("")
+        out += emit_edge_fwd(p, f64=True)
+        out.append("")
+        out += emit_edge_bwd(p, f64=True)
     out += ["};", ""]
     return out
 
@@ -391,6 +432,7 @@ def emit_table_source(t: "Table", name: str, desc: str, channels: int, symbols, 
         "// GENERATED by e3j_amd/codegen/gen_conv.py -- do not edit.",
         f"// {desc}",
         f"#include {include}",
+        "#include " + include.replace("unrolled.h", "unrolled_f64.h"),
         "",
         "namespace e3j_amd {",
         "namespace {",
@@ -399,14 +441,17 @@ def emit_table_source(t: "Table", name: str, desc: str, channels: int, symbols, 
     if lead == "builtin":
         lead = LAUNCH_LEADING[channels] if (t.X <= 64 and t.S <= 64) else None
     tile = launch.get("bwd_tile", [])
+    # float64 kernels: trailing layout, whole waves of channels, few enough coefficient classes
+    f64 = channels % 64 == 0 and 0 < len(t.classes) <= F64_MAX_CLASSES
     splits = sorted({v[2] for v in launch["fwd"] + launch["bwd"] + tile} |
-                    ({v[1] for v in lead["fwd"] + lead["bwd"]} if lead else set()))
+                    ({v[1] for v in lead["fwd"] + lead["bwd"]} if lead else set()) |
+                    (set(F64_SPLIT) if f64 else set()))
     part_names = {}
     for zs in splits:
         names = []
         for n, part in enumerate(split_parts(t, zs)):
             sname = f"Sig_{name}_z{zs}p{n}"
-            out += emit_part(sname, part)
+            out += emit_part(sname, part, f64=f64 and zs in F64_SPLIT)
             names.append(sname)
         part_names[zs] = ", ".join(names)
     fwd_args = ["    const float *, const float *, const float *, const int32_t *, const int32_t *,",
@@ -437,6 +482,11 @@ def emit_table_source(t: "Table", name: str, desc: str, channels: int, symbols, 
     sender_minw = 2
     out += [f"template __global__ void unrolled_bwd_sender_kernel<{channels}, 4, {sender_minw}, "
             f"{part_names[sender_split]}>("] + bwd_args
+    if f64:
+        as_f64 = lambda lines: [ln.replace("float", "double").replace("unsigned);", "unsigned, F64Coefs);")  # noqa: E731
+                                for ln in lines]
+        out += [f"template __global__ void unrolled_fwd_f64_kernel<{channels}, 4, {part_names[F64_SPLIT[0]]}>("] + as_f64(fwd_args)
+        out += [f"template __global__ void unrolled_bwd_f64_kernel<{channels}, 4, {part_names[F64_SPLIT[1]]}>("] + as_f64(bwd_args)
     if lead:
         for wpb, zs in lead["fwd"]:
             out += [f"template __global__ void unrolled_fwd_leading_kernel<{channels}, {wpb}, {part_names[zs]}>("] + fwd_args
@@ -465,6 +515,21 @@ def emit_table_source(t: "Table", name: str, desc: str, channels: int, symbols, 
             f"static const float kVal[] = {{{vals}}};",
             f"static const uint8_t kIdx[] = {{{idxs}}};",
             ""]
+    if f64:
+        out += ["// class of equal magnitude of every entry (the float64 kernels read one coefficient per class)",
+                f"static const uint8_t kClass[] = {{{', '.join(str(c) for c in t.class_of)}}};",
+                "static int run_fwd_f64(const e3j_amd_conv_params &p, const double *x, const double *y, const double *s,",
+                "                       const int32_t *sender, const int32_t *row_ptr, const int32_t *perm, double *out,",
+                "                       hipStream_t stream) {",
+                f"    return launch_unrolled_fwd_f64<{channels}, 4, {part_names[F64_SPLIT[0]]}>(",
+                "        p, x, y, s, sender, row_ptr, perm, out, stream);",
+                "}",
+                "static int run_bwd_f64(const e3j_amd_conv_params &p, const double *x, const double *y, const double *s,",
+                "                       const double *dm, const int32_t *sender, const int32_t *row_ptr,",
+                "                       const int32_t *perm, double *dx, double *dy, double *ds, hipStream_t stream) {",
+                f"    return launch_unrolled_bwd_f64<{channels}, 4, {t.Y}, {t.X}, {part_names[F64_SPLIT[1]]}>(",
+                "        p, x, y, s, dm, sender, row_ptr, perm, dx, dy, ds, stream);",
+                "}", ""]
     out += ["static int run_fwd" + fwd_sig[0]] + fwd_sig[1:]
     out += [ln.replace("VARIANT", "tuning().fwd_variant.load(std::memory_order_relaxed)") for ln in switch(
         launch["fwd"], lambda v: f"launch_unrolled_fwd<{channels}, {v[0]}, {v[1]}, {(*v, 1)[3]}, {part_names[v[2]]}>("
@@ -497,6 +562,7 @@ def emit_table_source(t: "Table", name: str, desc: str, channels: int, symbols, 
             f'    "{desc}",',
             f"    {t.X}, {t.Y}, {t.Z}, {t.S}, {len(t.val)}, {channels}, E3J_AMD_LAYOUT_TRAILING, kVal, kIdx,",
             f"    &run_fwd, &run_bwd, {tiled}, &run_bwd_sender,",
+            f"    {len(t.classes)}, kClass, &run_fwd_f64, &run_bwd_f64," if f64 else "    0, nullptr, nullptr, nullptr,",
             "};", ""]
     if lead:
         out += ["static int run_fwd_leading" + fwd_sig[0]] + fwd_sig[1:]

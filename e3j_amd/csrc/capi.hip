@@ -100,11 +100,17 @@ int validate(const e3j_amd_conv_params *p, const char *op) {
                                 "the signs in the table)");
     if (p->signature >= 0) {
         const Signature &sg = signature(p->signature);
-        if (p->val_dtype != E3J_AMD_F32 || sg.num_x != p->num_x || sg.num_y != p->num_y ||
+        const bool dtype_served = p->val_dtype == E3J_AMD_F32 ||
+                                  (p->val_dtype == E3J_AMD_F64 && sg.fwd_f64 != nullptr && sg.bwd_f64 != nullptr);
+        if (!dtype_served || sg.num_x != p->num_x || sg.num_y != p->num_y ||
             sg.num_out != p->num_out || sg.num_scalars != p->num_scalars ||
             sg.channels != p->channels || sg.layout != p->layout)
             return set_error(E3J_AMD_INVALID_ARGUMENT,
-                             name + ": operand shapes do not match signature " + sg.name);
+                             name + ": operand shapes or value dtype do not match signature " + sg.name);
+        if (p->val_dtype == E3J_AMD_F64 && p->coef_classes == nullptr)
+            return set_error(E3J_AMD_INVALID_ARGUMENT,
+                             name + ": float64 operands on an unrolled kernel need coef_classes "
+                                    "(e3j_amd_find_signature_f64)");
     }
     return E3J_AMD_OK;
 }
@@ -120,7 +126,17 @@ bool aligned16(std::initializer_list<const void *> ptrs) {
     return true;
 }
 bool signature_fits(const e3j_amd_conv_params *p, std::initializer_list<const void *> ptrs) {
-    return p->signature >= 0 && aligned16(ptrs);
+    return p->signature >= 0 && p->val_dtype == E3J_AMD_F32 && aligned16(ptrs);
+}
+// float64 operands on the float64 kernels of a signature (validate() has checked that they exist);
+// rows are moved as 8-byte elements, so any float64 array is aligned enough
+bool signature_fits_f64(const e3j_amd_conv_params *p) {
+    return p->signature >= 0 && p->val_dtype == E3J_AMD_F64;
+}
+int f64_receiver_rows_only(const char *op) {
+    return set_error(E3J_AMD_UNIMPLEMENTED,
+                     std::string(op) + ": the float64 unrolled kernels serve the forward pass and the "
+                                       "receiver-grouped backward; pass signature = -1 for the table-driven kernel");
 }
 // Falling back to the table-driven kernel is only right when no sign flip was asked for.
 int flip_without_kernel(const e3j_amd_conv_params *p, const char *op) {
@@ -151,7 +167,16 @@ int run_backward(const e3j_amd_conv_params *p, bool group_is_receiver, const voi
         (p->signature < 0 && missing(coef, p->num_coef)))
         return set_error(E3J_AMD_INVALID_ARGUMENT, std::string(op) + ": null operand");
     if (p->num_nodes == 0) return E3J_AMD_OK;
-    if (group_is_receiver && signature_fits(p, {x, s, dm, dx, ds}) &&
+    if (signature_fits_f64(p)) {
+        if (!group_is_receiver) return f64_receiver_rows_only(op);
+        rc = signature(p->signature).bwd_f64(*p, static_cast<const double *>(x), static_cast<const double *>(y),
+                                             static_cast<const double *>(s), static_cast<const double *>(dm),
+                                             other, row_ptr, edge_perm, static_cast<double *>(dx),
+                                             static_cast<double *>(dy), static_cast<double *>(ds), stream);
+        if (rc == E3J_AMD_OK)
+            rc = launch_zero_padding(*p, other, row_ptr, edge_perm, static_cast<double *>(dy),
+                                     static_cast<double *>(ds), stream);
+    } else if (group_is_receiver && signature_fits(p, {x, s, dm, dx, ds}) &&
         signature(p->signature).bwd != nullptr) {
         rc = signature(p->signature).bwd(*p, static_cast<const float *>(x),
                                          static_cast<const float *>(y), static_cast<const float *>(s),
@@ -308,6 +333,15 @@ int e3j_amd_convolution_fwd(const e3j_amd_conv_params *p, const void *coef, cons
         missing(sender, p->num_edges) || missing(y, p->num_edges) || missing(s, p->num_edges) ||
         (p->signature < 0 && missing(coef, p->num_coef)))
         return set_error(E3J_AMD_INVALID_ARGUMENT, "convolution: null operand");
+    if (signature_fits_f64(p)) {
+        if (p->row_cap != 0 || p->segments != nullptr)
+            return set_error(E3J_AMD_UNIMPLEMENTED, "convolution: row_cap / segments are taken by the float32 "
+                                                    "unrolled kernels only");
+        rc = signature(p->signature).fwd_f64(*p, static_cast<const double *>(x), static_cast<const double *>(y),
+                                             static_cast<const double *>(s), sender, receiver_ptr, edge_perm,
+                                             static_cast<double *>(out), stream);
+        return finish(p, stream, rc, "convolution");
+    }
     const bool split_rows = p->row_cap > 0 || p->segments != nullptr;
     if (p->row_cap < 0 || p->max_segments < 0 || p->row_piece < 0 || p->row_piece > p->row_cap)
         return set_error(E3J_AMD_INVALID_ARGUMENT, "convolution: row_cap / row_piece / max_segments");
@@ -490,9 +524,9 @@ int e3j_amd_convolution_bwd_tiled(const e3j_amd_conv_params *p, const void *x, c
         schedule == nullptr)
         return set_error(E3J_AMD_INVALID_ARGUMENT, std::string(op) + ": null operand");
     if (p->num_nodes == 0) return E3J_AMD_OK;
-    if (p->signature < 0 || signature(p->signature).bwd_tiled == nullptr)
+    if (p->signature < 0 || p->val_dtype != E3J_AMD_F32 || signature(p->signature).bwd_tiled == nullptr)
         return set_error(E3J_AMD_UNIMPLEMENTED,
-                         std::string(op) + ": needs a compile-time-unrolled kernel of the trailing layout "
+                         std::string(op) + ": needs a float32 compile-time-unrolled kernel of the trailing layout "
                                            "with at least 64 channels; e3j_amd_convolution_bwd_receiver "
                                            "serves the other cases");
     if (!aligned16({x, s, dm, dx, ds}))
@@ -521,6 +555,86 @@ int e3j_amd_find_signature(const void *coef_host, int32_t coef_idx_bytes, int32_
     if (coef_idx_bytes != 1 && coef_idx_bytes != 4) return -1;
     const std::vector<TableEntry> entries = unpack_entries(coef_host, coef_idx_bytes, num_coef, false);
     return match_signature(entries, num_x, num_y, num_out, num_scalars, channels, layout, coef_scale, y_flip);
+}
+
+int e3j_amd_find_signature_f64(const void *coef_host, int32_t coef_idx_bytes, int32_t num_coef,
+                               int32_t num_x, int32_t num_y, int32_t num_out, int32_t num_scalars,
+                               int32_t channels, int32_t layout, double *coef_classes, uint32_t *y_flip) {
+    if (y_flip) *y_flip = 0;
+    if (coef_host == nullptr || coef_classes == nullptr || num_coef <= 0) return -1;
+    if (coef_idx_bytes != 1 && coef_idx_bytes != 4) return -1;
+    struct Entry {
+        double val;
+        int32_t idx[4];
+        int32_t cls;
+    };
+    auto less = [](const Entry &a, const Entry &b) {
+        for (int t = 0; t < 4; t++)
+            if (a.idx[t] != b.idx[t]) return a.idx[t] < b.idx[t];
+        return false;
+    };
+    const size_t item = coef_idx_bytes == 1 ? sizeof(Coef4D<uint8_t, double>) : sizeof(Coef4D<int32_t, double>);
+    const unsigned char *bytes = static_cast<const unsigned char *>(coef_host);
+    std::vector<Entry> given((size_t)num_coef), own((size_t)num_coef);
+    for (int n = 0; n < num_coef; n++) {
+        std::memcpy(&given[n].val, bytes + n * item, sizeof(double));
+        for (int t = 0; t < 4; t++) {
+            if (coef_idx_bytes == 1) given[n].idx[t] = bytes[n * item + 8 + t];
+            else std::memcpy(&given[n].idx[t], bytes + n * item + 8 + 4 * t, 4);
+        }
+    }
+    std::stable_sort(given.begin(), given.end(), less);
+    const bool signs_allowed = y_flip != nullptr && num_y <= 32;
+    for (int id = 0; id < num_signatures(); id++) {
+        const Signature &sg = signature(id);
+        if (sg.fwd_f64 == nullptr || sg.bwd_f64 == nullptr || sg.coef_class == nullptr ||
+            sg.num_classes < 1 || sg.num_classes > kF64Classes)
+            continue;
+        if (sg.num_coef != num_coef || sg.num_x != num_x || sg.num_y != num_y || sg.num_out != num_out ||
+            sg.num_scalars != num_scalars || sg.channels != channels || sg.layout != layout)
+            continue;
+        for (int n = 0; n < num_coef; n++) {
+            own[n].val = sg.val[n];
+            own[n].cls = sg.coef_class[n];
+            for (int t = 0; t < 4; t++) own[n].idx[t] = sg.idx[4 * n + t];
+        }
+        std::stable_sort(own.begin(), own.end(), less);
+        // Same coordinates; the sign of every entry equal to the built-in one, or opposite for all
+        // entries of a y component; one magnitude per class of the built-in table.
+        double mags[kF64Classes];
+        bool have[kF64Classes] = {false};
+        uint32_t flip = 0, seen = 0;
+        bool same = true;
+        for (int n = 0; n < num_coef && same; n++) {
+            for (int t = 0; t < 4 && same; t++) same = given[n].idx[t] == own[n].idx[t];
+            if (!same) break;
+            const double v = given[n].val;
+            if (own[n].val == 0.0f || own[n].cls >= sg.num_classes) {  // (no built-in table holds zeros)
+                same = v == 0.0;
+                continue;
+            }
+            if (v == 0.0 || !std::isfinite(v)) { same = false; break; }
+            const int m = own[n].cls;
+            const double mag = std::fabs(v);
+            if (!have[m]) { mags[m] = mag; have[m] = true; }
+            else same = std::fabs(mag - mags[m]) <= 1e-13 * mags[m];
+            const bool opposite = (v < 0.0) != (own[n].val < 0.0f);
+            const int k = given[n].idx[2];
+            if (!signs_allowed) {
+                same = same && !opposite;
+            } else if ((seen >> k) & 1u) {
+                same = same && (((flip >> k) & 1u) != 0) == opposite;
+            } else {
+                seen |= 1u << k;
+                if (opposite) flip |= 1u << k;
+            }
+        }
+        if (!same) continue;
+        for (int m = 0; m < kF64Classes; m++) coef_classes[m] = m < sg.num_classes && have[m] ? mags[m] : 0.0;
+        if (y_flip) *y_flip = flip;
+        return id;
+    }
+    return -1;
 }
 
 }  // extern "C"

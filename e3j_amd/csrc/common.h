@@ -108,6 +108,8 @@ std::atomic<int> &table_plans();  // 1: plan the tables that can be planned (def
 // Zero the dy/ds rows of padding edges (float32 operands).
 int launch_zero_padding(const e3j_amd_conv_params &p, const int32_t *other, const int32_t *row_ptr,
                         const int32_t *perm, float *dy, float *ds, hipStream_t stream);
+int launch_zero_padding(const e3j_amd_conv_params &p, const int32_t *other, const int32_t *row_ptr,
+                        const int32_t *perm, double *dy, double *ds, hipStream_t stream);
 
 // Launch-shape variants of the unrolled kernels, from E3J_AMD_FWD_VARIANT /
 // E3J_AMD_BWD_VARIANT (read once; 0 = default).  For tuning runs.
@@ -176,6 +178,22 @@ struct Signature {
     int (*bwd_sender)(const e3j_amd_conv_params &p, const float *x, const float *y, const float *s,
                       const float *dm, const int32_t *receiver_t, const int32_t *sender_ptr,
                       const int32_t *edge_perm, float *dx, float *dy, float *ds, hipStream_t stream);
+    // float64 kernels (trailing layout, receiver rows; nullptr: none).  They read one coefficient
+    // per class of entries of equal magnitude from e3j_amd_conv_params.coef_classes: coef_class
+    // (num_coef) names the class of every entry, num_classes <= kF64Classes.
+    int32_t num_classes;
+    const uint8_t *coef_class;
+    int (*fwd_f64)(const e3j_amd_conv_params &p, const double *x, const double *y, const double *s,
+                   const int32_t *sender, const int32_t *receiver_ptr, const int32_t *edge_perm, double *out,
+                   hipStream_t stream);
+    int (*bwd_f64)(const e3j_amd_conv_params &p, const double *x, const double *y, const double *s,
+                   const double *dm, const int32_t *sender, const int32_t *receiver_ptr,
+                   const int32_t *edge_perm, double *dx, double *dy, double *ds, hipStream_t stream);
+};
+// the coefficient classes of a float64 launch, passed to the kernel by value
+constexpr int kF64Classes = E3J_AMD_F64_CLASSES;
+struct F64Coefs {
+    double v[kF64Classes];
 };
 // built-in signatures (generated/registry.hip), then the ones registered at run time (capi.hip)
 // A table entry on the host, and the lookup of a table among the signatures (capi.hip): the

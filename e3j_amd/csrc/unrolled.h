@@ -28,72 +28,83 @@
 
 namespace e3j_amd {
 
-template <int C>
+// C values of scalar type T per lane (T = double: the float64 kernels of unrolled_f64.h, which
+// share the generated arithmetic).
+template <int C, typename T = float>
 struct Vec {
-    float v[C];
+    T v[C];
 };
+// (keeps a scalar argument out of template deduction: the vector operand fixes T)
+template <typename T>
+struct SameAs {
+    using type = T;
+};
+template <typename T>
+using same_t = typename SameAs<T>::type;
+__device__ __forceinline__ float fma_t(float a, float b, float c) { return fmaf(a, b, c); }
+__device__ __forceinline__ double fma_t(double a, double b, double c) { return fma(a, b, c); }
 
-template <int C>
-__device__ __forceinline__ Vec<C> vzero() {
-    Vec<C> r;
+template <int C, typename T = float>
+__device__ __forceinline__ Vec<C, T> vzero() {
+    Vec<C, T> r;
 #pragma unroll
-    for (int t = 0; t < C; t++) r.v[t] = 0.f;
+    for (int t = 0; t < C; t++) r.v[t] = T(0);
     return r;
 }
 // Fixes the point in the instruction stream where `a` is computed: the value is an operand of
 // an (empty) statement the compiler keeps in program order.  Without it the instruction
 // selector emits a sum at its last use, and the operands of every term stay in registers
 // until then.
-template <int C>
-__device__ __forceinline__ void pin(Vec<C> &a) {
+template <int C, typename T>
+__device__ __forceinline__ void pin(Vec<C, T> &a) {
 #pragma unroll
     for (int t = 0; t < C; t++) asm volatile("" : "+v"(a.v[t]));
 }
-template <int C>
-__device__ __forceinline__ Vec<C> vmul(const Vec<C> &a, float w) {
-    Vec<C> r;
+template <int C, typename T>
+__device__ __forceinline__ Vec<C, T> vmul(const Vec<C, T> &a, same_t<T> w) {
+    Vec<C, T> r;
 #pragma unroll
     for (int t = 0; t < C; t++) r.v[t] = a.v[t] * w;
     return r;
 }
-template <int C>
-__device__ __forceinline__ Vec<C> vfma(const Vec<C> &a, float w, const Vec<C> &c) {
-    Vec<C> r;
+template <int C, typename T>
+__device__ __forceinline__ Vec<C, T> vfma(const Vec<C, T> &a, same_t<T> w, const Vec<C, T> &c) {
+    Vec<C, T> r;
 #pragma unroll
-    for (int t = 0; t < C; t++) r.v[t] = fmaf(a.v[t], w, c.v[t]);
+    for (int t = 0; t < C; t++) r.v[t] = fma_t(a.v[t], w, c.v[t]);
     return r;
 }
-template <int C>
-__device__ __forceinline__ Vec<C> vmulv(const Vec<C> &a, const Vec<C> &b) {
-    Vec<C> r;
+template <int C, typename T>
+__device__ __forceinline__ Vec<C, T> vmulv(const Vec<C, T> &a, const Vec<C, T> &b) {
+    Vec<C, T> r;
 #pragma unroll
     for (int t = 0; t < C; t++) r.v[t] = a.v[t] * b.v[t];
     return r;
 }
-template <int C>
-__device__ __forceinline__ Vec<C> vfmav(const Vec<C> &a, const Vec<C> &b, const Vec<C> &c) {
-    Vec<C> r;
+template <int C, typename T>
+__device__ __forceinline__ Vec<C, T> vfmav(const Vec<C, T> &a, const Vec<C, T> &b, const Vec<C, T> &c) {
+    Vec<C, T> r;
 #pragma unroll
-    for (int t = 0; t < C; t++) r.v[t] = fmaf(a.v[t], b.v[t], c.v[t]);
+    for (int t = 0; t < C; t++) r.v[t] = fma_t(a.v[t], b.v[t], c.v[t]);
     return r;
 }
 // sum over the channels of a lane of a * b (+ c): one fused multiply-add per channel
-template <int C>
-__device__ __forceinline__ float vdot(const Vec<C> &a, const Vec<C> &b, float c) {
+template <int C, typename T>
+__device__ __forceinline__ T vdot(const Vec<C, T> &a, const Vec<C, T> &b, same_t<T> c) {
 #pragma unroll
-    for (int t = 0; t < C; t++) c = fmaf(a.v[t], b.v[t], c);
+    for (int t = 0; t < C; t++) c = fma_t(a.v[t], b.v[t], c);
     return c;
 }
-template <int C>
-__device__ __forceinline__ float vdot(const Vec<C> &a, const Vec<C> &b) {
-    float c = a.v[0] * b.v[0];
+template <int C, typename T>
+__device__ __forceinline__ T vdot(const Vec<C, T> &a, const Vec<C, T> &b) {
+    T c = a.v[0] * b.v[0];
 #pragma unroll
-    for (int t = 1; t < C; t++) c = fmaf(a.v[t], b.v[t], c);
+    for (int t = 1; t < C; t++) c = fma_t(a.v[t], b.v[t], c);
     return c;
 }
-template <int C>
-__device__ __forceinline__ float hsum(const Vec<C> &a) {
-    float r = a.v[0];
+template <int C, typename T>
+__device__ __forceinline__ T hsum(const Vec<C, T> &a) {
+    T r = a.v[0];
 #pragma unroll
     for (int t = 1; t < C; t++) r += a.v[t];
     return r;
@@ -242,7 +253,27 @@ __device__ __forceinline__ float to_vgpr(float v) {
 // mask (never a register-array select, which the compiler would lower to a chain of
 // compares), and two cross-row exchanges finish the sum.  On return every lane holds
 // in v[0] the total of value `slot(lane)`.
-template <int NV, int LANES = kWave>
+template <int CTRL>
+__device__ __forceinline__ float dpp_move(float v) {
+    return __int_as_float(__builtin_amdgcn_mov_dpp(__float_as_int(v), CTRL, 0xf, 0xf, true));
+}
+template <int CTRL>
+__device__ __forceinline__ double dpp_move(double v) {  // the two halves travel alike
+    const int lo = __builtin_amdgcn_mov_dpp(__double2loint(v), CTRL, 0xf, 0xf, true);
+    const int hi = __builtin_amdgcn_mov_dpp(__double2hiint(v), CTRL, 0xf, 0xf, true);
+    return __hiloint2double(hi, lo);
+}
+// (a where mask is all ones, b where it is zero)
+__device__ __forceinline__ float pick_bits(float a, float b, unsigned mask) {
+    return __uint_as_float((__float_as_uint(a) & mask) | (__float_as_uint(b) & ~mask));
+}
+__device__ __forceinline__ double pick_bits(double a, double b, unsigned mask) {
+    const unsigned long long m = (unsigned long long)(long long)(int)mask;
+    return __longlong_as_double((long long)(((unsigned long long)__double_as_longlong(a) & m) |
+                                            ((unsigned long long)__double_as_longlong(b) & ~m)));
+}
+
+template <int NV, int LANES = kWave, typename T = float>
 struct WaveReduce {
     static_assert(NV >= 1 && NV <= 16, "at most 16 values");
     static_assert(LANES == 16 || LANES == 32 || LANES == 64, "sums run over groups of 16, 32 or 64 lanes");
@@ -250,24 +281,16 @@ struct WaveReduce {
     __device__ static __forceinline__ int slot(int lane) {
         return ((lane & 1) << 3) | ((lane & 2) << 1) | ((lane & 4) >> 1) | ((lane & 8) >> 3);
     }
-    template <int CTRL>
-    __device__ static __forceinline__ float dpp(float v) {
-        return __int_as_float(__builtin_amdgcn_mov_dpp(__float_as_int(v), CTRL, 0xf, 0xf, true));
-    }
-    // (a where mask is all ones, b where it is zero)
-    __device__ static __forceinline__ float pick(float a, float b, unsigned mask) {
-        return __uint_as_float((__float_as_uint(a) & mask) | (__float_as_uint(b) & ~mask));
-    }
     template <int CTRL, int N>
-    __device__ static __forceinline__ void level(float (&v)[P], unsigned upper) {
+    __device__ static __forceinline__ void level(T (&v)[P], unsigned upper) {
 #pragma unroll
         for (int t = 0; t < N / 2; t++) {
-            const float keep = pick(v[t + N / 2], v[t], upper);
-            const float send = pick(v[t], v[t + N / 2], upper);
-            v[t] = keep + dpp<CTRL>(send);
+            const T keep = pick_bits(v[t + N / 2], v[t], upper);
+            const T send = pick_bits(v[t], v[t + N / 2], upper);
+            v[t] = keep + dpp_move<CTRL>(send);
         }
     }
-    __device__ static __forceinline__ float run(float (&v)[P], int lane) {
+    __device__ static __forceinline__ T run(T (&v)[P], int lane) {
         level<0xB1, 16>(v, (lane & 1) ? ~0u : 0u);   // quad_perm [1,0,3,2]
         level<0x4E, 8>(v, (lane & 2) ? ~0u : 0u);    // quad_perm [2,3,0,1]
         level<0x124, 4>(v, (lane & 4) ? ~0u : 0u);   // row_ror:4 (the source lane differs in bit 2)
@@ -281,18 +304,18 @@ struct WaveReduce {
 // Any number of values: sixteen at a time.  `sink(k, total)` is called on the first 16 lanes of
 // every group of LANES lanes for the values k they hold (k < NV); `v` must be padded to a
 // multiple of 16.
-template <int NV, int LANES = kWave>
+template <int NV, int LANES = kWave, typename T = float>
 struct WaveReduceBlocks {
     static constexpr int P = (NV + 15) / 16 * 16;
     template <typename Sink>
-    __device__ static __forceinline__ void run(float (&v)[P], int lane, const Sink &sink) {
-        using Red = WaveReduce<16, LANES>;
+    __device__ static __forceinline__ void run(T (&v)[P], int lane, const Sink &sink) {
+        using Red = WaveReduce<16, LANES, T>;
 #pragma unroll
         for (int base = 0; base < P; base += 16) {
-            float part[16];
+            T part[16];
 #pragma unroll
             for (int t = 0; t < 16; t++) part[t] = v[base + t];
-            const float total = Red::run(part, lane);
+            const T total = Red::run(part, lane);
             const int k = base + Red::slot(lane);
             if (lane % LANES < 16 && k < NV) sink(k, total);
         }

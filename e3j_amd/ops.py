@@ -125,7 +125,9 @@ class _Table:
         """`(id, scale, y_flip)` of a built-in unrolled kernel, `(-1, 1.0, 0)` if none matches.
 
         `y_flip`: bit mask of the y components whose coefficients carry the opposite sign of
-        the built-in table (the parity signs of the SENDER ordering).
+        the built-in table (the parity signs of the SENDER ordering).  For a float64 table `scale`
+        is not a number but the array of coefficient classes the float64 kernels read
+        (`e3j_amd_conv_params.coef_classes`, kept alive by this table).
         """
         jit = config().jit
         key = (dims, channels, layout, jit)
@@ -134,7 +136,13 @@ class _Table:
             scale, flip = ctypes.c_float(1.0), ctypes.c_uint32(0)
             val_code = _lib.F32 if self.val_np_dtype == np.float32 else _lib.F64
 
+            classes = (ctypes.c_double * _lib.F64_CLASSES)()
+
             def find():
+                if self.val_np_dtype == np.float64:
+                    return int(_lib.load().e3j_amd_find_signature_f64(
+                        self.packed.ctypes.data, self.idx_bytes, self.num_coef, dims[0], dims[1], dims[2],
+                        dims[3], channels, layout.value, classes, ctypes.byref(flip)))
                 return int(_lib.load().e3j_amd_find_signature(
                     self.packed.ctypes.data, self.idx_bytes, val_code, self.num_coef, dims[0], dims[1],
                     dims[2], dims[3], channels, layout.value, ctypes.byref(scale), ctypes.byref(flip)))
@@ -153,7 +161,8 @@ class _Table:
                     "table-driven kernels serve it, an order of magnitude slower; config(jit=True) "
                     "(or E3J_AMD_JIT=1) compiles unrolled kernels for it with hipcc on first use",
                     TableDrivenKernelWarning, stacklevel=3)
-            hit = self._signature[key] = (sig, float(scale.value), int(flip.value))
+            hit = self._signature[key] = (sig, classes if self.val_np_dtype == np.float64 else float(scale.value),
+                                          int(flip.value))
         return hit
 
 
@@ -196,8 +205,10 @@ def _fill_params(meta: _Meta, x: torch.Tensor, y: torch.Tensor, s: torch.Tensor,
         num_nodes=int(x.shape[0]), num_edges=int(y.shape[0]), num_coef=table.num_coef,
         num_x=dims[0], num_y=dims[1], num_out=dims[2], num_scalars=dims[3], channels=int(channels),
         layout=layout.value, val_dtype=val_code, coef_idx_bytes=table.idx_bytes,
-        signature=sig, coef_scale=scale, debug=int(cfg.debug_level), y_flip=flip,
-        row_order=row_order.data_ptr() if row_order is not None else None)
+        signature=sig, coef_scale=scale if isinstance(scale, float) else 1.0, debug=int(cfg.debug_level),
+        y_flip=flip, row_order=row_order.data_ptr() if row_order is not None else None)
+    if sig >= 0 and not isinstance(scale, float):   # float64: the classes of the table (host memory of the table)
+        p.coef_classes = ctypes.cast(scale, ctypes.c_void_p).value
     return p, table
 
 
@@ -420,7 +431,7 @@ def _raw_forward(meta: _Meta, x, y, s, sender, receiver, graph=None) -> torch.Te
     # result is the same bits in every run, as for a row that one wave sums
     cap = 0
     fixed_order = bool(config().fixed_order_rows)
-    if (p.signature >= 0 and meta.layout == Layout.TRAILING_CHANNELS
+    if (p.signature >= 0 and meta.layout == Layout.TRAILING_CHANNELS and x.dtype == torch.float32
             and (fixed_order or not config().deterministic)
             and isinstance(graph, PreparedGraph) and y.shape[0] > 0
             and all(t.data_ptr() % 16 == 0 for t in (x, s, out))):
@@ -456,6 +467,8 @@ def _raw_backward(meta: _Meta, x, y, s, dm, sender, receiver, graph=None):
     deterministic = config().deterministic or x.dtype == torch.float16
     table = meta.table
     has_kernel = table.signature(*_shape(meta, x, y, s), meta.layout)[0] >= 0
+    if x.dtype == torch.float64 and deterministic:
+        has_kernel = False   # the float64 unrolled backward adds dx with atomics; rows that own dx: table-driven
     # SENDER ordering: the cotangents belong to the edges as given (dy[e], ds[e] come from
     # dm[receiver(e)]), not to the reversed edges the forward walks
     # (`src/e3j/ops/convolution.py:413-431`).  With an unrolled kernel for the table the edges
@@ -514,7 +527,8 @@ def _raw_backward(meta: _Meta, x, y, s, dm, sender, receiver, graph=None):
     # tiles of receivers whose dm rows fit the LDS of a workgroup: dx summed per (tile, sender)
     tile_rows = 0
     aligned = all(t.data_ptr() % 16 == 0 for t in (x, y, s, dm, dx, dy, ds))  # what the unrolled kernels take
-    if group_receiver and not ordered and y.shape[0] > 0 and p.layout == _lib.LAYOUT_TRAILING and aligned:
+    if (group_receiver and not ordered and y.shape[0] > 0 and p.layout == _lib.LAYOUT_TRAILING and aligned
+            and x.dtype == torch.float32):
         tile_rows = _tile_rows(p.signature)
     with torch.cuda.device(x.device):
         plan = _table_plan(p, table, x.device)  # noqa: F841 (kept alive until the call is enqueued)

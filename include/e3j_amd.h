@@ -112,8 +112,17 @@ typedef struct e3j_amd_conv_params {
      * kernel is launched; the plan is only read, so calls on any stream may share it.
      * E3J_AMD_PLAN_NONE: the call does not plan (a table the status call reported as not taken). */
     int32_t table_plan_state;
+    /* float64 operands on the unrolled kernels (signature >= 0, val_dtype = E3J_AMD_F64; trailing
+     * layout, receiver-grouped calls): HOST pointer to the E3J_AMD_F64_CLASSES doubles that
+     * e3j_amd_find_signature_f64 returned for the table.  The float64 kernels do not carry the
+     * table's values as literals with one scale factor (exact to float32 rounding only): they read
+     * one value per class of entries of equal magnitude from this array, which is copied into the
+     * launch, so a table of the signature's structure is served to float64 accuracy whatever its
+     * values.  coef_scale is not used then. */
+    const double *coef_classes;
 } e3j_amd_conv_params;
 enum { E3J_AMD_PLAN_BUILD = 0, E3J_AMD_PLAN_READY = 1, E3J_AMD_PLAN_NONE = 2 };
+enum { E3J_AMD_F64_CLASSES = 64 };
 
 /* Message of the last failure on the calling thread ("" if none). */
 const char *e3j_amd_last_error(void);
@@ -252,6 +261,18 @@ int e3j_amd_find_signature(const void *coef_host, int32_t coef_idx_bytes, int32_
                            int32_t num_scalars, int32_t channels, int32_t layout,
                            float *coef_scale,
                            uint32_t *y_flip);
+
+/* The same look-up for a float64 table (host memory, packed with double values), for float64
+ * operands on the unrolled kernels.  The table must have the entries of a built-in (or registered)
+ * table whose float64 kernels are built: the same coordinates, the same signs up to one sign per y
+ * component (*y_flip), and equal magnitudes (to 1e-13) wherever the built-in table has equal
+ * magnitudes.  The magnitudes themselves are free: coef_classes (E3J_AMD_F64_CLASSES doubles, host)
+ * receives one per class, for e3j_amd_conv_params.coef_classes.  Returns the id or -1.  No
+ * counterpart in the reference, whose kernel reads the table at run time for every dtype
+ * (tests/test_ops/test_dtype.py:56-71). */
+int e3j_amd_find_signature_f64(const void *coef_host, int32_t coef_idx_bytes, int32_t num_coef,
+                               int32_t num_x, int32_t num_y, int32_t num_out, int32_t num_scalars,
+                               int32_t channels, int32_t layout, double *coef_classes, uint32_t *y_flip);
 
 /* The table-driven kernels (calls with signature < 0, and calls whose operands an unrolled kernel
  * cannot take) come in two forms.  For a float32 or float16 table (float16: values held as half,

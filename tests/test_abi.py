@@ -33,10 +33,11 @@ def test_every_declared_symbol_is_exported():
 def test_params_struct_matches_header():
     header = open(os.path.join(ROOT, "include", "e3j_amd.h")).read()
     body = re.search(r"typedef struct e3j_amd_conv_params \{(.*?)\} e3j_amd_conv_params;", header, re.S).group(1)
-    fields = re.findall(r"^\s*(const int32_t \*|float \*|int32_t \*|uint32_t|int32_t|int64_t|float)\s*(\w+);", body, re.M)
+    fields = re.findall(r"^\s*(const int32_t \*|const double \*|float \*|int32_t \*|uint32_t|int32_t|int64_t|float)\s*(\w+);",
+                        body, re.M)
     assert [name for _, name in fields] == [name for name, _ in _lib.ConvParams._fields_]
     ctype = {"int32_t": C.c_int32, "uint32_t": C.c_uint32, "int64_t": C.c_int64, "float": C.c_float, "const int32_t *": C.c_void_p,
-             "float *": C.c_void_p, "int32_t *": C.c_void_p}
+             "float *": C.c_void_p, "int32_t *": C.c_void_p, "const double *": C.c_void_p}
     assert [ctype[t] for t, _ in fields] == [t for _, t in _lib.ConvParams._fields_]
 
 
