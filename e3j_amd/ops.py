@@ -148,7 +148,7 @@ class _Table:
                     dims[2], dims[3], channels, layout.value, ctypes.byref(scale), ctypes.byref(flip)))
 
             sig = find()
-            if sig < 0 and jit and self.val_np_dtype == np.float32 and self.num_coef > 0:
+            if sig < 0 and jit and self.val_np_dtype in (np.float32, np.float64) and self.num_coef > 0:
                 # not built in: generate and compile the kernels of this table, then look again
                 from . import jit as _jit
                 c = self.unpack()

@@ -364,3 +364,42 @@ def test_edge_features_and_regroup_validate_before_launching():
     assert lib.e3j_amd_rows_regroup(None, None, 3, 4, 8, None, None, 0, 0, None) == _lib.INVALID_ARGUMENT
     assert lib.e3j_amd_rows_regroup(None, None, 0, 4, 8, None, None, 0, 0, None) == _lib.OK
     assert lib.e3j_amd_rows_regroup(None, None, -1, 4, 8, None, None, 0, 0, None) == _lib.INVALID_ARGUMENT
+
+
+def test_float64_look_up_refuses_tables_of_another_structure():
+    """One magnitude per class: a table in which two entries of one class differ, or with a sign
+    that is not a sign of a whole y component, is not the built-in structure."""
+    from e3j_amd.convolution import Convolution
+    from tests import helpers as H
+    lib = _lib.load()
+    m = Convolution(("0e+1o+2e", "0e+1o+2e+3o"), "0e+1o+2e", graph_ordering="RECEIVER", avg_num_neighbors=3.0)
+    c = m.coef
+    idx4 = np.asarray(c.idx, dtype=np.int64)
+    val = np.asarray(c.val, dtype=np.float64)
+    dims = (m.source[0].dim, m.source[1].dim, m.target.dim, m.params.num_scalars)
+
+    def find(values):
+        packed = H.pack_table(idx4[:, :3], values, m._mix.mix_indices, val_dtype=np.float64)
+        classes = (C.c_double * _lib.F64_CLASSES)()
+        flip = C.c_uint32()
+        return lib.e3j_amd_find_signature_f64(packed.ctypes.data, 1, len(values), *dims, 64, 1, classes,
+                                              C.byref(flip)), list(classes), flip.value
+
+    sig, classes, flip = find(val)
+    assert sig >= 0 and flip == 0
+    assert sorted(set(np.round(np.abs(val), 15))) == sorted(set(np.round([v for v in classes if v > 0], 15)))
+    mags = np.abs(val)
+    twin = np.flatnonzero(mags == mags[0])
+    assert len(twin) > 1
+    one_off = val.copy()
+    one_off[twin[1]] *= 1.0 + 1e-9
+    assert find(one_off)[0] == -1
+    one_sign = val.copy()
+    k0 = idx4[0, 2]
+    members = np.flatnonzero(idx4[:, 2] == k0)
+    assert len(members) > 1
+    one_sign[members[0]] *= -1.0
+    assert find(one_sign)[0] == -1
+    whole_component = val.copy()
+    whole_component[members] *= -1.0
+    assert find(whole_component)[2] == 1 << int(k0)

@@ -175,43 +175,6 @@ def test_float64_through_the_c_abi_with_padding_permutation_and_sign_mask():
             other.data_ptr(), ptr.data_ptr(), perm_d.data_ptr(), xd.data_ptr(), yd.data_ptr(), sd.data_ptr(), stream))
 
 
-def test_float64_look_up_refuses_tables_of_another_structure():
-    """One magnitude per class: a table in which two entries of one class differ, or with a sign
-    that is not a sign of a whole y component, is not the built-in structure."""
-    lib = _lib.load()
-    m = Convolution(("0e+1o+2e", "0e+1o+2e+3o"), "0e+1o+2e", graph_ordering="RECEIVER", avg_num_neighbors=3.0)
-    c = m.coef
-    idx4 = np.asarray(c.idx, dtype=np.int64)
-    val = np.asarray(c.val, dtype=np.float64)
-    dims = (m.source[0].dim, m.source[1].dim, m.target.dim, m.params.num_scalars)
-
-    def find(values):
-        packed = H.pack_table(idx4[:, :3], values, m._mix.mix_indices, val_dtype=np.float64)
-        classes = (ctypes.c_double * _lib.F64_CLASSES)()
-        flip = ctypes.c_uint32()
-        return lib.e3j_amd_find_signature_f64(packed.ctypes.data, 1, len(values), *dims, 64, 1, classes,
-                                              ctypes.byref(flip)), list(classes), flip.value
-
-    sig, classes, flip = find(val)
-    assert sig >= 0 and flip == 0
-    assert sorted(set(np.round(np.abs(val), 15))) == sorted(set(np.round([v for v in classes if v > 0], 15)))
-    mags = np.abs(val)
-    twin = np.flatnonzero(mags == mags[0])
-    assert len(twin) > 1
-    one_off = val.copy()
-    one_off[twin[1]] *= 1.0 + 1e-9
-    assert find(one_off)[0] == -1
-    one_sign = val.copy()
-    k0 = idx4[0, 2]
-    members = np.flatnonzero(idx4[:, 2] == k0)
-    assert len(members) > 1
-    one_sign[members[0]] *= -1.0
-    assert find(one_sign)[0] == -1
-    whole_component = val.copy()
-    whole_component[members] *= -1.0
-    assert find(whole_component)[2] == 1 << int(k0)
-
-
 def test_float64_module_gradients_and_the_deterministic_mode():
     """The module in float64 through autograd on the unrolled kernels against the dense form, and
     `config(deterministic=True)`, which takes the table-driven rows that own their dx instead of
@@ -237,3 +200,33 @@ def test_float64_module_gradients_and_the_deterministic_mode():
     for a, b, g in zip(runs[0], runs[1], (gx, gy, gs)):
         assert torch.equal(a, b)
         torch.testing.assert_close(a, g, rtol=1e-11, atol=1e-12)
+
+
+def test_run_time_compiled_kernels_serve_a_float64_table():
+    """A random table of genuine float64 values (no float32 numbers) under `config(jit=True)`: the
+    kernels compiled for its structure take its values as coefficient classes."""
+    from e3j_amd import ConvolutionParams
+    rng = np.random.default_rng(31)
+    N, E, X, Y, Z, S, K, nnz = 40, 600, 5, 6, 7, 4, 64, 50
+    idx, val, mix = H.random_table(rng, nnz, X, Y, Z, S)
+    val = np.asarray(val, dtype=np.float64) * (1.0 + 1e-9 * rng.standard_normal(len(val)))
+    assert not np.array_equal(val, val.astype(np.float32).astype(np.float64))
+    snd, rcv = H.random_graph(rng, N, E)
+    x, y, s, dm = (a.astype(np.float64) * (1 + 1e-9) for a in H.random_operands(rng, N, E, X, Y, S, K, Z))
+    coef = H.pack_table(idx, val, mix, val_dtype=np.float64)
+    params = ConvolutionParams(num_out=Z, num_scalars=S)
+    dev = lambda a: torch.as_tensor(a).cuda()  # noqa: E731
+    with e3j_amd.config.use(jit=True):
+        sig = _Table.get(coef, np.float64).signature((X, Y, Z, S), K, e3j_amd.Layout.TRAILING_CHANNELS)[0]
+        assert sig >= 0
+        out = e3j_amd.convolution(coef, dev(x), dev(y), dev(s), dev(snd), dev(rcv), params, layout="TRAILING_CHANNELS")
+        grads = e3j_amd.convolution_bwd(coef, dev(x), dev(y), dev(s), dev(snd), dev(rcv), dev(dm), params,
+                                        layout="TRAILING_CHANNELS")
+    torch.cuda.synchronize()
+    ref = O.convolution_unfused(idx, val, mix, x, y, s, snd, rcv, Z, dtype=np.float64)
+    mag = O.convolution_unfused(idx, np.abs(val), mix, np.abs(x), np.abs(y), np.abs(s), snd, rcv, Z, dtype=np.float64)
+    assert_parity64(out.cpu().numpy(), ref, mag, "out")
+    refs = O.convolution_vjp(idx, val, mix, x, y, s, snd, rcv, dm, dtype=np.float64)
+    mgs = O.convolution_vjp(idx, np.abs(val), mix, np.abs(x), np.abs(y), np.abs(s), snd, rcv, np.abs(dm), dtype=np.float64)
+    for g, r, mg, what in zip(grads, refs, mgs, ("dx", "dy", "ds")):
+        assert_parity64(g.cpu().numpy(), r, mg, what)
