@@ -29,6 +29,7 @@
 
 #include <cstring>
 #include <map>
+#include <memory>
 #include <mutex>
 #include <tuple>
 #include <vector>
@@ -125,6 +126,9 @@ struct ResolvedTable {
     int32_t signature = -1;
     float scale = 1.0f;
     uint32_t flip = 0;
+    // float64 tables: the coefficient classes the float64 kernels read (shared with the calls that
+    // use them, so that clearing the cache never pulls them away from a call)
+    std::shared_ptr<const F64Coefs> classes;
 };
 
 class TableResolver {
@@ -132,11 +136,15 @@ class TableResolver {
     ResolvedTable resolve(const void *device_table, int32_t num_coef, int32_t idx_bytes, bool columns_ji,
                           const e3j_amd_conv_params &p, hipStream_t caller_stream) {
         ResolvedTable none;
-        if (p.val_dtype != E3J_AMD_F32 || num_coef <= 0 || device_table == nullptr) return none;
-        const size_t item = idx_bytes == 1 ? sizeof(Coef4D<uint8_t, float>) : sizeof(Coef4D<int32_t, float>);
+        const bool f64 = p.val_dtype == E3J_AMD_F64;
+        if ((p.val_dtype != E3J_AMD_F32 && !f64) || num_coef <= 0 || device_table == nullptr) return none;
+        // (the float64 kernels serve receiver rows in the trailing layout: the forward table only)
+        if (f64 && (columns_ji || p.layout != E3J_AMD_LAYOUT_TRAILING)) return none;
+        const size_t item = f64 ? (idx_bytes == 1 ? sizeof(Coef4D<uint8_t, double>) : sizeof(Coef4D<int32_t, double>))
+                                : (idx_bytes == 1 ? sizeof(Coef4D<uint8_t, float>) : sizeof(Coef4D<int32_t, float>));
         const size_t bytes = item * (size_t)num_coef;
-        const Shape shape{num_coef, idx_bytes, columns_ji ? 1 : 0, p.num_x, p.num_y, p.num_out, p.num_scalars,
-                          p.channels, p.layout};
+        const Shape shape{num_coef, idx_bytes + (f64 ? 16 : 0), columns_ji ? 1 : 0, p.num_x, p.num_y, p.num_out,
+                          p.num_scalars, p.channels, p.layout};
         hipStreamCaptureStatus capture = hipStreamCaptureStatusNone;
         if (hipStreamIsCapturing(caller_stream, &capture) != hipSuccess) {
             (void)hipGetLastError();
@@ -172,9 +180,17 @@ class TableResolver {
         }
         // the lookup itself runs without the lock (two threads may do the same one; both find the same)
         ResolvedTable entry;
-        const std::vector<TableEntry> entries = unpack_entries(key.second.data(), idx_bytes, num_coef, columns_ji);
-        entry.signature = match_signature(entries, p.num_x, p.num_y, p.num_out, p.num_scalars, p.channels,
-                                          p.layout, &entry.scale, &entry.flip);
+        if (f64) {
+            auto classes = std::make_shared<F64Coefs>();
+            entry.signature = e3j_amd_find_signature_f64(key.second.data(), idx_bytes, num_coef, p.num_x, p.num_y,
+                                                         p.num_out, p.num_scalars, p.channels, p.layout, classes->v,
+                                                         &entry.flip);
+            entry.classes = std::move(classes);
+        } else {
+            const std::vector<TableEntry> entries = unpack_entries(key.second.data(), idx_bytes, num_coef, columns_ji);
+            entry.signature = match_signature(entries, p.num_x, p.num_y, p.num_out, p.num_scalars, p.channels,
+                                              p.layout, &entry.scale, &entry.flip);
+        }
         if (entry.signature < 0) entry.signature = kNoKernel;
         {
             std::lock_guard<std::mutex> lock(mutex_);
@@ -200,11 +216,25 @@ TableResolver &resolver() {
     return r;
 }
 
-// Uses the id the frame names, or finds the kernels of the table the frame carries.
+struct Decoded {
+    e3j_amd_conv_params p;
+    hipStream_t stream;
+    std::shared_ptr<const F64Coefs> classes;  // what p.coef_classes points to, for the length of the call
+};
+
+// Uses the id the frame names, or finds the kernels of the table the frame carries.  float64
+// frames are always looked up: their kernels need the table's values (coef_classes), which no
+// attribute carries.
 void *choose_kernels(XlaCallFrame *f, const char *op, const XlaBuffer *coef, bool columns_ji,
-                     e3j_amd_conv_params *p, hipStream_t stream) {
+                     Decoded *d, hipStream_t stream) {
+    e3j_amd_conv_params *p = &d->p;
     bool named = false;
     (void)attr<int32_t>(f, "signature", kXlaS32, -1, &named);
+    if (p->val_dtype == E3J_AMD_F64) {
+        named = false;
+        p->signature = -1;
+        p->y_flip = 0;
+    }
     if (named) {
         // an id chosen by the host: at least the table sizes must agree with the operand
         if (p->signature >= 0 && p->signature < e3j_amd_num_signatures() &&
@@ -216,18 +246,15 @@ void *choose_kernels(XlaCallFrame *f, const char *op, const XlaBuffer *coef, boo
         return nullptr;
     }
     const ResolvedTable found = resolver().resolve(coef->data, p->num_coef, p->coef_idx_bytes, columns_ji, *p, stream);
-    if (found.signature >= 0) {
+    if (found.signature >= 0 && (p->val_dtype != E3J_AMD_F64 || found.classes)) {
         p->signature = found.signature;
         p->coef_scale = found.scale;
         p->y_flip = found.flip;
+        d->classes = found.classes;
+        p->coef_classes = found.classes ? found.classes->v : nullptr;
     }
     return nullptr;
 }
-
-struct Decoded {
-    e3j_amd_conv_params p;
-    hipStream_t stream;
-};
 
 // Fills sizes from the buffers, following the reference's handler
 // (lib/e3j_ops/ffi/e3j_ops.h:393-414,496-519).  Returns an XLA error or nullptr.
@@ -428,7 +455,7 @@ void *backward_handler(XlaCallFrame *f, Backward mode) {
     const int64_t numel = coef->dims[coef->rank - 1];
     d.p.num_coef = (int32_t)(count(coef) / numel / (stacked ? 3 : 1));
     const int32_t *perm_ptr = count(perm) ? static_cast<const int32_t *>(perm->data) : nullptr;
-    if (void *err = choose_kernels(f, op, coef, stacked != 0, &d.p, d.stream)) return err;
+    if (void *err = choose_kernels(f, op, coef, stacked != 0, &d, d.stream)) return err;
     // The reference's operands: the adjacency grouped by sender.  The unrolled kernels of that
     // grouping (trailing layout; a row owns its dx) pay a gather of dm rows per edge: faster than
     // a rebuild of the receiver rows (a dozen small launches) plus the receiver-grouped kernel on
@@ -541,7 +568,7 @@ void *e3j_amd_xla_convolution(void *call_frame) {
         (perm && count(perm) != 0 && count(perm) != d.p.num_edges))
         return make_error(f, E3J_AMD_INVALID_ARGUMENT, "convolution: adjacency operand sizes");
     d.p.num_coef = (int32_t)coef->dims[0];
-    if (void *err = choose_kernels(f, "convolution", coef, false, &d.p, d.stream)) return err;
+    if (void *err = choose_kernels(f, "convolution", coef, false, &d, d.stream)) return err;
     const int32_t *perm_ptr = (perm && count(perm)) ? static_cast<const int32_t *>(perm->data) : nullptr;
     const TablePlanMemory plan(f, &d.p);
     const int rc = e3j_amd_convolution_fwd(&d.p, coef->data, x->data, y->data, s->data,

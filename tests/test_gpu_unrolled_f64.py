@@ -230,3 +230,63 @@ def test_run_time_compiled_kernels_serve_a_float64_table():
     mgs = O.convolution_vjp(idx, np.abs(val), mix, np.abs(x), np.abs(y), np.abs(s), snd, rcv, np.abs(dm), dtype=np.float64)
     for g, r, mg, what in zip(grads, refs, mgs, ("dx", "dy", "ds")):
         assert_parity64(g.cpu().numpy(), r, mg, what)
+
+
+def test_float64_frames_of_the_ffi_targets_run_the_float64_kernels():
+    """`convolution` and `convolution_bwd_receiver` frames with float64 buffers and the reference's
+    attributes only: the handler reads the table back, finds the signature's structure and passes the
+    table's values as coefficient classes.  Same bits as the operators (the same kernels), and the
+    time of the unrolled kernels, not of the table-driven ones."""
+    import ctypes as C
+    from e3j_amd.graph import csr_row_ptr
+    from tests.xla_frame import F64, S32, U8, FakeXla
+    lib = _lib.load()
+    w = _with_neighbour_count(W.config2(0.2), 12.5)
+    m = w.module
+    coef = m._packed_coef("float64")
+    host, d = _f64(w)
+    n = w.num_nodes
+    ptr = csr_row_ptr(d["receiver"], n)
+    xla = FakeXla(stream=torch.cuda.current_stream().cuda_stream)
+    xla.allocate = lambda nbytes: torch.empty(nbytes, dtype=torch.uint8, device="cuda")
+
+    def buf(t, dtype):
+        xla._keep.append(t)
+        return xla.buffer(dtype, t.data_ptr(), tuple(t.shape))
+
+    attrs = lambda: {"num_nodes": (S32, C.c_int32(n)), "debug": (S32, C.c_int32(0))}  # noqa: E731
+    coef_d = torch.from_numpy(coef.copy()).cuda()
+    none = torch.zeros(0, dtype=torch.int32, device="cuda")
+    out = torch.full_like(d["dm"], float("nan"))
+    fwd = xla.frame([buf(coef_d, U8), buf(d["x"], F64), buf(d["y"], F64), buf(d["s"], F64), buf(d["sender"], S32),
+                     buf(ptr, S32)], [buf(out, F64)], attrs())
+    dx, dy, ds = (torch.full_like(d[f], float("nan")) for f in ("x", "y", "s"))
+    bwd = xla.frame([buf(coef_d, U8), buf(d["x"], F64), buf(d["y"], F64), buf(d["s"], F64), buf(d["dm"], F64),
+                     buf(d["sender"], S32), buf(ptr, S32), buf(none, S32)],
+                    [buf(dx, F64), buf(dy, F64), buf(ds, F64)], attrs())
+    assert lib.e3j_amd_xla_convolution(C.addressof(fwd)) is None, xla.errors
+    assert lib.e3j_amd_xla_convolution_bwd_receiver(C.addressof(bwd)) is None, xla.errors
+    torch.cuda.synchronize()
+    want = e3j_amd.convolution(coef, d["x"], d["y"], d["s"], d["sender"], d["receiver"], m.params, m.graph_ordering,
+                               layout=m.layout)
+    assert torch.equal(out, want)
+    idx, val, mix = w.table()
+    refs = O.convolution_vjp(idx, np.asarray(val, dtype=np.float64), mix, host["x"], host["y"], host["s"],
+                             host["sender"], host["receiver"], host["dm"], dtype=np.float64)
+    for g, r, what in zip((dx, dy, ds), refs, ("dx", "dy", "ds")):
+        np.testing.assert_allclose(g.cpu().numpy(), r, rtol=1e-11, atol=1e-12, err_msg=what)
+
+    def timed(fn, reps=5):
+        fn()
+        torch.cuda.synchronize()
+        a, b = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        a.record()
+        for _ in range(reps):
+            fn()
+        b.record()
+        torch.cuda.synchronize()
+        return a.elapsed_time(b) / reps
+
+    t_frame = timed(lambda: lib.e3j_amd_xla_convolution(C.addressof(fwd)))
+    print(f"float64 forward frame {t_frame:.3f} ms at {w.num_edges} edges, K={w.channels}")
+    assert t_frame < 0.5, "the table-driven float64 kernels take milliseconds at this size"
