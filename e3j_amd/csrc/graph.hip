@@ -271,16 +271,16 @@ __global__ __launch_bounds__(256) void tile_lists_kernel(
         __builtin_amdgcn_wave_barrier();
         for (int k = 2; k <= padded; k *= 2) {
             for (int j = k / 2; j > 0; j /= 2) {
-                for (int q = lane; q < padded; q += 64) {
-                    const int partner = q ^ j;
-                    if (partner > q) {
-                        const uint64_t a = keys[q], c = keys[partner];
-                        const bool ascending = (q & k) == 0;
-                        if ((a > c) == ascending) {
-                            keys[q] = c; keys[partner] = a;
-                            const uint16_t la = locals[q];
-                            locals[q] = locals[partner]; locals[partner] = la;
-                        }
+                // a lane per pair (q, q | j): q is the pair's number with a zero bit put in at j
+                for (int pr = lane; pr < padded / 2; pr += 64) {
+                    const int q = ((pr & ~(j - 1)) << 1) | (pr & (j - 1));
+                    const int partner = q | j;
+                    const uint64_t a = keys[q], c = keys[partner];
+                    const bool ascending = (q & k) == 0;
+                    if ((a > c) == ascending) {
+                        keys[q] = c; keys[partner] = a;
+                        const uint16_t la = locals[q];
+                        locals[q] = locals[partner]; locals[partner] = la;
                     }
                 }
                 __builtin_amdgcn_fence(__ATOMIC_ACQ_REL, "wavefront");
