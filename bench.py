@@ -118,9 +118,9 @@ def parse_args():
     ap.add_argument("--channels", type=int, default=None,
                     help="channel count of cfg3 (default 128; kernels are built for 32, 64, 128, 256)")
     ap.add_argument("--scale", type=float, default=1.0, help="fraction of the configuration's atoms")
-    ap.add_argument("--dtype", default="f32", choices=["f32", "f64"],
-                    help="f64: the same workload with float64 operands (a secondary figure: the float64 "
-                         "unrolled kernels of the trailing layout)")
+    ap.add_argument("--dtype", default="f32", choices=["f32", "f64", "f16"],
+                    help="f64 / f16: the same workload with float64 / float16 operands (secondary figures: the "
+                         "float64 and float16 unrolled kernels of the trailing layout)")
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--no-layouts", action="store_true",
                     help="skip the leading-channels sub-record of the default run")
@@ -315,36 +315,43 @@ MEASURED_TP_TRAFFIC_BYTES = {
 }
 
 
-def bench_float64(args, torch, device) -> int:
-    """Secondary figure: forward + VJP with float64 operands through the operators (graph preparation
-    in every step), the float64 unrolled kernels timed on their own through the C ABI, and the
-    table-driven kernels, which served float64 before, on an eighth of the workload."""
+def bench_other_dtype(args, torch, device) -> int:
+    """Secondary figure: forward + VJP with float64 or float16 operands through the operators (graph
+    preparation in every step), the unrolled kernels of that dtype timed on their own through the C
+    ABI, and the table-driven kernels, which served these dtypes before, on an eighth of the workload."""
     import numpy as np
     import e3j_amd
     from e3j_amd import _lib
     from e3j_amd.graph import csr_row_ptr, locality_order
     from e3j_amd.ops import _Table, clear_graph_cache
     lib = _lib.load()
+    f64 = args.dtype == "f64"
+    tdtype, ndtype, code, name = ((torch.float64, np.float64, _lib.F64, "float64") if f64
+                                  else (torch.float16, np.float16, _lib.F16, "float16"))
+    shrink = 1.0 if f64 else 0.25   # (sums of thirty messages stay inside the half range)
 
     def calls(w):
         module = w.module
-        table = _Table.get(module._packed_coef("float64"), np.float64)
+        table = _Table.get(module._packed_coef(name), ndtype)
         dims = (int(w.x.shape[1]), int(w.y.shape[1]), module.params.num_out, int(w.s.shape[1]))
         sig, classes, flip = table.signature(dims, w.channels, module.layout)
-        x, y, s, dm = (t.double() for t in (w.x, w.y, w.s, w.dm))
+        x, y, s, dm = ((t * shrink).to(tdtype) for t in (w.x, w.y, w.s, w.dm))
         ptr = csr_row_ptr(w.receiver, w.num_nodes)
         order = locality_order(w.sender, ptr, w.num_nodes, 2)
         out, dx, dy, ds = (torch.empty_like(t) for t in (dm, x, y, s))
         coef = table.device(device)
-        keep = (x, y, s, dm, ptr, order, out, dx, dy, ds, coef, classes)
+        keep_t = []
+        keep = (x, y, s, dm, ptr, order, out, dx, dy, ds, coef, classes, keep_t)
 
         def params(signature):
             p = _lib.ConvParams(num_nodes=w.num_nodes, num_edges=w.num_edges, num_coef=table.num_coef,
                                 num_x=dims[0], num_y=dims[1], num_out=dims[2], num_scalars=dims[3],
-                                channels=w.channels, layout=module.layout.value, val_dtype=_lib.F64,
-                                coef_idx_bytes=table.idx_bytes, signature=signature, coef_scale=1.0, debug=0, y_flip=flip)
+                                channels=w.channels, layout=module.layout.value, val_dtype=code,
+                                coef_idx_bytes=table.idx_bytes, signature=signature,
+                                coef_scale=classes if isinstance(classes, float) and signature >= 0 else 1.0,
+                                debug=0, y_flip=flip if signature >= 0 else 0)
             p.row_order = order.data_ptr()
-            if signature >= 0:
+            if signature >= 0 and f64:
                 p.coef_classes = ctypes.cast(classes, ctypes.c_void_p).value
             return p
 
@@ -356,18 +363,28 @@ def bench_float64(args, torch, device) -> int:
             bwd = lambda: _lib.check(lib.e3j_amd_convolution_bwd_receiver(  # noqa: E731
                 ctypes.byref(p), coef.data_ptr(), x.data_ptr(), y.data_ptr(), s.data_ptr(), dm.data_ptr(),
                 w.sender.data_ptr(), ptr.data_ptr(), None, dx.data_ptr(), dy.data_ptr(), ds.data_ptr(), stream()))
+            if p.signature < 0 and not f64:
+                # the table-driven kernels add dx with float atomics, which have no half form: their
+                # float16 backward runs on the sender-grouped adjacency, whose rows own their dx
+                from e3j_amd.graph import sort_edges
+                tperm, tother, tptr = sort_edges(w.sender, w.receiver, w.num_nodes)
+                keep_t.extend((tperm, tother, tptr))
+                bwd = lambda: _lib.check(lib.e3j_amd_convolution_bwd_sender(  # noqa: E731
+                    ctypes.byref(p), coef.data_ptr(), x.data_ptr(), y.data_ptr(), s.data_ptr(), dm.data_ptr(),
+                    tother.data_ptr(), tptr.data_ptr(), tperm.data_ptr(), dx.data_ptr(), dy.data_ptr(), ds.data_ptr(),
+                    stream()))
             return fwd, bwd
         return sig, params, pair, keep
 
     w = build_workload(args.config, args.scale, device, args.channels)
     if w.module.graph_ordering.value == "NONE" or args.layout != "trailing":
-        print("bench.py --dtype f64 times receiver-ordered workloads in the trailing layout", file=sys.stderr)
+        print("bench.py --dtype f64 / f16 times receiver-ordered workloads in the trailing layout", file=sys.stderr)
         return 2
     module = w.module
-    coef = module._packed_coef("float64")
+    coef = module._packed_coef(name)
     sig, params, pair, keep = calls(w)
     if sig < 0:
-        print("bench.py --dtype f64: no float64 unrolled kernel for this table", file=sys.stderr)
+        print(f"bench.py --dtype {args.dtype}: no {name} unrolled kernel for this table", file=sys.stderr)
         return 2
     xg, yg, sg = (t.requires_grad_(True) for t in keep[:3])
     dm = keep[3]
@@ -390,16 +407,17 @@ def bench_float64(args, torch, device) -> int:
     fwd_ms, bwd_ms = time_events(torch, fwd, args.steps, 2), time_events(torch, bwd, args.steps, 2)
     b32 = w.algorithmic_bytes()
     index_bytes = {"fwd": 4 * (w.num_edges + w.num_nodes + 1), "bwd": 4 * (2 * w.num_edges + w.num_nodes + 1)}
-    b64 = {k: 2 * (b32[k] - index_bytes[k]) + index_bytes[k] for k in ("fwd", "bwd")}   # values double, indices as they are
+    width = 2.0 if f64 else 0.5
+    b64 = {k: int(width * (b32[k] - index_bytes[k])) + index_bytes[k] for k in ("fwd", "bwd")}   # values resized, indices as they are
     frac = lambda nbytes, ms: nbytes / (ms * 1e-3) / 1e9 / HBM_PEAK_GBS  # noqa: E731
     result = {
-        "metric": "edges/sec fused Convolution fwd+VJP fp64", "value": w.num_edges / (ms_per_step * 1e-3),
+        "metric": f"edges/sec fused Convolution fwd+VJP {'fp64' if f64 else 'fp16'}", "value": w.num_edges / (ms_per_step * 1e-3),
         "unit": "edges/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup, "ms_per_step": ms_per_step,
-        "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": "f64", "data": "synthetic",
+        "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": args.dtype, "data": "synthetic",
         "config": {"workload": f"{args.config} x {args.scale}: {w.num_nodes} atoms, {w.num_edges} edges, K={w.channels}, "
-                               "float64 operands, receiver-ordered edges, trailing-channels layout, forward + VJP",
+                               f"{name} operands, receiver-ordered edges, trailing-channels layout, forward + VJP",
                    "signature": sig},
-        "roofline": {"bound": "hbm", "kernel": "convolution backward, float64 (unrolled_bwd_f64_kernel + dx, dy zero fills)",
+        "roofline": {"bound": "hbm", "kernel": f"convolution backward, {name} (unrolled_bwd_{args.dtype}_kernel + dx, dy zero fills)",
                      "achieved": b64["bwd"] / (bwd_ms * 1e-3) / 1e9, "peak": HBM_PEAK_GBS, "unit": "GB/s",
                      "frac": frac(b64["bwd"], bwd_ms), "traffic": None, "algorithmic_bytes": b64["bwd"], "ms": bwd_ms,
                      "forward": {"ms": fwd_ms, "algorithmic_bytes": b64["fwd"], "frac": frac(b64["fwd"], fwd_ms)}},
@@ -637,8 +655,8 @@ def main():
         return bench_radial_linear(args, torch, device)
     if args.config == "cfg5":
         return bench_energy(args, torch, device)
-    if args.dtype == "f64":
-        return bench_float64(args, torch, device)
+    if args.dtype != "f32":
+        return bench_other_dtype(args, torch, device)
 
     w = build_workload(args.config, args.scale, device, args.channels)
     w = w.with_layout("LEADING_CHANNELS" if args.layout == "leading" else "TRAILING_CHANNELS")

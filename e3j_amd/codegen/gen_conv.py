@@ -64,6 +64,10 @@ LAUNCH = {
 #: parts of the float64 kernels: (forward, backward).  A double takes the registers of two channels
 #: of a float kernel, so these are the splits the two-channel float kernels use.
 F64_SPLIT = (3, 4)
+#: float16 kernels (values held as half, computed in float): (channels per lane, parts forward,
+#: parts backward) by whether the channel count is a multiple of 128; the splits of the float
+#: kernels with as many channels per lane
+F16_SHAPE = {True: (2, 2, 3), False: (1, 1, 3)}
 #: the float64 kernels take one coefficient per class of equal magnitude as a kernel argument
 F64_MAX_CLASSES = 64
 #: `bwd_tile`: variants of the backward over tiles of receivers (trailing layout, at least 64
@@ -433,6 +437,7 @@ def emit_table_source(t: "Table", name: str, desc: str, channels: int, symbols, 
         f"// {desc}",
         f"#include {include}",
         "#include " + include.replace("unrolled.h", "unrolled_f64.h"),
+        "#include " + include.replace("unrolled.h", "unrolled_f16.h"),
         "",
         "namespace e3j_amd {",
         "namespace {",
@@ -443,9 +448,10 @@ def emit_table_source(t: "Table", name: str, desc: str, channels: int, symbols, 
     tile = launch.get("bwd_tile", [])
     # float64 kernels: trailing layout, whole waves of channels, few enough coefficient classes
     f64 = channels % 64 == 0 and 0 < len(t.classes) <= F64_MAX_CLASSES
+    f16 = channels % 64 == 0   # float16 kernels: trailing layout, whole waves of channels
     splits = sorted({v[2] for v in launch["fwd"] + launch["bwd"] + tile} |
                     ({v[1] for v in lead["fwd"] + lead["bwd"]} if lead else set()) |
-                    (set(F64_SPLIT) if f64 else set()))
+                    (set(F64_SPLIT) if f64 else set()) | (set(F16_SHAPE[channels % 128 == 0][1:]) if f16 else set()))
     part_names = {}
     for zs in splits:
         names = []
@@ -482,6 +488,11 @@ def emit_table_source(t: "Table", name: str, desc: str, channels: int, symbols, 
     sender_minw = 2
     out += [f"template __global__ void unrolled_bwd_sender_kernel<{channels}, 4, {sender_minw}, "
             f"{part_names[sender_split]}>("] + bwd_args
+    if f16:
+        as_f16 = lambda lines: [ln.replace("float *", "half_t *") for ln in lines]  # noqa: E731
+        h_cpl, h_fwd, h_bwd = F16_SHAPE[channels % 128 == 0]
+        out += [f"template __global__ void unrolled_fwd_f16_kernel<{channels}, {h_cpl}, 4, {part_names[h_fwd]}>("] + as_f16(fwd_args)
+        out += [f"template __global__ void unrolled_bwd_f16_kernel<{channels}, {h_cpl}, 4, {part_names[h_bwd]}>("] + as_f16(bwd_args)
     if f64:
         as_f64 = lambda lines: [ln.replace("float", "double").replace("unsigned);", "unsigned, F64Coefs);")  # noqa: E731
                                 for ln in lines]
@@ -515,6 +526,19 @@ def emit_table_source(t: "Table", name: str, desc: str, channels: int, symbols, 
             f"static const float kVal[] = {{{vals}}};",
             f"static const uint8_t kIdx[] = {{{idxs}}};",
             ""]
+    if f16:
+        out += ["static int run_fwd_f16(const e3j_amd_conv_params &p, const half_t *x, const half_t *y, const half_t *s,",
+                "                       const int32_t *sender, const int32_t *row_ptr, const int32_t *perm, half_t *out,",
+                "                       hipStream_t stream) {",
+                f"    return launch_unrolled_fwd_f16<{channels}, {h_cpl}, 4, {part_names[h_fwd]}>(",
+                "        p, x, y, s, sender, row_ptr, perm, out, stream);",
+                "}",
+                "static int run_bwd_f16(const e3j_amd_conv_params &p, const half_t *x, const half_t *y, const half_t *s,",
+                "                       const half_t *dm, const int32_t *sender, const int32_t *row_ptr,",
+                "                       const int32_t *perm, half_t *dx, half_t *dy, half_t *ds, hipStream_t stream) {",
+                f"    return launch_unrolled_bwd_f16<{channels}, {h_cpl}, 4, {t.Y}, {t.X}, {part_names[h_bwd]}>(",
+                "        p, x, y, s, dm, sender, row_ptr, perm, dx, dy, ds, stream);",
+                "}", ""]
     if f64:
         out += ["// class of equal magnitude of every entry (the float64 kernels read one coefficient per class)",
                 f"static const uint8_t kClass[] = {{{', '.join(str(c) for c in t.class_of)}}};",
@@ -563,6 +587,7 @@ def emit_table_source(t: "Table", name: str, desc: str, channels: int, symbols, 
             f"    {t.X}, {t.Y}, {t.Z}, {t.S}, {len(t.val)}, {channels}, E3J_AMD_LAYOUT_TRAILING, kVal, kIdx,",
             f"    &run_fwd, &run_bwd, {tiled}, &run_bwd_sender,",
             f"    {len(t.classes)}, kClass, &run_fwd_f64, &run_bwd_f64," if f64 else "    0, nullptr, nullptr, nullptr,",
+            "    &run_fwd_f16, &run_bwd_f16," if f16 else "    nullptr, nullptr,",
             "};", ""]
     if lead:
         out += ["static int run_fwd_leading" + fwd_sig[0]] + fwd_sig[1:]

@@ -101,7 +101,8 @@ int validate(const e3j_amd_conv_params *p, const char *op) {
     if (p->signature >= 0) {
         const Signature &sg = signature(p->signature);
         const bool dtype_served = p->val_dtype == E3J_AMD_F32 ||
-                                  (p->val_dtype == E3J_AMD_F64 && sg.fwd_f64 != nullptr && sg.bwd_f64 != nullptr);
+                                  (p->val_dtype == E3J_AMD_F64 && sg.fwd_f64 != nullptr && sg.bwd_f64 != nullptr) ||
+                                  (p->val_dtype == E3J_AMD_F16 && sg.fwd_f16 != nullptr && sg.bwd_f16 != nullptr);
         if (!dtype_served || sg.num_x != p->num_x || sg.num_y != p->num_y ||
             sg.num_out != p->num_out || sg.num_scalars != p->num_scalars ||
             sg.channels != p->channels || sg.layout != p->layout)
@@ -133,9 +134,12 @@ bool signature_fits(const e3j_amd_conv_params *p, std::initializer_list<const vo
 bool signature_fits_f64(const e3j_amd_conv_params *p) {
     return p->signature >= 0 && p->val_dtype == E3J_AMD_F64;
 }
+bool signature_fits_f16(const e3j_amd_conv_params *p) {
+    return p->signature >= 0 && p->val_dtype == E3J_AMD_F16;
+}
 int f64_receiver_rows_only(const char *op) {
     return set_error(E3J_AMD_UNIMPLEMENTED,
-                     std::string(op) + ": the float64 unrolled kernels serve the forward pass and the "
+                     std::string(op) + ": the float64 and float16 unrolled kernels serve the forward pass and the "
                                        "receiver-grouped backward; pass signature = -1 for the table-driven kernel");
 }
 // Falling back to the table-driven kernel is only right when no sign flip was asked for.
@@ -176,6 +180,15 @@ int run_backward(const e3j_amd_conv_params *p, bool group_is_receiver, const voi
         if (rc == E3J_AMD_OK)
             rc = launch_zero_padding(*p, other, row_ptr, edge_perm, static_cast<double *>(dy),
                                      static_cast<double *>(ds), stream);
+    } else if (signature_fits_f16(p)) {
+        if (!group_is_receiver) return f64_receiver_rows_only(op);
+        rc = signature(p->signature).bwd_f16(*p, static_cast<const half_t *>(x), static_cast<const half_t *>(y),
+                                             static_cast<const half_t *>(s), static_cast<const half_t *>(dm),
+                                             other, row_ptr, edge_perm, static_cast<half_t *>(dx),
+                                             static_cast<half_t *>(dy), static_cast<half_t *>(ds), stream);
+        if (rc == E3J_AMD_OK)
+            rc = launch_zero_padding(*p, other, row_ptr, edge_perm, static_cast<half_t *>(dy),
+                                     static_cast<half_t *>(ds), stream);
     } else if (group_is_receiver && signature_fits(p, {x, s, dm, dx, ds}) &&
         signature(p->signature).bwd != nullptr) {
         rc = signature(p->signature).bwd(*p, static_cast<const float *>(x),
@@ -237,7 +250,7 @@ bool entry_less(const TableEntry &a, const TableEntry &b) {
 // permutes the rows of a table when it balances them over warps (src/e3j/ops/convolution.py:178-208).
 int match_signature(std::vector<TableEntry> entries, int32_t num_x, int32_t num_y, int32_t num_out,
                     int32_t num_scalars, int32_t channels, int32_t layout, float *coef_scale,
-                    uint32_t *y_flip) {
+                    uint32_t *y_flip, double tolerance, bool float16_kernels) {
     if (coef_scale) *coef_scale = 1.0f;
     if (y_flip) *y_flip = 0;
     const int num_coef = (int)entries.size();
@@ -251,6 +264,7 @@ int match_signature(std::vector<TableEntry> entries, int32_t num_x, int32_t num_
             sg.num_out != num_out || sg.num_scalars != num_scalars || sg.channels != channels ||
             sg.layout != layout)
             continue;
+        if (float16_kernels && (sg.fwd_f16 == nullptr || sg.bwd_f16 == nullptr)) continue;
         for (int n = 0; n < num_coef; n++) {
             own[n].val = sg.val[n];
             for (int t = 0; t < 4; t++) own[n].idx[t] = sg.idx[4 * n + t];
@@ -271,8 +285,8 @@ int match_signature(std::vector<TableEntry> entries, int32_t num_x, int32_t num_
             for (int t = 0; t < 4 && same; t++) same = idx[t] == own[n].idx[t];
             if (!same) break;
             const double v = entries[n].val, want = scale * (double)own[n].val;
-            const bool plus = std::fabs(v - want) <= 4e-7 * std::fabs(want);
-            const bool minus = std::fabs(v + want) <= 4e-7 * std::fabs(want);
+            const bool plus = std::fabs(v - want) <= tolerance * std::fabs(want);
+            const bool minus = std::fabs(v + want) <= tolerance * std::fabs(want);
             if (plus) {
                 same = !signs_allowed || !((seen >> idx[2]) & 1u) || !((flip >> idx[2]) & 1u);
             } else if (minus && signs_allowed) {
@@ -340,6 +354,15 @@ int e3j_amd_convolution_fwd(const e3j_amd_conv_params *p, const void *coef, cons
         rc = signature(p->signature).fwd_f64(*p, static_cast<const double *>(x), static_cast<const double *>(y),
                                              static_cast<const double *>(s), sender, receiver_ptr, edge_perm,
                                              static_cast<double *>(out), stream);
+        return finish(p, stream, rc, "convolution");
+    }
+    if (signature_fits_f16(p)) {
+        if (p->row_cap != 0 || p->segments != nullptr)
+            return set_error(E3J_AMD_UNIMPLEMENTED, "convolution: row_cap / segments are taken by the float32 "
+                                                    "unrolled kernels only");
+        rc = signature(p->signature).fwd_f16(*p, static_cast<const half_t *>(x), static_cast<const half_t *>(y),
+                                             static_cast<const half_t *>(s), sender, receiver_ptr, edge_perm,
+                                             static_cast<half_t *>(out), stream);
         return finish(p, stream, rc, "convolution");
     }
     const bool split_rows = p->row_cap > 0 || p->segments != nullptr;
@@ -551,8 +574,26 @@ int e3j_amd_find_signature(const void *coef_host, int32_t coef_idx_bytes, int32_
                            float *coef_scale, uint32_t *y_flip) {
     if (coef_scale) *coef_scale = 1.0f;
     if (y_flip) *y_flip = 0;
-    if (coef_host == nullptr || val_dtype != E3J_AMD_F32 || num_coef <= 0) return -1;
+    if (coef_host == nullptr || (val_dtype != E3J_AMD_F32 && val_dtype != E3J_AMD_F16) || num_coef <= 0) return -1;
     if (coef_idx_bytes != 1 && coef_idx_bytes != 4) return -1;
+    if (val_dtype == E3J_AMD_F16) {
+        // a table of half values: every entry within half rounding (2^-11) of the built-in table times one
+        // factor; the float16 kernels then compute with the built-in float values
+        const size_t item = coef_idx_bytes == 1 ? sizeof(Coef4D<uint8_t, half_t>) : sizeof(Coef4D<int32_t, half_t>);
+        const unsigned char *bytes = static_cast<const unsigned char *>(coef_host);
+        std::vector<TableEntry> entries((size_t)num_coef);
+        for (int n = 0; n < num_coef; n++) {
+            half_t h;
+            std::memcpy(&h, bytes + n * item, sizeof(h));
+            entries[n].val = (float)h;
+            for (int t = 0; t < 4; t++) {
+                if (coef_idx_bytes == 1) entries[n].idx[t] = bytes[n * item + 2 + t];
+                else std::memcpy(&entries[n].idx[t], bytes + n * item + 4 + 4 * t, 4);
+            }
+        }
+        return match_signature(entries, num_x, num_y, num_out, num_scalars, channels, layout, coef_scale, y_flip,
+                               1.0 / 1024.0, true);
+    }
     const std::vector<TableEntry> entries = unpack_entries(coef_host, coef_idx_bytes, num_coef, false);
     return match_signature(entries, num_x, num_y, num_out, num_scalars, channels, layout, coef_scale, y_flip);
 }

@@ -110,6 +110,8 @@ int launch_zero_padding(const e3j_amd_conv_params &p, const int32_t *other, cons
                         const int32_t *perm, float *dy, float *ds, hipStream_t stream);
 int launch_zero_padding(const e3j_amd_conv_params &p, const int32_t *other, const int32_t *row_ptr,
                         const int32_t *perm, double *dy, double *ds, hipStream_t stream);
+int launch_zero_padding(const e3j_amd_conv_params &p, const int32_t *other, const int32_t *row_ptr,
+                        const int32_t *perm, half_t *dy, half_t *ds, hipStream_t stream);
 
 // Launch-shape variants of the unrolled kernels, from E3J_AMD_FWD_VARIANT /
 // E3J_AMD_BWD_VARIANT (read once; 0 = default).  For tuning runs.
@@ -189,6 +191,14 @@ struct Signature {
     int (*bwd_f64)(const e3j_amd_conv_params &p, const double *x, const double *y, const double *s,
                    const double *dm, const int32_t *sender, const int32_t *receiver_ptr,
                    const int32_t *edge_perm, double *dx, double *dy, double *ds, hipStream_t stream);
+    // float16 kernels (trailing layout, receiver rows; nullptr: none): values held as half, the float
+    // kernels' arithmetic, literals and scale factor
+    int (*fwd_f16)(const e3j_amd_conv_params &p, const half_t *x, const half_t *y, const half_t *s,
+                   const int32_t *sender, const int32_t *receiver_ptr, const int32_t *edge_perm, half_t *out,
+                   hipStream_t stream);
+    int (*bwd_f16)(const e3j_amd_conv_params &p, const half_t *x, const half_t *y, const half_t *s,
+                   const half_t *dm, const int32_t *sender, const int32_t *receiver_ptr,
+                   const int32_t *edge_perm, half_t *dx, half_t *dy, half_t *ds, hipStream_t stream);
 };
 // the coefficient classes of a float64 launch, passed to the kernel by value
 constexpr int kF64Classes = E3J_AMD_F64_CLASSES;
@@ -206,7 +216,7 @@ std::vector<TableEntry> unpack_entries(const void *packed_host, int32_t coef_idx
                                        bool columns_ji);
 int match_signature(std::vector<TableEntry> entries, int32_t num_x, int32_t num_y, int32_t num_out,
                     int32_t num_scalars, int32_t channels, int32_t layout, float *coef_scale,
-                    uint32_t *y_flip);
+                    uint32_t *y_flip, double tolerance = 4e-7, bool float16_kernels = false);
 int num_builtin_signatures();
 const Signature &builtin_signature(int id);
 int num_signatures();

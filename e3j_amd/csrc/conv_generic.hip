@@ -564,6 +564,10 @@ int launch_zero_padding(const e3j_amd_conv_params &p, const int32_t *other, cons
                         const int32_t *perm, double *dy, double *ds, hipStream_t stream) {
     return zero_padding<double>(p, other, row_ptr, perm, dy, ds, stream);
 }
+int launch_zero_padding(const e3j_amd_conv_params &p, const int32_t *other, const int32_t *row_ptr,
+                        const int32_t *perm, half_t *dy, half_t *ds, hipStream_t stream) {
+    return zero_padding<half_t>(p, other, row_ptr, perm, dy, ds, stream);
+}
 
 // The plan of a table the planned kernels can take (conv_planned.hip): in the caller's memory
 // (e3j_amd_conv_params.table_plan) or, without it, in memory of the stream's pool for the length

@@ -44,7 +44,8 @@ def _key(val: np.ndarray, idx4: np.ndarray, dims, channels: int) -> str:
     h.update(np.ascontiguousarray(idx4, dtype=np.int64).tobytes())
     h.update(repr((tuple(int(d) for d in dims), int(channels))).encode())
     for path in (gen_conv.__file__, os.path.join(_build.CSRC, "unrolled.h"),
-                 os.path.join(_build.CSRC, "unrolled_f64.h"), os.path.join(_build.CSRC, "common.h"), _PUBLIC_HEADER):
+                 os.path.join(_build.CSRC, "unrolled_f64.h"), os.path.join(_build.CSRC, "unrolled_f16.h"),
+                 os.path.join(_build.CSRC, "common.h"), _PUBLIC_HEADER):
         with open(path, "rb") as fh:      # kernels of another version of the templates are stale
             h.update(fh.read())
     return h.hexdigest()[:20]

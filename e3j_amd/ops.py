@@ -134,7 +134,8 @@ class _Table:
         hit = self._signature.get(key)
         if hit is None:
             scale, flip = ctypes.c_float(1.0), ctypes.c_uint32(0)
-            val_code = _lib.F32 if self.val_np_dtype == np.float32 else _lib.F64
+            val_code = {np.dtype(np.float32): _lib.F32, np.dtype(np.float64): _lib.F64,
+                        np.dtype(np.float16): _lib.F16}[self.val_np_dtype]
 
             classes = (ctypes.c_double * _lib.F64_CLASSES)()
 
@@ -148,7 +149,7 @@ class _Table:
                     dims[2], dims[3], channels, layout.value, ctypes.byref(scale), ctypes.byref(flip)))
 
             sig = find()
-            if sig < 0 and jit and self.val_np_dtype in (np.float32, np.float64) and self.num_coef > 0:
+            if sig < 0 and jit and self.num_coef > 0:
                 # not built in: generate and compile the kernels of this table, then look again
                 from . import jit as _jit
                 c = self.unpack()
@@ -463,12 +464,13 @@ def _raw_backward(meta: _Meta, x, y, s, dm, sender, receiver, graph=None):
     n = meta.num_nodes
     dx, dy, ds = torch.empty_like(x), torch.empty_like(y), torch.empty_like(s)
     lib = _lib.load()
-    # float16: dx by float atomics has no half-precision form, rows must own their dx
-    deterministic = config().deterministic or x.dtype == torch.float16
     table = meta.table
     has_kernel = table.signature(*_shape(meta, x, y, s), meta.layout)[0] >= 0
-    if x.dtype == torch.float64 and deterministic:
-        has_kernel = False   # the float64 unrolled backward adds dx with atomics; rows that own dx: table-driven
+    # float16 without an unrolled kernel: the table-driven kernels have no half-precision form of dx by
+    # atomics, rows must own their dx
+    deterministic = config().deterministic or (x.dtype == torch.float16 and not has_kernel)
+    if x.dtype != torch.float32 and deterministic:
+        has_kernel = False   # the float64 / float16 unrolled backward adds dx with atomics; rows that own dx: table-driven
     # SENDER ordering: the cotangents belong to the edges as given (dy[e], ds[e] come from
     # dm[receiver(e)]), not to the reversed edges the forward walks
     # (`src/e3j/ops/convolution.py:413-431`).  With an unrolled kernel for the table the edges

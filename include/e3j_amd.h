@@ -255,7 +255,10 @@ int e3j_amd_convolution_bwd_tiled(const e3j_amd_conv_params *p, const void *x, c
  * into the table for the SENDER ordering, src/e3j/ops/convolution.py:166-176), returned as
  * a bit mask for e3j_amd_conv_params.y_flip (tables with more than 32 y components match
  * only without signs).  Returns the signature id (>= 0) or -1.  Takes the place of the reference's
- * trace-time launch planning (src/e3j/ops/convolution.py:178-208). */
+ * trace-time launch planning (src/e3j/ops/convolution.py:178-208).
+ * val_dtype: E3J_AMD_F32, or E3J_AMD_F16 for a table of half values (float16 operands on the float16
+ * unrolled kernels: trailing layout, forward and receiver-grouped backward, operands 4-byte aligned);
+ * entries then agree within half rounding.  float64 tables: e3j_amd_find_signature_f64. */
 int e3j_amd_find_signature(const void *coef_host, int32_t coef_idx_bytes, int32_t val_dtype,
                            int32_t num_coef, int32_t num_x, int32_t num_y, int32_t num_out,
                            int32_t num_scalars, int32_t channels, int32_t layout,

@@ -306,6 +306,7 @@ def test_float16_through_the_operator_in_both_forms(plans):
     snd, rcv = H.random_graph(rng, N, E)
     x, y, s, dm = (a.astype(np.float16) for a in H.random_operands(rng, N, E, 16, 16, 23, K, 99))
     val16 = np.asarray(val).astype(np.float16)
+    val16[0] *= np.float16(1.25)   # no longer the built-in table: the table-driven kernels serve it
     coef = H.pack_table(idx, val16, mix, val_dtype=np.float16)
     lib = _lib.load()
     lib.e3j_amd_set_table_plans(plans)
