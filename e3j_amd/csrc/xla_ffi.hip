@@ -136,14 +136,15 @@ class TableResolver {
     ResolvedTable resolve(const void *device_table, int32_t num_coef, int32_t idx_bytes, bool columns_ji,
                           const e3j_amd_conv_params &p, hipStream_t caller_stream) {
         ResolvedTable none;
-        const bool f64 = p.val_dtype == E3J_AMD_F64;
-        if ((p.val_dtype != E3J_AMD_F32 && !f64) || num_coef <= 0 || device_table == nullptr) return none;
-        // (the float64 kernels serve receiver rows in the trailing layout: the forward table only)
-        if (f64 && (columns_ji || p.layout != E3J_AMD_LAYOUT_TRAILING)) return none;
-        const size_t item = f64 ? (idx_bytes == 1 ? sizeof(Coef4D<uint8_t, double>) : sizeof(Coef4D<int32_t, double>))
-                                : (idx_bytes == 1 ? sizeof(Coef4D<uint8_t, float>) : sizeof(Coef4D<int32_t, float>));
+        const bool f64 = p.val_dtype == E3J_AMD_F64, f16 = p.val_dtype == E3J_AMD_F16;
+        if (num_coef <= 0 || device_table == nullptr) return none;
+        // (the float64 and float16 kernels serve receiver rows in the trailing layout: the forward table only)
+        if ((f64 || f16) && (columns_ji || p.layout != E3J_AMD_LAYOUT_TRAILING)) return none;
+        const size_t item = f64   ? (idx_bytes == 1 ? sizeof(Coef4D<uint8_t, double>) : sizeof(Coef4D<int32_t, double>))
+                            : f16 ? (idx_bytes == 1 ? sizeof(Coef4D<uint8_t, half_t>) : sizeof(Coef4D<int32_t, half_t>))
+                                  : (idx_bytes == 1 ? sizeof(Coef4D<uint8_t, float>) : sizeof(Coef4D<int32_t, float>));
         const size_t bytes = item * (size_t)num_coef;
-        const Shape shape{num_coef, idx_bytes + (f64 ? 16 : 0), columns_ji ? 1 : 0, p.num_x, p.num_y, p.num_out,
+        const Shape shape{num_coef, idx_bytes + (f64 ? 16 : f16 ? 32 : 0), columns_ji ? 1 : 0, p.num_x, p.num_y, p.num_out,
                           p.num_scalars, p.channels, p.layout};
         hipStreamCaptureStatus capture = hipStreamCaptureStatusNone;
         if (hipStreamIsCapturing(caller_stream, &capture) != hipSuccess) {
@@ -186,6 +187,10 @@ class TableResolver {
                                                          p.num_out, p.num_scalars, p.channels, p.layout, classes->v,
                                                          &entry.flip);
             entry.classes = std::move(classes);
+        } else if (f16) {
+            entry.signature = e3j_amd_find_signature(key.second.data(), idx_bytes, E3J_AMD_F16, num_coef, p.num_x,
+                                                     p.num_y, p.num_out, p.num_scalars, p.channels, p.layout,
+                                                     &entry.scale, &entry.flip);
         } else {
             const std::vector<TableEntry> entries = unpack_entries(key.second.data(), idx_bytes, num_coef, columns_ji);
             entry.signature = match_signature(entries, p.num_x, p.num_y, p.num_out, p.num_scalars, p.channels,
@@ -456,6 +461,11 @@ void *backward_handler(XlaCallFrame *f, Backward mode) {
     d.p.num_coef = (int32_t)(count(coef) / numel / (stacked ? 3 : 1));
     const int32_t *perm_ptr = count(perm) ? static_cast<const int32_t *>(perm->data) : nullptr;
     if (void *err = choose_kernels(f, op, coef, stacked != 0, &d, d.stream)) return err;
+    if (mode == Backward::kSenderRows && d.p.val_dtype != E3J_AMD_F32) {
+        // the float64 and float16 unrolled kernels walk receiver rows only: sender rows stay table-driven
+        d.p.signature = -1;
+        d.p.y_flip = 0;
+    }
     // The reference's operands: the adjacency grouped by sender.  The unrolled kernels of that
     // grouping (trailing layout; a row owns its dx) pay a gather of dm rows per edge: faster than
     // a rebuild of the receiver rows (a dozen small launches) plus the receiver-grouped kernel on

@@ -178,3 +178,49 @@ def test_float16_module_through_autograd_and_the_deterministic_mode():
     for a, b, r, mg, what in zip(runs[0], runs[1], refs, mgs, ("dx", "dy", "ds")):
         assert torch.equal(a, b)
         assert_parity16(a, r, mg, f"deterministic {what}", 4.0)
+
+
+def test_float16_frames_of_the_ffi_targets_run_the_float16_kernels():
+    """`convolution` and `convolution_bwd_receiver` frames with float16 buffers and the reference's
+    attributes only: the handler finds the half-valued table among the signatures and runs the
+    float16 unrolled kernels, the operators' bits."""
+    import ctypes as C
+    from e3j_amd.graph import csr_row_ptr
+    from tests.xla_frame import F16, S32, U8, FakeXla
+    lib = _lib.load()
+    w = W.config2(0.2)
+    m = w.module
+    coef = m._packed_coef("float16")
+    host, d = _half(w)
+    n = w.num_nodes
+    ptr = csr_row_ptr(d["receiver"], n)
+    xla = FakeXla(stream=torch.cuda.current_stream().cuda_stream)
+
+    def buf(t, dtype):
+        xla._keep.append(t)
+        return xla.buffer(dtype, t.data_ptr(), tuple(t.shape))
+
+    attrs = lambda: {"num_nodes": (S32, C.c_int32(n)), "debug": (S32, C.c_int32(0))}  # noqa: E731
+    coef_d = torch.from_numpy(coef.copy()).cuda()
+    none = torch.zeros(0, dtype=torch.int32, device="cuda")
+    out = torch.full_like(d["dm"], float("nan"))
+    fwd = xla.frame([buf(coef_d, U8), buf(d["x"], F16), buf(d["y"], F16), buf(d["s"], F16), buf(d["sender"], S32),
+                     buf(ptr, S32)], [buf(out, F16)], attrs())
+    dx, dy, ds = (torch.full_like(d[f], float("nan")) for f in ("x", "y", "s"))
+    bwd = xla.frame([buf(coef_d, U8), buf(d["x"], F16), buf(d["y"], F16), buf(d["s"], F16), buf(d["dm"], F16),
+                     buf(d["sender"], S32), buf(ptr, S32), buf(none, S32)],
+                    [buf(dx, F16), buf(dy, F16), buf(ds, F16)], attrs())
+    assert lib.e3j_amd_xla_convolution(C.addressof(fwd)) is None, xla.errors
+    assert lib.e3j_amd_xla_convolution_bwd_receiver(C.addressof(bwd)) is None, xla.errors
+    torch.cuda.synchronize()
+    want = e3j_amd.convolution(coef, d["x"], d["y"], d["s"], d["sender"], d["receiver"], m.params, m.graph_ordering,
+                               layout=m.layout)
+    assert torch.equal(out, want)
+    idx, val, mix = w.table()
+    val = np.asarray(val).astype(np.float16).astype(np.float64)
+    args = (host["x"], host["y"], host["s"], host["sender"], host["receiver"])
+    mags = tuple(np.abs(t) for t in args[:3]) + args[3:]
+    refs = O.convolution_vjp(idx, val, mix, *args, host["dm"], dtype=np.float64)
+    mgs = O.convolution_vjp(idx, np.abs(val), mix, *mags, np.abs(host["dm"]), dtype=np.float64)
+    for g, r, mg, what, sums in zip((dx, dy, ds), refs, mgs, ("dx", "dy", "ds"), (4.0, 2.0, 1.0)):
+        assert_parity16(g, r, mg, what, sums)
