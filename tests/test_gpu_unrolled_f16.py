@@ -38,7 +38,6 @@ CASES = {
     "cfg3": lambda: W.config3(0.004),
     "cfg3_k256": lambda: W.config3(0.002, channels=256),
     "cfg2": lambda: W.config2(0.04),                      # y up to l = 3 on x up to l = 2
-    "cfg1": lambda: W.config1(0.2),
     "scalars_k64": lambda: W.make_workload("scalars", 200, "0e", 3, "0e+1o+2e+3o", 64, (51, 52, 53, 54)),
 }
 
@@ -61,8 +60,6 @@ def test_float16_unrolled_kernels_match_the_oracle(name):
     m = w.module
     coef = m._packed_coef("float16")
     dims = (int(w.x.shape[1]), int(w.y.shape[1]), m.params.num_out, int(w.s.shape[1]))
-    if w.channels % 64:
-        pytest.skip("the float16 kernels take whole waves of channels")
     sig, scale, flip = _Table.get(coef, np.float16).signature(dims, w.channels, m.layout)
     assert sig >= 0 and flip == 0, "the half-rounded table must resolve to the built-in signature"
     host, d = _half(w)
