@@ -57,6 +57,43 @@ def test_config1_and_config2_full_size_match_checker():
         _against_c_oracle(w, out, grads, w.name)
 
 
+def test_config2_full_size_in_float64_and_float16():
+    """Configuration 2 at full size with float64 and float16 operands on the unrolled kernels of those
+    dtypes, against the C checker's loops in float64: float64 within 64 float64 roundings of the
+    terms' magnitudes, float16 (operands and table rounded to half, results summed in half by the
+    atomics) within half-precision rounding of them."""
+    w = W.config2(device="cuda")
+    m = w.module
+    idx, val, mix = w.table()
+    Z = m.params.num_out
+    for dtype, name, scale in ((torch.float64, "float64", 1.0), (torch.float16, "float16", 0.25)):
+        coef = m._packed_coef(name)
+        x, y, s, dm = ((t * scale).to(dtype) for t in (w.x, w.y, w.s, w.dm))
+        out = e3j_amd.convolution(coef, x, y, s, w.sender, w.receiver, m.params, m.graph_ordering, layout=m.layout)
+        grads = e3j_amd.convolution_bwd(coef, x, y, s, w.sender, w.receiver, dm, m.params, m.graph_ordering,
+                                        layout=m.layout)
+        torch.cuda.synchronize()
+        assert out.dtype == dtype
+        host = [t.double().cpu().numpy() for t in (x, y, s, dm)]
+        snd, rcv = w.sender.cpu().numpy(), w.receiver.cpu().numpy()
+        v = np.asarray(val).astype(np.float16 if dtype == torch.float16 else np.float64).astype(np.float64)
+        args = (host[0], host[1], host[2], snd, rcv)
+        mag_args = tuple(np.abs(t) for t in args[:3]) + args[3:]
+        ref = c_oracle.convolution(idx, v, mix, *args, Z, dtype=np.float64)
+        mag = c_oracle.convolution(idx, np.abs(v), mix, *mag_args, Z, dtype=np.float64)
+        refs = c_oracle.convolution_vjp(idx, v, mix, *args, host[3], dtype=np.float64)
+        mags = c_oracle.convolution_vjp(idx, np.abs(v), mix, *mag_args, np.abs(host[3]), dtype=np.float64)
+        if dtype == torch.float64:
+            bound = lambda m_, sums: 64 * 2.0 ** -52 * m_ + 1e-300   # noqa: E731
+        else:   # (dx and the shared dy rows take one half rounding per addend)
+            bound = lambda m_, sums: 6 * sums * 2.0 ** -10 * m_ + 1e-3   # noqa: E731
+        for got, r, m_, what, sums in zip((out,) + tuple(grads), (ref,) + tuple(refs), (mag,) + tuple(mags),
+                                          ("out", "dx", "dy", "ds"), (1.0, 4.0, 2.0, 1.0)):
+            err = np.abs(got.double().cpu().numpy() - r)
+            assert np.isfinite(err).all() and (err <= bound(m_, sums)).all(), (
+                f"cfg2 {name} {what}: worst error {err.max():.3e}, {int((err > bound(m_, sums)).sum())} elements off")
+
+
 def test_config2_leading_layout_full_size_matches_checker():
     """The configuration as the baseline names it: channels before the irreps axis."""
     w = W.config2(device="cuda").with_layout("LEADING_CHANNELS")
