@@ -333,9 +333,12 @@ __global__ void zero_padding_edges_kernel(const int32_t *__restrict__ other,
     }
 }
 
-__global__ void fill_zero_kernel(uint32_t *__restrict__ p, size_t n_words) {
+// n_words whole words, then `tail_halves` (0 or 1) two-byte values behind them
+__global__ void fill_zero_kernel(uint32_t *__restrict__ p, size_t n_words, int tail_halves) {
     const size_t stride = (size_t)gridDim.x * blockDim.x;
-    for (size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x; i < n_words; i += stride) p[i] = 0u;
+    const size_t first = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
+    for (size_t i = first; i < n_words; i += stride) p[i] = 0u;
+    if (tail_halves && first == 0) *reinterpret_cast<uint16_t *>(p + n_words) = 0;
 }
 
 constexpr size_t kMaxLds = 160 * 1024;  // LDS per CU / per workgroup on gfx950
@@ -547,12 +550,13 @@ int reduce_ordered_dy(const e3j_amd_conv_params &p, const float *dy_slots, int s
 
 int launch_fill_zero(void *ptr, size_t bytes, hipStream_t stream) {
     if (bytes == 0) return E3J_AMD_OK;
-    if (bytes % 4 != 0 || (reinterpret_cast<uintptr_t>(ptr) % 4) != 0)
+    // whole 32-bit words, and one trailing half value (an odd number of float16 elements)
+    if (bytes % 2 != 0 || (reinterpret_cast<uintptr_t>(ptr) % 4) != 0)
         return set_error(E3J_AMD_INVALID_ARGUMENT, "fill: buffer must be 4-byte aligned");
     const size_t words = bytes / 4;
-    const size_t blocks = std::min<size_t>((words + 255) / 256, 8192);
+    const size_t blocks = std::max<size_t>(1, std::min<size_t>((words + 255) / 256, 8192));
     hipLaunchKernelGGL(fill_zero_kernel, dim3((unsigned)blocks), dim3(256), 0, stream,
-                       static_cast<uint32_t *>(ptr), words);
+                       static_cast<uint32_t *>(ptr), words, (int)(bytes % 4 / 2));
     return check_hip(hipGetLastError(), "fill launch");
 }
 
