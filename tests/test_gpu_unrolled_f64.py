@@ -290,3 +290,71 @@ def test_float64_frames_of_the_ffi_targets_run_the_float64_kernels():
     t_frame = timed(lambda: lib.e3j_amd_xla_convolution(C.addressof(fwd)))
     print(f"float64 forward frame {t_frame:.3f} ms at {w.num_edges} edges, K={w.channels}")
     assert t_frame < 0.5, "the table-driven float64 kernels take milliseconds at this size"
+
+
+@pytest.mark.parametrize("dtype", ["float64", "float16"])
+def test_float64_and_float16_entry_points_replay_from_a_captured_graph(dtype):
+    """Forward and backward of the float64 / float16 unrolled kernels recorded into a HIP graph (their
+    zero fills are kernels; the coefficient classes of a float64 call are copied into the launch when
+    it is recorded) and replayed on new operand values with eager work in between."""
+    from e3j_amd.graph import csr_row_ptr, locality_order
+    f64 = dtype == "float64"
+    w = _with_neighbour_count(W.config2(0.04), 12.5)
+    m = w.module
+    np_dtype, tdtype, code = (np.float64, torch.float64, _lib.F64) if f64 else (np.float16, torch.float16, _lib.F16)
+    table = _Table.get(m._packed_coef(dtype), np_dtype)
+    dims = (int(w.x.shape[1]), int(w.y.shape[1]), m.params.num_out, int(w.s.shape[1]))
+    sig, scale, flip = table.signature(dims, w.channels, m.layout)
+    assert sig >= 0
+    d = w.to("cuda")
+    ptr = csr_row_ptr(d.receiver, w.num_nodes)
+    order = locality_order(d.sender, ptr, w.num_nodes, 2)
+    lib = _lib.load()
+    p = _lib.ConvParams(num_nodes=w.num_nodes, num_edges=w.num_edges, num_coef=table.num_coef, num_x=dims[0],
+                        num_y=dims[1], num_out=dims[2], num_scalars=dims[3], channels=w.channels,
+                        layout=m.layout.value, val_dtype=code, coef_idx_bytes=table.idx_bytes, signature=sig,
+                        coef_scale=1.0 if f64 else scale, debug=0, y_flip=flip, row_order=order.data_ptr())
+    if f64:
+        p.coef_classes = ctypes.cast(scale, ctypes.c_void_p).value
+    coef = table.device(d.x.device)
+    x, y, s, dm = ((0.25 * t).to(tdtype) for t in (d.x, d.y, d.s, d.dm))
+    out = torch.empty_like(dm)
+    dx, dy, ds = torch.empty_like(x), torch.empty_like(y), torch.empty_like(s)
+
+    def launch(stream):
+        _lib.check(lib.e3j_amd_convolution_fwd(ctypes.byref(p), coef.data_ptr(), x.data_ptr(), y.data_ptr(),
+                                               s.data_ptr(), d.sender.data_ptr(), ptr.data_ptr(), None,
+                                               out.data_ptr(), stream))
+        _lib.check(lib.e3j_amd_convolution_bwd_receiver(
+            ctypes.byref(p), coef.data_ptr(), x.data_ptr(), y.data_ptr(), s.data_ptr(), dm.data_ptr(),
+            d.sender.data_ptr(), ptr.data_ptr(), None, dx.data_ptr(), dy.data_ptr(), ds.data_ptr(), stream))
+
+    side = torch.cuda.Stream()
+    side.wait_stream(torch.cuda.current_stream())
+    with torch.cuda.stream(side):
+        launch(side.cuda_stream)
+    torch.cuda.current_stream().wait_stream(side)
+    torch.cuda.synchronize()
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph, stream=side):
+        launch(side.cuda_stream)
+    if f64:
+        p.coef_classes = None   # the recorded launches hold their own copy of the classes
+    for trial in range(3):
+        gen = torch.Generator(device="cuda").manual_seed(200 + trial)
+        for t in (x, y, s, dm):
+            t.copy_(0.25 * torch.randn(t.shape, device="cuda", generator=gen))
+        (x.float().sum() + s.float().sum()).item()
+        graph.replay()
+        torch.cuda.synchronize()
+        replayed = [t.clone() for t in (out, dx, dy, ds)]
+        if f64:
+            p.coef_classes = ctypes.cast(scale, ctypes.c_void_p).value
+        launch(torch.cuda.current_stream().cuda_stream)
+        torch.cuda.synchronize()
+        if f64:
+            p.coef_classes = None
+        assert torch.equal(replayed[0], out) and torch.equal(replayed[3], ds), trial
+        tol = 1e-12 if f64 else 2e-2
+        for a, b in ((replayed[1], dx), (replayed[2], dy)):       # atomics: equal up to summation order
+            assert float((a.double() - b.double()).abs().max()) <= tol * float(b.double().abs().max()) + 1e-30, trial
