@@ -591,8 +591,9 @@ int e3j_amd_find_signature(const void *coef_host, int32_t coef_idx_bytes, int32_
                 else std::memcpy(&entries[n].idx[t], bytes + n * item + 4 + 4 * t, 4);
             }
         }
+        // (an entry and the entry the factor is taken from are each off by up to 2^-11: 2^-10 between them)
         return match_signature(entries, num_x, num_y, num_out, num_scalars, channels, layout, coef_scale, y_flip,
-                               1.0 / 1024.0, true);
+                               1.5 / 1024.0, true);
     }
     const std::vector<TableEntry> entries = unpack_entries(coef_host, coef_idx_bytes, num_coef, false);
     return match_signature(entries, num_x, num_y, num_out, num_scalars, channels, layout, coef_scale, y_flip);

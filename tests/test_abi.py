@@ -403,3 +403,27 @@ def test_float64_look_up_refuses_tables_of_another_structure():
     whole_component = val.copy()
     whole_component[members] *= -1.0
     assert find(whole_component)[2] == 1 << int(k0)
+
+
+@pytest.mark.parametrize("avg", [None, 4.0, 12.5, 30.0, 7.3])
+def test_half_valued_tables_resolve_to_their_signature(avg):
+    """A table of half values (the built-in table times a factor, every entry rounded to half on its
+    own) is found among the signatures that have float16 kernels, with the factor."""
+    lib = _lib.load()
+    m = Convolution(("0e+1o+2e+3o", "0e+1o+2e+3o"), "0e+1o+2e+3o", graph_ordering="RECEIVER", avg_num_neighbors=avg)
+    packed = m._packed_coef("float16")
+    scale, flip = C.c_float(), C.c_uint32()
+    for channels, found in ((64, True), (128, True), (32, False)):
+        sig = lib.e3j_amd_find_signature(packed.ctypes.data, 1, _lib.F16, packed.shape[0], 16, 16, 99, 23, channels, 1,
+                                         C.byref(scale), C.byref(flip))
+        assert (sig >= 0) == found
+        if found:
+            assert abs(scale.value * (avg or 1.0) - 1.0) < 2e-3 and flip.value == 0
+    # the same values with one entry off by a percent are another table
+    from e3j_amd.coef import Coef4D
+    c = Coef4D.unpack(packed, np.float16)
+    val = np.asarray(c.val).copy()
+    val[3] *= np.float16(1.01)
+    other = Coef4D(val, c.idx, val_dtype=np.float16, idx_dtype=c.idx_dtype).pack()
+    assert lib.e3j_amd_find_signature(other.ctypes.data, 1, _lib.F16, other.shape[0], 16, 16, 99, 23, 128, 1,
+                                      C.byref(scale), C.byref(flip)) == -1
