@@ -576,25 +576,9 @@ int e3j_amd_find_signature(const void *coef_host, int32_t coef_idx_bytes, int32_
     if (y_flip) *y_flip = 0;
     if (coef_host == nullptr || (val_dtype != E3J_AMD_F32 && val_dtype != E3J_AMD_F16) || num_coef <= 0) return -1;
     if (coef_idx_bytes != 1 && coef_idx_bytes != 4) return -1;
-    if (val_dtype == E3J_AMD_F16) {
-        // a table of half values: every entry within half rounding (2^-11) of the built-in table times one
-        // factor; the float16 kernels then compute with the built-in float values
-        const size_t item = coef_idx_bytes == 1 ? sizeof(Coef4D<uint8_t, half_t>) : sizeof(Coef4D<int32_t, half_t>);
-        const unsigned char *bytes = static_cast<const unsigned char *>(coef_host);
-        std::vector<TableEntry> entries((size_t)num_coef);
-        for (int n = 0; n < num_coef; n++) {
-            half_t h;
-            std::memcpy(&h, bytes + n * item, sizeof(h));
-            entries[n].val = (float)h;
-            for (int t = 0; t < 4; t++) {
-                if (coef_idx_bytes == 1) entries[n].idx[t] = bytes[n * item + 2 + t];
-                else std::memcpy(&entries[n].idx[t], bytes + n * item + 4 + 4 * t, 4);
-            }
-        }
-        // (an entry and the entry the factor is taken from are each off by up to 2^-11: 2^-10 between them)
-        return match_signature(entries, num_x, num_y, num_out, num_scalars, channels, layout, coef_scale, y_flip,
-                               1.5 / 1024.0, true);
-    }
+    if (val_dtype == E3J_AMD_F16)
+        return match_signature_f16(coef_host, coef_idx_bytes, num_coef, num_x, num_y, num_out, num_scalars, channels,
+                                   layout, false, coef_scale, y_flip);
     const std::vector<TableEntry> entries = unpack_entries(coef_host, coef_idx_bytes, num_coef, false);
     return match_signature(entries, num_x, num_y, num_out, num_scalars, channels, layout, coef_scale, y_flip);
 }
@@ -602,6 +586,40 @@ int e3j_amd_find_signature(const void *coef_host, int32_t coef_idx_bytes, int32_
 int e3j_amd_find_signature_f64(const void *coef_host, int32_t coef_idx_bytes, int32_t num_coef,
                                int32_t num_x, int32_t num_y, int32_t num_out, int32_t num_scalars,
                                int32_t channels, int32_t layout, double *coef_classes, uint32_t *y_flip) {
+    return match_signature_f64(coef_host, coef_idx_bytes, num_coef, num_x, num_y, num_out, num_scalars, channels,
+                               layout, false, coef_classes, y_flip);
+}
+
+}  // extern "C"
+
+namespace e3j_amd {
+
+int match_signature_f16(const void *coef_host, int32_t coef_idx_bytes, int32_t num_coef, int32_t num_x,
+                        int32_t num_y, int32_t num_out, int32_t num_scalars, int32_t channels, int32_t layout,
+                        bool columns_ji, float *coef_scale, uint32_t *y_flip) {
+    // a table of half values: every entry within half rounding (2^-11) of the built-in table times one
+    // factor; the float16 kernels then compute with the built-in float values
+    const size_t item = coef_idx_bytes == 1 ? sizeof(Coef4D<uint8_t, half_t>) : sizeof(Coef4D<int32_t, half_t>);
+    const unsigned char *bytes = static_cast<const unsigned char *>(coef_host);
+    std::vector<TableEntry> entries((size_t)num_coef);
+    for (int n = 0; n < num_coef; n++) {
+        half_t h;
+        std::memcpy(&h, bytes + n * item, sizeof(h));
+        entries[n].val = (float)h;
+        for (int t = 0; t < 4; t++) {
+            if (coef_idx_bytes == 1) entries[n].idx[t] = bytes[n * item + 2 + t];
+            else std::memcpy(&entries[n].idx[t], bytes + n * item + 4 + 4 * t, 4);
+        }
+        if (columns_ji) std::swap(entries[n].idx[0], entries[n].idx[1]);  // (j, i, k, l) of a dx table -> (i, j, k, l)
+    }
+    // (an entry and the entry the factor is taken from are each off by up to 2^-11: 2^-10 between them)
+    return match_signature(entries, num_x, num_y, num_out, num_scalars, channels, layout, coef_scale, y_flip,
+                           1.5 / 1024.0, true);
+}
+
+int match_signature_f64(const void *coef_host, int32_t coef_idx_bytes, int32_t num_coef, int32_t num_x,
+                        int32_t num_y, int32_t num_out, int32_t num_scalars, int32_t channels, int32_t layout,
+                        bool columns_ji, double *coef_classes, uint32_t *y_flip) {
     if (y_flip) *y_flip = 0;
     if (coef_host == nullptr || coef_classes == nullptr || num_coef <= 0) return -1;
     if (coef_idx_bytes != 1 && coef_idx_bytes != 4) return -1;
@@ -624,6 +642,7 @@ int e3j_amd_find_signature_f64(const void *coef_host, int32_t coef_idx_bytes, in
             if (coef_idx_bytes == 1) given[n].idx[t] = bytes[n * item + 8 + t];
             else std::memcpy(&given[n].idx[t], bytes + n * item + 8 + 4 * t, 4);
         }
+        if (columns_ji) std::swap(given[n].idx[0], given[n].idx[1]);  // (j, i, k, l) of a dx table -> (i, j, k, l)
     }
     std::stable_sort(given.begin(), given.end(), less);
     const bool signs_allowed = y_flip != nullptr && num_y <= 32;
@@ -679,4 +698,4 @@ int e3j_amd_find_signature_f64(const void *coef_host, int32_t coef_idx_bytes, in
     return -1;
 }
 
-}  // extern "C"
+}  // namespace e3j_amd

@@ -217,6 +217,14 @@ std::vector<TableEntry> unpack_entries(const void *packed_host, int32_t coef_idx
 int match_signature(std::vector<TableEntry> entries, int32_t num_x, int32_t num_y, int32_t num_out,
                     int32_t num_scalars, int32_t channels, int32_t layout, float *coef_scale,
                     uint32_t *y_flip, double tolerance = 4e-7, bool float16_kernels = false);
+// the same for tables of half values (float16 kernels) and of double values (float64 kernels: the
+// table's own magnitudes per class of the signature's entries into coef_classes[kF64Classes])
+int match_signature_f16(const void *coef_host, int32_t coef_idx_bytes, int32_t num_coef, int32_t num_x,
+                        int32_t num_y, int32_t num_out, int32_t num_scalars, int32_t channels, int32_t layout,
+                        bool columns_ji, float *coef_scale, uint32_t *y_flip);
+int match_signature_f64(const void *coef_host, int32_t coef_idx_bytes, int32_t num_coef, int32_t num_x,
+                        int32_t num_y, int32_t num_out, int32_t num_scalars, int32_t channels, int32_t layout,
+                        bool columns_ji, double *coef_classes, uint32_t *y_flip);
 int num_builtin_signatures();
 const Signature &builtin_signature(int id);
 int num_signatures();

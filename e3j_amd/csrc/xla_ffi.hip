@@ -138,8 +138,8 @@ class TableResolver {
         ResolvedTable none;
         const bool f64 = p.val_dtype == E3J_AMD_F64, f16 = p.val_dtype == E3J_AMD_F16;
         if (num_coef <= 0 || device_table == nullptr) return none;
-        // (the float64 and float16 kernels serve receiver rows in the trailing layout: the forward table only)
-        if ((f64 || f16) && (columns_ji || p.layout != E3J_AMD_LAYOUT_TRAILING)) return none;
+        // (the float64 and float16 kernels serve the trailing layout)
+        if ((f64 || f16) && p.layout != E3J_AMD_LAYOUT_TRAILING) return none;
         const size_t item = f64   ? (idx_bytes == 1 ? sizeof(Coef4D<uint8_t, double>) : sizeof(Coef4D<int32_t, double>))
                             : f16 ? (idx_bytes == 1 ? sizeof(Coef4D<uint8_t, half_t>) : sizeof(Coef4D<int32_t, half_t>))
                                   : (idx_bytes == 1 ? sizeof(Coef4D<uint8_t, float>) : sizeof(Coef4D<int32_t, float>));
@@ -183,14 +183,14 @@ class TableResolver {
         ResolvedTable entry;
         if (f64) {
             auto classes = std::make_shared<F64Coefs>();
-            entry.signature = e3j_amd_find_signature_f64(key.second.data(), idx_bytes, num_coef, p.num_x, p.num_y,
-                                                         p.num_out, p.num_scalars, p.channels, p.layout, classes->v,
-                                                         &entry.flip);
+            entry.signature = match_signature_f64(key.second.data(), idx_bytes, num_coef, p.num_x, p.num_y, p.num_out,
+                                                  p.num_scalars, p.channels, p.layout, columns_ji, classes->v,
+                                                  &entry.flip);
             entry.classes = std::move(classes);
         } else if (f16) {
-            entry.signature = e3j_amd_find_signature(key.second.data(), idx_bytes, E3J_AMD_F16, num_coef, p.num_x,
-                                                     p.num_y, p.num_out, p.num_scalars, p.channels, p.layout,
-                                                     &entry.scale, &entry.flip);
+            entry.signature = match_signature_f16(key.second.data(), idx_bytes, num_coef, p.num_x, p.num_y, p.num_out,
+                                                  p.num_scalars, p.channels, p.layout, columns_ji, &entry.scale,
+                                                  &entry.flip);
         } else {
             const std::vector<TableEntry> entries = unpack_entries(key.second.data(), idx_bytes, num_coef, columns_ji);
             entry.signature = match_signature(entries, p.num_x, p.num_y, p.num_out, p.num_scalars, p.channels,
@@ -461,11 +461,6 @@ void *backward_handler(XlaCallFrame *f, Backward mode) {
     d.p.num_coef = (int32_t)(count(coef) / numel / (stacked ? 3 : 1));
     const int32_t *perm_ptr = count(perm) ? static_cast<const int32_t *>(perm->data) : nullptr;
     if (void *err = choose_kernels(f, op, coef, stacked != 0, &d, d.stream)) return err;
-    if (mode == Backward::kSenderRows && d.p.val_dtype != E3J_AMD_F32) {
-        // the float64 and float16 unrolled kernels walk receiver rows only: sender rows stay table-driven
-        d.p.signature = -1;
-        d.p.y_flip = 0;
-    }
     // The reference's operands: the adjacency grouped by sender.  The unrolled kernels of that
     // grouping (trailing layout; a row owns its dx) pay a gather of dm rows per edge: faster than
     // a rebuild of the receiver rows (a dozen small launches) plus the receiver-grouped kernel on
@@ -473,12 +468,20 @@ void *backward_handler(XlaCallFrame *f, Backward mode) {
     // 0.44 ms), slower above (960k edges, 64 channels: 4.07 against 3.62 + 0.2 ms).  Large graphs
     // therefore get their receiver CSR rebuilt in scratch memory of the runtime; without such
     // memory run_backward keeps the sender rows (unrolled in the trailing layout, else table-driven).
-    const bool small_graph = d.p.layout == E3J_AMD_LAYOUT_TRAILING && d.p.num_edges < (1 << 18);
+    // (the sender-grouped unrolled kernels are float32 kernels: other dtypes always go by receiver rows)
+    const bool small_graph = d.p.layout == E3J_AMD_LAYOUT_TRAILING && d.p.num_edges < (1 << 18) &&
+                             d.p.val_dtype == E3J_AMD_F32;
     if (mode == Backward::kSenderRows && d.p.signature >= 0 && !small_graph) {
         bool done = false;
         void *err = backward_on_receiver_rows(f, op, &d, coef, stacked != 0, x, y, s, dm, other, row_ptr, perm_ptr,
                                               dx, dy, ds, &done);
         if (err != nullptr || done) return err;
+    }
+    if (mode == Backward::kSenderRows && d.p.val_dtype != E3J_AMD_F32) {
+        // no scratch to rebuild receiver rows in, and the float64 / float16 unrolled kernels walk
+        // receiver rows only: the sender rows stay with the table-driven kernel
+        d.p.signature = -1;
+        d.p.y_flip = 0;
     }
     if (ordered) {
         // the scratch of the atomic-free backward travels as a fourth result buffer (any dtype)

@@ -221,3 +221,23 @@ def test_float16_frames_of_the_ffi_targets_run_the_float16_kernels():
     mgs = O.convolution_vjp(idx, np.abs(val), mix, *mags, np.abs(host["dm"]), dtype=np.float64)
     for g, r, mg, what, sums in zip((dx, dy, ds), refs, mgs, ("dx", "dy", "ds"), (4.0, 2.0, 1.0)):
         assert_parity16(g, r, mg, what, sums)
+    # the reference's own backward frame: the three transposed tables stacked, the adjacency grouped by
+    # sender.  The handler finds the signature through the dx-transposed table, rebuilds receiver rows in
+    # scratch of the runtime and runs the float16 unrolled kernels on them.
+    from e3j_amd.coef import Coef4D
+    c = Coef4D.unpack(coef, np.float16)
+    stacked = np.stack([c.transpose(a).pack() for a in ((1, 0, 2, 3), (2, 0, 1, 3), (3, 0, 2, 1))])
+    perm_t, recv_t, sptr = O.transpose_graph(host["sender"], host["receiver"], n)
+    xla.allocate = lambda nbytes: torch.empty(nbytes, dtype=torch.uint8, device="cuda")
+    before = xla.allocations
+    dx2, dy2, ds2 = (torch.full_like(d[f], float("nan")) for f in ("x", "y", "s"))
+    stacked_d = torch.from_numpy(stacked.copy()).cuda()
+    ref_bwd = xla.frame([buf(stacked_d, U8), buf(d["x"], F16), buf(d["y"], F16), buf(d["s"], F16), buf(d["dm"], F16),
+                         buf(torch.as_tensor(recv_t.astype(np.int32)).cuda(), S32), buf(torch.as_tensor(sptr).cuda(), S32),
+                         buf(torch.as_tensor(perm_t.astype(np.int32)).cuda(), S32)],
+                        [buf(dx2, F16), buf(dy2, F16), buf(ds2, F16)], attrs())
+    assert lib.e3j_amd_xla_convolution_bwd(C.addressof(ref_bwd)) is None, xla.errors
+    torch.cuda.synchronize()
+    assert xla.allocations == before + 1, "the unrolled kernels run on receiver rows rebuilt in the runtime's scratch"
+    for g, r, mg, what, sums in zip((dx2, dy2, ds2), refs, mgs, ("dx", "dy", "ds"), (4.0, 2.0, 1.0)):
+        assert_parity16(g, r, mg, "reference frame " + what, sums)
