@@ -7,9 +7,10 @@
 // matrix M[i][j] = sum_k c_ijk * y[k].  A wave builds M once per edge in its strip of LDS (the
 // lanes share the table's non-empty cells), and then every lane (one channel) runs loops over
 // i and j whose bounds are compile-time numbers, so that x, the accumulators and the partial
-// sums sit in registers under constant indices; M is read as wave-uniform 16-byte LDS
-// broadcasts.  What depends on the table is data: the plan, built on the device by one
-// workgroup per call (no read-back, no compiler at run time):
+// sums sit in registers under constant indices; M is read four numbers to a 4-byte LDS read
+// (lane t takes number t % 4) and used through DPP operands.  What depends on the table is data:
+// the plan, built on the device by one workgroup per call (no read-back, no compiler at run
+// time):
 //   * the output coordinates in the order the loops visit them ("slots": sorted by the x
 //     coordinates their path touches, then by scalar, so that rows of one scalar are adjacent
 //     and blocks of 16 slots touch few groups of 4 x coordinates),
@@ -17,13 +18,16 @@
 //     inside those a bit per half of 8 slots: the loops skip the others with wave-uniform branches,
 //   * the non-empty cells (slot, j) with their (coefficient, k) lists in table order.
 // The backward pass (lib/e3j_ops/cuda/convolution/bwd.cuh:116-321) uses the same M: ds from the
-// forward's partial sums, dx[j] += M[i][j] * s[l(i)] * dm[i], and for dy the per-channel products
-// x[j] * s * dm[i] of a block of 64 cells are summed over the 64 channels with a transposing
-// butterfly (lane t ends with the total of cell t), multiplied with the cell's coefficients and
-// added into the wave's dy row in LDS.  Per edge a wave first copies the edge's scalar rows into its
-// LDS strip (the loops read them by the slot's scalar, a number of the plan) and gathers the x row
-// into registers; the table part of the plan sits in the workgroup's LDS, the per-slot numbers in
-// two vector registers of every wave that are read lane by lane.
+// forward's partial sums, dx[j] += M[i][j] * s[l(i)] * dm[i], and for dy the channel sums of the
+// products x[j] * (s * dm[i]) of a block of 16 slots, 16 x 16 cells, come from 16 matrix
+// instructions whose summed index is the channel (operands moved through a tile of LDS); a lane per
+// entry of the block then multiplies its cell's total with the coefficient and adds it into the
+// wave's dy row in LDS.  Per edge a wave issues the loads of the edge's operands (the x row, the
+// scalar rows, the first block of dm) together, builds M under them, and copies the scalar rows
+// into its LDS strip (the loops read them by the slot's scalar, a number of the plan); the next
+// edge's index, position and y are fetched one edge ahead.  The table part of the plan sits in the
+// workgroup's LDS, the per-slot numbers in two vector registers of every wave that are read lane by
+// lane.
 //
 // Tables the plan cannot take (an output coordinate with two different scalars, sizes beyond the
 // limits) run the kernels of conv_generic.hip: eligibility is a flag in the plan that both
@@ -64,10 +68,12 @@ __device__ __forceinline__ bool half_live(unsigned mask0, unsigned mask1, int b,
 struct PlanLayout {  // offsets in 32-bit words
     // slot_row, slot_l: output coordinate and scalar of a slot; first, count: the entries of a dense
     // cell (slot * 16 + j); cells: the non-empty cells packed as cell | first << 11 | count << 22;
-    // pairs: (coefficient bits, k) of the entries, cell by cell; coef, k, t, cell_list: working arrays
+    // pairs: (coefficient bits, k | cell within its block of 16 slots << 8) of the entries, cell by cell; coef, k, t, cell_list: working arrays
     // of the builder; zero_l: scalars no entry uses
     // slot_lw: 64 * scalar of the slot (the word offset of its row in a wave's LDS copy of s), 0 if none
-    int slot_row, slot_l, slot_lw, first, count, cell_list, cells, pairs, coef, k, t, zero_l, words;
+    // block_first: the first entry of each block of 16 slots in `pairs` (the entries of a block are
+    // adjacent: cells are numbered slot by slot), and the number of entries behind the last block
+    int slot_row, slot_l, slot_lw, first, count, cell_list, cells, pairs, coef, k, t, zero_l, block_first, words;
     PlanLayout(int num_coef, int num_scalars) {
         int at = kHeaderWords;
         auto take = [&](int n) { const int here = at; at += (n + 3) / 4 * 4; return here; };
@@ -76,6 +82,7 @@ struct PlanLayout {  // offsets in 32-bit words
         pairs = take(2 * num_coef);
         coef = take(num_coef); k = take(num_coef); t = take(num_coef);
         zero_l = take(num_scalars);
+        block_first = take(kSlots / 16 + 1);
         words = at;
     }
 };
@@ -197,7 +204,7 @@ __global__ __launch_bounds__(kBuildThreads) void plan_build_kernel(
         const int cell = slot_of_row[i] * kPlanX + j;
         const int at = plan[L.first + cell] + atomicAdd(&plan[L.count + cell], 1);
         plan[L.coef + at] = __float_as_int((float)coef[n].val);
-        plan[L.k + at] = k;
+        plan[L.k + at] = k | ((cell % (16 * kPlanX)) << 8);
         plan[L.t + at] = n;
     }
     __syncthreads();
@@ -231,6 +238,7 @@ __global__ __launch_bounds__(kBuildThreads) void plan_build_kernel(
         plan[L.pairs + 2 * n] = plan[L.coef + n];
         plan[L.pairs + 2 * n + 1] = plan[L.k + n];
     }
+    if (tid <= kSlots / 16) plan[L.block_first + tid] = tid < kSlots / 16 ? plan[L.first + tid * 16 * kPlanX] : num_coef;
     if (tid == 0) {
         plan[kEligible] = eligible; plan[kNumCells] = num_cells; plan[kChunkMask] = chunk_mask;
         plan[kNumZeroL] = num_zero_l; plan[kMaxRun] = max_run;
@@ -245,22 +253,29 @@ __device__ __forceinline__ void wave_lds_sync() {
     __builtin_amdgcn_wave_barrier();
 }
 
-typedef float f32x4 __attribute__((ext_vector_type(4)));
+// acc += (m of lane K of the lane's group of four lanes) * v, one instruction (a DPP operand).  The
+// loops read four wave-uniform numbers of M with one 4-byte LDS read (lane t takes number t % 4)
+// instead of a 16-byte broadcast to every lane: a quarter of the LDS return traffic.  (m comes
+// from an LDS read, never from a vector instruction just before: no wait states are owed.)
+// Keeps the eight reads before it together (the values are all in registers here): without it the
+// compiler moves each read next to its use and pays an LDS round trip per pair of values.
+__device__ __forceinline__ void together(float (&m)[8]) {
+    asm volatile("" : "+v"(m[0]), "+v"(m[1]), "+v"(m[2]), "+v"(m[3]), "+v"(m[4]), "+v"(m[5]), "+v"(m[6]), "+v"(m[7]));
+}
+template <int K>
+__device__ __forceinline__ void fma_quad(float &acc, float m, float v) {
+    asm("v_fmac_f32_dpp %0, %1, %2 quad_perm:[%3,%3,%3,%3] row_mask:0xf bank_mask:0xf"
+        : "+v"(acc) : "v"(m), "v"(v), "n"(K));
+}
 
 // The table part of the plan in LDS, shared by the waves of a workgroup: the packed cells, then
 // (coefficient, k) pairs.  Every thread of the workgroup calls this (it holds a barrier).
-// `dense` (backward): first | count << 11 of the first `dense_cells` dense cells behind them.
 __device__ __forceinline__ void stage_table(const int32_t *__restrict__ plan, const PlanLayout &L, int num_cells,
-                                            int num_coef, int32_t *tab, int dense_cells = 0) {
+                                            int num_coef, int32_t *tab) {
     const int tid = threadIdx.y * kWave + threadIdx.x, threads = blockDim.y * kWave;
     const int pairs = (num_cells + 1) & ~1;  // the pairs start at an even word
     for (int t = tid; t < num_cells; t += threads) tab[t] = plan[L.cells + t];
     for (int t = tid; t < 2 * num_coef; t += threads) tab[pairs + t] = plan[L.pairs + t];
-    int32_t *dense = tab + table_words(num_coef);
-    for (int t = tid; t < dense_cells; t += threads) {
-        const int cnt = plan[L.count + t];  // (an empty cell behind the last entry has first = 2048: dropped)
-        dense[t] = cnt > 0 ? plan[L.first + t] | (cnt << 11) : 0;
-    }
     __syncthreads();
 }
 
@@ -278,7 +293,7 @@ __device__ __forceinline__ void build_edge_matrix(const int32_t *tab, int num_ce
         float sum = 0.f;
         for (int r = 0; r < most; r++) {
             const int at = r < cnt ? first + r : first;
-            const int kk = tab[pairs + 2 * at + 1];
+            const int kk = tab[pairs + 2 * at + 1] & 255;
             const float cf = r < cnt ? __int_as_float(tab[pairs + 2 * at]) : 0.f;
             sum += cf * __shfl(yreg, kk, kWave);
         }
@@ -313,7 +328,7 @@ __device__ __forceinline__ void build_edge_matrix(const int32_t *tab, const Held
             if (it * kWave >= num_cells) break;  // (wave-uniform)
             const int first = (int)((held.w[it] >> 11) & 2047u), cnt = (int)(held.w[it] >> 22);
             const int at = r < cnt ? first + r : first;
-            const int kk = tab[pairs + 2 * at + 1];
+            const int kk = tab[pairs + 2 * at + 1] & 255;
             const float cf = r < cnt ? __int_as_float(tab[pairs + 2 * at]) : 0.f;
             sum[it] += cf * __shfl(yreg, kk, kWave);
         }
@@ -335,7 +350,7 @@ __device__ __forceinline__ void build_edge_matrix(const int32_t *tab, const Held
         float one = 0.f;
         for (int r = 0; r < most; r++) {
             const int at = r < cnt ? first + r : first;
-            const int kk = tab[pairs + 2 * at + 1];
+            const int kk = tab[pairs + 2 * at + 1] & 255;
             const float cf = r < cnt ? __int_as_float(tab[pairs + 2 * at]) : 0.f;
             one += cf * __shfl(yreg, kk, kWave);
         }
@@ -361,10 +376,6 @@ struct SlotWords {
 // know that a vector load of a wave-uniform address gives a wave-uniform value).
 __device__ __forceinline__ int uni(int v) { return __builtin_amdgcn_readfirstlane(v); }
 
-__device__ __forceinline__ int next_live(const int32_t *__restrict__ other, int e, int e1, int num_nodes) {
-    while (e < e1 && (unsigned)uni(other[e]) >= (unsigned)num_nodes) e++;  // padding edges are stepped over
-    return e;
-}
 
 // Rows of an operand behind a wave-uniform base: the lanes keep one 32-bit byte offset that
 // moves from row to row by the row stride, so that a load takes a scalar base, one offset
@@ -380,7 +391,7 @@ struct RowCursor {
         : base(reinterpret_cast<const char *>(row0)), at((unsigned)sizeof(Val) * lane_elems),
           step((unsigned)sizeof(Val) * stride_elems) {}
     __device__ __forceinline__ float row(unsigned r) const {  // r wave-uniform
-        return (float)*reinterpret_cast<const Val *>(base + (at + r * step));
+        return (float)*reinterpret_cast<const Val *>((base + (size_t)r * step) + at);
     }
 };
 // the lane's element of row r of an output operand (same addressing)
@@ -390,19 +401,63 @@ __device__ __forceinline__ Val *element_at(Val *row0, unsigned lane_elems, unsig
                                    (unsigned)sizeof(Val) * (lane_elems + r * stride_elems));
 }
 
-// The scalar rows of one edge into the wave's LDS copy, eight loads in flight.
+// The scalar rows of one edge on their way into the wave's LDS copy: the loads of 24 rows are issued
+// together with the edge's other loads, and the values are written to LDS once the edge's matrix is
+// built (the matrix needs LDS only, so it is built while the loads are in flight).  Rows past 24
+// follow in groups of eight.
+constexpr int kRowsAhead = 24;
 template <typename Val>
-__device__ __forceinline__ void stage_scalars(const Val *srow0, unsigned soff, unsigned sdim, int S, float *sbuf,
-                                              int lane) {
-    const RowCursor<Val> cur(srow0, soff, sdim);
-    for (int t0 = 0; t0 < S; t0 += 8) {
-        float v[8];
+struct ScalarRows {
+    float v[kRowsAhead];
+    __device__ __forceinline__ void load(const RowCursor<Val> &cur, int S) {
 #pragma unroll
-        for (int t = 0; t < 8; t++) v[t] = cur.row((unsigned)(t0 + t < S ? t0 + t : S - 1));  // (clamped: straight-line)
+        for (int t = 0; t < 8; t++) v[t] = cur.row((unsigned)(t < S ? t : S - 1));  // (clamped: straight-line)
+        if (S > 8) {
 #pragma unroll
-        for (int t = 0; t < 8; t++) sbuf[(t0 + t < S ? t0 + t : S - 1) * kWave + lane] = v[t];
+            for (int t = 8; t < 16; t++) v[t] = cur.row((unsigned)(t < S ? t : S - 1));
+        }
+        if (S > 16) {
+#pragma unroll
+            for (int t = 16; t < kRowsAhead; t++) v[t] = cur.row((unsigned)(t < S ? t : S - 1));
+        }
     }
-}
+    __device__ __forceinline__ void store(const RowCursor<Val> &cur, int S, float *sbuf, int lane) const {
+#pragma unroll
+        for (int t = 0; t < 8; t++) sbuf[(t < S ? t : S - 1) * kWave + lane] = v[t];
+        if (S > 8) {
+#pragma unroll
+            for (int t = 8; t < 16; t++) sbuf[(t < S ? t : S - 1) * kWave + lane] = v[t];
+        }
+        if (S > 16) {
+#pragma unroll
+            for (int t = 16; t < kRowsAhead; t++) sbuf[(t < S ? t : S - 1) * kWave + lane] = v[t];
+        }
+        for (int t0 = kRowsAhead; t0 < S; t0 += 8) {
+            float w[8];
+#pragma unroll
+            for (int t = 0; t < 8; t++) w[t] = cur.row((unsigned)(t0 + t < S ? t0 + t : S - 1));
+#pragma unroll
+            for (int t = 0; t < 8; t++) sbuf[(t0 + t < S ? t0 + t : S - 1) * kWave + lane] = w[t];
+        }
+    }
+};
+
+// The edge a wave works on, fetched one edge ahead of its use: the other end, the position of the
+// edge's operands and the wave's copy of y (lane k holds y[k]).
+struct EdgeAhead {
+    int other;
+    int64_t at;
+    float y;
+    template <typename Val>
+    __device__ __forceinline__ static EdgeAhead fetch(const int32_t *__restrict__ other, const int32_t *__restrict__ perm,
+                                                      const Val *__restrict__ y, int num_y, int e, int lane) {
+        EdgeAhead a;
+        a.other = uni(other[e]);
+        a.at = perm ? (int64_t)uni(perm[e]) : (int64_t)e;
+        a.y = lane < num_y ? (float)y[a.at * num_y + lane] : 0.f;
+        return a;
+    }
+};
 
 // Forward: a wave takes (row, 64 channels) and holds NB * 16 accumulators.
 template <typename Val, int NB, int XG>
@@ -439,23 +494,30 @@ __global__ __launch_bounds__(256, 2) void planned_fwd_kernel(
 #pragma unroll
     for (int t = 0; t < NB * 16; t++) acc[t] = 0.f;
 
-    const int e1 = uni(row_ptr[r + 1]);
-    for (int e = next_live(other, uni(row_ptr[r]), e1, num_nodes); e < e1; e = next_live(other, e + 1, e1, num_nodes)) {
-        const int snd = uni(other[e]);
-        const int64_t ee = perm ? (int64_t)uni(perm[e]) : (int64_t)e;
-        const float yreg = lane < num_y ? (float)y[ee * num_y + lane] : 0.f;
-        wave_lds_sync();  // the reads of the edge before are behind the writes below
-        stage_scalars(s + ee * ls.row, soff, (unsigned)ls.dim, S, sbuf, lane);
+    const int e0 = uni(row_ptr[r]), e1 = uni(row_ptr[r + 1]);
+    EdgeAhead next = {0, 0, 0.f};
+    if (e0 < e1) next = EdgeAhead::fetch(other, perm, y, num_y, e0, lane);
+    for (int e = e0; e < e1; e++) {
+        const EdgeAhead edge = next;
+        // this edge's loads, its matrix built under them (LDS only), then the next edge's numbers
+        const bool live = (unsigned)edge.other < (unsigned)num_nodes;  // (wave-uniform) padding edges are stepped over
+        const RowCursor<Val> sc(s + edge.at * ls.row, soff, (unsigned)ls.dim);
+        ScalarRows<Val> rows;
         float xv[XG * 4];
-        {
-            const RowCursor<Val> xc(x + (int64_t)snd * lx.row, xoff, (unsigned)lx.dim);
+        if (live) {
+            const RowCursor<Val> xc(x + (int64_t)edge.other * lx.row, xoff, (unsigned)lx.dim);
 #pragma unroll
-            for (int j = 0; j < XG * 4; j++) {
-                xv[j] = xc.row((unsigned)(j < X ? j : X - 1));
-                if (j >= X) xv[j] = 0.f;
-            }
+            for (int j = 0; j < XG * 4; j++) xv[j] = xc.row((unsigned)(j < X ? j : X - 1));
+            rows.load(sc, S);
+            wave_lds_sync();  // the reads of the edge before are behind the writes below
+            build_edge_matrix<XG>(tab, held, num_cells, max_run, edge.y, M, lane);
         }
-        build_edge_matrix<XG>(tab, held, num_cells, max_run, yreg, M, lane);
+        next = EdgeAhead::fetch(other, perm, y, num_y, e + 1 < e1 ? e + 1 : e, lane);
+        if (!live) continue;
+#pragma unroll
+        for (int j = 0; j < XG * 4; j++)
+            if (j >= X) xv[j] = 0.f;
+        rows.store(sc, S, sbuf, lane);
         wave_lds_sync();
 #pragma unroll
         for (int b = 0; b < NB; b++) {
@@ -472,14 +534,17 @@ __global__ __launch_bounds__(256, 2) void planned_fwd_kernel(
 #pragma unroll
                 for (int half = 0; half < 2; half++) {
                     if (!half_live<XG>(half0, half1, b, g, half)) continue;  // eight slots without a coefficient here
+                    float m[8];  // (read together, used together: one LDS round trip per half)
+#pragma unroll
+                    for (int uu = 0; uu < 8; uu++) m[uu] = M[((b * 16 + half * 8 + uu) * XG + g) * 4 + (lane & 3)];
+                    together(m);
 #pragma unroll
                     for (int uu = 0; uu < 8; uu++) {
                         const int u = half * 8 + uu;
-                        const f32x4 m = *reinterpret_cast<const f32x4 *>(&M[((b * 16 + u) * XG + g) * 4]);
-                        T[u] = __builtin_fmaf(m.x, xv[4 * g], T[u]);
-                        T[u] = __builtin_fmaf(m.y, xv[4 * g + 1], T[u]);
-                        T[u] = __builtin_fmaf(m.z, xv[4 * g + 2], T[u]);
-                        T[u] = __builtin_fmaf(m.w, xv[4 * g + 3], T[u]);
+                        fma_quad<0>(T[u], m[uu], xv[4 * g]);
+                        fma_quad<1>(T[u], m[uu], xv[4 * g + 1]);
+                        fma_quad<2>(T[u], m[uu], xv[4 * g + 2]);
+                        fma_quad<3>(T[u], m[uu], xv[4 * g + 3]);
                     }
                 }
             }
@@ -501,38 +566,34 @@ __global__ __launch_bounds__(256, 2) void planned_fwd_kernel(
     }
 }
 
-// The channel sums of 64 per-lane products, left one to a lane: v[t] (t < 32) of one wave is summed
-// over the lanes of each half of the wave with five halving steps (lanes whose bit N is clear keep
-// the lower half of the values and take their partner's partial sums of them; the partners are a
-// row swap for N = 16 and DPP lane permutations inside rows of 16 below that), which leaves the
-// partial sum of v[t % 32] over the lane's half in lane t; two such arrays are then finished with
-// one swap of wave halves, lanes 0..31 getting the totals of the first, 32..63 of the second.
-template <int N, int CTRL>  // N pairs (p, p + N) are left; partner lanes differ in bit N
-__device__ __forceinline__ void transpose_sum_step(float (&v)[32], int lane) {
-    const bool upper = (lane & N) != 0;
+// The channel sums of the per-lane products x[j] * s * dm[i] of a block of 16 slots, all 16 x 16 of
+// them with 16 matrix instructions: a wave writes its 16 values per lane (one row of 64 channels per
+// slot) to a tile of LDS and reads them back with lane t holding slot t % 16 of the channels
+// 16 (t / 16) .. + 15 (four 16-byte reads; rows 68 words apart), which is the first operand of
+// v_mfma_f32_16x16x4_f32 with the channels as the summed index; x of the edge, moved the same way
+// once per edge, is the second.  Lane t then holds, in register r, the total of the cell
+// (slot 4 (t / 16) + r, x coordinate t % 16).
+constexpr int kTileStride = 68;
+constexpr int kTileWords = 16 * kTileStride;
+typedef float f32x4 __attribute__((ext_vector_type(4)));
+struct ChannelOperand {
+    f32x4 q[4];
+    __device__ __forceinline__ void read(const float *tile, int lane) {
 #pragma unroll
-    for (int p = 0; p < N; p++) {
-        const float keep = upper ? v[p + N] : v[p];
-        const float send = upper ? v[p] : v[p + N];
-        v[p] = keep + __int_as_float(__builtin_amdgcn_update_dpp(0, __float_as_int(send), CTRL, 0xf, 0xf, true));
+        for (int n = 0; n < 4; n++)
+            q[n] = *reinterpret_cast<const f32x4 *>(&tile[(lane & 15) * kTileStride + 16 * (lane >> 4) + 4 * n]);
     }
-}
-__device__ __forceinline__ float transpose_sum_half(float (&v)[32], int lane) {
+};
+__device__ __forceinline__ f32x4 channel_sums(const ChannelOperand &a, const ChannelOperand &b) {
+    f32x4 d = {0.f, 0.f, 0.f, 0.f};
 #pragma unroll
-    for (int p = 0; p < 16; p++) {  // rows 1 and 3 of v[p] change places with rows 0 and 2 of v[p + 16]
-        const auto r = __builtin_amdgcn_permlane16_swap(__float_as_uint(v[p]), __float_as_uint(v[p + 16]), false, false);
-        v[p] = __uint_as_float(r[0]) + __uint_as_float(r[1]);
+    for (int n = 0; n < 4; n++) {
+        d = __builtin_amdgcn_mfma_f32_16x16x4f32(a.q[n].x, b.q[n].x, d, 0, 0, 0);
+        d = __builtin_amdgcn_mfma_f32_16x16x4f32(a.q[n].y, b.q[n].y, d, 0, 0, 0);
+        d = __builtin_amdgcn_mfma_f32_16x16x4f32(a.q[n].z, b.q[n].z, d, 0, 0, 0);
+        d = __builtin_amdgcn_mfma_f32_16x16x4f32(a.q[n].w, b.q[n].w, d, 0, 0, 0);
     }
-    transpose_sum_step<8, 0x140>(v, lane);  // row_mirror: lane ^ 15
-    transpose_sum_step<4, 0x141>(v, lane);  // row_half_mirror: lane ^ 7
-    transpose_sum_step<2, 0x4E>(v, lane);   // quad_perm [2, 3, 0, 1]: lane ^ 2
-    transpose_sum_step<1, 0xB1>(v, lane);   // quad_perm [1, 0, 3, 2]: lane ^ 1
-    return v[0];
-}
-// lanes 0..31: first.lower + first.upper, lanes 32..63: second.lower + second.upper
-__device__ __forceinline__ float join_halves(float first, float second) {
-    const auto r = __builtin_amdgcn_permlane32_swap(__float_as_uint(first), __float_as_uint(second), false, false);
-    return __uint_as_float(r[0]) + __uint_as_float(r[1]);
+    return d;
 }
 
 enum DyMode { kDyStore = 0, kDyAdd = 1, kDyAtomic = 2 };
@@ -556,12 +617,12 @@ __global__ __launch_bounds__(256, 2) void planned_bwd_kernel(
     const int max_run = plan[kMaxRun];
     const int num_zero_l = plan[kNumZeroL];
     int32_t *tab = reinterpret_cast<int32_t *>(planned_lds);
-    const int32_t *dense = tab + table_words(num_coef);
-    float *M = planned_lds + table_words(num_coef) + NB * 256 + wave * (kStrip + kPlanMaxY + S * kWave);
+    float *M = planned_lds + table_words(num_coef) + wave * (kStrip + kPlanMaxY + S * kWave + kTileWords);
     float *dyl = M + kStrip;
     float *sbuf = dyl + kPlanMaxY;
+    float *tile = sbuf + S * kWave;
     for (int t = lane; t < kStrip + kPlanMaxY; t += kWave) M[t] = 0.f;
-    stage_table(plan, L, num_cells, num_coef, tab, NB * 256);
+    stage_table(plan, L, num_cells, num_coef, tab);
     const int pairs = (num_cells + 1) & ~1;
     const int64_t item = (int64_t)blockIdx.x * blockDim.y + wave;
     // receiver rows: a wave per (row, 64 channels), dx by float atomics, dy shared between the
@@ -586,39 +647,68 @@ __global__ __launch_bounds__(256, 2) void planned_bwd_kernel(
         float dxa[XG * 4];
 #pragma unroll
         for (int j = 0; j < XG * 4; j++) dxa[j] = 0.f;
-        for (int e = next_live(other, e0, e1, num_nodes); e < e1; e = next_live(other, e + 1, e1, num_nodes)) {
-            const int o = uni(other[e]);
-            const int64_t ee = perm ? (int64_t)uni(perm[e]) : (int64_t)e;
+        EdgeAhead next = {0, 0, 0.f};
+        if (e0 < e1) next = EdgeAhead::fetch(other, perm, y, num_y, e0, lane);
+        for (int e = e0; e < e1; e++) {
+            const EdgeAhead edge = next;
+            const bool live = (unsigned)edge.other < (unsigned)num_nodes;  // (wave-uniform) padding edges are stepped over
+            const int o = edge.other;
+            const int64_t ee = edge.at;
             const int xnode = group_is_receiver ? o : g;
             const int znode = group_is_receiver ? g : o;
-            const float yreg = lane < num_y ? (float)y[ee * num_y + lane] : 0.f;
-            wave_lds_sync();
-            stage_scalars(s + ee * ls.row, soff, (unsigned)ls.dim, S, sbuf, lane);
+            // this edge's loads (x, scalars, the first block of dm), its matrix built under them (LDS
+            // only), then the next edge's numbers
+            const RowCursor<Val> sc(s + ee * ls.row, soff, (unsigned)ls.dim);
+            const RowCursor<Val> zc(dm + (int64_t)(live ? znode : 0) * lo.row, zoff, (unsigned)lo.dim);
+            ScalarRows<Val> rows;
             float xv[XG * 4];
-            {
+            float dz[16], dz_ahead[16];  // dm of the block at hand and of the block after it
+            auto load_dm = [&](int b, float (&to)[16]) {
+#pragma unroll
+                for (int u = 0; u < 16; u++) {
+                    const int row = slot_row[b * 16 + u];  // (-1: none)
+                    to[u] = zc.row((unsigned)(row < 0 ? 0 : row));
+                }
+            };
+            if (live) {
                 const RowCursor<Val> xc(x + (int64_t)xnode * lx.row, xoff, (unsigned)lx.dim);
 #pragma unroll
-                for (int j = 0; j < XG * 4; j++) {
-                    xv[j] = xc.row((unsigned)(j < X ? j : X - 1));
-                    if (j >= X || !active) xv[j] = 0.f;  // (idle lanes add nothing to dy)
-                }
+                for (int j = 0; j < XG * 4; j++) xv[j] = xc.row((unsigned)(j < X ? j : X - 1));
+                rows.load(sc, S);
+                load_dm(0, dz);
+                wave_lds_sync();  // the reads of the edge before are behind the writes below
+                build_edge_matrix<XG>(tab, num_cells, max_run, edge.y, M, lane);
             }
-            build_edge_matrix<XG>(tab, num_cells, max_run, yreg, M, lane);
+            next = EdgeAhead::fetch(other, perm, y, num_y, e + 1 < e1 ? e + 1 : e, lane);
+            if (!live) continue;
+#pragma unroll
+            for (int j = 0; j < XG * 4; j++)
+                if (j >= X || !active) xv[j] = 0.f;  // (idle lanes add nothing to dy)
+            rows.store(sc, S, sbuf, lane);
+#pragma unroll
+            for (int j = 0; j < 16; j++) tile[j * kTileStride + lane] = j < XG * 4 ? xv[j < XG * 4 ? j : 0] : 0.f;
             wave_lds_sync();
-            const RowCursor<Val> zc(dm + (int64_t)znode * lo.row, zoff, (unsigned)lo.dim);
+            ChannelOperand xop;
+            xop.read(tile, lane);
+            wave_lds_sync();  // (the tile is written again below)
             Val *dsrow0 = ds + ee * ls.row;
             const unsigned dsoff = (unsigned)c * (unsigned)ls.chan;
             int cur_l = -1;
             float dsa = 0.f;
 #pragma unroll
             for (int b = 0; b < NB; b++) {
-                if (((chunk_mask >> (b * XG)) & ((1u << XG) - 1u)) == 0) continue;
-                float sd[16], dz[16], T[16];
+                if (b + 1 < NB) load_dm(b + 1, dz_ahead);
+                const int entries0 = uni(plan[L.block_first + b]), entries1 = uni(plan[L.block_first + b + 1]);
+                if (((chunk_mask >> (b * XG)) & ((1u << XG) - 1u)) == 0) {
+#pragma unroll
+                    for (int u = 0; u < 16; u++) dz[u] = dz_ahead[u];
+                    continue;
+                }
+                float sd[16], T[16];
 #pragma unroll
                 for (int u = 0; u < 16; u++) {
-                    const int l = slot_l[b * 16 + u], row = slot_row[b * 16 + u];  // (-1: none)
+                    const int l = slot_l[b * 16 + u];  // (-1: none)
                     const float sv = sbuf[(l < 0 ? 0 : l) * kWave + lane];
-                    dz[u] = zc.row((unsigned)(row < 0 ? 0 : row));
                     if (l < 0) dz[u] = 0.f;
                     sd[u] = sv * dz[u];
                     T[u] = 0.f;
@@ -626,39 +716,48 @@ __global__ __launch_bounds__(256, 2) void planned_bwd_kernel(
 #pragma unroll
                 for (int gx = 0; gx < XG; gx++) {
                     if (!((chunk_mask >> (b * XG + gx)) & 1u)) continue;
-                    // lane t ends with the channel sum of cell (slot 16 b + t / 4, x coordinate 4 gx + t % 4):
-                    // the slots in two halves of eight, the first for lanes 0..31, the second for the rest
-                    float part[2];
 #pragma unroll
                     for (int half = 0; half < 2; half++) {
-                        if (!half_live<XG>(half0, half1, b, gx, half)) {  // eight slots without a coefficient here
-                            part[half] = 0.f;
-                            continue;
-                        }
-                        float G[32];
+                        if (!half_live<XG>(half0, half1, b, gx, half)) continue;  // eight slots without a coefficient here
+                        float m[8];
+#pragma unroll
+                        for (int uu = 0; uu < 8; uu++) m[uu] = M[((b * 16 + half * 8 + uu) * XG + gx) * 4 + (lane & 3)];
+                        together(m);
 #pragma unroll
                         for (int uu = 0; uu < 8; uu++) {
                             const int u = half * 8 + uu;
-                            const f32x4 m = *reinterpret_cast<const f32x4 *>(&M[((b * 16 + u) * XG + gx) * 4]);
-                            T[u] = __builtin_fmaf(m.x, xv[4 * gx], T[u]);
-                            T[u] = __builtin_fmaf(m.y, xv[4 * gx + 1], T[u]);
-                            T[u] = __builtin_fmaf(m.z, xv[4 * gx + 2], T[u]);
-                            T[u] = __builtin_fmaf(m.w, xv[4 * gx + 3], T[u]);
-                            dxa[4 * gx] = __builtin_fmaf(m.x, sd[u], dxa[4 * gx]);
-                            dxa[4 * gx + 1] = __builtin_fmaf(m.y, sd[u], dxa[4 * gx + 1]);
-                            dxa[4 * gx + 2] = __builtin_fmaf(m.z, sd[u], dxa[4 * gx + 2]);
-                            dxa[4 * gx + 3] = __builtin_fmaf(m.w, sd[u], dxa[4 * gx + 3]);
-#pragma unroll
-                            for (int jj = 0; jj < 4; jj++) G[uu * 4 + jj] = sd[u] * xv[4 * gx + jj];
+                            fma_quad<0>(T[u], m[uu], xv[4 * gx]);
+                            fma_quad<1>(T[u], m[uu], xv[4 * gx + 1]);
+                            fma_quad<2>(T[u], m[uu], xv[4 * gx + 2]);
+                            fma_quad<3>(T[u], m[uu], xv[4 * gx + 3]);
+                            fma_quad<0>(dxa[4 * gx], m[uu], sd[u]);
+                            fma_quad<1>(dxa[4 * gx + 1], m[uu], sd[u]);
+                            fma_quad<2>(dxa[4 * gx + 2], m[uu], sd[u]);
+                            fma_quad<3>(dxa[4 * gx + 3], m[uu], sd[u]);
                         }
-                        part[half] = transpose_sum_half(G, lane);
                     }
-                    const float total = join_halves(part[0], part[1]);
-                    const int where = dense[(b * 16 + lane / 4) * kPlanX + 4 * gx + lane % 4];
-                    const int first = where & 2047, cnt = where >> 11;
-                    for (int rr = 0; rr < cnt; rr++)
-                        atomicAdd(&dyl[tab[pairs + 2 * (first + rr) + 1]],
-                                  __int_as_float(tab[pairs + 2 * (first + rr)]) * total);
+                }
+                {   // dy: the channel sums of the block's cells, then the cells' entries
+#pragma unroll
+                    for (int u = 0; u < 16; u++) tile[u * kTileStride + lane] = sd[u];
+                    wave_lds_sync();
+                    ChannelOperand sdop;
+                    sdop.read(tile, lane);
+                    wave_lds_sync();  // (the tile is written again below)
+                    const f32x4 sums = channel_sums(sdop, xop);
+                    // the totals by cell in the tile, then a lane per entry of the block: coefficient x total
+                    // of the entry's cell, added to dy[k] of the wave's row in LDS
+#pragma unroll
+                    for (int r = 0; r < 4; r++) tile[(4 * (lane >> 4) + r) * kPlanX + (lane & 15)] = sums[r];
+                    wave_lds_sync();
+                    for (int n0 = entries0; n0 < entries1; n0 += kWave) {
+                        const int n = n0 + lane;
+                        if (n < entries1) {
+                            const int w = tab[pairs + 2 * n + 1];
+                            atomicAdd(&dyl[w & 255], __int_as_float(tab[pairs + 2 * n]) * tile[w >> 8]);
+                        }
+                    }
+                    wave_lds_sync();  // (the tile is written again by the next block)
                 }
                 // ds: the slots of one scalar are adjacent; a scalar's sum is stored when the next begins
 #pragma unroll
@@ -671,6 +770,8 @@ __global__ __launch_bounds__(256, 2) void planned_bwd_kernel(
                     }
                     dsa = __builtin_fmaf(dz[u], T[u], dsa);
                 }
+#pragma unroll
+                for (int u = 0; u < 16; u++) dz[u] = dz_ahead[u];
             }
             if (cur_l >= 0 && active) *element_at(dsrow0, dsoff, (unsigned)ls.dim, (unsigned)cur_l) = (Val)dsa;
             if (active)
@@ -774,8 +875,8 @@ int launch_planned_bwd_t(const e3j_amd_conv_params &p, bool group_is_receiver, c
     const int64_t items = group_is_receiver ? (int64_t)p.num_nodes * nchunks : (int64_t)p.num_nodes;
     const int64_t blocks = (items + kWavesPerBlock - 1) / kWavesPerBlock;
     if (blocks > 0x7fffffffLL) return set_error(E3J_AMD_INVALID_ARGUMENT, "convolution_bwd: grid too large");
-    const size_t lds = sizeof(float) * ((size_t)table_words(p.num_coef) + (size_t)nb * 256 +
-                                        (size_t)kWavesPerBlock * (nb * 16 * xg * 4 + kPlanMaxY + p.num_scalars * kWave));
+    const size_t lds = sizeof(float) * ((size_t)table_words(p.num_coef) +
+                                        (size_t)kWavesPerBlock * (nb * 16 * xg * 4 + kPlanMaxY + p.num_scalars * kWave + kTileWords));
     if (lds > 64 * 1024) {
         const int rc = check_hip(hipFuncSetAttribute(reinterpret_cast<const void *>(kernels[nb - 1][xg - 1]),
                                                      hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds),
