@@ -262,6 +262,15 @@ __device__ __forceinline__ void wave_lds_sync() {
 __device__ __forceinline__ void together(float (&m)[8]) {
     asm volatile("" : "+v"(m[0]), "+v"(m[1]), "+v"(m[2]), "+v"(m[3]), "+v"(m[4]), "+v"(m[5]), "+v"(m[6]), "+v"(m[7]));
 }
+// The reads before it are issued before the instructions behind it (the compiler would otherwise
+// move a read down to its use, and the read ahead of the next eight numbers of M with it).
+__device__ __forceinline__ void issued() { asm volatile("" ::: "memory"); }
+// The eight slots' numbers of M of (block b, group g of x coordinates, half): lane t takes number t % 4.
+template <int XG>
+__device__ __forceinline__ void read_half(const float *M, int b, int g, int half, int lane, float (&m)[8]) {
+#pragma unroll
+    for (int uu = 0; uu < 8; uu++) m[uu] = M[((b * 16 + half * 8 + uu) * XG + g) * 4 + (lane & 3)];
+}
 template <int K>
 __device__ __forceinline__ void fma_quad(float &acc, float m, float v) {
     asm("v_fmac_f32_dpp %0, %1, %2 quad_perm:[%3,%3,%3,%3] row_mask:0xf bank_mask:0xf"
@@ -390,9 +399,10 @@ struct RowCursor {
     __device__ __forceinline__ RowCursor(const Val *row0, unsigned lane_elems, unsigned stride_elems)
         : base(reinterpret_cast<const char *>(row0)), at((unsigned)sizeof(Val) * lane_elems),
           step((unsigned)sizeof(Val) * stride_elems) {}
-    __device__ __forceinline__ float row(unsigned r) const {  // r wave-uniform
-        return (float)*reinterpret_cast<const Val *>((base + (size_t)r * step) + at);
+    __device__ __forceinline__ Val raw(unsigned r) const {  // r wave-uniform; as held in memory
+        return *reinterpret_cast<const Val *>((base + (size_t)r * step) + at);
     }
+    __device__ __forceinline__ float row(unsigned r) const { return (float)raw(r); }
 };
 // the lane's element of row r of an output operand (same addressing)
 template <typename Val>
@@ -408,29 +418,29 @@ __device__ __forceinline__ Val *element_at(Val *row0, unsigned lane_elems, unsig
 constexpr int kRowsAhead = 24;
 template <typename Val>
 struct ScalarRows {
-    float v[kRowsAhead];
+    Val v[kRowsAhead];  // (as loaded: a conversion here would wait for the load)
     __device__ __forceinline__ void load(const RowCursor<Val> &cur, int S) {
 #pragma unroll
-        for (int t = 0; t < 8; t++) v[t] = cur.row((unsigned)(t < S ? t : S - 1));  // (clamped: straight-line)
+        for (int t = 0; t < 8; t++) v[t] = cur.raw((unsigned)(t < S ? t : S - 1));  // (clamped: straight-line)
         if (S > 8) {
 #pragma unroll
-            for (int t = 8; t < 16; t++) v[t] = cur.row((unsigned)(t < S ? t : S - 1));
+            for (int t = 8; t < 16; t++) v[t] = cur.raw((unsigned)(t < S ? t : S - 1));
         }
         if (S > 16) {
 #pragma unroll
-            for (int t = 16; t < kRowsAhead; t++) v[t] = cur.row((unsigned)(t < S ? t : S - 1));
+            for (int t = 16; t < kRowsAhead; t++) v[t] = cur.raw((unsigned)(t < S ? t : S - 1));
         }
     }
     __device__ __forceinline__ void store(const RowCursor<Val> &cur, int S, float *sbuf, int lane) const {
 #pragma unroll
-        for (int t = 0; t < 8; t++) sbuf[(t < S ? t : S - 1) * kWave + lane] = v[t];
+        for (int t = 0; t < 8; t++) sbuf[(t < S ? t : S - 1) * kWave + lane] = (float)v[t];
         if (S > 8) {
 #pragma unroll
-            for (int t = 8; t < 16; t++) sbuf[(t < S ? t : S - 1) * kWave + lane] = v[t];
+            for (int t = 8; t < 16; t++) sbuf[(t < S ? t : S - 1) * kWave + lane] = (float)v[t];
         }
         if (S > 16) {
 #pragma unroll
-            for (int t = 16; t < kRowsAhead; t++) sbuf[(t < S ? t : S - 1) * kWave + lane] = v[t];
+            for (int t = 16; t < kRowsAhead; t++) sbuf[(t < S ? t : S - 1) * kWave + lane] = (float)v[t];
         }
         for (int t0 = kRowsAhead; t0 < S; t0 += 8) {
             float w[8];
@@ -444,17 +454,18 @@ struct ScalarRows {
 
 // The edge a wave works on, fetched one edge ahead of its use: the other end, the position of the
 // edge's operands and the wave's copy of y (lane k holds y[k]).
+template <typename Val>
 struct EdgeAhead {
     int other;
     int64_t at;
-    float y;
-    template <typename Val>
+    Val y_held;  // (as loaded: a conversion here would wait for the load)
+    __device__ __forceinline__ float y(int num_y, int lane) const { return lane < num_y ? (float)y_held : 0.f; }
     __device__ __forceinline__ static EdgeAhead fetch(const int32_t *__restrict__ other, const int32_t *__restrict__ perm,
                                                       const Val *__restrict__ y, int num_y, int e, int lane) {
         EdgeAhead a;
         a.other = uni(other[e]);
         a.at = perm ? (int64_t)uni(perm[e]) : (int64_t)e;
-        a.y = lane < num_y ? (float)y[a.at * num_y + lane] : 0.f;
+        a.y_held = y[a.at * num_y + (lane < num_y ? lane : 0)];
         return a;
     }
 };
@@ -495,28 +506,28 @@ __global__ __launch_bounds__(256, 2) void planned_fwd_kernel(
     for (int t = 0; t < NB * 16; t++) acc[t] = 0.f;
 
     const int e0 = uni(row_ptr[r]), e1 = uni(row_ptr[r + 1]);
-    EdgeAhead next = {0, 0, 0.f};
-    if (e0 < e1) next = EdgeAhead::fetch(other, perm, y, num_y, e0, lane);
+    EdgeAhead<Val> next = {0, 0, Val(0)};
+    if (e0 < e1) next = EdgeAhead<Val>::fetch(other, perm, y, num_y, e0, lane);
     for (int e = e0; e < e1; e++) {
-        const EdgeAhead edge = next;
+        const EdgeAhead<Val> edge = next;
         // this edge's loads, its matrix built under them (LDS only), then the next edge's numbers
         const bool live = (unsigned)edge.other < (unsigned)num_nodes;  // (wave-uniform) padding edges are stepped over
         const RowCursor<Val> sc(s + edge.at * ls.row, soff, (unsigned)ls.dim);
         ScalarRows<Val> rows;
-        float xv[XG * 4];
+        Val x_held[XG * 4];  // (as loaded; converted once the matrix is built)
         if (live) {
             const RowCursor<Val> xc(x + (int64_t)edge.other * lx.row, xoff, (unsigned)lx.dim);
 #pragma unroll
-            for (int j = 0; j < XG * 4; j++) xv[j] = xc.row((unsigned)(j < X ? j : X - 1));
+            for (int j = 0; j < XG * 4; j++) x_held[j] = xc.raw((unsigned)(j < X ? j : X - 1));
             rows.load(sc, S);
             wave_lds_sync();  // the reads of the edge before are behind the writes below
-            build_edge_matrix<XG>(tab, held, num_cells, max_run, edge.y, M, lane);
+            build_edge_matrix<XG>(tab, held, num_cells, max_run, edge.y(num_y, lane), M, lane);
         }
-        next = EdgeAhead::fetch(other, perm, y, num_y, e + 1 < e1 ? e + 1 : e, lane);
+        next = EdgeAhead<Val>::fetch(other, perm, y, num_y, e + 1 < e1 ? e + 1 : e, lane);
         if (!live) continue;
+        float xv[XG * 4];
 #pragma unroll
-        for (int j = 0; j < XG * 4; j++)
-            if (j >= X) xv[j] = 0.f;
+        for (int j = 0; j < XG * 4; j++) xv[j] = j < X ? (float)x_held[j] : 0.f;
         rows.store(sc, S, sbuf, lane);
         wave_lds_sync();
 #pragma unroll
@@ -535,8 +546,7 @@ __global__ __launch_bounds__(256, 2) void planned_fwd_kernel(
                 for (int half = 0; half < 2; half++) {
                     if (!half_live<XG>(half0, half1, b, g, half)) continue;  // eight slots without a coefficient here
                     float m[8];  // (read together, used together: one LDS round trip per half)
-#pragma unroll
-                    for (int uu = 0; uu < 8; uu++) m[uu] = M[((b * 16 + half * 8 + uu) * XG + g) * 4 + (lane & 3)];
+                    read_half<XG>(M, b, g, half, lane, m);
                     together(m);
 #pragma unroll
                     for (int uu = 0; uu < 8; uu++) {
@@ -647,10 +657,10 @@ __global__ __launch_bounds__(256, 2) void planned_bwd_kernel(
         float dxa[XG * 4];
 #pragma unroll
         for (int j = 0; j < XG * 4; j++) dxa[j] = 0.f;
-        EdgeAhead next = {0, 0, 0.f};
-        if (e0 < e1) next = EdgeAhead::fetch(other, perm, y, num_y, e0, lane);
+        EdgeAhead<Val> next = {0, 0, Val(0)};
+        if (e0 < e1) next = EdgeAhead<Val>::fetch(other, perm, y, num_y, e0, lane);
         for (int e = e0; e < e1; e++) {
-            const EdgeAhead edge = next;
+            const EdgeAhead<Val> edge = next;
             const bool live = (unsigned)edge.other < (unsigned)num_nodes;  // (wave-uniform) padding edges are stepped over
             const int o = edge.other;
             const int64_t ee = edge.at;
@@ -661,29 +671,29 @@ __global__ __launch_bounds__(256, 2) void planned_bwd_kernel(
             const RowCursor<Val> sc(s + ee * ls.row, soff, (unsigned)ls.dim);
             const RowCursor<Val> zc(dm + (int64_t)(live ? znode : 0) * lo.row, zoff, (unsigned)lo.dim);
             ScalarRows<Val> rows;
-            float xv[XG * 4];
-            float dz[16], dz_ahead[16];  // dm of the block at hand and of the block after it
-            auto load_dm = [&](int b, float (&to)[16]) {
+            Val x_held[XG * 4];  // (as loaded; converted once the matrix is built)
+            Val dz_held[16], dz_ahead[16];  // dm of the block at hand and of the block after it, as loaded
+            auto load_dm = [&](int b, Val (&to)[16]) {
 #pragma unroll
                 for (int u = 0; u < 16; u++) {
                     const int row = slot_row[b * 16 + u];  // (-1: none)
-                    to[u] = zc.row((unsigned)(row < 0 ? 0 : row));
+                    to[u] = zc.raw((unsigned)(row < 0 ? 0 : row));
                 }
             };
             if (live) {
                 const RowCursor<Val> xc(x + (int64_t)xnode * lx.row, xoff, (unsigned)lx.dim);
 #pragma unroll
-                for (int j = 0; j < XG * 4; j++) xv[j] = xc.row((unsigned)(j < X ? j : X - 1));
+                for (int j = 0; j < XG * 4; j++) x_held[j] = xc.raw((unsigned)(j < X ? j : X - 1));
                 rows.load(sc, S);
-                load_dm(0, dz);
+                load_dm(0, dz_held);
                 wave_lds_sync();  // the reads of the edge before are behind the writes below
-                build_edge_matrix<XG>(tab, num_cells, max_run, edge.y, M, lane);
+                build_edge_matrix<XG>(tab, num_cells, max_run, edge.y(num_y, lane), M, lane);
             }
-            next = EdgeAhead::fetch(other, perm, y, num_y, e + 1 < e1 ? e + 1 : e, lane);
+            next = EdgeAhead<Val>::fetch(other, perm, y, num_y, e + 1 < e1 ? e + 1 : e, lane);
             if (!live) continue;
+            float xv[XG * 4];
 #pragma unroll
-            for (int j = 0; j < XG * 4; j++)
-                if (j >= X || !active) xv[j] = 0.f;  // (idle lanes add nothing to dy)
+            for (int j = 0; j < XG * 4; j++) xv[j] = j < X && active ? (float)x_held[j] : 0.f;  // (idle lanes add nothing to dy)
             rows.store(sc, S, sbuf, lane);
 #pragma unroll
             for (int j = 0; j < 16; j++) tile[j * kTileStride + lane] = j < XG * 4 ? xv[j < XG * 4 ? j : 0] : 0.f;
@@ -701,40 +711,42 @@ __global__ __launch_bounds__(256, 2) void planned_bwd_kernel(
                 const int entries0 = uni(plan[L.block_first + b]), entries1 = uni(plan[L.block_first + b + 1]);
                 if (((chunk_mask >> (b * XG)) & ((1u << XG) - 1u)) == 0) {
 #pragma unroll
-                    for (int u = 0; u < 16; u++) dz[u] = dz_ahead[u];
+                    for (int u = 0; u < 16; u++) dz_held[u] = dz_ahead[u];
                     continue;
                 }
-                float sd[16], T[16];
+                float sd[16], dz[16], T[16];
 #pragma unroll
                 for (int u = 0; u < 16; u++) {
                     const int l = slot_l[b * 16 + u];  // (-1: none)
                     const float sv = sbuf[(l < 0 ? 0 : l) * kWave + lane];
-                    if (l < 0) dz[u] = 0.f;
+                    dz[u] = l < 0 ? 0.f : (float)dz_held[u];
                     sd[u] = sv * dz[u];
                     T[u] = 0.f;
                 }
+                // the next half's numbers of M are read while the products of the one at hand run (read
+                // whether or not the half holds a coefficient: the count of reads in flight stays a
+                // compile-time number)
+                float m[2][8];
+                read_half<XG>(M, b, 0, 0, lane, m[0]);
 #pragma unroll
-                for (int gx = 0; gx < XG; gx++) {
-                    if (!((chunk_mask >> (b * XG + gx)) & 1u)) continue;
+                for (int it = 0; it < 2 * XG; it++) {
+                    const int gx = it / 2, half = it % 2;
+                    if (it + 1 < 2 * XG) read_half<XG>(M, b, (it + 1) / 2, (it + 1) % 2, lane, m[(it + 1) & 1]);
+                    issued();
+                    if (!half_live<XG>(half0, half1, b, gx, half)) continue;  // eight slots without a coefficient here
+                    together(m[it & 1]);
 #pragma unroll
-                    for (int half = 0; half < 2; half++) {
-                        if (!half_live<XG>(half0, half1, b, gx, half)) continue;  // eight slots without a coefficient here
-                        float m[8];
-#pragma unroll
-                        for (int uu = 0; uu < 8; uu++) m[uu] = M[((b * 16 + half * 8 + uu) * XG + gx) * 4 + (lane & 3)];
-                        together(m);
-#pragma unroll
-                        for (int uu = 0; uu < 8; uu++) {
-                            const int u = half * 8 + uu;
-                            fma_quad<0>(T[u], m[uu], xv[4 * gx]);
-                            fma_quad<1>(T[u], m[uu], xv[4 * gx + 1]);
-                            fma_quad<2>(T[u], m[uu], xv[4 * gx + 2]);
-                            fma_quad<3>(T[u], m[uu], xv[4 * gx + 3]);
-                            fma_quad<0>(dxa[4 * gx], m[uu], sd[u]);
-                            fma_quad<1>(dxa[4 * gx + 1], m[uu], sd[u]);
-                            fma_quad<2>(dxa[4 * gx + 2], m[uu], sd[u]);
-                            fma_quad<3>(dxa[4 * gx + 3], m[uu], sd[u]);
-                        }
+                    for (int uu = 0; uu < 8; uu++) {
+                        const int u = half * 8 + uu;
+                        const float mu = m[it & 1][uu];
+                        fma_quad<0>(T[u], mu, xv[4 * gx]);
+                        fma_quad<1>(T[u], mu, xv[4 * gx + 1]);
+                        fma_quad<2>(T[u], mu, xv[4 * gx + 2]);
+                        fma_quad<3>(T[u], mu, xv[4 * gx + 3]);
+                        fma_quad<0>(dxa[4 * gx], mu, sd[u]);
+                        fma_quad<1>(dxa[4 * gx + 1], mu, sd[u]);
+                        fma_quad<2>(dxa[4 * gx + 2], mu, sd[u]);
+                        fma_quad<3>(dxa[4 * gx + 3], mu, sd[u]);
                     }
                 }
                 {   // dy: the channel sums of the block's cells, then the cells' entries
@@ -771,7 +783,7 @@ __global__ __launch_bounds__(256, 2) void planned_bwd_kernel(
                     dsa = __builtin_fmaf(dz[u], T[u], dsa);
                 }
 #pragma unroll
-                for (int u = 0; u < 16; u++) dz[u] = dz_ahead[u];
+                for (int u = 0; u < 16; u++) dz_held[u] = dz_ahead[u];
             }
             if (cur_l >= 0 && active) *element_at(dsrow0, dsoff, (unsigned)ls.dim, (unsigned)cur_l) = (Val)dsa;
             if (active)
