@@ -32,13 +32,69 @@ COMMON_FLAGS = [
 ]
 
 
+# Sources whose kernels hold DPP instructions written as inline assembly.  The compiler's hazard
+# pass does not look inside inline assembly, so the build reads the assembly it wrote for them.
+DPP_ASM_SOURCES = ("conv_planned.hip", "conv_planned_f16.hip")
+
+
+def dpp_read_hazards(assembly: str) -> list[str]:
+    """The inline `v_fmac_f32_dpp` instructions of an assembly listing whose DPP operand (the first
+    source) was written by a vector instruction fewer than two wait states before: on gfx9 the
+    hardware does not wait for that, and the kernels are written so that the operand always
+    comes from an LDS read.  Returns one line of text per violation (none expected)."""
+    import re
+
+    def vgprs(token: str) -> set[int]:
+        m = re.match(r"v\[(\d+):(\d+)\]", token)
+        if m:
+            return set(range(int(m.group(1)), int(m.group(2)) + 1))
+        m = re.match(r"v(\d+)$", token)
+        return {int(m.group(1))} if m else set()
+
+    lines = [line.strip() for line in assembly.splitlines()]
+    lines = [line for line in lines if line and not line.startswith((";", ".", "//")) and not line.endswith(":")]
+    found = []
+    for i, line in enumerate(lines):
+        if not line.startswith("v_fmac_f32_dpp"):
+            continue
+        operands = [o.strip() for o in line.split(None, 1)[1].split(",")]
+        source = vgprs(operands[1].split()[0])
+        states = 0
+        for before in reversed(lines[max(i - 3, 0):i]):
+            if states >= 2:
+                break
+            if before.startswith("s_nop"):
+                states += int(before.split()[1]) + 1
+                continue
+            if before.startswith("v_") and not before.startswith(("v_readlane", "v_readfirstlane", "v_cmp")):
+                written = vgprs(before.split(None, 1)[1].split(",")[0].strip())
+                if written & source:
+                    found.append(f"{before}  ->  {line}")
+            states += 1
+    return found
+
+
 def _compile_one(src: str, extra: list[str]) -> str:
     rel = os.path.relpath(src, CSRC).replace(os.sep, "_")
     obj = os.path.join(OBJ_DIR, os.path.splitext(rel)[0] + ".o")
+    check_dpp = os.path.basename(src) in DPP_ASM_SOURCES
+    keep_temps = "-save-temps=obj" in extra
+    if check_dpp and not keep_temps:
+        extra = [*extra, "-save-temps=obj"]
     cmd = [HIPCC, *COMMON_FLAGS, *extra, "-c", src, "-o", obj]
     proc = subprocess.run(cmd, capture_output=True, text=True)
     if proc.returncode != 0:
         raise RuntimeError(f"hipcc failed for {src}:\n{' '.join(cmd)}\n{proc.stdout}\n{proc.stderr}")
+    if check_dpp:
+        listing = os.path.join(OBJ_DIR, f"{os.path.splitext(rel)[0]}-hip-amdgcn-amd-amdhsa-{ARCH}.s")
+        with open(listing) as f:
+            hazards = dpp_read_hazards(f.read())
+        if not keep_temps:  # (the listing came with the compiler's other intermediate files)
+            stem = os.path.join(OBJ_DIR, os.path.splitext(rel)[0])
+            for path in glob.glob(stem + "-h*") + glob.glob(stem + ".hip-*"):
+                os.remove(path)
+        if hazards:
+            raise RuntimeError(f"{src}: a DPP operand is read too soon after a vector write:\n" + "\n".join(hazards[:10]))
     return obj
 
 

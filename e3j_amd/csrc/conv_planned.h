@@ -256,7 +256,9 @@ __device__ __forceinline__ void wave_lds_sync() {
 // acc += (m of lane K of the lane's group of four lanes) * v, one instruction (a DPP operand).  The
 // loops read four wave-uniform numbers of M with one 4-byte LDS read (lane t takes number t % 4)
 // instead of a 16-byte broadcast to every lane: a quarter of the LDS return traffic.  (m comes
-// from an LDS read, never from a vector instruction just before: no wait states are owed.)
+// from an LDS read, never from a vector instruction just before, so no wait states are owed; the
+// compiler's hazard pass does not look inside inline assembly, and e3j_amd/build.py reads the
+// assembly listing of this file for a DPP operand written less than two wait states earlier.)
 // Keeps the eight reads before it together (the values are all in registers here): without it the
 // compiler moves each read next to its use and pays an LDS round trip per pair of values.
 __device__ __forceinline__ void together(float (&m)[8]) {

@@ -388,3 +388,35 @@ def test_run_time_tensor_product_signature_compiles_and_registers():
                                big.shape, 64)) == 3
     idx, val, _ = H.random_table(np.random.default_rng(0), 400, 4, 5, 300, 7)   # 300 outputs: outside the templates
     assert jit.register_tp(np.asarray(val, np.float32), idx.astype(np.int64), (300, 4, 5), 64) == []
+
+
+def test_build_reads_the_assembly_for_dpp_operands_written_too_late():
+    """The planned kernels use `v_fmac_f32_dpp` through inline assembly, which the compiler's hazard
+    pass does not see: the build scans the assembly for a DPP operand written by a vector
+    instruction fewer than two wait states earlier."""
+    from e3j_amd.build import dpp_read_hazards
+    fine = """
+        ds_read2_b32 v[2:3], v193 offset1:16
+        s_waitcnt lgkmcnt(0)
+        v_mov_b32_e32 v40, v0
+        v_fmac_f32_dpp v32, v2, v16 quad_perm:[0,0,0,0] row_mask:0xf bank_mask:0xf
+        v_fmac_f32_dpp v33, v3, v16 quad_perm:[0,0,0,0] row_mask:0xf bank_mask:0xf
+    """
+    assert dpp_read_hazards(fine) == []
+    late = """
+        v_mov_b32_e32 v2, v7
+        v_fmac_f32_dpp v32, v2, v16 quad_perm:[0,0,0,0] row_mask:0xf bank_mask:0xf
+    """
+    assert len(dpp_read_hazards(late)) == 1
+    spaced = """
+        v_mov_b32_e32 v2, v7
+        s_nop 1
+        v_fmac_f32_dpp v32, v2, v16 quad_perm:[0,0,0,0] row_mask:0xf bank_mask:0xf
+    """
+    assert dpp_read_hazards(spaced) == []
+    pair = """
+        v_mov_b64_e32 v[2:3], v[8:9]
+        v_add_f32_e32 v9, v9, v9
+        v_fmac_f32_dpp v32, v3, v16 quad_perm:[1,1,1,1] row_mask:0xf bank_mask:0xf
+    """
+    assert len(dpp_read_hazards(pair)) == 1
