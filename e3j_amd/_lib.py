@@ -88,6 +88,7 @@ class TpParams(ctypes.Structure):
         ("debug", ctypes.c_int32),
         ("signature", ctypes.c_int32),
         ("coef_scale", ctypes.c_float),
+        ("coef_classes", ctypes.c_void_p),
     ]
 
 
@@ -173,6 +174,7 @@ SYMBOLS = {
     "e3j_amd_tensor_product_fwd": (ctypes.c_int, [_TP_PARAMS] + [_P] * 5),
     "e3j_amd_tensor_product_bwd": (ctypes.c_int, [_TP_PARAMS] + [_P] * 7),
     "e3j_amd_tp_find_signature": (ctypes.c_int, [_P] + [ctypes.c_int32] * 9 + [ctypes.POINTER(ctypes.c_float)]),
+    "e3j_amd_tp_find_signature_f64": (ctypes.c_int, [_P] + [ctypes.c_int32] * 8 + [ctypes.POINTER(ctypes.c_double)]),
     "e3j_amd_tp_num_signatures": (ctypes.c_int, []),
     "e3j_amd_tp_register_signature": (ctypes.c_int, [_P]),
     "e3j_amd_tp_signature_name": (ctypes.c_char_p, [ctypes.c_int]),

@@ -18,7 +18,7 @@ from collections import OrderedDict
 import numpy as np
 
 from ..tensor_product import TensorProduct
-from .gen_conv import _lit
+from .gen_conv import F64_MAX_CLASSES, _f32_bits, _lit
 
 #: (name, x irreps, y irreps, output filter or None for the full product, channel counts)
 TP_TABLES = [
@@ -42,46 +42,78 @@ def _rows(val, idx, num_out):
     return rows
 
 
-def emit_sig(struct_name: str, val, idx, shape) -> list[str]:
-    Z, X, Y = (int(d) for d in shape)
-    rows = _rows(val, idx, Z)
-    out = [f"struct {struct_name} {{",
-           f"    static constexpr int X = {X}, Y = {Y}, Z = {Z};",
-           "",
-           "    template <typename Store>",
-           "    __device__ static __forceinline__ void fwd(const float *x, const float *y, const Store &st) {"]
+def coefficient_classes(val):
+    """Classes of equal magnitude in the order of their first entry (`class of each entry`, number
+    of classes): the float64 kernels read one value per class from a kernel argument."""
+    classes = OrderedDict()
+    for v in np.asarray(val, dtype=np.float32):
+        if v != 0:
+            classes.setdefault(_f32_bits(abs(float(v))), len(classes))
+    return [classes[_f32_bits(abs(float(v)))] if v != 0 else 255 for v in np.asarray(val, dtype=np.float32)], len(classes)
+
+
+def _emit_arith(val, idx, shape, f64: bool) -> list[str]:
+    """`fwd` and `bwd` of a table: coefficients as float literals with float operands, or (float64)
+    read from the coefficient classes `cf` under the sign of the entry."""
+    Z = int(shape[0])
+    T = "double" if f64 else "float"
+    fma = "fma" if f64 else "fmaf"
+    zero = "0.0" if f64 else "0.f"
+    class_of, _ = coefficient_classes(val)
+    rows = OrderedDict((i, []) for i in range(Z))
+    for n, (v, (i, j, k)) in enumerate(zip(val, idx)):
+        if v != 0:
+            c = float(np.float32(v))
+            text = (("-" if c < 0 else "") + f"cf.v[{class_of[n]}]") if f64 else _lit(c)
+            rows[int(i)].append((text, int(j), int(k)))
+    tail = ", const F64Coefs &cf" if f64 else ", TpNoCoefs = {}"
+    out = ["    template <typename Store>",
+           f"    __device__ static __forceinline__ void fwd(const {T} *x, const {T} *y, const Store &st{tail}) {{"]
     for i, terms in rows.items():
         if not terms:
-            out.append(f"        st.template put<{i}>(0.f);")
+            out.append(f"        st.template put<{i}>({zero});")
             continue
         out.append("        {")
         for n, (c, j, k) in enumerate(terms):
             if n == 0:
-                out.append(f"            float m = {_lit(c)} * (x[{j}] * y[{k}]);")
+                out.append(f"            {T} m = {c} * (x[{j}] * y[{k}]);")
             else:
-                out.append(f"            m = fmaf({_lit(c)}, x[{j}] * y[{k}], m);")
+                out.append(f"            m = {fma}({c}, x[{j}] * y[{k}], m);")
         out.append(f"            st.template put<{i}>(m);")
         out.append("        }")
     out += ["    }", "",
             "    // dx and dy are accumulated into: the caller clears them",
             "    template <typename Load>",
-            "    __device__ static __forceinline__ void bwd(const float *x, const float *y, const Load &ld,",
-            "                                                float *dx, float *dy) {"]
+            f"    __device__ static __forceinline__ void bwd(const {T} *x, const {T} *y, const Load &ld,",
+            f"                                                {T} *dx, {T} *dy{tail}) {{"]
     for i, terms in rows.items():
         if not terms:
             continue
         out.append("        {")
-        out.append(f"            const float g = ld.template get<{i}>();")
+        out.append(f"            const {T} g = ld.template get<{i}>();")
         scaled = OrderedDict()
         for c, j, k in terms:
             if c not in scaled:
                 scaled[c] = f"t{len(scaled)}"
-                out.append(f"            const float {scaled[c]} = {_lit(c)} * g;")
+                out.append(f"            const {T} {scaled[c]} = {c} * g;")
             t = scaled[c]
-            out.append(f"            dx[{j}] = fmaf({t}, y[{k}], dx[{j}]);")
-            out.append(f"            dy[{k}] = fmaf({t}, x[{j}], dy[{k}]);")
+            out.append(f"            dx[{j}] = {fma}({t}, y[{k}], dx[{j}]);")
+            out.append(f"            dy[{k}] = {fma}({t}, x[{j}], dy[{k}]);")
         out.append("        }")
-    out += ["    }", "};", ""]
+    out += ["    }"]
+    return out
+
+
+def emit_sig(struct_name: str, val, idx, shape, f64: bool = False) -> list[str]:
+    Z, X, Y = (int(d) for d in shape)
+    out = [f"struct {struct_name} {{",
+           f"    static constexpr int X = {X}, Y = {Y}, Z = {Z};",
+           ""]
+    out += _emit_arith(val, idx, shape, False)
+    if f64:
+        out += ["", "    // float64: one coefficient per class of equal magnitude, from the kernel's argument"]
+        out += _emit_arith(val, idx, shape, True)
+    out += ["};", ""]
     return out
 
 
@@ -102,12 +134,18 @@ def emit_source(name: str, desc: str, val, idx, shape, channels: int, symbols, i
            "namespace e3j_amd {",
            "namespace {",
            ""]
-    out += emit_sig(sig, val, idx, shape)
+    # float16 and float64 kernels: trailing layout, whole waves of channels
+    wide = not leading and channels % 64 == 0
+    class_of, num_classes = coefficient_classes(val)
+    if num_classes > F64_MAX_CLASSES:
+        wide = False
+    out += emit_sig(sig, val, idx, shape, f64=wide)
     out += ["}  // namespace", "",
             "// host pass only: the registry entries hold host function pointers",
             "#if !defined(__HIP_DEVICE_COMPILE__)",
             f"static const float kVal[] = {{{vals}}};",
-            f"static const uint8_t kIdx[] = {{{idxs}}};"]
+            f"static const uint8_t kIdx[] = {{{idxs}}};",
+            f"static const uint8_t kClass[] = {{{', '.join(str(c) for c in class_of)}}};"]
     layout = "E3J_AMD_LAYOUT_LEADING" if leading else "E3J_AMD_LAYOUT_TRAILING"
     for kind, symbol in zip((0, 1, 2), symbols):
         uniform = kind
@@ -119,7 +157,13 @@ def emit_source(name: str, desc: str, val, idx, shape, channels: int, symbols, i
                 f"    {X}, {Y}, {Z}, {len(val)}, {channels}, {uniform}, {layout}, kVal, kIdx,",
                 f"    &launch_tp_unrolled_fwd{suffix}<{args}>,",
                 f"    &launch_tp_unrolled_bwd{suffix}<{args}>,",
-                "};"]
+                f"    {num_classes}, kClass,"]
+        if wide:
+            out += [f"    &launch_tp_unrolled_fwd_f16<{args}>, &launch_tp_unrolled_bwd_f16<{args}>,",
+                    f"    &launch_tp_unrolled_fwd_f64<{args}>, &launch_tp_unrolled_bwd_f64<{args}>,"]
+        else:
+            out += ["    nullptr, nullptr, nullptr, nullptr,"]
+        out += ["};"]
     if plugin:  # accessor a run-time compiled library is loaded through
         out += ["", f"static const TpSignature *const kPlugin[] = {{{', '.join('&' + sym for sym in symbols)}}};",
                 'extern "C" const void *e3j_amd_tp_plugin_signature(int which) {',
@@ -128,6 +172,13 @@ def emit_source(name: str, desc: str, val, idx, shape, channels: int, symbols, i
     out += ["#else", "// device pass: the kernels must be instantiated"]
     fwd_args = "    const float *, const float *, float *, int64_t, {}float);"
     bwd_args = "    const float *, const float *, const float *, float *, float *, int64_t, {}float);"
+
+    def typed(kind: str, V: str) -> str:
+        """Argument list of a trailing-layout kernel for values held as `V`."""
+        A, cf = ("double", "F64Coefs") if V == "double" else ("float", "TpNoCoefs")
+        if kind == "fwd":
+            return f"    const {V} *, const {V} *, {V} *, int64_t, {A}, {cf});"
+        return f"    const {V} *, const {V} *, const {V} *, {V} *, {V} *, int64_t, {A}, {cf});"
     if leading:
         for uniform in ("false", "true"):
             out.append(f"template __global__ void tp_unrolled_fwd_leading_kernel<{sig}, 4, {uniform}>(")
@@ -142,20 +193,27 @@ def emit_source(name: str, desc: str, val, idx, shape, channels: int, symbols, i
         out.append(f"template __global__ void tp_unrolled_bwd_uniform_leading_lds_kernel<{sig}, 2>(")
         out.append(bwd_args.format("int, "))
     else:
-        for uniform in ("false", "true"):
-            out.append(f"template __global__ void tp_unrolled_fwd_kernel<{sig}, {channels}, 4, {uniform}>(")
-            out.append(fwd_args.format(""))
         narrow = channels < 64   # 16 or 32 channels: several rows side by side in a wave
-        out.append(f"template __global__ void tp_unrolled_fwd_inner{'_narrow' if narrow else ''}_kernel<{sig}, "
-                   f"{channels}{', 4' if narrow else ''}>(")
-        out.append(fwd_args.format(""))
-        out.append(f"template __global__ void tp_unrolled_bwd_inner_kernel<{sig}, {channels}, 4>(")
-        out.append(bwd_args.format(""))
-        out.append(f"template __global__ void tp_unrolled_bwd_map_kernel<{sig}, {channels}, 4>(")
-        out.append(bwd_args.format(""))
-        out.append(f"template __global__ void tp_unrolled_bwd_uniform{'_narrow' if narrow else ''}_kernel<{sig}, "
-                   f"{channels}{', 4' if narrow else ''}>(")
-        out.append(bwd_args.format(""))
+        for V in ("float", "half_t", "double") if wide else ("float",):
+            for uniform in ("false", "true"):
+                out.append(f"template __global__ void tp_unrolled_fwd_kernel<{sig}, {channels}, 4, {uniform}, {V}>(")
+                out.append(typed("fwd", V))
+            if narrow:
+                out.append(f"template __global__ void tp_unrolled_fwd_inner_narrow_kernel<{sig}, {channels}, 4>(")
+                out.append(fwd_args.format(""))
+            else:
+                out.append(f"template __global__ void tp_unrolled_fwd_inner_kernel<{sig}, {channels}, {V}>(")
+                out.append(typed("fwd", V))
+            out.append(f"template __global__ void tp_unrolled_bwd_inner_kernel<{sig}, {channels}, 4, {V}>(")
+            out.append(typed("bwd", V))
+            out.append(f"template __global__ void tp_unrolled_bwd_map_kernel<{sig}, {channels}, 4, {V}>(")
+            out.append(typed("bwd", V))
+            if narrow:
+                out.append(f"template __global__ void tp_unrolled_bwd_uniform_narrow_kernel<{sig}, {channels}, 4>(")
+                out.append(bwd_args.format(""))
+            else:
+                out.append(f"template __global__ void tp_unrolled_bwd_uniform_kernel<{sig}, {channels}, {V}>(")
+                out.append(typed("bwd", V))
     out += ["#endif", "", "}  // namespace e3j_amd", ""]
     return "\n".join(out)
 

@@ -255,15 +255,27 @@ int validate_tp(const e3j_amd_tp_params *p, const char *op) {
                                      ? sg.channels == p->channels_x
                                      : (tp_leading_channels_ok(p->channels_x, sg.uniform_y) &&
                                         p->num_rows * p->channels_x >= kWave);
-        if (!mode_ok || !channels_ok || p->val_dtype != E3J_AMD_F32 || p->layout != sg.layout ||
+        const bool dtype_ok = p->val_dtype == E3J_AMD_F32 || (p->val_dtype == E3J_AMD_F16 && sg.fwd_f16 != nullptr) ||
+                              (p->val_dtype == E3J_AMD_F64 && sg.fwd_f64 != nullptr);
+        if (!mode_ok || !channels_ok || !dtype_ok || p->layout != sg.layout ||
             sg.num_x != p->num_x || sg.num_y != p->num_y || sg.num_out != p->num_out)
             return set_error(E3J_AMD_INVALID_ARGUMENT,
                              name + ": operands do not match signature " + sg.name);
+        if (p->val_dtype == E3J_AMD_F64 && p->coef_classes == nullptr)
+            return set_error(E3J_AMD_INVALID_ARGUMENT,
+                             name + ": a float64 signature needs coef_classes (e3j_amd_tp_find_signature_f64)");
     }
     return E3J_AMD_OK;
 }
 
 bool absent(const void *ptr, int64_t count) { return count > 0 && ptr == nullptr; }
+
+// the coefficient classes of a float64 launch, from the caller's host array
+F64Coefs tp_classes(const e3j_amd_tp_params *p) {
+    F64Coefs c;
+    std::memcpy(c.v, p->coef_classes, sizeof(c.v));
+    return c;
+}
 
 // The unrolled kernels of the leading layout move columns in 16-byte pieces.
 const char *const kUnaligned = "tensor_product: the unrolled kernels of the leading layout need 16-byte "
@@ -294,9 +306,17 @@ extern "C" int e3j_amd_tensor_product_fwd(const e3j_amd_tp_params *p, const void
         return set_error(E3J_AMD_INVALID_ARGUMENT, "tensor_product: null operand");
     if (p->signature >= 0) {
         if (!pieces_aligned(p, {x, y, z})) return set_error(E3J_AMD_INVALID_ARGUMENT, kUnaligned);
-        const int rc = tp_signature(p->signature).fwd(p->num_rows, p->channels_x, p->coef_scale,
-                                                      static_cast<const float *>(x), static_cast<const float *>(y),
-                                                      static_cast<float *>(z), stream);
+        const TpSignature &sg = tp_signature(p->signature);
+        int rc;
+        if (p->val_dtype == E3J_AMD_F16)
+            rc = sg.fwd_f16(p->num_rows, p->channels_x, p->coef_scale, static_cast<const half_t *>(x),
+                            static_cast<const half_t *>(y), static_cast<half_t *>(z), stream);
+        else if (p->val_dtype == E3J_AMD_F64)
+            rc = sg.fwd_f64(p->num_rows, p->channels_x, tp_classes(p), static_cast<const double *>(x),
+                            static_cast<const double *>(y), static_cast<double *>(z), stream);
+        else
+            rc = sg.fwd(p->num_rows, p->channels_x, p->coef_scale, static_cast<const float *>(x),
+                        static_cast<const float *>(y), static_cast<float *>(z), stream);
         return finish_tp(p, stream, rc, "tensor_product");
     }
     const int rc = launch_product(p, p->mode, coef, x, p->num_x, p->channels_x, y, p->num_y, p->channels_y, z,
@@ -318,9 +338,20 @@ extern "C" int e3j_amd_tensor_product_bwd(const e3j_amd_tp_params *p, const void
         return set_error(E3J_AMD_INVALID_ARGUMENT, "tensor_product_bwd: null operand");
     if (p->signature >= 0) {
         if (!pieces_aligned(p, {x, y, dz, dx, dy})) return set_error(E3J_AMD_INVALID_ARGUMENT, kUnaligned);
-        const int rc = tp_signature(p->signature).bwd(
-            p->num_rows, p->channels_x, p->coef_scale, static_cast<const float *>(x), static_cast<const float *>(y),
-            static_cast<const float *>(dz), static_cast<float *>(dx), static_cast<float *>(dy), stream);
+        const TpSignature &sg = tp_signature(p->signature);
+        int rc;
+        if (p->val_dtype == E3J_AMD_F16)
+            rc = sg.bwd_f16(p->num_rows, p->channels_x, p->coef_scale, static_cast<const half_t *>(x),
+                            static_cast<const half_t *>(y), static_cast<const half_t *>(dz),
+                            static_cast<half_t *>(dx), static_cast<half_t *>(dy), stream);
+        else if (p->val_dtype == E3J_AMD_F64)
+            rc = sg.bwd_f64(p->num_rows, p->channels_x, tp_classes(p), static_cast<const double *>(x),
+                            static_cast<const double *>(y), static_cast<const double *>(dz),
+                            static_cast<double *>(dx), static_cast<double *>(dy), stream);
+        else
+            rc = sg.bwd(p->num_rows, p->channels_x, p->coef_scale, static_cast<const float *>(x),
+                        static_cast<const float *>(y), static_cast<const float *>(dz), static_cast<float *>(dx),
+                        static_cast<float *>(dy), stream);
         return finish_tp(p, stream, rc, "tensor_product_bwd");
     }
     // dx = product(table (j; i, k); dz, y), dy = product(table (k; i, j); dz, x).  The channel
@@ -363,46 +394,111 @@ extern "C" const char *e3j_amd_tp_signature_name(int id) {
     return (id >= 0 && id < num_tp_signatures()) ? tp_signature(id).name : "";
 }
 
+namespace {
+
+// entry n of a packed rank-3 table in host memory: value (as double) and the three indices
+template <typename Val>
+double tp_entry(const unsigned char *bytes, int coef_idx_bytes, int n, int32_t (&index)[3]) {
+    if (coef_idx_bytes == 1) {
+        Coef3<uint8_t, Val> e;
+        std::memcpy(&e, bytes + (size_t)n * sizeof(e), sizeof(e));
+        index[0] = e.i; index[1] = e.j; index[2] = e.k;
+        return (double)e.val;
+    }
+    Coef3<int32_t, Val> e;
+    std::memcpy(&e, bytes + (size_t)n * sizeof(e), sizeof(e));
+    index[0] = e.i; index[1] = e.j; index[2] = e.k;
+    return (double)e.val;
+}
+
+bool tp_sizes_match(const TpSignature &sg, int32_t num_coef, int32_t num_x, int32_t num_y, int32_t num_out,
+                    int32_t channels, int32_t kind, int32_t layout) {
+    if (sg.num_coef != num_coef || sg.num_x != num_x || sg.num_y != num_y || sg.num_out != num_out ||
+        sg.layout != layout || sg.uniform_y != kind)
+        return false;
+    return sg.layout == E3J_AMD_LAYOUT_TRAILING ? sg.channels == channels : tp_leading_channels_ok(channels, kind);
+}
+
+// float32 and float16 tables: one uniform positive factor is allowed between the caller's table and
+// the built-in one, taken from the entry of largest magnitude; every entry must agree with it
+// within `tolerance` (float32 rounding; for half values the rounding of the entry and of the
+// entry the factor is taken from)
+template <typename Val>
+int tp_find(const unsigned char *bytes, int32_t coef_idx_bytes, int32_t num_coef, int32_t num_x, int32_t num_y,
+            int32_t num_out, int32_t channels, int32_t kind, int32_t layout, double tolerance, bool half_kernels,
+            float *coef_scale) {
+    for (int id = 0; id < num_tp_signatures(); id++) {
+        const TpSignature &sg = tp_signature(id);
+        if (!tp_sizes_match(sg, num_coef, num_x, num_y, num_out, channels, kind, layout)) continue;
+        if (half_kernels && sg.fwd_f16 == nullptr) continue;
+        int big = 0;
+        for (int n = 1; n < num_coef; n++)
+            if (std::fabs(sg.val[n]) > std::fabs(sg.val[big])) big = n;
+        int32_t index[3];
+        const double scale = tp_entry<Val>(bytes, coef_idx_bytes, big, index) / (double)sg.val[big];
+        bool same = scale > 0.0 && std::isfinite(scale);
+        for (int n = 0; n < num_coef && same; n++) {
+            const double v = tp_entry<Val>(bytes, coef_idx_bytes, n, index);
+            for (int t = 0; t < 3 && same; t++) same = index[t] == (int32_t)sg.idx[3 * n + t];
+            const double want = scale * (double)sg.val[n];
+            same = same && std::fabs(v - want) <= tolerance * std::fabs(want);
+        }
+        if (same) {
+            if (coef_scale) *coef_scale = (float)scale;
+            return id;
+        }
+    }
+    return -1;
+}
+
+}  // namespace
+
 extern "C" int e3j_amd_tp_find_signature(const void *coef_host, int32_t coef_idx_bytes, int32_t val_dtype,
                                          int32_t num_coef, int32_t num_x, int32_t num_y, int32_t num_out,
                                          int32_t channels, int32_t kind, int32_t layout,
                                          float *coef_scale) {
     if (coef_scale) *coef_scale = 1.0f;
-    if (coef_host == nullptr || val_dtype != E3J_AMD_F32 || num_coef <= 0) return -1;
+    if (coef_host == nullptr || num_coef <= 0) return -1;
     if (coef_idx_bytes != 1 && coef_idx_bytes != 4) return -1;
-    const size_t item = coef_idx_bytes == 1 ? sizeof(Coef3<uint8_t, float>) : sizeof(Coef3<int32_t, float>);
+    const unsigned char *bytes = static_cast<const unsigned char *>(coef_host);
+    if (val_dtype == E3J_AMD_F32)
+        return tp_find<float>(bytes, coef_idx_bytes, num_coef, num_x, num_y, num_out, channels, kind, layout, 4e-7,
+                              false, coef_scale);
+    if (val_dtype == E3J_AMD_F16)
+        return tp_find<half_t>(bytes, coef_idx_bytes, num_coef, num_x, num_y, num_out, channels, kind, layout,
+                               1.5 / 1024.0, true, coef_scale);
+    return -1;
+}
+
+extern "C" int e3j_amd_tp_find_signature_f64(const void *coef_host, int32_t coef_idx_bytes, int32_t num_coef,
+                                             int32_t num_x, int32_t num_y, int32_t num_out, int32_t channels,
+                                             int32_t kind, int32_t layout, double *coef_classes) {
+    if (coef_host == nullptr || coef_classes == nullptr || num_coef <= 0) return -1;
+    if (coef_idx_bytes != 1 && coef_idx_bytes != 4) return -1;
     const unsigned char *bytes = static_cast<const unsigned char *>(coef_host);
     for (int id = 0; id < num_tp_signatures(); id++) {
         const TpSignature &sg = tp_signature(id);
-        if (sg.num_coef != num_coef || sg.num_x != num_x || sg.num_y != num_y || sg.num_out != num_out ||
-            sg.layout != layout || sg.uniform_y != kind)
-            continue;
-        if (sg.layout == E3J_AMD_LAYOUT_TRAILING ? sg.channels != channels
-                                                 : !tp_leading_channels_ok(channels, kind))
-            continue;
-        // one uniform positive factor is allowed between the tables, taken from the entry of
-        // largest magnitude; every entry must agree with it to float32 rounding
-        int big = 0;
-        for (int n = 1; n < num_coef; n++)
-            if (std::fabs(sg.val[n]) > std::fabs(sg.val[big])) big = n;
-        float vbig;
-        std::memcpy(&vbig, bytes + big * item, sizeof(float));
-        const double scale = (double)vbig / (double)sg.val[big];
-        bool same = scale > 0.0 && std::isfinite(scale);
+        if (!tp_sizes_match(sg, num_coef, num_x, num_y, num_out, channels, kind, layout)) continue;
+        if (sg.fwd_f64 == nullptr || sg.num_classes > kF64Classes) continue;
+        // same entries in the same order, the sign of every entry as built in, and within a class
+        // of equal built-in magnitude one magnitude (to float64 rounding): the kernels then
+        // compute with the caller's own values
+        double classes[kF64Classes];
+        bool seen[kF64Classes] = {};
+        for (int c = 0; c < kF64Classes; c++) classes[c] = 0.0;
+        bool same = true;
         for (int n = 0; n < num_coef && same; n++) {
-            float v;
-            std::memcpy(&v, bytes + n * item, sizeof(float));
-            for (int t = 0; t < 3 && same; t++) {
-                int32_t index;
-                if (coef_idx_bytes == 1) index = bytes[n * item + 4 + t];
-                else std::memcpy(&index, bytes + n * item + 4 + 4 * t, 4);
-                same = index == (int32_t)sg.idx[3 * n + t];
-            }
-            const double want = scale * (double)sg.val[n];
-            same = same && std::fabs((double)v - want) <= 4e-7 * std::fabs(want);
+            int32_t index[3];
+            const double v = tp_entry<double>(bytes, coef_idx_bytes, n, index);
+            for (int t = 0; t < 3 && same; t++) same = index[t] == (int32_t)sg.idx[3 * n + t];
+            const int c = sg.coef_class[n];
+            same = same && c < sg.num_classes && std::isfinite(v) && v != 0.0 && (v < 0.0) == (sg.val[n] < 0.f);
+            if (!same) break;
+            if (!seen[c]) { seen[c] = true; classes[c] = std::fabs(v); }
+            else same = std::fabs(std::fabs(v) - classes[c]) <= 1e-13 * classes[c];
         }
         if (same) {
-            if (coef_scale) *coef_scale = (float)scale;
+            std::memcpy(coef_classes, classes, sizeof(classes));
             return id;
         }
     }

@@ -1,6 +1,7 @@
-// Kernel templates of the compile-time-unrolled row-wise tensor product (gfx950, float32):
+// Kernel templates of the compile-time-unrolled row-wise tensor product (gfx950):
 // trailing-channels layout for channel counts that are multiples of 64, or 16 or 32 (first
-// part), and leading-channels layout (second part).
+// part: float32, and for whole waves of channels float16, held as half and computed in float,
+// and float64), and leading-channels layout (second part, float32).
 //
 // A generated `Sig` type supplies the straight-line Clebsch-Gordan arithmetic of one table
 // (`fwd`, `bwd`); the templates supply the wave <-> (row, 64-channel slice) mapping and the
@@ -31,6 +32,20 @@ struct TpSignature {
                hipStream_t stream);
     int (*bwd)(int64_t rows, int channels, float scale, const float *x, const float *y, const float *dz,
                float *dx, float *dy, hipStream_t stream);
+    // float16 (values held as half) and float64 forms, or null.  The float64 kernels read one
+    // coefficient per class of equal magnitude (`coef_class` of each entry, `num_classes` of them)
+    // from `classes` instead of carrying the values as literals: tables of this structure are
+    // served to float64 accuracy whatever their values were rounded to.
+    int32_t num_classes;
+    const uint8_t *coef_class;
+    int (*fwd_f16)(int64_t rows, int channels, float scale, const half_t *x, const half_t *y, half_t *z,
+                   hipStream_t stream);
+    int (*bwd_f16)(int64_t rows, int channels, float scale, const half_t *x, const half_t *y, const half_t *dz,
+                   half_t *dx, half_t *dy, hipStream_t stream);
+    int (*fwd_f64)(int64_t rows, int channels, const F64Coefs &classes, const double *x, const double *y, double *z,
+                   hipStream_t stream);
+    int (*bwd_f64)(int64_t rows, int channels, const F64Coefs &classes, const double *x, const double *y,
+                   const double *dz, double *dx, double *dy, hipStream_t stream);
 };
 // channel counts the leading-layout kernels take: MAP any multiple of 4 (16-byte pieces) with at
 // least 64 columns in all; uniform y and INNER (channel sums): whole waves per row that fit a block
@@ -44,37 +59,54 @@ const TpSignature &builtin_tp_signature(int id);
 int num_tp_signatures();
 const TpSignature &tp_signature(int id);
 
+// What the generated arithmetic takes beside its operands: nothing (the coefficients are
+// literals), or the coefficient classes of a float64 launch.
+struct TpNoCoefs {};
+// A: the type the arithmetic runs in for values held as V; Cf: the coefficient argument.
+template <typename V> struct TpValue { using A = float; using Cf = TpNoCoefs; };
+template <> struct TpValue<double> { using A = double; using Cf = F64Coefs; };
+template <typename V> using tp_arith = typename TpValue<V>::A;
+template <typename V> using tp_coefs = typename TpValue<V>::Cf;
+
 // Row of a (rows, dim, K) array seen by one lane: coordinate I lives at p[I * K].
-template <int K>
+template <int K, typename V = float>
 struct RowStore {
-    float *p;
+    V *p;
     bool on;  // lanes past the last row store nothing
     template <int I>
-    __device__ __forceinline__ void put(float v) const {
-        if (on) __builtin_nontemporal_store(v, p + I * K);
+    __device__ __forceinline__ void put(tp_arith<V> v) const {
+        if (on) __builtin_nontemporal_store((V)v, p + I * K);
     }
 };
-template <int K>
+template <int K, typename V = float>
 struct RowLoad {
-    const float *p;
-    float scale;
+    const V *p;
+    tp_arith<V> scale;
     template <int I>
-    __device__ __forceinline__ float get() const { return __builtin_nontemporal_load(p + I * K) * scale; }
+    __device__ __forceinline__ tp_arith<V> get() const {
+        return (tp_arith<V>)__builtin_nontemporal_load(p + I * K) * scale;
+    }
 };
 
 // Coordinates kept in registers (results of `fwd`, cotangents for `bwd`).
-template <int Z>
+template <int Z, typename A = float>
 struct RegStore {
-    float *v;
+    A *v;
     template <int I>
-    __device__ __forceinline__ void put(float a) const { v[I] = a; }
+    __device__ __forceinline__ void put(A a) const { v[I] = a; }
 };
-template <int Z>
+template <int Z, typename A = float>
 struct RegLoad {
-    const float *v;
+    const A *v;
     template <int I>
-    __device__ __forceinline__ float get() const { return v[I]; }
+    __device__ __forceinline__ A get() const { return v[I]; }
 };
+
+__device__ __forceinline__ double tp_vgpr(double v) {
+    asm volatile("" : "+v"(v));
+    return v;
+}
+__device__ __forceinline__ float tp_vgpr(float v) { return to_vgpr(v); }
 
 __device__ __forceinline__ int64_t tp_uniform(int64_t v) {
     const unsigned lo = __builtin_amdgcn_readfirstlane((unsigned)(v & 0xffffffffu));
@@ -107,57 +139,60 @@ struct TpTile {
     __host__ __device__ static int64_t items(int64_t rows) { return SUB > 1 ? (rows + SUB - 1) / SUB : rows * SL; }
 };
 
-template <typename Sig, int K, int WPB, bool kUniformY>
+template <typename Sig, int K, int WPB, bool kUniformY, typename V = float>
 __global__ __launch_bounds__(kWave * WPB) void tp_unrolled_fwd_kernel(
-    const float *__restrict__ x, const float *__restrict__ y, float *__restrict__ z, int64_t rows, float scale) {
+    const V *__restrict__ x, const V *__restrict__ y, V *__restrict__ z, int64_t rows, tp_arith<V> scale,
+    tp_coefs<V> cf) {
+    using A = tp_arith<V>;
     constexpr int X = Sig::X, Y = Sig::Y, Z = Sig::Z;
     const int64_t item = tp_uniform((int64_t)blockIdx.x * WPB + threadIdx.y);
     if (item >= TpTile<K>::items(rows)) return;
     const TpTile<K> t(item, threadIdx.x, rows);
     const int64_t r = t.r;
     const int c0 = t.c0;
-    float xv[X], yv[Y];
-    const float *xr = x + r * (X * K) + c0;
+    A xv[X], yv[Y];
+    const V *xr = x + r * (X * K) + c0;
 #pragma unroll
-    for (int j = 0; j < X; j++) xv[j] = __builtin_nontemporal_load(xr + j * K) * scale;
+    for (int j = 0; j < X; j++) xv[j] = (A)__builtin_nontemporal_load(xr + j * K) * scale;
     if (kUniformY) {
-        const float *yr = y + r * Y;
+        const V *yr = y + r * Y;
 #pragma unroll
-        for (int k = 0; k < Y; k++) yv[k] = yr[k];
+        for (int k = 0; k < Y; k++) yv[k] = (A)yr[k];
     } else {
-        const float *yr = y + r * (Y * K) + c0;
+        const V *yr = y + r * (Y * K) + c0;
 #pragma unroll
-        for (int k = 0; k < Y; k++) yv[k] = __builtin_nontemporal_load(yr + k * K);
+        for (int k = 0; k < Y; k++) yv[k] = (A)__builtin_nontemporal_load(yr + k * K);
     }
-    Sig::fwd(xv, yv, RowStore<K>{z + r * (Z * K) + c0, t.on});
+    Sig::fwd(xv, yv, RowStore<K, V>{z + r * (Z * K) + c0, t.on}, cf);
 }
 
 // MAP backward: dz is read once for both cotangents.
-template <typename Sig, int K, int WPB>
+template <typename Sig, int K, int WPB, typename V = float>
 __global__ __launch_bounds__(kWave * WPB) void tp_unrolled_bwd_map_kernel(
-    const float *__restrict__ x, const float *__restrict__ y, const float *__restrict__ dz,
-    float *__restrict__ dx, float *__restrict__ dy, int64_t rows, float scale) {
+    const V *__restrict__ x, const V *__restrict__ y, const V *__restrict__ dz,
+    V *__restrict__ dx, V *__restrict__ dy, int64_t rows, tp_arith<V> scale, tp_coefs<V> cf) {
+    using A = tp_arith<V>;
     constexpr int X = Sig::X, Y = Sig::Y, Z = Sig::Z;
     const int64_t item = tp_uniform((int64_t)blockIdx.x * WPB + threadIdx.y);
     if (item >= TpTile<K>::items(rows)) return;
     const TpTile<K> t(item, threadIdx.x, rows);
     const int64_t r = t.r;
     const int c0 = t.c0;
-    float xv[X], yv[Y], dxv[X], dyv[Y];
-    const float *xr = x + r * (X * K) + c0;
-    const float *yr = y + r * (Y * K) + c0;
+    A xv[X], yv[Y], dxv[X], dyv[Y];
+    const V *xr = x + r * (X * K) + c0;
+    const V *yr = y + r * (Y * K) + c0;
 #pragma unroll
-    for (int j = 0; j < X; j++) { xv[j] = __builtin_nontemporal_load(xr + j * K); dxv[j] = 0.f; }
+    for (int j = 0; j < X; j++) { xv[j] = (A)__builtin_nontemporal_load(xr + j * K); dxv[j] = A(0); }
 #pragma unroll
-    for (int k = 0; k < Y; k++) { yv[k] = __builtin_nontemporal_load(yr + k * K); dyv[k] = 0.f; }
-    Sig::bwd(xv, yv, RowLoad<K>{dz + r * (Z * K) + c0, scale}, dxv, dyv);
+    for (int k = 0; k < Y; k++) { yv[k] = (A)__builtin_nontemporal_load(yr + k * K); dyv[k] = A(0); }
+    Sig::bwd(xv, yv, RowLoad<K, V>{dz + r * (Z * K) + c0, scale}, dxv, dyv, cf);
     if (!t.on) return;
-    float *dxr = dx + r * (X * K) + c0;
-    float *dyr = dy + r * (Y * K) + c0;
+    V *dxr = dx + r * (X * K) + c0;
+    V *dyr = dy + r * (Y * K) + c0;
 #pragma unroll
-    for (int j = 0; j < X; j++) __builtin_nontemporal_store(dxv[j], dxr + j * K);
+    for (int j = 0; j < X; j++) __builtin_nontemporal_store((V)dxv[j], dxr + j * K);
 #pragma unroll
-    for (int k = 0; k < Y; k++) __builtin_nontemporal_store(dyv[k], dyr + k * K);
+    for (int k = 0; k < Y; k++) __builtin_nontemporal_store((V)dyv[k], dyr + k * K);
 }
 
 // Uniform-y backward: a wave per (row, slice); dy (rows, Y) is the channel sum: every wave
@@ -170,42 +205,43 @@ struct TpUniformGeometry {
     static constexpr int WPB = SL * RPB;
 };
 
-template <typename Sig, int K>
+template <typename Sig, int K, typename V = float>
 __global__ __launch_bounds__(kWave * TpUniformGeometry<K>::WPB) void tp_unrolled_bwd_uniform_kernel(
-    const float *__restrict__ x, const float *__restrict__ y, const float *__restrict__ dz,
-    float *__restrict__ dx, float *__restrict__ dy, int64_t rows, float scale) {
+    const V *__restrict__ x, const V *__restrict__ y, const V *__restrict__ dz,
+    V *__restrict__ dx, V *__restrict__ dy, int64_t rows, tp_arith<V> scale, tp_coefs<V> cf) {
+    using A = tp_arith<V>;
     constexpr int X = Sig::X, Y = Sig::Y, Z = Sig::Z;
     using G = TpUniformGeometry<K>;
-    using Red = WaveReduceBlocks<Y>;
-    __shared__ float partial[G::WPB][Red::P];
+    using Red = WaveReduceBlocks<Y, kWave, A>;
+    __shared__ A partial[G::WPB][Red::P];
     const int wave = threadIdx.y, lane = threadIdx.x;
     const int slice = wave % G::SL;
     const int64_t r = tp_uniform((int64_t)blockIdx.x * G::RPB + wave / G::SL);
     const bool valid = r < rows;  // uniform per wave; every wave reaches the barrier
     if (valid) {
-        float yv[Y], dyv[Red::P], xv[X], dxv[X];
-        const float *yr = y + r * Y;
+        A yv[Y], dyv[Red::P], xv[X], dxv[X];
+        const V *yr = y + r * Y;
 #pragma unroll
-        for (int k = 0; k < Y; k++) yv[k] = to_vgpr(yr[k]);
+        for (int k = 0; k < Y; k++) yv[k] = tp_vgpr((A)yr[k]);
 #pragma unroll
-        for (int k = 0; k < Red::P; k++) dyv[k] = 0.f;
+        for (int k = 0; k < Red::P; k++) dyv[k] = A(0);
         const int c0 = slice * kWave + lane;
-        const float *xr = x + r * (X * K) + c0;
+        const V *xr = x + r * (X * K) + c0;
 #pragma unroll
-        for (int j = 0; j < X; j++) { xv[j] = __builtin_nontemporal_load(xr + j * K); dxv[j] = 0.f; }
-        Sig::bwd(xv, yv, RowLoad<K>{dz + r * (Z * K) + c0, scale}, dxv, dyv);
-        float *dxr = dx + r * (X * K) + c0;
+        for (int j = 0; j < X; j++) { xv[j] = (A)__builtin_nontemporal_load(xr + j * K); dxv[j] = A(0); }
+        Sig::bwd(xv, yv, RowLoad<K, V>{dz + r * (Z * K) + c0, scale}, dxv, dyv, cf);
+        V *dxr = dx + r * (X * K) + c0;
 #pragma unroll
-        for (int j = 0; j < X; j++) __builtin_nontemporal_store(dxv[j], dxr + j * K);
-        float *mine = partial[wave];
-        Red::run(dyv, lane, [&](int k, float total) { mine[k] = total; });
+        for (int j = 0; j < X; j++) __builtin_nontemporal_store((V)dxv[j], dxr + j * K);
+        A *mine = partial[wave];
+        Red::run(dyv, lane, [&](int k, A total) { mine[k] = total; });
     }
     __syncthreads();
     if (valid && slice == 0 && lane < Y) {
-        float total = partial[wave][lane];
+        A total = partial[wave][lane];
 #pragma unroll
         for (int s2 = 1; s2 < G::SL; s2++) total += partial[wave + s2][lane];
-        dy[r * Y + lane] = total;
+        dy[r * Y + lane] = (V)total;
     }
 }
 
@@ -213,82 +249,85 @@ __global__ __launch_bounds__(kWave * TpUniformGeometry<K>::WPB) void tp_unrolled
 // on registers, reduces its 64 channels sixteen coordinates at a time, and the slices of a row
 // meet in LDS as in the uniform-y backward.  Its backward is the MAP backward with a
 // wave-uniform cotangent (scalar loads).
-template <int Z>
+template <int Z, typename V = float>
 struct UniformLoad {
-    const float *p;
-    float scale;
+    const V *p;
+    tp_arith<V> scale;
     template <int I>
-    __device__ __forceinline__ float get() const { return p[I] * scale; }
+    __device__ __forceinline__ tp_arith<V> get() const { return (tp_arith<V>)p[I] * scale; }
 };
 
 // sums of zv[0..Z) over the lanes of the wave into out[0..Z) (LDS, one row per wave)
-template <int Z>
-__device__ __forceinline__ void tp_reduce_columns(const float *zv, float *out, int lane) {
-    using Red = WaveReduceBlocks<Z>;
-    float padded[Red::P];
+template <int Z, typename A = float>
+__device__ __forceinline__ void tp_reduce_columns(const A *zv, A *out, int lane) {
+    using Red = WaveReduceBlocks<Z, kWave, A>;
+    A padded[Red::P];
 #pragma unroll
-    for (int t = 0; t < Red::P; t++) padded[t] = t < Z ? zv[t] : 0.f;
-    Red::run(padded, lane, [&](int i, float total) { out[i] = total; });
+    for (int t = 0; t < Red::P; t++) padded[t] = t < Z ? zv[t] : A(0);
+    Red::run(padded, lane, [&](int i, A total) { out[i] = total; });
 }
 
-template <typename Sig, int K>
+template <typename Sig, int K, typename V = float>
 __global__ __launch_bounds__(kWave * TpUniformGeometry<K>::WPB) void tp_unrolled_fwd_inner_kernel(
-    const float *__restrict__ x, const float *__restrict__ y, float *__restrict__ z, int64_t rows, float scale) {
+    const V *__restrict__ x, const V *__restrict__ y, V *__restrict__ z, int64_t rows, tp_arith<V> scale,
+    tp_coefs<V> cf) {
+    using A = tp_arith<V>;
     constexpr int X = Sig::X, Y = Sig::Y, Z = Sig::Z;
     using G = TpUniformGeometry<K>;
-    __shared__ float partial[G::WPB][Z];
+    __shared__ A partial[G::WPB][Z];
     const int wave = threadIdx.y, lane = threadIdx.x;
     const int slice = wave % G::SL;
     const int64_t r = tp_uniform((int64_t)blockIdx.x * G::RPB + wave / G::SL);
     const bool valid = r < rows;  // uniform per wave; every wave reaches the barrier
     if (valid) {
         const int c0 = slice * kWave + lane;
-        float xv[X], yv[Y], zv[Z];
-        const float *xr = x + r * (X * K) + c0;
-        const float *yr = y + r * (Y * K) + c0;
+        A xv[X], yv[Y], zv[Z];
+        const V *xr = x + r * (X * K) + c0;
+        const V *yr = y + r * (Y * K) + c0;
 #pragma unroll
-        for (int j = 0; j < X; j++) xv[j] = __builtin_nontemporal_load(xr + j * K) * scale;
+        for (int j = 0; j < X; j++) xv[j] = (A)__builtin_nontemporal_load(xr + j * K) * scale;
 #pragma unroll
-        for (int k = 0; k < Y; k++) yv[k] = __builtin_nontemporal_load(yr + k * K);
-        Sig::fwd(xv, yv, RegStore<Z>{zv});
-        tp_reduce_columns<Z>(zv, partial[wave], lane);
+        for (int k = 0; k < Y; k++) yv[k] = (A)__builtin_nontemporal_load(yr + k * K);
+        Sig::fwd(xv, yv, RegStore<Z, A>{zv}, cf);
+        tp_reduce_columns<Z, A>(zv, partial[wave], lane);
     }
     __syncthreads();
     if (valid && slice == 0) {
         for (int i = lane; i < Z; i += kWave) {
-            float total = partial[wave][i];
+            A total = partial[wave][i];
 #pragma unroll
             for (int s2 = 1; s2 < G::SL; s2++) total += partial[wave + s2][i];
-            z[r * Z + i] = total;
+            z[r * Z + i] = (V)total;
         }
     }
 }
 
-template <typename Sig, int K, int WPB>
+template <typename Sig, int K, int WPB, typename V = float>
 __global__ __launch_bounds__(kWave * WPB) void tp_unrolled_bwd_inner_kernel(
-    const float *__restrict__ x, const float *__restrict__ y, const float *__restrict__ dz,
-    float *__restrict__ dx, float *__restrict__ dy, int64_t rows, float scale) {
+    const V *__restrict__ x, const V *__restrict__ y, const V *__restrict__ dz,
+    V *__restrict__ dx, V *__restrict__ dy, int64_t rows, tp_arith<V> scale, tp_coefs<V> cf) {
+    using A = tp_arith<V>;
     constexpr int X = Sig::X, Y = Sig::Y, Z = Sig::Z;
     const int64_t item = tp_uniform((int64_t)blockIdx.x * WPB + threadIdx.y);
     if (item >= TpTile<K>::items(rows)) return;
     const TpTile<K> t(item, threadIdx.x, rows);
     const int64_t r = t.r;
     const int c0 = t.c0;
-    float xv[X], yv[Y], dxv[X], dyv[Y];
-    const float *xr = x + r * (X * K) + c0;
-    const float *yr = y + r * (Y * K) + c0;
+    A xv[X], yv[Y], dxv[X], dyv[Y];
+    const V *xr = x + r * (X * K) + c0;
+    const V *yr = y + r * (Y * K) + c0;
 #pragma unroll
-    for (int j = 0; j < X; j++) { xv[j] = __builtin_nontemporal_load(xr + j * K); dxv[j] = 0.f; }
+    for (int j = 0; j < X; j++) { xv[j] = (A)__builtin_nontemporal_load(xr + j * K); dxv[j] = A(0); }
 #pragma unroll
-    for (int k = 0; k < Y; k++) { yv[k] = __builtin_nontemporal_load(yr + k * K); dyv[k] = 0.f; }
-    Sig::bwd(xv, yv, UniformLoad<Z>{dz + r * Z, scale}, dxv, dyv);
+    for (int k = 0; k < Y; k++) { yv[k] = (A)__builtin_nontemporal_load(yr + k * K); dyv[k] = A(0); }
+    Sig::bwd(xv, yv, UniformLoad<Z, V>{dz + r * Z, scale}, dxv, dyv, cf);
     if (!t.on) return;
-    float *dxr = dx + r * (X * K) + c0;
-    float *dyr = dy + r * (Y * K) + c0;
+    V *dxr = dx + r * (X * K) + c0;
+    V *dyr = dy + r * (Y * K) + c0;
 #pragma unroll
-    for (int j = 0; j < X; j++) __builtin_nontemporal_store(dxv[j], dxr + j * K);
+    for (int j = 0; j < X; j++) __builtin_nontemporal_store((V)dxv[j], dxr + j * K);
 #pragma unroll
-    for (int k = 0; k < Y; k++) __builtin_nontemporal_store(dyv[k], dyr + k * K);
+    for (int k = 0; k < Y; k++) __builtin_nontemporal_store((V)dyv[k], dyr + k * K);
 }
 
 // 16 or 32 channels, kinds that sum over the channels: the groups of K lanes reduce on their
@@ -356,55 +395,90 @@ inline int tp_grid(int64_t items, int wpb, unsigned *blocks) {
     return E3J_AMD_OK;
 }
 
-// kKind: 0 MAP, 1 OUTER with a channel-free y, 2 INNER
-template <typename Sig, int K, int kKind>
-int launch_tp_unrolled_fwd(int64_t rows, int, float scale, const float *x, const float *y, float *z,
-                           hipStream_t stream) {
+// kKind: 0 MAP, 1 OUTER with a channel-free y, 2 INNER; V: the type the values are held in
+template <typename Sig, int K, int kKind, typename V>
+int launch_tp_unrolled_fwd_t(int64_t rows, tp_arith<V> scale, const tp_coefs<V> &cf, const V *x, const V *y, V *z,
+                             hipStream_t stream) {
     constexpr int WPB = 4;
     if (rows == 0) return E3J_AMD_OK;
     unsigned blocks;
     if constexpr (kKind == 2 && TpTile<K>::SUB > 1) {
+        static_assert(std::is_same<V, float>::value, "16 / 32 channels: float32 only");
         if (int rc = tp_grid(TpTile<K>::items(rows), WPB, &blocks)) return rc;
         hipLaunchKernelGGL((tp_unrolled_fwd_inner_narrow_kernel<Sig, K, WPB>), dim3(blocks), dim3(kWave, WPB), 0,
                            stream, x, y, z, rows, scale);
     } else if constexpr (kKind == 2) {
         using G = TpUniformGeometry<K>;
         if (int rc = tp_grid(rows, G::RPB, &blocks)) return rc;
-        hipLaunchKernelGGL((tp_unrolled_fwd_inner_kernel<Sig, K>), dim3(blocks), dim3(kWave, G::WPB), 0, stream,
-                           x, y, z, rows, scale);
+        hipLaunchKernelGGL((tp_unrolled_fwd_inner_kernel<Sig, K, V>), dim3(blocks), dim3(kWave, G::WPB), 0, stream,
+                           x, y, z, rows, scale, cf);
     } else {
         if (int rc = tp_grid(TpTile<K>::items(rows), WPB, &blocks)) return rc;
-        hipLaunchKernelGGL((tp_unrolled_fwd_kernel<Sig, K, WPB, kKind == 1>), dim3(blocks), dim3(kWave, WPB), 0,
-                           stream, x, y, z, rows, scale);
+        hipLaunchKernelGGL((tp_unrolled_fwd_kernel<Sig, K, WPB, kKind == 1, V>), dim3(blocks), dim3(kWave, WPB), 0,
+                           stream, x, y, z, rows, scale, cf);
     }
     return check_hip(hipGetLastError(), "tensor_product (unrolled) launch");
 }
 
-template <typename Sig, int K, int kKind>
-int launch_tp_unrolled_bwd(int64_t rows, int, float scale, const float *x, const float *y, const float *dz,
-                           float *dx, float *dy, hipStream_t stream) {
+template <typename Sig, int K, int kKind, typename V>
+int launch_tp_unrolled_bwd_t(int64_t rows, tp_arith<V> scale, const tp_coefs<V> &cf, const V *x, const V *y,
+                             const V *dz, V *dx, V *dy, hipStream_t stream) {
     constexpr int WPB = 4;
     if (rows == 0) return E3J_AMD_OK;
     unsigned blocks;
     if constexpr (kKind == 2) {
         if (int rc = tp_grid(TpTile<K>::items(rows), WPB, &blocks)) return rc;
-        hipLaunchKernelGGL((tp_unrolled_bwd_inner_kernel<Sig, K, WPB>), dim3(blocks), dim3(kWave, WPB), 0, stream,
-                           x, y, dz, dx, dy, rows, scale);
+        hipLaunchKernelGGL((tp_unrolled_bwd_inner_kernel<Sig, K, WPB, V>), dim3(blocks), dim3(kWave, WPB), 0, stream,
+                           x, y, dz, dx, dy, rows, scale, cf);
     } else if constexpr (kKind == 1 && TpTile<K>::SUB > 1) {
+        static_assert(std::is_same<V, float>::value, "16 / 32 channels: float32 only");
         if (int rc = tp_grid(TpTile<K>::items(rows), WPB, &blocks)) return rc;
         hipLaunchKernelGGL((tp_unrolled_bwd_uniform_narrow_kernel<Sig, K, WPB>), dim3(blocks), dim3(kWave, WPB), 0,
                            stream, x, y, dz, dx, dy, rows, scale);
     } else if constexpr (kKind == 1) {
         using G = TpUniformGeometry<K>;
         if (int rc = tp_grid(rows, G::RPB, &blocks)) return rc;
-        hipLaunchKernelGGL((tp_unrolled_bwd_uniform_kernel<Sig, K>), dim3(blocks), dim3(kWave, G::WPB), 0, stream,
-                           x, y, dz, dx, dy, rows, scale);
+        hipLaunchKernelGGL((tp_unrolled_bwd_uniform_kernel<Sig, K, V>), dim3(blocks), dim3(kWave, G::WPB), 0, stream,
+                           x, y, dz, dx, dy, rows, scale, cf);
     } else {
         if (int rc = tp_grid(TpTile<K>::items(rows), WPB, &blocks)) return rc;
-        hipLaunchKernelGGL((tp_unrolled_bwd_map_kernel<Sig, K, WPB>), dim3(blocks), dim3(kWave, WPB), 0, stream,
-                           x, y, dz, dx, dy, rows, scale);
+        hipLaunchKernelGGL((tp_unrolled_bwd_map_kernel<Sig, K, WPB, V>), dim3(blocks), dim3(kWave, WPB), 0, stream,
+                           x, y, dz, dx, dy, rows, scale, cf);
     }
     return check_hip(hipGetLastError(), "tensor_product_bwd (unrolled) launch");
+}
+
+// the registry's entry points: float32, float16 (whole waves of channels), float64 (the same; the
+// uniform factor of the table is part of its coefficient classes)
+template <typename Sig, int K, int kKind>
+int launch_tp_unrolled_fwd(int64_t rows, int, float scale, const float *x, const float *y, float *z,
+                           hipStream_t stream) {
+    return launch_tp_unrolled_fwd_t<Sig, K, kKind, float>(rows, scale, TpNoCoefs{}, x, y, z, stream);
+}
+template <typename Sig, int K, int kKind>
+int launch_tp_unrolled_bwd(int64_t rows, int, float scale, const float *x, const float *y, const float *dz,
+                           float *dx, float *dy, hipStream_t stream) {
+    return launch_tp_unrolled_bwd_t<Sig, K, kKind, float>(rows, scale, TpNoCoefs{}, x, y, dz, dx, dy, stream);
+}
+template <typename Sig, int K, int kKind>
+int launch_tp_unrolled_fwd_f16(int64_t rows, int, float scale, const half_t *x, const half_t *y, half_t *z,
+                               hipStream_t stream) {
+    return launch_tp_unrolled_fwd_t<Sig, K, kKind, half_t>(rows, scale, TpNoCoefs{}, x, y, z, stream);
+}
+template <typename Sig, int K, int kKind>
+int launch_tp_unrolled_bwd_f16(int64_t rows, int, float scale, const half_t *x, const half_t *y, const half_t *dz,
+                               half_t *dx, half_t *dy, hipStream_t stream) {
+    return launch_tp_unrolled_bwd_t<Sig, K, kKind, half_t>(rows, scale, TpNoCoefs{}, x, y, dz, dx, dy, stream);
+}
+template <typename Sig, int K, int kKind>
+int launch_tp_unrolled_fwd_f64(int64_t rows, int, const F64Coefs &classes, const double *x, const double *y,
+                               double *z, hipStream_t stream) {
+    return launch_tp_unrolled_fwd_t<Sig, K, kKind, double>(rows, 1.0, classes, x, y, z, stream);
+}
+template <typename Sig, int K, int kKind>
+int launch_tp_unrolled_bwd_f64(int64_t rows, int, const F64Coefs &classes, const double *x, const double *y,
+                               const double *dz, double *dx, double *dy, hipStream_t stream) {
+    return launch_tp_unrolled_bwd_t<Sig, K, kKind, double>(rows, 1.0, classes, x, y, dz, dx, dy, stream);
 }
 
 // ---------------------------------------------------------------------------

@@ -68,20 +68,28 @@ class _Table:
     def signature(self, num_x: int, num_y: int, num_out: int, channels: int, kind: int,
                   layout: Layout = Layout.TRAILING_CHANNELS):
         """`(id, scale)` of a built-in unrolled kernel, `(-1, 1.0)` if none matches.  `kind`: 0 MAP,
-        1 OUTER with a channel-free y, 2 INNER."""
+        1 OUTER with a channel-free y, 2 INNER.  For a float64 table `scale` is the ctypes array of
+        its coefficient classes (`e3j_amd_tp_params.coef_classes`)."""
         kind = int(kind)
         key = (num_x, num_y, num_out, channels, kind, layout, config().jit)
         hit = self._signature.get(key)
         if hit is None:
             scale = ctypes.c_float(1.0)
+            classes = (ctypes.c_double * _lib.F64_CLASSES)()
+            f64 = self.val_np_dtype == np.float64
             sig = -1
 
             def find():
+                if f64:
+                    return int(_lib.load().e3j_amd_tp_find_signature_f64(
+                        self.packed.ctypes.data, self.idx_bytes, self.num_coef, num_x, num_y, num_out, channels,
+                        kind, layout.value, classes))
+                code = _lib.F16 if self.val_np_dtype == np.float16 else _lib.F32
                 return int(_lib.load().e3j_amd_tp_find_signature(
-                    self.packed.ctypes.data, self.idx_bytes, _lib.F32, self.num_coef, num_x, num_y, num_out,
+                    self.packed.ctypes.data, self.idx_bytes, code, self.num_coef, num_x, num_y, num_out,
                     channels, kind, layout.value, ctypes.byref(scale)))
 
-            if self.val_np_dtype == np.float32 and self.num_coef > 0:
+            if self.num_coef > 0:
                 sig = find()
                 if sig < 0 and config().jit:
                     # not built in: generate and compile the kernels of this table, then look again
@@ -91,7 +99,7 @@ class _Table:
                     if (channels % 64 == 0 or channels in (16, 32) or not trailing) and _jit.register_tp(
                             c.val, c.idx.astype(np.int64), (num_out, num_x, num_y), channels if trailing else 0):
                         sig = find()
-            hit = self._signature[key] = (sig, float(scale.value))
+            hit = self._signature[key] = (sig, classes if f64 else float(scale.value))
         return hit
 
     @classmethod
@@ -160,21 +168,28 @@ def _params(meta: _Meta, x: torch.Tensor, y: torch.Tensor, backward: bool, dz=No
     # unrolled kernels: float32, MAP, OUTER with a channel-free y, or INNER; the leading-layout ones
     # need 64 columns in all and 16-byte aligned operands
     sig, scale = -1, 1.0
-    usable = x.dtype == torch.float32 and (
-        meta.layout == Layout.TRAILING_CHANNELS or
-        (int(x.shape[0]) * cx >= 64 and all(t.data_ptr() % 16 == 0 for t in (x, y, dz) if t is not None)))
+    # (float16 / float64: trailing layout, whole waves of channels; the look-up knows)
+    usable = (meta.layout == Layout.TRAILING_CHANNELS or
+              (x.dtype == torch.float32 and int(x.shape[0]) * cx >= 64 and
+               all(t.data_ptr() % 16 == 0 for t in (x, y, dz) if t is not None)))
     if usable and meta.mode == MixingMode.MAP:
         sig, scale = meta.table.signature(num_x, num_y, meta.num_out, cx, 0, meta.layout)
     elif usable and meta.mode == MixingMode.OUTER and cy == 1 and cx > 1:
         sig, scale = meta.table.signature(num_x, num_y, meta.num_out, cx, 1, meta.layout)
     elif usable and meta.mode == MixingMode.INNER:
         sig, scale = meta.table.signature(num_x, num_y, meta.num_out, cx, 2, meta.layout)
-    return _lib.TpParams(
+    classes = None
+    if not isinstance(scale, float):   # float64: the coefficient classes take the place of the factor
+        classes, scale = scale, 1.0
+    p = _lib.TpParams(
         signature=sig, coef_scale=scale,
         num_rows=int(x.shape[0]), num_coef=meta.table.num_coef, num_x=num_x, num_y=num_y,
         num_out=meta.num_out, channels_x=cx, channels_y=cy, mode=meta.mode.value, layout=meta.layout.value,
         val_dtype=_VAL_DTYPES[x.dtype][0], coef_idx_bytes=meta.table.idx_bytes,
         coef_sorted=1 if (backward or meta.table.sorted) else 0, debug=int(config().debug_level))
+    if classes is not None and sig >= 0:
+        p.coef_classes = ctypes.cast(classes, ctypes.c_void_p).value   # (kept alive by the table's cache)
+    return p
 
 
 def _raw_forward(meta: _Meta, x: torch.Tensor, y: torch.Tensor) -> torch.Tensor:

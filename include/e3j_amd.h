@@ -489,6 +489,9 @@ typedef struct e3j_amd_tp_params {
     int32_t debug;
     int32_t signature;      /* id from e3j_amd_tp_find_signature, or -1: table-driven kernel */
     float   coef_scale;     /* unrolled kernels: table = coef_scale * built-in table */
+    /* float64 with a signature: the E3J_AMD_F64_CLASSES coefficient classes that
+     * e3j_amd_tp_find_signature_f64 returned for the table, in HOST memory (read during the call). */
+    const double *coef_classes;
 } e3j_amd_tp_params;
 int e3j_amd_tensor_product_fwd(const e3j_amd_tp_params *p, const void *coef, const void *x, const void *y,
                                void *z, void *stream);
@@ -501,19 +504,29 @@ int e3j_amd_tensor_product_fwd(const e3j_amd_tp_params *p, const void *coef, con
 int e3j_amd_tensor_product_bwd(const e3j_amd_tp_params *p, const void *coef_bwd, const void *x, const void *y,
                                const void *dz, void *dx, void *dy, void *stream);
 
-/* Compile-time-unrolled kernels of the tensor product exist for built-in Clebsch-Gordan tables,
- * float32 and three channel modes, `kind` 0 MAP, 1 OUTER with channels_y == 1, 2 INNER: in the
- * trailing layout for the channel counts they were built for (64, 128), in the leading layout
- * for any multiple of 4 channels (kinds 1 and 2, which sum over the channels: 64, 128 or 256),
- * operands 16-byte aligned and num_rows * channels >= 64.  The lookup compares a
- * packed forward table in HOST memory with the built-in ones (same entries in the same order, up
- * to one positive factor returned in *coef_scale) and returns an id for
- * e3j_amd_tp_params.signature, or -1.  With a signature the `coef` / `coef_bwd` operands of the
- * two entry points above are not read and may be NULL.  No counterpart in the reference, whose
- * kernels are table-driven only. */
+/* Compile-time-unrolled kernels of the tensor product exist for built-in Clebsch-Gordan tables
+ * and three channel modes, `kind` 0 MAP, 1 OUTER with channels_y == 1, 2 INNER: in the
+ * trailing layout for the channel counts they were built for (32, 64, 128; float16 and float64
+ * operands: 64, 128), in the leading layout (float32) for any multiple of 4 channels (kinds 1 and
+ * 2, which sum over the channels: 64, 128 or 256), operands 16-byte aligned and num_rows *
+ * channels >= 64.  The lookup compares a packed forward table in HOST memory (val_dtype
+ * E3J_AMD_F32 or E3J_AMD_F16) with the built-in ones (same entries in the same order, up to one
+ * positive factor returned in *coef_scale; half values within their rounding) and returns an id
+ * for e3j_amd_tp_params.signature, or -1.  With a signature the `coef` / `coef_bwd` operands of
+ * the two entry points above are not read and may be NULL.  No counterpart in the reference,
+ * whose kernels are table-driven only. */
 int e3j_amd_tp_find_signature(const void *coef_host, int32_t coef_idx_bytes, int32_t val_dtype,
                               int32_t num_coef, int32_t num_x, int32_t num_y, int32_t num_out,
                               int32_t channels, int32_t kind, int32_t layout, float *coef_scale);
+/* The same for a table of float64 values.  The float64 kernels carry no coefficient values: they
+ * read one value per class of entries that have one magnitude in the built-in table, so the
+ * caller's table may hold any values of that structure (float32-rounded ones, exact ones, a
+ * normalisation folded in), provided the entries of a class agree to float64 rounding and every
+ * sign is the built-in one.  coef_classes: E3J_AMD_F64_CLASSES doubles, filled on a match; pass
+ * them in e3j_amd_tp_params.coef_classes. */
+int e3j_amd_tp_find_signature_f64(const void *coef_host, int32_t coef_idx_bytes, int32_t num_coef,
+                                  int32_t num_x, int32_t num_y, int32_t num_out, int32_t channels,
+                                  int32_t kind, int32_t layout, double *coef_classes);
 int e3j_amd_tp_num_signatures(void);
 const char *e3j_amd_tp_signature_name(int id);
 /* Adds the kernels of one table compiled at run time (an entry produced by the generator of this

@@ -44,9 +44,9 @@ def test_params_struct_matches_header():
 def test_tensor_product_params_struct_matches_header():
     header = open(os.path.join(ROOT, "include", "e3j_amd.h")).read()
     body = re.search(r"typedef struct e3j_amd_tp_params \{(.*?)\} e3j_amd_tp_params;", header, re.S).group(1)
-    fields = re.findall(r"^\s*(int32_t|int64_t|float)\s*(\w+);", body, re.M)
+    fields = re.findall(r"^\s*(const double \*|int32_t|int64_t|float)\s*(\w+);", body, re.M)
     assert [name for _, name in fields] == [name for name, _ in _lib.TpParams._fields_]
-    ctype = {"int32_t": C.c_int32, "int64_t": C.c_int64, "float": C.c_float}
+    ctype = {"int32_t": C.c_int32, "int64_t": C.c_int64, "float": C.c_float, "const double *": C.c_void_p}
     assert [ctype[t] for t, _ in fields] == [t for _, t in _lib.TpParams._fields_]
     modes = re.search(r"E3J_AMD_MODE_OUTER = (\d), E3J_AMD_MODE_INNER = (\d), E3J_AMD_MODE_MAP = (\d)", header)
     assert tuple(map(int, modes.groups())) == (_lib.MODE_OUTER, _lib.MODE_INNER, _lib.MODE_MAP)

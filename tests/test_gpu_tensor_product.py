@@ -431,3 +431,138 @@ def test_float16_operands(mode, layout, idx_dtype):
     for got, r, m, name in ((z, ref, mag, "z"), (dx, rdx, mdx, "dx"), (dy, rdy, mdy, "dy")):
         err = np.abs(got.detach().float().cpu().numpy().astype(np.float64) - r)
         assert np.all(err <= 8 * eps * m + 1e-3), f"{name}: {err.max()} against magnitude {m.max()}"
+
+
+# ---------------------------------------------------------------------------
+# compile-time-unrolled kernels in float16 and float64 (trailing layout, whole waves of channels)
+# ---------------------------------------------------------------------------
+def _unrolled_case(spaces, mode, channels, np_dtype, factor, rows=77, seed=31):
+    rng = np.random.default_rng(seed)
+    tp = TensorProduct(spaces[:2], spaces[2], layout="TRAILING_CHANNELS", mode=mode)
+    Z, X, Y = tp.shape
+    idx = np.asarray(tp.indices, dtype=np.int64)
+    val = (factor * np.asarray(tp.values, dtype=np.float64)).astype(np_dtype)
+    x, y = _operands(rng, mode, "TRAILING_CHANNELS", channels, rows=rows, dims=(X, Y), has=(True, False))
+    x, y = (0.5 * x).astype(np_dtype), (0.5 * y).astype(np_dtype)
+    return tp, idx, val, x, y, rng
+
+
+@pytest.mark.parametrize("spaces,channels", [(BUILTIN[t], k) for t in range(3) for k in (64, 128)],
+                         ids=lambda v: str(v) if isinstance(v, int) else "-".join(str(a) for a in v))
+@pytest.mark.parametrize("mode", ["MAP", "OUTER", "INNER"])
+@pytest.mark.parametrize("dtype", ["float64", "float16"])
+def test_unrolled_kernels_in_float64_and_float16(spaces, channels, mode, dtype):
+    """The operator on a built-in table in float64 / float16: an unrolled kernel serves it (the
+    look-up says so) and the results match the float64 checker on the table's own values: within
+    64 float64 roundings of the sum of magnitudes, or within half-precision rounding (the
+    float16 kernels compute in float with the built-in table times one factor, which differs from
+    the half-rounded entries by their rounding)."""
+    from e3j_amd.tp_ops import _Table
+    np_dtype = np.dtype(dtype)
+    tp, idx, val, x, y, rng = _unrolled_case(spaces, mode, channels, np_dtype, 1.5)
+    Z, X, Y = tp.shape
+    packed = Coef(val, idx, dtype, "uint8").pack()
+    sig, _ = _Table.get(packed, np_dtype).signature(X, Y, Z, channels, KIND[mode])
+    assert sig >= 0, "a built-in unrolled kernel must serve this table"
+    p = TensorProductParams(num_out=Z, mode=mode, layout="TRAILING_CHANNELS")
+    xt, yt = (torch.from_numpy(a).to(DEV).requires_grad_(True) for a in (x, y))
+    z = e3j_amd.tensor_product(packed, xt, yt, p)
+    assert z.dtype == getattr(torch, dtype)
+    dz = (0.5 * rng.normal(size=tuple(z.shape))).astype(np_dtype)
+    dx, dy = torch.autograd.grad(z, (xt, yt), torch.from_numpy(dz).to(DEV))
+    f64 = lambda a: a.astype(np.float64)  # noqa: E731
+    v = f64(val)
+    lay = "TRAILING_CHANNELS"
+    ref = T.tensor_product_unfused(idx, v, f64(x), f64(y), Z, mode, lay)
+    mag = T.tensor_product_unfused(idx, np.abs(v), np.abs(f64(x)), np.abs(f64(y)), Z, mode, lay)
+    rdx, rdy = T.tensor_product_vjp(idx, v, f64(x), f64(y), f64(dz), mode, lay)
+    mdx, mdy = T.tensor_product_vjp(idx, np.abs(v), np.abs(f64(x)), np.abs(f64(y)), np.abs(f64(dz)), mode, lay)
+    for got, r, m, name in ((z, ref, mag, "z"), (dx, rdx, mdx, "dx"), (dy, rdy, mdy, "dy")):
+        err = np.abs(got.detach().double().cpu().numpy() - r)
+        bound = 64 * 2.0 ** -52 * m + 1e-300 if dtype == "float64" else 8 * 2.0 ** -10 * m + 1e-3
+        assert np.all(err <= bound), f"{name}: {err.max()} against magnitude {m.max()}"
+
+
+@pytest.mark.parametrize("mode", ["MAP", "OUTER", "INNER"])
+def test_float64_classes_serve_exact_and_rounded_tables(mode):
+    """The float64 kernels take their coefficients from the caller's table: a table of exact
+    double values (what a float64 front end builds) and the same table rounded to float32 both
+    find the signature, and each result follows its own table to float64 accuracy."""
+    from e3j_amd.tp_ops import _Table
+    spaces, K = BUILTIN[2], 64
+    tp, idx, _, x, y, rng = _unrolled_case(spaces, mode, K, np.dtype("float64"), 1.0, rows=33)
+    Z, X, Y = tp.shape
+    rounded = np.asarray(tp.values, dtype=np.float32).astype(np.float64)
+    # exact values: what the float32 entries were rounded from, recovered through their squares
+    # (squares of the entries of a Clebsch-Gordan table are small rationals)
+    from fractions import Fraction
+    exact = np.array([np.sign(v) * np.sqrt(float(Fraction(float(v) ** 2).limit_denominator(10000))) for v in rounded])
+    assert 0 < np.abs(exact - rounded).max() < 1e-7
+    p = TensorProductParams(num_out=Z, mode=mode, layout="TRAILING_CHANNELS")
+    xt, yt = torch.from_numpy(x).to(DEV), torch.from_numpy(y).to(DEV)
+    outs = []
+    for val in (rounded, exact):
+        packed = Coef(val, idx, "float64", "uint8").pack()
+        sig, classes = _Table.get(packed, np.dtype("float64")).signature(X, Y, Z, K, KIND[mode])
+        assert sig >= 0
+        z = e3j_amd.tensor_product(packed, xt, yt, p).cpu().numpy()
+        ref = T.tensor_product_unfused(idx, val, x, y, Z, mode, "TRAILING_CHANNELS")
+        mag = T.tensor_product_unfused(idx, np.abs(val), np.abs(x), np.abs(y), Z, mode, "TRAILING_CHANNELS")
+        assert np.all(np.abs(z - ref) <= 64 * 2.0 ** -52 * mag + 1e-300)
+        outs.append(z)
+    assert np.abs(outs[0] - outs[1]).max() > 1e-10   # (the two tables do differ)
+    # a table of another structure is refused: one entry of a class changed
+    broken = exact.copy()
+    broken[5] *= 1.0 + 1e-9
+    packed = Coef(broken, idx, "float64", "uint8").pack()
+    assert _Table.get(packed, np.dtype("float64")).signature(X, Y, Z, K, KIND[mode])[0] == -1
+
+
+@pytest.mark.parametrize("dtype", ["float64", "float16"])
+def test_unrolled_float64_float16_through_the_c_abi(dtype):
+    """The C ABI with a signature in float64 / float16 against the table-driven kernels of the
+    same call (signature -1), MAP mode, 301 rows."""
+    lib = _lib.load()
+    np_dtype, tdtype = np.dtype(dtype), getattr(torch, dtype)
+    tp = TensorProduct(("0e+1o+2e+3o", "0e+1o+2e+3o"), "0e+1o+2e+3o", layout="TRAILING_CHANNELS", mode="MAP")
+    Z, X, Y = tp.shape
+    K, R = 128, 301
+    from e3j_amd.tp_ops import _Table
+    table = _Table.get(tp.packed_coef(dtype), np_dtype)
+    sig, scale = table.signature(X, Y, Z, K, 0)
+    assert sig >= 0
+    g = torch.Generator(device="cpu").manual_seed(5)
+    x = (0.5 * torch.randn(R, X, K, generator=g)).to(tdtype).to(DEV)
+    y = (0.5 * torch.randn(R, Y, K, generator=g)).to(tdtype).to(DEV)
+    dz = (0.5 * torch.randn(R, Z, K, generator=g)).to(tdtype).to(DEV)
+    stream = int(torch.cuda.current_stream().cuda_stream)
+    results = []
+    for signature in (sig, -1):
+        p = _lib.TpParams(num_rows=R, num_coef=table.num_coef, num_x=X, num_y=Y, num_out=Z, channels_x=K,
+                          channels_y=K, mode=_lib.MODE_MAP, layout=_lib.LAYOUT_TRAILING,
+                          val_dtype=_lib.F64 if dtype == "float64" else _lib.F16, coef_idx_bytes=table.idx_bytes,
+                          coef_sorted=1, debug=1, signature=signature,
+                          coef_scale=scale if isinstance(scale, float) else 1.0)
+        if signature >= 0 and dtype == "float64":
+            p.coef_classes = ctypes.cast(scale, ctypes.c_void_p).value
+        z = torch.full((R, Z, K), float("nan"), device=DEV, dtype=tdtype)
+        dx, dy = torch.full_like(x, float("nan")), torch.full_like(y, float("nan"))
+        coef = None if signature >= 0 else table.device(x.device).data_ptr()
+        coef_bwd = None if signature >= 0 else table.device(x.device, backward=True).data_ptr()
+        _lib.check(lib.e3j_amd_tensor_product_fwd(ctypes.byref(p), coef, x.data_ptr(), y.data_ptr(), z.data_ptr(), stream))
+        _lib.check(lib.e3j_amd_tensor_product_bwd(ctypes.byref(p), coef_bwd, x.data_ptr(), y.data_ptr(), dz.data_ptr(),
+                                                  dx.data_ptr(), dy.data_ptr(), stream))
+        results.append((z, dx, dy))
+    tol = dict(rtol=1e-12, atol=1e-12) if dtype == "float64" else dict(rtol=2e-2, atol=2e-2)
+    for a, b, name in zip(results[0], results[1], ("z", "dx", "dy")):
+        assert torch.isfinite(a).all(), name
+        torch.testing.assert_close(a, b, msg=lambda m, name=name: f"{name}: {m}", **tol)
+    # a float64 signature without its classes is refused
+    if dtype == "float64":
+        p = _lib.TpParams(num_rows=R, num_coef=table.num_coef, num_x=X, num_y=Y, num_out=Z, channels_x=K,
+                          channels_y=K, mode=_lib.MODE_MAP, layout=_lib.LAYOUT_TRAILING, val_dtype=_lib.F64,
+                          coef_idx_bytes=table.idx_bytes, coef_sorted=1, debug=0, signature=sig, coef_scale=1.0)
+        rc = lib.e3j_amd_tensor_product_fwd(ctypes.byref(p), None, x.data_ptr(), y.data_ptr(), results[0][0].data_ptr(),
+                                            stream)
+        assert rc == _lib.INVALID_ARGUMENT and b"coef_classes" in lib.e3j_amd_last_error()
+    torch.cuda.synchronize()
