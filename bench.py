@@ -41,8 +41,8 @@ HBM_PEAK_GBS = 8000.0
 #: hash of the kernel sources.  A figure is only quoted while the sources it was
 #: measured on are the ones in the tree.
 TRAFFIC_FILE = os.path.join(ROOT, "profiles", "traffic.json")
-KERNEL_SOURCES = ("e3j_amd/csrc/unrolled.h", "e3j_amd/csrc/common.h", "e3j_amd/csrc/tp_unrolled.h",
-                  "e3j_amd/codegen/gen_conv.py", "e3j_amd/codegen/gen_tp.py")
+#: (the sources of the convolution's unrolled kernels: the workloads of the file are convolutions)
+KERNEL_SOURCES = ("e3j_amd/csrc/unrolled.h", "e3j_amd/csrc/common.h", "e3j_amd/codegen/gen_conv.py")
 
 
 def kernel_source_hash() -> str:

@@ -137,9 +137,8 @@ def emit_source(name: str, desc: str, val, idx, shape, channels: int, symbols, i
     # float16 and float64 kernels: trailing layout, whole waves of channels
     wide = not leading and channels % 64 == 0
     class_of, num_classes = coefficient_classes(val)
-    if num_classes > F64_MAX_CLASSES:
-        wide = False
-    out += emit_sig(sig, val, idx, shape, f64=wide)
+    wide64 = wide and num_classes <= F64_MAX_CLASSES   # (a table of more magnitudes than the argument holds: no float64 kernels)
+    out += emit_sig(sig, val, idx, shape, f64=wide64)
     out += ["}  // namespace", "",
             "// host pass only: the registry entries hold host function pointers",
             "#if !defined(__HIP_DEVICE_COMPILE__)",
@@ -158,11 +157,10 @@ def emit_source(name: str, desc: str, val, idx, shape, channels: int, symbols, i
                 f"    &launch_tp_unrolled_fwd{suffix}<{args}>,",
                 f"    &launch_tp_unrolled_bwd{suffix}<{args}>,",
                 f"    {num_classes}, kClass,"]
-        if wide:
-            out += [f"    &launch_tp_unrolled_fwd_f16<{args}>, &launch_tp_unrolled_bwd_f16<{args}>,",
-                    f"    &launch_tp_unrolled_fwd_f64<{args}>, &launch_tp_unrolled_bwd_f64<{args}>,"]
-        else:
-            out += ["    nullptr, nullptr, nullptr, nullptr,"]
+        out += [f"    &launch_tp_unrolled_fwd_f16<{args}>, &launch_tp_unrolled_bwd_f16<{args}>," if wide
+                else "    nullptr, nullptr,",
+                f"    &launch_tp_unrolled_fwd_f64<{args}>, &launch_tp_unrolled_bwd_f64<{args}>," if wide64
+                else "    nullptr, nullptr,"]
         out += ["};"]
     if plugin:  # accessor a run-time compiled library is loaded through
         out += ["", f"static const TpSignature *const kPlugin[] = {{{', '.join('&' + sym for sym in symbols)}}};",
@@ -194,7 +192,7 @@ def emit_source(name: str, desc: str, val, idx, shape, channels: int, symbols, i
         out.append(bwd_args.format("int, "))
     else:
         narrow = channels < 64   # 16 or 32 channels: several rows side by side in a wave
-        for V in ("float", "half_t", "double") if wide else ("float",):
+        for V in ("float",) + (("half_t",) if wide else ()) + (("double",) if wide64 else ()):
             for uniform in ("false", "true"):
                 out.append(f"template __global__ void tp_unrolled_fwd_kernel<{sig}, {channels}, 4, {uniform}, {V}>(")
                 out.append(typed("fwd", V))

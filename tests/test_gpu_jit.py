@@ -128,3 +128,43 @@ def test_tensor_product_tables_run_on_generated_kernels(mode, layout, channels):
     mdx, mdy = T.tensor_product_vjp(idx, np.abs(val_r), np.abs(f64(x)), np.abs(f64(y)), np.abs(f64(dz)), mode, layout)
     H.assert_parity(dx.cpu().numpy(), rdx, mdx, "dx", ulps=32.0)
     H.assert_parity(dy.cpu().numpy(), rdy, mdy, "dy", ulps=32.0)
+
+
+@pytest.mark.parametrize("dtype", ["float16", "float64"])
+def test_tensor_product_generated_kernels_in_float16_and_float64(dtype):
+    """A table that is not built in, compiled at run time, serves float16 and float64 operands too
+    (trailing layout, 64 channels).  The float64 kernels exist when the table has at most 64
+    distinct magnitudes: a real Clebsch-Gordan table (here 0e+1o (x) 0e+1o+2e, scaled) has few."""
+    from e3j_amd import TensorProduct
+    from e3j_amd.coef import Coef
+    from e3j_amd.tp_ops import TensorProductParams, _Table as TpTable
+    from oracle import tp_oracle as T
+    rng = np.random.default_rng(8)
+    np_dtype = np.dtype(dtype)
+    tp = TensorProduct(("0e+1o", "0e+1o+2e"), None, layout="TRAILING_CHANNELS", mode="MAP")
+    Z, X, Y = tp.shape
+    idx = np.asarray(tp.indices, dtype=np.int64)
+    val = (0.75 * np.asarray(tp.values, dtype=np.float64)).astype(np_dtype)
+    coef = Coef(val, idx, dtype, "uint8").pack()
+    K, R = 64, 53
+    x = (0.5 * rng.normal(size=(R, X, K))).astype(np_dtype)
+    y = (0.5 * rng.normal(size=(R, Y, K))).astype(np_dtype)
+    p = TensorProductParams(num_out=Z, mode="MAP", layout="TRAILING_CHANNELS")
+    with e3j_amd.config.use(jit=True):
+        sig = TpTable.get(coef, np_dtype).signature(X, Y, Z, K, 0)[0]
+        assert sig >= 0, "the table must run on kernels compiled for it"
+        xt, yt = dev(x).requires_grad_(True), dev(y).requires_grad_(True)
+        z = e3j_amd.tensor_product(coef, xt, yt, p)
+        dz = (0.5 * rng.normal(size=tuple(z.shape))).astype(np_dtype)
+        dx, dy = torch.autograd.grad(z, (xt, yt), dev(dz))
+    f64 = lambda a: a.astype(np.float64)  # noqa: E731
+    v = f64(val)
+    lay = "TRAILING_CHANNELS"
+    ref = T.tensor_product_unfused(idx, v, f64(x), f64(y), Z, "MAP", lay)
+    mag = T.tensor_product_unfused(idx, np.abs(v), np.abs(f64(x)), np.abs(f64(y)), Z, "MAP", lay)
+    rdx, rdy = T.tensor_product_vjp(idx, v, f64(x), f64(y), f64(dz), "MAP", lay)
+    mdx, mdy = T.tensor_product_vjp(idx, np.abs(v), np.abs(f64(x)), np.abs(f64(y)), np.abs(f64(dz)), "MAP", lay)
+    for got, r, m, name in ((z, ref, mag, "z"), (dx, rdx, mdx, "dx"), (dy, rdy, mdy, "dy")):
+        err = np.abs(got.detach().double().cpu().numpy() - r)
+        bound = 64 * 2.0 ** -52 * m + 1e-300 if dtype == "float64" else 8 * 2.0 ** -10 * m + 1e-3
+        assert np.all(err <= bound), f"{name}: {err.max()} against magnitude {m.max()}"
