@@ -472,9 +472,11 @@ struct EdgeAhead {
     }
 };
 
-// Forward: a wave takes (row, 64 channels) and holds NB * 16 accumulators.
+// Forward: a wave takes (row, 64 channels) and holds NB * 16 accumulators: up to three blocks of
+// them leave room for three waves per SIMD (cfg2's table, 43 output coordinates: 0.35 ms with
+// three, 0.43 ms with two), more for two.
 template <typename Val, int NB, int XG>
-__global__ __launch_bounds__(256, 2) void planned_fwd_kernel(
+__global__ __launch_bounds__(256, NB <= 3 ? 3 : 2) void planned_fwd_kernel(
     const int32_t *__restrict__ plan, PlanLayout L, const Val *__restrict__ x, RowLayout lx,
     const Val *__restrict__ y, int num_y, const Val *__restrict__ s, RowLayout ls,
     const int32_t *__restrict__ other, const int32_t *__restrict__ row_ptr, const int32_t *__restrict__ perm,
