@@ -543,15 +543,17 @@ def bench_tensor_product(args, torch, device) -> int:
     K, R = args.channels or 128, args.rows
     tp = TensorProduct(("0e+1o+2e+3o", "0e+1o+2e+3o"), "0e+1o+2e+3o", layout=layout, mode=args.mode)
     Z, X, Y = tp.shape
-    coef = tp.packed_coef("float32")
+    name = {"f32": "float32", "f64": "float64", "f16": "float16"}[args.dtype]
+    tdtype = getattr(torch, name)
+    coef = tp.packed_coef(name)
     params = TensorProductParams(num_out=Z, mode=args.mode, layout=layout)
     g = torch.Generator(device=device).manual_seed(0)
-    x = torch.randn((R, X, K) if trailing else (R, K, X), device=device, generator=g)
+    x = torch.randn((R, X, K) if trailing else (R, K, X), device=device, generator=g).to(tdtype)
     has_cy = args.mode != "OUTER"
-    y = torch.randn(((R, Y, K) if trailing else (R, K, Y)) if has_cy else (R, Y), device=device, generator=g)
+    y = torch.randn(((R, Y, K) if trailing else (R, K, Y)) if has_cy else (R, Y), device=device, generator=g).to(tdtype)
     meta = _make_meta(coef, x, y, params)
     z = _raw_forward(meta, x, y)
-    dz = torch.randn(tuple(z.shape), device=device, generator=g)
+    dz = torch.randn(tuple(z.shape), device=device, generator=g).to(tdtype)
     signature = _params(meta, x, y, backward=False).signature
     xg, yg = x.detach().requires_grad_(True), y.detach().requires_grad_(True)
 
@@ -569,18 +571,19 @@ def bench_tensor_product(args, torch, device) -> int:
     ms_per_step = (time.perf_counter() - t0) * 1e3 / args.steps
     fwd_ms = time_events(torch, lambda: _raw_forward(meta, x, y), args.steps, 2)
     bwd_ms = time_events(torch, lambda: _raw_backward(meta, x, y, dz), args.steps, 2)
-    fwd_bytes = 4 * (x.numel() + y.numel() + z.numel())
-    bwd_bytes = 4 * (2 * x.numel() + 2 * y.numel() + z.numel())
+    width = x.element_size()
+    fwd_bytes = width * (x.numel() + y.numel() + z.numel())
+    bwd_bytes = width * (2 * x.numel() + 2 * y.numel() + z.numel())
 
     def gbs(nbytes, ms):
         return nbytes / (ms * 1e-3) / 1e9
 
-    measured = MEASURED_TP_TRAFFIC_BYTES.get((args.mode, args.layout, R, K), {})
+    measured = MEASURED_TP_TRAFFIC_BYTES.get((args.mode, args.layout, R, K), {}) if args.dtype == "f32" else {}
     result = {
-        "metric": "rows/sec fused TensorProduct fwd+VJP fp32; achieved HBM GB/s vs peak",
+        "metric": "rows/sec fused TensorProduct fwd+VJP " + args.dtype.replace("f", "fp") + "; achieved HBM GB/s vs peak",
         "value": R / (ms_per_step * 1e-3), "unit": "rows/s", "n_gpus": 1, "steps": args.steps,
         "warmup": args.warmup, "ms_per_step": ms_per_step, "higher_is_better": True, "scaling": "weak",
-        "vs_baseline": None, "dtype": "f32", "data": "synthetic",
+        "vs_baseline": None, "dtype": args.dtype, "data": "synthetic",
         "config": {"workload": f"row-wise tensor product 0e+1o+2e+3o (x) 0e+1o+2e+3o -> l <= 3 ({len(tp.values)} "
                                f"coefficients, {Z} output coordinates), {R} rows, {K} channels, mode {args.mode}, "
                                f"{args.layout}-channels layout, forward + VJP (dx, dy)",
@@ -601,7 +604,7 @@ def bench_tensor_product(args, torch, device) -> int:
         from oracle import tp_oracle
         idx, val = np.asarray(tp.indices, dtype=np.int64), np.asarray(tp.values, dtype=np.float32)
         rows = 2048
-        xs, ys, dzs = (t[:rows].cpu().numpy() for t in (x, y, dz))
+        xs, ys, dzs = (t[:rows].float().cpu().numpy() for t in (x, y, dz))
         t0 = time.perf_counter()
         reps = 0
         while time.perf_counter() - t0 < args.cpu_seconds:

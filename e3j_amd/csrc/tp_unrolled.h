@@ -102,10 +102,11 @@ struct RegLoad {
     __device__ __forceinline__ A get() const { return v[I]; }
 };
 
-__device__ __forceinline__ double tp_vgpr(double v) {
-    asm volatile("" : "+v"(v));
-    return v;
-}
+// The wave-uniform y of the uniform-y backward: float values are moved to vector registers (the
+// arithmetic then never meets the limit of scalar operands per instruction); doubles stay where
+// the compiler puts them, in scalar registers, which leaves the kernel 32 vector registers more
+// (float64, l<=3, K=128, 262 144 rows: 10.1 ms instead of 11.8 ms).
+__device__ __forceinline__ double tp_vgpr(double v) { return v; }
 __device__ __forceinline__ float tp_vgpr(float v) { return to_vgpr(v); }
 
 __device__ __forceinline__ int64_t tp_uniform(int64_t v) {
@@ -205,6 +206,8 @@ struct TpUniformGeometry {
     static constexpr int WPB = SL * RPB;
 };
 
+// (float64, l<=3: more than 256 registers, one wave per SIMD resident; bounded to 256 it spills
+// and takes twice the time)
 template <typename Sig, int K, typename V = float>
 __global__ __launch_bounds__(kWave * TpUniformGeometry<K>::WPB) void tp_unrolled_bwd_uniform_kernel(
     const V *__restrict__ x, const V *__restrict__ y, const V *__restrict__ dz,
