@@ -163,6 +163,9 @@ SYMBOLS = {
     "e3j_amd_harmonics_bwd": (ctypes.c_int, [_P, _P, ctypes.c_int64] + [ctypes.c_int32] * 4 + [_P, _P]),
     "e3j_amd_edge_features_fwd": (ctypes.c_int, [ctypes.POINTER(EdgeFeaturesParams)] + [_P] * 9),
     "e3j_amd_edge_features_bwd": (ctypes.c_int, [ctypes.POINTER(EdgeFeaturesParams)] + [_P] * 10),
+    "e3j_amd_channel_mix": (ctypes.c_int, [_P, _P, _P, ctypes.c_int64, ctypes.c_int32, ctypes.c_int32,
+                                           ctypes.POINTER(ctypes.c_int32), ctypes.POINTER(ctypes.c_int32),
+                                           ctypes.c_int32, _P]),
     "e3j_amd_rows_regroup": (ctypes.c_int, [_P, _P, ctypes.c_int64, ctypes.c_int32, ctypes.c_int32, _P, _P,
                                             ctypes.c_int32, ctypes.c_int32, _P]),
     "e3j_amd_radial_linear_fwd": (ctypes.c_int, [_P, _P, _P, ctypes.c_int64, ctypes.c_int32, ctypes.c_int32, _P]),

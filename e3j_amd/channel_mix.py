@@ -2,10 +2,12 @@
 
 The convolution writes, for every output degree `l`, `mul` copies of `2l + 1` rows; the linear layer
 that follows mixes copies and channels per degree (`src/e3j/core/linear.py:125-243` in the reference:
-slices, a product per block, a join).  Here one kernel launch regroups all rows into the operands
-`A_l[(n, m), (u, k)]` of one library matrix product per degree (`csrc/channel_mix.hip`), a second
-puts the results into `(N, X, K)`; the backward pass runs the same two moves in the other direction,
-so that every cotangent row is written once.
+slices, a product per block, a join).  Here float32 rows of 64 or 128 channels are mixed by one
+launch of a matrix-core kernel each way (`e3j_amd_channel_mix`, `csrc/channel_mix.hip`); other
+dtypes and channel counts take one kernel launch that regroups all rows into the operands
+`A_l[(n, m), (u, k)]` of one library matrix product per degree, and a second that puts the results
+into `(N, X, K)`; the backward pass runs the same moves in the other direction, so that every
+cotangent row is written once.
 """
 
 from __future__ import annotations
@@ -87,7 +89,35 @@ class ChannelMix:
             hit = self._device[key] = torch.as_tensor(self._weights[l], dtype=like.dtype, device=like.device)
         return hit
 
+    def _fused(self, src: torch.Tensor, transpose: bool):
+        """The mixing (or its transpose) in one launch of the library's matrix-core kernel, or None
+        where that kernel does not apply (it takes float32 at 64 or 128 channels, up to 8 degrees)."""
+        import ctypes
+        K = self.channels
+        if src.dtype != torch.float32 or K not in (64, 128) or len(self.blocks) > 8 or src.data_ptr() % 16:
+            return None
+        key = ("fused", transpose, src.device)
+        w = self._device.get(key)
+        if w is None:
+            parts = [wl.reshape(m, K, K) for wl, (m, _) in zip(self._weights, self.blocks)]
+            if transpose:
+                parts = [p.transpose(0, 2, 1) for p in parts]
+            flat = np.concatenate([np.ascontiguousarray(p, dtype=np.float32).reshape(-1) for p in parts])
+            w = self._device[key] = torch.as_tensor(flat, device=src.device)
+        n = int(src.shape[0])
+        dst = torch.empty((n, self.rows_in if transpose else self.rows_out, K), dtype=src.dtype, device=src.device)
+        mul = (ctypes.c_int32 * len(self.blocks))(*[m for m, _ in self.blocks])
+        dim = (ctypes.c_int32 * len(self.blocks))(*[d for _, d in self.blocks])
+        with torch.cuda.device(src.device):
+            _lib.check(_lib.load().e3j_amd_channel_mix(
+                src.data_ptr(), dst.data_ptr(), w.data_ptr(), n, K, len(self.blocks), mul, dim, int(transpose),
+                int(torch.cuda.current_stream(src.device).cuda_stream)))
+        return dst
+
     def _forward(self, out: torch.Tensor, weights) -> torch.Tensor:
+        fused = self._fused(out, transpose=False)
+        if fused is not None:
+            return fused
         n, K = int(out.shape[0]), self.channels
         a_base, a_stride, c_base, c_stride, spans = self._tables(n, out.device)
         grouped = torch.empty(n * self.rows_in * K, dtype=out.dtype, device=out.device)
@@ -101,6 +131,9 @@ class ChannelMix:
         return x
 
     def _backward(self, dx: torch.Tensor, weights, n: int) -> torch.Tensor:
+        fused = self._fused(dx, transpose=True)
+        if fused is not None:
+            return fused
         K = self.channels
         a_base, a_stride, c_base, c_stride, spans = self._tables(n, dx.device)
         dmixed = torch.empty(n * self.rows_out * K, dtype=dx.dtype, device=dx.device)

@@ -433,6 +433,19 @@ int e3j_amd_edge_features_bwd(const e3j_amd_edge_features_params *p, const void 
 int e3j_amd_rows_regroup(const void *src, void *dst, int64_t num_nodes, int32_t rows, int32_t channels,
                          const int64_t *row_base, const int64_t *row_stride, int32_t to_plain,
                          int32_t val_dtype, void *stream);
+/* The same mixing in one launch on the matrix cores (float32, 64 or 128 channels, 16-byte aligned
+ * operands): no regrouped copies, no library products.  The convolution's output has, for each of
+ * num_degrees output degrees in row order, mul[l] copies of dim[l] = 2l + 1 rows (mul, dim: HOST
+ * arrays, num_degrees <= 8).  transpose = 0: src (num_nodes, sum mul dim, channels), weights the
+ * concatenation of W_l[u][k][c] (mul[l] x channels x channels each), dst (num_nodes, sum dim,
+ * channels) with dst[n, m_l, c] = sum_{u, k} src[n, base_l + u dim_l + m, k] W_l[u][k][c].
+ * transpose = 1 (the backward pass): src (num_nodes, sum dim, channels), weights the
+ * concatenation of the transposed W_l[u][c][k], dst (num_nodes, sum mul dim, channels) with
+ * dst[n, base_l + u dim_l + m, k] = sum_c src[n, m_l, c] W_l[u][k][c].  Every row of dst is
+ * written once.  No counterpart in the reference (src/e3j/core/linear.py:125-243 under XLA). */
+int e3j_amd_channel_mix(const void *src, void *dst, const void *weights, int64_t num_nodes, int32_t channels,
+                        int32_t num_degrees, const int32_t *mul, const int32_t *dim, int32_t transpose,
+                        void *stream);
 
 /* Last layer of the radial network that produces the convolution's per-edge, per-path weights:
  * s (num_edges, n) = h (num_edges, inner) w (inner, n), n = paths * channels, float32, row-major,

@@ -76,10 +76,13 @@ def test_edge_features_on_an_empty_edge_list_and_errors():
         edge_features(pos, none, none, None, torch.rand(1, 17, 4, device="cuda"), 3, 5.0)
 
 
-@pytest.mark.parametrize("dtype", [torch.float32, torch.float64])
-def test_channel_mix_matches_the_oracle(dtype):
+@pytest.mark.parametrize("dtype,K", [(torch.float32, 64), (torch.float32, 128), (torch.float32, 32),
+                                     (torch.float64, 64)])
+def test_channel_mix_matches_the_oracle(dtype, K):
+    """float32 at 64 and 128 channels: the matrix-core kernel, one launch each way; 32 channels and
+    float64: row regrouping around library products.  37 nodes: a whole tile of 32 and a partial one."""
     rng = np.random.default_rng(5)
-    blocks, K, n = [(4, 1), (6, 3), (7, 5), (6, 7)], 64, 37
+    blocks, n = [(4, 1), (6, 3), (7, 5), (6, 7)], 37
     Z = sum(m * d for m, d in blocks)
     out = rng.normal(size=(n, Z, K))
     weights = [rng.normal(size=(m, K, K)) / np.sqrt(m * K) for m, _ in blocks]
